@@ -1,0 +1,232 @@
+// Device-side helpers shared by every fusion-group kernel (gfx950, wave64).
+// This header is embedded into the library and handed to hiprtc together with the
+// kernel text that the fusion code generator writes for one module.
+#pragma once
+
+typedef unsigned char rx_u8;
+typedef unsigned short rx_u16;
+typedef unsigned int rx_u32;
+typedef unsigned long long rx_u64;
+typedef signed char rx_i8;
+typedef short rx_i16;
+typedef int rx_i32;
+typedef long long rx_i64;
+
+#define RX_DEV static __device__ __forceinline__
+#define RX_MEM __device__ __forceinline__
+
+template <typename T, int N>
+struct __attribute__((aligned(sizeof(T) * N))) rx_vec {
+  T v[N];
+};
+
+// ---------------------------------------------------------------------------
+// bit casts
+// ---------------------------------------------------------------------------
+RX_DEV rx_u32 rx_f2u(float f) { return __builtin_bit_cast(rx_u32, f); }
+RX_DEV float rx_u2f(rx_u32 u) { return __builtin_bit_cast(float, u); }
+
+// ---------------------------------------------------------------------------
+// bf16: storage is the upper half of binary32; conversion rounds to nearest even
+// ---------------------------------------------------------------------------
+RX_DEV float rx_bf16_to_f32(rx_u16 b) { return rx_u2f(((rx_u32)b) << 16); }
+RX_DEV rx_u16 rx_f32_to_bf16(float f) {
+  rx_u32 u = rx_f2u(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (rx_u16)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (rx_u16)(u >> 16);
+}
+RX_DEV float rx_round_bf16(float f) { return rx_bf16_to_f32(rx_f32_to_bf16(f)); }
+
+// ---------------------------------------------------------------------------
+// f16
+// ---------------------------------------------------------------------------
+RX_DEV float rx_f16_to_f32(rx_u16 b) { return (float)__builtin_bit_cast(_Float16, b); }
+RX_DEV rx_u16 rx_f32_to_f16(float f) { return __builtin_bit_cast(rx_u16, (_Float16)f); }
+RX_DEV float rx_round_f16(float f) { return (float)(_Float16)f; }
+
+// ---------------------------------------------------------------------------
+// f8E4M3FN (OCP e4m3: bias 7, no inf, S.1111.111 = NaN, max 448)
+// f8E5M2   (bias 15, inf and NaN as in binary16)
+// Round to nearest even; a value that rounds above the largest finite number
+// becomes NaN (e4m3fn) or inf (e5m2).
+// ---------------------------------------------------------------------------
+RX_DEV float rx_e4m3_to_f32(rx_u8 b) {
+  rx_u32 s = ((rx_u32)(b & 0x80u)) << 24;
+  rx_u32 e = (b >> 3) & 0xfu;
+  rx_u32 m = b & 7u;
+  if (e == 0xfu && m == 7u) return rx_u2f(s | 0x7fc00000u);
+  if (e == 0) {
+    float v = (float)m * 0.001953125f;  // m * 2^-9
+    return rx_u2f(rx_f2u(v) | s);
+  }
+  return rx_u2f(s | ((e + 120u) << 23) | (m << 20));
+}
+RX_DEV rx_u8 rx_f32_to_e4m3(float f) {
+  rx_u32 u = rx_f2u(f);
+  rx_u8 s = (rx_u8)((u >> 24) & 0x80u);
+  rx_u32 a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (rx_u8)(s | 0x7fu);       // NaN
+  if (a > 0x43e80000u) return (rx_u8)(s | 0x7fu);       // |x| > 464 rounds past 448 (inf too)
+  if (a < 0x3c800000u) {                                // |x| < 2^-6: subnormal range
+    float v = rx_u2f(a) * 512.0f;                       // in units of 2^-9
+    float r = __builtin_rintf(v);                       // ties to even
+    return (rx_u8)(s | (rx_u8)(int)r);                  // r == 8 lands on the first normal
+  }
+  rx_u32 r = a + 0x7ffffu + ((a >> 20) & 1u);           // RNE at 3 mantissa bits
+  rx_u32 e = (r >> 23) - 120u;
+  rx_u32 m = (r >> 20) & 7u;
+  return (rx_u8)(s | (e << 3) | m);
+}
+RX_DEV float rx_round_e4m3(float f) { return rx_e4m3_to_f32(rx_f32_to_e4m3(f)); }
+
+RX_DEV float rx_e5m2_to_f32(rx_u8 b) {
+  rx_u16 h = (rx_u16)(((rx_u16)b) << 8);
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+RX_DEV rx_u8 rx_f32_to_e5m2(float f) {
+  rx_u32 u = rx_f2u(f);
+  rx_u8 s = (rx_u8)((u >> 24) & 0x80u);
+  rx_u32 a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (rx_u8)(s | 0x7fu);
+  if (a >= 0x47700000u) return (rx_u8)(s | 0x7cu);      // >= 61440 rounds to inf
+  if (a < 0x38800000u) {                                // |x| < 2^-14: subnormal range
+    float v = rx_u2f(a) * 65536.0f;                     // units of 2^-16
+    float r = __builtin_rintf(v);
+    return (rx_u8)(s | (rx_u8)(int)r);
+  }
+  rx_u32 r = a + 0xfffffu + ((a >> 21) & 1u);
+  rx_u32 e = (r >> 23) - 112u;
+  rx_u32 m = (r >> 21) & 3u;
+  return (rx_u8)(s | (e << 2) | m);
+}
+RX_DEV float rx_round_e5m2(float f) { return rx_e5m2_to_f32(rx_f32_to_e5m2(f)); }
+
+// ---------------------------------------------------------------------------
+// elementwise math with StableHLO semantics
+// ---------------------------------------------------------------------------
+template <typename T> RX_DEV T rx_max(T a, T b) { return (a > b || a != a) ? a : b; }
+template <typename T> RX_DEV T rx_min(T a, T b) { return (a < b || a != a) ? a : b; }
+template <typename T> RX_DEV T rx_sign(T a) {
+  return a != a ? a : (T)((a > (T)0) - (a < (T)0));
+}
+RX_DEV float rx_logistic(float x) { return 1.0f / (1.0f + expf(-x)); }
+RX_DEV double rx_logistic(double x) { return 1.0 / (1.0 + exp(-x)); }
+RX_DEV float rx_rsqrt(float x) { return 1.0f / sqrtf(x); }
+RX_DEV double rx_rsqrt(double x) { return 1.0 / sqrt(x); }
+RX_DEV float rx_gelu_tanh(float x) {
+  return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+RX_DEV float rx_gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f)); }
+RX_DEV float rx_gelu_sigmoid(float x) { return x / (1.0f + expf(-1.702f * x)); }
+RX_DEV double rx_gelu_tanh(double x) {
+  return 0.5 * x * (1.0 + tanh(0.7978845608028654 * (x + 0.044715 * x * x * x)));
+}
+RX_DEV double rx_gelu_erf(double x) { return 0.5 * x * (1.0 + erf(x * 0.7071067811865476)); }
+RX_DEV double rx_gelu_sigmoid(double x) { return x / (1.0 + exp(-1.702 * x)); }
+template <typename T> RX_DEV T rx_idiv(T a, T b) {
+  if (b == 0) return (T)-1;
+  if (b == (T)-1) return (T)(0 - a);
+  return a / b;
+}
+template <typename T> RX_DEV T rx_irem(T a, T b) {
+  if (b == 0) return a;
+  if (b == (T)-1) return (T)0;
+  return a % b;
+}
+template <typename T> RX_DEV T rx_ipow(T a, T b) {
+  if (b < 0) return (a == 1) ? (T)1 : ((a == (T)-1) ? ((b & 1) ? (T)-1 : (T)1) : (T)0);
+  T r = 1;
+  while (b) {
+    if (b & 1) r *= a;
+    a *= a;
+    b >>= 1;
+  }
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// wavefront (64 lanes) reductions.  32-bit payloads move through DPP row
+// operations; 64-bit payloads are moved as two halves.  The combined value
+// ends up in every lane.
+// ---------------------------------------------------------------------------
+template <int CTRL, int ROW_MASK>
+RX_DEV rx_i32 rx_dpp(rx_i32 v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xf, false);
+}
+template <typename T, int CTRL, int ROW_MASK>
+RX_DEV T rx_dpp_t(T v) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, rx_dpp<CTRL, ROW_MASK>(__builtin_bit_cast(rx_i32, v)));
+  } else if constexpr (sizeof(T) == 8) {
+    rx_u64 u = __builtin_bit_cast(rx_u64, v);
+    rx_u32 lo = (rx_u32)rx_dpp<CTRL, ROW_MASK>((rx_i32)(rx_u32)u);
+    rx_u32 hi = (rx_u32)rx_dpp<CTRL, ROW_MASK>((rx_i32)(rx_u32)(u >> 32));
+    return __builtin_bit_cast(T, ((rx_u64)hi << 32) | lo);
+  } else {
+    rx_i32 w = (rx_i32)v;
+    return (T)rx_dpp<CTRL, ROW_MASK>(w);
+  }
+}
+template <typename T>
+RX_DEV T rx_readlane63(T v) {
+  if constexpr (sizeof(T) == 8) {
+    rx_u64 u = __builtin_bit_cast(rx_u64, v);
+    rx_u32 lo = (rx_u32)__builtin_amdgcn_readlane((rx_i32)(rx_u32)u, 63);
+    rx_u32 hi = (rx_u32)__builtin_amdgcn_readlane((rx_i32)(rx_u32)(u >> 32), 63);
+    return __builtin_bit_cast(T, ((rx_u64)hi << 32) | lo);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(rx_i32, v), 63));
+  } else {
+    return (T)__builtin_amdgcn_readlane((rx_i32)v, 63);
+  }
+}
+
+struct rx_op_add { template <typename T> RX_MEM T operator()(T a, T b) const { return a + b; } };
+struct rx_op_mul { template <typename T> RX_MEM T operator()(T a, T b) const { return a * b; } };
+struct rx_op_max { template <typename T> RX_MEM T operator()(T a, T b) const { return rx_max(a, b); } };
+struct rx_op_min { template <typename T> RX_MEM T operator()(T a, T b) const { return rx_min(a, b); } };
+struct rx_op_and { template <typename T> RX_MEM T operator()(T a, T b) const { return (T)(a & b); } };
+struct rx_op_or { template <typename T> RX_MEM T operator()(T a, T b) const { return (T)(a | b); } };
+
+// Combine over the 64 lanes of a wavefront; the result is uniform.
+// Rows of 16 lanes are folded with quad permutes and row mirrors, then the row
+// totals travel down with row_bcast:15 / row_bcast:31 and lane 63 holds the total.
+template <typename T, typename OP>
+RX_DEV T rx_wave_reduce(T v, OP op) {
+  v = op(v, rx_dpp_t<T, 0xB1, 0xf>(v));   // quad_perm [1,0,3,2]
+  v = op(v, rx_dpp_t<T, 0x4E, 0xf>(v));   // quad_perm [2,3,0,1]
+  v = op(v, rx_dpp_t<T, 0x141, 0xf>(v));  // row_half_mirror
+  v = op(v, rx_dpp_t<T, 0x140, 0xf>(v));  // row_mirror: every lane holds its row total
+  T t = rx_dpp_t<T, 0x142, 0xa>(v);       // row_bcast:15 into rows 1 and 3
+  rx_u32 lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if ((lane >> 4) & 1u) v = op(v, t);
+  t = rx_dpp_t<T, 0x143, 0xc>(v);         // row_bcast:31 into rows 2 and 3
+  if (lane >= 32u) v = op(v, t);
+  return rx_readlane63(v);
+}
+
+// Combine over a workgroup of NWAVES wavefronts through LDS; result uniform.
+template <typename T, typename OP, int NWAVES>
+RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
+  v = rx_wave_reduce(v, op);
+  if constexpr (NWAVES == 1) return v;
+  const int w = threadIdx.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[w] = v;
+  __syncthreads();
+  T r = lds[0];
+#pragma unroll
+  for (int i = 1; i < NWAVES; ++i) r = op(r, lds[i]);
+  return r;
+}
+
+// XCD-aware placement: workgroups are dealt round-robin to the 8 XCDs, each with
+// its own L2.  This maps hardware workgroup id -> logical tile so that each XCD
+// walks one contiguous range of tiles.
+RX_DEV rx_u32 rx_xcd_remap(rx_u32 bid, rx_u32 nblocks) {
+  const rx_u32 per = nblocks >> 3;
+  const rx_u32 main = per << 3;
+  if (bid >= main) return bid;
+  return (bid & 7u) * per + (bid >> 3);
+}

@@ -1,0 +1,742 @@
+// Runtime (client, device, buffers, executables, futures) and the C ABI declared
+// in include/reactant_mi355x.h.
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <set>
+#include <unordered_set>
+#include <vector>
+
+#include "../../include/reactant_mi355x.h"
+#include "rx_embedded.inc"
+#include "rx_ir.h"
+#include "rx_plan.h"
+
+#define RX_EXPORT extern "C" __attribute__((visibility("default")))
+
+extern "C" __attribute__((visibility("default"))) void (*ReactantThrowError)(const char*) = nullptr;
+
+namespace {
+
+using rx::Error;
+
+thread_local std::string g_last_error;
+
+void report_error(const std::string& msg) {
+  g_last_error = msg;
+  if (ReactantThrowError) ReactantThrowError(msg.c_str());
+}
+
+#define HIP_CHECK(expr)                                                                                   \
+  do {                                                                                                    \
+    hipError_t e_ = (expr);                                                                               \
+    if (e_ != hipSuccess) throw Error(std::string(#expr) + " failed: " + hipGetErrorString(e_));          \
+  } while (0)
+
+char* dup_cstr(const std::string& s) {
+  char* p = (char*)malloc(s.size() + 1);
+  memcpy(p, s.c_str(), s.size() + 1);
+  return p;
+}
+
+// ---------------------------------------------------------------------------
+// handle registry
+// ---------------------------------------------------------------------------
+std::mutex g_reg_mu;
+std::unordered_set<const void*> g_handles;
+void reg_add(const void* p) { std::lock_guard<std::mutex> l(g_reg_mu); g_handles.insert(p); }
+void reg_del(const void* p) { std::lock_guard<std::mutex> l(g_reg_mu); g_handles.erase(p); }
+bool reg_has(const void* p) { std::lock_guard<std::mutex> l(g_reg_mu); return g_handles.count(p) != 0; }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// objects behind the opaque handles
+// ---------------------------------------------------------------------------
+struct RxClient;
+
+struct RxDevice {
+  RxClient* client = nullptr;
+  int ordinal = 0;       // HIP device ordinal
+  int index = 0;         // position in the client's device list
+  hipStream_t stream = nullptr;
+  std::string kind;
+  std::string arch;
+  // caching allocator: device memory is kept and reused by size class, because hipMalloc and
+  // hipFree are slow and hipFree synchronizes.  All work of a device runs on one stream, so
+  // a block freed by the host may be handed out again immediately: stream order protects it.
+  std::mutex mu;
+  std::multimap<size_t, void*> free_blocks;
+  int64_t num_allocs = 0, bytes_in_use = 0, peak_bytes_in_use = 0, largest_alloc = 0, pool_bytes = 0, peak_pool_bytes = 0;
+  int64_t bytes_limit = 0;
+
+  static size_t round_size(size_t n) {
+    if (n == 0) n = 1;
+    if (n <= (1u << 20)) return (n + 255) & ~(size_t)255;
+    return (n + 65535) & ~(size_t)65535;
+  }
+  void* alloc(size_t n) {
+    const size_t r = round_size(n);
+    std::lock_guard<std::mutex> l(mu);
+    auto it = free_blocks.find(r);
+    void* p = nullptr;
+    if (it != free_blocks.end()) {
+      p = it->second;
+      free_blocks.erase(it);
+    } else {
+      HIP_CHECK(hipSetDevice(ordinal));
+      hipError_t e = hipMalloc(&p, r);
+      if (e != hipSuccess) {
+        // give cached blocks back to the driver and retry once
+        (void)hipGetLastError();
+        for (auto& kv : free_blocks) { (void)hipFree(kv.second); pool_bytes -= (int64_t)kv.first; }
+        free_blocks.clear();
+        e = hipMalloc(&p, r);
+        if (e != hipSuccess) {
+          (void)hipGetLastError();
+          throw Error("RESOURCE_EXHAUSTED: out of device memory allocating " + std::to_string(r) + " bytes (" + hipGetErrorString(e) + ")");
+        }
+      }
+      pool_bytes += (int64_t)r;
+      peak_pool_bytes = std::max(peak_pool_bytes, pool_bytes);
+    }
+    num_allocs++;
+    bytes_in_use += (int64_t)r;
+    peak_bytes_in_use = std::max(peak_bytes_in_use, bytes_in_use);
+    largest_alloc = std::max<int64_t>(largest_alloc, (int64_t)r);
+    return p;
+  }
+  void release(void* p, size_t n) {
+    const size_t r = round_size(n);
+    std::lock_guard<std::mutex> l(mu);
+    bytes_in_use -= (int64_t)r;
+    free_blocks.insert({r, p});
+  }
+  void drain() {
+    std::lock_guard<std::mutex> l(mu);
+    for (auto& kv : free_blocks) (void)hipFree(kv.second);
+    free_blocks.clear();
+    pool_bytes = 0;
+  }
+};
+
+struct Allocation {
+  RxDevice* dev;
+  void* ptr;
+  size_t bytes;
+  Allocation(RxDevice* d, size_t n) : dev(d), ptr(d->alloc(n)), bytes(n) {}
+  ~Allocation() { dev->release(ptr, bytes); }
+  Allocation(const Allocation&) = delete;
+};
+using Mem = std::shared_ptr<Allocation>;
+
+struct RxClient {
+  std::vector<std::unique_ptr<RxDevice>> devices;
+  std::atomic<bool> alive{true};
+};
+
+struct RxBuffer {
+  RxClient* client = nullptr;
+  RxDevice* device = nullptr;
+  Mem mem;                       // empty once donated
+  rx::TType ty;
+  bool donated = false;
+};
+
+struct RxFuture {
+  hipEvent_t ev = nullptr;
+  RxDevice* device = nullptr;
+  std::string error;
+};
+
+struct RxExecutable {
+  RxClient* client = nullptr;
+  RxDevice* device = nullptr;
+  rx::Plan plan;
+  hipModule_t module = nullptr;
+  std::vector<hipFunction_t> fns;   // per launch
+  std::vector<Mem> consts;          // per plan buffer (only Const kinds are set)
+  std::string report;
+  std::mutex mu;
+};
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// hiprtc
+// ---------------------------------------------------------------------------
+std::string rtc_compile(const std::string& source, const std::string& arch) {
+  hiprtcProgram prog;
+  const char* hdr_src[] = {kRxPreambleSrc, kRxGemmKernelsSrc};
+  const char* hdr_name[] = {"rx_preamble.h", "rx_gemm_kernels.h"};
+  hiprtcResult r = hiprtcCreateProgram(&prog, source.c_str(), "rx_module.hip", 2, hdr_src, hdr_name);
+  if (r != HIPRTC_SUCCESS) throw Error(std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r));
+  std::string archopt = "--offload-arch=" + arch;
+  std::vector<const char*> opts = {archopt.c_str(), "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
+                                   "-packed-fp32-ops", "-Wno-unused-value"};
+  r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
+  size_t ls = 0;
+  hiprtcGetProgramLogSize(prog, &ls);
+  std::string log(ls, '\0');
+  if (ls) hiprtcGetProgramLog(prog, &log[0]);
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    if (getenv("RX_DUMP_FAILED_SOURCE")) {
+      FILE* f = fopen(getenv("RX_DUMP_FAILED_SOURCE"), "w");
+      if (f) { fputs(source.c_str(), f); fclose(f); }
+    }
+    throw Error(std::string("kernel compilation failed (") + hiprtcGetErrorString(r) + "):\n" + log);
+  }
+  size_t cs = 0;
+  hiprtcGetCodeSize(prog, &cs);
+  std::string code(cs, '\0');
+  hiprtcGetCode(prog, &code[0]);
+  hiprtcDestroyProgram(&prog);
+  return code;
+}
+
+rx::PlanOptions plan_options() {
+  rx::PlanOptions o;
+  if (const char* e = getenv("RX_XCD_SLABS")) o.xcd_slabs = atoi(e) != 0;
+  if (const char* e = getenv("RX_SLAB_MIN_NUMEL")) o.slab_min_numel = atoll(e);
+  if (const char* e = getenv("RX_MFMA")) o.mfma = atoi(e) != 0;
+  if (const char* e = getenv("RX_ROW_FUSION")) o.row_fusion = atoi(e) != 0;
+  if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;
+  return o;
+}
+
+int64_t prim_numel(size_t nd, const int64_t* dims) {
+  int64_t n = 1;
+  for (size_t k = 0; k < nd; ++k) n *= dims[k];
+  return n;
+}
+
+template <typename F>
+auto guarded(F&& f, decltype(f()) fallback) -> decltype(f()) {
+  try {
+    return f();
+  } catch (const std::exception& e) {
+    report_error(e.what());
+    return fallback;
+  }
+}
+template <typename F>
+void guarded_void(F&& f) {
+  try {
+    f();
+  } catch (const std::exception& e) {
+    report_error(e.what());
+  }
+}
+
+void check_client(RxClient* c) { if (!c || !reg_has(c)) throw Error("INVALID_ARGUMENT: null or foreign client handle"); }
+void check_device(RxDevice* d) { if (!d || !reg_has(d)) throw Error("INVALID_ARGUMENT: null or foreign device handle"); }
+void check_buffer(RxBuffer* b) { if (!b || !reg_has(b)) throw Error("INVALID_ARGUMENT: null or foreign buffer handle"); }
+void check_exec(RxExecutable* e) { if (!e || !reg_has(e)) throw Error("INVALID_ARGUMENT: null or foreign executable handle"); }
+
+RxBuffer* new_buffer(RxClient* c, RxDevice* d, const rx::TType& ty, Mem mem) {
+  RxBuffer* b = new RxBuffer;
+  b->client = c;
+  b->device = d;
+  b->ty = ty;
+  b->mem = std::move(mem);
+  reg_add(b);
+  return b;
+}
+
+// AOT kernels ------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+// Core of XLAExecuteSharded / RxExecuteTimed
+void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uint8_t* donate, int num_results, RxBuffer** results, float* launch_ms,
+             RxFuture** futures) {
+  check_exec(ex);
+  if (dev) check_device(dev);
+  if (!dev) dev = ex->device;
+  if (dev != ex->device) throw Error("INVALID_ARGUMENT: executable was compiled for another device");
+  const rx::Plan& P = ex->plan;
+  if (num_args != (int)P.param_types.size())
+    throw Error("INVALID_ARGUMENT: executable expects " + std::to_string(P.param_types.size()) + " arguments, got " + std::to_string(num_args));
+  if (num_results != (int)P.result_types.size())
+    throw Error("Error: results.size()=" + std::to_string(P.result_types.size()) + " does not match num_results=" + std::to_string(num_results) + "\n");
+  for (int i = 0; i < num_args; ++i) {
+    check_buffer(args[i]);
+    if (args[i]->donated || !args[i]->mem) throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " was donated to an earlier execution");
+    if (!(args[i]->ty == P.param_types[i]))
+      throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " has type " + args[i]->ty.str() + ", executable expects " + P.param_types[i].str());
+    if (args[i]->device != dev) throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " lives on another device");
+  }
+  std::lock_guard<std::mutex> lock(ex->mu);
+  HIP_CHECK(hipSetDevice(dev->ordinal));
+  const size_t NB = P.buffers.size();
+  std::vector<Mem> bufs(NB);
+  std::vector<char> is_res(NB, 0);
+  for (int b : P.result_buffers) is_res[b] = 1;
+  for (size_t b = 0; b < NB; ++b) {
+    const auto& B = P.buffers[b];
+    if (B.kind == rx::BufferDesc::Param) {
+      RxBuffer* a = args[B.param_index];
+      bufs[b] = a->mem;
+    } else if (B.kind == rx::BufferDesc::Const) {
+      bufs[b] = ex->consts[b];
+    }
+  }
+  // donated arguments give up their storage now; the plan drops it after its last use
+  for (int i = 0; i < num_args; ++i) {
+    if (donate && donate[i]) {
+      args[i]->donated = true;
+      args[i]->mem.reset();
+    }
+  }
+  std::vector<hipEvent_t> evs;
+  if (launch_ms) {
+    evs.resize(P.launches.size() + 1);
+    for (auto& e : evs) HIP_CHECK(hipEventCreate(&e));
+    HIP_CHECK(hipEventRecord(evs[0], dev->stream));
+  }
+  std::vector<void*> ptrs;
+  std::vector<void*> argv;
+  for (size_t li = 0; li < P.launches.size(); ++li) {
+    const auto& L = P.launches[li];
+    ptrs.clear();
+    argv.clear();
+    for (int b : L.args) {
+      if (!bufs[b]) {
+        const auto& B = P.buffers[b];
+        if (B.kind == rx::BufferDesc::Param || B.kind == rx::BufferDesc::Const) throw Error("internal: unbound input buffer");
+        bufs[b] = std::make_shared<Allocation>(dev, (size_t)B.bytes);
+      }
+      ptrs.push_back(bufs[b]->ptr);
+    }
+    for (auto& p : ptrs) argv.push_back(&p);
+    HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
+                                    argv.data(), nullptr));
+    if (launch_ms) HIP_CHECK(hipEventRecord(evs[li + 1], dev->stream));
+    for (int b : L.args) {
+      const auto& B = P.buffers[b];
+      if (B.last_use == (int)li && !is_res[b]) bufs[b].reset();
+    }
+  }
+  for (int r = 0; r < num_results; ++r) {
+    const int b = P.result_buffers[r];
+    const auto& B = P.buffers[b];
+    Mem m = bufs[b];
+    if (B.kind == rx::BufferDesc::Const) {
+      // a constant returned as a result gets its own copy: the caller may donate it later
+      m = std::make_shared<Allocation>(dev, (size_t)B.bytes);
+      HIP_CHECK(hipMemcpyAsync(m->ptr, ex->consts[b]->ptr, (size_t)B.bytes, hipMemcpyDeviceToDevice, dev->stream));
+    } else if (B.kind == rx::BufferDesc::Param && !m) {
+      throw Error("internal: pass-through result lost its storage");
+    } else if (!m) {
+      m = std::make_shared<Allocation>(dev, (size_t)B.bytes);  // nothing wrote it (empty tensor)
+    }
+    results[r] = new_buffer(ex->client, dev, P.result_types[r], m);
+  }
+  if (futures) {
+    // one event shared by all result futures would need ref counting; events are cheap
+    for (int r = 0; r < num_results; ++r) {
+      RxFuture* f = new RxFuture;
+      f->device = dev;
+      HIP_CHECK(hipEventCreateWithFlags(&f->ev, hipEventDisableTiming));
+      HIP_CHECK(hipEventRecord(f->ev, dev->stream));
+      reg_add(f);
+      futures[r] = f;
+    }
+  }
+  if (launch_ms) {
+    HIP_CHECK(hipEventSynchronize(evs.back()));
+    for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[li], evs[li + 1]));
+    for (auto& e : evs) (void)hipEventDestroy(e);
+  }
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+RX_EXPORT int RxOwns(const void* h) { return h && reg_has(h) ? 1 : 0; }
+RX_EXPORT const char* RxLastError(void) { return g_last_error.c_str(); }
+RX_EXPORT void RxClearError(void) { g_last_error.clear(); }
+RX_EXPORT void InitializeLogs(void) {}
+RX_EXPORT void SetLogLevel(int) {}
+
+RX_EXPORT RxClient* MakeGPUClient(int node_id, int num_nodes, int64_t* allowed_devices, int64_t num_allowed_devices, double memory_fraction,
+                                  bool preallocate, const char* platform_name, const char** error, void* distributed_runtime_client) {
+  (void)preallocate;
+  (void)platform_name;
+  (void)distributed_runtime_client;
+  try {
+    if (num_nodes > 1 || node_id != 0) throw Error("INVALID_ARGUMENT: this backend runs one process on one GPU (num_nodes must be 1, node_id 0)");
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) throw Error(std::string("NOT_FOUND: no HIP device is visible (") + hipGetErrorString(e) + ")");
+    std::vector<int> ords;
+    if (allowed_devices && num_allowed_devices > 0) {
+      for (int64_t k = 0; k < num_allowed_devices; ++k) {
+        if (allowed_devices[k] < 0 || allowed_devices[k] >= count) throw Error("INVALID_ARGUMENT: allowed device " + std::to_string(allowed_devices[k]) + " does not exist");
+        ords.push_back((int)allowed_devices[k]);
+      }
+    } else ords.push_back(0);
+    auto c = std::make_unique<RxClient>();
+    for (size_t k = 0; k < ords.size(); ++k) {
+      auto d = std::make_unique<RxDevice>();
+      d->client = c.get();
+      d->ordinal = ords[k];
+      d->index = (int)k;
+      HIP_CHECK(hipSetDevice(d->ordinal));
+      hipDeviceProp_t prop;
+      HIP_CHECK(hipGetDeviceProperties(&prop, d->ordinal));
+      d->kind = prop.name;
+      d->arch = prop.gcnArchName;
+      if (d->arch.rfind("gfx950", 0) != 0)
+        throw Error("FAILED_PRECONDITION: device " + std::to_string(d->ordinal) + " is " + d->arch + "; this backend only targets gfx950 (MI355X)");
+      size_t fr = 0, tot = 0;
+      HIP_CHECK(hipMemGetInfo(&fr, &tot));
+      d->bytes_limit = (int64_t)((memory_fraction > 0 && memory_fraction <= 1 ? memory_fraction : 1.0) * (double)tot);
+      HIP_CHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+      reg_add(d.get());
+      c->devices.push_back(std::move(d));
+    }
+    RxClient* raw = c.release();
+    reg_add(raw);
+    return raw;
+  } catch (const std::exception& ex) {
+    g_last_error = ex.what();
+    if (error) *error = dup_cstr(ex.what());
+    else report_error(ex.what());
+    return nullptr;
+  }
+}
+
+RX_EXPORT void FreeClient(RxClient* c) {
+  guarded_void([&] {
+    check_client(c);
+    c->alive = false;
+    for (auto& d : c->devices) {
+      (void)hipSetDevice(d->ordinal);
+      (void)hipStreamSynchronize(d->stream);
+      d->drain();
+      (void)hipStreamDestroy(d->stream);
+      reg_del(d.get());
+    }
+    reg_del(c);
+    // Buffers freed after this point (late finalizers) still reach their RxDevice through the
+    // shared allocation, so the client object itself is kept alive for the life of the process.
+  });
+}
+
+RX_EXPORT int ClientNumDevices(RxClient* c) { return guarded([&] { check_client(c); return (int)c->devices.size(); }, 0); }
+RX_EXPORT int ClientNumAddressableDevices(RxClient* c) { return ClientNumDevices(c); }
+RX_EXPORT int ClientProcessIndex(RxClient* c) { return guarded([&] { check_client(c); return 0; }, 0); }
+RX_EXPORT RxDevice* ClientGetDevice(RxClient* c, int id) {
+  return guarded([&]() -> RxDevice* {
+    check_client(c);
+    if (id < 0 || id >= (int)c->devices.size()) throw Error("INVALID_ARGUMENT: no device with id " + std::to_string(id));
+    return c->devices[id].get();
+  }, nullptr);
+}
+RX_EXPORT RxDevice* ClientGetAddressableDevice(RxClient* c, int id) { return ClientGetDevice(c, id); }
+RX_EXPORT const char* ClientGetPlatformName(RxClient* c) {
+  return guarded([&]() -> const char* { check_client(c); return dup_cstr("rocm"); }, nullptr);
+}
+RX_EXPORT void ClientGetDevices(RxClient* c, RxDevice** out) {
+  guarded_void([&] { check_client(c); for (size_t k = 0; k < c->devices.size(); ++k) out[k] = c->devices[k].get(); });
+}
+RX_EXPORT void ClientGetAddressableDevices(RxClient* c, RxDevice** out) { ClientGetDevices(c, out); }
+RX_EXPORT const char* DeviceGetKind(RxDevice* d) {
+  return guarded([&]() -> const char* { check_device(d); return dup_cstr(d->kind); }, nullptr);
+}
+RX_EXPORT RxClient* DeviceToClient(RxDevice* d) { return guarded([&]() -> RxClient* { check_device(d); return d->client; }, nullptr); }
+RX_EXPORT int64_t PjRtDeviceGetLocalDeviceId(RxDevice* d) { return guarded([&]() -> int64_t { check_device(d); return d->index; }, -1); }
+RX_EXPORT int64_t PjRtDeviceGetGlobalDeviceId(RxDevice* d) { return PjRtDeviceGetLocalDeviceId(d); }
+RX_EXPORT int64_t PjRtDeviceGetLocalHardwareId(RxDevice* d) { return guarded([&]() -> int64_t { check_device(d); return d->ordinal; }, -1); }
+RX_EXPORT bool pjrt_device_is_addressable(RxDevice* d) { return guarded([&] { check_device(d); return true; }, false); }
+RX_EXPORT void PjRtDeviceGetAllocatorStats(RxDevice* d, JLAllocatorStats* s) {
+  guarded_void([&] {
+    check_device(d);
+    std::lock_guard<std::mutex> l(d->mu);
+    const int64_t none = INT64_MIN;
+    s->num_allocs = d->num_allocs;
+    s->bytes_in_use = d->bytes_in_use;
+    s->peak_bytes_in_use = d->peak_bytes_in_use;
+    s->largest_alloc_size = d->largest_alloc;
+    s->bytes_limit = d->bytes_limit;
+    s->bytes_reserved = 0;
+    s->peak_bytes_reserved = 0;
+    s->bytes_reservable_limit = none;
+    s->largest_free_block_bytes = d->free_blocks.empty() ? 0 : (int64_t)d->free_blocks.rbegin()->first;
+    s->pool_bytes = d->pool_bytes;
+    s->peak_pool_bytes = d->peak_pool_bytes;
+  });
+}
+
+RX_EXPORT RxBuffer* ArrayFromHostBuffer(RxClient* c, void* data, uint64_t ptype, size_t dim, const int64_t* cshape, RxDevice* d) {
+  return guarded([&]() -> RxBuffer* {
+    check_client(c);
+    check_device(d);
+    rx::TType ty;
+    ty.dt = rx::dt_from_code((int)ptype);
+    if (ty.dt == rx::DT::INVALID) throw Error("UNIMPLEMENTED: primitive type code " + std::to_string(ptype) + " is not supported");
+    for (size_t k = 0; k < dim; ++k) {
+      if (cshape[k] < 0) throw Error("INVALID_ARGUMENT: negative dimension");
+      ty.dims.push_back(cshape[k]);
+    }
+    const size_t bytes = (size_t)ty.bytes();
+    if (bytes && !data) throw Error("INVALID_ARGUMENT: null host pointer");
+    Mem m = std::make_shared<Allocation>(d, std::max<size_t>(bytes, 1));
+    if (bytes) {
+      HIP_CHECK(hipSetDevice(d->ordinal));
+      HIP_CHECK(hipMemcpyAsync(m->ptr, data, bytes, hipMemcpyHostToDevice, d->stream));
+      HIP_CHECK(hipStreamSynchronize(d->stream));  // host memory is only borrowed during the call
+    }
+    return new_buffer(c, d, ty, m);
+  }, nullptr);
+}
+
+RX_EXPORT RxBuffer* UninitPJRTBuffer(RxClient* c, RxDevice* d, uint64_t ptype, uint64_t shapeLen, uint64_t* shape) {
+  return guarded([&]() -> RxBuffer* {
+    check_client(c);
+    check_device(d);
+    rx::TType ty;
+    ty.dt = rx::dt_from_code((int)ptype);
+    if (ty.dt == rx::DT::INVALID) throw Error("UNIMPLEMENTED: primitive type code " + std::to_string(ptype) + " is not supported");
+    for (uint64_t k = 0; k < shapeLen; ++k) ty.dims.push_back((int64_t)shape[k]);
+    Mem m = std::make_shared<Allocation>(d, std::max<size_t>((size_t)ty.bytes(), 1));
+    return new_buffer(c, d, ty, m);
+  }, nullptr);
+}
+
+static void live_mem(RxBuffer* b) {
+  check_buffer(b);
+  if (b->donated || !b->mem) throw Error("INVALID_ARGUMENT: buffer was donated to an execution and can no longer be read");
+}
+
+RX_EXPORT void BufferToHost(RxBuffer* b, void* data) {
+  guarded_void([&] {
+    live_mem(b);
+    const size_t bytes = (size_t)b->ty.bytes();
+    if (!bytes) return;
+    HIP_CHECK(hipSetDevice(b->device->ordinal));
+    HIP_CHECK(hipMemcpyAsync(data, b->mem->ptr, bytes, hipMemcpyDeviceToHost, b->device->stream));
+    HIP_CHECK(hipStreamSynchronize(b->device->stream));
+  });
+}
+
+RX_EXPORT void CopyToBuffer(RxClient* c, RxBuffer* b, void* data, size_t offset, size_t size, RxBuffer** bufferP) {
+  (void)bufferP;
+  guarded_void([&] {
+    check_client(c);
+    live_mem(b);
+    if (offset + size > (size_t)b->ty.bytes()) throw Error("INVALID_ARGUMENT: copy range exceeds the buffer");
+    HIP_CHECK(hipSetDevice(b->device->ordinal));
+    HIP_CHECK(hipMemcpyAsync((char*)b->mem->ptr + offset, data, size, hipMemcpyHostToDevice, b->device->stream));
+    HIP_CHECK(hipStreamSynchronize(b->device->stream));
+  });
+}
+
+RX_EXPORT void CopyFromBuffer(RxClient* c, RxBuffer* b, void* data, size_t offset, size_t size, RxBuffer** bufferP) {
+  (void)bufferP;
+  guarded_void([&] {
+    check_client(c);
+    live_mem(b);
+    if (offset + size > (size_t)b->ty.bytes()) throw Error("INVALID_ARGUMENT: copy range exceeds the buffer");
+    HIP_CHECK(hipSetDevice(b->device->ordinal));
+    HIP_CHECK(hipMemcpyAsync(data, (char*)b->mem->ptr + offset, size, hipMemcpyDeviceToHost, b->device->stream));
+    HIP_CHECK(hipStreamSynchronize(b->device->stream));
+  });
+}
+
+RX_EXPORT const int64_t* BufferShape(RxBuffer* b) { return guarded([&]() -> const int64_t* { check_buffer(b); return b->ty.dims.data(); }, nullptr); }
+RX_EXPORT int64_t BufferNDimensions(RxBuffer* b) { return guarded([&]() -> int64_t { check_buffer(b); return (int64_t)b->ty.dims.size(); }, 0); }
+RX_EXPORT int BufferPrimitiveType(RxBuffer* b) { return guarded([&] { check_buffer(b); return rx::info(b->ty.dt).code; }, 0); }
+RX_EXPORT RxDevice* BufferToDevice(RxBuffer* b) { return guarded([&]() -> RxDevice* { check_buffer(b); return b->device; }, nullptr); }
+RX_EXPORT RxClient* BufferToClient(RxBuffer* b) { return guarded([&]() -> RxClient* { check_buffer(b); return b->client; }, nullptr); }
+RX_EXPORT uint8_t BufferOnCPU(RxBuffer* b) { return guarded([&]() -> uint8_t { check_buffer(b); return 0; }, 0); }
+RX_EXPORT void* UnsafeBufferPointer(RxBuffer* b) { return guarded([&]() -> void* { live_mem(b); return b->mem->ptr; }, nullptr); }
+RX_EXPORT RxBuffer* CopyBufferToDevice(RxBuffer* b, RxDevice* dst) {
+  return guarded([&]() -> RxBuffer* {
+    live_mem(b);
+    check_device(dst);
+    const size_t bytes = (size_t)b->ty.bytes();
+    Mem m = std::make_shared<Allocation>(dst, std::max<size_t>(bytes, 1));
+    if (bytes) {
+      HIP_CHECK(hipSetDevice(dst->ordinal));
+      HIP_CHECK(hipMemcpyAsync(m->ptr, b->mem->ptr, bytes, hipMemcpyDeviceToDevice, dst->stream));
+      if (dst != b->device) HIP_CHECK(hipStreamSynchronize(dst->stream));
+    }
+    return new_buffer(dst->client, dst, b->ty, m);
+  }, nullptr);
+}
+RX_EXPORT void PjRtBufferFree(RxBuffer* b) {
+  // called from finalizers: tolerate null and handles that are already gone
+  if (!b || !reg_has(b)) return;
+  reg_del(b);
+  delete b;
+}
+
+RX_EXPORT int RxCompileOffline(const char* text, size_t len, int with_source, char** report) {
+  try {
+    rx::Graph g = rx::parse_module(text, len);
+    rx::Plan p = rx::make_plan(g, plan_options());
+    std::string code = rtc_compile(p.source, "gfx950");
+    if (report) {
+      std::string r = p.report() + "code object: " + std::to_string(code.size()) + " bytes\n";
+      if (with_source) r += "----- source -----\n" + p.source;
+      *report = dup_cstr(r);
+    }
+    return 0;
+  } catch (const std::exception& e) {
+    g_last_error = e.what();
+    if (report) *report = dup_cstr(e.what());
+    return 1;
+  }
+}
+
+RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, size_t len, const char* opts, size_t nopts) {
+  (void)opts;
+  (void)nopts;
+  return guarded([&]() -> RxExecutable* {
+    check_client(c);
+    if (!text) throw Error("INVALID_ARGUMENT: null module text");
+    RxDevice* d = c->devices[0].get();
+    std::unique_ptr<RxExecutable> ex(new RxExecutable);
+    ex->client = c;
+    ex->device = d;
+    try {
+      rx::Graph g = rx::parse_module(text, len);
+      ex->plan = rx::make_plan(g, plan_options());
+    } catch (const std::exception& e) {
+      // same shape of message as the reference: module text followed by the status (API.cpp:1499-1505)
+      std::string mod(text, std::min<size_t>(len, 4000));
+      throw Error(mod + "\n" + e.what());
+    }
+    ex->report = ex->plan.report();
+    HIP_CHECK(hipSetDevice(d->ordinal));
+    if (!ex->plan.launches.empty()) {
+      std::string code = rtc_compile(ex->plan.source, d->arch);
+      HIP_CHECK(hipModuleLoadData(&ex->module, code.data()));
+      for (auto& L : ex->plan.launches) {
+        hipFunction_t f;
+        HIP_CHECK(hipModuleGetFunction(&f, ex->module, L.kernel.c_str()));
+        ex->fns.push_back(f);
+      }
+    }
+    ex->consts.resize(ex->plan.buffers.size());
+    for (size_t b = 0; b < ex->plan.buffers.size(); ++b) {
+      auto& B = ex->plan.buffers[b];
+      if (B.kind != rx::BufferDesc::Const) continue;
+      ex->consts[b] = std::make_shared<Allocation>(d, std::max<size_t>(B.data.size(), 1));
+      if (!B.data.empty()) HIP_CHECK(hipMemcpy(ex->consts[b]->ptr, B.data.data(), B.data.size(), hipMemcpyHostToDevice));
+    }
+    RxExecutable* raw = ex.release();
+    reg_add(raw);
+    return raw;
+  }, nullptr);
+}
+
+RX_EXPORT void ExecutableFree(RxExecutable* ex) {
+  if (!ex || !reg_has(ex)) return;
+  reg_del(ex);
+  if (ex->module) {
+    (void)hipSetDevice(ex->device->ordinal);
+    (void)hipStreamSynchronize(ex->device->stream);
+    (void)hipModuleUnload(ex->module);
+  }
+  delete ex;
+}
+RX_EXPORT RxClient* PjRtLoadedExecutableGetClient(RxExecutable* ex) { return guarded([&]() -> RxClient* { check_exec(ex); return ex->client; }, nullptr); }
+RX_EXPORT void PjRtLoadedExecutableGetHloModules(RxExecutable* ex, void** mods, int32_t* n) {
+  (void)mods;
+  guarded_void([&] { check_exec(ex); if (n) *n = 0; });
+}
+RX_EXPORT const char* RxExecutableReport(RxExecutable* ex) { return guarded([&]() -> const char* { check_exec(ex); return ex->report.c_str(); }, ""); }
+RX_EXPORT int RxExecutableNumLaunches(RxExecutable* ex) { return guarded([&] { check_exec(ex); return (int)ex->plan.launches.size(); }, 0); }
+RX_EXPORT int RxExecutableNumResults(RxExecutable* ex) { return guarded([&] { check_exec(ex); return (int)ex->plan.result_types.size(); }, 0); }
+RX_EXPORT void RxExecutableLaunchInfo(RxExecutable* ex, int i, const char** kernel, const char** kind, double* bytes, double* flops) {
+  guarded_void([&] {
+    check_exec(ex);
+    if (i < 0 || i >= (int)ex->plan.launches.size()) throw Error("INVALID_ARGUMENT: launch index out of range");
+    auto& L = ex->plan.launches[i];
+    if (kernel) *kernel = L.kernel.c_str();
+    if (kind) *kind = L.kind.c_str();
+    if (bytes) *bytes = L.algo_bytes;
+    if (flops) *flops = L.flops;
+  });
+}
+
+RX_EXPORT void XLAExecuteSharded(RxExecutable* ex, int num_args, RxBuffer** op_args, RxDevice* device, uint8_t* is_arg_donatable, int num_results,
+                                 RxBuffer** op_results, uint8_t* futures, RxFuture** future_results) {
+  guarded_void([&] {
+    if (futures) *futures = future_results ? 1 : 0;
+    execute(ex, num_args, op_args, device, is_arg_donatable, num_results, op_results, nullptr, future_results);
+  });
+}
+RX_EXPORT void RxExecuteTimed(RxExecutable* ex, int num_args, RxBuffer** op_args, RxDevice* device, uint8_t* is_arg_donatable, int num_results,
+                              RxBuffer** op_results, float* launch_ms) {
+  guarded_void([&] { execute(ex, num_args, op_args, device, is_arg_donatable, num_results, op_results, launch_ms, nullptr); });
+}
+
+RX_EXPORT void FreeFuture(RxFuture* f) {
+  if (!f || !reg_has(f)) return;
+  reg_del(f);
+  if (f->ev) (void)hipEventDestroy(f->ev);
+  delete f;
+}
+RX_EXPORT uint8_t FutureIsReady(RxFuture* f) {
+  return guarded([&]() -> uint8_t {
+    if (!f || !reg_has(f)) throw Error("INVALID_ARGUMENT: null or foreign future handle");
+    hipError_t e = hipEventQuery(f->ev);
+    if (e == hipSuccess) return 1;
+    if (e == hipErrorNotReady) { (void)hipGetLastError(); return 0; }
+    throw Error(std::string("execution failed: ") + hipGetErrorString(e));
+  }, 0);
+}
+RX_EXPORT void FutureAwait(RxFuture* f) {
+  guarded_void([&] {
+    if (!f || !reg_has(f)) throw Error("INVALID_ARGUMENT: null or foreign future handle");
+    hipError_t e = hipEventSynchronize(f->ev);
+    if (e != hipSuccess) throw Error(std::string("execution failed: ") + hipGetErrorString(e));
+  });
+}
+RX_EXPORT void RxDeviceSynchronize(RxDevice* d) {
+  guarded_void([&] { check_device(d); HIP_CHECK(hipSetDevice(d->ordinal)); HIP_CHECK(hipStreamSynchronize(d->stream)); });
+}
+
+RX_EXPORT float RxCalibrationCopy(RxDevice* d, size_t bytes, int iters) {
+  return guarded([&]() -> float {
+    check_device(d);
+    if (iters < 1) iters = 1;
+    bytes &= ~(size_t)15;
+    if (!bytes) throw Error("INVALID_ARGUMENT: copy size must be at least 16 bytes");
+    HIP_CHECK(hipSetDevice(d->ordinal));
+    Allocation src(d, bytes), dst(d, bytes);
+    HIP_CHECK(hipMemsetAsync(src.ptr, 1, bytes, d->stream));
+    const size_t n16 = bytes / 16;
+    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, 256 * 32);
+    hipEvent_t a, b;
+    HIP_CHECK(hipEventCreate(&a));
+    HIP_CHECK(hipEventCreate(&b));
+    hipLaunchKernelGGL(rx_copy16, dim3(grid), dim3(256), 0, d->stream, (const uint4*)src.ptr, (uint4*)dst.ptr, n16);  // warm-up
+    HIP_CHECK(hipEventRecord(a, d->stream));
+    for (int i = 0; i < iters; ++i) hipLaunchKernelGGL(rx_copy16, dim3(grid), dim3(256), 0, d->stream, (const uint4*)src.ptr, (uint4*)dst.ptr, n16);
+    HIP_CHECK(hipEventRecord(b, d->stream));
+    HIP_CHECK(hipEventSynchronize(b));
+    float ms = 0;
+    HIP_CHECK(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    return ms / (float)iters;
+  }, -1.0f);
+}

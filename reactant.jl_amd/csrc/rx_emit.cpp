@@ -1,0 +1,518 @@
+#include "rx_emit.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+namespace rx {
+
+std::string Ix::str() const {
+  if (var.empty()) return std::to_string(off);
+  if (off == 0) return var;
+  if (off > 0) return "(" + var + " + " + std::to_string(off) + ")";
+  return "(" + var + " - " + std::to_string(-off) + ")";
+}
+
+static Ix const_ix(int64_t v) {
+  Ix i;
+  i.off = v;
+  i.lo = i.hi = v;
+  return i;
+}
+
+static Ix shifted(const Ix& a, int64_t d) {
+  Ix r = a;
+  r.off += d;
+  r.lo += d;
+  r.hi += d;
+  return r;
+}
+
+bool Emitter::lookup(const std::string& key, std::string* out) const {
+  for (auto it = scopes_.rbegin(); it != scopes_.rend(); ++it) {
+    auto f = it->find(key);
+    if (f != it->end()) {
+      *out = f->second;
+      return true;
+    }
+  }
+  return false;
+}
+
+int Emitter::slot_of(int node) {
+  for (size_t k = 0; k < inputs.size(); ++k)
+    if (inputs[k] == node) return (int)k;
+  inputs.push_back(node);
+  return (int)inputs.size() - 1;
+}
+
+std::string Emitter::linear(const Index& ix, const std::vector<int64_t>& dims) const {
+  int64_t stride = 1, c = 0;
+  std::vector<std::string> terms;
+  for (int d = (int)dims.size() - 1; d >= 0; --d) {
+    c += ix[d].off * stride;
+    if (!ix[d].var.empty() && dims[d] > 1) {
+      std::string v = idx64 ? "(long long)" + ix[d].var : ix[d].var;
+      terms.push_back(stride == 1 ? v : v + " * " + std::to_string(stride) + (idx64 ? "LL" : ""));
+    } else if (!ix[d].var.empty()) {
+      // dimension of size 1: index is 0 whatever the variable says (range-checked by the caller)
+      c -= ix[d].off * stride;
+    }
+    stride *= dims[d];
+  }
+  std::string s;
+  for (auto& t : terms) s += (s.empty() ? "" : " + ") + t;
+  if (s.empty()) return std::to_string(c) + (idx64 ? "LL" : "");
+  if (c > 0) s += " + " + std::to_string(c) + (idx64 ? "LL" : "");
+  if (c < 0) s += " - " + std::to_string(-c) + (idx64 ? "LL" : "");
+  return s;
+}
+
+std::string Emitter::load_conv(DT dt, const std::string& raw) const {
+  switch (dt) {
+    case DT::BF16: return "rx_bf16_to_f32(" + raw + ")";
+    case DT::F16: return "rx_f16_to_f32(" + raw + ")";
+    case DT::F8E4M3FN: return "rx_e4m3_to_f32(" + raw + ")";
+    case DT::F8E5M2: return "rx_e5m2_to_f32(" + raw + ")";
+    case DT::I1: return "(" + raw + " != 0)";
+    default: return raw;
+  }
+}
+
+std::string Emitter::store_conv(DT dt, const std::string& val) {
+  switch (dt) {
+    case DT::BF16: return "rx_f32_to_bf16(" + val + ")";
+    case DT::F16: return "rx_f32_to_f16(" + val + ")";
+    case DT::F8E4M3FN: return "rx_f32_to_e4m3(" + val + ")";
+    case DT::F8E5M2: return "rx_f32_to_e5m2(" + val + ")";
+    case DT::I1: return "(rx_u8)((" + val + ") ? 1 : 0)";
+    default: return val;
+  }
+}
+
+std::string Emitter::round_narrow(DT dt, const std::string& e) {
+  switch (dt) {
+    case DT::BF16: return "rx_round_bf16(" + e + ")";
+    case DT::F16: return "rx_round_f16(" + e + ")";
+    case DT::F8E4M3FN: return "rx_round_e4m3(" + e + ")";
+    case DT::F8E5M2: return "rx_round_e5m2(" + e + ")";
+    default: return e;
+  }
+}
+
+static std::string float_lit(double v, bool dbl) {
+  if (std::isnan(v)) return dbl ? "__builtin_nan(\"\")" : "__builtin_nanf(\"\")";
+  if (std::isinf(v)) return std::string(v < 0 ? "(-" : "(") + (dbl ? "__builtin_inf()" : "__builtin_inff()") + ")";
+  char buf[64];
+  snprintf(buf, sizeof buf, "%a", v);
+  std::string s = buf;
+  if (!dbl) s += "f";
+  return "(" + s + ")";
+}
+
+std::string Emitter::literal(const Node& n) {
+  DT dt = n.ty.dt;
+  if (is_float(dt)) return float_lit(splat_as_double(n), dt == DT::F64);
+  if (dt == DT::I1) return splat_as_int(n) ? "true" : "false";
+  int64_t v = splat_as_int(n);
+  if (dt == DT::U64) return "(rx_u64)" + std::to_string((uint64_t)v) + "ULL";
+  if (dt == DT::I64) {
+    if (v == INT64_MIN) return "(rx_i64)(-9223372036854775807LL - 1)";
+    return "(rx_i64)" + std::to_string(v) + "LL";
+  }
+  return std::string("(") + info(dt).ctype + ")" + "(" + std::to_string(v) + ")";
+}
+
+Ix Emitter::temp_index(const std::string& expr, int64_t lo, int64_t hi) {
+  Ix r;
+  r.var = fresh("t");
+  r.lo = lo;
+  r.hi = hi;
+  line("const " + idx_t() + " " + r.var + " = " + expr + ";");
+  return r;
+}
+
+std::string Emitter::emit(int node, const Index& ix) {
+  auto b = bound.find(node);
+  if (b != bound.end()) return b->second;
+  const Node& n = g_.nodes[node];
+  if ((int)ix.size() != n.ty.rank()) throw Error("internal: index rank mismatch at node " + std::to_string(node));
+  std::string key = std::to_string(node) + ":";
+  for (auto& i : ix) key += i.key() + ",";
+  std::string r;
+  if (lookup(key, &r)) return r;
+  if (is_input_(node)) r = emit_load(node, ix);
+  else r = emit_op(n, ix);
+  scopes_.back()[key] = r;
+  return r;
+}
+
+std::string Emitter::emit_load(int node, const Index& ix) {
+  const Node& n = g_.nodes[node];
+  const auto& dims = n.ty.dims;
+  for (size_t d = 0; d < dims.size(); ++d) {
+    if (dims[d] == 1) continue;
+    if (ix[d].lo < 0 || ix[d].hi > dims[d] - 1)
+      throw Error("internal: index range check failed reading node " + std::to_string(node) + " dim " + std::to_string(d) +
+                  " range [" + std::to_string(ix[d].lo) + "," + std::to_string(ix[d].hi) + "] size " + std::to_string(dims[d]));
+  }
+  int slot = slot_of(node);
+  LoadRecord rec;
+  rec.node = node;
+  if (dims.size() == root_vars_.size() && !dims.empty()) {
+    rec.affine = true;
+    for (size_t d = 0; d < dims.size(); ++d) {
+      if (ix[d].var != root_vars_[d]) { rec.affine = false; break; }
+      rec.off.push_back(ix[d].off);
+    }
+  }
+  loads.push_back(rec);
+  bool direct = allow_direct_ && rec.affine && dims == root_dims_;
+  if (direct)
+    for (auto o : rec.off) direct = direct && o == 0;
+  std::string raw;
+  if (direct) {
+    direct_inputs.insert(slot);
+    raw = direct_expr(slot);
+  } else {
+    raw = "in" + std::to_string(slot) + "[" + (dims.empty() ? std::string("0") : linear(ix, dims)) + "]";
+  }
+  std::string v = fresh();
+  line(std::string("const ") + info(n.ty.dt).ctype + " " + v + " = " + load_conv(n.ty.dt, raw) + ";");
+  return v;
+}
+
+static std::string fn(const std::string& base, bool dbl) { return dbl ? base : base + "f"; }
+
+std::string Emitter::emit_op(const Node& n, const Index& ix) {
+  const DT dt = n.ty.dt;
+  const std::string CT = info(dt).ctype;
+  const bool dbl = dt == DT::F64;
+  auto def = [&](const std::string& expr) {
+    std::string v = fresh();
+    line("const " + CT + " " + v + " = " + (is_narrow_float(dt) ? round_narrow(dt, expr) : expr) + ";");
+    return v;
+  };
+  // index of a rank-0 or same-shape operand
+  auto opnd = [&](int k) {
+    const Node& o = g_.nodes[n.in[k]];
+    if (o.ty.rank() == 0 && n.ty.rank() != 0) return emit(n.in[k], Index{});
+    return emit(n.in[k], ix);
+  };
+  switch (n.k) {
+    case OpK::Param:
+      throw Error("internal: parameter reached the emitter without a buffer");
+    case OpK::Constant:
+      if (!n.splat) throw Error("internal: dense constant must be materialized");
+      return literal(n);
+    case OpK::Iota: {
+      std::string e = "(" + CT + ")" + ix[n.a0[0]].str();
+      return is_narrow_float(dt) ? def(e) : e;
+    }
+    case OpK::Unary: {
+      const DT sdt = g_.nodes[n.in[0]].ty.dt;
+      std::string x = opnd(0);
+      const std::string& op = n.op;
+      if (op == "is_finite") return def("isfinite(" + x + ")");
+      if (is_float(dt)) {
+        if (op == "sine") return def(fn("sin", dbl) + "(" + x + ")");
+        if (op == "cosine") return def(fn("cos", dbl) + "(" + x + ")");
+        if (op == "tan") return def(fn("tan", dbl) + "(" + x + ")");
+        if (op == "tanh") return def(fn("tanh", dbl) + "(" + x + ")");
+        if (op == "exponential") return def(fn("exp", dbl) + "(" + x + ")");
+        if (op == "exponential_minus_one") return def(fn("expm1", dbl) + "(" + x + ")");
+        if (op == "log") return def(fn("log", dbl) + "(" + x + ")");
+        if (op == "log_plus_one") return def(fn("log1p", dbl) + "(" + x + ")");
+        if (op == "sqrt") return def(fn("sqrt", dbl) + "(" + x + ")");
+        if (op == "cbrt") return def(fn("cbrt", dbl) + "(" + x + ")");
+        if (op == "rsqrt") return def("rx_rsqrt(" + x + ")");
+        if (op == "abs") return def(fn("fabs", dbl) + "(" + x + ")");
+        if (op == "negate") return def("(-" + x + ")");
+        if (op == "logistic") return def("rx_logistic(" + x + ")");
+        if (op == "floor") return def(fn("floor", dbl) + "(" + x + ")");
+        if (op == "ceil") return def(fn("ceil", dbl) + "(" + x + ")");
+        if (op == "sign") return def("rx_sign(" + x + ")");
+        if (op == "round_nearest_even") return def(fn("rint", dbl) + "(" + x + ")");
+        if (op == "round_nearest_afz") return def(fn("round", dbl) + "(" + x + ")");
+        if (op == "erf") return def(fn("erf", dbl) + "(" + x + ")");
+      } else if (dt == DT::I1) {
+        if (op == "not") return def("(!" + x + ")");
+        if (op == "abs" || op == "negate" || op == "sign") return x;
+      } else {
+        if (op == "not") return def("(" + CT + ")(~" + x + ")");
+        if (op == "negate") return def("(" + CT + ")(0 - " + x + ")");
+        if (op == "abs") return info(dt).is_signed ? def("(" + CT + ")(" + x + " < 0 ? 0 - " + x + " : " + x + ")") : x;
+        if (op == "sign") return def("(" + CT + ")((" + x + " > 0) - (" + x + " < 0))");
+      }
+      (void)sdt;
+      throw Error("unsupported unary op '" + op + "' on " + info(dt).mlir);
+    }
+    case OpK::Gelu: {
+      std::string x = opnd(0);
+      if (!is_float(dt)) throw Error("gelu on a non-float type");
+      std::string f = n.op == "TANH" ? "rx_gelu_tanh" : (n.op == "SIGMOID" ? "rx_gelu_sigmoid" : "rx_gelu_erf");
+      return def(f + "(" + x + ")");
+    }
+    case OpK::Binary: {
+      std::string a = opnd(0), b = opnd(1);
+      const std::string& op = n.op;
+      if (is_float(dt)) {
+        if (op == "add") return def("(" + a + " + " + b + ")");
+        if (op == "subtract") return def("(" + a + " - " + b + ")");
+        if (op == "multiply") return def("(" + a + " * " + b + ")");
+        if (op == "divide") return def("(" + a + " / " + b + ")");
+        if (op == "maximum") return def("rx_max(" + a + ", " + b + ")");
+        if (op == "minimum") return def("rx_min(" + a + ", " + b + ")");
+        if (op == "power") return def(fn("pow", dbl) + "(" + a + ", " + b + ")");
+        if (op == "remainder") return def(fn("fmod", dbl) + "(" + a + ", " + b + ")");
+        if (op == "atan2") return def(fn("atan2", dbl) + "(" + a + ", " + b + ")");
+      } else if (dt == DT::I1) {
+        if (op == "add" || op == "or" || op == "maximum") return def("(" + a + " || " + b + ")");
+        if (op == "multiply" || op == "and" || op == "minimum") return def("(" + a + " && " + b + ")");
+        if (op == "xor" || op == "subtract") return def("(" + a + " != " + b + ")");
+      } else {
+        auto c = [&](const std::string& e) { return def("(" + CT + ")(" + e + ")"); };
+        if (op == "add") return c(a + " + " + b);
+        if (op == "subtract") return c(a + " - " + b);
+        if (op == "multiply") return c(a + " * " + b);
+        if (op == "divide") return def("rx_idiv<" + CT + ">(" + a + ", " + b + ")");
+        if (op == "remainder") return def("rx_irem<" + CT + ">(" + a + ", " + b + ")");
+        if (op == "maximum") return c(a + " > " + b + " ? " + a + " : " + b);
+        if (op == "minimum") return c(a + " < " + b + " ? " + a + " : " + b);
+        if (op == "and") return c(a + " & " + b);
+        if (op == "or") return c(a + " | " + b);
+        if (op == "xor") return c(a + " ^ " + b);
+        if (op == "power") return def("rx_ipow<" + CT + ">(" + a + ", " + b + ")");
+        const int bits = info(dt).size * 8;
+        const std::string oob = "((rx_u64)" + b + " >= " + std::to_string(bits) + ")";
+        if (op == "shift_left") return c(oob + " ? 0 : (" + a + " << " + b + ")");
+        if (op == "shift_right_logical") {
+          std::string U = std::string("rx_u") + std::to_string(bits);
+          return c(oob + " ? 0 : (" + CT + ")((" + U + ")" + a + " >> " + b + ")");
+        }
+        if (op == "shift_right_arithmetic") return c(oob + " ? (" + a + " < 0 ? -1 : 0) : (" + a + " >> " + b + ")");
+      }
+      throw Error("unsupported binary op '" + op + "' on " + info(dt).mlir);
+    }
+    case OpK::Compare: {
+      std::string a = opnd(0), b = opnd(1);
+      const char* o = n.op == "EQ" ? "==" : n.op == "NE" ? "!=" : n.op == "LT" ? "<" : n.op == "LE" ? "<=" : n.op == "GT" ? ">" : n.op == "GE" ? ">=" : nullptr;
+      if (!o) throw Error("unknown comparison direction " + n.op);
+      return def("(" + a + " " + o + " " + b + ")");
+    }
+    case OpK::Select: {
+      std::string p = opnd(0), a = opnd(1), b = opnd(2);
+      return def("(" + p + " ? " + a + " : " + b + ")");
+    }
+    case OpK::Clamp: {
+      std::string lo = opnd(0), x = opnd(1), hi = opnd(2);
+      if (is_float(dt)) return def("rx_min(rx_max(" + x + ", " + lo + "), " + hi + ")");
+      return def("(" + CT + ")((" + x + " < " + lo + " ? " + lo + " : " + x + ") > " + hi + " ? " + hi + " : (" + x + " < " + lo + " ? " + lo + " : " + x + "))");
+    }
+    case OpK::Convert: {
+      const DT sdt = g_.nodes[n.in[0]].ty.dt;
+      std::string x = opnd(0);
+      if (sdt == dt) return x;
+      if (dt == DT::I1) return def("(" + x + " != 0)");
+      if (is_narrow_float(sdt) && is_narrow_float(dt)) return def(x);
+      if (is_narrow_float(sdt) && dt == DT::F32) return x;
+      return def("(" + CT + ")" + x);
+    }
+    case OpK::BroadcastInDim: {
+      const Node& o = g_.nodes[n.in[0]];
+      Index oi(o.ty.rank());
+      for (int k = 0; k < o.ty.rank(); ++k) {
+        if (o.ty.dims[k] == 1 && n.ty.dims[n.a0[k]] != 1) oi[k] = const_ix(0);
+        else oi[k] = ix[n.a0[k]];
+      }
+      return emit(n.in[0], oi);
+    }
+    case OpK::Transpose: {
+      Index oi(ix.size());
+      for (size_t i = 0; i < ix.size(); ++i) oi[n.a0[i]] = ix[i];
+      return emit(n.in[0], oi);
+    }
+    case OpK::Reshape: {
+      const Node& o = g_.nodes[n.in[0]];
+      // fast path: shapes equal after dropping unit dims
+      std::vector<int> rn, ro;
+      for (int k = 0; k < n.ty.rank(); ++k) if (n.ty.dims[k] != 1) rn.push_back(k);
+      for (int k = 0; k < o.ty.rank(); ++k) if (o.ty.dims[k] != 1) ro.push_back(k);
+      bool same = rn.size() == ro.size();
+      for (size_t k = 0; same && k < rn.size(); ++k) same = n.ty.dims[rn[k]] == o.ty.dims[ro[k]];
+      Index oi(o.ty.rank(), const_ix(0));
+      if (same) {
+        for (size_t k = 0; k < rn.size(); ++k) oi[ro[k]] = ix[rn[k]];
+        return emit(n.in[0], oi);
+      }
+      Ix lin = temp_index(linear(ix, n.ty.dims), 0, n.ty.numel() - 1);
+      int64_t stride = o.ty.numel();
+      for (int k = 0; k < o.ty.rank(); ++k) {
+        stride /= std::max<int64_t>(o.ty.dims[k], 1);
+        if (o.ty.dims[k] == 1) continue;
+        std::string e = lin.var;
+        if (stride > 1) e = "(" + e + " / " + std::to_string(stride) + ")";
+        if (k > 0) e = e + " % " + std::to_string(o.ty.dims[k]);
+        oi[k] = temp_index(e, 0, o.ty.dims[k] - 1);
+      }
+      return emit(n.in[0], oi);
+    }
+    case OpK::Slice: {
+      Index oi(ix.size());
+      for (size_t d = 0; d < ix.size(); ++d) {
+        if (n.a2[d] == 1) oi[d] = shifted(ix[d], n.a0[d]);
+        else if (ix[d].is_const()) oi[d] = const_ix(ix[d].off * n.a2[d] + n.a0[d]);
+        else oi[d] = temp_index(ix[d].str() + " * " + std::to_string(n.a2[d]) + " + " + std::to_string(n.a0[d]),
+                                ix[d].lo * n.a2[d] + n.a0[d], ix[d].hi * n.a2[d] + n.a0[d]);
+      }
+      return emit(n.in[0], oi);
+    }
+    case OpK::DynamicSlice: {
+      const Node& o = g_.nodes[n.in[0]];
+      Index oi(ix.size());
+      for (size_t d = 0; d < ix.size(); ++d) {
+        const Node& s = g_.nodes[n.in[1 + d]];
+        if (s.k != OpK::Constant) throw Error("dynamic_slice with non-constant start indices is not supported");
+        int64_t st = std::min(std::max<int64_t>(splat_as_int(s), 0), o.ty.dims[d] - n.a0[d]);
+        oi[d] = shifted(ix[d], st);
+      }
+      return emit(n.in[0], oi);
+    }
+    case OpK::Pad: {
+      const Node& o = g_.nodes[n.in[0]];
+      std::string pv = emit(n.in[1], Index{});
+      Index oi(ix.size());
+      std::vector<std::string> conds;
+      std::vector<std::string> pre;
+      bool never = false;
+      for (size_t d = 0; d < ix.size(); ++d) {
+        const int64_t low = n.a0[d], q = n.a2[d] + 1, sd = o.ty.dims[d];
+        Ix p = shifted(ix[d], -low);
+        if (q == 1) {
+          if (p.lo < 0) conds.push_back(p.str() + " >= 0");
+          if (p.hi > sd - 1) conds.push_back(p.str() + " < " + std::to_string(sd));
+          p.lo = std::max<int64_t>(p.lo, 0);
+          p.hi = std::min<int64_t>(p.hi, sd - 1);
+          if (p.lo > p.hi) never = true;
+          oi[d] = p;
+        } else {
+          if (p.lo < 0) conds.push_back(p.str() + " >= 0");
+          conds.push_back(p.str() + " % " + std::to_string(q) + " == 0");
+          if (p.hi / q > sd - 1) conds.push_back(p.str() + " / " + std::to_string(q) + " < " + std::to_string(sd));
+          Ix t;
+          t.var = fresh("t");
+          t.lo = std::max<int64_t>(0, p.lo / q);
+          t.hi = std::min<int64_t>(sd - 1, std::max<int64_t>(p.hi, 0) / q);
+          pre.push_back("const " + idx_t() + " " + t.var + " = " + p.str() + " / " + std::to_string(q) + ";");
+          if (t.lo > t.hi) never = true;
+          oi[d] = t;
+        }
+      }
+      if (never || o.ty.numel() == 0) return pv;
+      if (conds.empty() && pre.empty()) return emit(n.in[0], oi);
+      std::string v = fresh();
+      line(CT + " " + v + " = " + pv + ";");
+      std::string cond;
+      for (auto& c : conds) cond += (cond.empty() ? "" : " && ") + c;
+      line("if (" + (cond.empty() ? std::string("true") : cond) + ") {");
+      indent += 2;
+      push_scope();
+      for (auto& p : pre) line(p);
+      std::string inner = emit(n.in[0], oi);
+      line(v + " = " + inner + ";");
+      pop_scope();
+      indent -= 2;
+      line("}");
+      return v;
+    }
+    case OpK::DynamicUpdateSlice: {
+      const Node& o = g_.nodes[n.in[0]];
+      const Node& u = g_.nodes[n.in[1]];
+      Index ui(ix.size()), oi = ix;
+      std::vector<std::string> conds;
+      bool never = false;
+      for (size_t d = 0; d < ix.size(); ++d) {
+        const Node& s = g_.nodes[n.in[2 + d]];
+        if (s.k != OpK::Constant) throw Error("dynamic_update_slice with non-constant start indices is not supported");
+        int64_t st = std::min(std::max<int64_t>(splat_as_int(s), 0), o.ty.dims[d] - u.ty.dims[d]);
+        Ix p = shifted(ix[d], -st);
+        if (p.lo < 0) conds.push_back(p.str() + " >= 0");
+        if (p.hi > u.ty.dims[d] - 1) conds.push_back(p.str() + " < " + std::to_string(u.ty.dims[d]));
+        p.lo = std::max<int64_t>(p.lo, 0);
+        p.hi = std::min<int64_t>(p.hi, u.ty.dims[d] - 1);
+        if (p.lo > p.hi) never = true;
+        ui[d] = p;
+      }
+      if (never || u.ty.numel() == 0) return emit(n.in[0], oi);
+      if (conds.empty()) return emit(n.in[1], ui);
+      std::string v = fresh();
+      line(CT + " " + v + ";");
+      std::string cond;
+      for (auto& c : conds) cond += (cond.empty() ? "" : " && ") + c;
+      line("if (" + cond + ") {");
+      indent += 2;
+      push_scope();
+      std::string a = emit(n.in[1], ui);
+      line(v + " = " + a + ";");
+      pop_scope();
+      indent -= 2;
+      line("} else {");
+      indent += 2;
+      push_scope();
+      std::string b = emit(n.in[0], oi);
+      line(v + " = " + b + ";");
+      pop_scope();
+      indent -= 2;
+      line("}");
+      return v;
+    }
+    case OpK::Concatenate: {
+      const int d = (int)n.a0[0];
+      // static choice when the index range falls inside one operand
+      int64_t base = 0;
+      std::vector<int64_t> starts;
+      for (int id : n.in) { starts.push_back(base); base += g_.nodes[id].ty.dims[d]; }
+      for (size_t k = 0; k < n.in.size(); ++k) {
+        int64_t sz = g_.nodes[n.in[k]].ty.dims[d];
+        if (ix[d].lo >= starts[k] && ix[d].hi < starts[k] + sz) {
+          Index oi = ix;
+          oi[d] = shifted(ix[d], -starts[k]);
+          return emit(n.in[k], oi);
+        }
+      }
+      std::string v = fresh();
+      line(CT + " " + v + ";");
+      bool first = true;
+      for (size_t k = 0; k < n.in.size(); ++k) {
+        int64_t sz = g_.nodes[n.in[k]].ty.dims[d];
+        if (sz == 0) continue;
+        if (ix[d].hi < starts[k] || ix[d].lo >= starts[k] + sz) continue;
+        bool last = true;
+        for (size_t k2 = k + 1; k2 < n.in.size(); ++k2)
+          if (g_.nodes[n.in[k2]].ty.dims[d] > 0 && ix[d].hi >= starts[k2]) last = false;
+        std::string head = first ? "if (" : "} else if (";
+        if (last && !first) line("} else {");
+        else line(head + ix[d].str() + " < " + std::to_string(starts[k] + sz) + ") {");
+        first = false;
+        indent += 2;
+        push_scope();
+        Index oi = ix;
+        oi[d] = shifted(ix[d], -starts[k]);
+        oi[d].lo = std::max<int64_t>(oi[d].lo, 0);
+        oi[d].hi = std::min<int64_t>(oi[d].hi, sz - 1);
+        std::string a = emit(n.in[k], oi);
+        line(v + " = " + a + ";");
+        pop_scope();
+        indent -= 2;
+      }
+      line("}");
+      return v;
+    }
+    case OpK::Reduce:
+    case OpK::DotGeneral:
+      throw Error("internal: reduce/dot_general reached the emitter without a buffer or binding");
+  }
+  throw Error("internal: unhandled op kind");
+}
+
+}  // namespace rx

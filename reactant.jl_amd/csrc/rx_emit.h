@@ -1,0 +1,84 @@
+// Expression emitter: writes HIP text that evaluates a fused cone of StableHLO
+// nodes at one symbolic index.  Index-transforming ops (slice, pad, broadcast,
+// transpose, reshape, dynamic_update_slice, concatenate) become index arithmetic
+// on the producer side, so a stencil written as a slice/pad/add chain turns into
+// loads at constant offsets from the output index.
+#pragma once
+#include <functional>
+#include <map>
+#include <set>
+#include <sstream>
+
+#include "rx_ir.h"
+
+namespace rx {
+
+// One index component: value = var + off (var empty -> constant `off`), known to lie in [lo, hi].
+struct Ix {
+  std::string var;
+  int64_t off = 0;
+  int64_t lo = 0, hi = 0;
+  bool is_const() const { return var.empty(); }
+  std::string str() const;
+  std::string key() const { return var + "+" + std::to_string(off); }
+};
+using Index = std::vector<Ix>;
+
+struct LoadRecord {
+  int node;                     // materialized node that is read
+  std::vector<int64_t> off;     // constant offsets relative to the root index (valid if `affine`)
+  bool affine = false;          // index is root identity + constant offsets
+};
+
+class Emitter {
+ public:
+  Emitter(const Graph& g, std::function<bool(int)> is_input) : g_(g), is_input_(std::move(is_input)) {}
+
+  // kernel parameter order of inputs, filled as loads are emitted
+  std::vector<int> inputs;
+  std::map<int, std::string> bound;          // node id -> expression already in scope
+  std::vector<LoadRecord> loads;
+  bool idx64 = false;
+  int indent = 2;
+
+  // direct (vectorizable) loads: root dims + names of the root index variables
+  void set_root(const std::vector<int64_t>& dims, const std::vector<std::string>& vars, bool allow_direct) {
+    root_dims_ = dims;
+    root_vars_ = vars;
+    allow_direct_ = allow_direct;
+  }
+  std::set<int> direct_inputs;               // inputs that were read through the vector preload
+  // expression for lane `l` of the preloaded vector of input slot s
+  std::function<std::string(int slot)> direct_expr;
+
+  std::string emit(int node, const Index& ix);
+  std::string take_code() { std::string s = out_.str(); out_.str(""); return s; }
+  void line(const std::string& s) { out_ << std::string(indent, ' ') << s << "\n"; }
+  int slot_of(int node);
+  std::string load_conv(DT dt, const std::string& raw) const;          // storage -> compute
+  static std::string store_conv(DT dt, const std::string& val);        // compute -> storage
+  static std::string literal(const Node& n);
+  static std::string round_narrow(DT dt, const std::string& e);
+  std::string idx_t() const { return idx64 ? "long long" : "int"; }
+  std::string fresh(const char* p = "v") { return std::string(p) + std::to_string(tmp_++); }
+  void push_scope() { scopes_.emplace_back(); }
+  void pop_scope() { scopes_.pop_back(); }
+  std::string linear(const Index& ix, const std::vector<int64_t>& dims) const;
+
+ private:
+  const Graph& g_;
+  std::function<bool(int)> is_input_;
+  std::ostringstream out_;
+  std::vector<std::map<std::string, std::string>> scopes_{1};
+  int tmp_ = 0;
+  std::vector<int64_t> root_dims_;
+  std::vector<std::string> root_vars_;
+  bool allow_direct_ = false;
+
+  std::string emit_load(int node, const Index& ix);
+  std::string emit_op(const Node& n, const Index& ix);
+  bool lookup(const std::string& key, std::string* out) const;
+  Ix temp_index(const std::string& expr, int64_t lo, int64_t hi);
+};
+
+}  // namespace rx

@@ -1,0 +1,27 @@
+// Choice and instantiation of the MFMA GEMM skeletons (kernels/rx_gemm_kernels.h).
+#pragma once
+#include <string>
+
+#include "rx_ir.h"
+
+namespace rx {
+
+struct GemmChoice {
+  bool ok = false;
+  std::string kind;         // "gemm_f32" | "gemm_bf16" | "gemm_f16" | "gemm_f8"
+  std::string skeleton;     // template name in rx_gemm_kernels.h
+  std::string targs;        // template arguments before the epilogue type
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block = 256;
+  unsigned lds_bytes = 0;   // dynamic LDS (0: the skeleton declares static LDS)
+  std::string stype_a, stype_b;
+};
+
+// Returns ok=false when no skeleton covers the case (the caller then writes a scalar loop).
+GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_k_contig, bool b_k_contig);
+
+// Text of the `extern "C"` kernel <kbase>_gemm that runs the skeleton with epilogue type <kbase>_epi.
+// `epi_params` is the tail of the parameter list (epilogue operands and out0), `epi_ctor` builds `epi`.
+std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor);
+
+}  // namespace rx

@@ -1,0 +1,1242 @@
+// Fusion partitioner and kernel writer.
+//
+// Every live node is either MATERIALIZED (it owns a buffer: parameters, dense
+// constants, results, reduce and dot_general results, and producers whose
+// duplication into several consumers would be expensive) or FUSED into the
+// kernels of the materialized nodes that consume it.  Group classes:
+//   map      one elementwise/broadcast/slice/pad cone per output element
+//            (stencils are maps whose loads sit at constant offsets)
+//   reduce   cone -> full reduction: per-thread partials, wavefront DPP stage,
+//            LDS across the workgroup, then a second single-workgroup pass
+//   row      reductions over the minor dimension fused with the elementwise ops
+//            that consume them (softmax, RMSNorm): one workgroup or one
+//            wavefront per row, the row stays in registers between phases
+//   dot      dot_general with its elementwise epilogue (MFMA skeletons for
+//            f32/bf16/f16/f8, a scalar loop for everything else)
+#include "rx_plan.h"
+
+#include <algorithm>
+#include <cmath>
+#include <set>
+#include <sstream>
+
+#include "rx_emit.h"
+#include "rx_gemm.h"
+
+namespace rx {
+namespace {
+
+constexpr int kBlock = 256;
+
+using Ctx = std::pair<int, std::string>;
+
+bool is_index_op(OpK k) {
+  switch (k) {
+    case OpK::BroadcastInDim: case OpK::Reshape: case OpK::Transpose: case OpK::Slice: case OpK::Pad:
+    case OpK::DynamicUpdateSlice: case OpK::DynamicSlice: case OpK::Concatenate:
+      return true;
+    default:
+      return false;
+  }
+}
+
+bool is_arith(OpK k) {
+  switch (k) {
+    case OpK::Unary: case OpK::Binary: case OpK::Compare: case OpK::Select: case OpK::Clamp: case OpK::Gelu:
+      return true;
+    default:
+      return false;
+  }
+}
+
+const char* acc_ctype(DT dt) {
+  if (dt == DT::F64) return "double";
+  if (is_float(dt)) return "float";
+  return info(dt).ctype;
+}
+
+std::string red_identity(Red r, DT dt) {
+  const bool f = is_float(dt), d = dt == DT::F64;
+  switch (r) {
+    case Red::Add: case Red::Or: return dt == DT::I1 ? "false" : (f ? (d ? "0.0" : "0.0f") : "0");
+    case Red::Mul: case Red::And:
+      if (dt == DT::I1) return "true";
+      if (r == Red::And) return std::string("(") + info(dt).ctype + ")(~0ull)";
+      return f ? (d ? "1.0" : "1.0f") : "1";
+    case Red::Max:
+      if (f) return d ? "(-__builtin_inf())" : "(-__builtin_inff())";
+      if (dt == DT::I1) return "false";
+      if (!info(dt).is_signed) return "0";
+      switch (info(dt).size) { case 1: return "(rx_i8)(-128)"; case 2: return "(rx_i16)(-32768)"; case 4: return "(-2147483647 - 1)"; default: return "(-9223372036854775807LL - 1)"; }
+    case Red::Min:
+      if (f) return d ? "__builtin_inf()" : "__builtin_inff()";
+      if (dt == DT::I1) return "true";
+      if (!info(dt).is_signed) return std::string("(") + info(dt).ctype + ")(~0ull)";
+      switch (info(dt).size) { case 1: return "(rx_i8)127"; case 2: return "(rx_i16)32767"; case 4: return "2147483647"; default: return "9223372036854775807LL"; }
+  }
+  return "0";
+}
+
+const char* red_functor(Red r) {
+  switch (r) {
+    case Red::Add: return "rx_op_add()";
+    case Red::Mul: return "rx_op_mul()";
+    case Red::Max: return "rx_op_max()";
+    case Red::Min: return "rx_op_min()";
+    case Red::And: return "rx_op_and()";
+    case Red::Or: return "rx_op_or()";
+  }
+  return "rx_op_add()";
+}
+
+std::string red_apply(Red r, DT dt, const std::string& a, const std::string& b) {
+  if (dt == DT::I1) {
+    if (r == Red::Add || r == Red::Or || r == Red::Max) return "(" + a + " || " + b + ")";
+    return "(" + a + " && " + b + ")";
+  }
+  switch (r) {
+    case Red::Add: return "(" + a + " + " + b + ")";
+    case Red::Mul: return "(" + a + " * " + b + ")";
+    case Red::Max: return "rx_max(" + a + ", " + b + ")";
+    case Red::Min: return "rx_min(" + a + ", " + b + ")";
+    case Red::And: return "(" + a + " & " + b + ")";
+    case Red::Or: return "(" + a + " | " + b + ")";
+  }
+  return a;
+}
+
+struct Planner {
+  Graph g;  // canonicalized copy
+  PlanOptions opt;
+  Plan plan;
+  std::vector<char> live, mat;
+  std::vector<std::vector<int>> users;
+  std::vector<std::set<Ctx>> ctx;
+  std::vector<char> prev_mat;       // materialization decided by the previous analysis sweep (used for producers)
+  std::vector<char> force_mat;      // chosen cut points below a dot_general with several consumers
+  std::vector<int> buf_of;          // node -> buffer id (materialized nodes)
+  std::ostringstream src;
+  int kcount = 0;
+
+  Planner(const Graph& gin, const PlanOptions& o) : g(gin), opt(o) {}
+
+  // ------------------------------------------------------------------ rewrites
+  void canonicalize() {
+    const int N = (int)g.nodes.size();
+    std::vector<int> nuse(N, 0);
+    for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
+    for (int r : g.results) nuse[r]++;
+    for (auto& n : g.nodes) {
+      // dot_general(transpose(X), Y): read X directly
+      if (n.k == OpK::DotGeneral) {
+        for (int side = 0; side < 2; ++side) {
+          const Node& o = g.nodes[n.in[side]];
+          auto& batch = side == 0 ? n.a0 : n.a1;
+          auto& contr = side == 0 ? n.a2 : n.a3;
+          if (o.k == OpK::Transpose && o.ty.rank() == 2 && batch.empty() && contr.size() == 1) {
+            contr[0] = o.a0[contr[0]];
+            n.in[side] = o.in[0];
+          }
+        }
+        // operands widened from one narrow float type: contract the narrow data directly
+        const Node &a = g.nodes[n.in[0]], &b = g.nodes[n.in[1]];
+        if (a.k == OpK::Convert && b.k == OpK::Convert && n.ty.dt == DT::F32) {
+          DT sa = g.nodes[a.in[0]].ty.dt, sb = g.nodes[b.in[0]].ty.dt;
+          if (sa == sb && is_narrow_float(sa) && a.ty.dt == DT::F32 && b.ty.dt == DT::F32) {
+            n.in[0] = a.in[0];
+            n.in[1] = b.in[0];
+          }
+        }
+      }
+      // transpose(dot_general(X, Y)) on matrices: swap the operands instead
+      if (n.k == OpK::Transpose && n.ty.rank() == 2 && n.a0 == std::vector<int64_t>{1, 0}) {
+        const Node& d = g.nodes[n.in[0]];
+        if (d.k == OpK::DotGeneral && nuse[d.id] == 1 && d.a0.empty() && g.nodes[d.in[0]].ty.rank() == 2 &&
+            g.nodes[d.in[1]].ty.rank() == 2 && d.a2.size() == 1) {
+          Node nd = d;
+          nd.id = n.id;
+          nd.ty = n.ty;
+          nd.in = {d.in[1], d.in[0]};
+          nd.a2 = d.a3;
+          nd.a3 = d.a2;
+          n = nd;
+        }
+      }
+    }
+  }
+
+  // ------------------------------------------------------------------ analysis
+  int cone_cost(int id, int cap = 16) {
+    std::set<int> seen;
+    std::vector<int> st{id};
+    int cost = 0;
+    while (!st.empty() && cost <= cap) {
+      int x = st.back();
+      st.pop_back();
+      if (!seen.insert(x).second) continue;
+      const Node& n = g.nodes[x];
+      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::DotGeneral) continue;
+      if (n.k == OpK::Constant) continue;
+      if (x != id && prev_mat[x]) continue;
+      if (is_arith(n.k)) cost += (n.k == OpK::Unary || n.k == OpK::Gelu) ? 2 : 1;
+      for (int i : n.in) st.push_back(i);
+    }
+    return cost;
+  }
+
+  bool reaches_dot(int id) const {
+    std::set<int> seen;
+    std::vector<int> st{id};
+    while (!st.empty()) {
+      int x = st.back();
+      st.pop_back();
+      if (!seen.insert(x).second || seen.size() > 64) continue;
+      const Node& n = g.nodes[x];
+      if (n.k == OpK::DotGeneral) return true;
+      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce) continue;
+      if (x != id && prev_mat[x]) continue;
+      for (int i : n.in) st.push_back(i);
+    }
+    return false;
+  }
+
+  void analyze() {
+    const int N = (int)g.nodes.size();
+    live.assign(N, 0);
+    mat.assign(N, 0);
+    force_mat.assign(N, 0);
+    users.assign(N, {});
+    ctx.assign(N, {});
+    std::vector<int> st(g.results.begin(), g.results.end());
+    while (!st.empty()) {
+      int x = st.back();
+      st.pop_back();
+      if (live[x]) continue;
+      live[x] = 1;
+      for (int i : g.nodes[x].in) st.push_back(i);
+    }
+    for (int x = 0; x < N; ++x)
+      if (live[x]) for (int i : g.nodes[x].in) users[i].push_back(x);
+    std::vector<char> is_result(N, 0);
+    for (int r : g.results) is_result[r] = 1;
+
+    for (int x = N - 1; x >= 0; --x) {
+      if (!live[x]) continue;
+      const Node& n = g.nodes[x];
+      // contexts in which x is evaluated
+      std::set<Ctx> U;
+      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::DotGeneral ||
+                    (n.k == OpK::Constant && !n.splat);
+      for (int u : users[x]) {
+        const Node& un = g.nodes[u];
+        if (un.k == OpK::DotGeneral) { forced = true; continue; }
+        // start indices of dynamic slices must be constants; they are read at plan time
+        std::vector<Ctx> base;
+        if (mat[u]) base.push_back({u, ""});
+        else base.assign(ctx[u].begin(), ctx[u].end());
+        for (auto& c : base) {
+          std::string sig = c.second;
+          if (is_index_op(un.k)) {
+            for (size_t k = 0; k < un.in.size(); ++k)
+              if (un.in[k] == x) U.insert({c.first, sig + "/" + std::to_string(u) + ":" + std::to_string(k)});
+          } else if (n.ty.rank() == 0 && un.ty.rank() != 0) {
+            U.insert({c.first, sig + "/s"});
+          } else {
+            U.insert({c.first, sig});
+          }
+        }
+      }
+      if (n.ty.rank() == 0) {  // a 0-d value has a single index whatever the path
+        std::set<Ctx> V;
+        for (auto& c : U) V.insert({c.first, "0d"});
+        U.swap(V);
+      }
+      ctx[x] = U;
+      if (forced || force_mat[x]) { mat[x] = 1; continue; }
+      if (U.size() <= 1) continue;
+      // A value computed from a dot_general and read by several kernels: write it once, at the
+      // narrowest point of the single-consumer chain under it, so the dot keeps its epilogue.
+      {
+        std::set<int> roots;
+        for (auto& c : U) roots.insert(c.first);
+        if (roots.size() > 1 && reaches_dot(x)) {
+          int best = x, cur = x;
+          while (true) {
+            const Node& cn = g.nodes[cur];
+            if (!(cn.k == OpK::Convert || cn.k == OpK::Unary)) break;
+            int p = cn.in[0];
+            const Node& pn = g.nodes[p];
+            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce) break;
+            if (users[p].size() != 1 || is_result[p]) break;
+            cur = p;
+            if (info(pn.ty.dt).size < info(g.nodes[best].ty.dt).size) best = cur;
+          }
+          force_mat[best] = 1;
+          if (best == x) { mat[x] = 1; continue; }
+          continue;
+        }
+      }
+      int cost = cone_cost(x);
+      if (cost == 0) continue;
+      if (cost * ((int)U.size() - 1) <= 6) continue;
+      mat[x] = 1;
+    }
+  }
+
+  // ------------------------------------------------------------------ buffers
+  int buffer_for(int node) {
+    if (buf_of[node] >= 0) return buf_of[node];
+    const Node& n = g.nodes[node];
+    BufferDesc b;
+    b.ty = n.ty;
+    b.bytes = std::max<int64_t>(n.ty.bytes(), 1);
+    if (n.k == OpK::Param) { b.kind = BufferDesc::Param; b.param_index = (int)n.a0[0]; }
+    else if (n.k == OpK::Constant && !n.splat) { b.kind = BufferDesc::Const; b.data = n.data; }
+    else b.kind = BufferDesc::Temp;
+    plan.buffers.push_back(b);
+    return buf_of[node] = (int)plan.buffers.size() - 1;
+  }
+  int scratch(int64_t bytes) {
+    BufferDesc b;
+    b.kind = BufferDesc::Scratch;
+    b.bytes = bytes;
+    plan.buffers.push_back(b);
+    return (int)plan.buffers.size() - 1;
+  }
+
+  bool is_input(int root_or_self, int node) const {
+    (void)root_or_self;
+    return mat[node];
+  }
+
+  // ------------------------------------------------------------------ helpers
+  // Kernel text is written with the placeholder "@K@" in its symbol names; identical texts
+  // (the unrolled steps of a time loop) share one compiled kernel.
+  std::map<std::string, std::string> dedupe;
+  std::string finalize(const std::string& text) {
+    auto it = dedupe.find(text);
+    if (it != dedupe.end()) return it->second;
+    std::string base = "rxk" + std::to_string(kcount++);
+    dedupe[text] = base;
+    src << named(text, base);
+    return base;
+  }
+  static std::string named(std::string text, const std::string& base) {
+    size_t p = 0;
+    while ((p = text.find("@K@", p)) != std::string::npos) text.replace(p, 3, base);
+    return text;
+  }
+
+  static std::string ptr_decl(const std::string& stype, bool is_const, const std::string& name) {
+    return std::string(is_const ? "const " : "") + stype + "* __restrict__ " + name;
+  }
+
+  std::string signature(const std::string& kname, const std::vector<int>& inputs, const std::vector<std::pair<std::string, std::string>>& outs,
+                        int launch_bounds = kBlock) {
+    std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(launch_bounds) + ") void " + kname + "(";
+    bool first = true;
+    for (size_t k = 0; k < inputs.size(); ++k) {
+      s += (first ? "" : ", ") + ptr_decl(info(g.nodes[inputs[k]].ty.dt).stype, true, "in" + std::to_string(k));
+      first = false;
+    }
+    for (auto& o : outs) {
+      s += (first ? "" : ", ") + ptr_decl(o.first, false, o.second);
+      first = false;
+    }
+    return s + ")";
+  }
+
+  std::string describe(int root, const std::vector<int>& extra_roots = {}) {
+    std::set<int> seen;
+    std::vector<int> st{root};
+    for (int r : extra_roots) st.push_back(r);
+    std::map<std::string, int> cnt;
+    while (!st.empty()) {
+      int x = st.back();
+      st.pop_back();
+      if (!seen.insert(x).second) continue;
+      const Node& n = g.nodes[x];
+      if (x != root && mat[x] && std::find(extra_roots.begin(), extra_roots.end(), x) == extra_roots.end()) continue;
+      std::string nm;
+      switch (n.k) {
+        case OpK::Unary: case OpK::Binary: nm = n.op; break;
+        case OpK::Compare: nm = "compare"; break;
+        case OpK::Select: nm = "select"; break;
+        case OpK::Clamp: nm = "clamp"; break;
+        case OpK::Convert: nm = "convert"; break;
+        case OpK::Gelu: nm = "gelu"; break;
+        case OpK::BroadcastInDim: nm = "broadcast_in_dim"; break;
+        case OpK::Reshape: nm = "reshape"; break;
+        case OpK::Transpose: nm = "transpose"; break;
+        case OpK::Slice: nm = "slice"; break;
+        case OpK::Pad: nm = "pad"; break;
+        case OpK::DynamicUpdateSlice: nm = "dynamic_update_slice"; break;
+        case OpK::DynamicSlice: nm = "dynamic_slice"; break;
+        case OpK::Concatenate: nm = "concatenate"; break;
+        case OpK::Reduce: nm = "reduce"; break;
+        case OpK::DotGeneral: nm = "dot_general"; break;
+        case OpK::Iota: nm = "iota"; break;
+        default: break;
+      }
+      if (!nm.empty()) cnt[nm]++;
+      for (int i : n.in) st.push_back(i);
+    }
+    std::string s;
+    for (auto& kv : cnt) s += (s.empty() ? "" : " ") + kv.first + (kv.second > 1 ? "x" + std::to_string(kv.second) : "");
+    return s;
+  }
+
+  double algo_bytes(const std::vector<int>& inputs, const std::vector<int>& outs) {
+    double b = 0;
+    for (int i : inputs) b += (double)g.nodes[i].ty.bytes();
+    for (int o : outs) b += (double)g.nodes[o].ty.bytes();
+    return b;
+  }
+
+  static int pick_vec(const TType& t) {
+    if (t.rank() == 0) return 1;
+    int v = std::max(1, 16 / info(t.dt).size);
+    int64_t minor = t.dims.back();
+    while (v > 1 && minor % v != 0) v >>= 1;
+    return v;
+  }
+
+  // Decode a linear vector id into the root index variables (row-major, minor dim in vectors).
+  // Declares i0..i{n-2} and i{n-1}b (first lane of the vector).
+  static void decode_index(std::ostringstream& o, const std::string& it, const std::string& vid, const std::vector<int64_t>& dims, int vec,
+                           const std::string& pad) {
+    const int n = (int)dims.size();
+    if (n == 0) return;
+    std::string rest = vid;
+    const int64_t mv = dims[n - 1] / vec;
+    if (n == 1) {
+      o << pad << "const " << it << " i0b = " << rest << " * " << vec << ";\n";
+      return;
+    }
+    o << pad << "const " << it << " i" << n - 1 << "b = (" << rest << " % " << mv << ") * " << vec << ";\n";
+    o << pad << it << " rr = " << rest << " / " << mv << ";\n";
+    for (int d = n - 2; d >= 1; --d) {
+      o << pad << "const " << it << " i" << d << " = rr % " << dims[d] << ";\n";
+      o << pad << "rr /= " << dims[d] << ";\n";
+    }
+    o << pad << "const " << it << " i0 = rr;\n";
+  }
+
+  static Index root_index(const std::vector<int64_t>& dims) {
+    Index ix(dims.size());
+    for (size_t d = 0; d < dims.size(); ++d) {
+      ix[d].var = "i" + std::to_string(d);
+      ix[d].lo = 0;
+      ix[d].hi = dims[d] - 1;
+    }
+    return ix;
+  }
+
+  bool needs64(const std::vector<int>& nodes_touched) const {
+    for (int x : nodes_touched)
+      if (g.nodes[x].ty.numel() >= (int64_t)1 << 31) return true;
+    return false;
+  }
+
+  std::vector<int> cone_nodes(int root) const {
+    std::set<int> seen;
+    std::vector<int> st{root}, out;
+    while (!st.empty()) {
+      int x = st.back();
+      st.pop_back();
+      if (!seen.insert(x).second) continue;
+      out.push_back(x);
+      if (x != root && mat[x]) continue;
+      for (int i : g.nodes[x].in) st.push_back(i);
+    }
+    return out;
+  }
+
+  // ------------------------------------------------------------------ map kernels
+  void emit_map(int root) {
+    const Node& rn = g.nodes[root];
+    const auto& dims = rn.ty.dims;
+    const int n = rn.ty.rank();
+    const int vec = pick_vec(rn.ty);
+    const int64_t numel = rn.ty.numel();
+    if (numel == 0) return;
+    const int64_t nv = numel / vec;
+    const std::string kname = "@K@_map";
+    Emitter em(g, [&](int x) { return x != root && mat[x]; });
+    em.idx64 = needs64(cone_nodes(root));
+    const std::string it = em.idx_t();
+    std::vector<std::string> vars;
+    for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
+    em.set_root(dims, vars, vec > 1);
+    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.indent = 4;
+    Index ix = root_index(dims);
+    // evaluate the root op itself (it is materialized, so bypass the input test by emitting its op)
+    std::string val = em.emit(root, ix);
+    std::string body = em.take_code();
+
+    // shifted loads along the slowest dimension -> XCD slab order
+    bool slab = false;
+    if (opt.xcd_slabs && n >= 3 && dims[0] >= 8 && dims[1] >= 8 && numel >= opt.slab_min_numel) {
+      std::map<int, std::set<int64_t>> offs0;
+      for (auto& l : em.loads)
+        if (l.affine && (int)l.off.size() == n) offs0[l.node].insert(l.off[0]);
+      for (auto& kv : offs0) slab = slab || kv.second.size() > 1;
+    }
+
+    std::ostringstream o;
+    std::vector<std::pair<std::string, std::string>> outs{{info(rn.ty.dt).stype, "out0"}};
+    o << "// map: " << describe(root) << " -> " << rn.ty.str() << "\n";
+    o << signature(kname, em.inputs, outs) << " {\n";
+    unsigned grid;
+    if (!slab) {
+      const int64_t nblocks = (nv + kBlock - 1) / kBlock;
+      grid = (unsigned)nblocks;
+      o << "  const " << it << " vid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+      o << "  if (vid >= " << nv << ") return;\n";
+      decode_index(o, it, "vid", dims, vec, "  ");
+      o << "  const " << it << " lin0 = vid * " << vec << ";\n";
+    } else {
+      // XCD x owns rows [y0, y1) of dimension 1 for every index of dimension 0; inside an
+      // XCD the tiles advance along dimension 0 so that its L2 keeps the neighbouring planes.
+      int64_t plane = numel / dims[0];
+      int64_t rowlen = plane / dims[1];
+      int64_t ymax = (dims[1] + 7) / 8;
+      int64_t bps = (ymax * rowlen / vec + kBlock - 1) / kBlock;
+      grid = (unsigned)(8 * dims[0] * bps);
+      o << "  const unsigned xcd = blockIdx.x & 7u, lb = blockIdx.x >> 3;\n";
+      o << "  const " << it << " i0 = lb / " << bps << "u;\n";
+      o << "  const " << it << " cb = lb % " << bps << "u;\n";
+      o << "  const " << it << " y0 = (" << it << ")xcd * " << dims[1] << " / 8, y1 = (" << it << ")(xcd + 1) * " << dims[1] << " / 8;\n";
+      o << "  const " << it << " e = (cb * " << kBlock << " + threadIdx.x) * " << vec << ";\n";
+      o << "  if (e >= (y1 - y0) * " << rowlen << ") return;\n";
+      o << "  const " << it << " pe = y0 * " << rowlen << " + e;\n";
+      // decode pe inside the plane: dims[1..n-1]
+      {
+        std::string rest = "pe";
+        o << "  const " << it << " i" << n - 1 << "b = " << rest << " % " << dims[n - 1] << ";\n";
+        o << "  " << it << " rr = " << rest << " / " << dims[n - 1] << ";\n";
+        for (int d = n - 2; d >= 2; --d) {
+          o << "  const " << it << " i" << d << " = rr % " << dims[d] << ";\n";
+          o << "  rr /= " << dims[d] << ";\n";
+        }
+        if (n >= 3) o << "  const " << it << " i1 = rr;\n";
+      }
+      o << "  const " << it << " lin0 = i0 * " << plane << (em.idx64 ? "LL" : "") << " + pe;\n";
+    }
+    for (int slot : em.direct_inputs) {
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      o << "  const rx_vec<" << st << ", " << vec << "> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot
+        << " + lin0);\n";
+    }
+    const std::string ost = info(rn.ty.dt).stype;
+    if (n == 0) {
+      o << "  {\n" << body << "    out0[0] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n  }\n";
+    } else {
+      o << "  rx_vec<" << ost << ", " << vec << "> res;\n";
+      o << "#pragma unroll\n  for (int l = 0; l < " << vec << "; ++l) {\n";
+      o << "    const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
+      o << body;
+      o << "    res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n  }\n";
+      o << "  *reinterpret_cast<rx_vec<" << ost << ", " << vec << ">*>(out0 + lin0) = res;\n";
+    }
+    o << "}\n\n";
+    const std::string kb_final = finalize(o.str());
+
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = slab ? "map_stencil" : "map";
+    L.grid[0] = n == 0 ? 1 : grid;
+    L.block[0] = kBlock;
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    L.algo_bytes = algo_bytes(em.inputs, {root});
+    L.desc = describe(root);
+    plan.launches.push_back(L);
+  }
+
+  // ------------------------------------------------------------------ reductions
+  struct RedShape {
+    bool trailing = false;   // reduced dims are exactly the trailing dims
+    int64_t rows = 1, cols = 1;
+    int nkeep = 0;
+  };
+  RedShape red_shape(const Node& r) const {
+    const TType& in = g.nodes[r.in[0]].ty;
+    RedShape s;
+    std::vector<int64_t> dd = r.a0;
+    std::sort(dd.begin(), dd.end());
+    s.nkeep = in.rank() - (int)dd.size();
+    s.trailing = true;
+    for (size_t k = 0; k < dd.size(); ++k) s.trailing = s.trailing && dd[k] == s.nkeep + (int)k;
+    for (int d = 0; d < in.rank(); ++d) (d < s.nkeep ? s.rows : s.cols) *= in.dims[d];
+    return s;
+  }
+
+  // full reduction (all dims): two kernels
+  void emit_reduce_full(int root) {
+    const Node& rn = g.nodes[root];
+    const Node& inn = g.nodes[rn.in[0]];
+    const auto& dims = inn.ty.dims;
+    const int n = inn.ty.rank();
+    const DT dt = rn.ty.dt;
+    const std::string ACC = acc_ctype(dt);
+    const int vec = pick_vec(inn.ty);
+    const int64_t nv = inn.ty.numel() / vec;
+    const int U = 4;
+    int64_t tiles = (nv + (int64_t)kBlock * U - 1) / ((int64_t)kBlock * U);
+    const int G = (int)std::max<int64_t>(1, std::min<int64_t>(tiles, 2048));
+    const std::string k1 = "@K@_reduce", k2 = "@K@_reduce_final";
+
+    Emitter em(g, [&](int x) { return mat[x]; });
+    em.idx64 = needs64(cone_nodes(rn.in[0]));
+    const std::string it = em.idx_t();
+    std::vector<std::string> vars;
+    for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
+    em.set_root(dims, vars, vec > 1);
+    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.indent = 10;
+    std::string val = em.emit(rn.in[0], root_index(dims));
+    std::string body = em.take_code();
+
+    std::ostringstream o;
+    o << "// reduce (pass 1): " << describe(rn.in[0]) << " -> partials\n";
+    o << signature(k1, em.inputs, {{ACC, "partial"}}) << " {\n";
+    o << "  " << ACC << " acc[" << U << "];\n";
+    o << "#pragma unroll\n  for (int u = 0; u < " << U << "; ++u) acc[u] = " << red_identity(rn.red, dt) << ";\n";
+    o << "  for (" << it << " base = (" << it << ")blockIdx.x * " << kBlock * U << "; base < " << nv << "; base += (" << it << ")gridDim.x * " << kBlock * U
+      << ") {\n";
+    o << "#pragma unroll\n    for (int u = 0; u < " << U << "; ++u) {\n";
+    o << "      const " << it << " vid = base + u * " << kBlock << " + threadIdx.x;\n";
+    o << "      if (vid < " << nv << ") {\n";
+    decode_index(o, it, "vid", dims, vec, "        ");
+    o << "        const " << it << " lin0 = vid * " << vec << ";\n";
+    for (int slot : em.direct_inputs) {
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      o << "        const rx_vec<" << st << ", " << vec << "> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot
+        << " + lin0);\n";
+    }
+    o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
+    if (n > 0) o << "          const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
+    o << body;
+    o << "          acc[u] = " << red_apply(rn.red, dt, "acc[u]", "(" + ACC + ")" + val) << ";\n";
+    o << "        }\n      }\n    }\n  }\n";
+    o << "  " << ACC << " a = acc[0];\n";
+    o << "#pragma unroll\n  for (int u = 1; u < " << U << "; ++u) a = " << red_apply(rn.red, dt, "a", "acc[u]") << ";\n";
+    o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
+    o << "  a = rx_block_reduce<" << ACC << ", decltype(" << red_functor(rn.red) << "), " << kBlock / 64 << ">(a, " << red_functor(rn.red) << ", lds);\n";
+    o << "  if (threadIdx.x == 0) partial[blockIdx.x] = a;\n";
+    o << "}\n\n";
+
+    // pass 2
+    Emitter e2(g, [&](int x) { return mat[x]; });
+    e2.indent = 4;
+    std::string initv = e2.emit(rn.in[1], Index{});
+    std::string ibody = e2.take_code();
+    std::vector<int> in2 = e2.inputs;
+    o << "// reduce (pass 2): combine " << G << " partials, apply init -> " << rn.ty.str() << "\n";
+    {
+      std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + k2 + "(const " + ACC + "* __restrict__ partial";
+      for (size_t k = 0; k < in2.size(); ++k) s += ", " + ptr_decl(info(g.nodes[in2[k]].ty.dt).stype, true, "in" + std::to_string(k));
+      s += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
+      o << s << " {\n";
+    }
+    o << "  " << ACC << " a = " << red_identity(rn.red, dt) << ";\n";
+    o << "  for (int i = threadIdx.x; i < " << G << "; i += " << kBlock << ") a = " << red_apply(rn.red, dt, "a", "partial[i]") << ";\n";
+    o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
+    o << "  a = rx_block_reduce<" << ACC << ", decltype(" << red_functor(rn.red) << "), " << kBlock / 64 << ">(a, " << red_functor(rn.red) << ", lds);\n";
+    o << "  if (threadIdx.x == 0) {\n" << ibody;
+    o << "    const " << ACC << " r = " << red_apply(rn.red, dt, "a", "(" + ACC + ")" + initv) << ";\n";
+    std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
+    o << "    out0[0] = " << Emitter::store_conv(dt, rv) << ";\n  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+
+    int sc = scratch((int64_t)G * (dt == DT::F64 || info(dt).size == 8 ? 8 : 4));
+    Launch L1;
+    L1.kernel = named(k1, kb_final);
+    L1.kind = "reduce";
+    L1.grid[0] = G;
+    L1.block[0] = kBlock;
+    for (int i : em.inputs) L1.args.push_back(buffer_for(i));
+    L1.args.push_back(sc);
+    L1.algo_bytes = algo_bytes(em.inputs, {}) + info(dt).size;
+    L1.desc = describe(rn.in[0]) + " reduce";
+    plan.launches.push_back(L1);
+    Launch L2;
+    L2.kernel = named(k2, kb_final);
+    L2.kind = "reduce_final";
+    L2.grid[0] = 1;
+    L2.block[0] = kBlock;
+    L2.args.push_back(sc);
+    for (int i : in2) L2.args.push_back(buffer_for(i));
+    L2.args.push_back(buffer_for(root));
+    L2.desc = "combine partials";
+    plan.launches.push_back(L2);
+  }
+
+  // generic reduction: one thread per output element, sequential loops over reduced dims
+  void emit_reduce_generic(int root) {
+    const Node& rn = g.nodes[root];
+    const Node& inn = g.nodes[rn.in[0]];
+    const DT dt = rn.ty.dt;
+    const std::string ACC = acc_ctype(dt);
+    const int64_t nout = rn.ty.numel();
+    const std::string kname = "@K@_reduce_generic";
+    Emitter em(g, [&](int x) { return mat[x]; });
+    em.idx64 = needs64(cone_nodes(rn.in[0]));
+    const std::string it = em.idx_t();
+    em.set_root({}, {}, false);
+    std::vector<int> kept, red;
+    for (int d = 0; d < inn.ty.rank(); ++d)
+      (std::find(rn.a0.begin(), rn.a0.end(), d) == rn.a0.end() ? kept : red).push_back(d);
+    Index ix(inn.ty.rank());
+    for (size_t k = 0; k < kept.size(); ++k) { ix[kept[k]].var = "o" + std::to_string(k); ix[kept[k]].hi = inn.ty.dims[kept[k]] - 1; }
+    for (size_t k = 0; k < red.size(); ++k) { ix[red[k]].var = "r" + std::to_string(k); ix[red[k]].hi = inn.ty.dims[red[k]] - 1; }
+    em.indent = 4 + 2 * (int)red.size();
+    Emitter e2(g, [&](int x) { return mat[x]; });
+    e2.inputs = {};
+    std::string val = em.emit(rn.in[0], ix);
+    std::string body = em.take_code();
+    em.indent = 2;
+    std::string initv = em.emit(rn.in[1], Index{});
+    std::string ibody = em.take_code();
+    std::ostringstream o;
+    o << "// reduce (generic): " << describe(rn.in[0]) << " over dims -> " << rn.ty.str() << "\n";
+    o << signature(kname, em.inputs, {{info(dt).stype, "out0"}}) << " {\n";
+    o << "  const " << it << " oid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+    o << "  if (oid >= " << nout << ") return;\n";
+    o << "  " << it << " rr = oid;\n";
+    for (int k = (int)kept.size() - 1; k >= 0; --k) {
+      o << "  const " << it << " o" << k << " = rr % " << inn.ty.dims[kept[k]] << ";\n";
+      o << "  rr /= " << inn.ty.dims[kept[k]] << ";\n";
+    }
+    o << "  " << ACC << " acc = " << red_identity(rn.red, dt) << ";\n";
+    for (size_t k = 0; k < red.size(); ++k)
+      o << std::string(2 + 2 * k, ' ') << "for (" << it << " r" << k << " = 0; r" << k << " < " << inn.ty.dims[red[k]] << "; ++r" << k << ") {\n";
+    o << body;
+    o << std::string(4 + 2 * red.size(), ' ') << "acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n";
+    for (int k = (int)red.size() - 1; k >= 0; --k) o << std::string(2 + 2 * k, ' ') << "}\n";
+    o << ibody;
+    o << "  const " << ACC << " r = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + initv) << ";\n";
+    std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
+    o << "  out0[oid] = " << Emitter::store_conv(dt, rv) << ";\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = "reduce_generic";
+    L.grid[0] = (unsigned)((nout + kBlock - 1) / kBlock);
+    L.block[0] = kBlock;
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    L.algo_bytes = algo_bytes(em.inputs, {root});
+    L.desc = describe(rn.in[0]) + " reduce";
+    plan.launches.push_back(L);
+  }
+
+  // ------------------------------------------------------------------ row groups
+  // `root` is either a Reduce over the trailing dims (plain row reduction) or an
+  // elementwise node of shape [rows.., cols] whose cone contains row reductions `phases`.
+  void emit_row(int root, const std::vector<int>& phases) {
+    const Node& rn = g.nodes[root];
+    const bool root_is_reduce = rn.k == OpK::Reduce;
+    const TType& full = root_is_reduce ? g.nodes[rn.in[0]].ty : rn.ty;
+    const int n = full.rank();
+    int nkeep;
+    if (root_is_reduce) nkeep = red_shape(rn).nkeep;
+    else nkeep = red_shape(g.nodes[phases[0]]).nkeep;
+    int64_t rows = 1, cols = 1;
+    for (int d = 0; d < n; ++d) (d < nkeep ? rows : cols) *= full.dims[d];
+    int vec = pick_vec(full);
+    while (vec > 1 && cols % vec) vec >>= 1;
+    // lanes cooperating on one row
+    const int L = cols / vec >= 512 ? 256 : 64;
+    const int rows_per_block = kBlock / L;
+    const int64_t iters = (cols / vec + L - 1) / L;
+    const bool cache = iters <= 8;
+    const std::string kname = "@K@_row";
+
+    std::set<int> phase_set(phases.begin(), phases.end());
+    Emitter em(g, [&](int x) { return mat[x] && x != root && !phase_set.count(x); });
+    std::vector<int> touched = cone_nodes(root);
+    for (int p : phases) { auto c = cone_nodes(p); touched.insert(touched.end(), c.begin(), c.end()); }
+    em.idx64 = needs64(touched);
+    const std::string it = em.idx_t();
+    std::vector<std::string> vars;
+    for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
+    em.set_root(full.dims, vars, true);
+    em.direct_expr = [&](int slot) { return cache ? "c" + std::to_string(slot) + "[itv].v[l]" : "d" + std::to_string(slot) + ".v[l]"; };
+    Index ix = root_index(full.dims);
+
+    struct PhaseCode { int node; std::string body, val; };
+    std::vector<PhaseCode> pcs;
+    std::vector<int> order = phases;
+    std::sort(order.begin(), order.end());
+    em.indent = 6;
+    for (int p : order) {
+      PhaseCode pc;
+      pc.node = p;
+      em.push_scope();
+      pc.val = em.emit(g.nodes[p].in[0], ix);
+      pc.body = em.take_code();
+      em.pop_scope();
+      em.bound[p] = "r" + std::to_string(p);
+      pcs.push_back(pc);
+    }
+    std::string fbody, fval;
+    if (!root_is_reduce) {
+      em.push_scope();
+      fval = em.emit(root, ix);
+      fbody = em.take_code();
+      em.pop_scope();
+    }
+    // init values of the reductions (scalars)
+    em.indent = 2;
+    std::map<int, std::string> inits;
+    for (int p : order) inits[p] = em.emit(g.nodes[p].in[1], Index{});
+    std::string init_code = em.take_code();
+
+    std::ostringstream o;
+    std::vector<std::pair<std::string, std::string>> outs;
+    if (root_is_reduce) outs.push_back({info(rn.ty.dt).stype, "out0"});
+    else outs.push_back({info(rn.ty.dt).stype, "out0"});
+    o << "// row group (" << rows << " rows x " << cols << "): " << describe(root, phases) << "\n";
+    o << signature(kname, em.inputs, outs) << " {\n";
+    o << "  const int lane = threadIdx.x % " << L << ";\n";
+    o << "  const " << it << " row = (" << it << ")blockIdx.x * " << rows_per_block << " + threadIdx.x / " << L << ";\n";
+    if (L == 64) o << "  if (row >= " << rows << ") return;\n";  // whole wavefronts leave together
+    o << init_code;
+    // decode row -> leading index vars
+    {
+      o << "  " << it << " rr = row;\n";
+      for (int d = nkeep - 1; d >= 0; --d) {
+        o << "  const " << it << " i" << d << " = rr % " << full.dims[d] << ";\n";
+        o << "  rr /= " << full.dims[d] << ";\n";
+      }
+    }
+    o << "  const " << it << " rowbase = row * " << cols << (em.idx64 ? "LL" : "") << ";\n";
+    if (L == 256) o << "  __shared__ double lds_raw[" << kBlock / 64 << "];\n";
+    // column loop header: declares trailing index vars for vector `itv`
+    auto loop_open = [&](std::ostringstream& s) {
+      s << "#pragma unroll\n  for (int itv = 0; itv < " << iters << "; ++itv) {\n";
+      s << "    const " << it << " cv = (" << it << ")(itv * " << L << " + lane) * " << vec << ";\n";
+      s << "    if (cv < " << cols << ") {\n";
+      s << "      const " << it << " lin0 = rowbase + cv;\n";
+    };
+    auto decode_cols = [&](std::ostringstream& s) {
+      // column offset c = cv + l -> trailing dims
+      if (n - nkeep == 1) {
+        s << "        const " << it << " i" << n - 1 << " = cv + l;\n";
+      } else {
+        s << "        " << it << " cc = cv + l;\n";
+        for (int d = n - 1; d > nkeep; --d) {
+          s << "        const " << it << " i" << d << " = cc % " << full.dims[d] << ";\n";
+          s << "        cc /= " << full.dims[d] << ";\n";
+        }
+        s << "        const " << it << " i" << nkeep << " = cc;\n";
+      }
+    };
+    // preload of direct inputs
+    auto preload = [&](std::ostringstream& s, bool into_cache) {
+      for (int slot : em.direct_inputs) {
+        const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+        if (into_cache)
+          s << "      c" << slot << "[itv] = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot << " + lin0);\n";
+        else
+          s << "      const rx_vec<" << st << ", " << vec << "> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot
+            << " + lin0);\n";
+      }
+    };
+    if (cache) {
+      for (int slot : em.direct_inputs) {
+        const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+        o << "  rx_vec<" << st << ", " << vec << "> c" << slot << "[" << iters << "];\n";
+      }
+      if (!em.direct_inputs.empty()) {
+        loop_open(o);
+        preload(o, true);
+        o << "    }\n  }\n";
+      }
+    }
+    for (auto& pc : pcs) {
+      const Node& p = g.nodes[pc.node];
+      const DT dt = p.ty.dt;
+      const std::string ACC = acc_ctype(dt);
+      o << "  " << ACC << " a" << pc.node << " = " << red_identity(p.red, dt) << ";\n";
+      loop_open(o);
+      if (!cache) preload(o, false);
+      o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
+      decode_cols(o);
+      o << pc.body;
+      o << "        a" << pc.node << " = " << red_apply(p.red, dt, "a" + std::to_string(pc.node), "(" + ACC + ")" + pc.val) << ";\n";
+      o << "      }\n    }\n  }\n";
+      if (L == 64)
+        o << "  a" << pc.node << " = rx_wave_reduce(a" << pc.node << ", " << red_functor(p.red) << ");\n";
+      else
+        o << "  a" << pc.node << " = rx_block_reduce<" << ACC << ", decltype(" << red_functor(p.red) << "), " << kBlock / 64 << ">(a" << pc.node << ", "
+          << red_functor(p.red) << ", reinterpret_cast<" << ACC << "*>(lds_raw));\n";
+      std::string comb = red_apply(p.red, dt, "a" + std::to_string(pc.node), "(" + ACC + ")" + inits[pc.node]);
+      std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, comb) : std::string("(") + info(dt).ctype + ")(" + comb + ")";
+      o << "  const " << info(dt).ctype << " r" << pc.node << " = " << rv << ";\n";
+    }
+    if (root_is_reduce) {
+      o << "  if (lane == 0) out0[row] = " << Emitter::store_conv(rn.ty.dt, "r" + std::to_string(root)) << ";\n";
+    } else {
+      const std::string ost = info(rn.ty.dt).stype;
+      loop_open(o);
+      if (!cache) preload(o, false);
+      o << "      rx_vec<" << ost << ", " << vec << "> res;\n";
+      o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
+      decode_cols(o);
+      o << fbody;
+      o << "        res.v[l] = " << Emitter::store_conv(rn.ty.dt, fval) << ";\n      }\n";
+      o << "      *reinterpret_cast<rx_vec<" << ost << ", " << vec << ">*>(out0 + lin0) = res;\n";
+      o << "    }\n  }\n";
+    }
+    o << "}\n\n";
+    const std::string kb_final = finalize(o.str());
+
+    Launch Lc;
+    Lc.kernel = named(kname, kb_final);
+    Lc.kind = "row";
+    Lc.grid[0] = (unsigned)((rows + rows_per_block - 1) / rows_per_block);
+    Lc.block[0] = kBlock;
+    for (int i : em.inputs) Lc.args.push_back(buffer_for(i));
+    Lc.args.push_back(buffer_for(root));
+    Lc.algo_bytes = algo_bytes(em.inputs, {root});
+    Lc.desc = describe(root, phases);
+    plan.launches.push_back(Lc);
+    (void)L;
+  }
+
+  // Row reductions that can run inside the kernel of `root` (see header comment).
+  std::vector<int> row_phases(int root) {
+    const Node& rn = g.nodes[root];
+    std::vector<int> phases;
+    if (!opt.row_fusion || rn.ty.rank() < 2) return phases;
+    std::set<int> S{root};
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      for (int x = 0; x < (int)g.nodes.size(); ++x) {
+        if (!live[x] || S.count(x)) continue;
+        const Node& r = g.nodes[x];
+        if (r.k != OpK::Reduce) continue;
+        if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
+        const TType& in = g.nodes[r.in[0]].ty;
+        if (in.dims != rn.ty.dims) continue;
+        RedShape rs = red_shape(r);
+        if (!rs.trailing || rs.nkeep == 0 || rs.nkeep == in.rank()) continue;
+        if (!phases.empty() && red_shape(g.nodes[phases[0]]).nkeep != rs.nkeep) continue;
+        if (ctx[x].empty()) continue;
+        bool ok = true;
+        for (auto& c : ctx[x]) {
+          if (!S.count(c.first)) { ok = false; break; }
+          // path must be: (elementwise)* broadcast_in_dim(dims = 0..nkeep-1) (elementwise on the kept shape)*
+          const std::string& sig = c.second;
+          if (sig.size() < 2 || sig[0] != '/' || sig.find('/', 1) != std::string::npos) { ok = false; break; }
+          int bid = std::stoi(sig.substr(1, sig.find(':') - 1));
+          const Node& b = g.nodes[bid];
+          if (b.k != OpK::BroadcastInDim || b.ty.dims != rn.ty.dims || (int)b.a0.size() != rs.nkeep) { ok = false; break; }
+          for (int k = 0; k < rs.nkeep; ++k) ok = ok && b.a0[k] == k;
+          if (!ok) break;
+        }
+        if (!ok) continue;
+        S.insert(x);
+        phases.push_back(x);
+        changed = true;
+      }
+    }
+    return phases;
+  }
+
+  // ------------------------------------------------------------------ dot groups
+  struct DotForm {
+    bool ok = false;        // matrix (optionally batched) form the GEMM skeletons understand
+    int64_t batch = 1, M = 1, N = 1, K = 1;
+    bool a_k_contig = false;  // lhs stored [.., M, K] (true) or [.., K, M]
+    bool b_k_contig = false;  // rhs stored [.., N, K] (true) or [.., K, N]
+  };
+  DotForm dot_form(const Node& d) const {
+    DotForm f;
+    const TType &l = g.nodes[d.in[0]].ty, &r = g.nodes[d.in[1]].ty;
+    if (d.a2.size() != 1) return f;
+    if (d.a0.size() > 1) return f;
+    const int nb = (int)d.a0.size();
+    if (l.rank() != 2 + nb || r.rank() != 2 + nb) return f;
+    if (nb == 1 && (d.a0[0] != 0 || d.a1[0] != 0)) return f;
+    const int lc = (int)d.a2[0], rc = (int)d.a3[0];
+    f.batch = nb ? l.dims[0] : 1;
+    f.K = l.dims[lc];
+    f.a_k_contig = lc == nb + 1;
+    f.b_k_contig = rc == nb + 1;
+    f.M = l.dims[f.a_k_contig ? nb : nb + 1];
+    f.N = r.dims[f.b_k_contig ? nb : nb + 1];
+    f.ok = true;
+    return f;
+  }
+
+  // Emit the dot group rooted at `root`; `dot` is the DotGeneral node inside it
+  // (root == dot when there is no epilogue).
+  void emit_dot(int root, int dot) {
+    const Node& d = g.nodes[dot];
+    const Node& rn = g.nodes[root];
+    const TType &lt = g.nodes[d.in[0]].ty, &rt = g.nodes[d.in[1]].ty;
+    DotForm f = dot_form(d);
+    const std::string kbase = "@K@";
+    const int n = rn.ty.rank();
+
+    // Epilogue: the cone from the root down to the dot accumulator, evaluated on NV
+    // consecutive elements of the minor output dimension (vector loads of same-shaped
+    // operands such as C in alpha*A*B + beta*C, one vector store).
+    Emitter em(g, [&](int x) { return mat[x] && x != root; });
+    em.idx64 = needs64(cone_nodes(root)) || lt.numel() >= ((int64_t)1 << 31) || rt.numel() >= ((int64_t)1 << 31);
+    const std::string it = em.idx_t();
+    std::vector<std::string> vars;
+    for (int k = 0; k < n; ++k) vars.push_back("i" + std::to_string(k));
+    em.set_root(rn.ty.dims, vars, n > 0);
+    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.indent = 6;
+    const std::string DCT = info(d.ty.dt).ctype;
+    em.bound[dot] = "accv";
+    std::string val = root == dot ? std::string("accv") : em.emit(root, root_index(rn.ty.dims));
+    std::string ebody = em.take_code();
+    const std::string ACC = is_float(d.ty.dt) ? (d.ty.dt == DT::F64 ? "double" : "float") : info(d.ty.dt).ctype;
+
+    GemmChoice gc;
+    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig);
+    std::ostringstream o;
+    o << "// dot epilogue: " << describe(root) << "\n";
+    o << "struct " << kbase << "_epi {\n";
+    for (size_t k = 0; k < em.inputs.size(); ++k)
+      o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
+    const std::string ost = info(rn.ty.dt).stype;
+    o << "  " << ost << "* __restrict__ out0;\n";
+    o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const " << ACC << " (&acc)[NV]";
+    for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
+    o << ") const {\n";
+    {
+      Index rix = root_index(rn.ty.dims);
+      if (n > 0) rix[n - 1].var = "i" + std::to_string(n - 1) + "b";
+      o << "    const " << it << " lin0 = " << (n ? em.linear(rix, rn.ty.dims) : std::string("0")) << ";\n";
+    }
+    for (int slot : em.direct_inputs) {
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      o << "    const rx_vec<" << st << ", NV> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", NV>*>(in" << slot << " + lin0);\n";
+    }
+    o << "    rx_vec<" << ost << ", NV> res;\n";
+    o << "#pragma unroll\n    for (int l = 0; l < NV; ++l) {\n";
+    if (n > 0) o << "      const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
+    {
+      std::string accv = is_narrow_float(d.ty.dt) ? Emitter::round_narrow(d.ty.dt, "acc[l]") : std::string("(") + DCT + ")acc[l]";
+      o << "      const " << DCT << " accv = " << accv << ";\n";
+    }
+    o << ebody;
+    o << "      res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n    }\n";
+    o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+    o << "  }\n};\n\n";
+
+    std::vector<int> epi_inputs = em.inputs;
+    Launch L;
+    {
+      double kprod = 1;
+      for (auto c : d.a2) kprod *= (double)lt.dims[c];
+      L.flops = 2.0 * (double)d.ty.numel() * kprod;
+    }
+    std::vector<int> all_in{d.in[0], d.in[1]};
+    for (int i : epi_inputs) if (i != d.in[0] && i != d.in[1]) all_in.push_back(i);
+    L.algo_bytes = algo_bytes(all_in, {root});
+    L.desc = describe(root);
+
+    auto epi_ctor = [&]() {
+      std::string s = kbase + "_epi epi{";
+      for (size_t k = 0; k < epi_inputs.size(); ++k) s += "in" + std::to_string(k) + ", ";
+      return s + "out0};";
+    };
+    auto epi_params = [&]() {
+      std::string s;
+      for (size_t k = 0; k < epi_inputs.size(); ++k) s += ", const " + std::string(info(g.nodes[epi_inputs[k]].ty.dt).stype) + "* __restrict__ in" + std::to_string(k);
+      return s + ", " + ost + "* __restrict__ out0";
+    };
+
+    if (gc.ok) {
+      o << gemm_instance(gc, kbase, epi_params(), epi_ctor());
+      L.kernel = kbase + "_gemm";
+      L.kind = gc.kind;
+      L.grid[0] = gc.grid[0]; L.grid[1] = gc.grid[1]; L.grid[2] = gc.grid[2];
+      L.block[0] = gc.block;
+      L.lds_bytes = gc.lds_bytes;
+    } else {
+      // scalar contraction: one thread per output element; any dims, any element type
+      const int64_t nout = d.ty.numel();
+      o << "// dot_general (scalar loop) " << lt.str() << " x " << rt.str() << "\n";
+      o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << kbase << "_dot(const " << info(lt.dt).stype << "* __restrict__ A, const "
+        << info(rt.dt).stype << "* __restrict__ B" << epi_params() << ") {\n";
+      o << "  const " << it << " oid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+      o << "  if (oid >= " << nout << ") return;\n";
+      std::vector<int> lfree, rfree;
+      auto isin = [](const std::vector<int64_t>& v, int x) { return std::find(v.begin(), v.end(), (int64_t)x) != v.end(); };
+      for (int k = 0; k < lt.rank(); ++k) if (!isin(d.a0, k) && !isin(d.a2, k)) lfree.push_back(k);
+      for (int k = 0; k < rt.rank(); ++k) if (!isin(d.a1, k) && !isin(d.a3, k)) rfree.push_back(k);
+      o << "  " << it << " rr = oid;\n";
+      for (int k = d.ty.rank() - 1; k >= 0; --k) {
+        o << "  const " << it << " i" << k << " = rr % " << d.ty.dims[k] << ";\n";
+        o << "  rr /= " << d.ty.dims[k] << ";\n";
+      }
+      std::vector<std::string> li(lt.rank()), ri(rt.rank());
+      int od = 0;
+      for (size_t k = 0; k < d.a0.size(); ++k, ++od) { li[d.a0[k]] = "i" + std::to_string(od); ri[d.a1[k]] = "i" + std::to_string(od); }
+      for (int k : lfree) li[k] = "i" + std::to_string(od++);
+      for (int k : rfree) ri[k] = "i" + std::to_string(od++);
+      for (size_t k = 0; k < d.a2.size(); ++k) { li[d.a2[k]] = "k" + std::to_string(k); ri[d.a3[k]] = "k" + std::to_string(k); }
+      auto lin = [&](const std::vector<std::string>& ixs, const std::vector<int64_t>& dims) {
+        std::string s2 = "0";
+        int64_t stride = 1;
+        for (int k = (int)dims.size() - 1; k >= 0; --k) {
+          s2 += " + (" + it + ")" + ixs[k] + " * " + std::to_string(stride);
+          stride *= dims[k];
+        }
+        return s2;
+      };
+      o << "  " << ACC << " acc[1] = {0};\n";
+      for (size_t k = 0; k < d.a2.size(); ++k)
+        o << "  for (" << it << " k" << k << " = 0; k" << k << " < " << lt.dims[d.a2[k]] << "; ++k" << k << ")\n";
+      Emitter tmp(g, [](int) { return true; });
+      o << "    acc[0] += (" << ACC << ")" << tmp.load_conv(lt.dt, "A[" + lin(li, lt.dims) + "]") << " * (" << ACC << ")"
+        << tmp.load_conv(rt.dt, "B[" + lin(ri, rt.dims) + "]") << ";\n";
+      o << "  " << epi_ctor() << "\n";
+      o << "  epi(acc";
+      for (int k = 0; k < n; ++k) o << ", i" << k;
+      o << ");\n}\n\n";
+      L.kernel = kbase + "_dot";
+      L.kind = "dot_scalar";
+      L.grid[0] = (unsigned)((nout + kBlock - 1) / kBlock);
+      L.block[0] = kBlock;
+    }
+    const std::string kb_final = finalize(o.str());
+    L.kernel = named(L.kernel, kb_final);
+    L.args.push_back(buffer_for(d.in[0]));
+    L.args.push_back(buffer_for(d.in[1]));
+    for (int i : epi_inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    plan.launches.push_back(L);
+  }
+
+  // ------------------------------------------------------------------ driver
+  void run() {
+    canonicalize();
+    const int N = (int)g.nodes.size();
+    // Decisions about a node depend on which of its producers own buffers; sweep until stable.
+    prev_mat.assign(N, 0);
+    for (int sweep = 0; sweep < 6; ++sweep) {
+      analyze();
+      if (mat == prev_mat) break;
+      prev_mat = mat;
+    }
+    buf_of.assign(N, -1);
+    plan.aliasing_output = g.aliasing_output;
+    for (int p : g.params) { plan.param_types.push_back(g.nodes[p].ty); buffer_for(p); }
+
+    // dot epilogues: an elementwise root that consumes a dot result at the identity index
+    std::map<int, int> epilogue_of;  // dot node -> root that absorbs it
+    for (int x = 0; x < N; ++x) {
+      if (!live[x] || g.nodes[x].k != OpK::DotGeneral) continue;
+      if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
+      if (ctx[x].size() != 1) continue;
+      const Ctx& c = *ctx[x].begin();
+      if (!c.second.empty()) continue;
+      const Node& r = g.nodes[c.first];
+      if (r.k == OpK::Reduce || r.k == OpK::DotGeneral) continue;
+      if (r.ty.dims != g.nodes[x].ty.dims) continue;
+      // the root must not be the anchor of a row group (its reductions need the full row)
+      if (!row_phases(c.first).empty()) continue;
+      epilogue_of[x] = c.first;
+    }
+    std::set<int> absorbed_roots;
+    for (auto& kv : epilogue_of) absorbed_roots.insert(kv.second);
+    std::set<int> fused_reduces;
+
+    // kernels in topological order of their roots
+    std::vector<std::pair<int, std::function<void()>>> jobs;
+    for (int x = 0; x < N; ++x) {
+      if (!live[x] || !mat[x]) continue;
+      const Node& n = g.nodes[x];
+      if (n.k == OpK::Param || (n.k == OpK::Constant && !n.splat)) continue;
+      if (n.k == OpK::DotGeneral) {
+        auto e = epilogue_of.find(x);
+        if (e != epilogue_of.end()) continue;  // emitted with its root
+        jobs.push_back({x, [this, x] { emit_dot(x, x); }});
+        continue;
+      }
+      if (absorbed_roots.count(x)) {
+        int dot = -1;
+        for (auto& kv : epilogue_of) if (kv.second == x) dot = kv.first;
+        jobs.push_back({x, [this, x, dot] { emit_dot(x, dot); }});
+        continue;
+      }
+      if (n.k == OpK::Reduce) {
+        jobs.push_back({x, [this, x, &fused_reduces] {
+          if (fused_reduces.count(x)) return;
+          const Node& r = g.nodes[x];
+          RedShape rs = red_shape(r);
+          if (g.nodes[r.in[0]].ty.numel() == 0 || r.ty.numel() == 0) { emit_reduce_generic(x); return; }
+          if (rs.nkeep == 0) { emit_reduce_full(x); return; }
+          if (rs.trailing && rs.cols >= 64) { emit_row(x, {x}); return; }
+          emit_reduce_generic(x);
+        }});
+        continue;
+      }
+      jobs.push_back({x, [this, x, &fused_reduces] {
+        std::vector<int> ph = row_phases(x);
+        if (!ph.empty()) {
+          for (int p : ph) fused_reduces.insert(p);
+          emit_row(x, ph);
+        } else emit_map(x);
+      }});
+    }
+    // row groups claim their reductions before those would be emitted on their own
+    for (auto& j : jobs) {
+      const Node& n = g.nodes[j.first];
+      if (n.k != OpK::Reduce && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
+        for (int p : row_phases(j.first)) fused_reduces.insert(p);
+    }
+    for (auto& j : jobs) j.second();
+
+    for (int r : g.results) {
+      plan.result_types.push_back(g.nodes[r].ty);
+      int b = buffer_for(r);
+      plan.buffers[b].is_result = true;
+      plan.result_buffers.push_back(b);
+    }
+    // liveness over the launch list
+    for (size_t li = 0; li < plan.launches.size(); ++li) {
+      auto& L = plan.launches[li];
+      for (int b : L.args) {
+        auto& B = plan.buffers[b];
+        if (B.first_def < 0) B.first_def = (int)li;
+        B.last_use = (int)li;
+      }
+    }
+    plan.source = "#include \"rx_preamble.h\"\n#include \"rx_gemm_kernels.h\"\n\n" + src.str();
+  }
+};
+
+}  // namespace
+
+std::string Plan::report() const {
+  std::ostringstream o;
+  o << "buffers: " << buffers.size() << ", launches: " << launches.size() << "\n";
+  for (size_t i = 0; i < launches.size(); ++i) {
+    auto& L = launches[i];
+    o << "  [" << i << "] " << L.kernel << " kind=" << L.kind << " grid=" << L.grid[0] << "x" << L.grid[1] << "x" << L.grid[2] << " block=" << L.block[0]
+      << " lds=" << L.lds_bytes << " algo_bytes=" << (long long)L.algo_bytes << " flops=" << (long long)L.flops << " :: " << L.desc << "\n";
+  }
+  return o.str();
+}
+
+Plan make_plan(const Graph& g, const PlanOptions& opt) {
+  Planner p(g, opt);
+  p.run();
+  return std::move(p.plan);
+}
+
+}  // namespace rx

@@ -1,0 +1,52 @@
+// Fusion planning: rx::Graph -> fusion groups -> one HIP translation unit plus a
+// launch list.  The runtime compiles the text with hiprtc and replays the list.
+#pragma once
+#include "rx_ir.h"
+
+namespace rx {
+
+struct BufferDesc {
+  enum Kind { Param, Const, Temp, Scratch } kind = Temp;
+  TType ty;                    // element type / shape (Scratch: bytes only)
+  int64_t bytes = 0;
+  int param_index = -1;        // Param
+  std::vector<uint8_t> data;   // Const: storage bytes uploaded once at compile time
+  int first_def = -1;          // index of the launch that writes it (Temp/Scratch)
+  int last_use = -1;           // index of the last launch that touches it
+  bool is_result = false;
+};
+
+struct Launch {
+  std::string kernel;          // symbol in the translation unit
+  std::string kind;            // "map" | "reduce" | "reduce_final" | "row" | "dot" | "gemm_*"
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {1, 1, 1};
+  unsigned lds_bytes = 0;
+  std::vector<int> args;       // buffer ids, in kernel parameter order
+  int n_outputs = 1;           // trailing args written by the kernel
+  double algo_bytes = 0;       // compulsory HBM traffic: distinct inputs once + outputs once
+  double flops = 0;            // contraction flops (2*M*N*K) for dot groups
+  std::string desc;            // human-readable summary of the fused ops
+};
+
+struct Plan {
+  std::string source;                  // HIP text for all kernels of the module
+  std::vector<BufferDesc> buffers;
+  std::vector<Launch> launches;
+  std::vector<int> result_buffers;     // per @main result: buffer id
+  std::vector<TType> param_types, result_types;
+  std::vector<int> aliasing_output;    // per argument: result index it may alias, or -1
+  std::string report() const;          // text summary for debugging
+};
+
+struct PlanOptions {
+  bool xcd_slabs = true;        // XCD-aware tile order for kernels with shifted loads
+  int64_t slab_min_numel = 1 << 22;  // smallest output that uses it
+  bool mfma = true;             // use the MFMA GEMM skeletons for eligible dot_generals
+  bool row_fusion = true;       // fuse row reductions with their elementwise consumers
+  bool lds_stencil = true;      // stage inputs read at several offsets through LDS halo tiles
+};
+
+Plan make_plan(const Graph& g, const PlanOptions& opt);
+
+}  // namespace rx

@@ -1,0 +1,40 @@
+"""Shared helpers: run one StableHLO module on the GPU through the C ABI and in
+the oracle on identical bytes."""
+import numpy as np
+
+from oracle import stablehlo_interp as I
+
+
+def gpu_run(rx, client, text, args, exe=None):
+    """args: list of oracle Tensors.  Returns (list of oracle Tensors from the GPU, executable)."""
+    exe = exe or rx.xla_compile(client, text)
+    bufs = []
+    for a in args:
+        raw = np.frombuffer(a.to_bytes(), dtype=rx._STORAGE[a.dt]).reshape(a.shape)
+        bufs.append(rx.Buffer.from_host(client, raw, a.dt))
+    outs = exe.execute_sharded(bufs)
+    res = []
+    for ab in outs:
+        b = ab.synced_buffer()
+        raw = b.to_host()
+        res.append(I.Tensor.from_bytes(raw.tobytes(), b.dtype(), b.shape()))
+    return res, exe
+
+
+def oracle_run(text, args, hifi=True):
+    return I.run_text(text, args, hifi=hifi)
+
+
+def rel_err(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    den = np.maximum(np.abs(ref), 1e-30)
+    return float(np.max(np.abs(got - ref) / den)) if got.size else 0.0
+
+
+def max_rel_to_scale(got, ref):
+    """max |got-ref| / max|ref|: error relative to the magnitude of the result."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    scale = max(float(np.max(np.abs(ref))), 1e-30) if ref.size else 1.0
+    return float(np.max(np.abs(got - ref))) / scale if got.size else 0.0

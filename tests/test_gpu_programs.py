@@ -1,0 +1,104 @@
+"""GPU parity of the five benchmark programs at sizes the oracle finishes in
+seconds.  Tolerances are the ones the project states: integers bit-exact, fp32
+maps 1e-6 relative, fp32 reductions 1e-5*sqrt(n) relative, bf16/fp8 contractions
+1e-2 relative to an f32/f64-accumulated reference."""
+import numpy as np
+import pytest
+
+from _harness import gpu_run, oracle_run, max_rel_to_scale
+from _loader import load_programs
+from oracle import stablehlo_interp as I
+
+pytestmark = pytest.mark.gpu
+P = load_programs()
+
+
+@pytest.mark.parametrize("n", [1, 7, 64, 1000, 4096, 1 << 20])
+def test_sinsum_add(rx, client, n):
+    x = np.random.default_rng(0).uniform(-np.pi, np.pi, n).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-np.pi, np.pi, n).astype(np.float32)
+    args = [I.Tensor(x, "f32"), I.Tensor(y, "f32")]
+    text = P.sinsum_add(n)
+    got, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    exact = np.sum(np.sin(x.astype(np.float64)) + y.astype(np.float64))
+    scale = np.sum(np.abs(np.sin(x.astype(np.float64)) + y.astype(np.float64)))
+    # fp32 reduction: 1e-5*sqrt(n) relative (to the magnitude of the summands)
+    tol = 1e-5 * np.sqrt(n)
+    assert abs(float(got[0].a) - exact) <= tol * max(scale / max(n, 1), abs(exact), 1e-6) + 1e-6 * scale / np.sqrt(n)
+    assert abs(float(ref[0].a) - exact) <= tol * max(abs(exact), 1e-6) + 1e-6 * scale
+
+
+@pytest.mark.parametrize("shape,embed", [((6, 5, 4), "pad"), ((6, 5, 4), "dus"), ((32, 16, 8), "pad"),
+                                         ((64, 64, 32), "pad")])
+def test_stencil(rx, client, shape, embed):
+    nx, ny, nz = shape
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(0)
+    c = np.zeros(full)
+    c[3:-3, 3:-3, 3:-3] = rng.uniform(0, 1, (nz, ny, nx))
+    u, v, w = [np.random.default_rng(s).uniform(-1, 1, full) for s in (1, 2, 3)]
+    args = [I.Tensor(a, "f64") for a in (c, u, v, w)]
+    text = P.stencil(nx, ny, nz, steps=3, embed=embed)
+    got, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args)
+    # add/mul chains evaluated in the module's order with contraction off: bit-exact
+    assert np.array_equal(got[0].a, ref[0].a)
+
+
+def test_stencil_xcd_slab_order(rx, client, monkeypatch):
+    """Same parity with the XCD-slab tile order forced on a small grid."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    test_stencil(rx, client, (64, 40, 20), "pad")
+    test_stencil(rx, client, (30, 33, 9), "dus")
+
+
+@pytest.mark.parametrize("m,n,k,form", [(5, 7, 3, "propagated"), (5, 7, 3, "transposed"), (64, 48, 32, "propagated"),
+                                        (256, 256, 256, "propagated"), (128, 256, 64, "transposed")])
+def test_gemm_f32(rx, client, m, n, k, form):
+    A = np.random.default_rng(0).normal(size=(m, k)).astype(np.float32)
+    B = np.random.default_rng(1).normal(size=(k, n)).astype(np.float32)
+    C = np.random.default_rng(2).normal(size=(m, n)).astype(np.float32)
+    args = [I.Tensor(A.T.copy(), "f32"), I.Tensor(B.T.copy(), "f32"), I.Tensor(C.T.copy(), "f32")]
+    text = P.gemm(m, n, k, form=form)
+    got, _ = gpu_run(rx, client, text, args)
+    ref = 1.5 * (A.astype(np.float64) @ B.astype(np.float64)) + 1.2 * C.astype(np.float64)
+    assert max_rel_to_scale(got[0].a.T, ref) <= 1e-5 * np.sqrt(k)
+    orc = oracle_run(text, args, hifi=True)
+    assert max_rel_to_scale(orc[0].a.T, ref) <= 1e-6
+
+
+def _mlp_args(batch, widths, seed=0):
+    rng = np.random.default_rng(seed)
+    args = [I.tensor(rng.normal(size=(batch, widths[0])), "bf16")]
+    for l in range(len(widths) - 1):
+        lim = np.sqrt(6.0 / (widths[l] + widths[l + 1]))
+        args.append(I.tensor(np.random.default_rng(seed + 1 + l).uniform(-lim, lim, size=(widths[l], widths[l + 1])), "bf16"))
+        args.append(I.tensor(np.random.default_rng(seed + 4 + l).normal(size=(widths[l + 1],)) * 0.01, "bf16"))
+    return args
+
+
+@pytest.mark.parametrize("batch,widths,gelu", [(8, (16, 32, 32, 16), "chain"), (64, (32, 64, 64, 32), "op"),
+                                               (256, (128, 256, 256, 128), "chain")])
+def test_mlp_bf16(rx, client, batch, widths, gelu):
+    args = _mlp_args(batch, widths)
+    text = P.mlp(batch, widths, gelu=gelu)
+    got, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    # softmax output: rows sum to one, and agree with the f64-accumulated oracle to 1e-2 of the row scale
+    assert np.allclose(got[0].a.sum(axis=1), 1.0, atol=2e-2)
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-2
+
+
+@pytest.mark.parametrize("batch,k,n,layout,form", [(8, 32, 16, "nk", "convert"), (8, 32, 16, "kn", "direct"),
+                                                   (64, 128, 256, "nk", "convert"), (128, 256, 128, "kn", "convert")])
+def test_fp8_linear(rx, client, batch, k, n, layout, form):
+    a = I.tensor(np.random.default_rng(0).normal(size=(batch, k)), "bf16")
+    wq = I.tensor(np.random.default_rng(1).normal(size=(n, k) if layout == "nk" else (k, n)), "f8E4M3FN")
+    sw = I.Tensor(np.float32(0.0123), "f32")
+    text = P.fp8_linear(batch, k, n, weight_layout=layout, dot_form=form)
+    got, _ = gpu_run(rx, client, text, [a, wq, sw])
+    ref = oracle_run(text, [a, wq, sw], hifi=True)
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-2
+    # RMSNorm invariant: mean square of every row is 1 (up to bf16 rounding)
+    assert np.allclose((got[0].a.astype(np.float64) ** 2).mean(axis=1), 1.0, atol=2e-2)
