@@ -297,7 +297,9 @@ class Buffer:
     def from_host(client, raw, dtype, device=None):
         """`raw` is the C-ordered storage array in device (reversed-dims) layout."""
         device = device or client.default_device()
-        raw = np.ascontiguousarray(raw, dtype=_STORAGE[dtype])
+        raw = np.asarray(raw, dtype=_STORAGE[dtype])
+        if not raw.flags.c_contiguous:
+            raw = raw.copy(order="C")  # (np.ascontiguousarray would turn a 0-d array into 1-d)
         dims = (_i64 * raw.ndim)(*raw.shape)
         h = _call("ArrayFromHostBuffer", client.handle, raw.ctypes.data_as(_vp), PRIMITIVE_TYPE[dtype],
                   raw.ndim, dims, device.handle)
@@ -507,7 +509,7 @@ def to_rarray(x, dtype=None, client=None):
     if dtype is None:
         dtype = _NUMPY_DEFAULT[x.dtype]
     storage = encode(x, dtype)
-    raw = np.ascontiguousarray(storage.T)
+    raw = storage.T.copy(order="C")
     return ConcreteRArray(AsyncBuffer(Buffer.from_host(client, raw, dtype)), x.shape, dtype)
 
 
