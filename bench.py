@@ -1,0 +1,262 @@
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stencil] [--no-others] [--no-cpu]
+
+Prints ONE JSON line.  The headline workload is BASELINE.json configs[1]: the 3-D
+diffusion/advection stencil, Float64 512x512x256 with 3-cell halos, 10 timesteps
+traced into one module.  A "step" is one execution of that module (10 timesteps)
+with all inputs resident in HBM; `value` is achieved HBM GB/s counting only the
+algorithmic bytes (per timestep: read c,u,v,w + write c over the interior
+= 5*512*512*256*8 B).  `roofline` describes the dominant kernel (the fused stencil
+map kernel), timed with HIP events on the stream it runs on, inside the timed
+region.  `cpu_baseline` times the numpy oracle on a bounded sample of the same
+workload on the host cores.  `others` carries the remaining four configs
+(sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry.
+"""
+import argparse
+import importlib
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0
+PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f8": 5000.0}
+
+
+def _pkg():
+    d = os.path.join(ROOT, "reactant.jl_amd")
+    if "reactant_jl_amd" in sys.modules:
+        return sys.modules["reactant_jl_amd"]
+    spec = importlib.util.spec_from_file_location("reactant_jl_amd", os.path.join(d, "__init__.py"),
+                                                  submodule_search_locations=[d])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["reactant_jl_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def _upload(rx, client, arr, dt):
+    return rx.Buffer.from_host(client, arr, dt)
+
+
+def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
+    """Run warmup + steps executions.  `make_args(prev_results)` returns (buffers, donated).
+    Returns (seconds for the timed steps, per-launch mean ms over the timed steps, last results)."""
+    dev = client.default_device()
+    res = None
+    for _ in range(warmup):
+        bufs, don = make_args(res)
+        res, _ms = exe.execute_timed(bufs, don)
+    dev.synchronize()
+    nl = len(exe.launches())
+    acc = np.zeros(nl)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        bufs, don = make_args(res)
+        res, ms = exe.execute_timed(bufs, don)
+        acc += np.asarray(ms)
+    dev.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, acc / steps, res
+
+
+def _dominant(launches, mean_ms, kinds):
+    """Aggregate the launches whose kind is in `kinds`: (count, mean ms per launch, bytes/launch, flops/launch)."""
+    idx = [i for i, l in enumerate(launches) if l["kind"] in kinds]
+    if not idx:
+        return 0, 0.0, 0.0, 0.0
+    ms = float(np.mean([mean_ms[i] for i in idx]))
+    b = float(np.mean([launches[i]["algorithmic_bytes"] for i in idx]))
+    f = float(np.mean([launches[i]["flops"] for i in idx]))
+    return len(idx), ms, b, f
+
+
+# ----------------------------------------------------------------------------
+# workloads
+# ----------------------------------------------------------------------------
+def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=10):
+    H = 3
+    full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
+    c = np.zeros(full)
+    c[H:-H, H:-H, H:-H] = np.random.default_rng(0).uniform(0, 1, (nz, ny, nx))
+    text = P.stencil(nx, ny, nz, steps=nsteps)
+    exe = rx.xla_compile(client, text)
+    cb = _upload(rx, client, c, "f64")
+    vel = [_upload(rx, client, np.random.default_rng(s).uniform(-1, 1, full), "f64") for s in (1, 2, 3)]
+    del c
+
+    def make_args(prev):
+        cur = prev[0] if prev else cb
+        return [cur] + vel, [1, 0, 0, 0]   # the tracer field is donated, as `tf.aliasing_output` says
+
+    secs, mean_ms, _ = _time_steps(rx, client, exe, make_args, steps, warmup)
+    launches = exe.launches()
+    cells = nx * ny * nz
+    algo_step = 5.0 * cells * 8 * nsteps
+    nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil", "map"))
+    algo_launch = 5.0 * cells * 8
+    return {
+        "workload": "stencil f64 %dx%dx%d halo 3, %d timesteps per module" % (nx, ny, nz, nsteps),
+        "ms_per_step": 1e3 * secs / steps,
+        "value": algo_step / (secs / steps) / 1e9, "unit": "GB/s", "dtype": "f64",
+        "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"] if launches else None, "launches_per_step": nk,
+                     "kernel_ms": kms, "achieved": algo_launch / (kms * 1e-3) / 1e9 if kms else None,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": algo_launch / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None, "traffic": None},
+        "plan": exe.report(),
+    }
+
+
+def bench_sinsum(rx, client, P, steps, warmup, n=1 << 26):
+    x = np.random.default_rng(0).uniform(-np.pi, np.pi, n).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-np.pi, np.pi, n).astype(np.float32)
+    exe = rx.xla_compile(client, P.sinsum_add(n))
+    bx, by = _upload(rx, client, x, "f32"), _upload(rx, client, y, "f32")
+    secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: ([bx, by], [0, 0]), steps, warmup)
+    launches = exe.launches()
+    _, kms, _, _ = _dominant(launches, mean_ms, ("reduce",))
+    algo = 8.0 * n
+    got = float(rx.decode(res[0].to_host(), "f32"))
+    exact = float(np.sum(np.sin(x.astype(np.float64)) + y.astype(np.float64)))
+    return {"workload": "sinsum_add f32[2^26] x2 -> scalar", "ms_per_step": 1e3 * secs / steps,
+            "value": algo / (secs / steps) / 1e9, "unit": "GB/s", "dtype": "f32",
+            "check": {"got": got, "f64_reference": exact},
+            "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"], "kernel_ms": kms,
+                         "achieved": algo / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": algo / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None}}
+
+
+def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype):
+    launches = exe.launches()
+    dots = [i for i, l in enumerate(launches) if l["flops"] > 0]
+    flops = sum(launches[i]["flops"] for i in dots)
+    dms = sum(mean_ms[i] for i in dots)
+    big = max(dots, key=lambda i: launches[i]["flops"])
+    ach = launches[big]["flops"] / (mean_ms[big] * 1e-3) / 1e12
+    return {"workload": name, "ms_per_step": 1e3 * secs / steps, "value": flops / (secs / steps) / 1e12,
+            "unit": "TFLOP/s", "dtype": dtype,
+            "kernels": [{"kernel": l["kernel"], "kind": l["kind"], "ms": float(m)} for l, m in zip(launches, mean_ms)],
+            "dot_tflops_kernel_time_only": flops / (dms * 1e-3) / 1e12,
+            "roofline": {"bound": "mfma", "kernel": launches[big]["kernel"], "kernel_ms": float(mean_ms[big]),
+                         "achieved": ach, "peak": PEAK_TFLOPS[dtype_key], "unit": "TFLOP/s",
+                         "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": None}}
+
+
+def bench_gemm(rx, client, P, steps, warmup, n=4096):
+    A, B, C = [np.random.default_rng(s).normal(size=(n, n)).astype(np.float32) for s in (0, 1, 2)]
+    exe = rx.xla_compile(client, P.gemm(n, n, n))
+    bufs = [_upload(rx, client, a, "f32") for a in (A, B, C)]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
+    return _dot_entry("gemm f32 %d^3, alpha=1.5 beta=1.2" % n, exe, secs, steps, mean_ms, "f32", "f32")
+
+
+def bench_mlp(rx, client, P, steps, warmup, batch=8192, widths=(1024, 4096, 4096, 1024)):
+    exe = rx.xla_compile(client, P.mlp(batch, widths))
+    bufs = [_upload(rx, client, rx.encode(np.random.default_rng(0).normal(size=(batch, widths[0])).astype(np.float32), "bf16"), "bf16")]
+    for l in range(len(widths) - 1):
+        lim = np.sqrt(6.0 / (widths[l] + widths[l + 1]))
+        w = np.random.default_rng(1 + l).uniform(-lim, lim, size=(widths[l], widths[l + 1])).astype(np.float32)
+        b = (np.random.default_rng(4 + l).normal(size=(widths[l + 1],)) * 0.01).astype(np.float32)
+        bufs += [_upload(rx, client, rx.encode(w, "bf16"), "bf16"), _upload(rx, client, rx.encode(b, "bf16"), "bf16")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
+    return _dot_entry("mlp bf16 batch %d widths %s, bias+gelu, softmax" % (batch, "->".join(map(str, widths))), exe, secs,
+                      steps, mean_ms, "bf16", "bf16")
+
+
+def bench_fp8(rx, client, P, steps, warmup, n=8192):
+    exe = rx.xla_compile(client, P.fp8_linear(n, n, n))
+    a = rx.encode(np.random.default_rng(0).normal(size=(n, n)).astype(np.float32), "bf16")
+    w = np.random.default_rng(1).normal(size=(n, n)).astype(np.float32)
+    sw = np.float32(np.abs(w).max() / 448.0)
+    wq = rx.encode(w / sw, "f8E4M3FN")
+    bufs = [_upload(rx, client, a, "bf16"), _upload(rx, client, wq, "f8E4M3FN"), _upload(rx, client, np.asarray(sw), "f32")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
+    return _dot_entry("fp8 linear %d^3 e4m3 per-tensor scales, bf16 out + RMSNorm" % n, exe, secs, steps, mean_ms, "f8",
+                      "f8E4M3FN")
+
+
+def cpu_baseline_stencil(P, nx=256, ny=256, nz=128, nsteps=1):
+    """numpy oracle on a bounded sample (smaller grid, one timestep) of the same program."""
+    from oracle import stablehlo_interp as I
+    H = 3
+    full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
+    c = np.zeros(full)
+    c[H:-H, H:-H, H:-H] = np.random.default_rng(0).uniform(0, 1, (nz, ny, nx))
+    args = [I.Tensor(c, "f64")] + [I.Tensor(np.random.default_rng(s).uniform(-1, 1, full), "f64") for s in (1, 2, 3)]
+    funcs = I.parse_module(P.stencil(nx, ny, nz, steps=nsteps))
+    interp = I.Interpreter(funcs)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        interp.run(args)
+        reps += 1
+        if time.perf_counter() - t0 > 10.0 or reps >= 20:
+            break
+    secs = (time.perf_counter() - t0) / reps
+    algo = 5.0 * nx * ny * nz * 8 * nsteps
+    return {"value": algo / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "numpy oracle, %dx%dx%d interior, %d timestep, %d repetitions (%.2f s each)" % (nx, ny, nz, nsteps, reps, secs)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8"])
+    ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--small", action="store_true", help="reduced sizes (debugging only; not a valid result)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this backend runs on one GPU; --gpus %d is not supported (no collectives, no sharding)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    rx = _pkg()
+    P = importlib.import_module("reactant_jl_amd.programs")
+    client = rx.set_default_backend("gpu")
+    table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8}
+    small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
+             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024)}
+    kw = small[args.workload] if args.small else {}
+    main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
+    copy_ms = rx._call("RxCalibrationCopy", client.default_device().handle, 1 << 30, 10)
+    out = {
+        "metric": "achieved HBM GB/s (map/reduce/stencil) + dot_general TFLOP/s, % of peak, 1 GPU",
+        "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": main_res["dtype"], "data": "synthetic", "config": {"workload": main_res["workload"]},
+        "roofline": main_res["roofline"],
+        "copy_kernel_GBs": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9 if copy_ms > 0 else None,
+    }
+    if "check" in main_res:
+        out["check"] = main_res["check"]
+    if "kernels" in main_res:
+        out["kernels"] = main_res["kernels"]
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_stencil(P) if args.workload == "stencil" else None
+    if not args.no_others:
+        others = []
+        for name in ("sinsum", "gemm", "mlp", "fp8", "stencil"):
+            if name == args.workload:
+                continue
+            try:
+                r = table[name](rx, client, P, max(3, min(args.steps, 5)), 2, **(small[name] if args.small else {}))
+                r.pop("plan", None)
+                others.append(r)
+            except Exception as e:  # report, never hide
+                others.append({"workload": name, "error": str(e)[:400]})
+        out["others"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
