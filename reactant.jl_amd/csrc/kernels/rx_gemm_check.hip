@@ -1,0 +1,32 @@
+// Ahead-of-time build check of the GEMM skeletons: instantiates every MMA policy and
+// both operand orders with a plain store epilogue, so that device-code errors show up
+// when the library is built rather than when a module is compiled at run time.
+#include <hip/hip_runtime.h>
+#include "rx_preamble.h"
+#include "rx_gemm_kernels.h"
+
+template <typename OUT, int N>
+struct rx_check_epi {
+  OUT* out;
+  template <int NV>
+  __device__ __forceinline__ void operator()(const float (&acc)[NV], int m, int n) const {
+#pragma unroll
+    for (int l = 0; l < NV; ++l) out[(long long)m * N + n + l] = (OUT)acc[l];
+  }
+};
+
+#define RX_CHECK(NAME, MMA, BK, AKC, BKC)                                                                          \
+  extern "C" __global__ __launch_bounds__(256) void NAME(const MMA::elem* A, const MMA::elem* B, float* out) {      \
+    rx_check_epi<float, 512> epi{out};                                                                             \
+    rx_gemm_body<MMA, 128, 128, BK, 2, 2, AKC, BKC, 512, 512, 512, false, rx_check_epi<float, 512>>(A, B, epi);     \
+  }
+
+RX_CHECK(rx_check_f32_nn, rx_mma_f32, 16, true, false)
+RX_CHECK(rx_check_f32_tt, rx_mma_f32, 16, false, true)
+RX_CHECK(rx_check_bf16_nn, rx_mma_bf16, 64, true, false)
+RX_CHECK(rx_check_bf16_nt, rx_mma_bf16, 64, true, true)
+RX_CHECK(rx_check_bf16_tn, rx_mma_bf16, 64, false, false)
+RX_CHECK(rx_check_f16_nt, rx_mma_f16, 64, true, true)
+RX_CHECK(rx_check_f16_tn, rx_mma_f16, 64, false, false)
+RX_CHECK(rx_check_f8_nt, rx_mma_f8, 128, true, true)
+RX_CHECK(rx_check_f8_nn, rx_mma_f8, 128, true, false)

@@ -1,2 +1,283 @@
-// MFMA GEMM skeletons (filled in below)
+// MFMA GEMM skeleton for gfx950 (wave64).  One template covers f32, bf16, f16 and
+// f8E4M3FN operands with f32 accumulation, both storage orders of each operand,
+// an optional batch dimension, and an epilogue functor that the fusion code
+// generator writes for each dot_general group (alpha/beta, bias + gelu, dequant...).
+//
+//   D[m][n] = sum_k A(m,k) * B(k,n)
+//   A is stored [M][K] (A_KC, K contiguous) or [K][M];  B is stored [N][K] (B_KC) or [K][N].
+//
+// Tiling: a workgroup of WM x WN wavefronts computes a BM x BN tile; each wavefront
+// owns (BM/WM) x (BN/WN) as a grid of 32x32 MFMA tiles.  K is walked in steps of BK
+// through two LDS buffers: while the MFMAs consume buffer i, the global loads for
+// the next step are in flight in registers and are written to buffer i^1 afterwards
+// (one barrier per step).  LDS rows are padded so that the 16-byte fragment reads
+// of 16 consecutive rows fall into distinct banks.  An operand whose K is not the
+// contiguous dimension is kept in LDS as [k][m|n] and read with the LDS transpose
+// loads (ds_read_b64_tr_b16 / _b8), which hand each lane consecutive-k values.
+//
+// The MFMA is issued with the B fragment as the row operand, so a lane holds four
+// consecutive n for one m: the epilogue then works on 4-element vectors.
+//
+// The k index inside one MFMA is whatever the hardware assigns to (lane group,
+// register byte); A and B fragments are loaded with the same mapping, which is all
+// a contraction needs.
 #pragma once
+
+typedef float rx_f32x4 __attribute__((ext_vector_type(4)));
+typedef float rx_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 rx_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 rx_bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 rx_f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 rx_f16x4 __attribute__((ext_vector_type(4)));
+typedef short rx_i16x4 __attribute__((ext_vector_type(4)));
+typedef int rx_i32x8 __attribute__((ext_vector_type(8)));
+typedef int rx_i32x4 __attribute__((ext_vector_type(4)));
+typedef int rx_i32x2 __attribute__((ext_vector_type(2)));
+
+#define RX_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// ---------------------------------------------------------------------------
+// MMA policies.  KS = k extent consumed by one `mma` call; frag = per-lane operand.
+//   load_kc: operand tile in LDS as [o][k] (row stride `ld` elements), 32 rows from `row0`
+//   load_tr: operand tile in LDS as [k][o] (row stride `ld` elements), 32 columns from `col0`
+// ---------------------------------------------------------------------------
+struct rx_mma_f32 {
+  typedef float elem;
+  typedef rx_f32x4 frag;
+  static constexpr int KS = 8;
+  static constexpr int PAD = 4;   // elements of row padding in LDS
+  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
+    return *reinterpret_cast<const rx_f32x4*>(t + (row0 + (lane & 31)) * ld + kk + 4 * (lane >> 5));
+  }
+  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+    const elem* p = t + (kk + 4 * (lane >> 5)) * ld + col0 + (lane & 31);
+    frag f;
+    f[0] = p[0];
+    f[1] = p[ld];
+    f[2] = p[2 * ld];
+    f[3] = p[3 * ld];
+    return f;
+  }
+  RX_DEV void mma(rx_f32x16& c, const frag& rowop, const frag& colop) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c = __builtin_amdgcn_mfma_f32_32x32x2f32(rowop[j], colop[j], c, 0, 0, 0);
+  }
+};
+
+struct rx_mma_bf16 {
+  typedef rx_u16 elem;
+  typedef rx_bf16x8 frag;
+  static constexpr int KS = 16;
+  static constexpr int PAD = 8;
+  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
+    return *reinterpret_cast<const rx_bf16x8*>(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
+  }
+  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+    // 16-lane blocks: source lane i points at row k + i/4, columns 4*(i%4)..+3; after the
+    // transpose lane j of the block holds 4 consecutive k for column j.
+    const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
+    const elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
+    rx_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p));
+    rx_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p + 4 * ld));
+    struct { rx_i16x4 a, b; } both = {lo, hi};
+    return __builtin_bit_cast(rx_bf16x8, both);
+  }
+  RX_DEV void mma(rx_f32x16& c, const frag& rowop, const frag& colop) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rowop, colop, c, 0, 0, 0);
+  }
+};
+
+struct rx_mma_f16 {
+  typedef rx_u16 elem;
+  typedef rx_f16x8 frag;
+  static constexpr int KS = 16;
+  static constexpr int PAD = 8;
+  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
+    return *reinterpret_cast<const rx_f16x8*>(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
+  }
+  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+    const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
+    const elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
+    rx_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p));
+    rx_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p + 4 * ld));
+    struct { rx_i16x4 a, b; } both = {lo, hi};
+    return __builtin_bit_cast(rx_f16x8, both);
+  }
+  RX_DEV void mma(rx_f32x16& c, const frag& rowop, const frag& colop) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(rowop, colop, c, 0, 0, 0);
+  }
+};
+
+// f8E4M3FN x f8E4M3FN (OCP e4m3 on gfx950), 64 k per instruction
+struct rx_mma_f8 {
+  typedef rx_u8 elem;
+  typedef rx_i32x8 frag;
+  static constexpr int KS = 64;
+  static constexpr int PAD = 16;
+  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
+    const elem* p = t + (row0 + (lane & 31)) * ld + kk + 32 * (lane >> 5);
+    struct { rx_i32x4 a, b; } both = {*reinterpret_cast<const rx_i32x4*>(p), *reinterpret_cast<const rx_i32x4*>(p + 16)};
+    return __builtin_bit_cast(rx_i32x8, both);
+  }
+  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+    // 16-lane blocks: source lane i points at row k + i/2, columns 8*(i%2)..+7; after the
+    // transpose lane j of the block holds 8 consecutive k for column j.
+    const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
+    const elem* p = t + (kk + 32 * g + (i >> 1)) * ld + col0 + 16 * q + 8 * (i & 1);
+    struct { rx_i32x2 a, b, c, d; } all = {
+        __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p)),
+        __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p + 8 * ld)),
+        __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p + 16 * ld)),
+        __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p + 24 * ld))};
+    return __builtin_bit_cast(rx_i32x8, all);
+  }
+  RX_DEV void mma(rx_f32x16& c, const frag& rowop, const frag& colop) {
+    // formats 0/0 = e4m3 x e4m3; zero scale operands select the unscaled instruction
+    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(rowop, colop, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+// ---------------------------------------------------------------------------
+// cooperative copy of one operand tile: global (row-major, leading dim `gld`) ->
+// registers -> LDS (row stride `lld`).  ROWS x COLS elements, 16-byte vectors.
+// Rows / column vectors past the end of the matrix are clamped to the last valid
+// ones (their products are never stored).
+// ---------------------------------------------------------------------------
+template <typename E, int ROWS, int COLS, int NT>
+struct rx_tile_copy {
+  static constexpr int VE = 16 / (int)sizeof(E);           // elements per vector
+  static constexpr int VPR = COLS / VE;                    // vectors per row
+  static constexpr int TOTAL = ROWS * VPR;
+  static constexpr int PER = (TOTAL + NT - 1) / NT;        // vectors per thread
+  rx_u32x4 r[PER];
+
+  RX_MEM void load(const E* __restrict__ g, long long gld, int row0, int col0, int nrows, int ncols, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int v = tid + i * NT;
+      if (TOTAL % NT == 0 || v < TOTAL) {
+        int rr = row0 + v / VPR;
+        int cc = col0 + (v % VPR) * VE;
+        rr = rr < nrows ? rr : nrows - 1;
+        cc = cc + VE <= ncols ? cc : ncols - VE;
+        r[i] = *reinterpret_cast<const rx_u32x4*>(g + (long long)rr * gld + cc);
+      }
+    }
+  }
+  RX_MEM void store(E* lds, int lld, int tid) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int v = tid + i * NT;
+      if (TOTAL % NT == 0 || v < TOTAL) *reinterpret_cast<rx_u32x4*>(lds + (v / VPR) * lld + (v % VPR) * VE) = r[i];
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// the kernel body
+// ---------------------------------------------------------------------------
+template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, bool BATCHED, class Epi>
+RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
+  typedef typename MMA::elem E;
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;   // 32x32 tiles per wavefront
+  constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BK : BM;
+  constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BK : BN;
+  constexpr int A_LD = A_COLS + MMA::PAD, B_LD = B_COLS + MMA::PAD;
+  constexpr int A_SZ = A_ROWS * A_LD, B_SZ = B_ROWS * B_LD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
+  E* lds = reinterpret_cast<E*>(rx_smem);
+  E* ldsA[2] = {lds, lds + A_SZ + B_SZ};
+  E* ldsB[2] = {lds + A_SZ, lds + 2 * A_SZ + B_SZ};
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  // Tile order: consecutive workgroups share the same A rows (n fastest) inside groups of
+  // 8 row-tiles, so the operand tiles of concurrently running workgroups stay in L2.
+  constexpr int GM = (M + BM - 1) / BM, GN = (N + BN - 1) / BN;
+  int bm, bn;
+  {
+    const int bid = blockIdx.x;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * GN;
+    const int grp = bid / per_group;
+    const int first = grp * GROUP;
+    const int rows = (GM - first) < GROUP ? (GM - first) : GROUP;
+    const int in = bid % per_group;
+    bm = first + in % rows;
+    bn = in / rows;
+  }
+  const int m0 = bm * BM, n0 = bn * BN;
+  const long long batch = BATCHED ? blockIdx.y : 0;
+  const E* Ab = A + batch * (long long)M * K;
+  const E* Bb = B + batch * (long long)N * K;
+  constexpr long long A_GLD = A_KC ? K : M, B_GLD = B_KC ? K : N;
+
+  rx_f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  rx_tile_copy<E, A_ROWS, A_COLS, NT> ca;
+  rx_tile_copy<E, B_ROWS, B_COLS, NT> cb;
+  auto gload = [&](int k0) {
+    if (A_KC) ca.load(Ab, A_GLD, m0, k0, M, K, tid); else ca.load(Ab, A_GLD, k0, m0, K, M, tid);
+    if (B_KC) cb.load(Bb, B_GLD, n0, k0, N, K, tid); else cb.load(Bb, B_GLD, k0, n0, K, N, tid);
+  };
+  gload(0);
+  ca.store(ldsA[0], A_LD, tid);
+  cb.store(ldsB[0], B_LD, tid);
+  __syncthreads();
+
+  constexpr int KT = K / BK;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < KT) gload((kt + 1) * BK);
+    const E* sa = ldsA[cur];
+    const E* sb = ldsB[cur];
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += MMA::KS) {
+      typename MMA::frag fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int o = wm * (BM / WM) + 32 * i;
+        fa[i] = A_KC ? MMA::load_kc(sa, A_LD, o, kk, lane) : MMA::load_tr(sa, A_LD, o, kk, lane);
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int o = wn * (BN / WN) + 32 * j;
+        fb[j] = B_KC ? MMA::load_kc(sb, B_LD, o, kk, lane) : MMA::load_tr(sb, B_LD, o, kk, lane);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) MMA::mma(acc[i][j], fb[j], fa[i]);
+    }
+    if (kt + 1 < KT) {
+      ca.store(ldsA[cur ^ 1], A_LD, tid);
+      cb.store(ldsB[cur ^ 1], B_LD, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds D[n = 8*(r/4) + 4*(lane/32) + r%4][m = lane%32] of each 32x32 tile
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * (BM / WM) + 32 * i + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wn * (BN / WN) + 32 * j + 4 * (lane >> 5);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int n = nb + 8 * rg;
+        if (m < M && n < N) {
+          const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
+          if constexpr (BATCHED) epi(v, (int)batch, m, n); else epi(v, m, n);
+        }
+      }
+    }
+  }
+}

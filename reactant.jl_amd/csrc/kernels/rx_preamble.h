@@ -21,6 +21,50 @@ struct __attribute__((aligned(sizeof(T) * N))) rx_vec {
 };
 
 // ---------------------------------------------------------------------------
+// vector loads / stores.  The non-temporal forms mark data that is touched once
+// (streamed inputs, map outputs) so that it does not displace reusable lines.
+// ---------------------------------------------------------------------------
+typedef rx_u32 rx_u32x4 __attribute__((ext_vector_type(4)));
+typedef rx_u32 rx_u32x2 __attribute__((ext_vector_type(2)));
+
+template <typename V, typename T>
+static __device__ __forceinline__ V rx_load(const T* p) {
+  return *reinterpret_cast<const V*>(p);
+}
+template <typename V, typename T>
+static __device__ __forceinline__ V rx_load_nt(const T* p) {
+  if constexpr (sizeof(V) == 16) {
+    return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const rx_u32x4*>(p)));
+  } else if constexpr (sizeof(V) == 8) {
+    return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const rx_u32x2*>(p)));
+  } else if constexpr (sizeof(V) == 4) {
+    return __builtin_bit_cast(V, __builtin_nontemporal_load(reinterpret_cast<const rx_u32*>(p)));
+  } else {
+    return *reinterpret_cast<const V*>(p);
+  }
+}
+template <typename T, typename V>
+static __device__ __forceinline__ void rx_store(T* p, const V& v) {
+  *reinterpret_cast<V*>(p) = v;
+}
+template <typename T, typename V>
+static __device__ __forceinline__ void rx_store_nt(T* p, const V& v) {
+  if constexpr (sizeof(V) == 16) {
+    __builtin_nontemporal_store(__builtin_bit_cast(rx_u32x4, v), reinterpret_cast<rx_u32x4*>(p));
+  } else if constexpr (sizeof(V) == 8) {
+    __builtin_nontemporal_store(__builtin_bit_cast(rx_u32x2, v), reinterpret_cast<rx_u32x2*>(p));
+  } else if constexpr (sizeof(V) == 4) {
+    __builtin_nontemporal_store(__builtin_bit_cast(rx_u32, v), reinterpret_cast<rx_u32*>(p));
+  } else {
+    *reinterpret_cast<V*>(p) = v;
+  }
+}
+template <typename I>
+static __device__ __forceinline__ I rx_clamp_idx(I i, I hi) {
+  return i < 0 ? (I)0 : (i > hi ? hi : i);
+}
+
+// ---------------------------------------------------------------------------
 // bit casts
 // ---------------------------------------------------------------------------
 RX_DEV rx_u32 rx_f2u(float f) { return __builtin_bit_cast(rx_u32, f); }

@@ -208,7 +208,9 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_SLAB_MIN_NUMEL")) o.slab_min_numel = atoll(e);
   if (const char* e = getenv("RX_MFMA")) o.mfma = atoi(e) != 0;
   if (const char* e = getenv("RX_ROW_FUSION")) o.row_fusion = atoi(e) != 0;
-  if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;
+  if (const char* e = getenv("RX_SHIFTED_VEC")) o.shifted_vector_loads = atoi(e) != 0;
+  if (const char* e = getenv("RX_NT_LOADS")) o.nt_loads = atoi(e) != 0;
+  if (const char* e = getenv("RX_NT_STORES")) o.nt_stores = atoi(e) != 0;
   return o;
 }
 
@@ -630,6 +632,11 @@ RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, siz
       for (auto& L : ex->plan.launches) {
         hipFunction_t f;
         HIP_CHECK(hipModuleGetFunction(&f, ex->module, L.kernel.c_str()));
+        if (L.lds_bytes > 48 * 1024) {
+          // more dynamic LDS than the default limit: gfx950 has 160 KB per workgroup
+          hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(f), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.lds_bytes);
+          if (e != hipSuccess) (void)hipGetLastError();
+        }
         ex->fns.push_back(f);
       }
     }

@@ -168,12 +168,34 @@ std::string Emitter::emit_load(int node, const Index& ix) {
   }
   loads.push_back(rec);
   bool direct = allow_direct_ && rec.affine && dims == root_dims_;
+  bool shifted = false;
   if (direct)
-    for (auto o : rec.off) direct = direct && o == 0;
+    for (auto o : rec.off) shifted = shifted || o != 0;
+  if (shifted && !(allow_shifted && vec > 1)) direct = false;
   std::string raw;
   if (direct) {
-    direct_inputs.insert(slot);
-    raw = direct_expr(slot);
+    // element (l + o) of the row, o = offset in the minor dimension; outer offsets move whole vectors
+    const int nd = (int)dims.size();
+    int64_t stride = 1, delta = 0;
+    for (int d = nd - 1; d >= 0; --d) {
+      if (d < nd - 1) delta += rec.off[d] * stride;
+      stride *= dims[d];
+    }
+    const int64_t o = rec.off[nd - 1];
+    int64_t q = o >= 0 ? o / vec : -((-o + vec - 1) / vec);
+    const int64_t r = o - q * vec;
+    const int64_t D0 = delta + q * vec;
+    direct_vecs.insert({slot, D0});
+    std::string A = direct_expr(slot, D0);
+    if (r == 0) {
+      raw = A + ".v[l]";
+    } else {
+      direct_vecs.insert({slot, D0 + vec});
+      std::string B = direct_expr(slot, D0 + vec);
+      const std::string lr = "(l + " + std::to_string(r) + ")";
+      raw = "(" + lr + " < " + std::to_string(vec) + " ? " + A + ".v[" + lr + " % " + std::to_string(vec) + "] : " + B + ".v[" + lr + " % " +
+            std::to_string(vec) + "])";
+    }
   } else {
     raw = "in" + std::to_string(slot) + "[" + (dims.empty() ? std::string("0") : linear(ix, dims)) + "]";
   }

@@ -47,9 +47,13 @@ class Emitter {
     root_vars_ = vars;
     allow_direct_ = allow_direct;
   }
-  std::set<int> direct_inputs;               // inputs that were read through the vector preload
-  // expression for lane `l` of the preloaded vector of input slot s
-  std::function<std::string(int slot)> direct_expr;
+  // Vector preloads.  (slot, D): the aligned vector of input `slot` at element offset D from the
+  // vector of the output element; D != 0 arises from loads at constant offsets (stencils) and is
+  // only produced when `allow_shifted` is set.  `direct_expr(slot, D)` names the preloaded vector.
+  std::set<std::pair<int, int64_t>> direct_vecs;
+  std::function<std::string(int slot, int64_t D)> direct_expr;
+  bool allow_shifted = false;
+  int vec = 1;
 
   std::string emit(int node, const Index& ix);
   std::string take_code() { std::string s = out_.str(); out_.str(""); return s; }

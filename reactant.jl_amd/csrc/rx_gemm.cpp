@@ -1,9 +1,62 @@
 #include "rx_gemm.h"
 
+#include <cstdlib>
+#include <sstream>
+
 namespace rx {
 
-GemmChoice choose_gemm(DT, DT, DT, int64_t, int64_t, int64_t, int64_t, bool, bool) { return GemmChoice(); }
+GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc) {
+  GemmChoice c;
+  if (a != b) return c;
+  std::string mma;
+  int esize = 0, bk = 0;
+  if (a == DT::F32 && out == DT::F32) { mma = "rx_mma_f32"; c.kind = "gemm_f32"; esize = 4; bk = 16; }
+  else if (a == DT::BF16 && (out == DT::BF16 || out == DT::F32)) { mma = "rx_mma_bf16"; c.kind = "gemm_bf16"; esize = 2; bk = 64; }
+  else if (a == DT::F16 && (out == DT::F16 || out == DT::F32)) { mma = "rx_mma_f16"; c.kind = "gemm_f16"; esize = 2; bk = 64; }
+  else if (a == DT::F8E4M3FN && (out == DT::F32 || out == DT::BF16 || out == DT::F16)) { mma = "rx_mma_f8"; c.kind = "gemm_f8"; esize = 1; bk = 128; }
+  else return c;
+  const int ve = 16 / esize;
+  if (K % bk != 0 || K < bk) return c;
+  if (N % 4 != 0) return c;
+  if (!a_kc && M % ve != 0) return c;
+  if (!b_kc && N % ve != 0) return c;
+  if (M < 1 || N < 4) return c;
+  if (M * N < 64 * 64) return c;  // tiny products: the scalar loop is as good
+  if (M >= ((int64_t)1 << 30) || N >= ((int64_t)1 << 30) || K >= ((int64_t)1 << 30)) return c;
+  int BM = 128, BN = 128, WM = 2, WN = 2;
+  if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
+    int v[4];
+    if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
+  }
+  if (const char* e = getenv("RX_GEMM_BK")) bk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : bk;
+  const int pad = a == DT::F32 ? 4 : (esize == 2 ? 8 : 16);
+  const int64_t a_sz = a_kc ? (int64_t)BM * (bk + pad) : (int64_t)bk * (BM + pad);
+  const int64_t b_sz = b_kc ? (int64_t)BN * (bk + pad) : (int64_t)bk * (BN + pad);
+  c.lds_bytes = (unsigned)(2 * (a_sz + b_sz) * esize);
+  if (c.lds_bytes > 160 * 1024) return c;
+  c.block = WM * WN * 64;
+  const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
+  c.grid[0] = (unsigned)(gm * gn);
+  c.grid[1] = (unsigned)batch;
+  std::ostringstream t;
+  t << mma << ", " << BM << ", " << BN << ", " << bk << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false")
+    << ", " << M << ", " << N << ", " << K;
+  c.targs = t.str();
+  c.skeleton = "rx_gemm_body";
+  c.stype_a = mma + "::elem";
+  c.ok = true;
+  return c;
+}
 
-std::string gemm_instance(const GemmChoice&, const std::string&, const std::string&, const std::string&) { return ""; }
+std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched) {
+  std::ostringstream o;
+  o << "// dot_general on MFMA: " << c.kind << " <" << c.targs << ">\n";
+  o << "extern \"C\" __global__ __launch_bounds__(" << c.block << ") void " << kbase << "_gemm(const " << c.stype_a << "* __restrict__ A, const " << c.stype_a
+    << "* __restrict__ B" << epi_params << ") {\n";
+  o << "  " << epi_ctor << "\n";
+  o << "  " << c.skeleton << "<" << c.targs << ", " << (batched ? "true" : "false") << ", " << kbase << "_epi>(A, B, epi);\n";
+  o << "}\n\n";
+  return o.str();
+}
 
 }  // namespace rx

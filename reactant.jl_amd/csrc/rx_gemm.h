@@ -22,6 +22,6 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
 
 // Text of the `extern "C"` kernel <kbase>_gemm that runs the skeleton with epilogue type <kbase>_epi.
 // `epi_params` is the tail of the parameter list (epilogue operands and out0), `epi_ctor` builds `epi`.
-std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor);
+std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched);
 
 }  // namespace rx

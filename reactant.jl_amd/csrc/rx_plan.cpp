@@ -393,6 +393,11 @@ struct Planner {
     return b;
   }
 
+  static std::string vec_name(int slot, int64_t D) {
+    if (D == 0) return "d" + std::to_string(slot);
+    return "d" + std::to_string(slot) + (D < 0 ? "_m" + std::to_string(-D) : "_p" + std::to_string(D));
+  }
+
   static int pick_vec(const TType& t) {
     if (t.rank() == 0) return 1;
     int v = std::max(1, 16 / info(t.dt).size);
@@ -468,7 +473,9 @@ struct Planner {
     std::vector<std::string> vars;
     for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
     em.set_root(dims, vars, vec > 1);
-    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.vec = vec;
+    em.allow_shifted = opt.shifted_vector_loads;
+    em.direct_expr = vec_name;
     em.indent = 4;
     Index ix = root_index(dims);
     // evaluate the root op itself (it is materialized, so bypass the input test by emitting its op)
@@ -524,10 +531,28 @@ struct Planner {
       }
       o << "  const " << it << " lin0 = i0 * " << plane << (em.idx64 ? "LL" : "") << " + pe;\n";
     }
-    for (int slot : em.direct_inputs) {
-      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
-      o << "  const rx_vec<" << st << ", " << vec << "> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot
-        << " + lin0);\n";
+    {
+      // inputs read once, at the output's own position, stream through (non-temporal hint);
+      // inputs read at several offsets stay cacheable
+      std::map<int, int> nvec, nload;
+      for (auto& sd : em.direct_vecs) nvec[sd.first]++;
+      for (auto& l : em.loads) nload[em.slot_of(l.node)]++;
+      for (auto& sd : em.direct_vecs) {
+        const int slot = sd.first;
+        const int64_t D = sd.second;
+        const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+        const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+        std::string addr = "lin0";
+        if (D != 0) {
+          // neighbours of elements on the boundary fall outside the array; their values are never
+          // used (the pad / update-slice guard selects them away), so the address is clamped
+          const std::string sfx = em.idx64 ? "LL" : "";
+          addr = "rx_clamp_idx<" + it + ">(lin0 + " + std::to_string(D) + sfx + ", " + std::to_string(numel - vec) + sfx + ")";
+        }
+        const bool stream = opt.nt_loads && nvec[slot] == 1 && D == 0 && nload[slot] == 1;
+        o << "  const " << vt << " " << vec_name(slot, D) << " = " << (stream ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + " << addr
+          << ");\n";
+      }
     }
     const std::string ost = info(rn.ty.dt).stype;
     if (n == 0) {
@@ -538,7 +563,7 @@ struct Planner {
       o << "    const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
       o << body;
       o << "    res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n  }\n";
-      o << "  *reinterpret_cast<rx_vec<" << ost << ", " << vec << ">*>(out0 + lin0) = res;\n";
+      o << "  " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
     }
     o << "}\n\n";
     const std::string kb_final = finalize(o.str());
@@ -594,7 +619,8 @@ struct Planner {
     std::vector<std::string> vars;
     for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
     em.set_root(dims, vars, vec > 1);
-    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.vec = vec;
+    em.direct_expr = vec_name;
     em.indent = 10;
     std::string val = em.emit(rn.in[0], root_index(dims));
     std::string body = em.take_code();
@@ -611,9 +637,10 @@ struct Planner {
     o << "      if (vid < " << nv << ") {\n";
     decode_index(o, it, "vid", dims, vec, "        ");
     o << "        const " << it << " lin0 = vid * " << vec << ";\n";
-    for (int slot : em.direct_inputs) {
-      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
-      o << "        const rx_vec<" << st << ", " << vec << "> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot
+    for (auto& sd : em.direct_vecs) {
+      const int slot = sd.first;
+      const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">";
+      o << "        const " << vt << " " << vec_name(slot, 0) << " = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot
         << " + lin0);\n";
     }
     o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
@@ -764,7 +791,8 @@ struct Planner {
     std::vector<std::string> vars;
     for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
     em.set_root(full.dims, vars, true);
-    em.direct_expr = [&](int slot) { return cache ? "c" + std::to_string(slot) + "[itv].v[l]" : "d" + std::to_string(slot) + ".v[l]"; };
+    em.vec = vec;
+    em.direct_expr = [&](int slot, int64_t) { return cache ? "c" + std::to_string(slot) + "[itv]" : "d" + std::to_string(slot); };
     Index ix = root_index(full.dims);
 
     struct PhaseCode { int node; std::string body, val; };
@@ -837,7 +865,8 @@ struct Planner {
     };
     // preload of direct inputs
     auto preload = [&](std::ostringstream& s, bool into_cache) {
-      for (int slot : em.direct_inputs) {
+      for (auto& sd : em.direct_vecs) {
+        const int slot = sd.first;
         const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
         if (into_cache)
           s << "      c" << slot << "[itv] = *reinterpret_cast<const rx_vec<" << st << ", " << vec << ">*>(in" << slot << " + lin0);\n";
@@ -847,11 +876,12 @@ struct Planner {
       }
     };
     if (cache) {
-      for (int slot : em.direct_inputs) {
+      for (auto& sd : em.direct_vecs) {
+        const int slot = sd.first;
         const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
         o << "  rx_vec<" << st << ", " << vec << "> c" << slot << "[" << iters << "];\n";
       }
-      if (!em.direct_inputs.empty()) {
+      if (!em.direct_vecs.empty()) {
         loop_open(o);
         preload(o, true);
         o << "    }\n  }\n";
@@ -994,7 +1024,8 @@ struct Planner {
     std::vector<std::string> vars;
     for (int k = 0; k < n; ++k) vars.push_back("i" + std::to_string(k));
     em.set_root(rn.ty.dims, vars, n > 0);
-    em.direct_expr = [&](int slot) { return "d" + std::to_string(slot) + ".v[l]"; };
+    em.vec = 4;  // only unshifted vectors are used here; the width is the template parameter NV
+    em.direct_expr = vec_name;
     em.indent = 6;
     const std::string DCT = info(d.ty.dt).ctype;
     em.bound[dot] = "accv";
@@ -1019,7 +1050,8 @@ struct Planner {
       if (n > 0) rix[n - 1].var = "i" + std::to_string(n - 1) + "b";
       o << "    const " << it << " lin0 = " << (n ? em.linear(rix, rn.ty.dims) : std::string("0")) << ";\n";
     }
-    for (int slot : em.direct_inputs) {
+    for (auto& sd : em.direct_vecs) {
+      const int slot = sd.first;
       const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
       o << "    const rx_vec<" << st << ", NV> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", NV>*>(in" << slot << " + lin0);\n";
     }
@@ -1059,7 +1091,7 @@ struct Planner {
     };
 
     if (gc.ok) {
-      o << gemm_instance(gc, kbase, epi_params(), epi_ctor());
+      o << gemm_instance(gc, kbase, epi_params(), epi_ctor(), d.a0.size() == 1);
       L.kernel = kbase + "_gemm";
       L.kind = gc.kind;
       L.grid[0] = gc.grid[0]; L.grid[1] = gc.grid[1]; L.grid[2] = gc.grid[2];

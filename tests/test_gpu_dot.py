@@ -1,0 +1,78 @@
+"""dot_general on the MFMA skeletons: every operand order, element type and the
+batched form, against the f64-accumulating oracle.  Shapes are chosen so that the
+MFMA path is taken (the plan's launch kind is asserted), including tile edges."""
+import numpy as np
+import pytest
+
+from _harness import gpu_run, oracle_run, max_rel_to_scale
+from oracle import stablehlo_interp as I
+
+pytestmark = pytest.mark.gpu
+
+
+def _tt(shape, dt):
+    return "tensor<" + "x".join([str(s) for s in shape] + [dt]) + ">"
+
+
+def dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch=0):
+    bs = [batch] if batch else []
+    a_shape = bs + ([M, K] if a_kc else [K, M])
+    b_shape = bs + ([N, K] if b_kc else [K, N])
+    nb = len(bs)
+    lc = nb + (1 if a_kc else 0)
+    rc = nb + (1 if b_kc else 0)
+    battr = "batching_dims = [0] x [0], " if batch else ""
+    ta, tb, to = _tt(a_shape, dt), _tt(b_shape, dt), _tt(bs + [M, N], out_dt)
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%0 = stablehlo.dot_general %%arg0, %%arg1, %scontracting_dims = [%d] x [%d], "
+            "precision = [DEFAULT, DEFAULT] : (%s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
+            % (ta, tb, to, battr, lc, rc, ta, tb, to, to)), a_shape, b_shape
+
+
+CASES = []
+for a_kc in (True, False):
+    for b_kc in (True, False):
+        CASES += [("f32", "f32", 128, 128, 64, a_kc, b_kc, 0), ("f32", "f32", 200, 136, 48, a_kc, b_kc, 0),
+                  ("bf16", "bf16", 128, 256, 128, a_kc, b_kc, 0), ("bf16", "f32", 136, 200, 64, a_kc, b_kc, 0),
+                  ("f16", "f16", 128, 128, 64, a_kc, b_kc, 0),
+                  ("f8E4M3FN", "f32", 128, 128, 256, a_kc, b_kc, 0), ("f8E4M3FN", "f32", 144, 208, 128, a_kc, b_kc, 0)]
+CASES += [("f32", "f32", 128, 128, 32, True, False, 3), ("bf16", "bf16", 128, 128, 64, True, True, 2),
+          ("f8E4M3FN", "f32", 128, 128, 128, True, True, 2), ("bf16", "bf16", 256, 384, 512, True, False, 0)]
+
+
+@pytest.mark.parametrize("dt,out_dt,M,N,K,a_kc,b_kc,batch", CASES)
+def test_dot_general_mfma(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
+    text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch)
+    a = I.tensor(np.random.default_rng(0).normal(size=a_shape), dt)
+    b = I.tensor(np.random.default_rng(1).normal(size=b_shape), dt)
+    got, exe = gpu_run(rx, client, text, [a, b])
+    kinds = [l["kind"] for l in exe.launches()]
+    assert kinds == ["gemm_" + {"f32": "f32", "bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8"}[dt]], kinds
+    ref = oracle_run(text, [a, b], hifi=True)
+    err = max_rel_to_scale(got[0].a, ref[0].a)
+    if out_dt in ("bf16", "f16"):
+        assert err <= 1e-2
+    else:
+        assert err <= 1e-5 * np.sqrt(K)
+
+
+def test_int_dot_general_reference_vectors(rx, client):
+    """Known answers of the reference's own test (test/core/ops.jl:249-278)."""
+    t = ("module {\n  func.func @main(%arg0: tensor<4xi32>, %arg1: tensor<4xi32>) -> tensor<i32> {\n"
+         "    %0 = stablehlo.dot_general %arg0, %arg1, contracting_dims = [0] x [0] : (tensor<4xi32>, tensor<4xi32>) -> tensor<i32>\n"
+         "    return %0 : tensor<i32>\n  }\n}\n")
+    a = I.Tensor(np.array([1, 2, 3, 4], dtype=np.int32), "i32")
+    b = I.Tensor(np.array([5, 6, -7, -8], dtype=np.int32), "i32")
+    got, _ = gpu_run(rx, client, t, [a, b])
+    assert int(got[0].a) == -36
+    # Int32[1 2; 3 4]' * Int32[5 6; -7 -8] == [-16 -18; -18 -20]; Julia matrices arrive transposed
+    t2 = ("module {\n  func.func @main(%arg0: tensor<2x2xi32>, %arg1: tensor<2x2xi32>) -> tensor<2x2xi32> {\n"
+          "    %0 = stablehlo.dot_general %arg0, %arg1, contracting_dims = [1] x [1] : (tensor<2x2xi32>, tensor<2x2xi32>) -> tensor<2x2xi32>\n"
+          "    return %0 : tensor<2x2xi32>\n  }\n}\n")
+    A = np.array([[1, 2], [3, 4]], dtype=np.int32)
+    B = np.array([[5, 6], [-7, -8]], dtype=np.int32)
+    # Julia f1(x, y) contracts dim 1 of both: result[i, j] = sum_k A[k, i] * B[k, j]; raw buffers are A.T, B.T
+    # and raw dim 1 is Julia dim 1.
+    got, _ = gpu_run(rx, client, t2, [I.Tensor(A.T.copy(), "i32"), I.Tensor(B.T.copy(), "i32")])
+    assert np.array_equal(got[0].a, A.T @ B)
+    assert np.array_equal(A.T @ B, np.array([[-16, -18], [-18, -20]]))
