@@ -208,6 +208,8 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_SLAB_MIN_NUMEL")) o.slab_min_numel = atoll(e);
   if (const char* e = getenv("RX_MFMA")) o.mfma = atoi(e) != 0;
   if (const char* e = getenv("RX_ROW_FUSION")) o.row_fusion = atoi(e) != 0;
+  if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;
+  if (const char* e = getenv("RX_LDS_TILE")) { int v[3]; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) == 3) { o.lds_tile[0] = v[0]; o.lds_tile[1] = v[1]; o.lds_tile[2] = v[2]; } }
   if (const char* e = getenv("RX_SHIFTED_VEC")) o.shifted_vector_loads = atoi(e) != 0;
   if (const char* e = getenv("RX_NT_LOADS")) o.nt_loads = atoi(e) != 0;
   if (const char* e = getenv("RX_NT_STORES")) o.nt_stores = atoi(e) != 0;

@@ -173,7 +173,10 @@ std::string Emitter::emit_load(int node, const Index& ix) {
     for (auto o : rec.off) shifted = shifted || o != 0;
   if (shifted && !(allow_shifted && vec > 1)) direct = false;
   std::string raw;
-  if (direct) {
+  std::string hooked;
+  if (tile_hook && rec.affine && dims == root_dims_ && tile_hook(slot, rec.off, &hooked)) {
+    raw = hooked;
+  } else if (direct) {
     // element (l + o) of the row, o = offset in the minor dimension; outer offsets move whole vectors
     const int nd = (int)dims.size();
     int64_t stride = 1, delta = 0;

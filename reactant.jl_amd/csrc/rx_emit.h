@@ -54,6 +54,9 @@ class Emitter {
   std::function<std::string(int slot, int64_t D)> direct_expr;
   bool allow_shifted = false;
   int vec = 1;
+  // Loads of an input at root-index + constant offsets can be redirected (to an LDS halo tile):
+  // the hook returns true and the expression to read instead of global memory.
+  std::function<bool(int slot, const std::vector<int64_t>& off, std::string* expr)> tile_hook;
 
   std::string emit(int node, const Index& ix);
   std::string take_code() { std::string s = out_.str(); out_.str(""); return s; }

@@ -457,8 +457,194 @@ struct Planner {
     return out;
   }
 
+  // ------------------------------------------------------------------ stencil maps through LDS halo tiles
+  // A rank-3 map that reads some input at several constant offsets (a stencil): the workgroup
+  // owns a TZ x TY x TX block of outputs, loads that input's block plus halo into LDS once with
+  // aligned 16-byte loads, and every neighbour access becomes an LDS read.  Inputs read only at
+  // the output's own position are still streamed from global memory with vector loads.
+  bool emit_map_lds(int root) {
+    const Node& rn = g.nodes[root];
+    const auto& dims = rn.ty.dims;
+    if (!opt.lds_stencil || rn.ty.rank() != 3) return false;
+    const int vec = pick_vec(rn.ty);
+    const int64_t numel = rn.ty.numel();
+    if (numel < opt.slab_min_numel || vec < 2) return false;
+    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
+    auto make_emitter = [&](Emitter& em) {
+      em.idx64 = needs64(cone_nodes(root));
+      em.set_root(dims, {"i0", "i1", "i2"}, true);
+      em.vec = vec;
+      em.allow_shifted = false;
+      em.direct_expr = vec_name;
+      em.indent = 8;
+    };
+    // pass 1: find the stencil inputs and their halos
+    Emitter probe(g, [&](int x) { return x != root && mat[x]; });
+    make_emitter(probe);
+    probe.emit(root, root_index(dims));
+    struct Halo { int64_t lo[3] = {0, 0, 0}, hi[3] = {0, 0, 0}; int count = 0; bool ok = true; };
+    std::map<int, Halo> halos;  // keyed by node
+    std::map<int, std::set<std::vector<int64_t>>> offs;
+    for (auto& l : probe.loads) {
+      const Node& ln = g.nodes[l.node];
+      if (ln.ty.dims != dims) continue;
+      if (!l.affine) { halos[l.node].ok = false; continue; }
+      offs[l.node].insert(l.off);
+    }
+    std::vector<int> staged;
+    for (auto& kv : offs) {
+      if (kv.second.size() < 3 || !halos[kv.first].ok) continue;
+      Halo& h = halos[kv.first];
+      for (auto& o : kv.second)
+        for (int d = 0; d < 3; ++d) { h.lo[d] = std::max<int64_t>(h.lo[d], -o[d]); h.hi[d] = std::max<int64_t>(h.hi[d], o[d]); }
+      if (h.lo[0] > 4 || h.hi[0] > 4 || h.lo[1] > 4 || h.hi[1] > 4 || h.lo[2] > 8 || h.hi[2] > 8) continue;
+      const int es = info(g.nodes[kv.first].ty.dt).size;
+      if (es != 4 && es != 8) continue;
+      if (info(g.nodes[kv.first].ty.dt).size != info(rn.ty.dt).size) continue;  // same vector width as the output
+      staged.push_back(kv.first);
+    }
+    if (staged.empty()) return false;
+    int TZ = opt.lds_tile[0], TY = opt.lds_tile[1], TX = opt.lds_tile[2];
+    if (TX % vec || (TX / vec) * TY != kBlock) return false;
+    const int TXV = TX / vec;
+    // LDS geometry per staged input
+    struct Geo { int64_t pz, py, lx, hxl; int64_t bytes; };
+    std::map<int, Geo> geo;
+    int64_t lds_total = 0;
+    for (int s : staged) {
+      Halo& h = halos[s];
+      Geo ge;
+      ge.hxl = (h.lo[2] + vec - 1) / vec * vec;
+      const int64_t hxh = (h.hi[2] + vec - 1) / vec * vec;
+      ge.pz = TZ + h.lo[0] + h.hi[0];
+      ge.py = TY + h.lo[1] + h.hi[1];
+      ge.lx = TX + ge.hxl + hxh;
+      ge.bytes = ge.pz * ge.py * ge.lx * info(g.nodes[s].ty.dt).size;
+      geo[s] = ge;
+      lds_total += ge.bytes;
+    }
+    if (lds_total > 64 * 1024) return false;
+
+    // pass 2: emit with the staged inputs redirected to LDS
+    Emitter em(g, [&](int x) { return x != root && mat[x]; });
+    make_emitter(em);
+    em.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+      const int node = em.inputs[slot];
+      auto it = geo.find(node);
+      if (it == geo.end()) return false;
+      const Halo& h = halos[node];
+      const Geo& ge = it->second;
+      // position inside the tile: (lz + dz + hz_lo, ly + dy + hy_lo, hxl + lx + l + dx)
+      std::ostringstream e;
+      e << "lds" << slot << "[((lz + " << (off[0] + h.lo[0]) << ") * " << ge.py << " + (ly + " << (off[1] + h.lo[1]) << ")) * " << ge.lx << " + lxe + l + "
+        << (ge.hxl + off[2]) << "]";
+      *expr = e.str();
+      return true;
+    };
+    std::string val = em.emit(root, root_index(dims));
+    std::string body = em.take_code();
+    const std::string it = em.idx_t();
+    const std::string kname = "@K@_stencil";
+    const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + TZ - 1) / TZ;
+    const int64_t nblocks = ntx * nty * ntz;
+    std::ostringstream o;
+    o << "// stencil map through LDS halo tiles (" << TZ << "x" << TY << "x" << TX << " outputs per workgroup): " << describe(root) << " -> " << rn.ty.str() << "\n";
+    o << signature(kname, em.inputs, {{info(rn.ty.dt).stype, "out0"}}) << " {\n";
+    for (int s : staged) {
+      const int slot = em.slot_of(s);
+      const Geo& ge = geo[s];
+      o << "  __shared__ __attribute__((aligned(16))) " << info(g.nodes[s].ty.dt).stype << " lds" << slot << "[" << ge.pz * ge.py * ge.lx << "];\n";
+    }
+    o << "  const unsigned tile = rx_xcd_remap(blockIdx.x, " << nblocks << "u);\n";
+    o << "  const int x0 = (int)(tile % " << ntx << "u) * " << TX << ";\n";
+    o << "  const int y0 = (int)((tile / " << ntx << "u) % " << nty << "u) * " << TY << ";\n";
+    o << "  const int z0 = (int)(tile / " << ntx * nty << "u) * " << TZ << ";\n";
+    for (int s : staged) {
+      const int slot = em.slot_of(s);
+      const Geo& ge = geo[s];
+      const Halo& h = halos[s];
+      const std::string st = info(g.nodes[s].ty.dt).stype;
+      const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+      const int64_t lxv = ge.lx / vec;
+      const int64_t total = ge.pz * ge.py * lxv;
+      const int64_t nit = (total + kBlock - 1) / kBlock;
+      // all global loads of the tile are issued before the first LDS write
+      o << "  {\n    " << vt << " t[" << nit << "];\n";
+      o << "#pragma unroll\n    for (int q = 0; q < " << nit << "; ++q) {\n";
+      o << "      const int v = threadIdx.x + q * " << kBlock << ";\n";
+      o << "      const int xv = v % " << lxv << ", rw = v / " << lxv << ";\n";
+      o << "      const int yy = rw % " << ge.py << ", zz = rw / " << ge.py << ";\n";
+      // halo cells outside the array are clamped to valid addresses; their values are never used
+      o << "      const " << it << " gz = rx_clamp_idx<" << it << ">(z0 - " << h.lo[0] << " + zz, " << Z - 1 << ");\n";
+      o << "      const " << it << " gy = rx_clamp_idx<" << it << ">(y0 - " << h.lo[1] << " + yy, " << Y - 1 << ");\n";
+      o << "      const " << it << " gx = rx_clamp_idx<" << it << ">(x0 - " << ge.hxl << " + xv * " << vec << ", " << X - vec << ");\n";
+      o << "      t[q] = rx_load<" << vt << ">(in" << slot << " + (gz * " << Y << " + gy) * " << X << (em.idx64 ? "LL" : "") << " + gx);\n";
+      o << "    }\n";
+      o << "#pragma unroll\n    for (int q = 0; q < " << nit << "; ++q) {\n";
+      o << "      const int v = threadIdx.x + q * " << kBlock << ";\n";
+      o << "      if (v < " << total << ") rx_store(lds" << slot << " + v * " << vec << ", t[q]);\n";
+      o << "    }\n  }\n";
+    }
+    o << "  const int ly = threadIdx.x / " << TXV << ", lxe = (threadIdx.x % " << TXV << ") * " << vec << ";\n";
+    o << "  const " << it << " i1 = y0 + ly, i2b = x0 + lxe;\n";
+    o << "  const bool live = i1 < " << Y << " && i2b < " << X << ";\n";
+    // inputs read only at the output position: their loads for every plane of the tile are in
+    // flight while the halo tile settles in LDS
+    for (auto& sd : em.direct_vecs) {
+      const int slot = sd.first;
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+      o << "  " << vt << " " << vec_name(slot, 0) << "z[" << TZ << "];\n";
+    }
+    if (!em.direct_vecs.empty()) {
+      o << "  if (live) {\n#pragma unroll\n    for (int lz = 0; lz < " << TZ << "; ++lz) {\n";
+      o << "      const " << it << " i0c = rx_clamp_idx<" << it << ">(z0 + lz, " << Z - 1 << ");\n";
+      o << "      const " << it << " linc = (i0c * " << Y << " + i1) * " << X << (em.idx64 ? "LL" : "") << " + i2b;\n";
+      for (auto& sd : em.direct_vecs) {
+        const int slot = sd.first;
+        const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+        const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+        o << "      " << vec_name(slot, 0) << "z[lz] = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + linc);\n";
+      }
+      o << "    }\n  }\n";
+    }
+    o << "  __syncthreads();\n";
+    o << "  if (!live) return;\n";
+    o << "#pragma unroll\n  for (int lz = 0; lz < " << TZ << "; ++lz) {\n";
+    o << "    const " << it << " i0 = z0 + lz;\n";
+    o << "    if (i0 >= " << Z << ") break;\n";
+    o << "    const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << (em.idx64 ? "LL" : "") << " + i2b;\n";
+    for (auto& sd : em.direct_vecs) {
+      const int slot = sd.first;
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+      o << "    const " << vt << " " << vec_name(slot, 0) << " = " << vec_name(slot, 0) << "z[lz];\n";
+    }
+    const std::string ost = info(rn.ty.dt).stype;
+    o << "    rx_vec<" << ost << ", " << vec << "> res;\n";
+    o << "#pragma unroll\n    for (int l = 0; l < " << vec << "; ++l) {\n";
+    o << "      const " << it << " i2 = i2b + l;\n";
+    o << body;
+    o << "      res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n    }\n";
+    o << "    " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
+    o << "  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = "map_stencil_lds";
+    L.grid[0] = (unsigned)nblocks;
+    L.block[0] = kBlock;
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    L.algo_bytes = algo_bytes(em.inputs, {root});
+    L.desc = describe(root);
+    plan.launches.push_back(L);
+    return true;
+  }
+
   // ------------------------------------------------------------------ map kernels
   void emit_map(int root) {
+    if (emit_map_lds(root)) return;
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
     const int n = rn.ty.rank();

@@ -44,6 +44,8 @@ struct PlanOptions {
   int64_t slab_min_numel = 1 << 22;  // smallest output that uses it
   bool mfma = true;             // use the MFMA GEMM skeletons for eligible dot_generals
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
+  bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
+  int lds_tile[3] = {3, 8, 64};  // outputs per workgroup tile (slowest .. fastest dimension)
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once
   bool nt_stores = true;        // non-temporal hint on map outputs
