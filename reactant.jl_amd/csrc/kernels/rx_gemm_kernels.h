@@ -34,7 +34,10 @@ typedef int rx_i32x8 __attribute__((ext_vector_type(8)));
 typedef int rx_i32x4 __attribute__((ext_vector_type(4)));
 typedef int rx_i32x2 __attribute__((ext_vector_type(2)));
 
-#define RX_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define RX_LDS __attribute__((address_space(3)))
+#define RX_LDS_PTR(T, p) ((RX_LDS T*)(p))
+// LDS tiles are addressed through address_space(3) pointers throughout, so that every access is
+// a ds_read / ds_write (a generic pointer would turn them into slower flat accesses).
 
 // ---------------------------------------------------------------------------
 // MMA policies.  KS = k extent consumed by one `mma` call; frag = per-lane operand.
@@ -46,11 +49,11 @@ struct rx_mma_f32 {
   typedef rx_f32x4 frag;
   static constexpr int KS = 8;
   static constexpr int PAD = 4;   // elements of row padding in LDS
-  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
-    return *reinterpret_cast<const rx_f32x4*>(t + (row0 + (lane & 31)) * ld + kk + 4 * (lane >> 5));
+  RX_DEV frag load_kc(const RX_LDS elem* t, int ld, int row0, int kk, int lane) {
+    return *(const RX_LDS rx_f32x4*)(t + (row0 + (lane & 31)) * ld + kk + 4 * (lane >> 5));
   }
-  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
-    const elem* p = t + (kk + 4 * (lane >> 5)) * ld + col0 + (lane & 31);
+  RX_DEV frag load_tr(const RX_LDS elem* t, int ld, int col0, int kk, int lane) {
+    const RX_LDS elem* p = t + (kk + 4 * (lane >> 5)) * ld + col0 + (lane & 31);
     frag f;
     f[0] = p[0];
     f[1] = p[ld];
@@ -69,14 +72,14 @@ struct rx_mma_bf16 {
   typedef rx_bf16x8 frag;
   static constexpr int KS = 16;
   static constexpr int PAD = 8;
-  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
-    return *reinterpret_cast<const rx_bf16x8*>(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
+  RX_DEV frag load_kc(const RX_LDS elem* t, int ld, int row0, int kk, int lane) {
+    return *(const RX_LDS rx_bf16x8*)(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
   }
-  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+  RX_DEV frag load_tr(const RX_LDS elem* t, int ld, int col0, int kk, int lane) {
     // 16-lane blocks: source lane i points at row k + i/4, columns 4*(i%4)..+3; after the
     // transpose lane j of the block holds 4 consecutive k for column j.
     const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
-    const elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
+    const RX_LDS elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
     rx_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p));
     rx_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p + 4 * ld));
     struct { rx_i16x4 a, b; } both = {lo, hi};
@@ -92,12 +95,12 @@ struct rx_mma_f16 {
   typedef rx_f16x8 frag;
   static constexpr int KS = 16;
   static constexpr int PAD = 8;
-  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
-    return *reinterpret_cast<const rx_f16x8*>(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
+  RX_DEV frag load_kc(const RX_LDS elem* t, int ld, int row0, int kk, int lane) {
+    return *(const RX_LDS rx_f16x8*)(t + (row0 + (lane & 31)) * ld + kk + 8 * (lane >> 5));
   }
-  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+  RX_DEV frag load_tr(const RX_LDS elem* t, int ld, int col0, int kk, int lane) {
     const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
-    const elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
+    const RX_LDS elem* p = t + (kk + 8 * g + (i >> 2)) * ld + col0 + 16 * q + 4 * (i & 3);
     rx_i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p));
     rx_i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p + 4 * ld));
     struct { rx_i16x4 a, b; } both = {lo, hi};
@@ -114,16 +117,16 @@ struct rx_mma_f8 {
   typedef rx_i32x8 frag;
   static constexpr int KS = 64;
   static constexpr int PAD = 16;
-  RX_DEV frag load_kc(const elem* t, int ld, int row0, int kk, int lane) {
-    const elem* p = t + (row0 + (lane & 31)) * ld + kk + 32 * (lane >> 5);
-    struct { rx_i32x4 a, b; } both = {*reinterpret_cast<const rx_i32x4*>(p), *reinterpret_cast<const rx_i32x4*>(p + 16)};
+  RX_DEV frag load_kc(const RX_LDS elem* t, int ld, int row0, int kk, int lane) {
+    const RX_LDS elem* p = t + (row0 + (lane & 31)) * ld + kk + 32 * (lane >> 5);
+    struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(p), *(const RX_LDS rx_i32x4*)(p + 16)};
     return __builtin_bit_cast(rx_i32x8, both);
   }
-  RX_DEV frag load_tr(const elem* t, int ld, int col0, int kk, int lane) {
+  RX_DEV frag load_tr(const RX_LDS elem* t, int ld, int col0, int kk, int lane) {
     // 16-lane blocks: source lane i points at row k + i/2, columns 8*(i%2)..+7; after the
     // transpose lane j of the block holds 8 consecutive k for column j.
     const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
-    const elem* p = t + (kk + 32 * g + (i >> 1)) * ld + col0 + 16 * q + 8 * (i & 1);
+    const RX_LDS elem* p = t + (kk + 32 * g + (i >> 1)) * ld + col0 + 16 * q + 8 * (i & 1);
     struct { rx_i32x2 a, b, c, d; } all = {
         __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p)),
         __builtin_amdgcn_ds_read_tr8_b64_v2i32(RX_LDS_PTR(rx_i32x2, p + 8 * ld)),
@@ -164,11 +167,11 @@ struct rx_tile_copy {
       }
     }
   }
-  RX_MEM void store(E* lds, int lld, int tid) const {
+  RX_MEM void store(RX_LDS E* lds, int lld, int tid) const {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int v = tid + i * NT;
-      if (TOTAL % NT == 0 || v < TOTAL) *reinterpret_cast<rx_u32x4*>(lds + (v / VPR) * lld + (v % VPR) * VE) = r[i];
+      if (TOTAL % NT == 0 || v < TOTAL) *(RX_LDS rx_u32x4*)(lds + (v / VPR) * lld + (v % VPR) * VE) = r[i];
     }
   }
 };
@@ -186,9 +189,8 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
   constexpr int A_LD = A_COLS + MMA::PAD, B_LD = B_COLS + MMA::PAD;
   constexpr int A_SZ = A_ROWS * A_LD, B_SZ = B_ROWS * B_LD;
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
-  E* lds = reinterpret_cast<E*>(rx_smem);
-  E* ldsA[2] = {lds, lds + A_SZ + B_SZ};
-  E* ldsB[2] = {lds + A_SZ, lds + 2 * A_SZ + B_SZ};
+  RX_LDS E* lds = (RX_LDS E*)rx_smem;
+  constexpr int STAGE = A_SZ + B_SZ;   // buffer s: A at s*STAGE, B at s*STAGE + A_SZ
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -228,16 +230,16 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
     if (B_KC) cb.load(Bb, B_GLD, n0, k0, N, K, tid); else cb.load(Bb, B_GLD, k0, n0, K, N, tid);
   };
   gload(0);
-  ca.store(ldsA[0], A_LD, tid);
-  cb.store(ldsB[0], B_LD, tid);
+  ca.store(lds, A_LD, tid);
+  cb.store(lds + A_SZ, B_LD, tid);
   __syncthreads();
 
   constexpr int KT = K / BK;
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < KT) gload((kt + 1) * BK);
-    const E* sa = ldsA[cur];
-    const E* sb = ldsB[cur];
+    const RX_LDS E* sa = lds + cur * STAGE;
+    const RX_LDS E* sb = sa + A_SZ;
 #pragma unroll
     for (int kk = 0; kk < BK; kk += MMA::KS) {
       typename MMA::frag fa[TM], fb[TN];
@@ -257,8 +259,8 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
         for (int j = 0; j < TN; ++j) MMA::mma(acc[i][j], fb[j], fa[i]);
     }
     if (kt + 1 < KT) {
-      ca.store(ldsA[cur ^ 1], A_LD, tid);
-      cb.store(ldsB[cur ^ 1], B_LD, tid);
+      ca.store(lds + (cur ^ 1) * STAGE, A_LD, tid);
+      cb.store(lds + (cur ^ 1) * STAGE + A_SZ, B_LD, tid);
     }
     __syncthreads();
   }

@@ -23,7 +23,10 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (M < 1 || N < 4) return c;
   if (M * N < 64 * 64) return c;  // tiny products: the scalar loop is as good
   if (M >= ((int64_t)1 << 30) || N >= ((int64_t)1 << 30) || K >= ((int64_t)1 << 30)) return c;
+  // Large problems take 256x256 tiles on 8 wavefronts (each wavefront a 128x64 block of the
+  // tile: fewer LDS bytes per MFMA); when that would leave compute units idle, 128x128 on 4.
   int BM = 128, BN = 128, WM = 2, WN = 2;
+  if (((M + 255) / 256) * ((N + 255) / 256) * batch >= 256) { BM = 256; BN = 256; WM = 2; WN = 4; }
   if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
     int v[4];
     if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
