@@ -283,3 +283,252 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
     }
   }
 }
+
+// ===========================================================================
+// Second body: operand tiles travel global -> LDS directly (global_load_lds, 16 bytes per
+// lane, no VGPR staging) through a ring of S LDS stages, so S-1 K-steps of loads are in
+// flight while one is being multiplied.  A wavefront's load fills 1 KB of contiguous LDS in
+// lane order, which rules out row padding; bank conflicts are avoided instead by an XOR
+// swizzle of the 16-byte chunk index inside each row, applied on the global-address side
+// when loading and on the LDS-address side when reading fragments.
+// ===========================================================================
+
+// chunk position inside an LDS row of CPR 16-byte chunks
+//   KC tiles ([o][k], fragment reads of 16 consecutive rows at one chunk index)
+template <int CPR>
+RX_DEV int rx_swz_kc(int row, int c) {
+  constexpr int R = CPR >= 16 ? 1 : 16 / CPR;          // rows per 256 bytes of LDS
+  return c ^ ((row / R) & (CPR - 1));
+}
+//   TR tiles ([k][o]): which rows are read together depends on the element size
+template <int ESIZE, int CPR>
+RX_DEV int rx_swz_tr(int row, int c) {
+  if constexpr (ESIZE == 2) return c ^ (((row & 3) << 1) & (CPR - 1));        // 4 rows x 32 B per 16 lanes
+  else if constexpr (ESIZE == 1) return c ^ ((row & 7) & (CPR - 1));          // 8 rows x 16 B per 16 lanes
+  else return c ^ ((((row >> 2) & 1) << 3) & (CPR - 1));                      // rows k, k+4 read in one instruction
+}
+
+template <class MMA> struct rx_frag_sw;
+
+template <> struct rx_frag_sw<rx_mma_f32> {
+  template <int LD> RX_DEV rx_mma_f32::frag kc(const RX_LDS float* t, int row0, int kk, int lane) {
+    const int r = row0 + (lane & 31), c = (kk + 4 * (lane >> 5)) >> 2;
+    return *(const RX_LDS rx_f32x4*)(t + r * LD + rx_swz_kc<LD / 4>(r, c) * 4);
+  }
+  template <int LD> RX_DEV rx_mma_f32::frag tr(const RX_LDS float* t, int col0, int kk, int lane) {
+    const int col = col0 + (lane & 31), k = kk + 4 * (lane >> 5);
+    rx_mma_f32::frag f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f[j] = t[(k + j) * LD + rx_swz_tr<4, LD / 4>(k + j, col >> 2) * 4 + (col & 3)];
+    return f;
+  }
+};
+template <> struct rx_frag_sw<rx_mma_bf16> {
+  template <int LD> RX_DEV rx_bf16x8 kc(const RX_LDS rx_u16* t, int row0, int kk, int lane) {
+    const int r = row0 + (lane & 31), c = (kk + 8 * (lane >> 5)) >> 3;
+    return *(const RX_LDS rx_bf16x8*)(t + r * LD + rx_swz_kc<LD / 8>(r, c) * 8);
+  }
+  template <int LD> RX_DEV rx_bf16x8 tr(const RX_LDS rx_u16* t, int col0, int kk, int lane) {
+    const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
+    const int k = kk + 8 * g + (i >> 2), col = col0 + 16 * q + 4 * (i & 3);
+    const RX_LDS rx_u16* p0 = t + k * LD + rx_swz_tr<2, LD / 8>(k, col >> 3) * 8 + (col & 7);
+    const RX_LDS rx_u16* p1 = t + (k + 4) * LD + rx_swz_tr<2, LD / 8>(k + 4, col >> 3) * 8 + (col & 7);
+    struct { rx_i16x4 a, b; } both = {__builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p0)),
+                                      __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, p1))};
+    return __builtin_bit_cast(rx_bf16x8, both);
+  }
+};
+template <> struct rx_frag_sw<rx_mma_f16> {
+  template <int LD> RX_DEV rx_f16x8 kc(const RX_LDS rx_u16* t, int row0, int kk, int lane) {
+    return __builtin_bit_cast(rx_f16x8, rx_frag_sw<rx_mma_bf16>::kc<LD>(t, row0, kk, lane));
+  }
+  template <int LD> RX_DEV rx_f16x8 tr(const RX_LDS rx_u16* t, int col0, int kk, int lane) {
+    return __builtin_bit_cast(rx_f16x8, rx_frag_sw<rx_mma_bf16>::tr<LD>(t, col0, kk, lane));
+  }
+};
+template <> struct rx_frag_sw<rx_mma_f8> {
+  template <int LD> RX_DEV rx_i32x8 kc(const RX_LDS rx_u8* t, int row0, int kk, int lane) {
+    const int r = row0 + (lane & 31), c = (kk + 32 * (lane >> 5)) >> 4;
+    struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c) * 16),
+                                      *(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c + 1) * 16)};
+    return __builtin_bit_cast(rx_i32x8, both);
+  }
+  template <int LD> RX_DEV rx_i32x8 tr(const RX_LDS rx_u8* t, int col0, int kk, int lane) {
+    const int i = lane & 15, q = (lane >> 4) & 1, g = lane >> 5;
+    const int k = kk + 32 * g + (i >> 1), col = col0 + 16 * q + 8 * (i & 1);
+    rx_i32x2 r[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const int kh = k + 8 * h;
+      const RX_LDS rx_u8* p = t + kh * LD + rx_swz_tr<1, LD / 16>(kh, col >> 4) * 16 + (col & 15);
+      r[h] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RX_LDS rx_i32x2*)p);
+    }
+    struct { rx_i32x2 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
+    return __builtin_bit_cast(rx_i32x8, all);
+  }
+};
+
+template <int V> struct rx_int { static constexpr int value = V; };
+
+// wait until at most N of this wavefront's vector-memory operations are outstanding
+template <int N>
+RX_DEV void rx_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// Issue the direct loads of one ROWS x COLS operand tile.  Slot s (16-byte units, lane order)
+// of the LDS tile holds global chunk (row = s / CPR, c = swizzle^-1(pos = s % CPR)).
+template <typename E, int ROWS, int COLS, int NT, bool KC>
+RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0, int col0, int nrows, int ncols, RX_LDS E* lds, int tid) {
+  constexpr int VE = 16 / (int)sizeof(E), CPR = COLS / VE, TOTAL = ROWS * CPR;
+  static_assert(TOTAL % NT == 0, "tile must be a whole number of workgroup-wide loads");
+  const int wave_base = (tid >> 6) << 6;
+#pragma unroll
+  for (int i = 0; i < TOTAL / NT; ++i) {
+    const int s = i * NT + tid;
+    const int row = s / CPR, pos = s % CPR;
+    const int c = KC ? rx_swz_kc<CPR>(row, pos) : rx_swz_tr<(int)sizeof(E), CPR>(row, pos);   // XOR is its own inverse
+    int rr = row0 + row, cc = col0 + c * VE;
+    rr = rr < nrows ? rr : nrows - 1;
+    cc = cc + VE <= ncols ? cc : ncols - VE;
+    // the LDS address is per wavefront: base of this wavefront's 1 KB run; lanes fill it in order
+    RX_LDS E* dst = lds + (i * NT + wave_base) * VE;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(g + (long long)rr * gld + cc), (RX_LDS void*)dst, 16, 0, 0);
+  }
+}
+
+template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, bool BATCHED, class Epi>
+RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
+  typedef typename MMA::elem E;
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BK : BM;
+  constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BK : BN;
+  constexpr int A_SZ = A_ROWS * A_COLS, B_SZ = B_ROWS * B_COLS, STAGE = A_SZ + B_SZ;
+  constexpr int VE = 16 / (int)sizeof(E);
+  constexpr int LPS = (A_SZ + B_SZ) / VE / NT;     // loads per thread per stage
+  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
+  RX_LDS E* lds = (RX_LDS E*)rx_smem;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  constexpr int GM = (M + BM - 1) / BM, GN = (N + BN - 1) / BN;
+  int bm, bn;
+  {
+    const int bid = blockIdx.x;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * GN;
+    const int grp = bid / per_group;
+    const int first = grp * GROUP;
+    const int rows = (GM - first) < GROUP ? (GM - first) : GROUP;
+    const int in = bid % per_group;
+    bm = first + in % rows;
+    bn = in / rows;
+  }
+  const int m0 = bm * BM, n0 = bn * BN;
+  const long long batch = BATCHED ? blockIdx.y : 0;
+  const E* Ab = A + batch * (long long)M * K;
+  const E* Bb = B + batch * (long long)N * K;
+  constexpr long long A_GLD = A_KC ? K : M, B_GLD = B_KC ? K : N;
+
+  rx_f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto issue = [&](int kt) {
+    RX_LDS E* st = lds + (kt % S) * STAGE;
+    const int k0 = kt * BK;
+    if (A_KC) rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, A_GLD, m0, k0, M, K, st, tid);
+    else rx_tile_load_direct<E, A_ROWS, A_COLS, NT, false>(Ab, A_GLD, k0, m0, K, M, st, tid);
+    if (B_KC) rx_tile_load_direct<E, B_ROWS, B_COLS, NT, true>(Bb, B_GLD, n0, k0, N, K, st + A_SZ, tid);
+    else rx_tile_load_direct<E, B_ROWS, B_COLS, NT, false>(Bb, B_GLD, k0, n0, K, N, st + A_SZ, tid);
+  };
+  constexpr int KT = K / BK;
+  constexpr int NS = BK / MMA::KS;   // MFMA k-steps per tile
+  // Fragments are double-buffered in registers: the LDS reads of step s+1 are issued before the
+  // MFMAs of step s.  The barrier that publishes tile kt+1 sits before the LAST step of tile kt:
+  // by then every wavefront holds its last fragments of tile kt in registers, so stage kt%S is
+  // free for tile kt+S, and the first fragments of tile kt+1 load under the last MFMAs of tile kt.
+  typename MMA::frag fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int buf, const RX_LDS E* sa, int kk) {
+    const RX_LDS E* sb = sa + A_SZ;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int o = wm * (BM / WM) + 32 * i;
+      if constexpr (A_KC) fa[buf][i] = rx_frag_sw<MMA>::template kc<A_COLS>(sa, o, kk, lane);
+      else fa[buf][i] = rx_frag_sw<MMA>::template tr<A_COLS>(sa, o, kk, lane);
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int o = wn * (BN / WN) + 32 * j;
+      if constexpr (B_KC) fb[buf][j] = rx_frag_sw<MMA>::template kc<B_COLS>(sb, o, kk, lane);
+      else fb[buf][j] = rx_frag_sw<MMA>::template tr<B_COLS>(sb, o, kk, lane);
+    }
+  };
+  auto mma_all = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) MMA::mma(acc[i][j], fb[buf][j], fa[buf][i]);
+  };
+  auto publish = [&]() {
+    asm volatile("" ::: "memory");   // compiler-only fences: LDS reads must not move across the barrier
+    __builtin_amdgcn_s_barrier();    // bare barrier: __syncthreads() would also wait for the younger loads
+    asm volatile("" ::: "memory");
+  };
+#pragma unroll
+  for (int s = 0; s < S; ++s)
+    if (s < KT) issue(s);
+  if (KT >= S) rx_wait_vmcnt<(S - 1) * LPS>(); else rx_wait_vmcnt<0>();
+  publish();
+  load_frags(0, lds, 0);
+
+  // P = register buffer that holds step 0 of this tile (compile-time, so that the fragment
+  // arrays are never indexed dynamically); the next tile starts in buffer (P + NS) & 1.
+  auto tile = [&](auto P, int kt) {
+    constexpr int p = decltype(P)::value;
+    const RX_LDS E* sa = lds + (kt % S) * STAGE;
+#pragma unroll
+    for (int s = 0; s + 1 < NS; ++s) {
+      load_frags((p + s + 1) & 1, sa, (s + 1) * MMA::KS);
+      mma_all((p + s) & 1);
+    }
+    if (kt + 1 < KT) {
+      // tile kt+1 has landed once only the (S-2) tiles after it are still in flight
+      if (kt + S - 1 < KT) rx_wait_vmcnt<(S - 2) * LPS>(); else rx_wait_vmcnt<0>();
+      publish();
+      if (kt + S < KT) issue(kt + S);
+      load_frags((p + NS) & 1, lds + ((kt + 1) % S) * STAGE, 0);
+    }
+    mma_all((p + NS - 1) & 1);
+  };
+  if constexpr (NS % 2 == 0) {
+    for (int kt = 0; kt < KT; ++kt) tile(rx_int<0>{}, kt);
+  } else {
+    for (int kt = 0; kt < KT; kt += 2) {
+      tile(rx_int<0>{}, kt);
+      if (kt + 1 < KT) tile(rx_int<1>{}, kt + 1);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * (BM / WM) + 32 * i + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wn * (BN / WN) + 32 * j + 4 * (lane >> 5);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int n = nb + 8 * rg;
+        if (m < M && n < N) {
+          const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
+          if constexpr (BATCHED) epi(v, (int)batch, m, n); else epi(v, m, n);
+        }
+      }
+    }
+  }
+}

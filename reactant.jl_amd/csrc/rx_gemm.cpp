@@ -32,6 +32,35 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
     if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
   }
   if (const char* e = getenv("RX_GEMM_BK")) bk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : bk;
+  bool direct = true;   // global -> LDS direct loads through a ring of LDS stages
+  if (const char* e = getenv("RX_GEMM_DIRECT")) direct = atoi(e) != 0;
+  int stages = 2;
+  if (const char* e = getenv("RX_GEMM_STAGES")) stages = atoi(e) >= 2 ? atoi(e) : stages;
+  const int nt = WM * WN * 64;
+  if (direct) {
+    int dbk = bk;
+    if (const char* e = getenv("RX_GEMM_BK")) dbk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : dbk;
+    const int ks = a == DT::F32 ? 8 : (esize == 2 ? 16 : 64);
+    const int64_t a_ch = (int64_t)BM * dbk / ve, b_ch = (int64_t)BN * dbk / ve;
+    const int64_t stage_bytes = ((int64_t)BM + BN) * dbk * esize;
+    while (stages > 2 && stage_bytes * stages > 160 * 1024) --stages;
+    if (dbk % ks == 0 && K % dbk == 0 && a_ch % nt == 0 && b_ch % nt == 0 && stage_bytes * stages <= 160 * 1024 &&
+        (a_kc ? dbk : BM) % ve == 0 && (b_kc ? dbk : BN) % ve == 0) {
+      c.lds_bytes = (unsigned)(stage_bytes * stages);
+      c.block = nt;
+      const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
+      c.grid[0] = (unsigned)(gm * gn);
+      c.grid[1] = (unsigned)batch;
+      std::ostringstream t;
+      t << mma << ", " << BM << ", " << BN << ", " << dbk << ", " << WM << ", " << WN << ", " << stages << ", " << (a_kc ? "true" : "false") << ", "
+        << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K;
+      c.targs = t.str();
+      c.skeleton = "rx_gemm_body_dl";
+      c.stype_a = mma + "::elem";
+      c.ok = true;
+      return c;
+    }
+  }
   const int pad = a == DT::F32 ? 4 : (esize == 2 ? 8 : 16);
   const int64_t a_sz = a_kc ? (int64_t)BM * (bk + pad) : (int64_t)bk * (BM + pad);
   const int64_t b_sz = b_kc ? (int64_t)BN * (bk + pad) : (int64_t)bk * (BN + pad);
