@@ -101,7 +101,7 @@ def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=1
     launches = exe.launches()
     cells = nx * ny * nz
     algo_step = 5.0 * cells * 8 * nsteps
-    nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil", "map"))
+    nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil_lds", "map_stencil", "map"))
     algo_launch = 5.0 * cells * 8
     return {
         "workload": "stencil f64 %dx%dx%d halo 3, %d timesteps per module" % (nx, ny, nz, nsteps),

@@ -39,7 +39,11 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       order, Eigen K-blocking) ... PARITY UNPINNED; covered by tolerance only.
 
 Numerics: every op computes in its own element type (bf16/f8 results are rounded
-after each op).  With `hifi=True` reductions and contractions of f32/bf16/f8
+after each op).  With `excess=True` the interpreter instead follows what XLA does
+under its default `xla_allow_excess_precision`: elementwise arithmetic on
+bf16/f16/f8 tensors is carried in f32 and rounded only where a value must exist in
+its own type (convert, dot_general operands, function results).  Both are valid evaluations of the same module; the GPU path uses the
+second, and tests state which one they compare with.  With `hifi=True` reductions and contractions of f32/bf16/f8
 accumulate in float64 before the final rounding, which is the value both this
 oracle and the GPU path are compared to under the stated tolerances.
 """
@@ -120,9 +124,24 @@ class Tensor:
         return Tensor(a.reshape(shape), dt)
 
 
-def tensor(a, dt):
-    """Build a Tensor from numbers, rounding to the element type."""
+_EXCESS = [False]
+
+
+def tensor(a, dt, force=False):
+    """Build a Tensor from numbers, rounding to the element type.
+
+    In excess-precision mode (see Interpreter) results of elementwise arithmetic on
+    bf16/f16/f8 tensors are left unrounded in f32; `force` rounds regardless."""
+    if _EXCESS[0] and not force and dt in ("bf16", "f8E4M3FN", "f8E5M2", "f16"):
+        return Tensor(np.asarray(a, dtype=np.float32), dt)
     return Tensor(_round_to(a, dt), dt)
+
+
+def _rounded(t):
+    """A value as it is when written to a buffer (rounded to its element type)."""
+    if t.dt in ("bf16", "f8E4M3FN", "f8E5M2"):
+        return Tensor(_round_to(t.a, t.dt), t.dt)
+    return t
 
 
 # ----------------------------------------------------------------------------
@@ -1046,9 +1065,10 @@ def _pad(x, pv, low, high, interior, dt):
 
 
 class Interpreter:
-    def __init__(self, funcs, hifi=False):
+    def __init__(self, funcs, hifi=False, excess=False):
         self.funcs = funcs
         self.hifi = hifi
+        self.excess = excess
 
     def run(self, args, fname="main"):
         f = self.funcs[fname]
@@ -1059,7 +1079,11 @@ class Interpreter:
             if tuple(v.shape) != t.shape or v.dt != t.dt:
                 raise ValueError("argument %s: expected %r, got %s %s" % (nm, t, v.shape, v.dt))
             env[nm] = v
-        return self._block(f.ops, env)
+        _EXCESS[0] = self.excess
+        try:
+            return [_rounded(r) for r in self._block(f.ops, env)]
+        finally:
+            _EXCESS[0] = False
 
     def _block(self, ops, env):
         for op in ops:
@@ -1083,7 +1107,11 @@ class Interpreter:
         if n in _BINARY:
             return [_binary(n, xs[0], xs[1], op.types_out[0].dt)]
         if n == "convert":
-            return [_convert(xs[0], op.types_out[0].dt)]
+            prev, _EXCESS[0] = _EXCESS[0], False
+            try:
+                return [_convert(_rounded(xs[0]) if False else xs[0], op.types_out[0].dt)]
+            finally:
+                _EXCESS[0] = prev
         if n == "compare":
             with np.errstate(all="ignore"):
                 return [Tensor(_CMP[at["direction"]](xs[0].a, xs[1].a), "i1")]
@@ -1145,16 +1173,18 @@ class Interpreter:
         if n == "reduce":
             if len(xs) != 2:
                 raise NotImplementedError("variadic reduce")
-            return [_reduce(xs[0], xs[1], at["dimensions"], at["body"], op.types_out[0].dt, self.hifi)]
+            r = _reduce(xs[0], xs[1], at["dimensions"], at["body"], op.types_out[0].dt, self.hifi)
+            return [r if self.excess else _rounded(r)]
         if n == "dot_general":
-            return [_dot_general(xs[0], xs[1], at, op.types_out[0].dt, self.hifi)]
+            r = _dot_general(_rounded(xs[0]), _rounded(xs[1]), at, op.types_out[0].dt, self.hifi)
+            return [r if self.excess else _rounded(r)]
         if n == "enzymexla.math.gelu":
             dt = op.types_out[0].dt
             return [tensor(gelu(xs[0].a.astype(np.float64), at.get("approximation", "NONE")), dt)]
         if n == "optimization_barrier":
             return list(xs)
         if n == "call":
-            return Interpreter(self.funcs, self.hifi).run(list(xs), at["callee"])
+            return Interpreter(self.funcs, self.hifi, self.excess).run(list(xs), at["callee"])
         if n == "map":
             region = op.regions[0]
             env = {}
@@ -1177,6 +1207,6 @@ class Interpreter:
         return o2
 
 
-def run_text(text, args, hifi=False, fname="main"):
+def run_text(text, args, hifi=False, fname="main", excess=False):
     """Parse `text` and evaluate function `fname` on `args` (list of Tensor)."""
-    return Interpreter(parse_module(text), hifi=hifi).run(list(args), fname)
+    return Interpreter(parse_module(text), hifi=hifi, excess=excess).run(list(args), fname)

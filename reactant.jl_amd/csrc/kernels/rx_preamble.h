@@ -106,7 +106,20 @@ RX_DEV float rx_e4m3_to_f32(rx_u8 b) {
   }
   return rx_u2f(s | ((e + 120u) << 23) | (m << 20));
 }
+RX_DEV rx_u8 rx_f32_to_e4m3_sw(float f);
+// gfx950 converts f32 -> OCP e4m3 in hardware (round to nearest even).  Only finite values with
+// |x| <= 448 are given to it, so its overflow mode never matters: (448, 464] rounds to 448 and
+// everything above (or NaN) is the NaN code, as the format without infinity requires.
 RX_DEV rx_u8 rx_f32_to_e4m3(float f) {
+  const rx_u32 u = rx_f2u(f);
+  const rx_u32 a = u & 0x7fffffffu;
+  const rx_u8 s = (rx_u8)((u >> 24) & 0x80u);
+  if (a > 0x43e80000u) return (rx_u8)(s | 0x7fu);
+  const float c = rx_u2f(a > 0x43e00000u ? 0x43e00000u : a);   // min(|x|, 448)
+  const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false);
+  return (rx_u8)(s | (rx_u8)(packed & 0x7f));
+}
+RX_DEV rx_u8 rx_f32_to_e4m3_sw(float f) {
   rx_u32 u = rx_f2u(f);
   rx_u8 s = (rx_u8)((u >> 24) & 0x80u);
   rx_u32 a = u & 0x7fffffffu;
@@ -153,6 +166,14 @@ template <typename T> RX_DEV T rx_max(T a, T b) { return (a > b || a != a) ? a :
 template <typename T> RX_DEV T rx_min(T a, T b) { return (a < b || a != a) ? a : b; }
 template <typename T> RX_DEV T rx_sign(T a) {
   return a != a ? a : (T)((a > (T)0) - (a < (T)0));
+}
+// tanh for results that are rounded to a 16-bit or 8-bit float: 1 - 2/(e^{2x}+1) on the
+// hardware exp2 / reciprocal (relative error ~1e-6, far below half an ulp of bf16)
+RX_DEV float rx_tanh_fast(float x) {
+  const float ax = fabsf(x);
+  const float e = __builtin_amdgcn_exp2f(fminf(ax, 15.0f) * 2.8853900817779268f);   // e^{2|x|}
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return x != x ? x : (x < 0.0f ? -t : t);
 }
 RX_DEV float rx_logistic(float x) { return 1.0f / (1.0f + expf(-x)); }
 RX_DEV double rx_logistic(double x) { return 1.0 / (1.0 + exp(-x)); }

@@ -211,6 +211,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;
   if (const char* e = getenv("RX_LDS_TILE")) { int v[3]; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) == 3) { o.lds_tile[0] = v[0]; o.lds_tile[1] = v[1]; o.lds_tile[2] = v[2]; } }
   if (const char* e = getenv("RX_SHIFTED_VEC")) o.shifted_vector_loads = atoi(e) != 0;
+  if (const char* e = getenv("RX_EXCESS_PRECISION")) o.excess_precision = atoi(e) != 0;
   if (const char* e = getenv("RX_NT_LOADS")) o.nt_loads = atoi(e) != 0;
   if (const char* e = getenv("RX_NT_STORES")) o.nt_stores = atoi(e) != 0;
   return o;

@@ -213,9 +213,10 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
   const DT dt = n.ty.dt;
   const std::string CT = info(dt).ctype;
   const bool dbl = dt == DT::F64;
-  auto def = [&](const std::string& expr) {
+  auto def = [&](const std::string& expr, bool force_round = false) {
     std::string v = fresh();
-    line("const " + CT + " " + v + " = " + (is_narrow_float(dt) ? round_narrow(dt, expr) : expr) + ";");
+    const bool rnd = is_narrow_float(dt) && (force_round || !excess_precision);
+    line("const " + CT + " " + v + " = " + (rnd ? round_narrow(dt, expr) : expr) + ";");
     return v;
   };
   // index of a rank-0 or same-shape operand
@@ -232,7 +233,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       return literal(n);
     case OpK::Iota: {
       std::string e = "(" + CT + ")" + ix[n.a0[0]].str();
-      return is_narrow_float(dt) ? def(e) : e;
+      return is_narrow_float(dt) ? def(e, true) : e;
     }
     case OpK::Unary: {
       const DT sdt = g_.nodes[n.in[0]].ty.dt;
@@ -243,7 +244,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (op == "sine") return def(fn("sin", dbl) + "(" + x + ")");
         if (op == "cosine") return def(fn("cos", dbl) + "(" + x + ")");
         if (op == "tan") return def(fn("tan", dbl) + "(" + x + ")");
-        if (op == "tanh") return def(fn("tanh", dbl) + "(" + x + ")");
+        if (op == "tanh") return def((is_narrow_float(dt) ? std::string("rx_tanh_fast") : fn("tanh", dbl)) + "(" + x + ")");
         if (op == "exponential") return def(fn("exp", dbl) + "(" + x + ")");
         if (op == "exponential_minus_one") return def(fn("expm1", dbl) + "(" + x + ")");
         if (op == "log") return def(fn("log", dbl) + "(" + x + ")");
@@ -339,9 +340,9 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       std::string x = opnd(0);
       if (sdt == dt) return x;
       if (dt == DT::I1) return def("(" + x + " != 0)");
-      if (is_narrow_float(sdt) && is_narrow_float(dt)) return def(x);
+      if (is_narrow_float(sdt) && is_narrow_float(dt)) return def(x, true);
       if (is_narrow_float(sdt) && dt == DT::F32) return x;
-      return def("(" + CT + ")" + x);
+      return def("(" + CT + ")" + x, true);
     }
     case OpK::BroadcastInDim: {
       const Node& o = g_.nodes[n.in[0]];

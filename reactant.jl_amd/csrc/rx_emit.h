@@ -54,6 +54,10 @@ class Emitter {
   std::function<std::string(int slot, int64_t D)> direct_expr;
   bool allow_shifted = false;
   int vec = 1;
+  // Arithmetic on bf16/f16/f8 tensors is carried in f32 inside a kernel and rounded once, when a
+  // value is stored or explicitly converted (what XLA does under its default
+  // xla_allow_excess_precision).  With this off every op result is rounded to its element type.
+  bool excess_precision = true;
   // Loads of an input at root-index + constant offsets can be redirected (to an LDS halo tile):
   // the hook returns true and the expression to read instead of global memory.
   std::function<bool(int slot, const std::vector<int64_t>& off, std::string* expr)> tile_hook;

@@ -480,6 +480,7 @@ struct Planner {
     };
     // pass 1: find the stencil inputs and their halos
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
+    probe.excess_precision = opt.excess_precision;
     make_emitter(probe);
     probe.emit(root, root_index(dims));
     struct Halo { int64_t lo[3] = {0, 0, 0}, hi[3] = {0, 0, 0}; int count = 0; bool ok = true; };
@@ -527,6 +528,7 @@ struct Planner {
 
     // pass 2: emit with the staged inputs redirected to LDS
     Emitter em(g, [&](int x) { return x != root && mat[x]; });
+    em.excess_precision = opt.excess_precision;
     make_emitter(em);
     em.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
       const int node = em.inputs[slot];
@@ -654,6 +656,7 @@ struct Planner {
     const int64_t nv = numel / vec;
     const std::string kname = "@K@_map";
     Emitter em(g, [&](int x) { return x != root && mat[x]; });
+    em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(root));
     const std::string it = em.idx_t();
     std::vector<std::string> vars;
@@ -800,6 +803,7 @@ struct Planner {
     const std::string k1 = "@K@_reduce", k2 = "@K@_reduce_final";
 
     Emitter em(g, [&](int x) { return mat[x]; });
+    em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(rn.in[0]));
     const std::string it = em.idx_t();
     std::vector<std::string> vars;
@@ -843,6 +847,7 @@ struct Planner {
 
     // pass 2
     Emitter e2(g, [&](int x) { return mat[x]; });
+    e2.excess_precision = opt.excess_precision;
     e2.indent = 4;
     std::string initv = e2.emit(rn.in[1], Index{});
     std::string ibody = e2.take_code();
@@ -896,6 +901,7 @@ struct Planner {
     const int64_t nout = rn.ty.numel();
     const std::string kname = "@K@_reduce_generic";
     Emitter em(g, [&](int x) { return mat[x]; });
+    em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(rn.in[0]));
     const std::string it = em.idx_t();
     em.set_root({}, {}, false);
@@ -907,6 +913,7 @@ struct Planner {
     for (size_t k = 0; k < red.size(); ++k) { ix[red[k]].var = "r" + std::to_string(k); ix[red[k]].hi = inn.ty.dims[red[k]] - 1; }
     em.indent = 4 + 2 * (int)red.size();
     Emitter e2(g, [&](int x) { return mat[x]; });
+    e2.excess_precision = opt.excess_precision;
     e2.inputs = {};
     std::string val = em.emit(rn.in[0], ix);
     std::string body = em.take_code();
@@ -970,6 +977,7 @@ struct Planner {
 
     std::set<int> phase_set(phases.begin(), phases.end());
     Emitter em(g, [&](int x) { return mat[x] && x != root && !phase_set.count(x); });
+    em.excess_precision = opt.excess_precision;
     std::vector<int> touched = cone_nodes(root);
     for (int p : phases) { auto c = cone_nodes(p); touched.insert(touched.end(), c.begin(), c.end()); }
     em.idx64 = needs64(touched);
@@ -1091,7 +1099,9 @@ struct Planner {
         o << "  a" << pc.node << " = rx_block_reduce<" << ACC << ", decltype(" << red_functor(p.red) << "), " << kBlock / 64 << ">(a" << pc.node << ", "
           << red_functor(p.red) << ", reinterpret_cast<" << ACC << "*>(lds_raw));\n";
       std::string comb = red_apply(p.red, dt, "a" + std::to_string(pc.node), "(" + ACC + ")" + inits[pc.node]);
-      std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, comb) : std::string("(") + info(dt).ctype + ")(" + comb + ")";
+      // a reduction consumed inside the kernel stays in f32 under excess precision
+      const bool rnd = is_narrow_float(dt) && !(opt.excess_precision && !root_is_reduce);
+      std::string rv = rnd ? Emitter::round_narrow(dt, comb) : std::string("(") + info(dt).ctype + ")(" + comb + ")";
       o << "  const " << info(dt).ctype << " r" << pc.node << " = " << rv << ";\n";
     }
     if (root_is_reduce) {
@@ -1205,6 +1215,7 @@ struct Planner {
     // consecutive elements of the minor output dimension (vector loads of same-shaped
     // operands such as C in alpha*A*B + beta*C, one vector store).
     Emitter em(g, [&](int x) { return mat[x] && x != root; });
+    em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(root)) || lt.numel() >= ((int64_t)1 << 31) || rt.numel() >= ((int64_t)1 << 31);
     const std::string it = em.idx_t();
     std::vector<std::string> vars;
@@ -1245,7 +1256,7 @@ struct Planner {
     o << "#pragma unroll\n    for (int l = 0; l < NV; ++l) {\n";
     if (n > 0) o << "      const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
     {
-      std::string accv = is_narrow_float(d.ty.dt) ? Emitter::round_narrow(d.ty.dt, "acc[l]") : std::string("(") + DCT + ")acc[l]";
+      std::string accv = (is_narrow_float(d.ty.dt) && !(opt.excess_precision && root != dot)) ? Emitter::round_narrow(d.ty.dt, "acc[l]") : std::string("(") + DCT + ")acc[l]";
       o << "      const " << DCT << " accv = " << accv << ";\n";
     }
     o << ebody;

@@ -47,6 +47,7 @@ struct PlanOptions {
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
   int lds_tile[3] = {3, 8, 64};  // outputs per workgroup tile (slowest .. fastest dimension)
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
+  bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once
   bool nt_stores = true;        // non-temporal hint on map outputs
 };

@@ -21,8 +21,8 @@ def gpu_run(rx, client, text, args, exe=None):
     return res, exe
 
 
-def oracle_run(text, args, hifi=True):
-    return I.run_text(text, args, hifi=hifi)
+def oracle_run(text, args, hifi=True, excess=False):
+    return I.run_text(text, args, hifi=hifi, excess=excess)
 
 
 def rel_err(got, ref):

@@ -1,0 +1,302 @@
+"""Op-level GPU parity: the reference's own known-answer tests for the ops on the
+hot path (test/core/ops.jl, test/core/map_reduction.jl, test/core/math_ops.jl,
+src/TestUtils.jl fixture generator), plus bit-exact checks of conversions and
+index ops against the oracle."""
+import numpy as np
+import pytest
+
+from _harness import gpu_run, oracle_run, rel_err
+from oracle import stablehlo_interp as I
+from oracle import lowfloat as lf
+
+pytestmark = pytest.mark.gpu
+
+
+def _tt(shape, dt):
+    return "tensor<" + "x".join([str(s) for s in shape] + [dt]) + ">"
+
+
+def mod(args, ret, body):
+    sig = ", ".join("%%arg%d: %s" % (k, t) for k, t in enumerate(args))
+    return "module {\n  func.func @main(%s) -> %s {\n%s  }\n}\n" % (sig, ret, body)
+
+
+def construct_test_array(dtype, *dims):
+    """Reactant.TestUtils.construct_test_array (src/TestUtils.jl:9-23), Julia (column-major) order."""
+    n = int(np.prod(dims))
+    flat = np.arange(1, n + 1)
+    a = (flat / n).astype(dtype) if np.issubdtype(dtype, np.floating) else flat.astype(dtype)
+    return a.reshape(dims, order="F")
+
+
+def both(rx, client, text, args, hifi=True):
+    got, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=hifi)
+    return got, ref
+
+
+# ---- pad (test/core/ops.jl:534-557) -----------------------------------------------
+@pytest.mark.parametrize("low,high,interior,expect", [
+    ([1], [0], [0], [0, 1, 2, 3, 4]), ([0], [1], [0], [1, 2, 3, 4, 0]), ([0], [0], [1], [1, 0, 2, 0, 3, 0, 4])])
+def test_pad_1d_reference_vectors(rx, client, low, high, interior, expect):
+    n = len(expect)
+    text = mod([_tt([4], "i64"), "tensor<i64>"], _tt([n], "i64"),
+               "    %%0 = stablehlo.pad %%arg0, %%arg1, low = %s, high = %s, interior = %s : (tensor<4xi64>, tensor<i64>) -> %s\n"
+               "    return %%0 : %s\n" % (low, high, interior, _tt([n], "i64"), _tt([n], "i64")))
+    got, ref = both(rx, client, text, [I.Tensor(np.array([1, 2, 3, 4]), "i64"), I.Tensor(np.array(0), "i64")])
+    assert got[0].a.tolist() == expect and ref[0].a.tolist() == expect
+
+
+@pytest.mark.parametrize("low,high,interior,expect", [
+    ([1, 2], [0, 0], [0, 0], [[0, 0, 0, 0], [0, 0, 1, 2], [0, 0, 3, 4]]),
+    ([0, 0], [1, 2], [0, 0], [[1, 2, 0, 0], [3, 4, 0, 0], [0, 0, 0, 0]]),
+    ([0, 0], [0, 0], [1, 2], [[1, 0, 0, 2], [0, 0, 0, 0], [3, 0, 0, 4]])])
+def test_pad_2d_reference_vectors(rx, client, low, high, interior, expect):
+    # Julia [1 2; 3 4] arrives as raw [[1,3],[2,4]]; Julia dims (low etc.) are reversed on the wire
+    E = np.array(expect)
+    raw_in = np.array([[1, 2], [3, 4]]).T.copy()
+    rl, rh, ri = low[::-1], high[::-1], interior[::-1]
+    oshape = list(E.T.shape)
+    text = mod([_tt([2, 2], "i64"), "tensor<i64>"], _tt(oshape, "i64"),
+               "    %%0 = stablehlo.pad %%arg0, %%arg1, low = %s, high = %s, interior = %s : (tensor<2x2xi64>, tensor<i64>) -> %s\n"
+               "    return %%0 : %s\n" % (rl, rh, ri, _tt(oshape, "i64"), _tt(oshape, "i64")))
+    got, ref = both(rx, client, text, [I.Tensor(raw_in, "i64"), I.Tensor(np.array(0), "i64")])
+    assert np.array_equal(got[0].a.T, E) and np.array_equal(ref[0].a.T, E)
+
+
+def test_slice_reference_vectors(rx, client):
+    # Ops.slice(x, [2], [3]) == [2, 3]  (1-based inclusive -> [1:3])   test/core/ops.jl:815-819
+    text = mod([_tt([4], "i64")], _tt([2], "i64"),
+               "    %0 = stablehlo.slice %arg0 [1:3] : (tensor<4xi64>) -> tensor<2xi64>\n    return %0 : tensor<2xi64>\n")
+    got, ref = both(rx, client, text, [I.Tensor(np.array([1, 2, 3, 4]), "i64")])
+    assert got[0].a.tolist() == [2, 3] == ref[0].a.tolist()
+
+
+# ---- elementwise known answers (test/core/ops.jl:788-824) ------------------------
+def test_sine_sqrt_reference_vectors(rx, client):
+    x = np.array([0.0, np.pi / 2, np.pi, 3 * np.pi / 2, 2 * np.pi])
+    text = mod([_tt([5], "f64")], _tt([5], "f64"), "    %0 = stablehlo.sine %arg0 : tensor<5xf64>\n    return %0 : tensor<5xf64>\n")
+    got, ref = both(rx, client, text, [I.Tensor(x, "f64")])
+    assert np.allclose(got[0].a, [0, 1, 0, -1, 0], atol=1e-15) and np.allclose(ref[0].a, [0, 1, 0, -1, 0], atol=1e-15)
+    text = mod([_tt([4], "f64")], _tt([4], "f64"), "    %0 = stablehlo.sqrt %arg0 : tensor<4xf64>\n    return %0 : tensor<4xf64>\n")
+    got, ref = both(rx, client, text, [I.Tensor(np.array([1.0, 4.0, 9.0, 16.0]), "f64")])
+    assert got[0].a.tolist() == [1.0, 2.0, 3.0, 4.0] == ref[0].a.tolist()
+
+
+UNARY_F32 = ["sine", "cosine", "tanh", "exponential", "log", "sqrt", "rsqrt", "abs", "negate", "logistic", "floor", "ceil",
+             "sign", "exponential_minus_one", "log_plus_one", "cbrt", "round_nearest_even"]
+
+
+@pytest.mark.parametrize("op", UNARY_F32)
+def test_unary_f32_maps(rx, client, op):
+    """fp32 maps agree with the f64-evaluated library routine to 1e-6 relative (trig sweep on the
+    reference's fixture array, test/core/math_ops.jl:33-43, plus a seeded wide sweep)."""
+    fix = construct_test_array(np.float32, 4, 16)[:, :7]
+    rng = np.random.default_rng(0)
+    wide = rng.uniform(0.05, 8.0, 4096).astype(np.float32) if op in ("log", "sqrt", "rsqrt", "log_plus_one") \
+        else rng.uniform(-8.0, 8.0, 4096).astype(np.float32)
+    for x in (np.ascontiguousarray(fix.T), wide):
+        t = _tt(x.shape, "f32")
+        text = mod([t], t, "    %%0 = stablehlo.%s %%arg0 : %s\n    return %%0 : %s\n" % (op, t, t))
+        got, _ = gpu_run(rx, client, text, [I.Tensor(x, "f32")])
+        ref64 = oracle_run(text.replace("f32", "f64"), [I.Tensor(x.astype(np.float64), "f64")])[0].a
+        err = np.abs(got[0].a.astype(np.float64) - ref64) / np.maximum(np.abs(ref64), 1e-30)
+        ok = (err <= 1e-6) | (np.abs(got[0].a.astype(np.float64) - ref64) <= 1e-7)
+        assert ok.all(), (op, float(err.max()))
+
+
+BINARY = ["add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "remainder"]
+
+
+@pytest.mark.parametrize("op", BINARY)
+@pytest.mark.parametrize("dt", ["f32", "f64", "i32", "i64", "ui8"])
+def test_binary_ops(rx, client, op, dt):
+    rng = np.random.default_rng(1)
+    n = 1000
+    if dt.startswith("f"):
+        a = rng.uniform(0.5, 4.0, n).astype(I.NP_OF[dt])
+        b = rng.uniform(0.5, 3.0, n).astype(I.NP_OF[dt])
+    else:
+        a = rng.integers(0 if dt == "ui8" else -50, 50, n).astype(I.NP_OF[dt])
+        b = rng.integers(1, 5, n).astype(I.NP_OF[dt])
+        if op == "power":
+            a = (np.abs(a) % 6).astype(I.NP_OF[dt])
+            b = (b % 4).astype(I.NP_OF[dt])
+    t = _tt([n], dt)
+    text = mod([t, t], t, "    %%0 = stablehlo.%s %%arg0, %%arg1 : %s\n    return %%0 : %s\n" % (op, t, t))
+    got, ref = both(rx, client, text, [I.Tensor(a, dt), I.Tensor(b, dt)])
+    if dt.startswith("f"):
+        tol = 1e-6 if dt == "f32" else 1e-14
+        assert rel_err(got[0].a, ref[0].a) <= tol
+    else:
+        assert np.array_equal(got[0].a, ref[0].a)   # integers: bit-exact
+
+
+# ---- reductions (test/core/ops.jl:1207-1235, test/core/map_reduction.jl) ---------
+@pytest.mark.parametrize("dims,body,init", [([1], "multiply", 1), ([0, 2], "add", 0), ([0, 1, 2], "add", 0)])
+def test_int_reduce_reference(rx, client, dims, body, init):
+    A = construct_test_array(np.int64, 3, 4, 5)       # Julia 3x4x5
+    raw = np.ascontiguousarray(A.T)                   # wire layout 5x4x3
+    jd = [d + 1 for d in dims]                        # these are the Julia dims of the reference test ...
+    wire = sorted(2 - d for d in dims)                # ... which are reversed on the wire
+    oshape = [s for k, s in enumerate(raw.shape) if k not in wire]
+    text = mod([_tt(raw.shape, "i64"), "tensor<i64>"], _tt(oshape, "i64"),
+               "    %%0 = stablehlo.reduce(%%arg0 init: %%arg1) applies stablehlo.%s across dimensions = %s : (%s, tensor<i64>) -> %s\n"
+               "    return %%0 : %s\n" % (body, wire, _tt(raw.shape, "i64"), _tt(oshape, "i64"), _tt(oshape, "i64")))
+    got, ref = both(rx, client, text, [I.Tensor(raw, "i64"), I.Tensor(np.array(init), "i64")])
+    f = np.multiply.reduce if body == "multiply" else np.add.reduce
+    expect = A
+    for d in sorted(dims, reverse=True):
+        expect = f(expect, axis=d)
+    assert np.array_equal(np.asarray(got[0].a).T, np.asarray(expect))
+    assert np.array_equal(np.asarray(ref[0].a).T, np.asarray(expect))
+    assert jd
+
+
+def test_float_sum_closed_form(rx, client):
+    # sum(construct_test_array(Float64, 2, 10)) == 210/20 == 10.5   (test/core/map_reduction.jl:8-19)
+    A = construct_test_array(np.float64, 2, 10)
+    raw = np.ascontiguousarray(A.T)
+    text = mod([_tt(raw.shape, "f64")], "tensor<f64>",
+               "    %%c = stablehlo.constant dense<0.000000e+00> : tensor<f64>\n"
+               "    %%0 = stablehlo.reduce(%%arg0 init: %%c) applies stablehlo.add across dimensions = [0, 1] : (%s, tensor<f64>) -> tensor<f64>\n"
+               "    return %%0 : tensor<f64>\n" % _tt(raw.shape, "f64"))
+    got, ref = both(rx, client, text, [I.Tensor(raw, "f64")])
+    assert abs(float(got[0].a) - 10.5) < 1e-12 and abs(float(ref[0].a) - 10.5) < 1e-12
+
+
+@pytest.mark.parametrize("shape,dims", [((64, 1000), [1]), ((1000, 64), [0]), ((7, 33, 65), [2]), ((7, 33, 65), [1, 2]),
+                                        ((7, 33, 65), [0]), ((5, 6, 7), [0, 2]), ((300, 4096), [1]), ((3, 70), [1])])
+@pytest.mark.parametrize("body", ["add", "maximum", "minimum"])
+def test_partial_reductions_f32(rx, client, shape, dims, body):
+    x = np.random.default_rng(3).normal(size=shape).astype(np.float32)
+    oshape = [s for k, s in enumerate(shape) if k not in dims]
+    init = {"add": "0.000000e+00", "maximum": "0xFF800000", "minimum": "0x7F800000"}[body]
+    text = mod([_tt(shape, "f32")], _tt(oshape, "f32"),
+               "    %%c = stablehlo.constant dense<%s> : tensor<f32>\n"
+               "    %%0 = stablehlo.reduce(%%arg0 init: %%c) applies stablehlo.%s across dimensions = %s : (%s, tensor<f32>) -> %s\n"
+               "    return %%0 : %s\n" % (init, body, dims, _tt(shape, "f32"), _tt(oshape, "f32"), _tt(oshape, "f32")))
+    got, ref = both(rx, client, text, [I.Tensor(x, "f32")])
+    n = int(np.prod([shape[d] for d in dims]))
+    if body == "add":
+        scale = np.abs(x).sum(axis=tuple(dims))
+        assert np.all(np.abs(got[0].a.astype(np.float64) - ref[0].a) <= 1e-5 * np.sqrt(n) * np.maximum(scale / n, 1e-30) + 1e-6)
+    else:
+        assert np.array_equal(got[0].a, ref[0].a)
+
+
+def test_bool_and_int_widening_sum(rx, client):
+    # sum(::Array{Bool}) widens to Int64 before the reduce (src/TracedRArray.jl:200-216)
+    x = (np.random.default_rng(0).uniform(size=(17, 9)) > 0.5)
+    text = mod([_tt(x.shape, "i1")], "tensor<i64>",
+               "    %%c = stablehlo.constant dense<0> : tensor<i64>\n"
+               "    %%0 = stablehlo.convert %%arg0 : (%s) -> %s\n"
+               "    %%1 = stablehlo.reduce(%%0 init: %%c) applies stablehlo.add across dimensions = [0, 1] : (%s, tensor<i64>) -> tensor<i64>\n"
+               "    return %%1 : tensor<i64>\n" % (_tt(x.shape, "i1"), _tt(x.shape, "i64"), _tt(x.shape, "i64")))
+    got, ref = both(rx, client, text, [I.Tensor(x, "i1")])
+    assert int(got[0].a) == int(x.sum()) == int(ref[0].a)
+
+
+# ---- conversions: bit-exact --------------------------------------------------------
+def _interesting_f32():
+    vals = [0.0, -0.0, np.inf, -np.inf, np.nan, 448.0, 449.0, 463.99, 464.0, 464.01, 480.0, 1e9, 2.0 ** -6, 2.0 ** -9,
+            2.0 ** -10, 2.0 ** -10 * 1.0001, 2.0 ** -11, 57344.0, 61439.0, 61440.0, 65504.0, 1e-30, 3.0e38]
+    codes = np.arange(256, dtype=np.uint8)
+    rep = lf.e4m3fn_bits_to_f32(codes)
+    rep = rep[np.isfinite(rep)]
+    mids = (np.sort(rep)[1:] + np.sort(rep)[:-1]) / 2           # ties
+    rng = np.random.default_rng(0)
+    rnd = np.concatenate([rng.normal(size=20000) * s for s in (1e-3, 1.0, 100.0, 1000.0)])
+    bits = rng.integers(0, 2 ** 32, 20000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    x = np.concatenate([np.array(vals, dtype=np.float32), -np.array(vals, dtype=np.float32), rep, mids,
+                        np.nextafter(mids.astype(np.float32), np.float32(np.inf)), np.nextafter(mids.astype(np.float32), np.float32(-np.inf)),
+                        rnd.astype(np.float32), bits]).astype(np.float32)
+    return x
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f8E4M3FN", "f8E5M2", "f16"])
+def test_convert_f32_to_narrow_bit_exact(rx, client, dt):
+    x = _interesting_f32()
+    t, o = _tt(x.shape, "f32"), _tt(x.shape, dt)
+    text = mod([t], o, "    %%0 = stablehlo.convert %%arg0 : (%s) -> %s\n    return %%0 : %s\n" % (t, o, o))
+    got, ref = both(rx, client, text, [I.Tensor(x, "f32")])
+    gb, rb = np.frombuffer(got[0].to_bytes(), np.uint8), np.frombuffer(ref[0].to_bytes(), np.uint8)
+    nan = np.isnan(got[0].a) & np.isnan(ref[0].a)
+    esz = I.ITEMSIZE[dt]
+    same = (gb.reshape(-1, esz) == rb.reshape(-1, esz)).all(axis=1)
+    assert (same | nan).all(), x[~(same | nan)][:10]
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f8E4M3FN", "f8E5M2", "f16"])
+def test_convert_narrow_to_f32_exact(rx, client, dt):
+    n = 65536 if I.ITEMSIZE[dt] == 2 else 256
+    raw = np.arange(n, dtype=np.uint16 if n > 256 else np.uint8)
+    x = I.Tensor.from_bytes(raw.tobytes(), dt, (n,))
+    t, o = _tt([n], dt), _tt([n], "f32")
+    text = mod([t], o, "    %%0 = stablehlo.convert %%arg0 : (%s) -> %s\n    return %%0 : %s\n" % (t, o, o))
+    got, ref = both(rx, client, text, [x])
+    assert np.array_equal(got[0].a.view(np.uint32)[~np.isnan(ref[0].a)], ref[0].a.view(np.uint32)[~np.isnan(ref[0].a)])
+    assert np.array_equal(np.isnan(got[0].a), np.isnan(ref[0].a))
+
+
+# ---- index ops: bit-exact on integers --------------------------------------------------
+def test_index_op_chain(rx, client):
+    x = np.arange(4 * 6 * 8, dtype=np.int32).reshape(4, 6, 8)
+    t = _tt(x.shape, "i32")
+    body = ("    %%0 = stablehlo.transpose %%arg0, dims = [2, 0, 1] : (%s) -> tensor<8x4x6xi32>\n"
+            "    %%1 = stablehlo.slice %%0 [1:7:2, 0:4, 2:6] : (tensor<8x4x6xi32>) -> tensor<3x4x4xi32>\n"
+            "    %%2 = stablehlo.reshape %%1 : (tensor<3x4x4xi32>) -> tensor<12x4xi32>\n"
+            "    %%3 = stablehlo.iota dim = 1 : tensor<12x4xi32>\n"
+            "    %%4 = stablehlo.add %%2, %%3 : tensor<12x4xi32>\n"
+            "    %%5 = stablehlo.broadcast_in_dim %%arg1, dims = [1] : (tensor<4xi32>) -> tensor<12x4xi32>\n"
+            "    %%6 = stablehlo.multiply %%4, %%5 : tensor<12x4xi32>\n"
+            "    %%7 = stablehlo.concatenate %%6, %%2, dim = 0 : (tensor<12x4xi32>, tensor<12x4xi32>) -> tensor<24x4xi32>\n"
+            "    %%c = stablehlo.constant dense<-1> : tensor<i32>\n"
+            "    %%8 = stablehlo.pad %%7, %%c, low = [1, -1], high = [2, 1], interior = [0, 1] : (tensor<24x4xi32>, tensor<i32>) -> tensor<27x7xi32>\n"
+            "    return %%8 : tensor<27x7xi32>\n" % t)
+    text = mod([t, _tt([4], "i32")], "tensor<27x7xi32>", body)
+    got, ref = both(rx, client, text, [I.Tensor(x, "i32"), I.Tensor(np.array([3, -2, 7, 1], dtype=np.int32), "i32")])
+    assert np.array_equal(got[0].a, ref[0].a)
+
+
+def test_compare_select_clamp(rx, client):
+    rng = np.random.default_rng(5)
+    a = rng.normal(size=(33, 17)).astype(np.float32)
+    b = rng.normal(size=(33, 17)).astype(np.float32)
+    t, tb = _tt(a.shape, "f32"), _tt(a.shape, "i1")
+    body = ("    %%0 = stablehlo.compare  GT, %%arg0, %%arg1,  FLOAT : (%s, %s) -> %s\n"
+            "    %%1 = stablehlo.select %%0, %%arg0, %%arg1 : %s, %s\n"
+            "    %%lo = stablehlo.constant dense<-5.000000e-01> : tensor<f32>\n"
+            "    %%hi = stablehlo.constant dense<5.000000e-01> : tensor<f32>\n"
+            "    %%2 = stablehlo.clamp %%lo, %%1, %%hi : (tensor<f32>, %s, tensor<f32>) -> %s\n"
+            "    return %%2 : %s\n" % (t, t, tb, tb, t, t, t, t))
+    got, ref = both(rx, client, mod([t, t], t, body), [I.Tensor(a, "f32"), I.Tensor(b, "f32")])
+    assert np.array_equal(got[0].a, ref[0].a)
+
+
+def test_map_op_generic_form(rx, client):
+    """stablehlo.map in generic form (src/mlir/Dialects/StableHLO.jl:2686-2705 spec example)."""
+    a = np.arange(6, dtype=np.int64).reshape(2, 3)
+    b = np.arange(6, 12, dtype=np.int64).reshape(2, 3)
+    text = ('module {\n  func.func @main(%arg0: tensor<2x3xi64>, %arg1: tensor<2x3xi64>) -> tensor<2x3xi64> {\n'
+            '    %0 = "stablehlo.map"(%arg0, %arg1) ({\n'
+            '      ^bb0(%a: tensor<i64>, %b: tensor<i64>):\n'
+            '        %1 = stablehlo.multiply %a, %b : tensor<i64>\n'
+            '        stablehlo.return %1 : tensor<i64>\n'
+            '    }) {dimensions = array<i64: 0, 1>} : (tensor<2x3xi64>, tensor<2x3xi64>) -> tensor<2x3xi64>\n'
+            '    return %0 : tensor<2x3xi64>\n  }\n}\n')
+    got, ref = both(rx, client, text, [I.Tensor(a, "i64"), I.Tensor(b, "i64")])
+    assert np.array_equal(got[0].a, a * b) and np.array_equal(ref[0].a, a * b)
+
+
+def test_empty_and_scalar_shapes(rx, client):
+    t0 = _tt([0], "f32")
+    text = mod([t0], "tensor<f32>",
+               "    %%c = stablehlo.constant dense<1.500000e+00> : tensor<f32>\n"
+               "    %%0 = stablehlo.reduce(%%arg0 init: %%c) applies stablehlo.add across dimensions = [0] : (%s, tensor<f32>) -> tensor<f32>\n"
+               "    return %%0 : tensor<f32>\n" % t0)
+    got, ref = both(rx, client, text, [I.Tensor(np.zeros(0, np.float32), "f32")])
+    assert float(got[0].a) == 1.5 == float(ref[0].a)
+    text = mod(["tensor<f32>", "tensor<f32>"], "tensor<f32>", "    %0 = stablehlo.add %arg0, %arg1 : tensor<f32>\n    return %0 : tensor<f32>\n")
+    got, _ = gpu_run(rx, client, text, [I.Tensor(np.float32(2.0), "f32"), I.Tensor(np.float32(2.0), "f32")])
+    assert float(got[0].a) == 4.0   # test/core/ops.jl:1066-1082
