@@ -1,0 +1,152 @@
+"""CPU tests of the boundary and the host logic (no compute calls without a GPU):
+the shared library loads and exports every symbol the header declares, the error
+convention works, the StableHLO importer and the fusion planner accept what the
+reference prints and reject what they cannot run, and the kernel text written for
+each benchmark program compiles for gfx950 (hiprtc needs no device)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from _loader import load_pkg, load_programs, ROOT
+
+rx = load_pkg()
+P = load_programs()
+HEADER = os.path.join(ROOT, "include", "reactant_mi355x.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b([A-Za-z_][A-Za-z0-9_]*)\s*\(", text))
+    names -= {"defined", "void"}
+    funcs = {n for n in names if re.search(r"\b%s\s*\([^;{]*\)\s*;" % n, text)}
+    return funcs
+
+
+def test_library_exports_every_declared_symbol():
+    funcs = declared_symbols()
+    assert len(funcs) >= 45
+    lib = ctypes.CDLL(rx.LIB_PATH)
+    missing = [f for f in sorted(funcs) if not hasattr(lib, f)]
+    assert not missing, missing
+    # the throw hook is an exported data symbol (reference API.cpp:262)
+    hook = ctypes.c_void_p.in_dll(lib, "ReactantThrowError")
+    assert hook.value is None
+    # every declared function has a ctypes signature in the host mirror, and vice versa
+    assert funcs == set(rx.SIGNATURES), funcs ^ set(rx.SIGNATURES)
+
+
+def test_handles_are_validated_without_a_device():
+    assert rx.lib.RxOwns(None) == 0
+    assert rx.lib.RxOwns(ctypes.c_void_p(0x1234)) == 0
+    # calls on foreign handles fail cleanly with a message instead of dereferencing them
+    rx.lib.RxClearError()
+    assert rx.lib.ClientNumDevices(ctypes.c_void_p(0x1234)) == 0
+    assert b"client handle" in rx.lib.RxLastError()
+    rx.lib.RxClearError()
+    rx.lib.PjRtBufferFree(ctypes.c_void_p(0x1234))      # finalizer path: silently ignored
+    rx.lib.FreeFuture(None)
+    rx.lib.ExecutableFree(None)
+    assert rx.lib.RxLastError() == b""
+
+
+def test_throw_callback_is_invoked():
+    seen = []
+    CB = ctypes.CFUNCTYPE(None, ctypes.c_char_p)
+    cb = CB(lambda m: seen.append(m))
+    lib = ctypes.CDLL(rx.LIB_PATH)
+    hook = ctypes.c_void_p.in_dll(lib, "ReactantThrowError")
+    hook.value = ctypes.cast(cb, ctypes.c_void_p).value
+    try:
+        lib.BufferNDimensions.restype = ctypes.c_int64
+        lib.BufferNDimensions(ctypes.c_void_p(0x42))
+        assert seen and b"buffer handle" in seen[0]
+    finally:
+        hook.value = None
+        rx.lib.RxClearError()
+
+
+def test_client_creation_reports_errors_through_the_error_pointer():
+    import subprocess, sys
+    # in a child process: a machine without a GPU must get NULL + a message, not a crash
+    code = ("import sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+            "from _loader import load_pkg\nrx = load_pkg()\n"
+            "try:\n    rx.Client()\n    print('CLIENT-OK')\n"
+            "except rx.ReactantInternalError as e:\n    print('ERR:', e)\n" % (ROOT, os.path.join(ROOT, "tests")))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert "CLIENT-OK" in out.stdout or "ERR:" in out.stdout, out.stdout + out.stderr
+    # multi-node requests are refused before any device is touched
+    err = ctypes.c_char_p()
+    h = rx.lib.MakeGPUClient(0, 2, None, 0, 0.75, False, b"rocm", ctypes.byref(err), None)
+    assert not h and b"one process" in err.value
+    rx.lib.RxClearError()
+
+
+PROGRAMS = {
+    "sinsum_add": (lambda: P.sinsum_add(1 << 20), ["reduce", "reduce_final"]),
+    "stencil": (lambda: P.stencil(64, 64, 32, steps=3), ["map", "map", "map"]),
+    "stencil_full": (lambda: P.stencil(512, 512, 256, steps=2), ["map_stencil_lds", "map_stencil_lds"]),
+    "gemm": (lambda: P.gemm(512, 512, 512), ["gemm_f32"]),
+    "gemm_transposed": (lambda: P.gemm(512, 256, 128, form="transposed"), ["gemm_f32"]),
+    "mlp": (lambda: P.mlp(512, (256, 512, 512, 256)), ["gemm_bf16", "gemm_bf16", "gemm_bf16", "row"]),
+    "mlp_gelu_op": (lambda: P.mlp(512, (256, 512, 512, 256), gelu="op"), ["gemm_bf16", "gemm_bf16", "gemm_bf16", "row"]),
+    "fp8_linear": (lambda: P.fp8_linear(512, 512, 512), ["reduce", "reduce_final", "map", "gemm_f8", "row"]),
+    "fp8_linear_kn": (lambda: P.fp8_linear(512, 512, 512, weight_layout="kn", dot_form="direct"),
+                      ["reduce", "reduce_final", "map", "gemm_f8", "row"]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(PROGRAMS))
+def test_benchmark_programs_plan_and_compile_for_gfx950(name):
+    make, kinds = PROGRAMS[name]
+    report = rx.compile_offline(make())
+    got = re.findall(r"kind=(\w+)", report)
+    assert got == kinds, report
+    assert "code object:" in report
+
+
+def test_fusion_plan_of_the_full_size_stencil_is_one_kernel_per_timestep():
+    report = rx.compile_offline(P.stencil(512, 512, 256, steps=10))
+    launches = re.findall(r"\] (\w+) kind=(\w+)", report)
+    assert len(launches) == 10
+    assert len({k for k, _ in launches}) == 1           # ten launches of one compiled kernel
+    # compulsory traffic of one timestep on the halo'd arrays: 4 reads + 1 write of 262*518*518 doubles
+    assert "algo_bytes=%d" % (5 * 262 * 518 * 518 * 8) in report
+
+
+def test_generated_source_is_inspectable():
+    report = rx.compile_offline(P.sinsum_add(4096), with_source=True)
+    assert "rx_wave_reduce" in report or "rx_block_reduce" in report
+    assert "sinf(" in report and "extern \"C\" __global__" in report
+
+
+@pytest.mark.parametrize("text,needle", [
+    ("module { func.func @main(%a: tensor<4xf32>) -> tensor<4xf32> { %0 = stablehlo.frobnicate %a : tensor<4xf32>\n return %0 : tensor<4xf32> } }", "unsupported operation"),
+    ("module { func.func @main(%a: tensor<4xf32>) -> tensor<4xf32> { %0 = stablehlo.add %a, %b : tensor<4xf32>\n return %0 : tensor<4xf32> } }", "undefined value"),
+    ("module { func.func @main(%a: tensor<4xf32>, %b: tensor<5xf32>) -> tensor<4xf32> { %0 = stablehlo.add %a, %b : tensor<4xf32>\n return %0 : tensor<4xf32> } }", "type mismatch"),
+    ("module { func.func @main(%a: tensor<4xc64>) -> tensor<4xc64> { return %a : tensor<4xc64> } }", "unsupported element type"),
+    ("module { func.func @main(%a: tensor<4x3xf32>) -> tensor<2x2xf32> { %0 = stablehlo.slice %a [0:2, 2:4] : (tensor<4x3xf32>) -> tensor<2x2xf32>\n return %0 : tensor<2x2xf32> } }", "bounds out of range"),
+    ("module { func.func @main(%a: tensor<4xf32>) -> tensor<f32> { return %a : tensor<4xf32> } }", "declared"),
+    ("module { func.func @main(%a: tensor<4xf32> -> tensor<4xf32> { return %a : tensor<4xf32> } }", "parse error"),
+])
+def test_importer_rejects_bad_modules_with_a_message(text, needle):
+    with pytest.raises(rx.ReactantInternalError) as e:
+        rx.compile_offline(text)
+    assert needle in str(e.value)
+
+
+def test_host_side_array_conventions():
+    import numpy as np
+    # dims reversal: a Julia array of size (3, 4) travels as a row-major [4][3] buffer (src/xla/PJRT/Buffer.jl:9-17)
+    x = np.arange(12.0).reshape(3, 4)
+    raw = np.ascontiguousarray(rx.encode(x, "f64").T)
+    assert raw.shape == (4, 3) and raw[1, 2] == x[2, 1]
+    # narrow floats are packed to their storage bits and back
+    v = np.float32([1.0, -2.5, 0.3333, 448.0, 1e-3])
+    assert np.array_equal(rx.decode(rx.encode(v, "bf16"), "bf16"), np.float32([1.0, -2.5, 0.333984375, 448.0, 0.00099945068359375]))
+    assert rx.decode(rx.encode(v, "f8E4M3FN"), "f8E4M3FN").tolist() == [1.0, -2.5, 0.34375, 448.0, 0.001953125]
+    assert rx.PRIMITIVE_TYPE["f32"] == 11 and rx.PRIMITIVE_TYPE["bf16"] == 16 and rx.PRIMITIVE_TYPE["f8E4M3FN"] == 20
+    with pytest.raises(rx.ReactantInternalError):
+        rx.set_default_backend("tpu")
