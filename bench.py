@@ -27,6 +27,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of each dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+# scaled by the readings of a plain 1 GiB copy kernel (profiles/bench_all_configs_hbm_traffic.txt).
+# Counters cannot be read from inside this process, so the figures of that profile are quoted here;
+# they are reported only for the kernel and shape they were measured on.
+MEASURED_TRAFFIC_BYTES = {
+    "rx_stencil_k0_stencil": 3540.4e6,
+    "rx_sinsum_add_k0_reduce": 537.1e6,
+    "rx_gemm_k0_gemm": 741.5e6,
+    "rx_mlp_k1_gemm": 671.8e6,
+    "rx_fp8_linear_k2_gemm": 2365.8e6,
+}
+_FULL_SIZE = [True]   # cleared by --small: the table only holds the full-size shapes
+
+
+def _traffic(kernel):
+    return MEASURED_TRAFFIC_BYTES.get(kernel) if _FULL_SIZE[0] else None
+
+
 PEAK_HBM_GBS = 8000.0
 PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f8": 5000.0}
 
@@ -110,7 +128,8 @@ def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=1
         "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"] if launches else None, "launches_per_step": nk,
                      "kernel_ms": kms, "achieved": algo_launch / (kms * 1e-3) / 1e9 if kms else None,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": algo_launch / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None, "traffic": None},
+                     "frac": algo_launch / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None,
+                     "traffic": _traffic(launches[0]["kernel"]) if launches else None},
         "plan": exe.report(),
     }
 
@@ -131,7 +150,7 @@ def bench_sinsum(rx, client, P, steps, warmup, n=1 << 26):
             "check": {"got": got, "f64_reference": exact},
             "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"], "kernel_ms": kms,
                          "achieved": algo / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": algo / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None}}
+                         "frac": algo / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _traffic(launches[0]["kernel"])}}
 
 
 def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype):
@@ -147,7 +166,7 @@ def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype):
             "dot_tflops_kernel_time_only": flops / (dms * 1e-3) / 1e12,
             "roofline": {"bound": "mfma", "kernel": launches[big]["kernel"], "kernel_ms": float(mean_ms[big]),
                          "achieved": ach, "peak": PEAK_TFLOPS[dtype_key], "unit": "TFLOP/s",
-                         "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": None}}
+                         "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": _traffic(launches[big]["kernel"])}}
 
 
 def bench_gemm(rx, client, P, steps, warmup, n=4096):
@@ -226,6 +245,7 @@ def main():
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024)}
+    _FULL_SIZE[0] = not args.small
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
     copy_ms = rx._call("RxCalibrationCopy", client.default_device().handle, 1 << 30, 10)

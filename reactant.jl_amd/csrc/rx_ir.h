@@ -79,6 +79,7 @@ struct Node {
 
 struct Graph {
   std::string name;
+  std::string module_name;            // symbol of the module ("reactant_<fn>" in what Reactant prints), may be empty
   std::vector<Node> nodes;            // topologically ordered
   std::vector<int> params;            // node ids of @main arguments
   std::vector<int> results;           // node ids returned

@@ -352,13 +352,14 @@ struct P {
   Cur c;
   std::map<std::string, RawFunc> funcs;
   std::vector<std::string> func_order;
+  std::string module_name;
   P(const char* t, size_t n) : c(t, n) {}
 
   void parse() {
     while (!c.eof()) {
       if (c.peek() == '#') { while (c.i < c.n && c.s[c.i] != '\n') ++c.i; continue; }
       if (c.accept("module")) {
-        if (c.peek() == '@') c.sym();
+        if (c.peek() == '@') module_name = c.sym();
         if (c.accept("attributes")) c.balanced('{', '}');
         c.expect("{");
         continue;
@@ -1208,6 +1209,7 @@ Graph parse_module(const char* text, size_t len) {
   if (!mainf) throw Error("StableHLO import: module has no @main function");
   Builder b(p);
   b.g.name = mainf->name;
+  b.g.module_name = p.module_name;
   std::vector<int> args;
   for (size_t k = 0; k < mainf->args.size(); ++k) {
     Node n;

@@ -316,7 +316,12 @@ struct Planner {
   std::string finalize(const std::string& text) {
     auto it = dedupe.find(text);
     if (it != dedupe.end()) return it->second;
-    std::string base = "rxk" + std::to_string(kcount++);
+    // kernel symbols carry the module's name so that profiles of several programs stay readable
+    std::string mod;
+    for (char ch : g.module_name) mod += (isalnum((unsigned char)ch) ? ch : '_');
+    if (mod.rfind("reactant_", 0) == 0) mod = mod.substr(9);
+    if (mod.size() > 24) mod.resize(24);
+    std::string base = "rx_" + (mod.empty() ? std::string("mod") : mod) + "_k" + std::to_string(kcount++);
     dedupe[text] = base;
     src << named(text, base);
     return base;
