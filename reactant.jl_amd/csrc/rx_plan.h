@@ -45,7 +45,10 @@ struct PlanOptions {
   bool mfma = true;             // use the MFMA GEMM skeletons for eligible dot_generals
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
-  int lds_tile[3] = {3, 8, 64};  // outputs per workgroup tile (slowest .. fastest dimension)
+  int lds_tile[3] = {3, 4, 128};  // outputs per workgroup tile (slowest .. fastest dimension)
+  bool stencil_march = false;   // stencil maps: a workgroup marches along the slowest dimension with a ring of planes in LDS
+  int march_depth = 3;          // planes of global loads kept in flight (in registers) ahead of their use
+  int march_planes = 32;        // planes produced per workgroup when marching
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once
