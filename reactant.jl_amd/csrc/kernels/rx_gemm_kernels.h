@@ -303,8 +303,10 @@ RX_DEV int rx_swz_kc(int row, int c) {
 //   TR tiles ([k][o]): which rows are read together depends on the element size
 template <int ESIZE, int CPR>
 RX_DEV int rx_swz_tr(int row, int c) {
-  if constexpr (ESIZE == 2) return c ^ (((row & 3) << 1) & (CPR - 1));        // 4 rows x 32 B per 16 lanes
-  else if constexpr (ESIZE == 1) return c ^ ((row & 7) & (CPR - 1));          // 8 rows x 16 B per 16 lanes
+  // 32 lanes of a transpose read touch 4 rows x 64 B (16-bit) or 8 rows x 32 B (8-bit): each row
+  // is moved to its own 64 B / 32 B group so that the 32 lanes cover all 64 banks once
+  if constexpr (ESIZE == 2) return c ^ (((row & 3) << 2) & (CPR - 1));
+  else if constexpr (ESIZE == 1) return c ^ (((row & 7) << 1) & (CPR - 1));
   else return c ^ ((((row >> 2) & 1) << 3) & (CPR - 1));                      // rows k, k+4 read in one instruction
 }
 
@@ -369,6 +371,14 @@ template <> struct rx_frag_sw<rx_mma_f8> {
 };
 
 template <int V> struct rx_int { static constexpr int value = V; };
+
+// the instruction scheduler may not move anything across this point
+#ifndef RX_GEMM_INTERLEAVE
+#define RX_GEMM_INTERLEAVE 1
+#endif
+#ifndef RX_SCHED_FENCE
+#define RX_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#endif
 
 // wait until at most N of this wavefront's vector-memory operations are outstanding
 template <int N>
@@ -475,6 +485,24 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 #pragma unroll
       for (int j = 0; j < TN; ++j) MMA::mma(acc[i][j], fb[buf][j], fa[buf][i]);
   };
+  // Ask the scheduler for the pattern "one MFMA, one LDS read, ..." over a step: the reads of the
+  // next step trickle out under this step's MFMAs instead of going out in one burst.
+  constexpr int RD_A = A_KC ? (sizeof(E) == 1 ? 2 : 1) : (sizeof(E) == 2 ? 2 : 4);
+  constexpr int RD_B = B_KC ? (sizeof(E) == 1 ? 2 : 1) : (sizeof(E) == 2 ? 2 : 4);
+  constexpr int NRD = TM * RD_A + TN * RD_B;
+  constexpr int NMF = TM * TN * (sizeof(E) == 4 ? 4 : 1);
+  auto interleave = [&]() {
+#if RX_GEMM_INTERLEAVE
+    constexpr int PAIRS = NRD < NMF ? NRD : NMF;
+#pragma unroll
+    for (int k = 0; k < PAIRS; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+    }
+    if constexpr (NMF > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, NMF - PAIRS, 0);
+    if constexpr (NRD > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, NRD - PAIRS, 0);
+#endif
+  };
   auto publish = [&]() {
     asm volatile("" ::: "memory");   // compiler-only fences: LDS reads must not move across the barrier
     __builtin_amdgcn_s_barrier();    // bare barrier: __syncthreads() would also wait for the younger loads
@@ -494,8 +522,11 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
     const RX_LDS E* sa = lds + (kt % S) * STAGE;
 #pragma unroll
     for (int s = 0; s + 1 < NS; ++s) {
+      // keep the order "LDS reads of the next step, then the MFMAs of this step": the reads then
+      // complete under a full step of MFMAs instead of being waited for right after issue
       load_frags((p + s + 1) & 1, sa, (s + 1) * MMA::KS);
       mma_all((p + s) & 1);
+      interleave();
     }
     if (kt + 1 < KT) {
       // tile kt+1 has landed once only the (S-2) tiles after it are still in flight
@@ -505,6 +536,7 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
       load_frags((p + NS) & 1, lds + ((kt + 1) % S) * STAGE, 0);
     }
     mma_all((p + NS - 1) & 1);
+    if (kt + 1 < KT) interleave(); else RX_SCHED_FENCE();
   };
   if constexpr (NS % 2 == 0) {
     for (int kt = 0; kt < KT; ++kt) tile(rx_int<0>{}, kt);
