@@ -201,6 +201,7 @@ std::string Emitter::emit_load(int node, const Index& ix) {
     }
   } else {
     raw = "in" + std::to_string(slot) + "[" + (dims.empty() ? std::string("0") : linear(ix, dims)) + "]";
+    if (!dims.empty()) ++unsafe_loads_;
   }
   std::string v = fresh();
   line(std::string("const ") + info(n.ty.dt).ctype + " " + v + " = " + load_conv(n.ty.dt, raw) + ";");
@@ -437,10 +438,36 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       if (never || o.ty.numel() == 0) return pv;
       if (conds.empty() && pre.empty()) return emit(n.in[0], oi);
       std::string v = fresh();
-      line(CT + " " + v + " = " + pv + ";");
       std::string cond;
       for (auto& c : conds) cond += (cond.empty() ? "" : " && ") + c;
-      line("if (" + (cond.empty() ? std::string("true") : cond) + ") {");
+      if (cond.empty()) cond = "true";
+      if (branchless_guards) {
+        const int unsafe0 = unsafe_loads_;
+        const std::string before = take_code();
+        push_scope();
+        for (auto& p : pre) line(p);
+        std::string inner = emit(n.in[0], oi);
+        const std::string code = take_code();
+        out_ << before;
+        if (unsafe_loads_ == unsafe0) {
+          // straight-line: the values stay in scope of the enclosing block
+          out_ << code;
+          auto top = scopes_.back();
+          scopes_.pop_back();
+          for (auto& kv : top) scopes_.back().insert(kv);
+          line("const " + CT + " " + v + " = (" + cond + ") ? " + inner + " : " + pv + ";");
+          return v;
+        }
+        line(CT + " " + v + " = " + pv + ";");
+        line("if (" + cond + ") {");
+        out_ << code;
+        line("  " + v + " = " + inner + ";");
+        pop_scope();
+        line("}");
+        return v;
+      }
+      line(CT + " " + v + " = " + pv + ";");
+      line("if (" + cond + ") {");
       indent += 2;
       push_scope();
       for (auto& p : pre) line(p);
@@ -472,9 +499,36 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       if (never || u.ty.numel() == 0) return emit(n.in[0], oi);
       if (conds.empty()) return emit(n.in[1], ui);
       std::string v = fresh();
-      line(CT + " " + v + ";");
       std::string cond;
       for (auto& c : conds) cond += (cond.empty() ? "" : " && ") + c;
+      if (branchless_guards) {
+        const int unsafe0 = unsafe_loads_;
+        const std::string before = take_code();
+        push_scope();
+        std::string a = emit(n.in[1], ui);
+        const std::string code_a = take_code();
+        pop_scope();
+        push_scope();
+        std::string b = emit(n.in[0], oi);
+        const std::string code_b = take_code();
+        pop_scope();
+        out_ << before;
+        if (unsafe_loads_ == unsafe0) {
+          out_ << code_a << code_b;
+          line("const " + CT + " " + v + " = (" + cond + ") ? " + a + " : " + b + ";");
+          return v;
+        }
+        line(CT + " " + v + ";");
+        line("if (" + cond + ") {");
+        out_ << code_a;
+        line("  " + v + " = " + a + ";");
+        line("} else {");
+        out_ << code_b;
+        line("  " + v + " = " + b + ";");
+        line("}");
+        return v;
+      }
+      line(CT + " " + v + ";");
       line("if (" + cond + ") {");
       indent += 2;
       push_scope();

@@ -62,6 +62,11 @@ class Emitter {
   // the hook returns true and the expression to read instead of global memory.
   std::function<bool(int slot, const std::vector<int64_t>& off, std::string* expr)> tile_hook;
 
+  // pad / dynamic_update_slice guards: when everything read under a guard comes from a tile or a
+  // preloaded vector (so evaluating it at a point the guard excludes cannot fault), evaluate both
+  // sides and select, instead of branching per element
+  bool branchless_guards = false;
+
   std::string emit(int node, const Index& ix);
   std::string take_code() { std::string s = out_.str(); out_.str(""); return s; }
   void line(const std::string& s) { out_ << std::string(indent, ' ') << s << "\n"; }
@@ -82,6 +87,7 @@ class Emitter {
   std::ostringstream out_;
   std::vector<std::map<std::string, std::string>> scopes_{1};
   int tmp_ = 0;
+  int unsafe_loads_ = 0;   // loads emitted as plain global reads at a computed index
   std::vector<int64_t> root_dims_;
   std::vector<std::string> root_vars_;
   bool allow_direct_ = false;

@@ -115,6 +115,8 @@ struct Planner {
   std::vector<char> prev_mat;       // materialization decided by the previous analysis sweep (used for producers)
   std::vector<char> force_mat;      // chosen cut points below a dot_general with several consumers
   std::vector<int> buf_of;          // node -> buffer id (materialized nodes)
+  std::map<int, int> fuse_prev;     // stencil root -> the stencil step it evaluates in LDS instead of reading from memory
+  std::set<int> lds_only;           // the steps absorbed that way: no launch, no buffer
   std::ostringstream src;
   int kcount = 0;
 
@@ -604,37 +606,68 @@ struct Planner {
   // owns a TZ x TY x TX block of outputs, loads that input's block plus halo into LDS once with
   // aligned 16-byte loads, and every neighbour access becomes an LDS read.  Inputs read only at
   // the output's own position are still streamed from global memory with vector loads.
-  bool emit_map_lds(int root) {
+  // Tile order of the stencil kernels.  Workgroups are dealt round-robin to the 8 XCDs, each with
+  // its own L2.  The y-tiles are cut into slabs of `sy` tiles; XCD k owns slabs k, k+8, ... and
+  // walks each of them layer by layer in z, so the planes that consecutive layers share (and the
+  // rows that neighbouring tiles of a layer share) are still in that XCD's L2 when they are asked
+  // for again.  Declares x0, y0, z0; returns the number of workgroups to launch.
+  int64_t emit_tile_order(std::ostringstream& o, int64_t ntx, int64_t nty, int64_t ntz, int TX, int TY, int TZ, int64_t default_sy = 0) {
+    const int64_t nblocks = ntx * nty * ntz;
+    if (!(opt.xcd_slabs && nty >= 16)) {
+      o << "  const unsigned tile = rx_xcd_remap(blockIdx.x, " << nblocks << "u);\n";
+      o << "  const int x0 = (int)(tile % " << ntx << "u) * " << TX << ";\n";
+      o << "  const int y0 = (int)((tile / " << ntx << "u) % " << nty << "u) * " << TY << ";\n";
+      o << "  const int z0 = (int)(tile / " << ntx * nty << "u) * " << TZ << ";\n";
+      return nblocks;
+    }
+    int64_t sy = opt.slab_ytiles > 0 ? opt.slab_ytiles : default_sy > 0 ? default_sy : (nty + 7) / 8;
+    sy = std::min<int64_t>(sy, (nty + 7) / 8);
+    const int64_t nslabs = (nty + sy - 1) / sy, rounds = (nslabs + 7) / 8;
+    const int64_t per_slab = ntz * ntx * sy;
+    o << "  const unsigned xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;\n";
+    o << "  const unsigned slab = (j / " << per_slab << "u) * 8u + xcd, r = j % " << per_slab << "u;\n";
+    o << "  const unsigned tz = r / " << ntx * sy << "u, rr = r % " << ntx * sy << "u;\n";
+    o << "  const unsigned ty = slab * " << sy << "u + rr / " << ntx << "u;\n";
+    o << "  if (ty >= " << nty << "u) return;\n";
+    o << "  const int x0 = (int)(rr % " << ntx << "u) * " << TX << ";\n";
+    o << "  const int y0 = (int)ty * " << TY << ";\n";
+    o << "  const int z0 = (int)tz * " << TZ << ";\n";
+    return 8 * rounds * per_slab;
+  }
+
+  struct Halo { int64_t lo[3] = {0, 0, 0}, hi[3] = {0, 0, 0}; bool ok = true; };
+  struct StencilProbe {
+    int vec = 1;
+    std::vector<int> staged;       // same-shape inputs read at three or more constant offsets
+    std::map<int, Halo> halos;     // per staged input: how far the offsets reach in each dimension
+  };
+  void stencil_emitter(Emitter& em, int root, int vec, const std::vector<std::string>& vars) {
+    em.idx64 = needs64(cone_nodes(root));
+    em.set_root(g.nodes[root].ty.dims, vars, true);
+    em.vec = vec;
+    em.allow_shifted = false;
+    em.excess_precision = opt.excess_precision;
+    em.branchless_guards = opt.branchless_guards;
+    em.indent = 8;
+  }
+  bool probe_stencil(int root, StencilProbe* sp) {
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
-    if (!opt.lds_stencil || rn.ty.rank() != 3) return false;
-    const int vec = pick_vec(rn.ty);
-    const int64_t numel = rn.ty.numel();
-    if (numel < opt.slab_min_numel || vec < 2) return false;
-    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
-    auto make_emitter = [&](Emitter& em) {
-      em.idx64 = needs64(cone_nodes(root));
-      em.set_root(dims, {"i0", "i1", "i2"}, true);
-      em.vec = vec;
-      em.allow_shifted = false;
-      em.direct_expr = vec_name;
-      em.indent = 8;
-    };
-    // pass 1: find the stencil inputs and their halos
+    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::DotGeneral) return false;
+    sp->vec = pick_vec(rn.ty);
+    if (rn.ty.numel() < opt.slab_min_numel || sp->vec < 2) return false;
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
-    probe.excess_precision = opt.excess_precision;
-    make_emitter(probe);
+    stencil_emitter(probe, root, sp->vec, {"i0", "i1", "i2"});
+    probe.direct_expr = vec_name;
     probe.emit(root, root_index(dims));
-    struct Halo { int64_t lo[3] = {0, 0, 0}, hi[3] = {0, 0, 0}; int count = 0; bool ok = true; };
-    std::map<int, Halo> halos;  // keyed by node
     std::map<int, std::set<std::vector<int64_t>>> offs;
+    std::map<int, Halo> halos;
     for (auto& l : probe.loads) {
       const Node& ln = g.nodes[l.node];
       if (ln.ty.dims != dims) continue;
       if (!l.affine) { halos[l.node].ok = false; continue; }
       offs[l.node].insert(l.off);
     }
-    std::vector<int> staged;
     for (auto& kv : offs) {
       if (kv.second.size() < 3 || !halos[kv.first].ok) continue;
       Halo& h = halos[kv.first];
@@ -643,10 +676,37 @@ struct Planner {
       if (h.lo[0] > 4 || h.hi[0] > 4 || h.lo[1] > 4 || h.hi[1] > 4 || h.lo[2] > 8 || h.hi[2] > 8) continue;
       const int es = info(g.nodes[kv.first].ty.dt).size;
       if (es != 4 && es != 8) continue;
-      if (info(g.nodes[kv.first].ty.dt).size != info(rn.ty.dt).size) continue;  // same vector width as the output
-      staged.push_back(kv.first);
+      if (es != info(rn.ty.dt).size) continue;  // same vector width as the output
+      sp->staged.push_back(kv.first);
+      sp->halos[kv.first] = h;
     }
-    if (staged.empty()) return false;
+    return !sp->staged.empty();
+  }
+
+  bool emit_map_lds(int root) {
+    const Node& rn = g.nodes[root];
+    const auto& dims = rn.ty.dims;
+    StencilProbe sp;
+    if (!probe_stencil(root, &sp)) return false;
+    const int vec = sp.vec;
+    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
+    auto make_emitter = [&](Emitter& em) {
+      stencil_emitter(em, root, vec, {"i0", "i1", "i2"});
+      em.direct_expr = vec_name;
+    };
+    std::vector<int>& staged = sp.staged;
+    std::map<int, Halo>& halos = sp.halos;
+    {
+      auto pf = fuse_prev.find(root);
+      if (pf != fuse_prev.end()) {
+        const int prev = pf->second;
+        if (emit_map_lds2(root, prev, sp)) return true;
+        // not fused after all: the producer gets its own launch first
+        fuse_prev.erase(pf);
+        lds_only.erase(prev);
+        emit_map(prev);
+      }
+    }
     if (opt.stencil_march && staged.size() == 1) {
       const Halo& h = halos[staged[0]];
       if (emit_map_march(root, staged[0], h.lo, h.hi)) return true;
@@ -674,7 +734,6 @@ struct Planner {
 
     // pass 2: emit with the staged inputs redirected to LDS
     Emitter em(g, [&](int x) { return x != root && mat[x]; });
-    em.excess_precision = opt.excess_precision;
     make_emitter(em);
     em.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
       const int node = em.inputs[slot];
@@ -694,7 +753,6 @@ struct Planner {
     const std::string it = em.idx_t();
     const std::string kname = "@K@_stencil";
     const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + TZ - 1) / TZ;
-    const int64_t nblocks = ntx * nty * ntz;
     std::ostringstream o;
     o << "// stencil map through LDS halo tiles (" << TZ << "x" << TY << "x" << TX << " outputs per workgroup): " << describe(root) << " -> " << rn.ty.str() << "\n";
     o << signature(kname, em.inputs, {{info(rn.ty.dt).stype, "out0"}}) << " {\n";
@@ -703,10 +761,7 @@ struct Planner {
       const Geo& ge = geo[s];
       o << "  __shared__ __attribute__((aligned(16))) " << info(g.nodes[s].ty.dt).stype << " lds" << slot << "[" << ge.pz * ge.py * ge.lx << "];\n";
     }
-    o << "  const unsigned tile = rx_xcd_remap(blockIdx.x, " << nblocks << "u);\n";
-    o << "  const int x0 = (int)(tile % " << ntx << "u) * " << TX << ";\n";
-    o << "  const int y0 = (int)((tile / " << ntx << "u) % " << nty << "u) * " << TY << ";\n";
-    o << "  const int z0 = (int)(tile / " << ntx * nty << "u) * " << TZ << ";\n";
+    const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, TZ);
     for (int s : staged) {
       const int slot = em.slot_of(s);
       const Geo& ge = geo[s];
@@ -780,7 +835,7 @@ struct Planner {
     Launch L;
     L.kernel = named(kname, kb_final);
     L.kind = "map_stencil_lds";
-    L.grid[0] = (unsigned)nblocks;
+    L.grid[0] = (unsigned)launch_blocks;
     L.block[0] = kBlock;
     for (int i : em.inputs) L.args.push_back(buffer_for(i));
     L.args.push_back(buffer_for(root));
@@ -790,8 +845,221 @@ struct Planner {
     return true;
   }
 
+  // ------------------------------------------------------------------ two stencil steps in one kernel
+  // `root` is a stencil of `prev`, which is itself a stencil of some array A and has no other
+  // reader.  The workgroup loads A's tile with both halos into LDS, evaluates `prev` on the
+  // output tile plus root's halo into registers, writes those values over the A tile (after a
+  // barrier), and evaluates `root` from them.  `prev` never reaches global memory.  The values of
+  // `prev` are computed by the same expression at the same points as in a kernel of its own, so
+  // the result is bit-identical to the two-kernel form.
+  bool emit_map_lds2(int root, int prev, const StencilProbe& spR) {
+    const Node& rn = g.nodes[root];
+    const Node& pn = g.nodes[prev];
+    const auto& dims = rn.ty.dims;
+    if (pn.ty.dims != dims || pn.ty.dt != rn.ty.dt) return false;
+    StencilProbe spP;
+    if (!probe_stencil(prev, &spP) || spP.staged.size() != 1 || spP.vec != spR.vec) return false;
+    const int src = spP.staged[0];
+    if (g.nodes[src].ty.dims != dims) return false;
+    const int vec = spR.vec;
+    const Halo hR = spR.halos.at(prev), hP = spP.halos.at(src);
+    const int TZ = opt.lds_tile2[0], TY = opt.lds_tile2[1], TX = opt.lds_tile2[2];
+    if (TZ < 1 || TX % vec) return false;
+    const int TXV = TX / vec;
+    // NB threads cover PZ planes of the output tile at a time
+    const int NB = opt.lds2_threads;
+    if (NB < 64 || NB > 1024 || NB % 64 || NB % (TXV * TY)) return false;
+    const int PZ = NB / (TXV * TY);
+    if (TZ % PZ) return false;
+    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
+    auto up = [&](int64_t v) { return (v + vec - 1) / vec * vec; };
+    // region of `prev` values (B) and of A values (A), relative to the output tile origin
+    const int64_t bxl = up(hR.lo[2]), bxh = up(hR.hi[2]);
+    const int64_t BZ = TZ + hR.lo[0] + hR.hi[0], BY = TY + hR.lo[1] + hR.hi[1], BX = TX + bxl + bxh;
+    const int64_t axl = up(hP.lo[2]), axh = up(hP.hi[2]);
+    const int64_t AZ = BZ + hP.lo[0] + hP.hi[0], AY = BY + hP.lo[1] + hP.hi[1], AX = BX + axl + axh;
+    const int64_t BXV = BX / vec, AXV = AX / vec;
+    const int64_t totalA = AZ * AY * AXV, totalB = BZ * BY * BXV;
+    const int es = info(rn.ty.dt).size;
+    const int64_t lds_bytes = std::max(totalA, totalB) * vec * es;
+    if (lds_bytes > 80 * 1024) return false;
+    const int64_t nitA = (totalA + NB - 1) / NB, nitB = (totalB + NB - 1) / NB;
+    if (nitB * vec * es / 4 > 96) return false;   // registers that hold the first step's values
+    const std::string st = info(rn.ty.dt).stype;
+    const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+
+    // first step, evaluated at (j0, j1, j2) = a point of region B (clamped into the array)
+    Emitter eb(g, [&](int x) { return x != prev && mat[x]; });
+    stencil_emitter(eb, prev, vec, {"j0", "j1", "j2"});
+    eb.direct_expr = [](int slot, int64_t D) { return "b" + vec_name(slot, D); };
+    eb.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+      if (eb.inputs[slot] != src) return false;
+      std::ostringstream e;
+      e << "lds[((bz + " << (off[0] + hP.lo[0]) << ") * " << AY << " + (by + " << (off[1] + hP.lo[1]) << ")) * " << AX << " + bxe + l + " << (axl + off[2]) << "]";
+      *expr = e.str();
+      return true;
+    };
+    Index jb(3);
+    for (int d = 0; d < 3; ++d) { jb[d].var = "j" + std::to_string(d); jb[d].lo = 0; jb[d].hi = dims[d] - 1; }
+    std::string valB = eb.emit(prev, jb);
+    std::string bodyB = eb.take_code();
+    for (auto& dv : eb.direct_vecs) if (dv.second != 0) return false;
+
+    // second step, evaluated at the output point; slots continue the first step's numbering
+    Emitter ec(g, [&](int x) { return x != root && mat[x]; });
+    stencil_emitter(ec, root, vec, {"i0", "i1", "i2"});
+    ec.idx64 = ec.idx64 || eb.idx64;
+    ec.inputs = eb.inputs;
+    ec.direct_expr = vec_name;
+    ec.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+      if (ec.inputs[slot] != prev) return false;
+      std::ostringstream e;
+      e << "lds[((lz + " << (off[0] + hR.lo[0]) << ") * " << BY << " + (ly + " << (off[1] + hR.lo[1]) << ")) * " << BX << " + lxe + l + " << (bxl + off[2]) << "]";
+      *expr = e.str();
+      return true;
+    };
+    std::string valC = ec.emit(root, root_index(dims));
+    std::string bodyC = ec.take_code();
+    for (auto& dv : ec.direct_vecs) if (dv.second != 0) return false;
+    // every read of `prev` must have gone to the tile
+    for (auto& l : ec.loads) if (l.node == prev && !l.affine) return false;
+    const std::string it = ec.idx_t();
+    const bool i64 = ec.idx64;
+    const int prev_slot = ec.slot_of(prev);
+
+    const std::string kname = "@K@_stencil2";
+    const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + TZ - 1) / TZ;
+    std::ostringstream o;
+    o << "// two stencil steps through one LDS tile (" << TZ << "x" << TY << "x" << TX << " outputs per workgroup): " << describe(prev) << " ; " << describe(root)
+      << " -> " << rn.ty.str() << "\n";
+    {
+      std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(NB) + ") void " + kname + "(";
+      for (size_t k = 0; k < ec.inputs.size(); ++k) {
+        if ((int)k == prev_slot) continue;
+        s += ptr_decl(info(g.nodes[ec.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k)) + ", ";
+      }
+      s += ptr_decl(st, false, "out0") + ")";
+      o << s << " {\n";
+    }
+    o << "  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];\n";
+    o << "  " << st << "* const lds = reinterpret_cast<" << st << "*>(rx_smem);\n";
+    const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, TZ, std::max(1, 16 / TY));
+    const std::string LL = i64 ? "LL" : "";
+    // stage A: the source tile with both halos; out-of-array cells are clamped (never used)
+    {
+      const int sslot = ec.slot_of(src);
+      o << "  {\n    " << vt << " t[" << nitA << "];\n";
+      o << "#pragma unroll\n    for (int q = 0; q < " << nitA << "; ++q) {\n";
+      o << "      const int v = threadIdx.x + q * " << NB << ";\n";
+      o << "      const int xv = v % " << AXV << ", rw = v / " << AXV << ";\n";
+      o << "      const int yy = rw % " << AY << ", zz = rw / " << AY << ";\n";
+      o << "      const " << it << " gz = rx_clamp_idx<" << it << ">(z0 - " << (hR.lo[0] + hP.lo[0]) << " + zz, " << Z - 1 << ");\n";
+      o << "      const " << it << " gy = rx_clamp_idx<" << it << ">(y0 - " << (hR.lo[1] + hP.lo[1]) << " + yy, " << Y - 1 << ");\n";
+      o << "      const " << it << " gx = rx_clamp_idx<" << it << ">(x0 - " << (bxl + axl) << " + xv * " << vec << ", " << X - vec << ");\n";
+      o << "      t[q] = rx_load<" << vt << ">(in" << sslot << " + (gz * " << Y << " + gy) * " << X << LL << " + gx);\n";
+      o << "    }\n";
+      o << "#pragma unroll\n    for (int q = 0; q < " << nitA << "; ++q) {\n";
+      o << "      const int v = threadIdx.x + q * " << NB << ";\n";
+      o << "      if (v < " << totalA << ") rx_store(lds + v * " << vec << ", t[q]);\n";
+      o << "    }\n  }\n";
+    }
+    // loads of the streamed inputs of both steps are issued while the tile settles in LDS; points
+    // of region B outside the array are evaluated at clamped coordinates (their values are never used)
+    auto vts_of = [&](Emitter& em, int slot) { return "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">"; };
+    for (auto& dv : eb.direct_vecs) o << "  " << vts_of(eb, dv.first) << " b" << vec_name(dv.first, 0) << "q[" << nitB << "];\n";
+    if (!eb.direct_vecs.empty()) {
+      o << "#pragma unroll\n  for (int q = 0; q < " << nitB << "; ++q) {\n";
+      o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << totalB - 1 << ");\n";
+      o << "    const int bxv = v % " << BXV << ", brw = v / " << BXV << ";\n";
+      o << "    const int by = brw % " << BY << ", bz = brw / " << BY << ";\n";
+      o << "    const " << it << " j0 = rx_clamp_idx<" << it << ">(z0 - " << hR.lo[0] << " + bz, " << Z - 1 << ");\n";
+      o << "    const " << it << " j1 = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + by, " << Y - 1 << ");\n";
+      o << "    const " << it << " j2b = rx_clamp_idx<" << it << ">(x0 - " << bxl << " + bxv * " << vec << ", " << X - vec << ");\n";
+      o << "    const " << it << " linb = (j0 * " << Y << " + j1) * " << X << LL << " + j2b;\n";
+      for (auto& dv : eb.direct_vecs)
+        o << "    b" << vec_name(dv.first, 0) << "q[q] = " << "rx_load" << "<" << vts_of(eb, dv.first) << ">(in" << dv.first << " + linb);\n";
+      o << "  }\n";
+    }
+    o << "  const int lzb = threadIdx.x / " << TXV * TY << ", lrem = threadIdx.x % " << TXV * TY << ";\n";
+    o << "  const int ly = lrem / " << TXV << ", lxe = (lrem % " << TXV << ") * " << vec << ";\n";
+    o << "  const " << it << " i1 = rx_min<" << it << ">(y0 + ly, " << Y - 1 << "), i2b = rx_min<" << it << ">(x0 + lxe, " << X - vec << ");\n";
+    o << "  const bool live = y0 + ly < " << Y << " && x0 + lxe < " << X << ";\n";
+    o << "  __syncthreads();\n";
+    // stage B: first step on region B, kept in registers until every wavefront has read the tile
+    o << "  " << vt << " sb[" << nitB << "];\n";
+    o << "#pragma unroll\n  for (int q = 0; q < " << nitB << "; ++q) {\n";
+    o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << totalB - 1 << ");\n";
+    o << "    const int bxv = v % " << BXV << ", brw = v / " << BXV << ";\n";
+    o << "    const int by = brw % " << BY << ", bz = brw / " << BY << ", bxe = bxv * " << vec << ";\n";
+    o << "    const " << it << " j0 = rx_clamp_idx<" << it << ">(z0 - " << hR.lo[0] << " + bz, " << Z - 1 << ");\n";
+    o << "    const " << it << " j1 = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + by, " << Y - 1 << ");\n";
+    o << "    const " << it << " j2b = rx_clamp_idx<" << it << ">(x0 - " << bxl << " + bxe, " << X - vec << ");\n";
+    for (auto& dv : eb.direct_vecs)
+      o << "    const " << vts_of(eb, dv.first) << " b" << vec_name(dv.first, 0) << " = b" << vec_name(dv.first, 0) << "q[q];\n";
+    o << "#pragma unroll\n    for (int l = 0; l < " << vec << "; ++l) {\n";
+    o << "      const " << it << " j2 = j2b + l;\n";
+    o << bodyB;
+    o << "      sb[q].v[l] = " << Emitter::store_conv(pn.ty.dt, valB) << ";\n    }\n";
+    o << "  }\n";
+    // streamed inputs of the second step: in flight across the barriers
+    for (auto& dv : ec.direct_vecs) o << "  " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << "z[" << TZ / PZ << "];\n";
+    if (!ec.direct_vecs.empty()) {
+      o << "#pragma unroll\n  for (int lk = 0; lk < " << TZ / PZ << "; ++lk) {\n";
+      o << "    const int lz = lk * " << PZ << " + lzb;\n";
+      o << "    const " << it << " i0c = rx_clamp_idx<" << it << ">(z0 + lz, " << Z - 1 << ");\n";
+      o << "    const " << it << " linc = (i0c * " << Y << " + i1) * " << X << LL << " + i2b;\n";
+      for (auto& dv : ec.direct_vecs)
+        o << "    " << vec_name(dv.first, 0) << "z[lk] = " << "rx_load" << "<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + linc);\n";
+      o << "  }\n";
+    }
+    o << "  __syncthreads();\n";
+    o << "#pragma unroll\n  for (int q = 0; q < " << nitB << "; ++q) {\n";
+    o << "    const int v = threadIdx.x + q * " << NB << ";\n";
+    o << "    if (v < " << totalB << ") rx_store(lds + v * " << vec << ", sb[q]);\n";
+    o << "  }\n";
+    o << "  __syncthreads();\n";
+    // stage C: second step on the output tile
+    o << "  if (!live) return;\n";
+    o << "#pragma unroll\n  for (int lk = 0; lk < " << TZ / PZ << "; ++lk) {\n";
+    o << "    const int lz = lk * " << PZ << " + lzb;\n";
+    o << "    const " << it << " i0 = z0 + lz;\n";
+    o << "    if (i0 >= " << Z << ") break;\n";
+    o << "    const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
+    for (auto& dv : ec.direct_vecs)
+      o << "    const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = " << vec_name(dv.first, 0) << "z[lk];\n";
+    o << "    " << vt << " res;\n";
+    o << "#pragma unroll\n    for (int l = 0; l < " << vec << "; ++l) {\n";
+    o << "      const " << it << " i2 = i2b + l;\n";
+    o << bodyC;
+    o << "      res.v[l] = " << Emitter::store_conv(rn.ty.dt, valC) << ";\n    }\n";
+    o << "    " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
+    o << "  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = "map_stencil_lds2";
+    L.grid[0] = (unsigned)launch_blocks;
+    L.block[0] = NB;
+    L.lds_bytes = (unsigned)lds_bytes;
+    std::vector<int> ins;
+    for (size_t k = 0; k < ec.inputs.size(); ++k) {
+      if ((int)k == prev_slot) continue;
+      ins.push_back(ec.inputs[k]);
+      L.args.push_back(buffer_for(ec.inputs[k]));
+    }
+    L.args.push_back(buffer_for(root));
+    // both steps' compulsory traffic: the first step's inputs and output, then the second's
+    std::set<int> read2;
+    for (auto& l : ec.loads) read2.insert(l.node);
+    L.algo_bytes = algo_bytes(eb.inputs, {prev}) + algo_bytes(std::vector<int>(read2.begin(), read2.end()), {root});
+    L.desc = describe(prev) + " ; " + describe(root);
+    plan.launches.push_back(L);
+    return true;
+  }
+
   // ------------------------------------------------------------------ map kernels
   void emit_map(int root) {
+    if (lds_only.count(root)) return;   // evaluated inside its only reader's kernel
     if (emit_map_lds(root)) return;
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
@@ -1567,6 +1835,32 @@ struct Planner {
           emit_row(x, ph);
         } else emit_map(x);
       }});
+    }
+    // Two consecutive stencil steps share a kernel when the first step has no other reader.
+    if (opt.stencil_fuse_steps) {
+      std::vector<char> is_result(N, 0);
+      for (int r : g.results) is_result[r] = 1;
+      auto plain_map_root = [&](int x) {
+        const Node& n = g.nodes[x];
+        if (!live[x] || !mat[x]) return false;
+        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::DotGeneral) return false;
+        if (absorbed_roots.count(x) || !row_phases(x).empty()) return false;
+        return true;
+      };
+      for (int x = 0; x < N; ++x) {
+        if (!plain_map_root(x)) continue;
+        StencilProbe sp;
+        if (!probe_stencil(x, &sp) || sp.staged.size() != 1) continue;
+        const int s = sp.staged[0];
+        if (!plain_map_root(s) || is_result[s] || lds_only.count(s) || fuse_prev.count(s)) continue;
+        bool only = !ctx[s].empty();
+        for (auto& c : ctx[s]) only = only && c.first == x;
+        if (!only) continue;
+        StencilProbe sq;
+        if (!probe_stencil(s, &sq) || sq.staged.size() != 1) continue;
+        fuse_prev[x] = s;
+        lds_only.insert(s);
+      }
     }
     // row groups claim their reductions before those would be emitted on their own
     for (auto& j : jobs) {

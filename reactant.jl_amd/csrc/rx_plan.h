@@ -45,7 +45,12 @@ struct PlanOptions {
   bool mfma = true;             // use the MFMA GEMM skeletons for eligible dot_generals
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
+  int slab_ytiles = 0;          // stencil kernels: y-tiles per XCD slab (0: one slab per XCD)
   int lds_tile[3] = {3, 4, 128};  // outputs per workgroup tile (slowest .. fastest dimension)
+  bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
+  bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS
+  int lds_tile2[3] = {4, 8, 64};   // outputs per workgroup tile of the two-step kernel
+  int lds2_threads = 512;          // its workgroup size
   bool stencil_march = false;   // stencil maps: a workgroup marches along the slowest dimension with a ring of planes in LDS
   int march_depth = 3;          // planes of global loads kept in flight (in registers) ahead of their use
   int march_planes = 32;        // planes produced per workgroup when marching

@@ -46,6 +46,46 @@ def test_stencil(rx, client, shape, embed):
     assert np.array_equal(got[0].a, ref[0].a)
 
 
+def _stencil_case(rx, client, shape, embed, steps, elt="f64"):
+    nx, ny, nz = shape
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(0)
+    c = np.zeros(full)
+    c[3:-3, 3:-3, 3:-3] = rng.uniform(0, 1, (nz, ny, nx))
+    u, v, w = [np.random.default_rng(s).uniform(-1, 1, full) for s in (1, 2, 3)]
+    if elt == "f32":
+        c, u, v, w = [a.astype(np.float32) for a in (c, u, v, w)]
+    args = [I.Tensor(a, elt) for a in (c, u, v, w)]
+    text = P.stencil(nx, ny, nz, steps=steps, embed=embed, elt=elt)
+    got, exe = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args)
+    return got[0].a, ref[0].a, exe
+
+
+@pytest.mark.parametrize("shape,embed,steps", [((70, 21, 9), "pad", 2), ((70, 21, 9), "dus", 2), ((64, 40, 20), "pad", 4),
+                                               ((130, 17, 6), "pad", 3), ((58, 26, 5), "dus", 5), ((250, 10, 2), "pad", 2), ((20, 130, 4), "pad", 2),
+                                               ((20, 150, 4), "dus", 3)])
+def test_stencil_two_steps_per_kernel(rx, client, monkeypatch, shape, embed, steps):
+    """Pairs of steps share one kernel (the first step's field lives only in LDS): the values are
+    the same bits as the oracle's, for tiles cut by every array edge and an odd step left over."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    got, ref, exe = _stencil_case(rx, client, shape, embed, steps)
+    kinds = [l["kind"] for l in exe.launches()]
+    assert kinds.count("map_stencil_lds2") == steps // 2 and len(kinds) == steps // 2 + steps % 2
+    assert np.array_equal(got, ref)
+
+
+def test_stencil_two_steps_f32_and_unfused_agree(rx, client, monkeypatch):
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    got, ref, exe = _stencil_case(rx, client, (72, 24, 10), "pad", 2, elt="f32")
+    assert [l["kind"] for l in exe.launches()] == ["map_stencil_lds2"]
+    assert np.array_equal(got, ref)
+    monkeypatch.setenv("RX_STENCIL_FUSE", "0")
+    got1, _, exe1 = _stencil_case(rx, client, (72, 24, 10), "pad", 2, elt="f32")
+    assert [l["kind"] for l in exe1.launches()] == ["map_stencil_lds", "map_stencil_lds"]
+    assert np.array_equal(got1, got)
+
+
 def test_stencil_xcd_slab_order(rx, client, monkeypatch):
     """Same parity with the XCD-slab tile order forced on a small grid."""
     monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
