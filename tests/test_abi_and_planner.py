@@ -87,7 +87,7 @@ def test_client_creation_reports_errors_through_the_error_pointer():
 PROGRAMS = {
     "sinsum_add": (lambda: P.sinsum_add(1 << 20), ["reduce", "reduce_final"]),
     "stencil": (lambda: P.stencil(64, 64, 32, steps=3), ["map", "map", "map"]),
-    "stencil_full": (lambda: P.stencil(512, 512, 256, steps=2), ["map_stencil_lds", "map_stencil_lds"]),
+    "stencil_full": (lambda: P.stencil(512, 512, 256, steps=3), ["map_stencil_lds2", "map_stencil_lds"]),
     "gemm": (lambda: P.gemm(512, 512, 512), ["gemm_f32"]),
     "gemm_transposed": (lambda: P.gemm(512, 256, 128, form="transposed"), ["gemm_f32"]),
     "mlp": (lambda: P.mlp(512, (256, 512, 512, 256)), ["gemm_bf16", "gemm_bf16", "gemm_bf16", "row"]),
@@ -107,12 +107,21 @@ def test_benchmark_programs_plan_and_compile_for_gfx950(name):
     assert "code object:" in report
 
 
-def test_fusion_plan_of_the_full_size_stencil_is_one_kernel_per_timestep():
+def test_fusion_plan_of_the_full_size_stencil_is_one_kernel_per_two_timesteps():
     report = rx.compile_offline(P.stencil(512, 512, 256, steps=10))
     launches = re.findall(r"\] (\w+) kind=(\w+)", report)
-    assert len(launches) == 10
-    assert len({k for k, _ in launches}) == 1           # ten launches of one compiled kernel
-    # compulsory traffic of one timestep on the halo'd arrays: 4 reads + 1 write of 262*518*518 doubles
+    assert len(launches) == 5 and {k for _, k in launches} == {"map_stencil_lds2"}
+    assert len({k for k, _ in launches}) == 1           # five launches of one compiled kernel
+    # compulsory traffic of two timesteps on the halo'd arrays: 2 x (4 reads + 1 write) of 262*518*518 doubles
+    assert "algo_bytes=%d" % (2 * 5 * 262 * 518 * 518 * 8) in report
+    assert "buffers: 9," in report                      # 4 arguments + 5 fields; the odd steps own no buffer
+
+
+def test_fusion_plan_of_the_stencil_without_step_pairing(monkeypatch):
+    monkeypatch.setenv("RX_STENCIL_FUSE", "0")
+    report = rx.compile_offline(P.stencil(512, 512, 256, steps=10))
+    launches = re.findall(r"\] (\w+) kind=(\w+)", report)
+    assert len(launches) == 10 and {k for _, k in launches} == {"map_stencil_lds"}
     assert "algo_bytes=%d" % (5 * 262 * 518 * 518 * 8) in report
 
 
