@@ -7,8 +7,8 @@ diffusion/advection stencil, Float64 512x512x256 with 3-cell halos, 10 timesteps
 traced into one module.  A "step" is one execution of that module (10 timesteps)
 with all inputs resident in HBM; `value` is achieved HBM GB/s counting only the
 algorithmic bytes (per timestep: read c,u,v,w + write c over the interior
-= 5*512*512*256*8 B).  `roofline` describes the dominant kernel (the fused stencil
-map kernel), timed with HIP events on the stream it runs on, inside the timed
+= 5*512*512*256*8 B).  `roofline` describes the dominant kernel (the stencil kernel
+that advances two timesteps per launch: its algorithmic bytes are those of both), timed with HIP events on the stream it runs on, inside the timed
 region.  `cpu_baseline` times the numpy oracle on a bounded sample of the same
 workload on the host cores.  `others` carries the remaining four configs
 (sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry.
@@ -32,11 +32,11 @@ if ROOT not in sys.path:
 # Counters cannot be read from inside this process, so the figures of that profile are quoted here;
 # they are reported only for the kernel and shape they were measured on.
 MEASURED_TRAFFIC_BYTES = {
-    "rx_stencil_k0_stencil": 3540.4e6,
+    "rx_stencil_k0_stencil2": 3235.0e6,
     "rx_sinsum_add_k0_reduce": 537.1e6,
-    "rx_gemm_k0_gemm": 741.5e6,
+    "rx_gemm_k0_gemm": 745.7e6,
     "rx_mlp_k1_gemm": 671.8e6,
-    "rx_fp8_linear_k2_gemm": 2365.8e6,
+    "rx_fp8_linear_k2_gemm": 2351.6e6,
 }
 _FULL_SIZE = [True]   # cleared by --small: the table only holds the full-size shapes
 
@@ -119,13 +119,19 @@ def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=1
     launches = exe.launches()
     cells = nx * ny * nz
     algo_step = 5.0 * cells * 8 * nsteps
-    nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil_lds", "map_stencil", "map"))
-    algo_launch = 5.0 * cells * 8
+    # the dominant kernel: two timesteps per launch when the steps pair up, else one
+    nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil_lds2",))
+    per_launch = 2
+    if nk == 0:
+        nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil_lds", "map_stencil", "map"))
+        per_launch = 1
+    algo_launch = 5.0 * cells * 8 * per_launch
     return {
         "workload": "stencil f64 %dx%dx%d halo 3, %d timesteps per module" % (nx, ny, nz, nsteps),
         "ms_per_step": 1e3 * secs / steps,
         "value": algo_step / (secs / steps) / 1e9, "unit": "GB/s", "dtype": "f64",
         "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"] if launches else None, "launches_per_step": nk,
+                     "timesteps_per_launch": per_launch,
                      "kernel_ms": kms, "achieved": algo_launch / (kms * 1e-3) / 1e9 if kms else None,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": algo_launch / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None,
