@@ -113,11 +113,10 @@ RX_DEV rx_u8 rx_f32_to_e4m3_sw(float f);
 RX_DEV rx_u8 rx_f32_to_e4m3(float f) {
   const rx_u32 u = rx_f2u(f);
   const rx_u32 a = u & 0x7fffffffu;
-  const rx_u8 s = (rx_u8)((u >> 24) & 0x80u);
-  if (a > 0x43e80000u) return (rx_u8)(s | 0x7fu);
-  const float c = rx_u2f(a > 0x43e00000u ? 0x43e00000u : a);   // min(|x|, 448)
-  const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false);
-  return (rx_u8)(s | (rx_u8)(packed & 0x7f));
+  const float c = rx_u2f(a < 0x43e00000u ? a : 0x43e00000u);   // min(|x|, 448); NaN payloads compare above it too
+  const rx_u32 packed = (rx_u32)__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false);
+  const rx_u32 code = a > 0x43e80000u ? 0x7fu : (packed & 0x7fu);
+  return (rx_u8)(((u >> 24) & 0x80u) | code);
 }
 RX_DEV rx_u8 rx_f32_to_e4m3_sw(float f) {
   rx_u32 u = rx_f2u(f);
@@ -164,6 +163,11 @@ RX_DEV float rx_round_e5m2(float f) { return rx_e5m2_to_f32(rx_f32_to_e5m2(f)); 
 // ---------------------------------------------------------------------------
 template <typename T> RX_DEV T rx_max(T a, T b) { return (a > b || a != a) ? a : b; }
 template <typename T> RX_DEV T rx_min(T a, T b) { return (a < b || a != a) ? a : b; }
+// clamp between two constants lo <= hi (neither NaN); a NaN operand stays NaN
+RX_DEV float rx_clamp_ordered(float x, float lo, float hi) {
+  const float m = __builtin_amdgcn_fmed3f(x, lo, hi);
+  return x != x ? x : m;
+}
 template <typename T> RX_DEV T rx_sign(T a) {
   return a != a ? a : (T)((a > (T)0) - (a < (T)0));
 }

@@ -90,6 +90,12 @@ std::string Emitter::store_conv(DT dt, const std::string& val) {
   }
 }
 
+std::string Emitter::store_value(DT dt, const std::string& val) const {
+  auto it = rounded_.find(val);
+  if (it != rounded_.end() && it->second.first == dt) return store_conv(dt, "(" + it->second.second + ")");
+  return store_conv(dt, val);
+}
+
 std::string Emitter::round_narrow(DT dt, const std::string& e) {
   switch (dt) {
     case DT::BF16: return "rx_round_bf16(" + e + ")";
@@ -218,6 +224,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
     std::string v = fresh();
     const bool rnd = is_narrow_float(dt) && (force_round || !excess_precision);
     line("const " + CT + " " + v + " = " + (rnd ? round_narrow(dt, expr) : expr) + ";");
+    if (rnd) rounded_[v] = {dt, expr};
     return v;
   };
   // index of a rank-0 or same-shape operand
@@ -333,7 +340,19 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
     }
     case OpK::Clamp: {
       std::string lo = opnd(0), x = opnd(1), hi = opnd(2);
-      if (is_float(dt)) return def("rx_min(rx_max(" + x + ", " + lo + "), " + hi + ")");
+      if (is_float(dt)) {
+        // constant finite bounds in order: one median instruction, NaN of the operand passed through
+        auto const_bound = [&](int k, double* v) {
+          const Node* c = &g_.nodes[n.in[k]];
+          while (c->k == OpK::BroadcastInDim || c->k == OpK::Reshape) c = &g_.nodes[c->in[0]];
+          if (c->k != OpK::Constant || !c->splat) return false;
+          *v = splat_as_double(*c);
+          return true;
+        };
+        double lv, hv;
+        if (CT == "float" && const_bound(0, &lv) && const_bound(2, &hv) && lv <= hv) return def("rx_clamp_ordered(" + x + ", " + lo + ", " + hi + ")");
+        return def("rx_min(rx_max(" + x + ", " + lo + "), " + hi + ")");
+      }
       return def("(" + CT + ")((" + x + " < " + lo + " ? " + lo + " : " + x + ") > " + hi + " ? " + hi + " : (" + x + " < " + lo + " ? " + lo + " : " + x + "))");
     }
     case OpK::Convert: {

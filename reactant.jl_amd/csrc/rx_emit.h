@@ -73,6 +73,9 @@ class Emitter {
   int slot_of(int node);
   std::string load_conv(DT dt, const std::string& raw) const;          // storage -> compute
   static std::string store_conv(DT dt, const std::string& val);        // compute -> storage
+  // same, for a value this emitter produced: a value that was just rounded to `dt` is converted
+  // from its unrounded form (one conversion instead of round-trip plus conversion)
+  std::string store_value(DT dt, const std::string& val) const;
   static std::string literal(const Node& n);
   static std::string round_narrow(DT dt, const std::string& e);
   std::string idx_t() const { return idx64 ? "long long" : "int"; }
@@ -87,6 +90,7 @@ class Emitter {
   std::ostringstream out_;
   std::vector<std::map<std::string, std::string>> scopes_{1};
   int tmp_ = 0;
+  std::map<std::string, std::pair<DT, std::string>> rounded_;   // variable -> (type it was rounded to, unrounded expression)
   int unsafe_loads_ = 0;   // loads emitted as plain global reads at a computed index
   std::vector<int64_t> root_dims_;
   std::vector<std::string> root_vars_;

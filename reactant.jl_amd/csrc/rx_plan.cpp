@@ -580,7 +580,7 @@ struct Planner {
     o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
     o << "          const " << it << " i2 = i2b + l;\n";
     o << body;
-    o << "          res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n        }\n";
+    o << "          res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n        }\n";
     o << "        " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
     o << "      }\n";
     o << "      store_plane(z + " << hhi[0] + 1 << ", pre[(j + 1) % " << D << "]);\n";
@@ -828,7 +828,7 @@ struct Planner {
     o << "#pragma unroll\n    for (int l = 0; l < " << vec << "; ++l) {\n";
     o << "      const " << it << " i2 = i2b + l;\n";
     o << body;
-    o << "      res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n    }\n";
+    o << "      res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n    }\n";
     o << "    " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
     o << "  }\n}\n\n";
     const std::string kb_final = finalize(o.str());
@@ -1159,13 +1159,13 @@ struct Planner {
     }
     const std::string ost = info(rn.ty.dt).stype;
     if (n == 0) {
-      o << "  {\n" << body << "    out0[0] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n  }\n";
+      o << "  {\n" << body << "    out0[0] = " << em.store_value(rn.ty.dt, val) << ";\n  }\n";
     } else {
       o << "  rx_vec<" << ost << ", " << vec << "> res;\n";
       o << "#pragma unroll\n  for (int l = 0; l < " << vec << "; ++l) {\n";
       o << "    const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
       o << body;
-      o << "    res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n  }\n";
+      o << "    res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n  }\n";
       o << "  " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
     }
     o << "}\n\n";
@@ -1528,7 +1528,7 @@ struct Planner {
       o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
       decode_cols(o);
       o << fbody;
-      o << "        res.v[l] = " << Emitter::store_conv(rn.ty.dt, fval) << ";\n      }\n";
+      o << "        res.v[l] = " << em.store_value(rn.ty.dt, fval) << ";\n      }\n";
       o << "      *reinterpret_cast<rx_vec<" << ost << ", " << vec << ">*>(out0 + lin0) = res;\n";
       o << "    }\n  }\n";
     }
@@ -1674,7 +1674,7 @@ struct Planner {
       o << "      const " << DCT << " accv = " << accv << ";\n";
     }
     o << ebody;
-    o << "      res.v[l] = " << Emitter::store_conv(rn.ty.dt, val) << ";\n    }\n";
+    o << "      res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n    }\n";
     o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
     o << "  }\n};\n\n";
 
