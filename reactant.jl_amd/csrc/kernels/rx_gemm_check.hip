@@ -18,7 +18,7 @@ struct rx_check_epi {
 #define RX_CHECK(NAME, MMA, BK, AKC, BKC)                                                                          \
   extern "C" __global__ __launch_bounds__(256) void NAME(const MMA::elem* A, const MMA::elem* B, float* out) {      \
     rx_check_epi<float, 512> epi{out};                                                                             \
-    rx_gemm_body<MMA, 128, 128, BK, 2, 2, AKC, BKC, 512, 512, 512, false, rx_check_epi<float, 512>>(A, B, epi);     \
+    rx_gemm_body<MMA, 128, 128, BK, 2, 2, AKC, BKC, 512, 512, 512, 4, 8, false, rx_check_epi<float, 512>>(A, B, epi);     \
   }
 
 RX_CHECK(rx_check_f32_nn, rx_mma_f32, 16, true, false)

@@ -179,7 +179,26 @@ struct rx_tile_copy {
 // ---------------------------------------------------------------------------
 // the kernel body
 // ---------------------------------------------------------------------------
-template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, bool BATCHED, class Epi>
+// Tile order.  Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  The tile
+// grid is cut into blocks of RB x CB tiles; XCD k takes blocks k, k+8, ... and the
+// tiles of one block run side by side on that XCD, so they share RB row panels of A and CB
+// column panels of B in its L2.  The 8 blocks in flight are consecutive in row-major block
+// order, which keeps the panels they share in the memory-side cache.  The grid is padded to
+// whole blocks on every XCD (rx::gemm_grid on the host computes the same number); a workgroup
+// whose tile falls outside the grid returns false.
+template <int GM, int GN, int RB, int CB>
+RX_DEV bool rx_gemm_tile(unsigned bid, int* bm, int* bn) {
+  constexpr unsigned PER = RB * CB;
+  constexpr unsigned NBC = (GN + CB - 1) / CB;
+  const unsigned xcd = bid & 7u, j = bid >> 3;
+  const unsigned blk = (j / PER) * 8u + xcd, t = j % PER;
+  const unsigned br = blk / NBC, bc = blk % NBC;
+  *bm = (int)(br * RB + t % RB);
+  *bn = (int)(bc * CB + t / RB);
+  return *bm < GM && *bn < GN;
+}
+
+template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
 RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
   typedef typename MMA::elem E;
   constexpr int NT = WM * WN * 64;
@@ -194,21 +213,9 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  // Tile order: consecutive workgroups share the same A rows (n fastest) inside groups of
-  // 8 row-tiles, so the operand tiles of concurrently running workgroups stay in L2.
   constexpr int GM = (M + BM - 1) / BM, GN = (N + BN - 1) / BN;
   int bm, bn;
-  {
-    const int bid = blockIdx.x;
-    constexpr int GROUP = 8;
-    const int per_group = GROUP * GN;
-    const int grp = bid / per_group;
-    const int first = grp * GROUP;
-    const int rows = (GM - first) < GROUP ? (GM - first) : GROUP;
-    const int in = bid % per_group;
-    bm = first + in % rows;
-    bn = in / rows;
-  }
+  if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
   const int m0 = bm * BM, n0 = bn * BN;
   const long long batch = BATCHED ? blockIdx.y : 0;
   const E* Ab = A + batch * (long long)M * K;
@@ -407,7 +414,7 @@ RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0
   }
 }
 
-template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, bool BATCHED, class Epi>
+template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
 RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
   typedef typename MMA::elem E;
   constexpr int NT = WM * WN * 64;
@@ -424,17 +431,7 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
   const int wm = wave / WN, wn = wave % WN;
   constexpr int GM = (M + BM - 1) / BM, GN = (N + BN - 1) / BN;
   int bm, bn;
-  {
-    const int bid = blockIdx.x;
-    constexpr int GROUP = 8;
-    const int per_group = GROUP * GN;
-    const int grp = bid / per_group;
-    const int first = grp * GROUP;
-    const int rows = (GM - first) < GROUP ? (GM - first) : GROUP;
-    const int in = bid % per_group;
-    bm = first + in % rows;
-    bn = in / rows;
-  }
+  if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
   const int m0 = bm * BM, n0 = bn * BN;
   const long long batch = BATCHED ? blockIdx.y : 0;
   const E* Ab = A + batch * (long long)M * K;

@@ -36,6 +36,8 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (const char* e = getenv("RX_GEMM_DIRECT")) direct = atoi(e) != 0;
   int stages = 2;
   if (const char* e = getenv("RX_GEMM_STAGES")) stages = atoi(e) >= 2 ? atoi(e) : stages;
+  int rb = 4, cb = 8;   // tiles of one XCD's block (rows x columns of the tile grid)
+  if (const char* e = getenv("RX_GEMM_BLOCK")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2 && v[0] > 0 && v[1] > 0) { rb = v[0]; cb = v[1]; } }
   const int nt = WM * WN * 64;
   if (direct) {
     int dbk = bk;
@@ -49,11 +51,11 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       c.lds_bytes = (unsigned)(stage_bytes * stages);
       c.block = nt;
       const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
-      c.grid[0] = (unsigned)(gm * gn);
+      c.grid[0] = (unsigned)gemm_grid(gm, gn, rb, cb);
       c.grid[1] = (unsigned)batch;
       std::ostringstream t;
       t << mma << ", " << BM << ", " << BN << ", " << dbk << ", " << WM << ", " << WN << ", " << stages << ", " << (a_kc ? "true" : "false") << ", "
-        << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K;
+        << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
       c.targs = t.str();
       c.skeleton = "rx_gemm_body_dl";
       c.stype_a = mma + "::elem";
@@ -68,11 +70,11 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (c.lds_bytes > 160 * 1024) return c;
   c.block = WM * WN * 64;
   const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
-  c.grid[0] = (unsigned)(gm * gn);
+  c.grid[0] = (unsigned)gemm_grid(gm, gn, rb, cb);
   c.grid[1] = (unsigned)batch;
   std::ostringstream t;
   t << mma << ", " << BM << ", " << BN << ", " << bk << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false")
-    << ", " << M << ", " << N << ", " << K;
+    << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
   c.targs = t.str();
   c.skeleton = "rx_gemm_body";
   c.stype_a = mma + "::elem";

@@ -17,6 +17,14 @@ struct GemmChoice {
   std::string stype_a, stype_b;
 };
 
+// Workgroups to launch for a gm x gn grid of tiles: the kernels walk the tiles in blocks of 4 x 8,
+// eight blocks (one per XCD) at a time, and the grid is padded to whole rounds of eight blocks
+// (rx_gemm_tile in kernels/rx_gemm_kernels.h decodes the same order).
+inline int64_t gemm_grid(int64_t gm, int64_t gn, int rb = 4, int cb = 8) {
+  const int64_t blocks = ((gm + rb - 1) / rb) * ((gn + cb - 1) / cb);
+  return (blocks + 7) / 8 * 8 * rb * cb;
+}
+
 // Returns ok=false when no skeleton covers the case (the caller then writes a scalar loop).
 GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_k_contig, bool b_k_contig);
 
