@@ -74,12 +74,8 @@ RX_DEV float rx_u2f(rx_u32 u) { return __builtin_bit_cast(float, u); }
 // bf16: storage is the upper half of binary32; conversion rounds to nearest even
 // ---------------------------------------------------------------------------
 RX_DEV float rx_bf16_to_f32(rx_u16 b) { return rx_u2f(((rx_u32)b) << 16); }
-RX_DEV rx_u16 rx_f32_to_bf16(float f) {
-  rx_u32 u = rx_f2u(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (rx_u16)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (rx_u16)(u >> 16);
-}
+// gfx950 converts in hardware (v_cvt_pk_bf16_f32, round to nearest even, NaN stays NaN)
+RX_DEV rx_u16 rx_f32_to_bf16(float f) { return __builtin_bit_cast(rx_u16, (__bf16)f); }
 RX_DEV float rx_round_bf16(float f) { return rx_bf16_to_f32(rx_f32_to_bf16(f)); }
 
 // ---------------------------------------------------------------------------
