@@ -539,3 +539,51 @@ class Thunk:
 def compile(mlir_text, client=None):
     client = client or default_backend()
     return Thunk(xla_compile(client, mlir_text), client)
+
+
+# ----------------------------------------------------------------------------
+# Reactant.Serialization.export_to_enzymejax hand-off (src/serialization/EnzymeJAX.jl:124-172)
+# ----------------------------------------------------------------------------
+def load_enzymejax_export(mlir_path, npz_path=None):
+    """Read what `export_to_enzymejax` writes for one function: `<fn>_<id>.mlir` (the module as
+    `string(mod)`) and `<fn>_<id>_inputs.npz` with keys `arr_1 … arr_N` in `@main` argument order.
+    The arrays were saved with their dims reversed (`permutedims(arr, reverse(1:ndims(arr)))`,
+    ext/ReactantNPZExt.jl:9-22), i.e. already in the layout of the module's tensor types; numbers
+    are 0-d.  Returns (module text, [numpy arrays])."""
+    with open(mlir_path, "r") as f:
+        text = f.read()
+    if npz_path is None:
+        stem = mlir_path[:-5] if mlir_path.endswith(".mlir") else mlir_path
+        npz_path = stem + "_inputs.npz"
+    arrays = []
+    with np.load(npz_path, allow_pickle=False) as z:
+        keys = set(z.files)
+        k = 1
+        while "arr_%d" % k in keys:
+            arrays.append(np.asarray(z["arr_%d" % k]))
+            k += 1
+        if len(arrays) != len(keys):
+            raise ReactantInternalError("%s: expected keys arr_1 … arr_N, found %s" % (npz_path, sorted(keys)))
+    return text, arrays
+
+
+def run_enzymejax_export(mlir_path, npz_path=None, client=None):
+    """Compile an exported module, upload its saved inputs and run it once.  Returns the results
+    as numpy arrays in the module's (dim-reversed) layout — what the generated Python script's
+    `run_<fn>(*load_inputs())` returns (src/serialization/EnzymeJAX.jl:338-345,390-402); the
+    Julia-order array is `result.T` for every rank."""
+    client = client or default_backend()
+    text, arrays = load_enzymejax_export(mlir_path, npz_path)
+    exe = xla_compile(client, text)
+    bufs = []
+    for i, a in enumerate(arrays):
+        if a.dtype not in _NUMPY_DEFAULT:
+            raise ReactantInternalError("input arr_%d has dtype %s, which no tensor element type stores" % (i + 1, a.dtype))
+        dt = _NUMPY_DEFAULT[a.dtype]
+        bufs.append(Buffer.from_host(client, encode(a, dt), dt))
+    outs = exe.execute_sharded(bufs)
+    res = []
+    for ab in outs:
+        b = ab.synced_buffer()
+        res.append(decode(b.to_host(), b.dtype()))
+    return res

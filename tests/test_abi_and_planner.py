@@ -7,6 +7,8 @@ import ctypes
 import os
 import re
 
+import numpy as np
+
 import pytest
 
 from _loader import load_pkg, load_programs, ROOT
@@ -159,3 +161,20 @@ def test_host_side_array_conventions():
     assert rx.PRIMITIVE_TYPE["f32"] == 11 and rx.PRIMITIVE_TYPE["bf16"] == 16 and rx.PRIMITIVE_TYPE["f8E4M3FN"] == 20
     with pytest.raises(rx.ReactantInternalError):
         rx.set_default_backend("tpu")
+
+
+def test_enzymejax_export_files_are_read_in_argument_order(tmp_path):
+    """`<fn>_<id>.mlir` + `<fn>_<id>_inputs.npz` with keys arr_1.. (reference
+    src/serialization/EnzymeJAX.jl:124-172); no device needed to read them and plan the module."""
+    text = P.sinsum_add(8)
+    (tmp_path / "f_0.mlir").write_text(text)
+    a, b = np.arange(8, dtype=np.float32), -np.arange(8, dtype=np.float32)
+    np.savez(tmp_path / "f_0_inputs.npz", arr_2=b, arr_1=a)
+    got_text, arrays = rx.load_enzymejax_export(str(tmp_path / "f_0.mlir"))
+    assert got_text == text and len(arrays) == 2
+    assert np.array_equal(arrays[0], a) and np.array_equal(arrays[1], b)
+    assert "kind=reduce" in rx.compile_offline(got_text)
+    np.savez(tmp_path / "g_0_inputs.npz", x=a)
+    (tmp_path / "g_0.mlir").write_text(text)
+    with pytest.raises(rx.ReactantInternalError, match="arr_1"):
+        rx.load_enzymejax_export(str(tmp_path / "g_0.mlir"))
