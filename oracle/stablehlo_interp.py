@@ -32,6 +32,8 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       textbook triple loop
   gelu / softmax ... closed forms, scipy.special, test/nn/nnlib.jl:85-149
   stencil chains ... brute-force loops on small grids
+  while loops (src/Ops.jl:2349-2460; text form src/mlir/Dialects/StableHLO.jl:4850-4861)
+      ... plain Python loops, closed forms, equality with the unrolled module
   bf16 / f8E4M3FN convert and dot_general ... PARITY UNPINNED in the reference
       (it holds no test of these); pinned here only by the OCP closed-form
       tables, exact-product arguments and torch CPU casts.
@@ -606,6 +608,34 @@ class Parser:
                     if not c.accept(","):
                         break
             return op
+        if short == "while":
+            # %r:2 = stablehlo.while(%iterArg = %init0, %iterArg_0 = %init1) : t0, t1 [attributes {..}]
+            #   cond { ... stablehlo.return %p : tensor<i1> } do { ... stablehlo.return %a, %b : t0, t1 }
+            # (form in the docstring of the reference's binding, src/mlir/Dialects/StableHLO.jl:4850-4861)
+            names = []
+            c.expect("(")
+            while not c.accept(")"):
+                names.append(c.ssa())
+                c.expect("=")
+                op.operands.append(c.ssa())
+                c.accept(",")
+            if names:
+                c.expect(":")
+                while True:
+                    op.types_out.append(c.type())
+                    if not c.accept(","):
+                        break
+            op.types_in = list(op.types_out)
+            if c.accept("attributes"):
+                c.balanced("{", "}")
+            c.expect("cond")
+            c.expect("{")
+            op.regions.append(self.block())
+            c.expect("do")
+            c.expect("{")
+            op.regions.append(self.block())
+            op.attrs["iter_names"] = names
+            return op
         if name.startswith("chlo."):
             op.operands.append(c.ssa())
             while c.accept(","):
@@ -1089,6 +1119,11 @@ class Interpreter:
         for op in ops:
             if op.name == "return":
                 return [env[o] for o in op.operands]
+            if op.name == "while":
+                outs = self._while(op, env)
+                for r, v in zip(op.results, outs):
+                    env[r] = v
+                continue
             outs = self._eval(op, [env[o] for o in op.operands])
             if len(op.results) == 1:
                 env[op.results[0]] = outs[0]
@@ -1096,6 +1131,33 @@ class Interpreter:
                 for r, v in zip(op.results, outs):
                     env[r] = v
         return []
+
+    def _while(self, op, env):
+        """stablehlo.while: the regions see the enclosing values; the block arguments of both
+        regions are the loop-carried values."""
+        cur = [env[o] for o in op.operands]
+
+        def region_names(region):
+            if "iter_names" in op.attrs:
+                return op.attrs["iter_names"]
+            for o in region:
+                if o.name == "__block_args__":
+                    return [nm for nm, _ in o.attrs["args"]]
+            return []
+
+        cond, body = op.regions
+        for _ in range(1 << 20):
+            e = dict(env)
+            e.update(zip(region_names(cond), cur))
+            pred = self._block([o for o in cond if o.name != "__block_args__"], e)[0]
+            if not bool(np.asarray(pred.a).reshape(-1)[0]):
+                return cur
+            e = dict(env)
+            e.update(zip(region_names(body), cur))
+            cur = [_rounded(v) for v in self._block([o for o in body if o.name != "__block_args__"], e)]
+            if len(cur) != len(op.operands):
+                raise ValueError("while body returns %d values for %d loop-carried ones" % (len(cur), len(op.operands)))
+        raise ValueError("while loop did not terminate")
 
     def _eval(self, op, xs):
         n, at = op.name, op.attrs

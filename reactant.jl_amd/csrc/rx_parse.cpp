@@ -627,6 +627,34 @@ struct P {
       fn_type(o);
       return o;
     }
+    if (sh == "while") {
+      // %r:2 = stablehlo.while(%iterArg = %init0, %iterArg_0 = %init1) : t0, t1 [attributes {..}]
+      //   cond { ... stablehlo.return %p : tensor<i1> } do { ... stablehlo.return %a, %b : t0, t1 }
+      // (the form in the docstring of the reference's binding, src/mlir/Dialects/StableHLO.jl:4850-4861)
+      std::vector<std::string> names;
+      c.expect("(");
+      while (!c.accept(")")) {
+        names.push_back(c.ssa());
+        c.expect("=");
+        o.operands.push_back(c.ssa());
+        c.accept(",");
+      }
+      if (!names.empty()) {
+        c.expect(":");
+        do { o.tout.push_back(c.type()); } while (c.accept(","));
+      }
+      if (o.tout.size() != names.size()) c.fail("while: one type per loop-carried value expected");
+      o.tin = o.tout;
+      for (size_t k = 0; k < names.size(); ++k) o.block_args.push_back({names[k], o.tout[k]});
+      if (c.accept("attributes")) c.balanced('{', '}');
+      c.expect("cond");
+      c.expect("{");
+      o.regions.push_back(block());
+      c.expect("do");
+      c.expect("{");
+      o.regions.push_back(block());
+      return o;
+    }
     if (sh == "compare") {
       o.sa["direction"] = c.ident();
       c.expect(",");
@@ -951,8 +979,8 @@ struct Builder {
       if (o.name == "__block_args__") continue;
       std::vector<int> in;
       for (auto& s : o.operands) in.push_back(look(s));
-      if (o.name == "return") return in;
-      std::vector<int> outs = build(o, in, depth);
+      if (o.name == "return" || o.name == "stablehlo.return" || o.name == "func.return") return in;
+      std::vector<int> outs = o.name == "stablehlo.while" ? run_while(o, in, env, depth) : build(o, in, depth);
       if (outs.size() != o.results.size()) fail("result count mismatch on " + o.name);
       for (size_t k = 0; k < outs.size(); ++k) env[o.results[k]] = outs[k];
     }
@@ -960,6 +988,157 @@ struct Builder {
   }
 
   const TType& ty(int id) { return g.nodes[id].ty; }
+
+  // ---- loops with a static trip count -------------------------------------------------------
+  // `stablehlo.while` is unrolled while the module is imported: the condition region is
+  // evaluated on the current loop-carried values and must fold to a constant (an induction
+  // variable compared with a constant); each time it is true the body region is replayed.  This
+  // is the form `@trace for` loops take (reference src/Ops.jl:2349-2460); loops whose trip count
+  // depends on data are rejected.
+  static constexpr int kMaxTrip = 4096;
+  std::map<int, std::pair<bool, int64_t>> folded;
+
+  static bool is_int_dt(DT t) { return !is_float(t) && t != DT::INVALID; }
+  static int64_t wrap_to(DT t, int64_t v) {
+    switch (t) {
+      case DT::I1: return v != 0;
+      case DT::I8: return (int8_t)v;
+      case DT::I16: return (int16_t)v;
+      case DT::I32: return (int32_t)v;
+      case DT::U8: return (uint8_t)v;
+      case DT::U16: return (uint16_t)v;
+      case DT::U32: return (uint32_t)v;
+      default: return v;
+    }
+  }
+  static bool is_unsigned_dt(DT t) { return t == DT::U8 || t == DT::U16 || t == DT::U32 || t == DT::U64; }
+
+  // value of a one-element integer node that depends on constants only
+  bool fold_int(int id, int64_t* out) {
+    auto it = folded.find(id);
+    if (it != folded.end()) { *out = it->second.second; return it->second.first; }
+    const Node& n = g.nodes[id];
+    bool ok = false;
+    int64_t v = 0;
+    auto sub = [&](int k, int64_t* x) { return fold_int(n.in[k], x); };
+    if (is_int_dt(n.ty.dt) && n.ty.numel() == 1) {
+      int64_t a, b, c2;
+      switch (n.k) {
+        case OpK::Constant:
+          if (n.splat || n.data.size() == (size_t)info(n.ty.dt).size) { v = splat_as_int(n); ok = true; }
+          break;
+        case OpK::Convert:
+          if (is_int_dt(g.nodes[n.in[0]].ty.dt) && sub(0, &a)) { v = wrap_to(n.ty.dt, a); ok = true; }
+          break;
+        case OpK::Reshape:
+        case OpK::BroadcastInDim:
+          if (sub(0, &a)) { v = a; ok = true; }
+          break;
+        case OpK::Binary:
+          if (sub(0, &a) && sub(1, &b)) {
+            const bool un = is_unsigned_dt(n.ty.dt);
+            ok = true;
+            if (n.op == "add") v = (int64_t)((uint64_t)a + (uint64_t)b);
+            else if (n.op == "subtract") v = (int64_t)((uint64_t)a - (uint64_t)b);
+            else if (n.op == "multiply") v = (int64_t)((uint64_t)a * (uint64_t)b);
+            else if (n.op == "minimum") v = un ? (int64_t)std::min((uint64_t)a, (uint64_t)b) : std::min(a, b);
+            else if (n.op == "maximum") v = un ? (int64_t)std::max((uint64_t)a, (uint64_t)b) : std::max(a, b);
+            else if (n.op == "and") v = a & b;
+            else if (n.op == "or") v = a | b;
+            else if (n.op == "xor") v = a ^ b;
+            else ok = false;
+            v = wrap_to(n.ty.dt, v);
+          }
+          break;
+        case OpK::Unary:
+          if (sub(0, &a)) {
+            ok = true;
+            if (n.op == "negate") v = wrap_to(n.ty.dt, (int64_t)(0 - (uint64_t)a));
+            else if (n.op == "not") v = n.ty.dt == DT::I1 ? !a : wrap_to(n.ty.dt, ~a);
+            else ok = false;
+          }
+          break;
+        case OpK::Compare:
+          if (is_int_dt(g.nodes[n.in[0]].ty.dt) && sub(0, &a) && sub(1, &b)) {
+            const bool un = is_unsigned_dt(g.nodes[n.in[0]].ty.dt) || n.cmp_unsigned;
+            const bool lt = un ? (uint64_t)a < (uint64_t)b : a < b, eq = a == b;
+            ok = true;
+            if (n.op == "LT") v = lt;
+            else if (n.op == "LE") v = lt || eq;
+            else if (n.op == "GT") v = !lt && !eq;
+            else if (n.op == "GE") v = !lt;
+            else if (n.op == "EQ") v = eq;
+            else if (n.op == "NE") v = !eq;
+            else ok = false;
+          }
+          break;
+        case OpK::Select:
+          if (sub(0, &c2) && sub(1, &a) && sub(2, &b)) { v = c2 ? a : b; ok = true; }
+          break;
+        default:
+          break;
+      }
+    }
+    folded[id] = {ok, v};
+    *out = v;
+    return ok;
+  }
+
+  std::vector<int> run_while(const RawOp& o, const std::vector<int>& init, const std::map<std::string, int>& outer, int depth) {
+    if (depth > 16) fail("while: nesting depth exceeded");
+    if (o.regions.size() != 2) fail("while: expected a condition and a body region");
+    auto names_of = [&](const std::vector<RawOp>& region) {
+      std::vector<std::pair<std::string, TType>> a = o.block_args;
+      if (a.empty())
+        for (auto& r : region)
+          if (r.name == "__block_args__") { a = r.block_args; break; }
+      if (a.size() != init.size()) fail("while: " + std::to_string(a.size()) + " region arguments for " + std::to_string(init.size()) + " loop-carried values");
+      return a;
+    };
+    const auto cond_args = names_of(o.regions[0]), body_args = names_of(o.regions[1]);
+    for (size_t k = 0; k < init.size(); ++k) {
+      if (!(ty(init[k]) == cond_args[k].second)) fail("while: operand " + std::to_string(k) + " has type " + ty(init[k]).str() + ", region expects " + cond_args[k].second.str());
+      if (k < o.tout.size() && !(o.tout[k] == ty(init[k]))) fail("while: result " + std::to_string(k) + " type mismatch");
+    }
+    std::vector<int> cur = init;
+    for (int trip = 0;; ++trip) {
+      if (trip > kMaxTrip) fail("while: more than " + std::to_string(kMaxTrip) + " iterations");
+      std::map<std::string, int> env = outer;
+      for (size_t k = 0; k < cur.size(); ++k) env[cond_args[k].first] = cur[k];
+      std::vector<int> pred = run_block(o.regions[0], env, depth + 1);
+      if (pred.size() != 1 || ty(pred[0]).dt != DT::I1 || ty(pred[0]).numel() != 1) fail("while: the condition must return one tensor<i1>");
+      int64_t p = 0;
+      if (!fold_int(pred[0], &p))
+        fail("while: the condition does not fold to a constant; only loops with a static trip count are supported");
+      if (!p) return cur;
+      env = outer;
+      for (size_t k = 0; k < cur.size(); ++k) env[body_args[k].first] = cur[k];
+      std::vector<int> next = run_block(o.regions[1], env, depth + 1);
+      if (next.size() != cur.size()) fail("while: the body returns " + std::to_string(next.size()) + " values for " + std::to_string(cur.size()) + " loop-carried ones");
+      for (size_t k = 0; k < cur.size(); ++k)
+        if (!(ty(next[k]) == ty(cur[k]))) fail("while: the body changes the type of loop-carried value " + std::to_string(k));
+      cur = next;
+    }
+  }
+
+  // one-element integer values that depend on constants only become constants (loop counters
+  // after unrolling; start indices of dynamic slices must be constants when kernels are planned)
+  void fold_scalar_constants() {
+    for (size_t id = 0; id < g.nodes.size(); ++id) {
+      Node& n = g.nodes[id];
+      if (n.k == OpK::Constant || n.k == OpK::Param || n.in.empty()) continue;
+      if (!is_int_dt(n.ty.dt) || n.ty.numel() != 1) continue;
+      int64_t v;
+      if (!fold_int((int)id, &v)) continue;
+      n.k = OpK::Constant;
+      n.op.clear();
+      n.in.clear();
+      n.a0.clear(); n.a1.clear(); n.a2.clear(); n.a3.clear();
+      n.splat = true;
+      n.data.assign(info(n.ty.dt).size, 0);
+      store_scalar(n.ty.dt, (double)v, v, true, n.data.data());
+    }
+  }
 
   void check_same(const TType& a, const TType& b, const std::string& what) {
     if (!(a == b)) fail(what + ": type mismatch " + a.str() + " vs " + b.str());
@@ -1229,6 +1408,7 @@ Graph parse_module(const char* text, size_t len) {
     b.g.aliasing_output.push_back(alias);
   }
   b.g.results = b.inline_func(*mainf, args, 0);
+  b.fold_scalar_constants();
   if (b.g.results.size() != mainf->result_types.size()) throw Error("StableHLO import: @main returns the wrong number of values");
   for (size_t k = 0; k < b.g.results.size(); ++k)
     if (!(b.g.nodes[b.g.results[k]].ty == mainf->result_types[k]))

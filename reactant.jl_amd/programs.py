@@ -120,7 +120,7 @@ def sinsum_add(n, dt="f32"):
 STENCIL_DEFAULTS = dict(dt=0.05, dx=1.0, kappa=1.0)
 
 
-def stencil(nx, ny, nz, steps=10, halo=3, dt=0.05, dx=1.0, kappa=1.0, embed="pad", elt="f64"):
+def stencil(nx, ny, nz, steps=10, halo=3, dt=0.05, dx=1.0, kappa=1.0, embed="pad", elt="f64", loop="unrolled"):
     """c,u,v,w are Julia arrays (nx+2H, ny+2H, nz+2H): raw dims (nz+2H, ny+2H, nx+2H).
 
     Per step, on the interior:
@@ -128,7 +128,9 @@ def stencil(nx, ny, nz, steps=10, halo=3, dt=0.05, dx=1.0, kappa=1.0, embed="pad
         adv_a = ifelse(a > 0, a*(c - c[-1]), a*(c[+1] - c)) / dx      for a in (u,v,w)
         c_new = c + dt*(lap - (adv_x + adv_y + adv_z))
     and the interior is re-embedded with zero halos (`embed="pad"`) or written over
-    the previous field (`embed="dus"`).
+    the previous field (`embed="dus"`).  `loop="unrolled"` is a plain Julia `for` (the steps are
+    traced one after another); `loop="while"` is what `@trace for` gives: one `stablehlo.while`
+    carrying a counter and the field (src/Ops.jl:2349-2460).
     """
     H = halo
     full = [nz + 2 * H, ny + 2 * H, nx + 2 * H]
@@ -151,8 +153,7 @@ def stencil(nx, ny, nz, steps=10, halo=3, dt=0.05, dx=1.0, kappa=1.0, embed="pad
         return b.slice(x, full, elt, st, [s + n for s, n in zip(st, inner)])
 
     ui, vi, wi = sh("%arg1", 0, 0, 0), sh("%arg2", 0, 0, 0), sh("%arg3", 0, 0, 0)
-    c = "%arg0"
-    for _ in range(steps):
+    def step(c):
         ci = sh(c, 0, 0, 0)
         cxm, cxp = sh(c, 0, 0, -1), sh(c, 0, 0, 1)
         cym, cyp = sh(c, 0, -1, 0), sh(c, 0, 1, 0)
@@ -185,7 +186,29 @@ def stencil(nx, ny, nz, steps=10, halo=3, dt=0.05, dx=1.0, kappa=1.0, embed="pad
             b.lines.append("    %s = stablehlo.dynamic_update_slice %s, %s, %s, %s, %s : "
                            "(%s, %s, tensor<i64>, tensor<i64>, tensor<i64>) -> %s"
                            % (nc, c, cn, hidx, hidx, hidx, tf, ti, tf))
-        c = nc
+        return nc
+
+    c = "%arg0"
+    if loop == "while":
+        ti64 = _tt([], "i64")
+        c0, c1, cn_ = b.const(0, [], "i64"), b.const(1, [], "i64"), b.const(steps, [], "i64")
+        res = b.new(tf)
+        b.lines.append("    %s:2 = stablehlo.while(%%iterArg = %s, %%iterArg_0 = %s) : %s, %s" % (res, c0, c, ti64, tf))
+        b.lines.append("     cond {")
+        p = b.new(_tt([], "i1"))
+        b.lines.append("      %s = stablehlo.compare  LT, %%iterArg, %s,  SIGNED : (%s, %s) -> tensor<i1>" % (p, cn_, ti64, ti64))
+        b.lines.append("      stablehlo.return %s : tensor<i1>" % p)
+        b.lines.append("    } do {")
+        b.types["%iterArg"] = ti64
+        b.types["%iterArg_0"] = tf
+        inc = b.bin("add", "%iterArg", c1)
+        nc = step("%iterArg_0")
+        b.lines.append("      stablehlo.return %s, %s : %s, %s" % (inc, nc, ti64, tf))
+        b.lines.append("    }")
+        c = res + "#1"
+    else:
+        for _ in range(steps):
+            c = step(c)
     return (_HDR.format(name="stencil") +
             "  func.func @main(%%arg0: %s {tf.aliasing_output = 0 : i32}, %%arg1: %s, %%arg2: %s, "
             "%%arg3: %s) -> %s {\n" % (tf, tf, tf, tf, tf) + b.text() +

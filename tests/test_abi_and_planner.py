@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 from _loader import load_pkg, load_programs, ROOT
+import _while_modules as W
 
 rx = load_pkg()
 P = load_programs()
@@ -178,3 +179,21 @@ def test_enzymejax_export_files_are_read_in_argument_order(tmp_path):
     (tmp_path / "g_0.mlir").write_text(text)
     with pytest.raises(rx.ReactantInternalError, match="arr_1"):
         rx.load_enzymejax_export(str(tmp_path / "g_0.mlir"))
+
+
+def test_while_with_a_static_trip_count_is_unrolled_at_import():
+    """The `@trace for` form of the stencil plans exactly like the unrolled form (five launches of
+    the two-step kernel); counters fold to constants, so counter-indexed slices plan too."""
+    strip = lambda rep: re.sub(r"code object: \d+ bytes", "", rep)
+    assert strip(rx.compile_offline(P.stencil(512, 512, 256, steps=10, loop="while"))) == \
+        strip(rx.compile_offline(P.stencil(512, 512, 256, steps=10)))
+    rep = rx.compile_offline(W.SETINDEX)
+    assert rep.count("dynamic_update_slice") >= 1 and "kind=map" in rep
+    assert "launches: 2" in rx.compile_offline(W.GENERIC)
+
+
+@pytest.mark.parametrize("text", [W.DATA_DEPENDENT, W.COUNT])
+def test_while_with_a_data_dependent_trip_count_is_rejected(text):
+    """A bound or a starting value that is an argument: the loop cannot be unrolled."""
+    with pytest.raises(rx.ReactantInternalError, match="static trip count"):
+        rx.compile_offline(text)

@@ -300,3 +300,19 @@ def test_empty_and_scalar_shapes(rx, client):
     text = mod(["tensor<f32>", "tensor<f32>"], "tensor<f32>", "    %0 = stablehlo.add %arg0, %arg1 : tensor<f32>\n    return %0 : tensor<f32>\n")
     got, _ = gpu_run(rx, client, text, [I.Tensor(np.float32(2.0), "f32"), I.Tensor(np.float32(2.0), "f32")])
     assert float(got[0].a) == 4.0   # test/core/ops.jl:1066-1082
+
+
+# ---- stablehlo.while with a static trip count ------------------------------------------------
+def test_while_counter_indexed_update_slice(rx, client):
+    import _while_modules as W
+    x = np.array([10, 20, 30, 40], dtype=np.int64)
+    got, ref = both(rx, client, W.SETINDEX, [I.Tensor(x, "i64")])
+    assert np.array_equal(got[0].a, x + 2 * np.arange(1, 5)) and np.array_equal(got[0].a, ref[0].a)
+
+
+def test_while_generic_form_returns_counter_and_value(rx, client):
+    import _while_modules as W
+    v = np.array([0.5, -1.0, 3.0, 0.0], dtype=np.float32)
+    got, ref = both(rx, client, W.GENERIC, [I.Tensor(v, "f32")])
+    assert int(got[0].a) == 3 and np.array_equal(got[1].a, 8 * v)
+    assert np.array_equal(got[1].a, ref[1].a)

@@ -86,6 +86,20 @@ def test_stencil_two_steps_f32_and_unfused_agree(rx, client, monkeypatch):
     assert np.array_equal(got1, got)
 
 
+@pytest.mark.parametrize("embed", ["pad", "dus"])
+def test_stencil_traced_loop_form(rx, client, monkeypatch, embed):
+    """`@trace for`: the ten steps arrive as one stablehlo.while; same bits as the oracle's loop."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    nx, ny, nz = 40, 21, 9
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(3)
+    args = [I.Tensor(rng.uniform(-1, 1, full), "f64") for _ in range(4)]
+    text = P.stencil(nx, ny, nz, steps=5, embed=embed, loop="while")
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["map_stencil_lds2", "map_stencil_lds2", "map_stencil_lds"]
+    assert np.array_equal(got[0].a, oracle_run(text, args)[0].a)
+
+
 def test_stencil_xcd_slab_order(rx, client, monkeypatch):
     """Same parity with the XCD-slab tile order forced on a small grid."""
     monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")

@@ -12,6 +12,7 @@ import pytest
 from oracle import lowfloat as lf
 from oracle import stablehlo_interp as I
 from _loader import load_programs
+import _while_modules as W
 
 P = load_programs()
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
@@ -314,3 +315,37 @@ def test_parser_accepts_reference_text_samples():
     }"""
     r = run(m6, [])
     assert r[0].a.tolist() == [0, 0, 0] and r[1].a.tolist() == [1.0, 2.0]
+
+
+def test_while_loops_against_plain_loops():
+    """`stablehlo.while` in the oracle: the example of the reference's binding docstring
+    (src/mlir/Dialects/StableHLO.jl:4850-4861) against a Python loop for several starting
+    points (including one where the body never runs), a counter-indexed update-slice loop
+    against its closed form, the generic form, and a data-dependent trip count."""
+    for i0, s0 in [(1, 0), (0, 0), (7, -3), (10, 5), (12, 1)]:
+        i, acc = i0, s0
+        while i < 10:
+            acc, i = acc + 1, i + 1
+        r = I.run_text(W.COUNT, [I.Tensor(np.int64(i0), "i64"), I.Tensor(np.int64(s0), "i64")])
+        assert (int(r[0].a), int(r[1].a)) == (i, acc)
+    x = np.array([10, 20, 30, 40], dtype=np.int64)
+    r = I.run_text(W.SETINDEX, [I.Tensor(x, "i64")])
+    assert np.array_equal(r[0].a, x + 2 * np.arange(1, 5))
+    v = np.array([0.5, -1.0, 3.0, 0.0], dtype=np.float32)
+    r = I.run_text(W.GENERIC, [I.Tensor(v, "f32")])
+    assert int(r[0].a) == 3 and np.array_equal(r[1].a, 8 * v)
+    for n in (0, 1, 5):
+        r = I.run_text(W.DATA_DEPENDENT, [I.Tensor(x, "i64"), I.Tensor(np.int64(n), "i64")])
+        assert np.array_equal(r[0].a, x * 2 ** n)
+
+
+@pytest.mark.parametrize("embed", ["pad", "dus"])
+def test_while_form_of_the_stencil_equals_the_unrolled_form(embed):
+    """`@trace for` (one stablehlo.while carrying a counter and the field) and a plain `for`
+    (steps traced one after another) are the same computation: same bits."""
+    rng = np.random.default_rng(5)
+    full = (4 + 6, 5 + 6, 6 + 6)
+    args = [I.Tensor(rng.uniform(-1, 1, full), "f64") for _ in range(4)]
+    a = I.run_text(P.stencil(6, 5, 4, steps=4, embed=embed, loop="while"), args)[0].a
+    b = I.run_text(P.stencil(6, 5, 4, steps=4, embed=embed), args)[0].a
+    assert np.array_equal(a, b)
