@@ -501,6 +501,85 @@ class ConcreteRArray:
         a = self.to_array()
         return a.astype(dtype) if dtype is not None else a
 
+    # -- array operations that go through the device (src/ConcreteRArray.jl:423-446,783-805,
+    #    src/xla/PJRT/Buffer.jl:19-103,170-182).  Indices are 1-based, as in Julia. ------------
+    def _client(self):
+        return self.data.buffer.client
+
+    def _tensor_type(self):
+        return "tensor<" + "".join("%dx" % d for d in self.shape[::-1]) + self.dtype + ">"
+
+    def similar(self, dtype=None, shape=None):
+        """Base.similar: an uninitialized array on the same device."""
+        dtype, shape = dtype or self.dtype, tuple(shape if shape is not None else self.shape)
+        buf = Buffer.uninitialized(self._client(), shape[::-1], dtype)
+        return ConcreteRArray(AsyncBuffer(buf), shape, dtype)
+
+    def copy(self):
+        return ConcreteRArray(AsyncBuffer(self._buffer().copy()), self.shape, self.dtype)
+
+    def _swap(self, thunk, *extra):
+        """Run an updating function with this array donated and take over the result's buffer
+        (in-place updates are handle swaps: src/compiler/Codegen.jl:1151-1169)."""
+        out = thunk(self, *extra, donated=[True] + [False] * len(extra))
+        self.data, self.donated = out.data, False
+        return self
+
+    def fill(self, value):
+        """fill!(a, value): compiles `broadcast_in_dim` of a number and runs it."""
+        if 0 in self.shape:
+            raise ReactantInternalError("Cannot setindex! to empty buffer")
+        tt, st = self._tensor_type(), "tensor<%s>" % self.dtype
+        text = ("module @reactant_fill {\n  func.func @main(%%arg0: %s {tf.aliasing_output = 0 : i32}, %%arg1: %s) -> %s {\n"
+                "    %%0 = stablehlo.broadcast_in_dim %%arg1, dims = [] : (%s) -> %s\n    return %%0 : %s\n  }\n}\n"
+                % (tt, st, tt, st, tt, tt))
+        return self._swap(_cached_thunk(self._client(), text), to_rarray(np.asarray(value), self.dtype, self._client()))
+
+    def _index_module(self, store):
+        n = len(self.shape)
+        tt, st, it = self._tensor_type(), "tensor<%s>" % self.dtype, "tensor<i64>"
+        one = "tensor<" + "1x" * n + self.dtype + ">"
+        first = 2 if store else 1                                       # position of the first index argument
+        idx_args = "".join(", %%arg%d: %s" % (k + first, it) for k in range(n))
+        body = "    %c = stablehlo.constant dense<1> : tensor<i64>\n"
+        for k in range(n):
+            body += "    %%i%d = stablehlo.subtract %%arg%d, %%c : %s\n" % (k, k + first, it)
+        starts = ", ".join("%%i%d" % k for k in reversed(range(n)))     # dims are reversed on the device
+        its = ", ".join([it] * n)
+        if store:
+            body += "    %%u = stablehlo.reshape %%arg1 : (%s) -> %s\n" % (st, one)
+            body += "    %%r = stablehlo.dynamic_update_slice %%arg0, %%u, %s : (%s, %s, %s) -> %s\n" % (starts, tt, one, its, tt)
+            return ("module @reactant_mysetindex {\n  func.func @main(%%arg0: %s {tf.aliasing_output = 0 : i32}, %%arg1: %s%s) -> %s {\n%s"
+                    "    return %%r : %s\n  }\n}\n" % (tt, st, idx_args, tt, body, tt))
+        body += "    %%s = stablehlo.dynamic_slice %%arg0, %s, sizes = [%s] : (%s, %s) -> %s\n" % (starts, ", ".join(["1"] * n), tt, its, one)
+        body += "    %%r = stablehlo.reshape %%s : (%s) -> %s\n" % (one, st)
+        return ("module @reactant_mygetindex {\n  func.func @main(%%arg0: %s%s) -> %s {\n%s    return %%r : %s\n  }\n}\n"
+                % (tt, idx_args, st, body, st))
+
+    def _check_index(self, idx):
+        if len(idx) != len(self.shape) or not self.shape:
+            raise IndexError("expected %d indices" % len(self.shape))
+        for i, d in zip(idx, self.shape):
+            if not 1 <= int(i) <= d:
+                raise IndexError("index %r out of bounds for an array of size %r" % (tuple(idx), self.shape))
+
+    def setindex(self, value, *idx):
+        """a[i, j, ...] = value for one element (scalar indexing of a device array): compiles a
+        `dynamic_update_slice` whose start indices are arguments, so one executable serves
+        every position."""
+        self._check_index(idx)
+        cl = self._client()
+        nums = [to_rarray(np.asarray(value), self.dtype, cl)] + [to_rarray(np.int64(i), "i64", cl) for i in idx]
+        return self._swap(_cached_thunk(cl, self._index_module(True)), *nums)
+
+    def getindex(self, *idx):
+        """a[i, j, ...] for one element."""
+        self._check_index(idx)
+        cl = self._client()
+        nums = [to_rarray(np.int64(i), "i64", cl) for i in idx]
+        out = _cached_thunk(cl, self._index_module(False))(self, *nums)
+        return out.to_array()[()]
+
 
 def to_rarray(x, dtype=None, client=None):
     """Reactant.to_rarray: host array (Julia index order) -> device."""
@@ -539,6 +618,17 @@ class Thunk:
 def compile(mlir_text, client=None):
     client = client or default_backend()
     return Thunk(xla_compile(client, mlir_text), client)
+
+
+_THUNKS = {}
+
+
+def _cached_thunk(client, mlir_text):
+    """One executable per (client, module text): the small functions behind fill!/setindex!/getindex."""
+    key = (id(client), mlir_text)
+    if key not in _THUNKS:
+        _THUNKS[key] = compile(mlir_text, client)
+    return _THUNKS[key]
 
 
 # ----------------------------------------------------------------------------

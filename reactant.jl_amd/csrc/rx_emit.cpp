@@ -418,9 +418,15 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       Index oi(ix.size());
       for (size_t d = 0; d < ix.size(); ++d) {
         const Node& s = g_.nodes[n.in[1 + d]];
-        if (s.k != OpK::Constant) throw Error("dynamic_slice with non-constant start indices is not supported");
-        int64_t st = std::min(std::max<int64_t>(splat_as_int(s), 0), o.ty.dims[d] - n.a0[d]);
-        oi[d] = shifted(ix[d], st);
+        const int64_t room = o.ty.dims[d] - n.a0[d];   // start indices are clamped into [0, room]
+        if (s.k == OpK::Constant) {
+          oi[d] = shifted(ix[d], std::min(std::max<int64_t>(splat_as_int(s), 0), room));
+        } else {
+          // start index computed at run time (a 0-d integer value): clamp, then offset
+          const std::string e = emit(n.in[1 + d], Index{});
+          oi[d] = temp_index("(" + idx_t() + ")rx_clamp_idx<long long>((long long)(" + e + "), " + std::to_string(room) + "LL) + " + ix[d].str(),
+                             ix[d].lo, ix[d].hi + room);
+        }
       }
       return emit(n.in[0], oi);
     }
@@ -505,9 +511,15 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       bool never = false;
       for (size_t d = 0; d < ix.size(); ++d) {
         const Node& s = g_.nodes[n.in[2 + d]];
-        if (s.k != OpK::Constant) throw Error("dynamic_update_slice with non-constant start indices is not supported");
-        int64_t st = std::min(std::max<int64_t>(splat_as_int(s), 0), o.ty.dims[d] - u.ty.dims[d]);
-        Ix p = shifted(ix[d], -st);
+        const int64_t room = o.ty.dims[d] - u.ty.dims[d];   // start indices are clamped into [0, room]
+        Ix p;
+        if (s.k == OpK::Constant) {
+          p = shifted(ix[d], -std::min(std::max<int64_t>(splat_as_int(s), 0), room));
+        } else {
+          const std::string e = emit(n.in[2 + d], Index{});
+          p = temp_index(ix[d].str() + " - (" + idx_t() + ")rx_clamp_idx<long long>((long long)(" + e + "), " + std::to_string(room) + "LL)",
+                         ix[d].lo - room, ix[d].hi);
+        }
         if (p.lo < 0) conds.push_back(p.str() + " >= 0");
         if (p.hi > u.ty.dims[d] - 1) conds.push_back(p.str() + " < " + std::to_string(u.ty.dims[d]));
         p.lo = std::max<int64_t>(p.lo, 0);

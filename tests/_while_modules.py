@@ -73,3 +73,28 @@ DATA_DEPENDENT = """module { func.func @main(%x: tensor<4xi64>, %n: tensor<i64>)
   }
   return %r#1 : tensor<4xi64>
 } }"""
+
+# scalar `setindex!` / `getindex` on a device array (src/ConcreteRArray.jl:423-446): Julia a is 3x4,
+# the indices arrive as 1-based numbers, the module works on the dim-reversed 4x3 tensor
+SETINDEX_SCALAR = """module @reactant_mysetindex attributes {mhlo.num_partitions = 1 : i64, mhlo.num_replicas = 1 : i64} {
+  func.func @main(%arg0: tensor<4x3xf64> {tf.aliasing_output = 0 : i32}, %arg1: tensor<f64>, %arg2: tensor<i64>, %arg3: tensor<i64>) -> tensor<4x3xf64> {
+    %c = stablehlo.constant dense<1> : tensor<i64>
+    %0 = stablehlo.subtract %arg2, %c : tensor<i64>
+    %1 = stablehlo.subtract %arg3, %c : tensor<i64>
+    %2 = stablehlo.reshape %arg1 : (tensor<f64>) -> tensor<1x1xf64>
+    %3 = stablehlo.dynamic_update_slice %arg0, %2, %1, %0 : (tensor<4x3xf64>, tensor<1x1xf64>, tensor<i64>, tensor<i64>) -> tensor<4x3xf64>
+    return %3 : tensor<4x3xf64>
+  }
+}"""
+GETINDEX_BLOCK = """module @reactant_getblock attributes {mhlo.num_partitions = 1 : i64, mhlo.num_replicas = 1 : i64} {
+  func.func @main(%arg0: tensor<4x3xf64>, %arg1: tensor<i32>, %arg2: tensor<i32>) -> tensor<2x2xf64> {
+    %0 = stablehlo.dynamic_slice %arg0, %arg2, %arg1, sizes = [2, 2] : (tensor<4x3xf64>, tensor<i32>, tensor<i32>) -> tensor<2x2xf64>
+    return %0 : tensor<2x2xf64>
+  }
+}"""
+FILL = """module @reactant_fill attributes {mhlo.num_partitions = 1 : i64, mhlo.num_replicas = 1 : i64} {
+  func.func @main(%arg0: tensor<4x3xf32> {tf.aliasing_output = 0 : i32}, %arg1: tensor<f32>) -> tensor<4x3xf32> {
+    %0 = stablehlo.broadcast_in_dim %arg1, dims = [] : (tensor<f32>) -> tensor<4x3xf32>
+    return %0 : tensor<4x3xf32>
+  }
+}"""

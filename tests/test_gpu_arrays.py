@@ -1,0 +1,73 @@
+"""Operations on device arrays that compile a small function behind the scenes, as the reference
+does for arrays that do not live in host memory: `fill!`, scalar `setindex!`/`getindex`
+(src/ConcreteRArray.jl:423-446,783-805), `similar`/`copy` (src/xla/PJRT/Buffer.jl:19-103,170-182),
+and the same modules with run-time start indices against the oracle."""
+import numpy as np
+import pytest
+
+import _while_modules as W
+from _harness import gpu_run, oracle_run
+from oracle import stablehlo_interp as I
+
+pytestmark = pytest.mark.gpu
+
+
+def test_fill_setindex_getindex_on_a_device_array(rx, client):
+    a = np.arange(12, dtype=np.float64).reshape(3, 4)
+    x = rx.to_rarray(a, client=client)
+    assert x.getindex(2, 3) == a[1, 2]
+    x.setindex(-5.0, 2, 4)
+    x.setindex(7.5, 3, 1)
+    a[1, 3], a[2, 0] = -5.0, 7.5
+    assert np.array_equal(np.asarray(x), a)
+    assert [x.getindex(i + 1, j + 1) for i in range(3) for j in range(4)] == list(a.reshape(-1))
+    y = x.copy()
+    x.fill(2.0)
+    assert np.array_equal(np.asarray(x), np.full((3, 4), 2.0)) and np.array_equal(np.asarray(y), a)
+    z = x.similar()
+    assert z.shape == (3, 4) and z.dtype == "f64" and np.asarray(z).shape == (3, 4)
+    w = x.similar(dtype="i32", shape=(5,))
+    w.fill(9)
+    assert np.array_equal(np.asarray(w), np.full(5, 9, dtype=np.int32))
+    with pytest.raises(IndexError):
+        x.setindex(1.0, 4, 1)
+    with pytest.raises(IndexError):
+        x.getindex(0, 1)
+
+
+def test_one_executable_serves_every_position(rx, client):
+    x = rx.to_rarray(np.zeros((2, 3, 4), dtype=np.float32), client=client)
+    before = len(rx._THUNKS)
+    for i in range(2):
+        for j in range(3):
+            for k in range(4):
+                x.setindex(100 * i + 10 * j + k, i + 1, j + 1, k + 1)
+    assert len(rx._THUNKS) == before + 1
+    want = np.fromfunction(lambda i, j, k: 100 * i + 10 * j + k, (2, 3, 4)).astype(np.float32)
+    assert np.array_equal(np.asarray(x), want)
+
+
+@pytest.mark.parametrize("i,j", [(1, 1), (3, 4), (2, 3)])
+def test_update_slice_with_runtime_indices_matches_the_oracle(rx, client, i, j):
+    a = np.arange(12, dtype=np.float64).reshape(4, 3)
+    args = [I.Tensor(a, "f64"), I.Tensor(np.float64(-5), "f64"), I.Tensor(np.int64(i), "i64"), I.Tensor(np.int64(j), "i64")]
+    got, _ = gpu_run(rx, client, W.SETINDEX_SCALAR, args)
+    want = a.copy()
+    want[j - 1, i - 1] = -5
+    assert np.array_equal(got[0].a, want) and np.array_equal(got[0].a, oracle_run(W.SETINDEX_SCALAR, args)[0].a)
+
+
+@pytest.mark.parametrize("i,j,ei,ej", [(0, 0, 0, 0), (1, 2, 1, 2), (7, -2, 1, 0), (-3, 9, 0, 2)])
+def test_slice_with_runtime_indices_clamps_like_the_specification(rx, client, i, j, ei, ej):
+    """Start indices are clamped so that the slice stays inside the operand."""
+    a = np.arange(12, dtype=np.float64).reshape(4, 3)
+    args = [I.Tensor(a, "f64"), I.Tensor(np.int32(i), "i32"), I.Tensor(np.int32(j), "i32")]
+    got, _ = gpu_run(rx, client, W.GETINDEX_BLOCK, args)
+    assert np.array_equal(got[0].a, a[ej:ej + 2, ei:ei + 2])
+    assert np.array_equal(got[0].a, oracle_run(W.GETINDEX_BLOCK, args)[0].a)
+
+
+def test_fill_module(rx, client):
+    args = [I.Tensor(np.zeros((4, 3), np.float32), "f32"), I.Tensor(np.float32(1.25), "f32")]
+    got, _ = gpu_run(rx, client, W.FILL, args)
+    assert np.array_equal(got[0].a, np.full((4, 3), 1.25, np.float32))
