@@ -67,23 +67,25 @@ def _upload(rx, client, arr, dt):
 
 def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
     """Run warmup + steps executions.  `make_args(prev_results)` returns (buffers, donated).
+    The timed steps are queued without waiting in between; every kernel launch sits between two
+    HIP events recorded on the library's stream, read after the final synchronization.
     Returns (seconds for the timed steps, per-launch mean ms over the timed steps, last results)."""
     dev = client.default_device()
     res = None
     for _ in range(warmup):
         bufs, don = make_args(res)
-        res, _ms = exe.execute_timed(bufs, don)
+        res = exe.execute_profiled(bufs, don)
     dev.synchronize()
-    nl = len(exe.launches())
-    acc = np.zeros(nl)
+    exe.take_timings()
     t0 = time.perf_counter()
     for _ in range(steps):
         bufs, don = make_args(res)
-        res, ms = exe.execute_timed(bufs, don)
-        acc += np.asarray(ms)
+        res = exe.execute_profiled(bufs, don)
     dev.synchronize()
     t1 = time.perf_counter()
-    return t1 - t0, acc / steps, res
+    runs, mean_ms = exe.take_timings()
+    assert runs == steps
+    return t1 - t0, np.asarray(mean_ms), res
 
 
 def _dominant(launches, mean_ms, kinds):

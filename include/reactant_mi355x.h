@@ -135,6 +135,13 @@ void RxExecutableLaunchInfo(RxExecutable *exec, int index, const char **kernel, 
  * stream the kernels run on); launch_ms has RxExecutableNumLaunches entries. */
 void RxExecuteTimed(RxExecutable *exec, int num_args, RxBuffer **op_args, RxDevice *device,
                     uint8_t *is_arg_donatable, int num_results, RxBuffer **op_results, float *launch_ms);
+/* The same event pairs without blocking: the call returns as soon as the launches are queued
+ * and the events stay with the executable.  RxExecutableTakeTimings waits for the profiled
+ * executions queued so far, adds each launch's milliseconds into launch_ms_sum
+ * (RxExecutableNumLaunches entries), forgets them and returns how many executions it summed. */
+void RxExecuteProfiled(RxExecutable *exec, int num_args, RxBuffer **op_args, RxDevice *device,
+                       uint8_t *is_arg_donatable, int num_results, RxBuffer **op_results);
+int RxExecutableTakeTimings(RxExecutable *exec, double *launch_ms_sum);
 /* Blocks until all work queued on the device's stream has finished. */
 void RxDeviceSynchronize(RxDevice *device);
 /* Plain 16-byte-per-lane copy kernel of `bytes` bytes, `iters` times; returns

@@ -115,6 +115,8 @@ SIGNATURES = {
     "RxExecutableNumResults": (_i, [_vp]),
     "RxExecutableLaunchInfo": (None, [_vp, _i, _P(_cp), _P(_cp), _P(ctypes.c_double), _P(ctypes.c_double)]),
     "RxExecuteTimed": (None, [_vp, _i, _P(_vp), _vp, _P(_u8), _i, _P(_vp), _P(ctypes.c_float)]),
+    "RxExecuteProfiled": (None, [_vp, _i, _P(_vp), _vp, _P(_u8), _i, _P(_vp)]),
+    "RxExecutableTakeTimings": (_i, [_vp, _P(ctypes.c_double)]),
     "RxDeviceSynchronize": (None, [_vp]),
     "RxCalibrationCopy": (ctypes.c_float, [_vp, _sz, _i]),
 }
@@ -423,6 +425,24 @@ class LoadedExecutable:
         dev = (device or self.client.default_device()).handle
         _call("RxExecuteTimed", self.handle, n, args, dev, don, nres, res, ms)
         return [Buffer(res[k], self.client) for k in range(nres)], [ms[k] for k in range(nl)]
+
+    def execute_profiled(self, buffers, donated=None, device=None):
+        """Like execute_timed but does not wait: the event pairs are read later by take_timings()."""
+        n = len(buffers)
+        args = (_vp * n)(*[b.handle for b in buffers])
+        don = (_u8 * n)(*([1 if d else 0 for d in donated] if donated else [0] * n))
+        nres = self.num_results
+        res = (_vp * nres)()
+        dev = (device or self.client.default_device()).handle
+        _call("RxExecuteProfiled", self.handle, n, args, dev, don, nres, res)
+        return [Buffer(res[k], self.client) for k in range(nres)]
+
+    def take_timings(self):
+        """(number of profiled executions since the last call, per-launch mean milliseconds)."""
+        nl = _call("RxExecutableNumLaunches", self.handle)
+        acc = (ctypes.c_double * max(nl, 1))()
+        runs = _call("RxExecutableTakeTimings", self.handle, acc)
+        return runs, [acc[k] / max(runs, 1) for k in range(nl)]
 
     def free(self):
         if self.handle:

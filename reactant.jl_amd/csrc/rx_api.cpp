@@ -165,6 +165,8 @@ struct RxExecutable {
   std::vector<Mem> consts;          // per plan buffer (only Const kinds are set)
   std::string report;
   std::mutex mu;
+  // event lists of executions profiled without blocking (RxExecuteProfiled), oldest first
+  std::vector<std::vector<hipEvent_t>> pending_events;
 };
 
 namespace {
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, 
 
 // Core of XLAExecuteSharded / RxExecuteTimed
 void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uint8_t* donate, int num_results, RxBuffer** results, float* launch_ms,
-             RxFuture** futures) {
+             RxFuture** futures, bool profile_async = false) {
   check_exec(ex);
   if (dev) check_device(dev);
   if (!dev) dev = ex->device;
@@ -313,7 +315,8 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     }
   }
   std::vector<hipEvent_t> evs;
-  if (launch_ms) {
+  const bool timed = launch_ms || profile_async;
+  if (timed) {
     evs.resize(P.launches.size() + 1);
     for (auto& e : evs) HIP_CHECK(hipEventCreate(&e));
     HIP_CHECK(hipEventRecord(evs[0], dev->stream));
@@ -335,7 +338,7 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     for (auto& p : ptrs) argv.push_back(&p);
     HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
                                     argv.data(), nullptr));
-    if (launch_ms) HIP_CHECK(hipEventRecord(evs[li + 1], dev->stream));
+    if (timed) HIP_CHECK(hipEventRecord(evs[li + 1], dev->stream));
     for (int b : L.args) {
       const auto& B = P.buffers[b];
       if (B.last_use == (int)li && !is_res[b]) bufs[b].reset();
@@ -371,6 +374,8 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     HIP_CHECK(hipEventSynchronize(evs.back()));
     for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[li], evs[li + 1]));
     for (auto& e : evs) (void)hipEventDestroy(e);
+  } else if (profile_async) {
+    ex->pending_events.push_back(std::move(evs));   // read later by RxExecutableTakeTimings
   }
 }
 
@@ -672,6 +677,8 @@ RX_EXPORT void ExecutableFree(RxExecutable* ex) {
     (void)hipStreamSynchronize(ex->device->stream);
     (void)hipModuleUnload(ex->module);
   }
+  for (auto& evs : ex->pending_events)
+    for (auto& e : evs) (void)hipEventDestroy(e);
   delete ex;
 }
 RX_EXPORT RxClient* PjRtLoadedExecutableGetClient(RxExecutable* ex) { return guarded([&]() -> RxClient* { check_exec(ex); return ex->client; }, nullptr); }
@@ -704,6 +711,33 @@ RX_EXPORT void XLAExecuteSharded(RxExecutable* ex, int num_args, RxBuffer** op_a
 RX_EXPORT void RxExecuteTimed(RxExecutable* ex, int num_args, RxBuffer** op_args, RxDevice* device, uint8_t* is_arg_donatable, int num_results,
                               RxBuffer** op_results, float* launch_ms) {
   guarded_void([&] { execute(ex, num_args, op_args, device, is_arg_donatable, num_results, op_results, launch_ms, nullptr); });
+}
+
+RX_EXPORT void RxExecuteProfiled(RxExecutable* ex, int num_args, RxBuffer** op_args, RxDevice* device, uint8_t* is_arg_donatable, int num_results,
+                                 RxBuffer** op_results) {
+  guarded_void([&] { execute(ex, num_args, op_args, device, is_arg_donatable, num_results, op_results, nullptr, nullptr, true); });
+}
+RX_EXPORT int RxExecutableTakeTimings(RxExecutable* ex, double* launch_ms_sum) {
+  return guarded([&]() -> int {
+    check_exec(ex);
+    std::lock_guard<std::mutex> lock(ex->mu);
+    const size_t nl = ex->plan.launches.size();
+    for (size_t li = 0; li < nl; ++li) launch_ms_sum[li] = 0.0;
+    int runs = 0;
+    HIP_CHECK(hipSetDevice(ex->device->ordinal));
+    for (auto& evs : ex->pending_events) {
+      HIP_CHECK(hipEventSynchronize(evs.back()));
+      for (size_t li = 0; li < nl; ++li) {
+        float ms = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&ms, evs[li], evs[li + 1]));
+        launch_ms_sum[li] += ms;
+      }
+      for (auto& e : evs) (void)hipEventDestroy(e);
+      ++runs;
+    }
+    ex->pending_events.clear();
+    return runs;
+  }, 0);
 }
 
 RX_EXPORT void FreeFuture(RxFuture* f) {

@@ -71,3 +71,21 @@ def test_fill_module(rx, client):
     args = [I.Tensor(np.zeros((4, 3), np.float32), "f32"), I.Tensor(np.float32(1.25), "f32")]
     got, _ = gpu_run(rx, client, W.FILL, args)
     assert np.array_equal(got[0].a, np.full((4, 3), 1.25, np.float32))
+
+
+def test_profiled_execution_does_not_block_and_reports_every_launch(rx, client):
+    """RxExecuteProfiled / RxExecutableTakeTimings: same results as a plain execution, one timing
+    per kernel launch, summed over the executions queued since the last read."""
+    from _loader import load_programs
+    P = load_programs()
+    n = 1 << 16
+    x = np.random.default_rng(0).uniform(-3, 3, n).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-3, 3, n).astype(np.float32)
+    exe = rx.xla_compile(client, P.sinsum_add(n))
+    bufs = [rx.Buffer.from_host(client, a, "f32") for a in (x, y)]
+    want = exe.execute_sharded(bufs)[0].synced_buffer().to_host()
+    outs = [exe.execute_profiled(bufs)[0] for _ in range(5)]
+    runs, ms = exe.take_timings()
+    assert runs == 5 and len(ms) == len(exe.launches()) == 2 and all(m > 0 for m in ms)
+    assert all(np.array_equal(o.to_host(), want) for o in outs)
+    assert exe.take_timings()[0] == 0
