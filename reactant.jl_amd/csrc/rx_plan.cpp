@@ -1256,31 +1256,80 @@ struct Planner {
     o << "#pragma unroll\n  for (int u = 1; u < " << U << "; ++u) a = " << red_apply(rn.red, dt, "a", "acc[u]") << ";\n";
     o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
     o << "  a = rx_block_reduce<" << ACC << ", decltype(" << red_functor(rn.red) << "), " << kBlock / 64 << ">(a, " << red_functor(rn.red) << ", lds);\n";
-    o << "  if (threadIdx.x == 0) partial[blockIdx.x] = a;\n";
-    o << "}\n\n";
-
-    // pass 2
+    // the init value and the final store, evaluated by one thread
     Emitter e2(g, [&](int x) { return mat[x]; });
     e2.excess_precision = opt.excess_precision;
     e2.indent = 4;
     std::string initv = e2.emit(rn.in[1], Index{});
     std::string ibody = e2.take_code();
     std::vector<int> in2 = e2.inputs;
-    o << "// reduce (pass 2): combine " << G << " partials, apply init -> " << rn.ty.str() << "\n";
-    {
-      std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + k2 + "(const " + ACC + "* __restrict__ partial";
-      for (size_t k = 0; k < in2.size(); ++k) s += ", " + ptr_decl(info(g.nodes[in2[k]].ty.dt).stype, true, "in" + std::to_string(k));
-      s += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
-      o << s << " {\n";
-    }
-    o << "  " << ACC << " a = " << red_identity(rn.red, dt) << ";\n";
-    o << "  for (int i = threadIdx.x; i < " << G << "; i += " << kBlock << ") a = " << red_apply(rn.red, dt, "a", "partial[i]") << ";\n";
-    o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
-    o << "  a = rx_block_reduce<" << ACC << ", decltype(" << red_functor(rn.red) << "), " << kBlock / 64 << ">(a, " << red_functor(rn.red) << ", lds);\n";
-    o << "  if (threadIdx.x == 0) {\n" << ibody;
-    o << "    const " << ACC << " r = " << red_apply(rn.red, dt, "a", "(" + ACC + ")" + initv) << ";\n";
     std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
-    o << "    out0[0] = " << Emitter::store_conv(dt, rv) << ";\n  }\n}\n\n";
+    auto combine = [&](std::ostringstream& oo, const std::string& src) {
+      // partials are combined in index order by a fixed tree: the result does not depend on
+      // which workgroup finished last
+      oo << "  " << ACC << " c = " << red_identity(rn.red, dt) << ";\n";
+      oo << "  for (int i = threadIdx.x; i < " << G << "; i += " << kBlock << ") c = " << red_apply(rn.red, dt, "c", src + "[i]") << ";\n";
+      oo << "  c = rx_block_reduce<" << ACC << ", decltype(" << red_functor(rn.red) << "), " << kBlock / 64 << ">(c, " << red_functor(rn.red) << ", lds);\n";
+      oo << "  if (threadIdx.x == 0) {\n" << ibody;
+      oo << "    const " << ACC << " r = " << red_apply(rn.red, dt, "c", "(" + ACC + ")" + initv) << ";\n";
+      oo << "    out0[0] = " << Emitter::store_conv(dt, rv) << ";\n";
+    };
+    const bool single = opt.single_pass_reduce && G > 1;
+    if (single) {
+      // One launch: every workgroup publishes its partial, takes a ticket, and the one that draws
+      // the last ticket combines all partials.  The ticket counter lives in a buffer that is
+      // zero when the executable is loaded and is set back to zero by that last workgroup.
+      // (device-scope fences around the ticket make the partials of other XCDs visible)
+      std::string sig = signature(k1, em.inputs, {{ACC, "partial"}});
+      sig.pop_back();
+      sig += ", unsigned* __restrict__ ticket";
+      for (size_t k = 0; k < in2.size(); ++k) sig += ", " + ptr_decl(info(g.nodes[in2[k]].ty.dt).stype, true, "fin" + std::to_string(k));
+      sig += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
+      // the pass-1 text was written against `signature(k1, ...)`; swap the header
+      std::string text = o.str();
+      const std::string old_sig = signature(k1, em.inputs, {{ACC, "partial"}});
+      const size_t at = text.find(old_sig);
+      text.replace(at, old_sig.size(), sig);
+      o.str("");
+      o << text;
+      o << "  __shared__ bool last;\n";
+      o << "  if (threadIdx.x == 0) {\n";
+      o << "    partial[blockIdx.x] = a;\n";
+      o << "    __builtin_amdgcn_fence(__ATOMIC_RELEASE, \"agent\");\n";
+      o << "    last = atomicAdd(ticket, 1u) == gridDim.x - 1u;\n";
+      o << "  }\n";
+      o << "  __syncthreads();\n";
+      o << "  if (!last) return;\n";
+      o << "  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"agent\");\n";
+      o << "  const volatile " << ACC << "* all = partial;\n";
+      // the init-value operands were numbered for a kernel of their own
+      std::string ib = ibody;
+      std::ostringstream oc;
+      combine(oc, "all");
+      std::string ctext = oc.str();
+      for (size_t k = in2.size(); k-- > 0;) {
+        const std::string from = "in" + std::to_string(k) + "[", to = "fin" + std::to_string(k) + "[";
+        for (size_t p = ctext.find(from); p != std::string::npos; p = ctext.find(from, p + to.size())) {
+          if (p > 0 && (isalnum((unsigned char)ctext[p - 1]) || ctext[p - 1] == '_')) continue;
+          ctext.replace(p, from.size(), to);
+        }
+      }
+      o << ctext;
+      o << "    *ticket = 0u;\n  }\n}\n\n";
+    } else {
+      o << "  if (threadIdx.x == 0) partial[blockIdx.x] = a;\n";
+      o << "}\n\n";
+      o << "// reduce (pass 2): combine " << G << " partials, apply init -> " << rn.ty.str() << "\n";
+      {
+        std::string s2 = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + k2 + "(const " + ACC + "* __restrict__ partial";
+        for (size_t k = 0; k < in2.size(); ++k) s2 += ", " + ptr_decl(info(g.nodes[in2[k]].ty.dt).stype, true, "in" + std::to_string(k));
+        s2 += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
+        o << s2 << " {\n";
+      }
+      o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
+      combine(o, "partial");
+      o << "  }\n}\n\n";
+    }
     const std::string kb_final = finalize(o.str());
 
     int sc = scratch((int64_t)G * (dt == DT::F64 || info(dt).size == 8 ? 8 : 4));
@@ -1293,6 +1342,20 @@ struct Planner {
     L1.args.push_back(sc);
     L1.algo_bytes = algo_bytes(em.inputs, {}) + info(dt).size;
     L1.desc = describe(rn.in[0]) + " reduce";
+    if (single) {
+      BufferDesc cb;
+      cb.kind = BufferDesc::Const;          // lives with the executable; zero when loaded
+      cb.ty.dt = DT::U32;
+      cb.ty.dims = {1};
+      cb.bytes = 4;
+      cb.data.assign(4, 0);
+      plan.buffers.push_back(cb);
+      L1.args.push_back((int)plan.buffers.size() - 1);
+      for (int i : in2) L1.args.push_back(buffer_for(i));
+      L1.args.push_back(buffer_for(root));
+      plan.launches.push_back(L1);
+      return;
+    }
     plan.launches.push_back(L1);
     Launch L2;
     L2.kernel = named(k2, kb_final);

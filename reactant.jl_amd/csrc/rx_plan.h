@@ -47,6 +47,10 @@ struct PlanOptions {
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
   int slab_ytiles = 0;          // stencil kernels: y-tiles per XCD slab (0: one slab per XCD)
   int lds_tile[3] = {3, 4, 128};  // outputs per workgroup tile (slowest .. fastest dimension)
+  // full reductions in one launch: the last workgroup to finish combines the partials.  Off: the
+  // device-scope release fence every workgroup needs before taking its ticket (an L2 write-back on
+  // this multi-die part) made the sinsum kernel 2x slower than the two-launch form.
+  bool single_pass_reduce = false;
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS
   int lds_tile2[3] = {4, 8, 64};   // outputs per workgroup tile of the two-step kernel

@@ -197,3 +197,9 @@ def test_while_with_a_data_dependent_trip_count_is_rejected(text):
     """A bound or a starting value that is an argument: the loop cannot be unrolled."""
     with pytest.raises(rx.ReactantInternalError, match="static trip count"):
         rx.compile_offline(text)
+
+
+def test_single_launch_reduction_is_an_option(monkeypatch):
+    monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
+    rep = rx.compile_offline(P.sinsum_add(1 << 20), with_source=True)
+    assert re.findall(r"kind=(\w+)", rep) == ["reduce"] and "atomicAdd(ticket" in rep

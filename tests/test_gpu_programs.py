@@ -29,6 +29,23 @@ def test_sinsum_add(rx, client, n):
     assert abs(float(ref[0].a) - exact) <= tol * max(abs(exact), 1e-6) + 1e-6 * scale
 
 
+def test_sinsum_add_single_launch_reduction(rx, client, monkeypatch):
+    """The one-launch form of the full reduction (last workgroup combines) gives the same bits as
+    the two-launch form: partials are combined in the same order."""
+    n = 1 << 20
+    x = np.random.default_rng(0).uniform(-np.pi, np.pi, n).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-np.pi, np.pi, n).astype(np.float32)
+    args = [I.Tensor(x, "f32"), I.Tensor(y, "f32")]
+    two, exe2 = gpu_run(rx, client, P.sinsum_add(n), args)
+    monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
+    one, exe1 = gpu_run(rx, client, P.sinsum_add(n), args)
+    assert len(exe1.launches()) == 1 and len(exe2.launches()) == 2
+    for _ in range(3):      # the ticket counter is back at zero after every run
+        again, _ = gpu_run(rx, client, P.sinsum_add(n), args, exe=exe1)
+        assert again[0].a.tobytes() == one[0].a.tobytes()
+    assert one[0].a.tobytes() == two[0].a.tobytes()
+
+
 @pytest.mark.parametrize("shape,embed", [((6, 5, 4), "pad"), ((6, 5, 4), "dus"), ((32, 16, 8), "pad"),
                                          ((64, 64, 32), "pad")])
 def test_stencil(rx, client, shape, embed):
