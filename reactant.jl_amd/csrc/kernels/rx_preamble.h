@@ -285,6 +285,11 @@ RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
   return r;
 }
 
+// Workgroup barrier for data exchanged through LDS only: waits for this wavefront's LDS
+// operations, not for its outstanding global loads (a __syncthreads() drains those too, which
+// would serialize register prefetch with the compute phase that follows the barrier).
+RX_DEV void rx_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // XCD-aware placement: workgroups are dealt round-robin to the 8 XCDs, each with
 // its own L2.  This maps hardware workgroup id -> logical tile so that each XCD
 // walks one contiguous range of tiles.

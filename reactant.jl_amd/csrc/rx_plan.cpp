@@ -560,7 +560,7 @@ struct Planner {
       o << "#pragma unroll\n  for (int k = 0; k < " << D << "; ++k) nx" << slot << "[k] = " << ldf << "<" << vt << ">(in" << slot << " + rx_clamp_idx<" << it
         << ">(z0 + k, " << Z - 1 << ") * " << Y * X << (em.idx64 ? "LL" : "") << " + colc);\n";
     }
-    o << "  __syncthreads();\n";
+    o << "  rx_lds_barrier();\n";
     o << "  for (int zb = z0; zb < zend; zb += " << D << ") {\n";
     o << "#pragma unroll\n    for (int j = 0; j < " << D << "; ++j) {\n";
     o << "      const int z = zb + j;\n";
@@ -585,7 +585,7 @@ struct Planner {
     o << "      }\n";
     o << "      store_plane(z + " << hhi[0] + 1 << ", pre[(j + 1) % " << D << "]);\n";
     o << "      load_plane(z + " << hhi[0] + 1 + D << ", pre[(j + 1) % " << D << "]);\n";
-    o << "      __syncthreads();\n";
+    o << "      rx_lds_barrier();\n";
     o << "    }\n  }\n}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;
@@ -700,6 +700,7 @@ struct Planner {
       auto pf = fuse_prev.find(root);
       if (pf != fuse_prev.end()) {
         const int prev = pf->second;
+        if (opt.stencil_march2 && emit_map_march2(root, prev, sp)) return true;
         if (emit_map_lds2(root, prev, sp)) return true;
         // not fused after all: the producer gets its own launch first
         fuse_prev.erase(pf);
@@ -811,7 +812,7 @@ struct Planner {
       }
       o << "    }\n  }\n";
     }
-    o << "  __syncthreads();\n";
+    o << "  rx_lds_barrier();\n";
     o << "  if (!live) return;\n";
     o << "#pragma unroll\n  for (int lz = 0; lz < " << TZ << "; ++lz) {\n";
     o << "    const " << it << " i0 = z0 + lz;\n";
@@ -984,7 +985,7 @@ struct Planner {
     o << "  const int ly = lrem / " << TXV << ", lxe = (lrem % " << TXV << ") * " << vec << ";\n";
     o << "  const " << it << " i1 = rx_min<" << it << ">(y0 + ly, " << Y - 1 << "), i2b = rx_min<" << it << ">(x0 + lxe, " << X - vec << ");\n";
     o << "  const bool live = y0 + ly < " << Y << " && x0 + lxe < " << X << ";\n";
-    o << "  __syncthreads();\n";
+    o << "  rx_lds_barrier();\n";
     // stage B: first step on region B, kept in registers until every wavefront has read the tile
     o << "  " << vt << " sb[" << nitB << "];\n";
     o << "#pragma unroll\n  for (int q = 0; q < " << nitB << "; ++q) {\n";
@@ -1012,12 +1013,12 @@ struct Planner {
         o << "    " << vec_name(dv.first, 0) << "z[lk] = " << "rx_load" << "<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + linc);\n";
       o << "  }\n";
     }
-    o << "  __syncthreads();\n";
+    o << "  rx_lds_barrier();\n";
     o << "#pragma unroll\n  for (int q = 0; q < " << nitB << "; ++q) {\n";
     o << "    const int v = threadIdx.x + q * " << NB << ";\n";
     o << "    if (v < " << totalB << ") rx_store(lds + v * " << vec << ", sb[q]);\n";
     o << "  }\n";
-    o << "  __syncthreads();\n";
+    o << "  rx_lds_barrier();\n";
     // stage C: second step on the output tile
     o << "  if (!live) return;\n";
     o << "#pragma unroll\n  for (int lk = 0; lk < " << TZ / PZ << "; ++lk) {\n";
@@ -1049,6 +1050,225 @@ struct Planner {
     }
     L.args.push_back(buffer_for(root));
     // both steps' compulsory traffic: the first step's inputs and output, then the second's
+    std::set<int> read2;
+    for (auto& l : ec.loads) read2.insert(l.node);
+    L.algo_bytes = algo_bytes(eb.inputs, {prev}) + algo_bytes(std::vector<int>(read2.begin(), read2.end()), {root});
+    L.desc = describe(prev) + " ; " + describe(root);
+    plan.launches.push_back(L);
+    return true;
+  }
+
+  // ------------------------------------------------------------------ two stencil steps, marching
+  // Same pairing as emit_map_lds2, other traversal: a workgroup owns TY x TX output columns and
+  // walks ZC planes along the slowest dimension.  Two rings of planes live in LDS: the source
+  // field A (with both halos in y/x) and the first step's values B (with the second step's halo).
+  // Every iteration t brings one new plane of A (requested one iteration earlier into registers),
+  // evaluates one plane of B from the ring of A, and evaluates one output plane from the ring
+  // of B.  Halo planes in z are therefore read and computed once per workgroup, not once per
+  // tile, and only the y/x surface of the column is recomputed.
+  bool emit_map_march2(int root, int prev, const StencilProbe& spR) {
+    const Node& rn = g.nodes[root];
+    const Node& pn = g.nodes[prev];
+    const auto& dims = rn.ty.dims;
+    if (pn.ty.dims != dims || pn.ty.dt != rn.ty.dt) return false;
+    StencilProbe spP;
+    if (!probe_stencil(prev, &spP) || spP.staged.size() != 1 || spP.vec != spR.vec) return false;
+    const int src = spP.staged[0];
+    if (g.nodes[src].ty.dims != dims) return false;
+    const int vec = spR.vec;
+    const Halo hR = spR.halos.at(prev), hP = spP.halos.at(src);
+    const int TY = opt.march2_tile[0], TX = opt.march2_tile[1];
+    if (TX % vec) return false;
+    const int TXV = TX / vec, NB = TXV * TY;
+    if (NB < 64 || NB > 1024 || NB % 64) return false;
+    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
+    const int64_t ZC = std::max<int64_t>(1, std::min<int64_t>(opt.march_planes, Z));
+    auto up = [&](int64_t v) { return (v + vec - 1) / vec * vec; };
+    const int64_t bxl = up(hR.lo[2]), bxh = up(hR.hi[2]);
+    const int64_t BY = TY + hR.lo[1] + hR.hi[1], BX = TX + bxl + bxh, BXV = BX / vec;
+    const int64_t axl = up(hP.lo[2]), axh = up(hP.hi[2]);
+    const int64_t AY = BY + hP.lo[1] + hP.hi[1], AX = BX + axl + axh, AXV = AX / vec;
+    const int64_t APLANE = AY * AX, BPLANE = BY * BX, AV = AY * AXV, BV = BY * BXV;
+    const int64_t RA = hP.lo[0] + hP.hi[0] + 1, RB = hR.lo[0] + hR.hi[0] + 1;   // planes alive at once
+    const int es = info(rn.ty.dt).size;
+    if ((RA * APLANE + RB * BPLANE) * es > 64 * 1024) return false;
+    const int64_t NLA = (AV + NB - 1) / NB, NLB = (BV + NB - 1) / NB;
+    if (NLA > 8 || NLB > 4) return false;
+    const std::string st = info(rn.ty.dt).stype;
+    const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
+    const int64_t dA = hP.lo[0] + hP.hi[0], dB = hR.lo[0] + hR.hi[0];
+
+    Emitter eb(g, [&](int x) { return x != prev && mat[x]; });
+    stencil_emitter(eb, prev, vec, {"j0", "j1", "j2"});
+    eb.indent = 12;
+    eb.direct_expr = [](int slot, int64_t D) { return "b" + vec_name(slot, D); };
+    eb.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+      if (eb.inputs[slot] != src) return false;
+      std::ostringstream e;   // plane b + off0 is the plane brought in (hi0 - off0) iterations ago
+      e << "ldsA[sa" << (hP.hi[0] - off[0]) << " + (by + " << (off[1] + hP.lo[1]) << ") * " << AX << " + bxe + l + " << (axl + off[2]) << "]";
+      *expr = e.str();
+      return true;
+    };
+    Index jb(3);
+    for (int d = 0; d < 3; ++d) { jb[d].var = "j" + std::to_string(d); jb[d].lo = 0; jb[d].hi = dims[d] - 1; }
+    std::string valB = eb.emit(prev, jb);
+    std::string bodyB = eb.take_code();
+    for (auto& dv : eb.direct_vecs) if (dv.second != 0) return false;
+
+    Emitter ec(g, [&](int x) { return x != root && mat[x]; });
+    stencil_emitter(ec, root, vec, {"i0", "i1", "i2"});
+    ec.indent = 10;
+    ec.idx64 = ec.idx64 || eb.idx64;
+    ec.inputs = eb.inputs;
+    ec.direct_expr = vec_name;
+    ec.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+      if (ec.inputs[slot] != prev) return false;
+      std::ostringstream e;
+      e << "ldsB[sb" << (hR.hi[0] - off[0]) << " + (ly + " << (off[1] + hR.lo[1]) << ") * " << BX << " + lxe + l + " << (bxl + off[2]) << "]";
+      *expr = e.str();
+      return true;
+    };
+    std::string valC = ec.emit(root, root_index(dims));
+    std::string bodyC = ec.take_code();
+    for (auto& dv : ec.direct_vecs) if (dv.second != 0) return false;
+    for (auto& l : ec.loads) if (l.node == prev && !l.affine) return false;
+    const std::string it = ec.idx_t();
+    const std::string LL = ec.idx64 ? "LL" : "";
+    const int prev_slot = ec.slot_of(prev), sslot = ec.slot_of(src);
+    auto vts_of = [&](Emitter& em, int slot) { return "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">"; };
+
+    const std::string kname = "@K@_stencil2m";
+    const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + ZC - 1) / ZC;
+    std::ostringstream o;
+    o << "// two stencil steps, marching along dim 0 (" << TY << "x" << TX << " outputs per plane, " << ZC << " planes per workgroup, rings of " << RA << " and "
+      << RB << " planes in LDS): " << describe(prev) << " ; " << describe(root) << " -> " << rn.ty.str() << "\n";
+    {
+      std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(NB) + ") void " + kname + "(";
+      for (size_t k = 0; k < ec.inputs.size(); ++k) {
+        if ((int)k == prev_slot) continue;
+        s += ptr_decl(info(g.nodes[ec.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k)) + ", ";
+      }
+      s += ptr_decl(st, false, "out0") + ")";
+      o << s << " {\n";
+    }
+    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsA[" << RA * APLANE << "];\n";
+    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << RB * BPLANE << "];\n";
+    const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, (int)ZC, std::max(1, 32 / TY));
+    o << "  const int zend = z0 + " << ZC << " < " << Z << " ? z0 + " << ZC << " : " << Z << ";\n";
+    // plane-independent parts of the addresses (clamped into the array; clamped cells are never used)
+    o << "  " << it << " poffA[" << NLA << "], poffB[" << NLB << "];\n";
+    o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) {\n";
+    o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << AV - 1 << ");\n";
+    o << "    const int xv = v % " << AXV << ", yy = v / " << AXV << ";\n";
+    o << "    poffA[q] = rx_clamp_idx<" << it << ">(y0 - " << (hR.lo[1] + hP.lo[1]) << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - "
+      << (bxl + axl) << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
+    o << "#pragma unroll\n  for (int q = 0; q < " << NLB << "; ++q) {\n";
+    o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << BV - 1 << ");\n";
+    o << "    const int xv = v % " << BXV << ", yy = v / " << BXV << ";\n";
+    o << "    poffB[q] = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - " << bxl
+      << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
+    o << "  const int ly = threadIdx.x / " << TXV << ", lxe = (threadIdx.x % " << TXV << ") * " << vec << ";\n";
+    o << "  const " << it << " i1 = rx_min<" << it << ">(y0 + ly, " << Y - 1 << "), i2b = rx_min<" << it << ">(x0 + lxe, " << X - vec << ");\n";
+    o << "  const bool live = y0 + ly < " << Y << " && x0 + lxe < " << X << ";\n";
+    o << "  const " << it << " colc = i1 * " << X << " + i2b;\n";
+    o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", nit = zend - 1 + " << (hR.hi[0] + hP.hi[0]) << " - tA0 + 1, zb0 = z0 - " << hR.lo[0] << ";\n";
+    o << "  auto plane = [&](int p) { return (" << it << ")rx_clamp_idx<int>(p, " << Z - 1 << ") * " << Y * X << LL << "; };\n";
+    // Requests run D iterations ahead of their use: register slot (iteration % D) holds the A
+    // plane and the first step's streamed inputs that iteration needs.  The loop is unrolled D
+    // times so the slot is a compile-time index.
+    const int D = std::max(1, std::min(opt.march_depth, 4));
+    o << "  " << vt << " preA[" << D << "][" << NLA << "];\n";
+    for (int k = 0; k < D; ++k)
+      o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) preA[" << k << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << k
+        << ") + poffA[q]);\n";
+    for (auto& dv : eb.direct_vecs) {
+      o << "  " << vts_of(eb, dv.first) << " ub" << dv.first << "[" << D << "][" << NLB << "];\n";
+      for (int k = 0; k < D; ++k)
+        o << "#pragma unroll\n  for (int q = 0; q < " << NLB << "; ++q) ub" << dv.first << "[" << (k + dA) % D << "][q] = rx_load<" << vts_of(eb, dv.first)
+          << ">(in" << dv.first << " + plane(zb0 + " << k << ") + poffB[q]);\n";
+    }
+    for (auto& dv : ec.direct_vecs)
+      o << "  " << vts_of(ec, dv.first) << " uc" << dv.first << " = rx_load<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + plane(z0) + colc);\n";
+    o << "  for (int itb = 0; itb < nit; itb += " << D << ") {\n";
+    for (int P = 0; P < D; ++P) {
+      o << "    if (itb + " << P << " < nit) {\n";
+      o << "    const int itn = itb + " << P << ";\n";
+      o << "    const int t = tA0 + itn;\n";
+      // (i) the plane requested D iterations ago goes to the ring; request the plane D ahead
+      o << "    {\n      " << st << "* dst = ldsA + (itn % " << RA << ") * " << APLANE << ";\n";
+      o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
+      o << "        const int v = threadIdx.x + q * " << NB << ";\n";
+      o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[" << P << "][q]);\n      }\n";
+      o << "      if (itn + " << D << " < nit) {\n";
+      o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[" << P << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(t + " << D
+        << ") + poffA[q]);\n";
+      o << "      }\n    }\n";
+      o << "    rx_lds_barrier();\n";
+      // (ii) one plane of the first step
+      o << "    const int ib = itn - " << dA << ";\n";
+      o << "    if (ib >= 0) {\n";
+      o << "      const int b = zb0 + ib;\n";
+      for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((itn + " << (2 * RA - k) << ") % " << RA << ") * " << APLANE << ";\n";
+      o << "      " << st << "* dstb = ldsB + (ib % " << RB << ") * " << BPLANE << ";\n";
+      o << "      const " << it << " j0 = rx_clamp_idx<" << it << ">(b, " << Z - 1 << ");\n";
+      o << "#pragma unroll\n      for (int q = 0; q < " << NLB << "; ++q) {\n";
+      o << "        const int v = threadIdx.x + q * " << NB << ";\n";
+      o << "        if (v < " << BV << ") {\n";
+      o << "          const int bxv = v % " << BXV << ", by = v / " << BXV << ", bxe = bxv * " << vec << ";\n";
+      o << "          const " << it << " j1 = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + by, " << Y - 1 << ");\n";
+      o << "          const " << it << " j2b = rx_clamp_idx<" << it << ">(x0 - " << bxl << " + bxe, " << X - vec << ");\n";
+      for (auto& dv : eb.direct_vecs)
+        o << "          const " << vts_of(eb, dv.first) << " b" << vec_name(dv.first, 0) << " = ub" << dv.first << "[" << P << "][q];\n";
+      o << "          " << vt << " res;\n";
+      o << "#pragma unroll\n          for (int l = 0; l < " << vec << "; ++l) {\n";
+      o << "            const " << it << " j2 = j2b + l;\n";
+      o << bodyB;
+      o << "            res.v[l] = " << Emitter::store_conv(pn.ty.dt, valB) << ";\n          }\n";
+      o << "          rx_store(dstb + v * " << vec << ", res);\n";
+      o << "        }\n      }\n";
+      o << "      if (ib + " << D << " < nit - " << dA << ") {\n";
+      for (auto& dv : eb.direct_vecs) {
+        o << "#pragma unroll\n        for (int q = 0; q < " << NLB << "; ++q) ub" << dv.first << "[" << P << "][q] = rx_load<" << vts_of(eb, dv.first) << ">(in"
+          << dv.first << " + plane(b + " << D << ") + poffB[q]);\n";
+      }
+      o << "      }\n    }\n";
+      o << "    rx_lds_barrier();\n";
+      // (iii) one output plane of the second step
+      o << "    const int iz = ib - " << dB << ";\n";
+      o << "    if (iz >= 0) {\n";
+      o << "      const int z = z0 + iz;\n";
+      for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((ib + " << (2 * RB - k) << ") % " << RB << ") * " << BPLANE << ";\n";
+      o << "      if (live) {\n";
+      o << "        const " << it << " i0 = z;\n";
+      o << "        const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
+      for (auto& dv : ec.direct_vecs) o << "        const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uc" << dv.first << ";\n";
+      o << "        " << vt << " res;\n";
+      o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
+      o << "          const " << it << " i2 = i2b + l;\n";
+      o << bodyC;
+      o << "          res.v[l] = " << ec.store_value(rn.ty.dt, valC) << ";\n        }\n";
+      o << "        " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
+      o << "      }\n";
+      o << "      if (z + 1 < zend) {\n";
+      for (auto& dv : ec.direct_vecs)
+        o << "        uc" << dv.first << " = rx_load<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + plane(z + 1) + colc);\n";
+      o << "      }\n    }\n";
+      o << "    }\n";
+    }
+    o << "  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = "map_stencil_lds2";
+    L.grid[0] = (unsigned)launch_blocks;
+    L.block[0] = NB;
+    std::vector<int> ins;
+    for (size_t k = 0; k < ec.inputs.size(); ++k) {
+      if ((int)k == prev_slot) continue;
+      ins.push_back(ec.inputs[k]);
+      L.args.push_back(buffer_for(ec.inputs[k]));
+    }
+    L.args.push_back(buffer_for(root));
     std::set<int> read2;
     for (auto& l : ec.loads) read2.insert(l.node);
     L.algo_bytes = algo_bytes(eb.inputs, {prev}) + algo_bytes(std::vector<int>(read2.begin(), read2.end()), {root});
