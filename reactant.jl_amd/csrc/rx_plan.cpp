@@ -601,11 +601,6 @@ struct Planner {
     return true;
   }
 
-  // ------------------------------------------------------------------ stencil maps through LDS halo tiles
-  // A rank-3 map that reads some input at several constant offsets (a stencil): the workgroup
-  // owns a TZ x TY x TX block of outputs, loads that input's block plus halo into LDS once with
-  // aligned 16-byte loads, and every neighbour access becomes an LDS read.  Inputs read only at
-  // the output's own position are still streamed from global memory with vector loads.
   // Tile order of the stencil kernels.  Workgroups are dealt round-robin to the 8 XCDs, each with
   // its own L2.  The y-tiles are cut into slabs of `sy` tiles; XCD k owns slabs k, k+8, ... and
   // walks each of them layer by layer in z, so the planes that consecutive layers share (and the
@@ -683,6 +678,11 @@ struct Planner {
     return !sp->staged.empty();
   }
 
+  // ------------------------------------------------------------------ stencil maps through LDS halo tiles
+  // A rank-3 map that reads some input at several constant offsets (a stencil): the workgroup
+  // owns a TZ x TY x TX block of outputs, loads that input's block plus halo into LDS once with
+  // aligned 16-byte loads, and every neighbour access becomes an LDS read.  Inputs read only at
+  // the output's own position are still streamed from global memory with vector loads.
   bool emit_map_lds(int root) {
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
@@ -1082,7 +1082,9 @@ struct Planner {
     const int TXV = TX / vec, NB = TXV * TY;
     if (NB < 64 || NB > 1024 || NB % 64) return false;
     const int64_t Z = dims[0], Y = dims[1], X = dims[2];
-    const int64_t ZC = std::max<int64_t>(1, std::min<int64_t>(opt.march_planes, Z));
+    // planes per workgroup: the extent is cut into equal chunks of about march2_planes
+    const int64_t nchunks = std::max<int64_t>(1, (Z + opt.march2_planes - 1) / opt.march2_planes);
+    const int64_t ZC = (Z + nchunks - 1) / nchunks;
     auto up = [&](int64_t v) { return (v + vec - 1) / vec * vec; };
     const int64_t bxl = up(hR.lo[2]), bxh = up(hR.hi[2]);
     const int64_t BY = TY + hR.lo[1] + hR.hi[1], BX = TX + bxl + bxh, BXV = BX / vec;
@@ -1093,7 +1095,8 @@ struct Planner {
     const int es = info(rn.ty.dt).size;
     if ((RA * APLANE + RB * BPLANE) * es > 64 * 1024) return false;
     const int64_t NLA = (AV + NB - 1) / NB, NLB = (BV + NB - 1) / NB;
-    if (NLA > 8 || NLB > 4) return false;
+    if (NLA > 8) return false;
+    (void)NLB;
     const std::string st = info(rn.ty.dt).stype;
     const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
     const int64_t dA = hP.lo[0] + hP.hi[0], dB = hR.lo[0] + hR.hi[0];
@@ -1155,106 +1158,136 @@ struct Planner {
     o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << RB * BPLANE << "];\n";
     const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, (int)ZC, std::max(1, 32 / TY));
     o << "  const int zend = z0 + " << ZC << " < " << Z << " ? z0 + " << ZC << " : " << Z << ";\n";
+    // The first step is evaluated in two passes.  The inner pass maps thread -> point exactly as
+    // the second step does, so the streamed inputs it loads for plane b are still in its registers
+    // when the second step reaches that plane.  The shell pass covers the rest of region B (the
+    // second step's halo in y/x): NSH vectors, enumerated row by row.
+    const int64_t nTop = hR.lo[1] * BXV, nBot = hR.hi[1] * BXV, nL = bxl / vec, nR = bxh / vec, nS = nL + nR;
+    const int64_t NSH = nTop + nBot + (int64_t)TY * nS, NSP = (NSH + NB - 1) / NB;
+    if (NSP > 2) return false;
+    const int64_t h = hR.hi[0];   // the second step's plane z is the first step's plane b - h
     // plane-independent parts of the addresses (clamped into the array; clamped cells are never used)
-    o << "  " << it << " poffA[" << NLA << "], poffB[" << NLB << "];\n";
+    o << "  " << it << " poffA[" << NLA << "];\n";
     o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) {\n";
     o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << AV - 1 << ");\n";
     o << "    const int xv = v % " << AXV << ", yy = v / " << AXV << ";\n";
     o << "    poffA[q] = rx_clamp_idx<" << it << ">(y0 - " << (hR.lo[1] + hP.lo[1]) << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - "
       << (bxl + axl) << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
-    o << "#pragma unroll\n  for (int q = 0; q < " << NLB << "; ++q) {\n";
-    o << "    const int v = rx_min((int)threadIdx.x + q * " << NB << ", " << BV - 1 << ");\n";
-    o << "    const int xv = v % " << BXV << ", yy = v / " << BXV << ";\n";
-    o << "    poffB[q] = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - " << bxl
-      << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
     o << "  const int ly = threadIdx.x / " << TXV << ", lxe = (threadIdx.x % " << TXV << ") * " << vec << ";\n";
     o << "  const " << it << " i1 = rx_min<" << it << ">(y0 + ly, " << Y - 1 << "), i2b = rx_min<" << it << ">(x0 + lxe, " << X - vec << ");\n";
     o << "  const bool live = y0 + ly < " << Y << " && x0 + lxe < " << X << ";\n";
     o << "  const " << it << " colc = i1 * " << X << " + i2b;\n";
+    if (NSP > 0) {
+      o << "  int sby[" << NSP << "], sbxe[" << NSP << "];\n  " << it << " soff[" << NSP << "];\n";
+      o << "#pragma unroll\n  for (int q = 0; q < " << NSP << "; ++q) {\n";
+      o << "    const int s = rx_min((int)threadIdx.x + q * " << NB << ", " << NSH - 1 << ");\n";
+      o << "    int yy, xv;\n";
+      o << "    if (s < " << nTop << ") { yy = s / " << BXV << "; xv = s % " << BXV << "; }\n";
+      o << "    else if (s < " << nTop + nBot << ") { const int r = s - " << nTop << "; yy = " << hR.lo[1] + TY << " + r / " << BXV << "; xv = r % " << BXV << "; }\n";
+      if (nS > 0)
+        o << "    else { const int r = s - " << nTop + nBot << ", c = r % " << nS << "; yy = " << hR.lo[1] << " + r / " << nS << "; xv = c < " << nL << " ? c : c + " << TXV << "; }\n";
+      else
+        o << "    else { yy = 0; xv = 0; }\n";
+      o << "    sby[q] = yy; sbxe[q] = xv * " << vec << ";\n";
+      o << "    soff[q] = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - " << bxl
+        << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
+    }
     o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", nit = zend - 1 + " << (hR.hi[0] + hP.hi[0]) << " - tA0 + 1, zb0 = z0 - " << hR.lo[0] << ";\n";
     o << "  auto plane = [&](int p) { return (" << it << ")rx_clamp_idx<int>(p, " << Z - 1 << ") * " << Y * X << LL << "; };\n";
-    // Requests run D iterations ahead of their use: register slot (iteration % D) holds the A
-    // plane and the first step's streamed inputs that iteration needs.  The loop is unrolled D
-    // times so the slot is a compile-time index.
-    const int D = std::max(1, std::min(opt.march_depth, 4));
-    o << "  " << vt << " preA[" << D << "][" << NLA << "];\n";
-    for (int k = 0; k < D; ++k)
-      o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) preA[" << k << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << k
-        << ") + poffA[q]);\n";
-    for (auto& dv : eb.direct_vecs) {
-      o << "  " << vts_of(eb, dv.first) << " ub" << dv.first << "[" << D << "][" << NLB << "];\n";
-      for (int k = 0; k < D; ++k)
-        o << "#pragma unroll\n  for (int q = 0; q < " << NLB << "; ++q) ub" << dv.first << "[" << (k + dA) % D << "][q] = rx_load<" << vts_of(eb, dv.first)
-          << ">(in" << dv.first << " + plane(zb0 + " << k << ") + poffB[q]);\n";
-    }
-    for (auto& dv : ec.direct_vecs)
-      o << "  " << vts_of(ec, dv.first) << " uc" << dv.first << " = rx_load<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + plane(z0) + colc);\n";
-    o << "  for (int itb = 0; itb < nit; itb += " << D << ") {\n";
-    for (int P = 0; P < D; ++P) {
-      o << "    if (itb + " << P << " < nit) {\n";
-      o << "    const int itn = itb + " << P << ";\n";
-      o << "    const int t = tA0 + itn;\n";
-      // (i) the plane requested D iterations ago goes to the ring; request the plane D ahead
-      o << "    {\n      " << st << "* dst = ldsA + (itn % " << RA << ") * " << APLANE << ";\n";
-      o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
-      o << "        const int v = threadIdx.x + q * " << NB << ";\n";
-      o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[" << P << "][q]);\n      }\n";
-      o << "      if (itn + " << D << " < nit) {\n";
-      o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[" << P << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(t + " << D
-        << ") + poffA[q]);\n";
-      o << "      }\n    }\n";
-      o << "    rx_lds_barrier();\n";
-      // (ii) one plane of the first step
-      o << "    const int ib = itn - " << dA << ";\n";
-      o << "    if (ib >= 0) {\n";
-      o << "      const int b = zb0 + ib;\n";
-      for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((itn + " << (2 * RA - k) << ") % " << RA << ") * " << APLANE << ";\n";
-      o << "      " << st << "* dstb = ldsB + (ib % " << RB << ") * " << BPLANE << ";\n";
-      o << "      const " << it << " j0 = rx_clamp_idx<" << it << ">(b, " << Z - 1 << ");\n";
-      o << "#pragma unroll\n      for (int q = 0; q < " << NLB << "; ++q) {\n";
-      o << "        const int v = threadIdx.x + q * " << NB << ";\n";
-      o << "        if (v < " << BV << ") {\n";
-      o << "          const int bxv = v % " << BXV << ", by = v / " << BXV << ", bxe = bxv * " << vec << ";\n";
-      o << "          const " << it << " j1 = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + by, " << Y - 1 << ");\n";
-      o << "          const " << it << " j2b = rx_clamp_idx<" << it << ">(x0 - " << bxl << " + bxe, " << X - vec << ");\n";
-      for (auto& dv : eb.direct_vecs)
-        o << "          const " << vts_of(eb, dv.first) << " b" << vec_name(dv.first, 0) << " = ub" << dv.first << "[" << P << "][q];\n";
-      o << "          " << vt << " res;\n";
-      o << "#pragma unroll\n          for (int l = 0; l < " << vec << "; ++l) {\n";
-      o << "            const " << it << " j2 = j2b + l;\n";
-      o << bodyB;
-      o << "            res.v[l] = " << Emitter::store_conv(pn.ty.dt, valB) << ";\n          }\n";
-      o << "          rx_store(dstb + v * " << vec << ", res);\n";
-      o << "        }\n      }\n";
-      o << "      if (ib + " << D << " < nit - " << dA << ") {\n";
-      for (auto& dv : eb.direct_vecs) {
-        o << "#pragma unroll\n        for (int q = 0; q < " << NLB << "; ++q) ub" << dv.first << "[" << P << "][q] = rx_load<" << vts_of(eb, dv.first) << ">(in"
-          << dv.first << " + plane(b + " << D << ") + poffB[q]);\n";
+    // first requests: A plane tA0 and the streamed inputs of the first B plane
+    o << "  " << vt << " preA[" << NLA << "];\n";
+    o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0) + poffA[q]);\n";
+    std::set<int> stream_slots;
+    for (auto& dv : eb.direct_vecs) stream_slots.insert(dv.first);
+    for (auto& dv : ec.direct_vecs) stream_slots.insert(dv.first);
+    for (int sl : stream_slots) {
+      const std::string vts = vts_of(ec, sl);
+      o << "  " << vts << " uq" << sl << "[" << h + 1 << "], un" << sl << ";\n";
+      o << "  uq" << sl << "[0] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + colc);\n";
+      if (NSP > 0 && eb.direct_vecs.count({sl, 0})) {
+        o << "  " << vts << " us" << sl << "[" << NSP << "], usn" << sl << "[" << NSP << "];\n";
+        o << "#pragma unroll\n  for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + soff[q]);\n";
       }
-      o << "      }\n    }\n";
-      o << "    rx_lds_barrier();\n";
-      // (iii) one output plane of the second step
-      o << "    const int iz = ib - " << dB << ";\n";
-      o << "    if (iz >= 0) {\n";
-      o << "      const int z = z0 + iz;\n";
-      for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((ib + " << (2 * RB - k) << ") % " << RB << ") * " << BPLANE << ";\n";
-      o << "      if (live) {\n";
-      o << "        const " << it << " i0 = z;\n";
-      o << "        const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
-      for (auto& dv : ec.direct_vecs) o << "        const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uc" << dv.first << ";\n";
-      o << "        " << vt << " res;\n";
-      o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
-      o << "          const " << it << " i2 = i2b + l;\n";
-      o << bodyC;
-      o << "          res.v[l] = " << ec.store_value(rn.ty.dt, valC) << ";\n        }\n";
-      o << "        " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
-      o << "      }\n";
-      o << "      if (z + 1 < zend) {\n";
-      for (auto& dv : ec.direct_vecs)
-        o << "        uc" << dv.first << " = rx_load<" << vts_of(ec, dv.first) << ">(in" << dv.first << " + plane(z + 1) + colc);\n";
-      o << "      }\n    }\n";
-      o << "    }\n";
     }
+    // body of the first step for one vector of region B
+    auto emit_B = [&](const std::string& pad, const std::string& by, const std::string& bxe, const std::string& j1, const std::string& j2b,
+                      const std::function<std::string(int)>& stream, const std::string& ldsoff) {
+      o << pad << "{\n";
+      o << pad << "  const int by = " << by << ", bxe = " << bxe << ";\n";
+      o << pad << "  const " << it << " j1 = " << j1 << ", j2b = " << j2b << ";\n";
+      for (auto& dv : eb.direct_vecs) o << pad << "  const " << vts_of(eb, dv.first) << " b" << vec_name(dv.first, 0) << " = " << stream(dv.first) << ";\n";
+      o << pad << "  " << vt << " res;\n";
+      o << "#pragma unroll\n" << pad << "  for (int l = 0; l < " << vec << "; ++l) {\n";
+      o << pad << "    const " << it << " j2 = j2b + l;\n";
+      o << bodyB;
+      o << pad << "    res.v[l] = " << Emitter::store_conv(pn.ty.dt, valB) << ";\n" << pad << "  }\n";
+      o << pad << "  rx_store(dstb + " << ldsoff << ", res);\n";
+      o << pad << "}\n";
+    };
+    o << "  for (int itn = 0; itn < nit; ++itn) {\n";
+    o << "    const int t = tA0 + itn;\n";
+    // (i) the plane requested last iteration goes to the ring; request the next one
+    o << "    {\n      " << st << "* dst = ldsA + (itn % " << RA << ") * " << APLANE << ";\n";
+    o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
+    o << "        const int v = threadIdx.x + q * " << NB << ";\n";
+    o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[q]);\n      }\n";
+    o << "      if (itn + 1 < nit) {\n";
+    o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(t + 1) + poffA[q]);\n";
+    o << "      }\n    }\n";
+    o << "    rx_lds_barrier();\n";
+    // (ii) one plane of the first step
+    o << "    const int ib = itn - " << dA << ";\n";
+    o << "    if (ib >= 0) {\n";
+    o << "      const int b = zb0 + ib;\n";
+    o << "      const bool more = ib + 1 < nit - " << dA << ";\n";
+    o << "      if (more) {\n";
+    for (int sl : stream_slots) {
+      const std::string vts = vts_of(ec, sl);
+      o << "        un" << sl << " = rx_load<" << vts << ">(in" << sl << " + plane(b + 1) + colc);\n";
+      if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
+        o << "#pragma unroll\n        for (int q = 0; q < " << NSP << "; ++q) usn" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(b + 1) + soff[q]);\n";
+    }
+    o << "      }\n";
+    for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((itn + " << (2 * RA - k) << ") % " << RA << ") * " << APLANE << ";\n";
+    o << "      " << st << "* dstb = ldsB + (ib % " << RB << ") * " << BPLANE << ";\n";
+    o << "      const " << it << " j0 = rx_clamp_idx<" << it << ">(b, " << Z - 1 << ");\n";
+    emit_B("      ", "ly + " + std::to_string(hR.lo[1]), "lxe + " + std::to_string(bxl), "i1", "i2b",
+           [&](int sl) { return "uq" + std::to_string(sl) + "[0]"; }, "by * " + std::to_string(BX) + " + bxe");
+    for (int64_t q = 0; q < NSP; ++q) {
+      o << "      if ((int)threadIdx.x + " << q * NB << " < " << NSH << ") {\n";
+      const std::string qs = std::to_string(q);
+      emit_B("        ", "sby[" + qs + "]", "sbxe[" + qs + "]",
+             "rx_clamp_idx<" + it + ">(y0 - " + std::to_string(hR.lo[1]) + " + sby[" + qs + "], " + std::to_string(Y - 1) + ")",
+             "rx_clamp_idx<" + it + ">(x0 - " + std::to_string(bxl) + " + sbxe[" + qs + "], " + std::to_string(X - vec) + ")",
+             [&](int sl) { return "us" + std::to_string(sl) + "[" + qs + "]"; }, "by * " + std::to_string(BX) + " + bxe");
+      o << "      }\n";
+    }
+    o << "    }\n";
+    o << "    rx_lds_barrier();\n";
+    // (iii) one output plane of the second step
+    o << "    const int iz = ib - " << dB << ";\n";
+    o << "    if (iz >= 0 && live) {\n";
+    o << "      const int z = z0 + iz;\n";
+    for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((ib + " << (2 * RB - k) << ") % " << RB << ") * " << BPLANE << ";\n";
+    o << "      const " << it << " i0 = z;\n";
+    o << "      const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
+    for (auto& dv : ec.direct_vecs) o << "      const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uq" << dv.first << "[" << h << "];\n";
+    o << "      " << vt << " res;\n";
+    o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
+    o << "        const " << it << " i2 = i2b + l;\n";
+    o << bodyC;
+    o << "        res.v[l] = " << ec.store_value(rn.ty.dt, valC) << ";\n      }\n";
+    o << "      " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
+    o << "    }\n";
+    // the streamed inputs move one plane on
+    o << "    if (ib >= 0) {\n";
+    for (int sl : stream_slots) {
+      for (int64_t k = h; k >= 1; --k) o << "      uq" << sl << "[" << k << "] = uq" << sl << "[" << k - 1 << "];\n";
+      o << "      uq" << sl << "[0] = un" << sl << ";\n";
+      if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
+        o << "#pragma unroll\n      for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << "[q];\n";
+    }
+    o << "    }\n";
     o << "  }\n}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;

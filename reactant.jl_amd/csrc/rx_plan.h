@@ -55,8 +55,9 @@ struct PlanOptions {
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS
   int lds_tile2[3] = {4, 8, 64};   // outputs per workgroup tile of the two-step kernel
   int lds2_threads = 512;          // its workgroup size
-  bool stencil_march2 = false;     // two-step kernel marching along the slowest dimension instead of 3-D tiles
-  int march2_tile[2] = {16, 32};   // its outputs per plane (rows, columns)
+  bool stencil_march2 = true;      // two-step kernel marching along the slowest dimension instead of 3-D tiles
+  int march2_tile[2] = {8, 64};    // its outputs per plane (rows, columns)
+  int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
   bool stencil_march = false;   // stencil maps: a workgroup marches along the slowest dimension with a ring of planes in LDS
   int march_depth = 3;          // planes of global loads kept in flight (in registers) ahead of their use
   int march_planes = 32;        // planes produced per workgroup when marching

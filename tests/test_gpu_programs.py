@@ -82,14 +82,31 @@ def _stencil_case(rx, client, shape, embed, steps, elt="f64"):
 @pytest.mark.parametrize("shape,embed,steps", [((70, 21, 9), "pad", 2), ((70, 21, 9), "dus", 2), ((64, 40, 20), "pad", 4),
                                                ((130, 17, 6), "pad", 3), ((58, 26, 5), "dus", 5), ((250, 10, 2), "pad", 2), ((20, 130, 4), "pad", 2),
                                                ((20, 150, 4), "dus", 3)])
-def test_stencil_two_steps_per_kernel(rx, client, monkeypatch, shape, embed, steps):
+@pytest.mark.parametrize("march", ["1", "0"])
+def test_stencil_two_steps_per_kernel(rx, client, monkeypatch, shape, embed, steps, march):
     """Pairs of steps share one kernel (the first step's field lives only in LDS): the values are
-    the same bits as the oracle's, for tiles cut by every array edge and an odd step left over."""
+    the same bits as the oracle's, for tiles cut by every array edge and an odd step left over.
+    Both traversals: marching along the slowest dimension with plane rings, and 3-D tiles."""
     monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    monkeypatch.setenv("RX_STENCIL_MARCH2", march)
     got, ref, exe = _stencil_case(rx, client, shape, embed, steps)
-    kinds = [l["kind"] for l in exe.launches()]
+    launches = exe.launches()
+    kinds = [l["kind"] for l in launches]
     assert kinds.count("map_stencil_lds2") == steps // 2 and len(kinds) == steps // 2 + steps % 2
+    assert launches[0]["kernel"].endswith("_stencil2m" if march == "1" else "_stencil2")
     assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("planes,tile", [("3", "8,64"), ("5", "16,32"), ("100", "4,128"), ("7", "32,16")])
+def test_stencil_marching_chunks_and_tiles(rx, client, monkeypatch, planes, tile):
+    """The marching kernel with chunks shorter and longer than the grid and other plane tiles."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    monkeypatch.setenv("RX_MARCH2_PLANES", planes)
+    monkeypatch.setenv("RX_MARCH2_TILE", tile)
+    for shape, embed in [((70, 21, 9), "pad"), ((20, 130, 11), "dus")]:
+        got, ref, exe = _stencil_case(rx, client, shape, embed, 2)
+        assert exe.launches()[0]["kernel"].endswith("_stencil2m")
+        assert np.array_equal(got, ref)
 
 
 def test_stencil_two_steps_f32_and_unfused_agree(rx, client, monkeypatch):
