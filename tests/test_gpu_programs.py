@@ -97,6 +97,56 @@ def test_stencil_two_steps_per_kernel(rx, client, monkeypatch, shape, embed, ste
     assert np.array_equal(got, ref)
 
 
+def _lopsided_stencil(nx, ny, nz, steps, offsets, H=3):
+    """steps of c <- pad(sum of c at `offsets` (dz, dy, dx) + u) with one-sided neighbourhoods."""
+    full, inner = [nz + 2 * H, ny + 2 * H, nx + 2 * H], [nz, ny, nx]
+    tf = "tensor<%dx%dx%dxf64>" % tuple(full)
+    ti = "tensor<%dx%dx%dxf64>" % tuple(inner)
+    lines, k, c = ["    %z = stablehlo.constant dense<0.000000e+00> : tensor<f64>"], [0], "%arg0"
+
+    def new():
+        k[0] += 1
+        return "%%v%d" % k[0]
+
+    def sl(x, d):
+        r, st = new(), [H + d[0], H + d[1], H + d[2]]
+        lines.append("    %s = stablehlo.slice %s [%s] : (%s) -> %s" % (
+            r, x, ", ".join("%d:%d" % (a, a + n) for a, n in zip(st, inner)), tf, ti))
+        return r
+
+    u = sl("%arg1", (0, 0, 0))
+    for _ in range(steps):
+        acc = u
+        for d in offsets:
+            t, r = sl(c, d), new()
+            lines.append("    %s = stablehlo.add %s, %s : %s" % (r, acc, t, ti))
+            acc = r
+        c = new()
+        lines.append("    %s = stablehlo.pad %s, %%z, low = [%d, %d, %d], high = [%d, %d, %d], interior = [0, 0, 0] : (%s, tensor<f64>) -> %s"
+                     % (c, acc, H, H, H, H, H, H, ti, tf))
+    return ("module @reactant_lopsided {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n%s\n    return %s : %s\n  }\n}\n"
+            % (tf, tf, tf, "\n".join(lines), c, tf))
+
+
+@pytest.mark.parametrize("march", ["1", "0"])
+@pytest.mark.parametrize("offsets", [[(0, 0, 0), (-1, 0, 0), (0, 1, 0), (0, 0, -2)],
+                                     [(0, 0, 0), (2, 0, 0), (0, -2, 0), (0, 0, 1), (0, 0, 3)],
+                                     [(0, 0, 0), (0, -1, 0), (0, 1, 0), (0, 0, 1)]])
+def test_two_step_kernels_with_one_sided_neighbourhoods(rx, client, monkeypatch, offsets, march):
+    """Halos that differ per side and per dimension (including none in z): ring sizes, shell
+    enumeration and tile halos follow the offsets the module actually uses."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    monkeypatch.setenv("RX_STENCIL_MARCH2", march)
+    nx, ny, nz = 70, 19, 7
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(11)
+    args = [I.Tensor(rng.uniform(-1, 1, full), "f64") for _ in range(2)]
+    text = _lopsided_stencil(nx, ny, nz, 3, offsets)
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["map_stencil_lds2", "map_stencil_lds"]
+    assert np.array_equal(got[0].a, oracle_run(text, args)[0].a)
+
+
 @pytest.mark.parametrize("planes,tile", [("3", "8,64"), ("5", "16,32"), ("100", "4,128"), ("7", "32,16")])
 def test_stencil_marching_chunks_and_tiles(rx, client, monkeypatch, planes, tile):
     """The marching kernel with chunks shorter and longer than the grid and other plane tiles."""
