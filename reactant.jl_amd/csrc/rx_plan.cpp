@@ -1091,7 +1091,7 @@ struct Planner {
     const int64_t axl = up(hP.lo[2]), axh = up(hP.hi[2]);
     const int64_t AY = BY + hP.lo[1] + hP.hi[1], AX = BX + axl + axh, AXV = AX / vec;
     const int64_t APLANE = AY * AX, BPLANE = BY * BX, AV = AY * AXV, BV = BY * BXV;
-    const int64_t RA = hP.lo[0] + hP.hi[0] + 1, RB = hR.lo[0] + hR.hi[0] + 1;   // planes alive at once
+    const int64_t RA = hP.lo[0] + hP.hi[0] + 2, RB = hR.lo[0] + hR.hi[0] + 2;   // a stencil's reach plus the plane being written
     const int es = info(rn.ty.dt).size;
     if ((RA * APLANE + RB * BPLANE) * es > 64 * 1024) return false;
     const int64_t NLA = (AV + NB - 1) / NB, NLB = (BV + NB - 1) / NB;
@@ -1192,23 +1192,42 @@ struct Planner {
       o << "    soff[q] = rx_clamp_idx<" << it << ">(y0 - " << hR.lo[1] << " + yy, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(x0 - " << bxl
         << " + xv * " << vec << ", " << X - vec << ");\n  }\n";
     }
-    o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", nit = zend - 1 + " << (hR.hi[0] + hP.hi[0]) << " - tA0 + 1, zb0 = z0 - " << hR.lo[0] << ";\n";
+    // Schedule: iteration n evaluates first-step plane n (from source planes that were in the ring
+    // before the iteration began), the output plane whose first-step planes were all finished
+    // before the iteration began, and puts the next source plane into the ring -- three pieces of
+    // work that touch disjoint ring slots, so one barrier per iteration is enough.  The rings hold
+    // one plane more than a stencil's reach for that.
+    const int64_t RA1 = dA + 2, RB1 = dB + 2;
+    o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", zb0 = z0 - " << hR.lo[0] << ";\n";
+    o << "  const int nB = zend - z0 + " << dB << ", nit = nB + 1;\n";
     o << "  auto plane = [&](int p) { return (" << it << ")rx_clamp_idx<int>(p, " << Z - 1 << ") * " << Y * X << LL << "; };\n";
-    // first requests: A plane tA0 and the streamed inputs of the first B plane
+    // prologue: the source planes the first first-step plane needs
     o << "  " << vt << " preA[" << NLA << "];\n";
-    o << "#pragma unroll\n  for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0) + poffA[q]);\n";
+    o << "  {\n    " << vt << " pro[" << dA + 1 << "][" << NLA << "];\n";
+    for (int64_t k = 0; k <= dA; ++k)
+      o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) pro[" << k << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << k
+        << ") + poffA[q]);\n";
+    o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << dA + 1 << ") + poffA[q]);\n";
     std::set<int> stream_slots;
     for (auto& dv : eb.direct_vecs) stream_slots.insert(dv.first);
     for (auto& dv : ec.direct_vecs) stream_slots.insert(dv.first);
+    const int64_t QL = h + 2;   // plane b of the first step is plane b - h - 1 ... of the second, one iteration later
+    for (int64_t k = 0; k <= dA; ++k) {
+      o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) {\n";
+      o << "      const int v = threadIdx.x + q * " << NB << ";\n";
+      o << "      if (v < " << AV << ") rx_store(ldsA + " << k * APLANE << " + v * " << vec << ", pro[" << k << "][q]);\n    }\n";
+    }
+    o << "  }\n";
     for (int sl : stream_slots) {
       const std::string vts = vts_of(ec, sl);
-      o << "  " << vts << " uq" << sl << "[" << h + 1 << "], un" << sl << ";\n";
+      o << "  " << vts << " uq" << sl << "[" << QL << "], un" << sl << ";\n";
       o << "  uq" << sl << "[0] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + colc);\n";
       if (NSP > 0 && eb.direct_vecs.count({sl, 0})) {
         o << "  " << vts << " us" << sl << "[" << NSP << "], usn" << sl << "[" << NSP << "];\n";
         o << "#pragma unroll\n  for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + soff[q]);\n";
       }
     }
+    o << "  rx_lds_barrier();\n";
     // body of the first step for one vector of region B
     auto emit_B = [&](const std::string& pad, const std::string& by, const std::string& bxe, const std::string& j1, const std::string& j2b,
                       const std::function<std::string(int)>& stream, const std::string& ldsoff) {
@@ -1224,32 +1243,46 @@ struct Planner {
       o << pad << "  rx_store(dstb + " << ldsoff << ", res);\n";
       o << pad << "}\n";
     };
-    o << "  for (int itn = 0; itn < nit; ++itn) {\n";
-    o << "    const int t = tA0 + itn;\n";
-    // (i) the plane requested last iteration goes to the ring; request the next one
-    o << "    {\n      " << st << "* dst = ldsA + (itn % " << RA << ") * " << APLANE << ";\n";
+    o << "  for (int n = 0; n < nit; ++n) {\n";
+    // requests for the next iteration
+    o << "    if (n + 1 < nB) {\n";
+    for (int sl : stream_slots) {
+      const std::string vts = vts_of(ec, sl);
+      o << "      un" << sl << " = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + 1) + colc);\n";
+      if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
+        o << "#pragma unroll\n      for (int q = 0; q < " << NSP << "; ++q) usn" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + 1) + soff[q]);\n";
+    }
+    o << "    }\n";
+    // the source plane requested last iteration goes to the ring; request the one after it
+    o << "    if (n + 1 < nB) {\n";
+    o << "      " << st << "* dst = ldsA + ((n + " << dA + 1 << ") % " << RA1 << ") * " << APLANE << ";\n";
     o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
     o << "        const int v = threadIdx.x + q * " << NB << ";\n";
     o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[q]);\n      }\n";
-    o << "      if (itn + 1 < nit) {\n";
-    o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(t + 1) + poffA[q]);\n";
+    o << "      if (n + 2 < nB) {\n";
+    o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + n + " << dA + 2
+      << ") + poffA[q]);\n";
     o << "      }\n    }\n";
-    o << "    rx_lds_barrier();\n";
-    // (ii) one plane of the first step
-    o << "    const int ib = itn - " << dA << ";\n";
-    o << "    if (ib >= 0) {\n";
-    o << "      const int b = zb0 + ib;\n";
-    o << "      const bool more = ib + 1 < nit - " << dA << ";\n";
-    o << "      if (more) {\n";
-    for (int sl : stream_slots) {
-      const std::string vts = vts_of(ec, sl);
-      o << "        un" << sl << " = rx_load<" << vts << ">(in" << sl << " + plane(b + 1) + colc);\n";
-      if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
-        o << "#pragma unroll\n        for (int q = 0; q < " << NSP << "; ++q) usn" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(b + 1) + soff[q]);\n";
-    }
-    o << "      }\n";
-    for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((itn + " << (2 * RA - k) << ") % " << RA << ") * " << APLANE << ";\n";
-    o << "      " << st << "* dstb = ldsB + (ib % " << RB << ") * " << BPLANE << ";\n";
+    // one output plane of the second step
+    o << "    const int iz = n - " << dB + 1 << ";\n";
+    o << "    if (iz >= 0 && live) {\n";
+    o << "      const int z = z0 + iz;\n";
+    for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((n + " << (2 * RB1 - 1 - k) << ") % " << RB1 << ") * " << BPLANE << ";\n";
+    o << "      const " << it << " i0 = z;\n";
+    o << "      const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
+    for (auto& dv : ec.direct_vecs) o << "      const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uq" << dv.first << "[" << h + 1 << "];\n";
+    o << "      " << vt << " res;\n";
+    o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
+    o << "        const " << it << " i2 = i2b + l;\n";
+    o << bodyC;
+    o << "        res.v[l] = " << ec.store_value(rn.ty.dt, valC) << ";\n      }\n";
+    o << "      " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
+    o << "    }\n";
+    // one plane of the first step
+    o << "    if (n < nB) {\n";
+    o << "      const int b = zb0 + n;\n";
+    for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((n + " << (dA - k) << ") % " << RA1 << ") * " << APLANE << ";\n";
+    o << "      " << st << "* dstb = ldsB + (n % " << RB1 << ") * " << BPLANE << ";\n";
     o << "      const " << it << " j0 = rx_clamp_idx<" << it << ">(b, " << Z - 1 << ");\n";
     emit_B("      ", "ly + " + std::to_string(hR.lo[1]), "lxe + " + std::to_string(bxl), "i1", "i2b",
            [&](int sl) { return "uq" + std::to_string(sl) + "[0]"; }, "by * " + std::to_string(BX) + " + bxe");
@@ -1263,31 +1296,14 @@ struct Planner {
       o << "      }\n";
     }
     o << "    }\n";
-    o << "    rx_lds_barrier();\n";
-    // (iii) one output plane of the second step
-    o << "    const int iz = ib - " << dB << ";\n";
-    o << "    if (iz >= 0 && live) {\n";
-    o << "      const int z = z0 + iz;\n";
-    for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((ib + " << (2 * RB - k) << ") % " << RB << ") * " << BPLANE << ";\n";
-    o << "      const " << it << " i0 = z;\n";
-    o << "      const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
-    for (auto& dv : ec.direct_vecs) o << "      const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uq" << dv.first << "[" << h << "];\n";
-    o << "      " << vt << " res;\n";
-    o << "#pragma unroll\n      for (int l = 0; l < " << vec << "; ++l) {\n";
-    o << "        const " << it << " i2 = i2b + l;\n";
-    o << bodyC;
-    o << "        res.v[l] = " << ec.store_value(rn.ty.dt, valC) << ";\n      }\n";
-    o << "      " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
-    o << "    }\n";
     // the streamed inputs move one plane on
-    o << "    if (ib >= 0) {\n";
     for (int sl : stream_slots) {
-      for (int64_t k = h; k >= 1; --k) o << "      uq" << sl << "[" << k << "] = uq" << sl << "[" << k - 1 << "];\n";
-      o << "      uq" << sl << "[0] = un" << sl << ";\n";
+      for (int64_t k = QL - 1; k >= 1; --k) o << "    uq" << sl << "[" << k << "] = uq" << sl << "[" << k - 1 << "];\n";
+      o << "    uq" << sl << "[0] = un" << sl << ";\n";
       if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
-        o << "#pragma unroll\n      for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << "[q];\n";
+        o << "#pragma unroll\n    for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << "[q];\n";
     }
-    o << "    }\n";
+    o << "    rx_lds_barrier();\n";
     o << "  }\n}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;
