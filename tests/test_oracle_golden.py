@@ -349,3 +349,22 @@ def test_while_form_of_the_stencil_equals_the_unrolled_form(embed):
     a = I.run_text(P.stencil(6, 5, 4, steps=4, embed=embed, loop="while"), args)[0].a
     b = I.run_text(P.stencil(6, 5, 4, steps=4, embed=embed), args)[0].a
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("embed", ["pad", "dus"])
+def test_c_restatement_of_the_stencil_matches_the_interpreter(embed):
+    """oracle/stencil_cpu.c (the CPU baseline of the benchmark) against the numpy interpreter:
+    same bits, on a grid with odd extents and for several steps."""
+    from oracle import build_c
+    lib = build_c.load() if os.path.exists(build_c.SO) else None
+    if lib is None:
+        build_c.build()
+        lib = build_c.load()
+    nx, ny, nz = 13, 9, 7
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(2)
+    a = [rng.uniform(-1, 1, full) for _ in range(4)]
+    ref = I.run_text(P.stencil(nx, ny, nz, steps=3, embed=embed), [I.Tensor(x, "f64") for x in a])[0].a
+    got = build_c.stencil_steps(lib, *a, nx, ny, nz, 3, embed=embed)
+    assert np.array_equal(got, ref)
+    assert lib.rx_oracle_threads() >= 1
