@@ -147,6 +147,49 @@ def test_two_step_kernels_with_one_sided_neighbourhoods(rx, client, monkeypatch,
     assert np.array_equal(got[0].a, oracle_run(text, args)[0].a)
 
 
+@pytest.mark.parametrize("elt", ["f64", "f32"])
+def test_stencil_with_two_fields_read_at_offsets(rx, client, monkeypatch, elt):
+    """Both inputs are read at several offsets: both get an LDS halo tile in the one-step kernel,
+    and steps are not paired (a pair needs a single field carried from step to step)."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    nx, ny, nz, H = 72, 20, 6, 3
+    full, inner = [nz + 2 * H, ny + 2 * H, nx + 2 * H], [nz, ny, nx]
+    tf = "tensor<%dx%dx%dx%s>" % (*full, elt)
+    ti = "tensor<%dx%dx%dx%s>" % (*inner, elt)
+    lines, k = ["    %%z = stablehlo.constant dense<0.000000e+00> : tensor<%s>" % elt], [0]
+
+    def sl(x, d):
+        k[0] += 1
+        r, st = "%%s%d" % k[0], [H + d[0], H + d[1], H + d[2]]
+        lines.append("    %s = stablehlo.slice %s [%s] : (%s) -> %s" % (
+            r, x, ", ".join("%d:%d" % (a, a + n) for a, n in zip(st, inner)), tf, ti))
+        return r
+
+    c = "%arg0"
+    for step in range(2):
+        terms = [sl(c, d) for d in [(0, 0, -1), (0, 0, 1), (0, 1, 0), (-1, 0, 0)]] + \
+                [sl("%arg1", d) for d in [(1, 0, 0), (-1, 0, 0), (0, -1, 0), (0, 0, 2)]]
+        acc = terms[0]
+        for t in terms[1:]:
+            k[0] += 1
+            r = "%%a%d" % k[0]
+            lines.append("    %s = stablehlo.multiply %s, %s : %s" % (r, acc, t, ti) if step and t is terms[4] else
+                         "    %s = stablehlo.add %s, %s : %s" % (r, acc, t, ti))
+            acc = r
+        k[0] += 1
+        c = "%%p%d" % k[0]
+        lines.append("    %s = stablehlo.pad %s, %%z, low = [3, 3, 3], high = [3, 3, 3], interior = [0, 0, 0] : (%s, tensor<%s>) -> %s"
+                     % (c, acc, ti, elt, tf))
+    text = ("module @reactant_two_fields {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n%s\n    return %s : %s\n  }\n}\n"
+            % (tf, tf, tf, "\n".join(lines), c, tf))
+    rng = np.random.default_rng(4)
+    np_t = np.float64 if elt == "f64" else np.float32
+    args = [I.Tensor(rng.uniform(-1, 1, full).astype(np_t), elt) for _ in range(2)]
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["map_stencil_lds", "map_stencil_lds"]
+    assert np.array_equal(got[0].a, oracle_run(text, args)[0].a)
+
+
 @pytest.mark.parametrize("planes,tile", [("3", "8,64"), ("5", "16,32"), ("100", "4,128"), ("7", "32,16")])
 def test_stencil_marching_chunks_and_tiles(rx, client, monkeypatch, planes, tile):
     """The marching kernel with chunks shorter and longer than the grid and other plane tiles."""
