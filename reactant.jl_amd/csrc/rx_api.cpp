@@ -214,9 +214,6 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_STENCIL_MARCH2")) o.stencil_march2 = atoi(e) != 0;
   if (const char* e = getenv("RX_MARCH2_PLANES")) o.march2_planes = atoi(e) > 0 ? atoi(e) : o.march2_planes;
   if (const char* e = getenv("RX_MARCH2_TILE")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2) { o.march2_tile[0] = v[0]; o.march2_tile[1] = v[1]; } }
-  if (const char* e = getenv("RX_STENCIL_MARCH")) o.stencil_march = atoi(e) != 0;
-  if (const char* e = getenv("RX_MARCH_DEPTH")) o.march_depth = atoi(e) >= 1 && atoi(e) <= 8 ? atoi(e) : o.march_depth;
-  if (const char* e = getenv("RX_MARCH_PLANES")) o.march_planes = atoi(e) > 0 ? atoi(e) : o.march_planes;
   if (const char* e = getenv("RX_LDS_TILE")) { int v[3]; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) == 3) { o.lds_tile[0] = v[0]; o.lds_tile[1] = v[1]; o.lds_tile[2] = v[2]; } }
   if (const char* e = getenv("RX_LDS_TILE2")) { int v[3]; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) == 3) { o.lds_tile2[0] = v[0]; o.lds_tile2[1] = v[1]; o.lds_tile2[2] = v[2]; } }
   if (const char* e = getenv("RX_SLAB_YTILES")) o.slab_ytiles = atoi(e);

@@ -464,143 +464,6 @@ struct Planner {
     return out;
   }
 
-  // ------------------------------------------------------------------ stencil maps, marching
-  // Same idea as the tile kernel below, but a workgroup owns a TY x TX column and walks along
-  // the slowest dimension: the staged input lives in a ring of planes in LDS, each plane
-  // (tile + halo) is loaded from global memory exactly once per workgroup, one plane ahead of
-  // its first use, and the planes above and below an output come from the ring.
-  bool emit_map_march(int root, int staged, const int64_t (&hlo)[3], const int64_t (&hhi)[3]) {
-    const Node& rn = g.nodes[root];
-    const auto& dims = rn.ty.dims;
-    const int vec = pick_vec(rn.ty);
-    const int64_t Z = dims[0], Y = dims[1], X = dims[2];
-    const int TY = opt.lds_tile[1], TX = opt.lds_tile[2];
-    if (TX % vec || (TX / vec) * TY != kBlock) return false;
-    const int TXV = TX / vec;
-    const int R = 4;                       // ring slots (power of two)
-    if (hlo[0] + hhi[0] + 2 > R) return false;
-    const int64_t hxl = (hlo[2] + vec - 1) / vec * vec, hxh = (hhi[2] + vec - 1) / vec * vec;
-    const int64_t PY = TY + hlo[1] + hhi[1], LX = TX + hxl + hxh, LXV = LX / vec;
-    const int64_t PLANE = PY * LX, PV = PY * LXV;
-    const int64_t NLD = (PV + kBlock - 1) / kBlock;
-    const int es = info(g.nodes[staged].ty.dt).size;
-    if (R * PLANE * es > 64 * 1024) return false;
-    const int64_t TZB = std::min<int64_t>(opt.march_planes, Z);
-
-    Emitter em(g, [&](int x) { return x != root && mat[x]; });
-    em.excess_precision = opt.excess_precision;
-    em.idx64 = needs64(cone_nodes(root));
-    em.set_root(dims, {"i0", "i1", "i2"}, true);
-    em.vec = vec;
-    em.allow_shifted = false;
-    em.direct_expr = vec_name;
-    em.indent = 10;
-    em.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
-      if (em.inputs[slot] != staged) return false;
-      std::ostringstream e;
-      e << "lds[(((i0 + " << off[0] << ") & " << (R - 1) << ") * " << PY << " + (ly + " << (off[1] + hlo[1]) << ")) * " << LX << " + lxe + l + "
-        << (hxl + off[2]) << "]";
-      *expr = e.str();
-      return true;
-    };
-    std::string val = em.emit(root, root_index(dims));
-    std::string body = em.take_code();
-    const std::string it = em.idx_t();
-    const int sslot = em.slot_of(staged);
-    const std::string sst = info(g.nodes[staged].ty.dt).stype;
-    const std::string svt = "rx_vec<" + sst + ", " + std::to_string(vec) + ">";
-    const std::string kname = "@K@_stencil";
-    const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + TZB - 1) / TZB;
-    const int64_t nblocks = ntx * nty * ntz;
-    std::ostringstream o;
-    o << "// stencil map, marching along dim 0 with a ring of " << R << " LDS planes (" << TY << "x" << TX << " outputs per plane, " << TZB
-      << " planes per workgroup): " << describe(root) << " -> " << rn.ty.str() << "\n";
-    o << signature(kname, em.inputs, {{info(rn.ty.dt).stype, "out0"}}) << " {\n";
-    o << "  __shared__ __attribute__((aligned(16))) " << sst << " lds[" << R * PLANE << "];\n";
-    o << "  const unsigned tile = rx_xcd_remap(blockIdx.x, " << nblocks << "u);\n";
-    o << "  const int x0 = (int)(tile % " << ntx << "u) * " << TX << ";\n";
-    o << "  const int y0 = (int)((tile / " << ntx << "u) % " << nty << "u) * " << TY << ";\n";
-    o << "  const int z0 = (int)(tile / " << ntx * nty << "u) * " << TZB << ";\n";
-    o << "  const int zend = z0 + " << TZB << " < " << Z << " ? z0 + " << TZB << " : " << Z << ";\n";
-    // per-thread addresses of the plane loads (the same for every plane, only the plane index moves)
-    o << "  " << it << " poff[" << NLD << "];\n";
-    o << "#pragma unroll\n  for (int q = 0; q < " << NLD << "; ++q) {\n";
-    o << "    const int v = threadIdx.x + q * " << kBlock << ";\n";
-    o << "    const int xv = v % " << LXV << ", yy = (v / " << LXV << ") % " << PY << ";\n";
-    o << "    const " << it << " gy = rx_clamp_idx<" << it << ">(y0 - " << hlo[1] << " + yy, " << Y - 1 << ");\n";
-    o << "    const " << it << " gx = rx_clamp_idx<" << it << ">(x0 - " << hxl << " + xv * " << vec << ", " << X - vec << ");\n";
-    o << "    poff[q] = gy * " << X << " + gx;\n  }\n";
-    // halo cells outside the array are clamped to valid addresses; their values are never used
-    o << "  auto load_plane = [&](int p, " << svt << " (&t)[" << NLD << "]) {\n";
-    o << "    const " << it << " gz = rx_clamp_idx<" << it << ">(p, " << Z - 1 << ");\n";
-    o << "#pragma unroll\n    for (int q = 0; q < " << NLD << "; ++q) t[q] = rx_load<" << svt << ">(in" << sslot << " + gz * " << Y * X << (em.idx64 ? "LL" : "")
-      << " + poff[q]);\n  };\n";
-    o << "  auto store_plane = [&](int p, const " << svt << " (&t)[" << NLD << "]) {\n";
-    o << "    " << sst << "* dst = lds + (p & " << (R - 1) << ") * " << PLANE << ";\n";
-    o << "#pragma unroll\n    for (int q = 0; q < " << NLD << "; ++q) {\n      const int v = threadIdx.x + q * " << kBlock << ";\n";
-    o << "      if (v < " << PV << ") rx_store(dst + v * " << vec << ", t[q]);\n    }\n  };\n";
-    const int D = opt.march_depth;
-    const std::string ldf = opt.nt_loads ? "rx_load_nt" : "rx_load";
-    o << "  " << svt << " pre[" << D << "][" << NLD << "];\n";
-    // planes needed by the first output plane go straight to LDS
-    for (int64_t p = -hlo[0]; p <= hhi[0]; ++p) o << "  load_plane(z0 + " << p << ", pre[0]); store_plane(z0 + " << p << ", pre[0]);\n";
-    // Register pipeline: at step z (slot j = (z - z0) % D) the plane z+hi+D is requested into
-    // slot j and the plane z+hi+1, requested D steps earlier into slot (j+1) % D, is written to
-    // the ring.  The planes that the first D steps write are requested here.
-    for (int k = 1; k <= D; ++k) o << "  load_plane(z0 + " << hhi[0] + k << ", pre[" << k % D << "]);\n";
-    o << "  const int ly = threadIdx.x / " << TXV << ", lxe = (threadIdx.x % " << TXV << ") * " << vec << ";\n";
-    o << "  const " << it << " i1 = y0 + ly, i2b = x0 + lxe;\n";
-    o << "  const bool live = i1 < " << Y << " && i2b < " << X << ";\n";
-    o << "  const " << it << " colc = rx_clamp_idx<" << it << ">(i1, " << Y - 1 << ") * " << X << " + rx_clamp_idx<" << it << ">(i2b, " << X - vec << ");\n";
-    // inputs read only at the output position: plane z is requested D steps before step z
-    for (auto& sd : em.direct_vecs) {
-      const int slot = sd.first;
-      const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">";
-      o << "  " << vt << " nx" << slot << "[" << D << "];\n";
-      o << "#pragma unroll\n  for (int k = 0; k < " << D << "; ++k) nx" << slot << "[k] = " << ldf << "<" << vt << ">(in" << slot << " + rx_clamp_idx<" << it
-        << ">(z0 + k, " << Z - 1 << ") * " << Y * X << (em.idx64 ? "LL" : "") << " + colc);\n";
-    }
-    o << "  rx_lds_barrier();\n";
-    o << "  for (int zb = z0; zb < zend; zb += " << D << ") {\n";
-    o << "#pragma unroll\n    for (int j = 0; j < " << D << "; ++j) {\n";
-    o << "      const int z = zb + j;\n";
-    o << "      if (z >= zend) break;\n";
-    for (auto& sd : em.direct_vecs) {
-      const int slot = sd.first;
-      const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">";
-      o << "      const " << vt << " " << vec_name(slot, 0) << " = nx" << slot << "[j];\n";
-      o << "      nx" << slot << "[j] = " << ldf << "<" << vt << ">(in" << slot << " + rx_clamp_idx<" << it << ">(z + " << D << ", " << Z - 1 << ") * " << Y * X
-        << (em.idx64 ? "LL" : "") << " + colc);\n";
-    }
-    o << "      if (live) {\n";
-    o << "        const " << it << " i0 = z;\n";
-    o << "        const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << (em.idx64 ? "LL" : "") << " + i2b;\n";
-    const std::string ost = info(rn.ty.dt).stype;
-    o << "        rx_vec<" << ost << ", " << vec << "> res;\n";
-    o << "#pragma unroll\n        for (int l = 0; l < " << vec << "; ++l) {\n";
-    o << "          const " << it << " i2 = i2b + l;\n";
-    o << body;
-    o << "          res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n        }\n";
-    o << "        " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
-    o << "      }\n";
-    o << "      store_plane(z + " << hhi[0] + 1 << ", pre[(j + 1) % " << D << "]);\n";
-    o << "      load_plane(z + " << hhi[0] + 1 + D << ", pre[(j + 1) % " << D << "]);\n";
-    o << "      rx_lds_barrier();\n";
-    o << "    }\n  }\n}\n\n";
-    const std::string kb_final = finalize(o.str());
-    Launch L;
-    L.kernel = named(kname, kb_final);
-    L.kind = "map_stencil_lds";
-    L.grid[0] = (unsigned)nblocks;
-    L.block[0] = kBlock;
-    for (int i : em.inputs) L.args.push_back(buffer_for(i));
-    L.args.push_back(buffer_for(root));
-    L.algo_bytes = algo_bytes(em.inputs, {root});
-    L.desc = describe(root);
-    plan.launches.push_back(L);
-    return true;
-  }
-
   // Tile order of the stencil kernels.  Workgroups are dealt round-robin to the 8 XCDs, each with
   // its own L2.  The y-tiles are cut into slabs of `sy` tiles; XCD k owns slabs k, k+8, ... and
   // walks each of them layer by layer in z, so the planes that consecutive layers share (and the
@@ -707,10 +570,6 @@ struct Planner {
         lds_only.erase(prev);
         emit_map(prev);
       }
-    }
-    if (opt.stencil_march && staged.size() == 1) {
-      const Halo& h = halos[staged[0]];
-      if (emit_map_march(root, staged[0], h.lo, h.hi)) return true;
     }
     int TZ = opt.lds_tile[0], TY = opt.lds_tile[1], TX = opt.lds_tile[2];
     if (TX % vec || (TX / vec) * TY != kBlock) return false;

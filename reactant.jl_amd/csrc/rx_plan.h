@@ -58,9 +58,6 @@ struct PlanOptions {
   bool stencil_march2 = true;      // two-step kernel marching along the slowest dimension instead of 3-D tiles
   int march2_tile[2] = {8, 64};    // its outputs per plane (rows, columns)
   int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
-  bool stencil_march = false;   // stencil maps: a workgroup marches along the slowest dimension with a ring of planes in LDS
-  int march_depth = 3;          // planes of global loads kept in flight (in registers) ahead of their use
-  int march_planes = 32;        // planes produced per workgroup when marching
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once
