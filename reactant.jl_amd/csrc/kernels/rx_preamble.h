@@ -174,6 +174,13 @@ RX_DEV float rx_tanh_fast(float x) {
   const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
   return __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(e + 1.0f), 1.0f);
 }
+// x / y for a divisor that is the same for every element.  1/y in double is loop-invariant; the
+// double product is within 2^-52 of the exact quotient, and the quotient of two 24-bit numbers is
+// never closer than about 2^-49 (relative) to a midpoint between two floats, so rounding the
+// product to float gives the correctly rounded quotient.  Zero, infinite and NaN operands
+// behave as in the division (1/0 = inf, 0 * inf = NaN, ...); double has the range for
+// subnormal divisors.
+RX_DEV float rx_div_uniform(float x, float y) { return (float)((double)x * (1.0 / (double)y)); }
 RX_DEV float rx_logistic(float x) { return 1.0f / (1.0f + expf(-x)); }
 RX_DEV double rx_logistic(double x) { return 1.0 / (1.0 + exp(-x)); }
 RX_DEV float rx_rsqrt(float x) { return 1.0f / sqrtf(x); }

@@ -216,6 +216,25 @@ std::string Emitter::emit_load(int node, const Index& ix) {
 
 static std::string fn(const std::string& base, bool dbl) { return dbl ? base : base + "f"; }
 
+// The same value at every index: a rank-0 value, or broadcasts / elementwise ops of such values.
+bool Emitter::is_uniform(int node, int depth) const {
+  const Node& n = g_.nodes[node];
+  if (n.ty.rank() == 0) return true;
+  if (depth > 8) return false;
+  switch (n.k) {
+    case OpK::Constant: return n.splat;
+    case OpK::BroadcastInDim:
+    case OpK::Reshape:
+    case OpK::Convert:
+    case OpK::Unary:
+      return is_uniform(n.in[0], depth + 1);
+    case OpK::Binary:
+      return is_uniform(n.in[0], depth + 1) && is_uniform(n.in[1], depth + 1);
+    default:
+      return false;
+  }
+}
+
 std::string Emitter::emit_op(const Node& n, const Index& ix) {
   const DT dt = n.ty.dt;
   const std::string CT = info(dt).ctype;
@@ -294,7 +313,13 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (op == "add") return def("(" + a + " + " + b + ")");
         if (op == "subtract") return def("(" + a + " - " + b + ")");
         if (op == "multiply") return def("(" + a + " * " + b + ")");
-        if (op == "divide") return def("(" + a + " / " + b + ")");
+        if (op == "divide") {
+          // a divisor that is one value for the whole tensor (a broadcast scalar, e.g. a
+          // quantization scale): its reciprocal in double is loop-invariant, and the product in
+          // double rounds to the same float as the division (see rx_div_uniform)
+          if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
+          return def("(" + a + " / " + b + ")");
+        }
         if (op == "maximum") return def("rx_max(" + a + ", " + b + ")");
         if (op == "minimum") return def("rx_min(" + a + ", " + b + ")");
         if (op == "power") return def(fn("pow", dbl) + "(" + a + ", " + b + ")");

@@ -96,6 +96,7 @@ class Emitter {
   std::vector<std::string> root_vars_;
   bool allow_direct_ = false;
 
+  bool is_uniform(int node, int depth = 0) const;
   std::string emit_load(int node, const Index& ix);
   std::string emit_op(const Node& n, const Index& ix);
   bool lookup(const std::string& key, std::string* out) const;

@@ -316,3 +316,30 @@ def test_while_generic_form_returns_counter_and_value(rx, client):
     got, ref = both(rx, client, W.GENERIC, [I.Tensor(v, "f32")])
     assert int(got[0].a) == 3 and np.array_equal(got[1].a, 8 * v)
     assert np.array_equal(got[1].a, ref[1].a)
+
+
+# ---- division by a broadcast scalar ------------------------------------------------------------
+@pytest.mark.parametrize("divisor", [3.0, 0.1, 448.0, 1e-40, 3.4e38, 0.0, -7.25, float("inf")])
+def test_divide_by_a_broadcast_scalar_is_correctly_rounded(rx, client, divisor):
+    """x / s with s one value for the whole tensor is evaluated as a product with the double
+    reciprocal; it must round exactly like the IEEE division (bit-for-bit against numpy),
+    including subnormal and huge divisors, zeros, infinities and quotients next to a tie."""
+    n = 1 << 16
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 2 ** 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32).copy()
+    x[: n // 2] = rng.normal(size=n // 2).astype(np.float32) * np.float32(100)
+    # numerators that put the quotient half an ulp away from a float: (2k+1) * s in float
+    s32 = np.float32(divisor)
+    if np.isfinite(s32) and s32 != 0:
+        k = (rng.integers(2 ** 23, 2 ** 24, 4096) * 2 + 1).astype(np.float64)
+        with np.errstate(all="ignore"):
+            x[-4096:] = (k * np.float64(s32)).astype(np.float32)
+    text = mod([_tt([n], "f32"), "tensor<f32>"], _tt([n], "f32"),
+               "    %0 = stablehlo.broadcast_in_dim %arg1, dims = [] : (tensor<f32>) -> tensor<{n}xf32>\n".replace("{n}", str(n)) +
+               "    %1 = stablehlo.divide %arg0, %0 : tensor<{n}xf32>\n    return %1 : tensor<{n}xf32>\n".replace("{n}", str(n)))
+    got, _ = gpu_run(rx, client, text, [I.Tensor(x, "f32"), I.Tensor(s32, "f32")])
+    with np.errstate(all="ignore"):
+        want = x / s32
+    same = got[0].a.view(np.uint32) == want.view(np.uint32)
+    both_nan = np.isnan(got[0].a) & np.isnan(want)
+    assert (same | both_nan).all(), (x[~(same | both_nan)][:5], got[0].a[~(same | both_nan)][:5], want[~(same | both_nan)][:5])
