@@ -3,7 +3,7 @@
  *
  * Every entry point below keeps the name, argument order and ownership rules of
  * the reference export it replaces (deps/ReactantExtra/API.cpp, line cited per
- * function), so the Julia side (src/xla/PJRT/*.jl) can route a call here by
+ * function), so the Julia side (the files under src/xla/PJRT) can route a call here by
  * swapping the library it `@ccall`s.  Handles are opaque pointers.  The only
  * signature that differs is compilation: the reference passes an in-memory
  * MlirModule; this library takes the module as MLIR text (`string(mod)`).

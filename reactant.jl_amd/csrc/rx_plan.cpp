@@ -949,13 +949,12 @@ struct Planner {
     const int64_t BY = TY + hR.lo[1] + hR.hi[1], BX = TX + bxl + bxh, BXV = BX / vec;
     const int64_t axl = up(hP.lo[2]), axh = up(hP.hi[2]);
     const int64_t AY = BY + hP.lo[1] + hP.hi[1], AX = BX + axl + axh, AXV = AX / vec;
-    const int64_t APLANE = AY * AX, BPLANE = BY * BX, AV = AY * AXV, BV = BY * BXV;
+    const int64_t APLANE = AY * AX, BPLANE = BY * BX, AV = AY * AXV;
     const int64_t RA = hP.lo[0] + hP.hi[0] + 2, RB = hR.lo[0] + hR.hi[0] + 2;   // a stencil's reach plus the plane being written
     const int es = info(rn.ty.dt).size;
     if ((RA * APLANE + RB * BPLANE) * es > 64 * 1024) return false;
-    const int64_t NLA = (AV + NB - 1) / NB, NLB = (BV + NB - 1) / NB;
+    const int64_t NLA = (AV + NB - 1) / NB;   // 16-byte loads per thread for one source plane
     if (NLA > 8) return false;
-    (void)NLB;
     const std::string st = info(rn.ty.dt).stype;
     const std::string vt = "rx_vec<" + st + ", " + std::to_string(vec) + ">";
     const int64_t dA = hP.lo[0] + hP.hi[0], dB = hR.lo[0] + hR.hi[0];
@@ -1056,7 +1055,6 @@ struct Planner {
     // before the iteration began, and puts the next source plane into the ring -- three pieces of
     // work that touch disjoint ring slots, so one barrier per iteration is enough.  The rings hold
     // one plane more than a stencil's reach for that.
-    const int64_t RA1 = dA + 2, RB1 = dB + 2;
     o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", zb0 = z0 - " << hR.lo[0] << ";\n";
     o << "  const int nB = zend - z0 + " << dB << ", nit = nB + 1;\n";
     o << "  auto plane = [&](int p) { return (" << it << ")rx_clamp_idx<int>(p, " << Z - 1 << ") * " << Y * X << LL << "; };\n";
@@ -1114,7 +1112,7 @@ struct Planner {
     o << "    }\n";
     // the source plane requested last iteration goes to the ring; request the one after it
     o << "    if (n + 1 < nB) {\n";
-    o << "      " << st << "* dst = ldsA + ((n + " << dA + 1 << ") % " << RA1 << ") * " << APLANE << ";\n";
+    o << "      " << st << "* dst = ldsA + ((n + " << dA + 1 << ") % " << RA << ") * " << APLANE << ";\n";
     o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
     o << "        const int v = threadIdx.x + q * " << NB << ";\n";
     o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[q]);\n      }\n";
@@ -1126,7 +1124,7 @@ struct Planner {
     o << "    const int iz = n - " << dB + 1 << ";\n";
     o << "    if (iz >= 0 && live) {\n";
     o << "      const int z = z0 + iz;\n";
-    for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((n + " << (2 * RB1 - 1 - k) << ") % " << RB1 << ") * " << BPLANE << ";\n";
+    for (int64_t k = 0; k <= dB; ++k) o << "      const int sb" << k << " = ((n + " << (2 * RB - 1 - k) << ") % " << RB << ") * " << BPLANE << ";\n";
     o << "      const " << it << " i0 = z;\n";
     o << "      const " << it << " lin0 = (i0 * " << Y << " + i1) * " << X << LL << " + i2b;\n";
     for (auto& dv : ec.direct_vecs) o << "      const " << vts_of(ec, dv.first) << " " << vec_name(dv.first, 0) << " = uq" << dv.first << "[" << h + 1 << "];\n";
@@ -1140,8 +1138,8 @@ struct Planner {
     // one plane of the first step
     o << "    if (n < nB) {\n";
     o << "      const int b = zb0 + n;\n";
-    for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((n + " << (dA - k) << ") % " << RA1 << ") * " << APLANE << ";\n";
-    o << "      " << st << "* dstb = ldsB + (n % " << RB1 << ") * " << BPLANE << ";\n";
+    for (int64_t k = 0; k <= dA; ++k) o << "      const int sa" << k << " = ((n + " << (dA - k) << ") % " << RA << ") * " << APLANE << ";\n";
+    o << "      " << st << "* dstb = ldsB + (n % " << RB << ") * " << BPLANE << ";\n";
     o << "      const " << it << " j0 = rx_clamp_idx<" << it << ">(b, " << Z - 1 << ");\n";
     emit_B("      ", "ly + " + std::to_string(hR.lo[1]), "lxe + " + std::to_string(bxl), "i1", "i2b",
            [&](int sl) { return "uq" + std::to_string(sl) + "[0]"; }, "by * " + std::to_string(BX) + " + bxe");
