@@ -1,0 +1,109 @@
+"""The five benchmark configs at their full sizes on the GPU.
+
+The numpy interpreter is too slow for these shapes, so each config is checked the way its
+structure allows: the stencil bit for bit against the oracle's C restatement (which the CPU
+tests pin to the interpreter); the reduction and the f32 GEMM against float64 numpy; the MLP and
+the FP8 linear layer, whose rows are independent, on a sample of rows recomputed by the
+interpreter with the same weights (plus the row invariants of softmax and RMSNorm on every row)."""
+import numpy as np
+import pytest
+
+from _harness import gpu_run, oracle_run, max_rel_to_scale
+from _loader import load_programs
+from oracle import stablehlo_interp as I
+from oracle import lowfloat as lf
+
+pytestmark = pytest.mark.gpu
+P = load_programs()
+
+
+def _upload(rx, client, raw, dt):
+    return rx.Buffer.from_host(client, raw, dt)
+
+
+def _download(buf):
+    return buf.synced_buffer().to_host()
+
+
+def test_sinsum_add_2_pow_26(rx, client):
+    n = 1 << 26
+    x = np.random.default_rng(0).uniform(-np.pi, np.pi, n).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-np.pi, np.pi, n).astype(np.float32)
+    exe = rx.xla_compile(client, P.sinsum_add(n))
+    out = exe.execute_sharded([_upload(rx, client, x, "f32"), _upload(rx, client, y, "f32")])
+    got = float(_download(out[0]))
+    terms = np.sin(x.astype(np.float64)) + y.astype(np.float64)
+    exact, scale = float(terms.sum()), float(np.abs(terms).sum())
+    # fp32 reduction: 1e-5 * sqrt(n) relative to the mean magnitude of the summands
+    assert abs(got - exact) <= 1e-5 * np.sqrt(n) * scale / n
+
+
+def test_stencil_512x512x256_ten_steps_bit_exact(rx, client):
+    from oracle import build_c
+    lib = build_c.load()
+    nx, ny, nz, H = 512, 512, 256, 3
+    full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
+    c = np.zeros(full)
+    c[H:-H, H:-H, H:-H] = np.random.default_rng(0).random((nz, ny, nx))
+    u = 2.0 * np.random.default_rng(1).random(full) - 1.0
+    v = np.ascontiguousarray(u[::-1])
+    w = 0.5 * (u - v)
+    exe = rx.xla_compile(client, P.stencil(nx, ny, nz, steps=10))
+    assert [l["kind"] for l in exe.launches()] == ["map_stencil_lds2"] * 5
+    out = exe.execute_sharded([_upload(rx, client, a, "f64") for a in (c, u, v, w)])
+    got = _download(out[0])
+    want = build_c.stencil_steps(lib, c, u, v, w, nx, ny, nz, 10)
+    assert got.shape == want.shape and np.array_equal(got, want)
+    assert not np.any(got[:H]) and not np.any(got[:, :H]) and not np.any(got[:, :, -H:])   # halos stay zero
+
+
+def test_gemm_4096_f32_alpha_beta(rx, client):
+    n = 4096
+    A, B, C = [np.random.default_rng(s).normal(size=(n, n)).astype(np.float32) for s in (0, 1, 2)]
+    exe = rx.xla_compile(client, P.gemm(n, n, n))
+    out = exe.execute_sharded([_upload(rx, client, a, "f32") for a in (A, B, C)])
+    got = _download(out[0])
+    # buffers are the Julia arrays with dims reversed: C_raw = alpha * B_raw @ A_raw + beta * C_raw
+    want = 1.5 * (B.astype(np.float64) @ A.astype(np.float64)) + 1.2 * C.astype(np.float64)
+    assert max_rel_to_scale(got, want) <= 1e-5
+
+
+def _bf16(a):
+    return lf.f32_to_bf16_bits(np.asarray(a, dtype=np.float32))
+
+
+def test_mlp_8192_rows_sampled(rx, client):
+    batch, widths, rows = 8192, (1024, 4096, 4096, 1024), 48
+    rng = np.random.default_rng(0)
+    raw = [_bf16(rng.normal(size=(batch, widths[0])))]
+    for l in range(3):
+        lim = np.sqrt(6.0 / (widths[l] + widths[l + 1]))
+        raw.append(_bf16(np.random.default_rng(1 + l).uniform(-lim, lim, size=(widths[l], widths[l + 1]))))
+        raw.append(_bf16(np.random.default_rng(4 + l).normal(size=(widths[l + 1],)) * 0.01))
+    exe = rx.xla_compile(client, P.mlp(batch, widths))
+    out = exe.execute_sharded([_upload(rx, client, a, "bf16") for a in raw])
+    got = lf.bf16_bits_to_f32(_download(out[0])).reshape(batch, widths[-1])
+    assert np.allclose(got.sum(axis=1), 1.0, atol=2e-2)                    # every softmax row sums to one
+    pick = np.linspace(0, batch - 1, rows).astype(int)                     # rows are independent: recompute a sample
+    args = [I.Tensor.from_bytes(raw[0][pick].tobytes(), "bf16", (rows, widths[0]))]
+    args += [I.Tensor.from_bytes(a.tobytes(), "bf16", a.shape) for a in raw[1:]]
+    ref = oracle_run(P.mlp(rows, widths), args, hifi=True, excess=True)
+    assert max_rel_to_scale(got[pick], ref[0].a) <= 2e-2
+
+
+def test_fp8_linear_8192_rows_sampled(rx, client):
+    n, rows = 8192, 32
+    act = np.random.default_rng(0).normal(size=(n, n)).astype(np.float32)
+    act[0, 0] = 9.0                                                        # the per-tensor absmax sits in a sampled row
+    a_raw = _bf16(act)
+    codes = np.random.default_rng(1).integers(0, 256, size=(n, n), dtype=np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x38                                   # no NaN codes among the weights
+    sw = np.float32(0.0123)
+    exe = rx.xla_compile(client, P.fp8_linear(n, n, n))
+    out = exe.execute_sharded([_upload(rx, client, a_raw, "bf16"), _upload(rx, client, codes, "f8E4M3FN"), _upload(rx, client, sw, "f32")])
+    got = lf.bf16_bits_to_f32(_download(out[0])).reshape(n, n)
+    assert np.allclose((got.astype(np.float64) ** 2).mean(axis=1), 1.0, atol=2e-2)   # RMSNorm: unit mean square per row
+    args = [I.Tensor.from_bytes(a_raw[:rows].tobytes(), "bf16", (rows, n)),
+            I.Tensor.from_bytes(codes.tobytes(), "f8E4M3FN", (n, n)), I.Tensor(sw, "f32")]
+    ref = oracle_run(P.fp8_linear(rows, n, n), args, hifi=True, excess=True)
+    assert max_rel_to_scale(got[:rows], ref[0].a) <= 1e-2
