@@ -268,6 +268,8 @@ class Client:
 
     def close(self):
         if self.handle:
+            for key in [k for k in _THUNKS if k[0] == id(self)]:   # executables of this client go with it
+                del _THUNKS[key]
             lib.FreeClient(self.handle)
             self.handle = None
 
