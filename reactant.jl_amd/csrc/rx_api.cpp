@@ -315,10 +315,15 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       args[i]->mem.reset();
     }
   }
-  std::vector<hipEvent_t> evs;
+  // events of a timed execution; destroyed on every exit path unless handed to the executable
+  struct EventList {
+    std::vector<hipEvent_t> v;
+    ~EventList() { for (auto e : v) if (e) (void)hipEventDestroy(e); }
+  } evlist;
+  std::vector<hipEvent_t>& evs = evlist.v;
   const bool timed = launch_ms || profile_async;
   if (timed) {
-    evs.resize(P.launches.size() + 1);
+    evs.assign(P.launches.size() + 1, nullptr);
     for (auto& e : evs) HIP_CHECK(hipEventCreate(&e));
     HIP_CHECK(hipEventRecord(evs[0], dev->stream));
   }
@@ -374,9 +379,9 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
   if (launch_ms) {
     HIP_CHECK(hipEventSynchronize(evs.back()));
     for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[li], evs[li + 1]));
-    for (auto& e : evs) (void)hipEventDestroy(e);
   } else if (profile_async) {
     ex->pending_events.push_back(std::move(evs));   // read later by RxExecutableTakeTimings
+    evs.clear();
   }
 }
 
