@@ -667,8 +667,11 @@ RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, siz
       auto& B = ex->plan.buffers[b];
       if (B.kind != rx::BufferDesc::Const) continue;
       ex->consts[b] = std::make_shared<Allocation>(d, std::max<size_t>(B.data.size(), 1));
-      if (!B.data.empty()) HIP_CHECK(hipMemcpy(ex->consts[b]->ptr, B.data.data(), B.data.size(), hipMemcpyHostToDevice));
+      // on the device's stream: the block may have been recycled from a buffer whose last kernel
+      // is still queued there, and a copy on the null stream would not wait for it
+      if (!B.data.empty()) HIP_CHECK(hipMemcpyAsync(ex->consts[b]->ptr, B.data.data(), B.data.size(), hipMemcpyHostToDevice, d->stream));
     }
+    HIP_CHECK(hipStreamSynchronize(d->stream));   // pageable host data: wait before the plan may move
     RxExecutable* raw = ex.release();
     reg_add(raw);
     return raw;
