@@ -172,7 +172,28 @@ std::string Emitter::emit_load(int node, const Index& ix) {
       rec.off.push_back(ix[d].off);
     }
   }
+  bool permuted = false;
+  if (!rec.affine && dims.size() == root_vars_.size() && dims.size() >= 2) {
+    std::vector<char> used(dims.size(), 0);
+    permuted = true;
+    for (size_t d = 0; d < dims.size() && permuted; ++d) {
+      int which = -1;
+      for (size_t v = 0; v < root_vars_.size(); ++v)
+        if (ix[d].var == root_vars_[v] && ix[d].off == 0) which = (int)v;
+      if (which < 0 || used[which] || root_dims_[which] != dims[d]) permuted = false;
+      else { used[which] = 1; rec.root_var.push_back(which); }
+    }
+    if (!permuted) rec.root_var.clear();
+  }
   loads.push_back(rec);
+  if (permuted && perm_hook) {
+    std::string hooked;
+    if (perm_hook(slot, rec.root_var, &hooked)) {
+      std::string v = fresh();
+      line(std::string("const ") + info(n.ty.dt).ctype + " " + v + " = " + load_conv(n.ty.dt, hooked) + ";");
+      return v;
+    }
+  }
   bool direct = allow_direct_ && rec.affine && dims == root_dims_;
   bool shifted = false;
   if (direct)

@@ -28,6 +28,9 @@ struct LoadRecord {
   int node;                     // materialized node that is read
   std::vector<int64_t> off;     // constant offsets relative to the root index (valid if `affine`)
   bool affine = false;          // index is root identity + constant offsets
+  // per input dimension: which root variable indexes it with offset 0 (-1: anything else).  A
+  // permutation of the root variables that is not the identity marks a transposed read.
+  std::vector<int> root_var;
 };
 
 class Emitter {
@@ -61,6 +64,9 @@ class Emitter {
   // Loads of an input at root-index + constant offsets can be redirected (to an LDS halo tile):
   // the hook returns true and the expression to read instead of global memory.
   std::function<bool(int slot, const std::vector<int64_t>& off, std::string* expr)> tile_hook;
+  // Loads whose index is a non-identity permutation of the root variables (a transposed read) can
+  // be redirected too; `root_var[d]` is the root variable that indexes input dimension d.
+  std::function<bool(int slot, const std::vector<int>& root_var, std::string* expr)> perm_hook;
 
   // pad / dynamic_update_slice guards: when everything read under a guard comes from a tile or a
   // preloaded vector (so evaluating it at a point the guard excludes cannot fault), evaluate both

@@ -1183,10 +1183,137 @@ struct Planner {
     return true;
   }
 
+  // ------------------------------------------------------------------ maps with transposed reads
+  // A map that reads an input with its two fastest-varying roles swapped (out[.., a, b] uses
+  // in[.., b, .., a]: the output's minor index selects a slow dimension of the input) would read
+  // that input with a large stride per lane.  Here a workgroup owns a 64 x 64 tile of the two
+  // dimensions involved: the input tile is read along the input's own minor dimension
+  // (coalesced), parked in LDS with a one-element row pad, and read back transposed.
+  bool emit_map_transposed(int root) {
+    const Node& rn = g.nodes[root];
+    const auto& dims = rn.ty.dims;
+    const int n = rn.ty.rank();
+    if (!opt.lds_transpose || n < 2 || rn.ty.numel() < (1 << 16)) return false;
+    const int TS = 64, ROWS = kBlock / TS;
+    auto fresh_emitter = [&](Emitter& em) {
+      em.excess_precision = opt.excess_precision;
+      em.idx64 = needs64(cone_nodes(root));
+      std::vector<std::string> vars;
+      for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
+      em.set_root(dims, vars, false);
+      em.vec = 1;
+      em.indent = 6;
+    };
+    // pass 1: which reads are transposed, and against which root dimension
+    Emitter probe(g, [&](int x) { return x != root && mat[x]; });
+    fresh_emitter(probe);
+    probe.emit(root, root_index(dims));
+    int q = -1;                      // root dimension that indexes the staged inputs' minor dimension
+    std::map<int, std::vector<int>> staged;   // node -> root_var
+    for (auto& l : probe.loads) {
+      if (l.root_var.empty()) continue;
+      const int in_minor_var = l.root_var.back();
+      if (in_minor_var == n - 1) continue;                     // its minor dim already follows the output's
+      if (dims[in_minor_var] < 16 || dims[n - 1] < 16) continue;
+      const int es = info(g.nodes[l.node].ty.dt).size;
+      if (es != 2 && es != 4 && es != 8) continue;
+      if (q < 0) q = in_minor_var;
+      if (in_minor_var != q) continue;                          // one tiling serves one pairing
+      auto it2 = staged.find(l.node);
+      if (it2 != staged.end() && it2->second != l.root_var) continue;
+      staged[l.node] = l.root_var;
+    }
+    if (staged.empty()) return false;
+    int64_t lds_total = 0;
+    for (auto& kv : staged) lds_total += (int64_t)TS * (TS + 1) * info(g.nodes[kv.first].ty.dt).size;
+    if (lds_total > 64 * 1024) return false;
+
+    // pass 2: emit with the transposed reads redirected to the tiles
+    Emitter em(g, [&](int x) { return x != root && mat[x]; });
+    fresh_emitter(em);
+    em.perm_hook = [&](int slot, const std::vector<int>& rv, std::string* expr) {
+      auto it2 = staged.find(em.inputs[slot]);
+      if (it2 == staged.end() || it2->second != rv) return false;
+      *expr = "tile" + std::to_string(slot) + "[tb * " + std::to_string(TS + 1) + " + ta]";
+      return true;
+    };
+    std::string val = em.emit(root, root_index(dims));
+    std::string body = em.take_code();
+    const std::string it = em.idx_t();
+    const int64_t DQ = dims[q], DM = dims[n - 1];
+    const int64_t ntq = (DQ + TS - 1) / TS, ntm = (DM + TS - 1) / TS;
+    int64_t outer = 1;
+    for (int d = 0; d < n - 1; ++d) if (d != q) outer *= dims[d];
+    const int64_t nblocks = outer * ntq * ntm;
+    if (nblocks >= ((int64_t)1 << 31)) return false;
+    const std::string kname = "@K@_map_t";
+    std::ostringstream o;
+    o << "// map with transposed reads staged through 64x64 LDS tiles: " << describe(root) << " -> " << rn.ty.str() << "\n";
+    o << signature(kname, em.inputs, {{info(rn.ty.dt).stype, "out0"}}) << " {\n";
+    for (auto& kv : staged) {
+      const int slot = em.slot_of(kv.first);
+      o << "  __shared__ " << info(g.nodes[kv.first].ty.dt).stype << " tile" << slot << "[" << TS * (TS + 1) << "];\n";
+    }
+    // block -> (outer coordinates, tile of dimension q, tile of the minor dimension)
+    o << "  unsigned rest = blockIdx.x;\n";
+    o << "  const " << it << " m0 = (" << it << ")(rest % " << ntm << "u) * " << TS << "; rest /= " << ntm << "u;\n";
+    o << "  const " << it << " q0 = (" << it << ")(rest % " << ntq << "u) * " << TS << "; rest /= " << ntq << "u;\n";
+    for (int d = n - 2; d >= 0; --d) {
+      if (d == q) continue;
+      o << "  const " << it << " i" << d << " = (" << it << ")(rest % " << dims[d] << "u); rest /= " << dims[d] << "u;\n";
+    }
+    o << "  const int lane = threadIdx.x % " << TS << ", grp = threadIdx.x / " << TS << ";\n";
+    // phase 1: read each staged input along its own minor dimension
+    for (auto& kv : staged) {
+      const int slot = em.slot_of(kv.first);
+      const Node& in = g.nodes[kv.first];
+      const auto& rv = kv.second;
+      // linear offset of the tile origin's row: every input dim d is indexed by root var rv[d]
+      std::vector<int64_t> stride(in.ty.rank(), 1);
+      for (int d = in.ty.rank() - 2; d >= 0; --d) stride[d] = stride[d + 1] * in.ty.dims[d + 1];
+      std::string base = "0";
+      int64_t stride_m = 0;
+      for (int d = 0; d < in.ty.rank(); ++d) {
+        if (rv[d] == n - 1) { stride_m = stride[d]; continue; }
+        if (rv[d] == q) continue;   // the input's minor dimension
+        base += " + i" + std::to_string(rv[d]) + " * " + std::to_string(stride[d]) + (em.idx64 ? "LL" : "");
+      }
+      o << "  {\n    const " << it << " base = " << base << ";\n";
+      o << "#pragma unroll\n    for (int r = 0; r < " << TS / ROWS << "; ++r) {\n";
+      o << "      const int tb = r * " << ROWS << " + grp, ta = lane;\n";
+      o << "      if (m0 + tb < " << DM << " && q0 + ta < " << DQ << ")\n";
+      o << "        tile" << slot << "[tb * " << TS + 1 << " + ta] = in" << slot << "[base + (m0 + tb) * " << stride_m << (em.idx64 ? "LL" : "") << " + (q0 + ta)];\n";
+      o << "    }\n  }\n";
+    }
+    o << "  __syncthreads();\n";
+    // phase 2: the map itself, lanes along the output's minor dimension
+    o << "#pragma unroll 4\n  for (int r = 0; r < " << TS / ROWS << "; ++r) {\n";
+    o << "    const int ta = r * " << ROWS << " + grp, tb = lane;\n";
+    o << "    const " << it << " i" << q << " = q0 + ta, i" << n - 1 << " = m0 + tb;\n";
+    o << "    if (i" << q << " < " << DQ << " && i" << n - 1 << " < " << DM << ") {\n";
+    o << body;
+    Index rix = root_index(dims);
+    o << "      out0[" << em.linear(rix, dims) << "] = " << em.store_value(rn.ty.dt, val) << ";\n";
+    o << "    }\n  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named(kname, kb_final);
+    L.kind = "map_transposed";
+    L.grid[0] = (unsigned)nblocks;
+    L.block[0] = kBlock;
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    L.algo_bytes = algo_bytes(em.inputs, {root});
+    L.desc = describe(root);
+    plan.launches.push_back(L);
+    return true;
+  }
+
   // ------------------------------------------------------------------ map kernels
   void emit_map(int root) {
     if (lds_only.count(root)) return;   // evaluated inside its only reader's kernel
     if (emit_map_lds(root)) return;
+    if (emit_map_transposed(root)) return;
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
     const int n = rn.ty.rank();

@@ -51,6 +51,7 @@ struct PlanOptions {
   // device-scope release fence every workgroup needs before taking its ticket (an L2 write-back on
   // this multi-die part) made the sinsum kernel 2x slower than the two-launch form.
   bool single_pass_reduce = false;
+  bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS
   int lds_tile2[3] = {4, 8, 64};   // outputs per workgroup tile of the two-step kernel

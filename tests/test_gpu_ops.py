@@ -5,7 +5,7 @@ index ops against the oracle."""
 import numpy as np
 import pytest
 
-from _harness import gpu_run, oracle_run, rel_err
+from _harness import gpu_run, oracle_run, rel_err, max_rel_to_scale
 from oracle import stablehlo_interp as I
 from oracle import lowfloat as lf
 
@@ -343,3 +343,57 @@ def test_divide_by_a_broadcast_scalar_is_correctly_rounded(rx, client, divisor):
     same = got[0].a.view(np.uint32) == want.view(np.uint32)
     both_nan = np.isnan(got[0].a) & np.isnan(want)
     assert (same | both_nan).all(), (x[~(same | both_nan)][:5], got[0].a[~(same | both_nan)][:5], want[~(same | both_nan)][:5])
+
+
+# ---- maps with transposed reads (64x64 tiles through LDS) ---------------------------------------
+def _tt_(shape, dt):
+    return "tensor<" + "".join("%dx" % d for d in shape) + dt + ">"
+
+
+@pytest.mark.parametrize("shape,perm,dt", [((300, 257), (1, 0), "f32"), ((257, 300), (1, 0), "f64"), ((64, 1030), (1, 0), "i32"),
+                                           ((9, 130, 70), (0, 2, 1), "f32"), ((70, 33, 129), (2, 1, 0), "f32"),
+                                           ((3, 66, 5, 80), (0, 3, 2, 1), "bf16"), ((130, 20, 70), (1, 2, 0), "f32")])
+def test_transpose_through_lds_tiles(rx, client, shape, perm, dt):
+    """Pure transposes of every kind that moves the minor dimension, with tiles cut by the edges;
+    bit-exact (a transpose moves values, it does not compute)."""
+    out_shape = tuple(shape[p] for p in perm)
+    text = ("module { func.func @main(%%a: %s) -> %s {\n  %%0 = stablehlo.transpose %%a, dims = [%s] : (%s) -> %s\n  return %%0 : %s } }"
+            % (_tt_(shape, dt), _tt_(out_shape, dt), ", ".join(map(str, perm)), _tt_(shape, dt), _tt_(out_shape, dt), _tt_(out_shape, dt)))
+    rng = np.random.default_rng(0)
+    x = I.tensor(rng.integers(-1000, 1000, size=shape), dt) if dt == "i32" else I.tensor(rng.normal(size=shape), dt)
+    got, exe = gpu_run(rx, client, text, [x])
+    assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
+    want = np.transpose(x.a, perm)
+    assert got[0].a.shape == want.shape and np.array_equal(got[0].a, want)
+    assert np.array_equal(got[0].a, oracle_run(text, [x])[0].a)
+
+
+def test_map_with_transposed_and_plain_operands(rx, client):
+    """sin(a') * b + c' in one kernel: two transposed reads share the tiling, one operand is read in place."""
+    m, n = 200, 330
+    ta, tb = _tt_((n, m), "f32"), _tt_((m, n), "f32")
+    text = ("module { func.func @main(%%a: %s, %%b: %s, %%c: %s) -> %s {\n"
+            "  %%0 = stablehlo.transpose %%a, dims = [1, 0] : (%s) -> %s\n  %%1 = stablehlo.sine %%0 : %s\n"
+            "  %%2 = stablehlo.multiply %%1, %%b : %s\n  %%3 = stablehlo.transpose %%c, dims = [1, 0] : (%s) -> %s\n"
+            "  %%4 = stablehlo.add %%2, %%3 : %s\n  return %%4 : %s } }" % (ta, tb, ta, tb, ta, tb, tb, tb, ta, tb, tb, tb))
+    rng = np.random.default_rng(1)
+    a, b, c = I.tensor(rng.normal(size=(n, m)), "f32"), I.tensor(rng.normal(size=(m, n)), "f32"), I.tensor(rng.normal(size=(n, m)), "f32")
+    got, exe = gpu_run(rx, client, text, [a, b, c])
+    assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
+    ref = oracle_run(text, [a, b, c])
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-6
+
+
+def test_transposed_reads_with_different_pairings_fall_back_per_operand(rx, client):
+    """out[i,j,k] = a[k,j,i] + b[i,k,j]: the minor dimensions of a and b pair with different output
+    dimensions; one of them is staged, the other is read with a stride -- same values either way."""
+    s = (40, 48, 56)
+    ta, tb, to = _tt_((56, 48, 40), "f32"), _tt_((40, 56, 48), "f32"), _tt_(s, "f32")
+    text = ("module { func.func @main(%%a: %s, %%b: %s) -> %s {\n"
+            "  %%0 = stablehlo.transpose %%a, dims = [2, 1, 0] : (%s) -> %s\n  %%1 = stablehlo.transpose %%b, dims = [0, 2, 1] : (%s) -> %s\n"
+            "  %%2 = stablehlo.add %%0, %%1 : %s\n  return %%2 : %s } }" % (ta, tb, to, ta, to, tb, to, to, to))
+    rng = np.random.default_rng(2)
+    a, b = I.tensor(rng.normal(size=(56, 48, 40)), "f32"), I.tensor(rng.normal(size=(40, 56, 48)), "f32")
+    got, exe = gpu_run(rx, client, text, [a, b])
+    assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
+    assert np.array_equal(got[0].a, np.transpose(a.a, (2, 1, 0)) + np.transpose(b.a, (0, 2, 1)))
