@@ -1650,9 +1650,28 @@ struct Planner {
     em.indent = 2;
     std::string initv = em.emit(rn.in[1], Index{});
     std::string ibody = em.take_code();
+    // Few outputs and a long reduction: one thread per output would leave most of the chip idle
+    // (a column sum of an 8192 x 8192 matrix has 8192 outputs).  The largest reduced dimension is
+    // then cut into `split` chunks (blockIdx.y); each chunk writes a partial per output and a
+    // second small kernel combines the partials in chunk order and applies the init value.
+    int64_t red_len = 1;
+    size_t ks = 0;
+    for (size_t k = 0; k < red.size(); ++k) {
+      red_len *= inn.ty.dims[red[k]];
+      if (inn.ty.dims[red[k]] > inn.ty.dims[red[ks]]) ks = k;
+    }
+    int64_t split = 1;
+    if (!red.empty() && nout > 0 && nout <= 32 * 1024 && red_len >= 64) {
+      const int64_t ds = inn.ty.dims[red[ks]];
+      split = std::min<int64_t>({ds, (512 * 1024 + nout - 1) / nout, 1024, std::max<int64_t>(1, red_len / 16)});
+    }
+    const bool two_pass = split >= 2;
+    const int64_t chunk = two_pass ? (inn.ty.dims[red[ks]] + split - 1) / split : 0;
+    if (two_pass) split = (inn.ty.dims[red[ks]] + chunk - 1) / chunk;
     std::ostringstream o;
-    o << "// reduce (generic): " << describe(rn.in[0]) << " over dims -> " << rn.ty.str() << "\n";
-    o << signature(kname, em.inputs, {{info(dt).stype, "out0"}}) << " {\n";
+    o << "// reduce (generic" << (two_pass ? ", reduced dimension cut into " + std::to_string(split) + " chunks" : std::string()) << "): " << describe(rn.in[0])
+      << " over dims -> " << rn.ty.str() << "\n";
+    o << signature(kname, em.inputs, {{two_pass ? ACC : std::string(info(dt).stype), two_pass ? "partial" : "out0"}}) << " {\n";
     o << "  const " << it << " oid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
     o << "  if (oid >= " << nout << ") return;\n";
     o << "  " << it << " rr = oid;\n";
@@ -1661,26 +1680,74 @@ struct Planner {
       o << "  rr /= " << inn.ty.dims[kept[k]] << ";\n";
     }
     o << "  " << ACC << " acc = " << red_identity(rn.red, dt) << ";\n";
-    for (size_t k = 0; k < red.size(); ++k)
-      o << std::string(2 + 2 * k, ' ') << "for (" << it << " r" << k << " = 0; r" << k << " < " << inn.ty.dims[red[k]] << "; ++r" << k << ") {\n";
+    for (size_t k = 0; k < red.size(); ++k) {
+      const std::string pad(2 + 2 * k, ' ');
+      if (two_pass && k == ks) {
+        o << pad << "const " << it << " r" << k << "_end = rx_min<" << it << ">(((" << it << ")blockIdx.y + 1) * " << chunk << ", " << inn.ty.dims[red[k]] << ");\n";
+        o << pad << "for (" << it << " r" << k << " = (" << it << ")blockIdx.y * " << chunk << "; r" << k << " < r" << k << "_end; ++r" << k << ") {\n";
+      } else {
+        o << pad << "for (" << it << " r" << k << " = 0; r" << k << " < " << inn.ty.dims[red[k]] << "; ++r" << k << ") {\n";
+      }
+    }
     o << body;
     o << std::string(4 + 2 * red.size(), ' ') << "acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n";
     for (int k = (int)red.size() - 1; k >= 0; --k) o << std::string(2 + 2 * k, ' ') << "}\n";
-    o << ibody;
-    o << "  const " << ACC << " r = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + initv) << ";\n";
     std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
-    o << "  out0[oid] = " << Emitter::store_conv(dt, rv) << ";\n}\n\n";
+    std::vector<int> fin_inputs;
+    if (!two_pass) {
+      o << ibody;
+      o << "  const " << ACC << " r = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + initv) << ";\n";
+      o << "  out0[oid] = " << Emitter::store_conv(dt, rv) << ";\n}\n\n";
+    } else {
+      o << "  partial[(" << it << ")blockIdx.y * " << nout << " + oid] = acc;\n}\n\n";
+      // the init value may read buffers of its own: evaluate it with a fresh numbering
+      Emitter e3(g, [&](int x) { return mat[x]; });
+      e3.excess_precision = opt.excess_precision;
+      e3.indent = 2;
+      std::string initv2 = e3.emit(rn.in[1], Index{});
+      std::string ibody2 = e3.take_code();
+      fin_inputs = e3.inputs;
+      o << "// reduce (generic): combine " << split << " partials per output, apply init -> " << rn.ty.str() << "\n";
+      std::string sg = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void @K@_reduce_combine(const " + ACC + "* __restrict__ partial";
+      for (size_t k = 0; k < fin_inputs.size(); ++k) sg += ", " + ptr_decl(info(g.nodes[fin_inputs[k]].ty.dt).stype, true, "in" + std::to_string(k));
+      sg += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
+      o << sg << " {\n";
+      o << "  const int oid = (int)blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+      o << "  if (oid >= " << nout << ") return;\n";
+      o << "  " << ACC << " acc = " << red_identity(rn.red, dt) << ";\n";
+      o << "  for (int s = 0; s < " << split << "; ++s) acc = " << red_apply(rn.red, dt, "acc", "partial[s * " + std::to_string(nout) + " + oid]") << ";\n";
+      o << ibody2;
+      o << "  const " << ACC << " r = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + initv2) << ";\n";
+      o << "  out0[oid] = " << Emitter::store_conv(dt, rv) << ";\n}\n\n";
+    }
     const std::string kb_final = finalize(o.str());
     Launch L;
     L.kernel = named(kname, kb_final);
     L.kind = "reduce_generic";
     L.grid[0] = (unsigned)((nout + kBlock - 1) / kBlock);
+    L.grid[1] = (unsigned)(two_pass ? split : 1);
     L.block[0] = kBlock;
     for (int i : em.inputs) L.args.push_back(buffer_for(i));
-    L.args.push_back(buffer_for(root));
     L.algo_bytes = algo_bytes(em.inputs, {root});
     L.desc = describe(rn.in[0]) + " reduce";
+    if (!two_pass) {
+      L.args.push_back(buffer_for(root));
+      plan.launches.push_back(L);
+      return;
+    }
+    const int sc = scratch(split * nout * (dt == DT::F64 || info(dt).size == 8 ? 8 : 4));
+    L.args.push_back(sc);
     plan.launches.push_back(L);
+    Launch L2;
+    L2.kernel = named("@K@_reduce_combine", kb_final);
+    L2.kind = "reduce_final";
+    L2.grid[0] = (unsigned)((nout + kBlock - 1) / kBlock);
+    L2.block[0] = kBlock;
+    L2.args.push_back(sc);
+    for (int i : fin_inputs) L2.args.push_back(buffer_for(i));
+    L2.args.push_back(buffer_for(root));
+    L2.desc = "combine partials";
+    plan.launches.push_back(L2);
   }
 
   // ------------------------------------------------------------------ row groups

@@ -166,7 +166,10 @@ def test_float_sum_closed_form(rx, client):
 
 
 @pytest.mark.parametrize("shape,dims", [((64, 1000), [1]), ((1000, 64), [0]), ((7, 33, 65), [2]), ((7, 33, 65), [1, 2]),
-                                        ((7, 33, 65), [0]), ((5, 6, 7), [0, 2]), ((300, 4096), [1]), ((3, 70), [1])])
+                                        ((7, 33, 65), [0]), ((5, 6, 7), [0, 2]), ((300, 4096), [1]), ((3, 70), [1]),
+                                        # few outputs, long reductions: the reduced dimension is cut into chunks
+                                        ((1000, 520), [0]), ((37, 130, 9), [0, 1]), ((130, 37, 9), [0, 1]), ((3, 1030, 2), [1]),
+                                        ((2049, 3), [0])])
 @pytest.mark.parametrize("body", ["add", "maximum", "minimum"])
 def test_partial_reductions_f32(rx, client, shape, dims, body):
     x = np.random.default_rng(3).normal(size=shape).astype(np.float32)
@@ -397,3 +400,16 @@ def test_transposed_reads_with_different_pairings_fall_back_per_operand(rx, clie
     got, exe = gpu_run(rx, client, text, [a, b])
     assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
     assert np.array_equal(got[0].a, np.transpose(a.a, (2, 1, 0)) + np.transpose(b.a, (0, 2, 1)))
+
+
+def test_chunked_integer_reduction_with_an_init_value(rx, client):
+    """A column sum whose reduced dimension is cut into chunks: exact in i32, the init value is
+    applied once (by the combining kernel), chunk sizes that do not divide the extent."""
+    shape = (1001, 77)
+    x = np.random.default_rng(8).integers(-1000, 1000, size=shape).astype(np.int32)
+    text = mod([_tt(shape, "i32"), "tensor<i32>"], _tt([77], "i32"),
+               "    %%0 = stablehlo.reduce(%%arg0 init: %%arg1) applies stablehlo.add across dimensions = [0] : (%s, tensor<i32>) -> %s\n"
+               "    return %%0 : %s\n" % (_tt(shape, "i32"), _tt([77], "i32"), _tt([77], "i32")))
+    got, exe = gpu_run(rx, client, text, [I.Tensor(x, "i32"), I.Tensor(np.int32(12345), "i32")])
+    assert [l["kind"] for l in exe.launches()] == ["reduce_generic", "reduce_final"]
+    assert np.array_equal(got[0].a, x.sum(axis=0, dtype=np.int32) + np.int32(12345))
