@@ -277,6 +277,35 @@ RX_DEV T rx_wave_reduce(T v, OP op) {
   return rx_readlane63(v);
 }
 
+// Value of lane (lane ^ 16): the one exchange that crosses rows of 16 lanes
+template <typename T>
+RX_DEV T rx_xor16(T v) {
+  const rx_i32 addr = (rx_i32)(((__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u))) ^ 16u) << 2);
+  if constexpr (sizeof(T) == 8) {
+    rx_u64 u = __builtin_bit_cast(rx_u64, v);
+    rx_u32 lo = (rx_u32)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)(rx_u32)u);
+    rx_u32 hi = (rx_u32)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)(rx_u32)(u >> 32));
+    return __builtin_bit_cast(T, ((rx_u64)hi << 32) | lo);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(rx_i32, v)));
+  } else {
+    return (T)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)v);
+  }
+}
+// Combine over aligned groups of W lanes (W a power of two up to 32); every lane of a group
+// ends up with its group's result.  Groups of a wavefront are independent: a group whose lanes
+// have all left the kernel is simply not there.
+template <int W, typename T, typename OP>
+RX_DEV T rx_group_reduce(T v, OP op) {
+  static_assert(W == 1 || W == 2 || W == 4 || W == 8 || W == 16 || W == 32, "group width");
+  if constexpr (W >= 2) v = op(v, rx_dpp_t<T, 0xB1, 0xf>(v));    // quad_perm [1,0,3,2]
+  if constexpr (W >= 4) v = op(v, rx_dpp_t<T, 0x4E, 0xf>(v));    // quad_perm [2,3,0,1]
+  if constexpr (W >= 8) v = op(v, rx_dpp_t<T, 0x141, 0xf>(v));   // row_half_mirror
+  if constexpr (W >= 16) v = op(v, rx_dpp_t<T, 0x140, 0xf>(v));  // row_mirror
+  if constexpr (W >= 32) v = op(v, rx_xor16(v));
+  return v;
+}
+
 // Combine over a workgroup of NWAVES wavefronts through LDS; result uniform.
 template <typename T, typename OP, int NWAVES>
 RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {

@@ -1765,8 +1765,13 @@ struct Planner {
     for (int d = 0; d < n; ++d) (d < nkeep ? rows : cols) *= full.dims[d];
     int vec = pick_vec(full);
     while (vec > 1 && cols % vec) vec >>= 1;
-    // lanes cooperating on one row
-    const int L = cols / vec >= 512 ? 256 : 64;
+    // lanes cooperating on one row: a workgroup for long rows, a wavefront for medium ones, an
+    // aligned group of 2..32 lanes for short ones (several rows per wavefront)
+    int L = cols / vec >= 512 ? 256 : 64;
+    if (cols / vec <= 32) {
+      L = 1;
+      while (L < cols / vec) L <<= 1;
+    }
     const int rows_per_block = kBlock / L;
     const int64_t iters = (cols / vec + L - 1) / L;
     const bool cache = iters <= 8;
@@ -1822,7 +1827,7 @@ struct Planner {
     o << signature(kname, em.inputs, outs) << " {\n";
     o << "  const int lane = threadIdx.x % " << L << ";\n";
     o << "  const " << it << " row = (" << it << ")blockIdx.x * " << rows_per_block << " + threadIdx.x / " << L << ";\n";
-    if (L == 64) o << "  if (row >= " << rows << ") return;\n";  // whole wavefronts leave together
+    if (L <= 64) o << "  if (row >= " << rows << ") return;\n";  // whole groups of lanes leave together
     o << init_code;
     // decode row -> leading index vars
     {
@@ -1892,6 +1897,8 @@ struct Planner {
       o << "      }\n    }\n  }\n";
       if (L == 64)
         o << "  a" << pc.node << " = rx_wave_reduce(a" << pc.node << ", " << red_functor(p.red) << ");\n";
+      else if (L < 64)
+        o << "  a" << pc.node << " = rx_group_reduce<" << L << ">(a" << pc.node << ", " << red_functor(p.red) << ");\n";
       else
         o << "  a" << pc.node << " = rx_block_reduce<" << ACC << ", decltype(" << red_functor(p.red) << "), " << kBlock / 64 << ">(a" << pc.node << ", "
           << red_functor(p.red) << ", reinterpret_cast<" << ACC << "*>(lds_raw));\n";

@@ -413,3 +413,28 @@ def test_chunked_integer_reduction_with_an_init_value(rx, client):
     got, exe = gpu_run(rx, client, text, [I.Tensor(x, "i32"), I.Tensor(np.int32(12345), "i32")])
     assert [l["kind"] for l in exe.launches()] == ["reduce_generic", "reduce_final"]
     assert np.array_equal(got[0].a, x.sum(axis=0, dtype=np.int32) + np.int32(12345))
+
+
+# ---- row groups on short rows: several rows share a wavefront --------------------------------------
+@pytest.mark.parametrize("rows,cols", [(1000, 3), (777, 5), (4099, 10), (300, 17), (129, 33), (515, 48), (64, 64), (9, 2)])
+def test_softmax_over_short_rows(rx, client, rows, cols):
+    """max / exp-sum / divide fused in one row kernel; rows of 2..64 elements are handled by
+    aligned groups of 1..32 lanes.  Against scipy-style softmax in float64 and the row-sum invariant."""
+    ty, to = _tt_((rows, cols), "f32"), _tt_((rows,), "f32")
+    text = ("module { func.func @main(%%a: %s) -> %s {\n"
+            " %%ninf = stablehlo.constant dense<0xFF800000> : tensor<f32>\n %%z = stablehlo.constant dense<0.0> : tensor<f32>\n"
+            " %%m = stablehlo.reduce(%%a init: %%ninf) applies stablehlo.maximum across dimensions = [1] : (%s, tensor<f32>) -> %s\n"
+            " %%mb = stablehlo.broadcast_in_dim %%m, dims = [0] : (%s) -> %s\n %%d = stablehlo.subtract %%a, %%mb : %s\n %%e = stablehlo.exponential %%d : %s\n"
+            " %%s = stablehlo.reduce(%%e init: %%z) applies stablehlo.add across dimensions = [1] : (%s, tensor<f32>) -> %s\n"
+            " %%sb = stablehlo.broadcast_in_dim %%s, dims = [0] : (%s) -> %s\n %%r = stablehlo.divide %%e, %%sb : %s\n return %%r : %s } }"
+            % (ty, ty, ty, to, to, ty, ty, ty, ty, to, to, ty, ty, ty))
+    x = np.random.default_rng(rows + cols).normal(size=(rows, cols)).astype(np.float32) * 3
+    got, exe = gpu_run(rx, client, text, [I.Tensor(x, "f32")])
+    assert [l["kind"] for l in exe.launches()] == ["row"]
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    want = e / e.sum(axis=1, keepdims=True)
+    assert np.max(np.abs(got[0].a - want)) <= 2e-6
+    assert np.allclose(got[0].a.sum(axis=1), 1.0, atol=1e-5)
+    ref = oracle_run(text, [I.Tensor(x, "f32")], hifi=True)
+    assert np.max(np.abs(got[0].a - ref[0].a)) <= 2e-6
