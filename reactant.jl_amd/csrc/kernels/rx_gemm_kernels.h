@@ -154,6 +154,9 @@ struct rx_tile_copy {
   static constexpr int PER = (TOTAL + NT - 1) / NT;        // vectors per thread
   rx_u32x4 r[PER];
 
+  // ZR / ZC: rows / column vectors past the end read as zero instead (the contracted dimension,
+  // whose tail must not contribute to the sums)
+  template <bool ZR, bool ZC>
   RX_MEM void load(const E* __restrict__ g, long long gld, int row0, int col0, int nrows, int ncols, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -161,9 +164,11 @@ struct rx_tile_copy {
       if (TOTAL % NT == 0 || v < TOTAL) {
         int rr = row0 + v / VPR;
         int cc = col0 + (v % VPR) * VE;
+        const bool zero = (ZR && rr >= nrows) || (ZC && cc + VE > ncols);
         rr = rr < nrows ? rr : nrows - 1;
         cc = cc + VE <= ncols ? cc : ncols - VE;
         r[i] = *reinterpret_cast<const rx_u32x4*>(g + (long long)rr * gld + cc);
+        if (zero) r[i] = rx_u32x4{0u, 0u, 0u, 0u};
       }
     }
   }
@@ -188,14 +193,20 @@ struct rx_tile_copy {
 // whose tile falls outside the grid returns false.
 template <int GM, int GN, int RB, int CB>
 RX_DEV bool rx_gemm_tile(unsigned bid, int* bm, int* bn) {
-  constexpr unsigned PER = RB * CB;
-  constexpr unsigned NBC = (GN + CB - 1) / CB;
-  const unsigned xcd = bid & 7u, j = bid >> 3;
-  const unsigned blk = (j / PER) * 8u + xcd, t = j % PER;
-  const unsigned br = blk / NBC, bc = blk % NBC;
-  *bm = (int)(br * RB + t % RB);
-  *bn = (int)(bc * CB + t / RB);
-  return *bm < GM && *bn < GN;
+  if constexpr (RB == 0) {   // small tile grids: no blocks, no padding (one workgroup per tile)
+    *bm = (int)(bid % (unsigned)GM);
+    *bn = (int)(bid / (unsigned)GM);
+    return *bn < GN;
+  } else {
+    constexpr unsigned PER = RB * CB;
+    constexpr unsigned NBC = (GN + CB - 1) / CB;
+    const unsigned xcd = bid & 7u, j = bid >> 3;
+    const unsigned blk = (j / PER) * 8u + xcd, t = j % PER;
+    const unsigned br = blk / NBC, bc = blk % NBC;
+    *bm = (int)(br * RB + t % RB);
+    *bn = (int)(bc * CB + t / RB);
+    return *bm < GM && *bn < GN;
+  }
 }
 
 template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
@@ -233,15 +244,16 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
   rx_tile_copy<E, A_ROWS, A_COLS, NT> ca;
   rx_tile_copy<E, B_ROWS, B_COLS, NT> cb;
   auto gload = [&](int k0) {
-    if (A_KC) ca.load(Ab, A_GLD, m0, k0, M, K, tid); else ca.load(Ab, A_GLD, k0, m0, K, M, tid);
-    if (B_KC) cb.load(Bb, B_GLD, n0, k0, N, K, tid); else cb.load(Bb, B_GLD, k0, n0, K, N, tid);
+    constexpr bool TAIL = K % BK != 0;   // only then can a tile reach past the contracted dimension
+    if (A_KC) ca.template load<false, TAIL>(Ab, A_GLD, m0, k0, M, K, tid); else ca.template load<TAIL, false>(Ab, A_GLD, k0, m0, K, M, tid);
+    if (B_KC) cb.template load<false, TAIL>(Bb, B_GLD, n0, k0, N, K, tid); else cb.template load<TAIL, false>(Bb, B_GLD, k0, n0, K, N, tid);
   };
   gload(0);
   ca.store(lds, A_LD, tid);
   cb.store(lds + A_SZ, B_LD, tid);
   __syncthreads();
 
-  constexpr int KT = K / BK;
+  constexpr int KT = (K + BK - 1) / BK;
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < KT) gload((kt + 1) * BK);

@@ -16,7 +16,9 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   else if (a == DT::F8E4M3FN && (out == DT::F32 || out == DT::BF16 || out == DT::F16)) { mma = "rx_mma_f8"; c.kind = "gemm_f8"; esize = 1; bk = 128; }
   else return c;
   const int ve = 16 / esize;
-  if (K % bk != 0 || K < bk) return c;
+  // 16-byte loads along the contracted dimension need whole vectors; a tail shorter than the
+  // K step is zero-filled by the register-staged skeleton
+  if (K < 1 || ((a_kc || b_kc) && K % ve != 0)) return c;
   if (N % 4 != 0) return c;
   if (!a_kc && M % ve != 0) return c;
   if (!b_kc && N % ve != 0) return c;
@@ -38,6 +40,8 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (const char* e = getenv("RX_GEMM_STAGES")) stages = atoi(e) >= 2 ? atoi(e) : stages;
   int rb = 4, cb = 8;   // tiles of one XCD's block (rows x columns of the tile grid)
   if (const char* e = getenv("RX_GEMM_BLOCK")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2 && v[0] > 0 && v[1] > 0) { rb = v[0]; cb = v[1]; } }
+  // a grid of few tiles (per batch entry) is not worth padding to whole XCD blocks
+  if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) < 64) rb = cb = 0;
   const int nt = WM * WN * 64;
   if (direct) {
     int dbk = bk;

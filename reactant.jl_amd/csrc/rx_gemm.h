@@ -21,6 +21,7 @@ struct GemmChoice {
 // eight blocks (one per XCD) at a time, and the grid is padded to whole rounds of eight blocks
 // (rx_gemm_tile in kernels/rx_gemm_kernels.h decodes the same order).
 inline int64_t gemm_grid(int64_t gm, int64_t gn, int rb = 4, int cb = 8) {
+  if (rb == 0) return gm * gn;   // plain order for small tile grids
   const int64_t blocks = ((gm + rb - 1) / rb) * ((gn + cb - 1) / cb);
   return (blocks + 7) / 8 * 8 * rb * cb;
 }

@@ -36,6 +36,13 @@ for a_kc in (True, False):
                   ("bf16", "bf16", 128, 256, 128, a_kc, b_kc, 0), ("bf16", "f32", 136, 200, 64, a_kc, b_kc, 0),
                   ("f16", "f16", 128, 128, 64, a_kc, b_kc, 0),
                   ("f8E4M3FN", "f32", 128, 128, 256, a_kc, b_kc, 0), ("f8E4M3FN", "f32", 144, 208, 128, a_kc, b_kc, 0)]
+# contracted dimension that is not a multiple of the K step (tail zero-filled), any operand order
+for a_kc in (True, False):
+    for b_kc in (True, False):
+        CASES += [("f32", "f32", 200, 136, 52, a_kc, b_kc, 0), ("bf16", "f32", 136, 200, 72, a_kc, b_kc, 0),
+                  ("f8E4M3FN", "f32", 144, 208, 176, a_kc, b_kc, 0)]
+CASES += [("f32", "f32", 96, 128, 37, False, False, 0), ("bf16", "bf16", 128, 136, 1000, True, False, 0),
+          ("f32", "f32", 1000, 1000, 1000, True, False, 0), ("f32", "f32", 128, 128, 8, True, True, 0)]
 CASES += [("f32", "f32", 128, 128, 32, True, False, 3), ("bf16", "bf16", 128, 128, 64, True, True, 2),
           ("f8E4M3FN", "f32", 128, 128, 128, True, True, 2), ("bf16", "bf16", 256, 384, 512, True, False, 0)]
 
