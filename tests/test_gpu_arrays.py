@@ -89,3 +89,39 @@ def test_profiled_execution_does_not_block_and_reports_every_launch(rx, client):
     assert runs == 5 and len(ms) == len(exe.launches()) >= 1 and all(m > 0 for m in ms)
     assert all(np.array_equal(o.to_host(), want) for o in outs)
     assert exe.take_timings()[0] == 0
+
+
+def test_calls_from_several_host_threads(rx, client):
+    """Calls arrive from any host thread (Julia tasks) and frees from finalizer threads: uploads,
+    executions of one shared executable, downloads and frees from four threads at once."""
+    import threading
+    from _loader import load_programs
+    P = load_programs()
+    n = 1 << 14
+    exe = rx.xla_compile(client, P.sinsum_add(n))
+    errors, results = [], {}
+
+    def work(k):
+        try:
+            rng = np.random.default_rng(k)
+            for rep in range(20):
+                x = rng.uniform(-3, 3, n).astype(np.float32)
+                y = rng.uniform(-3, 3, n).astype(np.float32)
+                bx, by = rx.Buffer.from_host(client, x, "f32"), rx.Buffer.from_host(client, y, "f32")
+                out = exe.execute_sharded([bx, by])[0].synced_buffer().to_host()
+                want = float((np.sin(x.astype(np.float64)) + y).sum())
+                if abs(float(out) - want) > 1e-5 * np.sqrt(n) * 4:
+                    errors.append((k, rep, float(out), want))
+                bx.free()
+                by.free()
+            results[k] = True
+        except Exception as e:      # noqa: BLE001 - reported below
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]
+    assert len(results) == 4
