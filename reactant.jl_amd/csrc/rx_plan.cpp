@@ -165,6 +165,166 @@ struct Planner {
         }
       }
     }
+    dots_to_reductions();
+  }
+
+  // A dot_general whose smaller operand has at most 8 free elements (matrix-vector, vector-matrix,
+  // inner products, a handful of right-hand sides) moves every element of the larger operand once and
+  // does a few flops on it: it is a reduction, not a matrix product.  It is rewritten into
+  // reduce(multiply(broadcast(big), broadcast(small))) laid out in the large operand's own dimension
+  // order, so that the row / column / full reduction kernels stream that operand with coalesced
+  // vector loads.  Narrow floats are multiplied and summed in f32 and rounded once.
+  struct DotAsReduce {
+    bool ok = false;
+    bool big_is_lhs = true;
+    std::vector<int> lfree, rfree;
+  };
+  DotAsReduce dot_as_reduction(const Node& d) const {
+    DotAsReduce r;
+    if (!opt.dot_as_reduce || d.k != OpK::DotGeneral || d.a2.empty()) return r;
+    const TType &lt = g.nodes[d.in[0]].ty, &rt = g.nodes[d.in[1]].ty;
+    if (lt.dt != rt.dt || lt.dt == DT::I1 || d.ty.dt == DT::I1) return r;
+    if (is_float(lt.dt) != is_float(d.ty.dt)) return r;
+    auto isin = [](const std::vector<int64_t>& v, int x) { return std::find(v.begin(), v.end(), (int64_t)x) != v.end(); };
+    int64_t mfree = 1, nfree = 1, kprod = 1;
+    for (int k = 0; k < lt.rank(); ++k) if (!isin(d.a0, k) && !isin(d.a2, k)) { r.lfree.push_back(k); mfree *= lt.dims[k]; }
+    for (int k = 0; k < rt.rank(); ++k) if (!isin(d.a1, k) && !isin(d.a3, k)) { r.rfree.push_back(k); nfree *= rt.dims[k]; }
+    for (auto c : d.a2) kprod *= lt.dims[c];
+    r.big_is_lhs = lt.numel() >= rt.numel();
+    if ((r.big_is_lhs ? nfree : mfree) > 8) return r;
+    if (kprod < 1 || d.ty.numel() < 1) return r;
+    // short contractions: one thread per output element walks them as fast
+    if (kprod < 128) return r;
+    r.ok = true;
+    return r;
+  }
+
+  void dots_to_reductions() {
+    bool any = false;
+    for (auto& n : g.nodes) any = any || dot_as_reduction(n).ok;
+    if (!any) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(g.nodes.size(), -1);
+    for (const Node& n : g.nodes) {
+      DotAsReduce f = dot_as_reduction(n);
+      if (!f.ok) {
+        Node c = n;
+        for (int& i : c.in) i = remap[i];
+        remap[n.id] = out.add(c);
+        continue;
+      }
+      const Node& d = n;
+      const int bigside = f.big_is_lhs ? 0 : 1;
+      const TType bt = g.nodes[d.in[bigside]].ty, st = g.nodes[d.in[1 - bigside]].ty;
+      const auto& bbatch = bigside == 0 ? d.a0 : d.a1;
+      const auto& sbatch = bigside == 0 ? d.a1 : d.a0;
+      const auto& bcontr = bigside == 0 ? d.a2 : d.a3;
+      const auto& scontr = bigside == 0 ? d.a3 : d.a2;
+      const auto& bfree = bigside == 0 ? f.lfree : f.rfree;
+      const auto& sfree = bigside == 0 ? f.rfree : f.lfree;
+      // product dims: the big operand's dims in order, the small operand's free dims after the big
+      // operand's last kept dim
+      int ins = 0;
+      for (int k = 0; k < bt.rank(); ++k)
+        if (std::find(bcontr.begin(), bcontr.end(), (int64_t)k) == bcontr.end()) ins = k + 1;
+      struct PD { int64_t size; int role; int idx; };  // role 0 batch(j) 1 lhs free(dim) 2 rhs free(dim) 3 contract(j)
+      std::vector<PD> pd;
+      std::vector<int64_t> bmap(bt.rank()), smap(st.rank(), -1);
+      auto push_big = [&](int k) {
+        PD e{bt.dims[k], 0, 0};
+        auto bi = std::find(bbatch.begin(), bbatch.end(), (int64_t)k);
+        auto ci = std::find(bcontr.begin(), bcontr.end(), (int64_t)k);
+        if (bi != bbatch.end()) { e.role = 0; e.idx = (int)(bi - bbatch.begin()); smap[sbatch[e.idx]] = (int64_t)pd.size(); }
+        else if (ci != bcontr.end()) { e.role = 3; e.idx = (int)(ci - bcontr.begin()); smap[scontr[e.idx]] = (int64_t)pd.size(); }
+        else { e.role = bigside == 0 ? 1 : 2; e.idx = k; }
+        bmap[k] = (int64_t)pd.size();
+        pd.push_back(e);
+      };
+      for (int k = 0; k < ins; ++k) push_big(k);
+      for (int k : sfree) { smap[k] = (int64_t)pd.size(); pd.push_back({st.dims[k], bigside == 0 ? 2 : 1, k}); }
+      for (int k = ins; k < bt.rank(); ++k) push_big(k);
+      (void)bfree;
+      std::vector<int64_t> pdims;
+      for (auto& e : pd) pdims.push_back(e.size);
+
+      const DT CT = (is_narrow_float(bt.dt) || is_narrow_float(d.ty.dt)) ? DT::F32 : d.ty.dt;
+      auto unary_node = [&](OpK k, int in, TType ty) {
+        Node c;
+        c.k = k;
+        c.ty = ty;
+        c.in = {in};
+        return c;
+      };
+      auto operand = [&](int src_old, const TType& sty, const std::vector<int64_t>& map) {
+        int cur = remap[src_old];
+        if (sty.dt != CT) cur = out.add(unary_node(OpK::Convert, cur, TType{CT, sty.dims}));
+        bool identity = sty.dims == pdims;
+        for (size_t k = 0; k < map.size(); ++k) identity = identity && map[k] == (int64_t)k;
+        if (!identity) {
+          Node b = unary_node(OpK::BroadcastInDim, cur, TType{CT, pdims});
+          b.a0 = map;
+          cur = out.add(b);
+        }
+        return cur;
+      };
+      const int pb = operand(d.in[bigside], bt, bmap);
+      const int ps = operand(d.in[1 - bigside], st, smap);
+      Node mul;
+      mul.k = OpK::Binary;
+      mul.op = "multiply";
+      mul.ty = TType{CT, pdims};
+      mul.in = bigside == 0 ? std::vector<int>{pb, ps} : std::vector<int>{ps, pb};
+      const int pm = out.add(mul);
+      Node zero;
+      zero.k = OpK::Constant;
+      zero.splat = true;
+      zero.ty = TType{CT, {}};
+      zero.data.assign((size_t)info(CT).size, 0);
+      const int pz = out.add(zero);
+      Node red;
+      red.k = OpK::Reduce;
+      red.red = Red::Add;
+      red.in = {pm, pz};
+      std::vector<PD> kept;
+      for (size_t k = 0; k < pd.size(); ++k) {
+        if (pd[k].role == 3) red.a0.push_back((int64_t)k);
+        else kept.push_back(pd[k]);
+      }
+      std::vector<int64_t> kdims;
+      for (auto& e : kept) kdims.push_back(e.size);
+      red.ty = TType{CT, kdims};
+      int cur = out.add(red);
+      if (CT != d.ty.dt) cur = out.add(unary_node(OpK::Convert, cur, TType{d.ty.dt, kdims}));
+      // result order of dot_general: batch dims, lhs free dims, rhs free dims
+      std::vector<std::pair<int, int>> want;
+      for (size_t j = 0; j < d.a0.size(); ++j) want.push_back({0, (int)j});
+      for (int k : f.lfree) want.push_back({1, k});
+      for (int k : f.rfree) want.push_back({2, k});
+      std::vector<int64_t> perm;
+      for (auto& w : want)
+        for (size_t k = 0; k < kept.size(); ++k)
+          if (kept[k].role == w.first && kept[k].idx == w.second) perm.push_back((int64_t)k);
+      if (perm.size() != kept.size() || (int)perm.size() != d.ty.rank()) throw Error("dot_general: internal error in the reduction form");
+      bool identity = true, same_order = true;
+      int64_t last = -1;
+      for (size_t k = 0; k < perm.size(); ++k) {
+        identity = identity && perm[k] == (int64_t)k;
+        if (kept[perm[k]].size != 1) { same_order = same_order && perm[k] > last; last = perm[k]; }
+      }
+      if (!identity) {
+        Node t = unary_node(same_order ? OpK::Reshape : OpK::Transpose, cur, d.ty);
+        if (!same_order) t.a0 = perm;
+        cur = out.add(t);
+      }
+      if (!(out.nodes[cur].ty == d.ty)) throw Error("dot_general: internal error in the reduction form (type)");
+      remap[n.id] = cur;
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // ------------------------------------------------------------------ analysis

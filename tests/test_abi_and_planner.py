@@ -203,3 +203,27 @@ def test_single_launch_reduction_is_an_option(monkeypatch):
     monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
     rep = rx.compile_offline(P.sinsum_add(1 << 20), with_source=True)
     assert re.findall(r"kind=(\w+)", rep) == ["reduce"] and "atomicAdd(ticket" in rep
+
+
+def _dot(lt, rt, ot, attrs):
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%0 = stablehlo.dot_general %%arg0, %%arg1, %s : (%s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
+            % (lt, rt, ot, attrs, lt, rt, ot, ot))
+
+
+def test_products_with_a_vector_like_operand_plan_as_reductions(monkeypatch):
+    mv = _dot("tensor<8192x8192xf32>", "tensor<8192xf32>", "tensor<8192xf32>", "contracting_dims = [1] x [0]")
+    rep = rx.compile_offline(mv)
+    assert "kind=row" in rep and "launches: 1" in rep and "dot" not in rep.split("code object")[0].replace("dot_general", "")
+    # contracting the slow dimension walks the matrix in storage order: a column reduction cut into chunks
+    mtv = _dot("tensor<8192x8192xf32>", "tensor<8192xf32>", "tensor<8192xf32>", "contracting_dims = [0] x [0]")
+    assert "kind=reduce_generic" in rx.compile_offline(mtv)
+    inner = _dot("tensor<67108864xf32>", "tensor<67108864xf32>", "tensor<f32>", "contracting_dims = [0] x [0]")
+    rep = rx.compile_offline(inner)
+    assert "kind=reduce " in rep and "kind=reduce_final" in rep
+    # a real matrix product is left to the MFMA skeleton, a short contraction to the scalar loop
+    assert "kind=gemm_f32" in rx.compile_offline(P.gemm(256, 256, 256))
+    short = _dot("tensor<4096x16xf32>", "tensor<16xf32>", "tensor<4096xf32>", "contracting_dims = [1] x [0]")
+    assert "kind=dot_scalar" in rx.compile_offline(short)
+    monkeypatch.setenv("RX_DOT_AS_REDUCE", "0")
+    assert "kind=dot_scalar" in rx.compile_offline(mv)

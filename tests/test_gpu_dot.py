@@ -1,6 +1,7 @@
-"""dot_general on the MFMA skeletons: every operand order, element type and the
-batched form, against the f64-accumulating oracle.  Shapes are chosen so that the
-MFMA path is taken (the plan's launch kind is asserted), including tile edges."""
+"""dot_general against the f64-accumulating oracle.  On the MFMA skeletons: every operand order,
+element type and the batched form, at shapes chosen so that the MFMA path is taken (the plan's
+launch kind is asserted), including tile edges.  With a vector-like operand (matrix-vector,
+inner products, a few right-hand sides): the multiply + reduce form, every layout."""
 import numpy as np
 import pytest
 
@@ -83,3 +84,75 @@ def test_int_dot_general_reference_vectors(rx, client):
     got, _ = gpu_run(rx, client, t2, [I.Tensor(A.T.copy(), "i32"), I.Tensor(B.T.copy(), "i32")])
     assert np.array_equal(got[0].a, A.T @ B)
     assert np.array_equal(A.T @ B, np.array([[-16, -18], [-18, -20]]))
+
+
+def _dot_text(ls, rs, os_, attrs, dt, out_dt=None):
+    lt, rt, ot = _tt(ls, dt), _tt(rs, dt), _tt(os_, out_dt or dt)
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%0 = stablehlo.dot_general %%arg0, %%arg1, %s : (%s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
+            % (lt, rt, ot, attrs, lt, rt, ot, ot))
+
+
+# products with a vector-like operand run as multiply + reduce: (lhs, rhs, out, attributes, type, kinds)
+VECTOR_CASES = [
+    ((300, 1000), (1000,), (300,), "contracting_dims = [1] x [0]", "f32", ["row"]),
+    ((1000, 300), (1000,), (300,), "contracting_dims = [0] x [0]", "f32", ["reduce_generic"]),
+    ((1000,), (1000, 300), (300,), "contracting_dims = [0] x [0]", "f32", ["reduce_generic"]),
+    ((1000,), (300, 1000), (300,), "contracting_dims = [0] x [1]", "f32", ["row"]),
+    ((100003,), (100003,), (), "contracting_dims = [0] x [0]", "f32", ["reduce", "reduce_final"]),
+    ((100003,), (100003,), (), "contracting_dims = [0] x [0]", "f64", ["reduce", "reduce_final"]),
+    ((100003,), (100003,), (), "contracting_dims = [0] x [0]", "i32", ["reduce", "reduce_final"]),
+    ((130, 70), (130, 70), (), "contracting_dims = [0, 1] x [0, 1]", "f64", ["reduce", "reduce_final"]),
+    ((130, 70), (70, 130), (), "contracting_dims = [0, 1] x [1, 0]", "f32", ["reduce", "reduce_final"]),
+    ((256, 520), (520, 3), (256, 3), "contracting_dims = [1] x [0]", "f32", ["row"]),
+    ((256, 520), (3, 520), (256, 3), "contracting_dims = [1] x [1]", "bf16", ["row", "map"]),
+    ((3, 520), (256, 520), (3, 256), "contracting_dims = [1] x [1]", "f32", ["row", "map"]),
+    ((2, 520), (520, 256), (2, 256), "contracting_dims = [1] x [0]", "f16", None),
+    ((520, 256), (520, 5), (256, 5), "contracting_dims = [0] x [0]", "f32", ["reduce_generic"]),
+    ((6, 200, 300), (6, 300), (6, 200), "batching_dims = [0] x [0], contracting_dims = [2] x [1]", "f32", ["row"]),
+    ((6, 300, 200), (6, 300), (6, 200), "batching_dims = [0] x [0], contracting_dims = [1] x [1]", "f32", ["reduce_generic"]),
+    ((6, 300), (6, 200, 300), (6, 200), "batching_dims = [0] x [0], contracting_dims = [1] x [2]", "bf16", ["row", "map"]),
+    ((200, 6, 300), (300, 6), (6, 200), "batching_dims = [1] x [1], contracting_dims = [2] x [0]", "f32", None),
+    ((300, 700), (700,), (300,), "contracting_dims = [1] x [0]", "i32", ["row"]),
+    ((300, 700), (700,), (300,), "contracting_dims = [1] x [0]", "f8E4M3FN", None),
+]
+
+
+@pytest.mark.parametrize("ls,rs,os_,attrs,dt,kinds", VECTOR_CASES)
+def test_dot_general_with_a_vector_like_operand(rx, client, ls, rs, os_, attrs, dt, kinds):
+    out_dt = "f32" if dt == "f8E4M3FN" else dt
+    text = _dot_text(list(ls), list(rs), list(os_), attrs, dt, out_dt)
+    rng = np.random.default_rng(5)
+    if dt == "i32":
+        a = I.Tensor(rng.integers(-2**20, 2**20, size=ls).astype(np.int32), dt)
+        b = I.Tensor(rng.integers(-2**20, 2**20, size=rs).astype(np.int32), dt)
+    else:
+        a = I.tensor(rng.normal(size=ls), dt)
+        b = I.tensor(rng.normal(size=rs), dt)
+    got, exe = gpu_run(rx, client, text, [a, b])
+    got_kinds = [l["kind"] for l in exe.launches()]
+    assert "dot_scalar" not in got_kinds and not any(k.startswith("gemm") for k in got_kinds), got_kinds
+    if kinds is not None:
+        assert got_kinds[0] == kinds[0], got_kinds
+    ref = oracle_run(text, [a, b], hifi=True)
+    assert got[0].a.shape == ref[0].a.shape
+    if dt == "i32":
+        assert np.array_equal(got[0].a, ref[0].a)
+        return
+    err = max_rel_to_scale(got[0].a, ref[0].a)
+    if out_dt in ("bf16", "f16"):
+        assert err <= 1e-2
+    elif dt == "f64":
+        assert err <= 1e-12
+    else:
+        assert err <= 1e-5 * np.sqrt(100003 if not os_ else 1000)
+
+
+def test_short_contractions_keep_the_scalar_loop(rx, client):
+    text = _dot_text([4096, 16], [16], [4096], "contracting_dims = [1] x [0]", "f32")
+    a = I.tensor(np.random.default_rng(0).normal(size=(4096, 16)), "f32")
+    b = I.tensor(np.random.default_rng(1).normal(size=(16,)), "f32")
+    got, exe = gpu_run(rx, client, text, [a, b])
+    assert [l["kind"] for l in exe.launches()] == ["dot_scalar"]
+    ref = oracle_run(text, [a, b], hifi=True)
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-5
