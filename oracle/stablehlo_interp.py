@@ -527,6 +527,28 @@ class Parser:
             if mo and key not in a:
                 g = mo.group(1) or ""
                 a[key] = [int(t) for t in g.replace(",", " ").split()]
+        for key in ("window_dimensions", "window_strides", "base_dilations", "window_dilations",
+                    "lhs_dilation", "rhs_dilation"):
+            mo = re.search(r"\b" + key + r"\s*=\s*array<i64(?::\s*([-\d,\s]*))?>", inner)
+            if mo and key not in a:
+                a[key] = [int(t) for t in (mo.group(1) or "").replace(",", " ").split()]
+        mo = re.search(r"\bwindow_reversal\s*=\s*array<i1(?::\s*([\w,\s]*))?>", inner)
+        if mo:
+            a["window_reversal"] = [t == "true" for t in (mo.group(1) or "").replace(",", " ").split()]
+        mo = re.search(r"\bpadding\s*=\s*dense<([^>]*)>\s*:\s*tensor<(\d+)x2xi64>", inner)
+        if mo:
+            vals = [int(t) for t in re.findall(r"-?\d+", mo.group(1))]
+            nrow = int(mo.group(2))
+            if len(vals) == 1:
+                vals = vals * (2 * nrow)
+            a["padding"] = [[vals[2 * k], vals[2 * k + 1]] for k in range(nrow)]
+        mo = re.search(r"#stablehlo\.conv<([^>]*->[^>]*)>", inner)
+        if mo:
+            a["dim_numbers"] = _parse_conv_dims(mo.group(1))
+        for key in ("feature_group_count", "batch_group_count"):
+            mo = re.search(r"\b" + key + r"\s*=\s*(\d+)", inner)
+            if mo:
+                a[key] = int(mo.group(1))
         mo = re.search(r"\bdimension\s*=\s*(\d+)", inner)
         if mo:
             a["dimension"] = int(mo.group(1))
@@ -583,7 +605,7 @@ class Parser:
             src = op.attrs.pop("__dense_src__")
             cc = _Cursor(src)
             op.attrs["value"] = _parse_dense(cc.balanced("<", ">"), op.types_out[0])
-        if op.name == "reduce":
+        if op.name in ("reduce", "reduce_window"):
             op.attrs["body"] = _reduce_body_kind(op.regions[0])
         return op
 
@@ -849,6 +871,55 @@ class Parser:
                 a["rhs_contracting_dimensions"] = [0]
                 op.name = "dot_general"
             return op
+        if short == "reverse":
+            op.operands.append(c.ssa())
+            c.expect(",")
+            c.expect("dims")
+            c.expect("=")
+            op.attrs["dimensions"] = c.int_list()
+            c.expect(":")
+            self.fn_type(op)
+            return op
+        if short == "convolution":
+            # stablehlo.convolution(%lhs, %rhs) dim_numbers = [b, f, 0, 1]x[o, i, 0, 1]->[b, f, 0, 1],
+            #   window = {stride = [1, 1], pad = [[0, 0], [0, 0]], lhs_dilate = [..], rhs_dilate = [..],
+            #   reverse = [false, false]} {batch_group_count = 1 : i64, feature_group_count = 1 : i64, ...}
+            c.expect("(")
+            op.operands.append(c.ssa())
+            c.expect(",")
+            op.operands.append(c.ssa())
+            c.expect(")")
+            c.expect("dim_numbers")
+            c.expect("=")
+            j = c.s.index("->", c.i)
+            j = c.s.index("]", j) + 1
+            op.attrs["dim_numbers"] = _parse_conv_dims(c.s[c.i:j])
+            c.i = j
+            c.expect(",")
+            c.expect("window")
+            c.expect("=")
+            win = c.balanced("{", "}")
+            for key, attr in (("stride", "window_strides"), ("lhs_dilate", "lhs_dilation"),
+                              ("rhs_dilate", "rhs_dilation")):
+                mo = re.search(r"\b" + key + r"\s*=\s*\[([-\d,\s]*)\]", win)
+                if mo:
+                    op.attrs[attr] = [int(t) for t in mo.group(1).replace(",", " ").split()]
+            mo = re.search(r"\bpad\s*=\s*\[((?:\s*\[[-\d,\s]*\]\s*,?)*)\]", win)
+            if mo:
+                vals = [int(t) for t in re.findall(r"-?\d+", mo.group(1))]
+                op.attrs["padding"] = [[vals[2 * k], vals[2 * k + 1]] for k in range(len(vals) // 2)]
+            mo = re.search(r"\breverse\s*=\s*\[([\w,\s]*)\]", win)
+            if mo:
+                op.attrs["window_reversal"] = [t in ("true", "1") for t in mo.group(1).replace(",", " ").split()]
+            if c.peek() == "{":
+                inner = c.balanced("{", "}")
+                for key in ("feature_group_count", "batch_group_count"):
+                    mo = re.search(r"\b" + key + r"\s*=\s*(\d+)", inner)
+                    if mo:
+                        op.attrs[key] = int(mo.group(1))
+            c.expect(":")
+            self.fn_type(op)
+            return op
         if short == "optimization_barrier":
             if c.peek() == "%":
                 op.operands.append(c.ssa())
@@ -870,6 +941,28 @@ class Parser:
             self.fn_type(op)
             return op
         raise ParseError("unsupported op %r" % name)
+
+
+def _parse_conv_dims(text):
+    """`[b, f, 0, 1]x[o, i, 0, 1]->[b, f, 0, 1]` -> positions of every role in the three tensors."""
+    groups = re.findall(r"\[([^\]]*)\]", text)
+    if len(groups) != 3:
+        raise ParseError("convolution dimension numbers %r" % text)
+    out = {}
+    for which, grp, names in (("lhs", groups[0], ("b", "f")), ("rhs", groups[1], ("o", "i")),
+                              ("out", groups[2], ("b", "f"))):
+        toks = [t.strip() for t in grp.split(",")]
+        nsp = len(toks) - 2
+        spatial = [None] * nsp
+        for pos, t in enumerate(toks):
+            if t == names[0]:
+                out[which + "_0"] = pos
+            elif t == names[1]:
+                out[which + "_1"] = pos
+            else:
+                spatial[int(t)] = pos
+        out[which + "_spatial"] = spatial
+    return out
 
 
 def _reduce_body_kind(region):
@@ -1071,6 +1164,143 @@ def _dot_general(x, y, at, dt_out, hifi):
     return Tensor(C.astype(NP_OF[dt_out]), dt_out)
 
 
+def _windows(a, window, strides, dilations):
+    """View of `a` with the window positions as extra leading axes:
+    out[k0..k_{r-1}, o0..o_{r-1}] = a[o_i * stride_i + k_i * dilation_i]."""
+    r = a.ndim
+    outs = []
+    for d in range(r):
+        span = (window[d] - 1) * dilations[d] + 1
+        outs.append(0 if a.shape[d] < span else (a.shape[d] - span) // strides[d] + 1)
+    shape = list(window) + outs
+    st = [a.strides[d] * dilations[d] for d in range(r)] + [a.strides[d] * strides[d] for d in range(r)]
+    if any(o == 0 for o in outs):
+        return np.zeros(shape, dtype=a.dtype)
+    return np.lib.stride_tricks.as_strided(a, shape=shape, strides=st, writeable=False)
+
+
+def _reduce_window(x, init, at, dt, hifi):
+    """stablehlo.reduce_window with a monoid body (what reference src/Ops.jl:3967-4011 builds; pooling
+    ext/ReactantNNlibExt/Ops.jl:1-32, cumulative ops src/TracedRArray.jl:1086-1108): the operand is
+    dilated (base dilation) and padded with the init value, then every window is reduced."""
+    r = x.a.ndim
+    window = at["window_dimensions"]
+    strides = at.get("window_strides") or [1] * r
+    bdil = at.get("base_dilations") or [1] * r
+    wdil = at.get("window_dilations") or [1] * r
+    pad = at.get("padding") or [[0, 0]] * r
+    pre = _prefix_form(x.a.shape, window, strides, bdil, wdil, pad)
+    if pre is not None and not at.get("__general__"):
+        return _prefix_scan(x, init, pre[0], pre[1], at["body"], dt, hifi)
+    padded = _pad(x, init, [p[0] for p in pad], [p[1] for p in pad], [b - 1 for b in bdil], x.dt)
+    w = _windows(np.ascontiguousarray(padded.a), window, strides, wdil)
+    return _reduce(Tensor(w, x.dt) if not is_float(x.dt) else _FloatView(w, x.dt), init, list(range(r)), at["body"], dt, hifi)
+
+
+def _prefix_form(shape, window, strides, bdil, wdil, pad):
+    """(dim, from_the_end) when every window is a prefix (or suffix) of one dimension: the window
+    spans that whole dimension and the operand is padded by its length minus one on one side."""
+    found = None
+    for d, n in enumerate(shape):
+        if window[d] == 1 and strides[d] == 1 and bdil[d] == 1 and tuple(pad[d]) == (0, 0):
+            continue
+        if found is not None or n < 2:
+            return None
+        if window[d] != n or strides[d] != 1 or bdil[d] != 1 or wdil[d] != 1:
+            return None
+        if tuple(pad[d]) == (n - 1, 0):
+            found = (d, False)
+        elif tuple(pad[d]) == (0, n - 1):
+            found = (d, True)
+        else:
+            return None
+    return found
+
+
+_ACCUMULATE = {"add": np.add, "multiply": np.multiply, "maximum": np.maximum, "minimum": np.minimum,
+               "and": np.bitwise_and, "or": np.bitwise_or}
+
+
+def _prefix_scan(x, init, dim, from_end, body, dt, hifi):
+    """The same values as the general window form for a monoid body whose init is its identity
+    (checked against the general form on small inputs by the tests), in linear time."""
+    a = x.a
+    if is_float(dt):
+        a = a.astype(np.float64 if (hifi or dt == "f64") else a.dtype)
+    if from_end:
+        a = np.flip(a, axis=dim)
+    with np.errstate(all="ignore"):
+        r = _ACCUMULATE[body].accumulate(a, axis=dim)
+        i0 = init.a.astype(r.dtype)
+        r = _ACCUMULATE[body](r, i0)
+    if from_end:
+        r = np.flip(r, axis=dim)
+    if is_float(dt):
+        return tensor(r, dt)
+    return Tensor(np.asarray(r).astype(NP_OF[dt]), dt)
+
+
+class _FloatView:
+    """Minimal stand-in for Tensor around an array that must not be copied or rounded."""
+    __slots__ = ("a", "dt")
+
+    def __init__(self, a, dt):
+        self.a, self.dt = a, dt
+
+
+def _convolution(x, w, at, dt_out, hifi):
+    """stablehlo.convolution (built by reference src/Ops.jl:1000-1073 from NNlib's conv,
+    ext/ReactantNNlibExt/Implementations.jl:42-79): correlation of the dilated, padded input with the
+    (optionally reversed, dilated) kernel, per feature group."""
+    dn = at["dim_numbers"]
+    nsp = len(dn["lhs_spatial"])
+    strides = at.get("window_strides") or [1] * nsp
+    pad = at.get("padding") or [[0, 0]] * nsp
+    ldil = at.get("lhs_dilation") or [1] * nsp
+    rdil = at.get("rhs_dilation") or [1] * nsp
+    rev = at.get("window_reversal") or [False] * nsp
+    G = at.get("feature_group_count", 1)
+    if at.get("batch_group_count", 1) != 1:
+        raise NotImplementedError("convolution with batch_group_count != 1")
+    acc = np.float64 if (hifi or x.dt == "f64") else (np.float32 if is_float(x.dt) else NP_OF[dt_out])
+    xa = np.transpose(x.a, [dn["lhs_0"], dn["lhs_1"]] + dn["lhs_spatial"]).astype(acc)     # [b, f, s...]
+    wa = np.transpose(w.a, [dn["rhs_0"], dn["rhs_1"]] + dn["rhs_spatial"]).astype(acc)     # [o, i, k...]
+    for d in range(nsp):
+        if rev[d]:
+            wa = np.flip(wa, axis=2 + d)
+    zero = Tensor(np.zeros((), dtype=acc), "f64" if acc == np.float64 else ("f32" if acc == np.float32 else dt_out))
+    xt = Tensor.__new__(Tensor)
+    xt.a, xt.dt = xa, zero.dt
+    xp = _pad(xt, zero, [0, 0] + [p[0] for p in pad], [0, 0] + [p[1] for p in pad],
+              [0, 0] + [l - 1 for l in ldil], zero.dt).a
+    B, C = xp.shape[0], xp.shape[1]
+    O, I = wa.shape[0], wa.shape[1]
+    if C != I * G or O % G != 0:
+        raise ValueError("convolution: feature counts do not match the group count")
+    ksz = list(wa.shape[2:])
+    win = _windows(np.ascontiguousarray(xp), [1, 1] + ksz, [1, 1] + list(strides), [1, 1] + list(rdil))
+    # win[1, 1, k..., b, c, o...]
+    win = win.reshape(ksz + [B, C] + list(win.shape[2 + nsp + 2:]))
+    osp = list(win.shape[nsp + 2:])
+    out = np.zeros([B, O] + osp, dtype=acc)
+    Og = O // G
+    kk = int(np.prod(ksz)) if ksz else 1
+    for g in range(G):
+        wg = wa[g * Og:(g + 1) * Og].reshape(Og, I, kk)                      # [o, i, k]
+        xg = win.reshape([kk, B, C, -1])[:, :, g * I:(g + 1) * I, :]        # [k, b, i, P]
+        out[:, g * Og:(g + 1) * Og] = np.einsum("oik,kbip->bop", wg, xg).reshape([B, Og] + osp)
+    # canonical [b, f, s...] -> the result's own dimension order
+    perm = [0] * (2 + nsp)
+    perm[dn["out_0"]] = 0
+    perm[dn["out_1"]] = 1
+    for d in range(nsp):
+        perm[dn["out_spatial"][d]] = 2 + d
+    res = np.transpose(out, perm)
+    if is_float(dt_out):
+        return tensor(res, dt_out)
+    return Tensor(res.astype(NP_OF[dt_out]), dt_out)
+
+
 def _pad(x, pv, low, high, interior, dt):
     a = x.a
     nd = a.ndim
@@ -1236,6 +1466,20 @@ class Interpreter:
             if len(xs) != 2:
                 raise NotImplementedError("variadic reduce")
             r = _reduce(xs[0], xs[1], at["dimensions"], at["body"], op.types_out[0].dt, self.hifi)
+            return [r if self.excess else _rounded(r)]
+        if n == "reverse":
+            return [Tensor(np.ascontiguousarray(np.flip(xs[0].a, axis=tuple(at["dimensions"]))), xs[0].dt)]
+        if n == "reduce_window":
+            if len(xs) != 2:
+                raise NotImplementedError("variadic reduce_window")
+            r = _reduce_window(xs[0], xs[1], at, op.types_out[0].dt, self.hifi)
+            if tuple(r.a.shape) != tuple(op.types_out[0].shape):
+                raise ValueError("reduce_window: result shape %s, declared %s" % (r.a.shape, op.types_out[0].shape))
+            return [r if self.excess else _rounded(r)]
+        if n == "convolution":
+            r = _convolution(_rounded(xs[0]), _rounded(xs[1]), at, op.types_out[0].dt, self.hifi)
+            if tuple(r.a.shape) != tuple(op.types_out[0].shape):
+                raise ValueError("convolution: result shape %s, declared %s" % (r.a.shape, op.types_out[0].shape))
             return [r if self.excess else _rounded(r)]
         if n == "dot_general":
             r = _dot_general(_rounded(xs[0]), _rounded(xs[1]), at, op.types_out[0].dt, self.hifi)

@@ -306,6 +306,33 @@ RX_DEV T rx_group_reduce(T v, OP op) {
   return v;
 }
 
+// Value held by lane `src` (0..63) of this wavefront.
+template <typename T>
+RX_DEV T rx_lane_from(T v, rx_u32 src) {
+  const rx_i32 addr = (rx_i32)(src << 2);
+  if constexpr (sizeof(T) == 8) {
+    rx_u64 u = __builtin_bit_cast(rx_u64, v);
+    rx_u32 lo = (rx_u32)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)(rx_u32)u);
+    rx_u32 hi = (rx_u32)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)(rx_u32)(u >> 32));
+    return __builtin_bit_cast(T, ((rx_u64)hi << 32) | lo);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(rx_i32, v)));
+  } else {
+    return (T)__builtin_amdgcn_ds_bpermute(addr, (rx_i32)v);
+  }
+}
+// Inclusive prefix combine over the 64 lanes of a wavefront (lane order).
+template <typename T, typename OP>
+RX_DEV T rx_wave_scan(T v, OP op) {
+  const rx_u32 lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+#pragma unroll
+  for (rx_u32 d = 1; d < 64u; d <<= 1) {
+    const T t = rx_lane_from(v, (lane - d) & 63u);
+    if (lane >= d) v = op(t, v);
+  }
+  return v;
+}
+
 // Combine over a workgroup of NWAVES wavefronts through LDS; result uniform.
 template <typename T, typename OP, int NWAVES>
 RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {

@@ -459,6 +459,35 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       }
       return emit(n.in[0], oi);
     }
+    case OpK::Reverse: {
+      const Node& o = g_.nodes[n.in[0]];
+      Index oi = ix;
+      for (auto d : n.a0) {
+        const int64_t last = o.ty.dims[d] - 1;
+        if (ix[d].is_const()) oi[d] = const_ix(last - ix[d].off);
+        else oi[d] = temp_index(std::to_string(last) + " - (" + ix[d].str() + ")", last - ix[d].hi, last - ix[d].lo);
+      }
+      return emit(n.in[0], oi);
+    }
+    case OpK::Window: {
+      const Node& o = g_.nodes[n.in[0]];
+      const int r = o.ty.rank();
+      Index oi(r);
+      for (int d = 0; d < r; ++d) {
+        const Ix& k = ix[d];
+        const Ix& p = ix[r + d];
+        const int64_t st = n.a1[d], dl = n.a2[d];
+        if (k.is_const() && p.is_const()) oi[d] = const_ix(p.off * st + k.off * dl);
+        else if (k.is_const() && st == 1) oi[d] = shifted(p, k.off * dl);
+        else if (p.is_const() && dl == 1) oi[d] = shifted(k, p.off * st);
+        else {
+          std::string e = st == 1 ? p.str() : "(" + p.str() + ") * " + std::to_string(st);
+          e += " + " + (dl == 1 ? k.str() : "(" + k.str() + ") * " + std::to_string(dl));
+          oi[d] = temp_index(e, p.lo * st + k.lo * dl, p.hi * st + k.hi * dl);
+        }
+      }
+      return emit(n.in[0], oi);
+    }
     case OpK::DynamicSlice: {
       const Node& o = g_.nodes[n.in[0]];
       Index oi(ix.size());
@@ -666,6 +695,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       return v;
     }
     case OpK::Reduce:
+    case OpK::Scan:
     case OpK::DotGeneral:
       throw Error("internal: reduce/dot_general reached the emitter without a buffer or binding");
   }

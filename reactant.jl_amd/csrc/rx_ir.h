@@ -52,7 +52,8 @@ enum class OpK : uint8_t {
   Param, Constant, Iota,
   Unary, Binary, Compare, Select, Clamp, Convert, Gelu,
   BroadcastInDim, Reshape, Transpose, Slice, Pad, DynamicUpdateSlice, DynamicSlice, Concatenate,
-  Reduce, DotGeneral,
+  Reverse, Window,
+  Reduce, DotGeneral, Scan,
 };
 
 enum class Red : uint8_t { Add, Mul, Max, Min, And, Or };
@@ -69,6 +70,10 @@ struct Node {
   //   DynamicSlice: a0 = sizes                       Concatenate, Iota: a0[0] = dimension
   //   Reduce: a0 = dimensions                        Param: a0[0] = argument index
   //   DotGeneral: a0/a1 = lhs/rhs batching, a2/a3 = lhs/rhs contracting
+  //   Reverse: a0 = dimensions
+  //   Window (rank r -> 2r): a0/a1/a2 = window sizes/strides/dilations;
+  //       out[k_0..k_{r-1}, o_0..o_{r-1}] = in[o_i * stride_i + k_i * dilation_i]
+  //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
   std::vector<int64_t> a0, a1, a2, a3;
   Red red = Red::Add;
   // Constant payload: either one splat element or dense bytes in storage format

@@ -521,8 +521,29 @@ struct P {
     for (const char* key : {"dimensions", "broadcast_dimensions", "permutation", "start_indices", "limit_indices",
                             "strides", "edge_padding_low", "edge_padding_high", "interior_padding", "slice_sizes",
                             "dimension", "iota_dimension", "lhs_batching_dimensions", "rhs_batching_dimensions",
-                            "lhs_contracting_dimensions", "rhs_contracting_dimensions"})
+                            "lhs_contracting_dimensions", "rhs_contracting_dimensions", "window_dimensions",
+                            "window_strides", "base_dilations", "window_dilations", "lhs_dilation", "rhs_dilation",
+                            "padding", "feature_group_count", "batch_group_count"})
       scan_int_array(in, key, o);
+    {
+      size_t q = in.find("#stablehlo.conv<");
+      if (q != std::string::npos) {
+        size_t arrow = in.find("->", q);
+        size_t e = arrow == std::string::npos ? arrow : in.find(']', arrow);
+        if (e != std::string::npos) o.sa["dim_numbers"] = in.substr(q + 16, e + 1 - (q + 16));
+      }
+      q = in.find("window_reversal");
+      if (q != std::string::npos) {
+        size_t e = in.find('>', q);
+        const std::string body = in.substr(q, e == std::string::npos ? std::string::npos : e - q);
+        std::vector<int64_t> v;
+        for (size_t k = 0; k < body.size(); ++k) {
+          if (body.compare(k, 4, "true") == 0) v.push_back(1);
+          else if (body.compare(k, 5, "false") == 0) v.push_back(0);
+        }
+        o.ia["window_reversal"] = v;
+      }
+    }
     size_t p = in.find("comparison_direction");
     if (p != std::string::npos) {
       size_t q = in.find("comparison_direction ", p + 20);
@@ -748,6 +769,78 @@ struct P {
         if (c.starts("dim")) { c.expect("dim"); c.expect("="); o.ia["dimension"] = {c.integer()}; }
         else o.operands.push_back(c.ssa());
       }
+      c.expect(":");
+      fn_type(o);
+      return o;
+    }
+    if (sh == "reverse") {
+      o.operands.push_back(c.ssa());
+      c.expect(",");
+      c.expect("dims");
+      c.expect("=");
+      o.ia["dimensions"] = c.int_list();
+      c.expect(":");
+      fn_type(o);
+      return o;
+    }
+    if (sh == "convolution") {
+      // stablehlo.convolution(%lhs, %rhs) dim_numbers = [b, f, 0, 1]x[o, i, 0, 1]->[b, f, 0, 1],
+      //   window = {stride = [1, 1], pad = [[0, 0], [0, 0]], lhs_dilate = [..], rhs_dilate = [..], reverse = [..]}
+      //   {batch_group_count = 1 : i64, feature_group_count = 1 : i64, precision_config = [..]} : (..) -> ..
+      c.expect("(");
+      o.operands.push_back(c.ssa());
+      c.expect(",");
+      o.operands.push_back(c.ssa());
+      c.expect(")");
+      c.expect("dim_numbers");
+      c.expect("=");
+      std::string dn = "[" + c.balanced('[', ']') + "]";
+      c.expect("x");
+      dn += "x[" + c.balanced('[', ']') + "]";
+      c.expect("->");
+      dn += "->[" + c.balanced('[', ']') + "]";
+      o.sa["dim_numbers"] = dn;
+      c.expect(",");
+      c.expect("window");
+      c.expect("=");
+      std::string win = c.balanced('{', '}');
+      // the window dictionary uses short keys; rename them to the attribute names
+      RawOp tmp;
+      for (const char* key : {"stride", "lhs_dilate", "rhs_dilate"}) scan_int_array(win, key, tmp);
+      if (tmp.ia.count("stride")) o.ia["window_strides"] = tmp.ia["stride"];
+      if (tmp.ia.count("lhs_dilate")) o.ia["lhs_dilation"] = tmp.ia["lhs_dilate"];
+      if (tmp.ia.count("rhs_dilate")) o.ia["rhs_dilation"] = tmp.ia["rhs_dilate"];
+      {
+        size_t q = win.find("pad");
+        if (q != std::string::npos && (q == 0 || !Cur::idc(win[q - 1]))) {
+          size_t b0 = win.find('[', q);
+          int depth = 0;
+          size_t e = b0;
+          for (; e < win.size(); ++e) {
+            if (win[e] == '[') ++depth;
+            if (win[e] == ']' && --depth == 0) break;
+          }
+          std::vector<int64_t> v;
+          std::string body = win.substr(b0, e - b0);
+          for (auto& ch : body) if (ch == '[' || ch == ']' || ch == ',') ch = ' ';
+          std::stringstream ss(body);
+          int64_t x;
+          while (ss >> x) v.push_back(x);
+          o.ia["padding"] = v;
+        }
+        q = win.find("reverse");
+        if (q != std::string::npos) {
+          size_t e = win.find(']', q);
+          const std::string body = win.substr(q, e == std::string::npos ? std::string::npos : e - q);
+          std::vector<int64_t> v;
+          for (size_t k = 0; k < body.size(); ++k) {
+            if (body.compare(k, 4, "true") == 0) v.push_back(1);
+            else if (body.compare(k, 5, "false") == 0) v.push_back(0);
+          }
+          o.ia["window_reversal"] = v;
+        }
+      }
+      if (c.peek() == '{') generic_attrs(c.balanced('{', '}'), o);
       c.expect(":");
       fn_type(o);
       return o;
@@ -1144,6 +1237,368 @@ struct Builder {
     if (!(a == b)) fail(what + ": type mismatch " + a.str() + " vs " + b.str());
   }
 
+  int add_node(OpK k, const TType& t, std::vector<int> in) {
+    Node n;
+    n.k = k;
+    n.ty = t;
+    n.in = std::move(in);
+    return g.add(n);
+  }
+  int zero_of(DT dt) {
+    Node z;
+    z.k = OpK::Constant;
+    z.splat = true;
+    z.ty = TType{dt, {}};
+    z.data.assign((size_t)info(dt).size, 0);
+    return g.add(z);
+  }
+  // the strided window view of `x`: [w_0..w_{r-1}, o_0..o_{r-1}]
+  int window_view(int x, const std::vector<int64_t>& w, const std::vector<int64_t>& st, const std::vector<int64_t>& dl,
+                  const std::string& what) {
+    const TType& t = ty(x);
+    const int r = t.rank();
+    Node n;
+    n.k = OpK::Window;
+    n.in = {x};
+    n.a0 = w; n.a1 = st; n.a2 = dl;
+    n.ty.dt = t.dt;
+    n.ty.dims = w;
+    for (int d = 0; d < r; ++d) {
+      if (w[d] < 1 || st[d] < 1 || dl[d] < 1) fail(what + ": window sizes, strides and dilations must be positive");
+      const int64_t span = (w[d] - 1) * dl[d] + 1;
+      n.ty.dims.push_back(t.dims[d] < span ? 0 : (t.dims[d] - span) / st[d] + 1);
+    }
+    return g.add(n);
+  }
+
+  // reduce_window (reference src/Ops.jl:3967-4011).  Pooling (ext/ReactantNNlibExt/Ops.jl:1-32)
+  // becomes pad + window view + reduce over the window dims; the form cumsum/cumprod build
+  // (src/TracedRArray.jl:1086-1108: the window spans one whole dimension, padded by its length
+  // minus one on one side) becomes a prefix scan.
+  int build_reduce_window(const RawOp& o, int x, int init, const TType& out) {
+    const TType xt = ty(x);
+    const int r = xt.rank();
+    if (ty(init).rank() != 0 || ty(init).dt != xt.dt || out.dt != xt.dt) fail("reduce_window: operand, init and result element types must match");
+    const Red red = body_kind(o);
+    auto get = [&](const char* key, int64_t dflt) {
+      std::vector<int64_t> v = o.ia.count(key) ? o.ia.at(key) : std::vector<int64_t>(r, dflt);
+      if ((int)v.size() != r) fail(std::string("reduce_window: ") + key + " must have one entry per dimension");
+      return v;
+    };
+    if (!o.ia.count("window_dimensions")) fail("reduce_window: window_dimensions missing");
+    const auto w = get("window_dimensions", 1), st = get("window_strides", 1), bd = get("base_dilations", 1), wd = get("window_dilations", 1);
+    std::vector<int64_t> pad = o.ia.count("padding") ? o.ia.at("padding") : std::vector<int64_t>(2 * r, 0);
+    if (pad.size() == 1) pad.assign(2 * r, pad[0]);
+    if ((int)pad.size() != 2 * r) fail("reduce_window: padding must be a (rank x 2) matrix");
+    std::vector<int64_t> lo(r), hi(r), interior(r);
+    bool any_pad = false;
+    for (int d = 0; d < r; ++d) {
+      lo[d] = pad[2 * d]; hi[d] = pad[2 * d + 1]; interior[d] = bd[d] - 1;
+      if (lo[d] < 0 || hi[d] < 0 || bd[d] < 1) fail("reduce_window: negative padding is not supported");
+      any_pad = any_pad || lo[d] || hi[d] || interior[d];
+    }
+    // prefix form
+    int sd = -1, others = 0;
+    for (int d = 0; d < r; ++d) {
+      const bool unit = w[d] == 1 && st[d] == 1 && lo[d] == 0 && hi[d] == 0 && bd[d] == 1;
+      if (unit) continue;
+      ++others;
+      const bool fwd = lo[d] == xt.dims[d] - 1 && hi[d] == 0, bwd = lo[d] == 0 && hi[d] == xt.dims[d] - 1;
+      if (w[d] == xt.dims[d] && st[d] == 1 && wd[d] == 1 && bd[d] == 1 && (fwd || bwd) && xt.dims[d] > 1) sd = d;
+    }
+    if (others == 1 && sd >= 0 && xt.numel() > 0 && xt.dt != DT::I1) {
+      if (!(out == xt)) fail("reduce_window: result shape mismatch");
+      Node n;
+      n.k = OpK::Scan;
+      n.ty = xt;
+      n.in = {x, init};
+      n.red = red;
+      n.a0 = {sd};
+      n.a1 = {lo[sd] == 0 ? 1 : 0};
+      return g.add(n);
+    }
+    int cur = x;
+    if (any_pad) {
+      Node pn;
+      pn.k = OpK::Pad;
+      pn.in = {x, init};
+      pn.a0 = lo; pn.a1 = hi; pn.a2 = interior;
+      pn.ty.dt = xt.dt;
+      for (int d = 0; d < r; ++d) pn.ty.dims.push_back(lo[d] + hi[d] + xt.dims[d] + std::max<int64_t>(xt.dims[d] - 1, 0) * interior[d]);
+      cur = g.add(pn);
+    }
+    const int win = window_view(cur, w, st, wd, "reduce_window");
+    const TType wt = ty(win);
+    if (std::vector<int64_t>(wt.dims.begin() + r, wt.dims.end()) != out.dims) fail("reduce_window: result shape mismatch");
+    Node rn;
+    rn.k = OpK::Reduce;
+    rn.in = {win, init};
+    rn.red = red;
+    for (int d = 0; d < r; ++d) rn.a0.push_back(d);
+    rn.ty = out;
+    return g.add(rn);
+  }
+
+  struct ConvDims { int d0 = -1, d1 = -1; std::vector<int> sp; };
+  // "[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]": position of the two named roles and of every spatial dim
+  static void parse_conv_dims(const std::string& text, ConvDims out[3]) {
+    size_t pos = 0;
+    const char* names[3] = {"bf", "oi", "bf"};
+    for (int which = 0; which < 3; ++which) {
+      size_t b = text.find('[', pos), e = text.find(']', b);
+      if (b == std::string::npos || e == std::string::npos) fail("convolution: malformed dimension numbers '" + text + "'");
+      std::vector<std::string> toks;
+      std::stringstream ss(text.substr(b + 1, e - b - 1));
+      std::string tok;
+      while (std::getline(ss, tok, ',')) {
+        std::string t;
+        for (char ch : tok) if (!isspace((unsigned char)ch)) t += ch;
+        toks.push_back(t);
+      }
+      if (toks.size() < 2) fail("convolution: malformed dimension numbers '" + text + "'");
+      out[which].sp.assign(toks.size() - 2, -1);
+      for (size_t k = 0; k < toks.size(); ++k) {
+        if (toks[k].size() == 1 && toks[k][0] == names[which][0]) out[which].d0 = (int)k;
+        else if (toks[k].size() == 1 && toks[k][0] == names[which][1]) out[which].d1 = (int)k;
+        else {
+          int64_t v = -1;
+          try { v = std::stoll(toks[k]); } catch (...) { v = -1; }
+          if (v < 0 || v >= (int64_t)out[which].sp.size() || out[which].sp[v] >= 0) fail("convolution: malformed dimension numbers '" + text + "'");
+          out[which].sp[v] = (int)k;
+        }
+      }
+      if (out[which].d0 < 0 || out[which].d1 < 0) fail("convolution: malformed dimension numbers '" + text + "'");
+      for (int v : out[which].sp) if (v < 0) fail("convolution: malformed dimension numbers '" + text + "'");
+      pos = e + 1;
+    }
+  }
+
+  // convolution (reference src/Ops.jl:1000-1073; NNlib's conv, ext/ReactantNNlibExt/Implementations.jl:42-79).
+  // It becomes one matrix product on the MFMA path: the weights [O, I*taps] against the matrix of
+  // input windows [I*taps, B*outputs] (one batch entry per feature group), which a map kernel writes
+  // with coalesced reads along the minor spatial dimension of the input.
+  int build_convolution(const RawOp& o_in, int x, int w, const TType& out) {
+    RawOp o = o_in;   // window attributes are renumbered below
+    if (!o.sa.count("dim_numbers")) fail("convolution: dimension numbers missing");
+    ConvDims cd[3];
+    parse_conv_dims(o.sa.at("dim_numbers"), cd);
+    const TType xt = ty(x), wt = ty(w);
+    const int r = xt.rank(), nsp = r - 2;
+    if (nsp < 0 || wt.rank() != r || out.rank() != r) fail("convolution: operand ranks do not match");
+    for (auto& c : cd) if ((int)c.sp.size() != nsp) fail("convolution: dimension numbers do not match the rank");
+    // Number the spatial dims in the order the input stores them, so that the canonical input keeps
+    // its minor dimension (reads stay coalesced) and needs no transpose in the usual layouts.
+    {
+      std::vector<int> order(nsp);
+      for (int d = 0; d < nsp; ++d) order[d] = d;
+      std::sort(order.begin(), order.end(), [&](int p, int q) { return cd[0].sp[p] < cd[0].sp[q]; });
+      auto permute = [&](const char* key) {
+        auto itv = o.ia.find(key);
+        if (itv == o.ia.end() || (int)itv->second.size() != nsp) return;
+        std::vector<int64_t> v(nsp);
+        for (int d = 0; d < nsp; ++d) v[d] = itv->second[order[d]];
+        o.ia[key] = v;
+      };
+      for (const char* key : {"window_strides", "lhs_dilation", "rhs_dilation", "window_reversal"}) permute(key);
+      auto pv = o.ia.find("padding");
+      if (pv != o.ia.end() && (int)pv->second.size() == 2 * nsp) {
+        std::vector<int64_t> v(2 * nsp);
+        for (int d = 0; d < nsp; ++d) { v[2 * d] = pv->second[2 * order[d]]; v[2 * d + 1] = pv->second[2 * order[d] + 1]; }
+        o.ia["padding"] = v;
+      }
+      for (auto& c : cd) {
+        std::vector<int> sp(nsp);
+        for (int d = 0; d < nsp; ++d) sp[d] = c.sp[order[d]];
+        c.sp = sp;
+      }
+    }
+    if (xt.dt != wt.dt || out.dt != xt.dt) fail("convolution: operand and result element types must match");
+    auto get = [&](const char* key, int64_t dflt) {
+      std::vector<int64_t> v = o.ia.count(key) ? o.ia.at(key) : std::vector<int64_t>(nsp, dflt);
+      if (v.empty()) v.assign(nsp, dflt);
+      if ((int)v.size() != nsp) fail(std::string("convolution: ") + key + " must have one entry per spatial dimension");
+      return v;
+    };
+    const auto st = get("window_strides", 1), ld = get("lhs_dilation", 1), rd = get("rhs_dilation", 1), rev = get("window_reversal", 0);
+    std::vector<int64_t> pad = o.ia.count("padding") ? o.ia.at("padding") : std::vector<int64_t>(2 * nsp, 0);
+    if (pad.size() == 1) pad.assign(2 * nsp, pad[0]);
+    if ((int)pad.size() != 2 * nsp) fail("convolution: padding must be a (spatial rank x 2) matrix");
+    const int64_t G = o.ia.count("feature_group_count") && !o.ia.at("feature_group_count").empty() ? o.ia.at("feature_group_count")[0] : 1;
+    const int64_t BG = o.ia.count("batch_group_count") && !o.ia.at("batch_group_count").empty() ? o.ia.at("batch_group_count")[0] : 1;
+    if (BG != 1) fail("convolution: batch_group_count other than 1 is not supported");
+    if (G < 1) fail("convolution: feature_group_count must be positive");
+
+    // canonical orders: input [b, f, s...], kernel [o, i, k...]
+    auto canon = [&](int node, const ConvDims& c) {
+      std::vector<int64_t> perm{c.d0, c.d1};
+      for (int v : c.sp) perm.push_back(v);
+      bool identity = true;
+      for (size_t k = 0; k < perm.size(); ++k) identity = identity && perm[k] == (int64_t)k;
+      if (identity) return node;
+      const TType t = ty(node);
+      Node n;
+      n.k = OpK::Transpose;
+      n.in = {node};
+      n.a0 = perm;
+      n.ty.dt = t.dt;
+      for (auto pdim : perm) n.ty.dims.push_back(t.dims[pdim]);
+      return g.add(n);
+    };
+    int xc = canon(x, cd[0]);
+    int wc = canon(w, cd[1]);
+    {
+      std::vector<int64_t> rdims;
+      for (int d = 0; d < nsp; ++d) if (rev[d]) rdims.push_back(2 + d);
+      if (!rdims.empty()) {
+        Node n;
+        n.k = OpK::Reverse;
+        n.in = {wc};
+        n.ty = ty(wc);
+        n.a0 = rdims;
+        wc = g.add(n);
+      }
+    }
+    const TType xct = ty(xc), wct = ty(wc);
+    const int64_t B = xct.dims[0], C = xct.dims[1], O = wct.dims[0], I = wct.dims[1];
+    if (C != I * G || O % G != 0) fail("convolution: feature counts do not match feature_group_count");
+    // dilate and pad the input
+    {
+      std::vector<int64_t> lo(r, 0), hi(r, 0), interior(r, 0);
+      bool any = false;
+      for (int d = 0; d < nsp; ++d) {
+        lo[2 + d] = pad[2 * d]; hi[2 + d] = pad[2 * d + 1]; interior[2 + d] = ld[d] - 1;
+        if (lo[2 + d] < 0 || hi[2 + d] < 0 || ld[d] < 1) fail("convolution: negative padding is not supported");
+        any = any || lo[2 + d] || hi[2 + d] || interior[2 + d];
+      }
+      if (any) {
+        Node pn;
+        pn.k = OpK::Pad;
+        pn.in = {xc, zero_of(xct.dt)};
+        pn.a0 = lo; pn.a1 = hi; pn.a2 = interior;
+        pn.ty.dt = xct.dt;
+        for (int d = 0; d < r; ++d) pn.ty.dims.push_back(lo[d] + hi[d] + xct.dims[d] + std::max<int64_t>(xct.dims[d] - 1, 0) * interior[d]);
+        xc = g.add(pn);
+      }
+    }
+    std::vector<int64_t> wsz{1, 1}, wst{1, 1}, wdl{1, 1};
+    int64_t taps = 1;
+    for (int d = 0; d < nsp; ++d) { wsz.push_back(wct.dims[2 + d]); wst.push_back(st[d]); wdl.push_back(rd[d]); taps *= wct.dims[2 + d]; }
+    const int win = window_view(xc, wsz, wst, wdl, "convolution");     // [1, 1, k..., B, C, o...]
+    const TType wint = ty(win);
+    std::vector<int64_t> osp(wint.dims.begin() + r + 2, wint.dims.end());
+    int64_t P = 1;
+    for (auto v : osp) P *= v;
+    // expected result shape
+    {
+      std::vector<int64_t> want(r);
+      want[cd[2].d0] = B; want[cd[2].d1] = O;
+      for (int d = 0; d < nsp; ++d) want[cd[2].sp[d]] = osp[d];
+      if (want != out.dims) fail("convolution: result shape mismatch");
+    }
+    if (out.numel() == 0 || taps * I == 0) {
+      // nothing to contract or nothing to produce: zeros
+      Node bz;
+      bz.k = OpK::BroadcastInDim;
+      bz.in = {zero_of(out.dt)};
+      bz.ty = out;
+      return g.add(bz);
+    }
+    // [k..., B, C, o...] -> [C, k..., B, o...]: rows of the window matrix are (feature, tap), columns (batch entry, output)
+    std::vector<int64_t> d1(wint.dims.begin() + 2, wint.dims.end());
+    int cur = add_node(OpK::Reshape, TType{xct.dt, d1}, {win});
+    {
+      Node t;
+      t.k = OpK::Transpose;
+      t.in = {cur};
+      t.a0.push_back(nsp + 1);
+      for (int d = 0; d < nsp; ++d) t.a0.push_back(d);
+      t.a0.push_back(nsp);
+      for (int d = 0; d < nsp; ++d) t.a0.push_back(nsp + 2 + d);
+      t.ty.dt = xct.dt;
+      for (auto pdim : t.a0) t.ty.dims.push_back(d1[pdim]);
+      cur = g.add(t);
+    }
+    // The MFMA skeletons read 16-byte vectors along the contracted dimension of the weights and along
+    // the columns of the window matrix: both are padded with zeros to whole vectors (the extra
+    // columns are sliced off the product).
+    const int64_t K = I * taps, N = B * P;
+    int64_t Kp = K, Np = N;
+    if (xct.dt == DT::F32 || xct.dt == DT::BF16 || xct.dt == DT::F16) {
+      const int64_t ve = 16 / info(xct.dt).size;
+      Kp = (K + ve - 1) / ve * ve;
+      Np = (N + ve - 1) / ve * ve;
+    }
+    auto padded = [&](int node, std::vector<int64_t> hi) {
+      bool any = false;
+      for (auto v : hi) any = any || v != 0;
+      if (!any) return node;
+      const TType t = ty(node);
+      Node pn;
+      pn.k = OpK::Pad;
+      pn.in = {node, zero_of(t.dt)};
+      pn.a0.assign(t.rank(), 0);
+      pn.a1 = hi;
+      pn.a2.assign(t.rank(), 0);
+      pn.ty.dt = t.dt;
+      for (int d = 0; d < t.rank(); ++d) pn.ty.dims.push_back(t.dims[d] + hi[d]);
+      return g.add(pn);
+    };
+    Node dot;
+    dot.k = OpK::DotGeneral;
+    int lhs, rhs;
+    if (G == 1) {
+      lhs = padded(add_node(OpK::Reshape, TType{xct.dt, {O, K}}, {wc}), {0, Kp - K});
+      rhs = padded(add_node(OpK::Reshape, TType{xct.dt, {K, N}}, {cur}), {Kp - K, Np - N});
+      dot.a2 = {1}; dot.a3 = {0};
+      dot.ty = TType{out.dt, {O, Np}};
+    } else {
+      lhs = padded(add_node(OpK::Reshape, TType{xct.dt, {G, O / G, K}}, {wc}), {0, 0, Kp - K});
+      rhs = padded(add_node(OpK::Reshape, TType{xct.dt, {G, K, N}}, {cur}), {0, Kp - K, Np - N});
+      dot.a0 = {0}; dot.a1 = {0}; dot.a2 = {2}; dot.a3 = {1};
+      dot.ty = TType{out.dt, {G, O / G, Np}};
+    }
+    dot.in = {lhs, rhs};
+    cur = g.add(dot);
+    if (Np != N) {
+      Node sl;
+      sl.k = OpK::Slice;
+      sl.in = {cur};
+      const TType t = ty(cur);
+      sl.a0.assign(t.rank(), 0);
+      sl.a1 = t.dims;
+      sl.a1.back() = N;
+      sl.a2.assign(t.rank(), 1);
+      sl.ty = t;
+      sl.ty.dims.back() = N;
+      cur = g.add(sl);
+    }
+    // [O, B, o...] -> the result's own dimension order
+    std::vector<int64_t> obd{O, B};
+    for (auto v : osp) obd.push_back(v);
+    std::vector<int64_t> perm(r);
+    perm[cd[2].d0] = 1; perm[cd[2].d1] = 0;
+    for (int d = 0; d < nsp; ++d) perm[cd[2].sp[d]] = 2 + d;
+    bool same_order = true;   // dims of more than one element keep their order: a reshape is enough
+    {
+      int64_t last = -1;
+      for (int k = 0; k < r; ++k)
+        if (obd[perm[k]] != 1) { same_order = same_order && perm[k] > last; last = perm[k]; }
+    }
+    if (same_order) {
+      cur = add_node(OpK::Reshape, out, {cur});
+    } else {
+      cur = add_node(OpK::Reshape, TType{out.dt, obd}, {cur});
+      Node t;
+      t.k = OpK::Transpose;
+      t.in = {cur};
+      t.a0 = perm;
+      t.ty = out;
+      cur = g.add(t);
+    }
+    if (!(ty(cur) == out)) fail("convolution: internal shape error");
+    return cur;
+  }
+
   std::vector<int> build(const RawOp& o, const std::vector<int>& in, int depth) {
     std::string sh = o.name;
     if (sh.rfind("stablehlo.", 0) == 0) sh = sh.substr(10);
@@ -1330,6 +1785,23 @@ struct Builder {
       if (kept != n.ty.dims) fail("reduce: result shape mismatch");
       if (ty(in[1]).rank() != 0) fail("reduce: init must be 0-d");
       return {g.add(n)};
+    }
+    if (sh == "reverse") {
+      need(1);
+      n.k = OpK::Reverse;
+      n.ty = out1();
+      check_same(n.ty, ty(in[0]), o.name);
+      n.a0 = o.ia.at("dimensions");
+      for (auto d : n.a0) if (d < 0 || d >= n.ty.rank()) fail("reverse: dimension out of range");
+      return {g.add(n)};
+    }
+    if (sh == "reduce_window") {
+      if (in.size() != 2) fail("variadic reduce_window is not supported");
+      return {build_reduce_window(o, in[0], in[1], out1())};
+    }
+    if (sh == "convolution") {
+      need(2);
+      return {build_convolution(o, in[0], in[1], out1())};
     }
     if (sh == "map") {
       // elementwise application of a scalar body: inline the body on full tensors

@@ -33,7 +33,7 @@ using Ctx = std::pair<int, std::string>;
 bool is_index_op(OpK k) {
   switch (k) {
     case OpK::BroadcastInDim: case OpK::Reshape: case OpK::Transpose: case OpK::Slice: case OpK::Pad:
-    case OpK::DynamicUpdateSlice: case OpK::DynamicSlice: case OpK::Concatenate:
+    case OpK::DynamicUpdateSlice: case OpK::DynamicSlice: case OpK::Concatenate: case OpK::Reverse: case OpK::Window:
       return true;
     default:
       return false;
@@ -117,6 +117,7 @@ struct Planner {
   std::vector<int> buf_of;          // node -> buffer id (materialized nodes)
   std::map<int, int> fuse_prev;     // stencil root -> the stencil step it evaluates in LDS instead of reading from memory
   std::set<int> lds_only;           // the steps absorbed that way: no launch, no buffer
+  std::map<int, int> reshape_alias; // materialized reshape of a materialized value: the same bytes, no launch
   std::ostringstream src;
   int kcount = 0;
 
@@ -337,7 +338,7 @@ struct Planner {
       st.pop_back();
       if (!seen.insert(x).second) continue;
       const Node& n = g.nodes[x];
-      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::DotGeneral) continue;
+      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral) continue;
       if (n.k == OpK::Constant) continue;
       if (x != id && prev_mat[x]) continue;
       if (is_arith(n.k)) cost += (n.k == OpK::Unary || n.k == OpK::Gelu) ? 2 : 1;
@@ -355,7 +356,7 @@ struct Planner {
       if (!seen.insert(x).second || seen.size() > 64) continue;
       const Node& n = g.nodes[x];
       if (n.k == OpK::DotGeneral) return true;
-      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce) continue;
+      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan) continue;
       if (x != id && prev_mat[x]) continue;
       for (int i : n.in) st.push_back(i);
     }
@@ -387,7 +388,7 @@ struct Planner {
       const Node& n = g.nodes[x];
       // contexts in which x is evaluated
       std::set<Ctx> U;
-      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::DotGeneral ||
+      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral ||
                     (n.k == OpK::Constant && !n.splat);
       for (int u : users[x]) {
         const Node& un = g.nodes[u];
@@ -428,7 +429,7 @@ struct Planner {
             if (!(cn.k == OpK::Convert || cn.k == OpK::Unary)) break;
             int p = cn.in[0];
             const Node& pn = g.nodes[p];
-            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce) break;
+            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce || pn.k == OpK::Scan) break;
             if (users[p].size() != 1 || is_result[p]) break;
             cur = p;
             if (info(pn.ty.dt).size < info(g.nodes[best].ty.dt).size) best = cur;
@@ -448,6 +449,10 @@ struct Planner {
   // ------------------------------------------------------------------ buffers
   int buffer_for(int node) {
     if (buf_of[node] >= 0) return buf_of[node];
+    {
+      auto al = reshape_alias.find(node);
+      if (al != reshape_alias.end()) return buf_of[node] = buffer_for(al->second);
+    }
     const Node& n = g.nodes[node];
     BufferDesc b;
     b.ty = n.ty;
@@ -540,6 +545,9 @@ struct Planner {
         case OpK::DynamicUpdateSlice: nm = "dynamic_update_slice"; break;
         case OpK::DynamicSlice: nm = "dynamic_slice"; break;
         case OpK::Concatenate: nm = "concatenate"; break;
+        case OpK::Reverse: nm = "reverse"; break;
+        case OpK::Window: nm = "window"; break;
+        case OpK::Scan: nm = "scan"; break;
         case OpK::Reduce: nm = "reduce"; break;
         case OpK::DotGeneral: nm = "dot_general"; break;
         case OpK::Iota: nm = "iota"; break;
@@ -671,7 +679,7 @@ struct Planner {
   bool probe_stencil(int root, StencilProbe* sp) {
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
-    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::DotGeneral) return false;
+    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::Scan || rn.k == OpK::DotGeneral) return false;
     sp->vec = pick_vec(rn.ty);
     if (rn.ty.numel() < opt.slab_min_numel || sp->vec < 2) return false;
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
@@ -1910,6 +1918,201 @@ struct Planner {
     plan.launches.push_back(L2);
   }
 
+  // ------------------------------------------------------------------ prefix scans
+  // Inclusive prefix combine along one dimension (what cumsum / cumprod / cummax arrive as).  The
+  // scanned dimension is cut into chunks; a first kernel reduces every chunk, the scan kernel
+  // starts each chunk from the combination of the chunk totals before it.  Along the minor
+  // dimension a workgroup scans a chunk in tiles of 1024 elements (4 per lane, wavefront scan,
+  // wavefront totals through LDS); along any other dimension a thread walks its chunk and the
+  // lanes lie along the minor dimension, so both forms read and write coalesced.
+  void emit_scan(int root) {
+    const Node& rn = g.nodes[root];
+    const TType& ty = rn.ty;
+    const DT dt = ty.dt;
+    const int a = (int)rn.a0[0];
+    const bool rev = rn.a1[0] != 0;
+    const std::string ACC = acc_ctype(dt);
+    const std::string OP = red_functor(rn.red);
+    const std::string IDENT = red_identity(rn.red, dt);
+    const int64_t n = ty.dims[a];
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < a; ++d) outer *= ty.dims[d];
+    for (int d = a + 1; d < ty.rank(); ++d) inner *= ty.dims[d];
+    // short rows are walked by one thread each (a row is a few cache lines, all of them used)
+    const bool rowwise = inner == 1 && n >= 256 && outer * ((n + 4095) / 4096) < ((int64_t)1 << 31);
+    Emitter em(g, [&](int x) { return mat[x]; });
+    em.excess_precision = opt.excess_precision;
+    em.idx64 = needs64(cone_nodes(rn.in[0])) || ty.numel() >= ((int64_t)1 << 31);
+    const std::string it = em.idx_t();
+    em.set_root({}, {}, false);
+    Index ix(ty.rank());
+    for (int d = 0; d < ty.rank(); ++d) {
+      ix[d].var = d == a ? std::string("j") : (d < a ? "o" : "q") + std::to_string(d);
+      ix[d].hi = ty.dims[d] - 1;
+    }
+    em.indent = rowwise ? 8 : 4;
+    const std::string val = em.emit(rn.in[0], ix);
+    const std::string body = em.take_code();
+    em.indent = 2;
+    const std::string initv = em.emit(rn.in[1], Index{});
+    const std::string ibody = em.take_code();
+    const std::string ost = info(dt).stype;
+    const std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
+    const std::string jexpr = rev ? std::to_string(n - 1) + " - p" : std::string("p");
+    auto decompose = [&](std::ostringstream& o, const std::string& var, int d0, int d1) {
+      o << "  " << it << " rr_" << var << " = " << var << ";\n";
+      for (int d = d1 - 1; d >= d0; --d) {
+        o << "  const " << it << " " << (d < a ? "o" : "q") << d << " = rr_" << var << " % " << ty.dims[d] << ";\n";
+        o << "  rr_" << var << " /= " << ty.dims[d] << ";\n";
+      }
+      o << "  (void)rr_" << var << ";\n";
+    };
+    std::ostringstream o;
+    Launch L1, L2;
+    int64_t NC = 1, CH = n;
+    if (rowwise) {
+      constexpr int V = 4, TILE = kBlock * V;
+      NC = std::max<int64_t>(1, std::min<int64_t>((n + 4 * TILE - 1) / (4 * TILE), std::max<int64_t>(1, 2048 / std::max<int64_t>(outer, 1))));
+      CH = ((n + NC - 1) / NC + TILE - 1) / TILE * TILE;
+      NC = (n + CH - 1) / CH;
+      auto head = [&](const std::string& kname, bool with_tot, bool with_out) {
+        std::string sg = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + kname + "(";
+        bool first = true;
+        for (size_t k = 0; k < em.inputs.size(); ++k) {
+          sg += (first ? "" : ", ") + ptr_decl(info(g.nodes[em.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k));
+          first = false;
+        }
+        if (with_tot) { sg += (first ? "" : ", ") + ptr_decl(ACC, with_out, "tot"); first = false; }
+        if (with_out) sg += (first ? "" : ", ") + ptr_decl(ost, false, "out0");
+        return sg + ")";
+      };
+      auto prologue = [&](std::ostringstream& oo) {
+        oo << "  const " << it << " c = (" << it << ")(blockIdx.x % " << NC << "u), row = (" << it << ")(blockIdx.x / " << NC << "u);\n";
+        decompose(oo, "row", 0, a);
+        for (int d = a + 1; d < ty.rank(); ++d) oo << "  const " << it << " q" << d << " = 0;\n";
+        oo << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << CH << ", " << n << ");\n";
+      };
+      o << "// scan along the minor dimension of " << ty.str() << " (" << NC << " chunk" << (NC > 1 ? "s" : "") << " per row): " << describe(rn.in[0]) << "\n";
+      if (NC > 1) {
+        o << head("@K@_scan_totals", true, false) << " {\n";
+        o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
+        prologue(o);
+        o << "  " << ACC << " acc = " << IDENT << ";\n";
+        o << "  for (" << it << " pb = c * " << CH << " + (" << it << ")threadIdx.x * " << V << "; pb < pend; pb += " << TILE << ") {\n";
+        o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+        o << "        const " << it << " j = " << jexpr << ";\n" << body;
+        o << "        acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n      }\n    }\n  }\n";
+        o << "  acc = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(acc, " << OP << ", lds);\n";
+        o << "  if (threadIdx.x == 0) tot[row * " << NC << " + c] = acc;\n}\n\n";
+      }
+      o << head("@K@_scan", NC > 1, true) << " {\n";
+      o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n  __shared__ " << ACC << " wsum[" << kBlock / 64 << "];\n";
+      prologue(o);
+      o << ibody;
+      o << "  " << ACC << " carry = " << IDENT << ";\n";
+      o << "  if (c == 0) carry = (" << ACC << ")" << initv << ";\n";
+      if (NC > 1) {
+        o << "  {\n    " << ACC << " part = " << IDENT << ";\n";
+        o << "    for (" << it << " s = threadIdx.x; s < c; s += " << kBlock << ") part = " << red_apply(rn.red, dt, "part", "tot[row * " + std::to_string(NC) + " + s]") << ";\n";
+        o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
+        o << "    if (c != 0) carry = " << red_apply(rn.red, dt, "(" + ACC + ")" + initv, "part") << ";\n  }\n";
+      } else {
+        o << "  (void)lds;\n";
+      }
+      o << "  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;\n";
+      o << "  for (" << it << " tb = c * " << CH << "; tb < pend; tb += " << TILE << ") {\n";
+      o << "    const " << it << " pb = tb + (" << it << ")threadIdx.x * " << V << ";\n";
+      o << "    " << ACC << " v[" << V << "];\n";
+      o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      v[l] = " << IDENT << ";\n      if (p < pend) {\n";
+      o << "        const " << it << " j = " << jexpr << ";\n" << body;
+      o << "        v[l] = (" << ACC << ")" << val << ";\n      }\n    }\n";
+      o << "#pragma unroll\n    for (int l = 1; l < " << V << "; ++l) v[l] = " << red_apply(rn.red, dt, "v[l - 1]", "v[l]") << ";\n";
+      o << "    const " << ACC << " incl = rx_wave_scan(v[" << V - 1 << "], " << OP << ");\n";
+      o << "    __syncthreads();\n    if (lane == 63) wsum[w] = incl;\n    __syncthreads();\n";
+      o << "    " << ACC << " pre = carry;\n    " << ACC << " total = wsum[0];\n";
+      o << "#pragma unroll\n    for (int i = 0; i < " << kBlock / 64 << "; ++i) {\n      if (i < w) pre = " << red_apply(rn.red, dt, "pre", "wsum[i]") << ";\n";
+      o << "      if (i > 0) total = " << red_apply(rn.red, dt, "total", "wsum[i]") << ";\n    }\n";
+      o << "    const " << ACC << " below = rx_lane_from(incl, (rx_u32)(lane - 1) & 63u);\n";
+      o << "    if (lane > 0) pre = " << red_apply(rn.red, dt, "pre", "below") << ";\n";
+      o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+      o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pre", "v[l]") << ";\n";
+      o << "        out0[row * " << n << " + (" << jexpr << ")] = " << Emitter::store_conv(dt, rv) << ";\n      }\n    }\n";
+      o << "    carry = " << red_apply(rn.red, dt, "carry", "total") << ";\n  }\n}\n\n";
+      L1.grid[0] = L2.grid[0] = (unsigned)(NC * outer);
+    } else {
+      const int64_t lines = outer * inner;
+      NC = std::max<int64_t>(1, std::min<int64_t>(65536 / std::max<int64_t>(lines, 1), n / 16));
+      CH = (n + NC - 1) / NC;
+      NC = (n + CH - 1) / CH;
+      auto head = [&](const std::string& kname, bool with_tot, bool with_out) {
+        std::string sg = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + kname + "(";
+        bool first = true;
+        for (size_t k = 0; k < em.inputs.size(); ++k) {
+          sg += (first ? "" : ", ") + ptr_decl(info(g.nodes[em.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k));
+          first = false;
+        }
+        if (with_tot) { sg += (first ? "" : ", ") + ptr_decl(ACC, with_out, "tot"); first = false; }
+        if (with_out) sg += (first ? "" : ", ") + ptr_decl(ost, false, "out0");
+        return sg + ")";
+      };
+      // thread id -> (outer index, chunk, inner index); the inner index is the fastest
+      auto prologue = [&](std::ostringstream& oo) {
+        oo << "  const " << it << " tid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+        oo << "  if (tid >= " << lines * NC << ") return;\n";
+        oo << "  const " << it << " qi = tid % " << inner << ";\n";
+        oo << "  const " << it << " c = (tid / " << inner << ") % " << NC << ";\n";
+        oo << "  const " << it << " oi = tid / " << inner * NC << ";\n";
+        decompose(oo, "qi", a + 1, ty.rank());
+        decompose(oo, "oi", 0, a);
+        oo << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << CH << ", " << n << ");\n";
+      };
+      o << "// scan along dimension " << a << " of " << ty.str() << " (" << NC << " chunk" << (NC > 1 ? "s" : "") << " per line): " << describe(rn.in[0]) << "\n";
+      if (NC > 1) {
+        o << head("@K@_scan_totals", true, false) << " {\n";
+        prologue(o);
+        o << "  " << ACC << " acc = " << IDENT << ";\n";
+        o << "  for (" << it << " p = c * " << CH << "; p < pend; ++p) {\n";
+        o << "    const " << it << " j = " << jexpr << ";\n" << body;
+        o << "    acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n  }\n";
+        o << "  tot[(oi * " << NC << " + c) * " << inner << " + qi] = acc;\n}\n\n";
+      }
+      o << head("@K@_scan", NC > 1, true) << " {\n";
+      prologue(o);
+      o << ibody;
+      o << "  " << ACC << " acc = (" << ACC << ")" << initv << ";\n";
+      if (NC > 1)
+        o << "  for (" << it << " s = 0; s < c; ++s) acc = " << red_apply(rn.red, dt, "acc", "tot[(oi * " + std::to_string(NC) + " + s) * " + std::to_string(inner) + " + qi]") << ";\n";
+      o << "  for (" << it << " p = c * " << CH << "; p < pend; ++p) {\n";
+      o << "    const " << it << " j = " << jexpr << ";\n" << body;
+      o << "    acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n";
+      o << "    const " << ACC << " r = acc;\n";
+      o << "    out0[(oi * " << n << " + j) * " << inner << " + qi] = " << Emitter::store_conv(dt, rv) << ";\n  }\n}\n\n";
+      L1.grid[0] = L2.grid[0] = (unsigned)((lines * NC + kBlock - 1) / kBlock);
+    }
+    const std::string kb_final = finalize(o.str());
+    int sc = -1;
+    if (NC > 1) {
+      sc = scratch(outer * inner * NC * (int64_t)(ACC == "double" || info(dt).size == 8 ? 8 : 4));
+      L1.kernel = named("@K@_scan_totals", kb_final);
+      L1.kind = "scan_totals";
+      L1.block[0] = kBlock;
+      for (int i : em.inputs) L1.args.push_back(buffer_for(i));
+      L1.args.push_back(sc);
+      L1.algo_bytes = algo_bytes(em.inputs, {});
+      L1.desc = describe(rn.in[0]) + " chunk totals";
+      plan.launches.push_back(L1);
+    }
+    L2.kernel = named("@K@_scan", kb_final);
+    L2.kind = "scan";
+    L2.block[0] = kBlock;
+    for (int i : em.inputs) L2.args.push_back(buffer_for(i));
+    if (NC > 1) L2.args.push_back(sc);
+    L2.args.push_back(buffer_for(root));
+    L2.algo_bytes = algo_bytes(em.inputs, {root});
+    L2.desc = describe(rn.in[0]) + " scan";
+    plan.launches.push_back(L2);
+  }
+
   // ------------------------------------------------------------------ row groups
   // `root` is either a Reduce over the trailing dims (plain row reduction) or an
   // elementwise node of shape [rows.., cols] whose cone contains row reductions `phases`.
@@ -2338,7 +2541,7 @@ struct Planner {
       const Ctx& c = *ctx[x].begin();
       if (!c.second.empty()) continue;
       const Node& r = g.nodes[c.first];
-      if (r.k == OpK::Reduce || r.k == OpK::DotGeneral) continue;
+      if (r.k == OpK::Reduce || r.k == OpK::Scan || r.k == OpK::DotGeneral) continue;
       if (r.ty.dims != g.nodes[x].ty.dims) continue;
       // the root must not be the anchor of a row group (its reductions need the full row)
       if (!row_phases(c.first).empty()) continue;
@@ -2347,6 +2550,29 @@ struct Planner {
     std::set<int> absorbed_roots;
     for (auto& kv : epilogue_of) absorbed_roots.insert(kv.second);
     std::set<int> fused_reduces;
+
+    // A reshape that must own a buffer and reads a value that owns one is the same bytes in the same
+    // (row-major) order: it shares that buffer and costs no launch.  A result may share only a
+    // temporary of this module that nothing else returns.
+    {
+      std::vector<char> is_result(N, 0);
+      for (int r : g.results) is_result[r] = 1;
+      std::set<int> returned_bases;
+      for (int x = 0; x < N; ++x) {
+        if (!live[x] || !mat[x]) continue;
+        const Node& n = g.nodes[x];
+        if (n.k != OpK::Reshape || absorbed_roots.count(x)) continue;
+        int base = n.in[0];
+        if (!mat[base]) continue;
+        while (reshape_alias.count(base)) base = reshape_alias[base];
+        if (is_result[x]) {
+          const Node& bn = g.nodes[base];
+          if (bn.k == OpK::Param || bn.k == OpK::Constant || is_result[base] || returned_bases.count(base)) continue;
+          returned_bases.insert(base);
+        }
+        reshape_alias[x] = base;
+      }
+    }
 
     // kernels in topological order of their roots
     std::vector<std::pair<int, std::function<void()>>> jobs;
@@ -2366,6 +2592,11 @@ struct Planner {
         jobs.push_back({x, [this, x, dot] { emit_dot(x, dot); }});
         continue;
       }
+      if (n.k == OpK::Scan) {
+        jobs.push_back({x, [this, x] { emit_scan(x); }});
+        continue;
+      }
+      if (reshape_alias.count(x)) continue;
       if (n.k == OpK::Reduce) {
         jobs.push_back({x, [this, x, &fused_reduces] {
           if (fused_reduces.count(x)) return;
@@ -2393,7 +2624,8 @@ struct Planner {
       auto plain_map_root = [&](int x) {
         const Node& n = g.nodes[x];
         if (!live[x] || !mat[x]) return false;
-        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::DotGeneral) return false;
+        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral) return false;
+        if (reshape_alias.count(x)) return false;
         if (absorbed_roots.count(x) || !row_phases(x).empty()) return false;
         return true;
       };
@@ -2415,7 +2647,7 @@ struct Planner {
     // row groups claim their reductions before those would be emitted on their own
     for (auto& j : jobs) {
       const Node& n = g.nodes[j.first];
-      if (n.k != OpK::Reduce && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
+      if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
         for (int p : row_phases(j.first)) fused_reduces.insert(p);
     }
     for (auto& j : jobs) j.second();

@@ -1,0 +1,138 @@
+"""Module text for windowed ops in the forms the reference prints them: `stablehlo.reduce_window`
+(generic form; built by src/Ops.jl:3967-4011 for pooling, ext/ReactantNNlibExt/Ops.jl:1-32, and for
+cumsum/cumprod, src/TracedRArray.jl:1086-1108), `stablehlo.convolution` (src/Ops.jl:1000-1073) and
+`stablehlo.reverse` (kernel flip, ext/ReactantNNlibExt/Implementations.jl:53-55)."""
+
+INIT = {("add", True): "0.000000e+00", ("multiply", True): "1.000000e+00", ("maximum", True): "0xFF800000",
+        ("minimum", True): "0x7F800000", ("add", False): "0", ("multiply", False): "1"}
+
+
+def tt(shape, dt):
+    return "tensor<" + "".join("%dx" % d for d in shape) + dt + ">"
+
+
+def _init_literal(body, dt):
+    if dt.startswith("f") or dt == "bf16":
+        if body == "maximum":
+            return {"f64": "0xFFF0000000000000", "f32": "0xFF800000", "bf16": "0xFF80", "f16": "0xFC00"}[dt]
+        if body == "minimum":
+            return {"f64": "0x7FF0000000000000", "f32": "0x7F800000", "bf16": "0x7F80", "f16": "0x7C00"}[dt]
+        return INIT[(body, True)]
+    if body == "maximum":
+        return {"i32": "-2147483648", "i64": "-9223372036854775808"}[dt]
+    if body == "minimum":
+        return {"i32": "2147483647", "i64": "9223372036854775807"}[dt]
+    return INIT[(body, False)]
+
+
+def window_out_shape(shape, window, strides, padding, base_dil, win_dil):
+    out = []
+    for d, n in enumerate(shape):
+        dil = n + max(n - 1, 0) * (base_dil[d] - 1)
+        padded = dil + padding[d][0] + padding[d][1]
+        span = (window[d] - 1) * win_dil[d] + 1
+        out.append(0 if padded < span else (padded - span) // strides[d] + 1)
+    return out
+
+
+def reduce_window(shape, dt, body, window, strides=None, padding=None, base_dil=None, win_dil=None):
+    r = len(shape)
+    strides = strides or [1] * r
+    padding = padding or [[0, 0]] * r
+    base_dil = base_dil or [1] * r
+    win_dil = win_dil or [1] * r
+    out = window_out_shape(shape, window, strides, padding, base_dil, win_dil)
+    arr = lambda v: "array<i64: " + ", ".join(str(x) for x in v) + ">"
+    pad = "dense<[" + ", ".join("[%d, %d]" % (p[0], p[1]) for p in padding) + "]> : tensor<%dx2xi64>" % r
+    ti, to, ts = tt(shape, dt), tt(out, dt), tt([], dt)
+    return ("module {\n  func.func @main(%%arg0: %s) -> %s {\n"
+            "    %%cst = stablehlo.constant dense<%s> : %s\n"
+            "    %%0 = \"stablehlo.reduce_window\"(%%arg0, %%cst) <{base_dilations = %s, padding = %s, "
+            "window_dilations = %s, window_dimensions = %s, window_strides = %s}> ({\n"
+            "    ^bb0(%%arg1: %s, %%arg2: %s):\n"
+            "      %%1 = stablehlo.%s %%arg1, %%arg2 : %s\n"
+            "      stablehlo.return %%1 : %s\n"
+            "    }) : (%s, %s) -> %s\n"
+            "    return %%0 : %s\n  }\n}\n"
+            % (ti, to, _init_literal(body, dt), ts, arr(base_dil), pad, arr(win_dil), arr(window), arr(strides),
+               ts, ts, body, ts, ts, ti, ts, to, to)), out
+
+
+def cumulative(shape, dt, dim, body="add", reverse=False):
+    """What Base.cumsum / cumprod of a traced array print (src/TracedRArray.jl:1086-1108)."""
+    r = len(shape)
+    window = [1] * r
+    window[dim] = shape[dim]
+    padding = [[0, 0] for _ in range(r)]
+    padding[dim] = [0, shape[dim] - 1] if reverse else [shape[dim] - 1, 0]
+    return reduce_window(shape, dt, body, window, padding=padding)[0]
+
+
+def conv_out_shape(x_sp, k_sp, strides, padding, lhs_dil, rhs_dil):
+    out = []
+    for d, n in enumerate(x_sp):
+        dil = n + max(n - 1, 0) * (lhs_dil[d] - 1)
+        padded = dil + padding[d][0] + padding[d][1]
+        span = (k_sp[d] - 1) * rhs_dil[d] + 1
+        out.append(0 if padded < span else (padded - span) // strides[d] + 1)
+    return out
+
+
+def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]", strides=None, padding=None,
+                lhs_dil=None, rhs_dil=None, groups=1, flip=False, generic=False, epilogue=None):
+    """`dims` uses the textual dimension numbers; spatial dim s of the input has the size
+    x_shape[position of s].  With `flip` the kernel's spatial dims are reversed first (NNlib's true
+    convolution).  `epilogue="bias_relu"` adds a per-feature bias and a relu, the fused form LuxLib emits."""
+    import re
+    groups_txt = re.findall(r"\[([^\]]*)\]", dims)
+    pos = []
+    for gtxt in groups_txt:
+        toks = [t.strip() for t in gtxt.split(",")]
+        pos.append({t: k for k, t in enumerate(toks)})
+    nsp = len(x_shape) - 2
+    strides = strides or [1] * nsp
+    padding = padding or [[0, 0]] * nsp
+    lhs_dil = lhs_dil or [1] * nsp
+    rhs_dil = rhs_dil or [1] * nsp
+    x_sp = [x_shape[pos[0][str(s)]] for s in range(nsp)]
+    k_sp = [w_shape[pos[1][str(s)]] for s in range(nsp)]
+    o_sp = conv_out_shape(x_sp, k_sp, strides, padding, lhs_dil, rhs_dil)
+    out = [0] * len(x_shape)
+    out[pos[2]["b"]] = x_shape[pos[0]["b"]]
+    out[pos[2]["f"]] = w_shape[pos[1]["o"]]
+    for s in range(nsp):
+        out[pos[2][str(s)]] = o_sp[s]
+    tx, tw, to = tt(x_shape, dt), tt(w_shape, dt), tt(out, dt)
+    lst = lambda v: "[" + ", ".join(str(x) for x in v) + "]"
+    body = ""
+    wname = "%arg1"
+    if flip:
+        rd = sorted(pos[1][str(s)] for s in range(nsp))
+        body += "    %%w = stablehlo.reverse %%arg1, dims = %s : %s\n" % (lst(rd), tw)
+        wname = "%w"
+    if generic:
+        arr = lambda v: "array<i64: " + ", ".join(str(x) for x in v) + ">"
+        pad = "dense<[" + ", ".join("[%d, %d]" % (p[0], p[1]) for p in padding) + "]> : tensor<%dx2xi64>" % nsp
+        body += ("    %%0 = \"stablehlo.convolution\"(%%arg0, %s) <{batch_group_count = 1 : i64, dimension_numbers = "
+                 "#stablehlo.conv<%s>, feature_group_count = %d : i64, lhs_dilation = %s, padding = %s, "
+                 "precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>], rhs_dilation = %s, "
+                 "window_strides = %s}> : (%s, %s) -> %s\n"
+                 % (wname, dims, groups, arr(lhs_dil), pad, arr(rhs_dil), arr(strides), tx, tw, to))
+    else:
+        body += ("    %%0 = stablehlo.convolution(%%arg0, %s) dim_numbers = %s, window = {stride = %s, pad = %s, "
+                 "lhs_dilate = %s, rhs_dilate = %s} {batch_group_count = 1 : i64, feature_group_count = %d : i64, "
+                 "precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>]} : (%s, %s) -> %s\n"
+                 % (wname, dims, lst(strides), "[" + ", ".join(lst(p) for p in padding) + "]", lst(lhs_dil), lst(rhs_dil),
+                    groups, tx, tw, to))
+    args = "%%arg0: %s, %%arg1: %s" % (tx, tw)
+    res = "%0"
+    if epilogue == "bias_relu":
+        nf = out[pos[2]["f"]]
+        tb = tt([nf], dt)
+        args += ", %%arg2: %s" % tb
+        body += "    %%b = stablehlo.broadcast_in_dim %%arg2, dims = [%d] : (%s) -> %s\n" % (pos[2]["f"], tb, to)
+        body += "    %%1 = stablehlo.add %%0, %%b : %s\n" % to
+        body += "    %%z = stablehlo.constant dense<0.000000e+00> : %s\n" % to
+        body += "    %%2 = stablehlo.maximum %%1, %%z : %s\n" % to
+        res = "%2"
+    return ("module {\n  func.func @main(%s) -> %s {\n%s    return %s : %s\n  }\n}\n" % (args, to, body, res, to)), out
