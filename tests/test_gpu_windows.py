@@ -1,0 +1,210 @@
+"""Windowed ops on the GPU against the oracle: reverse, reduce_window in its pooling forms (window
+view + reduction) and its cumulative forms (prefix scans), convolution (window matrix + matrix
+product).  Cases follow the reference's tests: test/core/ops.jl:609-618 (reverse),
+test/core/map_reduction.jl:165-229 (cumsum / cumprod), test/nn/convolution.jl:160-217 (groups x
+stride x padding x dilation grid, 1-d flip vectors)."""
+import numpy as np
+import pytest
+
+from _harness import gpu_run, oracle_run, max_rel_to_scale
+from oracle import stablehlo_interp as I
+import _nn_modules as NN
+
+pytestmark = pytest.mark.gpu
+
+
+def _args(shapes, dt, seed=0, lo=None):
+    rng = np.random.default_rng(seed)
+    out = []
+    for sh in shapes:
+        if dt[0] == "i":
+            out.append(I.Tensor(rng.integers(-1000, 1000, size=sh).astype(I.NP_OF[dt]), dt))
+        elif lo is not None:
+            out.append(I.tensor(rng.uniform(lo[0], lo[1], size=sh), dt))
+        else:
+            out.append(I.tensor(rng.normal(size=sh), dt))
+    return out
+
+
+def _close(got, ref, tol):
+    assert got.shape == ref.shape
+    same_inf = np.array_equal(np.isinf(got), np.isinf(ref)) and np.array_equal(np.isnan(got), np.isnan(ref))
+    assert same_inf
+    fin = np.isfinite(ref)
+    if fin.any():
+        scale = max(float(np.max(np.abs(ref[fin]))), 1e-30)
+        assert float(np.max(np.abs(got[fin].astype(np.float64) - ref[fin].astype(np.float64)))) / scale <= tol
+
+
+def test_reverse_reference_vectors(rx, client):
+    t = ("module {\n func.func @main(%arg0: tensor<4xi64>) -> tensor<4xi64> {\n"
+         "  %0 = stablehlo.reverse %arg0, dims = [0] : tensor<4xi64>\n  return %0 : tensor<4xi64>\n }\n}\n")
+    got, _ = gpu_run(rx, client, t, [I.Tensor(np.array([1, 2, 3, 4]), "i64")])
+    assert got[0].a.tolist() == [4, 3, 2, 1]
+    t2 = ("module {\n func.func @main(%arg0: tensor<3x5x4xf32>) -> tensor<3x5x4xf32> {\n"
+          "  %0 = stablehlo.reverse %arg0, dims = [0, 2] : tensor<3x5x4xf32>\n"
+          "  %1 = stablehlo.negate %0 : tensor<3x5x4xf32>\n  return %1 : tensor<3x5x4xf32>\n }\n}\n")
+    a = _args([(3, 5, 4)], "f32")
+    got, _ = gpu_run(rx, client, t2, a)
+    assert np.array_equal(got[0].a, -a[0].a[::-1, :, ::-1])
+
+
+def test_cumulative_reference_cases(rx, client):
+    a = I.tensor(np.arange(1, 11) / 10, "f32")
+    for body, lib in (("add", np.cumsum), ("multiply", np.cumprod)):
+        got, exe = gpu_run(rx, client, NN.cumulative([10], "f32", 0, body), [a])
+        assert [l["kind"] for l in exe.launches()] == ["scan"]
+        assert np.allclose(got[0].a, lib(a.a.astype(np.float64)), rtol=1e-6)
+    b = I.tensor(np.arange(1, 61).reshape(5, 4, 3) / 60, "f32")
+    for raw in range(3):
+        for body, lib in (("add", np.cumsum), ("multiply", np.cumprod)):
+            got, _ = gpu_run(rx, client, NN.cumulative([5, 4, 3], "f32", raw, body), [b])
+            assert np.allclose(got[0].a, lib(b.a.astype(np.float64), axis=raw), rtol=1e-6)
+
+
+# (shape, dtype, dim, body, from the end, launch kinds)
+SCANS = [
+    ([1 << 22], "f32", 0, "add", False, ["scan_totals", "scan"]),
+    ([100003], "f64", 0, "add", False, ["scan_totals", "scan"]),
+    ([100003], "i32", 0, "add", True, ["scan_totals", "scan"]),
+    ([512, 3000], "f32", 1, "add", False, ["scan"]),
+    ([3, 70001], "f32", 1, "maximum", True, None),
+    ([3000, 512], "f32", 0, "add", False, None),
+    ([100000, 8], "f32", 0, "add", False, ["scan_totals", "scan"]),
+    ([7, 300, 33], "f32", 1, "add", True, None),
+    ([64, 1000], "f64", 1, "multiply", True, ["scan"]),
+    ([1000, 64], "f32", 0, "minimum", False, None),
+    ([300, 1000], "i32", 1, "add", False, ["scan"]),
+    ([300, 1000], "i64", 0, "add", False, None),
+    ([100000, 10], "f32", 1, "add", False, ["scan"]),
+    ([2, 1500], "bf16", 1, "add", False, ["scan"]),
+    ([2, 300], "bf16", 0, "maximum", False, ["scan"]),
+]
+
+
+@pytest.mark.parametrize("shape,dt,dim,body,rev,kinds", SCANS)
+def test_prefix_scans(rx, client, shape, dt, dim, body, rev, kinds):
+    text = NN.cumulative(shape, dt, dim, body, rev)
+    args = _args([shape], dt, seed=7, lo=(0.98, 1.02) if body == "multiply" else None)
+    got, exe = gpu_run(rx, client, text, args)
+    got_kinds = [l["kind"] for l in exe.launches()]
+    assert set(got_kinds) <= {"scan_totals", "scan"}, got_kinds
+    if kinds is not None:
+        assert got_kinds == kinds
+    ref = oracle_run(text, args, hifi=True)
+    if dt[0] == "i" or body in ("maximum", "minimum"):
+        assert np.array_equal(got[0].a, ref[0].a)
+    elif dt == "bf16":
+        _close(got[0].a, ref[0].a, 1e-2)
+    elif dt == "f64":
+        _close(got[0].a, ref[0].a, 1e-12)
+    else:
+        _close(got[0].a, ref[0].a, 1e-5 * np.sqrt(shape[dim]))
+
+
+def test_scan_of_a_fused_producer_and_into_a_consumer(rx, client):
+    """cumsum(abs2.(x)) ./ sum: the producer is evaluated inside the scan kernels, the consumer reads its result."""
+    t = ("module {\n func.func @main(%arg0: tensor<64x5000xf32>) -> tensor<64x5000xf32> {\n"
+         "  %sq = stablehlo.multiply %arg0, %arg0 : tensor<64x5000xf32>\n"
+         "  %c = stablehlo.constant dense<0.000000e+00> : tensor<f32>\n"
+         "  %0 = \"stablehlo.reduce_window\"(%sq, %c) <{base_dilations = array<i64: 1, 1>, padding = dense<[[0, 0], [4999, 0]]> : tensor<2x2xi64>, "
+         "window_dilations = array<i64: 1, 1>, window_dimensions = array<i64: 1, 5000>, window_strides = array<i64: 1, 1>}> ({\n"
+         "  ^bb0(%a: tensor<f32>, %b: tensor<f32>):\n    %s = stablehlo.add %a, %b : tensor<f32>\n    stablehlo.return %s : tensor<f32>\n"
+         "  }) : (tensor<64x5000xf32>, tensor<f32>) -> tensor<64x5000xf32>\n"
+         "  %h = stablehlo.constant dense<5.000000e-01> : tensor<64x5000xf32>\n"
+         "  %1 = stablehlo.multiply %0, %h : tensor<64x5000xf32>\n"
+         "  return %1 : tensor<64x5000xf32>\n }\n}\n")
+    args = _args([(64, 5000)], "f32", seed=2)
+    got, exe = gpu_run(rx, client, t, args)
+    assert [l["kind"] for l in exe.launches()] == ["scan_totals", "scan", "map"]
+    ref = np.cumsum(args[0].a.astype(np.float64) ** 2, axis=1) * 0.5
+    _close(got[0].a, ref, 1e-5 * np.sqrt(5000))
+
+
+POOLS = [
+    ([8, 16, 32, 32], "f32", "maximum", [1, 1, 2, 2], [1, 1, 2, 2], None, None, None),
+    ([8, 16, 32, 32], "f32", "add", [1, 1, 2, 2], [1, 1, 2, 2], None, None, None),
+    ([2, 3, 17, 19], "f32", "add", [1, 1, 3, 3], [1, 1, 2, 2], [[0, 0], [0, 0], [1, 1], [1, 1]], None, None),
+    ([2, 3, 17, 19], "f32", "maximum", [1, 1, 3, 2], [1, 1, 1, 2], [[0, 0], [0, 0], [2, 1], [0, 3]], [1, 1, 2, 1], [1, 1, 2, 3]),
+    ([4, 6, 40], "f64", "minimum", [1, 1, 5], [1, 1, 3], [[0, 0], [0, 0], [2, 2]], None, None),
+    ([2, 4, 9, 10, 11], "f32", "maximum", [1, 1, 2, 2, 2], [1, 1, 2, 2, 2], None, None, None),
+    ([4, 4, 28, 28], "bf16", "maximum", [1, 1, 3, 3], [1, 1, 2, 2], [[0, 0], [0, 0], [1, 1], [1, 1]], None, None),
+    ([6, 50, 50], "i32", "add", [1, 3, 3], [1, 1, 1], [[0, 0], [1, 1], [1, 1]], None, None),
+]
+
+
+@pytest.mark.parametrize("shape,dt,body,window,strides,padding,bd,wd", POOLS)
+def test_pooling_windows(rx, client, shape, dt, body, window, strides, padding, bd, wd):
+    text, out_shape = NN.reduce_window(shape, dt, body, window, strides, padding, bd, wd)
+    args = _args([shape], dt, seed=11)
+    got, exe = gpu_run(rx, client, text, args)
+    assert all(l["kind"] in ("reduce_generic", "reduce_final", "row") for l in exe.launches())
+    ref = oracle_run(text, args, hifi=True)
+    assert list(got[0].a.shape) == out_shape
+    if dt[0] == "i" or body in ("maximum", "minimum"):
+        assert np.array_equal(got[0].a, ref[0].a)
+    else:
+        _close(got[0].a, ref[0].a, 1e-6 * np.prod(window))
+
+
+def test_conv_1d_flip_reference_vectors(rx, client):
+    x = I.tensor(np.array([[[1.0, 2.0, 3.0]]]), "f32")
+    for flip, want in ((False, [8.0, 14.0, 8.0]), (True, [4.0, 10.0, 12.0])):
+        for generic in (False, True):
+            text, _ = NN.convolution([1, 1, 3], [1, 1, 3], "f32", dims="[b, f, 0]x[o, i, 0]->[b, f, 0]", padding=[[1, 1]], flip=flip, generic=generic)
+            got, _ = gpu_run(rx, client, text, [x, x])
+            assert got[0].a.reshape(-1).tolist() == want
+
+
+CONV_GRID = [(g, s, p, d) for g in (1, 2, 4) for s in ((1, 1), (2, 2), (3, 3))
+             for p in ((0, 0), (2, 2), (0, 2), (2, 0)) for d in ((1, 1), (1, 2))]
+
+
+@pytest.mark.parametrize("groups", [1, 2, 4])
+def test_convolution_reference_grid(rx, client, groups):
+    """x 16x16x8x2, weight 4x4x(8/groups)x4 in Julia order, i.e. raw [2, 8, 16, 16] and [4, 8/groups, 4, 4]."""
+    xs, ws = [2, 8, 16, 16], [4, 8 // groups, 4, 4]
+    args = _args([xs, ws], "f32", seed=groups)
+    for (g, s, p, d) in CONV_GRID:
+        if g != groups:
+            continue
+        # Julia's dim 1 is the raw minor dim: spatial dim 0 sits at raw position 3
+        text, out_shape = NN.convolution(xs, ws, "f32", strides=list(s), padding=[[p[0], p[0]], [p[1], p[1]]],
+                                         rhs_dil=list(d), groups=g, flip=True)
+        got, _ = gpu_run(rx, client, text, args)
+        ref = oracle_run(text, args, hifi=True)
+        assert list(got[0].a.shape) == out_shape
+        _close(got[0].a, ref[0].a, 1e-5 * np.sqrt(8 // g * 16))
+
+
+CONVS = [
+    # x, w, dtype, dims, kwargs, expected kind of the product
+    ([4, 64, 56, 56], [64, 64, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "gemm_f32"),
+    ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
+    ([1, 3, 33, 35], [16, 3, 5, 5], "f32", None, dict(strides=[2, 2], padding=[[2, 2], [2, 2]]), "gemm_f32"),
+    ([16, 16, 8, 2], [4, 4, 8, 4], "f32", "[1, 0, f, b]x[1, 0, i, o]->[1, 0, f, b]", dict(), None),
+    ([2, 16, 16, 8], [4, 4, 8, 4], "f32", "[b, 1, 0, f]x[1, 0, i, o]->[b, 1, 0, f]", dict(padding=[[1, 2], [0, 1]]), None),
+    ([3, 5, 40], [7, 5, 3], "f32", "[b, f, 0]x[o, i, 0]->[b, f, 0]", dict(lhs_dil=[2], padding=[[2, 2]]), None),
+    ([2, 3, 8, 8, 8], [3, 3, 3, 3, 3], "f32", "[b, f, 2, 1, 0]x[o, i, 2, 1, 0]->[b, f, 2, 1, 0]", dict(padding=[[1, 1], [1, 1], [1, 1]]), None),
+    ([2, 6, 20, 20], [12, 3, 3, 3], "f64", None, dict(groups=2, generic=True), None),
+    ([8, 32, 14, 14], [32, 1, 3, 3], "f32", None, dict(groups=32, padding=[[1, 1], [1, 1]]), None),
+]
+
+
+@pytest.mark.parametrize("xs,ws,dt,dims,kw,kind", CONVS)
+def test_convolution_layouts_and_types(rx, client, xs, ws, dt, dims, kw, kind):
+    kw = dict(kw)
+    if dims:
+        kw["dims"] = dims
+    text, out_shape = NN.convolution(xs, ws, dt, **kw)
+    shapes = [xs, ws] + ([[out_shape[1]]] if kw.get("epilogue") else [])
+    args = _args(shapes, dt, seed=21)
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    if kind:
+        assert kind in kinds, kinds
+    ref = oracle_run(text, args, hifi=True)
+    assert list(got[0].a.shape) == out_shape
+    taps = int(np.prod(ws[1:])) if not dims or dims.startswith("[b, f") else int(np.prod(ws)) // max(ws)
+    tol = 1e-2 if dt == "bf16" else (1e-12 if dt == "f64" else 1e-5 * np.sqrt(taps))
+    _close(got[0].a, ref[0].a, tol)

@@ -1,0 +1,172 @@
+"""Pins for the oracle's windowed ops (reverse, reduce_window, convolution): the reference's own
+known answers, library routines and brute-force loops.  CPU only."""
+import itertools
+
+import numpy as np
+import pytest
+from scipy import signal
+
+from oracle import stablehlo_interp as I
+import _nn_modules as NN
+
+
+def run(text, arrays, dt="f32", hifi=False):
+    return I.run_text(text, [I.tensor(a, dt) if dt[0] in "fb" else I.Tensor(np.asarray(a), dt) for a in arrays], hifi=hifi)[0].a
+
+
+def test_reverse_reference_vectors():
+    """test/core/ops.jl:609-618; Julia matrices arrive with their dims reversed."""
+    t = ("module {\n func.func @main(%arg0: tensor<4xi64>) -> tensor<4xi64> {\n"
+         "  %0 = stablehlo.reverse %arg0, dims = [0] : tensor<4xi64>\n  return %0 : tensor<4xi64>\n }\n}\n")
+    assert run(t, [np.array([1, 2, 3, 4])], "i64").tolist() == [4, 3, 2, 1]
+    x = np.array([[1, 2], [3, 4]])                       # Julia [1 2; 3 4]
+    for jdim, want in ((1, [[3, 4], [1, 2]]), (2, [[2, 1], [4, 3]])):
+        raw_dim = 2 - jdim
+        t = ("module {\n func.func @main(%%arg0: tensor<2x2xi64>) -> tensor<2x2xi64> {\n"
+             "  %%0 = stablehlo.reverse %%arg0, dims = [%d] : tensor<2x2xi64>\n  return %%0 : tensor<2x2xi64>\n }\n}\n" % raw_dim)
+        got = run(t, [x.T.copy()], "i64").T
+        assert got.tolist() == want
+
+
+def test_conv_1d_flip_reference_vectors():
+    """test/nn/convolution.jl:206-217: x = W = [1, 2, 3], pad 1, flipped and not."""
+    x = np.array([[[1.0, 2.0, 3.0]]])
+    for flip, want in ((False, [0 * 1 + 1 * 2 + 2 * 3, 1 * 1 + 2 * 2 + 3 * 3, 1 * 2 + 2 * 3 + 3 * 0]),
+                       (True, [3 * 0 + 2 * 1 + 1 * 2, 3 * 1 + 2 * 2 + 1 * 3, 3 * 2 + 2 * 3 + 1 * 0])):
+        text, out = NN.convolution([1, 1, 3], [1, 1, 3], "f32", dims="[b, f, 0]x[o, i, 0]->[b, f, 0]", padding=[[1, 1]], flip=flip)
+        assert out == [1, 1, 3]
+        assert run(text, [x, x]).reshape(-1).tolist() == want
+        text, _ = NN.convolution([1, 1, 3], [1, 1, 3], "f32", dims="[b, f, 0]x[o, i, 0]->[b, f, 0]", padding=[[1, 1]], flip=flip, generic=True)
+        assert run(text, [x, x]).reshape(-1).tolist() == want
+
+
+def test_cumulative_reference_cases():
+    """test/core/map_reduction.jl:165-229: cumsum / cumprod of 1:10 ./ 10 and of a 3x4x5 array along
+    each Julia dim (raw dim = 3 - Julia dim) against numpy's accumulate."""
+    a = (np.arange(1, 11) / 10).astype(np.float32)
+    assert np.allclose(run(NN.cumulative([10], "f32", 0), [a]), np.cumsum(a), rtol=1e-6)
+    assert np.allclose(run(NN.cumulative([10], "f32", 0, "multiply"), [a]), np.cumprod(a), rtol=1e-6)
+    b = (np.arange(1, 61).reshape(5, 4, 3) / 60).astype(np.float32)      # raw view of reshape(1:60, (3, 4, 5)) ./ 60
+    for raw in range(3):
+        assert np.allclose(run(NN.cumulative([5, 4, 3], "f32", raw), [b]), np.cumsum(b, axis=raw), rtol=1e-6)
+        assert np.allclose(run(NN.cumulative([5, 4, 3], "f32", raw, "multiply"), [b]), np.cumprod(b, axis=raw), rtol=1e-6)
+
+
+def test_prefix_fast_path_equals_the_general_window_form():
+    rng = np.random.default_rng(0)
+    for shape, dim, body, rev in (([37], 0, "add", False), ([6, 11], 0, "maximum", True), ([6, 11], 1, "multiply", False),
+                                  ([3, 5, 4], 1, "minimum", True), ([9, 2], 0, "add", True)):
+        x = rng.uniform(0.5, 1.5, size=shape)
+        text = NN.cumulative(shape, "f64", dim, body, rev)
+        fast = I.Interpreter(I.parse_module(text)).run([I.tensor(x, "f64")])[0].a
+        # force the general path: pad with the init value, gather every window, reduce
+        funcs = I.parse_module(text)
+        for fn in funcs.values():
+            for op in fn.ops:
+                if op.name == "reduce_window":
+                    op.attrs["__general__"] = True
+        slow = I.Interpreter(funcs).run([I.tensor(x, "f64")])[0].a
+        assert np.allclose(fast, slow, rtol=1e-13, atol=0), (shape, dim, body, rev)
+    ints = rng.integers(-50, 50, size=(7, 13)).astype(np.int32)
+    assert np.array_equal(run(NN.cumulative([7, 13], "i32", 1), [ints], "i32"), np.cumsum(ints, axis=1, dtype=np.int32))
+
+
+def brute_pool(x, body, window, strides, padding, base_dil, win_dil):
+    r = x.ndim
+    ident = {"add": 0.0, "maximum": -np.inf, "minimum": np.inf, "multiply": 1.0}[body]
+    f = {"add": lambda p, q: p + q, "maximum": max, "minimum": min, "multiply": lambda p, q: p * q}[body]
+    dil = [n + max(n - 1, 0) * (base_dil[d] - 1) for d, n in enumerate(x.shape)]
+    big = np.full([dil[d] + padding[d][0] + padding[d][1] for d in range(r)], ident)
+    for idx in itertools.product(*[range(n) for n in x.shape]):
+        big[tuple(padding[d][0] + idx[d] * base_dil[d] for d in range(r))] = x[idx]
+    out_shape = NN.window_out_shape(list(x.shape), window, strides, padding, base_dil, win_dil)
+    out = np.zeros(out_shape)
+    for o in itertools.product(*[range(n) for n in out_shape]):
+        acc = ident
+        for k in itertools.product(*[range(w) for w in window]):
+            acc = f(acc, big[tuple(o[d] * strides[d] + k[d] * win_dil[d] for d in range(r))])
+        out[o] = acc
+    return out
+
+
+@pytest.mark.parametrize("body", ["add", "maximum", "minimum"])
+def test_reduce_window_against_brute_force(body):
+    rng = np.random.default_rng(3)
+    x = rng.normal(size=(2, 3, 7, 9))
+    for window, strides, padding, bd, wd in (
+            ([1, 1, 2, 2], [1, 1, 2, 2], [[0, 0]] * 4, [1] * 4, [1] * 4),
+            ([1, 1, 3, 3], [1, 1, 2, 1], [[0, 0], [0, 0], [1, 1], [2, 0]], [1] * 4, [1] * 4),
+            ([1, 2, 3, 2], [1, 1, 1, 2], [[0, 0], [1, 0], [2, 1], [0, 3]], [1, 1, 2, 1], [1, 1, 2, 3])):
+        text, out_shape = NN.reduce_window(list(x.shape), "f64", body, window, strides, padding, bd, wd)
+        got = run(text, [x], "f64")
+        want = brute_pool(x, body, window, strides, padding, bd, wd)
+        assert list(got.shape) == out_shape
+        assert np.array_equal(np.isinf(got), np.isinf(want))
+        fin = np.isfinite(want)
+        assert np.allclose(got[fin], want[fin], rtol=1e-13)
+
+
+def brute_conv(x, w, strides, padding, lhs_dil, rhs_dil, groups):
+    """x [b, c, s...], w [o, i, k...] -> [b, o, s...]: plain loops."""
+    nsp = x.ndim - 2
+    B, C = x.shape[:2]
+    O, Ich = w.shape[:2]
+    dil = [n + max(n - 1, 0) * (lhs_dil[d] - 1) for d, n in enumerate(x.shape[2:])]
+    big = np.zeros([B, C] + [dil[d] + padding[d][0] + padding[d][1] for d in range(nsp)])
+    for idx in itertools.product(*[range(n) for n in x.shape[2:]]):
+        big[(slice(None), slice(None)) + tuple(padding[d][0] + idx[d] * lhs_dil[d] for d in range(nsp))] = x[(slice(None), slice(None)) + idx]
+    osp = NN.conv_out_shape(list(x.shape[2:]), list(w.shape[2:]), strides, padding, lhs_dil, rhs_dil)
+    out = np.zeros([B, O] + osp)
+    og = O // groups
+    for b in range(B):
+        for o in range(O):
+            g = o // og
+            for pos in itertools.product(*[range(n) for n in osp]):
+                acc = 0.0
+                for i in range(Ich):
+                    for k in itertools.product(*[range(n) for n in w.shape[2:]]):
+                        acc += big[(b, g * Ich + i) + tuple(pos[d] * strides[d] + k[d] * rhs_dil[d] for d in range(nsp))] * w[(o, i) + k]
+                out[(b, o) + pos] = acc
+    return out
+
+
+def test_convolution_against_brute_force_and_scipy():
+    rng = np.random.default_rng(4)
+    # the grid of test/nn/convolution.jl:165-181 on a smaller image: groups, strides, padding, dilation
+    for groups in (1, 2, 4):
+        x = rng.normal(size=(2, 8, 9, 10))
+        w = rng.normal(size=(4, 8 // groups, 3, 2))
+        for strides, padding, rd in (([1, 1], [[0, 0], [0, 0]], [1, 1]), ([2, 2], [[2, 2], [0, 0]], [1, 2]),
+                                     ([3, 3], [[0, 0], [2, 2]], [1, 1]), ([1, 2], [[2, 1], [0, 3]], [2, 1])):
+            text, out_shape = NN.convolution(list(x.shape), list(w.shape), "f64", strides=strides, padding=padding,
+                                             rhs_dil=rd, groups=groups, dims="[b, f, 0, 1]x[o, i, 0, 1]->[b, f, 0, 1]")
+            got = run(text, [x, w], "f64")
+            want = brute_conv(x, w, strides, padding, [1, 1], rd, groups)
+            assert list(got.shape) == out_shape
+            assert np.allclose(got, want, rtol=1e-12, atol=1e-12), (groups, strides, padding, rd)
+    # input dilation (what the gradient with respect to the input uses), one spatial dim
+    x = rng.normal(size=(2, 3, 11))
+    w = rng.normal(size=(5, 3, 4))
+    text, _ = NN.convolution([2, 3, 11], [5, 3, 4], "f64", dims="[b, f, 0]x[o, i, 0]->[b, f, 0]", lhs_dil=[3], padding=[[3, 2]])
+    assert np.allclose(run(text, [x, w], "f64"), brute_conv(x, w, [1], [[3, 2]], [3], [1], 1), rtol=1e-12, atol=1e-12)
+    # one channel, no padding: scipy's cross-correlation; flipped kernel: scipy's convolution
+    img = rng.normal(size=(12, 13))
+    ker = rng.normal(size=(3, 4))
+    for flip, lib in ((False, signal.correlate2d), (True, signal.convolve2d)):
+        text, _ = NN.convolution([1, 1, 12, 13], [1, 1, 3, 4], "f64", dims="[b, f, 0, 1]x[o, i, 0, 1]->[b, f, 0, 1]", flip=flip)
+        assert np.allclose(run(text, [img[None, None], ker[None, None]], "f64")[0, 0], lib(img, ker, mode="valid"), rtol=1e-12, atol=1e-12)
+
+
+def test_convolution_layouts_agree():
+    """The same convolution written with the reference's Julia-order dimension numbers
+    ([0, 1, f, b]-style, src/Ops.jl:1029-1043 on unreversed dims) and in the reversed raw order."""
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(2, 3, 7, 6))          # [b, f, h, w]
+    w = rng.normal(size=(4, 3, 3, 2))          # [o, i, kh, kw]
+    t1, _ = NN.convolution([2, 3, 7, 6], [4, 3, 3, 2], "f64", dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]", strides=[1, 2], padding=[[0, 1], [1, 0]])
+    a = run(t1, [x, w], "f64")
+    # the same data seen as [w, h, f, b]; spatial dim 0 is still the image's w
+    xt, wt = np.ascontiguousarray(x.transpose(3, 2, 1, 0)), np.ascontiguousarray(w.transpose(3, 2, 1, 0))
+    t2, _ = NN.convolution(list(xt.shape), list(wt.shape), "f64", dims="[0, 1, f, b]x[0, 1, i, o]->[0, 1, f, b]", strides=[1, 2], padding=[[0, 1], [1, 0]])
+    b = run(t2, [xt, wt], "f64")
+    assert np.allclose(a, b.transpose(3, 2, 1, 0), rtol=1e-13, atol=1e-13)
