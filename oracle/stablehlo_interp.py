@@ -2,7 +2,8 @@
 
 A CPU restatement, in numpy, of the StableHLO subset that Reactant hands to its
 runtime for the data-parallel hot path (elementwise/broadcast maps, reductions,
-slice/pad/dynamic_update_slice stencil chains, dot_general, convert).
+slice/pad/dynamic_update_slice stencil chains, dot_general, convert) and for the
+windowed ops next to it (reverse, reduce_window, convolution).
 
 The arithmetic of this path is not in the reference repository: it lives in XLA
 (un-vendored; pulled through Enzyme-JAX commit 51a4cd6c..., see the reference's
@@ -34,6 +35,12 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
   stencil chains ... brute-force loops on small grids
   while loops (src/Ops.jl:2349-2460; text form src/mlir/Dialects/StableHLO.jl:4850-4861)
       ... plain Python loops, closed forms, equality with the unrolled module
+  reverse, reduce_window, convolution (src/Ops.jl:1000-1073,3967-4011;
+      ext/ReactantNNlibExt/Implementations.jl:42-79, Ops.jl:1-32; src/TracedRArray.jl:1086-1108)
+      ... reference KATs (test/core/ops.jl:609-618, test/nn/convolution.jl:206-217,
+      test/core/map_reduction.jl:165-229), brute-force loops over the reference's
+      groups x stride x padding x dilation grid, scipy.signal.correlate2d / convolve2d,
+      numpy accumulate (tests/test_oracle_windows.py)
   bf16 / f8E4M3FN convert and dot_general ... PARITY UNPINNED in the reference
       (it holds no test of these); pinned here only by the OCP closed-form
       tables, exact-product arguments and torch CPU casts.

@@ -27,8 +27,14 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (M >= ((int64_t)1 << 30) || N >= ((int64_t)1 << 30) || K >= ((int64_t)1 << 30)) return c;
   // Large problems take 256x256 tiles on 8 wavefronts (each wavefront a 128x64 block of the
   // tile: fewer LDS bytes per MFMA); when that would leave compute units idle, 128x128 on 4.
+  // Products that leave most compute units without a 128x128 tile take 64x64 tiles (1000^3 f32:
+  // 16 -> 48 TFLOP/s, 1024^3 bf16: 130 -> 240); an operand with at most 64 rows (the output
+  // features of a convolution) gets a 64-wide tile so that no MFMA works on padding.
   int BM = 128, BN = 128, WM = 2, WN = 2;
-  if (((M + 255) / 256) * ((N + 255) / 256) * batch >= 256) { BM = 256; BN = 256; WM = 2; WN = 4; }
+  if (M <= 64 && N > 64) { BM = 64; BN = 128; }
+  else if (N <= 64 && M > 64) { BM = 128; BN = 64; }
+  else if (M > 128 && N > 128 && ((M + 255) / 256) * ((N + 255) / 256) * batch >= 256) { BM = 256; BN = 256; WM = 2; WN = 4; }
+  else if (((M + 127) / 128) * ((N + 127) / 128) * batch < 128) { BM = 64; BN = 64; }
   if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
     int v[4];
     if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
@@ -42,6 +48,9 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (const char* e = getenv("RX_GEMM_BLOCK")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2 && v[0] > 0 && v[1] > 0) { rb = v[0]; cb = v[1]; } }
   // a grid of few tiles (per batch entry) is not worth padding to whole XCD blocks
   if (((M + BM - 1) / BM) * ((N + BN - 1) / BN) < 64) rb = cb = 0;
+  // a tile grid with fewer rows (columns) than a block: make the block that flat
+  else if ((M + BM - 1) / BM < rb) { const int64_t gm = (M + BM - 1) / BM; cb = (int)(rb * cb / gm); rb = (int)gm; }
+  else if ((N + BN - 1) / BN < cb) { const int64_t gn = (N + BN - 1) / BN; rb = (int)(rb * cb / gn); cb = (int)gn; }
   const int nt = WM * WN * 64;
   if (direct) {
     int dbk = bk;

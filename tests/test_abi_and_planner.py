@@ -227,3 +227,24 @@ def test_products_with_a_vector_like_operand_plan_as_reductions(monkeypatch):
     assert "kind=dot_scalar" in rx.compile_offline(short)
     monkeypatch.setenv("RX_DOT_AS_REDUCE", "0")
     assert "kind=dot_scalar" in rx.compile_offline(mv)
+
+
+def test_windowed_ops_plan(monkeypatch):
+    import _nn_modules as NN
+    # cumsum over 2^24 elements: chunk totals, then the scan proper
+    rep = rx.compile_offline(NN.cumulative([1 << 24], "f32", 0))
+    assert "kind=scan_totals" in rep and "kind=scan " in rep and "launches: 2" in rep
+    # rows of a matrix: one workgroup per row chunk, no totals needed when a row is one chunk
+    assert "launches: 1" in rx.compile_offline(NN.cumulative([4096, 4096], "f32", 1))
+    # pooling: the window view is index arithmetic inside a reduction kernel
+    rep = rx.compile_offline(NN.reduce_window([8, 16, 32, 32], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])[0])
+    assert "launches: 1" in rep and "window reduce" in rep
+    # convolution: window matrix (one map), MFMA product with a 64-row tile, bias + relu + layout in one map;
+    # the reshaped weights share the argument's buffer
+    rep = rx.compile_offline(NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0])
+    kinds = [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
+    assert kinds == ["map", "gemm_f32", "map"], rep
+    assert "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rx.compile_offline(
+        NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]])[0], with_source=True)
+    with pytest.raises(Exception, match="batch_group_count"):
+        rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 8, 4, 4], "f32")[0].replace("batch_group_count = 1", "batch_group_count = 2"))
