@@ -88,6 +88,20 @@ def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
     return t1 - t0, np.asarray(mean_ms), res
 
 
+def _time_plain(client, exe, bufs, steps, warmup):
+    """The same K steps without the event pair around every launch (two records per launch cost a
+    few microseconds of stream time each, which shows on steps of less than 0.1 ms).  Seconds per step."""
+    dev = client.default_device()
+    for _ in range(warmup):
+        exe.execute_sharded(bufs)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        exe.execute_sharded(bufs)
+    dev.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
 def _dominant(launches, mean_ms, kinds):
     """Aggregate the launches whose kind is in `kinds`: (count, mean ms per launch, bytes/launch, flops/launch)."""
     idx = [i for i, l in enumerate(launches) if l["kind"] in kinds]
@@ -151,25 +165,28 @@ def bench_sinsum(rx, client, P, steps, warmup, n=1 << 26):
     launches = exe.launches()
     _, kms, _, _ = _dominant(launches, mean_ms, ("reduce",))
     algo = 8.0 * n
+    plain = _time_plain(client, exe, [bx, by], steps, warmup)
     got = float(rx.decode(res[0].to_host(), "f32"))
     exact = float(np.sum(np.sin(x.astype(np.float64)) + y.astype(np.float64)))
     return {"workload": "sinsum_add f32[2^26] x2 -> scalar", "ms_per_step": 1e3 * secs / steps,
             "value": algo / (secs / steps) / 1e9, "unit": "GB/s", "dtype": "f32",
+            "without_launch_events": {"ms_per_step": 1e3 * plain, "value": algo / plain / 1e9},
             "check": {"got": got, "f64_reference": exact},
             "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"], "kernel_ms": kms,
                          "achieved": algo / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": algo / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _traffic(launches[0]["kernel"])}}
 
 
-def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype):
+def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype, plain=None):
     launches = exe.launches()
     dots = [i for i, l in enumerate(launches) if l["flops"] > 0]
     flops = sum(launches[i]["flops"] for i in dots)
     dms = sum(mean_ms[i] for i in dots)
     big = max(dots, key=lambda i: launches[i]["flops"])
     ach = launches[big]["flops"] / (mean_ms[big] * 1e-3) / 1e12
+    extra = {} if plain is None else {"without_launch_events": {"ms_per_step": 1e3 * plain, "value": flops / plain / 1e12}}
     return {"workload": name, "ms_per_step": 1e3 * secs / steps, "value": flops / (secs / steps) / 1e12,
-            "unit": "TFLOP/s", "dtype": dtype,
+            "unit": "TFLOP/s", "dtype": dtype, **extra,
             "kernels": [{"kernel": l["kernel"], "kind": l["kind"], "ms": float(m)} for l, m in zip(launches, mean_ms)],
             "dot_tflops_kernel_time_only": flops / (dms * 1e-3) / 1e12,
             "roofline": {"bound": "mfma", "kernel": launches[big]["kernel"], "kernel_ms": float(mean_ms[big]),
@@ -182,7 +199,8 @@ def bench_gemm(rx, client, P, steps, warmup, n=4096):
     exe = rx.xla_compile(client, P.gemm(n, n, n))
     bufs = [_upload(rx, client, a, "f32") for a in (A, B, C)]
     secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
-    return _dot_entry("gemm f32 %d^3, alpha=1.5 beta=1.2" % n, exe, secs, steps, mean_ms, "f32", "f32")
+    return _dot_entry("gemm f32 %d^3, alpha=1.5 beta=1.2" % n, exe, secs, steps, mean_ms, "f32", "f32",
+                      plain=_time_plain(client, exe, bufs, steps, warmup))
 
 
 def bench_mlp(rx, client, P, steps, warmup, batch=8192, widths=(1024, 4096, 4096, 1024)):
@@ -195,7 +213,7 @@ def bench_mlp(rx, client, P, steps, warmup, batch=8192, widths=(1024, 4096, 4096
         bufs += [_upload(rx, client, rx.encode(w, "bf16"), "bf16"), _upload(rx, client, rx.encode(b, "bf16"), "bf16")]
     secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
     return _dot_entry("mlp bf16 batch %d widths %s, bias+gelu, softmax" % (batch, "->".join(map(str, widths))), exe, secs,
-                      steps, mean_ms, "bf16", "bf16")
+                      steps, mean_ms, "bf16", "bf16", plain=_time_plain(client, exe, bufs, steps, warmup))
 
 
 def bench_fp8(rx, client, P, steps, warmup, n=8192):
@@ -207,7 +225,7 @@ def bench_fp8(rx, client, P, steps, warmup, n=8192):
     bufs = [_upload(rx, client, a, "bf16"), _upload(rx, client, wq, "f8E4M3FN"), _upload(rx, client, np.asarray(sw), "f32")]
     secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
     return _dot_entry("fp8 linear %d^3 e4m3 per-tensor scales, bf16 out + RMSNorm" % n, exe, secs, steps, mean_ms, "f8",
-                      "f8E4M3FN")
+                      "f8E4M3FN", plain=_time_plain(client, exe, bufs, steps, warmup))
 
 
 def cpu_baseline_stencil(P, nx=512, ny=512, nz=256, nsteps=10):
