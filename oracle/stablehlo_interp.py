@@ -41,6 +41,9 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       test/core/map_reduction.jl:165-229), brute-force loops over the reference's
       groups x stride x padding x dilation grid, scipy.signal.correlate2d / convolve2d,
       numpy accumulate (tests/test_oracle_windows.py)
+  batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
+      (zero mean / unit variance of the normalized batch, numpy mean and var, the affine
+      special case); the reference holds no known answer for them
   bf16 / f8E4M3FN convert and dot_general ... PARITY UNPINNED in the reference
       (it holds no test of these); pinned here only by the OCP closed-form
       tables, exact-product arguments and torch CPU casts.
@@ -552,10 +555,13 @@ class Parser:
         mo = re.search(r"#stablehlo\.conv<([^>]*->[^>]*)>", inner)
         if mo:
             a["dim_numbers"] = _parse_conv_dims(mo.group(1))
-        for key in ("feature_group_count", "batch_group_count"):
+        for key in ("feature_group_count", "batch_group_count", "feature_index"):
             mo = re.search(r"\b" + key + r"\s*=\s*(\d+)", inner)
             if mo:
                 a[key] = int(mo.group(1))
+        mo = re.search(r"\bepsilon\s*=\s*([-+\w.]+)", inner)
+        if mo:
+            a["epsilon"] = float(mo.group(1))
         mo = re.search(r"\bdimension\s*=\s*(\d+)", inner)
         if mo:
             a["dimension"] = int(mo.group(1))
@@ -1204,6 +1210,34 @@ def _reduce_window(x, init, at, dt, hifi):
     return _reduce(Tensor(w, x.dt) if not is_float(x.dt) else _FloatView(w, x.dt), init, list(range(r)), at["body"], dt, hifi)
 
 
+def _batch_norm(xs, at, training, hifi):
+    """stablehlo.batch_norm_inference / batch_norm_training (reference src/Ops.jl:4012-4092) as the
+    specification writes them: per-feature mean and biased variance over the other dims (training),
+    then (x - mean) / sqrt(variance + epsilon) * scale + offset, every step in the element type."""
+    x = xs[0]
+    dt = x.dt
+    f = at["feature_index"]
+    others = [d for d in range(x.a.ndim) if d != f]
+    shp = [1] * x.a.ndim
+    shp[f] = x.a.shape[f]
+    bc = lambda v: v.a.reshape(shp)
+    if training:
+        scale, offset = xs[1], xs[2]
+        count = tensor(np.asarray(float(np.prod([x.a.shape[d] for d in others]))), dt)
+        zero = tensor(np.zeros(()), dt)
+        mean = _binary("divide", _reduce(x, zero, others, "add", dt, hifi), count, dt)
+        c = _binary("subtract", x, Tensor(np.broadcast_to(bc(mean), x.a.shape), dt), dt)
+        var = _binary("divide", _reduce(_binary("multiply", c, c, dt), zero, others, "add", dt, hifi), count, dt)
+    else:
+        scale, offset, mean, var = xs[1:5]
+    full = lambda v: Tensor(np.broadcast_to(bc(v), x.a.shape), dt)
+    centered = _binary("subtract", x, full(mean), dt)
+    stddev = _unary("sqrt", _binary("add", var, tensor(np.asarray(at["epsilon"]), dt), dt), dt)
+    normalized = _binary("divide", centered, full(stddev), dt)
+    res = _binary("add", _binary("multiply", normalized, full(scale), dt), full(offset), dt)
+    return [res, mean, var] if training else [res]
+
+
 def _prefix_form(shape, window, strides, bdil, wdil, pad):
     """(dim, from_the_end) when every window is a prefix (or suffix) of one dimension: the window
     spans that whole dimension and the operand is padded by its length minus one on one side."""
@@ -1474,6 +1508,8 @@ class Interpreter:
                 raise NotImplementedError("variadic reduce")
             r = _reduce(xs[0], xs[1], at["dimensions"], at["body"], op.types_out[0].dt, self.hifi)
             return [r if self.excess else _rounded(r)]
+        if n in ("batch_norm_inference", "batch_norm_training"):
+            return _batch_norm(xs, at, n == "batch_norm_training", self.hifi)
         if n == "reverse":
             return [Tensor(np.ascontiguousarray(np.flip(xs[0].a, axis=tuple(at["dimensions"]))), xs[0].dt)]
         if n == "reduce_window":

@@ -523,7 +523,7 @@ struct P {
                             "dimension", "iota_dimension", "lhs_batching_dimensions", "rhs_batching_dimensions",
                             "lhs_contracting_dimensions", "rhs_contracting_dimensions", "window_dimensions",
                             "window_strides", "base_dilations", "window_dilations", "lhs_dilation", "rhs_dilation",
-                            "padding", "feature_group_count", "batch_group_count"})
+                            "padding", "feature_group_count", "batch_group_count", "feature_index"})
       scan_int_array(in, key, o);
     {
       size_t q = in.find("#stablehlo.conv<");
@@ -531,6 +531,17 @@ struct P {
         size_t arrow = in.find("->", q);
         size_t e = arrow == std::string::npos ? arrow : in.find(']', arrow);
         if (e != std::string::npos) o.sa["dim_numbers"] = in.substr(q + 16, e + 1 - (q + 16));
+      }
+      q = in.find("epsilon");
+      if (q != std::string::npos) {
+        size_t e1 = in.find('=', q);
+        if (e1 != std::string::npos) {
+          ++e1;
+          while (e1 < in.size() && in[e1] == ' ') ++e1;
+          size_t e2 = e1;
+          while (e2 < in.size() && (isalnum((unsigned char)in[e2]) || in[e2] == '.' || in[e2] == '-' || in[e2] == '+')) ++e2;
+          o.sa["epsilon"] = in.substr(e1, e2 - e1);
+        }
       }
       q = in.find("window_reversal");
       if (q != std::string::npos) {
@@ -1339,6 +1350,86 @@ struct Builder {
     return g.add(rn);
   }
 
+  int binary_node(const char* op, int a, int b) {
+    Node n;
+    n.k = OpK::Binary;
+    n.op = op;
+    n.ty = ty(a);
+    n.in = {a, b};
+    return g.add(n);
+  }
+  int splat_of(const TType& t, double v) {
+    Node c;
+    c.k = OpK::Constant;
+    c.splat = true;
+    c.ty = TType{t.dt, {}};
+    c.data.assign((size_t)info(t.dt).size, 0);
+    store_scalar(t.dt, v, (int64_t)v, false, c.data.data());
+    const int id = g.add(c);
+    if (t.rank() == 0) return id;
+    Node b;
+    b.k = OpK::BroadcastInDim;
+    b.in = {id};
+    b.ty = t;
+    return g.add(b);
+  }
+  int feature_bcast(int v, const TType& full, int feature) {
+    Node b;
+    b.k = OpK::BroadcastInDim;
+    b.in = {v};
+    b.a0 = {feature};
+    b.ty = full;
+    return g.add(b);
+  }
+  // batch_norm_inference / batch_norm_training (reference src/Ops.jl:4012-4092), written out as the
+  // specification defines them: per-feature mean and biased variance over all other dims (training),
+  // then (x - mean) / sqrt(variance + epsilon) * scale + offset.
+  std::vector<int> build_batch_norm(const RawOp& o, const std::vector<int>& in, bool training) {
+    if (in.size() != (training ? 3u : 5u)) fail(o.name + ": wrong operand count");
+    if (!o.ia.count("feature_index") || o.ia.at("feature_index").empty()) fail(o.name + ": feature_index missing");
+    if (!o.sa.count("epsilon")) fail(o.name + ": epsilon missing");
+    const TType xt = ty(in[0]);
+    const int f = (int)o.ia.at("feature_index")[0];
+    if (!is_float(xt.dt) || f < 0 || f >= xt.rank()) fail(o.name + ": float operand and a valid feature_index expected");
+    const TType ft{xt.dt, {xt.dims[f]}};
+    for (size_t k = 1; k < in.size(); ++k) if (!(ty(in[k]) == ft)) fail(o.name + ": per-feature operands must be " + ft.str());
+    if (o.tout.empty() || !(o.tout[0] == xt)) fail(o.name + ": result type mismatch");
+    double eps = 0;
+    try { eps = std::stod(o.sa.at("epsilon")); } catch (...) { fail(o.name + ": malformed epsilon"); }
+    int mean, var;
+    if (training) {
+      std::vector<int64_t> rdims;
+      double count = 1;
+      for (int d = 0; d < xt.rank(); ++d) if (d != f) { rdims.push_back(d); count *= (double)xt.dims[d]; }
+      auto feature_mean = [&](int v) {
+        Node r;
+        r.k = OpK::Reduce;
+        r.red = Red::Add;
+        r.in = {v, zero_of(xt.dt)};
+        r.a0 = rdims;
+        r.ty = ft;
+        return binary_node("divide", g.add(r), splat_of(ft, count));
+      };
+      mean = feature_mean(in[0]);
+      const int c = binary_node("subtract", in[0], feature_bcast(mean, xt, f));
+      var = feature_mean(binary_node("multiply", c, c));
+    } else {
+      mean = in[3];
+      var = in[4];
+    }
+    const int centered = binary_node("subtract", in[0], feature_bcast(mean, xt, f));
+    Node sq;
+    sq.k = OpK::Unary;
+    sq.op = "sqrt";
+    sq.ty = ft;
+    sq.in = {binary_node("add", var, splat_of(ft, eps))};
+    const int stddev = g.add(sq);
+    const int normalized = binary_node("divide", centered, feature_bcast(stddev, xt, f));
+    const int res = binary_node("add", binary_node("multiply", normalized, feature_bcast(in[1], xt, f)), feature_bcast(in[2], xt, f));
+    if (training) return {res, mean, var};
+    return {res};
+  }
+
   struct ConvDims { int d0 = -1, d1 = -1; std::vector<int> sp; };
   // "[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]": position of the two named roles and of every spatial dim
   static void parse_conv_dims(const std::string& text, ConvDims out[3]) {
@@ -1795,6 +1886,7 @@ struct Builder {
       for (auto d : n.a0) if (d < 0 || d >= n.ty.rank()) fail("reverse: dimension out of range");
       return {g.add(n)};
     }
+    if (sh == "batch_norm_inference" || sh == "batch_norm_training") return build_batch_norm(o, in, sh == "batch_norm_training");
     if (sh == "reduce_window") {
       if (in.size() != 2) fail("variadic reduce_window is not supported");
       return {build_reduce_window(o, in[0], in[1], out1())};

@@ -136,3 +136,18 @@ def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1,
         body += "    %%2 = stablehlo.maximum %%1, %%z : %s\n" % to
         res = "%2"
     return ("module {\n  func.func @main(%s) -> %s {\n%s    return %s : %s\n  }\n}\n" % (args, to, body, res, to)), out
+
+
+def batch_norm(shape, dt, feature_index, epsilon=1e-5, training=False):
+    """`stablehlo.batch_norm_inference` / `batch_norm_training` in the generic form they print in
+    (built by the reference's src/Ops.jl:4012-4092)."""
+    tx, tf = tt(shape, dt), tt([shape[feature_index]], dt)
+    if training:
+        return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg2: %s) -> (%s, %s, %s) {\n"
+                "    %%0:3 = \"stablehlo.batch_norm_training\"(%%arg0, %%arg1, %%arg2) <{epsilon = %e : f32, feature_index = %d : i64}> : "
+                "(%s, %s, %s) -> (%s, %s, %s)\n    return %%0#0, %%0#1, %%0#2 : %s, %s, %s\n  }\n}\n"
+                % (tx, tf, tf, tx, tf, tf, epsilon, feature_index, tx, tf, tf, tx, tf, tf, tx, tf, tf))
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg2: %s, %%arg3: %s, %%arg4: %s) -> %s {\n"
+            "    %%0 = \"stablehlo.batch_norm_inference\"(%%arg0, %%arg1, %%arg2, %%arg3, %%arg4) <{epsilon = %e : f32, feature_index = %d : i64}> : "
+            "(%s, %s, %s, %s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
+            % (tx, tf, tf, tf, tf, tx, epsilon, feature_index, tx, tf, tf, tf, tf, tx, tx))

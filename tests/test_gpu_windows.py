@@ -208,3 +208,21 @@ def test_convolution_layouts_and_types(rx, client, xs, ws, dt, dims, kw, kind):
     taps = int(np.prod(ws[1:])) if not dims or dims.startswith("[b, f") else int(np.prod(ws)) // max(ws)
     tol = 1e-2 if dt == "bf16" else (1e-12 if dt == "f64" else 1e-5 * np.sqrt(taps))
     _close(got[0].a, ref[0].a, tol)
+
+
+@pytest.mark.parametrize("shape,dt,feature,training", [([4, 16, 14, 14], "f32", 1, False), ([14, 14, 16, 4], "f32", 2, False),
+                                                       ([64, 33], "f32", 1, True), ([8, 6, 30, 30], "f32", 1, True),
+                                                       ([4, 16, 14, 14], "bf16", 1, False), ([5, 7, 9], "f64", 0, True)])
+def test_batch_norm(rx, client, shape, dt, feature, training):
+    text = NN.batch_norm(shape, dt, feature, 1e-3, training)
+    rng = np.random.default_rng(13)
+    nf = shape[feature]
+    args = [I.tensor(rng.normal(1.0, 2.0, size=shape), dt), I.tensor(rng.uniform(0.5, 1.5, size=nf), dt), I.tensor(rng.normal(size=nf), dt)]
+    if not training:
+        args += [I.tensor(rng.normal(size=nf), dt), I.tensor(rng.uniform(0.5, 2.0, size=nf), dt)]
+    got, exe = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True, excess=(dt == "bf16"))
+    assert len(got) == (3 if training else 1)
+    tol = {"f32": 2e-5, "bf16": 1e-2, "f64": 1e-12}[dt]
+    for g, r in zip(got, ref):
+        _close(g.a, r.a, tol)

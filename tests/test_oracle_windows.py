@@ -170,3 +170,20 @@ def test_convolution_layouts_agree():
     t2, _ = NN.convolution(list(xt.shape), list(wt.shape), "f64", dims="[0, 1, f, b]x[0, 1, i, o]->[0, 1, f, b]", strides=[1, 2], padding=[[0, 1], [1, 0]])
     b = run(t2, [xt, wt], "f64")
     assert np.allclose(a, b.transpose(3, 2, 1, 0), rtol=1e-13, atol=1e-13)
+
+
+def test_batch_norm_closed_forms():
+    """Normalizing with a batch's own statistics gives zero mean and unit (biased) variance per
+    feature; inference with mean 0, variance 1 - eps, scale s, offset b is s * x + b."""
+    rng = np.random.default_rng(8)
+    x = rng.normal(2.0, 3.0, size=(6, 5, 7))
+    ones, zeros = np.ones(5), np.zeros(5)
+    out, mean, var = [t.a for t in I.run_text(NN.batch_norm([6, 5, 7], "f64", 1, 1e-5, training=True),
+                                              [I.tensor(a, "f64") for a in (x, ones, zeros)])]
+    assert np.allclose(mean, x.mean(axis=(0, 2)), rtol=1e-13)
+    assert np.allclose(var, x.var(axis=(0, 2)), rtol=1e-12)
+    assert np.allclose(out.mean(axis=(0, 2)), 0, atol=1e-12)
+    assert np.allclose(out.var(axis=(0, 2)), var / (var + 1e-5), rtol=1e-10)
+    s, b = rng.normal(size=5), rng.normal(size=5)
+    got = I.run_text(NN.batch_norm([6, 5, 7], "f64", 1, 0.25), [I.tensor(a, "f64") for a in (x, s, b, zeros, ones * 0.75)])[0].a
+    assert np.allclose(got, x * s[None, :, None] + b[None, :, None], rtol=1e-13, atol=1e-13)
