@@ -151,3 +151,78 @@ def batch_norm(shape, dt, feature_index, epsilon=1e-5, training=False):
             "    %%0 = \"stablehlo.batch_norm_inference\"(%%arg0, %%arg1, %%arg2, %%arg3, %%arg4) <{epsilon = %e : f32, feature_index = %d : i64}> : "
             "(%s, %s, %s, %s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
             % (tx, tf, tf, tf, tf, tx, epsilon, feature_index, tx, tf, tf, tf, tf, tx, tx))
+
+
+def vgg_block(batch=2, cin=3, cmid=8, hw=16, classes=10, dt="f32"):
+    """conv3x3(pad 1) + batch norm (inference) + relu + maxpool 2x2 + conv3x3 + bias + relu +
+    global mean pool + dense + softmax: the op sequence of the VGG forward pass of
+    benchmark/nn/vision.jl:24-34 at toy sizes.  Arguments: x, w1, bn scale/offset/mean/var, w2, b2, wd, bd."""
+    h2 = hw // 2
+    X, W1, F1 = tt([batch, cin, hw, hw], dt), tt([cmid, cin, 3, 3], dt), tt([cmid], dt)
+    A1 = tt([batch, cmid, hw, hw], dt)
+    P1 = tt([batch, cmid, h2, h2], dt)
+    W2, F2 = tt([2 * cmid, cmid, 3, 3], dt), tt([2 * cmid], dt)
+    A2 = tt([batch, 2 * cmid, h2, h2], dt)
+    G, WD, BD, OUT, S = tt([batch, 2 * cmid], dt), tt([2 * cmid, classes], dt), tt([classes], dt), tt([batch, classes], dt), tt([], dt)
+    R = tt([batch], dt)
+    conv = ("stablehlo.convolution(%s, %s) dim_numbers = [b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0], window = {stride = [1, 1], "
+            "pad = [[1, 1], [1, 1]], rhs_dilate = [1, 1]} {batch_group_count = 1 : i64, feature_group_count = 1 : i64} : (%s, %s) -> %s")
+    pool = ("\"stablehlo.reduce_window\"(%s, %s) <{base_dilations = array<i64: 1, 1, 1, 1>, padding = dense<0> : tensor<4x2xi64>, "
+            "window_dilations = array<i64: 1, 1, 1, 1>, window_dimensions = array<i64: 1, 1, 2, 2>, window_strides = array<i64: 1, 1, 2, 2>}> ({\n"
+            "    ^bb0(%%p: %s, %%q: %s):\n      %%m = stablehlo.maximum %%p, %%q : %s\n      stablehlo.return %%m : %s\n    }) : (%s, %s) -> %s")
+    lines = [
+        "%c1 = " + conv % ("%arg0", "%arg1", X, W1, A1),
+        "%bn = \"stablehlo.batch_norm_inference\"(%c1, %arg2, %arg3, %arg4, %arg5) <{epsilon = 1.000000e-05 : f32, feature_index = 1 : i64}> : "
+        "(" + ", ".join([A1, F1, F1, F1, F1]) + ") -> " + A1,
+        "%z1 = stablehlo.constant dense<0.000000e+00> : " + A1,
+        "%r1 = stablehlo.maximum %bn, %z1 : " + A1,
+        "%ninf = stablehlo.constant dense<0xFF800000> : " + S if dt == "f32" else "%ninf = stablehlo.constant dense<0xFFF0000000000000> : " + S,
+        "%p1 = " + pool % ("%r1", "%ninf", S, S, S, S, A1, S, P1),
+        "%c2 = " + conv % ("%p1", "%arg6", P1, W2, A2),
+        "%b2 = stablehlo.broadcast_in_dim %arg7, dims = [1] : (" + F2 + ") -> " + A2,
+        "%a2 = stablehlo.add %c2, %b2 : " + A2,
+        "%z2 = stablehlo.constant dense<0.000000e+00> : " + A2,
+        "%r2 = stablehlo.maximum %a2, %z2 : " + A2,
+        "%zero = stablehlo.constant dense<0.000000e+00> : " + S,
+        "%gs = stablehlo.reduce(%r2 init: %zero) applies stablehlo.add across dimensions = [2, 3] : (" + A2 + ", " + S + ") -> " + G,
+        "%cnt = stablehlo.constant dense<" + "%.6e" % float(h2 * h2) + "> : " + G,
+        "%gm = stablehlo.divide %gs, %cnt : " + G,
+        "%d = stablehlo.dot_general %gm, %arg8, contracting_dims = [1] x [0] : (" + G + ", " + WD + ") -> " + OUT,
+        "%bd = stablehlo.broadcast_in_dim %arg9, dims = [1] : (" + BD + ") -> " + OUT,
+        "%lg = stablehlo.add %d, %bd : " + OUT,
+        "%mx = stablehlo.reduce(%lg init: %ninf) applies stablehlo.maximum across dimensions = [1] : (" + OUT + ", " + S + ") -> " + R,
+        "%mxb = stablehlo.broadcast_in_dim %mx, dims = [0] : (" + R + ") -> " + OUT,
+        "%sh = stablehlo.subtract %lg, %mxb : " + OUT,
+        "%ex = stablehlo.exponential %sh : " + OUT,
+        "%sm = stablehlo.reduce(%ex init: %zero) applies stablehlo.add across dimensions = [1] : (" + OUT + ", " + S + ") -> " + R,
+        "%smb = stablehlo.broadcast_in_dim %sm, dims = [0] : (" + R + ") -> " + OUT,
+        "%out = stablehlo.divide %ex, %smb : " + OUT,
+    ]
+    args = [X, W1, F1, F1, F1, F1, W2, F2, WD, BD]
+    sig = ", ".join("%%arg%d: %s" % (k, t) for k, t in enumerate(args))
+    shapes = [[batch, cin, hw, hw], [cmid, cin, 3, 3], [cmid], [cmid], [cmid], [cmid], [2 * cmid, cmid, 3, 3], [2 * cmid],
+              [2 * cmid, classes], [classes]]
+    return ("module {\n  func.func @main(%s) -> %s {\n    %s\n    return %%out : %s\n  }\n}\n" % (sig, OUT, "\n    ".join(lines), OUT)), shapes
+
+
+def attention_block(batch_heads=6, seq=40, dim=16, dt="f32"):
+    """softmax(q k^T / sqrt(d)) v on [batch*heads, seq, dim] operands: the two batched products and the
+    row softmax of NNlib.dot_product_attention, which the ViT of benchmark/nn/vision.jl:5-22 runs."""
+    Q, SC, S, R = tt([batch_heads, seq, dim], dt), tt([batch_heads, seq, seq], dt), tt([], dt), tt([batch_heads, seq], dt)
+    lines = [
+        "%s0 = stablehlo.dot_general %arg0, %arg1, batching_dims = [0] x [0], contracting_dims = [2] x [2] : (" + Q + ", " + Q + ") -> " + SC,
+        "%sc = stablehlo.constant dense<" + "%.9e" % (1.0 / dim ** 0.5) + "> : " + SC,
+        "%s1 = stablehlo.multiply %s0, %sc : " + SC,
+        "%ninf = stablehlo.constant dense<" + _init_literal("maximum", dt) + "> : " + S,
+        "%zero = stablehlo.constant dense<0.000000e+00> : " + S,
+        "%mx = stablehlo.reduce(%s1 init: %ninf) applies stablehlo.maximum across dimensions = [2] : (" + SC + ", " + S + ") -> " + R,
+        "%mxb = stablehlo.broadcast_in_dim %mx, dims = [0, 1] : (" + R + ") -> " + SC,
+        "%sh = stablehlo.subtract %s1, %mxb : " + SC,
+        "%ex = stablehlo.exponential %sh : " + SC,
+        "%sm = stablehlo.reduce(%ex init: %zero) applies stablehlo.add across dimensions = [2] : (" + SC + ", " + S + ") -> " + R,
+        "%smb = stablehlo.broadcast_in_dim %sm, dims = [0, 1] : (" + R + ") -> " + SC,
+        "%p = stablehlo.divide %ex, %smb : " + SC,
+        "%out = stablehlo.dot_general %p, %arg2, batching_dims = [0] x [0], contracting_dims = [2] x [1] : (" + SC + ", " + Q + ") -> " + Q,
+    ]
+    sig = ", ".join("%%arg%d: %s" % (k, Q) for k in range(3))
+    return ("module {\n  func.func @main(%s) -> %s {\n    %s\n    return %%out : %s\n  }\n}\n" % (sig, Q, "\n    ".join(lines), Q)), [[batch_heads, seq, dim]] * 3

@@ -226,3 +226,33 @@ def test_batch_norm(rx, client, shape, dt, feature, training):
     tol = {"f32": 2e-5, "bf16": 1e-2, "f64": 1e-12}[dt]
     for g, r in zip(got, ref):
         _close(g.a, r.a, tol)
+
+
+@pytest.mark.parametrize("sizes", [dict(batch=2, cin=3, cmid=8, hw=16, classes=10), dict(batch=4, cin=3, cmid=64, hw=32, classes=100)])
+def test_vgg_style_forward_pass(rx, client, sizes):
+    text, shapes = NN.vgg_block(**sizes)
+    rng = np.random.default_rng(17)
+    args = []
+    for k, sh in enumerate(shapes):
+        if k == 5:      # running variance
+            args.append(I.tensor(rng.uniform(0.5, 2.0, size=sh), "f32"))
+        elif len(sh) == 4 and k > 0:
+            args.append(I.tensor(rng.normal(size=sh) / np.sqrt(np.prod(sh[1:])), "f32"))
+        else:
+            args.append(I.tensor(rng.normal(size=sh), "f32"))
+    got, exe = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    assert got[0].a.shape == (sizes["batch"], sizes["classes"])
+    assert np.allclose(got[0].a.sum(axis=1), 1.0, atol=1e-5)
+    _close(got[0].a, ref[0].a, 1e-4)
+    if sizes["cmid"] >= 64:
+        assert any(l["kind"] == "gemm_f32" for l in exe.launches())
+
+
+@pytest.mark.parametrize("bh,seq,dim,dt,tol", [(6, 40, 16, "f32", 1e-5), (8, 256, 64, "f32", 1e-4), (8, 256, 64, "bf16", 2e-2)])
+def test_attention_block(rx, client, bh, seq, dim, dt, tol):
+    text, shapes = NN.attention_block(bh, seq, dim, dt)
+    args = _args(shapes, dt, seed=19)
+    got, exe = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True, excess=(dt == "bf16"))
+    _close(got[0].a, ref[0].a, tol)
