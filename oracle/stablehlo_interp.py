@@ -1326,9 +1326,10 @@ def _convolution(x, w, at, dt_out, hifi):
     out = np.zeros([B, O] + osp, dtype=acc)
     Og = O // G
     kk = int(np.prod(ksz)) if ksz else 1
+    npos = int(np.prod(osp)) if osp else 1
     for g in range(G):
         wg = wa[g * Og:(g + 1) * Og].reshape(Og, I, kk)                      # [o, i, k]
-        xg = win.reshape([kk, B, C, -1])[:, :, g * I:(g + 1) * I, :]        # [k, b, i, P]
+        xg = win.reshape([kk, B, C, npos])[:, :, g * I:(g + 1) * I, :]      # [k, b, i, P]
         out[:, g * Og:(g + 1) * Og] = np.einsum("oik,kbip->bop", wg, xg).reshape([B, Og] + osp)
     # canonical [b, f, s...] -> the result's own dimension order
     perm = [0] * (2 + nsp)

@@ -344,8 +344,10 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       ptrs.push_back(bufs[b]->ptr);
     }
     for (auto& p : ptrs) argv.push_back(&p);
-    HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
-                                    argv.data(), nullptr));
+    // a kernel over an empty tensor has no workgroups: nothing to launch
+    if (L.grid[0] != 0 && L.grid[1] != 0 && L.grid[2] != 0)
+      HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
+                                      argv.data(), nullptr));
     if (timed) HIP_CHECK(hipEventRecord(evs[li + 1], dev->stream));
     for (int b : L.args) {
       const auto& B = P.buffers[b];

@@ -256,3 +256,26 @@ def test_attention_block(rx, client, bh, seq, dim, dt, tol):
     got, exe = gpu_run(rx, client, text, args)
     ref = oracle_run(text, args, hifi=True, excess=(dt == "bf16"))
     _close(got[0].a, ref[0].a, tol)
+
+
+EDGES = [
+    ("scan of an empty tensor", lambda: (NN.cumulative([5, 0], "f32", 0), [[5, 0]])),
+    ("scan along a dimension of one element", lambda: (NN.cumulative([1, 7], "f32", 0), [[1, 7]])),
+    ("scan of two elements", lambda: (NN.cumulative([2], "f32", 0), [[2]])),
+    ("window larger than the operand", lambda: (NN.reduce_window([2, 3], "f32", "add", [3, 1])[0], [[2, 3]])),
+    ("window of one element", lambda: (NN.reduce_window([4, 5], "f32", "maximum", [1, 1])[0], [[4, 5]])),
+    ("convolution of an empty batch", lambda: (NN.convolution([0, 3, 8, 8], [4, 3, 3, 3], "f32")[0], [[0, 3, 8, 8], [4, 3, 3, 3]])),
+    ("1x1 convolution", lambda: (NN.convolution([2, 16, 9, 9], [8, 16, 1, 1], "f32")[0], [[2, 16, 9, 9], [8, 16, 1, 1]])),
+    ("kernel larger than the image", lambda: (NN.convolution([1, 2, 3, 3], [2, 2, 5, 5], "f32")[0], [[1, 2, 3, 3], [2, 2, 5, 5]])),
+    ("convolution without spatial dims", lambda: (NN.convolution([5, 7], [3, 7], "f32", dims="[b, f]x[o, i]->[b, f]")[0], [[5, 7], [3, 7]])),
+]
+
+
+@pytest.mark.parametrize("name,make", EDGES, ids=[e[0] for e in EDGES])
+def test_degenerate_windows(rx, client, name, make):
+    text, shapes = make()
+    args = _args(shapes, "f32", seed=23)
+    got, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    assert got[0].a.shape == ref[0].a.shape
+    assert np.allclose(got[0].a, ref[0].a, rtol=1e-5, atol=1e-6)
