@@ -1944,11 +1944,22 @@ struct Planner {
     em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(rn.in[0])) || ty.numel() >= ((int64_t)1 << 31);
     const std::string it = em.idx_t();
-    em.set_root({}, {}, false);
+    // forward scans along the minor dimension whose rows are whole vectors read and write 16 bytes per lane
+    const int vecw = (rowwise && !rev && a == ty.rank() - 1 && pick_vec(ty) > 1) ? pick_vec(ty) : 1;
+    const int V = vecw > 1 ? vecw : 4;
     Index ix(ty.rank());
+    std::vector<std::string> vars;
     for (int d = 0; d < ty.rank(); ++d) {
       ix[d].var = d == a ? std::string("j") : (d < a ? "o" : "q") + std::to_string(d);
       ix[d].hi = ty.dims[d] - 1;
+      vars.push_back(ix[d].var);
+    }
+    if (vecw > 1) {
+      em.set_root(ty.dims, vars, true);
+      em.vec = vecw;
+      em.direct_expr = vec_name;
+    } else {
+      em.set_root({}, {}, false);
     }
     em.indent = rowwise ? 8 : 4;
     const std::string val = em.emit(rn.in[0], ix);
@@ -1971,7 +1982,18 @@ struct Planner {
     Launch L1, L2;
     int64_t NC = 1, CH = n;
     if (rowwise) {
-      constexpr int V = 4, TILE = kBlock * V;
+      const int TILE = kBlock * V;
+      // preloads of the inputs that are read at the scan's own index, one vector per lane
+      auto preload = [&](std::ostringstream& oo, const std::string& pad) {
+        if (vecw == 1) return;
+        oo << pad << "const " << it << " lin0 = row * " << n << " + pb;\n";
+        for (auto& sd : em.direct_vecs) {
+          const int slot = sd.first;
+          const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vecw) + ">";
+          oo << pad << vt << " " << vec_name(slot, 0) << " = {};\n";
+          oo << pad << "if (pb < pend) " << vec_name(slot, 0) << " = rx_load<" << vt << ">(in" << slot << " + lin0);\n";
+        }
+      };
       NC = std::max<int64_t>(1, std::min<int64_t>((n + 4 * TILE - 1) / (4 * TILE), std::max<int64_t>(1, 2048 / std::max<int64_t>(outer, 1))));
       CH = ((n + NC - 1) / NC + TILE - 1) / TILE * TILE;
       NC = (n + CH - 1) / CH;
@@ -1997,11 +2019,46 @@ struct Planner {
         o << head("@K@_scan_totals", true, false) << " {\n";
         o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n";
         prologue(o);
-        o << "  " << ACC << " acc = " << IDENT << ";\n";
-        o << "  for (" << it << " pb = c * " << CH << " + (" << it << ")threadIdx.x * " << V << "; pb < pend; pb += " << TILE << ") {\n";
-        o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
-        o << "        const " << it << " j = " << jexpr << ";\n" << body;
-        o << "        acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n      }\n    }\n  }\n";
+        if (vecw > 1) {
+          // Rows of whole vectors: a vector that starts inside the chunk lies inside it.  Four tiles per
+          // iteration, their loads issued together (one 16-byte load in flight per lane does not
+          // cover the memory latency), each with its own accumulator.
+          constexpr int U = 4;
+          o << "  " << ACC << " accu[" << U << "];\n#pragma unroll\n  for (int u = 0; u < " << U << "; ++u) accu[u] = " << IDENT << ";\n";
+          o << "  " << it << " pb = c * " << CH << " + (" << it << ")threadIdx.x * " << V << ";\n";
+          auto one = [&](const std::string& pbexpr, int u, const std::string& pad) {
+            // the generated expression names its preloaded vectors; give every tile of the group its own
+            std::string b = body, vv = val;
+            for (auto& sd : em.direct_vecs) {
+              const std::string from = vec_name(sd.first, 0), to = from + "u" + std::to_string(u);
+              for (std::string* t : {&b, &vv})
+                for (size_t q = t->find(from + "."); q != std::string::npos; q = t->find(from + ".", q + to.size())) t->replace(q, from.size(), to);
+            }
+            o << pad << "{\n" << pad << "  const " << it << " pbu = " << pbexpr << ";\n";
+            o << "#pragma unroll\n" << pad << "  for (int l = 0; l < " << V << "; ++l) {\n" << pad << "    const " << it << " j = pbu + l;\n" << b;
+            o << pad << "    accu[" << u << "] = " << red_apply(rn.red, dt, "accu[" + std::to_string(u) + "]", "(" + ACC + ")" + vv) << ";\n" << pad << "  }\n" << pad << "}\n";
+          };
+          auto loads = [&](const std::string& pbexpr, int u, const std::string& pad) {
+            for (auto& sd : em.direct_vecs) {
+              const int slot = sd.first;
+              const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vecw) + ">";
+              o << pad << "const " << vt << " " << vec_name(slot, 0) << "u" << u << " = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + row * " << n << " + " << pbexpr << ");\n";
+            }
+          };
+          o << "  for (; pb + " << (U - 1) * TILE << " < pend; pb += " << U * TILE << ") {\n";
+          for (int u = 0; u < U; ++u) loads("pb + " + std::to_string(u * TILE), u, "    ");
+          for (int u = 0; u < U; ++u) one("pb + " + std::to_string(u * TILE), u, "    ");
+          o << "  }\n  for (; pb < pend; pb += " << TILE << ") {\n";
+          loads("pb", 0, "    ");
+          one("pb", 0, "    ");
+          o << "  }\n  " << ACC << " acc = accu[0];\n#pragma unroll\n  for (int u = 1; u < " << U << "; ++u) acc = " << red_apply(rn.red, dt, "acc", "accu[u]") << ";\n";
+        } else {
+          o << "  " << ACC << " acc = " << IDENT << ";\n";
+          o << "  for (" << it << " pb = c * " << CH << " + (" << it << ")threadIdx.x * " << V << "; pb < pend; pb += " << TILE << ") {\n";
+          o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+          o << "        const " << it << " j = " << jexpr << ";\n" << body;
+          o << "        acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n      }\n    }\n  }\n";
+        }
         o << "  acc = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(acc, " << OP << ", lds);\n";
         o << "  if (threadIdx.x == 0) tot[row * " << NC << " + c] = acc;\n}\n\n";
       }
@@ -2023,6 +2080,7 @@ struct Planner {
       o << "  for (" << it << " tb = c * " << CH << "; tb < pend; tb += " << TILE << ") {\n";
       o << "    const " << it << " pb = tb + (" << it << ")threadIdx.x * " << V << ";\n";
       o << "    " << ACC << " v[" << V << "];\n";
+      preload(o, "    ");
       o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      v[l] = " << IDENT << ";\n      if (p < pend) {\n";
       o << "        const " << it << " j = " << jexpr << ";\n" << body;
       o << "        v[l] = (" << ACC << ")" << val << ";\n      }\n    }\n";
@@ -2034,9 +2092,17 @@ struct Planner {
       o << "      if (i > 0) total = " << red_apply(rn.red, dt, "total", "wsum[i]") << ";\n    }\n";
       o << "    const " << ACC << " below = rx_lane_from(incl, (rx_u32)(lane - 1) & 63u);\n";
       o << "    if (lane > 0) pre = " << red_apply(rn.red, dt, "pre", "below") << ";\n";
-      o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
-      o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pre", "v[l]") << ";\n";
-      o << "        out0[row * " << n << " + (" << jexpr << ")] = " << Emitter::store_conv(dt, rv) << ";\n      }\n    }\n";
+      if (vecw > 1) {
+        o << "    if (pb < pend) {\n      rx_vec<" << ost << ", " << V << "> res;\n";
+        o << "#pragma unroll\n      for (int l = 0; l < " << V << "; ++l) {\n";
+        o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pre", "v[l]") << ";\n";
+        o << "        res.v[l] = " << Emitter::store_conv(dt, rv) << ";\n      }\n";
+        o << "      *reinterpret_cast<rx_vec<" << ost << ", " << V << ">*>(out0 + lin0) = res;\n    }\n";
+      } else {
+        o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+        o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pre", "v[l]") << ";\n";
+        o << "        out0[row * " << n << " + (" << jexpr << ")] = " << Emitter::store_conv(dt, rv) << ";\n      }\n    }\n";
+      }
       o << "    carry = " << red_apply(rn.red, dt, "carry", "total") << ";\n  }\n}\n\n";
       L1.grid[0] = L2.grid[0] = (unsigned)(NC * outer);
     } else {
