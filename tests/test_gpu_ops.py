@@ -438,3 +438,32 @@ def test_softmax_over_short_rows(rx, client, rows, cols):
     assert np.allclose(got[0].a.sum(axis=1), 1.0, atol=1e-5)
     ref = oracle_run(text, [I.Tensor(x, "f32")], hifi=True)
     assert np.max(np.abs(got[0].a - ref[0].a)) <= 2e-6
+
+
+def test_reshapes_that_share_a_buffer(rx, client):
+    """A reshape of a value that owns a buffer costs no launch; results stay independent buffers."""
+    t = ("module {\n func.func @main(%arg0: tensor<6x4xf32>) -> (tensor<24xf32>, tensor<3x8xf32>, tensor<2x12xf32>, tensor<4x6xf32>, tensor<6x4xf32>) {\n"
+         "  %0 = stablehlo.reshape %arg0 : (tensor<6x4xf32>) -> tensor<24xf32>\n"             # reshape of an argument: a copy
+         "  %1 = stablehlo.exponential %arg0 : tensor<6x4xf32>\n"
+         "  %2 = stablehlo.reshape %1 : (tensor<6x4xf32>) -> tensor<3x8xf32>\n"              # shares the temporary
+         "  %3 = stablehlo.reshape %1 : (tensor<6x4xf32>) -> tensor<2x12xf32>\n"             # second result on the same value: its own copy
+         "  %4 = stablehlo.negate %arg0 : tensor<6x4xf32>\n"
+         "  %5 = stablehlo.reshape %4 : (tensor<6x4xf32>) -> tensor<4x6xf32>\n"              # the value itself is returned too
+         "  return %0, %2, %3, %5, %4 : tensor<24xf32>, tensor<3x8xf32>, tensor<2x12xf32>, tensor<4x6xf32>, tensor<6x4xf32>\n }\n}\n")
+    x = I.tensor(np.random.default_rng(0).normal(size=(6, 4)), "f32")
+    got, exe = gpu_run(rx, client, t, [x])
+    ref = oracle_run(t, [x])
+    for g, r in zip(got, ref):
+        assert g.a.shape == r.a.shape
+        assert np.allclose(g.a, r.a, rtol=1e-6)
+    assert len(exe.launches()) == 5          # copy, exp, copy of exp, negate, copy of negate; one reshape is free
+    # a reshape between two kernels is always free
+    t2 = ("module {\n func.func @main(%arg0: tensor<64x32xf32>, %arg1: tensor<16x128xf32>) -> tensor<16x16xf32> {\n"
+          "  %0 = stablehlo.exponential %arg0 : tensor<64x32xf32>\n"
+          "  %1 = stablehlo.reshape %0 : (tensor<64x32xf32>) -> tensor<16x128xf32>\n"
+          "  %2 = stablehlo.dot_general %1, %arg1, contracting_dims = [1] x [1] : (tensor<16x128xf32>, tensor<16x128xf32>) -> tensor<16x16xf32>\n"
+          "  return %2 : tensor<16x16xf32>\n }\n}\n")
+    a = [I.tensor(np.random.default_rng(1).normal(size=(64, 32)), "f32"), I.tensor(np.random.default_rng(2).normal(size=(16, 128)), "f32")]
+    got, exe = gpu_run(rx, client, t2, a)
+    assert len(exe.launches()) == 2
+    assert max_rel_to_scale(got[0].a, oracle_run(t2, a, hifi=True)[0].a) <= 1e-5
