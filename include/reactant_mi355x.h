@@ -131,8 +131,9 @@ int RxExecutableNumLaunches(RxExecutable *exec);
 int RxExecutableNumResults(RxExecutable *exec);
 void RxExecutableLaunchInfo(RxExecutable *exec, int index, const char **kernel, const char **kind,
                             double *algorithmic_bytes, double *flops);
-/* XLAExecuteSharded with a HIP event pair around every kernel launch (on the
- * stream the kernels run on); launch_ms has RxExecutableNumLaunches entries. */
+/* XLAExecuteSharded with a HIP event pair attached to every kernel launch (start and stop
+ * of the dispatch itself, on the stream the kernels run on); launch_ms has
+ * RxExecutableNumLaunches entries. */
 void RxExecuteTimed(RxExecutable *exec, int num_args, RxBuffer **op_args, RxDevice *device,
                     uint8_t *is_arg_donatable, int num_results, RxBuffer **op_results, float *launch_ms);
 /* The same event pairs without blocking: the call returns as soon as the launches are queued

@@ -1,6 +1,7 @@
 // Runtime (client, device, buffers, executables, futures) and the C ABI declared
 // in include/reactant_mi355x.h.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 
 #include <atomic>
@@ -323,11 +324,13 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     ~EventList() { for (auto e : v) if (e) (void)hipEventDestroy(e); }
   } evlist;
   std::vector<hipEvent_t>& evs = evlist.v;
+  // A timed execution gives every launch its own start and stop event, attached to the dispatch
+  // itself (hipExtModuleLaunchKernel): the pair reads the kernel's own begin and end time stamps and
+  // puts no marker packets between the kernels.
   const bool timed = launch_ms || profile_async;
   if (timed) {
-    evs.assign(P.launches.size() + 1, nullptr);
+    evs.assign(2 * P.launches.size(), nullptr);
     for (auto& e : evs) HIP_CHECK(hipEventCreate(&e));
-    HIP_CHECK(hipEventRecord(evs[0], dev->stream));
   }
   std::vector<void*> ptrs;
   std::vector<void*> argv;
@@ -345,10 +348,17 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     }
     for (auto& p : ptrs) argv.push_back(&p);
     // a kernel over an empty tensor has no workgroups: nothing to launch
-    if (L.grid[0] != 0 && L.grid[1] != 0 && L.grid[2] != 0)
+    const bool empty = L.grid[0] == 0 || L.grid[1] == 0 || L.grid[2] == 0;
+    if (timed && !empty) {
+      HIP_CHECK(hipExtModuleLaunchKernel(ex->fns[li], L.grid[0] * L.block[0], L.grid[1] * L.block[1], L.grid[2] * L.block[2], L.block[0], L.block[1],
+                                         L.block[2], L.lds_bytes, dev->stream, argv.data(), nullptr, evs[2 * li], evs[2 * li + 1], 0));
+    } else if (timed) {
+      HIP_CHECK(hipEventRecord(evs[2 * li], dev->stream));
+      HIP_CHECK(hipEventRecord(evs[2 * li + 1], dev->stream));
+    } else if (!empty) {
       HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
                                       argv.data(), nullptr));
-    if (timed) HIP_CHECK(hipEventRecord(evs[li + 1], dev->stream));
+    }
     for (int b : L.args) {
       const auto& B = P.buffers[b];
       if (B.last_use == (int)li && !is_res[b]) bufs[b].reset();
@@ -381,8 +391,8 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     }
   }
   if (launch_ms) {
-    HIP_CHECK(hipEventSynchronize(evs.back()));
-    for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[li], evs[li + 1]));
+    if (!evs.empty()) HIP_CHECK(hipEventSynchronize(evs.back()));
+    for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[2 * li], evs[2 * li + 1]));
   } else if (profile_async) {
     ex->pending_events.push_back(std::move(evs));   // read later by RxExecutableTakeTimings
     evs.clear();
@@ -739,10 +749,10 @@ RX_EXPORT int RxExecutableTakeTimings(RxExecutable* ex, double* launch_ms_sum) {
     int runs = 0;
     HIP_CHECK(hipSetDevice(ex->device->ordinal));
     for (auto& evs : ex->pending_events) {
-      HIP_CHECK(hipEventSynchronize(evs.back()));
+      if (!evs.empty()) HIP_CHECK(hipEventSynchronize(evs.back()));
       for (size_t li = 0; li < nl; ++li) {
         float ms = 0.f;
-        HIP_CHECK(hipEventElapsedTime(&ms, evs[li], evs[li + 1]));
+        HIP_CHECK(hipEventElapsedTime(&ms, evs[2 * li], evs[2 * li + 1]));
         launch_ms_sum[li] += ms;
       }
       for (auto& e : evs) (void)hipEventDestroy(e);
