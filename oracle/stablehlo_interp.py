@@ -41,6 +41,8 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       test/core/map_reduction.jl:165-229), brute-force loops over the reference's
       groups x stride x padding x dilation grid, scipy.signal.correlate2d / convolve2d,
       numpy accumulate (tests/test_oracle_windows.py)
+  reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy
+      max / argmax / argmin with ties, first and last index
   batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
       (zero mean / unit variance of the normalized batch, numpy mean and var, the affine
       special case); the reference holds no known answer for them
@@ -618,7 +620,9 @@ class Parser:
             src = op.attrs.pop("__dense_src__")
             cc = _Cursor(src)
             op.attrs["value"] = _parse_dense(cc.balanced("<", ">"), op.types_out[0])
-        if op.name in ("reduce", "reduce_window"):
+        if op.name == "reduce":
+            op.attrs["body"] = _reduce_body_kind(op.regions[0], len(op.operands) // 2)
+        if op.name == "reduce_window":
             op.attrs["body"] = _reduce_body_kind(op.regions[0])
         return op
 
@@ -808,16 +812,20 @@ class Parser:
             op.types_out = [c.type()]
             return op
         if short == "reduce":
-            c.expect("(")
+            # (%x init: %c) or, for several operands, (%x init: %c), (%y init: %d)
             inputs, inits = [], []
             while True:
-                inputs.append(c.ssa())
-                c.expect("init")
-                c.expect(":")
-                inits.append(c.ssa())
+                c.expect("(")
+                while True:
+                    inputs.append(c.ssa())
+                    c.expect("init")
+                    c.expect(":")
+                    inits.append(c.ssa())
+                    if not c.accept(","):
+                        break
+                c.expect(")")
                 if not c.accept(","):
                     break
-            c.expect(")")
             op.operands = inputs + inits
             if c.accept("applies"):
                 body = c.ident()
@@ -836,21 +844,27 @@ class Parser:
                 c.expect(":")
                 self.fn_type(op)
                 c.expect("reducer")
-                c.expect("(")
-                args = []
-                while not c.accept(")"):
-                    nm = c.ssa()
-                    c.expect(":")
-                    t = c.type()
-                    c.skip_loc()
-                    args.append((nm, t))
-                    c.accept(",")
+                # one (lhs, rhs) group per reduced operand; the region's arguments are all lhs, then all rhs
+                lhs, rhs = [], []
+                while c.accept("("):
+                    grp = []
+                    while not c.accept(")"):
+                        nm = c.ssa()
+                        c.expect(":")
+                        t = c.type()
+                        c.skip_loc()
+                        grp.append((nm, t))
+                        c.accept(",")
+                    if len(grp) != 2:
+                        raise ParseError("reducer group with %d arguments" % len(grp))
+                    lhs.append(grp[0])
+                    rhs.append(grp[1])
                 c.expect("{")
                 lab = Op("__block_args__")
-                lab.attrs["args"] = args
+                lab.attrs["args"] = lhs + rhs
                 region = [lab] + self.block()
                 op.regions.append(region)
-                op.attrs["body"] = _reduce_body_kind(region)
+                op.attrs["body"] = _reduce_body_kind(region, len(inputs))
             return op
         if short in ("dot_general", "dot"):
             op.operands.append(c.ssa())
@@ -978,10 +992,12 @@ def _parse_conv_dims(text):
     return out
 
 
-def _reduce_body_kind(region):
+def _reduce_body_kind(region, ninputs=1):
     body = [o for o in region if o.name not in ("__block_args__", "return")]
-    if len(body) == 1 and body[0].name in ("add", "multiply", "maximum", "minimum", "and", "or"):
+    if ninputs == 1 and len(body) == 1 and body[0].name in ("add", "multiply", "maximum", "minimum", "and", "or"):
         return body[0].name
+    if ninputs > 1:
+        return "__region__"     # evaluated by folding the region over the reduced elements
     raise ParseError("reduce body is not a single monoid op")
 
 
@@ -1431,6 +1447,28 @@ class Interpreter:
                 raise ValueError("while body returns %d values for %d loop-carried ones" % (len(cur), len(op.operands)))
         raise ValueError("while loop did not terminate")
 
+    def _variadic_reduce(self, op, xs):
+        """stablehlo.reduce over several operands with an arbitrary body (argmax / findfirst,
+        reference src/Ops.jl:1536-1596): the region is folded over the reduced elements from the
+        init values, in row-major order of the reduced dims, on all kept positions at once."""
+        k = len(xs) // 2
+        ins, inits = xs[:k], xs[k:]
+        dims = sorted(op.attrs["dimensions"])
+        shape = ins[0].a.shape
+        kept = [d for d in range(len(shape)) if d not in dims]
+        kshape = [shape[d] for d in kept]
+        flat = [np.transpose(t.a, kept + dims).reshape(kshape + [-1]) for t in ins]
+        acc = [Tensor(np.broadcast_to(i.a, kshape).copy(), i.dt) for i in inits]
+        region = op.regions[0]
+        names = [nm for nm, _ in region[0].attrs["args"]] if region[0].name == "__block_args__" else []
+        body = [self._retarget(o, tuple(kshape)) for o in region if o.name != "__block_args__"]
+        for j in range(flat[0].shape[-1]):
+            env = {}
+            vals = acc + [Tensor(f[..., j], t.dt) for f, t in zip(flat, ins)]
+            env.update(zip(names, vals))
+            acc = [_rounded(v) for v in self._block(body, env)]
+        return acc
+
     def _eval(self, op, xs):
         n, at = op.name, op.attrs
         if n == "constant":
@@ -1504,6 +1542,8 @@ class Interpreter:
             shp[d] = t.shape[d]
             r = np.broadcast_to(np.arange(t.shape[d]).reshape(shp), t.shape)
             return [tensor(r, t.dt) if is_float(t.dt) else Tensor(r.astype(NP_OF[t.dt]), t.dt)]
+        if n == "reduce" and len(xs) != 2:
+            return self._variadic_reduce(op, xs)
         if n == "reduce":
             if len(xs) != 2:
                 raise NotImplementedError("variadic reduce")

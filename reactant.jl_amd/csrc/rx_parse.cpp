@@ -865,15 +865,18 @@ struct P {
       return o;
     }
     if (sh == "reduce") {
-      c.expect("(");
+      // (%x init: %c) or, for several operands, (%x init: %c), (%y init: %d)
       std::vector<std::string> ins, inits;
       do {
-        ins.push_back(c.ssa());
-        c.expect("init");
-        c.expect(":");
-        inits.push_back(c.ssa());
+        c.expect("(");
+        do {
+          ins.push_back(c.ssa());
+          c.expect("init");
+          c.expect(":");
+          inits.push_back(c.ssa());
+        } while (c.accept(","));
+        c.expect(")");
       } while (c.accept(","));
-      c.expect(")");
       o.operands = ins;
       o.operands.insert(o.operands.end(), inits.begin(), inits.end());
       if (c.accept("applies")) {
@@ -896,15 +899,24 @@ struct P {
         c.expect("reducer");
         RawOp lab;
         lab.name = "__block_args__";
-        c.expect("(");
-        while (!c.accept(")")) {
-          std::string nm = c.ssa();
-          c.expect(":");
-          TType t = c.type();
-          c.skip_loc();
-          lab.block_args.push_back({nm, t});
-          c.accept(",");
+        // one (lhs, rhs) group per reduced operand; the region's arguments are all lhs, then all rhs
+        std::vector<std::pair<std::string, TType>> lhs, rhs;
+        while (c.accept("(")) {
+          std::vector<std::pair<std::string, TType>> grp;
+          while (!c.accept(")")) {
+            std::string nm = c.ssa();
+            c.expect(":");
+            TType t = c.type();
+            c.skip_loc();
+            grp.push_back({nm, t});
+            c.accept(",");
+          }
+          if (grp.size() != 2) throw Error("StableHLO import: reducer group must name two arguments");
+          lhs.push_back(grp[0]);
+          rhs.push_back(grp[1]);
         }
+        lab.block_args = lhs;
+        lab.block_args.insert(lab.block_args.end(), rhs.begin(), rhs.end());
         c.expect("{");
         std::vector<RawOp> region;
         region.push_back(std::move(lab));
@@ -1430,6 +1442,99 @@ struct Builder {
     return {res};
   }
 
+  // The reduce over (value, index) pairs that argmax / argmin / findmax / findmin print
+  // (reference src/Ops.jl:1571-1596): body `c = a1 <dir> a2; return select(c, a1, a2), select(c, i1, i2)`
+  // with the indices an iota along the one reduced dimension.  It becomes two monoid reductions:
+  // the extreme value, then the first (non-strict comparison) or last (strict) index that holds it.
+  // A slice in which no element equals the extreme (NaNs) gets the largest / smallest index value.
+  std::vector<int> build_arg_reduce(const RawOp& o, const std::vector<int>& in) {
+    const char* what = "reduce over two operands: only the argmax / argmin form (compare, select, select over a value and an iota) is supported";
+    if (o.regions.empty() || o.tout.size() != 2) fail(what);
+    const auto& region = o.regions[0];
+    if (region.empty() || region[0].name != "__block_args__" || region[0].block_args.size() != 4) fail(what);
+    const std::string a1 = region[0].block_args[0].first, i1 = region[0].block_args[1].first, a2 = region[0].block_args[2].first,
+                      i2 = region[0].block_args[3].first;
+    std::vector<const RawOp*> body;
+    for (size_t k = 1; k < region.size(); ++k) body.push_back(&region[k]);
+    if (body.size() != 4) fail(what);
+    auto short_name = [](const RawOp& r) { return r.name.rfind("stablehlo.", 0) == 0 ? r.name.substr(10) : r.name; };
+    const RawOp &cmp = *body[0], &s0 = *body[1], &s1 = *body[2], &ret = *body[3];
+    if (short_name(cmp) != "compare" || short_name(s0) != "select" || short_name(s1) != "select" || short_name(ret) != "return") fail(what);
+    if (cmp.operands.size() != 2 || cmp.operands[0] != a1 || cmp.operands[1] != a2 || cmp.results.size() != 1) fail(what);
+    const std::string c = cmp.results[0];
+    const RawOp *sv = nullptr, *si = nullptr;
+    for (const RawOp* sel : {&s0, &s1}) {
+      if (sel->operands.size() != 3 || sel->operands[0] != c || sel->results.size() != 1) fail(what);
+      if (sel->operands[1] == a1 && sel->operands[2] == a2) sv = sel;
+      else if (sel->operands[1] == i1 && sel->operands[2] == i2) si = sel;
+    }
+    if (!sv || !si || ret.operands.size() != 2 || ret.operands[0] != sv->results[0] || ret.operands[1] != si->results[0]) fail(what);
+    const std::string dir = cmp.sa.count("direction") ? cmp.sa.at("direction") : "";
+    const bool is_max = dir == "GE" || dir == "GT", is_min = dir == "LE" || dir == "LT";
+    if (!is_max && !is_min) fail(what);
+    const bool first = dir == "GE" || dir == "LE";
+    const std::vector<int64_t> dims = o.ia.at("dimensions");
+    const Node& idx = g.nodes[in[1]];
+    if (dims.size() != 1 || idx.k != OpK::Iota || idx.a0.empty() || idx.a0[0] != dims[0]) fail(what);
+    const TType xt = ty(in[0]), it = ty(in[1]);
+    if (xt.dims != it.dims || !is_int_dt(it.dt) || it.dt == DT::I1 || ty(in[2]).rank() != 0 || ty(in[3]).rank() != 0) fail(what);
+    std::vector<int64_t> kept;
+    for (int k = 0; k < xt.rank(); ++k) if (k != dims[0]) kept.push_back(xt.dims[k]);
+    if (o.tout[0].dims != kept || o.tout[1].dims != kept || o.tout[0].dt != xt.dt || o.tout[1].dt != it.dt) fail("reduce: result type mismatch");
+    Node m;
+    m.k = OpK::Reduce;
+    m.red = is_max ? Red::Max : Red::Min;
+    m.in = {in[0], in[2]};
+    m.a0 = dims;
+    m.ty = o.tout[0];
+    const int mv = g.add(m);
+    // positions that hold the extreme keep their index, the others the neutral index
+    Node mb;
+    mb.k = OpK::BroadcastInDim;
+    mb.in = {mv};
+    mb.ty = xt;
+    for (int k = 0; k < xt.rank(); ++k) if (k != dims[0]) mb.a0.push_back(k);
+    const int mbv = g.add(mb);
+    Node eq;
+    eq.k = OpK::Compare;
+    eq.op = "EQ";
+    eq.in = {in[0], mbv};
+    eq.ty = TType{DT::I1, xt.dims};
+    const int eqv = g.add(eq);
+    Node lim;
+    lim.k = OpK::Constant;
+    lim.splat = true;
+    lim.ty = TType{it.dt, {}};
+    lim.data.assign((size_t)info(it.dt).size, 0);
+    {
+      const int bits = 8 * info(it.dt).size;
+      const bool sgn = info(it.dt).is_signed;
+      uint64_t v;
+      if (first) v = sgn ? ((uint64_t)1 << (bits - 1)) - 1 : (bits == 64 ? ~(uint64_t)0 : ((uint64_t)1 << bits) - 1);
+      else v = sgn ? (uint64_t)1 << (bits - 1) : 0;   // smallest value (two's complement bit pattern)
+      memcpy(lim.data.data(), &v, (size_t)info(it.dt).size);
+    }
+    const int limv = g.add(lim);
+    Node limb;
+    limb.k = OpK::BroadcastInDim;
+    limb.in = {limv};
+    limb.ty = it;
+    const int limbv = g.add(limb);
+    Node sel;
+    sel.k = OpK::Select;
+    sel.in = {eqv, in[1], limbv};
+    sel.ty = it;
+    const int selv = g.add(sel);
+    Node r;
+    r.k = OpK::Reduce;
+    r.red = first ? Red::Min : Red::Max;
+    r.in = {selv, limv};
+    r.a0 = dims;
+    r.ty = o.tout[1];
+    (void)in[3];
+    return {mv, g.add(r)};
+  }
+
   struct ConvDims { int d0 = -1, d1 = -1; std::vector<int> sp; };
   // "[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]": position of the two named roles and of every spatial dim
   static void parse_conv_dims(const std::string& text, ConvDims out[3]) {
@@ -1863,8 +1968,9 @@ struct Builder {
       n.a0 = o.ia.count("iota_dimension") ? o.ia.at("iota_dimension") : o.ia.at("dimension");
       return {g.add(n)};
     }
+    if (sh == "reduce" && in.size() == 4) return build_arg_reduce(o, in);
     if (sh == "reduce") {
-      if (in.size() != 2) fail("variadic reduce is not supported");
+      if (in.size() != 2) fail("reduce over more than two operands is not supported");
       n.k = OpK::Reduce;
       n.ty = out1();
       n.a0 = o.ia.at("dimensions");

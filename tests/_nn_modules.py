@@ -226,3 +226,32 @@ def attention_block(batch_heads=6, seq=40, dim=16, dt="f32"):
     ]
     sig = ", ".join("%%arg%d: %s" % (k, Q) for k in range(3))
     return ("module {\n  func.func @main(%s) -> %s {\n    %s\n    return %%out : %s\n  }\n}\n" % (sig, Q, "\n    ".join(lines), Q)), [[batch_heads, seq, dim]] * 3
+
+
+def argreduce(shape, dt, dim, direction="GE", idt="i64", generic=False):
+    """The variadic reduce that argmax / argmin / findmax print (reference src/Ops.jl:1571-1596):
+    (value, index) pairs over `dim`, keeping the left pair when `a1 <direction> a2`.  Returns the
+    module text; results are (values, zero-based indices)."""
+    out = [s for d, s in enumerate(shape) if d != dim]
+    tx, ti, tvo, tio = tt(shape, dt), tt(shape, idt), tt(out, dt), tt(out, idt)
+    sv, si = tt([], dt), tt([], idt)
+    vinit = _init_literal("maximum" if direction in ("GE", "GT") else "minimum", dt)
+    if generic:
+        red = ("    %%r:2 = \"stablehlo.reduce\"(%%arg0, %%io, %%cv, %%ci) <{dimensions = array<i64: %d>}> ({\n"
+               "    ^bb0(%%a1: %s, %%i1: %s, %%a2: %s, %%i2: %s):\n" % (dim, sv, si, sv, si))
+        tail = "    }) : (%s, %s, %s, %s) -> (%s, %s)\n" % (tx, ti, sv, si, tvo, tio)
+    else:
+        red = ("    %%r:2 = stablehlo.reduce(%%arg0 init: %%cv), (%%io init: %%ci) across dimensions = [%d] : (%s, %s, %s, %s) -> (%s, %s)\n"
+               "     reducer(%%a1: %s, %%a2: %s) (%%i1: %s, %%i2: %s)  {\n" % (dim, tx, ti, sv, si, tvo, tio, sv, sv, si, si))
+        tail = "    }\n"
+    body = ("      %%c = stablehlo.compare %s, %%a1, %%a2 : (%s, %s) -> tensor<i1>\n"
+            "      %%v = stablehlo.select %%c, %%a1, %%a2 : tensor<i1>, %s\n"
+            "      %%i = stablehlo.select %%c, %%i1, %%i2 : tensor<i1>, %s\n"
+            "      stablehlo.return %%v, %%i : %s, %s\n" % (direction, sv, sv, sv, si, sv, si))
+    return ("module {\n  func.func @main(%%arg0: %s) -> (%s, %s) {\n"
+            "    %%io = stablehlo.iota dim = %d : %s\n"
+            "    %%cv = stablehlo.constant dense<%s> : %s\n"
+            "    %%ci = stablehlo.constant dense<-1> : %s\n"
+            "%s%s%s"
+            "    return %%r#0, %%r#1 : %s, %s\n  }\n}\n"
+            % (tx, tvo, tio, dim, ti, vinit, sv, si, red, body, tail, tvo, tio))

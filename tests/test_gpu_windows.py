@@ -279,3 +279,27 @@ def test_degenerate_windows(rx, client, name, make):
     ref = oracle_run(text, args, hifi=True)
     assert got[0].a.shape == ref[0].a.shape
     assert np.allclose(got[0].a, ref[0].a, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,dt,dim,direction,generic", [
+    ([2, 3], "f64", 0, "GE", False), ([2, 3], "f64", 1, "LE", False),          # the shapes of test/core/sorting.jl:109-139
+    ([4, 3, 2], "f64", 0, "GE", False), ([4, 3, 2], "f64", 1, "GE", True), ([4, 3, 2], "f64", 2, "LE", False),
+    ([4096, 1000], "f32", 1, "GE", False), ([4096, 1000], "f32", 0, "LE", True), ([100000], "f32", 0, "GE", False),
+    ([64, 50, 30], "bf16", 1, "GT", False), ([300, 70], "i32", 1, "LT", False),
+])
+def test_argmax_and_argmin(rx, client, shape, dt, dim, direction, generic):
+    """The (value, index) reduce of argmax / argmin / findmax (src/Ops.jl:1571-1596), with many ties."""
+    text = NN.argreduce(shape, dt, dim, direction, generic=generic)
+    rng = np.random.default_rng(31)
+    if dt == "i32":
+        x = I.Tensor(rng.integers(-3, 4, size=shape).astype(np.int32), dt)
+    else:
+        x = I.tensor(rng.integers(-8, 9, size=shape) / 4.0, dt)
+    got, exe = gpu_run(rx, client, text, [x])
+    ref = oracle_run(text, [x])
+    assert len(got) == 2
+    assert np.array_equal(got[0].a, ref[0].a)
+    assert np.array_equal(got[1].a, ref[1].a)
+    lib = np.argmax if direction in ("GE", "GT") else np.argmin
+    if direction in ("GE", "LE"):
+        assert np.array_equal(got[1].a, lib(x.a, axis=dim))

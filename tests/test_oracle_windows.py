@@ -187,3 +187,20 @@ def test_batch_norm_closed_forms():
     s, b = rng.normal(size=5), rng.normal(size=5)
     got = I.run_text(NN.batch_norm([6, 5, 7], "f64", 1, 0.25), [I.tensor(a, "f64") for a in (x, s, b, zeros, ones * 0.75)])[0].a
     assert np.allclose(got, x * s[None, :, None] + b[None, :, None], rtol=1e-13, atol=1e-13)
+
+
+def test_argmax_reduce_against_numpy():
+    """findmax / argmax arrive as a reduce over (value, index) pairs (src/Ops.jl:1571-1596); the
+    folded region must agree with numpy's max / argmax (first index on ties) along every dim."""
+    rng = np.random.default_rng(9)
+    x = rng.integers(0, 5, size=(4, 6, 5)).astype(np.float64)        # many ties
+    for dim in range(3):
+        for generic in (False, True):
+            v, i = [t.a for t in I.run_text(NN.argreduce([4, 6, 5], "f64", dim, "GE", generic=generic), [I.tensor(x, "f64")])]
+            assert np.array_equal(v, x.max(axis=dim)) and np.array_equal(i, x.argmax(axis=dim))
+        v, i = [t.a for t in I.run_text(NN.argreduce([4, 6, 5], "f64", dim, "LE"), [I.tensor(x, "f64")])]
+        assert np.array_equal(v, x.min(axis=dim)) and np.array_equal(i, x.argmin(axis=dim))
+        # the strict comparison keeps the later of two equal values
+        v, i = [t.a for t in I.run_text(NN.argreduce([4, 6, 5], "f64", dim, "GT"), [I.tensor(x, "f64")])]
+        last = x.shape[dim] - 1 - np.flip(x, axis=dim).argmax(axis=dim)
+        assert np.array_equal(v, x.max(axis=dim)) and np.array_equal(i, last)
