@@ -573,3 +573,113 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
     }
   }
 }
+
+// ---------------------------------------------------------------------------
+// f64 operands: v_mfma_f64_16x16x4_f64, f64 accumulation.  Same tiling, tile order, operand
+// layouts and epilogue interface as rx_gemm_body; a wavefront owns (BM/WM) x (BN/WN) as a grid of
+// 16x16 MFMA tiles.  One fragment is two k values per lane (one 16-byte LDS read where k is
+// contiguous): lane group g = lane / 16 takes k = 2g for the first MFMA of a pair and k = 2g + 1
+// for the second; A and B use the same assignment, which is all a contraction needs.  The B
+// fragment is the row operand, with its rows permuted so that a lane ends with four consecutive n of one m.
+// ---------------------------------------------------------------------------
+typedef double rx_f64x2 __attribute__((ext_vector_type(2)));
+typedef double rx_f64x4 __attribute__((ext_vector_type(4)));
+
+template <int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
+RX_DEV void rx_gemm_body_f64(const double* __restrict__ A, const double* __restrict__ B, const Epi& epi) {
+  typedef double E;
+  constexpr int NT = WM * WN * 64;
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;   // 16x16 tiles per wavefront
+  constexpr int PAD = 2, KS = 8;
+  static_assert(BK % KS == 0 && (BM / WM) % 16 == 0 && (BN / WN) % 16 == 0, "tile shape");
+  constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BK : BM;
+  constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BK : BN;
+  constexpr int A_LD = A_COLS + PAD, B_LD = B_COLS + PAD;
+  constexpr int A_SZ = A_ROWS * A_LD, B_SZ = B_ROWS * B_LD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
+  RX_LDS E* lds = (RX_LDS E*)rx_smem;
+  constexpr int STAGE = A_SZ + B_SZ;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  constexpr int GM = (M + BM - 1) / BM, GN = (N + BN - 1) / BN;
+  int bm, bn;
+  if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
+  const int m0 = bm * BM, n0 = bn * BN;
+  const long long batch = BATCHED ? blockIdx.y : 0;
+  const E* Ab = A + batch * (long long)M * K;
+  const E* Bb = B + batch * (long long)N * K;
+  constexpr long long A_GLD = A_KC ? K : M, B_GLD = B_KC ? K : N;
+
+  rx_f64x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = rx_f64x4{0.0, 0.0, 0.0, 0.0};
+
+  rx_tile_copy<E, A_ROWS, A_COLS, NT> ca;
+  rx_tile_copy<E, B_ROWS, B_COLS, NT> cb;
+  auto gload = [&](int k0) {
+    constexpr bool TAIL = K % BK != 0;
+    if (A_KC) ca.template load<false, TAIL>(Ab, A_GLD, m0, k0, M, K, tid); else ca.template load<TAIL, false>(Ab, A_GLD, k0, m0, K, M, tid);
+    if (B_KC) cb.template load<false, TAIL>(Bb, B_GLD, n0, k0, N, K, tid); else cb.template load<TAIL, false>(Bb, B_GLD, k0, n0, K, N, tid);
+  };
+  // The two k values of this lane for the fragment at k offset kk, operand row/column o + idx.
+  // The instruction leaves row 4*r + lane/16 of its row operand in accumulator register r; feeding
+  // it row 4*(i%4) + i/4 of the B tile from lane i makes those four rows consecutive n.
+  const int idx_a = lane & 15, idx_b = 4 * (lane & 3) + ((lane & 15) >> 2);
+  auto frag = [&](const RX_LDS E* t, int ld, bool kc, int o, int kk, int idx) {
+    const int r = o + idx, k = kk + 2 * (lane >> 4);
+    if (kc) return *(const RX_LDS rx_f64x2*)(t + r * ld + k);
+    rx_f64x2 f;
+    f[0] = t[k * ld + r];
+    f[1] = t[(k + 1) * ld + r];
+    return f;
+  };
+  gload(0);
+  ca.store(lds, A_LD, tid);
+  cb.store(lds + A_SZ, B_LD, tid);
+  __syncthreads();
+
+  constexpr int KT = (K + BK - 1) / BK;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < KT) gload((kt + 1) * BK);
+    const RX_LDS E* sa = lds + cur * STAGE;
+    const RX_LDS E* sb = sa + A_SZ;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += KS) {
+      rx_f64x2 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = frag(sa, A_LD, A_KC, wm * (BM / WM) + 16 * i, kk, idx_a);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[j] = frag(sb, B_LD, B_KC, wn * (BN / WN) + 16 * j, kk, idx_b);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fb[j][0], fa[i][0], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fb[j][1], fa[i][1], acc[i][j], 0, 0, 0);
+        }
+    }
+    if (kt + 1 < KT) {
+      ca.store(lds + (cur ^ 1) * STAGE, A_LD, tid);
+      cb.store(lds + (cur ^ 1) * STAGE + A_SZ, B_LD, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds D[n = 4*(lane/16) + r][m = lane%16] of each 16x16 tile
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * (BM / WM) + 16 * i + (lane & 15);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * (BN / WN) + 16 * j + 4 * (lane >> 4);
+      if (m < M && n < N) {
+        const double v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+        if constexpr (BATCHED) epi(v, (int)batch, m, n); else epi(v, m, n);
+      }
+    }
+  }
+}

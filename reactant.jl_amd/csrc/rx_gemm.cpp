@@ -5,9 +5,53 @@
 
 namespace rx {
 
+// f64: the register-staged skeleton on v_mfma_f64_16x16x4_f64
+static GemmChoice choose_gemm_f64(int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc) {
+  GemmChoice c;
+  const int ve = 2, bk = 16;
+  if (K < 1 || ((a_kc || b_kc) && K % ve != 0)) return c;
+  if (N % 4 != 0 || M < 1 || N < 4) return c;
+  if (!a_kc && M % ve != 0) return c;
+  if (!b_kc && N % ve != 0) return c;
+  if (M * N < 64 * 64) return c;
+  if (M >= ((int64_t)1 << 30) || N >= ((int64_t)1 << 30) || K >= ((int64_t)1 << 30)) return c;
+  // 4096^3: 256x128 tiles on 8 wavefronts 60-62 TFLOP/s, 128x128 on 4 wavefronts 47, 64x64 52-54;
+  // 1024^3: 64x64 32, 128x128 11
+  int BM = 64, BN = 64, WM = 2, WN = 2;
+  if (((M + 255) / 256) * ((N + 127) / 128) * batch >= 256) { BM = 256; BN = 128; WM = 4; WN = 2; }
+  else if (((M + 127) / 128) * ((N + 127) / 128) * batch >= 512) { BM = 128; BN = 128; }
+  if (const char* e = getenv("RX_GEMM_TILE_F64")) {  // "BM,BN,WM,WN" for tuning runs
+    int v[4];
+    if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
+  }
+  int rb = 4, cb = 8;
+  const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
+  if (gm * gn < 64) rb = cb = 0;
+  else if (gm < rb) { cb = (int)(rb * cb / gm); rb = (int)gm; }
+  else if (gn < cb) { rb = (int)(rb * cb / gn); cb = (int)gn; }
+  const int pad = 2;
+  const int64_t a_sz = a_kc ? (int64_t)BM * (bk + pad) : (int64_t)bk * (BM + pad);
+  const int64_t b_sz = b_kc ? (int64_t)BN * (bk + pad) : (int64_t)bk * (BN + pad);
+  c.lds_bytes = (unsigned)(2 * (a_sz + b_sz) * 8);
+  if (c.lds_bytes > 160 * 1024) return c;
+  c.block = WM * WN * 64;
+  c.grid[0] = (unsigned)gemm_grid(gm, gn, rb, cb);
+  c.grid[1] = (unsigned)batch;
+  std::ostringstream t;
+  t << BM << ", " << BN << ", " << bk << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false")
+    << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
+  c.targs = t.str();
+  c.skeleton = "rx_gemm_body_f64";
+  c.stype_a = "double";
+  c.kind = "gemm_f64";
+  c.ok = true;
+  return c;
+}
+
 GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc) {
   GemmChoice c;
   if (a != b) return c;
+  if (a == DT::F64 && out == DT::F64) return choose_gemm_f64(batch, M, N, K, a_kc, b_kc);
   std::string mma;
   int esize = 0, bk = 0;
   if (a == DT::F32 && out == DT::F32) { mma = "rx_mma_f32"; c.kind = "gemm_f32"; esize = 4; bk = 16; }

@@ -42,6 +42,12 @@ for a_kc in (True, False):
     for b_kc in (True, False):
         CASES += [("f32", "f32", 200, 136, 52, a_kc, b_kc, 0), ("bf16", "f32", 136, 200, 72, a_kc, b_kc, 0),
                   ("f8E4M3FN", "f32", 144, 208, 176, a_kc, b_kc, 0)]
+# f64 on v_mfma_f64_16x16x4_f64: every operand order, tile edges, a K tail, batched
+for a_kc in (True, False):
+    for b_kc in (True, False):
+        CASES += [("f64", "f64", 128, 128, 64, a_kc, b_kc, 0), ("f64", "f64", 200, 136, 50, a_kc, b_kc, 0),
+                  ("f64", "f64", 72, 64, 16, a_kc, b_kc, 3)]
+CASES += [("f64", "f64", 512, 384, 256, True, False, 0), ("f64", "f64", 1000, 1000, 300, True, True, 0)]
 CASES += [("f32", "f32", 96, 128, 37, False, False, 0), ("bf16", "bf16", 128, 136, 1000, True, False, 0),
           ("f32", "f32", 1000, 1000, 1000, True, False, 0), ("f32", "f32", 128, 128, 8, True, True, 0)]
 CASES += [("f32", "f32", 128, 128, 32, True, False, 3), ("bf16", "bf16", 128, 128, 64, True, True, 2),
@@ -55,11 +61,13 @@ def test_dot_general_mfma(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
     b = I.tensor(np.random.default_rng(1).normal(size=b_shape), dt)
     got, exe = gpu_run(rx, client, text, [a, b])
     kinds = [l["kind"] for l in exe.launches()]
-    assert kinds == ["gemm_" + {"f32": "f32", "bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8"}[dt]], kinds
+    assert kinds == ["gemm_" + {"f32": "f32", "bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8", "f64": "f64"}[dt]], kinds
     ref = oracle_run(text, [a, b], hifi=True)
     err = max_rel_to_scale(got[0].a, ref[0].a)
     if out_dt in ("bf16", "f16"):
         assert err <= 1e-2
+    elif out_dt == "f64":
+        assert err <= 1e-14 * np.sqrt(K)
     else:
         assert err <= 1e-5 * np.sqrt(K)
 
