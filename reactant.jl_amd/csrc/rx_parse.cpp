@@ -1719,8 +1719,8 @@ struct Builder {
     // columns are sliced off the product).
     const int64_t K = I * taps, N = B * P;
     int64_t Kp = K, Np = N;
-    if (xct.dt == DT::F32 || xct.dt == DT::BF16 || xct.dt == DT::F16) {
-      const int64_t ve = 16 / info(xct.dt).size;
+    if (xct.dt == DT::F32 || xct.dt == DT::BF16 || xct.dt == DT::F16 || xct.dt == DT::F64) {
+      const int64_t ve = std::max<int64_t>(4, 16 / info(xct.dt).size);
       Kp = (K + ve - 1) / ve * ve;
       Np = (N + ve - 1) / ve * ve;
     }

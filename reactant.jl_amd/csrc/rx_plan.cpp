@@ -167,6 +167,87 @@ struct Planner {
       }
     }
     dots_to_reductions();
+    align_dots();
+  }
+
+  // A matrix product that misses the MFMA path only because a dimension is not a whole number of
+  // 16-byte vectors (an odd N, a K of 27) is padded with zeros to the next multiple and the
+  // padding sliced off the result: two small copies instead of the scalar loop.
+  void align_dots() {
+    if (!opt.mfma) return;
+    struct Fix { int64_t Mp, Np, Kp; };
+    std::map<int, Fix> fixes;
+    for (const Node& d : g.nodes) {
+      if (d.k != OpK::DotGeneral) continue;
+      DotForm f = dot_form(d);
+      if (!f.ok || d.ty.rank() < 2) continue;
+      const DT a = g.nodes[d.in[0]].ty.dt, b = g.nodes[d.in[1]].ty.dt;
+      if (a != b || !is_float(a) || a == DT::F8E5M2) continue;
+      if (choose_gemm(a, b, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig).ok) continue;
+      if ((double)f.M * (double)f.N * (double)f.K * (double)f.batch < (double)(1 << 22)) continue;   // small: the scalar loop will do
+      const int64_t ve = 16 / info(a).size;
+      auto up = [](int64_t x, int64_t m) { return (x + m - 1) / m * m; };
+      Fix fx;
+      fx.Kp = up(f.K, ve);
+      fx.Mp = f.a_k_contig ? f.M : up(f.M, ve);
+      fx.Np = up(f.N, f.b_k_contig ? 4 : std::max<int64_t>(4, ve));
+      if (fx.Kp == f.K && fx.Mp == f.M && fx.Np == f.N) continue;
+      if (!choose_gemm(a, b, d.ty.dt, f.batch, fx.Mp, fx.Np, fx.Kp, f.a_k_contig, f.b_k_contig).ok) continue;
+      fixes[d.id] = fx;
+    }
+    if (fixes.empty()) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(g.nodes.size(), -1);
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      for (int& i : c.in) i = remap[i];
+      auto fi = fixes.find(n.id);
+      if (fi == fixes.end()) { remap[n.id] = out.add(c); continue; }
+      const Fix& fx = fi->second;
+      DotForm f = dot_form(n);
+      const int nb = (int)n.a0.size();
+      auto padded = [&](int node, bool kc, int64_t rows_to, int64_t k_to) {
+        // operand dims [batch.., rows, K] (kc) or [batch.., K, rows]
+        const TType t = out.nodes[node].ty;
+        std::vector<int64_t> want = t.dims;
+        want[nb + (kc ? 0 : 1)] = rows_to;
+        want[nb + (kc ? 1 : 0)] = k_to;
+        if (want == t.dims) return node;
+        Node z;
+        z.k = OpK::Constant;
+        z.splat = true;
+        z.ty = TType{t.dt, {}};
+        z.data.assign((size_t)info(t.dt).size, 0);
+        const int zi = out.add(z);
+        Node pn;
+        pn.k = OpK::Pad;
+        pn.in = {node, zi};
+        pn.a0.assign(t.rank(), 0);
+        pn.a2.assign(t.rank(), 0);
+        for (int k = 0; k < t.rank(); ++k) pn.a1.push_back(want[k] - t.dims[k]);
+        pn.ty = TType{t.dt, want};
+        return out.add(pn);
+      };
+      c.in[0] = padded(c.in[0], f.a_k_contig, fx.Mp, fx.Kp);
+      c.in[1] = padded(c.in[1], f.b_k_contig, fx.Np, fx.Kp);
+      c.ty.dims[nb] = fx.Mp;
+      c.ty.dims[nb + 1] = fx.Np;
+      int cur = out.add(c);
+      Node sl;
+      sl.k = OpK::Slice;
+      sl.in = {cur};
+      sl.a0.assign(n.ty.rank(), 0);
+      sl.a1 = n.ty.dims;
+      sl.a2.assign(n.ty.rank(), 1);
+      sl.ty = n.ty;
+      remap[n.id] = out.add(sl);
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // A dot_general whose smaller operand has at most 8 free elements (matrix-vector, vector-matrix,
