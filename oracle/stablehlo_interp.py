@@ -41,6 +41,8 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       test/core/map_reduction.jl:165-229), brute-force loops over the reference's
       groups x stride x padding x dilation grid, scipy.signal.correlate2d / convolve2d,
       numpy accumulate (tests/test_oracle_windows.py)
+  gather (src/Ops.jl:2269-2345; NNlib.gather, ext/ReactantNNlibExt/Implementations.jl:426-438)
+      ... reference KATs (test/nn/scatter_gather.jl:5-99), numpy fancy indexing with clamping
   reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy
       max / argmax / argmin with ties, first and last index
   batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
@@ -557,6 +559,15 @@ class Parser:
         mo = re.search(r"#stablehlo\.conv<([^>]*->[^>]*)>", inner)
         if mo:
             a["dim_numbers"] = _parse_conv_dims(mo.group(1))
+        mo = re.search(r"#stablehlo\.gather<([^>]*)>", inner)
+        if mo:
+            d = mo.group(1)
+            for k in ("offset_dims", "collapsed_slice_dims", "operand_batching_dims", "start_indices_batching_dims",
+                      "start_index_map"):
+                m2 = re.search(k + r"\s*=\s*\[([-\d,\s]*)\]", d)
+                a[k] = [int(t) for t in m2.group(1).replace(",", " ").split()] if m2 else []
+            m2 = re.search(r"index_vector_dim\s*=\s*(\d+)", d)
+            a["index_vector_dim"] = int(m2.group(1)) if m2 else 0
         for key in ("feature_group_count", "batch_group_count", "feature_index"):
             mo = re.search(r"\b" + key + r"\s*=\s*(\d+)", inner)
             if mo:
@@ -1226,6 +1237,47 @@ def _reduce_window(x, init, at, dt, hifi):
     return _reduce(Tensor(w, x.dt) if not is_float(x.dt) else _FloatView(w, x.dt), init, list(range(r)), at["body"], dt, hifi)
 
 
+def _gather(operand, start, at, tout):
+    """stablehlo.gather as the specification writes it (built by reference src/Ops.jl:2269-2345 for
+    indexing with index arrays and by NNlib.gather, ext/ReactantNNlibExt/Implementations.jl:426-438):
+    every result position reads the operand at the clamped start index found at its batch position,
+    plus its offset inside the slice."""
+    offset_dims = at.get("offset_dims", [])
+    collapsed = at.get("collapsed_slice_dims", [])
+    obatch = at.get("operand_batching_dims", [])
+    sbatch = at.get("start_indices_batching_dims", [])
+    smap = at.get("start_index_map", [])
+    ivd = at.get("index_vector_dim", 0)
+    sizes = at["slice_sizes"]
+    a, st = operand.a, start.a.astype(np.int64)
+    rshape = tuple(tout.shape)
+    grid = np.indices(rshape) if rshape else np.zeros((0,), dtype=np.int64)
+    batch_dims = [d for d in range(len(rshape)) if d not in offset_dims]
+    batch_idx = [grid[d] for d in batch_dims]
+    off_idx = [grid[d] for d in offset_dims]
+    op_index = []
+    oi = 0
+    for d in range(a.ndim):
+        if d in collapsed or d in obatch:
+            comp = np.zeros(rshape, dtype=np.int64)
+        else:
+            comp = off_idx[oi].astype(np.int64)
+            oi += 1
+        if d in obatch:
+            ds = sbatch[obatch.index(d)]
+            comp = comp + batch_idx[ds - (0 if ds < ivd else 1)]
+        if d in smap:
+            k = smap.index(d)
+            sel = list(batch_idx)
+            if ivd < st.ndim:
+                sel.insert(ivd, np.full(rshape, k, dtype=np.int64))
+            s0 = st[tuple(sel)] if st.ndim else np.full(rshape, st[()])
+            comp = comp + np.clip(s0, 0, a.shape[d] - sizes[d])
+        op_index.append(comp)
+    res = a[tuple(op_index)] if a.ndim else np.broadcast_to(a, rshape)
+    return Tensor(np.ascontiguousarray(res), operand.dt)
+
+
 def _batch_norm(xs, at, training, hifi):
     """stablehlo.batch_norm_inference / batch_norm_training (reference src/Ops.jl:4012-4092) as the
     specification writes them: per-feature mean and biased variance over the other dims (training),
@@ -1549,6 +1601,8 @@ class Interpreter:
                 raise NotImplementedError("variadic reduce")
             r = _reduce(xs[0], xs[1], at["dimensions"], at["body"], op.types_out[0].dt, self.hifi)
             return [r if self.excess else _rounded(r)]
+        if n == "gather":
+            return [_gather(xs[0], xs[1], at, op.types_out[0])]
         if n in ("batch_norm_inference", "batch_norm_training"):
             return _batch_norm(xs, at, n == "batch_norm_training", self.hifi)
         if n == "reverse":

@@ -488,6 +488,45 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       }
       return emit(n.in[0], oi);
     }
+    case OpK::Gather: {
+      // result index -> (batch index into start_indices, offset index into the slice); the operand
+      // index is the clamped start read at the batch index, plus the offset
+      const Node& o = g_.nodes[n.in[0]];
+      const Node& st = g_.nodes[n.in[1]];
+      const int r = o.ty.rank(), rs = st.ty.rank();
+      const int ivd = (int)n.a4[0];
+      auto has = [](const std::vector<int64_t>& v, int x) { return std::find(v.begin(), v.end(), (int64_t)x) != v.end(); };
+      std::vector<Ix> batch;   // result index components of the non-offset dims, in order
+      for (int d = 0; d < n.ty.rank(); ++d) if (!has(n.a0, d)) batch.push_back(ix[d]);
+      // offset component per operand dim
+      Index off(r, const_ix(0));
+      {
+        size_t j = 0;
+        for (int d = 0; d < r; ++d) {
+          if (has(n.a1, d) || has(n.a5, d)) continue;
+          off[d] = ix[n.a0[j++]];
+        }
+      }
+      Index oi = off;
+      // operand batching dims take the batch index component of their start_indices dim
+      for (size_t b = 0; b < n.a5.size(); ++b) {
+        const int ds = (int)n.a6[b];
+        oi[n.a5[b]] = batch[ds - (ds < ivd ? 0 : 1)];
+      }
+      for (size_t k = 0; k < n.a2.size(); ++k) {
+        const int d = (int)n.a2[k];
+        Index si(rs);
+        size_t bi = 0;
+        for (int q = 0; q < rs; ++q) si[q] = q == ivd ? const_ix((int64_t)k) : batch[bi++];
+        const std::string e = emit(n.in[1], si);
+        const int64_t room = o.ty.dims[d] - n.a3[d];
+        const Ix& f = off[d];
+        oi[d] = temp_index("(" + idx_t() + ")rx_clamp_idx<long long>((long long)(" + e + "), " + std::to_string(room) + "LL)" +
+                               (f.is_const() && f.off == 0 ? std::string() : " + " + f.str()),
+                           f.lo, f.hi + room);
+      }
+      return emit(n.in[0], oi);
+    }
     case OpK::DynamicSlice: {
       const Node& o = g_.nodes[n.in[0]];
       Index oi(ix.size());

@@ -52,7 +52,7 @@ enum class OpK : uint8_t {
   Param, Constant, Iota,
   Unary, Binary, Compare, Select, Clamp, Convert, Gelu,
   BroadcastInDim, Reshape, Transpose, Slice, Pad, DynamicUpdateSlice, DynamicSlice, Concatenate,
-  Reverse, Window,
+  Reverse, Window, Gather,
   Reduce, DotGeneral, Scan,
 };
 
@@ -73,8 +73,10 @@ struct Node {
   //   Reverse: a0 = dimensions
   //   Window (rank r -> 2r): a0/a1/a2 = window sizes/strides/dilations;
   //       out[k_0..k_{r-1}, o_0..o_{r-1}] = in[o_i * stride_i + k_i * dilation_i]
+  //   Gather (operand, start_indices): a0 = offset_dims, a1 = collapsed_slice_dims, a2 = start_index_map,
+  //       a3 = slice_sizes, a4[0] = index_vector_dim, a5 = operand_batching_dims, a6 = start_indices_batching_dims
   //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
-  std::vector<int64_t> a0, a1, a2, a3;
+  std::vector<int64_t> a0, a1, a2, a3, a4, a5, a6;
   Red red = Red::Add;
   // Constant payload: either one splat element or dense bytes in storage format
   bool splat = false;

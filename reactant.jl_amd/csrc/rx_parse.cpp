@@ -523,7 +523,9 @@ struct P {
                             "dimension", "iota_dimension", "lhs_batching_dimensions", "rhs_batching_dimensions",
                             "lhs_contracting_dimensions", "rhs_contracting_dimensions", "window_dimensions",
                             "window_strides", "base_dilations", "window_dilations", "lhs_dilation", "rhs_dilation",
-                            "padding", "feature_group_count", "batch_group_count", "feature_index"})
+                            "padding", "feature_group_count", "batch_group_count", "feature_index", "offset_dims",
+                            "collapsed_slice_dims", "operand_batching_dims", "start_indices_batching_dims", "start_index_map",
+                            "index_vector_dim"})
       scan_int_array(in, key, o);
     {
       size_t q = in.find("#stablehlo.conv<");
@@ -1990,6 +1992,53 @@ struct Builder {
       check_same(n.ty, ty(in[0]), o.name);
       n.a0 = o.ia.at("dimensions");
       for (auto d : n.a0) if (d < 0 || d >= n.ty.rank()) fail("reverse: dimension out of range");
+      return {g.add(n)};
+    }
+    if (sh == "gather") {
+      need(2);
+      n.k = OpK::Gather;
+      n.ty = out1();
+      const TType& ot = ty(in[0]);
+      const TType& st = ty(in[1]);
+      auto get = [&](const char* key) { return o.ia.count(key) ? o.ia.at(key) : std::vector<int64_t>{}; };
+      n.a0 = get("offset_dims");
+      n.a1 = get("collapsed_slice_dims");
+      n.a2 = get("start_index_map");
+      n.a3 = get("slice_sizes");
+      n.a4 = get("index_vector_dim");
+      n.a5 = get("operand_batching_dims");
+      n.a6 = get("start_indices_batching_dims");
+      if (n.a4.size() != 1) fail("gather: index_vector_dim missing");
+      const int r = ot.rank(), rs = st.rank(), ivd = (int)n.a4[0];
+      if (!is_int_dt(st.dt) || st.dt == DT::I1) fail("gather: start indices must be integers");
+      if ((int)n.a3.size() != r) fail("gather: slice_sizes must have one entry per operand dimension");
+      if (ivd < 0 || ivd > rs) fail("gather: index_vector_dim out of range");
+      if ((int64_t)n.a2.size() != (ivd < rs ? st.dims[ivd] : 1)) fail("gather: start_index_map does not match the index vector length");
+      if (n.a5.size() != n.a6.size()) fail("gather: batching dimension lists differ in length");
+      auto in_range = [&](const std::vector<int64_t>& v, int hi) { for (auto x : v) if (x < 0 || x >= hi) return false; return true; };
+      if (!in_range(n.a1, r) || !in_range(n.a2, r) || !in_range(n.a5, r) || !in_range(n.a6, rs) || !in_range(n.a0, n.ty.rank())) fail("gather: dimension number out of range");
+      for (int d = 0; d < r; ++d) {
+        if (n.a3[d] < 0 || n.a3[d] > ot.dims[d]) fail("gather: slice size exceeds the operand");
+        const bool dropped = std::find(n.a1.begin(), n.a1.end(), (int64_t)d) != n.a1.end() || std::find(n.a5.begin(), n.a5.end(), (int64_t)d) != n.a5.end();
+        if (dropped && n.a3[d] != 1) fail("gather: collapsed and batching dimensions need slice size 1");
+      }
+      // result shape: batch dims of the start indices (without the index vector) interleaved with the kept slice sizes
+      {
+        std::vector<int64_t> bdims, odims;
+        for (int q = 0; q < rs; ++q) if (q != ivd) bdims.push_back(st.dims[q]);
+        for (int d = 0; d < r; ++d) {
+          const bool dropped = std::find(n.a1.begin(), n.a1.end(), (int64_t)d) != n.a1.end() || std::find(n.a5.begin(), n.a5.end(), (int64_t)d) != n.a5.end();
+          if (!dropped) odims.push_back(n.a3[d]);
+        }
+        if (n.a0.size() != odims.size() || (int)(bdims.size() + odims.size()) != n.ty.rank()) fail("gather: result rank mismatch");
+        size_t bi = 0, oi2 = 0;
+        for (int d = 0; d < n.ty.rank(); ++d) {
+          const bool is_off = std::find(n.a0.begin(), n.a0.end(), (int64_t)d) != n.a0.end();
+          const int64_t want = is_off ? odims[oi2++] : bdims[bi++];
+          if (n.ty.dims[d] != want) fail("gather: result shape mismatch");
+        }
+      }
+      if (n.ty.dt != ot.dt) fail("gather: element type mismatch");
       return {g.add(n)};
     }
     if (sh == "batch_norm_inference" || sh == "batch_norm_training") return build_batch_norm(o, in, sh == "batch_norm_training");

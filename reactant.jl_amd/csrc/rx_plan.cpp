@@ -33,7 +33,7 @@ using Ctx = std::pair<int, std::string>;
 bool is_index_op(OpK k) {
   switch (k) {
     case OpK::BroadcastInDim: case OpK::Reshape: case OpK::Transpose: case OpK::Slice: case OpK::Pad:
-    case OpK::DynamicUpdateSlice: case OpK::DynamicSlice: case OpK::Concatenate: case OpK::Reverse: case OpK::Window:
+    case OpK::DynamicUpdateSlice: case OpK::DynamicSlice: case OpK::Concatenate: case OpK::Reverse: case OpK::Window: case OpK::Gather:
       return true;
     default:
       return false;
@@ -628,6 +628,7 @@ struct Planner {
         case OpK::Concatenate: nm = "concatenate"; break;
         case OpK::Reverse: nm = "reverse"; break;
         case OpK::Window: nm = "window"; break;
+        case OpK::Gather: nm = "gather"; break;
         case OpK::Scan: nm = "scan"; break;
         case OpK::Reduce: nm = "reduce"; break;
         case OpK::DotGeneral: nm = "dot_general"; break;

@@ -255,3 +255,23 @@ def argreduce(shape, dt, dim, direction="GE", idt="i64", generic=False):
             "%s%s%s"
             "    return %%r#0, %%r#1 : %s, %s\n  }\n}\n"
             % (tx, tvo, tio, dim, ti, vinit, sv, si, red, body, tail, tvo, tio))
+
+
+def gather(operand_shape, start_shape, out_shape, dt, offset_dims, collapsed_slice_dims, start_index_map, index_vector_dim,
+           slice_sizes, operand_batching_dims=(), start_indices_batching_dims=(), idt="i64", one_based=False):
+    """`stablehlo.gather` in the generic form it prints in.  With `one_based` the indices are
+    decremented first, as the reference's Ops.gather does (src/Ops.jl:2313)."""
+    to, ts, tr = tt(operand_shape, dt), tt(start_shape, idt), tt(out_shape, dt)
+    lst = lambda v: "[" + ", ".join(str(x) for x in v) + "]"
+    dn = "offset_dims = %s, collapsed_slice_dims = %s, " % (lst(offset_dims), lst(collapsed_slice_dims))
+    if operand_batching_dims:
+        dn += "operand_batching_dims = %s, start_indices_batching_dims = %s, " % (lst(operand_batching_dims), lst(start_indices_batching_dims))
+    dn += "start_index_map = %s, index_vector_dim = %d" % (lst(start_index_map), index_vector_dim)
+    pre, idx = "", "%arg1"
+    if one_based:
+        pre = ("    %%one = stablehlo.constant dense<1> : %s\n    %%idx = stablehlo.subtract %%arg1, %%one : %s\n" % (ts, ts))
+        idx = "%idx"
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n%s"
+            "    %%0 = \"stablehlo.gather\"(%%arg0, %s) <{dimension_numbers = #stablehlo.gather<%s>, indices_are_sorted = false, "
+            "slice_sizes = array<i64: %s>}> : (%s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
+            % (to, ts, tr, pre, idx, dn, ", ".join(str(x) for x in slice_sizes), to, ts, tr, tr))

@@ -303,3 +303,44 @@ def test_argmax_and_argmin(rx, client, shape, dt, dim, direction, generic):
     lib = np.argmax if direction in ("GE", "GT") else np.argmin
     if direction in ("GE", "LE"):
         assert np.array_equal(got[1].a, lib(x.a, axis=dim))
+
+
+def test_gather_reference_vectors(rx, client):
+    """NNlib.gather known answers (test/nn/scatter_gather.jl:5-99)."""
+    src = I.tensor(np.array([3, 4, 5, 6, 7]), "f32")
+    index = np.array([[1, 2, 3, 4], [4, 2, 1, 3], [3, 5, 5, 3]])
+    t = NN.gather([5], [1, 3, 4], [3, 4], "f32", [], [0], [0], 0, [1], one_based=True)
+    got, _ = gpu_run(rx, client, t, [src, I.Tensor(index.reshape(1, 3, 4), "i64")])
+    assert got[0].a.tolist() == [[3, 4, 5, 6], [6, 4, 3, 5], [5, 7, 7, 5]]
+    src2 = I.tensor(np.array([[3, 5, 7], [4, 6, 8]]), "f32")
+    index2 = np.array([[1, 2, 3], [2, 2, 1], [3, 1, 3]])
+    t = NN.gather([2, 3], [1, 3, 3], [2, 3, 3], "f32", [0], [1], [1], 0, [2, 1], one_based=True)
+    got, _ = gpu_run(rx, client, t, [src2, I.Tensor(index2.reshape(1, 3, 3), "i64")])
+    assert got[0].a[:, :, 1].tolist() == [[5, 5, 3], [6, 6, 4]] and got[0].a[:, :, 2].tolist() == [[7, 3, 7], [8, 4, 8]]
+
+
+GATHERS = [
+    # operand, start indices, result, dtype, offset_dims, collapsed, start_index_map, index_vector_dim, slice_sizes, batching
+    ([7, 5, 6], [1000, 3], [1000, 1], "f32", [1], [0, 1], [0, 1, 2], 1, [1, 1, 1], None),          # x[idx] (gather_getindex)
+    ([50000, 64], [32, 128], [32, 128, 64], "bf16", [2], [0], [0], 2, [1, 64], None),               # embedding lookup
+    ([50000, 64], [4096], [4096, 64], "f32", [1], [0], [0], 1, [1, 64], None),                      # index vector dim past the end
+    ([64, 50000], [1, 3000], [64, 3000], "f32", [0], [1], [1], 0, [64, 1], None),                   # columns (NNlib.gather layout)
+    ([4, 2000], [4, 50], [4, 50, 33], "f64", [2], [], [1], 2, [1, 33], ([0], [0])),                 # windows with a batching dim
+    ([30, 40], [17, 2], [17, 5, 7], "i32", [1, 2], [], [0, 1], 1, [5, 7], None),                    # 2-d patches
+]
+
+
+@pytest.mark.parametrize("os_,ss,rs,dt,od,cd,sim,ivd,sz,bat", GATHERS)
+def test_gather(rx, client, os_, ss,rs, dt, od, cd, sim, ivd, sz, bat):
+    kw = {} if bat is None else dict(operand_batching_dims=bat[0], start_indices_batching_dims=bat[1])
+    text = NN.gather(os_, ss, rs, dt, od, cd, sim, ivd, sz, idt="i32" if dt == "i32" else "i64", **kw)
+    rng = np.random.default_rng(37)
+    x = _args([os_], dt, seed=37)[0]
+    hi = max(os_)
+    idt = "i32" if dt == "i32" else "i64"
+    idx = I.Tensor(rng.integers(-3, hi + 3, size=ss).astype(I.NP_OF[idt]), idt)     # some starts out of range: clamped
+    got, exe = gpu_run(rx, client, text, [x, idx])
+    ref = oracle_run(text, [x, idx])
+    assert got[0].a.shape == ref[0].a.shape
+    assert np.array_equal(got[0].a, ref[0].a)
+    assert [l["kind"] for l in exe.launches()] == ["map"]

@@ -204,3 +204,50 @@ def test_argmax_reduce_against_numpy():
         v, i = [t.a for t in I.run_text(NN.argreduce([4, 6, 5], "f64", dim, "GT"), [I.tensor(x, "f64")])]
         last = x.shape[dim] - 1 - np.flip(x, axis=dim).argmax(axis=dim)
         assert np.array_equal(v, x.max(axis=dim)) and np.array_equal(i, last)
+
+
+def test_gather_reference_vectors():
+    """test/nn/scatter_gather.jl:5-99 (NNlib.gather known answers) with the dimension numbers of
+    ext/ReactantNNlibExt/Implementations.jl:426-438, written on the tensors as the traced program
+    sees them (Julia dim order, one-based indices)."""
+    src = np.array([3, 4, 5, 6, 7], dtype=np.float32)
+    index = np.array([[1, 2, 3, 4], [4, 2, 1, 3], [3, 5, 5, 3]])
+    output = np.array([[3, 4, 5, 6], [6, 4, 3, 5], [5, 7, 7, 5]], dtype=np.float32)
+    t = NN.gather([5], [1, 3, 4], [3, 4], "f32", [], [0], [0], 0, [1], one_based=True)
+    got = I.run_text(t, [I.tensor(src, "f32"), I.Tensor(index.reshape(1, 3, 4), "i64")])[0].a
+    assert np.array_equal(got, output)
+    # 2-d source, columns gathered: output[:, i, j] = src[:, index[i, j]]
+    src2 = np.array([[3, 5, 7], [4, 6, 8]], dtype=np.float32)
+    index2 = np.array([[1, 2, 3], [2, 2, 1], [3, 1, 3]])
+    want = np.zeros((2, 3, 3), dtype=np.float32)
+    want[:, :, 0] = [[3, 5, 7], [4, 6, 8]]
+    want[:, :, 1] = [[5, 5, 3], [6, 6, 4]]
+    want[:, :, 2] = [[7, 3, 7], [8, 4, 8]]
+    t = NN.gather([2, 3], [1, 3, 3], [2, 3, 3], "f32", [0], [1], [1], 0, [2, 1], one_based=True)
+    got = I.run_text(t, [I.tensor(src2, "f32"), I.Tensor(index2.reshape(1, 3, 3), "i64")])[0].a
+    assert np.array_equal(got, want)
+
+
+def test_gather_against_numpy_indexing():
+    rng = np.random.default_rng(12)
+    x = rng.normal(size=(7, 5, 6))
+    # x[idx] on a flattened view: the reference's gather_getindex (src/Ops.jl:2269-2298)
+    idx = rng.integers(0, 7, size=(11, 3))
+    idx[:, 1] = rng.integers(0, 5, size=11)
+    idx[:, 2] = rng.integers(0, 6, size=11)
+    t = NN.gather([7, 5, 6], [11, 3], [11, 1], "f64", [1], [0, 1], [0, 1, 2], 1, [1, 1, 1])
+    got = I.run_text(t, [I.tensor(x, "f64"), I.Tensor(idx, "i64")])[0].a
+    assert np.array_equal(got[:, 0], x[idx[:, 0], idx[:, 1], idx[:, 2]])
+    # rows of a table (an embedding lookup), out-of-range rows clamped
+    table = rng.normal(size=(10, 4))
+    ids = np.array([[0, 9, 3], [12, -2, 5]])
+    t = NN.gather([10, 4], [2, 3], [2, 3, 4], "f64", [2], [0], [0], 2, [1, 4])
+    got = I.run_text(t, [I.tensor(table, "f64"), I.Tensor(ids, "i64")])[0].a
+    assert np.array_equal(got, table[np.clip(ids, 0, 9)])
+    # windows: slices of 3 starting at given offsets, with a batching dimension
+    y = rng.normal(size=(4, 20))
+    starts = rng.integers(-2, 22, size=(4, 5))
+    t = NN.gather([4, 20], [4, 5], [4, 5, 3], "f64", [2], [], [1], 2, [1, 3], operand_batching_dims=[0], start_indices_batching_dims=[0])
+    got = I.run_text(t, [I.tensor(y, "f64"), I.Tensor(starts, "i64")])[0].a
+    want = np.stack([[y[b, np.clip(s, 0, 17):np.clip(s, 0, 17) + 3] for s in starts[b]] for b in range(4)])
+    assert np.array_equal(got, want)
