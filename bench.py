@@ -228,6 +228,62 @@ def bench_fp8(rx, client, P, steps, warmup, n=8192):
                       "f8E4M3FN", plain=_time_plain(client, exe, bufs, steps, warmup))
 
 
+# ----------------------------------------------------------------------------
+# windowed ops next to the hot path (not part of the default run: --workload conv|cumsum|maxpool)
+# ----------------------------------------------------------------------------
+def _window_entry(name, exe, secs, steps, mean_ms, algo_bytes, flops, dtype, bound_kind):
+    launches = exe.launches()
+    big = int(np.argmax(mean_ms))
+    entry = {"workload": name, "ms_per_step": 1e3 * secs / steps, "dtype": dtype,
+             "kernels": [{"kernel": l["kernel"], "kind": l["kind"], "ms": float(m)} for l, m in zip(launches, mean_ms)]}
+    if flops:
+        ach = flops / (secs / steps) / 1e12
+        entry.update(value=ach, unit="TFLOP/s")
+        dot = [i for i, l in enumerate(launches) if l["flops"] > 0]
+        kms = float(mean_ms[dot[0]]) if dot else float(mean_ms[big])
+        kach = flops / (kms * 1e-3) / 1e12
+        entry["roofline"] = {"bound": "mfma", "kernel": launches[dot[0] if dot else big]["kernel"], "kernel_ms": kms, "achieved": kach,
+                             "peak": PEAK_TFLOPS[bound_kind], "unit": "TFLOP/s", "frac": kach / PEAK_TFLOPS[bound_kind], "traffic": None}
+    else:
+        entry.update(value=algo_bytes / (secs / steps) / 1e9, unit="GB/s")
+        # every launch of these programs is a pass over the data: the roofline is quoted on their sum
+        kms = float(np.sum(mean_ms))
+        entry["roofline"] = {"bound": "hbm", "kernel": launches[big]["kernel"], "kernel_ms": kms, "achieved": algo_bytes / (kms * 1e-3) / 1e9,
+                             "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": algo_bytes / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None}
+    return entry
+
+
+def bench_conv(rx, client, P, steps, warmup, batch=32, cin=64, cout=64, hw=56):
+    """3x3 convolution, padding 1, bias + relu (a VGG/ResNet body layer) in f32."""
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    text, out_shape = NN.convolution([batch, cin, hw, hw], [cout, cin, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")
+    exe = rx.xla_compile(client, text)
+    rng = np.random.default_rng(0)
+    bufs = [_upload(rx, client, rng.normal(size=s).astype(np.float32), "f32") for s in ([batch, cin, hw, hw], [cout, cin, 3, 3], [cout])]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
+    flops = 2.0 * batch * cout * hw * hw * cin * 9
+    return _window_entry("conv 3x3 pad 1 f32 %dx%dx%dx%d -> %d features, bias + relu" % (batch, cin, hw, hw, cout), exe, secs, steps, mean_ms,
+                         0.0, flops, "f32", "f32")
+
+
+def bench_cumsum(rx, client, P, steps, warmup, n=1 << 26):
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    exe = rx.xla_compile(client, NN.cumulative([n], "f32", 0))
+    bufs = [_upload(rx, client, np.random.default_rng(0).normal(size=n).astype(np.float32), "f32")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0]), steps, warmup)
+    return _window_entry("cumsum f32[2^%d]" % int(np.log2(n)), exe, secs, steps, mean_ms, 8.0 * n, 0.0, "f32", None)
+
+
+def bench_maxpool(rx, client, P, steps, warmup, batch=64, c=64, hw=112):
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    text, out_shape = NN.reduce_window([batch, c, hw, hw], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])
+    exe = rx.xla_compile(client, text)
+    bufs = [_upload(rx, client, np.random.default_rng(0).normal(size=(batch, c, hw, hw)).astype(np.float32), "f32")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0]), steps, warmup)
+    return _window_entry("maxpool 2x2 stride 2 f32 %dx%dx%dx%d" % (batch, c, hw, hw), exe, secs, steps, mean_ms,
+                         4.0 * batch * c * hw * hw * 1.25, 0.0, "f32", None)
+
+
 def cpu_baseline_stencil(P, nx=512, ny=512, nz=256, nsteps=10):
     """The oracle's C restatement of the stencil (oracle/stencil_cpu.c, OpenMP on all host cores,
     same bits as the GPU result) on the full grid, a bounded number of repetitions of the
@@ -278,7 +334,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--small", action="store_true", help="reduced sizes (debugging only; not a valid result)")
@@ -290,9 +346,11 @@ def main():
     rx = _pkg()
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
-    table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8}
+    table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
+             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
-             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024)}
+             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
+             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4)}
     _FULL_SIZE[0] = not args.small
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
