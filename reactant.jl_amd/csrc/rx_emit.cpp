@@ -437,6 +437,69 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         for (size_t k = 0; k < rn.size(); ++k) oi[ro[k]] = ix[rn[k]];
         return emit(n.in[0], oi);
       }
+      // Dims that regroup independently ([C*T, B*P] <-> [C, T, B, P]) are converted group by group:
+      // a group's index arithmetic involves only its own variables, so the part that does not
+      // depend on the minor output index is computed once per thread, not once per element.
+      {
+        const auto& nd = n.ty.dims;
+        const auto& od = o.ty.dims;
+        struct Grp { size_t a0, a1, b0, b1; };
+        std::vector<Grp> groups;
+        size_t a = 0, b = 0;
+        bool ok = n.ty.numel() > 0;
+        while (ok && a < nd.size() && b < od.size()) {
+          Grp gq{a, a, b, b};
+          int64_t pa = nd[a++], pb = od[b++];
+          while (pa != pb) {
+            if (pa < pb) { if (a >= nd.size()) { ok = false; break; } pa *= nd[a++]; }
+            else { if (b >= od.size()) { ok = false; break; } pb *= od[b++]; }
+          }
+          gq.a1 = a; gq.b1 = b;
+          groups.push_back(gq);
+        }
+        for (; ok && a < nd.size(); ++a) ok = nd[a] == 1;     // trailing unit dims carry no index
+        for (; ok && b < od.size(); ++b) ok = od[b] == 1;
+        if (ok && groups.size() > 1) {
+          for (auto& gq : groups) {
+            if (gq.a1 - gq.a0 == 1 && gq.b1 - gq.b0 == 1) { oi[gq.b0] = ix[gq.a0]; continue; }
+            // linear index inside the group
+            std::string e;
+            int64_t total = 1, lo = 0, hi = 0;
+            bool all_const = true;
+            for (size_t k = gq.a0; k < gq.a1; ++k) {
+              total *= nd[k];
+              if (nd[k] == 1) continue;
+              all_const = all_const && ix[k].is_const();
+            }
+            {
+              int64_t stride = total;
+              for (size_t k = gq.a0; k < gq.a1; ++k) {
+                stride /= std::max<int64_t>(nd[k], 1);
+                if (nd[k] == 1) continue;
+                const std::string term = stride == 1 ? "(" + ix[k].str() + ")" : "(" + ix[k].str() + ") * " + std::to_string(stride);
+                e += (e.empty() ? "" : " + ") + term;
+                lo += ix[k].lo * stride;
+                hi += ix[k].hi * stride;
+              }
+            }
+            if (e.empty()) e = "0";
+            Ix lin = temp_index(e, lo, hi);
+            int64_t stride = total;
+            for (size_t k = gq.b0; k < gq.b1; ++k) {
+              stride /= std::max<int64_t>(od[k], 1);
+              if (od[k] == 1) continue;
+              std::string c2 = lin.var;
+              if (stride > 1) c2 = "(" + c2 + " / " + std::to_string(stride) + ")";
+              bool first = true;
+              for (size_t q = gq.b0; q < k; ++q) first = first && od[q] == 1;
+              if (!first) c2 = c2 + " % " + std::to_string(od[k]);
+              oi[k] = temp_index(c2, 0, od[k] - 1);
+            }
+            (void)all_const;
+          }
+          return emit(n.in[0], oi);
+        }
+      }
       Ix lin = temp_index(linear(ix, n.ty.dims), 0, n.ty.numel() - 1);
       int64_t stride = o.ty.numel();
       for (int k = 0; k < o.ty.rank(); ++k) {
