@@ -172,6 +172,23 @@ struct rx_tile_copy {
       }
     }
   }
+  // The same tile taken from a functor instead of memory: fn(batch, row, col) is element (row, col)
+  // of the operand as it would be stored; positions outside the matrix are zero.
+  template <class FN>
+  RX_MEM void load_fn(const FN& fn, long long batch, int row0, int col0, int nrows, int ncols, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int v = tid + i * NT;
+      if (TOTAL % NT == 0 || v < TOTAL) {
+        const int rr = row0 + v / VPR;
+        const int cc = col0 + (v % VPR) * VE;
+        union { E e[VE]; rx_u32x4 q; } u;
+#pragma unroll
+        for (int k = 0; k < VE; ++k) u.e[k] = (rr < nrows && cc + k < ncols) ? fn(batch, rr, cc + k) : E(0);
+        r[i] = u.q;
+      }
+    }
+  }
   RX_MEM void store(RX_LDS E* lds, int lld, int tid) const {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -209,8 +226,15 @@ RX_DEV bool rx_gemm_tile(unsigned bid, int* bm, int* bn) {
   }
 }
 
-template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
-RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
+// An operand can also be a functor (LA / LB other than rx_no_fn): the fusion code generator
+// writes one when the operand is a cheap expansion of smaller data (the window matrix of a
+// convolution, a broadcast), so that the expanded matrix never exists in memory.
+struct rx_no_fn { static constexpr bool none = true; };
+
+template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
+          class LA = rx_no_fn, class LB = rx_no_fn>
+RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi, const LA& la = LA(),
+                         const LB& lb = LB()) {
   typedef typename MMA::elem E;
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;   // 32x32 tiles per wavefront
@@ -245,8 +269,16 @@ RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typenam
   rx_tile_copy<E, B_ROWS, B_COLS, NT> cb;
   auto gload = [&](int k0) {
     constexpr bool TAIL = K % BK != 0;   // only then can a tile reach past the contracted dimension
-    if (A_KC) ca.template load<false, TAIL>(Ab, A_GLD, m0, k0, M, K, tid); else ca.template load<TAIL, false>(Ab, A_GLD, k0, m0, K, M, tid);
-    if (B_KC) cb.template load<false, TAIL>(Bb, B_GLD, n0, k0, N, K, tid); else cb.template load<TAIL, false>(Bb, B_GLD, k0, n0, K, N, tid);
+    if constexpr (!LA::none) {
+      if (A_KC) ca.load_fn(la, batch, m0, k0, M, K, tid); else ca.load_fn(la, batch, k0, m0, K, M, tid);
+    } else {
+      if (A_KC) ca.template load<false, TAIL>(Ab, A_GLD, m0, k0, M, K, tid); else ca.template load<TAIL, false>(Ab, A_GLD, k0, m0, K, M, tid);
+    }
+    if constexpr (!LB::none) {
+      if (B_KC) cb.load_fn(lb, batch, n0, k0, N, K, tid); else cb.load_fn(lb, batch, k0, n0, K, N, tid);
+    } else {
+      if (B_KC) cb.template load<false, TAIL>(Bb, B_GLD, n0, k0, N, K, tid); else cb.template load<TAIL, false>(Bb, B_GLD, k0, n0, K, N, tid);
+    }
   };
   gload(0);
   ca.store(lds, A_LD, tid);

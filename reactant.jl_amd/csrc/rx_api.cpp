@@ -222,6 +222,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_SINGLE_PASS_REDUCE")) o.single_pass_reduce = atoi(e) != 0;
   if (const char* e = getenv("RX_LDS_TRANSPOSE")) o.lds_transpose = atoi(e) != 0;
   if (const char* e = getenv("RX_DOT_AS_REDUCE")) o.dot_as_reduce = atoi(e) != 0;
+  if (const char* e = getenv("RX_FUSE_DOT_OPERANDS")) o.fuse_dot_operands = atoi(e) != 0;
   if (const char* e = getenv("RX_BRANCHLESS")) o.branchless_guards = atoi(e) != 0;
   if (const char* e = getenv("RX_STENCIL_FUSE")) o.stencil_fuse_steps = atoi(e) != 0;
   if (const char* e = getenv("RX_SHIFTED_VEC")) o.shifted_vector_loads = atoi(e) != 0;

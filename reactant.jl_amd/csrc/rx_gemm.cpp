@@ -48,10 +48,10 @@ static GemmChoice choose_gemm_f64(int64_t batch, int64_t M, int64_t N, int64_t K
   return c;
 }
 
-GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc) {
+GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc, bool staged_only) {
   GemmChoice c;
   if (a != b) return c;
-  if (a == DT::F64 && out == DT::F64) return choose_gemm_f64(batch, M, N, K, a_kc, b_kc);
+  if (a == DT::F64 && out == DT::F64) return staged_only ? c : choose_gemm_f64(batch, M, N, K, a_kc, b_kc);
   std::string mma;
   int esize = 0, bk = 0;
   if (a == DT::F32 && out == DT::F32) { mma = "rx_mma_f32"; c.kind = "gemm_f32"; esize = 4; bk = 16; }
@@ -84,7 +84,7 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
     if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
   }
   if (const char* e = getenv("RX_GEMM_BK")) bk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : bk;
-  bool direct = true;   // global -> LDS direct loads through a ring of LDS stages
+  bool direct = !staged_only;   // global -> LDS direct loads through a ring of LDS stages
   if (const char* e = getenv("RX_GEMM_DIRECT")) direct = atoi(e) != 0;
   int stages = 2;
   if (const char* e = getenv("RX_GEMM_STAGES")) stages = atoi(e) >= 2 ? atoi(e) : stages;
@@ -139,14 +139,26 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   return c;
 }
 
-std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched) {
+std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched,
+                          const GemmOperandFn& fa, const GemmOperandFn& fb) {
   std::ostringstream o;
   o << "// dot_general on MFMA: " << c.kind << " <" << c.targs << ">\n";
-  o << "extern \"C\" __global__ __launch_bounds__(" << c.block << ") void " << kbase << "_gemm(const " << c.stype_a << "* __restrict__ A, const " << c.stype_a
-    << "* __restrict__ B" << epi_params << ") {\n";
+  const bool fn = !fa.type.empty() || !fb.type.empty();
+  o << "extern \"C\" __global__ __launch_bounds__(" << c.block << ") void " << kbase << "_gemm(";
+  // operands that are read from memory come first, then what the operand functors read, then the epilogue's operands
+  std::string params;
+  if (fa.type.empty()) params += ", const " + c.stype_a + "* __restrict__ A";
+  if (fb.type.empty()) params += ", const " + c.stype_a + "* __restrict__ B";
+  params += fa.params + fb.params + epi_params;
+  o << params.substr(2) << ") {\n";
+  if (!fa.type.empty()) o << "  const " << c.stype_a << "* A = nullptr;\n  " << fa.ctor << "\n";
+  if (!fb.type.empty()) o << "  const " << c.stype_a << "* B = nullptr;\n  " << fb.ctor << "\n";
   o << "  " << epi_ctor << "\n";
-  o << "  " << c.skeleton << "<" << c.targs << ", " << (batched ? "true" : "false") << ", " << kbase << "_epi>(A, B, epi);\n";
-  o << "}\n\n";
+  o << "  " << c.skeleton << "<" << c.targs << ", " << (batched ? "true" : "false") << ", " << kbase << "_epi";
+  if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn" : fa.type) << ", " << (fb.type.empty() ? "rx_no_fn" : fb.type);
+  o << ">(A, B, epi";
+  if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn()" : "la") << ", " << (fb.type.empty() ? "rx_no_fn()" : "lb");
+  o << ");\n}\n\n";
   return o.str();
 }
 

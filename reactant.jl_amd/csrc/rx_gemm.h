@@ -27,10 +27,18 @@ inline int64_t gemm_grid(int64_t gm, int64_t gn, int rb = 4, int cb = 8) {
 }
 
 // Returns ok=false when no skeleton covers the case (the caller then writes a scalar loop).
-GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_k_contig, bool b_k_contig);
+// `staged_only`: an operand is a functor, which only the register-staged skeleton can read.
+GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_k_contig, bool b_k_contig,
+                       bool staged_only = false);
 
 // Text of the `extern "C"` kernel <kbase>_gemm that runs the skeleton with epilogue type <kbase>_epi.
 // `epi_params` is the tail of the parameter list (epilogue operands and out0), `epi_ctor` builds `epi`.
-std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched);
+// An operand computed by a functor: `type` names the functor struct ("" = read from memory), `params` the
+// kernel parameters it needs (", const T* name" ...), `ctor` the statement that builds it as `la` / `lb`.
+struct GemmOperandFn {
+  std::string type, params, ctor;
+};
+std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched,
+                          const GemmOperandFn& fa = {}, const GemmOperandFn& fb = {});
 
 }  // namespace rx

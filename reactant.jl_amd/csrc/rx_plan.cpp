@@ -118,6 +118,7 @@ struct Planner {
   std::map<int, int> fuse_prev;     // stencil root -> the stencil step it evaluates in LDS instead of reading from memory
   std::set<int> lds_only;           // the steps absorbed that way: no launch, no buffer
   std::map<int, int> reshape_alias; // materialized reshape of a materialized value: the same bytes, no launch
+  std::set<std::pair<int, int>> fused_operands;   // (dot_general, side): the operand is evaluated inside the GEMM's tile loads
   std::ostringstream src;
   int kcount = 0;
 
@@ -168,6 +169,55 @@ struct Planner {
     }
     dots_to_reductions();
     align_dots();
+  }
+
+  // A dot_general operand that is a cheap expansion of much smaller data -- the window matrix of a
+  // convolution, a broadcast -- is not written to memory: the GEMM evaluates it while it loads
+  // its tiles (a functor in place of the operand pointer), reading the small data through the caches.
+  void decide_fused_operands() {
+    fused_operands.clear();
+    if (!opt.mfma || !opt.fuse_dot_operands) return;
+    const int N = (int)g.nodes.size();
+    std::vector<int> nuse(N, 0);
+    for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
+    for (int r : g.results) nuse[r]++;
+    auto is_leaf = [](const Node& n) {
+      return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral;
+    };
+    for (const Node& d : g.nodes) {
+      if (d.k != OpK::DotGeneral || d.ty.rank() < 2) continue;
+      DotForm f = dot_form(d);
+      if (!f.ok) continue;
+      const DT a = g.nodes[d.in[0]].ty.dt, b = g.nodes[d.in[1]].ty.dt;
+      if (!choose_gemm(a, b, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, true).ok) continue;
+      for (int side = 0; side < 2; ++side) {
+        const int x = d.in[side];
+        const Node& xn = g.nodes[x];
+        if (is_leaf(xn) || xn.k == OpK::Constant || nuse[x] != 1) continue;
+        // every tile row (column) of the product evaluates the operand again; with more than one or two
+        // of them the expanded matrix is cheaper (3x3 256 -> 256 features on 14x14 images: 0.12 ms
+        // with the window matrix in memory, 0.15 ms evaluated four times over)
+        if ((side == 1 ? f.M : f.N) > 128) continue;
+        std::set<int> seen;
+        std::vector<int> st{x};
+        double leaf = 0;
+        int count = 0;
+        bool ok = true;
+        while (!st.empty() && ok) {
+          const int y = st.back();
+          st.pop_back();
+          if (!seen.insert(y).second) continue;
+          const Node& yn = g.nodes[y];
+          if (is_leaf(yn)) { leaf += (double)yn.ty.numel(); continue; }
+          if (yn.k == OpK::Constant) continue;
+          if (yn.k == OpK::Gather) { ok = false; break; }   // data-dependent addresses: keep the plain path
+          if (++count > 48) ok = false;
+          for (int i : yn.in) st.push_back(i);
+        }
+        if (!ok || (double)xn.ty.numel() < 3.0 * leaf) continue;
+        fused_operands.insert({d.id, side});
+      }
+    }
   }
 
   // A matrix product that misses the MFMA path only because a dimension is not a whole number of
@@ -473,7 +523,12 @@ struct Planner {
                     (n.k == OpK::Constant && !n.splat);
       for (int u : users[x]) {
         const Node& un = g.nodes[u];
-        if (un.k == OpK::DotGeneral) { forced = true; continue; }
+        if (un.k == OpK::DotGeneral) {
+          const int side = un.in[0] == x ? 0 : 1;
+          if (fused_operands.count({u, side})) U.insert({u, "/operand" + std::to_string(side)});
+          else forced = true;
+          continue;
+        }
         // start indices of dynamic slices must be constants; they are read at plan time
         std::vector<Ctx> base;
         if (mat[u]) base.push_back({u, ""});
@@ -2545,9 +2600,52 @@ struct Planner {
     std::string ebody = em.take_code();
     const std::string ACC = is_float(d.ty.dt) ? (d.ty.dt == DT::F64 ? "double" : "float") : info(d.ty.dt).ctype;
 
+    const bool fuse_a = fused_operands.count({dot, 0}) != 0, fuse_b = fused_operands.count({dot, 1}) != 0;
     GemmChoice gc;
-    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig);
+    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, fuse_a || fuse_b);
+    if ((fuse_a || fuse_b) && !gc.ok) throw Error("internal: a fused dot_general operand without a GEMM skeleton");
     std::ostringstream o;
+    // operand functors: element (row, column) of the operand as it would be stored, evaluated from the fused cone
+    GemmOperandFn fn_a, fn_b;
+    std::vector<int> in_a, in_b;
+    auto make_operand_fn = [&](int side, GemmOperandFn& fn, std::vector<int>& inputs) {
+      const int x = d.in[side];
+      const TType& xt = g.nodes[x].ty;
+      Emitter e(g, [&](int y) { return mat[y] != 0; });
+      e.excess_precision = opt.excess_precision;
+      e.idx64 = needs64(cone_nodes(x));
+      e.set_root({}, {}, false);
+      e.indent = 4;
+      const std::string eit = e.idx_t();
+      const int nbd = (int)d.a0.size();
+      Index ix(xt.rank());
+      for (int k = 0; k < xt.rank(); ++k) {
+        ix[k].var = k < nbd ? "ob" : (k == nbd ? "r" : "c");
+        ix[k].hi = xt.dims[k] - 1;
+      }
+      const std::string v = e.emit(x, ix);
+      const std::string code = e.take_code();
+      inputs = e.inputs;
+      const std::string tag = side == 0 ? "opa" : "opb";
+      const std::string E = info(xt.dt).stype;
+      o << "// dot operand " << (side == 0 ? "A" : "B") << " computed on the fly: " << describe(x) << "\n";
+      o << "struct " << kbase << "_" << tag << " {\n  static constexpr bool none = false;\n";
+      for (size_t k = 0; k < inputs.size(); ++k) o << "  const " << info(g.nodes[inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
+      o << "  __device__ __forceinline__ " << E << " operator()(long long ob_, int r_, int c_) const {\n";
+      o << "    const " << eit << " ob = (" << eit << ")ob_, r = (" << eit << ")r_, c = (" << eit << ")c_;\n    (void)ob;\n";
+      o << code;
+      o << "    return " << e.store_value(xt.dt, v) << ";\n  }\n};\n\n";
+      fn.type = kbase + "_" + tag;
+      fn.ctor = fn.type + " " + (side == 0 ? "la" : "lb") + "{";
+      for (size_t k = 0; k < inputs.size(); ++k) {
+        const std::string pn = (side == 0 ? "fa" : "fb") + std::to_string(k);
+        fn.params += ", const " + std::string(info(g.nodes[inputs[k]].ty.dt).stype) + "* __restrict__ " + pn;
+        fn.ctor += (k ? ", " : "") + pn;
+      }
+      fn.ctor += "};";
+    };
+    if (fuse_a) make_operand_fn(0, fn_a, in_a);
+    if (fuse_b) make_operand_fn(1, fn_b, in_b);
     o << "// dot epilogue: " << describe(root) << "\n";
     o << "struct " << kbase << "_epi {\n";
     for (size_t k = 0; k < em.inputs.size(); ++k)
@@ -2586,8 +2684,10 @@ struct Planner {
       for (auto c : d.a2) kprod *= (double)lt.dims[c];
       L.flops = 2.0 * (double)d.ty.numel() * kprod;
     }
-    std::vector<int> all_in{d.in[0], d.in[1]};
-    for (int i : epi_inputs) if (i != d.in[0] && i != d.in[1]) all_in.push_back(i);
+    std::vector<int> all_in;
+    if (fuse_a) all_in.insert(all_in.end(), in_a.begin(), in_a.end()); else all_in.push_back(d.in[0]);
+    if (fuse_b) all_in.insert(all_in.end(), in_b.begin(), in_b.end()); else all_in.push_back(d.in[1]);
+    for (int i : epi_inputs) if (std::find(all_in.begin(), all_in.end(), i) == all_in.end()) all_in.push_back(i);
     L.algo_bytes = algo_bytes(all_in, {root});
     L.desc = describe(root);
 
@@ -2603,7 +2703,7 @@ struct Planner {
     };
 
     if (gc.ok) {
-      o << gemm_instance(gc, kbase, epi_params(), epi_ctor(), d.a0.size() == 1);
+      o << gemm_instance(gc, kbase, epi_params(), epi_ctor(), d.a0.size() == 1, fn_a, fn_b);
       L.kernel = kbase + "_gemm";
       L.kind = gc.kind;
       L.grid[0] = gc.grid[0]; L.grid[1] = gc.grid[1]; L.grid[2] = gc.grid[2];
@@ -2658,8 +2758,10 @@ struct Planner {
     }
     const std::string kb_final = finalize(o.str());
     L.kernel = named(L.kernel, kb_final);
-    L.args.push_back(buffer_for(d.in[0]));
-    L.args.push_back(buffer_for(d.in[1]));
+    if (!fuse_a) L.args.push_back(buffer_for(d.in[0]));
+    if (!fuse_b) L.args.push_back(buffer_for(d.in[1]));
+    for (int i : in_a) L.args.push_back(buffer_for(i));
+    for (int i : in_b) L.args.push_back(buffer_for(i));
     for (int i : epi_inputs) L.args.push_back(buffer_for(i));
     L.args.push_back(buffer_for(root));
     plan.launches.push_back(L);
@@ -2668,6 +2770,7 @@ struct Planner {
   // ------------------------------------------------------------------ driver
   void run() {
     canonicalize();
+    decide_fused_operands();
     const int N = (int)g.nodes.size();
     // Decisions about a node depend on which of its producers own buffers; sweep until stable.
     prev_mat.assign(N, 0);

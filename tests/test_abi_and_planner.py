@@ -239,12 +239,19 @@ def test_windowed_ops_plan(monkeypatch):
     # pooling: the window view is index arithmetic inside a reduction kernel
     rep = rx.compile_offline(NN.reduce_window([8, 16, 32, 32], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])[0])
     assert "launches: 1" in rep and "window reduce" in rep
-    # convolution: window matrix (one map), MFMA product with a 64-row tile, bias + relu + layout in one map;
-    # the reshaped weights share the argument's buffer
-    rep = rx.compile_offline(NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0])
-    kinds = [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
-    assert kinds == ["map", "gemm_f32", "map"], rep
-    assert "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rx.compile_offline(
-        NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]])[0], with_source=True)
+    # convolution with few output features: one MFMA product (64-row tiles) that evaluates the window matrix while
+    # it loads its tiles, then bias + relu + layout in one map; the reshaped weights share the argument's buffer
+    conv = NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0]
+    kinds = lambda rep: [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
+    rep = rx.compile_offline(conv, with_source=True)
+    assert kinds(rep) == ["gemm_f32", "map"], rep
+    assert "rx_gemm_body<rx_mma_f32, 64, 128" in rep and "dot operand B computed on the fly" in rep
+    # many output features: every tile row would evaluate the window matrix again, so it is written once instead
+    rep = rx.compile_offline(NN.convolution([32, 256, 14, 14], [256, 256, 3, 3], "f32", padding=[[1, 1], [1, 1]])[0])
+    assert kinds(rep) == ["map", "gemm_f32", "map"], rep
+    monkeypatch.setenv("RX_FUSE_DOT_OPERANDS", "0")
+    rep = rx.compile_offline(conv, with_source=True)
+    assert kinds(rep) == ["map", "gemm_f32", "map"] and "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rep
+    monkeypatch.delenv("RX_FUSE_DOT_OPERANDS")
     with pytest.raises(Exception, match="batch_group_count"):
         rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 8, 4, 4], "f32")[0].replace("batch_group_count = 1", "batch_group_count = 2"))

@@ -188,6 +188,8 @@ CONVS = [
     ([2, 3, 8, 8, 8], [3, 3, 3, 3, 3], "f32", "[b, f, 2, 1, 0]x[o, i, 2, 1, 0]->[b, f, 2, 1, 0]", dict(padding=[[1, 1], [1, 1], [1, 1]]), None),
     ([2, 6, 20, 20], [12, 3, 3, 3], "f64", None, dict(groups=2, generic=True), None),
     ([8, 32, 14, 14], [32, 1, 3, 3], "f32", None, dict(groups=32, padding=[[1, 1], [1, 1]]), None),
+    # more than 128 output features: the window matrix is written to memory instead of being evaluated by the product
+    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "gemm_f32"),
 ]
 
 
