@@ -35,6 +35,7 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
   stencil chains ... brute-force loops on small grids
   while loops (src/Ops.jl:2349-2460; text form src/mlir/Dialects/StableHLO.jl:4850-4861)
       ... plain Python loops, closed forms, equality with the unrolled module
+  if / case (src/Ops.jl:2449-2470,2838,3198) ... plain Python branches
   reverse, reduce_window, convolution (src/Ops.jl:1000-1073,3967-4011;
       ext/ReactantNNlibExt/Implementations.jl:42-79, Ops.jl:1-32; src/TracedRArray.jl:1086-1108)
       ... reference KATs (test/core/ops.jl:609-618, test/nn/convolution.jl:206-217,
@@ -1461,6 +1462,16 @@ class Interpreter:
                 return [env[o] for o in op.operands]
             if op.name == "while":
                 outs = self._while(op, env)
+                for r, v in zip(op.results, outs):
+                    env[r] = v
+                continue
+            if op.name in ("if", "case"):
+                # only the selected region runs (reference src/Ops.jl:2449-2470,2838,3198); an index
+                # outside [0, n) selects the last branch
+                sel = env[op.operands[0]].a.reshape(-1)[0]
+                nbr = len(op.regions)
+                k = (0 if bool(sel) else 1) if op.name == "if" else (int(sel) if 0 <= int(sel) < nbr else nbr - 1)
+                outs = self._block([o for o in op.regions[k] if o.name != "__block_args__"], dict(env))
                 for r, v in zip(op.results, outs):
                     env[r] = v
                 continue

@@ -1098,7 +1098,9 @@ struct Builder {
       std::vector<int> in;
       for (auto& s : o.operands) in.push_back(look(s));
       if (o.name == "return" || o.name == "stablehlo.return" || o.name == "func.return") return in;
-      std::vector<int> outs = o.name == "stablehlo.while" ? run_while(o, in, env, depth) : build(o, in, depth);
+      std::vector<int> outs = o.name == "stablehlo.while" ? run_while(o, in, env, depth)
+                              : (o.name == "stablehlo.if" || o.name == "stablehlo.case") ? run_branches(o, in, env, depth)
+                                                                                         : build(o, in, depth);
       if (outs.size() != o.results.size()) fail("result count mismatch on " + o.name);
       for (size_t k = 0; k < outs.size(); ++k) env[o.results[k]] = outs[k];
     }
@@ -1200,6 +1202,74 @@ struct Builder {
     folded[id] = {ok, v};
     *out = v;
     return ok;
+  }
+
+  // `stablehlo.if` / `stablehlo.case` (what `@trace if` prints, reference src/Ops.jl:2449-2470,2838,3198).
+  // A predicate that folds to a constant selects its branch while importing.  Otherwise every
+  // branch is evaluated and the results are selected element by element: regions of this op set
+  // have no side effects, so the values are those of running the one branch.
+  std::vector<int> run_branches(const RawOp& o, const std::vector<int>& in, const std::map<std::string, int>& outer, int depth) {
+    if (depth > 16) fail(o.name + ": nesting depth exceeded");
+    const bool is_if = o.name == "stablehlo.if";
+    if (in.size() != 1 || ty(in[0]).numel() != 1 || ty(in[0]).rank() != 0) fail(o.name + ": expected one 0-d predicate / index operand");
+    if (is_if ? (o.regions.size() != 2 || ty(in[0]).dt != DT::I1) : (o.regions.empty() || !is_int_dt(ty(in[0]).dt) || ty(in[0]).dt == DT::I1))
+      fail(o.name + ": malformed regions or operand type");
+    const int nbr = (int)o.regions.size();
+    int64_t folded_v = 0;
+    const bool is_const = fold_int(in[0], &folded_v);
+    auto run_one = [&](int k) {
+      std::map<std::string, int> env = outer;
+      std::vector<int> r = run_block(o.regions[k], env, depth + 1);
+      if (r.size() != o.tout.size()) fail(o.name + ": a branch returns " + std::to_string(r.size()) + " values for " + std::to_string(o.tout.size()) + " results");
+      for (size_t q = 0; q < r.size(); ++q) if (!(ty(r[q]) == o.tout[q])) fail(o.name + ": branch result " + std::to_string(q) + " has type " + ty(r[q]).str());
+      return r;
+    };
+    if (is_const) {
+      // if: region 0 is the true branch; case: an index outside [0, n) selects the last branch
+      const int k = is_if ? (folded_v ? 0 : 1) : (int)((folded_v < 0 || folded_v >= nbr) ? nbr - 1 : folded_v);
+      return run_one(k);
+    }
+    std::vector<std::vector<int>> vals;
+    for (int k = 0; k < nbr; ++k) vals.push_back(run_one(k));
+    auto select_node = [&](int pred, int a, int b) {
+      const TType t = ty(a);
+      int p = pred;
+      if (t.rank() != 0) {
+        Node bc;
+        bc.k = OpK::BroadcastInDim;
+        bc.in = {pred};
+        bc.ty = TType{DT::I1, t.dims};
+        p = g.add(bc);
+      }
+      Node sn;
+      sn.k = OpK::Select;
+      sn.in = {p, a, b};
+      sn.ty = t;
+      return g.add(sn);
+    };
+    std::vector<int> out;
+    for (size_t q = 0; q < o.tout.size(); ++q) {
+      if (is_if) { out.push_back(select_node(in[0], vals[0][q], vals[1][q])); continue; }
+      // case: start from the last branch (also the out-of-range choice), override with index == k
+      int cur = vals[nbr - 1][q];
+      for (int k = nbr - 2; k >= 0; --k) {
+        Node c;
+        c.k = OpK::Constant;
+        c.splat = true;
+        c.ty = ty(in[0]);
+        c.data.assign((size_t)info(c.ty.dt).size, 0);
+        store_scalar(c.ty.dt, (double)k, k, true, c.data.data());
+        const int ci = g.add(c);
+        Node eq;
+        eq.k = OpK::Compare;
+        eq.op = "EQ";
+        eq.in = {in[0], ci};
+        eq.ty = TType{DT::I1, {}};
+        cur = select_node(g.add(eq), vals[k][q], cur);
+      }
+      out.push_back(cur);
+    }
+    return out;
   }
 
   std::vector<int> run_while(const RawOp& o, const std::vector<int>& init, const std::map<std::string, int>& outer, int depth) {

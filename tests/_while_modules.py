@@ -98,3 +98,58 @@ FILL = """module @reactant_fill attributes {mhlo.num_partitions = 1 : i64, mhlo.
     return %0 : tensor<4x3xf32>
   }
 }"""
+
+
+# `@trace if` (reference src/Ops.jl:2449-2470, 2838): both regions see the enclosing values
+IF = """module {
+  func.func @main(%arg0: tensor<8xf32>, %arg1: tensor<f32>) -> (tensor<8xf32>, tensor<f32>) {
+    %z = stablehlo.constant dense<0.000000e+00> : tensor<f32>
+    %p = stablehlo.compare GT, %arg1, %z : (tensor<f32>, tensor<f32>) -> tensor<i1>
+    %0:2 = "stablehlo.if"(%p) ({
+      %1 = stablehlo.sine %arg0 : tensor<8xf32>
+      %one = stablehlo.constant dense<1.000000e+00> : tensor<f32>
+      stablehlo.return %1, %one : tensor<8xf32>, tensor<f32>
+    }, {
+      %b = stablehlo.broadcast_in_dim %arg1, dims = [] : (tensor<f32>) -> tensor<8xf32>
+      %2 = stablehlo.multiply %arg0, %b : tensor<8xf32>
+      %3 = stablehlo.negate %arg1 : tensor<f32>
+      stablehlo.return %2, %3 : tensor<8xf32>, tensor<f32>
+    }) : (tensor<i1>) -> (tensor<8xf32>, tensor<f32>)
+    return %0#0, %0#1 : tensor<8xf32>, tensor<f32>
+  }
+}
+"""
+
+# `stablehlo.case` (src/Ops.jl:2890-3210): three branches on an i32 index; out-of-range indices take the last one
+CASE = """module {
+  func.func @main(%arg0: tensor<4x5xf64>, %arg1: tensor<i32>) -> tensor<4x5xf64> {
+    %0 = "stablehlo.case"(%arg1) ({
+      %1 = stablehlo.exponential %arg0 : tensor<4x5xf64>
+      stablehlo.return %1 : tensor<4x5xf64>
+    }, {
+      %2 = stablehlo.multiply %arg0, %arg0 : tensor<4x5xf64>
+      stablehlo.return %2 : tensor<4x5xf64>
+    }, {
+      %3 = stablehlo.negate %arg0 : tensor<4x5xf64>
+      stablehlo.return %3 : tensor<4x5xf64>
+    }) : (tensor<i32>) -> tensor<4x5xf64>
+    return %0 : tensor<4x5xf64>
+  }
+}
+"""
+
+# a predicate that is a constant selects its branch while the module is imported
+IF_CONST = """module {
+  func.func @main(%arg0: tensor<8xf32>) -> tensor<8xf32> {
+    %p = stablehlo.constant dense<false> : tensor<i1>
+    %0 = "stablehlo.if"(%p) ({
+      %1 = stablehlo.sine %arg0 : tensor<8xf32>
+      stablehlo.return %1 : tensor<8xf32>
+    }, {
+      %2 = stablehlo.cosine %arg0 : tensor<8xf32>
+      stablehlo.return %2 : tensor<8xf32>
+    }) : (tensor<i1>) -> tensor<8xf32>
+    return %0 : tensor<8xf32>
+  }
+}
+"""

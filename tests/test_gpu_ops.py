@@ -467,3 +467,24 @@ def test_reshapes_that_share_a_buffer(rx, client):
     got, exe = gpu_run(rx, client, t2, a)
     assert len(exe.launches()) == 2
     assert max_rel_to_scale(got[0].a, oracle_run(t2, a, hifi=True)[0].a) <= 1e-5
+
+
+def test_conditionals(rx, client):
+    """stablehlo.if / stablehlo.case: every branch is evaluated and the results selected."""
+    import _while_modules as W
+    x = I.tensor(np.arange(8) / 4, "f32")
+    exe = None
+    for s in (2.0, -3.0, 0.0):
+        args = [x, I.tensor(np.float32(s), "f32")]
+        got, exe = gpu_run(rx, client, W.IF, args, exe=exe)
+        ref = oracle_run(W.IF, args)
+        assert rel_err(got[0].a, ref[0].a) <= 1e-6 and float(got[1].a) == float(ref[1].a)
+    y = I.tensor(np.random.default_rng(0).normal(size=(4, 5)), "f64")
+    exe = None
+    for idx in (0, 1, 2, 7, -1):
+        args = [y, I.Tensor(np.int32(idx), "i32")]
+        got, exe = gpu_run(rx, client, W.CASE, args, exe=exe)
+        assert rel_err(got[0].a, oracle_run(W.CASE, args)[0].a) <= 1e-14
+    got, exe = gpu_run(rx, client, W.IF_CONST, [x])
+    assert rel_err(got[0].a, np.cos(x.a)) <= 1e-6
+    assert "select" not in exe.report() and ":: cosine" in exe.report()

@@ -368,3 +368,18 @@ def test_c_restatement_of_the_stencil_matches_the_interpreter(embed):
     got = build_c.stencil_steps(lib, *a, nx, ny, nz, 3, embed=embed)
     assert np.array_equal(got, ref)
     assert lib.rx_oracle_threads() >= 1
+
+
+def test_conditionals_against_plain_python():
+    x = np.arange(8, dtype=np.float32) / 4
+    for s in (2.0, -3.0):
+        a, b = I.run_text(W.IF, [I.tensor(x, "f32"), I.tensor(np.float32(s), "f32")])
+        if s > 0:
+            assert np.allclose(a.a, np.sin(x), rtol=1e-6) and float(b.a) == 1.0
+        else:
+            assert np.array_equal(a.a, x * np.float32(s)) and float(b.a) == -s
+    y = np.random.default_rng(0).normal(size=(4, 5))
+    for idx, want in ((0, np.exp(y)), (1, y * y), (2, -y), (7, -y), (-1, -y)):
+        got = I.run_text(W.CASE, [I.tensor(y, "f64"), I.Tensor(np.int32(idx), "i32")])[0].a
+        assert np.allclose(got, want, rtol=1e-14)
+    assert np.allclose(I.run_text(W.IF_CONST, [I.tensor(x, "f32")])[0].a, np.cos(x), rtol=1e-6)
