@@ -170,3 +170,39 @@ def test_short_contractions_keep_the_scalar_loop(rx, client):
     assert [l["kind"] for l in exe.launches()] == ["dot_scalar"]
     ref = oracle_run(text, [a, b], hifi=True)
     assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-5
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_operand_evaluated_inside_the_product_with_an_epilogue(rx, client, dt):
+    """A dot operand that expands smaller data (here a broadcast vector, scaled) is a functor of the
+    GEMM, on either side, next to an epilogue with an operand of its own."""
+    M, K, N = 64, 256, 4096
+    tA, tw, tB, tC, ts = _tt([M, K], dt), _tt([K], dt), _tt([K, N], dt), _tt([M, N], dt), _tt([N], dt)
+    text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg2: %s, %%arg3: %s) -> %s {\n"
+            "    %%wb = stablehlo.broadcast_in_dim %%arg1, dims = [0] : (%s) -> %s\n"
+            "    %%sb = stablehlo.broadcast_in_dim %%arg3, dims = [1] : (%s) -> %s\n"
+            "    %%b = stablehlo.multiply %%wb, %%sb : %s\n"
+            "    %%0 = stablehlo.dot_general %%arg0, %%b, contracting_dims = [1] x [0] : (%s, %s) -> %s\n"
+            "    %%1 = stablehlo.add %%0, %%arg2 : %s\n"
+            "    %%z = stablehlo.constant dense<0.000000e+00> : %s\n"
+            "    %%2 = stablehlo.maximum %%1, %%z : %s\n"
+            "    return %%2 : %s\n  }\n}\n" % (tA, tw, tC, ts, tC, tw, tB, ts, tB, tB, tA, tB, tC, tC, tC, tC, tC))
+    rng = np.random.default_rng(3)
+    args = [I.tensor(rng.normal(size=(M, K)), dt), I.tensor(rng.normal(size=(K,)), dt), I.tensor(rng.normal(size=(M, N)), dt),
+            I.tensor(rng.uniform(0.5, 1.5, size=(N,)), dt)]
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt], exe.report()
+    ref = oracle_run(text, args, hifi=True, excess=(dt == "bf16"))
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= (2e-2 if dt == "bf16" else 1e-5 * np.sqrt(K))
+    # the same product transposed: the expanded operand is now the left one
+    text2 = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg3: %s) -> %s {\n"
+             "    %%wb = stablehlo.broadcast_in_dim %%arg1, dims = [0] : (%s) -> %s\n"
+             "    %%sb = stablehlo.broadcast_in_dim %%arg3, dims = [1] : (%s) -> %s\n"
+             "    %%b = stablehlo.multiply %%wb, %%sb : %s\n"
+             "    %%0 = stablehlo.dot_general %%b, %%arg0, contracting_dims = [0] x [1] : (%s, %s) -> %s\n"
+             "    return %%0 : %s\n  }\n}\n" % (tA, tw, ts, _tt([N, M], dt), tw, tB, ts, tB, tB, tB, tA, _tt([N, M], dt), _tt([N, M], dt)))
+    args2 = [args[0], args[1], args[3]]
+    got, exe = gpu_run(rx, client, text2, args2)
+    assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt], exe.report()
+    ref = oracle_run(text2, args2, hifi=True, excess=(dt == "bf16"))
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= (2e-2 if dt == "bf16" else 1e-5 * np.sqrt(K))
