@@ -107,3 +107,39 @@ def test_fp8_linear_8192_rows_sampled(rx, client):
             I.Tensor.from_bytes(codes.tobytes(), "f8E4M3FN", (n, n)), I.Tensor(sw, "f32")]
     ref = oracle_run(P.fp8_linear(rows, n, n), args, hifi=True, excess=True)
     assert max_rel_to_scale(got[:rows], ref[0].a) <= 1e-2
+
+
+def test_tensors_of_more_than_2_31_elements(rx, client):
+    """Index arithmetic switches to 64 bits when a tensor has 2^31 elements or more: an elementwise
+    map with a shifted slice and a pad, a full reduction, a row and a column reduction, bit for bit
+    on i8 data (2 GiB per tensor)."""
+    n = (1 << 31) + 4096
+    t = "tensor<%dxi8>" % n
+    mapped = ("module { func.func @main(%%a: %s) -> %s {\n %%c = stablehlo.constant dense<3> : %s\n %%0 = stablehlo.multiply %%a, %%c : %s\n"
+              " %%1 = stablehlo.slice %%0 [5:%d] : (%s) -> tensor<%dxi8>\n %%z = stablehlo.constant dense<7> : tensor<i8>\n"
+              " %%2 = stablehlo.pad %%1, %%z, low = [2], high = [3], interior = [0] : (tensor<%dxi8>, tensor<i8>) -> %s\n return %%2 : %s } }"
+              % (t, t, t, t, n, t, n - 5, n - 5, t, t))
+    summed = ("module { func.func @main(%%a: %s) -> tensor<i64> {\n %%0 = stablehlo.convert %%a : (%s) -> tensor<%dxi64>\n"
+              " %%z = stablehlo.constant dense<0> : tensor<i64>\n"
+              " %%1 = stablehlo.reduce(%%0 init: %%z) applies stablehlo.add across dimensions = [0] : (tensor<%dxi64>, tensor<i64>) -> tensor<i64>\n"
+              " return %%1 : tensor<i64> } }" % (t, t, n, n))
+    rng = np.random.default_rng(0)
+    x = rng.integers(-20, 21, size=n, dtype=np.int8)
+    bx = rx.Buffer.from_host(client, x, "i8")
+    out = rx.xla_compile(client, mapped).execute_sharded([bx])[0].synced_buffer().to_host()
+    assert np.array_equal(out[2:n - 3], (x[5:] * np.int8(3)).astype(np.int8)) and (out[:2] == 7).all() and (out[n - 3:] == 7).all()
+    del out
+    total = rx.xla_compile(client, summed).execute_sharded([bx])[0].synced_buffer().to_host()
+    assert int(total) == int(x.sum(dtype=np.int64))
+    del bx, x
+    R, C = (1 << 16) + 1, 1 << 15
+    t2 = "tensor<%dx%dxi8>" % (R, C)
+    sums = ("module { func.func @main(%%a: %s) -> (tensor<%dxi32>, tensor<%dxi32>) {\n %%0 = stablehlo.convert %%a : (%s) -> tensor<%dx%dxi32>\n"
+            " %%z = stablehlo.constant dense<0> : tensor<i32>\n"
+            " %%1 = stablehlo.reduce(%%0 init: %%z) applies stablehlo.add across dimensions = [1] : (tensor<%dx%dxi32>, tensor<i32>) -> tensor<%dxi32>\n"
+            " %%2 = stablehlo.reduce(%%0 init: %%z) applies stablehlo.add across dimensions = [0] : (tensor<%dx%dxi32>, tensor<i32>) -> tensor<%dxi32>\n"
+            " return %%1, %%2 : tensor<%dxi32>, tensor<%dxi32> } }" % (t2, R, C, t2, R, C, R, C, R, R, C, C, R, C))
+    x2 = rng.integers(-20, 21, size=(R, C), dtype=np.int8)
+    outs = rx.xla_compile(client, sums).execute_sharded([rx.Buffer.from_host(client, x2, "i8")])
+    assert np.array_equal(outs[0].synced_buffer().to_host(), x2.sum(axis=1, dtype=np.int32))
+    assert np.array_equal(outs[1].synced_buffer().to_host(), x2.sum(axis=0, dtype=np.int32))
