@@ -2,16 +2,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stencil] [--no-others] [--no-cpu]
 
-Prints ONE JSON line.  The headline workload is BASELINE.json configs[1]: the 3-D
-diffusion/advection stencil, Float64 512x512x256 with 3-cell halos, 10 timesteps
-traced into one module.  A "step" is one execution of that module (10 timesteps)
+Prints ONE JSON line.  The headline workload is the 3-D diffusion/advection stencil,
+Float64 512x512x256 with 3-cell halos, 10 timesteps traced into one module.  A "step" is one execution of that module (10 timesteps)
 with all inputs resident in HBM; `value` is achieved HBM GB/s counting only the
 algorithmic bytes (per timestep: read c,u,v,w + write c over the interior
 = 5*512*512*256*8 B).  `roofline` describes the dominant kernel (the stencil kernel
 that advances two timesteps per launch: its algorithmic bytes are those of both), timed with HIP events on the stream it runs on, inside the timed
 region.  `cpu_baseline` times the oracle's C/OpenMP restatement of the stencil on the
 host cores (a bounded number of repetitions of the same module).  `others` carries the remaining four configs
-(sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry.
+(sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry; their step time is that
+of plain executions, and the pass with an event pair on every launch is reported beside it.
+`--workload conv|cumsum|maxpool` run one of the windowed ops instead (never part of `others`).
 """
 import argparse
 import importlib
