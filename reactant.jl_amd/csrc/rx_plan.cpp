@@ -168,7 +168,126 @@ struct Planner {
       }
     }
     dots_to_reductions();
+    normalize_dots();
     align_dots();
+  }
+
+  // A dot_general with several batch, free or contracting dims, or with them in another order than
+  // [batch, rows, k] / [batch, k, rows], is brought to the (batched) matrix form the GEMM skeletons
+  // understand: each operand is reshaped when its dims are already grouped that way (free of
+  // charge) and transposed first when they are not; the result is reshaped back.
+  void normalize_dots() {
+    if (!opt.mfma) return;
+    struct Form {
+      std::vector<int64_t> perm[2];   // operand dims in the order batch.., free.., contract.. (or batch.., contract.., free..)
+      bool kc[2];                     // contract dims last
+      bool transpose[2];
+      int64_t B, M, N, K;
+    };
+    std::map<int, Form> forms;
+    for (const Node& d : g.nodes) {
+      if (d.k != OpK::DotGeneral || d.a2.empty()) continue;
+      if (dot_form(d).ok) continue;
+      const TType &lt = g.nodes[d.in[0]].ty, &rt = g.nodes[d.in[1]].ty;
+      if (lt.numel() == 0 || rt.numel() == 0 || d.ty.numel() == 0) continue;
+      Form f;
+      // contracting pairs in the order of the lhs dims
+      std::vector<std::pair<int64_t, int64_t>> cp;
+      for (size_t k = 0; k < d.a2.size(); ++k) cp.push_back({d.a2[k], d.a3[k]});
+      std::sort(cp.begin(), cp.end());
+      auto isin = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+      f.B = f.M = f.N = f.K = 1;
+      for (auto b : d.a0) f.B *= lt.dims[b];
+      for (auto& c : cp) f.K *= lt.dims[c.first];
+      for (int side = 0; side < 2; ++side) {
+        const TType& t = side == 0 ? lt : rt;
+        const auto& batch = side == 0 ? d.a0 : d.a1;
+        const auto& contr = side == 0 ? d.a2 : d.a3;
+        std::vector<int64_t> fr, ct;
+        for (int k = 0; k < t.rank(); ++k) if (!isin(batch, k) && !isin(contr, k)) fr.push_back(k);
+        for (auto& c : cp) ct.push_back(side == 0 ? c.first : c.second);
+        for (auto k : fr) (side == 0 ? f.M : f.N) *= t.dims[k];
+        std::vector<int64_t> p_kc = batch, p_tr = batch;
+        p_kc.insert(p_kc.end(), fr.begin(), fr.end());
+        p_kc.insert(p_kc.end(), ct.begin(), ct.end());
+        p_tr.insert(p_tr.end(), ct.begin(), ct.end());
+        p_tr.insert(p_tr.end(), fr.begin(), fr.end());
+        auto identity = [](const std::vector<int64_t>& p) { for (size_t k = 0; k < p.size(); ++k) if (p[k] != (int64_t)k) return false; return true; };
+        if (identity(p_kc)) { f.perm[side] = p_kc; f.kc[side] = true; f.transpose[side] = false; }
+        else if (identity(p_tr)) { f.perm[side] = p_tr; f.kc[side] = false; f.transpose[side] = false; }
+        else { f.perm[side] = p_kc; f.kc[side] = true; f.transpose[side] = true; }
+      }
+      // worth it only if the matrix form reaches a skeleton (possibly after padding to whole vectors) or the reduction form
+      const DT a = lt.dt, b = rt.dt;
+      const int64_t ve = 16 / info(a).size;
+      auto up = [](int64_t x, int64_t m) { return (x + m - 1) / m * m; };
+      if (!choose_gemm(a, b, d.ty.dt, f.B, f.kc[0] ? f.M : up(f.M, ve), up(f.N, std::max<int64_t>(4, ve)), up(f.K, ve), f.kc[0], f.kc[1]).ok) continue;
+      forms[d.id] = f;
+    }
+    if (forms.empty()) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(g.nodes.size(), -1);
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      for (int& i : c.in) i = remap[i];
+      auto fi = forms.find(n.id);
+      if (fi == forms.end()) { remap[n.id] = out.add(c); continue; }
+      const Form& f = fi->second;
+      const bool batched = !n.a0.empty();
+      int opnd[2];
+      for (int side = 0; side < 2; ++side) {
+        int cur = c.in[side];
+        const TType t = out.nodes[cur].ty;
+        if (f.transpose[side]) {
+          Node tr;
+          tr.k = OpK::Transpose;
+          tr.in = {cur};
+          tr.a0 = f.perm[side];
+          tr.ty.dt = t.dt;
+          for (auto pdim : f.perm[side]) tr.ty.dims.push_back(t.dims[pdim]);
+          cur = out.add(tr);
+        }
+        const int64_t rows = side == 0 ? f.M : f.N;
+        std::vector<int64_t> md;
+        if (batched) md.push_back(f.B);
+        if (f.kc[side]) { md.push_back(rows); md.push_back(f.K); } else { md.push_back(f.K); md.push_back(rows); }
+        if (out.nodes[cur].ty.dims != md) {
+          Node rs;
+          rs.k = OpK::Reshape;
+          rs.in = {cur};
+          rs.ty = TType{t.dt, md};
+          cur = out.add(rs);
+        }
+        opnd[side] = cur;
+      }
+      Node dn;
+      dn.k = OpK::DotGeneral;
+      dn.op = n.op;
+      dn.in = {opnd[0], opnd[1]};
+      const int64_t nb = batched ? 1 : 0;
+      if (batched) { dn.a0 = {0}; dn.a1 = {0}; }
+      dn.a2 = {nb + (f.kc[0] ? 1 : 0)};
+      dn.a3 = {nb + (f.kc[1] ? 1 : 0)};
+      dn.ty.dt = n.ty.dt;
+      if (batched) dn.ty.dims.push_back(f.B);
+      dn.ty.dims.push_back(f.M);
+      dn.ty.dims.push_back(f.N);
+      int cur = out.add(dn);
+      if (out.nodes[cur].ty.dims != n.ty.dims) {
+        Node rs;
+        rs.k = OpK::Reshape;
+        rs.in = {cur};
+        rs.ty = n.ty;
+        cur = out.add(rs);
+      }
+      remap[n.id] = cur;
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // A dot_general operand that is a cheap expansion of much smaller data -- the window matrix of a

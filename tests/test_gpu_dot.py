@@ -206,3 +206,28 @@ def test_operand_evaluated_inside_the_product_with_an_epilogue(rx, client, dt):
     assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt], exe.report()
     ref = oracle_run(text2, args2, hifi=True, excess=(dt == "bf16"))
     assert max_rel_to_scale(got[0].a, ref[0].a) <= (2e-2 if dt == "bf16" else 1e-5 * np.sqrt(K))
+
+
+GENERAL_DOTS = [
+    # lhs, rhs, out, attributes, dtype: forms that are reshaped (and where needed transposed) into batched matrix products
+    ([64, 96, 12], [96, 80, 12], [12, 64, 80], "batching_dims = [2] x [2], contracting_dims = [1] x [0]", "f32"),       # NNlib.batched_mul layout
+    ([3, 4, 64, 96], [3, 4, 96, 80], [3, 4, 64, 80], "batching_dims = [0, 1] x [0, 1], contracting_dims = [3] x [2]", "bf16"),
+    ([128, 8, 16], [8, 16, 192], [128, 192], "contracting_dims = [1, 2] x [0, 1]", "f32"),
+    ([16, 8, 128], [128, 12, 16], [16, 8, 12, 16], "contracting_dims = [2] x [0]", "f32"),
+    ([128, 8, 16], [16, 8, 192], [128, 192], "contracting_dims = [1, 2] x [1, 0]", "f64"),
+    ([5, 64, 7, 32], [32, 5, 96], [5, 64, 7, 96], "batching_dims = [0] x [1], contracting_dims = [3] x [0]", "f32"),
+]
+
+
+@pytest.mark.parametrize("ls,rs,os_,attrs,dt", GENERAL_DOTS)
+def test_dot_general_with_grouped_or_permuted_dims(rx, client, ls, rs, os_, attrs, dt):
+    text = _dot_text(ls, rs, os_, attrs, dt)
+    rng = np.random.default_rng(11)
+    a, b = I.tensor(rng.normal(size=ls), dt), I.tensor(rng.normal(size=rs), dt)
+    got, exe = gpu_run(rx, client, text, [a, b])
+    kinds = [l["kind"] for l in exe.launches()]
+    assert any(k.startswith("gemm_") for k in kinds) and "dot_scalar" not in kinds, kinds
+    ref = oracle_run(text, [a, b], hifi=True)
+    assert got[0].a.shape == ref[0].a.shape
+    err = max_rel_to_scale(got[0].a, ref[0].a)
+    assert err <= {"bf16": 1e-2, "f64": 1e-13, "f32": 1e-4}[dt]
