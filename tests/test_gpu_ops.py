@@ -322,12 +322,14 @@ def test_while_generic_form_returns_counter_and_value(rx, client):
 
 
 # ---- division by a broadcast scalar ------------------------------------------------------------
-@pytest.mark.parametrize("divisor", [3.0, 0.1, 448.0, 1e-40, 3.4e38, 0.0, -7.25, float("inf")])
+@pytest.mark.parametrize("divisor", [3.0, 0.1, 448.0, 1e-40, 3.4e38, 0.0, -7.25, float("inf"), 1.9999999, 0.99999994, 0.012125223,
+                                     3.6379788e-12, 3.63797e-12, 5.4975581e11, 5.49756e11, -1.0000001])
 def test_divide_by_a_broadcast_scalar_is_correctly_rounded(rx, client, divisor):
     """x / s with s one value for the whole tensor is evaluated as a product with the double
     reciprocal; it must round exactly like the IEEE division (bit-for-bit against numpy),
-    including subnormal and huge divisors, zeros, infinities and quotients next to a tie."""
-    n = 1 << 16
+    including subnormal and huge divisors, divisors with an all-ones mantissa, zeros, infinities
+    and quotients next to a tie."""
+    n = 1 << 20
     rng = np.random.default_rng(5)
     x = rng.integers(0, 2 ** 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32).copy()
     x[: n // 2] = rng.normal(size=n // 2).astype(np.float32) * np.float32(100)
