@@ -1733,10 +1733,16 @@ struct Builder {
     {
       std::vector<int64_t> lo(r, 0), hi(r, 0), interior(r, 0);
       bool any = false;
+      // negative padding (the gradient forms produce it) crops the dilated input: pad by the
+      // non-negative parts, then slice the rest off
+      std::vector<int64_t> crop_lo(r, 0), crop_hi(r, 0);
+      bool any_crop = false;
       for (int d = 0; d < nsp; ++d) {
-        lo[2 + d] = pad[2 * d]; hi[2 + d] = pad[2 * d + 1]; interior[2 + d] = ld[d] - 1;
-        if (lo[2 + d] < 0 || hi[2 + d] < 0 || ld[d] < 1) fail("convolution: negative padding is not supported");
+        if (ld[d] < 1) fail("convolution: lhs_dilation must be positive");
+        lo[2 + d] = std::max<int64_t>(pad[2 * d], 0); hi[2 + d] = std::max<int64_t>(pad[2 * d + 1], 0); interior[2 + d] = ld[d] - 1;
+        crop_lo[2 + d] = std::max<int64_t>(-pad[2 * d], 0); crop_hi[2 + d] = std::max<int64_t>(-pad[2 * d + 1], 0);
         any = any || lo[2 + d] || hi[2 + d] || interior[2 + d];
+        any_crop = any_crop || crop_lo[2 + d] || crop_hi[2 + d];
       }
       if (any) {
         Node pn;
@@ -1746,6 +1752,22 @@ struct Builder {
         pn.ty.dt = xct.dt;
         for (int d = 0; d < r; ++d) pn.ty.dims.push_back(lo[d] + hi[d] + xct.dims[d] + std::max<int64_t>(xct.dims[d] - 1, 0) * interior[d]);
         xc = g.add(pn);
+      }
+      if (any_crop) {
+        const TType t = ty(xc);
+        Node sl;
+        sl.k = OpK::Slice;
+        sl.in = {xc};
+        sl.a0 = crop_lo;
+        sl.a2.assign(r, 1);
+        sl.ty.dt = t.dt;
+        for (int d = 0; d < r; ++d) {
+          const int64_t lim = t.dims[d] - crop_hi[d];
+          if (lim < crop_lo[d]) fail("convolution: negative padding removes more than the input holds");
+          sl.a1.push_back(lim);
+          sl.ty.dims.push_back(lim - crop_lo[d]);
+        }
+        xc = g.add(sl);
       }
     }
     std::vector<int64_t> wsz{1, 1}, wst{1, 1}, wdl{1, 1};

@@ -346,3 +346,21 @@ def test_gather(rx, client, os_, ss,rs, dt, od, cd, sim, ivd, sz, bat):
     assert got[0].a.shape == ref[0].a.shape
     assert np.array_equal(got[0].a, ref[0].a)
     assert [l["kind"] for l in exe.launches()] == ["map"]
+
+
+def test_convolution_gradient_forms(rx, client):
+    """Filter and data gradients of a convolution as the reference builds them
+    (ext/ReactantNNlibExt/Implementations.jl:85-251): batch and feature roles swapped, input
+    dilation, reversed kernel.  The oracle's values for these forms are pinned against the
+    definition of the derivative in tests/test_oracle_windows.py."""
+    from test_oracle_windows import _grad_cases, conv_grad_modules
+    rng = np.random.default_rng(41)
+    cases = _grad_cases() + [dict(W=28, H=28, ci=16, co=32, B=8, kw=3, kh=3, s=(1, 1), p=(1, 1), d=(1, 1)),
+                             dict(W=32, H=32, ci=8, co=16, B=4, kw=5, kh=5, s=(2, 2), p=(2, 2), d=(1, 1))]
+    for c in cases:
+        tf, td, xs, ws, ys = conv_grad_modules(c, "f32")
+        x, w, dy = I.tensor(rng.normal(size=xs), "f32"), I.tensor(rng.normal(size=ws), "f32"), I.tensor(rng.normal(size=ys), "f32")
+        got, _ = gpu_run(rx, client, tf, [x, dy])
+        _close(got[0].a, oracle_run(tf, [x, dy], hifi=True)[0].a, 1e-5 * np.sqrt(ys[0] * ys[1] * ys[3]))
+        got, _ = gpu_run(rx, client, td, [dy, w])
+        _close(got[0].a, oracle_run(td, [dy, w], hifi=True)[0].a, 1e-5 * np.sqrt(ws[0] * ws[1] * ws[3]))

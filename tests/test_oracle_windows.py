@@ -251,3 +251,68 @@ def test_gather_against_numpy_indexing():
     got = I.run_text(t, [I.tensor(y, "f64"), I.Tensor(starts, "i64")])[0].a
     want = np.stack([[y[b, np.clip(s, 0, 17):np.clip(s, 0, 17) + 3] for s in starts[b]] for b in range(4)])
     assert np.array_equal(got, want)
+
+
+def _grad_cases():
+    """x [w, h, cin, b], w [kw, kh, cin, cout] (Julia dim order, as the traced program sees them), forward
+    cross-correlation with stride s, padding p (symmetric per dim), dilation d."""
+    return [dict(W=9, H=8, ci=3, co=4, B=2, kw=3, kh=2, s=(1, 1), p=(0, 0), d=(1, 1)),
+            dict(W=10, H=9, ci=2, co=3, B=2, kw=3, kh=3, s=(2, 1), p=(1, 2), d=(1, 1)),
+            dict(W=11, H=10, ci=2, co=2, B=3, kw=2, kh=3, s=(1, 2), p=(2, 0), d=(2, 1))]
+
+
+def _dil(n, d):
+    return max(0, 1 + d * (n - 1))
+
+
+def conv_grad_modules(c, dt):
+    """The two gradient convolutions as ext/ReactantNNlibExt/Implementations.jl:85-251 builds them."""
+    ow = (c["W"] + 2 * c["p"][0] - _dil(c["kw"], c["d"][0])) // c["s"][0] + 1
+    oh = (c["H"] + 2 * c["p"][1] - _dil(c["kh"], c["d"][1])) // c["s"][1] + 1
+    xs, ws, ys = [c["W"], c["H"], c["ci"], c["B"]], [c["kw"], c["kh"], c["ci"], c["co"]], [ow, oh, c["co"], c["B"]]
+    lhs_shape, k_shape, o_shape = (c["W"], c["H"]), (_dil(c["kw"], c["d"][0]), _dil(c["kh"], c["d"][1])), (_dil(ow, c["s"][0]), _dil(oh, c["s"][1]))
+    # filter gradient: x is the input with batch = cin, feature = b; dy is the kernel with o = cout, i = b
+    padf = [[c["p"][i], o_shape[i] - lhs_shape[i] + k_shape[i] - c["p"][i] - 1] for i in range(2)]
+    tf, outf = NN.convolution(xs, ys, dt, dims="[0, 1, b, f]x[0, 1, o, i]->[0, 1, b, f]", strides=list(c["d"]), padding=padf, rhs_dil=list(c["s"]))
+    assert outf == ws, (outf, ws)
+    # data gradient: dy is the input (dilated by the stride), the reversed kernel has o = cin, i = cout
+    padd = []
+    for i in range(2):
+        before = k_shape[i] - c["p"][i] - 1
+        padd.append([before, lhs_shape[i] + k_shape[i] - 1 - o_shape[i] - before])
+    td, outd = NN.convolution(ys, ws, dt, dims="[0, 1, f, b]x[0, 1, o, i]->[0, 1, f, b]", padding=padd, lhs_dil=list(c["s"]), rhs_dil=list(c["d"]), flip=True)
+    assert outd == xs, (outd, xs)
+    return tf, td, xs, ws, ys
+
+
+def conv_grads_brute(c, x, w, dy):
+    """Derivatives of sum(y * dy), y the forward cross-correlation, from the definition."""
+    ow, oh = dy.shape[0], dy.shape[1]
+    dw, dx = np.zeros_like(w), np.zeros_like(x)
+    for kx in range(c["kw"]):
+        for ky in range(c["kh"]):
+            for ox in range(ow):
+                ix = ox * c["s"][0] + kx * c["d"][0] - c["p"][0]
+                if not 0 <= ix < c["W"]:
+                    continue
+                for oy in range(oh):
+                    iy = oy * c["s"][1] + ky * c["d"][1] - c["p"][1]
+                    if not 0 <= iy < c["H"]:
+                        continue
+                    dw[kx, ky] += x[ix, iy] @ dy[ox, oy].T                 # [ci, b] x [b, co]
+                    dx[ix, iy] += w[kx, ky] @ dy[ox, oy]                   # [ci, co] x [co, b]
+    return dw, dx
+
+
+def test_convolution_gradient_forms_against_the_definition():
+    """The dimension-number forms of the filter and data gradients (batch and feature roles swapped,
+    input dilation, reversed kernel) give the derivatives of the forward pass."""
+    rng = np.random.default_rng(6)
+    for c in _grad_cases():
+        tf, td, xs, ws, ys = conv_grad_modules(c, "f64")
+        x, w, dy = rng.normal(size=xs), rng.normal(size=ws), rng.normal(size=ys)
+        dw, dx = conv_grads_brute(c, x, w, dy)
+        got_w = I.run_text(tf, [I.tensor(x, "f64"), I.tensor(dy, "f64")])[0].a
+        got_x = I.run_text(td, [I.tensor(dy, "f64"), I.tensor(w, "f64")])[0].a
+        assert np.allclose(got_w, dw, rtol=1e-12, atol=1e-12), c
+        assert np.allclose(got_x, dx, rtol=1e-12, atol=1e-12), c
