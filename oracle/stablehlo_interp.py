@@ -1370,8 +1370,18 @@ def _convolution(x, w, at, dt_out, hifi):
     rdil = at.get("rhs_dilation") or [1] * nsp
     rev = at.get("window_reversal") or [False] * nsp
     G = at.get("feature_group_count", 1)
-    if at.get("batch_group_count", 1) != 1:
-        raise NotImplementedError("convolution with batch_group_count != 1")
+    BG = at.get("batch_group_count", 1)
+    if BG != 1:
+        # the specification: split the input along its batch dim and the kernel along its output
+        # feature dim into BG parts, convolve part with part, concatenate along the output features
+        if G != 1:
+            raise ValueError("convolution: batch_group_count and feature_group_count cannot both exceed 1")
+        at1 = dict(at)
+        at1["batch_group_count"] = 1
+        xs = np.split(x.a, BG, axis=dn["lhs_0"])
+        ws = np.split(w.a, BG, axis=dn["rhs_0"])
+        parts = [_convolution(_FloatView(xg, x.dt), _FloatView(wg, w.dt), at1, dt_out, hifi).a for xg, wg in zip(xs, ws)]
+        return Tensor(np.concatenate(parts, axis=dn["out_1"]), dt_out) if not is_float(dt_out) else tensor(np.concatenate(parts, axis=dn["out_1"]), dt_out)
     acc = np.float64 if (hifi or x.dt == "f64") else (np.float32 if is_float(x.dt) else NP_OF[dt_out])
     xa = np.transpose(x.a, [dn["lhs_0"], dn["lhs_1"]] + dn["lhs_spatial"]).astype(acc)     # [b, f, s...]
     wa = np.transpose(w.a, [dn["rhs_0"], dn["rhs_1"]] + dn["rhs_spatial"]).astype(acc)     # [o, i, k...]

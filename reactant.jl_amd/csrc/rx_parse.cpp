@@ -1693,7 +1693,7 @@ struct Builder {
     if ((int)pad.size() != 2 * nsp) fail("convolution: padding must be a (spatial rank x 2) matrix");
     const int64_t G = o.ia.count("feature_group_count") && !o.ia.at("feature_group_count").empty() ? o.ia.at("feature_group_count")[0] : 1;
     const int64_t BG = o.ia.count("batch_group_count") && !o.ia.at("batch_group_count").empty() ? o.ia.at("batch_group_count")[0] : 1;
-    if (BG != 1) fail("convolution: batch_group_count other than 1 is not supported");
+    if (BG < 1 || (BG > 1 && G > 1)) fail("convolution: batch_group_count and feature_group_count cannot both exceed 1");
     if (G < 1) fail("convolution: feature_group_count must be positive");
 
     // canonical orders: input [b, f, s...], kernel [o, i, k...]
@@ -1729,6 +1729,8 @@ struct Builder {
     const TType xct = ty(xc), wct = ty(wc);
     const int64_t B = xct.dims[0], C = xct.dims[1], O = wct.dims[0], I = wct.dims[1];
     if (C != I * G || O % G != 0) fail("convolution: feature counts do not match feature_group_count");
+    if (B % BG != 0 || O % BG != 0) fail("convolution: batch and output feature counts must be multiples of batch_group_count");
+    const int64_t Bo = B / BG;    // batch entries of the result
     // dilate and pad the input
     {
       std::vector<int64_t> lo(r, 0), hi(r, 0), interior(r, 0);
@@ -1781,7 +1783,7 @@ struct Builder {
     // expected result shape
     {
       std::vector<int64_t> want(r);
-      want[cd[2].d0] = B; want[cd[2].d1] = O;
+      want[cd[2].d0] = Bo; want[cd[2].d1] = O;
       for (int d = 0; d < nsp; ++d) want[cd[2].sp[d]] = osp[d];
       if (want != out.dims) fail("convolution: result shape mismatch");
     }
@@ -1808,10 +1810,30 @@ struct Builder {
       for (auto pdim : t.a0) t.ty.dims.push_back(d1[pdim]);
       cur = g.add(t);
     }
+    // batch groups (the filter gradient of a grouped convolution): output features of group g see only
+    // the batch entries of group g, i.e. one product per group: [C, k..., (g, b'), o...] -> [g, C, k..., b', o...]
+    if (BG > 1) {
+      const TType t = ty(cur);
+      std::vector<int64_t> sd;
+      for (int d = 0; d <= nsp; ++d) sd.push_back(t.dims[d]);
+      sd.push_back(BG);
+      sd.push_back(Bo);
+      for (int d = 0; d < nsp; ++d) sd.push_back(t.dims[nsp + 2 + d]);
+      cur = add_node(OpK::Reshape, TType{t.dt, sd}, {cur});
+      Node tr;
+      tr.k = OpK::Transpose;
+      tr.in = {cur};
+      tr.a0.push_back(nsp + 1);
+      for (int d = 0; d <= nsp; ++d) tr.a0.push_back(d);
+      for (int d = nsp + 2; d < (int)sd.size(); ++d) tr.a0.push_back(d);
+      tr.ty.dt = t.dt;
+      for (auto pdim : tr.a0) tr.ty.dims.push_back(sd[pdim]);
+      cur = g.add(tr);
+    }
     // The MFMA skeletons read 16-byte vectors along the contracted dimension of the weights and along
     // the columns of the window matrix: both are padded with zeros to whole vectors (the extra
     // columns are sliced off the product).
-    const int64_t K = I * taps, N = B * P;
+    const int64_t K = I * taps, N = Bo * P;
     int64_t Kp = K, Np = N;
     if (xct.dt == DT::F32 || xct.dt == DT::BF16 || xct.dt == DT::F16 || xct.dt == DT::F64) {
       const int64_t ve = std::max<int64_t>(4, 16 / info(xct.dt).size);
@@ -1836,7 +1858,12 @@ struct Builder {
     Node dot;
     dot.k = OpK::DotGeneral;
     int lhs, rhs;
-    if (G == 1) {
+    if (BG > 1) {
+      lhs = padded(add_node(OpK::Reshape, TType{xct.dt, {BG, O / BG, K}}, {wc}), {0, 0, Kp - K});
+      rhs = padded(add_node(OpK::Reshape, TType{xct.dt, {BG, K, N}}, {cur}), {0, Kp - K, Np - N});
+      dot.a0 = {0}; dot.a1 = {0}; dot.a2 = {2}; dot.a3 = {1};
+      dot.ty = TType{out.dt, {BG, O / BG, Np}};
+    } else if (G == 1) {
       lhs = padded(add_node(OpK::Reshape, TType{xct.dt, {O, K}}, {wc}), {0, Kp - K});
       rhs = padded(add_node(OpK::Reshape, TType{xct.dt, {K, N}}, {cur}), {Kp - K, Np - N});
       dot.a2 = {1}; dot.a3 = {0};
@@ -1863,7 +1890,7 @@ struct Builder {
       cur = g.add(sl);
     }
     // [O, B, o...] -> the result's own dimension order
-    std::vector<int64_t> obd{O, B};
+    std::vector<int64_t> obd{O, Bo};
     for (auto v : osp) obd.push_back(v);
     std::vector<int64_t> perm(r);
     perm[cd[2].d0] = 1; perm[cd[2].d1] = 0;

@@ -82,7 +82,7 @@ def conv_out_shape(x_sp, k_sp, strides, padding, lhs_dil, rhs_dil):
 
 
 def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0]", strides=None, padding=None,
-                lhs_dil=None, rhs_dil=None, groups=1, flip=False, generic=False, epilogue=None):
+                lhs_dil=None, rhs_dil=None, groups=1, flip=False, generic=False, epilogue=None, batch_groups=1):
     """`dims` uses the textual dimension numbers; spatial dim s of the input has the size
     x_shape[position of s].  With `flip` the kernel's spatial dims are reversed first (NNlib's true
     convolution).  `epilogue="bias_relu"` adds a per-feature bias and a relu, the fused form LuxLib emits."""
@@ -101,7 +101,7 @@ def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1,
     k_sp = [w_shape[pos[1][str(s)]] for s in range(nsp)]
     o_sp = conv_out_shape(x_sp, k_sp, strides, padding, lhs_dil, rhs_dil)
     out = [0] * len(x_shape)
-    out[pos[2]["b"]] = x_shape[pos[0]["b"]]
+    out[pos[2]["b"]] = x_shape[pos[0]["b"]] // batch_groups
     out[pos[2]["f"]] = w_shape[pos[1]["o"]]
     for s in range(nsp):
         out[pos[2][str(s)]] = o_sp[s]
@@ -116,17 +116,17 @@ def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1,
     if generic:
         arr = lambda v: "array<i64: " + ", ".join(str(x) for x in v) + ">"
         pad = "dense<[" + ", ".join("[%d, %d]" % (p[0], p[1]) for p in padding) + "]> : tensor<%dx2xi64>" % nsp
-        body += ("    %%0 = \"stablehlo.convolution\"(%%arg0, %s) <{batch_group_count = 1 : i64, dimension_numbers = "
+        body += ("    %%0 = \"stablehlo.convolution\"(%%arg0, %s) <{batch_group_count = %d : i64, dimension_numbers = "
                  "#stablehlo.conv<%s>, feature_group_count = %d : i64, lhs_dilation = %s, padding = %s, "
                  "precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>], rhs_dilation = %s, "
                  "window_strides = %s}> : (%s, %s) -> %s\n"
-                 % (wname, dims, groups, arr(lhs_dil), pad, arr(rhs_dil), arr(strides), tx, tw, to))
+                 % (wname, batch_groups, dims, groups, arr(lhs_dil), pad, arr(rhs_dil), arr(strides), tx, tw, to))
     else:
         body += ("    %%0 = stablehlo.convolution(%%arg0, %s) dim_numbers = %s, window = {stride = %s, pad = %s, "
-                 "lhs_dilate = %s, rhs_dilate = %s} {batch_group_count = 1 : i64, feature_group_count = %d : i64, "
+                 "lhs_dilate = %s, rhs_dilate = %s} {batch_group_count = %d : i64, feature_group_count = %d : i64, "
                  "precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>]} : (%s, %s) -> %s\n"
                  % (wname, dims, lst(strides), "[" + ", ".join(lst(p) for p in padding) + "]", lst(lhs_dil), lst(rhs_dil),
-                    groups, tx, tw, to))
+                    batch_groups, groups, tx, tw, to))
     args = "%%arg0: %s, %%arg1: %s" % (tx, tw)
     res = "%0"
     if epilogue == "bias_relu":

@@ -254,5 +254,5 @@ def test_windowed_ops_plan(monkeypatch):
     rep = rx.compile_offline(conv, with_source=True)
     assert kinds(rep) == ["map", "gemm_f32", "map"] and "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rep
     monkeypatch.delenv("RX_FUSE_DOT_OPERANDS")
-    with pytest.raises(Exception, match="batch_group_count"):
-        rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 8, 4, 4], "f32")[0].replace("batch_group_count = 1", "batch_group_count = 2"))
+    with pytest.raises(Exception, match="batch_group_count and feature_group_count"):
+        rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 4, 4, 4], "f32", groups=2)[0].replace("batch_group_count = 1", "batch_group_count = 2"))

@@ -364,3 +364,15 @@ def test_convolution_gradient_forms(rx, client):
         _close(got[0].a, oracle_run(tf, [x, dy], hifi=True)[0].a, 1e-5 * np.sqrt(ys[0] * ys[1] * ys[3]))
         got, _ = gpu_run(rx, client, td, [dy, w])
         _close(got[0].a, oracle_run(td, [dy, w], hifi=True)[0].a, 1e-5 * np.sqrt(ws[0] * ws[1] * ws[3]))
+
+
+def test_grouped_filter_gradient(rx, client):
+    """`batch_group_count`: the filter gradient of a grouped convolution, one product per group."""
+    from test_oracle_windows import grouped_filter_grad_module
+    rng = np.random.default_rng(43)
+    for groups, c in ((2, dict(W=9, H=8, ci=4, co=6, B=2, kw=3, kh=2, s=(1, 1), p=(1, 0), d=(1, 1))),
+                      (4, dict(W=28, H=28, ci=32, co=64, B=8, kw=3, kh=3, s=(1, 1), p=(1, 1), d=(1, 1)))):
+        tf, xs, ws, ys = grouped_filter_grad_module(c, groups, "f32")
+        x, dy = I.tensor(rng.normal(size=xs), "f32"), I.tensor(rng.normal(size=ys), "f32")
+        got, _ = gpu_run(rx, client, tf, [x, dy])
+        _close(got[0].a, oracle_run(tf, [x, dy], hifi=True)[0].a, 1e-5 * np.sqrt(ys[0] * ys[1] * ys[3]))

@@ -316,3 +316,34 @@ def test_convolution_gradient_forms_against_the_definition():
         got_x = I.run_text(td, [I.tensor(dy, "f64"), I.tensor(w, "f64")])[0].a
         assert np.allclose(got_w, dw, rtol=1e-12, atol=1e-12), c
         assert np.allclose(got_x, dx, rtol=1e-12, atol=1e-12), c
+
+
+def grouped_filter_grad_module(c, groups, dt):
+    """Filter gradient of a grouped convolution: `batch_group_count = groups`
+    (ext/ReactantNNlibExt/Implementations.jl:85-140)."""
+    ow = (c["W"] + 2 * c["p"][0] - _dil(c["kw"], c["d"][0])) // c["s"][0] + 1
+    oh = (c["H"] + 2 * c["p"][1] - _dil(c["kh"], c["d"][1])) // c["s"][1] + 1
+    xs, ys = [c["W"], c["H"], c["ci"], c["B"]], [ow, oh, c["co"], c["B"]]
+    ws = [c["kw"], c["kh"], c["ci"] // groups, c["co"]]
+    lhs_shape, k_shape, o_shape = (c["W"], c["H"]), (_dil(c["kw"], c["d"][0]), _dil(c["kh"], c["d"][1])), (_dil(ow, c["s"][0]), _dil(oh, c["s"][1]))
+    padf = [[c["p"][i], o_shape[i] - lhs_shape[i] + k_shape[i] - c["p"][i] - 1] for i in range(2)]
+    tf, outf = NN.convolution(xs, ys, dt, dims="[0, 1, b, f]x[0, 1, o, i]->[0, 1, b, f]", strides=list(c["d"]), padding=padf,
+                              rhs_dil=list(c["s"]), batch_groups=groups)
+    assert outf == ws, (outf, ws)
+    return tf, xs, ws, ys
+
+
+def test_grouped_filter_gradient_against_the_definition():
+    rng = np.random.default_rng(7)
+    for groups, c in ((2, dict(W=9, H=8, ci=4, co=6, B=2, kw=3, kh=2, s=(1, 1), p=(1, 0), d=(1, 1))),
+                      (3, dict(W=10, H=7, ci=6, co=3, B=3, kw=2, kh=2, s=(2, 1), p=(0, 1), d=(1, 2)))):
+        tf, xs, ws, ys = grouped_filter_grad_module(c, groups, "f64")
+        x, dy = rng.normal(size=xs), rng.normal(size=ys)
+        cpg, opg = c["ci"] // groups, c["co"] // groups
+        dw = np.zeros(ws)
+        for g in range(groups):
+            cg = dict(c, ci=cpg, co=opg)
+            dwg, _ = conv_grads_brute(cg, x[:, :, g * cpg:(g + 1) * cpg], np.zeros([c["kw"], c["kh"], cpg, opg]), dy[:, :, g * opg:(g + 1) * opg])
+            dw[:, :, :, g * opg:(g + 1) * opg] = dwg
+        got = I.run_text(tf, [I.tensor(x, "f64"), I.tensor(dy, "f64")])[0].a
+        assert np.allclose(got, dw, rtol=1e-12, atol=1e-12), (groups, c)
