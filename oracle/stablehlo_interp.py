@@ -44,6 +44,9 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       numpy accumulate (tests/test_oracle_windows.py)
   gather (src/Ops.jl:2269-2345; NNlib.gather, ext/ReactantNNlibExt/Implementations.jl:426-438)
       ... reference KATs (test/nn/scatter_gather.jl:5-99), numpy fancy indexing with clamping
+  scatter (src/Ops.jl:2150-2268) ... numpy indexed assignment and np.add.at, dropped
+      out-of-range updates (whole windows, as XLA does; the StableHLO text says per element:
+      PARITY UNPINNED between the two readings, the reference holds no case that tells them apart)
   reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy
       max / argmax / argmin with ties, first and last index
   batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
@@ -560,6 +563,15 @@ class Parser:
         mo = re.search(r"#stablehlo\.conv<([^>]*->[^>]*)>", inner)
         if mo:
             a["dim_numbers"] = _parse_conv_dims(mo.group(1))
+        mo = re.search(r"#stablehlo\.scatter<([^>]*)>", inner)
+        if mo:
+            d = mo.group(1)
+            for k in ("update_window_dims", "inserted_window_dims", "input_batching_dims", "scatter_indices_batching_dims",
+                      "scatter_dims_to_operand_dims"):
+                m2 = re.search(k + r"\s*=\s*\[([-\d,\s]*)\]", d)
+                a[k] = [int(t) for t in m2.group(1).replace(",", " ").split()] if m2 else []
+            m2 = re.search(r"index_vector_dim\s*=\s*(\d+)", d)
+            a["index_vector_dim"] = int(m2.group(1)) if m2 else 0
         mo = re.search(r"#stablehlo\.gather<([^>]*)>", inner)
         if mo:
             d = mo.group(1)
@@ -1520,6 +1532,47 @@ class Interpreter:
                 raise ValueError("while body returns %d values for %d loop-carried ones" % (len(cur), len(op.operands)))
         raise ValueError("while loop did not terminate")
 
+    def _scatter(self, op, xs):
+        """stablehlo.scatter (built by reference src/Ops.jl:2150-2268), update by update in row-major
+        order of the update tensor.  As XLA does, an update window that does not lie wholly inside
+        the operand is dropped as a whole."""
+        at = op.attrs
+        operand, start, upd = xs
+        uwd, iwd = at.get("update_window_dims", []), at.get("inserted_window_dims", [])
+        ibd, sbd = at.get("input_batching_dims", []), at.get("scatter_indices_batching_dims", [])
+        sdo, ivd = at.get("scatter_dims_to_operand_dims", []), at.get("index_vector_dim", 0)
+        res = operand.a.copy()
+        st = start.a.astype(np.int64)
+        region = op.regions[0]
+        names = [nm for nm, _ in region[0].attrs["args"]]
+        body = [o for o in region if o.name != "__block_args__"]
+        wdims = [d for d in range(res.ndim) if d not in iwd and d not in ibd]      # operand dim of each window dim
+        for uidx in np.ndindex(*upd.a.shape):
+            spos = [uidx[d] for d in range(upd.a.ndim) if d not in uwd]
+            widx = [uidx[d] for d in uwd]
+            target = [0] * res.ndim
+            for j, d in enumerate(wdims):
+                target[d] = widx[j]
+            for b, d in enumerate(ibd):
+                ds = sbd[b]
+                target[d] += spos[ds - (0 if ds < ivd else 1)]
+            start_of = dict()
+            for k, d in enumerate(sdo):
+                sel = list(spos)
+                if ivd < st.ndim:
+                    sel.insert(ivd, k)
+                start_of[d] = int(st[tuple(sel)]) if st.ndim else int(st[()])
+                target[d] += start_of[d]
+            ok = all(0 <= target[d] < res.shape[d] for d in range(res.ndim))
+            for j, d in enumerate(wdims):
+                w0 = target[d] - widx[j]
+                ok = ok and w0 >= 0 and w0 + upd.a.shape[uwd[j]] <= res.shape[d]
+            if not ok:
+                continue
+            env = {names[0]: Tensor(res[tuple(target)], operand.dt), names[1]: Tensor(upd.a[uidx], upd.dt)}
+            res[tuple(target)] = _rounded(self._block(body, env)[0]).a
+        return Tensor(res, operand.dt)
+
     def _variadic_reduce(self, op, xs):
         """stablehlo.reduce over several operands with an arbitrary body (argmax / findfirst,
         reference src/Ops.jl:1536-1596): the region is folded over the reduced elements from the
@@ -1624,6 +1677,10 @@ class Interpreter:
             return [r if self.excess else _rounded(r)]
         if n == "gather":
             return [_gather(xs[0], xs[1], at, op.types_out[0])]
+        if n == "scatter":
+            if len(xs) != 3:
+                raise NotImplementedError("scatter over several operands")
+            return [self._scatter(op, xs)]
         if n in ("batch_norm_inference", "batch_norm_training"):
             return _batch_norm(xs, at, n == "batch_norm_training", self.hifi)
         if n == "reverse":

@@ -348,6 +348,51 @@ RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
   return r;
 }
 
+// Read-modify-write on one element in global memory (scatter with a combining update).  Sums of
+// 32/64-bit integers and floats use the hardware atomics; everything else is a compare-and-swap
+// loop on the 32- or 64-bit word (or, for 8/16-bit integers, on the aligned word that holds it).
+template <typename T, typename OP>
+RX_DEV void rx_atomic_rmw(T* p, T v, OP op) {
+  if constexpr (sizeof(T) == 4) {
+    rx_u32* w = (rx_u32*)p;
+    rx_u32 old = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), want;
+    do {
+      want = __builtin_bit_cast(rx_u32, (T)op(__builtin_bit_cast(T, old), v));
+    } while (!__hip_atomic_compare_exchange_weak(w, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  } else if constexpr (sizeof(T) == 8) {
+    rx_u64* w = (rx_u64*)p;
+    rx_u64 old = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), want;
+    do {
+      want = __builtin_bit_cast(rx_u64, (T)op(__builtin_bit_cast(T, old), v));
+    } while (!__hip_atomic_compare_exchange_weak(w, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  } else {
+    const unsigned long long addr = (unsigned long long)p;
+    rx_u32* w = (rx_u32*)(addr & ~3ull);
+    const unsigned shift = (unsigned)(addr & 3ull) * 8u;
+    const rx_u32 mask = (sizeof(T) == 1 ? 0xffu : 0xffffu) << shift;
+    rx_u32 old = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), want;
+    do {
+      T cur;
+      if constexpr (sizeof(T) == 1) cur = __builtin_bit_cast(T, (rx_u8)((old & mask) >> shift));
+      else cur = __builtin_bit_cast(T, (rx_u16)((old & mask) >> shift));
+      const T nv = (T)op(cur, v);
+      rx_u32 bits;
+      if constexpr (sizeof(T) == 1) bits = (rx_u32)__builtin_bit_cast(rx_u8, nv);
+      else bits = (rx_u32)__builtin_bit_cast(rx_u16, nv);
+      want = (old & ~mask) | (bits << shift);
+    } while (!__hip_atomic_compare_exchange_weak(w, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+  }
+}
+template <typename T> RX_DEV void rx_atomic_add(T* p, T v) {
+  if constexpr (sizeof(T) >= 4) (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else rx_atomic_rmw(p, v, rx_op_add());
+}
+template <typename T> RX_DEV void rx_atomic_mul(T* p, T v) { rx_atomic_rmw(p, v, rx_op_mul()); }
+template <typename T> RX_DEV void rx_atomic_max(T* p, T v) { rx_atomic_rmw(p, v, rx_op_max()); }
+template <typename T> RX_DEV void rx_atomic_min(T* p, T v) { rx_atomic_rmw(p, v, rx_op_min()); }
+template <typename T> RX_DEV void rx_atomic_and(T* p, T v) { rx_atomic_rmw(p, v, rx_op_and()); }
+template <typename T> RX_DEV void rx_atomic_or(T* p, T v) { rx_atomic_rmw(p, v, rx_op_or()); }
+
 // Workgroup barrier for data exchanged through LDS only: waits for this wavefront's LDS
 // operations, not for its outstanding global loads (a __syncthreads() drains those too, which
 // would serialize register prefetch with the compute phase that follows the barrier).

@@ -53,7 +53,7 @@ enum class OpK : uint8_t {
   Unary, Binary, Compare, Select, Clamp, Convert, Gelu,
   BroadcastInDim, Reshape, Transpose, Slice, Pad, DynamicUpdateSlice, DynamicSlice, Concatenate,
   Reverse, Window, Gather,
-  Reduce, DotGeneral, Scan,
+  Reduce, DotGeneral, Scan, Scatter,
 };
 
 enum class Red : uint8_t { Add, Mul, Max, Min, And, Or };
@@ -75,6 +75,9 @@ struct Node {
   //       out[k_0..k_{r-1}, o_0..o_{r-1}] = in[o_i * stride_i + k_i * dilation_i]
   //   Gather (operand, start_indices): a0 = offset_dims, a1 = collapsed_slice_dims, a2 = start_index_map,
   //       a3 = slice_sizes, a4[0] = index_vector_dim, a5 = operand_batching_dims, a6 = start_indices_batching_dims
+  //   Scatter (operand, scatter_indices, updates): a0 = update_window_dims, a1 = inserted_window_dims,
+  //       a2 = scatter_dims_to_operand_dims, a4[0] = index_vector_dim, a5 = input_batching_dims,
+  //       a6 = scatter_indices_batching_dims; op = "assign" or "combine" (then `red` is the monoid)
   //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
   std::vector<int64_t> a0, a1, a2, a3, a4, a5, a6;
   Red red = Red::Add;

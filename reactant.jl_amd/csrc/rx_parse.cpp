@@ -525,7 +525,8 @@ struct P {
                             "window_strides", "base_dilations", "window_dilations", "lhs_dilation", "rhs_dilation",
                             "padding", "feature_group_count", "batch_group_count", "feature_index", "offset_dims",
                             "collapsed_slice_dims", "operand_batching_dims", "start_indices_batching_dims", "start_index_map",
-                            "index_vector_dim"})
+                            "index_vector_dim", "update_window_dims", "inserted_window_dims", "input_batching_dims",
+                            "scatter_indices_batching_dims", "scatter_dims_to_operand_dims"})
       scan_int_array(in, key, o);
     {
       size_t q = in.find("#stablehlo.conv<");
@@ -2111,6 +2112,64 @@ struct Builder {
       check_same(n.ty, ty(in[0]), o.name);
       n.a0 = o.ia.at("dimensions");
       for (auto d : n.a0) if (d < 0 || d >= n.ty.rank()) fail("reverse: dimension out of range");
+      return {g.add(n)};
+    }
+    if (sh == "scatter") {
+      // one operand / one update tensor; the update computation is an assignment (returns its second
+      // argument) or a single monoid op of both arguments (reference src/Ops.jl:2150-2268)
+      if (in.size() != 3) fail("scatter over several operands is not supported");
+      n.k = OpK::Scatter;
+      n.ty = out1();
+      const TType &ot = ty(in[0]), &st = ty(in[1]), &ut = ty(in[2]);
+      if (!(n.ty == ot) || ut.dt != ot.dt) fail("scatter: operand, updates and result types must agree");
+      if (!is_int_dt(st.dt) || st.dt == DT::I1) fail("scatter: indices must be integers");
+      auto get = [&](const char* key) { return o.ia.count(key) ? o.ia.at(key) : std::vector<int64_t>{}; };
+      n.a0 = get("update_window_dims");
+      n.a1 = get("inserted_window_dims");
+      n.a2 = get("scatter_dims_to_operand_dims");
+      n.a4 = get("index_vector_dim");
+      n.a5 = get("input_batching_dims");
+      n.a6 = get("scatter_indices_batching_dims");
+      if (n.a4.size() != 1) fail("scatter: index_vector_dim missing");
+      const int r = ot.rank(), rs = st.rank(), ru = ut.rank(), ivd = (int)n.a4[0];
+      if (ivd < 0 || ivd > rs) fail("scatter: index_vector_dim out of range");
+      if ((int64_t)n.a2.size() != (ivd < rs ? st.dims[ivd] : 1)) fail("scatter: scatter_dims_to_operand_dims does not match the index vector length");
+      if (n.a5.size() != n.a6.size()) fail("scatter: batching dimension lists differ in length");
+      auto in_range = [&](const std::vector<int64_t>& v, int hi) { for (auto x : v) if (x < 0 || x >= hi) return false; return true; };
+      if (!in_range(n.a0, ru) || !in_range(n.a1, r) || !in_range(n.a2, r) || !in_range(n.a5, r) || !in_range(n.a6, rs)) fail("scatter: dimension number out of range");
+      if ((int)(n.a0.size() + n.a1.size() + n.a5.size()) != r) fail("scatter: window dims do not cover the operand");
+      // updates shape: scatter dims follow the index tensor (without the index vector), window dims fit the operand
+      {
+        std::vector<int64_t> sdims;
+        for (int q = 0; q < rs; ++q) if (q != ivd) sdims.push_back(st.dims[q]);
+        if ((int)(sdims.size() + n.a0.size()) != ru) fail("scatter: updates rank mismatch");
+        size_t si = 0, wi = 0;
+        std::vector<int> wdim;   // operand dim of each window dim
+        for (int d = 0; d < r; ++d)
+          if (std::find(n.a1.begin(), n.a1.end(), (int64_t)d) == n.a1.end() && std::find(n.a5.begin(), n.a5.end(), (int64_t)d) == n.a5.end()) wdim.push_back(d);
+        for (int d = 0; d < ru; ++d) {
+          const bool is_win = std::find(n.a0.begin(), n.a0.end(), (int64_t)d) != n.a0.end();
+          if (is_win) { if (ut.dims[d] > ot.dims[wdim[wi++]]) fail("scatter: update window exceeds the operand"); }
+          else if (ut.dims[d] != sdims[si++]) fail("scatter: updates shape does not match the indices");
+        }
+      }
+      // update computation
+      if (o.regions.empty() || o.regions[0].empty() || o.regions[0][0].name != "__block_args__" || o.regions[0][0].block_args.size() != 2)
+        fail("scatter: update computation with two arguments expected");
+      const auto& region = o.regions[0];
+      const std::string a_cur = region[0].block_args[0].first, a_upd = region[0].block_args[1].first;
+      std::vector<const RawOp*> body;
+      for (size_t k = 1; k < region.size(); ++k) body.push_back(&region[k]);
+      if (body.size() == 1 && body[0]->operands.size() == 1 && body[0]->operands[0] == a_upd) n.op = "assign";
+      else if (body.size() == 2 && body[0]->operands.size() == 2 && body[1]->operands.size() == 1 && body[0]->results.size() == 1 &&
+               body[1]->operands[0] == body[0]->results[0] &&
+               ((body[0]->operands[0] == a_cur && body[0]->operands[1] == a_upd) || (body[0]->operands[0] == a_upd && body[0]->operands[1] == a_cur))) {
+        RawOp tmp;
+        tmp.sa["body"] = body[0]->name.substr(body[0]->name.rfind('.') + 1);
+        n.red = body_kind(tmp);
+        n.op = "combine";
+      } else fail("scatter: the update computation must return its second argument or one monoid op of both");
+      if (n.op == "combine" && is_narrow_float(ot.dt)) fail("scatter: combining updates of 8- or 16-bit floats is not supported");
       return {g.add(n)};
     }
     if (sh == "gather") {

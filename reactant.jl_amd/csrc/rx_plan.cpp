@@ -301,7 +301,7 @@ struct Planner {
     for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
     for (int r : g.results) nuse[r]++;
     auto is_leaf = [](const Node& n) {
-      return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral;
+      return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral;
     };
     for (const Node& d : g.nodes) {
       if (d.k != OpK::DotGeneral || d.ty.rank() < 2) continue;
@@ -588,7 +588,7 @@ struct Planner {
       st.pop_back();
       if (!seen.insert(x).second) continue;
       const Node& n = g.nodes[x];
-      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral) continue;
+      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) continue;
       if (n.k == OpK::Constant) continue;
       if (x != id && prev_mat[x]) continue;
       if (is_arith(n.k)) cost += (n.k == OpK::Unary || n.k == OpK::Gelu) ? 2 : 1;
@@ -606,7 +606,7 @@ struct Planner {
       if (!seen.insert(x).second || seen.size() > 64) continue;
       const Node& n = g.nodes[x];
       if (n.k == OpK::DotGeneral) return true;
-      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan) continue;
+      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter) continue;
       if (x != id && prev_mat[x]) continue;
       for (int i : n.in) st.push_back(i);
     }
@@ -638,7 +638,7 @@ struct Planner {
       const Node& n = g.nodes[x];
       // contexts in which x is evaluated
       std::set<Ctx> U;
-      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral ||
+      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral ||
                     (n.k == OpK::Constant && !n.splat);
       for (int u : users[x]) {
         const Node& un = g.nodes[u];
@@ -684,7 +684,7 @@ struct Planner {
             if (!(cn.k == OpK::Convert || cn.k == OpK::Unary)) break;
             int p = cn.in[0];
             const Node& pn = g.nodes[p];
-            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce || pn.k == OpK::Scan) break;
+            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce || pn.k == OpK::Scan || pn.k == OpK::Scatter) break;
             if (users[p].size() != 1 || is_result[p]) break;
             cur = p;
             if (info(pn.ty.dt).size < info(g.nodes[best].ty.dt).size) best = cur;
@@ -804,6 +804,7 @@ struct Planner {
         case OpK::Window: nm = "window"; break;
         case OpK::Gather: nm = "gather"; break;
         case OpK::Scan: nm = "scan"; break;
+        case OpK::Scatter: nm = "scatter"; break;
         case OpK::Reduce: nm = "reduce"; break;
         case OpK::DotGeneral: nm = "dot_general"; break;
         case OpK::Iota: nm = "iota"; break;
@@ -935,7 +936,7 @@ struct Planner {
   bool probe_stencil(int root, StencilProbe* sp) {
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
-    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::Scan || rn.k == OpK::DotGeneral) return false;
+    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::Scan || rn.k == OpK::Scatter || rn.k == OpK::DotGeneral) return false;
     sp->vec = pick_vec(rn.ty);
     if (rn.ty.numel() < opt.slab_min_numel || sp->vec < 2) return false;
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
@@ -1734,10 +1735,14 @@ struct Planner {
   }
 
   // ------------------------------------------------------------------ map kernels
-  void emit_map(int root) {
-    if (lds_only.count(root)) return;   // evaluated inside its only reader's kernel
-    if (emit_map_lds(root)) return;
-    if (emit_map_transposed(root)) return;
+  // `value` >= 0: write that node's values (same type as `root`) into root's buffer instead of
+  // evaluating root itself (the copy of the operand a scatter starts from).
+  void emit_map(int root, int value = -1) {
+    if (value < 0) {
+      if (lds_only.count(root)) return;   // evaluated inside its only reader's kernel
+      if (emit_map_lds(root)) return;
+      if (emit_map_transposed(root)) return;
+    }
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
     const int n = rn.ty.rank();
@@ -1748,7 +1753,7 @@ struct Planner {
     const std::string kname = "@K@_map";
     Emitter em(g, [&](int x) { return x != root && mat[x]; });
     em.excess_precision = opt.excess_precision;
-    em.idx64 = needs64(cone_nodes(root));
+    em.idx64 = needs64(cone_nodes(value >= 0 ? value : root)) || numel >= ((int64_t)1 << 31);
     const std::string it = em.idx_t();
     std::vector<std::string> vars;
     for (int d = 0; d < n; ++d) vars.push_back("i" + std::to_string(d));
@@ -1759,7 +1764,7 @@ struct Planner {
     em.indent = 4;
     Index ix = root_index(dims);
     // evaluate the root op itself (it is materialized, so bypass the input test by emitting its op)
-    std::string val = em.emit(root, ix);
+    std::string val = em.emit(value >= 0 ? value : root, ix);
     std::string body = em.take_code();
 
     // shifted loads along the slowest dimension -> XCD slab order
@@ -1773,7 +1778,7 @@ struct Planner {
 
     std::ostringstream o;
     std::vector<std::pair<std::string, std::string>> outs{{info(rn.ty.dt).stype, "out0"}};
-    o << "// map: " << describe(root) << " -> " << rn.ty.str() << "\n";
+    o << "// map: " << (value >= 0 ? "copy of " + describe(value) : describe(root)) << " -> " << rn.ty.str() << "\n";
     o << signature(kname, em.inputs, outs) << " {\n";
     unsigned grid;
     if (!slab) {
@@ -1856,7 +1861,124 @@ struct Planner {
     for (int i : em.inputs) L.args.push_back(buffer_for(i));
     L.args.push_back(buffer_for(root));
     L.algo_bytes = algo_bytes(em.inputs, {root});
-    L.desc = describe(root);
+    L.desc = value >= 0 ? "copy of the scatter operand" : describe(root);
+    plan.launches.push_back(L);
+  }
+
+  // ------------------------------------------------------------------ scatter
+  // The result starts as a copy of the operand (a map kernel); then one thread per element of
+  // `updates` finds its target -- the start index read from the index tensor at its scatter
+  // position, plus its offset inside the update window -- skips it if the window leaves the
+  // operand (the specification drops such updates, it does not clamp them), and stores or
+  // combines.  Combining uses the hardware atomics (the order of colliding float additions is
+  // not fixed); colliding assignments leave one of the values, as the specification allows.
+  void emit_scatter(int root) {
+    const Node& rn = g.nodes[root];
+    const TType& ot = rn.ty;
+    const TType& st = g.nodes[rn.in[1]].ty;
+    const TType& ut = g.nodes[rn.in[2]].ty;
+    emit_map(root, rn.in[0]);
+    if (ut.numel() == 0 || ot.numel() == 0) return;
+    const int r = ot.rank(), rs = st.rank(), ru = ut.rank();
+    const int ivd = (int)rn.a4[0];
+    auto has = [](const std::vector<int64_t>& v, int x) { return std::find(v.begin(), v.end(), (int64_t)x) != v.end(); };
+    Emitter em(g, [&](int x) { return mat[x] != 0; });
+    em.excess_precision = opt.excess_precision;
+    em.idx64 = needs64(cone_nodes(rn.in[1])) || needs64(cone_nodes(rn.in[2])) || ot.numel() >= ((int64_t)1 << 31) || ut.numel() >= ((int64_t)1 << 31);
+    const std::string it = em.idx_t();
+    em.set_root({}, {}, false);
+    em.indent = 2;
+    Index ux(ru);
+    for (int d = 0; d < ru; ++d) { ux[d].var = "u" + std::to_string(d); ux[d].hi = ut.dims[d] - 1; }
+    // scatter position = update index without the window dims
+    std::vector<Ix> spos;
+    for (int d = 0; d < ru; ++d) if (!has(rn.a0, d)) spos.push_back(ux[d]);
+    // window offset per operand dim
+    std::vector<std::string> off(r, "0");
+    {
+      size_t j = 0;
+      for (int d = 0; d < r; ++d) {
+        if (has(rn.a1, d) || has(rn.a5, d)) continue;
+        off[d] = ux[rn.a0[j++]].str();
+      }
+    }
+    for (size_t b = 0; b < rn.a5.size(); ++b) {
+      const int ds = (int)rn.a6[b];
+      off[rn.a5[b]] = spos[ds - (ds < ivd ? 0 : 1)].str();
+    }
+    std::ostringstream body;
+    std::vector<std::string> target(r);
+    std::string guard;
+    std::vector<std::string> start_code;
+    for (int d = 0; d < r; ++d) target[d] = "(long long)(" + off[d] + ")";
+    for (size_t k = 0; k < rn.a2.size(); ++k) {
+      const int d = (int)rn.a2[k];
+      Index si(rs);
+      size_t bi = 0;
+      for (int q = 0; q < rs; ++q) {
+        if (q == ivd) { si[q].off = (int64_t)k; si[q].lo = si[q].hi = (int64_t)k; }
+        else si[q] = spos[bi++];
+      }
+      const std::string e = em.emit(rn.in[1], si);
+      target[d] = "((long long)(" + e + ") + (long long)(" + off[d] + "))";
+    }
+    const std::string val = em.emit(rn.in[2], ux);
+    const std::string code = em.take_code();
+    std::ostringstream o;
+    const std::string ost = info(ot.dt).stype;
+    o << "// scatter (" << (rn.op == "assign" ? std::string("assign") : std::string("combine")) << "): " << describe(rn.in[2]) << " -> " << ot.str() << "\n";
+    o << signature("@K@_scatter", em.inputs, {{ost, "out0"}}) << " {\n";
+    o << "  const " << it << " uid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
+    o << "  if (uid >= " << ut.numel() << ") return;\n";
+    o << "  " << it << " rr = uid;\n";
+    for (int d = ru - 1; d >= 0; --d) {
+      o << "  const " << it << " u" << d << " = rr % " << ut.dims[d] << ";\n";
+      o << "  rr /= " << ut.dims[d] << ";\n";
+    }
+    o << "  (void)rr;\n" << code;
+    std::string lin = "0";
+    int64_t stride = 1;
+    for (int d = r - 1; d >= 0; --d) {
+      o << "  const long long t" << d << "_ = " << target[d] << ";\n";
+      guard += (guard.empty() ? "" : " && ") + std::string("t") + std::to_string(d) + "_ >= 0 && t" + std::to_string(d) + "_ < " + std::to_string(ot.dims[d]) + "LL";
+      lin += " + t" + std::to_string(d) + "_ * " + std::to_string(stride) + "LL";
+      stride *= ot.dims[d];
+    }
+    // The whole update window must lie inside the operand, not just this element: test the window's corners.
+    {
+      std::string wguard;
+      size_t j = 0;
+      for (int d = 0; d < r; ++d) {
+        if (has(rn.a1, d) || has(rn.a5, d)) continue;
+        const int ud = (int)rn.a0[j++];
+        // start of the window in dim d = target - own offset; the window spans ut.dims[ud] elements
+        wguard += (wguard.empty() ? "" : " && ") + std::string("(t") + std::to_string(d) + "_ - (long long)u" + std::to_string(ud) + ") >= 0 && (t" +
+                  std::to_string(d) + "_ - (long long)u" + std::to_string(ud) + ") + " + std::to_string(ut.dims[ud]) + "LL <= " + std::to_string(ot.dims[d]) + "LL";
+      }
+      if (!wguard.empty()) guard += " && " + wguard;
+    }
+    if (guard.empty()) guard = "true";
+    o << "  if (" << guard << ") {\n";
+    o << "    " << ost << "* p = out0 + (" << lin << ");\n";
+    const std::string sv = em.store_value(ot.dt, val);
+    if (rn.op == "assign") {
+      o << "    *p = " << sv << ";\n";
+    } else {
+      const char* fn = rn.red == Red::Add ? "rx_atomic_add" : rn.red == Red::Mul ? "rx_atomic_mul" : rn.red == Red::Max ? "rx_atomic_max"
+                       : rn.red == Red::Min ? "rx_atomic_min" : rn.red == Red::And ? "rx_atomic_and" : "rx_atomic_or";
+      o << "    " << fn << "(p, " << sv << ");\n";
+    }
+    o << "  }\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named("@K@_scatter", kb_final);
+    L.kind = "scatter";
+    L.grid[0] = (unsigned)((ut.numel() + kBlock - 1) / kBlock);
+    L.block[0] = kBlock;
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    L.algo_bytes = algo_bytes(em.inputs, {});
+    L.desc = describe(rn.in[2]) + " scatter";
     plan.launches.push_back(L);
   }
 
@@ -2911,7 +3033,7 @@ struct Planner {
       const Ctx& c = *ctx[x].begin();
       if (!c.second.empty()) continue;
       const Node& r = g.nodes[c.first];
-      if (r.k == OpK::Reduce || r.k == OpK::Scan || r.k == OpK::DotGeneral) continue;
+      if (r.k == OpK::Reduce || r.k == OpK::Scan || r.k == OpK::Scatter || r.k == OpK::DotGeneral) continue;
       if (r.ty.dims != g.nodes[x].ty.dims) continue;
       // the root must not be the anchor of a row group (its reductions need the full row)
       if (!row_phases(c.first).empty()) continue;
@@ -2966,6 +3088,10 @@ struct Planner {
         jobs.push_back({x, [this, x] { emit_scan(x); }});
         continue;
       }
+      if (n.k == OpK::Scatter) {
+        jobs.push_back({x, [this, x] { emit_scatter(x); }});
+        continue;
+      }
       if (reshape_alias.count(x)) continue;
       if (n.k == OpK::Reduce) {
         jobs.push_back({x, [this, x, &fused_reduces] {
@@ -2994,7 +3120,7 @@ struct Planner {
       auto plain_map_root = [&](int x) {
         const Node& n = g.nodes[x];
         if (!live[x] || !mat[x]) return false;
-        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::DotGeneral) return false;
+        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) return false;
         if (reshape_alias.count(x)) return false;
         if (absorbed_roots.count(x) || !row_phases(x).empty()) return false;
         return true;
@@ -3017,7 +3143,7 @@ struct Planner {
     // row groups claim their reductions before those would be emitted on their own
     for (auto& j : jobs) {
       const Node& n = g.nodes[j.first];
-      if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
+      if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::Scatter && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
         for (int p : row_phases(j.first)) fused_reduces.insert(p);
     }
     for (auto& j : jobs) j.second();

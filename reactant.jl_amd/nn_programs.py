@@ -278,3 +278,24 @@ def gather(operand_shape, start_shape, out_shape, dt, offset_dims, collapsed_sli
             "    %%0 = \"stablehlo.gather\"(%%arg0, %s) <{dimension_numbers = #stablehlo.gather<%s>, indices_are_sorted = false, "
             "slice_sizes = array<i64: %s>}> : (%s, %s) -> %s\n    return %%0 : %s\n  }\n}\n"
             % (to, ts, tr, pre, idx, dn, ", ".join(str(x) for x in slice_sizes), to, ts, tr, tr))
+
+
+def scatter(operand_shape, index_shape, update_shape, dt, update_window_dims, inserted_window_dims, scatter_dims_to_operand_dims,
+            index_vector_dim, body="assign", input_batching_dims=(), scatter_indices_batching_dims=(), idt="i64"):
+    """`stablehlo.scatter` in the generic form it prints in (reference src/Ops.jl:2150-2268).  `body` is
+    "assign" (the update replaces the element, what `setindex!` with index arrays prints) or the name of
+    a binary op combining the element with the update ("add", "maximum", ...)."""
+    to, ti, tu, ts = tt(operand_shape, dt), tt(index_shape, idt), tt(update_shape, dt), tt([], dt)
+    lst = lambda v: "[" + ", ".join(str(x) for x in v) + "]"
+    dn = "update_window_dims = %s, inserted_window_dims = %s, " % (lst(update_window_dims), lst(inserted_window_dims))
+    if input_batching_dims:
+        dn += "input_batching_dims = %s, scatter_indices_batching_dims = %s, " % (lst(input_batching_dims), lst(scatter_indices_batching_dims))
+    dn += "scatter_dims_to_operand_dims = %s, index_vector_dim = %d" % (lst(scatter_dims_to_operand_dims), index_vector_dim)
+    if body == "assign":
+        region = "      stablehlo.return %%u : %s\n" % ts
+    else:
+        region = "      %%r = stablehlo.%s %%c, %%u : %s\n      stablehlo.return %%r : %s\n" % (body, ts, ts)
+    return ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg2: %s) -> %s {\n"
+            "    %%0 = \"stablehlo.scatter\"(%%arg0, %%arg1, %%arg2) <{indices_are_sorted = false, scatter_dimension_numbers = "
+            "#stablehlo.scatter<%s>, unique_indices = false}> ({\n    ^bb0(%%c: %s, %%u: %s):\n%s    }) : (%s, %s, %s) -> %s\n"
+            "    return %%0 : %s\n  }\n}\n" % (to, ti, tu, to, dn, ts, ts, region, to, ti, tu, to, to))

@@ -376,3 +376,41 @@ def test_grouped_filter_gradient(rx, client):
         x, dy = I.tensor(rng.normal(size=xs), "f32"), I.tensor(rng.normal(size=ys), "f32")
         got, _ = gpu_run(rx, client, tf, [x, dy])
         _close(got[0].a, oracle_run(tf, [x, dy], hifi=True)[0].a, 1e-5 * np.sqrt(ys[0] * ys[1] * ys[3]))
+
+
+SCATTERS = [
+    # operand, indices, updates, dtype, update_window_dims, inserted_window_dims, scatter_dims_to_operand_dims, index_vector_dim, body, batching
+    ([600, 700], [5000, 2], [5000], "f32", [], [0, 1], [0, 1], 1, "assign", None),        # setindex! with index pairs
+    ([600, 700], [5000, 2], [5000], "f32", [], [0, 1], [0, 1], 1, "add", None),
+    ([1000, 64], [4096], [4096, 64], "f32", [1], [0], [0], 1, "add", None),                # gradient of an embedding lookup
+    ([1000, 64], [4096], [4096, 64], "f64", [1], [0], [0], 1, "add", None),
+    ([50, 40], [300, 1], [300, 40], "i32", [1], [0], [0], 1, "maximum", None),
+    ([200], [77, 1], [77, 5], "f32", [1], [], [0], 1, "add", None),                         # windows, some sticking out
+    ([8, 300], [8, 60], [8, 60], "i64", [], [1], [1], 2, "add", ([0], [0])),              # a batching dim
+    ([300], [1000, 1], [1000], "i8", [], [0], [0], 1, "add", None),
+    ([300], [1000, 1], [1000], "f32", [], [0], [0], 1, "minimum", None),
+]
+
+
+@pytest.mark.parametrize("os_,is_,us,dt,uwd,iwd,sdo,ivd,body,bat", SCATTERS)
+def test_scatter(rx, client, os_, is_, us, dt, uwd, iwd, sdo, ivd, body, bat):
+    kw = {} if bat is None else dict(input_batching_dims=bat[0], scatter_indices_batching_dims=bat[1])
+    text = NN.scatter(os_, is_, us, dt, uwd, iwd, sdo, ivd, body=body, **kw)
+    rng = np.random.default_rng(47)
+    dest = _args([os_], dt, seed=47)[0] if dt[0] == "f" else I.Tensor(rng.integers(-50, 50, size=os_).astype(I.NP_OF[dt]), dt)
+    upd = _args([us], dt, seed=48)[0] if dt[0] == "f" else I.Tensor(rng.integers(-3, 4, size=us).astype(I.NP_OF[dt]), dt)
+    hi = max(os_)
+    idx = rng.integers(-2, hi + 2, size=is_)
+    if body == "assign":
+        # colliding assignments may leave either value: use distinct in-range targets (plus some out of range)
+        flat = rng.permutation(os_[0] * os_[1])[: is_[0]]
+        idx = np.stack([flat // os_[1], flat % os_[1]], axis=1)
+        idx[::50] = [os_[0] + 3, 0]
+    idx = I.Tensor(idx.astype(np.int64), "i64")
+    got, exe = gpu_run(rx, client, text, [dest, idx, upd])
+    assert [l["kind"] for l in exe.launches()] == ["map", "scatter"]
+    ref = oracle_run(text, [dest, idx, upd])
+    if dt[0] == "f" and body == "add":
+        _close(got[0].a, ref[0].a, 1e-5 if dt == "f32" else 1e-13)
+    else:
+        assert np.array_equal(got[0].a, ref[0].a)

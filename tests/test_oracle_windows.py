@@ -347,3 +347,32 @@ def test_grouped_filter_gradient_against_the_definition():
             dw[:, :, :, g * opg:(g + 1) * opg] = dwg
         got = I.run_text(tf, [I.tensor(x, "f64"), I.tensor(dy, "f64")])[0].a
         assert np.allclose(got, dw, rtol=1e-12, atol=1e-12), (groups, c)
+
+
+def test_scatter_against_numpy():
+    """setindex! with index arrays (src/Ops.jl:2150-2172) and scatter-add, against numpy's indexed
+    assignment / np.add.at; out-of-range updates are dropped."""
+    rng = np.random.default_rng(14)
+    dest = rng.normal(size=(6, 7))
+    idx = np.array([[0, 0], [5, 6], [2, 3], [9, 1], [3, -1], [4, 4]])          # two of them out of range
+    upd = rng.normal(size=6)
+    t = NN.scatter([6, 7], [6, 2], [6], "f64", [], [0, 1], [0, 1], 1)
+    got = I.run_text(t, [I.tensor(dest, "f64"), I.Tensor(idx, "i64"), I.tensor(upd, "f64")])[0].a
+    want = dest.copy()
+    for k in (0, 1, 2, 5):
+        want[idx[k, 0], idx[k, 1]] = upd[k]
+    assert np.array_equal(got, want)
+    # rows added into a table, with repeated rows (what the gradient of an embedding lookup is)
+    table = rng.normal(size=(10, 4))
+    ids = np.array([3, 3, 0, 9, 3, 11])
+    rows = rng.normal(size=(6, 4))
+    t = NN.scatter([10, 4], [6], [6, 4], "f64", [1], [0], [0], 1, body="add")
+    got = I.run_text(t, [I.tensor(table, "f64"), I.Tensor(ids, "i64"), I.tensor(rows, "f64")])[0].a
+    want = table.copy()
+    np.add.at(want, ids[:5], rows[:5])
+    assert np.allclose(got, want, rtol=1e-14)
+    # a window that sticks out of the operand is dropped as a whole
+    base = np.zeros((8,))
+    t = NN.scatter([8], [3, 1], [3, 3], "f64", [1], [], [0], 1, body="add")
+    got = I.run_text(t, [I.tensor(base, "f64"), I.Tensor(np.array([[0], [6], [4]]), "i64"), I.tensor(np.ones((3, 3)), "f64")])[0].a
+    assert got.tolist() == [1, 1, 1, 0, 1, 1, 1, 0]
