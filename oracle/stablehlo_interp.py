@@ -44,7 +44,8 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       numpy accumulate (tests/test_oracle_windows.py)
   gather (src/Ops.jl:2269-2345; NNlib.gather, ext/ReactantNNlibExt/Implementations.jl:426-438)
       ... reference KATs (test/nn/scatter_gather.jl:5-99), numpy fancy indexing with clamping
-  scatter (src/Ops.jl:2150-2268) ... numpy indexed assignment and np.add.at, dropped
+  scatter (src/Ops.jl:2150-2268) ... reference KATs (NNlib.scatter, test/nn/scatter_gather.jl:254-428,
+      seven operations, four shapes), numpy indexed assignment and np.add.at; dropped
       out-of-range updates (whole windows, as XLA does; the StableHLO text says per element:
       PARITY UNPINNED between the two readings, the reference holds no case that tells them apart)
   reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy

@@ -255,6 +255,7 @@ RX_DEV T rx_readlane63(T v) {
 
 struct rx_op_add { template <typename T> RX_MEM T operator()(T a, T b) const { return a + b; } };
 struct rx_op_mul { template <typename T> RX_MEM T operator()(T a, T b) const { return a * b; } };
+struct rx_op_div { template <typename T> RX_MEM T operator()(T a, T b) const { return a / b; } };
 struct rx_op_max { template <typename T> RX_MEM T operator()(T a, T b) const { return rx_max(a, b); } };
 struct rx_op_min { template <typename T> RX_MEM T operator()(T a, T b) const { return rx_min(a, b); } };
 struct rx_op_and { template <typename T> RX_MEM T operator()(T a, T b) const { return (T)(a & b); } };
@@ -388,6 +389,7 @@ template <typename T> RX_DEV void rx_atomic_add(T* p, T v) {
   else rx_atomic_rmw(p, v, rx_op_add());
 }
 template <typename T> RX_DEV void rx_atomic_mul(T* p, T v) { rx_atomic_rmw(p, v, rx_op_mul()); }
+template <typename T> RX_DEV void rx_atomic_div(T* p, T v) { rx_atomic_rmw(p, v, rx_op_div()); }
 template <typename T> RX_DEV void rx_atomic_max(T* p, T v) { rx_atomic_rmw(p, v, rx_op_max()); }
 template <typename T> RX_DEV void rx_atomic_min(T* p, T v) { rx_atomic_rmw(p, v, rx_op_min()); }
 template <typename T> RX_DEV void rx_atomic_and(T* p, T v) { rx_atomic_rmw(p, v, rx_op_and()); }

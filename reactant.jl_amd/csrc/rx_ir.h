@@ -77,7 +77,7 @@ struct Node {
   //       a3 = slice_sizes, a4[0] = index_vector_dim, a5 = operand_batching_dims, a6 = start_indices_batching_dims
   //   Scatter (operand, scatter_indices, updates): a0 = update_window_dims, a1 = inserted_window_dims,
   //       a2 = scatter_dims_to_operand_dims, a4[0] = index_vector_dim, a5 = input_batching_dims,
-  //       a6 = scatter_indices_batching_dims; op = "assign" or "combine" (then `red` is the monoid)
+  //       a6 = scatter_indices_batching_dims; op = "assign", "subtract", "divide" or "combine" (then `red` is the monoid)
   //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
   std::vector<int64_t> a0, a1, a2, a3, a4, a5, a6;
   Red red = Red::Add;

@@ -2164,12 +2164,21 @@ struct Builder {
       else if (body.size() == 2 && body[0]->operands.size() == 2 && body[1]->operands.size() == 1 && body[0]->results.size() == 1 &&
                body[1]->operands[0] == body[0]->results[0] &&
                ((body[0]->operands[0] == a_cur && body[0]->operands[1] == a_upd) || (body[0]->operands[0] == a_upd && body[0]->operands[1] == a_cur))) {
-        RawOp tmp;
-        tmp.sa["body"] = body[0]->name.substr(body[0]->name.rfind('.') + 1);
-        n.red = body_kind(tmp);
-        n.op = "combine";
-      } else fail("scatter: the update computation must return its second argument or one monoid op of both");
-      if (n.op == "combine" && is_narrow_float(ot.dt)) fail("scatter: combining updates of 8- or 16-bit floats is not supported");
+        const std::string bname = body[0]->name.substr(body[0]->name.rfind('.') + 1);
+        const bool in_order = body[0]->operands[0] == a_cur;
+        // element - update and element / update (NNlib.scatter!(-, ...) and (/, ...), reference
+        // ext/ReactantNNlibExt/Implementations.jl:477-530): the order of the updates of one element
+        // does not matter to the exact result, as for the monoids
+        if (bname == "subtract" && in_order && ot.dt != DT::I1) n.op = "subtract";
+        else if (bname == "divide" && in_order && is_float(ot.dt)) n.op = "divide";
+        else {
+          RawOp tmp;
+          tmp.sa["body"] = bname;
+          n.red = body_kind(tmp);
+          n.op = "combine";
+        }
+      } else fail("scatter: the update computation must return its second argument or one op of both (a monoid, element - update, element / update)");
+      if (n.op != "assign" && is_narrow_float(ot.dt)) fail("scatter: combining updates of 8- or 16-bit floats is not supported");
       return {g.add(n)};
     }
     if (sh == "gather") {

@@ -1926,7 +1926,7 @@ struct Planner {
     const std::string code = em.take_code();
     std::ostringstream o;
     const std::string ost = info(ot.dt).stype;
-    o << "// scatter (" << (rn.op == "assign" ? std::string("assign") : std::string("combine")) << "): " << describe(rn.in[2]) << " -> " << ot.str() << "\n";
+    o << "// scatter (" << rn.op << "): " << describe(rn.in[2]) << " -> " << ot.str() << "\n";
     o << signature("@K@_scatter", em.inputs, {{ost, "out0"}}) << " {\n";
     o << "  const " << it << " uid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
     o << "  if (uid >= " << ut.numel() << ") return;\n";
@@ -1963,6 +1963,10 @@ struct Planner {
     const std::string sv = em.store_value(ot.dt, val);
     if (rn.op == "assign") {
       o << "    *p = " << sv << ";\n";
+    } else if (rn.op == "subtract") {
+      o << "    rx_atomic_add(p, (" << ost << ")(-(" << sv << ")));\n";
+    } else if (rn.op == "divide") {
+      o << "    rx_atomic_div(p, " << sv << ");\n";
     } else {
       const char* fn = rn.red == Red::Add ? "rx_atomic_add" : rn.red == Red::Mul ? "rx_atomic_mul" : rn.red == Red::Max ? "rx_atomic_max"
                        : rn.red == Red::Min ? "rx_atomic_min" : rn.red == Red::And ? "rx_atomic_and" : "rx_atomic_or";

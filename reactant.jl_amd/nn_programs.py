@@ -299,3 +299,37 @@ def scatter(operand_shape, index_shape, update_shape, dt, update_window_dims, in
             "    %%0 = \"stablehlo.scatter\"(%%arg0, %%arg1, %%arg2) <{indices_are_sorted = false, scatter_dimension_numbers = "
             "#stablehlo.scatter<%s>, unique_indices = false}> ({\n    ^bb0(%%c: %s, %%u: %s):\n%s    }) : (%s, %s, %s) -> %s\n"
             "    return %%0 : %s\n  }\n}\n" % (to, ti, tu, to, dn, ts, ts, region, to, ti, tu, to, to))
+
+
+def nnlib_scatter(op, dst_shape, src_shape, idx_shape, dt="f32"):
+    """The module `NNlib.scatter!(op, dst, src, idx)` traces to for an integer index array
+    (reference ext/ReactantNNlibExt/Implementations.jl:477-530 over src/Ops.jl:2204-2268): the index
+    array gets a leading unit dim that holds the index vector, one is subtracted from it inside the
+    module, the leading `ndims(src) - ndims(idx)` dims of `src` are the update window and the
+    trailing dims of `dst` are indexed.  Arguments: dst, idx (i64, one-based), src.  `op` is "add",
+    "subtract", "maximum", "minimum", "multiply", "divide" or "mean" (two additive scatters into
+    zeros, then dst + sum / count where the count is not zero)."""
+    nd, nw = len(dst_shape), len(src_shape) - len(idx_shape)
+    ishape = [1] + list(idx_shape)
+    to, ti, tu, ts = tt(dst_shape, dt), tt(ishape, "i64"), tt(src_shape, dt), tt([], dt)
+    lst = lambda v: "[" + ", ".join(str(x) for x in v) + "]"
+    dn = ("update_window_dims = %s, inserted_window_dims = %s, scatter_dims_to_operand_dims = %s, index_vector_dim = 0"
+          % (lst(range(nw)), lst(range(nw, nd)), lst(range(nd - 1, nd))))
+
+    def one(res, dst, upd, body):
+        return ("    %s = \"stablehlo.scatter\"(%s, %%idx0, %s) <{indices_are_sorted = false, scatter_dimension_numbers = "
+                "#stablehlo.scatter<%s>, unique_indices = false}> ({\n    ^bb0(%%c: %s, %%u: %s):\n"
+                "      %%r = stablehlo.%s %%c, %%u : %s\n      stablehlo.return %%r : %s\n    }) : (%s, %s, %s) -> %s\n"
+                % (res, dst, upd, dn, ts, ts, body, ts, ts, to, ti, tu, to))
+
+    head = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg2: %s) -> %s {\n"
+            "    %%one = stablehlo.constant dense<1> : %s\n    %%idx0 = stablehlo.subtract %%arg1, %%one : %s\n" % (to, ti, tu, to, ti, ti))
+    if op != "mean":
+        return head + one("%0", "%arg0", "%arg2", op) + "    return %%0 : %s\n  }\n}\n" % to
+    tb = tt(dst_shape, "i1")
+    return (head + "    %%z = stablehlo.constant dense<0.0> : %s\n    %%ones = stablehlo.constant dense<1.0> : %s\n" % (to, tu)
+            + one("%ns", "%z", "%ones", "add") + one("%sum", "%z", "%arg2", "add")
+            + "    %%isz = stablehlo.compare EQ, %%ns, %%z : (%s, %s) -> %s\n" % (to, to, tb)
+            + "    %%q = stablehlo.divide %%sum, %%ns : %s\n" % to
+            + "    %%sd = stablehlo.select %%isz, %%sum, %%q : %s, %s\n" % (tb, to)
+            + "    %%0 = stablehlo.add %%arg0, %%sd : %s\n    return %%0 : %s\n  }\n}\n" % (to, to))

@@ -414,3 +414,32 @@ def test_scatter(rx, client, os_, is_, us, dt, uwd, iwd, sdo, ivd, body, bat):
         _close(got[0].a, ref[0].a, 1e-5 if dt == "f32" else 1e-13)
     else:
         assert np.array_equal(got[0].a, ref[0].a)
+
+
+def _nnlib_scatter_cases():
+    import _nnlib_scatter_cases as C
+    return [pytest.param(*c[1:], id=c[0]) for c in C.cases()]
+
+
+@pytest.mark.parametrize("op,dst,src,idx,want", _nnlib_scatter_cases())
+def test_scatter_nnlib_reference_vectors(rx, client, op, dst, src, idx, want):
+    """NNlib.scatter! / scatter known answers (test/nn/scatter_gather.jl:254-428), all seven operations
+    (element - update and element / update included) through the module the reference's lowering builds."""
+    text = NN.nnlib_scatter(op, list(dst.shape), list(src.shape), list(idx.shape))
+    args = [I.tensor(dst, "f32"), I.Tensor(idx.reshape((1,) + idx.shape), "i64"), I.tensor(src, "f32")]
+    got, _ = gpu_run(rx, client, text, args)
+    np.testing.assert_allclose(got[0].a, want, rtol=1e-6)
+    assert np.array_equal(got[0].a, oracle_run(text, args)[0].a) or op in ("add", "subtract", "multiply", "divide", "mean")
+
+
+def test_scatter_subtract_divide_large(rx, client):
+    """element - update and element / update with many colliding updates, against the oracle."""
+    rng = np.random.default_rng(53)
+    for body, tol in (("subtract", 1e-5), ("divide", 1e-5)):
+        text = NN.scatter([1000, 64], [4096], [4096, 64], "f32", [1], [0], [0], 1, body=body)
+        dest = I.tensor(rng.normal(size=(1000, 64)), "f32")
+        upd = I.tensor(rng.uniform(0.5, 1.5, size=(4096, 64)), "f32")
+        idx = I.Tensor(rng.integers(-2, 1002, size=(4096,)).astype(np.int64), "i64")
+        got, exe = gpu_run(rx, client, text, [dest, idx, upd])
+        assert [l["kind"] for l in exe.launches()] == ["map", "scatter"]
+        _close(got[0].a, oracle_run(text, [dest, idx, upd])[0].a, tol)

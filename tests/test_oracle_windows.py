@@ -376,3 +376,19 @@ def test_scatter_against_numpy():
     t = NN.scatter([8], [3, 1], [3, 3], "f64", [1], [], [0], 1, body="add")
     got = I.run_text(t, [I.tensor(base, "f64"), I.Tensor(np.array([[0], [6], [4]]), "i64"), I.tensor(np.ones((3, 3)), "f64")])[0].a
     assert got.tolist() == [1, 1, 1, 0, 1, 1, 1, 0]
+
+
+def _nnlib_scatter_cases():
+    import _nnlib_scatter_cases as C
+    return [pytest.param(*c[1:], id=c[0]) for c in C.cases()]
+
+
+@pytest.mark.parametrize("op,dst,src,idx,want", _nnlib_scatter_cases())
+def test_scatter_nnlib_reference_vectors(op, dst, src, idx, want):
+    """NNlib.scatter! / scatter known answers (test/nn/scatter_gather.jl:254-428) through the module the
+    reference's lowering builds (ext/ReactantNNlibExt/Implementations.jl:477-530): pins the roles of
+    update_window_dims, inserted_window_dims, scatter_dims_to_operand_dims and index_vector_dim, and
+    the argument order of the update computation (element first: subtract and divide)."""
+    text = NN.nnlib_scatter(op, list(dst.shape), list(src.shape), list(idx.shape))
+    got = I.run_text(text, [I.tensor(dst, "f32"), I.Tensor(idx.reshape((1,) + idx.shape), "i64"), I.tensor(src, "f32")])[0].a
+    np.testing.assert_allclose(got, want, rtol=1e-6)
