@@ -12,7 +12,8 @@ region.  `cpu_baseline` times the oracle's C/OpenMP restatement of the stencil o
 host cores (a bounded number of repetitions of the same module).  `others` carries the remaining four configs
 (sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry; their step time is that
 of plain executions, and the pass with an event pair on every launch is reported beside it.
-`--workload conv|cumsum|maxpool` run one of the windowed ops instead (never part of `others`).
+`--workload conv|cumsum|maxpool` run one of the windowed ops instead, `--workload polybench` the
+reference's polybench stencil suite (never part of `others`).
 """
 import argparse
 import importlib
@@ -288,6 +289,45 @@ def bench_maxpool(rx, client, P, steps, warmup, batch=64, c=64, hw=112):
                          4.0 * batch * c * hw * hw * 1.25, 0.0, "f32", None)
 
 
+def bench_polybench(rx, client, P, steps, warmup, scale=1):
+    """The reference's polybench stencil suite at its own sizes (benchmark/polybench/stencil.jl:71,170,
+    229,301; f32, vectorized forms as traced loops): seconds per whole program (all its time steps),
+    and the same programs with one launch per update step for comparison.  `value` is array cells
+    updated per second over the four programs."""
+    PB = importlib.import_module("reactant_jl_amd.polybench_programs")
+    rng = np.random.default_rng(0)
+    progs, total_cells, total_s = [], 0.0, 0.0
+    for name in ("heat_3d", "jacobi_1d", "jacobi_2d", "fdtd_2d"):
+        sz = dict(PB.POLYBENCH_SIZES[name])
+        for key in ("tsteps", "tmax"):
+            if key in sz:
+                sz[key] = max(2, sz[key] // scale)
+        shapes = {"heat_3d": [(sz.get("n"),) * 3] * 2, "jacobi_1d": [(sz.get("n"),)] * 2, "jacobi_2d": [(sz.get("n"),) * 2] * 2,
+                  "fdtd_2d": [(sz.get("ny"), sz.get("nx"))] * 3 + [(sz.get("tmax"),)]}[name]
+        trips = sz.get("tsteps", sz.get("tmax"))
+        updates = {"heat_3d": 2, "jacobi_1d": 2, "jacobi_2d": 2, "fdtd_2d": 3}[name]
+        cells = float(np.prod(shapes[0])) * trips * updates
+        text = PB.build(name, **sz)
+        bufs = [_upload(rx, client, rng.random(s, dtype=np.float32), "f32") for s in shapes]
+        exe = rx.xla_compile(client, text)
+        secs = _time_plain(client, exe, bufs, steps, warmup)
+        os.environ["RX_CHAIN_STEPS"] = "1"
+        try:
+            exe1 = rx.xla_compile(client, text)
+        finally:
+            del os.environ["RX_CHAIN_STEPS"]
+        secs1 = _time_plain(client, exe1, bufs, max(2, steps // 2), 1)
+        kinds = [l["kind"] for l in exe.launches()]
+        progs.append({"program": name, "sizes": sz, "ms": 1e3 * secs, "launches": len(kinds), "chain_kernels": kinds.count("map_chain"),
+                      "ms_one_launch_per_step": 1e3 * secs1, "launches_one_per_step": len(exe1.launches()),
+                      "Gcells_per_s": cells / secs / 1e9})
+        total_cells += cells
+        total_s += secs
+    return {"workload": "polybench stencils f32 (heat_3d 128^3 x256, jacobi_1d 2048 x1024, jacobi_2d 512^2 x1024, fdtd_2d 1024x2048 x256)",
+            "ms_per_step": 1e3 * total_s, "value": total_cells / total_s / 1e9, "unit": "Gcell/s", "dtype": "f32", "programs": progs,
+            "roofline": None}
+
+
 def cpu_baseline_stencil(P, nx=512, ny=512, nz=256, nsteps=10):
     """The oracle's C restatement of the stencil (oracle/stencil_cpu.c, OpenMP on all host cores,
     same bits as the GPU result) on the full grid, a bounded number of repetitions of the
@@ -338,7 +378,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "polybench"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--small", action="store_true", help="reduced sizes (debugging only; not a valid result)")
@@ -351,10 +391,10 @@ def main():
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
-             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool}
+             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "polybench": bench_polybench}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
-             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4)}
+             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "polybench": dict(scale=16)}
     _FULL_SIZE[0] = not args.small
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
@@ -371,6 +411,8 @@ def main():
         out["check"] = main_res["check"]
     if "kernels" in main_res:
         out["kernels"] = main_res["kernels"]
+    if "programs" in main_res:
+        out["programs"] = main_res["programs"]
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_stencil(P) if args.workload == "stencil" else None
     if not args.no_others:

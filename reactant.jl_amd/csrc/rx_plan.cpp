@@ -16,6 +16,7 @@
 #include "rx_plan.h"
 
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <set>
 #include <sstream>
@@ -1734,6 +1735,276 @@ struct Planner {
     return true;
   }
 
+  // ------------------------------------------------------------------ chains of update steps through LDS
+  // A time loop over small arrays (the reference's polybench stencils, benchmark/polybench/stencil.jl)
+  // unrolls into a run of steps, each a dynamic_update_slice over one array (a "field") with values
+  // computed from neighbouring elements of the others.  With one launch per step such a loop is bound
+  // by the gap between dependent launches, not by memory.  A chain kernel runs K consecutive steps per
+  // launch: a workgroup loads its tile of every field plus a halo as wide as the K steps reach,
+  // updates the fields in LDS step by step on regions that shrink by each step's reach (neighbouring
+  // workgroups recompute each other's halos), and writes its tile of the fields that changed.
+  // Versions of a field that are superseded inside the kernel never reach memory.
+  struct ChainProbe {
+    int base = -1;                 // the array the step's update is written over
+    std::map<int, Halo> reads;     // inputs of the field's shape and type, and how far the step reads around a point
+    std::vector<int> others;       // every other input (read from memory as in a map kernel)
+  };
+  std::map<int, std::vector<int>> chain_at;   // first step of a chain -> all its steps
+  std::set<int> chain_member;                 // steps emitted by a chain kernel
+
+  // steps per kernel: a 1-d tile's halo grows by a cell or two per step, so long chains stay cheap
+  int chain_cap(int rank) const { return opt.chain_steps > 0 ? opt.chain_steps : rank == 1 ? 64 : 16; }
+
+  bool probe_chain_step(int x, ChainProbe* cp) {
+    const Node& n = g.nodes[x];
+    const int r = n.ty.rank();
+    if (n.k != OpK::DynamicUpdateSlice || r < 1 || r > 3 || r > opt.chain_max_rank) return false;
+    const int es = info(n.ty.dt).size;
+    if (es != 4 && es != 8) return false;
+    if (n.ty.numel() < 2 || n.ty.numel() >= opt.slab_min_numel) return false;
+    int b = n.in[0];
+    while (!mat[b] && g.nodes[b].k == OpK::DynamicUpdateSlice) b = g.nodes[b].in[0];
+    if (!mat[b] || !(g.nodes[b].ty == n.ty)) return false;
+    Emitter probe(g, [&](int y) { return y != x && mat[y]; });
+    std::vector<std::string> vars;
+    Index ix(r);
+    for (int d = 0; d < r; ++d) {
+      vars.push_back("g" + std::to_string(d));
+      ix[d].var = vars[d]; ix[d].lo = 0; ix[d].hi = n.ty.dims[d] - 1;
+    }
+    probe.set_root(n.ty.dims, vars, false);
+    probe.excess_precision = opt.excess_precision;
+    try { probe.emit(x, ix); } catch (const Error&) { return false; }
+    cp->base = b;
+    bool saw_base = false;
+    for (auto& l : probe.loads) {
+      const Node& ln = g.nodes[l.node];
+      if (ln.ty == n.ty) {
+        if (!l.affine) return false;
+        Halo& h = cp->reads[l.node];
+        for (int d = 0; d < r; ++d) { h.lo[d] = std::max<int64_t>(h.lo[d], -l.off[d]); h.hi[d] = std::max<int64_t>(h.hi[d], l.off[d]); }
+        saw_base = saw_base || l.node == b;
+      } else cp->others.push_back(l.node);
+    }
+    if (!saw_base) return false;
+    for (auto& kv : cp->reads)
+      for (int d = 0; d < r; ++d) if (kv.second.lo[d] > 4 || kv.second.hi[d] > 4) return false;
+    return true;
+  }
+
+  // every kernel that reads `v` is one of `group` (or `also`)
+  bool read_only_by(int v, const std::set<int>& group, int also) {
+    std::vector<int> st{v};
+    std::set<int> seen;
+    while (!st.empty()) {
+      int y = st.back();
+      st.pop_back();
+      for (int u : users[y]) {
+        if (!live[u]) continue;
+        if (mat[u]) { if (!group.count(u) && u != also) return false; }
+        else if (seen.insert(u).second) st.push_back(u);
+      }
+    }
+    return true;
+  }
+
+  // Kernel for a prefix of `steps`; returns how many steps it covers (0: none, nothing emitted).
+  size_t emit_chain(const std::vector<int>& steps, const std::vector<ChainProbe>& probes) {
+    const Node& n0 = g.nodes[steps[0]];
+    const int r = n0.ty.rank();
+    const auto& D = n0.ty.dims;
+    const int es = info(n0.ty.dt).size;
+    const std::string st = info(n0.ty.dt).stype;
+    int64_t T[3] = {1, 1, 1};
+    {
+      const int64_t dflt[3][3] = {{256, 1, 1}, {32, 64, 1}, {8, 8, 32}};
+      for (int d = 0; d < r; ++d) {
+        T[d] = opt.chain_tile[d] > 0 && opt.chain_tile[r - 1] > 0 ? opt.chain_tile[d] : dflt[r - 1][d];
+        T[d] = std::min<int64_t>(T[d], D[d]);
+      }
+    }
+    for (size_t k = std::min<size_t>(steps.size(), (size_t)chain_cap(r)); k >= 2; --k) {
+      // fields of the first k steps: version at kernel entry, and which field each node is a version of
+      std::vector<int> entry;
+      std::map<int, int> field_of;
+      for (size_t i = 0; i < k; ++i) {
+        for (auto& kv : probes[i].reads)
+          if (!field_of.count(kv.first)) { field_of[kv.first] = (int)entry.size(); entry.push_back(kv.first); }
+        field_of[steps[i]] = field_of[probes[i].base];
+      }
+      const int nf = (int)entry.size();
+      std::vector<std::array<int64_t, 3>> lo(k), hi(k);
+      int64_t HL[3] = {0, 0, 0}, HH[3] = {0, 0, 0};
+      for (size_t i = 0; i < k; ++i) {
+        lo[i] = {0, 0, 0}; hi[i] = {0, 0, 0};
+        for (auto& kv : probes[i].reads)
+          for (int d = 0; d < r; ++d) { lo[i][d] = std::max(lo[i][d], kv.second.lo[d]); hi[i][d] = std::max(hi[i][d], kv.second.hi[d]); }
+        for (int d = 0; d < r; ++d) { HL[d] += lo[i][d]; HH[d] += hi[i][d]; }
+      }
+      int64_t E[3] = {1, 1, 1}, box = 1, tile = 1;
+      for (int d = 0; d < r; ++d) { E[d] = T[d] + HL[d] + HH[d]; box *= E[d]; tile *= T[d]; }
+      const int64_t lds_bytes = box * nf * es;
+      if (lds_bytes > opt.chain_lds_bytes || (double)box > opt.chain_redundancy * (double)tile) continue;
+      const int NB = opt.chain_threads > 0 ? opt.chain_threads : box >= 4096 ? 1024 : box >= 1024 ? 512 : 256;
+      if (NB < 64 || NB > 1024 || NB % 64) continue;
+
+      // the steps' bodies, evaluated at the array position (g0, g1, g2) whose cell in the box is `li`
+      std::vector<std::string> vars;
+      Index ix(r);
+      for (int d = 0; d < r; ++d) {
+        vars.push_back("g" + std::to_string(d));
+        ix[d].var = vars[d]; ix[d].lo = 0; ix[d].hi = D[d] - 1;
+      }
+      std::vector<int> inputs, cur = entry, writes(k);
+      std::vector<std::string> bodies(k), vals(k);
+      std::set<int> group(steps.begin(), steps.begin() + k);
+      bool ok = true;
+      for (size_t i = 0; i < k && ok; ++i) {
+        const int x = steps[i];
+        Emitter em(g, [&, x](int y) { return y != x && mat[y]; });
+        em.inputs = inputs;
+        em.set_root(D, vars, false);
+        em.excess_precision = opt.excess_precision;
+        em.branchless_guards = opt.branchless_guards;
+        em.indent = 6;
+        em.tile_hook = [&](int slot, const std::vector<int64_t>& off, std::string* expr) {
+          const int node = em.inputs[slot];
+          auto f = field_of.find(node);
+          if (f == field_of.end() || !(g.nodes[node].ty == n0.ty)) return false;
+          if (cur[f->second] != node) { ok = false; return false; }
+          int64_t delta = 0, stride = 1;
+          for (int d = r - 1; d >= 0; --d) { delta += off[d] * stride; stride *= E[d]; }
+          *expr = "lds" + std::to_string(f->second) + "[li + (" + std::to_string(delta) + ")]";
+          return true;
+        };
+        vals[i] = em.store_value(n0.ty.dt, em.emit(x, ix));
+        bodies[i] = em.take_code();
+        for (auto& l : em.loads) if (group.count(l.node) && !(l.affine && g.nodes[l.node].ty == n0.ty)) ok = false;
+        inputs = em.inputs;
+        writes[i] = field_of[probes[i].base];
+        cur[writes[i]] = x;
+      }
+      if (!ok) continue;
+
+      std::ostringstream o;
+      const std::string kname = "@K@_chain";
+      o << "// " << k << " update steps through LDS tiles (";
+      for (int d = 0; d < r; ++d) o << (d ? "x" : "") << T[d];
+      o << " outputs per workgroup, box ";
+      for (int d = 0; d < r; ++d) o << (d ? "x" : "") << E[d];
+      o << ", " << nf << " fields): " << describe(steps[0]) << " ... -> " << n0.ty.str() << "\n";
+      std::vector<int> arg_nodes;
+      {
+        std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(NB) + ") void " + kname + "(";
+        bool first = true;
+        for (size_t q = 0; q < inputs.size(); ++q) {
+          if (group.count(inputs[q])) continue;
+          s += (first ? "" : ", ") + ptr_decl(info(g.nodes[inputs[q]].ty.dt).stype, true, "in" + std::to_string(q));
+          first = false;
+          arg_nodes.push_back(inputs[q]);
+        }
+        for (int f = 0; f < nf; ++f)
+          if (cur[f] != entry[f]) { s += (first ? "" : ", ") + ptr_decl(st, false, "out" + std::to_string(f)); first = false; }
+        o << s << ") {\n";
+      }
+      auto slot_in = [&](int node) {
+        for (size_t q = 0; q < inputs.size(); ++q) if (inputs[q] == node) return (int)q;
+        return -1;
+      };
+      o << "  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];\n";
+      for (int f = 0; f < nf; ++f) o << "  " << st << "* const lds" << f << " = reinterpret_cast<" << st << "*>(rx_smem) + " << f * box << ";\n";
+      int64_t nt[3] = {1, 1, 1}, ntiles = 1;
+      for (int d = 0; d < r; ++d) { nt[d] = (D[d] + T[d] - 1) / T[d]; ntiles *= nt[d]; }
+      o << "  int tb = blockIdx.x;\n";
+      for (int d = r - 1; d >= 0; --d) {
+        o << "  const int t" << d << " = (tb % " << nt[d] << ") * " << T[d] << ";\n";
+        if (d) o << "  tb /= " << nt[d] << ";\n";
+      }
+      // Loops over the cells of a region run a fixed number of rounds per thread without branches
+      // (cells past the end repeat the last one, array positions are clamped into the array, and
+      // only the final LDS or global store is predicated), so that the compiler can keep the loads
+      // of several rounds in flight.
+      // decode cell p of a region with extents ext[] whose first cell sits at (t - back[]) in the array
+      auto open_loop = [&](int64_t total, const int64_t* ext, const int64_t* back, const char* ind) {
+        const int64_t rounds = (total + NB - 1) / NB;
+        o << "#pragma unroll " << std::min<int64_t>(rounds, 8) << "\n";
+        o << "  for (int q = 0; q < " << rounds << "; ++q) {\n";
+        o << ind << "const int p = threadIdx.x + q * " << NB << ";\n";
+        o << ind << "int rr = rx_min(p, " << total - 1 << ");\n";
+        for (int d = r - 1; d >= 0; --d) {
+          if (d) { o << ind << "const int c" << d << " = rr % " << ext[d] << ";\n" << ind << "rr /= " << ext[d] << ";\n"; }
+          else o << ind << "const int c0 = rr;\n";
+        }
+        std::string in_arr = "p < " + std::to_string(total);
+        for (int d = 0; d < r; ++d) {
+          o << ind << "const int a" << d << " = t" << d << " - " << back[d] << " + c" << d << ";\n";
+          o << ind << "const int g" << d << " = rx_clamp_idx<int>(a" << d << ", " << D[d] - 1 << ");\n";
+          in_arr += " && a" + std::to_string(d) + " == g" + std::to_string(d);
+        }
+        o << ind << "const bool live = " << in_arr << ";\n";
+      };
+      auto box_index = [&](const int64_t* back) {   // cell of the box that holds array position a
+        std::string e;
+        for (int d = 0; d < r; ++d) {
+          const std::string c = "(c" + std::to_string(d) + " + " + std::to_string(HL[d] - back[d]) + ")";
+          e = d ? "(" + e + ") * " + std::to_string(E[d]) + " + " + c : c;
+        }
+        return e;
+      };
+      auto array_index = [&]() {
+        std::string e;
+        for (int d = 0; d < r; ++d) e = d ? "(" + e + ") * " + std::to_string(D[d]) + " + g" + std::to_string(d) : "g0";
+        return e;
+      };
+      // stage every field's box
+      {
+        open_loop(box, E, HL, "    ");
+        o << "    const int lin = " << array_index() << ";\n";
+        for (int f = 0; f < nf; ++f) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
+        o << "    if (p < " << box << ") {\n";
+        for (int f = 0; f < nf; ++f) o << "      lds" << f << "[p] = s" << f << ";\n";
+        o << "    }\n  }\n  __syncthreads();\n";
+      }
+      for (size_t i = 0; i < k; ++i) {
+        int64_t back[3] = {0, 0, 0}, ext[3] = {1, 1, 1}, total = 1;
+        for (int d = 0; d < r; ++d) {
+          int64_t fwd = 0;
+          for (size_t j = i + 1; j < k; ++j) { back[d] += lo[j][d]; fwd += hi[j][d]; }
+          ext[d] = T[d] + back[d] + fwd;
+          total *= ext[d];
+        }
+        o << "  // step " << i << ": " << describe(steps[i]) << "\n";
+        open_loop(total, ext, back, "    ");
+        o << "    {\n      const int li = " << box_index(back) << ";\n";
+        o << bodies[i];
+        o << "      if (live) lds" << writes[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
+      }
+      {
+        const int64_t zero[3] = {0, 0, 0};
+        open_loop(tile, T, zero, "    ");
+        o << "    if (live) {\n      const int li = " << box_index(zero) << ";\n      const int lin = " << array_index() << ";\n";
+        for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = lds" << f << "[li];\n";
+        o << "    }\n  }\n}\n\n";
+      }
+      const std::string kb_final = finalize(o.str());
+      Launch L;
+      L.kernel = named(kname, kb_final);
+      L.kind = "map_chain";
+      L.grid[0] = (unsigned)ntiles;
+      L.block[0] = NB;
+      L.lds_bytes = (unsigned)lds_bytes;
+      for (int a : arg_nodes) L.args.push_back(buffer_for(a));
+      std::vector<int> outs;
+      for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) { L.args.push_back(buffer_for(cur[f])); outs.push_back(cur[f]); }
+      L.n_outputs = (int)outs.size();
+      L.algo_bytes = algo_bytes(arg_nodes, outs);
+      L.desc = std::to_string(k) + " steps: " + describe(steps[0]) + " ...";
+      plan.launches.push_back(L);
+      return k;
+    }
+    return 0;
+  }
+
   // ------------------------------------------------------------------ map kernels
   // `value` >= 0: write that node's values (same type as `root`) into root's buffer instead of
   // evaluating root itself (the copy of the operand a scatter starts from).
@@ -3142,6 +3413,63 @@ struct Planner {
         if (!probe_stencil(s, &sq) || sq.staged.size() != 1) continue;
         fuse_prev[x] = s;
         lds_only.insert(s);
+      }
+    }
+    // Runs of update steps over small arrays share chain kernels.
+    if (opt.chain_steps == 0 || opt.chain_steps >= 2) {
+      std::vector<char> is_result(N, 0);
+      for (int r : g.results) is_result[r] = 1;
+      size_t i = 0;
+      while (i < jobs.size()) {
+        std::vector<int> steps;
+        std::vector<ChainProbe> probes;
+        std::set<int> group;
+        std::map<int, int> field_of;
+        std::vector<int> cur;
+        for (size_t j = i; j < jobs.size() && (steps.empty() || steps.size() < (size_t)chain_cap(g.nodes[steps[0]].ty.rank())); ++j) {
+          const int x = jobs[j].first;
+          if (absorbed_roots.count(x) || reshape_alias.count(x) || !row_phases(x).empty()) break;
+          ChainProbe q;
+          if (!probe_chain_step(x, &q)) break;
+          if (!steps.empty() && !(g.nodes[x].ty == g.nodes[steps[0]].ty)) break;
+          bool ok = true;
+          // what a step reads is either outside the kernel or the latest version of a field
+          for (auto& kv : q.reads) ok = ok && (!group.count(kv.first) || cur[field_of[kv.first]] == kv.first);
+          for (int y : q.others) ok = ok && !group.count(y);
+          // the step overwrites its field in place: it may read that field only at its own position
+          const Halo& hb = q.reads[q.base];
+          for (int d = 0; d < 3; ++d) ok = ok && hb.lo[d] == 0 && hb.hi[d] == 0;
+          // a version superseded inside the kernel exists nowhere else
+          if (ok && group.count(q.base)) ok = !is_result[q.base] && read_only_by(q.base, group, x);
+          if (!ok) break;
+          for (auto& kv : q.reads)
+            if (!field_of.count(kv.first)) { field_of[kv.first] = (int)cur.size(); cur.push_back(kv.first); }
+          const int fw = field_of[q.base];
+          field_of[x] = fw;
+          cur[fw] = x;
+          group.insert(x);
+          steps.push_back(x);
+          probes.push_back(q);
+        }
+        if (steps.size() < 2) { ++i; continue; }
+        chain_at[steps[0]] = steps;
+        auto plain0 = jobs[i].second;
+        jobs[i].second = [this, steps, probes, plain0] {
+          size_t at = 0;
+          while (steps.size() - at >= 2) {
+            const size_t used = emit_chain(std::vector<int>(steps.begin() + at, steps.end()), std::vector<ChainProbe>(probes.begin() + at, probes.end()));
+            if (!used) break;
+            for (size_t q = 0; q < used; ++q) chain_member.insert(steps[at + q]);
+            at += used;
+          }
+          if (!chain_member.count(steps[0])) plain0();
+        };
+        for (size_t q = 1; q < steps.size(); ++q) {
+          auto plain = jobs[i + q].second;
+          const int x = steps[q];
+          jobs[i + q].second = [this, x, plain] { if (!chain_member.count(x)) plain(); };
+        }
+        i += steps.size();
       }
     }
     // row groups claim their reductions before those would be emitted on their own

@@ -61,6 +61,15 @@ struct PlanOptions {
   bool stencil_march2 = true;      // two-step kernel marching along the slowest dimension instead of 3-D tiles
   int march2_tile[2] = {8, 64};    // its outputs per plane (rows, columns)
   int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
+  // Runs of in-place update steps over small arrays (time loops of stencils): up to `chain_steps`
+  // consecutive steps per launch, the arrays held in LDS tiles in between (0: 64 for vectors, 16
+  // otherwise; 1: off)
+  int chain_steps = 0;
+  int chain_tile[3] = {0, 0, 0};     // outputs per workgroup (slowest .. fastest dimension of the array's rank; zeros: default per rank)
+  int64_t chain_lds_bytes = 64 * 1024;  // LDS a workgroup may use for the tiles
+  int chain_max_rank = 2;            // rank-3 steps are bound by index arithmetic in such a kernel, not by launches: left as maps
+  int chain_threads = 0;             // workgroup size (0: by the number of staged cells)
+  double chain_redundancy = 3.0;     // largest ratio of staged cells (tile plus halo) to tile cells
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once

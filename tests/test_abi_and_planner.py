@@ -256,3 +256,20 @@ def test_windowed_ops_plan(monkeypatch):
     monkeypatch.delenv("RX_FUSE_DOT_OPERANDS")
     with pytest.raises(Exception, match="batch_group_count and feature_group_count"):
         rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 4, 4, 4], "f32", groups=2)[0].replace("batch_group_count = 1", "batch_group_count = 2"))
+
+
+def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
+    """The reference's polybench stencils (benchmark/polybench/stencil.jl) at its sizes: 1024 or 256
+    trips of a `stablehlo.while` unroll into runs of update steps, which share chain kernels."""
+    import importlib
+    PB = importlib.import_module("reactant_jl_amd.polybench_programs")
+    kinds = lambda rep: [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
+    k = kinds(rx.compile_offline(PB.build("jacobi_1d")))            # 2048 half steps, 64 per launch
+    assert k == ["map_chain"] * 32
+    rep = rx.compile_offline(PB.build("jacobi_2d"), with_source=True)
+    assert kinds(rep) == ["map_chain"] * 128 and "16 update steps through LDS tiles (32x64 outputs per workgroup, box 64x96, 2 fields)" in rep
+    k = kinds(rx.compile_offline(PB.build("fdtd_2d", tmax=32)))      # the last launch fuses the updates nobody returns
+    assert k.count("map_chain") == len(k) - 1 and len(k) <= 8
+    assert kinds(rx.compile_offline(PB.build("heat_3d", tsteps=8))) == ["map"] * 16     # rank 3: one launch per step
+    monkeypatch.setenv("RX_CHAIN_STEPS", "1")
+    assert kinds(rx.compile_offline(PB.build("jacobi_1d", tsteps=16))) == ["map"] * 32

@@ -392,3 +392,29 @@ def test_scatter_nnlib_reference_vectors(op, dst, src, idx, want):
     text = NN.nnlib_scatter(op, list(dst.shape), list(src.shape), list(idx.shape))
     got = I.run_text(text, [I.tensor(dst, "f32"), I.Tensor(idx.reshape((1,) + idx.shape), "i64"), I.tensor(src, "f32")])[0].a
     np.testing.assert_allclose(got, want, rtol=1e-6)
+
+
+def test_polybench_stencil_modules_follow_the_julia_loops():
+    """The four vectorized polybench programs (benchmark/polybench/stencil.jl) as `stablehlo.while`
+    modules over dim-reversed tensors, against loop nests written from the Julia source on arrays
+    indexed like the Julia ones: pins the module builders (offsets, update boxes, the reversal of
+    dims) and the oracle's while / dynamic_update_slice on them, bit for bit."""
+    import _polybench_cases as C
+    rng = np.random.default_rng(5)
+    f = lambda *s: rng.random(s, dtype=np.float32)
+    rt = lambda a: I.tensor(np.ascontiguousarray(a.T), "f32")          # Julia array -> dim-reversed tensor
+    A, B = f(37), f(37)
+    out = I.run_text(C.P.jacobi_1d(37, 5), [rt(A), rt(B)])
+    for got, want in zip(out, C.jacobi_1d(5, A, B)):
+        assert np.array_equal(got.a.T, want)
+    A, B = f(13, 13), f(13, 13)
+    out = I.run_text(C.P.jacobi_2d(13, 4), [rt(A), rt(B)])
+    for got, want in zip(out, C.jacobi_2d(4, A, B)):
+        assert np.array_equal(got.a.T, want)
+    A, B = f(9, 9, 9), f(9, 9, 9)
+    out = I.run_text(C.P.heat_3d(9, 3), [rt(A), rt(B)])
+    for got, want in zip(out, C.heat_3d(3, A, B)):
+        assert np.array_equal(got.a.T, want)
+    EX, EY, HZ, fict = f(11, 7), f(11, 7), f(11, 7), f(6)
+    out = I.run_text(C.P.fdtd_2d(11, 7, 6), [rt(EX), rt(EY), rt(HZ), I.tensor(fict, "f32")])
+    assert np.array_equal(out[0].a.T, C.fdtd_2d(EX, EY, HZ, fict))
