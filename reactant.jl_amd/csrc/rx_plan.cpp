@@ -2005,6 +2005,45 @@ struct Planner {
     return 0;
   }
 
+  // ------------------------------------------------------------------ updates in place
+  // root = dynamic_update_slice(base, update, constant starts) where `base` is a temporary that no
+  // later kernel reads: the result takes over base's buffer and the kernel touches only the box
+  // that changes (range `setindex!` on a traced array, src/Indexing.jl:438-443, costs the bytes of
+  // the range, not of the array).  Returns the box as (start, length) per dimension.
+  bool update_in_place_box(int root, std::vector<std::pair<int64_t, int64_t>>* box) {
+    if (!opt.in_place_updates) return false;
+    const Node& n = g.nodes[root];
+    if (n.k != OpK::DynamicUpdateSlice) return false;
+    const int base = n.in[0];
+    const Node& bn = g.nodes[base];
+    if (!mat[base] || !(bn.ty == n.ty) || bn.k == OpK::Param || bn.k == OpK::Constant) return false;
+    if (reshape_alias.count(base) || reshape_alias.count(root)) return false;
+    for (auto& kv : reshape_alias) if (kv.second == base) return false;
+    for (int r : g.results) if (r == base) return false;
+    const Node& un = g.nodes[n.in[1]];
+    if (un.ty.numel() == 0) return false;
+    box->clear();
+    for (int d = 0; d < n.ty.rank(); ++d) {
+      const Node& sn = g.nodes[n.in[2 + d]];
+      if (sn.k != OpK::Constant) return false;
+      const int64_t room = n.ty.dims[d] - un.ty.dims[d];
+      box->push_back({std::min(std::max<int64_t>(splat_as_int(sn), 0), room), un.ty.dims[d]});
+    }
+    // every other kernel that reads base runs before this one (kernels run in node order)
+    std::vector<int> st{base};
+    std::set<int> seen;
+    while (!st.empty()) {
+      int y = st.back();
+      st.pop_back();
+      for (int u : users[y]) {
+        if (!live[u] || u == root) continue;
+        if (mat[u]) { if (u > root) return false; }
+        else if (seen.insert(u).second) st.push_back(u);
+      }
+    }
+    return true;
+  }
+
   // ------------------------------------------------------------------ map kernels
   // `value` >= 0: write that node's values (same type as `root`) into root's buffer instead of
   // evaluating root itself (the copy of the operand a scatter starts from).
@@ -2037,6 +2076,31 @@ struct Planner {
     // evaluate the root op itself (it is materialized, so bypass the input test by emitting its op)
     std::string val = em.emit(value >= 0 ? value : root, ix);
     std::string body = em.take_code();
+    // an update that can take over its operand's buffer: the kernel reads that operand only at the
+    // position it writes
+    std::vector<std::pair<int64_t, int64_t>> box;
+    bool inplace = value < 0 && n >= 1 && update_in_place_box(root, &box);
+    if (inplace)
+      for (auto& l : em.loads)
+        if (l.node == rn.in[0]) {
+          bool own = l.affine;
+          for (auto off : l.off) own = own && off == 0;
+          inplace = inplace && own;
+        }
+
+    // does the update itself use the old values (x[r] .+= ...), or only the copy around the box?
+    bool update_reads_base = false;
+    if (inplace) {
+      std::vector<int> st{rn.in[1]};
+      std::set<int> seen;
+      while (!st.empty() && !update_reads_base) {
+        int y = st.back();
+        st.pop_back();
+        if (y == rn.in[0]) { update_reads_base = true; break; }
+        if (mat[y] || !seen.insert(y).second) continue;
+        for (int i : g.nodes[y].in) st.push_back(i);
+      }
+    }
 
     // shifted loads along the slowest dimension -> XCD slab order
     bool slab = false;
@@ -2087,6 +2151,16 @@ struct Planner {
       }
       o << "  const " << it << " lin0 = i0 * " << plane << (em.idx64 ? "LL" : "") << " + pe;\n";
     }
+    if (inplace) {
+      std::string outside;
+      for (int d = 0; d < n; ++d) {
+        const std::string v = "i" + std::to_string(d) + (d == n - 1 ? "b" : "");
+        const int64_t lo = box[d].first, hi = box[d].first + box[d].second;
+        outside += (d ? " || " : "") + (d == n - 1 ? v + " + " + std::to_string(vec) + " <= " + std::to_string(lo) : v + " < " + std::to_string(lo)) + " || " + v +
+                   " >= " + std::to_string(hi);
+      }
+      o << "  if (" << outside << ") return;   // outside the box that changes: the buffer already holds the operand\n";
+    }
     {
       // inputs read once, at the output's own position, stream through (non-temporal hint);
       // inputs read at several offsets stay cacheable
@@ -2106,6 +2180,13 @@ struct Planner {
           addr = "rx_clamp_idx<" + it + ">(lin0 + " + std::to_string(D) + sfx + ", " + std::to_string(numel - vec) + sfx + ")";
         }
         const bool stream = opt.nt_loads && nvec[slot] == 1 && D == 0 && nload[slot] == 1;
+        if (inplace && !update_reads_base && em.inputs[slot] == rn.in[0] && D == 0) {
+          // the old values matter only where a vector sticks out of the box
+          const std::string v = "i" + std::to_string(n - 1) + "b";
+          o << "  const " << vt << " " << vec_name(slot, D) << " = (" << v << " < " << box[n - 1].first << " || " << v << " + " << vec << " > "
+            << box[n - 1].first + box[n - 1].second << ") ? rx_load<" << vt << ">(in" << slot << " + lin0) : " << vt << "{};\n";
+          continue;
+        }
         o << "  const " << vt << " " << vec_name(slot, D) << " = " << (stream ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + " << addr
           << ");\n";
       }
@@ -2122,16 +2203,32 @@ struct Planner {
       o << "  " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + lin0, res);\n";
     }
     o << "}\n\n";
-    const std::string kb_final = finalize(o.str());
+    std::string ktext = o.str();
+    if (inplace) {
+      // the operand and the result are the same memory
+      for (size_t q; (q = ktext.find("* __restrict__ ")) != std::string::npos;) ktext.replace(q, 15, "* ");
+      buf_of[root] = buffer_for(rn.in[0]);
+    }
+    const std::string kb_final = finalize(ktext);
 
     Launch L;
     L.kernel = named(kname, kb_final);
-    L.kind = slab ? "map_stencil" : "map";
+    L.kind = inplace ? "map_in_place" : slab ? "map_stencil" : "map";
     L.grid[0] = n == 0 ? 1 : grid;
     L.block[0] = kBlock;
     for (int i : em.inputs) L.args.push_back(buffer_for(i));
     L.args.push_back(buffer_for(root));
     L.algo_bytes = algo_bytes(em.inputs, {root});
+    if (inplace) {
+      // the operand is not copied: its box is written (and read, if the update uses the old values)
+      std::vector<int> others;
+      bool reads_base = false;
+      for (int i : em.inputs) { if (i == rn.in[0]) reads_base = true; else others.push_back(i); }
+      (void)reads_base;   // unless the update uses them, old values are read only where a vector straddles the edge of the box
+      double boxb = info(rn.ty.dt).size;
+      for (auto& b : box) boxb *= (double)b.second;
+      L.algo_bytes = algo_bytes(others, {}) + boxb * (update_reads_base ? 2 : 1);
+    }
     L.desc = value >= 0 ? "copy of the scatter operand" : describe(root);
     plan.launches.push_back(L);
   }

@@ -70,6 +70,7 @@ struct PlanOptions {
   int chain_max_rank = 2;            // rank-3 steps are bound by index arithmetic in such a kernel, not by launches: left as maps
   int chain_threads = 0;             // workgroup size (0: by the number of staged cells)
   double chain_redundancy = 3.0;     // largest ratio of staged cells (tile plus halo) to tile cells
+  bool in_place_updates = true;   // dynamic_update_slice over a temporary nobody reads later writes only its box, into the operand's buffer
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)
   bool nt_loads = true;         // non-temporal hint on inputs that are read exactly once

@@ -270,6 +270,9 @@ def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
     assert kinds(rep) == ["map_chain"] * 128 and "16 update steps through LDS tiles (32x64 outputs per workgroup, box 64x96, 2 fields)" in rep
     k = kinds(rx.compile_offline(PB.build("fdtd_2d", tmax=32)))      # the last launch fuses the updates nobody returns
     assert k.count("map_chain") == len(k) - 1 and len(k) <= 8
-    assert kinds(rx.compile_offline(PB.build("heat_3d", tsteps=8))) == ["map"] * 16     # rank 3: one launch per step
+    # rank 3: one launch per step; once the arrays are temporaries each step writes only its box, in place
+    assert kinds(rx.compile_offline(PB.build("heat_3d", tsteps=8))) == ["map"] * 2 + ["map_in_place"] * 14
     monkeypatch.setenv("RX_CHAIN_STEPS", "1")
+    assert kinds(rx.compile_offline(PB.build("jacobi_1d", tsteps=16))) == ["map"] * 2 + ["map_in_place"] * 30
+    monkeypatch.setenv("RX_IN_PLACE", "0")
     assert kinds(rx.compile_offline(PB.build("jacobi_1d", tsteps=16))) == ["map"] * 32

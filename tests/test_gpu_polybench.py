@@ -66,11 +66,11 @@ def test_polybench_reference_sizes(rx, client, name):
 
 def test_heat_3d_reference_size(rx, client):
     """benchmark/polybench/stencil.jl:170 (128^3), a quarter of its 256 time steps: one map launch
-    per half step (rank-3 steps are not chained)."""
+    per half step (rank-3 steps are not chained), in place once the arrays are temporaries."""
     text = P.build("heat_3d", tsteps=64)
     args = _fields([(128, 128, 128)] * 2, "f32", seed=4)
     got, exe = gpu_run(rx, client, text, args)
-    assert _kinds(exe) == ["map"] * 128
+    assert _kinds(exe) == ["map"] * 2 + ["map_in_place"] * 126
     for g_, r_ in zip(got, oracle_run(text, args)):
         assert np.array_equal(g_.a, r_.a)
 
@@ -82,8 +82,12 @@ def test_chained_and_unchained_plans_agree(rx, client, monkeypatch):
     assert "map_chain" in _kinds(exe)
     monkeypatch.setenv("RX_CHAIN_STEPS", "1")
     plain, exe1 = gpu_run(rx, client, text, args)
-    assert "map_chain" not in _kinds(exe1) and len(exe1.launches()) > len(exe.launches())
+    assert "map_chain" not in _kinds(exe1) and "map_in_place" in _kinds(exe1) and len(exe1.launches()) > len(exe.launches())
     assert np.array_equal(chained[0].a, plain[0].a)
+    monkeypatch.setenv("RX_IN_PLACE", "0")
+    copied, exe2 = gpu_run(rx, client, text, args)
+    assert set(_kinds(exe2)) == {"map"}
+    assert np.array_equal(chained[0].a, copied[0].a)
 
 
 @pytest.mark.parametrize("tile,steps,threads", [("7,13", "5", "64"), ("64,64", "16", "1024"), ("3,200", "2", "256"), ("16,16", "9", "128")])
@@ -158,3 +162,51 @@ def test_intermediate_version_that_is_returned_ends_the_chain(rx, client):
     assert "map_chain" in _kinds(exe)
     for g_, r_ in zip(got, oracle_run(text, args)):
         assert np.array_equal(g_.a, r_.a)
+
+
+IN_PLACE = [
+    # array, box start, box shape, dtype
+    ((1000,), (3,), (900,), "f32"),
+    ((1000,), (0,), (1000,), "f32"),             # the whole array
+    ((64, 130), (5, 1), (50, 127), "f32"),       # rows whose vectors straddle both edges of the box
+    ((64, 130), (63, 129), (1, 1), "f64"),       # one element
+    ((20, 30, 44), (1, 2, 3), (18, 20, 37), "i32"),
+    ((7, 9, 11, 16), (1, 0, 2, 5), (5, 9, 8, 6), "f32"),
+    ((300, 300), (100, 0), (17, 300), "i8"),     # 16 elements per vector
+]
+
+
+@pytest.mark.parametrize("shape,start,box,dt", IN_PLACE)
+def test_range_setindex_writes_in_place(rx, client, shape, start, box, dt):
+    """y = f(x), a temporary that is worth storing; s = sum(y); y[range] = z + y[range]; return y and y + s:
+    the update takes over the temporary's buffer and writes only the box (the sum reads it before)."""
+    t, tb = P._tt(shape, dt), P._tt(box, dt)
+    lim = ", ".join("%d:%d" % (s, s + n) for s, n in zip(start, box))
+    idx = "".join("    %%s%d = stablehlo.constant dense<%d> : tensor<i64>\n" % (d, s) for d, s in enumerate(start))
+    text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> (%s, %s) {\n" % (t, tb, t, t)
+            + "    %%y0 = stablehlo.add %%arg0, %%arg0 : %s\n" % t
+            + "".join("    %%a%d = stablehlo.add %%y%d, %%arg0 : %s\n    %%y%d = stablehlo.multiply %%a%d, %%a%d : %s\n" % (k, k, t, k + 1, k, k, t) for k in range(4))
+            + "    %%y = stablehlo.subtract %%y4, %%arg0 : %s\n" % t
+            + "    %%sum = stablehlo.reduce(%%y init: %%z0) applies stablehlo.add across dimensions = [%s] : (%s, %s) -> %s\n"
+            % (", ".join(str(d) for d in range(len(shape))), t, P._tt([], dt), P._tt([], dt))
+            + "    %%old = stablehlo.slice %%y [%s] : (%s) -> %s\n" % (lim, t, tb)
+            + "    %%new = stablehlo.add %%arg1, %%old : %s\n" % tb + idx
+            + "    %%r = stablehlo.dynamic_update_slice %%y, %%new, %s : (%s, %s, %s) -> %s\n"
+            % (", ".join("%%s%d" % d for d in range(len(shape))), t, tb, ", ".join(["tensor<i64>"] * len(shape)), t)
+            + "    %%sb = stablehlo.broadcast_in_dim %%sum, dims = [] : (%s) -> %s\n" % (P._tt([], dt), t)
+            + "    %%w = stablehlo.add %%r, %%sb : %s\n" % t
+            + "    return %%r, %%w : %s, %s\n  }\n}\n" % (t, t))
+    text = text.replace("    %y0 = ", "    %%z0 = stablehlo.constant dense<%s> : %s\n    %%y0 = " % ("0.0" if dt[0] == "f" else "0", P._tt([], dt)), 1).replace("%%", "%")
+    if dt[0] == "f":
+        args = _fields([shape, box], dt, seed=1)
+    else:
+        rng = np.random.default_rng(1)
+        args = [I.Tensor(rng.integers(-20, 20, size=s).astype(I.NP_OF[dt]), dt) for s in (shape, box)]
+    got, exe = gpu_run(rx, client, text, args)
+    assert "map_in_place" in _kinds(exe), _kinds(exe)
+    ref = oracle_run(text, args)
+    assert np.array_equal(got[0].a, ref[0].a)
+    if dt[0] == "f":
+        np.testing.assert_allclose(got[1].a, ref[1].a, rtol=1e-4)
+    else:
+        assert np.array_equal(got[1].a, ref[1].a)
