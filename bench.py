@@ -12,8 +12,8 @@ region.  `cpu_baseline` times the oracle's C/OpenMP restatement of the stencil o
 host cores (a bounded number of repetitions of the same module).  `others` carries the remaining four configs
 (sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry; their step time is that
 of plain executions, and the pass with an event pair on every launch is reported beside it.
-`--workload conv|cumsum|maxpool` run one of the windowed ops instead, `--workload polybench` the
-reference's polybench stencil suite (never part of `others`).
+`--workload conv|cumsum|maxpool` run one of the windowed ops instead, `--workload polybench` /
+`polybench_linalg` the reference's polybench stencil and linear-algebra suites (never part of `others`).
 """
 import argparse
 import importlib
@@ -328,6 +328,47 @@ def bench_polybench(rx, client, P, steps, warmup, scale=1):
             "roofline": None}
 
 
+def bench_polybench_linalg(rx, client, P, steps, warmup, scale=1):
+    """The BLAS / linear-algebra / data-mining programs of the reference's polybench suite at its sizes
+    (benchmark/polybench/blas.jl, linalg_kernels.jl, data_mining.jl; f32, vectorized forms): seconds per
+    program.  Matrix-product programs report TFLOP/s of their products, matrix-vector programs GB/s of
+    the matrix bytes they must read.  `value` is the suite's total time in ms (lower is better)."""
+    PB = importlib.import_module("reactant_jl_amd.polybench_programs")
+    rng = np.random.default_rng(0)
+    # flops of the products / matrix bytes read once, per program
+    def work(name, kw):
+        n = kw.get("n", 0)
+        if name == "gemm": return 2.0 * n * n * kw["m"], 0
+        if name in ("syr2k",): return 4.0 * n ** 3, 0
+        if name in ("syrk", "correlation", "covariance"): return 2.0 * n ** 3, 0
+        if name == "2mm": return 4.0 * n ** 3, 0
+        if name == "3mm": return 2.0 * (kw["p"] * kw["q"] * kw["r"] + kw["r"] * kw["s"] * kw["p"] + kw["p"] * kw["r"] * kw["p"]), 0
+        if name == "doitgen": return 2.0 * kw["r"] * kw["q"] * kw["p"] * kw["p"], 0
+        if name == "gemver": return 0, 4.0 * n * n * 4        # read A, write Â, read Â twice
+        if name == "gesummv": return 0, 2.0 * n * n * 4
+        if name == "atax": return 0, 2.0 * n * n * 4
+        if name == "bicg": return 0, 2.0 * n * kw["m"] * 4
+        if name == "mvt": return 0, 2.0 * n * n * 4
+        return 0, 0
+    progs, total = [], 0.0
+    for name in PB.LINALG_SIZES:
+        kw = {k: max(8, v // scale) for k, v in PB.LINALG_SIZES[name].items()}
+        text, shapes = PB.linalg(name, **kw)
+        bufs = [_upload(rx, client, np.asarray(rng.random(tuple(reversed(s)), dtype=np.float32)), "f32") for s in shapes]
+        exe = rx.xla_compile(client, text)
+        secs = _time_plain(client, exe, bufs, steps, warmup)
+        flops, nbytes = work(name, kw)
+        e = {"program": name, "sizes": kw, "ms": 1e3 * secs, "launches": [l["kind"] for l in exe.launches()]}
+        if flops:
+            e["TFLOP_per_s"] = flops / secs / 1e12
+        if nbytes:
+            e["GB_per_s"] = nbytes / secs / 1e9
+        progs.append(e)
+        total += secs
+    return {"workload": "polybench BLAS / linear-algebra / data-mining programs f32 at the reference's sizes", "ms_per_step": 1e3 * total,
+            "value": 1e3 * total, "unit": "ms", "dtype": "f32", "programs": progs, "roofline": None, "higher_is_better": False}
+
+
 def cpu_baseline_stencil(P, nx=512, ny=512, nz=256, nsteps=10):
     """The oracle's C restatement of the stencil (oracle/stencil_cpu.c, OpenMP on all host cores,
     same bits as the GPU result) on the full grid, a bounded number of repetitions of the
@@ -378,7 +419,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "polybench"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "polybench", "polybench_linalg"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--small", action="store_true", help="reduced sizes (debugging only; not a valid result)")
@@ -391,10 +432,10 @@ def main():
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
-             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "polybench": bench_polybench}
+             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
-             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "polybench": dict(scale=16)}
+             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
@@ -402,7 +443,7 @@ def main():
     out = {
         "metric": "achieved HBM GB/s (map/reduce/stencil) + dot_general TFLOP/s, % of peak, 1 GPU",
         "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": main_res.get("higher_is_better", True), "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic", "config": {"workload": main_res["workload"]},
         "roofline": main_res["roofline"],
         "copy_kernel_GBs": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9 if copy_ms > 0 else None,

@@ -3409,6 +3409,11 @@ struct Planner {
       if (r.ty.dims != g.nodes[x].ty.dims) continue;
       // the root must not be the anchor of a row group (its reductions need the full row)
       if (!row_phases(c.first).empty()) continue;
+      // a root takes one product into its kernel; a second one feeding the same root (A*B' + B*A') runs
+      // on its own and is read back as an input
+      bool taken = false;
+      for (auto& kv : epilogue_of) taken = taken || kv.second == c.first;
+      if (taken) continue;
       epilogue_of[x] = c.first;
     }
     std::set<int> absorbed_roots;

@@ -95,3 +95,60 @@ def random_update_program(rng, shape, nfields, nsteps, dt="f32", results=None, s
     sig = ", ".join("%s: %s" % (a, t) for a in names)
     return (P._HDR.format(name="update_steps") + "  func.func @main(%s) -> %s {\n" % (sig, "(%s)" % rt if len(results) > 1 else rt)
             + b.text() + "    return %s : %s\n  }\n}\n" % (", ".join(cur[i] for i in results), rt))
+
+
+# The BLAS / linear-algebra / data-mining programs of the suite (benchmark/polybench/blas.jl,
+# linalg_kernels.jl, data_mining.jl) as numpy formulas on arrays indexed like the Julia ones,
+# evaluated in float64; arguments in the order of the Julia functions (numbers first where they are).
+def _f64(xs):
+    return [np.asarray(x, dtype=np.float64) for x in xs]
+
+
+LINALG_REFERENCE = {
+    "gemm": lambda al, be, A, B, C: [al * (A @ B) + be * C],
+    "gemver": lambda al, be, u1, u2, v1, v2, A, y, z: (lambda Ah: (lambda x: [Ah, x, al * (Ah @ x)])(be * (Ah.T @ y) + z))(A + np.outer(u1, v1) + np.outer(u2, v2)),
+    "gesummv": lambda al, be, A, B, x: [(al * A + be * B) @ x],
+    "syr2k": lambda al, be, A, B, C: [al * (A @ B.T) + al * (B @ A.T) + be * C],
+    "syrk": lambda al, be, A, C: [al * (A @ A.T) + be * C],
+    "2mm": lambda al, be, A, B, C, D: [al * (A @ B @ C) + be * D],
+    "3mm": lambda A, B, C, D: [(A @ B) @ (C @ D)],
+    "atax": lambda A, x: [A.T @ (A @ x)],
+    "bicg": lambda A, p, r: [A.T @ r, A @ p],
+    "doitgen": lambda A, x: [np.einsum("rqs,sp->rqp", A, x)],
+    "mvt": lambda x1, x2, y1, y2, A: [x1 + A @ y1, x2 + A.T @ y2],
+    "covariance": lambda D: (lambda X: [X.T @ X / (D.shape[0] - 1)])(D - D.mean(axis=0, keepdims=True)),
+}
+
+
+def _correlation(D):
+    n = D.shape[0]
+    X = D - D.mean(axis=0, keepdims=True)
+    sig = np.sqrt((X * X).sum(axis=0, keepdims=True))
+    sig = np.where(sig <= 0.1, 1.0, sig)
+    Xn = X / (sig / np.sqrt(n - 1))
+    return [Xn.T @ Xn / (n - 1)]
+
+
+LINALG_REFERENCE["correlation"] = _correlation
+
+LINALG_SMALL = {
+    "gemm": dict(n=96, m=160), "gemver": dict(n=200), "gesummv": dict(n=300), "syr2k": dict(n=128), "syrk": dict(n=130),
+    "2mm": dict(n=144), "3mm": dict(p=40, q=72, r=136, s=264), "atax": dict(n=257), "bicg": dict(n=120, m=333),
+    "doitgen": dict(r=6, q=10, p=36), "mvt": dict(n=310), "correlation": dict(n=150), "covariance": dict(n=150),
+}
+
+
+def linalg_args(shapes, seed=0):
+    """Arguments as Julia arrays (numbers for the 0-d ones), rand(Float32) like the reference's drivers."""
+    rng = np.random.default_rng(seed)
+    return [np.float32(rng.random()) if s == () else rng.random(s, dtype=np.float32) for s in shapes]
+
+
+def to_tensor(I, a):
+    """Julia array -> the dim-reversed tensor the module takes"""
+    a = np.asarray(a, dtype=np.float32)
+    return I.tensor(np.ascontiguousarray(a.T) if a.ndim else a, "f32")
+
+
+def from_tensor(t):
+    return np.asarray(t.a).T

@@ -210,3 +210,28 @@ def test_range_setindex_writes_in_place(rx, client, shape, start, box, dt):
         np.testing.assert_allclose(got[1].a, ref[1].a, rtol=1e-4)
     else:
         assert np.array_equal(got[1].a, ref[1].a)
+
+
+LINALG_MEDIUM = {
+    "gemm": dict(n=512, m=1024), "gemver": dict(n=1024), "gesummv": dict(n=1024), "syr2k": dict(n=512), "syrk": dict(n=512),
+    "2mm": dict(n=512), "3mm": dict(p=128, q=256, r=512, s=1024), "atax": dict(n=1024), "bicg": dict(n=512, m=1024),
+    "doitgen": dict(r=32, q=64, p=128), "mvt": dict(n=1024), "correlation": dict(n=512), "covariance": dict(n=512),
+}
+
+
+@pytest.mark.parametrize("size", ["small", "medium"])
+@pytest.mark.parametrize("name", sorted(C.LINALG_SMALL))
+def test_polybench_linalg_programs(rx, client, name, size):
+    """The BLAS / linear-algebra / data-mining programs of benchmark/polybench (matrix products with
+    scaled and transposed operands, two products feeding one sum, matrix-vector products as reductions,
+    column statistics) against the oracle with f64 accumulation; f32 tolerance 1e-5 sqrt(k) of the result's scale."""
+    kw = C.LINALG_SMALL[name] if size == "small" else LINALG_MEDIUM[name]
+    text, shapes = P.linalg(name, **kw)
+    args = [C.to_tensor(I, a) for a in C.linalg_args(shapes, seed=len(name) + len(size))]
+    got, exe = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    k = max(max(s) if s else 1 for s in shapes)
+    for g_, r_ in zip(got, ref):
+        assert g_.a.shape == r_.a.shape
+        scale = max(1.0, float(np.max(np.abs(r_.a))))
+        assert float(np.max(np.abs(g_.a.astype(np.float64) - r_.a.astype(np.float64)))) <= 1e-5 * np.sqrt(k) * scale

@@ -418,3 +418,25 @@ def test_polybench_stencil_modules_follow_the_julia_loops():
     EX, EY, HZ, fict = f(11, 7), f(11, 7), f(11, 7), f(6)
     out = I.run_text(C.P.fdtd_2d(11, 7, 6), [rt(EX), rt(EY), rt(HZ), I.tensor(fict, "f32")])
     assert np.array_equal(out[0].a.T, C.fdtd_2d(EX, EY, HZ, fict))
+
+
+def _linalg_names():
+    import _polybench_cases as C
+    return sorted(C.LINALG_SMALL)
+
+
+@pytest.mark.parametrize("name", _linalg_names())
+def test_polybench_linalg_modules_follow_the_julia_formulas(name):
+    """The vectorized BLAS / linear-algebra / data-mining programs of benchmark/polybench as modules over
+    dim-reversed tensors, against the Julia formulas evaluated by numpy in float64: pins the builders
+    (which operand of a dot_general is which, the adjoints, Julia's broadcasting of row and column vectors)."""
+    import _polybench_cases as C
+    text, shapes = C.P.linalg(name, **C.LINALG_SMALL[name])
+    args = C.linalg_args(shapes, seed=len(name))
+    got = I.run_text(text, [C.to_tensor(I, a) for a in args], hifi=True)
+    want = C.LINALG_REFERENCE[name](*C._f64(args))
+    assert len(got) == len(want)
+    for g_, w_ in zip(got, want):
+        g_ = C.from_tensor(g_)
+        assert g_.shape == w_.shape
+        assert np.max(np.abs(g_ - w_)) <= 2e-6 * max(1.0, np.max(np.abs(w_)))
