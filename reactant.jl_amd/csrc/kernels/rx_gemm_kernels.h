@@ -458,7 +458,10 @@ RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0
   }
 }
 
-template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
+// SPLIT > 1: workgroup (x, y) contracts the y-th of SPLIT equal slices of K and hands the epilogue
+// (y, m, n): partial products that a reduction over the leading index adds up (few output tiles, long K).
+template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
+          int SPLIT = 1>
 RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
   typedef typename MMA::elem E;
   constexpr int NT = WM * WN * 64;
@@ -481,6 +484,8 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
   const E* Ab = A + batch * (long long)M * K;
   const E* Bb = B + batch * (long long)N * K;
   constexpr long long A_GLD = A_KC ? K : M, B_GLD = B_KC ? K : N;
+  static_assert(SPLIT >= 1 && K % (SPLIT * BK) == 0 && !(BATCHED && SPLIT > 1), "split of K");
+  const int kbase = SPLIT > 1 ? (int)blockIdx.y * (K / SPLIT) : 0;
 
   rx_f32x16 acc[TM][TN];
 #pragma unroll
@@ -492,13 +497,13 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 
   auto issue = [&](int kt) {
     RX_LDS E* st = lds + (kt % S) * STAGE;
-    const int k0 = kt * BK;
+    const int k0 = kbase + kt * BK;
     if (A_KC) rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, A_GLD, m0, k0, M, K, st, tid);
     else rx_tile_load_direct<E, A_ROWS, A_COLS, NT, false>(Ab, A_GLD, k0, m0, K, M, st, tid);
     if (B_KC) rx_tile_load_direct<E, B_ROWS, B_COLS, NT, true>(Bb, B_GLD, n0, k0, N, K, st + A_SZ, tid);
     else rx_tile_load_direct<E, B_ROWS, B_COLS, NT, false>(Bb, B_GLD, k0, n0, K, N, st + A_SZ, tid);
   };
-  constexpr int KT = K / BK;
+  constexpr int KT = K / SPLIT / BK;
   constexpr int NS = BK / MMA::KS;   // MFMA k-steps per tile
   // Fragments are double-buffered in registers: the LDS reads of step s+1 are issued before the
   // MFMAs of step s.  The barrier that publishes tile kt+1 sits before the LAST step of tile kt:
@@ -599,7 +604,9 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
         const int n = nb + 8 * rg;
         if (m < M && n < N) {
           const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
-          if constexpr (BATCHED) epi(v, (int)batch, m, n); else epi(v, m, n);
+          if constexpr (BATCHED) epi(v, (int)batch, m, n);
+          else if constexpr (SPLIT > 1) epi(v, (int)blockIdx.y, m, n);
+          else epi(v, m, n);
         }
       }
     }

@@ -48,9 +48,10 @@ static GemmChoice choose_gemm_f64(int64_t batch, int64_t M, int64_t N, int64_t K
   return c;
 }
 
-GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc, bool staged_only) {
+GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_kc, bool b_kc, bool staged_only, int split) {
   GemmChoice c;
   if (a != b) return c;
+  if (split > 1 && (staged_only || batch != 1 || a == DT::F64)) return c;
   if (a == DT::F64 && out == DT::F64) return staged_only ? c : choose_gemm_f64(batch, M, N, K, a_kc, b_kc);
   std::string mma;
   int esize = 0, bk = 0;
@@ -78,7 +79,7 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (M <= 64 && N > 64) { BM = 64; BN = 128; }
   else if (N <= 64 && M > 64) { BM = 128; BN = 64; }
   else if (M > 128 && N > 128 && ((M + 255) / 256) * ((N + 255) / 256) * batch >= 256) { BM = 256; BN = 256; WM = 2; WN = 4; }
-  else if (((M + 127) / 128) * ((N + 127) / 128) * batch < 128) { BM = 64; BN = 64; }
+  else if (((M + 127) / 128) * ((N + 127) / 128) * batch * split < 128) { BM = 64; BN = 64; }
   if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
     int v[4];
     if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
@@ -103,13 +104,14 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
     const int64_t a_ch = (int64_t)BM * dbk / ve, b_ch = (int64_t)BN * dbk / ve;
     const int64_t stage_bytes = ((int64_t)BM + BN) * dbk * esize;
     while (stages > 2 && stage_bytes * stages > 160 * 1024) --stages;
-    if (dbk % ks == 0 && K % dbk == 0 && a_ch % nt == 0 && b_ch % nt == 0 && stage_bytes * stages <= 160 * 1024 &&
+    if (dbk % ks == 0 && K % ((int64_t)dbk * split) == 0 && a_ch % nt == 0 && b_ch % nt == 0 && stage_bytes * stages <= 160 * 1024 &&
         (a_kc ? dbk : BM) % ve == 0 && (b_kc ? dbk : BN) % ve == 0) {
       c.lds_bytes = (unsigned)(stage_bytes * stages);
       c.block = nt;
       const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
       c.grid[0] = (unsigned)gemm_grid(gm, gn, rb, cb);
-      c.grid[1] = (unsigned)batch;
+      c.grid[1] = (unsigned)(split > 1 ? split : batch);
+      c.split = split;
       std::ostringstream t;
       t << mma << ", " << BM << ", " << BN << ", " << dbk << ", " << WM << ", " << WN << ", " << stages << ", " << (a_kc ? "true" : "false") << ", "
         << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
@@ -120,6 +122,7 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       return c;
     }
   }
+  if (split > 1) return c;   // only the direct-to-LDS skeleton slices K
   const int pad = a == DT::F32 ? 4 : (esize == 2 ? 8 : 16);
   const int64_t a_sz = a_kc ? (int64_t)BM * (bk + pad) : (int64_t)bk * (BM + pad);
   const int64_t b_sz = b_kc ? (int64_t)BN * (bk + pad) : (int64_t)bk * (BN + pad);
@@ -156,6 +159,7 @@ std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const s
   o << "  " << epi_ctor << "\n";
   o << "  " << c.skeleton << "<" << c.targs << ", " << (batched ? "true" : "false") << ", " << kbase << "_epi";
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn" : fa.type) << ", " << (fb.type.empty() ? "rx_no_fn" : fb.type);
+  if (c.split > 1) o << ", " << c.split;
   o << ">(A, B, epi";
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn()" : "la") << ", " << (fb.type.empty() ? "rx_no_fn()" : "lb");
   o << ");\n}\n\n";

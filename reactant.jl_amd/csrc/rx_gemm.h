@@ -15,6 +15,7 @@ struct GemmChoice {
   unsigned block = 256;
   unsigned lds_bytes = 0;   // dynamic LDS (0: the skeleton declares static LDS)
   std::string stype_a, stype_b;
+  int split = 1;            // slices of K, one per blockIdx.y (partial products; rx_gemm_body_dl only)
 };
 
 // Workgroups to launch for a gm x gn grid of tiles: the kernels walk the tiles in blocks of 4 x 8,
@@ -29,7 +30,7 @@ inline int64_t gemm_grid(int64_t gm, int64_t gn, int rb = 4, int cb = 8) {
 // Returns ok=false when no skeleton covers the case (the caller then writes a scalar loop).
 // `staged_only`: an operand is a functor, which only the register-staged skeleton can read.
 GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, int64_t K, bool a_k_contig, bool b_k_contig,
-                       bool staged_only = false);
+                       bool staged_only = false, int split = 1);
 
 // Text of the `extern "C"` kernel <kbase>_gemm that runs the skeleton with epilogue type <kbase>_epi.
 // `epi_params` is the tail of the parameter list (epilogue operands and out0), `epi_ctor` builds `epi`.

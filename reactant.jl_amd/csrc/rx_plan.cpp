@@ -171,6 +171,7 @@ struct Planner {
     dots_to_reductions();
     normalize_dots();
     align_dots();
+    split_dots();
   }
 
   // A dot_general with several batch, free or contracting dims, or with them in another order than
@@ -305,7 +306,7 @@ struct Planner {
       return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral;
     };
     for (const Node& d : g.nodes) {
-      if (d.k != OpK::DotGeneral || d.ty.rank() < 2) continue;
+      if (d.k != OpK::DotGeneral || d.ty.rank() < 2 || !d.a4.empty()) continue;
       DotForm f = dot_form(d);
       if (!f.ok) continue;
       const DT a = g.nodes[d.in[0]].ty.dt, b = g.nodes[d.in[1]].ty.dt;
@@ -414,6 +415,74 @@ struct Planner {
       sl.a2.assign(n.ty.rank(), 1);
       sl.ty = n.ty;
       remap[n.id] = out.add(sl);
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
+  }
+
+  // A matrix product with few output tiles and a long contraction (the last product of a chain, a
+  // Gram matrix of tall data, the filter gradient of a convolution) leaves most compute units idle:
+  // K is cut into S slices, workgroup (tile, s) contracts slice s into a partial product
+  // [S, M, N] in f32, and a reduction over the leading index adds the slices up.
+  void split_dots() {
+    if (!opt.mfma || !opt.split_k) return;
+    std::map<int, int> splits;
+    for (const Node& d : g.nodes) {
+      if (d.k != OpK::DotGeneral || d.ty.rank() != 2 || !d.a0.empty()) continue;
+      DotForm f = dot_form(d);
+      if (!f.ok || f.batch != 1) continue;
+      const DT a = g.nodes[d.in[0]].ty.dt, b = g.nodes[d.in[1]].ty.dt;
+      if (a != b || !is_float(a) || a == DT::F64 || !is_float(d.ty.dt)) continue;
+      if (!choose_gemm(a, b, d.ty.dt, 1, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig).ok) continue;
+      const int64_t tiles = ((f.M + 63) / 64) * ((f.N + 63) / 64);
+      if (tiles >= 256 || f.K < 1024) continue;
+      // enough slices for two workgroups per compute unit, each slice at least 512 long
+      int S = 1;
+      while (S < 256 && tiles * S < 512 && f.K / (2 * S) >= 512) S *= 2;
+      for (; S > 1; S /= 2) {
+        if (f.K % S) continue;
+        GemmChoice c = choose_gemm(a, b, DT::F32, 1, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, false, S);
+        if (c.ok && c.split == S) break;
+      }
+      if (S > 1) splits[d.id] = S;
+    }
+    if (splits.empty()) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(g.nodes.size(), -1);
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      for (int& i : c.in) i = remap[i];
+      auto si = splits.find(n.id);
+      if (si == splits.end()) { remap[n.id] = out.add(c); continue; }
+      const int S = si->second;
+      c.a4 = {S};
+      c.ty = TType{DT::F32, {S, n.ty.dims[0], n.ty.dims[1]}};
+      const int part = out.add(c);
+      Node zero;
+      zero.k = OpK::Constant;
+      zero.splat = true;
+      zero.ty = TType{DT::F32, {}};
+      zero.data.assign(4, 0);
+      const int pz = out.add(zero);
+      Node red;
+      red.k = OpK::Reduce;
+      red.red = Red::Add;
+      red.in = {part, pz};
+      red.a0 = {0};
+      red.ty = TType{DT::F32, n.ty.dims};
+      int cur = out.add(red);
+      if (n.ty.dt != DT::F32) {
+        Node cv;
+        cv.k = OpK::Convert;
+        cv.ty = n.ty;
+        cv.in = {cur};
+        cur = out.add(cv);
+      }
+      remap[n.id] = cur;
     }
     for (int p : g.params) out.params.push_back(remap[p]);
     for (int r : g.results) out.results.push_back(remap[r]);
@@ -3215,8 +3284,10 @@ struct Planner {
 
     const bool fuse_a = fused_operands.count({dot, 0}) != 0, fuse_b = fused_operands.count({dot, 1}) != 0;
     GemmChoice gc;
-    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, fuse_a || fuse_b);
+    const int ksplit = d.a4.empty() ? 1 : (int)d.a4[0];
+    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, fuse_a || fuse_b, ksplit);
     if ((fuse_a || fuse_b) && !gc.ok) throw Error("internal: a fused dot_general operand without a GEMM skeleton");
+    if (ksplit > 1 && (!gc.ok || gc.split != ksplit || root != dot)) throw Error("internal: a dot_general cut along K without the skeleton that slices K");
     std::ostringstream o;
     // operand functors: element (row, column) of the operand as it would be stored, evaluated from the fused cone
     GemmOperandFn fn_a, fn_b;
@@ -3295,7 +3366,7 @@ struct Planner {
     {
       double kprod = 1;
       for (auto c : d.a2) kprod *= (double)lt.dims[c];
-      L.flops = 2.0 * (double)d.ty.numel() * kprod;
+      L.flops = 2.0 * (double)d.ty.numel() * kprod / (double)(d.a4.empty() ? 1 : d.a4[0]);
     }
     std::vector<int> all_in;
     if (fuse_a) all_in.insert(all_in.end(), in_a.begin(), in_a.end()); else all_in.push_back(d.in[0]);

@@ -231,3 +231,37 @@ def test_dot_general_with_grouped_or_permuted_dims(rx, client, ls, rs, os_, attr
     assert got[0].a.shape == ref[0].a.shape
     err = max_rel_to_scale(got[0].a, ref[0].a)
     assert err <= {"bf16": 1e-2, "f64": 1e-13, "f32": 1e-4}[dt]
+
+
+SPLIT_CASES = [
+    # dt, out, M, N, K, a_kc, b_kc, slices
+    ("f32", "f32", 256, 256, 2048, True, False, 8),
+    ("f32", "f32", 128, 192, 8192, False, True, 16),
+    ("f32", "f32", 256, 2048, 4096, True, True, 2),
+    ("bf16", "bf16", 128, 128, 16384, True, False, 16),
+    ("bf16", "f32", 320, 192, 4096, False, False, 16),
+    ("f16", "f16", 64, 512, 4096, True, True, 16),
+    ("f8E4M3FN", "f32", 256, 128, 8192, True, True, 16),
+    ("f8E4M3FN", "bf16", 128, 128, 4096, False, True, 16),
+]
+
+
+@pytest.mark.parametrize("dt,out_dt,M,N,K,a_kc,b_kc,slices", SPLIT_CASES)
+def test_long_contractions_with_few_output_tiles_are_cut_along_k(rx, client, monkeypatch, dt, out_dt, M, N, K, a_kc, b_kc, slices):
+    """Few 64x64 output tiles and a long K: partial products of K slices in f32 ([S, M, N]), then a
+    reduction over the slices (and the rounding to the result type)."""
+    text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc)
+    a = I.tensor(np.random.default_rng(0).normal(size=a_shape), dt)
+    b = I.tensor(np.random.default_rng(1).normal(size=b_shape), dt)
+    got, exe = gpu_run(rx, client, text, [a, b])
+    L = exe.launches()
+    assert [l["kind"] for l in L][:2] == ["gemm_" + {"f32": "f32", "bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8"}[dt], "reduce_generic"], L
+    import re
+    assert int(re.search(r"kind=gemm_\w+ grid=\d+x(\d+)x1", exe.report()).group(1)) in (slices // 4, slices // 2, slices, 2 * slices)
+    ref = oracle_run(text, [a, b], hifi=True)
+    err = max_rel_to_scale(got[0].a, ref[0].a)
+    assert err <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
+    monkeypatch.setenv("RX_SPLIT_K", "0")
+    whole, exe1 = gpu_run(rx, client, text, [a, b])
+    assert len(exe1.launches()) == 1
+    assert max_rel_to_scale(whole[0].a, ref[0].a) <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
