@@ -48,6 +48,9 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       seven operations, four shapes), numpy indexed assignment and np.add.at; dropped
       out-of-range updates (whole windows, as XLA does; the StableHLO text says per element:
       PARITY UNPINNED between the two readings, the reference holds no case that tells them apart)
+  select_and_scatter (the gradient of pooling) ... torch's max_pool2d backward (a library routine) on
+      padded, strided and overlapping windows; the tie rules (GE keeps the first element, GT the last)
+      by a constant operand; the reference holds no known answer for it
   reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy
       max / argmax / argmin with ties, first and last index
   batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
@@ -1533,6 +1536,58 @@ class Interpreter:
                 raise ValueError("while body returns %d values for %d loop-carried ones" % (len(cur), len(op.operands)))
         raise ValueError("while loop did not terminate")
 
+    def _select_and_scatter(self, op, xs):
+        """stablehlo.select_and_scatter as the specification writes it (the gradient of pooling): per
+        window of the padded operand, walk the elements that lie inside the operand in row-major
+        order keeping `selected` unless select(selected, element) is false; then
+        result[selected] = scatter(result[selected], source[window]), windows in row-major order,
+        starting from an operand-shaped array of the init value.  The select region runs on all
+        windows at once, one window element at a time."""
+        operand, source, init = xs
+        at = op.attrs
+        r = operand.a.ndim
+        window = at["window_dimensions"]
+        strides = at.get("window_strides") or [1] * r
+        pad = at.get("padding") or [[0, 0]] * r
+        lo = [p[0] for p in pad]
+        oshape = source.a.shape
+        grid = np.indices(oshape) if oshape else np.zeros((0,), dtype=np.int64)
+        sel_val = np.zeros(oshape, dtype=operand.a.dtype)
+        sel_pos = [np.full(oshape, -1, dtype=np.int64) for _ in range(r)]
+        have = np.zeros(oshape, dtype=bool)
+        region = op.regions[0]
+        names = [nm for nm, _ in region[0].attrs["args"]]
+        body = [self._retarget(o_, tuple(oshape)) for o_ in region if o_.name != "__block_args__"]
+        for k in np.ndindex(*window):
+            pos = [grid[d] * strides[d] + k[d] - lo[d] for d in range(r)]
+            valid = np.ones(oshape, dtype=bool)
+            for d in range(r):
+                valid &= (pos[d] >= 0) & (pos[d] < operand.a.shape[d])
+            cl = tuple(np.clip(pos[d], 0, operand.a.shape[d] - 1) for d in range(r))
+            val = operand.a[cl]
+            keep = self._block(body, {names[0]: Tensor(sel_val, operand.dt), names[1]: Tensor(val, operand.dt)})[0].a.astype(bool)
+            take = valid & (~have | ~keep)
+            sel_val = np.where(take, val, sel_val)
+            for d in range(r):
+                sel_pos[d] = np.where(take, pos[d], sel_pos[d])
+            have |= valid
+        res = np.broadcast_to(init.a, operand.a.shape).astype(operand.a.dtype).copy()
+        sregion = op.regions[1]
+        snames = [nm for nm, _ in sregion[0].attrs["args"]]
+        sbody = [o_ for o_ in sregion if o_.name != "__block_args__"]
+        flat_idx = [p_[have] for p_ in sel_pos]
+        upd = source.a[have]
+        if len(sbody) == 2 and sbody[0].name == "add":
+            acc = res.astype(np.float64) if (self.hifi and is_float(operand.dt)) else res
+            np.add.at(acc, tuple(flat_idx), upd.astype(acc.dtype))
+            res = acc.astype(res.dtype) if acc is not res else res
+        else:
+            for n_ in range(upd.shape[0]):
+                tgt = tuple(int(f[n_]) for f in flat_idx)
+                env = {snames[0]: Tensor(res[tgt], operand.dt), snames[1]: Tensor(upd[n_], operand.dt)}
+                res[tgt] = _rounded(self._block(sbody, env)[0]).a
+        return Tensor(res, operand.dt)
+
     def _scatter(self, op, xs):
         """stablehlo.scatter (built by reference src/Ops.jl:2150-2268), update by update in row-major
         order of the update tensor.  As XLA does, an update window that does not lie wholly inside
@@ -1684,6 +1739,8 @@ class Interpreter:
             return [self._scatter(op, xs)]
         if n in ("batch_norm_inference", "batch_norm_training"):
             return _batch_norm(xs, at, n == "batch_norm_training", self.hifi)
+        if n == "select_and_scatter":
+            return [self._select_and_scatter(op, xs)]
         if n == "reverse":
             return [Tensor(np.ascontiguousarray(np.flip(xs[0].a, axis=tuple(at["dimensions"]))), xs[0].dt)]
         if n == "reduce_window":

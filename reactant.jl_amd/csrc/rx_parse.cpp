@@ -1435,6 +1435,169 @@ struct Builder {
     return g.add(rn);
   }
 
+  // select_and_scatter in the form the gradient of max / min pooling takes (select: one compare of
+  // the two values, scatter: add).  Per window: the position of the extreme (the first one in
+  // row-major window order for GE / LE, the last for GT / LT) from an index reduction over the
+  // window view, turned into operand coordinates; then a scatter-add of `source` into an operand-shaped
+  // array of `init`.  Padding never wins against data (it holds -inf / +inf); a window made of padding
+  // only lands outside the operand and is dropped by the scatter.
+  int build_select_and_scatter(const RawOp& o, int x, int src, int init, const TType& out) {
+    const char* what = "select_and_scatter: only the pooling-gradient form is supported (select = one GE / GT / LE / LT compare, scatter = add)";
+    const TType xt = ty(x), st_ = ty(src);
+    const int r = xt.rank();
+    if (!(out == xt) || !is_float(xt.dt) || is_narrow_float(xt.dt) || st_.dt != xt.dt || ty(init).rank() != 0 || r < 1) fail(what);
+    if (o.regions.size() != 2) fail(what);
+    auto body_of = [&](const std::vector<RawOp>& region, std::string* a, std::string* b) {
+      if (region.size() != 3 || region[0].name != "__block_args__" || region[0].block_args.size() != 2) fail(what);
+      *a = region[0].block_args[0].first; *b = region[0].block_args[1].first;
+      const RawOp& ret = region[2];
+      if (region[1].results.size() != 1 || ret.operands.size() != 1 || ret.operands[0] != region[1].results[0]) fail(what);
+      return &region[1];
+    };
+    std::string a, b;
+    const RawOp* cmp = body_of(o.regions[0], &a, &b);
+    if (cmp->name.substr(cmp->name.rfind('.') + 1) != "compare" || cmp->operands.size() != 2 || cmp->operands[0] != a || cmp->operands[1] != b) fail(what);
+    const std::string dir = cmp->sa.count("direction") ? cmp->sa.at("direction") : "";
+    const bool is_max = dir == "GE" || dir == "GT", is_min = dir == "LE" || dir == "LT";
+    if (!is_max && !is_min) fail(what);
+    const bool first = dir == "GE" || dir == "LE";
+    const RawOp* add = body_of(o.regions[1], &a, &b);
+    if (add->name.substr(add->name.rfind('.') + 1) != "add" || add->operands.size() != 2 ||
+        !((add->operands[0] == a && add->operands[1] == b) || (add->operands[0] == b && add->operands[1] == a))) fail(what);
+    auto get = [&](const char* key, int64_t dflt) {
+      std::vector<int64_t> v = o.ia.count(key) ? o.ia.at(key) : std::vector<int64_t>(r, dflt);
+      if ((int)v.size() != r) fail(std::string("select_and_scatter: ") + key + " must have one entry per dimension");
+      return v;
+    };
+    if (!o.ia.count("window_dimensions")) fail("select_and_scatter: window_dimensions missing");
+    const auto w = get("window_dimensions", 1), st = get("window_strides", 1);
+    std::vector<int64_t> pad = o.ia.count("padding") ? o.ia.at("padding") : std::vector<int64_t>(2 * r, 0);
+    if (pad.size() == 1) pad.assign(2 * r, pad[0]);
+    if ((int)pad.size() != 2 * r) fail("select_and_scatter: padding must be a (rank x 2) matrix");
+    std::vector<int64_t> lo(r), hi(r), zeros(r, 0), ones(r, 1);
+    bool any_pad = false;
+    for (int d = 0; d < r; ++d) {
+      lo[d] = pad[2 * d]; hi[d] = pad[2 * d + 1];
+      if (lo[d] < 0 || hi[d] < 0) fail("select_and_scatter: negative padding is not supported");
+      any_pad = any_pad || lo[d] || hi[d];
+    }
+    int cur = x;
+    if (any_pad) {
+      Node c;
+      c.k = OpK::Constant;
+      c.splat = true;
+      c.ty = TType{xt.dt, {}};
+      c.data.assign((size_t)info(xt.dt).size, 0);
+      store_scalar(xt.dt, is_max ? -INFINITY : INFINITY, 0, false, c.data.data());
+      const int pv = g.add(c);
+      Node pn;
+      pn.k = OpK::Pad;
+      pn.in = {x, pv};
+      pn.a0 = lo; pn.a1 = hi; pn.a2 = zeros;
+      pn.ty.dt = xt.dt;
+      for (int d = 0; d < r; ++d) pn.ty.dims.push_back(lo[d] + hi[d] + xt.dims[d]);
+      cur = g.add(pn);
+    }
+    const int win = window_view(cur, w, st, ones, "select_and_scatter");       // [w.., o..]
+    const TType wt = ty(win);
+    const std::vector<int64_t> odims(wt.dims.begin() + r, wt.dims.end());
+    if (odims != st_.dims) fail("select_and_scatter: source shape does not match the windows");
+    int64_t wn = 1;
+    for (int d = 0; d < r; ++d) wn *= w[d];
+    std::vector<int64_t> fdims{wn};
+    fdims.insert(fdims.end(), odims.begin(), odims.end());
+    const TType ft{xt.dt, fdims}, it{DT::I64, fdims}, ot{DT::I64, odims};
+    const int flat = add_node(OpK::Reshape, ft, {win});
+    // the extreme of every window, and the flat window offset that holds it
+    Node m;
+    m.k = OpK::Reduce;
+    m.red = is_max ? Red::Max : Red::Min;
+    {
+      Node c;
+      c.k = OpK::Constant;
+      c.splat = true;
+      c.ty = TType{xt.dt, {}};
+      c.data.assign((size_t)info(xt.dt).size, 0);
+      store_scalar(xt.dt, is_max ? -INFINITY : INFINITY, 0, false, c.data.data());
+      m.in = {flat, g.add(c)};
+    }
+    m.a0 = {0};
+    m.ty = TType{xt.dt, odims};
+    const int mv = g.add(m);
+    Node mb;
+    mb.k = OpK::BroadcastInDim;
+    mb.in = {mv};
+    mb.ty = ft;
+    for (int d = 0; d < r; ++d) mb.a0.push_back(d + 1);
+    const int mbv = g.add(mb);
+    Node eq;
+    eq.k = OpK::Compare;
+    eq.op = "EQ";
+    eq.in = {flat, mbv};
+    eq.ty = TType{DT::I1, fdims};
+    const int eqv = g.add(eq);
+    Node io;
+    io.k = OpK::Iota;
+    io.ty = it;
+    io.a0 = {0};
+    const int iov = g.add(io);
+    const int limv = splat_of(it, first ? (double)wn : -1.0);
+    Node sel;
+    sel.k = OpK::Select;
+    sel.in = {eqv, iov, limv};
+    sel.ty = it;
+    const int selv = g.add(sel);
+    Node jr;
+    jr.k = OpK::Reduce;
+    jr.red = first ? Red::Min : Red::Max;
+    jr.in = {selv, splat_of(TType{DT::I64, {}}, first ? (double)wn : -1.0)};
+    jr.a0 = {0};
+    jr.ty = ot;
+    const int jv = g.add(jr);
+    // operand coordinates of the selected element: o_d * stride_d + j_d - lo_d, stacked along a new last dim
+    std::vector<int64_t> idims = odims;
+    idims.push_back(1);
+    std::vector<int> parts;
+    int64_t inner = wn;
+    for (int d = 0; d < r; ++d) {
+      inner /= w[d];
+      int jd = binary_node("divide", jv, splat_of(ot, (double)inner));
+      jd = binary_node("remainder", jd, splat_of(ot, (double)w[d]));
+      Node od;
+      od.k = OpK::Iota;
+      od.ty = ot;
+      od.a0 = {d};
+      int pos = binary_node("multiply", g.add(od), splat_of(ot, (double)st[d]));
+      pos = binary_node("add", pos, jd);
+      pos = binary_node("subtract", pos, splat_of(ot, (double)lo[d]));
+      parts.push_back(add_node(OpK::Reshape, TType{DT::I64, idims}, {pos}));
+    }
+    int index = parts[0];
+    if (r > 1) {
+      Node cc;
+      cc.k = OpK::Concatenate;
+      cc.in = parts;
+      cc.a0 = {r};
+      cc.ty = TType{DT::I64, odims};
+      cc.ty.dims.push_back(r);
+      index = g.add(cc);
+    }
+    Node ib;
+    ib.k = OpK::BroadcastInDim;
+    ib.in = {init};
+    ib.ty = xt;
+    const int base = g.add(ib);
+    Node sc;
+    sc.k = OpK::Scatter;
+    sc.ty = xt;
+    sc.in = {base, index, src};
+    for (int d = 0; d < r; ++d) { sc.a1.push_back(d); sc.a2.push_back(d); }
+    sc.a4 = {r};
+    sc.op = "combine";
+    sc.red = Red::Add;
+    return g.add(sc);
+  }
+
   int binary_node(const char* op, int a, int b) {
     Node n;
     n.k = OpK::Binary;
@@ -2232,6 +2395,10 @@ struct Builder {
     if (sh == "reduce_window") {
       if (in.size() != 2) fail("variadic reduce_window is not supported");
       return {build_reduce_window(o, in[0], in[1], out1())};
+    }
+    if (sh == "select_and_scatter") {
+      need(3);
+      return {build_select_and_scatter(o, in[0], in[1], in[2], out1())};
     }
     if (sh == "convolution") {
       need(2);

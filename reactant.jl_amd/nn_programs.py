@@ -333,3 +333,26 @@ def nnlib_scatter(op, dst_shape, src_shape, idx_shape, dt="f32"):
             + "    %%q = stablehlo.divide %%sum, %%ns : %s\n" % to
             + "    %%sd = stablehlo.select %%isz, %%sum, %%q : %s, %s\n" % (tb, to)
             + "    %%0 = stablehlo.add %%arg0, %%sd : %s\n    return %%0 : %s\n  }\n}\n" % (to, to))
+
+
+def select_and_scatter(x_shape, dt, window, strides=None, padding=None, direction="GE"):
+    """`stablehlo.select_and_scatter` in the form the gradient of a pooling layer takes (what the
+    reverse pass of `reduce_window` with a maximum body becomes): select = one compare of the two
+    window elements, scatter = add, init 0.  Arguments: the pooled array and the gradient of the pooled
+    result.  Returns (text, source shape)."""
+    r = len(x_shape)
+    strides = strides or [1] * r
+    padding = padding or [[0, 0]] * r
+    s_shape = window_out_shape(x_shape, window, strides, padding, [1] * r, [1] * r)
+    tx, tsrc, t0, tb = tt(x_shape, dt), tt(s_shape, dt), tt([], dt), tt([], "i1")
+    pad = "[" + ", ".join("[%d, %d]" % (p[0], p[1]) for p in padding) + "]"
+    lst = lambda v: ", ".join(str(int(x)) for x in v)
+    text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%cst = stablehlo.constant dense<0.000000e+00> : %s\n"
+            "    %%0 = \"stablehlo.select_and_scatter\"(%%arg0, %%arg1, %%cst) <{padding = dense<%s> : tensor<%dx2xi64>, "
+            "window_dimensions = array<i64: %s>, window_strides = array<i64: %s>}> ({\n"
+            "    ^bb0(%%a: %s, %%b: %s):\n      %%c = stablehlo.compare  %s, %%a, %%b,  FLOAT : (%s, %s) -> %s\n      stablehlo.return %%c : %s\n    }, {\n"
+            "    ^bb0(%%a: %s, %%b: %s):\n      %%c = stablehlo.add %%a, %%b : %s\n      stablehlo.return %%c : %s\n    }) : (%s, %s, %s) -> %s\n"
+            "    return %%0 : %s\n  }\n}\n"
+            % (tx, tsrc, tx, t0, pad, r, lst(window), lst(strides), t0, t0, direction, t0, t0, tb, tb, t0, t0, t0, t0, tx, tsrc, t0, tx, tx))
+    return text, s_shape

@@ -443,3 +443,35 @@ def test_scatter_subtract_divide_large(rx, client):
         got, exe = gpu_run(rx, client, text, [dest, idx, upd])
         assert [l["kind"] for l in exe.launches()] == ["map", "scatter"]
         _close(got[0].a, oracle_run(text, [dest, idx, upd])[0].a, tol)
+
+
+SELECT_AND_SCATTER = [
+    # x shape, dtype, window, strides, padding, direction
+    ([8, 16, 32, 32], "f32", [1, 1, 2, 2], [1, 1, 2, 2], None, "GE"),                               # 2x2 max pooling, VGG
+    ([4, 8, 33, 29], "f32", [1, 1, 3, 3], [1, 1, 2, 2], [[0, 0], [0, 0], [1, 1], [1, 1]], "GE"),   # overlapping, padded
+    ([2, 4, 20, 20], "f64", [1, 1, 3, 3], [1, 1, 1, 1], None, "GE"),                                # every element in nine windows
+    ([3, 5, 40], "f32", [1, 1, 4], [1, 1, 4], None, "GT"),
+    ([2, 3, 8, 9, 10], "f32", [1, 1, 2, 2, 2], [1, 1, 2, 2, 2], None, "LE"),                        # 3-d min pooling
+    ([64, 64, 56, 56], "f32", [1, 1, 2, 2], [1, 1, 2, 2], None, "GE"),
+]
+
+
+@pytest.mark.parametrize("xs,dt,w,st,pd,direction", SELECT_AND_SCATTER)
+def test_select_and_scatter(rx, client, xs, dt, w, st, pd, direction):
+    """The gradient of pooling: the window's extreme found by an index reduction over the window view,
+    then a scatter-add; against the oracle (itself checked against torch's max_pool2d backward)."""
+    text, ss = NN.select_and_scatter(xs, dt, w, st, pd, direction=direction)
+    x, dy = _args([xs], dt, seed=61)[0], _args([ss], dt, seed=62)[0]
+    got, exe = gpu_run(rx, client, text, [x, dy])
+    assert [l["kind"] for l in exe.launches()][-1] == "scatter"
+    ref = oracle_run(text, [x, dy])
+    _close(got[0].a, ref[0].a, 1e-5 if dt == "f32" else 1e-13)
+
+
+def test_select_and_scatter_ties(rx, client):
+    x = I.tensor(np.ones((2, 3, 8, 8)), "f32")
+    dy = _args([[2, 3, 4, 4]], "f32", seed=63)[0]
+    for direction in ("GE", "GT", "LE", "LT"):
+        text, _ = NN.select_and_scatter([2, 3, 8, 8], "f32", [1, 1, 2, 2], [1, 1, 2, 2], None, direction=direction)
+        got, _ = gpu_run(rx, client, text, [x, dy])
+        assert np.array_equal(got[0].a, oracle_run(text, [x, dy])[0].a), direction

@@ -440,3 +440,49 @@ def test_polybench_linalg_modules_follow_the_julia_formulas(name):
         g_ = C.from_tensor(g_)
         assert g_.shape == w_.shape
         assert np.max(np.abs(g_ - w_)) <= 2e-6 * max(1.0, np.max(np.abs(w_)))
+
+
+SAS_CASES = [
+    # x shape, window, strides, padding
+    ([2, 3, 8, 8], [1, 1, 2, 2], [1, 1, 2, 2], None),
+    ([2, 3, 9, 11], [1, 1, 3, 3], [1, 1, 2, 2], [[0, 0], [0, 0], [1, 1], [1, 1]]),
+    ([1, 2, 7, 7], [1, 1, 3, 3], [1, 1, 1, 1], None),                              # overlapping windows
+    ([3, 1, 10, 6], [1, 1, 2, 3], [1, 1, 2, 3], [[0, 0], [0, 0], [1, 1], [0, 0]]),
+]
+
+
+@pytest.mark.parametrize("xs,w,st,pd", SAS_CASES)
+def test_select_and_scatter_is_the_gradient_of_max_pooling(xs, w, st, pd):
+    """The oracle's select_and_scatter (GE select, add scatter) against torch's max_pool2d backward, a
+    library routine; ties are rare in random data, the tie rule is pinned below."""
+    import torch
+    rng = np.random.default_rng(3)
+    text, ss = NN.select_and_scatter(xs, "f32", w, st, pd)
+    x, dy = rng.normal(size=xs).astype(np.float32), rng.normal(size=ss).astype(np.float32)
+    got = I.run_text(text, [I.tensor(x, "f32"), I.tensor(dy, "f32")])[0].a
+    xt = torch.tensor(x, requires_grad=True)
+    y = torch.nn.functional.max_pool2d(xt, kernel_size=(w[2], w[3]), stride=(st[2], st[3]), padding=(pd[2][0], pd[3][0]) if pd else 0)
+    assert list(y.shape) == ss
+    y.backward(torch.tensor(dy))
+    np.testing.assert_allclose(got, xt.grad.numpy(), rtol=0, atol=1e-6)
+
+
+def test_select_and_scatter_ties_and_padding():
+    """On a constant operand GE keeps the first element of a window (row-major) and GT moves on to the
+    last; elements of the padding are never selected; LE / LT select minima the same way."""
+    x = np.ones((1, 1, 4, 4), np.float32)
+    dy = np.arange(1, 5, dtype=np.float32).reshape(1, 1, 2, 2)
+    for direction, corner in (("GE", (0, 0)), ("GT", (1, 1)), ("LE", (0, 0)), ("LT", (1, 1))):
+        text, ss = NN.select_and_scatter([1, 1, 4, 4], "f32", [1, 1, 2, 2], [1, 1, 2, 2], None, direction=direction)
+        got = I.run_text(text, [I.tensor(x, "f32"), I.tensor(dy, "f32")])[0].a[0, 0]
+        want = np.zeros((4, 4), np.float32)
+        for i in range(2):
+            for j in range(2):
+                want[2 * i + corner[0], 2 * j + corner[1]] = dy[0, 0, i, j]
+        assert np.array_equal(got, want), direction
+    # one row of padding above and below: windows (rows -1..0) and (rows 3..4) select inside the operand
+    text, ss = NN.select_and_scatter([1, 1, 4, 2], "f32", [1, 1, 2, 2], [1, 1, 2, 2], [[0, 0], [0, 0], [1, 1], [0, 0]])
+    assert ss == [1, 1, 3, 1]
+    x = -np.arange(8, dtype=np.float32).reshape(1, 1, 4, 2) - 100.0            # all far below zero
+    got = I.run_text(text, [I.tensor(x, "f32"), I.tensor(np.array([1, 10, 100], np.float32).reshape(1, 1, 3, 1), "f32")])[0].a[0, 0]
+    assert np.array_equal(got, np.array([[1, 0], [10, 0], [0, 0], [100, 0]], np.float32))
