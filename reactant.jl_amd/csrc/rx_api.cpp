@@ -230,6 +230,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_CHAIN_STEPS")) o.chain_steps = atoi(e);
   if (const char* e = getenv("RX_CHAIN_TILE")) { int v[3] = {0, 0, 0}; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) >= 1) { o.chain_tile[0] = v[0]; o.chain_tile[1] = v[1]; o.chain_tile[2] = v[2]; } }
   if (const char* e = getenv("RX_CHAIN_MAX_RANK")) o.chain_max_rank = atoi(e);
+  if (const char* e = getenv("RX_CHAIN_FIXED")) o.chain_fixed_cells = atoi(e) != 0;
   if (const char* e = getenv("RX_CHAIN_THREADS")) o.chain_threads = atoi(e);
   if (const char* e = getenv("RX_CHAIN_LDS_BYTES")) o.chain_lds_bytes = atoll(e);
   if (const char* e = getenv("RX_CHAIN_REDUNDANCY")) o.chain_redundancy = atof(e);

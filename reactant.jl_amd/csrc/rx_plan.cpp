@@ -1886,7 +1886,10 @@ struct Planner {
     const std::string st = info(n0.ty.dt).stype;
     int64_t T[3] = {1, 1, 1};
     {
-      const int64_t dflt[3][3] = {{256, 1, 1}, {32, 64, 1}, {8, 8, 32}};
+      // vectors: one cell per thread (a step costs an LDS round trip and a barrier, whatever the tile);
+      // matrices: 32x64 tiles, 32x32 when that is what it takes to give every compute unit a tile
+      int64_t dflt[3][3] = {{128, 1, 1}, {32, 64, 1}, {8, 8, 32}};
+      if (r == 2 && ((D[0] + 31) / 32) * ((D[1] + 63) / 64) < 256) dflt[1][1] = 32;
       for (int d = 0; d < r; ++d) {
         T[d] = opt.chain_tile[d] > 0 && opt.chain_tile[r - 1] > 0 ? opt.chain_tile[d] : dflt[r - 1][d];
         T[d] = std::min<int64_t>(T[d], D[d]);
@@ -1914,7 +1917,7 @@ struct Planner {
       for (int d = 0; d < r; ++d) { E[d] = T[d] + HL[d] + HH[d]; box *= E[d]; tile *= T[d]; }
       const int64_t lds_bytes = box * nf * es;
       if (lds_bytes > opt.chain_lds_bytes || (double)box > opt.chain_redundancy * (double)tile) continue;
-      const int NB = opt.chain_threads > 0 ? opt.chain_threads : box >= 4096 ? 1024 : box >= 1024 ? 512 : 256;
+      const int NB = opt.chain_threads > 0 ? opt.chain_threads : (int)std::min<int64_t>(1024, (box + 63) / 64 * 64);
       if (NB < 64 || NB > 1024 || NB % 64) continue;
 
       // the steps' bodies, evaluated at the array position (g0, g1, g2) whose cell in the box is `li`
@@ -1926,6 +1929,7 @@ struct Planner {
       }
       std::vector<int> inputs, cur = entry, writes(k);
       std::vector<std::string> bodies(k), vals(k);
+      int64_t margin = 0;   // farthest neighbour read, in cells: the tiles sit that far inside the LDS allocation
       std::set<int> group(steps.begin(), steps.begin() + k);
       bool ok = true;
       for (size_t i = 0; i < k && ok; ++i) {
@@ -1943,6 +1947,7 @@ struct Planner {
           if (cur[f->second] != node) { ok = false; return false; }
           int64_t delta = 0, stride = 1;
           for (int d = r - 1; d >= 0; --d) { delta += off[d] * stride; stride *= E[d]; }
+          margin = std::max<int64_t>(margin, delta < 0 ? -delta : delta);
           *expr = "lds" + std::to_string(f->second) + "[li + (" + std::to_string(delta) + ")]";
           return true;
         };
@@ -1981,7 +1986,7 @@ struct Planner {
         return -1;
       };
       o << "  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];\n";
-      for (int f = 0; f < nf; ++f) o << "  " << st << "* const lds" << f << " = reinterpret_cast<" << st << "*>(rx_smem) + " << f * box << ";\n";
+      for (int f = 0; f < nf; ++f) o << "  " << st << "* const lds" << f << " = reinterpret_cast<" << st << "*>(rx_smem) + " << margin + f * box << ";\n";
       int64_t nt[3] = {1, 1, 1}, ntiles = 1;
       for (int d = 0; d < r; ++d) { nt[d] = (D[d] + T[d] - 1) / T[d]; ntiles *= nt[d]; }
       o << "  int tb = blockIdx.x;\n";
@@ -1989,6 +1994,9 @@ struct Planner {
         o << "  const int t" << d << " = (tb % " << nt[d] << ") * " << T[d] << ";\n";
         if (d) o << "  tb /= " << nt[d] << ";\n";
       }
+      const int64_t R = (box + NB - 1) / NB;   // box cells per thread
+      const bool fixed = R <= 8 && opt.chain_fixed_cells;
+      if (!fixed) {
       // Loops over the cells of a region run a fixed number of rounds per thread without branches
       // (cells past the end repeat the last one, array positions are clamped into the array, and
       // only the final LDS or global store is predicated), so that the compiler can keep the loads
@@ -2055,13 +2063,82 @@ struct Planner {
         for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = lds" << f << "[li];\n";
         o << "    }\n  }\n}\n\n";
       }
+      } else {
+        // Every thread owns the box cells p = threadIdx.x + q * NB for the whole kernel: their array
+        // coordinates are worked out once and kept in registers, a step only tests whether a cell lies
+        // in its region, and a cell's index in an LDS tile is p itself.  Rounds that cannot meet a
+        // step's region are left out when the text is written.  Nothing branches inside a round (only
+        // the final store is predicated), so the loads of several rounds stay in flight.
+        auto array_index = [&]() {
+          std::string e;
+          for (int d = 0; d < r; ++d) e = d ? "(" + e + ") * " + std::to_string(D[d]) + " + g" + std::to_string(d) : "g0";
+          return e;
+        };
+        for (int d = 0; d < r; ++d) o << "  int C" << d << "[" << R << "], G" << d << "[" << R << "];\n";
+        o << "  bool IN[" << R << "];\n";
+        o << "#pragma unroll\n  for (int q = 0; q < " << R << "; ++q) {\n";
+        o << "    const int p = threadIdx.x + q * " << NB << ";\n    int rr = rx_min(p, " << box - 1 << ");\n";
+        for (int d = r - 1; d >= 0; --d) {
+          if (d) o << "    const int c" << d << " = rr % " << E[d] << ";\n    rr /= " << E[d] << ";\n";
+          else o << "    const int c0 = rr;\n";
+        }
+        std::string in_arr = "p < " + std::to_string(box);
+        for (int d = 0; d < r; ++d) {
+          o << "    const int a" << d << " = t" << d << " - " << HL[d] << " + c" << d << ";\n";
+          o << "    const int g" << d << " = rx_clamp_idx<int>(a" << d << ", " << D[d] - 1 << ");\n";
+          o << "    C" << d << "[q] = c" << d << "; G" << d << "[q] = g" << d << ";\n";
+          in_arr += " && a" + std::to_string(d) + " == g" + std::to_string(d);
+        }
+        o << "    IN[q] = " << in_arr << ";\n";
+        o << "    const int lin = " << array_index() << ";\n";
+        for (int f = 0; f < nf; ++f) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
+        o << "    if (p < " << box << ") {\n";
+        for (int f = 0; f < nf; ++f) o << "      lds" << f << "[p] = s" << f << ";\n";
+        o << "    }\n  }\n  __syncthreads();\n";
+        const int64_t plane = box / E[0];
+        auto rounds_of = [&](int64_t r0, int64_t r1, int64_t* qlo, int64_t* qhi) {   // rounds that hold cells of box rows [r0, r1)
+          *qlo = r0 * plane / NB;
+          *qhi = std::min<int64_t>(R, (r1 * plane + NB - 1) / NB);
+        };
+        auto open_round = [&](const int64_t* first, const int64_t* ext) {
+          int64_t qlo, qhi;
+          rounds_of(first[0], first[0] + ext[0], &qlo, &qhi);
+          o << "#pragma unroll\n  for (int q = " << qlo << "; q < " << qhi << "; ++q) {\n";
+          o << "    const int li = rx_min((int)threadIdx.x + q * " << NB << ", " << box - 1 << ");\n";
+          std::string live = "IN[q]";
+          for (int d = 0; d < r; ++d) {
+            o << "    const int g" << d << " = G" << d << "[q];\n";
+            live += " && (unsigned)(C" + std::to_string(d) + "[q] - " + std::to_string(first[d]) + ") < " + std::to_string(ext[d]) + "u";
+          }
+          o << "    const bool live = " << live << ";\n";
+        };
+        for (size_t i = 0; i < k; ++i) {
+          int64_t first[3] = {0, 0, 0}, ext[3] = {1, 1, 1};
+          for (int d = 0; d < r; ++d) {
+            int64_t back = 0, fwd = 0;
+            for (size_t j = i + 1; j < k; ++j) { back += lo[j][d]; fwd += hi[j][d]; }
+            first[d] = HL[d] - back;
+            ext[d] = T[d] + back + fwd;
+          }
+          o << "  // step " << i << ": " << describe(steps[i]) << "\n";
+          open_round(first, ext);
+          o << "    {\n" << bodies[i];
+          o << "      if (live) lds" << writes[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
+        }
+        {
+          open_round(HL, T);
+          o << "    if (live) {\n      const int lin = " << array_index() << ";\n";
+          for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = lds" << f << "[li];\n";
+          o << "    }\n  }\n}\n\n";
+        }
+      }
       const std::string kb_final = finalize(o.str());
       Launch L;
       L.kernel = named(kname, kb_final);
       L.kind = "map_chain";
       L.grid[0] = (unsigned)ntiles;
       L.block[0] = NB;
-      L.lds_bytes = (unsigned)lds_bytes;
+      L.lds_bytes = (unsigned)(lds_bytes + 2 * margin * es);
       for (int a : arg_nodes) L.args.push_back(buffer_for(a));
       std::vector<int> outs;
       for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) { L.args.push_back(buffer_for(cur[f])); outs.push_back(cur[f]); }

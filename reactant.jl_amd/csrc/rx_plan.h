@@ -69,8 +69,9 @@ struct PlanOptions {
   int chain_tile[3] = {0, 0, 0};     // outputs per workgroup (slowest .. fastest dimension of the array's rank; zeros: default per rank)
   int64_t chain_lds_bytes = 64 * 1024;  // LDS a workgroup may use for the tiles
   int chain_max_rank = 2;            // rank-3 steps are bound by index arithmetic in such a kernel, not by launches: left as maps
+  bool chain_fixed_cells = true;     // a thread keeps the same box cells (and their coordinates in registers) through all steps
   int chain_threads = 0;             // workgroup size (0: by the number of staged cells)
-  double chain_redundancy = 3.0;     // largest ratio of staged cells (tile plus halo) to tile cells
+  double chain_redundancy = 4.1;     // largest ratio of staged cells (tile plus halo) to tile cells
   bool in_place_updates = true;   // dynamic_update_slice over a temporary nobody reads later writes only its box, into the operand's buffer
   bool shifted_vector_loads = true;  // loads at constant offsets become aligned vector loads of neighbouring vectors
   bool excess_precision = true; // narrow-float arithmetic stays in f32 inside a kernel (rounded at stores and converts)

@@ -267,7 +267,7 @@ def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
     k = kinds(rx.compile_offline(PB.build("jacobi_1d")))            # 2048 half steps, 64 per launch
     assert k == ["map_chain"] * 32
     rep = rx.compile_offline(PB.build("jacobi_2d"), with_source=True)
-    assert kinds(rep) == ["map_chain"] * 128 and "16 update steps through LDS tiles (32x64 outputs per workgroup, box 64x96, 2 fields)" in rep
+    assert kinds(rep) == ["map_chain"] * 128 and "16 update steps through LDS tiles (32x32 outputs per workgroup, box 64x64, 2 fields)" in rep
     k = kinds(rx.compile_offline(PB.build("fdtd_2d", tmax=32)))      # the last launch fuses the updates nobody returns
     assert k.count("map_chain") == len(k) - 1 and len(k) <= 8
     # rank 3: one launch per step; once the arrays are temporaries each step writes only its box, in place
