@@ -1116,7 +1116,7 @@ struct Builder {
   // variable compared with a constant); each time it is true the body region is replayed.  This
   // is the form `@trace for` loops take (reference src/Ops.jl:2349-2460); loops whose trip count
   // depends on data are rejected.
-  static constexpr int kMaxTrip = 4096;
+  static constexpr int kMaxTrip = 65536;
   std::map<int, std::pair<bool, int64_t>> folded;
 
   static bool is_int_dt(DT t) { return !is_float(t) && t != DT::INVALID; }

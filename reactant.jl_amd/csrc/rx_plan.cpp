@@ -17,7 +17,9 @@
 
 #include <algorithm>
 #include <array>
+#include <chrono>
 #include <cmath>
+#include <cstdio>
 #include <set>
 #include <sstream>
 
@@ -3264,19 +3266,32 @@ struct Planner {
   }
 
   // Row reductions that can run inside the kernel of `root` (see header comment).
+  // All calls come after the analysis has settled, so the answers are kept; the reductions of the
+  // module are listed once (a time loop unrolls into thousands of roots and no reduction at all).
+  std::map<int, std::vector<int>> row_phase_cache;
+  std::vector<int> row_reduces;
+  bool row_reduces_listed = false;
   std::vector<int> row_phases(int root) {
+    auto hit = row_phase_cache.find(root);
+    if (hit != row_phase_cache.end()) return hit->second;
+    return row_phase_cache[root] = row_phases_uncached(root);
+  }
+  std::vector<int> row_phases_uncached(int root) {
     const Node& rn = g.nodes[root];
     std::vector<int> phases;
     if (!opt.row_fusion || rn.ty.rank() < 2) return phases;
+    if (!row_reduces_listed) {
+      row_reduces_listed = true;
+      for (int x = 0; x < (int)g.nodes.size(); ++x)
+        if (live[x] && g.nodes[x].k == OpK::Reduce && std::find(g.results.begin(), g.results.end(), x) == g.results.end()) row_reduces.push_back(x);
+    }
     std::set<int> S{root};
     bool changed = true;
     while (changed) {
       changed = false;
-      for (int x = 0; x < (int)g.nodes.size(); ++x) {
-        if (!live[x] || S.count(x)) continue;
+      for (int x : row_reduces) {
+        if (S.count(x)) continue;
         const Node& r = g.nodes[x];
-        if (r.k != OpK::Reduce) continue;
-        if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
         const TType& in = g.nodes[r.in[0]].ty;
         if (in.dims != rn.ty.dims) continue;
         RedShape rs = red_shape(r);
@@ -3530,8 +3545,18 @@ struct Planner {
 
   // ------------------------------------------------------------------ driver
   void run() {
+    const bool timing = getenv("RX_PLAN_TIMING") != nullptr;
+    auto t_prev = std::chrono::steady_clock::now();
+    auto lap = [&](const char* what) {
+      if (!timing) return;
+      auto t = std::chrono::steady_clock::now();
+      fprintf(stderr, "[plan] %s: %.3f s\n", what, std::chrono::duration<double>(t - t_prev).count());
+      t_prev = t;
+    };
     canonicalize();
+    lap("canonicalize");
     decide_fused_operands();
+    lap("decide_fused_operands");
     const int N = (int)g.nodes.size();
     // Decisions about a node depend on which of its producers own buffers; sweep until stable.
     prev_mat.assign(N, 0);
@@ -3540,6 +3565,7 @@ struct Planner {
       if (mat == prev_mat) break;
       prev_mat = mat;
     }
+    lap("analysis sweeps");
     buf_of.assign(N, -1);
     plan.aliasing_output = g.aliasing_output;
     for (int p : g.params) { plan.param_types.push_back(g.nodes[p].ty); buffer_for(p); }
@@ -3591,6 +3617,7 @@ struct Planner {
       }
     }
 
+    lap("epilogues and aliases");
     // kernels in topological order of their roots
     std::vector<std::pair<int, std::function<void()>>> jobs;
     for (int x = 0; x < N; ++x) {
@@ -3728,7 +3755,9 @@ struct Planner {
       if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::Scatter && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
         for (int p : row_phases(j.first)) fused_reduces.insert(p);
     }
+    lap("job list, chains");
     for (auto& j : jobs) j.second();
+    lap("emit");
 
     for (int r : g.results) {
       plan.result_types.push_back(g.nodes[r].ty);

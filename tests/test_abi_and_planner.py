@@ -276,3 +276,17 @@ def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
     assert kinds(rx.compile_offline(PB.build("jacobi_1d", tsteps=16))) == ["map"] * 2 + ["map_in_place"] * 30
     monkeypatch.setenv("RX_IN_PLACE", "0")
     assert kinds(rx.compile_offline(PB.build("jacobi_1d", tsteps=16))) == ["map"] * 32
+
+
+def test_long_time_loops_import_and_plan_in_linear_time():
+    """8192 trips of a two-step loop body (16384 update steps): import, planning and compilation stay
+    linear in the trip count (a few seconds); more than 65536 trips are refused with a message."""
+    import importlib
+    import time
+    PB = importlib.import_module("reactant_jl_amd.polybench_programs")
+    t0 = time.time()
+    rep = rx.compile_offline(PB.build("jacobi_2d", tsteps=8192))
+    assert "launches: 1024" in rep
+    assert time.time() - t0 < 60
+    with pytest.raises(Exception, match="more than 65536 iterations"):
+        rx.compile_offline(PB.build("jacobi_1d", n=64, tsteps=70000))
