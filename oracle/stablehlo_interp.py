@@ -48,6 +48,8 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       seven operations, four shapes), numpy indexed assignment and np.add.at; dropped
       out-of-range updates (whole windows, as XLA does; the StableHLO text says per element:
       PARITY UNPINNED between the two readings, the reference holds no case that tells them apart)
+  chlo unary math ops, popcnt, count_leading_zeros (src/Ops.jl:398-436) ... scipy / numpy routines, checked
+      against inverse pairs, recurrences and values the mathematics fixes (tests/test_oracle_golden.py)
   select_and_scatter (the gradient of pooling) ... torch's max_pool2d backward (a library routine) on
       padded, strided and overlapping windows; the tie rules (GE keeps the first element, GT the last)
       by a constant operand; the reference holds no known answer for it
@@ -363,7 +365,9 @@ class _Cursor:
 
 _UNARY = {"sine", "cosine", "tanh", "exponential", "log", "sqrt", "rsqrt", "abs", "negate",
           "logistic", "floor", "ceil", "sign", "not", "exponential_minus_one", "log_plus_one",
-          "round_nearest_even", "round_nearest_afz", "cbrt", "tan", "is_finite"}
+          "round_nearest_even", "round_nearest_afz", "cbrt", "tan", "is_finite", "popcnt", "count_leading_zeros"}
+_CHLO_UNARY = {"chlo.erf", "chlo.erfc", "chlo.acos", "chlo.acosh", "chlo.asin", "chlo.asinh", "chlo.atan", "chlo.atanh", "chlo.cosh",
+               "chlo.sinh", "chlo.lgamma", "chlo.digamma", "chlo.erf_inv", "chlo.is_inf", "chlo.is_pos_inf", "chlo.is_neg_inf"}
 _BINARY = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "remainder",
            "and", "or", "xor", "atan2", "shift_left", "shift_right_logical",
            "shift_right_arithmetic"}
@@ -1067,6 +1071,15 @@ def _unary(name, x, dt):
             elif name == "round_nearest_afz": r = np.trunc(w + np.copysign(0.5, w))
             elif name == "is_finite": return Tensor(np.isfinite(w), "i1")
             elif name == "chlo.erf": r = _erf(w.astype(np.float64)).astype(w.dtype)
+            elif name in ("chlo.is_inf", "chlo.is_pos_inf", "chlo.is_neg_inf"):
+                return Tensor(np.isinf(w) & ((w > 0) if name == "chlo.is_pos_inf" else (w < 0) if name == "chlo.is_neg_inf" else True), "i1")
+            elif name in _CHLO_UNARY:
+                # the chlo math ops of reference src/Ops.jl:398-436, by numpy / scipy.special in float64
+                import scipy.special as sp
+                f = {"chlo.erfc": sp.erfc, "chlo.acos": np.arccos, "chlo.acosh": np.arccosh, "chlo.asin": np.arcsin, "chlo.asinh": np.arcsinh,
+                     "chlo.atan": np.arctan, "chlo.atanh": np.arctanh, "chlo.cosh": np.cosh, "chlo.sinh": np.sinh, "chlo.lgamma": sp.gammaln,
+                     "chlo.digamma": sp.digamma, "chlo.erf_inv": sp.erfinv}[name]
+                r = f(w.astype(np.float64)).astype(w.dtype)
             else: raise NotImplementedError(name)
         return tensor(r, dt)
     if name == "not":
@@ -1077,6 +1090,13 @@ def _unary(name, x, dt):
         return Tensor((-a.astype(np.int64)).astype(a.dtype) if dt != "i1" else a, dt)
     if name == "sign":
         return Tensor(np.sign(a).astype(a.dtype), dt)
+    if name == "popcnt":
+        # of the two's-complement bit pattern (numpy counts the bits of |a| for signed types)
+        return Tensor(np.bitwise_count(a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])).astype(a.dtype), dt)
+    if name == "count_leading_zeros":
+        bits = 8 * a.dtype.itemsize
+        u = a.astype({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize]).astype(object)
+        return Tensor(np.array([bits - int(v).bit_length() for v in u.reshape(-1)], dtype=a.dtype).reshape(a.shape), dt)
     raise NotImplementedError("%s on %s" % (name, dt))
 
 
@@ -1656,8 +1676,9 @@ class Interpreter:
         if n == "constant":
             t = op.types_out[0]
             return [Tensor(at["value"], t.dt)]
-        if n in _UNARY or n == "chlo.erf":
-            return [_unary(n, xs[0], op.types_out[0].dt if n != "is_finite" else xs[0].dt)]
+        if n in _UNARY or n in _CHLO_UNARY:
+            classify = n in ("is_finite", "chlo.is_inf", "chlo.is_pos_inf", "chlo.is_neg_inf")     # float in, i1 out
+            return [_unary(n, xs[0], xs[0].dt if classify else op.types_out[0].dt)]
         if n in _BINARY:
             return [_binary(n, xs[0], xs[1], op.types_out[0].dt)]
         if n == "convert":

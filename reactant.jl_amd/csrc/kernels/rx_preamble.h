@@ -253,6 +253,38 @@ RX_DEV T rx_readlane63(T v) {
   }
 }
 
+// digamma: reflection below zero, the recurrence psi(x) = psi(x + 1) - 1 / x up to x >= 10, then the
+// asymptotic series; carried in double (poles at the non-positive integers give NaN)
+template <typename T>
+RX_DEV T rx_digamma(T xin) {
+  double x = (double)xin, r = 0.0;
+  if (x <= 0.0 && floor(x) == x) return (T)__builtin_nan("");
+  if (x < 0.0) {
+    r = -3.14159265358979323846 / tan(3.14159265358979323846 * x);
+    x = 1.0 - x;
+  }
+  while (x < 10.0) { r -= 1.0 / x; x += 1.0; }
+  const double f = 1.0 / (x * x);
+  r += log(x) - 0.5 / x -
+       f * (1.0 / 12.0 - f * (1.0 / 120.0 - f * (1.0 / 252.0 - f * (1.0 / 240.0 - f * (1.0 / 132.0 - f * (691.0 / 32760.0 - f * (1.0 / 12.0)))))));
+  return (T)r;
+}
+// bits set / leading zero bits of an integer of any width (the value's own width counts)
+template <typename T>
+RX_DEV int rx_popcnt(T v) {
+  if constexpr (sizeof(T) == 8) return __popcll((unsigned long long)v);
+  else if constexpr (sizeof(T) == 4) return __popc((unsigned)v);
+  else if constexpr (sizeof(T) == 2) return __popc((unsigned)(unsigned short)v);
+  else return __popc((unsigned)(unsigned char)v);
+}
+template <typename T>
+RX_DEV int rx_clz(T v) {
+  if constexpr (sizeof(T) == 8) return v == 0 ? 64 : __clzll((long long)v);
+  else if constexpr (sizeof(T) == 4) return v == 0 ? 32 : __clz((int)v);
+  else if constexpr (sizeof(T) == 2) return (unsigned short)v == 0 ? 16 : __clz((int)(unsigned)(unsigned short)v) - 16;
+  else return (unsigned char)v == 0 ? 8 : __clz((int)(unsigned)(unsigned char)v) - 24;
+}
+
 struct rx_op_add { template <typename T> RX_MEM T operator()(T a, T b) const { return a + b; } };
 struct rx_op_mul { template <typename T> RX_MEM T operator()(T a, T b) const { return a * b; } };
 struct rx_op_div { template <typename T> RX_MEM T operator()(T a, T b) const { return a / b; } };

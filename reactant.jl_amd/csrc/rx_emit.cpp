@@ -288,7 +288,14 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       std::string x = opnd(0);
       const std::string& op = n.op;
       if (op == "is_finite") return def("isfinite(" + x + ")");
+      if (op == "is_inf") return def("isinf(" + x + ")");
+      if (op == "is_pos_inf") return def("(isinf(" + x + ") && " + x + " > 0)");
+      if (op == "is_neg_inf") return def("(isinf(" + x + ") && " + x + " < 0)");
       if (is_float(dt)) {
+        for (const char* m : {"acos", "acosh", "asin", "asinh", "atan", "atanh", "cosh", "sinh", "erfc", "lgamma"})
+          if (op == m) return def(fn(m, dbl) + "(" + x + ")");
+        if (op == "erf_inv") return def(fn("erfinv", dbl) + "(" + x + ")");
+        if (op == "digamma") return def("rx_digamma(" + x + ")");
         if (op == "sine") return def(fn("sin", dbl) + "(" + x + ")");
         if (op == "cosine") return def(fn("cos", dbl) + "(" + x + ")");
         if (op == "tan") return def(fn("tan", dbl) + "(" + x + ")");
@@ -317,6 +324,8 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (op == "negate") return def("(" + CT + ")(0 - " + x + ")");
         if (op == "abs") return info(dt).is_signed ? def("(" + CT + ")(" + x + " < 0 ? 0 - " + x + " : " + x + ")") : x;
         if (op == "sign") return def("(" + CT + ")((" + x + " > 0) - (" + x + " < 0))");
+        if (op == "popcnt") return def("(" + CT + ")rx_popcnt(" + x + ")");
+        if (op == "count_leading_zeros") return def("(" + CT + ")rx_clz(" + x + ")");
       }
       (void)sdt;
       throw Error("unsupported unary op '" + op + "' on " + info(dt).mlir);

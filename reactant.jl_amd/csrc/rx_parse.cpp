@@ -340,7 +340,10 @@ struct RawFunc {
 
 const char* kUnary[] = {"sine", "cosine", "tanh", "exponential", "log", "sqrt", "rsqrt", "abs", "negate", "logistic",
                         "floor", "ceil", "sign", "not", "exponential_minus_one", "log_plus_one", "round_nearest_even",
-                        "round_nearest_afz", "cbrt", "tan", "is_finite", nullptr};
+                        "round_nearest_afz", "cbrt", "tan", "is_finite", "popcnt", "count_leading_zeros", nullptr};
+// the `chlo` unary ops of reference src/Ops.jl:398-436,618-640 (evaluated by the device math library)
+const char* kChloUnary[] = {"chlo.erf", "chlo.erfc", "chlo.acos", "chlo.acosh", "chlo.asin", "chlo.asinh", "chlo.atan", "chlo.atanh", "chlo.cosh",
+                            "chlo.sinh", "chlo.lgamma", "chlo.digamma", "chlo.erf_inv", "chlo.is_inf", "chlo.is_pos_inf", "chlo.is_neg_inf", nullptr};
 const char* kBinary[] = {"add", "subtract", "multiply", "divide", "maximum", "minimum", "power", "remainder", "and", "or",
                          "xor", "atan2", "shift_left", "shift_right_logical", "shift_right_arithmetic", nullptr};
 bool in_list(const char** l, const std::string& s) {
@@ -2099,12 +2102,13 @@ struct Builder {
       fill_constant(n, o.dense, [&](const std::string& m) { fail("constant: " + m); });
       return {g.add(n)};
     }
-    if (in_list(kUnary, sh) || sh == "chlo.erf" || sh == "chlo.erfc" ) {
+    if (in_list(kUnary, sh) || in_list(kChloUnary, sh)) {
       need(1);
       n.k = OpK::Unary;
-      n.op = sh == "chlo.erf" ? "erf" : sh;
+      n.op = sh.rfind("chlo.", 0) == 0 ? sh.substr(5) : sh;
       n.ty = out1();
-      if (sh == "is_finite") n.ty.dt = DT::I1;
+      if (sh == "is_finite" || sh == "chlo.is_inf" || sh == "chlo.is_pos_inf" || sh == "chlo.is_neg_inf") n.ty.dt = DT::I1;
+      if (in_list(kChloUnary, sh) && !is_float(ty(in[0]).dt)) fail(o.name + ": a float operand is expected");
       if (n.ty.dims != ty(in[0]).dims) fail(o.name + ": shape mismatch");
       return {g.add(n)};
     }

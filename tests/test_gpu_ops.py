@@ -490,3 +490,59 @@ def test_conditionals(rx, client):
     got, exe = gpu_run(rx, client, W.IF_CONST, [x])
     assert rel_err(got[0].a, np.cos(x.a)) <= 1e-6
     assert "select" not in exe.report() and ":: cosine" in exe.report()
+
+
+CHLO_UNARY = {   # op -> range of the sweep
+    "acos": (-0.99, 0.99), "asin": (-0.99, 0.99), "atan": (-20.0, 20.0), "acosh": (1.01, 50.0), "asinh": (-50.0, 50.0),
+    "atanh": (-0.99, 0.99), "cosh": (-8.0, 8.0), "sinh": (-8.0, 8.0), "erfc": (-3.0, 3.0), "lgamma": (2.5, 30.0),
+    "digamma": (0.1, 30.0), "erf_inv": (-0.999, 0.999), "erf": (-3.0, 3.0),
+}
+
+
+@pytest.mark.parametrize("op", sorted(CHLO_UNARY))
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_chlo_unary_maps(rx, client, op, dt):
+    """The `chlo` math ops of reference src/Ops.jl:398-436 against scipy / numpy in float64: 1e-6 relative for
+    f32 (5e-6 for digamma near its zero), 1e-12 for f64."""
+    lo, hi = CHLO_UNARY[op]
+    x = np.random.default_rng(5).uniform(lo, hi, 4096).astype(I.NP_OF[dt])
+    t = _tt(x.shape, dt)
+    text = mod([t], t, "    %%0 = chlo.%s %%arg0 : %s -> %s\n    return %%0 : %s\n" % (op, t, t, t))
+    got, _ = gpu_run(rx, client, text, [I.Tensor(x, dt)])
+    ref64 = oracle_run(text.replace(dt, "f64"), [I.Tensor(x.astype(np.float64), "f64")])[0].a
+    diff = np.abs(got[0].a.astype(np.float64) - ref64)
+    rel = (5e-6 if op == "digamma" else 1e-6) if dt == "f32" else 1e-12
+    assert ((diff <= rel * np.maximum(np.abs(ref64), 1e-30)) | (diff <= rel)).all(), (op, float((diff / np.maximum(np.abs(ref64), 1e-30)).max()))
+
+
+def test_digamma_below_zero_and_classification_ops(rx, client):
+    x = np.array([-2.5, -0.5, -1.25, -7.75, 0.25], np.float64)
+    t = _tt(x.shape, "f64")
+    text = mod([t], t, "    %%0 = chlo.digamma %%arg0 : %s -> %s\n    return %%0 : %s\n" % (t, t, t))
+    got, ref = both(rx, client, text, [I.Tensor(x, "f64")])
+    assert np.allclose(got[0].a, ref[0].a, rtol=1e-11)
+    y = np.array([1.0, np.inf, -np.inf, np.nan, 0.0], np.float32)
+    t, tb = _tt(y.shape, "f32"), _tt(y.shape, "i1")
+    for op, want in (("is_inf", [0, 1, 1, 0, 0]), ("is_pos_inf", [0, 1, 0, 0, 0]), ("is_neg_inf", [0, 0, 1, 0, 0])):
+        text = mod([t], tb, "    %%0 = chlo.%s %%arg0 : %s -> %s\n    return %%0 : %s\n" % (op, t, tb, tb))
+        got, ref = both(rx, client, text, [I.Tensor(y, "f32")])
+        assert got[0].a.astype(int).tolist() == want == ref[0].a.astype(int).tolist()
+
+
+@pytest.mark.parametrize("dt", ["i8", "ui16", "i32", "ui32", "i64"])
+def test_popcnt_and_count_leading_zeros(rx, client, dt):
+    """stablehlo.popcnt / count_leading_zeros at the element's own width, bit for bit."""
+    npdt = I.NP_OF[dt]
+    bits = 8 * np.dtype(npdt).itemsize
+    rng = np.random.default_rng(9)
+    raw = rng.integers(0, 1 << 62, 3000, dtype=np.uint64) >> rng.integers(0, 62, 3000).astype(np.uint64)
+    x = np.concatenate([np.array([0, 1, (1 << bits) - 1, 1 << (bits - 1)], dtype=np.uint64), raw & np.uint64((1 << bits) - 1)]).astype(
+        {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[bits // 8]).view(npdt)
+    t = _tt(x.shape, dt)
+    for op in ("popcnt", "count_leading_zeros"):
+        text = mod([t], t, "    %%0 = stablehlo.%s %%arg0 : %s\n    return %%0 : %s\n" % (op, t, t))
+        got, ref = both(rx, client, text, [I.Tensor(x, dt)])
+        assert np.array_equal(got[0].a, ref[0].a), op
+    # known answers at this width
+    text = mod([t], t, "    %%0 = stablehlo.count_leading_zeros %%arg0 : %s\n    return %%0 : %s\n" % (t, t))
+    assert oracle_run(text, [I.Tensor(x, dt)])[0].a[:4].tolist() == [bits, bits - 1, 0, 0]

@@ -383,3 +383,29 @@ def test_conditionals_against_plain_python():
         got = I.run_text(W.CASE, [I.tensor(y, "f64"), I.Tensor(np.int32(idx), "i32")])[0].a
         assert np.allclose(got, want, rtol=1e-14)
     assert np.allclose(I.run_text(W.IF_CONST, [I.tensor(x, "f32")])[0].a, np.cos(x), rtol=1e-6)
+
+
+def test_chlo_math_ops_satisfy_their_identities():
+    """The oracle's chlo unary ops (scipy / numpy routines, reference src/Ops.jl:398-436) against what the
+    mathematics fixes: inverse pairs, the hyperbolic identity, digamma's recurrence and psi(1) = -gamma,
+    lgamma at the integers, erfc = 1 - erf; popcnt / count_leading_zeros on known values."""
+    import math
+    from oracle import stablehlo_interp as I
+
+    def run(op, x, dt="f64"):
+        t = "tensor<%dx%s>" % (len(x), dt)
+        text = "module {\n func.func @main(%%arg0: %s) -> %s {\n  %%0 = %s %%arg0 : %s%s\n  return %%0 : %s\n }\n}\n" % (
+            t, t, op, t, " -> " + t if op.startswith("chlo.") else "", t)
+        return I.run_text(text, [I.Tensor(np.asarray(x, dtype=I.NP_OF[dt]), dt)])[0].a
+
+    x = np.linspace(0.05, 0.95, 19)
+    assert np.allclose(np.cos(run("chlo.acos", x)), x) and np.allclose(np.sin(run("chlo.asin", x)), x) and np.allclose(np.tan(run("chlo.atan", x)), x)
+    assert np.allclose(np.cosh(run("chlo.acosh", 1 + x)), 1 + x) and np.allclose(np.sinh(run("chlo.asinh", x)), x) and np.allclose(np.tanh(run("chlo.atanh", x)), x)
+    assert np.allclose(run("chlo.cosh", x) ** 2 - run("chlo.sinh", x) ** 2, 1.0)
+    assert np.allclose(run("chlo.erf", run("chlo.erf_inv", x)), x) and np.allclose(run("chlo.erfc", x), 1 - run("chlo.erf", x))
+    assert np.allclose(run("chlo.lgamma", [1.0, 2.0, 5.0, 11.0]), [0.0, 0.0, math.log(24.0), math.log(3628800.0)])
+    assert np.allclose(run("chlo.digamma", [1.0]), [-0.5772156649015329])
+    assert np.allclose(run("chlo.digamma", x + 1) - run("chlo.digamma", x), 1 / x)
+    assert run("stablehlo.popcnt", [0, 1, 255, -1, 1 << 20], "i32").tolist() == [0, 1, 8, 32, 1]
+    assert run("stablehlo.count_leading_zeros", [0, 1, 255, -1, 1 << 20], "i32").tolist() == [32, 31, 24, 0, 11]
+    assert run("stablehlo.count_leading_zeros", [0, 1, 127, -1], "i8").tolist() == [8, 7, 1, 0]
