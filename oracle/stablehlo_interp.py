@@ -737,6 +737,15 @@ class Parser:
             c.expect(":")
             self.fn_type(op)
             return op
+        if short == "get_dimension_size":
+            op.operands.append(c.ssa())
+            c.expect(",")
+            c.expect("dim")
+            c.expect("=")
+            op.attrs["dimension"] = int(c.integer())
+            c.expect(":")
+            self.fn_type(op)
+            return op
         if short == "compare":
             op.attrs["direction"] = c.ident()
             c.expect(",")
@@ -1681,6 +1690,16 @@ class Interpreter:
             return [_unary(n, xs[0], xs[0].dt if classify else op.types_out[0].dt)]
         if n in _BINARY:
             return [_binary(n, xs[0], xs[1], op.types_out[0].dt)]
+        if n == "bitcast_convert":
+            # the same bits read as another type of the same width (src/Ops.jl bitcast_convert)
+            to = op.types_out[0].dt
+            src = np.ascontiguousarray(xs[0].a)
+            if src.dtype.itemsize != np.dtype(NP_OF[to]).itemsize or not xs[0].dt in NP_OF or xs[0].dt in ("bf16", "f16", "f8E4M3FN", "f8E5M2", "i1") or to in ("bf16", "f16", "f8E4M3FN", "f8E5M2", "i1"):
+                raise NotImplementedError("bitcast_convert between %s and %s" % (xs[0].dt, to))
+            return [Tensor(src.view(NP_OF[to]).copy(), to)]
+        if n == "get_dimension_size":
+            d = at["dimension"] if not isinstance(at["dimension"], list) else at["dimension"][0]
+            return [Tensor(np.array(xs[0].a.shape[d], dtype=NP_OF[op.types_out[0].dt]), op.types_out[0].dt)]
         if n == "convert":
             prev, _EXCESS[0] = _EXCESS[0], False
             try:

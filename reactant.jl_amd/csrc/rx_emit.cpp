@@ -288,6 +288,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       std::string x = opnd(0);
       const std::string& op = n.op;
       if (op == "is_finite") return def("isfinite(" + x + ")");
+      if (op == "bitcast") return sdt == dt ? x : def("__builtin_bit_cast(" + CT + ", " + x + ")");
       if (op == "is_inf") return def("isinf(" + x + ")");
       if (op == "is_pos_inf") return def("(isinf(" + x + ") && " + x + " > 0)");
       if (op == "is_neg_inf") return def("(isinf(" + x + ") && " + x + " < 0)");

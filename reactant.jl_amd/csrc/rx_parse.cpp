@@ -665,6 +665,17 @@ struct P {
       fn_type(o);
       return o;
     }
+    if (sh == "get_dimension_size") {
+      // %0 = stablehlo.get_dimension_size %arg0, dim = 1 : (tensor<..>) -> tensor<i32>
+      o.operands.push_back(c.ssa());
+      c.expect(",");
+      c.expect("dim");
+      c.expect("=");
+      o.ia["dimension"] = {c.integer()};
+      c.expect(":");
+      fn_type(o);
+      return o;
+    }
     if (sh == "while") {
       // %r:2 = stablehlo.while(%iterArg = %init0, %iterArg_0 = %init1) : t0, t1 [attributes {..}]
       //   cond { ... stablehlo.return %p : tensor<i1> } do { ... stablehlo.return %a, %b : t0, t1 }
@@ -2128,6 +2139,24 @@ struct Builder {
       check_same(ty(in[0]), ty(in[1]), o.name);
       check_same(n.ty, ty(in[0]), o.name);
       return {g.add(n)};
+    }
+    if (sh == "bitcast_convert") {
+      // the same bits as another type of the same width (32- and 64-bit types, 8/16-bit integers)
+      need(1);
+      n.k = OpK::Unary;
+      n.op = "bitcast";
+      n.ty = out1();
+      const DT s_ = ty(in[0]).dt, d_ = n.ty.dt;
+      if (n.ty.dims != ty(in[0]).dims || info(s_).size != info(d_).size || is_narrow_float(s_) || is_narrow_float(d_) || s_ == DT::I1 || d_ == DT::I1)
+        fail("bitcast_convert: only between types of one width (no 8/16-bit floats, no i1)");
+      return {g.add(n)};
+    }
+    if (sh == "get_dimension_size") {
+      need(1);
+      if (!o.ia.count("dimension") || o.ia.at("dimension").empty()) fail("get_dimension_size: dimension missing");
+      const int64_t d_ = o.ia.at("dimension")[0];
+      if (d_ < 0 || d_ >= ty(in[0]).rank()) fail("get_dimension_size: dimension out of range");
+      return {splat_of(out1(), (double)ty(in[0]).dims[d_])};
     }
     if (sh == "convert") {
       need(1);

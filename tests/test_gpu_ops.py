@@ -546,3 +546,22 @@ def test_popcnt_and_count_leading_zeros(rx, client, dt):
     # known answers at this width
     text = mod([t], t, "    %%0 = stablehlo.count_leading_zeros %%arg0 : %s\n    return %%0 : %s\n" % (t, t))
     assert oracle_run(text, [I.Tensor(x, dt)])[0].a[:4].tolist() == [bits, bits - 1, 0, 0]
+
+
+def test_bitcast_convert_and_get_dimension_size(rx, client):
+    """bitcast_convert between types of one width (known bit patterns: 1.0f = 0x3F800000, -2.0 = 0xC000...), and
+    get_dimension_size, which folds to a constant."""
+    x = np.array([1.0, -2.0, 0.0, np.inf, 1e-45], np.float32)
+    t, ti = _tt(x.shape, "f32"), _tt(x.shape, "ui32")
+    text = mod([t], ti, "    %%0 = stablehlo.bitcast_convert %%arg0 : (%s) -> %s\n    return %%0 : %s\n" % (t, ti, ti))
+    got, ref = both(rx, client, text, [I.Tensor(x, "f32")])
+    assert got[0].a.tolist() == [0x3F800000, 0xC0000000, 0, 0x7F800000, 1] == ref[0].a.tolist()
+    y = np.random.default_rng(2).integers(-2 ** 62, 2 ** 62, 1000)
+    t, tf = _tt(y.shape, "i64"), _tt(y.shape, "f64")
+    text = mod([t], tf, "    %%0 = stablehlo.bitcast_convert %%arg0 : (%s) -> %s\n    return %%0 : %s\n" % (t, tf, tf))
+    got, ref = both(rx, client, text, [I.Tensor(y, "i64")])
+    assert np.array_equal(got[0].a.view(np.int64), y) and np.array_equal(ref[0].a.view(np.int64), y)
+    t = _tt([7, 5, 3], "f32")
+    text = mod([t], "tensor<i32>", "    %%0 = stablehlo.get_dimension_size %%arg0, dim = 1 : (%s) -> tensor<i32>\n    return %%0 : tensor<i32>\n" % t)
+    got, ref = both(rx, client, text, [I.Tensor(np.zeros((7, 5, 3), np.float32), "f32")])
+    assert int(got[0].a) == 5 == int(ref[0].a)
