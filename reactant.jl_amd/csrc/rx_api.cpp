@@ -208,7 +208,8 @@ std::string rtc_compile(const std::string& source, const std::string& arch) {
 rx::PlanOptions plan_options() {
   rx::PlanOptions o;
   if (const char* e = getenv("RX_XCD_SLABS")) o.xcd_slabs = atoi(e) != 0;
-  if (const char* e = getenv("RX_SLAB_MIN_NUMEL")) o.slab_min_numel = atoll(e);
+  if (const char* e = getenv("RX_SLAB_MIN_NUMEL")) o.slab_min_numel = o.slab_order_min_numel = atoll(e);
+  if (const char* e = getenv("RX_SLAB_ORDER_MIN_NUMEL")) o.slab_order_min_numel = atoll(e);
   if (const char* e = getenv("RX_MFMA")) o.mfma = atoi(e) != 0;
   if (const char* e = getenv("RX_ROW_FUSION")) o.row_fusion = atoi(e) != 0;
   if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;

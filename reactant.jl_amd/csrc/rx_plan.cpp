@@ -2252,7 +2252,7 @@ struct Planner {
 
     // shifted loads along the slowest dimension -> XCD slab order
     bool slab = false;
-    if (opt.xcd_slabs && n >= 3 && dims[0] >= 8 && dims[1] >= 8 && numel >= opt.slab_min_numel) {
+    if (opt.xcd_slabs && n >= 3 && dims[0] >= 8 && dims[1] >= 8 && numel >= opt.slab_order_min_numel) {
       std::map<int, std::set<int64_t>> offs0;
       for (auto& l : em.loads)
         if (l.affine && (int)l.off.size() == n) offs0[l.node].insert(l.off[0]);

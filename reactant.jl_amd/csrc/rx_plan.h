@@ -42,6 +42,7 @@ struct Plan {
 struct PlanOptions {
   bool xcd_slabs = true;        // XCD-aware tile order for kernels with shifted loads
   int64_t slab_min_numel = 1 << 22;  // smallest output that uses it
+  int64_t slab_order_min_numel = 1 << 22;  // smallest plain map with loads shifted along the slowest dimension that takes the XCD slab order
   bool mfma = true;             // use the MFMA GEMM skeletons for eligible dot_generals
   bool dot_as_reduce = true;    // dot_generals with a vector-like operand run as multiply + reduce
   bool fuse_dot_operands = true;  // a dot operand that expands much smaller data is evaluated inside the GEMM's tile loads
