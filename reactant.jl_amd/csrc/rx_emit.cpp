@@ -606,7 +606,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       for (size_t d = 0; d < ix.size(); ++d) {
         const Node& s = g_.nodes[n.in[1 + d]];
         const int64_t room = o.ty.dims[d] - n.a0[d];   // start indices are clamped into [0, room]
-        if (s.k == OpK::Constant) {
+        if (s.k == OpK::Constant && s.splat) {
           oi[d] = shifted(ix[d], std::min(std::max<int64_t>(splat_as_int(s), 0), room));
         } else {
           // start index computed at run time (a 0-d integer value): clamp, then offset
@@ -700,7 +700,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         const Node& s = g_.nodes[n.in[2 + d]];
         const int64_t room = o.ty.dims[d] - u.ty.dims[d];   // start indices are clamped into [0, room]
         Ix p;
-        if (s.k == OpK::Constant) {
+        if (s.k == OpK::Constant && s.splat) {
           p = shifted(ix[d], -std::min(std::max<int64_t>(splat_as_int(s), 0), room));
         } else {
           const std::string e = emit(n.in[2 + d], Index{});

@@ -1324,6 +1324,32 @@ struct Builder {
     }
   }
 
+  // An unrolled loop that reads `a[i]` (dynamic_slice at the loop counter) leaves one dynamic_slice per
+  // trip, alike but for the folded start.  Written into the kernel text the starts would make every
+  // trip's kernel a different one (hundreds of compilations for a time loop); kept as 0-d constants in
+  // memory, the trips share one kernel text that reads its start from its own 8-byte buffer.
+  void keep_loop_slice_starts_in_memory() {
+    std::map<std::pair<int, std::vector<int64_t>>, std::vector<int>> groups;
+    std::vector<int> other_uses(g.nodes.size(), 0);
+    for (int r : g.results) other_uses[r]++;
+    for (const Node& n : g.nodes) {
+      bool all_const = n.k == OpK::DynamicSlice;
+      for (size_t k = 0; k < n.in.size(); ++k) {
+        if (n.k == OpK::DynamicSlice && k >= 1) all_const = all_const && g.nodes[n.in[k]].k == OpK::Constant && g.nodes[n.in[k]].ty.rank() == 0;
+        else other_uses[n.in[k]]++;
+      }
+      if (all_const) groups[{n.in[0], n.a0}].push_back(n.id);
+    }
+    for (auto& kv : groups) {
+      if (kv.second.size() < 8) continue;
+      for (int id : kv.second)
+        for (size_t k = 1; k < g.nodes[id].in.size(); ++k) {
+          Node& c = g.nodes[g.nodes[id].in[k]];
+          if (other_uses[c.id] == 0 && c.data.size() == (size_t)info(c.ty.dt).size) c.splat = false;
+        }
+    }
+  }
+
   // one-element integer values that depend on constants only become constants (loop counters
   // after unrolling; start indices of dynamic slices must be constants when kernels are planned)
   void fold_scalar_constants() {
@@ -2515,6 +2541,7 @@ Graph parse_module(const char* text, size_t len) {
   }
   b.g.results = b.inline_func(*mainf, args, 0);
   b.fold_scalar_constants();
+  b.keep_loop_slice_starts_in_memory();
   if (b.g.results.size() != mainf->result_types.size()) throw Error("StableHLO import: @main returns the wrong number of values");
   for (size_t k = 0; k < b.g.results.size(); ++k)
     if (!(b.g.nodes[b.g.results[k]].ty == mainf->result_types[k]))

@@ -2173,7 +2173,7 @@ struct Planner {
     box->clear();
     for (int d = 0; d < n.ty.rank(); ++d) {
       const Node& sn = g.nodes[n.in[2 + d]];
-      if (sn.k != OpK::Constant) return false;
+      if (sn.k != OpK::Constant || !sn.splat) return false;
       const int64_t room = n.ty.dims[d] - un.ty.dims[d];
       box->push_back({std::min(std::max<int64_t>(splat_as_int(sn), 0), room), un.ty.dims[d]});
     }
