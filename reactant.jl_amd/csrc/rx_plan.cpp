@@ -1069,6 +1069,9 @@ struct Planner {
       }
     }
     int TZ = opt.lds_tile[0], TY = opt.lds_tile[1], TX = opt.lds_tile[2];
+    // the tile is given for 8-byte elements (two per vector); with more elements per vector the rows
+    // take fewer threads, so the tile gets more rows
+    if (TX % vec == 0 && (TX / vec) * TY != kBlock && kBlock % (TX / vec) == 0) TY = kBlock / (TX / vec);
     if (TX % vec || (TX / vec) * TY != kBlock) return false;
     const int TXV = TX / vec;
     // LDS geometry per staged input
