@@ -1832,13 +1832,19 @@ struct Planner {
   bool probe_chain_step(int x, ChainProbe* cp) {
     const Node& n = g.nodes[x];
     const int r = n.ty.rank();
-    if (n.k != OpK::DynamicUpdateSlice || r < 1 || r > 3 || r > opt.chain_max_rank) return false;
+    if (r < 1 || r > 3 || r > opt.chain_max_rank) return false;
+    if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) return false;
     const int es = info(n.ty.dt).size;
     if (es != 4 && es != 8) return false;
     if (n.ty.numel() < 2 || n.ty.numel() >= opt.slab_min_numel) return false;
-    int b = n.in[0];
-    while (!mat[b] && g.nodes[b].k == OpK::DynamicUpdateSlice) b = g.nodes[b].in[0];
-    if (!mat[b] || !(g.nodes[b].ty == n.ty)) return false;
+    // an update (x[r] = ...) supersedes the array it is written over; any other step (u = f(u), a pad
+    // around a computed interior) supersedes the array it reads the farthest around a point
+    int b = -1;
+    if (n.k == OpK::DynamicUpdateSlice) {
+      b = n.in[0];
+      while (!mat[b] && g.nodes[b].k == OpK::DynamicUpdateSlice) b = g.nodes[b].in[0];
+      if (!mat[b] || !(g.nodes[b].ty == n.ty)) return false;
+    }
     Emitter probe(g, [&](int y) { return y != x && mat[y]; });
     std::vector<std::string> vars;
     Index ix(r);
@@ -1859,6 +1865,17 @@ struct Planner {
         for (int d = 0; d < r; ++d) { h.lo[d] = std::max<int64_t>(h.lo[d], -l.off[d]); h.hi[d] = std::max<int64_t>(h.hi[d], l.off[d]); }
         saw_base = saw_base || l.node == b;
       } else cp->others.push_back(l.node);
+    }
+    if (b < 0) {
+      int64_t best = -1;
+      for (auto& kv : cp->reads) {
+        int64_t reach = 0;
+        for (int d = 0; d < r; ++d) reach += kv.second.lo[d] + kv.second.hi[d];
+        if (reach > best) { best = reach; b = kv.first; }
+      }
+      if (b < 0 || best == 0) return false;   // a plain elementwise step gains nothing from a tile
+      cp->base = b;
+      saw_base = true;
     }
     if (!saw_base) return false;
     for (auto& kv : cp->reads)
@@ -1910,6 +1927,22 @@ struct Planner {
         field_of[steps[i]] = field_of[probes[i].base];
       }
       const int nf = (int)entry.size();
+      // a step that reads the array it supersedes at other positions than its own cannot update it in
+      // place: such arrays get a second tile, written and read in turns
+      std::vector<char> two_tiles(nf, 0);
+      for (size_t i = 0; i < k; ++i) {
+        const Halo& hb = probes[i].reads.at(probes[i].base);
+        for (int d = 0; d < r; ++d) if (hb.lo[d] || hb.hi[d]) two_tiles[field_of[probes[i].base]] = 1;
+      }
+      // an array that no step writes and every step reads at its own position only stays in memory
+      std::vector<char> has_tile(nf, 0);
+      for (size_t i = 0; i < k; ++i) {
+        has_tile[field_of[probes[i].base]] = 1;
+        for (auto& kv : probes[i].reads)
+          for (int d = 0; d < r; ++d) if (kv.second.lo[d] || kv.second.hi[d]) has_tile[field_of[kv.first]] = 1;
+      }
+      int ntiles_lds = 0;
+      for (int f = 0; f < nf; ++f) ntiles_lds += has_tile[f] ? 1 + two_tiles[f] : 0;
       std::vector<std::array<int64_t, 3>> lo(k), hi(k);
       int64_t HL[3] = {0, 0, 0}, HH[3] = {0, 0, 0};
       for (size_t i = 0; i < k; ++i) {
@@ -1920,7 +1953,8 @@ struct Planner {
       }
       int64_t E[3] = {1, 1, 1}, box = 1, tile = 1;
       for (int d = 0; d < r; ++d) { E[d] = T[d] + HL[d] + HH[d]; box *= E[d]; tile *= T[d]; }
-      const int64_t lds_bytes = box * nf * es;
+      const int64_t lds_bytes = box * ntiles_lds * es;
+      if (getenv("RX_CHAIN_DEBUG")) fprintf(stderr, "[chain] k=%zu box=%lld tile=%lld tiles_in_lds=%d bytes=%lld\n", k, (long long)box, (long long)tile, ntiles_lds, (long long)lds_bytes);
       if (lds_bytes > opt.chain_lds_bytes || (double)box > opt.chain_redundancy * (double)tile) continue;
       const int NB = opt.chain_threads > 0 ? opt.chain_threads : (int)std::min<int64_t>(1024, (box + 63) / 64 * 64);
       if (NB < 64 || NB > 1024 || NB % 64) continue;
@@ -1933,7 +1967,10 @@ struct Planner {
         ix[d].var = vars[d]; ix[d].lo = 0; ix[d].hi = D[d] - 1;
       }
       std::vector<int> inputs, cur = entry, writes(k);
-      std::vector<std::string> bodies(k), vals(k);
+      std::vector<std::string> bodies(k), vals(k), wname(k);
+      // tile that holds the current version of a field: lds<f> or its twin lds<f>b
+      std::vector<char> side(nf, 0);
+      auto tile_name = [&](int f) { return "lds" + std::to_string(f) + (side[f] ? "b" : ""); };
       int64_t margin = 0;   // farthest neighbour read, in cells: the tiles sit that far inside the LDS allocation
       std::set<int> group(steps.begin(), steps.begin() + k);
       bool ok = true;
@@ -1950,10 +1987,11 @@ struct Planner {
           auto f = field_of.find(node);
           if (f == field_of.end() || !(g.nodes[node].ty == n0.ty)) return false;
           if (cur[f->second] != node) { ok = false; return false; }
+          if (!has_tile[f->second]) return false;
           int64_t delta = 0, stride = 1;
           for (int d = r - 1; d >= 0; --d) { delta += off[d] * stride; stride *= E[d]; }
           margin = std::max<int64_t>(margin, delta < 0 ? -delta : delta);
-          *expr = "lds" + std::to_string(f->second) + "[li + (" + std::to_string(delta) + ")]";
+          *expr = tile_name(f->second) + "[li + (" + std::to_string(delta) + ")]";
           return true;
         };
         vals[i] = em.store_value(n0.ty.dt, em.emit(x, ix));
@@ -1961,6 +1999,13 @@ struct Planner {
         for (auto& l : em.loads) if (group.count(l.node) && !(l.affine && g.nodes[l.node].ty == n0.ty)) ok = false;
         inputs = em.inputs;
         writes[i] = field_of[probes[i].base];
+        {
+          const Halo& hb = probes[i].reads.at(probes[i].base);
+          bool self = false;
+          for (int d = 0; d < r; ++d) self = self || hb.lo[d] || hb.hi[d];
+          if (self) side[writes[i]] = !side[writes[i]];
+          wname[i] = tile_name(writes[i]);
+        }
         cur[writes[i]] = x;
       }
       if (!ok) continue;
@@ -1991,7 +2036,14 @@ struct Planner {
         return -1;
       };
       o << "  extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];\n";
-      for (int f = 0; f < nf; ++f) o << "  " << st << "* const lds" << f << " = reinterpret_cast<" << st << "*>(rx_smem) + " << margin + f * box << ";\n";
+      {
+        int slot = 0;
+        for (int f = 0; f < nf; ++f) {
+          if (!has_tile[f]) continue;
+          o << "  " << st << "* const lds" << f << " = reinterpret_cast<" << st << "*>(rx_smem) + " << margin + slot++ * box << ";\n";
+          if (two_tiles[f]) o << "  " << st << "* const lds" << f << "b = reinterpret_cast<" << st << "*>(rx_smem) + " << margin + slot++ * box << ";\n";
+        }
+      }
       int64_t nt[3] = {1, 1, 1}, ntiles = 1;
       for (int d = 0; d < r; ++d) { nt[d] = (D[d] + T[d] - 1) / T[d]; ntiles *= nt[d]; }
       o << "  int tb = blockIdx.x;\n";
@@ -2042,9 +2094,9 @@ struct Planner {
       {
         open_loop(box, E, HL, "    ");
         o << "    const int lin = " << array_index() << ";\n";
-        for (int f = 0; f < nf; ++f) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
+        for (int f = 0; f < nf; ++f) if (has_tile[f]) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
         o << "    if (p < " << box << ") {\n";
-        for (int f = 0; f < nf; ++f) o << "      lds" << f << "[p] = s" << f << ";\n";
+        for (int f = 0; f < nf; ++f) if (has_tile[f]) o << "      lds" << f << "[p] = s" << f << ";\n";
         o << "    }\n  }\n  __syncthreads();\n";
       }
       for (size_t i = 0; i < k; ++i) {
@@ -2059,13 +2111,13 @@ struct Planner {
         open_loop(total, ext, back, "    ");
         o << "    {\n      const int li = " << box_index(back) << ";\n";
         o << bodies[i];
-        o << "      if (live) lds" << writes[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
+        o << "      if (live) " << wname[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
       }
       {
         const int64_t zero[3] = {0, 0, 0};
         open_loop(tile, T, zero, "    ");
         o << "    if (live) {\n      const int li = " << box_index(zero) << ";\n      const int lin = " << array_index() << ";\n";
-        for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = lds" << f << "[li];\n";
+        for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = " << tile_name(f) << "[li];\n";
         o << "    }\n  }\n}\n\n";
       }
       } else {
@@ -2096,9 +2148,9 @@ struct Planner {
         }
         o << "    IN[q] = " << in_arr << ";\n";
         o << "    const int lin = " << array_index() << ";\n";
-        for (int f = 0; f < nf; ++f) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
+        for (int f = 0; f < nf; ++f) if (has_tile[f]) o << "    const " << st << " s" << f << " = in" << slot_in(entry[f]) << "[lin];\n";
         o << "    if (p < " << box << ") {\n";
-        for (int f = 0; f < nf; ++f) o << "      lds" << f << "[p] = s" << f << ";\n";
+        for (int f = 0; f < nf; ++f) if (has_tile[f]) o << "      lds" << f << "[p] = s" << f << ";\n";
         o << "    }\n  }\n  __syncthreads();\n";
         const int64_t plane = box / E[0];
         auto rounds_of = [&](int64_t r0, int64_t r1, int64_t* qlo, int64_t* qhi) {   // rounds that hold cells of box rows [r0, r1)
@@ -2128,12 +2180,12 @@ struct Planner {
           o << "  // step " << i << ": " << describe(steps[i]) << "\n";
           open_round(first, ext);
           o << "    {\n" << bodies[i];
-          o << "      if (live) lds" << writes[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
+          o << "      if (live) " << wname[i] << "[li] = " << vals[i] << ";\n    }\n  }\n  __syncthreads();\n";
         }
         {
           open_round(HL, T);
           o << "    if (live) {\n      const int lin = " << array_index() << ";\n";
-          for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = lds" << f << "[li];\n";
+          for (int f = 0; f < nf; ++f) if (cur[f] != entry[f]) o << "      out" << f << "[lin] = " << tile_name(f) << "[li];\n";
           o << "    }\n  }\n}\n\n";
         }
       }
@@ -3716,9 +3768,6 @@ struct Planner {
           // what a step reads is either outside the kernel or the latest version of a field
           for (auto& kv : q.reads) ok = ok && (!group.count(kv.first) || cur[field_of[kv.first]] == kv.first);
           for (int y : q.others) ok = ok && !group.count(y);
-          // the step overwrites its field in place: it may read that field only at its own position
-          const Halo& hb = q.reads[q.base];
-          for (int d = 0; d < 3; ++d) ok = ok && hb.lo[d] == 0 && hb.hi[d] == 0;
           // a version superseded inside the kernel exists nowhere else
           if (ok && group.count(q.base)) ok = !is_result[q.base] && read_only_by(q.base, group, x);
           if (!ok) break;
@@ -3731,6 +3780,7 @@ struct Planner {
           steps.push_back(x);
           probes.push_back(q);
         }
+        if (getenv("RX_CHAIN_DEBUG")) fprintf(stderr, "[chain] job %zu (node %d, %s): run of %zu steps\n", i, jobs[i].first, g.nodes[jobs[i].first].ty.str().c_str(), steps.size());
         if (steps.size() < 2) { ++i; continue; }
         chain_at[steps[0]] = steps;
         auto plain0 = jobs[i].second;

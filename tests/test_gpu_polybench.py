@@ -235,3 +235,44 @@ def test_polybench_linalg_programs(rx, client, name, size):
         assert g_.a.shape == r_.a.shape
         scale = max(1.0, float(np.max(np.abs(r_.a))))
         assert float(np.max(np.abs(g_.a.astype(np.float64) - r_.a.astype(np.float64)))) <= 1e-5 * np.sqrt(k) * scale
+
+
+@pytest.mark.parametrize("shape,nfields,nsteps,dt", [((500,), 1, 20, "f32"), ((300,), 2, 25, "f64"), ((48, 70), 2, 12, "f32"), ((40, 40), 1, 9, "i32"),
+                                                     ((12, 20, 24), 2, 5, "f32")])
+def test_steps_that_read_the_array_they_supersede_use_two_tiles(rx, client, monkeypatch, shape, nfields, nsteps, dt):
+    """u = f(u shifted): the new version cannot overwrite the old one in place; the chain kernel keeps two
+    LDS tiles for such an array and writes them in turns."""
+    monkeypatch.setenv("RX_CHAIN_MAX_RANK", "3")
+    monkeypatch.setenv("RX_CHAIN_REDUNDANCY", "8")
+    for seed in (0, 1):
+        rng = np.random.default_rng(10 * seed + nsteps)
+        text = C.random_update_program(rng, shape, nfields, nsteps, dt, None, self_offsets=True)
+        args = _fields([shape] * nfields, dt, seed=seed)
+        got, exe = gpu_run(rx, client, text, args)
+        for g_, r_ in zip(got, oracle_run(text, args)):
+            assert np.array_equal(g_.a, r_.a)
+    assert "map_chain" in _kinds(exe)
+
+
+def test_pad_form_time_loop_of_one_array(rx, client, monkeypatch):
+    """u = pad(f(u interior neighbours)) repeated (a heat equation written out of place, the form of the
+    3-d diffusion / advection program): chained at small sizes, same bits as one launch per step."""
+    import importlib
+    PR = importlib.import_module("reactant_jl_amd.programs")
+    monkeypatch.setenv("RX_CHAIN_MAX_RANK", "3")
+    monkeypatch.setenv("RX_CHAIN_REDUNDANCY", "20")
+    monkeypatch.setenv("RX_CHAIN_TILE", "4,8,16")
+    nx, ny, nz = 30, 17, 8
+    text = PR.stencil(nx, ny, nz, steps=6, embed="pad")
+    full = (nz + 6, ny + 6, nx + 6)
+    rng = np.random.default_rng(4)
+    c = np.zeros(full)
+    c[3:-3, 3:-3, 3:-3] = rng.random((nz, ny, nx))
+    args = [I.Tensor(c, "f64")] + [I.Tensor(rng.uniform(-1, 1, full), "f64") for _ in range(3)]
+    got, exe = gpu_run(rx, client, text, args)
+    assert "map_chain" in _kinds(exe), _kinds(exe)
+    ref = oracle_run(text, args)
+    assert np.array_equal(got[0].a, ref[0].a)
+    monkeypatch.setenv("RX_CHAIN_STEPS", "1")
+    plain, exe1 = gpu_run(rx, client, text, args)
+    assert "map_chain" not in _kinds(exe1) and np.array_equal(plain[0].a, got[0].a)
