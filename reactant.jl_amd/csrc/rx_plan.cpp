@@ -1827,12 +1827,14 @@ struct Planner {
   std::set<int> chain_member;                 // steps emitted by a chain kernel
 
   // steps per kernel: a 1-d tile's halo grows by a cell or two per step, so long chains stay cheap
-  int chain_cap(int rank) const { return opt.chain_steps > 0 ? opt.chain_steps : rank == 1 ? 64 : 16; }
+  int chain_cap(int rank) const { return opt.chain_steps > 0 ? opt.chain_steps : rank == 1 ? 64 : rank == 2 ? 16 : 4; }
 
   bool probe_chain_step(int x, ChainProbe* cp) {
     const Node& n = g.nodes[x];
     const int r = n.ty.rank();
-    if (r < 1 || r > 3 || r > opt.chain_max_rank) return false;
+    // rank 3: only small arrays, whose steps are bound by the launch gap (32^3 and 64^3 heat steps: 1.6x and 1.4x
+    // faster in chains of four); at 128^3 the redundant halo cells cost more than the launches saved
+    if (r < 1 || r > 3 || (r > opt.chain_max_rank && !(r == 3 && n.ty.numel() <= opt.chain_rank3_numel))) return false;
     if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) return false;
     const int es = info(n.ty.dt).size;
     if (es != 4 && es != 8) return false;
@@ -1910,7 +1912,7 @@ struct Planner {
     {
       // vectors: one cell per thread (a step costs an LDS round trip and a barrier, whatever the tile);
       // matrices: 32x64 tiles, 32x32 when that is what it takes to give every compute unit a tile
-      int64_t dflt[3][3] = {{128, 1, 1}, {32, 64, 1}, {8, 8, 32}};
+      int64_t dflt[3][3] = {{128, 1, 1}, {32, 64, 1}, {8, 8, 16}};
       if (r == 2 && ((D[0] + 31) / 32) * ((D[1] + 63) / 64) < 256) dflt[1][1] = 32;
       for (int d = 0; d < r; ++d) {
         T[d] = opt.chain_tile[d] > 0 && opt.chain_tile[r - 1] > 0 ? opt.chain_tile[d] : dflt[r - 1][d];
@@ -1955,7 +1957,7 @@ struct Planner {
       for (int d = 0; d < r; ++d) { E[d] = T[d] + HL[d] + HH[d]; box *= E[d]; tile *= T[d]; }
       const int64_t lds_bytes = box * ntiles_lds * es;
       if (getenv("RX_CHAIN_DEBUG")) fprintf(stderr, "[chain] k=%zu box=%lld tile=%lld tiles_in_lds=%d bytes=%lld\n", k, (long long)box, (long long)tile, ntiles_lds, (long long)lds_bytes);
-      if (lds_bytes > opt.chain_lds_bytes || (double)box > opt.chain_redundancy * (double)tile) continue;
+      if (lds_bytes > opt.chain_lds_bytes || (double)box > (r == 3 ? 2.0 : 1.0) * opt.chain_redundancy * (double)tile) continue;
       const int NB = opt.chain_threads > 0 ? opt.chain_threads : (int)std::min<int64_t>(1024, (box + 63) / 64 * 64);
       if (NB < 64 || NB > 1024 || NB % 64) continue;
 

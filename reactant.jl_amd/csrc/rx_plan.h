@@ -69,6 +69,7 @@ struct PlanOptions {
   int chain_steps = 0;
   int chain_tile[3] = {0, 0, 0};     // outputs per workgroup (slowest .. fastest dimension of the array's rank; zeros: default per rank)
   int64_t chain_lds_bytes = 64 * 1024;  // LDS a workgroup may use for the tiles
+  int64_t chain_rank3_numel = 1 << 18;  // rank-3 steps up to this many elements are chained all the same (four per launch)
   int chain_max_rank = 2;            // rank-3 steps are bound by index arithmetic in such a kernel, not by launches: left as maps
   bool chain_fixed_cells = true;     // a thread keeps the same box cells (and their coordinates in registers) through all steps
   int chain_threads = 0;             // workgroup size (0: by the number of staged cells)
