@@ -265,3 +265,19 @@ def test_long_contractions_with_few_output_tiles_are_cut_along_k(rx, client, mon
     whole, exe1 = gpu_run(rx, client, text, [a, b])
     assert len(exe1.launches()) == 1
     assert max_rel_to_scale(whole[0].a, ref[0].a) <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
+
+
+def test_a_root_fed_by_several_products(rx, client):
+    """(A*B + C*D) .* (E'*F'): one product joins the elementwise root's kernel, the others run on their own
+    and are read back (syr2k of the reference's polybench suite is the two-product case)."""
+    t = _tt([256, 256], "f32")
+    text = ("module {\n func.func @main(%a: T, %b: T, %c: T, %d: T, %e: T, %f: T) -> T {\n"
+            "  %0 = stablehlo.dot_general %a, %b, contracting_dims = [1] x [0] : (T, T) -> T\n"
+            "  %1 = stablehlo.dot_general %c, %d, contracting_dims = [1] x [0] : (T, T) -> T\n"
+            "  %2 = stablehlo.dot_general %e, %f, contracting_dims = [0] x [1] : (T, T) -> T\n"
+            "  %3 = stablehlo.add %0, %1 : T\n  %4 = stablehlo.multiply %3, %2 : T\n  return %4 : T\n }\n}\n").replace("T", t)
+    rng = np.random.default_rng(0)
+    args = [I.tensor(rng.normal(size=(256, 256)), "f32") for _ in range(6)]
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["gemm_f32"] * 3
+    assert max_rel_to_scale(got[0].a, oracle_run(text, args, hifi=True)[0].a) <= 1e-5 * 16
