@@ -55,6 +55,9 @@ Parity status per function (what pins it, see tests/test_oracle_*.py):
       by a constant operand; the reference holds no known answer for it
   reduce over several operands (argmax / argmin / findfirst, src/Ops.jl:1536-1596) ... numpy
       max / argmax / argmin with ties, first and last index
+  convert float -> integer outside the integer's range ... saturates, NaN -> 0 (XLA's choice; StableHLO
+      leaves it implementation-defined and the reference holds no case: PARITY UNPINNED); in range it is
+      truncation, pinned by Python's int()
   batch_norm_inference / batch_norm_training (src/Ops.jl:4012-4092) ... closed forms
       (zero mean / unit variance of the normalized batch, numpy mean and var, the affine
       special case); the reference holds no known answer for them
@@ -1109,6 +1112,28 @@ def _unary(name, x, dt):
     raise NotImplementedError("%s on %s" % (name, dt))
 
 
+def _int_divide(a, b):
+    """Integer quotient truncated toward zero in the operands' own width; x / 0 = all ones, and for
+    signed types x / -1 = -x with wrap-around (MIN / -1 = MIN), which is what XLA returns for the cases
+    that the specification leaves to the implementation."""
+    if a.dtype == np.bool_:
+        return a | ~b  # x / 1 = x, x / 0 = all ones
+    signed = np.issubdtype(a.dtype, np.signedinteger)
+    with np.errstate(all="ignore"):
+        one = np.ones((), a.dtype)
+        safe = np.where(b == 0, one, b).astype(a.dtype)
+        if signed:
+            minus1 = safe == -1
+            safe = np.where(minus1, one, safe).astype(a.dtype)
+        q = (a // safe).astype(a.dtype)                      # floor
+        rem = (a - q * safe).astype(a.dtype)
+        if signed:
+            q = (q + ((rem != 0) & ((a < 0) != (safe < 0)))).astype(a.dtype)   # floor -> truncation
+            q = np.where(minus1, (0 - a).astype(a.dtype), q).astype(a.dtype)
+        q = np.where(b == 0, np.array(-1).astype(a.dtype), q).astype(a.dtype)
+    return q
+
+
 def _binary(name, x, y, dt):
     a, b = x.a, y.a
     if is_float(dt):
@@ -1129,13 +1154,10 @@ def _binary(name, x, y, dt):
         elif name == "subtract": r = a - b
         elif name == "multiply": r = a * b if dt != "i1" else a & b
         elif name == "divide":
-            safe = np.where(b == 0, 1, b)
-            r = (np.trunc(a.astype(np.float64) / safe)).astype(a.dtype) if a.dtype.itemsize < 8 else \
-                (np.sign(a) * np.sign(safe) * (np.abs(a) // np.abs(safe))).astype(a.dtype)
-            r = np.where(b == 0, -1, r).astype(a.dtype)
+            r = _int_divide(a, b)
         elif name == "remainder":
-            safe = np.where(b == 0, 1, b)
-            r = np.where(b == 0, a, np.fmod(a, safe)).astype(a.dtype)
+            # the dividend minus quotient x divisor (sign of the dividend; x % 0 = x, MIN % -1 = 0)
+            r = np.where(b == 0, a, a - _int_divide(a, b) * b).astype(a.dtype)
         elif name == "maximum": r = np.maximum(a, b)
         elif name == "minimum": r = np.minimum(a, b)
         elif name == "and": r = a & b
@@ -1181,10 +1203,16 @@ def _convert(x, dt_out):
         if dt_out in ("bf16", "f8E4M3FN", "f8E5M2"):
             return tensor(a.astype(np.float32), dt_out)
         return Tensor(a.astype(NP_OF[dt_out]), dt_out)
-    # to integer: truncation toward zero
+    # to integer: truncation toward zero; beyond the type's range the nearest limit, NaN -> 0 (what XLA
+    # does; StableHLO leaves it to the implementation and the reference holds no case: PARITY UNPINNED)
     if is_float(din):
+        info = np.iinfo(NP_OF[dt_out])
         with np.errstate(all="ignore"):
-            return Tensor(np.trunc(a).astype(NP_OF[dt_out]), dt_out)
+            t = np.trunc(np.asarray(a, dtype=np.float64))
+            r = np.where(np.isnan(t), 0.0, t)
+            out = np.clip(r, float(info.min), float(info.max))
+            res = np.where(out >= float(info.max), info.max, np.where(out <= float(info.min), info.min, out.astype(NP_OF[dt_out])))
+            return Tensor(res.astype(NP_OF[dt_out]), dt_out)
     return Tensor(a.astype(NP_OF[dt_out]), dt_out)
 
 

@@ -195,15 +195,33 @@ RX_DEV double rx_gelu_tanh(double x) {
 }
 RX_DEV double rx_gelu_erf(double x) { return 0.5 * x * (1.0 + erf(x * 0.7071067811865476)); }
 RX_DEV double rx_gelu_sigmoid(double x) { return x / (1.0 + exp(-1.702 * x)); }
+// Integer division as XLA defines the cases C++ leaves undefined: x / 0 = all ones, x % 0 = x, and
+// for signed types x / -1 = -x with wrap-around (so MIN / -1 = MIN) and x % -1 = 0.  For an unsigned
+// type (T)-1 is the largest value, an ordinary divisor.
 template <typename T> RX_DEV T rx_idiv(T a, T b) {
   if (b == 0) return (T)-1;
-  if (b == (T)-1) return (T)(0 - a);
+  if constexpr ((T)-1 < (T)0) {
+    if (b == (T)-1) return (T)(0 - a);
+  }
   return a / b;
 }
 template <typename T> RX_DEV T rx_irem(T a, T b) {
   if (b == 0) return a;
-  if (b == (T)-1) return (T)0;
+  if constexpr ((T)-1 < (T)0) {
+    if (b == (T)-1) return (T)0;
+  }
   return a % b;
+}
+// float -> integer conversion: truncation toward zero; values beyond the type's range give the
+// nearest limit and NaN gives 0 (a plain C++ cast is undefined for those).
+template <typename T, typename F> RX_DEV T rx_f2i(F x) {
+  constexpr bool sgn = (T)-1 < (T)0;
+  constexpr T hi = sgn ? (T)(((unsigned long long)1 << (8 * sizeof(T) - 1)) - 1) : (T)~(T)0;
+  constexpr T lo = sgn ? (T)(-(long long)hi - 1) : (T)0;
+  if (!(x == x)) return (T)0;
+  if (x <= (F)lo) return lo;
+  if (x >= (F)hi) return hi;   // (F)hi may round up to 2^k: such x are out of range as well
+  return (T)x;
 }
 template <typename T> RX_DEV T rx_ipow(T a, T b) {
   if (b < 0) return (a == 1) ? (T)1 : ((a == (T)-1) ? ((b & 1) ? (T)-1 : (T)1) : (T)0);

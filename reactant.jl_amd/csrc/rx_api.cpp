@@ -93,12 +93,21 @@ struct RxDevice {
       free_blocks.erase(it);
     } else {
       HIP_CHECK(hipSetDevice(ordinal));
-      hipError_t e = hipMalloc(&p, r);
-      if (e != hipSuccess) {
-        // give cached blocks back to the driver and retry once
-        (void)hipGetLastError();
+      auto trim = [&] {   // give cached blocks back to the driver
         for (auto& kv : free_blocks) { (void)hipFree(kv.second); pool_bytes -= (int64_t)kv.first; }
         free_blocks.clear();
+      };
+      // the client's memory fraction bounds what this allocator holds, cached blocks included
+      if (bytes_limit > 0 && pool_bytes + (int64_t)r > bytes_limit) {
+        trim();
+        if (pool_bytes + (int64_t)r > bytes_limit)
+          throw Error("RESOURCE_EXHAUSTED: allocating " + std::to_string(r) + " bytes would exceed the client's memory limit of " +
+                      std::to_string(bytes_limit) + " bytes (" + std::to_string(pool_bytes) + " in use)");
+      }
+      hipError_t e = hipMalloc(&p, r);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        trim();
         e = hipMalloc(&p, r);
         if (e != hipSuccess) {
           (void)hipGetLastError();
@@ -114,17 +123,24 @@ struct RxDevice {
     largest_alloc = std::max<int64_t>(largest_alloc, (int64_t)r);
     return p;
   }
+  bool closed = false;   // the client is gone: nothing will ask for a cached block again
   void release(void* p, size_t n) {
     const size_t r = round_size(n);
     std::lock_guard<std::mutex> l(mu);
     bytes_in_use -= (int64_t)r;
+    if (closed) {   // a buffer freed late (a finalizer after FreeClient): hand the block straight back
+      (void)hipSetDevice(ordinal);
+      (void)hipFree(p);
+      pool_bytes -= (int64_t)r;
+      return;
+    }
     free_blocks.insert({r, p});
   }
-  void drain() {
+  void drain(bool close) {
     std::lock_guard<std::mutex> l(mu);
-    for (auto& kv : free_blocks) (void)hipFree(kv.second);
+    for (auto& kv : free_blocks) { (void)hipFree(kv.second); pool_bytes -= (int64_t)kv.first; }
     free_blocks.clear();
-    pool_bytes = 0;
+    closed = closed || close;
   }
 };
 
@@ -322,13 +338,8 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       bufs[b] = ex->consts[b];
     }
   }
-  // donated arguments give up their storage now; the plan drops it after its last use
-  for (int i = 0; i < num_args; ++i) {
-    if (donate && donate[i]) {
-      args[i]->donated = true;
-      args[i]->mem.reset();
-    }
-  }
+  // Donated arguments give up their storage only once everything that can fail has succeeded (at the
+  // end of this function): an out-of-memory or launch error must leave the caller's arrays intact.
   // events of a timed execution; destroyed on every exit path unless handed to the executable
   struct EventList {
     std::vector<hipEvent_t> v;
@@ -375,6 +386,17 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       if (B.last_use == (int)li && !is_res[b]) bufs[b].reset();
     }
   }
+  // result handles and futures made so far; released again if a later step throws
+  struct Pending {
+    std::vector<RxBuffer*> bufs;
+    std::vector<RxFuture*> futs;
+    ~Pending() {
+      for (RxBuffer* b : bufs) { reg_del(b); delete b; }
+      for (RxFuture* f : futs) { if (f->ev) (void)hipEventDestroy(f->ev); delete f; }
+    }
+  } pending;
+  std::vector<RxBuffer*>& new_results = pending.bufs;
+  std::vector<RxFuture*>& new_futures = pending.futs;
   for (int r = 0; r < num_results; ++r) {
     const int b = P.result_buffers[r];
     const auto& B = P.buffers[b];
@@ -385,26 +407,43 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       HIP_CHECK(hipMemcpyAsync(m->ptr, ex->consts[b]->ptr, (size_t)B.bytes, hipMemcpyDeviceToDevice, dev->stream));
     } else if (B.kind == rx::BufferDesc::Param && !m) {
       throw Error("internal: pass-through result lost its storage");
+    } else if (B.kind == rx::BufferDesc::Param && !(donate && donate[B.param_index])) {
+      // an argument returned unchanged and not donated: the result is a buffer of its own, so that
+      // writing into it (CopyToBuffer) or donating it later leaves the caller's argument alone
+      m = std::make_shared<Allocation>(dev, std::max<size_t>((size_t)B.bytes, 1));
+      if (B.bytes) HIP_CHECK(hipMemcpyAsync(m->ptr, bufs[b]->ptr, (size_t)B.bytes, hipMemcpyDeviceToDevice, dev->stream));
     } else if (!m) {
       m = std::make_shared<Allocation>(dev, (size_t)B.bytes);  // nothing wrote it (empty tensor)
     }
-    results[r] = new_buffer(ex->client, dev, P.result_types[r], m);
+    new_results.push_back(new_buffer(ex->client, dev, P.result_types[r], m));
   }
   if (futures) {
     // one event shared by all result futures would need ref counting; events are cheap
     for (int r = 0; r < num_results; ++r) {
-      RxFuture* f = new RxFuture;
+      std::unique_ptr<RxFuture> f(new RxFuture);
       f->device = dev;
       HIP_CHECK(hipEventCreateWithFlags(&f->ev, hipEventDisableTiming));
       HIP_CHECK(hipEventRecord(f->ev, dev->stream));
-      reg_add(f);
-      futures[r] = f;
+      new_futures.push_back(f.release());
     }
   }
   if (launch_ms) {
     if (!evs.empty()) HIP_CHECK(hipEventSynchronize(evs.back()));
     for (size_t li = 0; li < P.launches.size(); ++li) HIP_CHECK(hipEventElapsedTime(&launch_ms[li], evs[2 * li], evs[2 * li + 1]));
-  } else if (profile_async) {
+  }
+  // nothing below can fail: publish the results and take the donated arguments' storage
+  for (int r = 0; r < num_results; ++r) results[r] = new_results[r];
+  new_results.clear();
+  if (futures)
+    for (int r = 0; r < num_results; ++r) { reg_add(new_futures[r]); futures[r] = new_futures[r]; }
+  new_futures.clear();
+  for (int i = 0; i < num_args; ++i) {
+    if (donate && donate[i]) {
+      args[i]->donated = true;
+      args[i]->mem.reset();
+    }
+  }
+  if (profile_async && !launch_ms) {
     ex->pending_events.push_back(std::move(evs));   // read later by RxExecutableTakeTimings
     evs.clear();
   }
@@ -476,7 +515,7 @@ RX_EXPORT void FreeClient(RxClient* c) {
     for (auto& d : c->devices) {
       (void)hipSetDevice(d->ordinal);
       (void)hipStreamSynchronize(d->stream);
-      d->drain();
+      d->drain(true);
       (void)hipStreamDestroy(d->stream);
       reg_del(d.get());
     }
@@ -682,7 +721,11 @@ RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, siz
         if (L.lds_bytes > 48 * 1024) {
           // more dynamic LDS than the default limit: gfx950 has 160 KB per workgroup
           hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(f), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.lds_bytes);
-          if (e != hipSuccess) (void)hipGetLastError();
+          if (e != hipSuccess) {
+            (void)hipGetLastError();
+            throw Error("kernel " + L.kernel + " needs " + std::to_string(L.lds_bytes) + " bytes of LDS, which the device refused (" +
+                        hipGetErrorString(e) + ")");
+          }
         }
         ex->fns.push_back(f);
       }

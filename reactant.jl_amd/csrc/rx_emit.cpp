@@ -418,6 +418,8 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       if (dt == DT::I1) return def("(" + x + " != 0)");
       if (is_narrow_float(sdt) && is_narrow_float(dt)) return def(x, true);
       if (is_narrow_float(sdt) && dt == DT::F32) return x;
+      // float -> integer: toward zero, saturating at the type's limits, NaN -> 0 (a plain cast is undefined there)
+      if (is_float(sdt) && !is_float(dt)) return def("rx_f2i<" + CT + ">(" + x + ")", true);
       return def("(" + CT + ")" + x, true);
     }
     case OpK::BroadcastInDim: {

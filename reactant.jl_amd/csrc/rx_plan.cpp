@@ -122,6 +122,8 @@ struct Planner {
   std::set<int> lds_only;           // the steps absorbed that way: no launch, no buffer
   std::map<int, int> reshape_alias; // materialized reshape of a materialized value: the same bytes, no launch
   std::set<std::pair<int, int>> fused_operands;   // (dot_general, side): the operand is evaluated inside the GEMM's tile loads
+  std::map<int, int> epilogue_of;   // dot_general -> the elementwise root that absorbs it (the product is launched there)
+  std::map<int, int> row_anchor;    // reduction fused into a row kernel -> the root of that kernel
   std::ostringstream src;
   int kcount = 0;
 
@@ -2234,7 +2236,7 @@ struct Planner {
       const int64_t room = n.ty.dims[d] - un.ty.dims[d];
       box->push_back({std::min(std::max<int64_t>(splat_as_int(sn), 0), room), un.ty.dims[d]});
     }
-    // every other kernel that reads base runs before this one (kernels run in node order)
+    // every other kernel that reads base is launched before this one
     std::vector<int> st{base};
     std::set<int> seen;
     while (!st.empty()) {
@@ -2242,11 +2244,25 @@ struct Planner {
       st.pop_back();
       for (int u : users[y]) {
         if (!live[u] || u == root) continue;
-        if (mat[u]) { if (u > root) return false; }
+        if (mat[u]) { if (launch_position(u) > root) return false; }
         else if (seen.insert(u).second) st.push_back(u);
       }
     }
     return true;
+  }
+
+  // Kernels are launched in the node order of their jobs, but some values are computed by a job
+  // that comes later than their own node: a product absorbed by its epilogue runs at the
+  // epilogue's root, a reduction fused into a row kernel at the row anchor, a stencil step that
+  // lives in LDS only inside the kernel of the step that reads it.
+  int launch_position(int u) const {
+    auto e = epilogue_of.find(u);
+    if (e != epilogue_of.end()) return e->second;
+    auto r = row_anchor.find(u);
+    if (r != row_anchor.end()) return r->second;
+    if (lds_only.count(u))
+      for (auto& kv : fuse_prev) if (kv.second == u) return kv.first;
+    return u;
   }
 
   // ------------------------------------------------------------------ map kernels
@@ -3628,7 +3644,7 @@ struct Planner {
     for (int p : g.params) { plan.param_types.push_back(g.nodes[p].ty); buffer_for(p); }
 
     // dot epilogues: an elementwise root that consumes a dot result at the identity index
-    std::map<int, int> epilogue_of;  // dot node -> root that absorbs it
+    epilogue_of.clear();
     for (int x = 0; x < N; ++x) {
       if (!live[x] || g.nodes[x].k != OpK::DotGeneral) continue;
       if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
@@ -3808,7 +3824,7 @@ struct Planner {
     for (auto& j : jobs) {
       const Node& n = g.nodes[j.first];
       if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::Scatter && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
-        for (int p : row_phases(j.first)) fused_reduces.insert(p);
+        for (int p : row_phases(j.first)) { fused_reduces.insert(p); row_anchor[p] = j.first; }
     }
     lap("job list, chains");
     for (auto& j : jobs) j.second();

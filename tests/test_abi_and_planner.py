@@ -291,3 +291,14 @@ def test_long_time_loops_import_and_plan_in_linear_time():
     assert time.time() - t0 < 60
     with pytest.raises(Exception, match="more than 65536 iterations"):
         rx.compile_offline(PB.build("jacobi_1d", n=64, tsteps=70000))
+
+
+def test_update_in_place_waits_for_readers_that_are_launched_late():
+    """A product absorbed by its epilogue is launched at the epilogue, a reduction fused into a row
+    kernel at that kernel's root: when either comes after a `dynamic_update_slice` of the value it
+    reads, the update must write a buffer of its own (kind map, not map_in_place)."""
+    import _inplace_modules as M
+    kinds = lambda rep: re.findall(r"kind=(\w+)", rep)
+    assert kinds(rx.compile_offline(M.DOT_EPILOGUE_AFTER_UPDATE)) == ["map", "map", "gemm_f32"]
+    assert kinds(rx.compile_offline(M.ROW_REDUCE_AFTER_UPDATE)) == ["gemm_f32", "map", "row"]
+    assert kinds(rx.compile_offline(M.UPDATE_AFTER_ALL_READERS)) == ["map", "gemm_f32", "map_in_place"]

@@ -125,3 +125,53 @@ def test_calls_from_several_host_threads(rx, client):
         t.join()
     assert not errors, errors[:3]
     assert len(results) == 4
+
+
+PASS_THROUGH = """module {
+  func.func @main(%a: tensor<256xf32>, %b: tensor<256xf32>) -> (tensor<256xf32>, tensor<256xf32>) {
+    %0 = stablehlo.add %a, %b : tensor<256xf32>
+    return %a, %0 : tensor<256xf32>, tensor<256xf32>
+  }
+}
+"""
+
+
+def test_an_argument_returned_unchanged_is_a_buffer_of_its_own_unless_donated(rx, client):
+    a = np.arange(256, dtype=np.float32)
+    exe = rx.xla_compile(client, PASS_THROUGH)
+    ba, bb = rx.Buffer.from_host(client, a, "f32"), rx.Buffer.from_host(client, a, "f32")
+    out = [r.synced_buffer() for r in exe.execute_sharded([ba, bb])]
+    assert out[0].unsafe_pointer() != ba.unsafe_pointer()
+    out[0].copy_from_host(np.full(256, -1.0, dtype=np.float32))          # writes the result only
+    assert np.array_equal(ba.to_host(), a) and np.array_equal(out[0].to_host(), np.full(256, -1.0, dtype=np.float32))
+    assert np.array_equal(out[1].to_host(), 2 * a)
+    # donated: the result takes the argument's storage over, the argument can no longer be read
+    p = ba.unsafe_pointer()
+    out = [r.synced_buffer() for r in exe.execute_sharded([ba, bb], donated=[True, False])]
+    assert out[0].unsafe_pointer() == p and np.array_equal(out[0].to_host(), a)
+    with pytest.raises(rx.ReactantInternalError, match="donated"):
+        ba.to_host()
+
+
+def test_memory_limit_is_enforced_and_a_failed_execution_keeps_donated_arguments(rx):
+    """A client with a small memory fraction: an allocation beyond it fails with RESOURCE_EXHAUSTED
+    (src/accelerators/GPU.jl:7-37 passes the fraction), and an execution that fails that way leaves
+    the argument it was asked to donate readable."""
+    small = rx.Client(memory_fraction=2e-4)                                # about 58 MB of 288 GB
+    try:
+        limit = small.default_device().allocator_stats()["bytes_limit"]
+        assert 0 < limit < (1 << 28)
+        n = int(limit // 4 * 0.6)
+        x = np.ones(n, dtype=np.float32)
+        bx = rx.Buffer.from_host(small, x, "f32")                          # 60 % of the limit: fits
+        with pytest.raises(rx.ReactantInternalError, match="RESOURCE_EXHAUSTED"):
+            rx.Buffer.from_host(small, x, "f32")                           # a second one does not
+        t = "tensor<%dxf32>" % n
+        exe = rx.xla_compile(small, "module { func.func @main(%%a: %s) -> %s { %%0 = stablehlo.add %%a, %%a : %s\n return %%0 : %s } }" % (t, t, t, t))
+        with pytest.raises(rx.ReactantInternalError, match="RESOURCE_EXHAUSTED"):
+            exe.execute_sharded([bx], donated=[True])                      # the result does not fit beside the argument
+        assert float(bx.to_host()[n - 1]) == 1.0                           # still the caller's
+        exe.free()
+        bx.free()
+    finally:
+        small.close()

@@ -565,3 +565,49 @@ def test_bitcast_convert_and_get_dimension_size(rx, client):
     text = mod([t], "tensor<i32>", "    %%0 = stablehlo.get_dimension_size %%arg0, dim = 1 : (%s) -> tensor<i32>\n    return %%0 : tensor<i32>\n" % t)
     got, ref = both(rx, client, text, [I.Tensor(np.zeros((7, 5, 3), np.float32), "f32")])
     assert int(got[0].a) == 5 == int(ref[0].a)
+
+
+# ---- integer division at the edges, float -> integer conversion beyond the range -------------
+@pytest.mark.parametrize("dt", ["ui8", "ui16", "ui32", "ui64", "i8", "i16", "i32", "i64"])
+@pytest.mark.parametrize("op", ["divide", "remainder"])
+def test_integer_division_edge_cases(rx, client, op, dt):
+    """Divisors 0, 1 and the all-ones pattern (the largest value of an unsigned type, -1 of a signed
+    one), dividends including the type's limits; bit-exact against the oracle, whose rules are pinned
+    against Python integers in tests/test_oracle_golden.py."""
+    info = np.iinfo(I.NP_OF[dt])
+    av = [0, 1, 2, 5, 100, info.max, info.max - 1, info.min, info.min + 1 if info.min else 7]
+    bv = [0, 1, 2, 3, info.max, info.max - 1, -1 if info.min else info.max, info.min if info.min else 4]
+    a = np.array([x for x in av for _ in bv], dtype=I.NP_OF[dt])
+    b = np.array([y for _ in av for y in bv], dtype=I.NP_OF[dt])
+    t = _tt([a.size], dt)
+    text = mod([t, t], t, "    %%0 = stablehlo.%s %%arg0, %%arg1 : %s\n    return %%0 : %s\n" % (op, t, t))
+    got, ref = both(rx, client, text, [I.Tensor(a, dt), I.Tensor(b, dt)])
+    assert np.array_equal(got[0].a, ref[0].a), (got[0].a.tolist(), ref[0].a.tolist())
+
+
+@pytest.mark.parametrize("dst", ["i8", "ui8", "i16", "ui16", "i32", "ui32", "i64", "ui64"])
+@pytest.mark.parametrize("src", ["f32", "f64", "bf16"])
+def test_convert_float_to_integer_saturates(rx, client, src, dst):
+    """Truncation toward zero inside the range, the nearest limit beyond it, 0 for NaN."""
+    vals = [0.0, 0.9, -0.9, 3.9, -3.9, 127.0, 128.0, -128.0, -129.0, 255.0, 256.0, 300.0, -200.0, 32767.0, 32768.0, -32769.0, 65535.0,
+            65536.0, 2147483520.0, 2147483648.0, -2147483648.0, -2147483904.0, 4294967040.0, 4294967296.0, 9.2233715e18, 9.3e18,
+            -9.3e18, 1.8446743e19, 1.9e19, 1e30, -1e30, float("inf"), float("-inf"), float("nan")]
+    x = I.tensor(np.array(vals, dtype=np.float64), src)
+    ts, td = _tt([len(vals)], src), _tt([len(vals)], dst)
+    text = mod([ts], td, "    %%0 = stablehlo.convert %%arg0 : (%s) -> %s\n    return %%0 : %s\n" % (ts, td, td))
+    got, ref = both(rx, client, text, [x])
+    assert np.array_equal(got[0].a, ref[0].a), (got[0].a.tolist(), ref[0].a.tolist())
+
+
+# ---- an update in place must wait for every reader of the buffer it takes over ---------------
+@pytest.mark.parametrize("name", ["dot_epilogue_after_update", "row_reduce_after_update", "update_after_all_readers"])
+def test_update_slice_and_late_readers(rx, client, name):
+    import _inplace_modules as M
+    text, nargs, shapes = M.CASES[name]
+    rng = np.random.default_rng(11)
+    args = [I.Tensor(rng.uniform(0.5, 1.5, s).astype(np.float32), "f32") for s in shapes]
+    got, ref = both(rx, client, text, args)
+    assert np.array_equal(got[0].a[:16], args[nargs - 2].a)           # the updated rows: copies
+    assert rel_err(got[0].a, ref[0].a) <= 1e-5, name                  # the rest: a sum or a product of positive numbers
+    assert max_rel_to_scale(got[1].a, ref[1].a) <= 1e-5, name        # positive operands: no cancellation
+    assert rel_err(got[1].a, ref[1].a) <= 1e-4, name

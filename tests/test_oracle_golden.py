@@ -409,3 +409,41 @@ def test_chlo_math_ops_satisfy_their_identities():
     assert run("stablehlo.popcnt", [0, 1, 255, -1, 1 << 20], "i32").tolist() == [0, 1, 8, 32, 1]
     assert run("stablehlo.count_leading_zeros", [0, 1, 255, -1, 1 << 20], "i32").tolist() == [32, 31, 24, 0, 11]
     assert run("stablehlo.count_leading_zeros", [0, 1, 127, -1], "i8").tolist() == [8, 7, 1, 0]
+
+
+def test_integer_division_rules_against_python_integers():
+    """Quotients truncate toward zero and remainders take the dividend's sign (C and XLA alike);
+    x / 0 is all ones and x % 0 is x; MIN / -1 wraps to MIN and MIN % -1 is 0; the all-ones divisor
+    of an unsigned type is an ordinary number."""
+    for dt in ("i8", "i16", "i32", "i64", "ui8", "ui16", "ui32", "ui64"):
+        info = np.iinfo(I.NP_OF[dt])
+        bits = info.bits
+        vals = sorted({0, 1, 2, 3, 7, 100, info.max, info.max - 1, info.min, info.min + 1, -1 if info.min else info.max, -7 if info.min else 9})
+        a = np.array([x for x in vals for _ in vals], dtype=I.NP_OF[dt])
+        b = np.array([y for _ in vals for y in vals], dtype=I.NP_OF[dt])
+        q = I._binary("divide", I.Tensor(a, dt), I.Tensor(b, dt), dt).a
+        r = I._binary("remainder", I.Tensor(a, dt), I.Tensor(b, dt), dt).a
+
+        def wrap(v):
+            v &= (1 << bits) - 1
+            return v - (1 << bits) if info.min and v >> (bits - 1) else v
+        for x, y, qq, rr in zip(a.tolist(), b.tolist(), q.tolist(), r.tolist()):
+            if y == 0:
+                eq, er = wrap(-1), x
+            else:
+                t = abs(x) // abs(y) * (1 if (x < 0) == (y < 0) else -1)
+                eq, er = wrap(t), x - t * y
+            assert (qq, rr) == (eq, er), (dt, x, y, qq, rr, eq, er)
+
+
+def test_float_to_integer_conversion_against_python_int():
+    """In range: Python's int() (truncation).  Beyond the range the oracle saturates and maps NaN to 0,
+    which is XLA's choice and not fixed by the specification (parity unpinned there)."""
+    rng = np.random.default_rng(5)
+    for dt in ("i8", "ui8", "i16", "ui16", "i32", "ui32", "i64", "ui64"):
+        info = np.iinfo(I.NP_OF[dt])
+        x = rng.uniform(max(info.min, -2.0 ** 52), min(info.max, 2.0 ** 52), 500)
+        got = I._convert(I.Tensor(x, "f64"), dt).a.tolist()
+        assert got == [int(v) for v in x.tolist()], dt
+        edge = I._convert(I.Tensor(np.array([1e30, -1e30, np.nan, np.inf, -np.inf]), "f64"), dt).a.tolist()
+        assert edge == [info.max, info.min, 0, info.max, info.min], (dt, edge)
