@@ -143,6 +143,20 @@ void RxExecuteTimed(RxExecutable *exec, int num_args, RxBuffer **op_args, RxDevi
 void RxExecuteProfiled(RxExecutable *exec, int num_args, RxBuffer **op_args, RxDevice *device,
                        uint8_t *is_arg_donatable, int num_results, RxBuffer **op_results);
 int RxExecutableTakeTimings(RxExecutable *exec, double *launch_ms_sum);
+/* No counterpart in the reference.  For callers that cannot allocate device memory while they run
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the launch
+ * list of `exec`, like XLAExecuteSharded, but the caller passes the result buffers too (existing
+ * buffers of the executable's result types, distinct from the arguments and from each other; they
+ * are overwritten), and every temporary of the plan (partial results of the two-pass reductions,
+ * tensors handed from one kernel to the next) lives in a static device array of
+ * RxNoAllocScratchBytes() = 4 MiB that each GPU the library runs on holds until the process ends.
+ * No hipMalloc / hipFree, no event, no handle is created; nothing is donated; the kernels are queued
+ * on the device's stream and the call does not wait for them.  Returns 0, or 1 with a message
+ * (RxLastError) when the temporaries of the plan exceed the array ("RESOURCE_EXHAUSTED"), or a
+ * buffer has the wrong type or device.  All calls on one GPU share the array: calls through one
+ * client are ordered by its stream, calls through different clients of the same GPU race. */
+int RxExecuteNoAlloc(RxExecutable *exec, int num_args, RxBuffer **op_args, int num_results, RxBuffer **op_results);
+size_t RxNoAllocScratchBytes(void);
 /* Blocks until all work queued on the device's stream has finished. */
 void RxDeviceSynchronize(RxDevice *device);
 /* Plain 16-byte-per-lane copy kernel of `bytes` bytes, `iters` times; returns

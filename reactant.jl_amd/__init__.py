@@ -117,6 +117,8 @@ SIGNATURES = {
     "RxExecuteTimed": (None, [_vp, _i, _P(_vp), _vp, _P(_u8), _i, _P(_vp), _P(ctypes.c_float)]),
     "RxExecuteProfiled": (None, [_vp, _i, _P(_vp), _vp, _P(_u8), _i, _P(_vp)]),
     "RxExecutableTakeTimings": (_i, [_vp, _P(ctypes.c_double)]),
+    "RxExecuteNoAlloc": (_i, [_vp, _i, _P(_vp), _i, _P(_vp)]),
+    "RxNoAllocScratchBytes": (_sz, []),
     "RxDeviceSynchronize": (None, [_vp]),
     "RxCalibrationCopy": (ctypes.c_float, [_vp, _sz, _i]),
 }
@@ -438,6 +440,14 @@ class LoadedExecutable:
         dev = (device or self.client.default_device()).handle
         _call("RxExecuteProfiled", self.handle, n, args, dev, don, nres, res)
         return [Buffer(res[k], self.client) for k in range(nres)]
+
+    def execute_no_alloc(self, buffers, results):
+        """Queue the launch list with caller-owned result buffers and every temporary in the library's
+        static device array (4 MiB): nothing is allocated, nothing is donated, no future is returned."""
+        n, nres = len(buffers), len(results)
+        args = (_vp * n)(*[b.handle for b in buffers])
+        res = (_vp * nres)(*[b.handle for b in results])
+        _call("RxExecuteNoAlloc", self.handle, n, args, nres, res)
 
     def take_timings(self):
         """(number of profiled executions since the last call, per-launch mean milliseconds)."""

@@ -24,6 +24,14 @@
 
 extern "C" __attribute__((visibility("default"))) void (*ReactantThrowError)(const char*) = nullptr;
 
+// Device memory of RxExecuteNoAlloc: every temporary of an executable's plan (partial results of the
+// two-pass reductions, intermediate tensors between kernels) is placed here instead of coming from
+// the allocator.  One copy per GPU, held until the process ends.  Host code never uses this name as
+// an address: each device's address is looked up once (hipGetSymbolAddress, in MakeGPUClient) and
+// kept in RxDevice::scratch_ptr.
+#define RX_NOALLOC_SCRATCH_BYTES (4u << 20)
+static __device__ __align__(256) unsigned char scratch[RX_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 using rx::Error;
@@ -68,6 +76,8 @@ struct RxDevice {
   int ordinal = 0;       // HIP device ordinal
   int index = 0;         // position in the client's device list
   hipStream_t stream = nullptr;
+  void* scratch_ptr = nullptr;   // this device's copy of `scratch` (RxExecuteNoAlloc)
+  std::mutex scratch_mu;         // held while a call that uses it queues its kernels
   std::string kind;
   std::string arch;
   // caching allocator: device memory is kept and reused by size class, because hipMalloc and
@@ -494,6 +504,7 @@ RX_EXPORT RxClient* MakeGPUClient(int node_id, int num_nodes, int64_t* allowed_d
       HIP_CHECK(hipMemGetInfo(&fr, &tot));
       d->bytes_limit = (int64_t)((memory_fraction > 0 && memory_fraction <= 1 ? memory_fraction : 1.0) * (double)tot);
       HIP_CHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+      HIP_CHECK(hipGetSymbolAddress(&d->scratch_ptr, HIP_SYMBOL(scratch)));   // with this device current: its own copy
       reg_add(d.get());
       c->devices.push_back(std::move(d));
     }
@@ -816,6 +827,88 @@ RX_EXPORT int RxExecutableTakeTimings(RxExecutable* ex, double* launch_ms_sum) {
     return runs;
   }, 0);
 }
+
+// The launch list of `ex` with caller-owned results and every temporary inside the device's static
+// scratch array: no allocation, no event, no handle is created.
+RX_EXPORT int RxExecuteNoAlloc(RxExecutable* ex, int num_args, RxBuffer** args, int num_results, RxBuffer** results) {
+  return guarded([&]() -> int {
+    check_exec(ex);
+    RxDevice* dev = ex->device;
+    const rx::Plan& P = ex->plan;
+    if (num_args != (int)P.param_types.size())
+      throw Error("INVALID_ARGUMENT: executable expects " + std::to_string(P.param_types.size()) + " arguments, got " + std::to_string(num_args));
+    if (num_results != (int)P.result_types.size())
+      throw Error("INVALID_ARGUMENT: executable returns " + std::to_string(P.result_types.size()) + " results, got room for " + std::to_string(num_results));
+    for (int i = 0; i < num_args; ++i) {
+      check_buffer(args[i]);
+      if (args[i]->donated || !args[i]->mem) throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " was donated to an earlier execution");
+      if (!(args[i]->ty == P.param_types[i]))
+        throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " has type " + args[i]->ty.str() + ", executable expects " + P.param_types[i].str());
+      if (args[i]->device != dev) throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " lives on another device");
+    }
+    for (int r = 0; r < num_results; ++r) {
+      check_buffer(results[r]);
+      if (results[r]->donated || !results[r]->mem) throw Error("INVALID_ARGUMENT: result buffer " + std::to_string(r) + " was donated to an earlier execution");
+      if (!(results[r]->ty == P.result_types[r]))
+        throw Error("INVALID_ARGUMENT: result buffer " + std::to_string(r) + " has type " + results[r]->ty.str() + ", executable returns " + P.result_types[r].str());
+      if (results[r]->device != dev) throw Error("INVALID_ARGUMENT: result buffer " + std::to_string(r) + " lives on another device");
+      for (int i = 0; i < num_args; ++i)
+        if (args[i]->mem->ptr == results[r]->mem->ptr) throw Error("INVALID_ARGUMENT: result buffer " + std::to_string(r) + " is also argument " + std::to_string(i));
+      for (int q = 0; q < r; ++q)
+        if (results[q]->mem->ptr == results[r]->mem->ptr) throw Error("INVALID_ARGUMENT: result buffers " + std::to_string(q) + " and " + std::to_string(r) + " are the same");
+    }
+    if (!dev->scratch_ptr) throw Error("internal: the device's scratch array was not resolved");
+    // where every plan buffer lives: arguments, constants of the executable, the caller's results
+    // (first result that returns the buffer), everything else at 256-byte steps in the scratch array
+    const size_t NB = P.buffers.size();
+    std::vector<void*> where(NB, nullptr);
+    std::vector<int> first_result(NB, -1);
+    for (int r = 0; r < num_results; ++r)
+      if (first_result[P.result_buffers[r]] < 0) first_result[P.result_buffers[r]] = r;
+    size_t used = 0;
+    for (size_t b = 0; b < NB; ++b) {
+      const auto& B = P.buffers[b];
+      if (B.kind == rx::BufferDesc::Param) where[b] = args[B.param_index]->mem->ptr;
+      else if (B.kind == rx::BufferDesc::Const) where[b] = ex->consts[b]->ptr;
+      else if (first_result[b] >= 0) where[b] = results[first_result[b]]->mem->ptr;
+      else if (B.first_def >= 0 || B.last_use >= 0) {
+        where[b] = (char*)dev->scratch_ptr + used;
+        used += ((size_t)B.bytes + 255) & ~(size_t)255;
+      }
+    }
+    if (used > RX_NOALLOC_SCRATCH_BYTES)
+      throw Error("RESOURCE_EXHAUSTED: the temporaries of this executable take " + std::to_string(used) + " bytes; RxExecuteNoAlloc holds at most " +
+                  std::to_string(RX_NOALLOC_SCRATCH_BYTES) + " (use XLAExecuteSharded)");
+    std::lock_guard<std::mutex> lock(ex->mu);
+    std::lock_guard<std::mutex> slock(dev->scratch_mu);
+    HIP_CHECK(hipSetDevice(dev->ordinal));
+    std::vector<void*> ptrs, argv;
+    for (size_t li = 0; li < P.launches.size(); ++li) {
+      const auto& L = P.launches[li];
+      if (L.grid[0] == 0 || L.grid[1] == 0 || L.grid[2] == 0) continue;
+      ptrs.clear();
+      argv.clear();
+      for (int b : L.args) {
+        if (!where[b]) throw Error("internal: unbound buffer in launch " + std::to_string(li));
+        ptrs.push_back(where[b]);
+      }
+      for (auto& p : ptrs) argv.push_back(&p);
+      HIP_CHECK(hipModuleLaunchKernel(ex->fns[li], L.grid[0], L.grid[1], L.grid[2], L.block[0], L.block[1], L.block[2], L.lds_bytes, dev->stream,
+                                      argv.data(), nullptr));
+    }
+    // results that no kernel of this call wrote in place: arguments and constants returned as they
+    // are, and a buffer returned more than once
+    for (int r = 0; r < num_results; ++r) {
+      const int b = P.result_buffers[r];
+      const auto& B = P.buffers[b];
+      void* src = where[b];
+      if (src && src != results[r]->mem->ptr && B.bytes && P.result_types[r].bytes())
+        HIP_CHECK(hipMemcpyAsync(results[r]->mem->ptr, src, (size_t)P.result_types[r].bytes(), hipMemcpyDeviceToDevice, dev->stream));
+    }
+    return 0;
+  }, 1);
+}
+RX_EXPORT size_t RxNoAllocScratchBytes(void) { return RX_NOALLOC_SCRATCH_BYTES; }
 
 RX_EXPORT void FreeFuture(RxFuture* f) {
   if (!f || !reg_has(f)) return;
