@@ -566,6 +566,9 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
   auto tile = [&](auto P, int kt) {
     constexpr int p = decltype(P)::value;
     const RX_LDS E* sa = lds + (kt % S) * STAGE;
+    // 16-bit operands: the wavefronts of the main loop run at raised priority (measured: the 8192 x 4096 x 4096 bf16
+    // layer 5 % faster; 8-bit operands 2 % slower, so they keep the default)
+    if constexpr (sizeof(E) == 2) __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int s = 0; s + 1 < NS; ++s) {
       // keep the order "LDS reads of the next step, then the MFMAs of this step": the reads then

@@ -2,6 +2,7 @@
 
 #include <cstdlib>
 #include <sstream>
+#include <stdexcept>
 
 namespace rx {
 
@@ -75,6 +76,13 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   // Products that leave most compute units without a 128x128 tile take 64x64 tiles (1000^3 f32:
   // 16 -> 48 TFLOP/s, 1024^3 bf16: 130 -> 240); an operand with at most 64 rows (the output
   // features of a convolution) gets a 64-wide tile so that no MFMA works on padding.
+  // A tuning override (RX_GEMM_TILE / _BK / _STAGES / _DIRECT) is honoured or refused with an error: a setting that
+  // does not fit must not end in the scalar loop unnoticed.
+  bool tuned = false;
+  auto refuse = [&](const char* why) {
+    throw std::runtime_error(std::string("RX_GEMM_* tuning override cannot be honoured for ") + c.kind + " " + std::to_string(M) + "x" + std::to_string(N) + "x" +
+                             std::to_string(K) + ": " + why);
+  };
   int BM = 128, BN = 128, WM = 2, WN = 2;
   if (M <= 64 && N > 64) { BM = 64; BN = 128; }
   else if (N <= 64 && M > 64) { BM = 128; BN = 64; }
@@ -82,13 +90,21 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   else if (((M + 127) / 128) * ((N + 127) / 128) * batch * split < 128) { BM = 64; BN = 64; }
   if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
     int v[4];
-    if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; }
+    if (sscanf(e, "%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3]) == 4) { BM = v[0]; BN = v[1]; WM = v[2]; WN = v[3]; tuned = true; }
+    else refuse("RX_GEMM_TILE wants BM,BN,WM,WN");
+    if (BM < 32 || BN < 32 || WM < 1 || WN < 1 || BM % (32 * WM) != 0 || BN % (32 * WN) != 0 || WM * WN > 16) refuse("tile is not a whole number of 32x32 blocks per wavefront");
   }
-  if (const char* e = getenv("RX_GEMM_BK")) bk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : bk;
+  const int ks_step = a == DT::F32 ? 8 : (esize == 2 ? 16 : 64);
+  if (const char* e = getenv("RX_GEMM_BK")) {
+    const int v = atoi(e);
+    if (v <= 0 || v % ks_step != 0) refuse("RX_GEMM_BK is not a multiple of the MFMA k step");
+    if (K % v == 0) { bk = v; tuned = true; }   // products whose K it does not divide keep the default
+  }
   bool direct = !staged_only;   // global -> LDS direct loads through a ring of LDS stages
-  if (const char* e = getenv("RX_GEMM_DIRECT")) direct = atoi(e) != 0;
+  bool direct_forced = false;
+  if (const char* e = getenv("RX_GEMM_DIRECT")) { direct = atoi(e) != 0 && !staged_only; direct_forced = atoi(e) != 0 && !staged_only; }
   int stages = 2;
-  if (const char* e = getenv("RX_GEMM_STAGES")) stages = atoi(e) >= 2 ? atoi(e) : stages;
+  if (const char* e = getenv("RX_GEMM_STAGES")) { if (atoi(e) < 2) refuse("RX_GEMM_STAGES < 2"); stages = atoi(e); }
   int rb = 4, cb = 8;   // tiles of one XCD's block (rows x columns of the tile grid)
   if (const char* e = getenv("RX_GEMM_BLOCK")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2 && v[0] > 0 && v[1] > 0) { rb = v[0]; cb = v[1]; } }
   // a grid of few tiles (per batch entry) is not worth padding to whole XCD blocks
@@ -98,9 +114,8 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   else if ((N + BN - 1) / BN < cb) { const int64_t gn = (N + BN - 1) / BN; rb = (int)(rb * cb / gn); cb = (int)gn; }
   const int nt = WM * WN * 64;
   if (direct) {
-    int dbk = bk;
-    if (const char* e = getenv("RX_GEMM_BK")) dbk = atoi(e) > 0 && K % atoi(e) == 0 ? atoi(e) : dbk;
-    const int ks = a == DT::F32 ? 8 : (esize == 2 ? 16 : 64);
+    const int dbk = bk;
+    const int ks = ks_step;
     const int64_t a_ch = (int64_t)BM * dbk / ve, b_ch = (int64_t)BN * dbk / ve;
     const int64_t stage_bytes = ((int64_t)BM + BN) * dbk * esize;
     while (stages > 2 && stage_bytes * stages > 160 * 1024) --stages;
@@ -121,13 +136,18 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       c.ok = true;
       return c;
     }
+    if (direct_forced) refuse("the direct-to-LDS skeleton does not tile this shape");
+    if (tuned && stage_bytes * 2 > 160 * 1024) refuse("two LDS stages of this tile exceed 160 KB");
   }
   if (split > 1) return c;   // only the direct-to-LDS skeleton slices K
   const int pad = a == DT::F32 ? 4 : (esize == 2 ? 8 : 16);
   const int64_t a_sz = a_kc ? (int64_t)BM * (bk + pad) : (int64_t)bk * (BM + pad);
   const int64_t b_sz = b_kc ? (int64_t)BN * (bk + pad) : (int64_t)bk * (BN + pad);
   c.lds_bytes = (unsigned)(2 * (a_sz + b_sz) * esize);
-  if (c.lds_bytes > 160 * 1024) return c;
+  if (c.lds_bytes > 160 * 1024) {
+    if (tuned) refuse("the register-staged skeleton needs more than 160 KB of LDS for this tile and K step");
+    return c;
+  }
   c.block = WM * WN * 64;
   const int64_t gm = (M + BM - 1) / BM, gn = (N + BN - 1) / BN;
   c.grid[0] = (unsigned)gemm_grid(gm, gn, rb, cb);

@@ -302,3 +302,21 @@ def test_update_in_place_waits_for_readers_that_are_launched_late():
     assert kinds(rx.compile_offline(M.DOT_EPILOGUE_AFTER_UPDATE)) == ["map", "map", "gemm_f32"]
     assert kinds(rx.compile_offline(M.ROW_REDUCE_AFTER_UPDATE)) == ["gemm_f32", "map", "row"]
     assert kinds(rx.compile_offline(M.UPDATE_AFTER_ALL_READERS)) == ["map", "gemm_f32", "map_in_place"]
+
+
+def test_gemm_tuning_overrides_are_honoured_or_refused(monkeypatch):
+    # a K step whose two LDS stages exceed 160 KB used to end in the scalar loop without a word
+    fp8 = P.fp8_linear(512, 512, 512)
+    monkeypatch.setenv("RX_GEMM_TILE", "256,256,2,4")
+    monkeypatch.setenv("RX_GEMM_BK", "256")
+    with pytest.raises(rx.ReactantInternalError, match="tuning override cannot be honoured"):
+        rx.compile_offline(fp8)
+    monkeypatch.setenv("RX_GEMM_BK", "100")   # not a multiple of the MFMA k step
+    with pytest.raises(rx.ReactantInternalError, match="multiple of the MFMA k step"):
+        rx.compile_offline(fp8)
+    monkeypatch.setenv("RX_GEMM_BK", "128")
+    assert "kind=gemm_f8" in rx.compile_offline(fp8)
+    monkeypatch.delenv("RX_GEMM_BK")
+    monkeypatch.setenv("RX_GEMM_TILE", "96,96,2,2")
+    with pytest.raises(rx.ReactantInternalError, match="32x32 blocks"):
+        rx.compile_offline(fp8)
