@@ -38,3 +38,27 @@ def max_rel_to_scale(got, ref):
     ref = np.asarray(ref, dtype=np.float64)
     scale = max(float(np.max(np.abs(ref))), 1e-30) if ref.size else 1.0
     return float(np.max(np.abs(got - ref))) / scale if got.size else 0.0
+
+
+def abs_args(args):
+    """The operands with every element replaced by its magnitude (exact in the operand's own type)."""
+    return [I.Tensor(np.abs(a.a), a.dt) for a in args]
+
+
+def contraction_err(got, ref, bound):
+    """max over the entries of |got - ref|_ij / bound_ij, where bound_ij = (|A| . |B|)_ij plus the magnitudes the
+    epilogue adds: the componentwise error of a contraction.  One large entry cannot set the scale for the others,
+    so a wrong small entry (a dropped K tail in one tile, a bad bias lane) shows."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    bound = np.asarray(bound, dtype=np.float64)
+    assert got.shape == ref.shape == bound.shape, (got.shape, ref.shape, bound.shape)
+    if not got.size:
+        return 0.0
+    assert np.all(bound >= 0)
+    return float(np.max(np.abs(got - ref) / np.maximum(bound, 1e-300)))
+
+
+def dot_bound(text, args):
+    """(|A| . |B|) of a module that is one dot_general (any dimension numbers), by running the oracle on the magnitudes."""
+    return np.asarray(I.run_text(text, abs_args(args), hifi=True)[0].a, dtype=np.float64)

@@ -5,10 +5,24 @@ inner products, a few right-hand sides): the multiply + reduce form, every layou
 import numpy as np
 import pytest
 
-from _harness import gpu_run, oracle_run, max_rel_to_scale
+from _harness import gpu_run, oracle_run, max_rel_to_scale, contraction_err, dot_bound
 from oracle import stablehlo_interp as I
 
 pytestmark = pytest.mark.gpu
+
+
+def cw_tol(dt, out_dt):
+    """Bound on |got - ref|_ij / (|A| . |B|)_ij, the componentwise error of a contraction accumulated in f32 (f64 for f64
+    operands): the rounding of the result type for 16-bit results (half an ulp of bf16 is 2^-9, of f16 2^-12, relative to
+    the entry, which is at most the bound), the accumulation for wider ones.  All are below the 1e-2 (16- and 8-bit
+    operands) and 1e-5 sqrt(K) (f32) the specification of this backend allows."""
+    if out_dt == "bf16":
+        return 4e-3
+    if out_dt == "f16":
+        return 1e-3
+    if dt == "f64":
+        return 1e-14
+    return 1e-4 if dt.startswith("f8") else 1e-6
 
 
 def _tt(shape, dt):
@@ -69,7 +83,8 @@ def test_dot_general_mfma(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
     kinds = [l["kind"] for l in exe.launches() if l["kind"] != "map"]     # maps: the padding copies and the final slice
     assert kinds == ["gemm_" + {"f32": "f32", "bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8", "f64": "f64"}[dt]], kinds
     ref = oracle_run(text, [a, b], hifi=True)
-    err = max_rel_to_scale(got[0].a, ref[0].a)
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol(dt, out_dt)
+    err = max_rel_to_scale(got[0].a, ref[0].a)     # second figure: the error against the largest entry
     if out_dt in ("bf16", "f16"):
         assert err <= 1e-2
     elif out_dt == "f64":
@@ -153,6 +168,7 @@ def test_dot_general_with_a_vector_like_operand(rx, client, ls, rs, os_, attrs, 
     if dt == "i32":
         assert np.array_equal(got[0].a, ref[0].a)
         return
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol(dt, out_dt)
     err = max_rel_to_scale(got[0].a, ref[0].a)
     if out_dt in ("bf16", "f16"):
         assert err <= 1e-2
@@ -169,6 +185,7 @@ def test_short_contractions_keep_the_scalar_loop(rx, client):
     got, exe = gpu_run(rx, client, text, [a, b])
     assert [l["kind"] for l in exe.launches()] == ["dot_scalar"]
     ref = oracle_run(text, [a, b], hifi=True)
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol("f32", "f32")
     assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-5
 
 
@@ -193,6 +210,9 @@ def test_operand_evaluated_inside_the_product_with_an_epilogue(rx, client, dt):
     got, exe = gpu_run(rx, client, text, args)
     assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt], exe.report()
     ref = oracle_run(text, args, hifi=True, excess=(dt == "bf16"))
+    # on magnitudes the module is |A| . (|w| |s|) + |C| (the maximum with zero changes nothing): the bound with the epilogue's term;
+    # the expanded operand is rounded to bf16 before the product, which doubles the allowance
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, args)) <= (2 if dt == "bf16" else 1) * cw_tol(dt, dt)
     assert max_rel_to_scale(got[0].a, ref[0].a) <= (2e-2 if dt == "bf16" else 1e-5 * np.sqrt(K))
     # the same product transposed: the expanded operand is now the left one
     text2 = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s, %%arg3: %s) -> %s {\n"
@@ -205,6 +225,7 @@ def test_operand_evaluated_inside_the_product_with_an_epilogue(rx, client, dt):
     got, exe = gpu_run(rx, client, text2, args2)
     assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt], exe.report()
     ref = oracle_run(text2, args2, hifi=True, excess=(dt == "bf16"))
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text2, args2)) <= (2 if dt == "bf16" else 1) * cw_tol(dt, dt)
     assert max_rel_to_scale(got[0].a, ref[0].a) <= (2e-2 if dt == "bf16" else 1e-5 * np.sqrt(K))
 
 
@@ -229,6 +250,7 @@ def test_dot_general_with_grouped_or_permuted_dims(rx, client, ls, rs, os_, attr
     assert any(k.startswith("gemm_") for k in kinds) and "dot_scalar" not in kinds, kinds
     ref = oracle_run(text, [a, b], hifi=True)
     assert got[0].a.shape == ref[0].a.shape
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol(dt, dt)
     err = max_rel_to_scale(got[0].a, ref[0].a)
     assert err <= {"bf16": 1e-2, "f64": 1e-13, "f32": 1e-4}[dt]
 
@@ -259,11 +281,14 @@ def test_long_contractions_with_few_output_tiles_are_cut_along_k(rx, client, mon
     import re
     assert int(re.search(r"kind=gemm_\w+ grid=\d+x(\d+)x1", exe.report()).group(1)) in (slices // 4, slices // 2, slices, 2 * slices)
     ref = oracle_run(text, [a, b], hifi=True)
+    bound = dot_bound(text, [a, b])
+    assert contraction_err(got[0].a, ref[0].a, bound) <= cw_tol(dt, out_dt)
     err = max_rel_to_scale(got[0].a, ref[0].a)
     assert err <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
     monkeypatch.setenv("RX_SPLIT_K", "0")
     whole, exe1 = gpu_run(rx, client, text, [a, b])
     assert len(exe1.launches()) == 1
+    assert contraction_err(whole[0].a, ref[0].a, bound) <= cw_tol(dt, out_dt)
     assert max_rel_to_scale(whole[0].a, ref[0].a) <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
 
 
@@ -280,4 +305,7 @@ def test_a_root_fed_by_several_products(rx, client):
     args = [I.tensor(rng.normal(size=(256, 256)), "f32") for _ in range(6)]
     got, exe = gpu_run(rx, client, text, args)
     assert [l["kind"] for l in exe.launches()] == ["gemm_f32"] * 3
-    assert max_rel_to_scale(got[0].a, oracle_run(text, args, hifi=True)[0].a) <= 1e-5 * 16
+    ref = oracle_run(text, args, hifi=True)[0].a
+    # on magnitudes the module is (|A||B| + |C||D|) (|E||F|): the first-order bound of the product of the two factors' errors
+    assert contraction_err(got[0].a, ref, dot_bound(text, args)) <= 2 * cw_tol("f32", "f32")
+    assert max_rel_to_scale(got[0].a, ref) <= 1e-5 * 16

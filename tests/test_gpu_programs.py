@@ -5,7 +5,7 @@ maps 1e-6 relative, fp32 reductions 1e-5*sqrt(n) relative, bf16/fp8 contractions
 import numpy as np
 import pytest
 
-from _harness import gpu_run, oracle_run, max_rel_to_scale
+from _harness import gpu_run, oracle_run, max_rel_to_scale, contraction_err, abs_args
 from _loader import load_programs
 from oracle import stablehlo_interp as I
 
@@ -244,6 +244,9 @@ def test_gemm_f32(rx, client, m, n, k, form):
     text = P.gemm(m, n, k, form=form)
     got, _ = gpu_run(rx, client, text, args)
     ref = 1.5 * (A.astype(np.float64) @ B.astype(np.float64)) + 1.2 * C.astype(np.float64)
+    # componentwise: against 1.5 |A| |B| + 1.2 |C|, entry by entry
+    bound = 1.5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + 1.2 * np.abs(C).astype(np.float64)
+    assert contraction_err(got[0].a.T, ref, bound) <= 1e-6
     assert max_rel_to_scale(got[0].a.T, ref) <= 1e-5 * np.sqrt(k)
     orc = oracle_run(text, args, hifi=True)
     assert max_rel_to_scale(orc[0].a.T, ref) <= 1e-6
@@ -277,6 +280,17 @@ def test_mlp_bf16(rx, client, batch, widths, gelu):
     # in test_gpu_dot.py)
     assert max_rel_to_scale(got[0].a, ref[0].a) <= 2e-2
     assert max_rel_to_scale(got[0].a, strict[0].a) <= 3e-2
+    # every layer on its own, fed with the oracle's activations of the layer before, is held to 1e-2 componentwise:
+    # |got - ref|_ij <= 1e-2 (|h| . |W| + |b|)_ij  (gelu has slope <= 1.13 and is rounded to bf16 once)
+    h = args[0]
+    for l in range(len(widths) - 1):
+        layer = P.mlp(batch, widths[l:l + 2], gelu=gelu, softmax=False)
+        largs = [h, args[1 + 2 * l], args[2 + 2 * l]]
+        got_l, _ = gpu_run(rx, client, layer, largs)
+        ref_l = oracle_run(layer, largs, hifi=True, excess=True)
+        bound = (np.abs(h.a.astype(np.float64)) @ np.abs(largs[1].a.astype(np.float64))) + np.abs(largs[2].a.astype(np.float64))[None, :]
+        assert contraction_err(got_l[0].a, ref_l[0].a, bound) <= 1e-2, l
+        h = ref_l[0]
 
 
 @pytest.mark.parametrize("batch,k,n,layout,form", [(8, 32, 16, "nk", "convert"), (8, 32, 16, "kn", "direct"),
@@ -289,5 +303,8 @@ def test_fp8_linear(rx, client, batch, k, n, layout, form):
     got, _ = gpu_run(rx, client, text, [a, wq, sw])
     ref = oracle_run(text, [a, wq, sw], hifi=True, excess=True)
     assert max_rel_to_scale(got[0].a, ref[0].a) <= 1e-2
+    # rows are normalised one by one: each row against its own largest entry
+    g64, r64 = got[0].a.astype(np.float64), ref[0].a.astype(np.float64)
+    assert float(np.max(np.max(np.abs(g64 - r64), axis=1) / np.max(np.abs(r64), axis=1))) <= 1e-2
     # RMSNorm invariant: mean square of every row is 1 (up to bf16 rounding)
     assert np.allclose((got[0].a.astype(np.float64) ** 2).mean(axis=1), 1.0, atol=2e-2)
