@@ -9,9 +9,13 @@ algorithmic bytes (per timestep: read c,u,v,w + write c over the interior
 = 5*512*512*256*8 B).  `roofline` describes the dominant kernel (the stencil kernel
 that advances two timesteps per launch: its algorithmic bytes are those of both), timed with HIP events on the stream it runs on, inside the timed
 region.  `cpu_baseline` times the oracle's C/OpenMP restatement of the stencil on the
-host cores (a bounded number of repetitions of the same module).  `others` carries the remaining four configs
-(sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry; their step time is that
-of plain executions, and the pass with an event pair on every launch is reported beside it.
+host cores (a bounded number of repetitions of the same module, same inputs).  `others` carries the remaining four configs
+(sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry, its own `check` against the oracle and
+its own `cpu_baseline`; their step time is the median over groups of plain executions, and the pass with an event pair
+on every launch is reported beside it.  Every workload's result is verified after its timed region (`check`):
+the stencil bit for bit against the C restatement, the others on sampled rows against float64 / the numpy oracle.
+`roofline.traffic` is read from profiles/bench_all_configs_hbm_traffic.txt (rocprofv3 counters) and is null when the
+kernel name or launch size there does not match this run's launch list.
 `--workload conv|cumsum|maxpool` run one of the windowed ops instead, `--workload polybench` /
 `polybench_linalg` the reference's polybench stencil and linear-algebra suites (never part of `others`).
 """
@@ -29,22 +33,51 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of each dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
-# scaled by the readings of a plain 1 GiB copy kernel (profiles/bench_all_configs_hbm_traffic.txt).
-# Counters cannot be read from inside this process, so the figures of that profile are quoted here;
-# they are reported only for the kernel and shape they were measured on.
-MEASURED_TRAFFIC_BYTES = {
-    "rx_stencil_k0_stencil2m": 3549.6e6,
-    "rx_sinsum_add_k0_reduce": 537.1e6,
-    "rx_gemm_k0_gemm": 547.5e6,
-    "rx_mlp_k1_gemm": 470.1e6,
-    "rx_fp8_linear_k2_gemm": 965.7e6,
-}
-_FULL_SIZE = [True]   # cleared by --small: the table only holds the full-size shapes
+# HBM bytes per launch of each kernel as rocprofv3 counted them (FETCH_SIZE / WRITE_SIZE scaled by the readings of a
+# plain 1 GiB copy kernel): counters cannot be read from inside this process, so the tracked summary of that profile is
+# the one source of the figures.  A row is used only if its kernel name and its launch size (work-items) are the ones
+# of this run's launch list; otherwise `traffic` is null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_all_configs_hbm_traffic.txt")
+_FULL_SIZE = [True]   # cleared by --small
+OPTS = {"check": True, "cpu": True}
 
 
-def _traffic(kernel):
-    return MEASURED_TRAFFIC_BYTES.get(kernel) if _FULL_SIZE[0] else None
+def _traffic_table():
+    table = {}
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                t = line.split()
+                if len(t) == 5 and t[0].startswith("rx_") and t[1].isdigit():
+                    table[(t[0], int(t[1]))] = float(t[4]) * 1e6
+    except OSError:
+        pass
+    return table
+
+
+def _launch_sizes(exe):
+    """kernel name -> work-items per launch, from the plan report ("[i] name kind=... grid=AxBxC block=N")."""
+    import re
+    out = {}
+    for m in re.finditer(r"\] (\S+) kind=\S+ grid=(\d+)x(\d+)x(\d+) block=(\d+)", exe.report()):
+        out[m.group(1)] = int(m.group(2)) * int(m.group(3)) * int(m.group(4)) * int(m.group(5))
+    return out
+
+
+def _traffic(exe, kernel):
+    if not _FULL_SIZE[0]:
+        return None
+    return _traffic_table().get((kernel, _launch_sizes(exe).get(kernel, -1)))
+
+
+def _hbm_roofline(exe, kernel, kms, algo_bytes, **extra):
+    tr = _traffic(exe, kernel)
+    return {"bound": "hbm", "kernel": kernel, **extra, "kernel_ms": kms,
+            "achieved": algo_bytes / (kms * 1e-3) / 1e9 if kms else None, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": algo_bytes / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None,
+            "traffic": tr,
+            # what the memory system actually moved, as a fraction of the HBM peak (counter bytes / kernel time)
+            "traffic_frac": tr / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if (tr and kms) else None}
 
 
 PEAK_HBM_GBS = 8000.0
@@ -92,16 +125,44 @@ def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
 
 def _time_plain(client, exe, bufs, steps, warmup):
     """K steps as a caller runs them: queued without waiting, no event pair on the launches (a pair
-    costs a few microseconds of stream time, which shows on steps of less than 0.1 ms).  Seconds per step."""
+    costs a few microseconds of stream time, which shows on steps of less than 0.1 ms).  The K steps run in up to
+    five groups, each queued whole and timed by the host clock around a synchronization; returns the median of
+    the groups' seconds per step."""
     dev = client.default_device()
     for _ in range(warmup):
         exe.execute_sharded(bufs)
     dev.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        exe.execute_sharded(bufs)
-    dev.synchronize()
-    return (time.perf_counter() - t0) / steps
+    groups = max(1, min(5, steps // 2))
+    per = max(1, steps // groups)
+    times = []
+    for _ in range(groups):
+        t0 = time.perf_counter()
+        for _ in range(per):
+            exe.execute_sharded(bufs)
+        dev.synchronize()
+        times.append((time.perf_counter() - t0) / per)
+    return float(np.median(times))
+
+
+def _cpu_threads():
+    """Threads numpy's BLAS uses on this host (the GEMM-shaped CPU baselines run on it)."""
+    try:
+        import threadpoolctl
+        n = [i.get("num_threads", 1) for i in threadpoolctl.threadpool_info() if i.get("user_api") == "blas"]
+        return int(max(n)) if n else 1
+    except Exception:
+        return 1
+
+
+def _timed_reps(fn, budget_s, max_reps):
+    """Run fn() until `budget_s` seconds or `max_reps` repetitions; (seconds per repetition, repetitions, last result)."""
+    t0, reps, res = time.perf_counter(), 0, None
+    while True:
+        res = fn()
+        reps += 1
+        if time.perf_counter() - t0 > budget_s or reps >= max_reps:
+            break
+    return (time.perf_counter() - t0) / reps, reps, res
 
 
 def _dominant(launches, mean_ms, kinds):
@@ -118,6 +179,14 @@ def _dominant(launches, mean_ms, kinds):
 # ----------------------------------------------------------------------------
 # workloads
 # ----------------------------------------------------------------------------
+def _oracle_c():
+    try:
+        from oracle import build_c
+        return build_c, build_c.load()
+    except (ImportError, OSError):
+        return None, None
+
+
 def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=10):
     H = 3
     full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
@@ -126,8 +195,8 @@ def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=1
     text = P.stencil(nx, ny, nz, steps=nsteps)
     exe = rx.xla_compile(client, text)
     cb = _upload(rx, client, c, "f64")
-    vel = [_upload(rx, client, np.random.default_rng(s).uniform(-1, 1, full), "f64") for s in (1, 2, 3)]
-    del c
+    host_vel = [np.random.default_rng(s).uniform(-1, 1, full) for s in (1, 2, 3)]
+    vel = [_upload(rx, client, a, "f64") for a in host_vel]
 
     def make_args(prev):
         cur = prev[0] if prev else cb
@@ -144,18 +213,37 @@ def bench_stencil(rx, client, P, steps, warmup, nx=512, ny=512, nz=256, nsteps=1
         nk, kms, _b, _f = _dominant(launches, mean_ms, ("map_stencil_lds", "map_stencil", "map"))
         per_launch = 1
     algo_launch = 5.0 * cells * 8 * per_launch
-    return {
+    res = {
         "workload": "stencil f64 %dx%dx%d halo 3, %d timesteps per module" % (nx, ny, nz, nsteps),
         "ms_per_step": 1e3 * secs / steps,
         "value": algo_step / (secs / steps) / 1e9, "unit": "GB/s", "dtype": "f64",
-        "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"] if launches else None, "launches_per_step": nk,
-                     "timesteps_per_launch": per_launch,
-                     "kernel_ms": kms, "achieved": algo_launch / (kms * 1e-3) / 1e9 if kms else None,
-                     "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": algo_launch / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS if kms else None,
-                     "traffic": _traffic(launches[0]["kernel"]) if launches else None},
+        "roofline": _hbm_roofline(exe, launches[0]["kernel"], kms, algo_launch, launches_per_step=nk, timesteps_per_launch=per_launch),
         "plan": exe.report(),
     }
+    # after the timed region: one module call from the initial field, bit for bit against the C restatement of the
+    # same ten timesteps on the same inputs; that CPU run is also the first repetition of the CPU baseline
+    build_c, lib = _oracle_c() if (OPTS["check"] or OPTS["cpu"]) else (None, None)
+    if lib is not None:
+        t0 = time.perf_counter()
+        want = build_c.stencil_steps(lib, c, *host_vel, nx, ny, nz, nsteps)
+        first = time.perf_counter() - t0
+        if OPTS["check"]:
+            out = exe.execute_sharded([_upload(rx, client, c, "f64")] + vel)
+            got = rx.decode(out[0].synced_buffer().to_host(), "f64").reshape(full)
+            res["check"] = {"against": "oracle/stencil_cpu.c, same inputs, %d timesteps" % nsteps, "cells": int(got.size),
+                            "bit_exact": bool(np.array_equal(got, want)), "mismatches": int(np.count_nonzero(got != want))}
+            del got, out
+        if OPTS["cpu"]:
+            per, reps, _ = _timed_reps(lambda: build_c.stencil_steps(lib, c, *host_vel, nx, ny, nz, nsteps), 10.0, 9)
+            per = (per * reps + first) / (reps + 1)
+            res["cpu_baseline"] = {"value": algo_step / per / 1e9, "unit": "GB/s", "cores": int(lib.rx_oracle_threads()), "kind": "port",
+                                   "sample": "C restatement of the stencil (oracle/stencil_cpu.c, OpenMP), the GPU run's inputs, full %dx%dx%d grid, "
+                                             "%d timesteps per repetition, %d repetitions (%.2f s each)" % (nx, ny, nz, nsteps, reps + 1, per)}
+    elif OPTS["check"] or OPTS["cpu"]:
+        res["check"] = {"skipped": "oracle/_build/liboracle_c.so is not built"}
+        if OPTS["cpu"]:
+            res["cpu_baseline"] = cpu_baseline_stencil_numpy(P)
+    return res
 
 
 def bench_sinsum(rx, client, P, steps, warmup, n=1 << 26):
@@ -168,16 +256,30 @@ def bench_sinsum(rx, client, P, steps, warmup, n=1 << 26):
     _, kms, _, _ = _dominant(launches, mean_ms, ("reduce",))
     algo = 8.0 * n
     plain = _time_plain(client, exe, [bx, by], steps, warmup)
-    got = float(rx.decode(res[0].to_host(), "f32"))
-    exact = float(np.sum(np.sin(x.astype(np.float64)) + y.astype(np.float64)))
     # the step time is that of the plain executions; the pass with an event pair on every launch gives the kernel times
-    return {"workload": "sinsum_add f32[2^26] x2 -> scalar", "ms_per_step": 1e3 * plain,
-            "value": algo / plain / 1e9, "unit": "GB/s", "dtype": "f32",
-            "with_launch_events": {"ms_per_step": 1e3 * secs / steps, "value": algo / (secs / steps) / 1e9},
-            "check": {"got": got, "f64_reference": exact},
-            "roofline": {"bound": "hbm", "kernel": launches[0]["kernel"], "kernel_ms": kms,
-                         "achieved": algo / (kms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": algo / (kms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": _traffic(launches[0]["kernel"])}}
+    out = {"workload": "sinsum_add f32[2^26] x2 -> scalar", "ms_per_step": 1e3 * plain,
+           "value": algo / plain / 1e9, "unit": "GB/s", "dtype": "f32",
+           "with_launch_events": {"ms_per_step": 1e3 * secs / steps, "value": algo / (secs / steps) / 1e9},
+           "roofline": _hbm_roofline(exe, launches[0]["kernel"], kms, algo)}
+    if OPTS["check"]:
+        got = float(rx.decode(res[0].to_host(), "f32"))
+        terms = np.sin(x.astype(np.float64)) + y.astype(np.float64)
+        exact, mag = float(np.sum(terms)), float(np.sum(np.abs(terms)))
+        # f32 accumulation over n terms: within 1e-6 of the sum of magnitudes (far inside the 1e-5 sqrt(n) allowance)
+        out["check"] = {"against": "float64 numpy", "got": got, "f64_reference": exact, "err_over_sum_of_magnitudes": abs(got - exact) / mag,
+                        "pass": bool(abs(got - exact) <= 1e-6 * mag)}
+    if OPTS["cpu"]:
+        build_c, lib = _oracle_c()
+        if lib is not None:
+            per, reps, _ = _timed_reps(lambda: build_c.sinsum_add(lib, x, y), 3.0, 20)
+            out["cpu_baseline"] = {"value": algo / per / 1e9, "unit": "GB/s", "cores": int(lib.rx_oracle_threads()), "kind": "port",
+                                   "sample": "C restatement (oracle/reduce_cpu.c, OpenMP), full 2^%d vectors, %d repetitions (%.3f s each)"
+                                             % (int(np.log2(n)), reps, per)}
+        else:
+            per, reps, _ = _timed_reps(lambda: float(np.sum(np.sin(x) + y, dtype=np.float64)), 3.0, 5)
+            out["cpu_baseline"] = {"value": algo / per / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                   "sample": "numpy, full vectors, %d repetitions (%.3f s each)" % (reps, per)}
+    return out
 
 
 def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype, plain=None):
@@ -194,43 +296,118 @@ def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype, plain=None):
             "unit": "TFLOP/s", "dtype": dtype, **extra,
             "kernels": [{"kernel": l["kernel"], "kind": l["kind"], "ms": float(m)} for l, m in zip(launches, mean_ms)],
             "dot_tflops_kernel_time_only": flops / (dms * 1e-3) / 1e12,
+            # the whole step against the same peak: what a caller gets, epilogues and the launches around the products included
+            "whole_step_frac": flops / step / 1e12 / PEAK_TFLOPS[dtype_key],
             "roofline": {"bound": "mfma", "kernel": launches[big]["kernel"], "kernel_ms": float(mean_ms[big]),
                          "achieved": ach, "peak": PEAK_TFLOPS[dtype_key], "unit": "TFLOP/s",
-                         "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": _traffic(launches[big]["kernel"])}}
+                         "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": _traffic(exe, launches[big]["kernel"])}}
+
+
+def _cw_err(got, ref, bound):
+    return float(np.max(np.abs(np.asarray(got, np.float64) - np.asarray(ref, np.float64)) / np.maximum(np.asarray(bound, np.float64), 1e-300)))
 
 
 def bench_gemm(rx, client, P, steps, warmup, n=4096):
     A, B, C = [np.random.default_rng(s).normal(size=(n, n)).astype(np.float32) for s in (0, 1, 2)]
     exe = rx.xla_compile(client, P.gemm(n, n, n))
     bufs = [_upload(rx, client, a, "f32") for a in (A, B, C)]
-    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
-    return _dot_entry("gemm f32 %d^3, alpha=1.5 beta=1.2" % n, exe, secs, steps, mean_ms, "f32", "f32",
-                      plain=_time_plain(client, exe, bufs, steps, warmup))
+    secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
+    out = _dot_entry("gemm f32 %d^3, alpha=1.5 beta=1.2" % n, exe, secs, steps, mean_ms, "f32", "f32",
+                     plain=_time_plain(client, exe, bufs, steps, warmup))
+    if OPTS["check"]:
+        # buffers are the Julia arrays with dims reversed: C_raw = 1.5 B_raw A_raw + 1.2 C_raw; a sample of rows in float64,
+        # every entry against 1e-6 (1.5 |B||A| + 1.2 |C|)
+        got = rx.decode(res[0].to_host(), "f32").reshape(n, n)
+        pick = np.unique(np.concatenate([np.arange(4), np.linspace(0, n - 1, 56).astype(int), np.arange(n - 4, n)]))
+        Bs, A64 = B[pick].astype(np.float64), A.astype(np.float64)
+        want = 1.5 * (Bs @ A64) + 1.2 * C[pick].astype(np.float64)
+        err = _cw_err(got[pick], want, 1.5 * (np.abs(Bs) @ np.abs(A64)) + 1.2 * np.abs(C[pick]).astype(np.float64))
+        out["check"] = {"against": "float64 numpy, %d rows" % len(pick), "componentwise_err": err, "tolerance": 1e-6, "pass": bool(err <= 1e-6)}
+    if OPTS["cpu"]:
+        per, reps, _ = _timed_reps(lambda: np.float32(1.5) * (B @ A) + np.float32(1.2) * C, 4.0, 10)
+        out["cpu_baseline"] = {"value": (2.0 * n ** 3 + 3.0 * n * n) / per / 1e12, "unit": "TFLOP/s", "cores": _cpu_threads(), "kind": "port",
+                               "sample": "numpy float32 restatement (OpenBLAS sgemm + axpby), full %d^3, %d repetitions (%.3f s each)" % (n, reps, per)}
+    return out
+
+
+def _rows_args(I, raw, pick, dts):
+    """Oracle tensors of the sampled rows of the first operand and of the other operands whole."""
+    args = [I.Tensor.from_bytes(np.ascontiguousarray(raw[0][pick]).tobytes(), dts[0], (len(pick),) + raw[0].shape[1:])]
+    for a, dt in zip(raw[1:], dts[1:]):
+        args.append(I.Tensor.from_bytes(np.ascontiguousarray(a).tobytes(), dt, a.shape))
+    return args
 
 
 def bench_mlp(rx, client, P, steps, warmup, batch=8192, widths=(1024, 4096, 4096, 1024)):
     exe = rx.xla_compile(client, P.mlp(batch, widths))
-    bufs = [_upload(rx, client, rx.encode(np.random.default_rng(0).normal(size=(batch, widths[0])).astype(np.float32), "bf16"), "bf16")]
+    raw = [rx.encode(np.random.default_rng(0).normal(size=(batch, widths[0])).astype(np.float32), "bf16")]
     for l in range(len(widths) - 1):
         lim = np.sqrt(6.0 / (widths[l] + widths[l + 1]))
         w = np.random.default_rng(1 + l).uniform(-lim, lim, size=(widths[l], widths[l + 1])).astype(np.float32)
         b = (np.random.default_rng(4 + l).normal(size=(widths[l + 1],)) * 0.01).astype(np.float32)
-        bufs += [_upload(rx, client, rx.encode(w, "bf16"), "bf16"), _upload(rx, client, rx.encode(b, "bf16"), "bf16")]
-    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
-    return _dot_entry("mlp bf16 batch %d widths %s, bias+gelu, softmax" % (batch, "->".join(map(str, widths))), exe, secs,
-                      steps, mean_ms, "bf16", "bf16", plain=_time_plain(client, exe, bufs, steps, warmup))
+        raw += [rx.encode(w, "bf16"), rx.encode(b, "bf16")]
+    bufs = [_upload(rx, client, a, "bf16") for a in raw]
+    secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
+    out = _dot_entry("mlp bf16 batch %d widths %s, bias+gelu, softmax" % (batch, "->".join(map(str, widths))), exe, secs,
+                     steps, mean_ms, "bf16", "bf16", plain=_time_plain(client, exe, bufs, steps, warmup))
+    if OPTS["check"] or OPTS["cpu"]:
+        # rows are independent: the numpy oracle recomputes a sample of them (float64 accumulation, bf16 rounding where the
+        # module stores); that run is also the CPU baseline, scaled by rows
+        from oracle import stablehlo_interp as I
+        rows = min(256, batch)
+        pick = np.linspace(0, batch - 1, rows).astype(int)
+        args = _rows_args(I, raw, pick, ["bf16"] * len(raw))
+        text = P.mlp(rows, widths)
+        t0 = time.perf_counter()
+        ref = I.run_text(text, args, hifi=True, excess=True)[0].a.astype(np.float64)
+        per = time.perf_counter() - t0
+        if OPTS["check"]:
+            got = rx.decode(res[0].to_host(), "bf16").astype(np.float64).reshape(batch, widths[-1])
+            err = float(np.max(np.abs(got[pick] - ref)) / np.max(np.abs(ref)))
+            rowsum = float(np.max(np.abs(got.sum(axis=1) - 1.0)))
+            out["check"] = {"against": "numpy oracle, %d sampled rows; softmax row sums on every row" % rows, "max_err_over_max_entry": err,
+                            "tolerance": 2e-2, "max_row_sum_deviation": rowsum, "pass": bool(err <= 2e-2 and rowsum <= 2e-2)}
+        if OPTS["cpu"]:
+            flops = sum(l["flops"] for l in exe.launches())
+            out["cpu_baseline"] = {"value": flops * rows / batch / per / 1e12, "unit": "TFLOP/s", "cores": _cpu_threads(), "kind": "port",
+                                   "sample": "numpy oracle (float64 OpenBLAS; operands decoded to float64 before the timed run), %d of %d rows, one run of %.2f s, scaled by rows" % (rows, batch, per)}
+    return out
 
 
 def bench_fp8(rx, client, P, steps, warmup, n=8192):
     exe = rx.xla_compile(client, P.fp8_linear(n, n, n))
-    a = rx.encode(np.random.default_rng(0).normal(size=(n, n)).astype(np.float32), "bf16")
+    act = np.random.default_rng(0).normal(size=(n, n)).astype(np.float32)
+    act[0, 0] = 9.0   # the per-tensor absmax sits in a row that the check samples
+    a = rx.encode(act, "bf16")
     w = np.random.default_rng(1).normal(size=(n, n)).astype(np.float32)
     sw = np.float32(np.abs(w).max() / 448.0)
     wq = rx.encode(w / sw, "f8E4M3FN")
+    del act, w
     bufs = [_upload(rx, client, a, "bf16"), _upload(rx, client, wq, "f8E4M3FN"), _upload(rx, client, np.asarray(sw), "f32")]
-    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
-    return _dot_entry("fp8 linear %d^3 e4m3 per-tensor scales, bf16 out + RMSNorm" % n, exe, secs, steps, mean_ms, "f8",
-                      "f8E4M3FN", plain=_time_plain(client, exe, bufs, steps, warmup))
+    secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
+    out = _dot_entry("fp8 linear %d^3 e4m3 per-tensor scales, bf16 out + RMSNorm" % n, exe, secs, steps, mean_ms, "f8",
+                     "f8E4M3FN", plain=_time_plain(client, exe, bufs, steps, warmup))
+    if OPTS["check"] or OPTS["cpu"]:
+        from oracle import stablehlo_interp as I
+        rows = min(128, n)
+        args = [I.Tensor.from_bytes(np.ascontiguousarray(a[:rows]).tobytes(), "bf16", (rows, n)),
+                I.Tensor.from_bytes(np.ascontiguousarray(wq).tobytes(), "f8E4M3FN", (n, n)), I.Tensor(sw, "f32")]
+        text = P.fp8_linear(rows, n, n)
+        t0 = time.perf_counter()
+        ref = I.run_text(text, args, hifi=True, excess=True)[0].a.astype(np.float64)
+        per = time.perf_counter() - t0
+        if OPTS["check"]:
+            got = rx.decode(res[0].to_host(), "bf16").astype(np.float64).reshape(n, n)
+            err = float(np.max(np.max(np.abs(got[:rows] - ref), axis=1) / np.max(np.abs(ref), axis=1)))
+            ms = float(np.max(np.abs((got ** 2).mean(axis=1) - 1.0)))
+            out["check"] = {"against": "numpy oracle, first %d rows (the absmax is in row 0); RMSNorm mean square on every row" % rows,
+                            "max_err_over_row_max": err, "tolerance": 1e-2, "max_mean_square_deviation": ms, "pass": bool(err <= 1e-2 and ms <= 2e-2)}
+        if OPTS["cpu"]:
+            flops = sum(l["flops"] for l in exe.launches())
+            out["cpu_baseline"] = {"value": flops * rows / n / per / 1e12, "unit": "TFLOP/s", "cores": _cpu_threads(), "kind": "port",
+                                   "sample": "numpy oracle (float64 OpenBLAS; operands decoded to float64 before the timed run), %d of %d rows, one run of "
+                                             "%.2f s, scaled by rows" % (rows, n, per)}
+    return out
 
 
 # ----------------------------------------------------------------------------
@@ -369,49 +546,34 @@ def bench_polybench_linalg(rx, client, P, steps, warmup, scale=1):
             "value": 1e3 * total, "unit": "ms", "dtype": "f32", "programs": progs, "roofline": None, "higher_is_better": False}
 
 
-def cpu_baseline_stencil(P, nx=512, ny=512, nz=256, nsteps=10):
-    """The oracle's C restatement of the stencil (oracle/stencil_cpu.c, OpenMP on all host cores,
-    same bits as the GPU result) on the full grid, a bounded number of repetitions of the
-    10-timestep module.  If that library was not built, the numpy interpreter on a smaller grid."""
-    H = 3
-    try:
-        from oracle import build_c
-        lib = build_c.load()
-    except (ImportError, OSError):
-        lib = None
-    if lib is None:
-        from oracle import stablehlo_interp as I
-        nx, ny, nz, nsteps = 256, 256, 128, 1
-        full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
-        c = np.zeros(full)
-        c[H:-H, H:-H, H:-H] = np.random.default_rng(0).uniform(0, 1, (nz, ny, nx))
-        args = [I.Tensor(c, "f64")] + [I.Tensor(np.random.default_rng(s).uniform(-1, 1, full), "f64") for s in (1, 2, 3)]
-        interp = I.Interpreter(I.parse_module(P.stencil(nx, ny, nz, steps=nsteps)))
-        t0, reps = time.perf_counter(), 0
-        while True:
-            interp.run(args)
-            reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 20:
-                break
-        secs = (time.perf_counter() - t0) / reps
-        return {"value": 5.0 * nx * ny * nz * 8 * nsteps / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "numpy oracle, %dx%dx%d interior, %d timestep, %d repetitions (%.2f s each)" % (nx, ny, nz, nsteps, reps, secs)}
+def cpu_baseline_stencil_numpy(P):
+    """Fallback when the C restatement is not built: the numpy interpreter on a smaller grid, one timestep."""
+    from oracle import stablehlo_interp as I
+    H, nx, ny, nz, nsteps = 3, 256, 256, 128, 1
     full = (nz + 2 * H, ny + 2 * H, nx + 2 * H)
     c = np.zeros(full)
-    c[H:-H, H:-H, H:-H] = np.random.default_rng(0).random((nz, ny, nx))
-    u = 2.0 * np.random.default_rng(1).random(full) - 1.0
-    v, w = -u, u[::-1].copy()          # timing does not depend on the values; two generators' worth of time saved
-    build_c.stencil_steps(lib, c, u, v, w, nx, ny, nz, 1)      # touch every page once
-    t0, reps = time.perf_counter(), 0
-    while True:
-        build_c.stencil_steps(lib, c, u, v, w, nx, ny, nz, nsteps)
-        reps += 1
-        if time.perf_counter() - t0 > 12.0 or reps >= 10:
-            break
-    secs = (time.perf_counter() - t0) / reps
-    return {"value": 5.0 * nx * ny * nz * 8 * nsteps / secs / 1e9, "unit": "GB/s", "cores": int(lib.rx_oracle_threads()), "kind": "port",
-            "sample": "C restatement of the stencil (OpenMP), full %dx%dx%d grid, %d timesteps per repetition, %d repetitions (%.2f s each)"
-                      % (nx, ny, nz, nsteps, reps, secs)}
+    c[H:-H, H:-H, H:-H] = np.random.default_rng(0).uniform(0, 1, (nz, ny, nx))
+    args = [I.Tensor(c, "f64")] + [I.Tensor(np.random.default_rng(s).uniform(-1, 1, full), "f64") for s in (1, 2, 3)]
+    interp = I.Interpreter(I.parse_module(P.stencil(nx, ny, nz, steps=nsteps)))
+    secs, reps, _ = _timed_reps(lambda: interp.run(args), 10.0, 20)
+    return {"value": 5.0 * nx * ny * nz * 8 * nsteps / secs / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "numpy oracle, %dx%dx%d interior, %d timestep, %d repetitions (%.2f s each)" % (nx, ny, nz, nsteps, reps, secs)}
+
+
+def reference_probe():
+    """Is the reference itself (Julia + Reactant with its XLA-CPU backend) installed on this host?  If it is, its CPU
+    backend could be timed beside these figures; this records what was found."""
+    import shutil
+    import subprocess
+    julia = shutil.which("julia")
+    if julia is None:
+        return {"julia": None, "reactant": False, "note": "no julia on PATH: the CPU baselines are restatements (kind \"port\"), not Reactant's XLA-CPU backend"}
+    try:
+        r = subprocess.run([julia, "-e", "using Reactant; print(\"ok\")"], capture_output=True, text=True, timeout=180)
+        ok = r.returncode == 0 and "ok" in r.stdout
+    except Exception:
+        ok = False
+    return {"julia": julia, "reactant": ok, "note": "Reactant %s" % ("loads: its CPU backend can be timed with the same programs" if ok else "is not installed")}
 
 
 def main():
@@ -421,7 +583,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "polybench", "polybench_linalg"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--no-check", action="store_true", help="skip the verification of the results after the timed regions (profiling runs)")
     ap.add_argument("--small", action="store_true", help="reduced sizes (debugging only; not a valid result)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -437,6 +600,7 @@ def main():
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
              "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
+    OPTS["check"], OPTS["cpu"] = not args.no_check, not args.no_cpu
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
     copy_ms = rx._call("RxCalibrationCopy", client.default_device().handle, 1 << 30, 10)
@@ -448,21 +612,23 @@ def main():
         "roofline": main_res["roofline"],
         "copy_kernel_GBs": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9 if copy_ms > 0 else None,
     }
-    if "check" in main_res:
-        out["check"] = main_res["check"]
+    for key in ("check", "cpu_baseline", "whole_step_frac"):
+        if key in main_res:
+            out[key] = main_res[key]
     if "kernels" in main_res:
         out["kernels"] = main_res["kernels"]
     if "programs" in main_res:
         out["programs"] = main_res["programs"]
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_stencil(P) if args.workload == "stencil" else None
+        out.setdefault("cpu_baseline", None)
+        out["reference_probe"] = reference_probe()
     if not args.no_others:
         others = []
         for name in ("sinsum", "gemm", "mlp", "fp8", "stencil"):
             if name == args.workload:
                 continue
             try:
-                r = table[name](rx, client, P, max(3, min(args.steps, 5)), 2, **(small[name] if args.small else {}))
+                r = table[name](rx, client, P, args.steps, args.warmup, **(small[name] if args.small else {}))
                 r.pop("plan", None)
                 others.append(r)
             except Exception as e:  # report, never hide

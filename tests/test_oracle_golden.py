@@ -370,6 +370,29 @@ def test_c_restatement_of_the_stencil_matches_the_interpreter(embed):
     assert lib.rx_oracle_threads() >= 1
 
 
+def test_c_restatement_of_sinsum_add_is_pinned():
+    """oracle/reduce_cpu.c (a CPU baseline of the benchmark): closed forms that a dropped term, a wrong sign or a swapped
+    operand would miss (sum over a whole period of sine is the sum of y alone; sin(pi/2) = 1 counts the elements), and
+    the numpy interpreter's float64 evaluation of the same module on seeded data."""
+    from oracle import build_c
+    if not os.path.exists(build_c.SO) or os.path.getmtime(build_c.SO) < os.path.getmtime(os.path.join(os.path.dirname(build_c.SO), "..", "reduce_cpu.c")):
+        build_c.build(force=True)
+    lib = build_c.load()
+    n = 1 << 12
+    half_pi = np.full(n, np.pi / 2, dtype=np.float32)
+    assert build_c.sinsum_add(lib, half_pi, np.zeros(n, dtype=np.float32)) == pytest.approx(n, rel=1e-7)
+    assert build_c.sinsum_add(lib, half_pi, np.full(n, -3.0, dtype=np.float32)) == pytest.approx(-2.0 * n, rel=1e-7)
+    period = (2 * np.pi * np.arange(n) / n).astype(np.float32)
+    y = np.arange(n, dtype=np.float32) / n
+    assert build_c.sinsum_add(lib, period, y) == pytest.approx(float(y.astype(np.float64).sum()), abs=1e-3)
+    assert build_c.sinsum_add(lib, -half_pi, y) == pytest.approx(float(y.astype(np.float64).sum()) - n, rel=1e-6)   # sine is odd
+    x = np.random.default_rng(0).uniform(-np.pi, np.pi, 100003).astype(np.float32)
+    y = np.random.default_rng(1).uniform(-np.pi, np.pi, 100003).astype(np.float32)
+    ref = float(I.run_text(P.sinsum_add(100003), [I.tensor(x, "f32"), I.tensor(y, "f32")], hifi=True)[0].a)
+    mag = float(np.sum(np.abs(np.sin(x.astype(np.float64)) + y.astype(np.float64))))
+    assert abs(build_c.sinsum_add(lib, x, y) - ref) <= 1e-6 * mag
+
+
 def test_conditionals_against_plain_python():
     x = np.arange(8, dtype=np.float32) / 4
     for s in (2.0, -3.0):
