@@ -303,6 +303,21 @@ def _dot_entry(name, exe, secs, steps, mean_ms, dtype_key, dtype, plain=None):
                          "frac": ach / PEAK_TFLOPS[dtype_key], "traffic": _traffic(exe, launches[big]["kernel"])}}
 
 
+def _mfma_ceiling(rx, client, entry, kind):
+    """What the MFMA pipe sustains on this device with operands in registers and nothing else running (about 10 ms per
+    launch, clock settled under the power limit), beside the published peak: with pseudo-random operands, as a GEMM on
+    N(0,1) data toggles the multipliers, and with all-zero operands."""
+    try:
+        dev = client.default_device()
+        tf_r, mhz_r = rx.mfma_ceiling(dev, kind, False)
+        tf_z, mhz_z = rx.mfma_ceiling(dev, kind, True)
+    except Exception as e:  # report, never hide
+        entry["sustained_mfma"] = {"error": str(e)[:200]}
+        return
+    entry["sustained_mfma"] = {"random_operands": {"TFLOP/s": tf_r, "clock_MHz": mhz_r}, "zero_operands": {"TFLOP/s": tf_z, "clock_MHz": mhz_z},
+                               "kernel_frac_of_random": entry["roofline"]["achieved"] / tf_r if tf_r else None}
+
+
 def _cw_err(got, ref, bound):
     return float(np.max(np.abs(np.asarray(got, np.float64) - np.asarray(ref, np.float64)) / np.maximum(np.asarray(bound, np.float64), 1e-300)))
 
@@ -350,6 +365,7 @@ def bench_mlp(rx, client, P, steps, warmup, batch=8192, widths=(1024, 4096, 4096
     secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
     out = _dot_entry("mlp bf16 batch %d widths %s, bias+gelu, softmax" % (batch, "->".join(map(str, widths))), exe, secs,
                      steps, mean_ms, "bf16", "bf16", plain=_time_plain(client, exe, bufs, steps, warmup))
+    _mfma_ceiling(rx, client, out, "bf16")
     if OPTS["check"] or OPTS["cpu"]:
         # rows are independent: the numpy oracle recomputes a sample of them (float64 accumulation, bf16 rounding where the
         # module stores); that run is also the CPU baseline, scaled by rows
@@ -387,6 +403,7 @@ def bench_fp8(rx, client, P, steps, warmup, n=8192):
     secs, mean_ms, res = _time_steps(rx, client, exe, lambda prev: (bufs, [0, 0, 0]), steps, warmup)
     out = _dot_entry("fp8 linear %d^3 e4m3 per-tensor scales, bf16 out + RMSNorm" % n, exe, secs, steps, mean_ms, "f8",
                      "f8E4M3FN", plain=_time_plain(client, exe, bufs, steps, warmup))
+    _mfma_ceiling(rx, client, out, "f8")
     if OPTS["check"] or OPTS["cpu"]:
         from oracle import stablehlo_interp as I
         rows = min(128, n)
@@ -612,7 +629,7 @@ def main():
         "roofline": main_res["roofline"],
         "copy_kernel_GBs": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9 if copy_ms > 0 else None,
     }
-    for key in ("check", "cpu_baseline", "whole_step_frac"):
+    for key in ("check", "cpu_baseline", "whole_step_frac", "sustained_mfma"):
         if key in main_res:
             out[key] = main_res[key]
     if "kernels" in main_res:

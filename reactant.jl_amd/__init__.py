@@ -121,6 +121,7 @@ SIGNATURES = {
     "RxNoAllocScratchBytes": (_sz, []),
     "RxDeviceSynchronize": (None, [_vp]),
     "RxCalibrationCopy": (ctypes.c_float, [_vp, _sz, _i]),
+    "RxMfmaCeiling": (_i, [_vp, _i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
 }
 for _name, (_res, _args) in SIGNATURES.items():
     _fn = getattr(lib, _name)
@@ -470,6 +471,14 @@ def xla_compile(client, mlir_text):
     data = mlir_text.encode() if isinstance(mlir_text, str) else bytes(mlir_text)
     h = _call("ClientCompileFromText", client.handle, data, len(data), None, 0)
     return LoadedExecutable(h, client)
+
+
+def mfma_ceiling(device, kind, zero_operands=False):
+    """(TFLOP/s, average shader clock in MHz) the MFMA pipe sustains on `device` with nothing else running:
+    kind "bf16" (v_mfma_f32_32x32x16_bf16) or "f8" (v_mfma_f32_32x32x64_f8f6f4), pseudo-random or all-zero operands."""
+    tf, mhz = ctypes.c_double(), ctypes.c_double()
+    _call("RxMfmaCeiling", device.handle, {"bf16": 0, "f8": 1}[kind], 1 if zero_operands else 0, ctypes.byref(tf), ctypes.byref(mhz))
+    return tf.value, mhz.value
 
 
 def compile_offline(mlir_text, with_source=False):

@@ -314,6 +314,64 @@ __global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, 
   for (; i < n16; i += stride) dst[i] = src[i];
 }
 
+// The rate the MFMA pipe sustains when nothing else runs: every wavefront of the chip (one per SIMD) issues
+// independent MFMAs back to back on operands that stay in registers, for long enough that the clock settles under
+// the power limit.  KIND 0: v_mfma_f32_32x32x16_bf16, KIND 1: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3), the
+// instructions of the GEMM skeletons.  Operands are seeded pseudo-random values of moderate exponent, or all zero
+// (no toggling in the multipliers).  Every wavefront reports its shader-clock and real-time ticks.
+typedef float rx_probe_f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 rx_probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef int rx_probe_i32x8 __attribute__((ext_vector_type(8)));
+typedef int rx_probe_i32x4 __attribute__((ext_vector_type(4)));
+template <int KIND>
+__global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, int iters, int zero) {
+  const int tid = threadIdx.x;
+  rx_probe_i32x8 a[4], b[4];
+  unsigned s = (blockIdx.x * 256u + (unsigned)tid) * 2654435761u + 12345u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      s = s * 1664525u + 1013904223u;
+      unsigned x = KIND == 0 ? ((s & 0x807f807fu) | 0x3f003f00u) : (s & 0xbfbfbfbfu);
+      a[i][r] = zero ? 0 : (int)x;
+      s = s * 1664525u + 1013904223u;
+      x = KIND == 0 ? ((s & 0x807f807fu) | 0x3f003f00u) : (s & 0xbfbfbfbfu);
+      b[i][r] = zero ? 0 : (int)x;
+    }
+  rx_probe_bf16x8 av[4], bv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const rx_probe_i32x4 x = {a[i][0], a[i][1], a[i][2], a[i][3]}, y = {b[i][4], b[i][5], b[i][6], b[i][7]};
+    av[i] = __builtin_bit_cast(rx_probe_bf16x8, x);
+    bv[i] = __builtin_bit_cast(rx_probe_bf16x8, y);
+  }
+  rx_probe_f32x16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  const unsigned long long t0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+    if constexpr (KIND == 0) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[q & 7] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[q & 3], bv[q >> 2], acc[q & 7], 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q & 7] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[q & 3], b[q >> 1], acc[q & 7], 0, 0, 0, 0, 0, 0);
+    }
+  }
+  const unsigned long long t1 = clock64(), w1 = wall_clock64();
+  float sum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sum += acc[i][0] + acc[i][7];
+  if (sum == 1.2345f) ticks[2 * 1024] = 1;   // keeps the accumulators alive
+  if ((tid & 63) == 0) {
+    ticks[(blockIdx.x * 4 + (tid >> 6)) * 2] = t1 - t0;
+    ticks[(blockIdx.x * 4 + (tid >> 6)) * 2 + 1] = w1 - w0;
+  }
+}
+
 // Core of XLAExecuteSharded / RxExecuteTimed
 void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uint8_t* donate, int num_results, RxBuffer** results, float* launch_ms,
              RxFuture** futures, bool profile_async = false) {
@@ -934,6 +992,43 @@ RX_EXPORT void FutureAwait(RxFuture* f) {
 }
 RX_EXPORT void RxDeviceSynchronize(RxDevice* d) {
   guarded_void([&] { check_device(d); HIP_CHECK(hipSetDevice(d->ordinal)); HIP_CHECK(hipStreamSynchronize(d->stream)); });
+}
+
+RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tflops, double* clock_mhz) {
+  return guarded([&]() -> int {
+    check_device(d);
+    if (kind != 0 && kind != 1) throw Error("INVALID_ARGUMENT: kind is 0 (bf16) or 1 (f8E4M3FN)");
+    HIP_CHECK(hipSetDevice(d->ordinal));
+    Allocation ticks(d, (2 * 1024 + 8) * sizeof(unsigned long long));
+    HIP_CHECK(hipMemsetAsync(ticks.ptr, 0, (2 * 1024 + 8) * sizeof(unsigned long long), d->stream));
+    // 256 workgroups of four wavefronts: one wavefront per SIMD of the chip.  About 10 ms per launch, so that the
+    // clock has settled under the power limit; the second launch is the one that is timed.
+    const int iters = 40000;
+    const double flop_per_iter = kind == 0 ? 16 * 2.0 * 32 * 32 * 16 : 8 * 2.0 * 32 * 32 * 64;
+    hipEvent_t a, b;
+    HIP_CHECK(hipEventCreate(&a));
+    HIP_CHECK(hipEventCreate(&b));
+    auto launch = [&]() {
+      if (kind == 0) hipLaunchKernelGGL(rx_mfma_probe<0>, dim3(256), dim3(256), 0, d->stream, (unsigned long long*)ticks.ptr, iters, zero_operands);
+      else hipLaunchKernelGGL(rx_mfma_probe<1>, dim3(256), dim3(256), 0, d->stream, (unsigned long long*)ticks.ptr, iters, zero_operands);
+    };
+    launch();
+    HIP_CHECK(hipEventRecord(a, d->stream));
+    launch();
+    HIP_CHECK(hipEventRecord(b, d->stream));
+    HIP_CHECK(hipEventSynchronize(b));
+    float ms = 0;
+    HIP_CHECK(hipEventElapsedTime(&ms, a, b));
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
+    std::vector<unsigned long long> h(2 * 1024);
+    HIP_CHECK(hipMemcpy(h.data(), ticks.ptr, h.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    double c = 0, w = 0;
+    for (int i = 0; i < 1024; ++i) { c += (double)h[2 * i]; w += (double)h[2 * i + 1]; }
+    if (tflops) *tflops = flop_per_iter * iters * 1024 / (ms * 1e-3) / 1e12;
+    if (clock_mhz) *clock_mhz = w > 0 ? c / w * 100.0 : 0.0;   // the real-time counter ticks at 100 MHz
+    return 0;
+  }, 1);
 }
 
 RX_EXPORT float RxCalibrationCopy(RxDevice* d, size_t bytes, int iters) {
