@@ -30,3 +30,16 @@ RX_CHECK(rx_check_f16_nt, rx_mma_f16, 64, true, true)
 RX_CHECK(rx_check_f16_tn, rx_mma_f16, 64, false, false)
 RX_CHECK(rx_check_f8_nt, rx_mma_f8, 128, true, true)
 RX_CHECK(rx_check_f8_nn, rx_mma_f8, 128, true, false)
+
+// the direct-to-LDS body, with the 32x32 and the 16x16 MFMA shapes of 16-bit operands and the 8-bit one
+#define RX_CHECK_DL(NAME, MMA, BM, BN, BK, WM, WN, AKC, BKC)                                                              \
+  extern "C" __global__ __launch_bounds__(WM * WN * 64) void NAME(const MMA::elem* A, const MMA::elem* B, float* out) {     \
+    rx_check_epi<float, 512> epi{out};                                                                                     \
+    rx_gemm_body_dl<MMA, BM, BN, BK, WM, WN, 2, AKC, BKC, 512, 512, 512, 0, 0, false, rx_check_epi<float, 512>>(A, B, epi);  \
+  }
+RX_CHECK_DL(rx_check_dl_bf16_nn, rx_mma_bf16, 256, 256, 64, 2, 4, true, false)
+RX_CHECK_DL(rx_check_dl_bf16x16_nn, rx_mma_bf16_16, 256, 256, 64, 2, 4, true, false)
+RX_CHECK_DL(rx_check_dl_bf16x16_nt, rx_mma_bf16_16, 256, 128, 64, 2, 4, true, true)
+RX_CHECK_DL(rx_check_dl_bf16x16_tn, rx_mma_bf16_16, 128, 256, 64, 4, 2, false, false)
+RX_CHECK_DL(rx_check_dl_f16x16_tt, rx_mma_f16_16, 128, 128, 64, 2, 2, false, true)
+RX_CHECK_DL(rx_check_dl_f8_nt, rx_mma_f8, 256, 256, 128, 2, 4, true, true)

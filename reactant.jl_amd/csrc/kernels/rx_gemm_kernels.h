@@ -361,6 +361,14 @@ RX_DEV int rx_swz_tr(int row, int c) {
   else return c ^ ((((row >> 2) & 1) << 3) & (CPR - 1));                      // rows k, k+4 read in one instruction
 }
 
+//   TR tiles of 16-bit elements read by the 16 x 16 x 32 MFMA's fragments: the four 16-lane blocks of a transpose read
+//   take rows k, k+8, k+16, k+24, so one 32-lane phase reads rows k..k+3 and k+8..k+11, 32 bytes of each; every
+//   one of those eight rows gets its own 32-byte group of the 256 bytes that the 64 banks hold
+template <int CPR>
+RX_DEV int rx_swz_tr16(int row, int c) {
+  return c ^ ((((row & 3) | (((row >> 3) & 1) << 2)) << 1) & (CPR - 1));
+}
+
 template <class MMA> struct rx_frag_sw;
 
 template <> struct rx_frag_sw<rx_mma_f32> {
@@ -421,6 +429,98 @@ template <> struct rx_frag_sw<rx_mma_f8> {
   }
 };
 
+// ---------------------------------------------------------------------------
+// 16-bit operands on v_mfma_f32_16x16x32_{bf16,f16}: under the power limit of this part the 16 x 16 x 32
+// instruction sustains about 13 % more flops than 32 x 32 x 16 on the same operand data (measured with MFMAs
+// alone on register operands), and a GEMM is power-bound.  The skeleton keeps its 32 x 32 bookkeeping: one
+// "macro" step is 32 x 32 x 32 as four MFMAs, a fragment is the two 16-row halves of 32 rows (8 k per lane
+// each: lane = row % 16 + 16 * k group), and sub-accumulator (a, b) -- rows 16a.. of the column operand, rows
+// 16b.. of the row operand -- sits at registers 4 * (2a + b) .. + 3 of the 16.
+// ---------------------------------------------------------------------------
+typedef float rx_f32x4v __attribute__((ext_vector_type(4)));
+
+template <bool BF>
+struct rx_mma_16b_16 {
+  typedef rx_u16 elem;
+  typedef rx_i32x8 frag;
+  static constexpr int KS = 32;
+  static constexpr int PAD = 8;
+  RX_DEV void mma(rx_f32x16& c, const frag& rowop, const frag& colop) {
+    const rx_i32x4 r0 = {rowop[0], rowop[1], rowop[2], rowop[3]}, r1 = {rowop[4], rowop[5], rowop[6], rowop[7]};
+    const rx_i32x4 c0 = {colop[0], colop[1], colop[2], colop[3]}, c1 = {colop[4], colop[5], colop[6], colop[7]};
+    rx_f32x4v s[4] = {{c[0], c[1], c[2], c[3]}, {c[4], c[5], c[6], c[7]}, {c[8], c[9], c[10], c[11]}, {c[12], c[13], c[14], c[15]}};
+    if constexpr (BF) {
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r0), __builtin_bit_cast(rx_bf16x8, c0), s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r1), __builtin_bit_cast(rx_bf16x8, c0), s[1], 0, 0, 0);
+      s[2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r0), __builtin_bit_cast(rx_bf16x8, c1), s[2], 0, 0, 0);
+      s[3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r1), __builtin_bit_cast(rx_bf16x8, c1), s[3], 0, 0, 0);
+    } else {
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r0), __builtin_bit_cast(rx_f16x8, c0), s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r1), __builtin_bit_cast(rx_f16x8, c0), s[1], 0, 0, 0);
+      s[2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r0), __builtin_bit_cast(rx_f16x8, c1), s[2], 0, 0, 0);
+      s[3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r1), __builtin_bit_cast(rx_f16x8, c1), s[3], 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c[4 * q + e] = s[q][e];
+  }
+};
+typedef rx_mma_16b_16<true> rx_mma_bf16_16;
+typedef rx_mma_16b_16<false> rx_mma_f16_16;
+
+template <bool BF> struct rx_frag_sw<rx_mma_16b_16<BF>> {
+  template <int LD> RX_DEV rx_i32x8 kc(const RX_LDS rx_u16* t, int row0, int kk, int lane) {
+    const int r0 = row0 + (lane & 15), r1 = r0 + 16, c = (kk >> 3) + (lane >> 4);
+    struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(t + r0 * LD + rx_swz_kc<LD / 8>(r0, c) * 8),
+                                      *(const RX_LDS rx_i32x4*)(t + r1 * LD + rx_swz_kc<LD / 8>(r1, c) * 8)};
+    return __builtin_bit_cast(rx_i32x8, both);
+  }
+  template <int LD> RX_DEV rx_i32x8 tr(const RX_LDS rx_u16* t, int col0, int kk, int lane) {
+    // a 16-lane block is one k group: source lane i points at row k + i/4, columns 4*(i%4)..+3; after the transpose
+    // lane j of the block holds 4 consecutive k for column j
+    const int i = lane & 15, g = lane >> 4;
+    const int k = kk + 8 * g + (i >> 2);
+    rx_i16x4 r[4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int col = col0 + 16 * h + 4 * (i & 3);
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int kq = k + 4 * q;
+        r[2 * h + q] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(RX_LDS_PTR(rx_i16x4, t + kq * LD + rx_swz_tr16<LD / 8>(kq, col >> 3) * 8 + (col & 7)));
+      }
+    }
+    struct { rx_i16x4 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
+    return __builtin_bit_cast(rx_i32x8, all);
+  }
+};
+
+// What differs between the MFMA shapes outside the fragment readers: the swizzle of [k][o] tiles, the instruction
+// counts that the schedule hints use, and where register group rg (four consecutive n) of a 32 x 32 tile lies.
+template <class MMA> struct rx_mma_traits {
+  static constexpr int TR_SWZ = 0;        // rx_swz_tr
+  static constexpr int MFMA_PER_MMA = sizeof(typename MMA::elem) == 4 ? 4 : 1;
+  static constexpr int RD_KC = sizeof(typename MMA::elem) == 1 ? 2 : 1;
+  static constexpr int RD_TR = sizeof(typename MMA::elem) == 2 ? 2 : 4;
+  static constexpr bool RAISE_PRIO = sizeof(typename MMA::elem) == 2;
+  RX_DEV void coords(int lane, int rg, int* dm, int* dn) {
+    *dm = lane & 31;
+    *dn = 8 * rg + 4 * (lane >> 5);
+  }
+};
+template <bool BF> struct rx_mma_traits<rx_mma_16b_16<BF>> {
+  static constexpr int TR_SWZ = 1;        // rx_swz_tr16
+  static constexpr int MFMA_PER_MMA = 4;
+  static constexpr int RD_KC = 2;
+  static constexpr int RD_TR = 4;
+  static constexpr bool RAISE_PRIO = false;   // measured: raised priority costs this shape 7 % once the epilogue runs
+  RX_DEV void coords(int lane, int rg, int* dm, int* dn) {
+    *dm = 16 * (rg >> 1) + (lane & 15);
+    *dn = 16 * (rg & 1) + 4 * (lane >> 4);
+  }
+};
+
 template <int V> struct rx_int { static constexpr int value = V; };
 
 // the instruction scheduler may not move anything across this point
@@ -439,7 +539,7 @@ RX_DEV void rx_wait_vmcnt() {
 
 // Issue the direct loads of one ROWS x COLS operand tile.  Slot s (16-byte units, lane order)
 // of the LDS tile holds global chunk (row = s / CPR, c = swizzle^-1(pos = s % CPR)).
-template <typename E, int ROWS, int COLS, int NT, bool KC>
+template <typename E, int ROWS, int COLS, int NT, bool KC, int TR_SWZ = 0>
 RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0, int col0, int nrows, int ncols, RX_LDS E* lds, int tid) {
   constexpr int VE = 16 / (int)sizeof(E), CPR = COLS / VE, TOTAL = ROWS * CPR;
   static_assert(TOTAL % NT == 0, "tile must be a whole number of workgroup-wide loads");
@@ -448,7 +548,7 @@ RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0
   for (int i = 0; i < TOTAL / NT; ++i) {
     const int s = i * NT + tid;
     const int row = s / CPR, pos = s % CPR;
-    const int c = KC ? rx_swz_kc<CPR>(row, pos) : rx_swz_tr<(int)sizeof(E), CPR>(row, pos);   // XOR is its own inverse
+    const int c = KC ? rx_swz_kc<CPR>(row, pos) : (TR_SWZ == 1 ? rx_swz_tr16<CPR>(row, pos) : rx_swz_tr<(int)sizeof(E), CPR>(row, pos));   // XOR is its own inverse
     int rr = row0 + row, cc = col0 + c * VE;
     rr = rr < nrows ? rr : nrows - 1;
     cc = cc + VE <= ncols ? cc : ncols - VE;
@@ -464,6 +564,7 @@ template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, b
           int SPLIT = 1>
 RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
   typedef typename MMA::elem E;
+  typedef rx_mma_traits<MMA> TRAITS;
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BK : BM;
@@ -499,9 +600,9 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
     RX_LDS E* st = lds + (kt % S) * STAGE;
     const int k0 = kbase + kt * BK;
     if (A_KC) rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, A_GLD, m0, k0, M, K, st, tid);
-    else rx_tile_load_direct<E, A_ROWS, A_COLS, NT, false>(Ab, A_GLD, k0, m0, K, M, st, tid);
+    else rx_tile_load_direct<E, A_ROWS, A_COLS, NT, false, TRAITS::TR_SWZ>(Ab, A_GLD, k0, m0, K, M, st, tid);
     if (B_KC) rx_tile_load_direct<E, B_ROWS, B_COLS, NT, true>(Bb, B_GLD, n0, k0, N, K, st + A_SZ, tid);
-    else rx_tile_load_direct<E, B_ROWS, B_COLS, NT, false>(Bb, B_GLD, k0, n0, K, N, st + A_SZ, tid);
+    else rx_tile_load_direct<E, B_ROWS, B_COLS, NT, false, TRAITS::TR_SWZ>(Bb, B_GLD, k0, n0, K, N, st + A_SZ, tid);
   };
   constexpr int KT = K / SPLIT / BK;
   constexpr int NS = BK / MMA::KS;   // MFMA k-steps per tile
@@ -533,19 +634,20 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
   };
   // Ask the scheduler for the pattern "one MFMA, one LDS read, ..." over a step: the reads of the
   // next step trickle out under this step's MFMAs instead of going out in one burst.
-  constexpr int RD_A = A_KC ? (sizeof(E) == 1 ? 2 : 1) : (sizeof(E) == 2 ? 2 : 4);
-  constexpr int RD_B = B_KC ? (sizeof(E) == 1 ? 2 : 1) : (sizeof(E) == 2 ? 2 : 4);
+  constexpr int RD_A = A_KC ? TRAITS::RD_KC : TRAITS::RD_TR;
+  constexpr int RD_B = B_KC ? TRAITS::RD_KC : TRAITS::RD_TR;
   constexpr int NRD = TM * RD_A + TN * RD_B;
-  constexpr int NMF = TM * TN * (sizeof(E) == 4 ? 4 : 1);
+  constexpr int NMF = TM * TN * TRAITS::MFMA_PER_MMA;
   auto interleave = [&]() {
 #if RX_GEMM_INTERLEAVE
     constexpr int PAIRS = NRD < NMF ? NRD : NMF;
+    constexpr int MPP = NMF / PAIRS;   // MFMAs per LDS read when there are more MFMAs than reads
 #pragma unroll
     for (int k = 0; k < PAIRS; ++k) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+      __builtin_amdgcn_sched_group_barrier(0x008, MPP, 0);   // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);     // DS read
     }
-    if constexpr (NMF > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, NMF - PAIRS, 0);
+    if constexpr (NMF > PAIRS * MPP) __builtin_amdgcn_sched_group_barrier(0x008, NMF - PAIRS * MPP, 0);
     if constexpr (NRD > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, NRD - PAIRS, 0);
 #endif
   };
@@ -568,7 +670,7 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
     const RX_LDS E* sa = lds + (kt % S) * STAGE;
     // 16-bit operands: the wavefronts of the main loop run at raised priority (measured: the 8192 x 4096 x 4096 bf16
     // layer 5 % faster; 8-bit operands 2 % slower, so they keep the default)
-    if constexpr (sizeof(E) == 2) __builtin_amdgcn_s_setprio(3);
+    if constexpr (TRAITS::RAISE_PRIO) __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int s = 0; s + 1 < NS; ++s) {
       // keep the order "LDS reads of the next step, then the MFMAs of this step": the reads then
@@ -598,13 +700,14 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m0 + wm * (BM / WM) + 32 * i + (lane & 31);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int nb = n0 + wn * (BN / WN) + 32 * j + 4 * (lane >> 5);
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        const int n = nb + 8 * rg;
+        int dm, dn;
+        TRAITS::coords(lane, rg, &dm, &dn);
+        const int m = m0 + wm * (BM / WM) + 32 * i + dm;
+        const int n = n0 + wn * (BN / WN) + 32 * j + dn;
         if (m < M && n < N) {
           const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
           if constexpr (BATCHED) epi(v, (int)batch, m, n);

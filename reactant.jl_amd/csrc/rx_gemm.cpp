@@ -87,6 +87,11 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   if (M <= 64 && N > 64) { BM = 64; BN = 128; }
   else if (N <= 64 && M > 64) { BM = 128; BN = 64; }
   else if (M > 128 && N > 128 && ((M + 255) / 256) * ((N + 255) / 256) * batch >= 256) { BM = 256; BN = 256; WM = 2; WN = 4; }
+  // 16-bit operands whose 256x256 tiles would leave compute units idle but whose 256x128 tiles fill the chip (the
+  // 8192 x 1024 x 4096 layer of the MLP: 256 tiles, one per compute unit): 8 wavefronts, each a 128x32 block of the
+  // tile, against 128x128 tiles on 4 wavefronts 75 -> 67 us
+  else if (esize == 2 && M >= N && M > 128 && N > 64 && ((M + 255) / 256) * ((N + 127) / 128) * batch >= 256) { BM = 256; BN = 128; WM = 2; WN = 4; }
+  else if (esize == 2 && N > M && N > 128 && M > 64 && ((M + 127) / 128) * ((N + 255) / 256) * batch >= 256) { BM = 128; BN = 256; WM = 4; WN = 2; }
   else if (((M + 127) / 128) * ((N + 127) / 128) * batch * split < 128) { BM = 64; BN = 64; }
   if (const char* e = getenv("RX_GEMM_TILE")) {  // "BM,BN,WM,WN" for tuning runs
     int v[4];
@@ -115,7 +120,10 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   const int nt = WM * WN * 64;
   if (direct) {
     const int dbk = bk;
-    const int ks = ks_step;
+    // 16-bit operands take the 16x16x32 MFMA here (kernels/rx_gemm_kernels.h, rx_mma_16b_16): k step 32
+    const bool mfma16 = esize == 2 && dbk % 32 == 0 && !(getenv("RX_GEMM_MFMA32") && atoi(getenv("RX_GEMM_MFMA32")) != 0);
+    const std::string dmma = mfma16 ? mma + "_16" : mma;
+    const int ks = mfma16 ? 32 : ks_step;
     const int64_t a_ch = (int64_t)BM * dbk / ve, b_ch = (int64_t)BN * dbk / ve;
     const int64_t stage_bytes = ((int64_t)BM + BN) * dbk * esize;
     while (stages > 2 && stage_bytes * stages > 160 * 1024) --stages;
@@ -128,11 +136,11 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       c.grid[1] = (unsigned)(split > 1 ? split : batch);
       c.split = split;
       std::ostringstream t;
-      t << mma << ", " << BM << ", " << BN << ", " << dbk << ", " << WM << ", " << WN << ", " << stages << ", " << (a_kc ? "true" : "false") << ", "
+      t << dmma << ", " << BM << ", " << BN << ", " << dbk << ", " << WM << ", " << WN << ", " << stages << ", " << (a_kc ? "true" : "false") << ", "
         << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
       c.targs = t.str();
       c.skeleton = "rx_gemm_body_dl";
-      c.stype_a = mma + "::elem";
+      c.stype_a = dmma + "::elem";
       c.ok = true;
       return c;
     }
