@@ -16,7 +16,7 @@ on every launch is reported beside it.  Every workload's result is verified afte
 the stencil bit for bit against the C restatement, the others on sampled rows against float64 / the numpy oracle.
 `roofline.traffic` is read from profiles/bench_all_configs_hbm_traffic.txt (rocprofv3 counters) and is null when the
 kernel name or launch size there does not match this run's launch list.
-`--workload conv|cumsum|maxpool` run one of the windowed ops instead, `--workload polybench` /
+`--workload conv|cumsum|maxpool|colsum|transpose` run one of the windowed / layout ops instead, `--workload polybench` /
 `polybench_linalg` the reference's polybench stencil and linear-algebra suites (never part of `others`).
 """
 import argparse
@@ -483,6 +483,27 @@ def bench_maxpool(rx, client, P, steps, warmup, batch=64, c=64, hw=112):
                          4.0 * batch * c * hw * hw * 1.25, 0.0, "f32", None)
 
 
+def bench_colsum(rx, client, P, steps, warmup, n=8192):
+    """Column sums of an n x n f32 matrix (a reduction that keeps the minor dimension)."""
+    t, o = "tensor<%dx%dxf32>" % (n, n), "tensor<%dxf32>" % n
+    text = ("module { func.func @main(%%a: %s) -> %s { %%c = stablehlo.constant dense<0.0> : tensor<f32>\n"
+            " %%0 = stablehlo.reduce(%%a init: %%c) applies stablehlo.add across dimensions = [0] : (%s, tensor<f32>) -> %s\n return %%0 : %s } }" % (t, o, t, o, o))
+    exe = rx.xla_compile(client, text)
+    bufs = [_upload(rx, client, np.random.default_rng(0).normal(size=(n, n)).astype(np.float32), "f32")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0]), steps, warmup)
+    return _window_entry("column sums f32 %dx%d" % (n, n), exe, secs, steps, mean_ms, 4.0 * n * n, 0.0, "f32", None)
+
+
+def bench_transpose(rx, client, P, steps, warmup, n=8192):
+    """Transpose of an n x n f32 matrix (a map that reads its input with the two minor roles swapped)."""
+    t = "tensor<%dx%dxf32>" % (n, n)
+    text = "module { func.func @main(%%a: %s) -> %s { %%0 = stablehlo.transpose %%a, dims = [1, 0] : (%s) -> %s\n return %%0 : %s } }" % (t, t, t, t, t)
+    exe = rx.xla_compile(client, text)
+    bufs = [_upload(rx, client, np.random.default_rng(0).normal(size=(n, n)).astype(np.float32), "f32")]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0]), steps, warmup)
+    return _window_entry("transpose f32 %dx%d" % (n, n), exe, secs, steps, mean_ms, 8.0 * n * n, 0.0, "f32", None)
+
+
 def bench_polybench(rx, client, P, steps, warmup, scale=1):
     """The reference's polybench stencil suite at its own sizes (benchmark/polybench/stencil.jl:71,170,
     229,301; f32, vectorized forms as traced loops): seconds per whole program (all its time steps),
@@ -598,7 +619,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "polybench", "polybench_linalg"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-check", action="store_true", help="skip the verification of the results after the timed regions (profiling runs)")
@@ -612,10 +633,10 @@ def main():
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
-             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
+             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "colsum": bench_colsum, "transpose": bench_transpose, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
-             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
+             "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "colsum": dict(n=1024), "transpose": dict(n=1024), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
     OPTS["check"], OPTS["cpu"] = not args.no_check, not args.no_cpu
     kw = small[args.workload] if args.small else {}

@@ -316,10 +316,11 @@ __global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, 
 
 // The rate the MFMA pipe sustains when nothing else runs: every wavefront of the chip (one per SIMD) issues
 // independent MFMAs back to back on operands that stay in registers, for long enough that the clock settles under
-// the power limit.  KIND 0: v_mfma_f32_32x32x16_bf16, KIND 1: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3), the
+// the power limit.  KIND 0: v_mfma_f32_16x16x32_bf16, KIND 1: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3), the
 // instructions of the GEMM skeletons.  Operands are seeded pseudo-random values of moderate exponent, or all zero
 // (no toggling in the multipliers).  Every wavefront reports its shader-clock and real-time ticks.
 typedef float rx_probe_f32x16 __attribute__((ext_vector_type(16)));
+typedef float rx_probe_f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 rx_probe_bf16x8 __attribute__((ext_vector_type(8)));
 typedef int rx_probe_i32x8 __attribute__((ext_vector_type(8)));
 typedef int rx_probe_i32x4 __attribute__((ext_vector_type(4)));
@@ -347,15 +348,19 @@ __global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, 
     bv[i] = __builtin_bit_cast(rx_probe_bf16x8, y);
   }
   rx_probe_f32x16 acc[8];
+  rx_probe_f32x4 acc4[16];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc4[i] = rx_probe_f32x4{0.f, 0.f, 0.f, 0.f};
   const unsigned long long t0 = clock64(), w0 = wall_clock64();
   for (int it = 0; it < iters; ++it) {
     if constexpr (KIND == 0) {
+      // written as instructions so that the sixteen accumulators stay in the vector registers they start in
 #pragma unroll
-      for (int q = 0; q < 16; ++q) acc[q & 7] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[q & 3], bv[q >> 2], acc[q & 7], 0, 0, 0);
+      for (int q = 0; q < 32; ++q) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc4[q & 15]) : "v"(av[q & 3]), "v"(bv[(q >> 2) & 3]));
     } else {
 #pragma unroll
       for (int q = 0; q < 8; ++q) acc[q & 7] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[q & 3], b[q >> 1], acc[q & 7], 0, 0, 0, 0, 0, 0);
@@ -365,6 +370,8 @@ __global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, 
   float sum = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) sum += acc[i][0] + acc[i][7];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) sum += acc4[i][0] + acc4[i][3];
   if (sum == 1.2345f) ticks[2 * 1024] = 1;   // keeps the accumulators alive
   if ((tid & 63) == 0) {
     ticks[(blockIdx.x * 4 + (tid >> 6)) * 2] = t1 - t0;
@@ -1004,7 +1011,7 @@ RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tf
     // 256 workgroups of four wavefronts: one wavefront per SIMD of the chip.  About 10 ms per launch, so that the
     // clock has settled under the power limit; the second launch is the one that is timed.
     const int iters = 40000;
-    const double flop_per_iter = kind == 0 ? 16 * 2.0 * 32 * 32 * 16 : 8 * 2.0 * 32 * 32 * 64;
+    const double flop_per_iter = kind == 0 ? 32 * 2.0 * 16 * 16 * 32 : 8 * 2.0 * 32 * 32 * 64;
     hipEvent_t a, b;
     HIP_CHECK(hipEventCreate(&a));
     HIP_CHECK(hipEventCreate(&b));
