@@ -118,6 +118,25 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   else if ((M + BM - 1) / BM < rb) { const int64_t gm = (M + BM - 1) / BM; cb = (int)(rb * cb / gm); rb = (int)gm; }
   else if ((N + BN - 1) / BN < cb) { const int64_t gn = (N + BN - 1) / BN; rb = (int)(rb * cb / gn); cb = (int)gn; }
   const int nt = WM * WN * 64;
+  // 8-bit operands on 256x256 tiles: the streaming skeleton on the 16x16x128 MFMA (kernels/rx_gemm_kernels.h,
+  // rx_gemm_body_f8s).  It wants whole K tiles of 128 and operands below 4 GB (32-bit buffer offsets), and has no
+  // K-sliced form; RX_GEMM_F8_STREAM=0 keeps the 32x32x64 skeleton.
+  if (direct && esize == 1 && BM == 256 && BN == 256 && WM == 2 && WN == 4 && split == 1 && bk == 128 && K % 128 == 0 && stages == 2 &&
+      M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32) && !(getenv("RX_GEMM_F8_STREAM") && atoi(getenv("RX_GEMM_F8_STREAM")) == 0)) {
+    c.lds_bytes = (unsigned)(2 * (BM + BN) * 128);
+    c.block = nt;
+    c.grid[0] = (unsigned)gemm_grid((M + BM - 1) / BM, (N + BN - 1) / BN, rb, cb);
+    c.grid[1] = (unsigned)batch;
+    c.split = 1;
+    std::ostringstream t;
+    t << BM << ", " << BN << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false") << ", " << M << ", " << N
+      << ", " << K << ", " << rb << ", " << cb;
+    c.targs = t.str();
+    c.skeleton = "rx_gemm_body_f8s";
+    c.stype_a = "rx_u8";
+    c.ok = true;
+    return c;
+  }
   if (direct) {
     const int dbk = bk;
     // 16-bit operands take the 16x16x32 MFMA here (kernels/rx_gemm_kernels.h, rx_mma_16b_16): k step 32

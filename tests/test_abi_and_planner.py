@@ -320,3 +320,19 @@ def test_gemm_tuning_overrides_are_honoured_or_refused(monkeypatch):
     monkeypatch.setenv("RX_GEMM_TILE", "96,96,2,2")
     with pytest.raises(rx.ReactantInternalError, match="32x32 blocks"):
         rx.compile_offline(fp8)
+
+
+def test_fp8_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
+    # 8-bit operands on 256x256 tiles with whole K tiles of 128: the 16x16x128 MFMA skeleton (with_source shows the call)
+    big = P.fp8_linear(8192, 8192, 8192)
+    assert "rx_gemm_body_f8s<256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    monkeypatch.setenv("RX_GEMM_F8_STREAM", "0")
+    src = rx.compile_offline(big, with_source=True)
+    assert "rx_gemm_body_f8s<" not in src and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in src
+    monkeypatch.delenv("RX_GEMM_F8_STREAM")
+    # K = 8256 is whole 16-byte vectors but not whole K tiles of 128: not the direct-to-LDS skeletons
+    odd = rx.compile_offline(P.fp8_linear(8192, 8256, 8192), with_source=True)
+    assert "rx_gemm_body_f8s<" not in odd and "kind=gemm_f8" in odd
+    # a different stage count is a request for the ring skeleton
+    monkeypatch.setenv("RX_GEMM_STAGES", "2")
+    assert "rx_gemm_body_f8s<" in rx.compile_offline(big, with_source=True)

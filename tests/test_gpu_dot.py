@@ -93,6 +93,35 @@ def test_dot_general_mfma(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
         assert err <= 1e-5 * np.sqrt(K)
 
 
+STREAM_F8_CASES = [
+    # out, M, N, K, a_kc, b_kc, batch: 256 or more tiles of 256x256, ragged last tiles, one to five K tiles of 128
+    ("f32", 4000, 4112, 128, True, True, 0),
+    ("bf16", 4000, 4112, 256, True, False, 0),
+    ("f32", 4000, 4112, 384, False, False, 0),
+    ("bf16", 4016, 4100, 640, False, True, 0),
+    ("f32", 2048, 2064, 512, True, True, 4),
+    ("bf16", 2040, 2064, 256, True, False, 5),
+]
+
+
+@pytest.mark.parametrize("out_dt,M,N,K,a_kc,b_kc,batch", STREAM_F8_CASES)
+def test_fp8_streaming_skeleton(rx, client, out_dt, M, N, K, a_kc, b_kc, batch):
+    """8-bit operands on 256x256 tiles take the skeleton that streams one operand through the 16x16x128 MFMA: every
+    operand order, batched, rows past the end of an operand (read as zero by the buffer loads), odd and even tile counts
+    along K."""
+    dt = "f8E4M3FN"
+    text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch)
+    assert "rx_gemm_body_f8s<" in rx.compile_offline(text, with_source=True)
+    a = I.tensor(np.random.default_rng(5).normal(size=a_shape), dt)
+    b = I.tensor(np.random.default_rng(6).normal(size=b_shape), dt)
+    got, exe = gpu_run(rx, client, text, [a, b])
+    assert [l["kind"] for l in exe.launches()] == ["gemm_f8"], exe.report()
+    ref = oracle_run(text, [a, b], hifi=True)
+    assert got[0].a.shape == ref[0].a.shape
+    assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol(dt, out_dt)
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= (1e-2 if out_dt == "bf16" else 1e-5 * np.sqrt(K))
+
+
 def test_int_dot_general_reference_vectors(rx, client):
     """Known answers of the reference's own test (test/core/ops.jl:249-278)."""
     t = ("module {\n  func.func @main(%arg0: tensor<4xi32>, %arg1: tensor<4xi32>) -> tensor<i32> {\n"
