@@ -720,10 +720,11 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 }
 
 // ===========================================================================
-// 8-bit operands on v_mfma_f32_16x16x128_f8f6f4, one operand streamed.
-// Under the power limit of this part the 16 x 16 x 128 instruction sustains about 8 % more flops than 32 x 32 x 64
-// on the same data, but its fragments (16 rows x 128 k: 8 registers) do not fit the skeleton above twice.  Here the
-// wavefront's (BM/WM) x (BN/WN) tile is NA x NB blocks of 16 x 16 and a K tile is one MFMA deep (128): the NB
+// 8- and 16-bit operands on the 16 x 16 MFMA shapes, one operand streamed.
+// Under the power limit of this part v_mfma_f32_16x16x128_f8f6f4 sustains about 8 % more flops than 32 x 32 x 64
+// on the same data (16 x 16 x 32 against 32 x 32 x 16 for 16-bit operands: 13 %), but 16 x 16 x 128 fragments (16
+// rows x 128 bytes of k: 8 registers) do not fit the skeleton above twice.  Here the wavefront's (BM/WM) x (BN/WN)
+// tile is NA x NB blocks of 16 x 16 and a K tile is 128 bytes deep -- one 8-bit MFMA, two 16-bit ones: the NB
 // fragments of the B operand stay in registers for the whole K tile (two sets: the next tile's are read under the
 // last MFMAs of this one), the NA fragments of A stream through four buffers, block i + D being read from LDS while
 // block i is multiplied.  128 accumulator + 64 + 32 fragment registers.
@@ -732,7 +733,10 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 // offset, and rows past the end of the operand are outside the buffer's range and read as zero: no address
 // arithmetic and no clamping in the main loop.  Two LDS stages per operand, A stages first so that one address
 // register per operand reaches both of its stages.
-// Measured on 8192^3 (e4m3, bf16 result): 484-491 us against 538-560 us for the skeleton above on the same devices.
+// Measured against the skeleton above on the same devices: 8192^3 e4m3 484-491 us against 538-560; bf16
+// 8192 x 4096 x 4096 with bias + GELU 235-238 us against 245-257 ([m][k] x [k][n]; no difference for [m][k] x [n][k]),
+// K = 1024: 74 against 77; 256 x 128 tiles of 8192 x 1024 x 4096: 65 against 66.5.  128 x 128 tiles on four wavefronts
+// gain nothing and stay with the skeleton above.
 // ===========================================================================
 template <int I, int N, class F>
 RX_DEV void rx_static_for(F&& f) {
@@ -742,80 +746,137 @@ RX_DEV void rx_static_for(F&& f) {
   }
 }
 
-//   [k][o] tiles of 8-bit elements read by 16 x 16 x 128 fragments: one 32-lane phase of a transpose read takes rows
-//   k..k+7 and k+32..k+39, 16 bytes of each; every one of the sixteen rows gets its own 16-byte group of the 64 banks
-template <int CPR>
-RX_DEV int rx_swz_tr8_16(int row, int c) {
-  return c ^ (((row & 7) | (((row >> 5) & 1) << 3)) & (CPR - 1));
+//   [k][o] tiles read by the 16 x 16 fragments.  8-bit: one 32-lane phase of a transpose read takes rows k..k+7 and
+//   k+32..k+39, 16 bytes of each; 16-bit: rows k..k+3 and k+16..k+19, 32 bytes of each.  Every one of those rows gets
+//   its own group of the 256 bytes that the 64 banks hold.
+template <int ESZ, int CPR>
+RX_DEV int rx_swz_tr_s(int row, int c) {
+  if constexpr (ESZ == 1) return c ^ (((row & 7) | (((row >> 5) & 1) << 3)) & (CPR - 1));
+  else return c ^ ((((row & 3) | (((row >> 4) & 1) << 2)) << 1) & (CPR - 1));
 }
 
-struct rx_frag_f8_16 {
-  // 16 rows x 128 k, lane = row % 16 + 16 * (k / 32): 32 consecutive k per lane
+// Element policies: the MFMAs of one 16 x 16 x (128 bytes of k) product, and the row bit that the [k][o] swizzle takes
+// beyond the low ones.  The first operand's rows become the rows of the 16 x 16 result: a lane ends with four
+// consecutive rows of one column.
+struct rx_el_f8 {
+  typedef rx_u8 elem;
+  static constexpr int VARBIT = 5, NMF = 1;
+  RX_DEV void mma(rx_f32x4v& c, const rx_i32x8& rowop, const rx_i32x8& colop) {
+    // formats 0/0 = e4m3 x e4m3; zero scale operands select the unscaled instruction
+    c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rowop, colop, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+template <bool BF> struct rx_el_16 {
+  typedef rx_u16 elem;
+  static constexpr int VARBIT = 4, NMF = 2;
+  RX_DEV void mma(rx_f32x4v& c, const rx_i32x8& rowop, const rx_i32x8& colop) {
+    // a lane's 32 bytes are k = 16g .. 16g+15 (g = lane / 16): the first 16 bytes go to the first MFMA, the rest to
+    // the second; both operands split the same way, which is all a contraction needs
+    const rx_i32x4 r0 = {rowop[0], rowop[1], rowop[2], rowop[3]}, r1 = {rowop[4], rowop[5], rowop[6], rowop[7]};
+    const rx_i32x4 c0 = {colop[0], colop[1], colop[2], colop[3]}, c1 = {colop[4], colop[5], colop[6], colop[7]};
+    if constexpr (BF) {
+      c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r0), __builtin_bit_cast(rx_bf16x8, c0), c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(rx_bf16x8, r1), __builtin_bit_cast(rx_bf16x8, c1), c, 0, 0, 0);
+    } else {
+      c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r0), __builtin_bit_cast(rx_f16x8, c0), c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(rx_f16x8, r1), __builtin_bit_cast(rx_f16x8, c1), c, 0, 0, 0);
+    }
+  }
+};
+typedef rx_el_16<true> rx_el_bf16;
+typedef rx_el_16<false> rx_el_f16;
+
+// Fragments of 16 rows x 128 bytes of k.  LDS addresses and LD (one LDS row) are in bytes.
+template <class EL> struct rx_frag_s {
+  // [o][k] tiles: lane = row % 16 + 16 * g reads the 32 bytes at 32 * g of its row
   template <int LD> RX_DEV rx_i32x8 kc(const RX_LDS rx_u8* t, int row0, int lane) {
     const int r = row0 + (lane & 15), c = 2 * (lane >> 4);
     struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c) * 16),
                                       *(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c + 1) * 16)};
     return __builtin_bit_cast(rx_i32x8, both);
   }
-  // a 16-lane block is one k group of 32: source lane i points at row k + i/2, columns 8*(i%2)..+7; after the
-  // transpose lane j of the block holds 8 consecutive k for column j
+  // [k][o] tiles, col0 in elements: transpose reads, four per fragment
   template <int LD> RX_DEV rx_i32x8 tr(const RX_LDS rx_u8* t, int col0, int lane) {
     const int i = lane & 15, g = lane >> 4;
-    const int k = 32 * g + (i >> 1), col = col0 + 8 * (i & 1);
-    rx_i32x2 r[4];
+    if constexpr (sizeof(typename EL::elem) == 1) {
+      // a 16-lane block is one k group of 32: source lane i points at row k + i/2, columns 8*(i%2)..+7; after the
+      // transpose lane j of the block holds 8 consecutive k for column j
+      const int k = 32 * g + (i >> 1), col = col0 + 8 * (i & 1);
+      rx_i32x2 r[4];
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-      const int kh = k + 8 * h;
-      r[h] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RX_LDS rx_i32x2*)(t + kh * LD + rx_swz_tr8_16<LD / 16>(kh, col >> 4) * 16 + (col & 15)));
+      for (int h = 0; h < 4; ++h) {
+        const int kh = k + 8 * h;
+        r[h] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RX_LDS rx_i32x2*)(t + kh * LD + rx_swz_tr_s<1, LD / 16>(kh, col >> 4) * 16 + (col & 15)));
+      }
+      struct { rx_i32x2 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
+      return __builtin_bit_cast(rx_i32x8, all);
+    } else {
+      // a 16-lane block is one k group of 16: source lane i points at row k + i/4, columns 4*(i%4)..+3; after the
+      // transpose lane j of the block holds 4 consecutive k for column j.  Read h covers k = 16g + 4h .. + 3.
+      const int k = 16 * g + (i >> 2), colb = (col0 + 4 * (i & 3)) * 2;
+      rx_i16x4 r[4];
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const int kh = k + 4 * h;
+        r[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RX_LDS rx_i16x4*)(t + kh * LD + rx_swz_tr_s<2, LD / 16>(kh, colb >> 4) * 16 + (colb & 15)));
+      }
+      struct { rx_i16x4 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
+      return __builtin_bit_cast(rx_i32x8, all);
     }
-    struct { rx_i32x2 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
-    return __builtin_bit_cast(rx_i32x8, all);
   }
 };
 
-// Direct loads of one operand's ROWS x COLS byte tile per K tile.  Slot s (16-byte units, lane order) of the LDS tile
-// holds global chunk (row = s / CPR, c = swizzle^-1(pos = s % CPR)); load i of a thread covers rows i * RSTEP.. of the
-// tile, and the swizzle of a slot is the same for every i (NVAR = 1) or alternates with i (NVAR = 2).
-template <int ROWS, int COLS, int NT, bool KC>
-struct rx_dma_f8 {
+// Direct loads of one operand's tile of ROWS rows x COLS bytes per K tile.  Slot s (16-byte units, lane order) of the
+// LDS tile holds global chunk (row = s / CPR, c = swizzle^-1(pos = s % CPR)); load i of a thread covers rows
+// i * RSTEP.. of the tile.  The swizzle of a thread's slot is the same for every i, except that the [k][o] swizzle
+// takes row bit VARBIT, which i * RSTEP may toggle: then there are two offsets.
+template <class EL, int ROWS, int COLS, int NT, bool KC>
+struct rx_dma_s {
+  static constexpr int ESZ = sizeof(typename EL::elem);
   static constexpr int CPR = COLS / 16, NL = ROWS * CPR / NT, RSTEP = NT / CPR;
-  static_assert(ROWS * CPR % NT == 0 && RSTEP % 32 == 0, "tile must be a whole number of workgroup-wide loads");
-  static constexpr int NVAR = (KC || RSTEP % 64 == 0 || NL == 1) ? 1 : 2;
+  static_assert(ROWS * CPR % NT == 0 && RSTEP % 16 == 0, "tile must be a whole number of workgroup-wide loads");
+  static constexpr int VSTEP = 1 << EL::VARBIT;
+  static constexpr int NVAR = (KC || RSTEP > VSTEP || NL * RSTEP <= VSTEP) ? 1 : 2;
+  static constexpr int I1 = VSTEP / RSTEP;     // first load whose rows have the bit set
   __amdgpu_buffer_rsrc_t rsrc;
   unsigned voff[NVAR];
-  unsigned gld;
-  // base: the operand (of this batch entry), ld: its row length, o0: first row (column) of the tile, bytes: operand size
-  __device__ __forceinline__ void init(const rx_u8* base, unsigned ld, int o0, unsigned bytes, int tid) {
+  unsigned gldb;   // bytes per operand row
+  // base: the operand (of this batch entry), ldb: bytes per row of it, o0b: first row of the tile ([o][k]) or byte
+  // offset of its first column ([k][o]), bytes: operand size
+  __device__ __forceinline__ void init(const void* base, unsigned ldb, int o0b, unsigned bytes, int tid) {
     rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);
-    gld = ld;
+    gldb = ldb;
 #pragma unroll
     for (int v = 0; v < NVAR; ++v) {
-      const int s = v * NT + tid;
+      const int i0 = v * I1;
+      const int s = i0 * NT + tid;
       const int row = s / CPR, pos = s % CPR;
-      if constexpr (KC) voff[v] = (unsigned)(o0 + row) * ld + rx_swz_kc<CPR>(row, pos) * 16;          // rows are o, columns k
-      else voff[v] = (unsigned)(row - v * RSTEP) * ld + o0 + rx_swz_tr8_16<CPR>(row, pos) * 16;       // rows are k, columns o
+      if constexpr (KC) voff[v] = (unsigned)(o0b + row) * ldb + rx_swz_kc<CPR>(row, pos) * 16;
+      else voff[v] = (unsigned)(row - i0 * RSTEP) * ldb + o0b + rx_swz_tr_s<ESZ, CPR>(row, pos) * 16;
     }
   }
-  // kbyte: scalar byte offset of the K tile (k0 for [o][k] operands, k0 * ld for [k][o]); wave: wavefront index, scalar
+  // kbyte: scalar byte offset of the K tile (k0 bytes for [o][k] operands, k0 rows for [k][o]); wave: wavefront index, scalar
   __device__ __forceinline__ void issue(unsigned kbyte, RX_LDS rx_u8* lds, int wave) const {
 #pragma unroll
     for (int i = 0; i < NL; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (RX_LDS void*)(lds + (i * NT + wave * 64) * 16), 16, voff[i % NVAR], kbyte + i * RSTEP * gld, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (RX_LDS void*)(lds + (i * NT + wave * 64) * 16), 16, voff[NVAR == 1 ? 0 : ((i * RSTEP / VSTEP) & 1)],
+                                               kbyte + i * RSTEP * gldb, 0, 0);
   }
 };
 
-template <int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2>
-RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restrict__ B, const Epi& epi) {
-  constexpr int BK = 128, NBUF = 4;
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2>
+RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi) {
+  constexpr int ESZ = sizeof(typename EL::elem);
+  constexpr int BKB = 128, BK = BKB / ESZ, NBUF = 4;
   constexpr int NT = WM * WN * 64;
   constexpr int NA = BM / WM / 16, NB = BN / WN / 16;
   static_assert(NA % NBUF == 0 && D >= 1 && D < NBUF && D <= NA, "streaming depth");
-  constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BK : BM;
-  constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BK : BN;
-  constexpr int A_SZ = BM * BK, B_SZ = BN * BK;
-  typedef rx_dma_f8<A_ROWS, A_COLS, NT, A_KC> DMA_A;
-  typedef rx_dma_f8<B_ROWS, B_COLS, NT, B_KC> DMA_B;
-  static_assert((long long)M * K < (1ll << 32) && (long long)N * K < (1ll << 32), "32-bit operand offsets");
+  constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BKB : BM * ESZ;   // LDS tiles: rows x bytes
+  constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BKB : BN * ESZ;
+  constexpr int A_SZ = BM * BKB, B_SZ = BN * BKB;
+  typedef rx_dma_s<EL, A_ROWS, A_COLS, NT, A_KC> DMA_A;
+  typedef rx_dma_s<EL, B_ROWS, B_COLS, NT, B_KC> DMA_B;
+  static_assert((long long)M * K * ESZ < (1ll << 32) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
   static_assert(K % BK == 0, "whole K tiles");
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
   RX_LDS rx_u8* const ldsa = (RX_LDS rx_u8*)rx_smem;
@@ -828,9 +889,9 @@ RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restric
   if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
   const int m0 = bm * BM, n0 = bn * BN;
   const long long batch = BATCHED ? blockIdx.y : 0;
-  constexpr unsigned A_GLD = A_KC ? K : M, B_GLD = B_KC ? K : N;
+  constexpr unsigned A_GLDB = (A_KC ? K : M) * ESZ, B_GLDB = (B_KC ? K : N) * ESZ;
   constexpr int KT = K / BK;
-  constexpr unsigned KA = A_KC ? BK : BK * A_GLD, KB = B_KC ? BK : BK * B_GLD;   // byte step of one K tile
+  constexpr unsigned KA = A_KC ? BKB : BK * A_GLDB, KB = B_KC ? BKB : BK * B_GLDB;   // byte step of one K tile
 
   rx_f32x4v acc[NA][NB];
 #pragma unroll
@@ -840,8 +901,8 @@ RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restric
 
   DMA_A dma_a;
   DMA_B dma_b;
-  dma_a.init(A + batch * (long long)M * K, A_GLD, m0, (unsigned)((long long)M * K), tid);
-  dma_b.init(B + batch * (long long)N * K, B_GLD, n0, (unsigned)((long long)N * K), tid);
+  dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * K * ESZ), tid);
+  dma_b.init(B + batch * (long long)N * K, B_GLDB, B_KC ? n0 : n0 * ESZ, (unsigned)((long long)N * K * ESZ), tid);
   // tile kt lies in stage kt % 2 of both operands
   auto issue = [&](int kt, auto ST) {
     constexpr int st = decltype(ST)::value;
@@ -852,14 +913,14 @@ RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restric
   auto read_a = [&](auto BUF, auto ST, int blk) {
     const RX_LDS rx_u8* st = ldsa + decltype(ST)::value * A_SZ;
     const int o = wm * (BM / WM) + 16 * blk;
-    if constexpr (A_KC) fa[decltype(BUF)::value] = rx_frag_f8_16::kc<A_COLS>(st, o, lane);
-    else fa[decltype(BUF)::value] = rx_frag_f8_16::tr<A_COLS>(st, o, lane);
+    if constexpr (A_KC) fa[decltype(BUF)::value] = rx_frag_s<EL>::template kc<A_COLS>(st, o, lane);
+    else fa[decltype(BUF)::value] = rx_frag_s<EL>::template tr<A_COLS>(st, o, lane);
   };
   auto read_b = [&](auto J, auto ST) {
     constexpr int j = decltype(J)::value, st = decltype(ST)::value;
     const int o = wn * (BN / WN) + 16 * j;
-    if constexpr (B_KC) fb[st][j] = rx_frag_f8_16::kc<B_COLS>(ldsb + st * B_SZ, o, lane);
-    else fb[st][j] = rx_frag_f8_16::tr<B_COLS>(ldsb + st * B_SZ, o, lane);
+    if constexpr (B_KC) fb[st][j] = rx_frag_s<EL>::template kc<B_COLS>(ldsb + st * B_SZ, o, lane);
+    else fb[st][j] = rx_frag_s<EL>::template tr<B_COLS>(ldsb + st * B_SZ, o, lane);
   };
   auto publish = [&]() {
     asm volatile("" ::: "memory");   // compiler-only fences: LDS reads must not move across the barrier
@@ -879,6 +940,7 @@ RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restric
   // fragments of tile kt+1 are read with its first D blocks of A, BPB of them per block.
   constexpr int BPB = (NB + D - 1) / D;
   constexpr int RDS_A = A_KC ? 2 : 4, RDS_B = B_KC ? 2 : 4;   // LDS read instructions per fragment
+  constexpr int NMB = NB * EL::NMF;                           // MFMAs per block of A
   // MODE 0: tile kt+2 exists, 1: it may not, 2: last tile
   auto tile = [&](auto P, auto MODE, int kt) {
     constexpr int p = decltype(P)::value, mode = decltype(MODE)::value;
@@ -901,19 +963,25 @@ RX_DEV void rx_gemm_body_f8s(const rx_u8* __restrict__ A, const rx_u8* __restric
         read_a(rx_int<t % NBUF>{}, nxt, t - NA);
         rx_static_for<nb0, nb1>([&](auto J) { read_b(J, nxt); });
       }
+      // the B fragment is the row operand: a lane ends with four consecutive n of one m
       rx_static_for<0, NB>([&](auto J) {
         constexpr int j = decltype(J)::value;
-        // formats 0/0 = e4m3 x e4m3; zero scale operands select the unscaled instruction.  The B fragment is the row
-        // operand: a lane ends with four consecutive n of one m
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[p][j], fa[i % NBUF], acc[i][j], 0, 0, 0, 0, 0, 0);
+        EL::mma(acc[i][j], fb[p][j], fa[i % NBUF]);
       });
       // ask the scheduler to let this block's LDS reads trickle out between its MFMAs
       constexpr int nrd = t < NA ? RDS_A : (last ? 0 : RDS_A + (nb1 - nb0) * RDS_B);
       if constexpr (nrd == 0) {
-        __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NMB, 0);
+      } else if constexpr (nrd <= NMB) {
+        constexpr int mpr = NMB / nrd;           // MFMAs per read
+        rx_static_for<0, nrd>([&](auto Q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, mpr, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        });
+        if constexpr (NMB > nrd * mpr) __builtin_amdgcn_sched_group_barrier(0x008, NMB - nrd * mpr, 0);
       } else {
-        constexpr int per = (nrd + NB - 1) / NB;
-        rx_static_for<0, NB>([&](auto Q) {
+        constexpr int per = (nrd + NMB - 1) / NMB;
+        rx_static_for<0, NMB>([&](auto Q) {
           constexpr int q = decltype(Q)::value;
           constexpr int n = (q + 1) * per <= nrd ? per : (q * per < nrd ? nrd - q * per : 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);

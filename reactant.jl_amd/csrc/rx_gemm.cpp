@@ -118,22 +118,25 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
   else if ((M + BM - 1) / BM < rb) { const int64_t gm = (M + BM - 1) / BM; cb = (int)(rb * cb / gm); rb = (int)gm; }
   else if ((N + BN - 1) / BN < cb) { const int64_t gn = (N + BN - 1) / BN; rb = (int)(rb * cb / gn); cb = (int)gn; }
   const int nt = WM * WN * 64;
-  // 8-bit operands on 256x256 tiles: the streaming skeleton on the 16x16x128 MFMA (kernels/rx_gemm_kernels.h,
-  // rx_gemm_body_f8s).  It wants whole K tiles of 128 and operands below 4 GB (32-bit buffer offsets), and has no
-  // K-sliced form; RX_GEMM_F8_STREAM=0 keeps the 32x32x64 skeleton.
-  if (direct && esize == 1 && BM == 256 && BN == 256 && WM == 2 && WN == 4 && split == 1 && bk == 128 && K % 128 == 0 && stages == 2 &&
-      M * K < ((int64_t)1 << 32) && N * K < ((int64_t)1 << 32) && !(getenv("RX_GEMM_F8_STREAM") && atoi(getenv("RX_GEMM_F8_STREAM")) == 0)) {
+  // 8- and 16-bit operands on the eight-wavefront tiles whose wavefronts own 128 rows (256x256, 256x128): the
+  // streaming skeleton on the 16x16 MFMA shapes (kernels/rx_gemm_kernels.h, rx_gemm_body_s).  It wants whole K tiles
+  // of 128 bytes and operands below 4 GB (32-bit buffer offsets), and has no K-sliced form; RX_GEMM_STREAM=0 keeps the
+  // ring skeleton.
+  if (direct && (esize == 1 || esize == 2) && BM == 256 && (BN == 256 || BN == 128) && WM == 2 && WN == 4 && split == 1 && bk * esize == 128 &&
+      K % bk == 0 && stages == 2 && M * K * esize < ((int64_t)1 << 32) && N * K * esize < ((int64_t)1 << 32) &&
+      !(getenv("RX_GEMM_STREAM") && atoi(getenv("RX_GEMM_STREAM")) == 0) && !(getenv("RX_GEMM_MFMA32") && atoi(getenv("RX_GEMM_MFMA32")) != 0)) {
+    const std::string el = a == DT::F8E4M3FN ? "rx_el_f8" : (a == DT::BF16 ? "rx_el_bf16" : "rx_el_f16");
     c.lds_bytes = (unsigned)(2 * (BM + BN) * 128);
     c.block = nt;
     c.grid[0] = (unsigned)gemm_grid((M + BM - 1) / BM, (N + BN - 1) / BN, rb, cb);
     c.grid[1] = (unsigned)batch;
     c.split = 1;
     std::ostringstream t;
-    t << BM << ", " << BN << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false") << ", " << M << ", " << N
-      << ", " << K << ", " << rb << ", " << cb;
+    t << el << ", " << BM << ", " << BN << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false") << ", " << M
+      << ", " << N << ", " << K << ", " << rb << ", " << cb;
     c.targs = t.str();
-    c.skeleton = "rx_gemm_body_f8s";
-    c.stype_a = "rx_u8";
+    c.skeleton = "rx_gemm_body_s";
+    c.stype_a = el + "::elem";
     c.ok = true;
     return c;
   }

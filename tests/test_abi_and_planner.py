@@ -322,17 +322,21 @@ def test_gemm_tuning_overrides_are_honoured_or_refused(monkeypatch):
         rx.compile_offline(fp8)
 
 
-def test_fp8_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
-    # 8-bit operands on 256x256 tiles with whole K tiles of 128: the 16x16x128 MFMA skeleton (with_source shows the call)
+def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
+    # 8- and 16-bit operands on eight-wavefront tiles with whole K tiles of 128 bytes: the 16x16 MFMA skeleton that streams
+    # one operand (with_source shows the call)
     big = P.fp8_linear(8192, 8192, 8192)
-    assert "rx_gemm_body_f8s<256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
-    monkeypatch.setenv("RX_GEMM_F8_STREAM", "0")
+    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    mlp = rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
+    assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in mlp      # the 4096^2 layer
+    assert "rx_gemm_body_s<rx_el_bf16, 256, 128, 2, 4, true, false, 8192, 1024, 4096" in mlp      # the last layer: 256x128 tiles
+    monkeypatch.setenv("RX_GEMM_STREAM", "0")
     src = rx.compile_offline(big, with_source=True)
-    assert "rx_gemm_body_f8s<" not in src and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in src
-    monkeypatch.delenv("RX_GEMM_F8_STREAM")
+    assert "rx_gemm_body_s<" not in src and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in src
+    monkeypatch.delenv("RX_GEMM_STREAM")
     # K = 8256 is whole 16-byte vectors but not whole K tiles of 128: not the direct-to-LDS skeletons
     odd = rx.compile_offline(P.fp8_linear(8192, 8256, 8192), with_source=True)
-    assert "rx_gemm_body_f8s<" not in odd and "kind=gemm_f8" in odd
-    # a different stage count is a request for the ring skeleton
-    monkeypatch.setenv("RX_GEMM_STAGES", "2")
-    assert "rx_gemm_body_f8s<" in rx.compile_offline(big, with_source=True)
+    assert "rx_gemm_body_s<" not in odd and "kind=gemm_f8" in odd
+    # the 32x32 MFMA shapes are a request for the ring skeleton
+    monkeypatch.setenv("RX_GEMM_MFMA32", "1")
+    assert "rx_gemm_body_dl<rx_mma_bf16, 256, 256, 64" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)

@@ -93,33 +93,42 @@ def test_dot_general_mfma(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
         assert err <= 1e-5 * np.sqrt(K)
 
 
-STREAM_F8_CASES = [
-    # out, M, N, K, a_kc, b_kc, batch: 256 or more tiles of 256x256, ragged last tiles, one to five K tiles of 128
-    ("f32", 4000, 4112, 128, True, True, 0),
-    ("bf16", 4000, 4112, 256, True, False, 0),
-    ("f32", 4000, 4112, 384, False, False, 0),
-    ("bf16", 4016, 4100, 640, False, True, 0),
-    ("f32", 2048, 2064, 512, True, True, 4),
-    ("bf16", 2040, 2064, 256, True, False, 5),
+STREAM_CASES = [
+    # dt, out, M, N, K, a_kc, b_kc, batch: 256 or more eight-wavefront tiles, ragged last tiles, one to five K tiles of 128 bytes
+    ("f8E4M3FN", "f32", 4000, 4112, 128, True, True, 0),
+    ("f8E4M3FN", "bf16", 4000, 4112, 256, True, False, 0),
+    ("f8E4M3FN", "f32", 4000, 4112, 384, False, False, 0),
+    ("f8E4M3FN", "bf16", 4016, 4100, 640, False, True, 0),
+    ("f8E4M3FN", "f32", 2048, 2064, 512, True, True, 4),
+    ("f8E4M3FN", "bf16", 2040, 2064, 256, True, False, 5),
+    ("bf16", "bf16", 4000, 4104, 64, True, False, 0),
+    ("bf16", "f32", 4000, 4104, 128, True, True, 0),
+    ("bf16", "bf16", 4000, 4104, 192, False, False, 0),
+    ("f16", "f16", 4008, 4100, 320, False, True, 0),
+    ("f16", "f32", 2040, 2056, 256, True, False, 5),
+    # 256x128 tiles (the tall products whose 256x256 tiles would not fill the chip)
+    ("bf16", "bf16", 8000, 1032, 192, True, False, 0),
+    ("bf16", "f32", 8000, 1028, 128, True, True, 0),
+    ("f16", "f16", 8000, 1032, 64, False, False, 0),
+    ("bf16", "bf16", 8000, 1028, 320, False, True, 0),
 ]
 
 
-@pytest.mark.parametrize("out_dt,M,N,K,a_kc,b_kc,batch", STREAM_F8_CASES)
-def test_fp8_streaming_skeleton(rx, client, out_dt, M, N, K, a_kc, b_kc, batch):
-    """8-bit operands on 256x256 tiles take the skeleton that streams one operand through the 16x16x128 MFMA: every
-    operand order, batched, rows past the end of an operand (read as zero by the buffer loads), odd and even tile counts
-    along K."""
-    dt = "f8E4M3FN"
+@pytest.mark.parametrize("dt,out_dt,M,N,K,a_kc,b_kc,batch", STREAM_CASES)
+def test_streaming_skeleton(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
+    """8- and 16-bit operands on the eight-wavefront tiles take the skeleton that streams one operand through the 16x16
+    MFMA shapes: every operand order, batched, rows past the end of an operand (read as zero by the buffer loads), odd and
+    even tile counts along K."""
     text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch)
-    assert "rx_gemm_body_f8s<" in rx.compile_offline(text, with_source=True)
+    assert "rx_gemm_body_s<" in rx.compile_offline(text, with_source=True)
     a = I.tensor(np.random.default_rng(5).normal(size=a_shape), dt)
     b = I.tensor(np.random.default_rng(6).normal(size=b_shape), dt)
     got, exe = gpu_run(rx, client, text, [a, b])
-    assert [l["kind"] for l in exe.launches()] == ["gemm_f8"], exe.report()
+    assert [l["kind"] for l in exe.launches()] == ["gemm_" + {"bf16": "bf16", "f16": "f16", "f8E4M3FN": "f8"}[dt]], exe.report()
     ref = oracle_run(text, [a, b], hifi=True)
     assert got[0].a.shape == ref[0].a.shape
     assert contraction_err(got[0].a, ref[0].a, dot_bound(text, [a, b])) <= cw_tol(dt, out_dt)
-    assert max_rel_to_scale(got[0].a, ref[0].a) <= (1e-2 if out_dt == "bf16" else 1e-5 * np.sqrt(K))
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
 
 
 def test_int_dot_general_reference_vectors(rx, client):
