@@ -399,6 +399,37 @@ RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
   return r;
 }
 
+// A workgroup's partial result handed to another workgroup of the same launch without a fence: the value travels in
+// 32-bit pieces, each in the low half of a 64-bit word whose high half is a flag, and each word is written by one
+// relaxed device-scope atomic store -- a reader that sees the flag sees the piece.  Slots are zero before the launch;
+// the reader clears what it has read.  The wait is bounded (about a second): no correct run exhausts it.
+template <typename T>
+RX_DEV void rx_publish_partial(unsigned long long* slot, T v) {
+  constexpr int NW = (sizeof(T) + 3) / 4;
+  rx_u32 w[NW] = {};
+  __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+  for (int k = 0; k < NW; ++k) __hip_atomic_store(slot + k, (1ull << 32) | w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+RX_DEV T rx_await_partial(unsigned long long* slot) {
+  constexpr int NW = (sizeof(T) + 3) / 4;
+  rx_u32 w[NW];
+#pragma unroll
+  for (int k = 0; k < NW; ++k) {
+    unsigned long long x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spin = 0; (x >> 32) == 0 && spin < (1 << 20); ++spin) {
+      __builtin_amdgcn_s_sleep(2);
+      x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    w[k] = (rx_u32)x;
+    __hip_atomic_store(slot + k, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  T v;
+  __builtin_memcpy(&v, w, sizeof(T));
+  return v;
+}
+
 // Read-modify-write on one element in global memory (scatter with a combining update).  Sums of
 // 32/64-bit integers and floats use the hardware atomics; everything else is a compare-and-swap
 // loop on the 32- or 64-bit word (or, for 8/16-bit integers, on the aligned word that holds it).

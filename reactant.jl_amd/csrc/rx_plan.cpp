@@ -2667,14 +2667,18 @@ struct Planner {
       oo << "    out0[0] = " << Emitter::store_conv(dt, rv) << ";\n";
     };
     const bool single = opt.single_pass_reduce && G > 1;
+    const int NW = (dt == DT::F64 || info(dt).size == 8) ? 2 : 1;   // 32-bit words of one partial
     if (single) {
-      // One launch: every workgroup publishes its partial, takes a ticket, and the one that draws
-      // the last ticket combines all partials.  The ticket counter lives in a buffer that is
-      // zero when the executable is loaded and is set back to zero by that last workgroup.
-      // (device-scope fences around the ticket make the partials of other XCDs visible)
+      // One launch.  Every workgroup publishes its partial as self-validating 64-bit words -- 32 bits of the value
+      // under a flag, written by one relaxed device-scope atomic store each, so no fence (an L2 write-back on this
+      // multi-die part) is needed to order value and flag.  The workgroup with the last index then waits for every
+      // slot, clears it for the next run, and combines the partials in index order by the same fixed tree as the
+      // two-launch form: the result is bit-identical to it and does not depend on timing.  The slots live in a
+      // buffer that is zero when the executable is loaded.  The wait is bounded: a slot that never arrives (which
+      // no correct run produces) ends it after about a second with whatever the slot holds.
       std::string sig = signature(k1, em.inputs, {{ACC, "partial"}});
       sig.pop_back();
-      sig += ", unsigned* __restrict__ ticket";
+      sig += ", unsigned long long* __restrict__ slots";
       for (size_t k = 0; k < in2.size(); ++k) sig += ", " + ptr_decl(info(g.nodes[in2[k]].ty.dt).stype, true, "fin" + std::to_string(k));
       sig += ", " + ptr_decl(info(dt).stype, false, "out0") + ")";
       // the pass-1 text was written against `signature(k1, ...)`; swap the header
@@ -2684,18 +2688,12 @@ struct Planner {
       text.replace(at, old_sig.size(), sig);
       o.str("");
       o << text;
-      o << "  __shared__ bool last;\n";
-      o << "  if (threadIdx.x == 0) {\n";
-      o << "    partial[blockIdx.x] = a;\n";
-      o << "    __builtin_amdgcn_fence(__ATOMIC_RELEASE, \"agent\");\n";
-      o << "    last = atomicAdd(ticket, 1u) == gridDim.x - 1u;\n";
-      o << "  }\n";
-      o << "  __syncthreads();\n";
-      o << "  if (!last) return;\n";
-      o << "  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"agent\");\n";
-      o << "  const volatile " << ACC << "* all = partial;\n";
+      o << "  if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(slots + (size_t)blockIdx.x * " << NW << ", a);\n";
+      o << "  if (blockIdx.x != gridDim.x - 1u) return;\n";
+      // the combining workgroup keeps what it collected in the partials buffer: it reads that buffer alone
+      o << "  " << ACC << "* all = partial;\n";
+      o << "  for (int i = threadIdx.x; i < " << G << "; i += " << kBlock << ") all[i] = rx_await_partial<" << ACC << ">(slots + (size_t)i * " << NW << ");\n";
       // the init-value operands were numbered for a kernel of their own
-      std::string ib = ibody;
       std::ostringstream oc;
       combine(oc, "all");
       std::string ctext = oc.str();
@@ -2707,7 +2705,7 @@ struct Planner {
         }
       }
       o << ctext;
-      o << "    *ticket = 0u;\n  }\n}\n\n";
+      o << "  }\n}\n\n";
     } else {
       o << "  if (threadIdx.x == 0) partial[blockIdx.x] = a;\n";
       o << "}\n\n";
@@ -2737,10 +2735,10 @@ struct Planner {
     if (single) {
       BufferDesc cb;
       cb.kind = BufferDesc::Const;          // lives with the executable; zero when loaded
-      cb.ty.dt = DT::U32;
-      cb.ty.dims = {1};
-      cb.bytes = 4;
-      cb.data.assign(4, 0);
+      cb.ty.dt = DT::U64;
+      cb.ty.dims = {(int64_t)G * NW};
+      cb.bytes = (int64_t)G * NW * 8;
+      cb.data.assign((size_t)cb.bytes, 0);
       plan.buffers.push_back(cb);
       L1.args.push_back((int)plan.buffers.size() - 1);
       for (int i : in2) L1.args.push_back(buffer_for(i));

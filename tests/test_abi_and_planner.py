@@ -203,7 +203,11 @@ def test_while_with_a_data_dependent_trip_count_is_rejected(text):
 def test_single_launch_reduction_is_an_option(monkeypatch):
     monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
     rep = rx.compile_offline(P.sinsum_add(1 << 20), with_source=True)
-    assert re.findall(r"kind=(\w+)", rep) == ["reduce"] and "atomicAdd(ticket" in rep
+    # partials travel as flagged 64-bit words (no fence, no ticket); the last workgroup collects them
+    assert re.findall(r"kind=(\w+)", rep) == ["reduce"] and "rx_publish_partial<float>" in rep and "rx_await_partial<float>" in rep
+    f64 = P.sinsum_add(1 << 20).replace("f32", "f64")
+    rep = rx.compile_offline(f64, with_source=True)
+    assert "rx_publish_partial<double>(slots + (size_t)blockIdx.x * 2" in rep      # two 32-bit pieces per partial
 
 
 def _dot(lt, rt, ot, attrs):

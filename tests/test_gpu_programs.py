@@ -40,10 +40,36 @@ def test_sinsum_add_single_launch_reduction(rx, client, monkeypatch):
     monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
     one, exe1 = gpu_run(rx, client, P.sinsum_add(n), args)
     assert len(exe1.launches()) == 1 and len(exe2.launches()) == 2
-    for _ in range(3):      # the ticket counter is back at zero after every run
+    for _ in range(3):      # the slots are back at zero after every run
         again, _ = gpu_run(rx, client, P.sinsum_add(n), args, exe=exe1)
         assert again[0].a.tobytes() == one[0].a.tobytes()
     assert one[0].a.tobytes() == two[0].a.tobytes()
+
+
+@pytest.mark.parametrize("dt,op,init", [("f64", "add", "0.000000e+00"), ("i32", "maximum", "-2147483648"), ("i64", "add", "0"),
+                                        ("bf16", "minimum", "0x7F80")])
+def test_single_launch_reduction_of_other_types(rx, client, monkeypatch, dt, op, init):
+    """Partials of 8 bytes travel as two flagged words, narrower ones as one: same bits as the two-launch form, run after run."""
+    shape = (1500, 700)      # not a whole number of workgroup tiles
+    text = ("module {\n  func.func @main(%%arg0: tensor<1500x700x%s>) -> tensor<%s> {\n"
+            "    %%c = stablehlo.constant dense<%s> : tensor<%s>\n"
+            "    %%0 = stablehlo.reduce(%%arg0 init: %%c) applies stablehlo.%s across dimensions = [0, 1] : (tensor<1500x700x%s>, tensor<%s>) -> tensor<%s>\n"
+            "    return %%0 : tensor<%s>\n  }\n}\n" % (dt, dt, init, dt, op, dt, dt, dt, dt))
+    rng = np.random.default_rng(4)
+    a = I.tensor(rng.integers(-1000, 1000, shape) if dt.startswith("i") else rng.normal(size=shape), dt)
+    two, exe2 = gpu_run(rx, client, text, [a])
+    monkeypatch.setenv("RX_SINGLE_PASS_REDUCE", "1")
+    one, exe1 = gpu_run(rx, client, text, [a])
+    assert len(exe1.launches()) == 1 and len(exe2.launches()) == 2
+    assert one[0].a.tobytes() == two[0].a.tobytes()
+    for _ in range(2):
+        again, _ = gpu_run(rx, client, text, [a], exe=exe1)
+        assert again[0].a.tobytes() == one[0].a.tobytes()
+    ref = oracle_run(text, [a])
+    if dt.startswith("i") or op != "add":
+        assert one[0].a.tobytes() == ref[0].a.tobytes()
+    else:
+        assert abs(float(one[0].a) - float(ref[0].a)) <= 1e-9 * np.sum(np.abs(np.asarray(a.a, dtype=np.float64)))
 
 
 @pytest.mark.parametrize("shape,embed", [((6, 5, 4), "pad"), ((6, 5, 4), "dus"), ((32, 16, 8), "pad"),
