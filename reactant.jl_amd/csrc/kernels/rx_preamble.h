@@ -403,13 +403,33 @@ RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
 // 32-bit pieces, each in the low half of a 64-bit word whose high half is a flag, and each word is written by one
 // relaxed device-scope atomic store -- a reader that sees the flag sees the piece.  Slots are zero before the launch;
 // the reader clears what it has read.  The wait is bounded (about a second): no correct run exhausts it.
+// A flag is a nonzero 32-bit epoch: readers that clear what they read use epoch 1 throughout; where a slot has several
+// readers nothing is cleared, and the epoch changes from launch to launch instead.
 template <typename T>
-RX_DEV void rx_publish_partial(unsigned long long* slot, T v) {
+RX_DEV void rx_publish_partial(unsigned long long* slot, T v, rx_u32 epoch = 1u) {
   constexpr int NW = (sizeof(T) + 3) / 4;
   rx_u32 w[NW] = {};
   __builtin_memcpy(w, &v, sizeof(T));
 #pragma unroll
-  for (int k = 0; k < NW; ++k) __hip_atomic_store(slot + k, (1ull << 32) | w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (int k = 0; k < NW; ++k) __hip_atomic_store(slot + k, ((unsigned long long)epoch << 32) | w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// the same wait for a partial that several workgroups read: the slot keeps its value
+template <typename T>
+RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch) {
+  constexpr int NW = (sizeof(T) + 3) / 4;
+  rx_u32 w[NW];
+#pragma unroll
+  for (int k = 0; k < NW; ++k) {
+    unsigned long long x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int spin = 0; (rx_u32)(x >> 32) != epoch && spin < (1 << 16); ++spin) {
+      __builtin_amdgcn_s_sleep(2);
+      x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    w[k] = (rx_u32)x;
+  }
+  T v;
+  __builtin_memcpy(&v, w, sizeof(T));
+  return v;
 }
 template <typename T>
 RX_DEV T rx_await_partial(unsigned long long* slot) {

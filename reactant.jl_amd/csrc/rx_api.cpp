@@ -247,6 +247,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_SLAB_YTILES")) o.slab_ytiles = atoi(e);
   if (const char* e = getenv("RX_LDS2_THREADS")) o.lds2_threads = atoi(e);
   if (const char* e = getenv("RX_SINGLE_PASS_REDUCE")) o.single_pass_reduce = atoi(e) != 0;
+  if (const char* e = getenv("RX_SINGLE_PASS_SCAN")) o.single_pass_scan = atoi(e) != 0;
   if (const char* e = getenv("RX_LDS_TRANSPOSE")) o.lds_transpose = atoi(e) != 0;
   if (const char* e = getenv("RX_DOT_AS_REDUCE")) o.dot_as_reduce = atoi(e) != 0;
   if (const char* e = getenv("RX_FUSE_DOT_OPERANDS")) o.fuse_dot_operands = atoi(e) != 0;

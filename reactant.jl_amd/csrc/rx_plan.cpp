@@ -3015,6 +3015,147 @@ struct Planner {
         for (int d = a + 1; d < ty.rank(); ++d) oo << "  const " << it << " q" << d << " = 0;\n";
         oo << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << CH << ", " << n << ");\n";
       };
+      // Long rows in one launch.  A workgroup owns a chunk of T tiles, keeps its values in registers, publishes the
+      // chunk's total as flagged 64-bit words (rx_publish_partial: no fence), and builds its carry from what the
+      // chunks before it published.  So that nobody waits for a chain, totals exist at three levels: per chunk, per
+      // group of 32 chunks (summed and published by the group's last chunk) and per 32 groups (by their last chunk);
+      // a chunk's carry is the supergroups before it, the groups before it in its supergroup and the chunks before it
+      // in its group -- at most a few dozen slots, combined in an order that depends on the chunk index alone, so the
+      // result does not depend on timing.  Every workgroup waits only for lower-numbered ones, which the dispatcher
+      // started no later (workgroups start in index order on each die -- an assumption about the dispatcher, which is
+      // why this form is an option, RX_SINGLE_PASS_SCAN=1, and the two-launch form the default); waits are bounded, a
+      // wait that expires continues with what the slot holds.  Nothing is cleared between runs: a flag is the row's epoch, a word that
+      // the row's last chunk advances once its carry is complete -- by then every chunk of the row has published, so
+      // has read the epoch (one counter of finished workgroups would cost 60 ns each: atomics on one address from
+      // eight dies).  The data is read once and written once.
+      {
+        constexpr int GS = 32;
+        // tiles per chunk: 2^26 f32 takes 0.274 / 0.188 / 0.141 / 0.131 / 0.170 ms with 2 / 4 / 8 / 16 / 32 (few tiles: too
+        // many workgroups polling; many: registers)
+        const int T = getenv("RX_SCAN_T") ? std::max(1, std::min(32, atoi(getenv("RX_SCAN_T")))) : 16;
+        const int64_t sCH = (int64_t)T * TILE;
+        const int64_t sNC = (n + sCH - 1) / sCH;
+        const int64_t sNG = (sNC + GS - 1) / GS, sNS = (sNG + GS - 1) / GS, SL = sNC + sNG + sNS;
+        const int NW = (ACC == "double" || info(dt).size == 8) ? 2 : 1;
+        const int64_t slot_words = outer * SL * NW + outer;   // + one epoch word per row
+        if (opt.single_pass_scan && sNC > 1 && sNC * outer < ((int64_t)1 << 30) && slot_words * 8 <= ((int64_t)64 << 20)) {
+          auto slot_of = [&](const std::string& idx) { return "slots + (row * " + std::to_string(SL) + " + " + idx + ") * " + std::to_string(NW); };
+          std::string sg = head("@K@_scan", false, false);
+          sg.pop_back();
+          sg += std::string(em.inputs.empty() ? "" : ", ") + "unsigned long long* __restrict__ slots, " + ptr_decl(ost, false, "out0") + ")";
+          o << "// scan along the minor dimension of " << ty.str() << " (" << sNC << " chunks per row, one launch): " << describe(rn.in[0]) << "\n";
+          o << sg << " {\n";
+          o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n  __shared__ " << ACC << " wsum[" << T * (kBlock / 64) << "];\n";
+          o << "  const " << it << " c = (" << it << ")(blockIdx.x % " << sNC << "u), row = (" << it << ")(blockIdx.x / " << sNC << "u);\n";
+          decompose(o, "row", 0, a);
+          for (int d = a + 1; d < ty.rank(); ++d) o << "  const " << it << " q" << d << " = 0;\n";
+          o << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << sCH << ", " << n << ");\n";
+          o << ibody;
+          o << "  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;\n";
+          o << "  const rx_u32 epoch = (rx_u32)slots[" << outer * SL * NW << " + row] + 1u;\n";
+          o << "  " << ACC << " v[" << T << "][" << V << "], pre[" << T << "], incl[" << T << "];\n";
+          // all loads of the chunk first (rows of whole vectors), so that a workgroup has its whole chunk in flight
+          if (vecw > 1) {
+            for (auto& sd : em.direct_vecs) {
+              const int slot = sd.first;
+              const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vecw) + ">";
+              o << "  " << vt << " " << vec_name(slot, 0) << "t[" << T << "];\n";
+            }
+            o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
+            o << "    const " << it << " pb = c * " << sCH << " + t * " << TILE << " + (" << it << ")threadIdx.x * " << V << ";\n";
+            for (auto& sd : em.direct_vecs) {
+              const int slot = sd.first;
+              const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vecw) + ">";
+              o << "    " << vec_name(slot, 0) << "t[t] = " << vt << "{};\n";
+              o << "    if (pb < pend) " << vec_name(slot, 0) << "t[t] = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + row * " << n << " + pb);\n";
+            }
+            o << "  }\n";
+          }
+          o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
+          o << "    const " << it << " pb = c * " << sCH << " + t * " << TILE << " + (" << it << ")threadIdx.x * " << V << ";\n";
+          if (vecw > 1) {
+            o << "    const " << it << " lin0 = row * " << n << " + pb;\n    (void)lin0;\n";
+            for (auto& sd : em.direct_vecs) o << "    const auto& " << vec_name(sd.first, 0) << " = " << vec_name(sd.first, 0) << "t[t];\n";
+          }
+          o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      v[t][l] = " << IDENT << ";\n      if (p < pend) {\n";
+          o << "        const " << it << " j = " << jexpr << ";\n" << body;
+          o << "        v[t][l] = (" << ACC << ")" << val << ";\n      }\n    }\n";
+          o << "#pragma unroll\n    for (int l = 1; l < " << V << "; ++l) v[t][l] = " << red_apply(rn.red, dt, "v[t][l - 1]", "v[t][l]") << ";\n";
+          o << "    incl[t] = rx_wave_scan(v[t][" << V - 1 << "], " << OP << ");\n";
+          o << "    if (lane == 63) wsum[t * " << kBlock / 64 << " + w] = incl[t];\n  }\n";
+          o << "  __syncthreads();\n";
+          o << "  " << ACC << " run = " << IDENT << ";\n";
+          o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
+          o << "    " << ACC << " pt = run;\n    " << ACC << " total = wsum[t * " << kBlock / 64 << "];\n";
+          o << "#pragma unroll\n    for (int i = 0; i < " << kBlock / 64 << "; ++i) {\n      if (i < w) pt = " << red_apply(rn.red, dt, "pt", "wsum[t * " + std::to_string(kBlock / 64) + " + i]") << ";\n";
+          o << "      if (i > 0) total = " << red_apply(rn.red, dt, "total", "wsum[t * " + std::to_string(kBlock / 64) + " + i]") << ";\n    }\n";
+          o << "    const " << ACC << " below = rx_lane_from(incl[t], (rx_u32)(lane - 1) & 63u);\n";
+          o << "    if (lane > 0) pt = " << red_apply(rn.red, dt, "pt", "below") << ";\n";
+          o << "    pre[t] = pt;\n";
+          o << "    run = " << red_apply(rn.red, dt, "run", "total") << ";\n  }\n";
+          // publish, duties of the last chunk of a group / of 32 groups
+          o << "  if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of("c") << ", run, epoch);\n";
+          o << "  if (c % " << GS << " == " << GS - 1 << ") {\n";
+          o << "    " << ACC << " part = " << IDENT << ";\n";
+          o << "    if (threadIdx.x < " << GS << ") part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + threadIdx.x)") << ", epoch);\n";
+          o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
+          o << "    if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS)) << ", part, epoch);\n";
+          o << "    if ((c / " << GS << ") % " << GS << " == " << GS - 1 << ") {\n";
+          o << "      " << ACC << " gp = " << IDENT << ";\n";
+          o << "      if (threadIdx.x < " << GS << ") gp = rx_peek_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS) + " - " + std::to_string(GS - 1) + " + threadIdx.x") << ", epoch);\n";
+          o << "      gp = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(gp, " << OP << ", lds);\n";
+          o << "      if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC + sNG) + " + c / " + std::to_string(GS * GS)) << ", gp, epoch);\n";
+          o << "    }\n  }\n";
+          // carry
+          o << "  " << ACC << " carry = (" << ACC << ")" << initv << ";\n";
+          o << "  {\n    const " << it << " ns = c / " << GS * GS << ", ng = (c / " << GS << ") % " << GS << ", na = c % " << GS << ";\n";
+          o << "    " << ACC << " part = " << IDENT << ";\n";
+          o << "    for (" << it << " k = threadIdx.x; k < ns + ng + na; k += " << kBlock << ") {\n";
+          o << "      const " << it << " idx = k < ns ? " << sNC + sNG << " + k : (k < ns + ng ? " << sNC << " + ns * " << GS << " + (k - ns) : (c / " << GS << ") * " << GS << " + (k - ns - ng));\n";
+          o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch)") << ";\n    }\n";
+          o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
+          o << "    if (c != 0) carry = " << red_apply(rn.red, dt, "carry", "part") << ";\n  }\n";
+          // the row's last chunk has, through its carry, heard from every chunk of the row: the next run's epoch
+          o << "  if (c == " << sNC - 1 << " && threadIdx.x == 0) slots[" << outer * SL * NW << " + row] = (unsigned long long)(epoch == 0xffffffffu ? 0u : epoch);\n";
+          // results
+          o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
+          o << "    const " << it << " pb = c * " << sCH << " + t * " << TILE << " + (" << it << ")threadIdx.x * " << V << ";\n";
+          o << "    const " << ACC << " pt = " << red_apply(rn.red, dt, "carry", "pre[t]") << ";\n";
+          if (vecw > 1) {
+            o << "    if (pb < pend) {\n      rx_vec<" << ost << ", " << V << "> res;\n";
+            o << "#pragma unroll\n      for (int l = 0; l < " << V << "; ++l) {\n";
+            o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pt", "v[t][l]") << ";\n";
+            o << "        res.v[l] = " << Emitter::store_conv(dt, rv) << ";\n      }\n";
+            o << "      *reinterpret_cast<rx_vec<" << ost << ", " << V << ">*>(out0 + row * " << n << " + pb) = res;\n    }\n";
+          } else {
+            o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+            o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pt", "v[t][l]") << ";\n";
+            o << "        out0[row * " << n << " + (" << jexpr << ")] = " << Emitter::store_conv(dt, rv) << ";\n      }\n    }\n";
+          }
+          o << "  }\n}\n\n";
+          const std::string kb_single = finalize(o.str());
+          BufferDesc cb;
+          cb.kind = BufferDesc::Const;          // lives with the executable; zero when loaded
+          cb.ty.dt = DT::U64;
+          cb.ty.dims = {slot_words};
+          cb.bytes = slot_words * 8;
+          cb.data.assign((size_t)cb.bytes, 0);
+          plan.buffers.push_back(cb);
+          const int slots_buf = (int)plan.buffers.size() - 1;
+          Launch L;
+          L.kernel = named("@K@_scan", kb_single);
+          L.kind = "scan";
+          L.grid[0] = (unsigned)(sNC * outer);
+          L.block[0] = kBlock;
+          for (int i : em.inputs) L.args.push_back(buffer_for(i));
+          L.args.push_back(slots_buf);
+          L.args.push_back(buffer_for(root));
+          L.algo_bytes = algo_bytes(em.inputs, {root});
+          L.desc = describe(rn.in[0]) + " scan";
+          plan.launches.push_back(L);
+          return;
+        }
+      }
       o << "// scan along the minor dimension of " << ty.str() << " (" << NC << " chunk" << (NC > 1 ? "s" : "") << " per row): " << describe(rn.in[0]) << "\n";
       if (NC > 1) {
         o << head("@K@_scan_totals", true, false) << " {\n";

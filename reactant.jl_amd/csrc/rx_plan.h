@@ -55,6 +55,7 @@ struct PlanOptions {
   // device-scope release fence every workgroup needs before taking its ticket (an L2 write-back on
   // this multi-die part) made the sinsum kernel 2x slower than the two-launch form.
   bool single_pass_reduce = false;
+  bool single_pass_scan = false;     // long scanned rows in one launch (chunk totals travel as flagged words)
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS

@@ -102,6 +102,49 @@ def test_prefix_scans(rx, client, shape, dt, dim, body, rev, kinds):
         _close(got[0].a, ref[0].a, 1e-5 * np.sqrt(shape[dim]))
 
 
+# long rows in one launch: chunks of 16 tiles (16384 elements of 4 bytes), totals per chunk / 32 chunks / 1024 chunks
+ONE_LAUNCH_SCANS = [
+    ([1 << 25], "f32", 0, "add", False),         # 2048 chunks: 64 groups, 2 supergroups
+    ([3000001], "f32", 0, "add", False),          # ragged last chunk, partial last group, scalar loads (odd length)
+    ([3000000], "i32", 0, "add", True),           # from the end; integers are exact
+    ([9000000], "i64", 0, "add", False),          # two flagged words per total; more than one supergroup
+    ([1200000], "f64", 0, "multiply", False),
+    ([3, 700000], "f32", 1, "maximum", True),     # several rows, each with its own slots
+    ([5, 40000], "bf16", 1, "add", False),
+    ([2, 16385], "f32", 1, "add", False),         # two chunks, the second of one element
+]
+
+
+@pytest.mark.parametrize("shape,dt,dim,body,rev", ONE_LAUNCH_SCANS)
+def test_prefix_scans_of_long_rows_in_one_launch(rx, client, monkeypatch, shape, dt, dim, body, rev):
+    """The one-launch form of a scan over long rows against the oracle and against the two-launch form (bit for bit where
+    the operation is exact), three runs of one executable: the slots are cleared by the run that used them."""
+    text = NN.cumulative(shape, dt, dim, body, rev)
+    args = _args([shape], dt, seed=9, lo=(0.999999, 1.000001) if body == "multiply" else None)
+    monkeypatch.setenv("RX_SINGLE_PASS_SCAN", "0")
+    two, exe2 = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe2.launches()] == ["scan_totals", "scan"]
+    monkeypatch.setenv("RX_SINGLE_PASS_SCAN", "1")
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["scan"]
+    ref = oracle_run(text, args, hifi=True)
+    exact = dt[0] == "i" or body in ("maximum", "minimum")
+    for run in range(3):
+        if exact:
+            assert np.array_equal(got[0].a, ref[0].a) and got[0].a.tobytes() == two[0].a.tobytes()
+        elif dt == "bf16":
+            _close(got[0].a, ref[0].a, 1e-2)
+        elif dt == "f64":
+            _close(got[0].a, ref[0].a, 1e-12)
+        else:
+            _close(got[0].a, ref[0].a, 1e-5 * np.sqrt(shape[dim]))
+        if run == 0:
+            first = got[0].a.tobytes()
+        else:
+            assert got[0].a.tobytes() == first        # fixed combination order: the same bits every run
+        got, _ = gpu_run(rx, client, text, args, exe=exe)
+
+
 def test_scan_of_a_fused_producer_and_into_a_consumer(rx, client):
     """cumsum(abs2.(x)) ./ sum: the producer is evaluated inside the scan kernels, the consumer reads its result."""
     t = ("module {\n func.func @main(%arg0: tensor<64x5000xf32>) -> tensor<64x5000xf32> {\n"
