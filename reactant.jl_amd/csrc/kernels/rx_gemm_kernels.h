@@ -747,12 +747,12 @@ RX_DEV void rx_static_for(F&& f) {
 }
 
 //   [k][o] tiles read by the 16 x 16 fragments.  8-bit: one 32-lane phase of a transpose read takes rows k..k+7 and
-//   k+32..k+39, 16 bytes of each; 16-bit: rows k..k+3 and k+16..k+19, 32 bytes of each.  Every one of those rows gets
+//   k+16..k+23, 16 bytes of each; 16-bit: rows k..k+3 and k+8..k+11, 32 bytes of each.  Every one of those rows gets
 //   its own group of the 256 bytes that the 64 banks hold.
 template <int ESZ, int CPR>
 RX_DEV int rx_swz_tr_s(int row, int c) {
-  if constexpr (ESZ == 1) return c ^ (((row & 7) | (((row >> 5) & 1) << 3)) & (CPR - 1));
-  else return c ^ ((((row & 3) | (((row >> 4) & 1) << 2)) << 1) & (CPR - 1));
+  if constexpr (ESZ == 1) return c ^ (((row & 7) | (((row >> 4) & 1) << 3)) & (CPR - 1));
+  else return rx_swz_tr16<CPR>(row, c);
 }
 
 // Element policies: the MFMAs of one 16 x 16 x (128 bytes of k) product, and the row bit that the [k][o] swizzle takes
@@ -760,7 +760,7 @@ RX_DEV int rx_swz_tr_s(int row, int c) {
 // consecutive rows of one column.
 struct rx_el_f8 {
   typedef rx_u8 elem;
-  static constexpr int VARBIT = 5, NMF = 1;
+  static constexpr int VARBIT = 4, NMF = 1;
   RX_DEV void mma(rx_f32x4v& c, const rx_i32x8& rowop, const rx_i32x8& colop) {
     // formats 0/0 = e4m3 x e4m3; zero scale operands select the unscaled instruction
     c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(rowop, colop, c, 0, 0, 0, 0, 0, 0);
@@ -768,10 +768,10 @@ struct rx_el_f8 {
 };
 template <bool BF> struct rx_el_16 {
   typedef rx_u16 elem;
-  static constexpr int VARBIT = 4, NMF = 2;
+  static constexpr int VARBIT = 3, NMF = 2;
   RX_DEV void mma(rx_f32x4v& c, const rx_i32x8& rowop, const rx_i32x8& colop) {
-    // a lane's 32 bytes are k = 16g .. 16g+15 (g = lane / 16): the first 16 bytes go to the first MFMA, the rest to
-    // the second; both operands split the same way, which is all a contraction needs
+    // a lane's first 16 bytes are k = 8g .. 8g+7 (g = lane / 16) for the first MFMA, its second 16 bytes
+    // k = 32 + 8g .. for the second
     const rx_i32x4 r0 = {rowop[0], rowop[1], rowop[2], rowop[3]}, r1 = {rowop[4], rowop[5], rowop[6], rowop[7]};
     const rx_i32x4 c0 = {colop[0], colop[1], colop[2], colop[3]}, c1 = {colop[4], colop[5], colop[6], colop[7]};
     if constexpr (BF) {
@@ -786,38 +786,42 @@ template <bool BF> struct rx_el_16 {
 typedef rx_el_16<true> rx_el_bf16;
 typedef rx_el_16<false> rx_el_f16;
 
-// Fragments of 16 rows x 128 bytes of k.  LDS addresses and LD (one LDS row) are in bytes.
+// Fragments of 16 rows x 128 bytes of k.  LDS addresses and LD (one LDS row) are in bytes.  A lane (row % 16, g = lane
+// / 16) holds the 16 bytes at 16 g and the 16 bytes at 64 + 16 g of its row: the four 16-lane blocks of one 16-byte
+// read then take neighbouring chunks, which the XOR swizzle keeps on different banks (blocks two chunks apart, as 32
+// contiguous bytes per lane would have it, collide two ways: measured with SQ_LDS_BANK_CONFLICT).  Which k a lane holds
+// does not matter to a contraction as long as both operands agree, and the transposing reads below do.
 template <class EL> struct rx_frag_s {
-  // [o][k] tiles: lane = row % 16 + 16 * g reads the 32 bytes at 32 * g of its row
+  // [o][k] tiles
   template <int LD> RX_DEV rx_i32x8 kc(const RX_LDS rx_u8* t, int row0, int lane) {
-    const int r = row0 + (lane & 15), c = 2 * (lane >> 4);
+    const int r = row0 + (lane & 15), c = lane >> 4;
     struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c) * 16),
-                                      *(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c + 1) * 16)};
+                                      *(const RX_LDS rx_i32x4*)(t + r * LD + rx_swz_kc<LD / 16>(r, c + 4) * 16)};
     return __builtin_bit_cast(rx_i32x8, both);
   }
   // [k][o] tiles, col0 in elements: transpose reads, four per fragment
   template <int LD> RX_DEV rx_i32x8 tr(const RX_LDS rx_u8* t, int col0, int lane) {
     const int i = lane & 15, g = lane >> 4;
     if constexpr (sizeof(typename EL::elem) == 1) {
-      // a 16-lane block is one k group of 32: source lane i points at row k + i/2, columns 8*(i%2)..+7; after the
-      // transpose lane j of the block holds 8 consecutive k for column j
-      const int k = 32 * g + (i >> 1), col = col0 + 8 * (i & 1);
+      // source lane i of a 16-lane block points at row k + i/2, columns 8*(i%2)..+7; after the transpose lane j of the
+      // block holds 8 consecutive k for column j.  Read h covers k = 16g + 8(h%2) + 64(h/2) .. + 7.
+      const int k = 16 * g + (i >> 1), col = col0 + 8 * (i & 1);
       rx_i32x2 r[4];
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
-        const int kh = k + 8 * h;
+        const int kh = k + 8 * (h & 1) + 64 * (h >> 1);
         r[h] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((RX_LDS rx_i32x2*)(t + kh * LD + rx_swz_tr_s<1, LD / 16>(kh, col >> 4) * 16 + (col & 15)));
       }
       struct { rx_i32x2 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
       return __builtin_bit_cast(rx_i32x8, all);
     } else {
-      // a 16-lane block is one k group of 16: source lane i points at row k + i/4, columns 4*(i%4)..+3; after the
-      // transpose lane j of the block holds 4 consecutive k for column j.  Read h covers k = 16g + 4h .. + 3.
-      const int k = 16 * g + (i >> 2), colb = (col0 + 4 * (i & 3)) * 2;
+      // source lane i of a 16-lane block points at row k + i/4, columns 4*(i%4)..+3; after the transpose lane j of the
+      // block holds 4 consecutive k for column j.  Read h covers k = 8g + 4(h%2) + 32(h/2) .. + 3.
+      const int k = 8 * g + (i >> 2), colb = (col0 + 4 * (i & 3)) * 2;
       rx_i16x4 r[4];
 #pragma unroll
       for (int h = 0; h < 4; ++h) {
-        const int kh = k + 4 * h;
+        const int kh = k + 4 * (h & 1) + 32 * (h >> 1);
         r[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RX_LDS rx_i16x4*)(t + kh * LD + rx_swz_tr_s<2, LD / 16>(kh, colb >> 4) * 16 + (colb & 15)));
       }
       struct { rx_i16x4 a, b, c, d; } all = {r[0], r[1], r[2], r[3]};
