@@ -136,6 +136,10 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       << ", " << N << ", " << K << ", " << rb << ", " << cb;
     c.targs = t.str();
     c.skeleton = "rx_gemm_body_s";
+    if (const char* e = getenv("RX_GEMM_STREAM_DEPTH")) {
+      if (atoi(e) < 1 || atoi(e) > 3) refuse("RX_GEMM_STREAM_DEPTH is 1, 2 or 3");
+      c.depth = atoi(e);
+    }
     c.stype_a = el + "::elem";
     c.ok = true;
     return c;
@@ -210,6 +214,7 @@ std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const s
   o << "  " << c.skeleton << "<" << c.targs << ", " << (batched ? "true" : "false") << ", " << kbase << "_epi";
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn" : fa.type) << ", " << (fb.type.empty() ? "rx_no_fn" : fb.type);
   if (c.split > 1) o << ", " << c.split;
+  if (c.depth > 0) o << ", " << c.depth;
   o << ">(A, B, epi";
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn()" : "la") << ", " << (fb.type.empty() ? "rx_no_fn()" : "lb");
   o << ");\n}\n\n";
