@@ -617,8 +617,8 @@ def reference_probe():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
