@@ -6,6 +6,7 @@
 // A file whose first line is "// expect-error" must be rejected by the importer or the planner with a
 // message (a thrown rx error is the expected outcome); any other file must plan.
 #include <cstdio>
+#include <cstdlib>
 #include <fstream>
 #include <sstream>
 #include <string>
@@ -32,7 +33,10 @@ int main(int argc, char** argv) {
     const bool expect_error = text.rfind("// expect-error", 0) == 0;
     try {
       rx::Graph g = rx::parse_module(text.data(), text.size());
-      rx::Plan p = rx::make_plan(g, rx::PlanOptions());
+      rx::PlanOptions opt;
+      if (const char* e = std::getenv("RX_SINGLE_PASS_REDUCE")) opt.single_pass_reduce = std::atoi(e) != 0;   // the optional one-launch forms
+      if (const char* e = std::getenv("RX_SINGLE_PASS_SCAN")) opt.single_pass_scan = std::atoi(e) != 0;
+      rx::Plan p = rx::make_plan(g, opt);
       if (expect_error) {
         std::fprintf(stderr, "%s: planned, but a rejection was expected\n", argv[i]);
         ++failures;

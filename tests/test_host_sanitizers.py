@@ -73,9 +73,11 @@ def test_importer_and_planner_are_clean_under_asan_and_ubsan(tmp_path):
         f = tmp_path / (name + ".mlir")
         f.write_text("// expect-error\n" + text)
         files.append(str(f))
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
-    r = subprocess.run([HOSTCHECK] + files, capture_output=True, text=True, timeout=900, env=env)
-    report = r.stdout[-3000:] + "\n" + r.stderr[-6000:]
-    assert "AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr and "LeakSanitizer" not in r.stderr, report
-    assert r.returncode == 0, report
-    assert r.stdout.count("launches") == len(mods) and r.stdout.count("rejected as expected") == len(rejected), report
+    # once with the default plan options, once with the optional one-launch reductions and scans
+    for extra in ({}, {"RX_SINGLE_PASS_REDUCE": "1", "RX_SINGLE_PASS_SCAN": "1"}):
+        env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1", **extra)
+        r = subprocess.run([HOSTCHECK] + files, capture_output=True, text=True, timeout=900, env=env)
+        report = r.stdout[-3000:] + "\n" + r.stderr[-6000:]
+        assert "AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr and "LeakSanitizer" not in r.stderr, report
+        assert r.returncode == 0, report
+        assert r.stdout.count("launches") == len(mods) and r.stdout.count("rejected as expected") == len(rejected), report
