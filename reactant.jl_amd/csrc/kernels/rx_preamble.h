@@ -413,18 +413,20 @@ RX_DEV void rx_publish_partial(unsigned long long* slot, T v, rx_u32 epoch = 1u)
 #pragma unroll
   for (int k = 0; k < NW; ++k) __hip_atomic_store(slot + k, ((unsigned long long)epoch << 32) | w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// the same wait for a partial that several workgroups read: the slot keeps its value
+// the same wait for a partial that several workgroups read: the slot keeps its value.  `limit` polls (about 1.5 us each);
+// a wait that expires sets the fault word (pinned host memory, checked by the host) and continues with what the slot holds
 template <typename T>
-RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch) {
+RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch, int limit, unsigned* fault) {
   constexpr int NW = (sizeof(T) + 3) / 4;
   rx_u32 w[NW];
 #pragma unroll
   for (int k = 0; k < NW; ++k) {
     unsigned long long x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    for (int spin = 0; (rx_u32)(x >> 32) != epoch && spin < (1 << 16); ++spin) {
+    for (int spin = 0; (rx_u32)(x >> 32) != epoch && spin < limit; ++spin) {
       __builtin_amdgcn_s_sleep(2);
       x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    if ((rx_u32)(x >> 32) != epoch) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     w[k] = (rx_u32)x;
   }
   T v;

@@ -77,6 +77,10 @@ struct RxDevice {
   int index = 0;         // position in the client's device list
   hipStream_t stream = nullptr;
   void* scratch_ptr = nullptr;   // this device's copy of `scratch` (RxExecuteNoAlloc)
+  // A word in pinned host memory that kernels can write: set when a kernel's bounded wait for another workgroup of
+  // its launch expired (its results are then invalid).  Checked wherever the host has waited for the device.
+  unsigned* fault_host = nullptr;
+  void* fault_dev = nullptr;
   std::mutex scratch_mu;         // held while a call that uses it queues its kernels
   std::string kind;
   std::string arch;
@@ -182,6 +186,16 @@ struct RxFuture {
   RxDevice* device = nullptr;
   std::string error;
 };
+
+// Called after the host has waited for a device: a kernel whose wait for another workgroup expired has set the word.
+static void check_fault(RxDevice* d) {
+  if (!d || !d->fault_host) return;
+  volatile unsigned* w = d->fault_host;
+  if (*w == 0) return;
+  *w = 0;
+  throw Error("INTERNAL: a kernel's bounded wait for another workgroup of its launch expired; results produced since the last "
+              "synchronization are invalid (RX_SINGLE_PASS_SCAN=0 selects the scan that does not wait)");
+}
 
 struct RxExecutable {
   RxClient* client = nullptr;
@@ -437,6 +451,7 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
     ptrs.clear();
     argv.clear();
     for (int b : L.args) {
+      if (P.buffers[b].kind == rx::BufferDesc::Fault) { ptrs.push_back(dev->fault_dev); continue; }
       if (!bufs[b]) {
         const auto& B = P.buffers[b];
         if (B.kind == rx::BufferDesc::Param || B.kind == rx::BufferDesc::Const) throw Error("internal: unbound input buffer");
@@ -571,6 +586,9 @@ RX_EXPORT RxClient* MakeGPUClient(int node_id, int num_nodes, int64_t* allowed_d
       d->bytes_limit = (int64_t)((memory_fraction > 0 && memory_fraction <= 1 ? memory_fraction : 1.0) * (double)tot);
       HIP_CHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
       HIP_CHECK(hipGetSymbolAddress(&d->scratch_ptr, HIP_SYMBOL(scratch)));   // with this device current: its own copy
+      HIP_CHECK(hipHostMalloc((void**)&d->fault_host, 64, hipHostMallocMapped));
+      *d->fault_host = 0;
+      HIP_CHECK(hipHostGetDevicePointer(&d->fault_dev, d->fault_host, 0));
       reg_add(d.get());
       c->devices.push_back(std::move(d));
     }
@@ -594,6 +612,7 @@ RX_EXPORT void FreeClient(RxClient* c) {
       (void)hipStreamSynchronize(d->stream);
       d->drain(true);
       (void)hipStreamDestroy(d->stream);
+      if (d->fault_host) { (void)hipHostFree(d->fault_host); d->fault_host = nullptr; d->fault_dev = nullptr; }
       reg_del(d.get());
     }
     reg_del(c);
@@ -696,6 +715,7 @@ RX_EXPORT void BufferToHost(RxBuffer* b, void* data) {
     HIP_CHECK(hipSetDevice(b->device->ordinal));
     HIP_CHECK(hipMemcpyAsync(data, b->mem->ptr, bytes, hipMemcpyDeviceToHost, b->device->stream));
     HIP_CHECK(hipStreamSynchronize(b->device->stream));
+    check_fault(b->device);
   });
 }
 
@@ -720,6 +740,7 @@ RX_EXPORT void CopyFromBuffer(RxClient* c, RxBuffer* b, void* data, size_t offse
     HIP_CHECK(hipSetDevice(b->device->ordinal));
     HIP_CHECK(hipMemcpyAsync(data, (char*)b->mem->ptr + offset, size, hipMemcpyDeviceToHost, b->device->stream));
     HIP_CHECK(hipStreamSynchronize(b->device->stream));
+    check_fault(b->device);
   });
 }
 
@@ -936,6 +957,7 @@ RX_EXPORT int RxExecuteNoAlloc(RxExecutable* ex, int num_args, RxBuffer** args, 
       const auto& B = P.buffers[b];
       if (B.kind == rx::BufferDesc::Param) where[b] = args[B.param_index]->mem->ptr;
       else if (B.kind == rx::BufferDesc::Const) where[b] = ex->consts[b]->ptr;
+      else if (B.kind == rx::BufferDesc::Fault) where[b] = dev->fault_dev;
       else if (first_result[b] >= 0) where[b] = results[first_result[b]]->mem->ptr;
       else if (B.first_def >= 0 || B.last_use >= 0) {
         where[b] = (char*)dev->scratch_ptr + used;
@@ -994,7 +1016,7 @@ RX_EXPORT uint8_t FutureIsReady(RxFuture* f) {
     if (!f || !reg_has(f)) throw Error("INVALID_ARGUMENT: null or foreign future handle");
     future_event(f);
     hipError_t e = hipEventQuery(f->ev);
-    if (e == hipSuccess) return 1;
+    if (e == hipSuccess) { check_fault(f->device); return 1; }
     if (e == hipErrorNotReady) { (void)hipGetLastError(); return 0; }
     throw Error(std::string("execution failed: ") + hipGetErrorString(e));
   }, 0);
@@ -1005,10 +1027,11 @@ RX_EXPORT void FutureAwait(RxFuture* f) {
     future_event(f);
     hipError_t e = hipEventSynchronize(f->ev);
     if (e != hipSuccess) throw Error(std::string("execution failed: ") + hipGetErrorString(e));
+    check_fault(f->device);
   });
 }
 RX_EXPORT void RxDeviceSynchronize(RxDevice* d) {
-  guarded_void([&] { check_device(d); HIP_CHECK(hipSetDevice(d->ordinal)); HIP_CHECK(hipStreamSynchronize(d->stream)); });
+  guarded_void([&] { check_device(d); HIP_CHECK(hipSetDevice(d->ordinal)); HIP_CHECK(hipStreamSynchronize(d->stream)); check_fault(d); });
 }
 
 RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tflops, double* clock_mhz) {

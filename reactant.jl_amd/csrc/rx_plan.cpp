@@ -3022,9 +3022,10 @@ struct Planner {
       // a chunk's carry is the supergroups before it, the groups before it in its supergroup and the chunks before it
       // in its group -- at most a few dozen slots, combined in an order that depends on the chunk index alone, so the
       // result does not depend on timing.  Every workgroup waits only for lower-numbered ones, which the dispatcher
-      // started no later (workgroups start in index order on each die -- an assumption about the dispatcher, which is
-      // why this form is an option, RX_SINGLE_PASS_SCAN=1, and the two-launch form the default); waits are bounded, a
-      // wait that expires continues with what the slot holds.  Nothing is cleared between runs: a flag is the row's epoch, a word that
+      // started no later (workgroups start in index order on each die: an assumption about the dispatcher).  Waits are
+      // bounded: one that expires sets the device's fault word, and the next call that waits for the device raises an
+      // error instead of handing out the result; RX_SINGLE_PASS_SCAN=0 selects the two-launch form, which never
+      // waits.  Nothing is cleared between runs: a flag is the row's epoch, a word that
       // the row's last chunk advances once its carry is complete -- by then every chunk of the row has published, so
       // has read the epoch (one counter of finished workgroups would cost 60 ns each: atomics on one address from
       // eight dies).  The data is read once and written once.
@@ -3042,7 +3043,9 @@ struct Planner {
           auto slot_of = [&](const std::string& idx) { return "slots + (row * " + std::to_string(SL) + " + " + idx + ") * " + std::to_string(NW); };
           std::string sg = head("@K@_scan", false, false);
           sg.pop_back();
-          sg += std::string(em.inputs.empty() ? "" : ", ") + "unsigned long long* __restrict__ slots, " + ptr_decl(ost, false, "out0") + ")";
+          sg += std::string(em.inputs.empty() ? "" : ", ") + "unsigned long long* __restrict__ slots, unsigned* __restrict__ fault, " + ptr_decl(ost, false, "out0") + ")";
+          // polls before a wait gives up (about 0.1 s); RX_SCAN_SPIN_LIMIT exists so that a test can make a wait expire
+          const int spin_limit = getenv("RX_SCAN_SPIN_LIMIT") ? std::max(0, atoi(getenv("RX_SCAN_SPIN_LIMIT"))) : (1 << 16);
           o << "// scan along the minor dimension of " << ty.str() << " (" << sNC << " chunks per row, one launch): " << describe(rn.in[0]) << "\n";
           o << sg << " {\n";
           o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n  __shared__ " << ACC << " wsum[" << T * (kBlock / 64) << "];\n";
@@ -3097,12 +3100,12 @@ struct Planner {
           o << "  if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of("c") << ", run, epoch);\n";
           o << "  if (c % " << GS << " == " << GS - 1 << ") {\n";
           o << "    " << ACC << " part = " << IDENT << ";\n";
-          o << "    if (threadIdx.x < " << GS << ") part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + threadIdx.x)") << ", epoch);\n";
+          o << "    if (threadIdx.x < " << GS << ") part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + threadIdx.x)") << ", epoch, " << spin_limit << ", fault);\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
           o << "    if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS)) << ", part, epoch);\n";
           o << "    if ((c / " << GS << ") % " << GS << " == " << GS - 1 << ") {\n";
           o << "      " << ACC << " gp = " << IDENT << ";\n";
-          o << "      if (threadIdx.x < " << GS << ") gp = rx_peek_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS) + " - " + std::to_string(GS - 1) + " + threadIdx.x") << ", epoch);\n";
+          o << "      if (threadIdx.x < " << GS << ") gp = rx_peek_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS) + " - " + std::to_string(GS - 1) + " + threadIdx.x") << ", epoch, " << spin_limit << ", fault);\n";
           o << "      gp = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(gp, " << OP << ", lds);\n";
           o << "      if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC + sNG) + " + c / " + std::to_string(GS * GS)) << ", gp, epoch);\n";
           o << "    }\n  }\n";
@@ -3112,7 +3115,7 @@ struct Planner {
           o << "    " << ACC << " part = " << IDENT << ";\n";
           o << "    for (" << it << " k = threadIdx.x; k < ns + ng + na; k += " << kBlock << ") {\n";
           o << "      const " << it << " idx = k < ns ? " << sNC + sNG << " + k : (k < ns + ng ? " << sNC << " + ns * " << GS << " + (k - ns) : (c / " << GS << ") * " << GS << " + (k - ns - ng));\n";
-          o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch)") << ";\n    }\n";
+          o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch, " + std::to_string(spin_limit) + ", fault)") << ";\n    }\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
           o << "    if (c != 0) carry = " << red_apply(rn.red, dt, "carry", "part") << ";\n  }\n";
           // the row's last chunk has, through its carry, heard from every chunk of the row: the next run's epoch
@@ -3142,6 +3145,13 @@ struct Planner {
           cb.data.assign((size_t)cb.bytes, 0);
           plan.buffers.push_back(cb);
           const int slots_buf = (int)plan.buffers.size() - 1;
+          BufferDesc fb;
+          fb.kind = BufferDesc::Fault;
+          fb.ty.dt = DT::U32;
+          fb.ty.dims = {1};
+          fb.bytes = 4;
+          plan.buffers.push_back(fb);
+          const int fault_buf = (int)plan.buffers.size() - 1;
           Launch L;
           L.kernel = named("@K@_scan", kb_single);
           L.kind = "scan";
@@ -3149,6 +3159,7 @@ struct Planner {
           L.block[0] = kBlock;
           for (int i : em.inputs) L.args.push_back(buffer_for(i));
           L.args.push_back(slots_buf);
+          L.args.push_back(fault_buf);
           L.args.push_back(buffer_for(root));
           L.algo_bytes = algo_bytes(em.inputs, {root});
           L.desc = describe(rn.in[0]) + " scan";

@@ -6,7 +6,9 @@
 namespace rx {
 
 struct BufferDesc {
-  enum Kind { Param, Const, Temp, Scratch } kind = Temp;
+  // Fault: the device's fault word, a 32-bit word in pinned host memory that a kernel sets when a bounded wait for
+  // another workgroup expires; the runtime checks it wherever the host waits for the device
+  enum Kind { Param, Const, Temp, Scratch, Fault } kind = Temp;
   TType ty;                    // element type / shape (Scratch: bytes only)
   int64_t bytes = 0;
   int param_index = -1;        // Param
@@ -55,7 +57,7 @@ struct PlanOptions {
   // device-scope release fence every workgroup needs before taking its ticket (an L2 write-back on
   // this multi-die part) made the sinsum kernel 2x slower than the two-launch form.
   bool single_pass_reduce = false;
-  bool single_pass_scan = false;     // long scanned rows in one launch (chunk totals travel as flagged words)
+  bool single_pass_scan = true;      // long scanned rows in one launch (chunk totals travel as flagged words)
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS

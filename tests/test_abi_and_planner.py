@@ -237,9 +237,14 @@ def test_products_with_a_vector_like_operand_plan_as_reductions(monkeypatch):
 
 def test_windowed_ops_plan(monkeypatch):
     import _nn_modules as NN
-    # cumsum over 2^24 elements: chunk totals, then the scan proper
+    # cumsum over 2^24 elements: one launch whose workgroups hand their chunk totals on as flagged words
+    rep = rx.compile_offline(NN.cumulative([1 << 24], "f32", 0), with_source=True)
+    assert "kind=scan " in rep and "launches: 1" in rep and "rx_peek_partial<float>" in rep and "unsigned* __restrict__ fault" in rep
+    # the form that does not wait for other workgroups: chunk totals, then the scan proper
+    monkeypatch.setenv("RX_SINGLE_PASS_SCAN", "0")
     rep = rx.compile_offline(NN.cumulative([1 << 24], "f32", 0))
     assert "kind=scan_totals" in rep and "kind=scan " in rep and "launches: 2" in rep
+    monkeypatch.delenv("RX_SINGLE_PASS_SCAN")
     # rows of a matrix: one workgroup per row chunk, no totals needed when a row is one chunk
     assert "launches: 1" in rx.compile_offline(NN.cumulative([4096, 4096], "f32", 1))
     # pooling: the window view is index arithmetic inside a reduction kernel
