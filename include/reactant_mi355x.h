@@ -107,7 +107,9 @@ void XLAExecuteSharded(RxExecutable *exec, int num_args, RxBuffer **op_args, RxD
                        uint8_t *is_arg_donatable, int num_results, RxBuffer **op_results, uint8_t *futures,
                        RxFuture **future_results);
 /* A future completes when its device's stream has reached the point at which the future was first asked
- * (FutureIsReady / FutureAwait), which is no earlier than the end of the call that returned it. */
+ * (FutureIsReady / FutureAwait), which is no earlier than the end of the call that returned it.
+ * Calls that wait for the device (these, BufferToHost, CopyFromBuffer) also report a kernel whose bounded wait for
+ * another workgroup of its launch expired: they raise once, and the results of that execution are invalid. */
 void FreeFuture(RxFuture *future);                                   /* API.cpp:1358 */
 uint8_t FutureIsReady(RxFuture *future);                             /* API.cpp:1360 */
 void FutureAwait(RxFuture *future);                                  /* API.cpp:1364 */
