@@ -182,7 +182,8 @@ struct RxBuffer {
 };
 
 struct RxFuture {
-  hipEvent_t ev = nullptr;
+  hipEvent_t ev = nullptr;       // recorded when the future is first asked (future_event)
+  bool done = false;             // known complete without an event (its client was freed, which waits for the stream)
   RxDevice* device = nullptr;
   std::string error;
 };
@@ -1006,7 +1007,8 @@ RX_EXPORT void FreeFuture(RxFuture* f) {
 }
 // The event of a future, recorded on its device's stream the first time the future is asked about.
 static void future_event(RxFuture* f) {
-  if (f->ev) return;
+  if (f->ev || f->done) return;
+  if (!f->device->client || !f->device->client->alive.load()) { f->done = true; return; }   // FreeClient drained the stream
   HIP_CHECK(hipSetDevice(f->device->ordinal));
   HIP_CHECK(hipEventCreateWithFlags(&f->ev, hipEventDisableTiming));
   HIP_CHECK(hipEventRecord(f->ev, f->device->stream));
@@ -1015,6 +1017,7 @@ RX_EXPORT uint8_t FutureIsReady(RxFuture* f) {
   return guarded([&]() -> uint8_t {
     if (!f || !reg_has(f)) throw Error("INVALID_ARGUMENT: null or foreign future handle");
     future_event(f);
+    if (f->done) return 1;
     hipError_t e = hipEventQuery(f->ev);
     if (e == hipSuccess) { check_fault(f->device); return 1; }
     if (e == hipErrorNotReady) { (void)hipGetLastError(); return 0; }
@@ -1025,6 +1028,7 @@ RX_EXPORT void FutureAwait(RxFuture* f) {
   guarded_void([&] {
     if (!f || !reg_has(f)) throw Error("INVALID_ARGUMENT: null or foreign future handle");
     future_event(f);
+    if (f->done) return;
     hipError_t e = hipEventSynchronize(f->ev);
     if (e != hipSuccess) throw Error(std::string("execution failed: ") + hipGetErrorString(e));
     check_fault(f->device);

@@ -175,3 +175,29 @@ def test_memory_limit_is_enforced_and_a_failed_execution_keeps_donated_arguments
         bx.free()
     finally:
         small.close()
+
+
+def test_futures_are_asked_late_or_never(rx):
+    """A future records its event when it is first asked (src/xla/PJRT/Future.jl:1-28 only ever polls or awaits): asking
+    after more work was queued, asking twice, never asking, and asking after the client was freed all behave."""
+    own = rx.Client()
+    try:
+        n = 1 << 22
+        t = "tensor<%dxf32>" % n
+        exe = rx.xla_compile(own, "module { func.func @main(%%a: %s) -> %s { %%0 = stablehlo.add %%a, %%a : %s\n return %%0 : %s } }" % (t, t, t, t))
+        x = np.arange(n, dtype=np.float32)
+        bx = rx.Buffer.from_host(own, x, "f32")
+        first = exe.execute_sharded([bx])[0]
+        later = [exe.execute_sharded([bx])[0] for _ in range(20)]          # more work behind the first call
+        assert first.future is not None
+        first.future.wait()                                                # waits for a point at or after the first call's end
+        assert first.future.is_ready()                                     # asked again: the same event
+        assert np.array_equal(first.buffer.to_host(), 2 * x)
+        while not later[-1].future.is_ready():                             # polling alone makes progress
+            pass
+        assert np.array_equal(later[-1].buffer.to_host(), 2 * x)
+        unasked = later[3].future                                          # never asked before the client goes away
+    finally:
+        own.close()
+    assert unasked.is_ready()                                              # FreeClient waited for the stream
+    unasked.wait()
