@@ -346,6 +346,13 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     # K = 8256 is whole 16-byte vectors but not whole K tiles of 128: not the direct-to-LDS skeletons
     odd = rx.compile_offline(P.fp8_linear(8192, 8256, 8192), with_source=True)
     assert "rx_gemm_body_s<" not in odd and "kind=gemm_f8" in odd
+    # an operand of 4 GB or more is beyond the 32-bit buffer offsets of the streaming skeleton: the ring skeleton takes it
+    huge = rx.compile_offline(_dot("tensor<65536x65536xf8E4M3FN>", "tensor<8192x65536xf8E4M3FN>", "tensor<65536x8192xf32>", "contracting_dims = [1] x [1]"),
+                              with_source=True)
+    assert "rx_gemm_body_s<" not in huge and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in huge
+    below = rx.compile_offline(_dot("tensor<32768x65536xf8E4M3FN>", "tensor<8192x65536xf8E4M3FN>", "tensor<32768x8192xf32>", "contracting_dims = [1] x [1]"),
+                               with_source=True)
+    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 32768, 8192, 65536" in below
     # the 32x32 MFMA shapes are a request for the ring skeleton
     monkeypatch.setenv("RX_GEMM_MFMA32", "1")
     assert "rx_gemm_body_dl<rx_mma_bf16, 256, 256, 64" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
