@@ -1560,13 +1560,21 @@ struct Planner {
     o << "  const int tA0 = z0 - " << (hR.lo[0] + hP.lo[0]) << ", zb0 = z0 - " << hR.lo[0] << ";\n";
     o << "  const int nB = zend - z0 + " << dB << ", nit = nB + 1;\n";
     o << "  auto plane = [&](int p) { return (" << it << ")rx_clamp_idx<int>(p, " << Z - 1 << ") * " << Y * X << LL << "; };\n";
+    // Requests run PD planes ahead of their use: with one plane ahead the bytes in flight (3 workgroups of 256 threads
+    // per CU, about 90 bytes each) divided by the memory latency are what the kernel moves, not what the memory
+    // system can (measured: 5.3 TB/s against 6.5 for a plain copy).  Registers that receive a request are named by the
+    // iteration's parity, so the loop body is instantiated for both.
+    const int PD = opt.march2_prefetch == 2 ? 2 : 1;
+    auto par = [&](const std::string& e) { return PD == 2 ? "[" + e + "]" : std::string(); };
     // prologue: the source planes the first first-step plane needs
-    o << "  " << vt << " preA[" << NLA << "];\n";
+    o << "  " << vt << " preA" << (PD == 2 ? "[2]" : "") << "[" << NLA << "];\n";
     o << "  {\n    " << vt << " pro[" << dA + 1 << "][" << NLA << "];\n";
     for (int64_t k = 0; k <= dA; ++k)
       o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) pro[" << k << "][q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << k
         << ") + poffA[q]);\n";
-    o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << dA + 1 << ") + poffA[q]);\n";
+    o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) preA" << par("0") << "[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << dA + 1 << ") + poffA[q]);\n";
+    if (PD == 2)
+      o << "#pragma unroll\n    for (int q = 0; q < " << NLA << "; ++q) preA[1][q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + " << dA + 2 << ") + poffA[q]);\n";
     std::set<int> stream_slots;
     for (auto& dv : eb.direct_vecs) stream_slots.insert(dv.first);
     for (auto& dv : ec.direct_vecs) stream_slots.insert(dv.first);
@@ -1579,11 +1587,14 @@ struct Planner {
     o << "  }\n";
     for (int sl : stream_slots) {
       const std::string vts = vts_of(ec, sl);
-      o << "  " << vts << " uq" << sl << "[" << QL << "], un" << sl << ";\n";
+      o << "  " << vts << " uq" << sl << "[" << QL << "], un" << sl << (PD == 2 ? "[2]" : "") << ";\n";
       o << "  uq" << sl << "[0] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + colc);\n";
+      if (PD == 2) o << "  un" << sl << "[1] = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + 1) + colc);\n";
       if (NSP > 0 && eb.direct_vecs.count({sl, 0})) {
-        o << "  " << vts << " us" << sl << "[" << NSP << "], usn" << sl << "[" << NSP << "];\n";
+        o << "  " << vts << " us" << sl << "[" << NSP << "], usn" << sl << (PD == 2 ? "[2]" : "") << "[" << NSP << "];\n";
         o << "#pragma unroll\n  for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0) + soff[q]);\n";
+        if (PD == 2)
+          o << "#pragma unroll\n  for (int q = 0; q < " << NSP << "; ++q) usn" << sl << "[1][q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + 1) + soff[q]);\n";
       }
     }
     o << "  rx_lds_barrier();\n";
@@ -1602,14 +1613,15 @@ struct Planner {
       o << pad << "  rx_store(dstb + " << ldsoff << ", res);\n";
       o << pad << "}\n";
     };
-    o << "  for (int n = 0; n < nit; ++n) {\n";
-    // requests for the next iteration
-    o << "    if (n + 1 < nB) {\n";
+    if (PD == 2) o << "  auto iter = [&](auto PAR, const int n) __attribute__((always_inline)) {\n    constexpr int P = decltype(PAR)::value;\n";
+    else o << "  for (int n = 0; n < nit; ++n) {\n";
+    // requests for the iteration PD ahead
+    o << "    if (n + " << PD << " < nB) {\n";
     for (int sl : stream_slots) {
       const std::string vts = vts_of(ec, sl);
-      o << "      un" << sl << " = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + 1) + colc);\n";
+      o << "      un" << sl << par("P") << " = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + " << PD << ") + colc);\n";
       if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
-        o << "#pragma unroll\n      for (int q = 0; q < " << NSP << "; ++q) usn" << sl << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + 1) + soff[q]);\n";
+        o << "#pragma unroll\n      for (int q = 0; q < " << NSP << "; ++q) usn" << sl << par("P") << "[q] = rx_load<" << vts << ">(in" << sl << " + plane(zb0 + n + " << PD << ") + soff[q]);\n";
     }
     o << "    }\n";
     // the source plane requested last iteration goes to the ring; request the one after it
@@ -1617,9 +1629,9 @@ struct Planner {
     o << "      " << st << "* dst = ldsA + ((n + " << dA + 1 << ") % " << RA << ") * " << APLANE << ";\n";
     o << "#pragma unroll\n      for (int q = 0; q < " << NLA << "; ++q) {\n";
     o << "        const int v = threadIdx.x + q * " << NB << ";\n";
-    o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA[q]);\n      }\n";
-    o << "      if (n + 2 < nB) {\n";
-    o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + n + " << dA + 2
+    o << "        if (v < " << AV << ") rx_store(dst + v * " << vec << ", preA" << par("P") << "[q]);\n      }\n";
+    o << "      if (n + " << PD + 1 << " < nB) {\n";
+    o << "#pragma unroll\n        for (int q = 0; q < " << NLA << "; ++q) preA" << par("P") << "[q] = rx_load<" << vt << ">(in" << sslot << " + plane(tA0 + n + " << dA + 1 + PD
       << ") + poffA[q]);\n";
     o << "      }\n    }\n";
     // one output plane of the second step
@@ -1658,12 +1670,13 @@ struct Planner {
     // the streamed inputs move one plane on
     for (int sl : stream_slots) {
       for (int64_t k = QL - 1; k >= 1; --k) o << "    uq" << sl << "[" << k << "] = uq" << sl << "[" << k - 1 << "];\n";
-      o << "    uq" << sl << "[0] = un" << sl << ";\n";
+      o << "    uq" << sl << "[0] = un" << sl << par("P ^ 1") << ";\n";
       if (NSP > 0 && eb.direct_vecs.count({sl, 0}))
-        o << "#pragma unroll\n    for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << "[q];\n";
+        o << "#pragma unroll\n    for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << par("P ^ 1") << "[q];\n";
     }
     o << "    rx_lds_barrier();\n";
-    o << "  }\n}\n\n";
+    if (PD == 2) o << "  };\n  for (int n = 0; n < nit; n += 2) {\n    iter(rx_int<0>{}, n);\n    if (n + 1 < nit) iter(rx_int<1>{}, n + 1);\n  }\n}\n\n";
+    else o << "  }\n}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;
     L.kernel = named(kname, kb_final);
@@ -1726,8 +1739,17 @@ struct Planner {
       staged[l.node] = l.root_var;
     }
     if (staged.empty()) return false;
+    // Whole 16-byte vectors on both sides where the two dimensions allow it: a tile of 64 input columns x 128 input
+    // rows (64 x 64 for 8-byte elements) is read with 16-byte loads, parked with a row pitch of 64 + V, and written as
+    // output rows of 512 bytes, each lane storing the V elements it gathered from V tile rows (8192^2 f32 transpose:
+    // 134 -> 105 us; the 4-byte form moves a 256-byte row segment per wavefront instruction).
+    const int es_out = info(rn.ty.dt).size;
+    int V = (es_out == 2 || es_out == 4 || es_out == 8) ? 16 / es_out : 1;
+    for (auto& kv : staged) if ((int)info(g.nodes[kv.first].ty.dt).size != es_out) V = 1;
+    if (V > 1 && (q < 0 || dims[q] % V != 0 || dims[n - 1] % V != 0 || dims[q] < 64 || dims[n - 1] < 64 || !opt.transpose_vectors)) V = 1;
+    const int TQ = TS, TM = V > 1 ? (es_out == 8 ? 64 : 128) : TS, LD = V > 1 ? TQ + V : TS + 1;
     int64_t lds_total = 0;
-    for (auto& kv : staged) lds_total += (int64_t)TS * (TS + 1) * info(g.nodes[kv.first].ty.dt).size;
+    for (auto& kv : staged) lds_total += (int64_t)TM * LD * info(g.nodes[kv.first].ty.dt).size;
     if (lds_total > 64 * 1024) return false;
 
     // pass 2: emit with the transposed reads redirected to the tiles
@@ -1736,14 +1758,14 @@ struct Planner {
     em.perm_hook = [&](int slot, const std::vector<int>& rv, std::string* expr) {
       auto it2 = staged.find(em.inputs[slot]);
       if (it2 == staged.end() || it2->second != rv) return false;
-      *expr = "tile" + std::to_string(slot) + "[tb * " + std::to_string(TS + 1) + " + ta]";
+      *expr = "tile" + std::to_string(slot) + "[tb * " + std::to_string(LD) + " + ta]";
       return true;
     };
     std::string val = em.emit(root, root_index(dims));
     std::string body = em.take_code();
     const std::string it = em.idx_t();
     const int64_t DQ = dims[q], DM = dims[n - 1];
-    const int64_t ntq = (DQ + TS - 1) / TS, ntm = (DM + TS - 1) / TS;
+    const int64_t ntq = (DQ + TQ - 1) / TQ, ntm = (DM + TM - 1) / TM;
     int64_t outer = 1;
     for (int d = 0; d < n - 1; ++d) if (d != q) outer *= dims[d];
     const int64_t nblocks = outer * ntq * ntm;
@@ -1754,12 +1776,12 @@ struct Planner {
     o << signature(kname, em.inputs, {{info(rn.ty.dt).stype, "out0"}}) << " {\n";
     for (auto& kv : staged) {
       const int slot = em.slot_of(kv.first);
-      o << "  __shared__ " << info(g.nodes[kv.first].ty.dt).stype << " tile" << slot << "[" << TS * (TS + 1) << "];\n";
+      o << "  __shared__ __attribute__((aligned(16))) " << info(g.nodes[kv.first].ty.dt).stype << " tile" << slot << "[" << TM * LD << "];\n";
     }
     // block -> (outer coordinates, tile of dimension q, tile of the minor dimension)
     o << "  unsigned rest = blockIdx.x;\n";
-    o << "  const " << it << " m0 = (" << it << ")(rest % " << ntm << "u) * " << TS << "; rest /= " << ntm << "u;\n";
-    o << "  const " << it << " q0 = (" << it << ")(rest % " << ntq << "u) * " << TS << "; rest /= " << ntq << "u;\n";
+    o << "  const " << it << " m0 = (" << it << ")(rest % " << ntm << "u) * " << TM << "; rest /= " << ntm << "u;\n";
+    o << "  const " << it << " q0 = (" << it << ")(rest % " << ntq << "u) * " << TQ << "; rest /= " << ntq << "u;\n";
     for (int d = n - 2; d >= 0; --d) {
       if (d == q) continue;
       o << "  const " << it << " i" << d << " = (" << it << ")(rest % " << dims[d] << "u); rest /= " << dims[d] << "u;\n";
@@ -1781,6 +1803,17 @@ struct Planner {
         base += " + i" + std::to_string(rv[d]) + " * " + std::to_string(stride[d]) + (em.idx64 ? "LL" : "");
       }
       o << "  {\n    const " << it << " base = " << base << ";\n";
+      if (V > 1) {
+        const int LPR = TQ / V, RPP = kBlock / LPR;    // lanes per input row, rows per pass
+        const std::string vts = "rx_vec<" + std::string(info(in.ty.dt).stype) + ", " + std::to_string(V) + ">";
+        o << "#pragma unroll\n    for (int r = 0; r < " << TM / RPP << "; ++r) {\n";
+        o << "      const int tb = r * " << RPP << " + (int)threadIdx.x / " << LPR << ", ta = ((int)threadIdx.x % " << LPR << ") * " << V << ";\n";
+        o << "      if (m0 + tb < " << DM << " && q0 + ta < " << DQ << ")\n";
+        o << "        rx_store(tile" << slot << " + tb * " << LD << " + ta, rx_load_nt<" << vts << ">(in" << slot << " + base + (m0 + tb) * " << stride_m << (em.idx64 ? "LL" : "")
+          << " + (q0 + ta)));\n";
+        o << "    }\n  }\n";
+        continue;
+      }
       o << "#pragma unroll\n    for (int r = 0; r < " << TS / ROWS << "; ++r) {\n";
       o << "      const int tb = r * " << ROWS << " + grp, ta = lane;\n";
       o << "      if (m0 + tb < " << DM << " && q0 + ta < " << DQ << ")\n";
@@ -1788,6 +1821,27 @@ struct Planner {
       o << "    }\n  }\n";
     }
     o << "  __syncthreads();\n";
+    if (V > 1) {
+      // phase 2 on vectors: a lane owns V consecutive elements of an output row
+      const int OPR = TM / V, ORP = kBlock / OPR;      // lanes per output row, output rows per pass
+      const std::string vto = "rx_vec<" + std::string(info(rn.ty.dt).stype) + ", " + std::to_string(V) + ">";
+      o << "#pragma unroll 4\n  for (int r = 0; r < " << TQ / ORP << "; ++r) {\n";
+      o << "    const int ta = r * " << ORP << " + (int)threadIdx.x / " << OPR << ", tbv = ((int)threadIdx.x % " << OPR << ") * " << V << ";\n";
+      o << "    const " << it << " i" << q << " = q0 + ta;\n";
+      o << "    if (i" << q << " < " << DQ << " && m0 + tbv < " << DM << ") {\n";
+      o << "      " << vto << " res;\n";
+      o << "#pragma unroll\n      for (int e = 0; e < " << V << "; ++e) {\n";
+      o << "      const int tb = tbv + e;\n";
+      o << "      const " << it << " i" << n - 1 << " = m0 + tb;\n";
+      o << body;
+      o << "      res.v[e] = " << em.store_value(rn.ty.dt, val) << ";\n      }\n";
+      {
+        Index rix = root_index(dims);
+        rix[n - 1].var = "(m0 + tbv)";
+        o << "      " << (opt.nt_stores ? "rx_store_nt" : "rx_store") << "(out0 + " << em.linear(rix, dims) << ", res);\n";
+      }
+      o << "    }\n  }\n}\n\n";
+    } else {
     // phase 2: the map itself, lanes along the output's minor dimension
     o << "#pragma unroll 4\n  for (int r = 0; r < " << TS / ROWS << "; ++r) {\n";
     o << "    const int ta = r * " << ROWS << " + grp, tb = lane;\n";
@@ -1797,6 +1851,7 @@ struct Planner {
     Index rix = root_index(dims);
     o << "      out0[" << em.linear(rix, dims) << "] = " << em.store_value(rn.ty.dt, val) << ";\n";
     o << "    }\n  }\n}\n\n";
+    }
     const std::string kb_final = finalize(o.str());
     Launch L;
     L.kernel = named(kname, kb_final);

@@ -357,7 +357,11 @@ def _tt_(shape, dt):
 
 @pytest.mark.parametrize("shape,perm,dt", [((300, 257), (1, 0), "f32"), ((257, 300), (1, 0), "f64"), ((64, 1030), (1, 0), "i32"),
                                            ((9, 130, 70), (0, 2, 1), "f32"), ((70, 33, 129), (2, 1, 0), "f32"),
-                                           ((3, 66, 5, 80), (0, 3, 2, 1), "bf16"), ((130, 20, 70), (1, 2, 0), "f32")])
+                                           ((3, 66, 5, 80), (0, 3, 2, 1), "bf16"), ((130, 20, 70), (1, 2, 0), "f32"),
+                                           # both dimensions whole 16-byte vectors: the vector form, tiles of 64 x 128 (64 x 64 for f64) cut by the edges
+                                           ((300, 260), (1, 0), "f32"), ((520, 264), (1, 0), "f64"), ((1000, 1000), (1, 0), "i32"),
+                                           ((3, 72, 5, 80), (0, 3, 2, 1), "bf16"), ((132, 20, 68), (1, 2, 0), "f32"), ((256, 256), (1, 0), "f32"),
+                                           ((5, 128, 192), (0, 2, 1), "f16")])
 def test_transpose_through_lds_tiles(rx, client, shape, perm, dt):
     """Pure transposes of every kind that moves the minor dimension, with tiles cut by the edges;
     bit-exact (a transpose moves values, it does not compute)."""
