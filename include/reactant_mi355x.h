@@ -169,7 +169,7 @@ void RxDeviceSynchronize(RxDevice *device);
 float RxCalibrationCopy(RxDevice *device, size_t bytes, int iters);
 /* Measurement aid, no counterpart in the reference: the rate the MFMA pipe sustains on this device when nothing
  * else runs (one wavefront per SIMD issuing independent MFMAs on register operands for about 10 ms, so that the
- * clock settles under the power limit).  kind 0: v_mfma_f32_16x16x32_bf16, kind 1: v_mfma_f32_32x32x64_f8f6f4 on
+ * clock settles under the power limit).  kind 0: v_mfma_f32_16x16x32_bf16, kind 1: v_mfma_f32_16x16x128_f8f6f4 on
  * e4m3; operands pseudo-random, or all zero (`zero_operands` != 0: no toggling in the multipliers).  Writes the
  * TFLOP/s and the average shader clock in MHz; returns 0, or 1 with a message (RxLastError). */
 int RxMfmaCeiling(RxDevice *device, int kind, int zero_operands, double *tflops, double *clock_mhz);

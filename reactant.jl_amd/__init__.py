@@ -475,7 +475,7 @@ def xla_compile(client, mlir_text):
 
 def mfma_ceiling(device, kind, zero_operands=False):
     """(TFLOP/s, average shader clock in MHz) the MFMA pipe sustains on `device` with nothing else running:
-    kind "bf16" (v_mfma_f32_16x16x32_bf16) or "f8" (v_mfma_f32_32x32x64_f8f6f4), pseudo-random or all-zero operands."""
+    kind "bf16" (v_mfma_f32_16x16x32_bf16) or "f8" (v_mfma_f32_16x16x128_f8f6f4), pseudo-random or all-zero operands."""
     tf, mhz = ctypes.c_double(), ctypes.c_double()
     _call("RxMfmaCeiling", device.handle, {"bf16": 0, "f8": 1}[kind], 1 if zero_operands else 0, ctypes.byref(tf), ctypes.byref(mhz))
     return tf.value, mhz.value

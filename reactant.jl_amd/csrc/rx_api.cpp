@@ -334,8 +334,8 @@ __global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, 
 
 // The rate the MFMA pipe sustains when nothing else runs: every wavefront of the chip (one per SIMD) issues
 // independent MFMAs back to back on operands that stay in registers, for long enough that the clock settles under
-// the power limit.  KIND 0: v_mfma_f32_16x16x32_bf16, KIND 1: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3), the
-// instructions of the GEMM skeletons.  Operands are seeded pseudo-random values of moderate exponent, or all zero
+// the power limit.  KIND 0: v_mfma_f32_16x16x32_bf16, KIND 1: v_mfma_f32_16x16x128_f8f6f4 (e4m3 x e4m3), the
+// instructions of the streaming GEMM skeleton.  Operands are seeded pseudo-random values of moderate exponent, or all zero
 // (no toggling in the multipliers).  Every wavefront reports its shader-clock and real-time ticks.
 typedef float rx_probe_f32x16 __attribute__((ext_vector_type(16)));
 typedef float rx_probe_f32x4 __attribute__((ext_vector_type(4)));
@@ -381,7 +381,7 @@ __global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, 
       for (int q = 0; q < 32; ++q) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc4[q & 15]) : "v"(av[q & 3]), "v"(bv[(q >> 2) & 3]));
     } else {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) acc[q & 7] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[q & 3], b[q >> 1], acc[q & 7], 0, 0, 0, 0, 0, 0);
+      for (int q = 0; q < 16; ++q) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+v"(acc4[q & 15]) : "v"(a[q & 3]), "v"(b[(q >> 2) & 3]));
     }
   }
   const unsigned long long t1 = clock64(), w1 = wall_clock64();
@@ -1050,7 +1050,7 @@ RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tf
     // 256 workgroups of four wavefronts: one wavefront per SIMD of the chip.  About 10 ms per launch, so that the
     // clock has settled under the power limit; the second launch is the one that is timed.
     const int iters = 40000;
-    const double flop_per_iter = kind == 0 ? 32 * 2.0 * 16 * 16 * 32 : 8 * 2.0 * 32 * 32 * 64;
+    const double flop_per_iter = kind == 0 ? 32 * 2.0 * 16 * 16 * 32 : 16 * 2.0 * 16 * 16 * 128;
     hipEvent_t a, b;
     HIP_CHECK(hipEventCreate(&a));
     HIP_CHECK(hipEventCreate(&b));
@@ -1087,7 +1087,9 @@ RX_EXPORT float RxCalibrationCopy(RxDevice* d, size_t bytes, int iters) {
     Allocation src(d, bytes), dst(d, bytes);
     HIP_CHECK(hipMemsetAsync(src.ptr, 1, bytes, d->stream));
     const size_t n16 = bytes / 16;
-    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, 256 * 32);
+    // one 16-byte element per thread, workgroups in address order: 6.2-6.5 TB/s of read + write on this part; a
+    // grid-stride loop over 8192 workgroups, whose accesses drift apart, reaches 4.6
+    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, 0x7fffffffu);
     hipEvent_t a, b;
     HIP_CHECK(hipEventCreate(&a));
     HIP_CHECK(hipEventCreate(&b));
