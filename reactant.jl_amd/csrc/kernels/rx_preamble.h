@@ -357,6 +357,13 @@ RX_DEV T rx_group_reduce(T v, OP op) {
   return v;
 }
 
+// Makes the compiler have `x` in a register at this point of the program (so whatever it was computed from can
+// be dropped here, instead of the computation moving to where `x` is used).
+template <typename T>
+RX_DEV void rx_pin(T& x) {
+  if constexpr (sizeof(T) == 4 || sizeof(T) == 8) asm volatile("" : "+v"(x));
+}
+
 // Value held by lane `src` (0..63) of this wavefront.
 template <typename T>
 RX_DEV T rx_lane_from(T v, rx_u32 src) {

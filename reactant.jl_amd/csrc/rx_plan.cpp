@@ -3089,11 +3089,14 @@ struct Planner {
       };
       // Long rows in one launch.  A workgroup owns a chunk of T tiles, keeps its values in registers, publishes the
       // chunk's total as flagged 64-bit words (rx_publish_partial: no fence), and builds its carry from what the
-      // chunks before it published.  So that nobody waits for a chain, totals exist at three levels: per chunk, per
-      // group of 32 chunks (summed and published by the group's last chunk) and per 32 groups (by their last chunk);
-      // a chunk's carry is the supergroups before it, the groups before it in its supergroup and the chunks before it
-      // in its group -- at most a few dozen slots, combined in an order that depends on the chunk index alone, so the
-      // result does not depend on timing.  Every workgroup waits only for lower-numbered ones, which the dispatcher
+      // chunks before it published.  Totals exist per chunk and per group of 256 chunks (summed and published by the
+      // group's last chunk).  A chunk's carry is the totals of the groups up to the last but one before its own, then
+      // the chunks of the group before its own and of its own group up to itself: at most 511 chunk slots and one
+      // slot per older group, all requested at once and combined in an order that depends on the chunk index alone,
+      // so the result does not depend on timing.  A group's total is first needed by chunks that start 256 chunks
+      // after the one that publishes it, so nobody waits for a sum of sums: with groups of 32 whose totals the next
+      // group needs at once, a chunk waited 5.4 us on average, with this window 3.7 (2^26 f32, time stamps inside
+      // the kernel).  Every workgroup waits only for lower-numbered ones, which the dispatcher
       // started no later (workgroups start in index order on each die: an assumption about the dispatcher).  Waits are
       // bounded: one that expires sets the device's fault word, and the next call that waits for the device raises an
       // error instead of handing out the result; RX_SINGLE_PASS_SCAN=0 selects the two-launch form, which never
@@ -3102,13 +3105,13 @@ struct Planner {
       // has read the epoch (one counter of finished workgroups would cost 60 ns each: atomics on one address from
       // eight dies).  The data is read once and written once.
       {
-        constexpr int GS = 32;
-        // tiles per chunk: 2^26 f32 takes 0.274 / 0.188 / 0.141 / 0.131 / 0.170 ms with 2 / 4 / 8 / 16 / 32 (few tiles: too
-        // many workgroups polling; many: registers)
+        constexpr int GS = kBlock;
+        // tiles per chunk: 2^26 f32 takes 121 / 99 / 97 us with 8 / 16 / 32 (few tiles: too many workgroups polling;
+        // 32: 182 registers)
         const int T = getenv("RX_SCAN_T") ? std::max(1, std::min(32, atoi(getenv("RX_SCAN_T")))) : 16;
         const int64_t sCH = (int64_t)T * TILE;
         const int64_t sNC = (n + sCH - 1) / sCH;
-        const int64_t sNG = (sNC + GS - 1) / GS, sNS = (sNG + GS - 1) / GS, SL = sNC + sNG + sNS;
+        const int64_t sNG = (sNC + GS - 1) / GS, SL = sNC + sNG;
         const int NW = (ACC == "double" || info(dt).size == 8) ? 2 : 1;
         const int64_t slot_words = outer * SL * NW + outer;   // + one epoch word per row
         if (opt.single_pass_scan && sNC > 1 && sNC * outer < ((int64_t)1 << 30) && slot_words * 8 <= ((int64_t)64 << 20)) {
@@ -3128,7 +3131,7 @@ struct Planner {
           o << ibody;
           o << "  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;\n";
           o << "  const rx_u32 epoch = (rx_u32)slots[" << outer * SL * NW << " + row] + 1u;\n";
-          o << "  " << ACC << " v[" << T << "][" << V << "], pre[" << T << "], incl[" << T << "];\n";
+          o << "  " << ACC << " v[" << T << "][" << V << "], pre[" << T << "];\n";
           // all loads of the chunk first (rows of whole vectors), so that a workgroup has its whole chunk in flight
           if (vecw > 1) {
             for (auto& sd : em.direct_vecs) {
@@ -3156,37 +3159,33 @@ struct Planner {
           o << "        const " << it << " j = " << jexpr << ";\n" << body;
           o << "        v[t][l] = (" << ACC << ")" << val << ";\n      }\n    }\n";
           o << "#pragma unroll\n    for (int l = 1; l < " << V << "; ++l) v[t][l] = " << red_apply(rn.red, dt, "v[t][l - 1]", "v[t][l]") << ";\n";
-          o << "    incl[t] = rx_wave_scan(v[t][" << V - 1 << "], " << OP << ");\n";
-          o << "    if (lane == 63) wsum[t * " << kBlock / 64 << " + w] = incl[t];\n  }\n";
+          o << "    const " << ACC << " incl = rx_wave_scan(v[t][" << V - 1 << "], " << OP << ");\n";
+          o << "    if (lane == 63) wsum[t * " << kBlock / 64 << " + w] = incl;\n";
+          o << "    pre[t] = rx_lane_from(incl, (rx_u32)(lane - 1) & 63u);\n  }\n";
           o << "  __syncthreads();\n";
           o << "  " << ACC << " run = " << IDENT << ";\n";
           o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
           o << "    " << ACC << " pt = run;\n    " << ACC << " total = wsum[t * " << kBlock / 64 << "];\n";
           o << "#pragma unroll\n    for (int i = 0; i < " << kBlock / 64 << "; ++i) {\n      if (i < w) pt = " << red_apply(rn.red, dt, "pt", "wsum[t * " + std::to_string(kBlock / 64) + " + i]") << ";\n";
           o << "      if (i > 0) total = " << red_apply(rn.red, dt, "total", "wsum[t * " + std::to_string(kBlock / 64) + " + i]") << ";\n    }\n";
-          o << "    const " << ACC << " below = rx_lane_from(incl[t], (rx_u32)(lane - 1) & 63u);\n";
-          o << "    if (lane > 0) pt = " << red_apply(rn.red, dt, "pt", "below") << ";\n";
-          o << "    pre[t] = pt;\n";
+          o << "    if (lane > 0) pt = " << red_apply(rn.red, dt, "pt", "pre[t]") << ";\n";
+          // pinned here: left to itself the compiler computes these after the waits below and keeps the wavefront
+          // totals of every tile in registers until then (186 registers instead of 102, half the resident workgroups)
+          o << "    pre[t] = pt;\n    rx_pin(pre[t]);\n";
           o << "    run = " << red_apply(rn.red, dt, "run", "total") << ";\n  }\n";
-          // publish, duties of the last chunk of a group / of 32 groups
+          // publish; the last chunk of a group also publishes the group's total
           o << "  if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of("c") << ", run, epoch);\n";
           o << "  if (c % " << GS << " == " << GS - 1 << ") {\n";
-          o << "    " << ACC << " part = " << IDENT << ";\n";
-          o << "    if (threadIdx.x < " << GS << ") part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + threadIdx.x)") << ", epoch, " << spin_limit << ", fault);\n";
+          o << "    " << ACC << " part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + (" + it + ")threadIdx.x)") << ", epoch, " << spin_limit << ", fault);\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
           o << "    if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS)) << ", part, epoch);\n";
-          o << "    if ((c / " << GS << ") % " << GS << " == " << GS - 1 << ") {\n";
-          o << "      " << ACC << " gp = " << IDENT << ";\n";
-          o << "      if (threadIdx.x < " << GS << ") gp = rx_peek_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS) + " - " + std::to_string(GS - 1) + " + threadIdx.x") << ", epoch, " << spin_limit << ", fault);\n";
-          o << "      gp = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(gp, " << OP << ", lds);\n";
-          o << "      if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC + sNG) + " + c / " + std::to_string(GS * GS)) << ", gp, epoch);\n";
-          o << "    }\n  }\n";
+          o << "  }\n";
           // carry
           o << "  " << ACC << " carry = (" << ACC << ")" << initv << ";\n";
-          o << "  {\n    const " << it << " ns = c / " << GS * GS << ", ng = (c / " << GS << ") % " << GS << ", na = c % " << GS << ";\n";
+          o << "  {\n    const " << it << " g = c / " << GS << ", ngr = g >= 2 ? g - 1 : 0, c0 = (g >= 1 ? g - 1 : 0) * " << GS << ";\n";
           o << "    " << ACC << " part = " << IDENT << ";\n";
-          o << "    for (" << it << " k = threadIdx.x; k < ns + ng + na; k += " << kBlock << ") {\n";
-          o << "      const " << it << " idx = k < ns ? " << sNC + sNG << " + k : (k < ns + ng ? " << sNC << " + ns * " << GS << " + (k - ns) : (c / " << GS << ") * " << GS << " + (k - ns - ng));\n";
+          o << "    for (" << it << " k = threadIdx.x; k < ngr + (c - c0); k += " << kBlock << ") {\n";
+          o << "      const " << it << " idx = k < ngr ? " << sNC << " + k : c0 + (k - ngr);\n";
           o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch, " + std::to_string(spin_limit) + ", fault)") << ";\n    }\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
           o << "    if (c != 0) carry = " << red_apply(rn.red, dt, "carry", "part") << ";\n  }\n";
