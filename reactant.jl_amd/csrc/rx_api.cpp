@@ -256,6 +256,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_LDS_STENCIL")) o.lds_stencil = atoi(e) != 0;
   if (const char* e = getenv("RX_STENCIL_MARCH2")) o.stencil_march2 = atoi(e) != 0;
   if (const char* e = getenv("RX_TRANSPOSE_VECTORS")) o.transpose_vectors = atoi(e) != 0;
+  if (const char* e = getenv("RX_TRANSPOSE_BLOCK")) o.transpose_block = std::max(1, std::min(64, atoi(e)));
   if (const char* e = getenv("RX_MARCH2_PREFETCH")) o.march2_prefetch = atoi(e) == 2 ? 2 : 1;
   if (const char* e = getenv("RX_MARCH2_PLANES")) o.march2_planes = atoi(e) > 0 ? atoi(e) : o.march2_planes;
   if (const char* e = getenv("RX_MARCH2_TILE")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2) { o.march2_tile[0] = v[0]; o.march2_tile[1] = v[1]; } }
