@@ -174,6 +174,14 @@ RX_DEV float rx_tanh_fast(float x) {
   const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
   return __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(e + 1.0f), 1.0f);
 }
+// 0.5 x (1 + tanh(a (x + b x^3))) = x / (1 + e^(-2 a (x + b x^3))) for results that are rounded to a 16-bit or 8-bit
+// float; k1 = -2 a log2(e), k3 = k1 b.  The exponential saturates to 0 or inf at the ends, which gives x and -0 as the
+// chain does; x = -inf gives NaN as the chain does (-inf * 0); NaN propagates.  Where 1 + tanh cancels (x < -3) the
+// chain in float32 is off by up to |x| 2^-23 in absolute terms; this form is not.
+RX_DEV float rx_gelu_chain_fast(float x, float k1, float k3) {
+  const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(k3, x * x, k1));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
 // x / y for a divisor that is the same for every element.  1/y in double is loop-invariant; the
 // double product is within 2^-52 of the exact quotient, and the quotient of two 24-bit numbers is
 // never closer than about 2^-49 (relative) to a midpoint between two floats, so rounding the

@@ -105,6 +105,7 @@ class Emitter {
   bool is_uniform(int node, int depth = 0) const;
   std::string emit_load(int node, const Index& ix);
   std::string emit_op(const Node& n, const Index& ix);
+  bool match_gelu_chain(const Node& n, int* xnode, double* ka, double* kb) const;
   bool lookup(const std::string& key, std::string* out) const;
   Ix temp_index(const std::string& expr, int64_t lo, int64_t hi);
 };

@@ -331,6 +331,19 @@ def test_gemm_tuning_overrides_are_honoured_or_refused(monkeypatch):
         rx.compile_offline(fp8)
 
 
+def test_gelu_chain_is_recognised_for_narrow_results(monkeypatch):
+    """0.5 x (1 + tanh(a (x + b x^3))) in a bf16 program is evaluated as x / (1 + e^(...)) with folded constants; the
+    f32 program, and a bf16 program that must round after every op, keep the chain."""
+    P = load_programs()
+    src = rx.compile_offline(P.mlp(64, (32, 64, 64, 32)), with_source=True)
+    assert src.count("rx_gelu_chain_fast(") == 3 and "rx_tanh_fast" not in src
+    src32 = rx.compile_offline(P.mlp(64, (32, 64, 64, 32), dt="f32"), with_source=True)
+    assert "rx_gelu_chain_fast" not in src32 and "tanhf(" in src32
+    monkeypatch.setenv("RX_EXCESS_PRECISION", "0")
+    strict = rx.compile_offline(P.mlp(64, (32, 64, 64, 32)), with_source=True)
+    assert "rx_gelu_chain_fast" not in strict
+
+
 def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     # 8- and 16-bit operands on eight-wavefront tiles with whole K tiles of 128 bytes: the 16x16 MFMA skeleton that streams
     # one operand (with_source shows the call)

@@ -319,6 +319,39 @@ def test_mlp_bf16(rx, client, batch, widths, gelu):
         h = ref_l[0]
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_gelu_chain_on_every_value(rx, client, dt):
+    """The tanh chain that gelu lowers to, as a map of its own over every 16-bit pattern (infinities, NaNs, zeros and
+    subnormals included): the kernel evaluates it in the logistic form with folded constants.  Each result is within
+    one ulp of the chain evaluated in float64 and rounded once (plus |x| 2^-22, what one float32 rounding of
+    1 + tanh costs the chain itself: where that sum cancels, the logistic form is the more accurate of the two);
+    non-finite results agree in kind."""
+    n = 1 << 16
+    b = P._B()
+    b.types["%arg0"] = P._tt([n], dt)
+    h = P._gelu_tanh(b, "%arg0", [n], dt)
+    text = ("module {\n  func.func @main(%%arg0: %s) -> %s {\n" % (P._tt([n], dt), P._tt([n], dt)) + b.text()
+            + "    return %s : %s\n  }\n}\n" % (h, P._tt([n], dt)))
+    bits = np.arange(n, dtype=np.uint16)
+    x = I.Tensor.from_bytes(bits.tobytes(), dt, (n,))
+    got, exe = gpu_run(rx, client, text, [x])
+    assert "rx_gelu_chain_fast" in rx.compile_offline(text, with_source=True)
+    with np.errstate(all="ignore"):
+        xv = x.a.astype(np.float64)
+    c0 = float(I.tensor(np.array([np.sqrt(2.0 / np.pi)]), dt).a[0])
+    c1 = float(I.tensor(np.array([0.044715]), dt).a[0])
+    with np.errstate(all="ignore"):
+        exact = 0.5 * xv * (1.0 + np.tanh(c0 * (xv + c1 * xv * xv * xv)))
+        ref = I.tensor(exact, dt).a.astype(np.float64)
+    g = got[0].a.astype(np.float64)
+    assert np.array_equal(np.isnan(g), np.isnan(ref))
+    fin = np.isfinite(ref)
+    assert np.array_equal(g[~fin & ~np.isnan(ref)], ref[~fin & ~np.isnan(ref)])
+    ulp = np.spacing(np.abs(ref[fin]).astype(np.float32)).astype(np.float64) * (2.0 ** (24 - (8 if dt == "bf16" else 11)))
+    tiny = 2.0 ** (-133 if dt == "bf16" else -24)
+    assert np.all(np.abs(g[fin] - ref[fin]) <= np.maximum(ulp, tiny) + np.abs(xv[fin]) * 2.0 ** -22)
+
+
 @pytest.mark.parametrize("batch,k,n,layout,form", [(8, 32, 16, "nk", "convert"), (8, 32, 16, "kn", "direct"),
                                                    (64, 128, 256, "nk", "convert"), (128, 256, 128, "kn", "convert")])
 def test_fp8_linear(rx, client, batch, k, n, layout, form):
