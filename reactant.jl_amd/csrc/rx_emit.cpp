@@ -387,6 +387,10 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
     case OpK::Gelu: {
       std::string x = opnd(0);
       if (!is_float(dt)) throw Error("gelu on a non-float type");
+      if (n.op == "TANH" && is_narrow_float(dt)) {
+        const double k1 = -2.0 * 1.4426950408889634 * 0.7978845608028654;
+        return def("rx_gelu_chain_fast(" + x + ", " + float_lit(k1, false) + ", " + float_lit(k1 * 0.044715, false) + ")");
+      }
       std::string f = n.op == "TANH" ? "rx_gelu_tanh" : (n.op == "SIGMOID" ? "rx_gelu_sigmoid" : "rx_gelu_erf");
       return def(f + "(" + x + ")");
     }
