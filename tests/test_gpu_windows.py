@@ -104,10 +104,10 @@ def test_prefix_scans(rx, client, shape, dt, dim, body, rev, kinds):
 
 # long rows in one launch: chunks of 16 tiles (16384 elements of 4 bytes), totals per chunk / 32 chunks / 1024 chunks
 ONE_LAUNCH_SCANS = [
-    ([1 << 25], "f32", 0, "add", False),         # 2048 chunks: 64 groups, 2 supergroups
+    ([1 << 25], "f32", 0, "add", False),         # 2048 chunks: 8 groups of 256; carries use group totals from two groups back
     ([3000001], "f32", 0, "add", False),          # ragged last chunk, partial last group, scalar loads (odd length)
     ([3000000], "i32", 0, "add", True),           # from the end; integers are exact
-    ([9000000], "i64", 0, "add", False),          # two flagged words per total; more than one supergroup
+    ([9000000], "i64", 0, "add", False),          # two flagged words per total; 1099 chunks, five groups
     ([1200000], "f64", 0, "multiply", False),
     ([3, 700000], "f32", 1, "maximum", True),     # several rows, each with its own slots
     ([5, 40000], "bf16", 1, "add", False),
