@@ -968,11 +968,15 @@ struct Planner {
   // walks each of them layer by layer in z, so the planes that consecutive layers share (and the
   // rows that neighbouring tiles of a layer share) are still in that XCD's L2 when they are asked
   // for again.  Declares x0, y0, z0; returns the number of workgroups to launch.
-  int64_t emit_tile_order(std::ostringstream& o, int64_t ntx, int64_t nty, int64_t ntz, int TX, int TY, int TZ, int64_t default_sy = 0) {
+  // `bid` is the expression of the block number within the region (a launch can hold two regions with tile shapes of
+  // their own), `x_base` the region's first column.
+  int64_t emit_tile_order(std::ostringstream& o, int64_t ntx, int64_t nty, int64_t ntz, int TX, int TY, int TZ, int64_t default_sy = 0,
+                          const std::string& bid = "blockIdx.x", int64_t x_base = 0) {
     const int64_t nblocks = ntx * nty * ntz;
+    const std::string xb = x_base ? std::to_string(x_base) + " + " : std::string();
     if (!(opt.xcd_slabs && nty >= 16)) {
-      o << "  const unsigned tile = rx_xcd_remap(blockIdx.x, " << nblocks << "u);\n";
-      o << "  const int x0 = (int)(tile % " << ntx << "u) * " << TX << ";\n";
+      o << "  const unsigned tile = rx_xcd_remap(" << bid << ", " << nblocks << "u);\n";
+      o << "  const int x0 = " << xb << "(int)(tile % " << ntx << "u) * " << TX << ";\n";
       o << "  const int y0 = (int)((tile / " << ntx << "u) % " << nty << "u) * " << TY << ";\n";
       o << "  const int z0 = (int)(tile / " << ntx * nty << "u) * " << TZ << ";\n";
       return nblocks;
@@ -981,12 +985,12 @@ struct Planner {
     sy = std::min<int64_t>(sy, (nty + 7) / 8);
     const int64_t nslabs = (nty + sy - 1) / sy, rounds = (nslabs + 7) / 8;
     const int64_t per_slab = ntz * ntx * sy;
-    o << "  const unsigned xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;\n";
+    o << "  const unsigned xcd = " << bid << " & 7u, j = " << bid << " >> 3;\n";
     o << "  const unsigned slab = (j / " << per_slab << "u) * 8u + xcd, r = j % " << per_slab << "u;\n";
     o << "  const unsigned tz = r / " << ntx * sy << "u, rr = r % " << ntx * sy << "u;\n";
     o << "  const unsigned ty = slab * " << sy << "u + rr / " << ntx << "u;\n";
     o << "  if (ty >= " << nty << "u) return;\n";
-    o << "  const int x0 = (int)(rr % " << ntx << "u) * " << TX << ";\n";
+    o << "  const int x0 = " << xb << "(int)(rr % " << ntx << "u) * " << TX << ";\n";
     o << "  const int y0 = (int)ty * " << TY << ";\n";
     o << "  const int z0 = (int)tz * " << TZ << ";\n";
     return 8 * rounds * per_slab;
@@ -1438,14 +1442,22 @@ struct Planner {
     if (g.nodes[src].ty.dims != dims) return false;
     const int vec = spR.vec;
     const Halo hR = spR.halos.at(prev), hP = spP.halos.at(src);
-    const int TY = opt.march2_tile[0], TX = opt.march2_tile[1];
-    if (TX % vec) return false;
-    const int TXV = TX / vec, NB = TXV * TY;
-    if (NB < 64 || NB > 1024 || NB % 64) return false;
     const int64_t Z = dims[0], Y = dims[1], X = dims[2];
     // planes per workgroup: the extent is cut into equal chunks of about march2_planes
     const int64_t nchunks = std::max<int64_t>(1, (Z + opt.march2_planes - 1) / opt.march2_planes);
     const int64_t ZC = (Z + nchunks - 1) / nchunks;
+    // A launch holds one or two regions of columns [x_lo, x_hi), each with a tile shape of its own (same number of
+    // threads); `bid` is the block number within the region.
+    struct Region {
+      std::string text, note;
+      int64_t blocks = 0, lds_a = 0, lds_b = 0;
+      int nb = 0, prev_slot = -1;
+      std::vector<int> inputs, first_inputs, reads2;
+    };
+    auto gen = [&](int TY, int TX, int64_t x_lo, int64_t x_hi, const std::string& bid, Region* R) -> bool {
+    if (TX % vec) return false;
+    const int TXV = TX / vec, NB = TXV * TY;
+    if (NB < 64 || NB > 1024 || NB % 64) return false;
     auto up = [&](int64_t v) { return (v + vec - 1) / vec * vec; };
     const int64_t bxl = up(hR.lo[2]), bxh = up(hR.hi[2]);
     const int64_t BY = TY + hR.lo[1] + hR.hi[1], BX = TX + bxl + bxh, BXV = BX / vec;
@@ -1500,23 +1512,9 @@ struct Planner {
     const int prev_slot = ec.slot_of(prev), sslot = ec.slot_of(src);
     auto vts_of = [&](Emitter& em, int slot) { return "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vec) + ">"; };
 
-    const std::string kname = "@K@_stencil2m";
-    const int64_t ntx = (X + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + ZC - 1) / ZC;
+    const int64_t ntx = (x_hi - x_lo + TX - 1) / TX, nty = (Y + TY - 1) / TY, ntz = (Z + ZC - 1) / ZC;
     std::ostringstream o;
-    o << "// two stencil steps, marching along dim 0 (" << TY << "x" << TX << " outputs per plane, " << ZC << " planes per workgroup, rings of " << RA << " and "
-      << RB << " planes in LDS): " << describe(prev) << " ; " << describe(root) << " -> " << rn.ty.str() << "\n";
-    {
-      std::string s = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(NB) + ") void " + kname + "(";
-      for (size_t k = 0; k < ec.inputs.size(); ++k) {
-        if ((int)k == prev_slot) continue;
-        s += ptr_decl(info(g.nodes[ec.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k)) + ", ";
-      }
-      s += ptr_decl(st, false, "out0") + ")";
-      o << s << " {\n";
-    }
-    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsA[" << RA * APLANE << "];\n";
-    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << RB * BPLANE << "];\n";
-    const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, (int)ZC, std::max(1, 32 / TY));
+    const int64_t launch_blocks = emit_tile_order(o, ntx, nty, ntz, TX, TY, (int)ZC, std::max(1, 32 / TY), bid, x_lo);
     o << "  const int zend = z0 + " << ZC << " < " << Z << " ? z0 + " << ZC << " : " << Z << ";\n";
     // The first step is evaluated in two passes.  The inner pass maps thread -> point exactly as
     // the second step does, so the streamed inputs it loads for plane b are still in its registers
@@ -1675,24 +1673,78 @@ struct Planner {
         o << "#pragma unroll\n    for (int q = 0; q < " << NSP << "; ++q) us" << sl << "[q] = usn" << sl << par("P ^ 1") << "[q];\n";
     }
     o << "    rx_lds_barrier();\n";
-    if (PD == 2) o << "  };\n  for (int n = 0; n < nit; n += 2) {\n    iter(rx_int<0>{}, n);\n    if (n + 1 < nit) iter(rx_int<1>{}, n + 1);\n  }\n}\n\n";
-    else o << "  }\n}\n\n";
+    if (PD == 2) o << "  };\n  for (int n = 0; n < nit; n += 2) {\n    iter(rx_int<0>{}, n);\n    if (n + 1 < nit) iter(rx_int<1>{}, n + 1);\n  }\n";
+    else o << "  }\n";
+    R->text = o.str();
+    R->blocks = launch_blocks;
+    R->lds_a = RA * APLANE;
+    R->lds_b = RB * BPLANE;
+    R->nb = (int)NB;
+    R->prev_slot = prev_slot;
+    R->inputs = ec.inputs;
+    R->first_inputs = eb.inputs;
+    std::set<int> read2;
+    for (auto& l : ec.loads) read2.insert(l.node);
+    R->reads2.assign(read2.begin(), read2.end());
+    std::ostringstream note;
+    note << TY << "x" << TX << " outputs per plane, " << ZC << " planes per workgroup, rings of " << RA << " and " << RB << " planes in LDS";
+    R->note = note.str();
+    return true;
+    };
+    const int TY0 = opt.march2_tile[0], TX0 = opt.march2_tile[1];
+    std::vector<Region> regions(1);
+    // A last tile column that is nearly empty (518 columns in tiles of 64: eight full ones and six columns) costs as
+    // many workgroups as a full one, each as long-lived.  Those columns go to tiles a quarter as wide and four times as
+    // tall instead: the same number of threads, and for symmetric halos the same planes in LDS.
+    const int64_t rem = X % TX0;
+    bool split = false;
+    if (opt.march2_edge && rem > 0 && rem * 4 <= TX0 && X / TX0 >= 2 && (TX0 / 4) % spR.vec == 0 && TX0 / 4 >= 2 * spR.vec) {
+      std::vector<Region> two(2);
+      if (gen(TY0, TX0, 0, X - rem, "blockIdx.x", &two[0]) &&
+          gen(TY0 * 4, TX0 / 4, X - rem, X, "(blockIdx.x - " + std::to_string(two[0].blocks) + "u)", &two[1]) &&
+          two[0].nb == two[1].nb && two[0].inputs == two[1].inputs && two[0].prev_slot == two[1].prev_slot &&
+          std::max(two[0].lds_a, two[1].lds_a) + std::max(two[0].lds_b, two[1].lds_b) <= (two[0].lds_a + two[0].lds_b) * 5 / 4) {
+        regions = two;
+        split = true;
+      }
+    }
+    if (!split && !gen(TY0, TX0, 0, X, "blockIdx.x", &regions[0])) return false;
+    const Region& R0 = regions[0];
+    const std::string st = info(rn.ty.dt).stype;
+    const std::string kname = "@K@_stencil2m";
+    std::ostringstream o;
+    o << "// two stencil steps, marching along dim 0 (" << R0.note;
+    if (split) o << "; the last " << rem << " columns in tiles of " << regions[1].note;
+    o << "): " << describe(prev) << " ; " << describe(root) << " -> " << rn.ty.str() << "\n";
+    {
+      std::string sg = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(R0.nb) + ") void " + kname + "(";
+      for (size_t k = 0; k < R0.inputs.size(); ++k) {
+        if ((int)k == R0.prev_slot) continue;
+        sg += ptr_decl(info(g.nodes[R0.inputs[k]].ty.dt).stype, true, "in" + std::to_string(k)) + ", ";
+      }
+      sg += ptr_decl(st, false, "out0") + ")";
+      o << sg << " {\n";
+    }
+    int64_t lds_a = 0, lds_b = 0, launch_blocks = 0;
+    for (auto& R : regions) { lds_a = std::max(lds_a, R.lds_a); lds_b = std::max(lds_b, R.lds_b); launch_blocks += R.blocks; }
+    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsA[" << lds_a << "];\n";
+    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << lds_b << "];\n";
+    if (split) o << "  if (blockIdx.x < " << R0.blocks << "u) {\n" << R0.text << "  } else {\n" << regions[1].text << "  }\n";
+    else o << R0.text;
+    o << "}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;
     L.kernel = named(kname, kb_final);
     L.kind = "map_stencil_lds2";
     L.grid[0] = (unsigned)launch_blocks;
-    L.block[0] = NB;
-    std::vector<int> ins;
-    for (size_t k = 0; k < ec.inputs.size(); ++k) {
-      if ((int)k == prev_slot) continue;
-      ins.push_back(ec.inputs[k]);
-      L.args.push_back(buffer_for(ec.inputs[k]));
+    L.block[0] = R0.nb;
+    for (size_t k = 0; k < R0.inputs.size(); ++k) {
+      if ((int)k == R0.prev_slot) continue;
+      L.args.push_back(buffer_for(R0.inputs[k]));
     }
     L.args.push_back(buffer_for(root));
-    std::set<int> read2;
-    for (auto& l : ec.loads) read2.insert(l.node);
-    L.algo_bytes = algo_bytes(eb.inputs, {prev}) + algo_bytes(std::vector<int>(read2.begin(), read2.end()), {root});
+    // both steps' compulsory traffic: the first step's inputs and output, then the second's
+    L.algo_bytes = algo_bytes(R0.first_inputs, {prev}) + algo_bytes(R0.reads2, {root});
     L.desc = describe(prev) + " ; " + describe(root);
     plan.launches.push_back(L);
     return true;

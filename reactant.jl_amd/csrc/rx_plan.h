@@ -65,6 +65,7 @@ struct PlanOptions {
   int lds2_threads = 512;          // its workgroup size
   bool stencil_march2 = true;      // two-step kernel marching along the slowest dimension instead of 3-D tiles
   int march2_tile[2] = {8, 64};    // its outputs per plane (rows, columns)
+  bool march2_edge = true;         // a nearly empty last tile column is covered by tiles a quarter as wide, four times as tall
   int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
   bool transpose_vectors = true;   // transposing maps move 16-byte vectors where the dimensions allow it
   int transpose_block = 8;         // their tiles are taken in blocks of this many by this many (1: plain order)
