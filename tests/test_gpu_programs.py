@@ -228,6 +228,25 @@ def test_stencil_marching_chunks_and_tiles(rx, client, monkeypatch, planes, tile
         assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("shape,elt,tile", [((134, 70, 9), "f64", "8,64"), ((200, 33, 5), "f32", "8,64"), ((390, 20, 12), "f32", "8,64"),
+                                            ((262, 9, 30), "f64", "8,64")])
+def test_stencil_edge_columns_in_tiles_of_their_own(rx, client, monkeypatch, shape, elt, tile):
+    """A nearly empty last tile column is covered by tiles a quarter as wide and four times as tall in the same launch:
+    same bits as the oracle's and as the kernel with one tile shape."""
+    monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
+    monkeypatch.setenv("RX_MARCH2_TILE", tile)
+    monkeypatch.setenv("RX_MARCH2_PLANES", "4")
+    text = P.stencil(*shape, steps=2, elt=elt)
+    assert "columns in tiles of" in rx.compile_offline(text, with_source=True)
+    got, ref, exe = _stencil_case(rx, client, shape, "pad", 2, elt=elt)
+    assert exe.launches()[0]["kernel"].endswith("_stencil2m")
+    assert np.array_equal(got, ref)
+    monkeypatch.setenv("RX_MARCH2_EDGE", "0")
+    assert "columns in tiles of" not in rx.compile_offline(text, with_source=True)
+    one, _, exe1 = _stencil_case(rx, client, shape, "pad", 2, elt=elt)
+    assert np.array_equal(one, got)
+
+
 def test_stencil_two_steps_f32_and_unfused_agree(rx, client, monkeypatch):
     monkeypatch.setenv("RX_SLAB_MIN_NUMEL", "1")
     got, ref, exe = _stencil_case(rx, client, (72, 24, 10), "pad", 2, elt="f32")
