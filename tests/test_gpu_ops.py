@@ -377,6 +377,14 @@ def test_transpose_through_lds_tiles(rx, client, shape, perm, dt):
     assert np.array_equal(got[0].a, oracle_run(text, [x])[0].a)
 
 
+@pytest.mark.parametrize("block", ["1", "3", "16"])
+@pytest.mark.parametrize("shape,perm,dt", [((1100, 1300), (1, 0), "f32"), ((3, 700, 129), (0, 2, 1), "f32"), ((2, 1000, 72), (0, 2, 1), "f64")])
+def test_transposing_tiles_in_blocks_of_other_sizes(rx, client, monkeypatch, block, shape, perm, dt):
+    """The order in which the tiles are taken (blocks of B x B, ragged at the edges of the tile grid) does not change a value."""
+    monkeypatch.setenv("RX_TRANSPOSE_BLOCK", block)
+    test_transpose_through_lds_tiles(rx, client, shape, perm, dt)
+
+
 def test_map_with_transposed_and_plain_operands(rx, client):
     """sin(a') * b + c' in one kernel: two transposed reads share the tiling, one operand is read in place."""
     m, n = 200, 330

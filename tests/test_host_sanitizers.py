@@ -31,6 +31,12 @@ def corpus():
         "fp8_small": P.fp8_linear(8, 32, 16), "fp8_kn": P.fp8_linear(128, 256, 128, weight_layout="kn"),
         "fp8_direct": P.fp8_linear(8, 32, 16, weight_layout="kn", dot_form="direct"), "fp8_full": P.fp8_linear(8192, 8192, 8192),
         "cumsum": NN.cumulative([1 << 20], "f32", 0), "cumsum_rows": NN.cumulative([512, 384], "f32", 1, reverse=True),
+        "cumsum_long": NN.cumulative([1 << 26], "f32", 0), "cumsum_long_rows": NN.cumulative([3, 9000000], "i64", 1),
+        "transpose": "module { func.func @main(%a: tensor<520x264xf64>) -> tensor<264x520xf64> { %0 = stablehlo.transpose %a, dims = [1, 0] : "
+                     "(tensor<520x264xf64>) -> tensor<264x520xf64>\n return %0 : tensor<264x520xf64> } }",
+        "transpose_batched": "module { func.func @main(%a: tensor<5x1000x72xf32>) -> tensor<5x72x1000xf32> { %0 = stablehlo.transpose %a, dims = [0, 2, 1] : "
+                             "(tensor<5x1000x72xf32>) -> tensor<5x72x1000xf32>\n return %0 : tensor<5x72x1000xf32> } }",
+        "stencil_edge": P.stencil(134, 70, 9, steps=2), "stencil_edge_f32": P.stencil(390, 20, 12, steps=3, elt="f32"),
         "maxpool": NN.reduce_window([4, 8, 32, 32], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])[0],
         "conv": NN.convolution([2, 8, 16, 16], [4, 8, 3, 3], "f32", padding=[[1, 1], [1, 1]])[0],
         "conv_groups": NN.convolution([2, 8, 16, 16], [4, 4, 3, 3], "f32", groups=2)[0],
