@@ -3197,7 +3197,10 @@ struct Planner {
           o << "  const " << it << " c = (" << it << ")(blockIdx.x % " << sNC << "u), row = (" << it << ")(blockIdx.x / " << sNC << "u);\n";
           decompose(o, "row", 0, a);
           for (int d = a + 1; d < ty.rank(); ++d) o << "  const " << it << " q" << d << " = 0;\n";
-          o << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << sCH << ", " << n << ");\n";
+          // rows that are a whole number of chunks need none of the guards below
+          const bool whole = n % sCH == 0;
+          const std::string in_chunk = whole ? "true" : "pb < pend", in_row = whole ? "true" : "p < pend";
+          o << "  const " << it << " pend = rx_min<" << it << ">((c + 1) * " << sCH << ", " << n << ");\n  (void)pend;\n";
           o << ibody;
           o << "  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;\n";
           o << "  const rx_u32 epoch = (rx_u32)slots[" << outer * SL * NW << " + row] + 1u;\n";
@@ -3215,7 +3218,7 @@ struct Planner {
               const int slot = sd.first;
               const std::string vt = "rx_vec<" + std::string(info(g.nodes[em.inputs[slot]].ty.dt).stype) + ", " + std::to_string(vecw) + ">";
               o << "    " << vec_name(slot, 0) << "t[t] = " << vt << "{};\n";
-              o << "    if (pb < pend) " << vec_name(slot, 0) << "t[t] = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + row * " << n << " + pb);\n";
+              o << "    if (" << in_chunk << ") " << vec_name(slot, 0) << "t[t] = " << (opt.nt_loads ? "rx_load_nt" : "rx_load") << "<" << vt << ">(in" << slot << " + row * " << n << " + pb);\n";
             }
             o << "  }\n";
           }
@@ -3225,7 +3228,7 @@ struct Planner {
             o << "    const " << it << " lin0 = row * " << n << " + pb;\n    (void)lin0;\n";
             for (auto& sd : em.direct_vecs) o << "    const auto& " << vec_name(sd.first, 0) << " = " << vec_name(sd.first, 0) << "t[t];\n";
           }
-          o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      v[t][l] = " << IDENT << ";\n      if (p < pend) {\n";
+          o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      v[t][l] = " << IDENT << ";\n      if (" << in_row << ") {\n";
           o << "        const " << it << " j = " << jexpr << ";\n" << body;
           o << "        v[t][l] = (" << ACC << ")" << val << ";\n      }\n    }\n  }\n";
           // The chunk's total goes out before the scans inside the chunk, in an order of its own (values of a lane,
@@ -3275,13 +3278,13 @@ struct Planner {
           o << "    const " << it << " pb = c * " << sCH << " + t * " << TILE << " + (" << it << ")threadIdx.x * " << V << ";\n";
           o << "    const " << ACC << " pt = " << red_apply(rn.red, dt, "carry", "pre[t]") << ";\n";
           if (vecw > 1) {
-            o << "    if (pb < pend) {\n      rx_vec<" << ost << ", " << V << "> res;\n";
+            o << "    if (" << in_chunk << ") {\n      rx_vec<" << ost << ", " << V << "> res;\n";
             o << "#pragma unroll\n      for (int l = 0; l < " << V << "; ++l) {\n";
             o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pt", "v[t][l]") << ";\n";
             o << "        res.v[l] = " << Emitter::store_conv(dt, rv) << ";\n      }\n";
             o << "      *reinterpret_cast<rx_vec<" << ost << ", " << V << ">*>(out0 + row * " << n << " + pb) = res;\n    }\n";
           } else {
-            o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (p < pend) {\n";
+            o << "#pragma unroll\n    for (int l = 0; l < " << V << "; ++l) {\n      const " << it << " p = pb + l;\n      if (" << in_row << ") {\n";
             o << "        const " << ACC << " r = " << red_apply(rn.red, dt, "pt", "v[t][l]") << ";\n";
             o << "        out0[row * " << n << " + (" << jexpr << ")] = " << Emitter::store_conv(dt, rv) << ";\n      }\n    }\n";
           }
