@@ -11,7 +11,7 @@ that advances two timesteps per launch: its algorithmic bytes are those of both)
 region.  `cpu_baseline` times the oracle's C/OpenMP restatement of the stencil on the
 host cores (a bounded number of repetitions of the same module, same inputs).  `others` carries the remaining four configs
 (sinsum_add, f32 GEMM, bf16 MLP, FP8 linear), each with its own roofline entry, its own `check` against the oracle and
-its own `cpu_baseline`; their step time is the median over groups of plain executions, and the pass with an event pair
+its own `cpu_baseline`; their step time is the median over five runs of the K plain executions, and the pass with an event pair
 on every launch is reported beside it.  Every workload's result is verified after its timed region (`check`):
 the stencil bit for bit against the C restatement, the others on sampled rows against float64 / the numpy oracle.
 `roofline.traffic` is read from profiles/bench_all_configs_hbm_traffic.txt (rocprofv3 counters) and is null when the
@@ -125,22 +125,20 @@ def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
 
 def _time_plain(client, exe, bufs, steps, warmup):
     """K steps as a caller runs them: queued without waiting, no event pair on the launches (a pair
-    costs a few microseconds of stream time, which shows on steps of less than 0.1 ms).  The K steps run in up to
-    five groups, each queued whole and timed by the host clock around a synchronization; returns the median of
-    the groups' seconds per step."""
+    costs a few microseconds of stream time, which shows on steps of less than 0.1 ms).  The K steps are run five
+    times, each run queued whole and timed by the host clock around a synchronization (whose wake-up, some tens of
+    microseconds, is spread over the K steps of a run); returns the median of the runs' seconds per step."""
     dev = client.default_device()
     for _ in range(warmup):
         exe.execute_sharded(bufs)
     dev.synchronize()
-    groups = max(1, min(5, steps // 2))
-    per = max(1, steps // groups)
     times = []
-    for _ in range(groups):
+    for _ in range(5):
         t0 = time.perf_counter()
-        for _ in range(per):
+        for _ in range(steps):
             exe.execute_sharded(bufs)
         dev.synchronize()
-        times.append((time.perf_counter() - t0) / per)
+        times.append((time.perf_counter() - t0) / steps)
     return float(np.median(times))
 
 
