@@ -44,17 +44,18 @@ RX_CHECK_DL(rx_check_dl_bf16x16_tn, rx_mma_bf16_16, 128, 256, 64, 4, 2, false, f
 RX_CHECK_DL(rx_check_dl_f16x16_tt, rx_mma_f16_16, 128, 128, 64, 2, 2, false, true)
 RX_CHECK_DL(rx_check_dl_f8_nt, rx_mma_f8, 256, 256, 128, 2, 4, true, true)
 
-// the streaming body (16x16 MFMA shapes), 8- and 16-bit operands, all four operand layouts, 256x256 and 256x128 tiles
-#define RX_CHECK_S(NAME, EL, BM, BN, AKC, BKC, K)                                                                        \
+// the streaming body (16x16 MFMA shapes), 8- and 16-bit operands, all four operand layouts, 256x256 tiles (wavefronts of 128x64) and 256x128 tiles (64x64; 128x32 by request)
+#define RX_CHECK_S(NAME, EL, BM, BN, WM, WN, AKC, BKC, K)                                                                \
   extern "C" __global__ __launch_bounds__(512) void NAME(const EL::elem* A, const EL::elem* B, float* out) {              \
     rx_check_epi<float, 512> epi{out};                                                                                     \
-    rx_gemm_body_s<EL, BM, BN, 2, 4, AKC, BKC, 512, 512, K, 0, 0, false, rx_check_epi<float, 512>>(A, B, epi);              \
+    rx_gemm_body_s<EL, BM, BN, WM, WN, AKC, BKC, 512, 512, K, 0, 0, false, rx_check_epi<float, 512>>(A, B, epi);            \
   }
-RX_CHECK_S(rx_check_s_f8_nt, rx_el_f8, 256, 256, true, true, 512)
-RX_CHECK_S(rx_check_s_f8_nn, rx_el_f8, 256, 256, true, false, 384)
-RX_CHECK_S(rx_check_s_f8_tn, rx_el_f8, 256, 128, false, false, 128)
-RX_CHECK_S(rx_check_s_f8_tt, rx_el_f8, 256, 256, false, true, 256)
-RX_CHECK_S(rx_check_s_bf16_nn, rx_el_bf16, 256, 256, true, false, 512)
-RX_CHECK_S(rx_check_s_bf16_nt, rx_el_bf16, 256, 128, true, true, 64)
-RX_CHECK_S(rx_check_s_f16_tn, rx_el_f16, 256, 256, false, false, 192)
-RX_CHECK_S(rx_check_s_f16_tt, rx_el_f16, 256, 128, false, true, 128)
+RX_CHECK_S(rx_check_s_f8_nt, rx_el_f8, 256, 256, 2, 4, true, true, 512)
+RX_CHECK_S(rx_check_s_f8_nn, rx_el_f8, 256, 256, 2, 4, true, false, 384)
+RX_CHECK_S(rx_check_s_f8_tn, rx_el_f8, 256, 128, 4, 2, false, false, 128)
+RX_CHECK_S(rx_check_s_f8_tt, rx_el_f8, 256, 256, 2, 4, false, true, 256)
+RX_CHECK_S(rx_check_s_bf16_nn, rx_el_bf16, 256, 256, 2, 4, true, false, 512)
+RX_CHECK_S(rx_check_s_bf16_nt, rx_el_bf16, 256, 128, 4, 2, true, true, 64)
+RX_CHECK_S(rx_check_s_bf16_nt24, rx_el_bf16, 256, 128, 2, 4, true, true, 64)
+RX_CHECK_S(rx_check_s_f16_tn, rx_el_f16, 256, 256, 2, 4, false, false, 192)
+RX_CHECK_S(rx_check_s_f16_tt, rx_el_f16, 256, 128, 4, 2, false, true, 128)

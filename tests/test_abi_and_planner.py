@@ -351,7 +351,7 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
     mlp = rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
     assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in mlp      # the 4096^2 layer
-    assert "rx_gemm_body_s<rx_el_bf16, 256, 128, 2, 4, true, false, 8192, 1024, 4096" in mlp      # the last layer: 256x128 tiles
+    assert "rx_gemm_body_s<rx_el_bf16, 256, 128, 4, 2, true, false, 8192, 1024, 4096" in mlp      # the last layer: 256x128 tiles, wavefronts of 64x64
     monkeypatch.setenv("RX_GEMM_STREAM", "0")
     src = rx.compile_offline(big, with_source=True)
     assert "rx_gemm_body_s<" not in src and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in src
