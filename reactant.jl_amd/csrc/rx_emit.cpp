@@ -256,6 +256,29 @@ bool Emitter::is_uniform(int node, int depth) const {
   }
 }
 
+// The value does not vary along the node's last dimension (a row's reduction result broadcast back over the row).
+bool Emitter::minor_uniform(int node, int depth) const {
+  const Node& n = g_.nodes[node];
+  if (n.ty.rank() == 0) return true;
+  if (depth > 8) return false;
+  switch (n.k) {
+    case OpK::Constant: return n.splat;
+    case OpK::BroadcastInDim: {
+      const Node& o = g_.nodes[n.in[0]];
+      for (size_t d = 0; d < n.a0.size(); ++d)
+        if (n.a0[d] == n.ty.rank() - 1 && o.ty.dims[d] != 1) return false;
+      return true;
+    }
+    case OpK::Convert:
+    case OpK::Unary:
+      return minor_uniform(n.in[0], depth + 1);
+    case OpK::Binary:
+      return minor_uniform(n.in[0], depth + 1) && minor_uniform(n.in[1], depth + 1);
+    default:
+      return false;
+  }
+}
+
 // n = (0.5 * x) * (1 + tanh(a * (x + b * ((x * x) * x)))) in any operand order, every intermediate value computed in
 // this kernel and of n's type; a, b constants.
 bool Emitter::match_gelu_chain(const Node& n, int* xnode, double* ka, double* kb) const {
@@ -354,7 +377,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (op == "cosine") return def(fn("cos", dbl) + "(" + x + ")");
         if (op == "tan") return def(fn("tan", dbl) + "(" + x + ")");
         if (op == "tanh") return def((is_narrow_float(dt) ? std::string("rx_tanh_fast") : fn("tanh", dbl)) + "(" + x + ")");
-        if (op == "exponential") return def(fn("exp", dbl) + "(" + x + ")");
+        if (op == "exponential") return def((is_narrow_float(dt) ? std::string("rx_exp_fast") : fn("exp", dbl)) + "(" + x + ")");
         if (op == "exponential_minus_one") return def(fn("expm1", dbl) + "(" + x + ")");
         if (op == "log") return def(fn("log", dbl) + "(" + x + ")");
         if (op == "log_plus_one") return def(fn("log1p", dbl) + "(" + x + ")");
@@ -419,6 +442,10 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
           // quantization scale): its reciprocal in double is loop-invariant, and the product in
           // double rounds to the same float as the division (see rx_div_uniform)
           if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
+          // a result that is rounded to a narrow float, divided by a value that is the same along the minor dimension
+          // (the sum of a softmax row): its reciprocal, a division of its own that the compiler computes once per
+          // row, times the dividend -- within an ulp of float32 of the quotient
+          if (CT == "float" && is_narrow_float(dt) && excess_precision && minor_uniform(n.in[1])) return def("(" + a + " * (1.0f / " + b + "))");
           return def("(" + a + " / " + b + ")");
         }
         if (op == "maximum") return def("rx_max(" + a + ", " + b + ")");

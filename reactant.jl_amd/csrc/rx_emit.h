@@ -103,6 +103,7 @@ class Emitter {
   bool allow_direct_ = false;
 
   bool is_uniform(int node, int depth = 0) const;
+  bool minor_uniform(int node, int depth = 0) const;
   std::string emit_load(int node, const Index& ix);
   std::string emit_op(const Node& n, const Index& ix);
   bool match_gelu_chain(const Node& n, int* xnode, double* ka, double* kb) const;

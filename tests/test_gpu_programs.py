@@ -371,6 +371,67 @@ def test_gelu_chain_on_every_value(rx, client, dt):
     assert np.all(np.abs(g[fin] - ref[fin]) <= np.maximum(ulp, tiny) + np.abs(xv[fin]) * 2.0 ** -22)
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_exponential_of_every_narrow_value(rx, client, dt):
+    """exp over every 16-bit pattern: narrow results take the hardware 2^y on y = x log2(e).  Within one ulp of the
+    exponential evaluated in float64 and rounded once; overflow to inf, underflow to zero and NaN as the exact result;
+    results below the smallest normal float32 (bf16 subnormals) may be flushed to zero."""
+    n = 1 << 16
+    ty = P._tt([n], dt)
+    text = "module {\n  func.func @main(%%arg0: %s) -> %s {\n    %%0 = stablehlo.exponential %%arg0 : %s\n    return %%0 : %s\n  }\n}\n" % (ty, ty, ty, ty)
+    x = I.Tensor.from_bytes(np.arange(n, dtype=np.uint16).tobytes(), dt, (n,))
+    got, _ = gpu_run(rx, client, text, [x])
+    assert "rx_exp_fast" in rx.compile_offline(text, with_source=True)
+    with np.errstate(all="ignore"):
+        xv = x.a.astype(np.float64)
+        exact = np.exp(xv)
+        ref = I.tensor(exact, dt).a.astype(np.float64)
+    g = got[0].a.astype(np.float64)
+    assert np.array_equal(np.isnan(g), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    inf = ok & np.isinf(ref)
+    # at the overflow threshold the rounded exact result may be the largest finite value where the GPU gives inf, or the reverse
+    big = np.finfo(np.float32).max if dt == "bf16" else 65504.0
+    assert np.all((g[inf] == np.inf) | (g[inf] >= big * 0.99))
+    fin = ok & np.isfinite(ref)
+    ulp = np.spacing(np.abs(ref[fin]).astype(np.float32)).astype(np.float64) * (2.0 ** (24 - (8 if dt == "bf16" else 11)))
+    tiny = 2.0 ** -126 if dt == "bf16" else 2.0 ** -24
+    d = np.abs(g[fin] - ref[fin])
+    assert np.all((d <= np.maximum(ulp, tiny)) | (np.isinf(g[fin]) & (ref[fin] >= big * 0.99)))
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_softmax_rows_with_extreme_sums(rx, client, dt):
+    """Softmax over rows whose sums of exponentials are tiny, ordinary and huge: the division by the row's sum is a
+    multiplication by its reciprocal (computed once per row by a true division) for narrow results; against the oracle,
+    one ulp of the exact quotient."""
+    rows, cols = 64, 1000
+    rng = np.random.default_rng(5)
+    x = rng.normal(size=(rows, cols))
+    hi = 80.0 if dt == "bf16" else 3.0
+    x += np.linspace(-hi, hi, rows)[:, None]          # sums from e^-80 * 1000 to e^80 * 1000 (bf16); f16 holds no more than 65504
+    ty, tr = P._tt([rows, cols], dt), P._tt([rows], dt)
+    text = ("module {\n  func.func @main(%%arg0: %s) -> %s {\n"
+            "    %%c = stablehlo.constant dense<0.0> : tensor<%s>\n"
+            "    %%0 = stablehlo.exponential %%arg0 : %s\n"
+            "    %%1 = stablehlo.reduce(%%0 init: %%c) applies stablehlo.add across dimensions = [1] : (%s, tensor<%s>) -> %s\n"
+            "    %%2 = stablehlo.broadcast_in_dim %%1, dims = [0] : (%s) -> %s\n"
+            "    %%3 = stablehlo.divide %%0, %%2 : %s\n    return %%3 : %s\n  }\n}\n" % (ty, ty, dt, ty, ty, dt, tr, tr, ty, ty, ty))
+    a = I.tensor(x, dt)
+    got, exe = gpu_run(rx, client, text, [a])
+    assert "(1.0f / " in rx.compile_offline(text, with_source=True)
+    xv = a.a.astype(np.float64)
+    e = np.exp(xv)
+    exact = e / e.sum(axis=1, keepdims=True)
+    g = got[0].a.astype(np.float64)
+    rel = 2.0 ** -7 if dt == "bf16" else 2.0 ** -10
+    # the kernel keeps the exponentials and the row's sum in float32 and rounds once: one ulp of the exact quotient
+    assert np.all(np.abs(g - exact) <= 1.01 * rel * exact + (1e-40 if dt == "bf16" else 2.0 ** -24))
+    # the oracle may round the row's sum to the narrow type before it is broadcast (it is a tensor of that type)
+    ref = oracle_run(text, [a], hifi=True, excess=True)[0].a.astype(np.float64)
+    assert np.all(np.abs(g - ref) <= 2.5 * rel * np.maximum(np.abs(ref), np.abs(g)) + (1e-40 if dt == "bf16" else 2.0 ** -24))
+
+
 @pytest.mark.parametrize("batch,k,n,layout,form", [(8, 32, 16, "nk", "convert"), (8, 32, 16, "kn", "direct"),
                                                    (64, 128, 256, "nk", "convert"), (128, 256, 128, "kn", "convert")])
 def test_fp8_linear(rx, client, batch, k, n, layout, form):
