@@ -178,6 +178,9 @@ RX_DEV float rx_tanh_fast(float x) {
 // about |x| 2^-24 + 2^-23, far below half an ulp of f16); saturates to 0 and inf like expf; results below the smallest
 // normal float32 (which only a bf16 result can hold) are flushed to zero.
 RX_DEV float rx_exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+// 1 / (1 + e^-x) for results that are rounded to a 16-bit or 8-bit float, on the hardware's 2^y and reciprocal
+// (absolute error about 1e-7); exactly 0 and 1 at the ends, NaN propagates.
+RX_DEV float rx_logistic_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f)); }
 // 0.5 x (1 + tanh(a (x + b x^3))) = x / (1 + e^(-2 a (x + b x^3))) for results that are rounded to a 16-bit or 8-bit
 // float; k1 = -2 a log2(e), k3 = k1 b.  The exponential saturates to 0 or inf at the ends, which gives x and -0 as the
 // chain does; x = -inf gives NaN as the chain does (-inf * 0); NaN propagates.  Where 1 + tanh cancels (x < -3) the

@@ -386,7 +386,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (op == "rsqrt") return def("rx_rsqrt(" + x + ")");
         if (op == "abs") return def(fn("fabs", dbl) + "(" + x + ")");
         if (op == "negate") return def("(-" + x + ")");
-        if (op == "logistic") return def("rx_logistic(" + x + ")");
+        if (op == "logistic") return def((is_narrow_float(dt) ? "rx_logistic_fast(" : "rx_logistic(") + x + ")");
         if (op == "floor") return def(fn("floor", dbl) + "(" + x + ")");
         if (op == "ceil") return def(fn("ceil", dbl) + "(" + x + ")");
         if (op == "sign") return def("rx_sign(" + x + ")");

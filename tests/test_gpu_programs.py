@@ -401,6 +401,30 @@ def test_exponential_of_every_narrow_value(rx, client, dt):
 
 
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
+def test_logistic_of_every_narrow_value(rx, client, dt):
+    """1 / (1 + e^-x) over every 16-bit pattern (narrow results: hardware 2^y and reciprocal): one ulp of the float64
+    result rounded once, exactly 0 and 1 at the ends, NaN where the input is NaN; results below the smallest normal
+    float32 may be flushed to zero."""
+    n = 1 << 16
+    ty = P._tt([n], dt)
+    text = "module {\n  func.func @main(%%arg0: %s) -> %s {\n    %%0 = stablehlo.logistic %%arg0 : %s\n    return %%0 : %s\n  }\n}\n" % (ty, ty, ty, ty)
+    x = I.Tensor.from_bytes(np.arange(n, dtype=np.uint16).tobytes(), dt, (n,))
+    got, _ = gpu_run(rx, client, text, [x])
+    assert "rx_logistic_fast" in rx.compile_offline(text, with_source=True)
+    with np.errstate(all="ignore"):
+        xv = x.a.astype(np.float64)
+        exact = 1.0 / (1.0 + np.exp(-xv))
+        ref = I.tensor(exact, dt).a.astype(np.float64)
+    g = got[0].a.astype(np.float64)
+    assert np.array_equal(np.isnan(g), np.isnan(ref))
+    fin = ~np.isnan(ref)
+    ulp = np.spacing(np.abs(ref[fin]).astype(np.float32)).astype(np.float64) * (2.0 ** (24 - (8 if dt == "bf16" else 11)))
+    tiny = 2.0 ** -126 if dt == "bf16" else 2.0 ** -24
+    assert np.all(np.abs(g[fin] - ref[fin]) <= np.maximum(ulp, tiny))
+    assert g[fin].min() >= 0.0 and g[fin].max() <= 1.0
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
 def test_softmax_rows_with_extreme_sums(rx, client, dt):
     """Softmax over rows whose sums of exponentials are tiny, ordinary and huge: the division by the row's sum is a
     multiplication by its reciprocal (computed once per row by a true division) for narrow results; against the oracle,
