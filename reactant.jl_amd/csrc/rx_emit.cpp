@@ -441,11 +441,11 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
           // a divisor that is one value for the whole tensor (a broadcast scalar, e.g. a
           // quantization scale): its reciprocal in double is loop-invariant, and the product in
           // double rounds to the same float as the division (see rx_div_uniform)
-          if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
           // a result that is rounded to a narrow float, divided by a value that is the same along the minor dimension
-          // (the sum of a softmax row): its reciprocal, a division of its own that the compiler computes once per
-          // row, times the dividend -- within an ulp of float32 of the quotient
-          if (CT == "float" && is_narrow_float(dt) && excess_precision && minor_uniform(n.in[1])) return def("(" + a + " * (1.0f / " + b + "))");
+          // (the sum of a softmax row, a quantization scale): its reciprocal, a division of its own that the compiler
+          // computes once per row, times the dividend -- within an ulp of float32 of the quotient
+          if (CT == "float" && is_narrow_float(dt) && excess_precision && n.ty.rank() > 0 && minor_uniform(n.in[1])) return def("(" + a + " * (1.0f / " + b + "))");
+          if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
           return def("(" + a + " / " + b + ")");
         }
         if (op == "maximum") return def("rx_max(" + a + ", " + b + ")");
