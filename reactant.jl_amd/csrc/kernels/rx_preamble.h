@@ -114,6 +114,9 @@ RX_DEV rx_u8 rx_f32_to_e4m3(float f) {
   const rx_u32 code = a > 0x43e80000u ? 0x7fu : (packed & 0x7fu);
   return (rx_u8)(((u >> 24) & 0x80u) | code);
 }
+// The same for a value known to be finite with |x| <= 448, or NaN: the hardware conversion alone.  A NaN becomes the
+// code 0xff whatever its sign (rx_f32_to_e4m3 keeps the sign: 0x7f or 0xff; both are NaN).
+RX_DEV rx_u8 rx_f32_to_e4m3_inrange(float f) { return (rx_u8)__builtin_amdgcn_cvt_pk_fp8_f32(f, f, 0, false); }
 RX_DEV rx_u8 rx_f32_to_e4m3_sw(float f) {
   rx_u32 u = rx_f2u(f);
   rx_u8 s = (rx_u8)((u >> 24) & 0x80u);

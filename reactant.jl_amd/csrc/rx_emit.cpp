@@ -90,7 +90,23 @@ std::string Emitter::store_conv(DT dt, const std::string& val) {
   }
 }
 
+// `e` with casts to float and enclosing parentheses taken off
+static std::string bare_name(std::string e) {
+  for (;;) {
+    if (e.size() >= 2 && e.front() == '(' && e.back() == ')' && e.find(')') == e.size() - 1) e = e.substr(1, e.size() - 2);
+    else if (e.compare(0, 7, "(float)") == 0) e = e.substr(7);
+    else return e;
+  }
+}
+
 std::string Emitter::store_value(DT dt, const std::string& val) const {
+  // a value that a clamp has just put inside the range of e4m3 (what a quantization does): the hardware conversion
+  // by itself, without the range handling around it
+  if (dt == DT::F8E4M3FN) {
+    auto r = rounded_.find(val);
+    const std::string src = bare_name(r != rounded_.end() && r->second.first == dt ? r->second.second : val);
+    if (e4m3_range_.count(src)) return "rx_f32_to_e4m3_inrange(" + src + ")";
+  }
   auto it = rounded_.find(val);
   if (it != rounded_.end() && it->second.first == dt) return store_conv(dt, "(" + it->second.second + ")");
   return store_conv(dt, val);
@@ -503,7 +519,11 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
           return true;
         };
         double lv, hv;
-        if (CT == "float" && const_bound(0, &lv) && const_bound(2, &hv) && lv <= hv) return def("rx_clamp_ordered(" + x + ", " + lo + ", " + hi + ")");
+        if (CT == "float" && const_bound(0, &lv) && const_bound(2, &hv) && lv <= hv) {
+          const std::string v = def("rx_clamp_ordered(" + x + ", " + lo + ", " + hi + ")");
+          if (lv >= -448.0 && hv <= 448.0 && dt == DT::F32) e4m3_range_.insert(v);
+          return v;
+        }
         return def("rx_min(rx_max(" + x + ", " + lo + "), " + hi + ")");
       }
       return def("(" + CT + ")((" + x + " < " + lo + " ? " + lo + " : " + x + ") > " + hi + " ? " + hi + " : (" + x + " < " + lo + " ? " + lo + " : " + x + "))");

@@ -97,6 +97,7 @@ class Emitter {
   std::vector<std::map<std::string, std::string>> scopes_{1};
   int tmp_ = 0;
   std::map<std::string, std::pair<DT, std::string>> rounded_;   // variable -> (type it was rounded to, unrounded expression)
+  std::set<std::string> e4m3_range_;   // float values known to lie in [-448, 448] (or to be NaN)
   int unsafe_loads_ = 0;   // loads emitted as plain global reads at a computed index
   std::vector<int64_t> root_dims_;
   std::vector<std::string> root_vars_;

@@ -230,6 +230,22 @@ def test_convert_f32_to_narrow_bit_exact(rx, client, dt):
     assert (same | nan).all(), x[~(same | nan)][:10]
 
 
+def test_convert_of_a_clamped_value_to_e4m3_bit_exact(rx, client):
+    """clamp(x, -448, 448) followed by the conversion to e4m3 (a quantization): the conversion is the hardware
+    instruction alone there; the same bytes as the oracle's on every interesting float32 (ties, subnormals, both
+    zeros, values far outside the range), NaN stays NaN."""
+    x = _interesting_f32()
+    t, o = _tt(x.shape, "f32"), _tt(x.shape, "f8E4M3FN")
+    text = mod([t], o, "    %%lo = stablehlo.constant dense<-448.0> : %s\n    %%hi = stablehlo.constant dense<448.0> : %s\n"
+               "    %%0 = stablehlo.clamp %%lo, %%arg0, %%hi : %s\n    %%1 = stablehlo.convert %%0 : (%s) -> %s\n    return %%1 : %s\n" % (t, t, t, t, o, o))
+    assert "rx_f32_to_e4m3_inrange" in rx.compile_offline(text, with_source=True)
+    got, ref = both(rx, client, text, [I.Tensor(x, "f32")])
+    gb, rb = np.frombuffer(got[0].to_bytes(), np.uint8), np.frombuffer(ref[0].to_bytes(), np.uint8)
+    nan = np.isnan(got[0].a) & np.isnan(ref[0].a)
+    assert ((gb == rb) | nan).all(), x[~((gb == rb) | nan)][:10]
+    assert np.array_equal(np.isnan(got[0].a), np.isnan(ref[0].a))
+
+
 @pytest.mark.parametrize("dt", ["bf16", "f8E4M3FN", "f8E5M2", "f16"])
 def test_convert_narrow_to_f32_exact(rx, client, dt):
     n = 65536 if I.ITEMSIZE[dt] == 2 else 256
