@@ -400,6 +400,37 @@ def test_exponential_of_every_narrow_value(rx, client, dt):
     assert np.all((d <= np.maximum(ulp, tiny)) | (np.isinf(g[fin]) & (ref[fin] >= big * 0.99)))
 
 
+def test_division_by_a_row_value_special_cases(rx, client):
+    """bf16 rows divided by a per-row value (the reciprocal form): divisors that are zero, infinite, NaN, huge, tiny and
+    subnormal against dividends of every kind.  Finite quotients within an ulp of the exact one (or both zero / both
+    beyond the largest bf16), infinities and NaNs where IEEE division has them."""
+    big, tiny = 3.0e38, 1.2e-38
+    divisors = np.array([1.0, -3.0, 0.0, -0.0, np.inf, -np.inf, np.nan, big, -big, tiny, 4.0e-39, 1.0e-30, 7.0e20, 0.333], dtype=np.float64)
+    dividends = np.array([0.0, -0.0, 1.0, -1.0, 2.5, np.inf, -np.inf, np.nan, big, -big, tiny, 1.0e-20, 6.0e15, 0.1, 100.0, -7.0], dtype=np.float64)
+    rows, cols = len(divisors), 64
+    x = np.tile(np.resize(dividends, cols), (rows, 1))
+    ty, tr = P._tt([rows, cols], "bf16"), P._tt([rows], "bf16")
+    text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%0 = stablehlo.broadcast_in_dim %%arg1, dims = [0] : (%s) -> %s\n"
+            "    %%1 = stablehlo.divide %%arg0, %%0 : %s\n    return %%1 : %s\n  }\n}\n" % (ty, tr, ty, tr, ty, ty, ty))
+    assert "(1.0f / " in rx.compile_offline(text, with_source=True)
+    a, b = I.tensor(x, "bf16"), I.tensor(divisors, "bf16")
+    got, _ = gpu_run(rx, client, text, [a, b])
+    g = got[0].a.astype(np.float64)
+    with np.errstate(all="ignore"):
+        exact = a.a.astype(np.float64) / b.a.astype(np.float64)[:, None]
+        ref = I.tensor(exact, "bf16").a.astype(np.float64)
+    assert np.array_equal(np.isnan(g), np.isnan(ref)), (g[np.isnan(g) != np.isnan(ref)], ref[np.isnan(g) != np.isnan(ref)])
+    ok = ~np.isnan(ref)
+    top = 3.3895313892515355e38          # the largest bf16
+    both_huge = ok & (np.abs(g) >= top) & (np.abs(ref) >= top) & (np.sign(g) == np.sign(ref))
+    fin = ok & np.isfinite(ref) & ~both_huge
+    assert np.array_equal(np.isinf(g[ok & ~both_huge]), np.isinf(ref[ok & ~both_huge]))
+    ulp = np.spacing(np.abs(ref[fin]).astype(np.float32)).astype(np.float64) * 2.0 ** 16
+    assert np.all(np.abs(g[fin] - ref[fin]) <= np.maximum(ulp, 2.0 ** -126)), (g[fin][np.abs(g[fin] - ref[fin]) > np.maximum(ulp, 2.0 ** -126)], ref[fin][np.abs(g[fin] - ref[fin]) > np.maximum(ulp, 2.0 ** -126)])
+    assert np.array_equal(np.signbit(g[fin & (ref == 0)]), np.signbit(ref[fin & (ref == 0)]))
+
+
 @pytest.mark.parametrize("dt", ["bf16", "f16"])
 def test_logistic_of_every_narrow_value(rx, client, dt):
     """1 / (1 + e^-x) over every 16-bit pattern (narrow results: hardware 2^y and reciprocal): one ulp of the float64
