@@ -1,4 +1,4 @@
-"""TEST INFRASTRUCTURE (oracle).  Builds the C restatements in this directory (stencil_cpu.c, reduce_cpu.c) with gcc
+"""TEST INFRASTRUCTURE (oracle).  Builds the C restatements in this directory (stencil_cpu.c, reduce_cpu.c, dense_cpu.c) with gcc
 (-O3 -fopenmp -ffp-contract=off, baseline x86-64 so the library runs on any host) into oracle/_build/liboracle_c.so and loads it with ctypes."""
 import ctypes
 import os
@@ -9,7 +9,7 @@ SO = os.path.join(HERE, "_build", "liboracle_c.so")
 
 
 def build(force=False):
-    srcs = [os.path.join(HERE, f) for f in ("stencil_cpu.c", "reduce_cpu.c")]
+    srcs = [os.path.join(HERE, f) for f in ("stencil_cpu.c", "reduce_cpu.c", "dense_cpu.c")]
     if not force and os.path.exists(SO) and all(os.path.getmtime(SO) >= os.path.getmtime(s) for s in srcs):
         return SO
     os.makedirs(os.path.dirname(SO), exist_ok=True)
@@ -30,7 +30,41 @@ def load():
     fp = ctypes.POINTER(ctypes.c_float)
     lib.rx_oracle_sinsum_add.restype = ctypes.c_double
     lib.rx_oracle_sinsum_add.argtypes = [fp, fp, ctypes.c_longlong]
+    ll = ctypes.c_longlong
+    lib.rx_oracle_bias_gelu_bf16.restype = None
+    lib.rx_oracle_bias_gelu_bf16.argtypes = [fp, fp, ll, ll]
+    lib.rx_oracle_softmax_rows_bf16.restype = None
+    lib.rx_oracle_softmax_rows_bf16.argtypes = [fp, ll, ll]
+    lib.rx_oracle_scale_rmsnorm_bf16.restype = None
+    lib.rx_oracle_scale_rmsnorm_bf16.argtypes = [fp, ctypes.c_float, ctypes.c_float, ll, ll]
     return lib
+
+
+def mlp_f32(lib, x, weights, biases, softmax=True):
+    """The dense network of programs.mlp in single precision: x [batch][w0], weights[l] [w_l][w_{l+1}], biases[l] [w_{l+1}],
+    all float32 arrays holding bf16 values.  Each layer is numpy's sgemm, then bias + gelu rounded to bf16 (C, OpenMP);
+    softmax over the last layer's rows.  Returns float32 [batch][w_last]."""
+    import numpy as np
+    fp = ctypes.POINTER(ctypes.c_float)
+    h = np.ascontiguousarray(x, dtype=np.float32)
+    for w, b in zip(weights, biases):
+        h = np.ascontiguousarray(h @ w)
+        b = np.ascontiguousarray(b, dtype=np.float32)
+        lib.rx_oracle_bias_gelu_bf16(h.ctypes.data_as(fp), b.ctypes.data_as(fp), h.shape[0], h.shape[1])
+    if softmax:
+        lib.rx_oracle_softmax_rows_bf16(h.ctypes.data_as(fp), h.shape[0], h.shape[1])
+    return h
+
+
+def fp8_linear_f32(lib, q, w, scale, eps=1e-6):
+    """The product and what follows it in programs.fp8_linear, in single precision: q [batch][k] and w [n][k] are float32
+    arrays holding e4m3 values (products of two such values and their sums over k <= 2^16 terms are formed by sgemm in
+    float32), scale = scale_a * scale_w.  Returns bf16(rmsnorm(bf16(scale * q w^T))) as float32 [batch][n]."""
+    import numpy as np
+    fp = ctypes.POINTER(ctypes.c_float)
+    h = np.ascontiguousarray(q @ w.T)
+    lib.rx_oracle_scale_rmsnorm_bf16(h.ctypes.data_as(fp), ctypes.c_float(float(scale)), ctypes.c_float(float(eps)), h.shape[0], h.shape[1])
+    return h
 
 
 def sinsum_add(lib, x, y):

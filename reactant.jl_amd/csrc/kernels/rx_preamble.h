@@ -199,6 +199,15 @@ RX_DEV float rx_gelu_chain_fast(float x, float k1, float k3) {
 // behave as in the division (1/0 = inf, 0 * inf = NaN, ...); double has the range for
 // subnormal divisors.
 RX_DEV float rx_div_uniform(float x, float y) { return (float)((double)x * (1.0 / (double)y)); }
+// x / y for a result that is rounded to a narrow float, where y does not vary along the minor dimension (the sum of a
+// softmax row): x times the reciprocal of y, a division that is computed once per row.  The reciprocal of a divisor
+// below 2^-128 would overflow although the quotient is finite (1e-20 / 1e-39), so divisors below 2^-64 are scaled by
+// 2^64 first and the product is scaled back: both scalings are exact, the result stays within an ulp of float32 of
+// the quotient, and zero, infinite and NaN operands behave as in the division.
+RX_DEV float rx_div_minor_uniform(float x, float y) {
+  const float s = __builtin_fabsf(y) < 0x1p-64f ? 0x1p64f : 1.0f;
+  return (x * (1.0f / (y * s))) * s;
+}
 RX_DEV float rx_logistic(float x) { return 1.0f / (1.0f + expf(-x)); }
 RX_DEV double rx_logistic(double x) { return 1.0 / (1.0 + exp(-x)); }
 RX_DEV float rx_rsqrt(float x) { return 1.0f / sqrtf(x); }
@@ -424,10 +433,21 @@ RX_DEV T rx_block_reduce(T v, OP op, T* lds /* NWAVES entries */) {
   return r;
 }
 
+// true for every thread of the workgroup if p is true for any of them (w: one word of LDS)
+RX_DEV bool rx_block_any(bool p, int* w) {
+  if (threadIdx.x == 0) *w = 0;
+  __syncthreads();
+  if (p) *w = 1;
+  __syncthreads();
+  const bool r = *w != 0;
+  __syncthreads();
+  return r;
+}
+
 // A workgroup's partial result handed to another workgroup of the same launch without a fence: the value travels in
 // 32-bit pieces, each in the low half of a 64-bit word whose high half is a flag, and each word is written by one
 // relaxed device-scope atomic store -- a reader that sees the flag sees the piece.  Slots are zero before the launch;
-// the reader clears what it has read.  The wait is bounded (about a second): no correct run exhausts it.
+// the reader clears what it has read.  The wait is bounded (2^20 polls of about 1.5 us): no correct run exhausts it.
 // A flag is a nonzero 32-bit epoch: readers that clear what they read use epoch 1 throughout; where a slot has several
 // readers nothing is cleared, and the epoch changes from launch to launch instead.
 template <typename T>
@@ -438,10 +458,11 @@ RX_DEV void rx_publish_partial(unsigned long long* slot, T v, rx_u32 epoch = 1u)
 #pragma unroll
   for (int k = 0; k < NW; ++k) __hip_atomic_store(slot + k, ((unsigned long long)epoch << 32) | w[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// the same wait for a partial that several workgroups read: the slot keeps its value.  `limit` polls (about 1.5 us each);
-// a wait that expires sets the fault word (pinned host memory, checked by the host) and continues with what the slot holds
+// the same wait for a partial that several workgroups read: the slot keeps its value.  `limit` polls (about 1.5 us each:
+// 2^16 polls are about 0.1 s); a wait that expires sets the fault word (pinned host memory, checked by the host) and
+// *bad, and continues with what the slot holds
 template <typename T>
-RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch, int limit, unsigned* fault) {
+RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch, int limit, unsigned* fault, bool* bad) {
   constexpr int NW = (sizeof(T) + 3) / 4;
   rx_u32 w[NW];
 #pragma unroll
@@ -451,7 +472,10 @@ RX_DEV T rx_peek_partial(unsigned long long* slot, rx_u32 epoch, int limit, unsi
       __builtin_amdgcn_s_sleep(2);
       x = __hip_atomic_load(slot + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    if ((rx_u32)(x >> 32) != epoch) __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if ((rx_u32)(x >> 32) != epoch) {
+      __hip_atomic_store(fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      *bad = true;
+    }
     w[k] = (rx_u32)x;
   }
   T v;

@@ -81,7 +81,11 @@ struct RxDevice {
   // its launch expired (its results are then invalid).  Checked wherever the host has waited for the device.
   unsigned* fault_host = nullptr;
   void* fault_dev = nullptr;
+  // set once the fault word has been found set: executables whose kernels wait for other workgroups are then rebuilt
+  // in the form that does not wait, and new ones are compiled in that form
+  std::atomic<bool> waits_failed{false};
   std::mutex scratch_mu;         // held while a call that uses it queues its kernels
+  std::mutex future_mu;          // held while a future of this device creates and records its event
   std::string kind;
   std::string arch;
   // caching allocator: device memory is kept and reused by size class, because hipMalloc and
@@ -194,8 +198,10 @@ static void check_fault(RxDevice* d) {
   volatile unsigned* w = d->fault_host;
   if (*w == 0) return;
   *w = 0;
+  d->waits_failed = true;
   throw Error("INTERNAL: a kernel's bounded wait for another workgroup of its launch expired; results produced since the last "
-              "synchronization are invalid (RX_SINGLE_PASS_SCAN=0 selects the scan that does not wait)");
+              "synchronization are invalid.  Executables of this device that wait between workgroups (the one-launch scan) are "
+              "rebuilt in the form that does not wait when they are next executed, so the call can be repeated");
 }
 
 struct RxExecutable {
@@ -206,6 +212,8 @@ struct RxExecutable {
   std::vector<hipFunction_t> fns;   // per launch
   std::vector<Mem> consts;          // per plan buffer (only Const kinds are set)
   std::string report;
+  std::string text;                 // the module as compiled: a rebuild after a failed wait starts from it
+  bool waits = false;               // some kernel of the plan waits for other workgroups of its launch (has a fault-word argument)
   std::mutex mu;
   // event lists of executions profiled without blocking (RxExecuteProfiled), oldest first
   std::vector<std::vector<hipEvent_t>> pending_events;
@@ -399,6 +407,8 @@ __global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, 
   }
 }
 
+void rebuild_without_waits(RxExecutable* ex);
+
 // Core of XLAExecuteSharded / RxExecuteTimed
 void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uint8_t* donate, int num_results, RxBuffer** results, float* launch_ms,
              RxFuture** futures, bool profile_async = false) {
@@ -406,6 +416,8 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
   if (dev) check_device(dev);
   if (!dev) dev = ex->device;
   if (dev != ex->device) throw Error("INVALID_ARGUMENT: executable was compiled for another device");
+  std::lock_guard<std::mutex> lock(ex->mu);
+  rebuild_without_waits(ex);
   const rx::Plan& P = ex->plan;
   if (num_args != (int)P.param_types.size())
     throw Error("INVALID_ARGUMENT: executable expects " + std::to_string(P.param_types.size()) + " arguments, got " + std::to_string(num_args));
@@ -418,12 +430,33 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " has type " + args[i]->ty.str() + ", executable expects " + P.param_types[i].str());
     if (args[i]->device != dev) throw Error("INVALID_ARGUMENT: argument " + std::to_string(i) + " lives on another device");
   }
-  std::lock_guard<std::mutex> lock(ex->mu);
   HIP_CHECK(hipSetDevice(dev->ordinal));
   const size_t NB = P.buffers.size();
   std::vector<Mem> bufs(NB);
   std::vector<char> is_res(NB, 0);
   for (int b : P.result_buffers) is_res[b] = 1;
+  // A donated argument hands its storage to the plan's buffer now, so that the block goes back to the pool at the
+  // argument's last use inside this execution (the time loop of the stencil donates four fields of half a gigabyte).
+  // If a later step throws, the guard below gives the storage back where it is still alive; where the plan has already
+  // released it, the argument stays consumed.
+  struct Donation {
+    int num_args;
+    RxBuffer** args;
+    uint8_t* donate;
+    const rx::Plan& P;
+    std::vector<Mem>& bufs;
+    bool committed = false;
+    ~Donation() {
+      if (!donate) return;
+      for (size_t b = 0; b < P.buffers.size(); ++b) {
+        const auto& B = P.buffers[b];
+        if (B.kind != rx::BufferDesc::Param || !donate[B.param_index]) continue;
+        RxBuffer* a = args[B.param_index];
+        if (committed || !bufs[b]) { a->donated = true; a->mem.reset(); }
+        else if (!a->mem) a->mem = bufs[b];
+      }
+    }
+  } donation{num_args, args, donate, P, bufs};
   for (size_t b = 0; b < NB; ++b) {
     const auto& B = P.buffers[b];
     if (B.kind == rx::BufferDesc::Param) {
@@ -433,8 +466,9 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
       bufs[b] = ex->consts[b];
     }
   }
-  // Donated arguments give up their storage only once everything that can fail has succeeded (at the
-  // end of this function): an out-of-memory or launch error must leave the caller's arrays intact.
+  if (donate)
+    for (int i = 0; i < num_args; ++i)
+      if (donate[i]) args[i]->mem.reset();   // the plan's buffer holds it from here on
   // events of a timed execution; destroyed on every exit path unless handed to the executable
   struct EventList {
     std::vector<hipEvent_t> v;
@@ -533,12 +567,7 @@ void execute(RxExecutable* ex, int num_args, RxBuffer** args, RxDevice* dev, uin
   if (futures)
     for (int r = 0; r < num_results; ++r) { reg_add(new_futures[r]); futures[r] = new_futures[r]; }
   new_futures.clear();
-  for (int i = 0; i < num_args; ++i) {
-    if (donate && donate[i]) {
-      args[i]->donated = true;
-      args[i]->mem.reset();
-    }
-  }
+  donation.committed = true;   // its destructor marks the donated arguments as consumed
   if (profile_async && !launch_ms) {
     ex->pending_events.push_back(std::move(evs));   // read later by RxExecutableTakeTimings
     evs.clear();
@@ -795,6 +824,67 @@ RX_EXPORT int RxCompileOffline(const char* text, size_t len, int with_source, ch
   }
 }
 
+namespace {
+// Parse, plan and load the module text of an executable: kernels through hiprtc, constants to the device.
+void load_plan(RxExecutable* ex, rx::PlanOptions opt) {
+  RxDevice* d = ex->device;
+  if (d->waits_failed) opt.single_pass_scan = false;   // a wait between workgroups has expired on this device before
+  try {
+    rx::Graph g = rx::parse_module(ex->text.data(), ex->text.size());
+    ex->plan = rx::make_plan(g, opt);
+  } catch (const std::exception& e) {
+    // same shape of message as the reference: module text followed by the status (API.cpp:1499-1505)
+    throw Error(ex->text.substr(0, 4000) + "\n" + e.what());
+  }
+  ex->report = ex->plan.report();
+  ex->waits = false;
+  for (auto& B : ex->plan.buffers) ex->waits = ex->waits || B.kind == rx::BufferDesc::Fault;
+  HIP_CHECK(hipSetDevice(d->ordinal));
+  ex->fns.clear();
+  if (!ex->plan.launches.empty()) {
+    std::string code = rtc_compile(ex->plan.source, d->arch);
+    HIP_CHECK(hipModuleLoadData(&ex->module, code.data()));
+    for (auto& L : ex->plan.launches) {
+      hipFunction_t f;
+      HIP_CHECK(hipModuleGetFunction(&f, ex->module, L.kernel.c_str()));
+      if (L.lds_bytes > 48 * 1024) {
+        // more dynamic LDS than the default limit: gfx950 has 160 KB per workgroup
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(f), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.lds_bytes);
+        if (e != hipSuccess) {
+          (void)hipGetLastError();
+          throw Error("kernel " + L.kernel + " needs " + std::to_string(L.lds_bytes) + " bytes of LDS, which the device refused (" +
+                      hipGetErrorString(e) + ")");
+        }
+      }
+      ex->fns.push_back(f);
+    }
+  }
+  ex->consts.assign(ex->plan.buffers.size(), Mem());
+  for (size_t b = 0; b < ex->plan.buffers.size(); ++b) {
+    auto& B = ex->plan.buffers[b];
+    if (B.kind != rx::BufferDesc::Const) continue;
+    ex->consts[b] = std::make_shared<Allocation>(d, std::max<size_t>(B.data.size(), 1));
+    // on the device's stream: the block may have been recycled from a buffer whose last kernel
+    // is still queued there, and a copy on the null stream would not wait for it
+    if (!B.data.empty()) HIP_CHECK(hipMemcpyAsync(ex->consts[b]->ptr, B.data.data(), B.data.size(), hipMemcpyHostToDevice, d->stream));
+  }
+  HIP_CHECK(hipStreamSynchronize(d->stream));   // pageable host data: wait before the plan may move
+}
+
+// After a wait between workgroups has expired on the device (check_fault), an executable whose kernels wait is rebuilt
+// from its module text in the form that does not wait (two launches per scan).  Called with ex->mu held.
+void rebuild_without_waits(RxExecutable* ex) {
+  if (!ex->waits || !ex->device->waits_failed) return;
+  HIP_CHECK(hipSetDevice(ex->device->ordinal));
+  HIP_CHECK(hipStreamSynchronize(ex->device->stream));   // kernels of the old module may still be queued
+  if (ex->module) { (void)hipModuleUnload(ex->module); ex->module = nullptr; }
+  for (auto& evs : ex->pending_events)   // timings of the old plan's launches
+    for (auto& e : evs) (void)hipEventDestroy(e);
+  ex->pending_events.clear();
+  load_plan(ex, plan_options());
+}
+}  // namespace
+
 RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, size_t len, const char* opts, size_t nopts) {
   (void)opts;
   (void)nopts;
@@ -805,44 +895,8 @@ RX_EXPORT RxExecutable* ClientCompileFromText(RxClient* c, const char* text, siz
     std::unique_ptr<RxExecutable> ex(new RxExecutable);
     ex->client = c;
     ex->device = d;
-    try {
-      rx::Graph g = rx::parse_module(text, len);
-      ex->plan = rx::make_plan(g, plan_options());
-    } catch (const std::exception& e) {
-      // same shape of message as the reference: module text followed by the status (API.cpp:1499-1505)
-      std::string mod(text, std::min<size_t>(len, 4000));
-      throw Error(mod + "\n" + e.what());
-    }
-    ex->report = ex->plan.report();
-    HIP_CHECK(hipSetDevice(d->ordinal));
-    if (!ex->plan.launches.empty()) {
-      std::string code = rtc_compile(ex->plan.source, d->arch);
-      HIP_CHECK(hipModuleLoadData(&ex->module, code.data()));
-      for (auto& L : ex->plan.launches) {
-        hipFunction_t f;
-        HIP_CHECK(hipModuleGetFunction(&f, ex->module, L.kernel.c_str()));
-        if (L.lds_bytes > 48 * 1024) {
-          // more dynamic LDS than the default limit: gfx950 has 160 KB per workgroup
-          hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(f), hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.lds_bytes);
-          if (e != hipSuccess) {
-            (void)hipGetLastError();
-            throw Error("kernel " + L.kernel + " needs " + std::to_string(L.lds_bytes) + " bytes of LDS, which the device refused (" +
-                        hipGetErrorString(e) + ")");
-          }
-        }
-        ex->fns.push_back(f);
-      }
-    }
-    ex->consts.resize(ex->plan.buffers.size());
-    for (size_t b = 0; b < ex->plan.buffers.size(); ++b) {
-      auto& B = ex->plan.buffers[b];
-      if (B.kind != rx::BufferDesc::Const) continue;
-      ex->consts[b] = std::make_shared<Allocation>(d, std::max<size_t>(B.data.size(), 1));
-      // on the device's stream: the block may have been recycled from a buffer whose last kernel
-      // is still queued there, and a copy on the null stream would not wait for it
-      if (!B.data.empty()) HIP_CHECK(hipMemcpyAsync(ex->consts[b]->ptr, B.data.data(), B.data.size(), hipMemcpyHostToDevice, d->stream));
-    }
-    HIP_CHECK(hipStreamSynchronize(d->stream));   // pageable host data: wait before the plan may move
+    ex->text.assign(text, len);
+    load_plan(ex.get(), plan_options());
     RxExecutable* raw = ex.release();
     reg_add(raw);
     return raw;
@@ -926,6 +980,10 @@ RX_EXPORT int RxExecuteNoAlloc(RxExecutable* ex, int num_args, RxBuffer** args, 
   return guarded([&]() -> int {
     check_exec(ex);
     RxDevice* dev = ex->device;
+    std::lock_guard<std::mutex> lock(ex->mu);
+    if (ex->waits && dev->waits_failed)
+      throw Error("FAILED_PRECONDITION: a wait between workgroups expired on this device earlier; this executable has to be rebuilt in the form "
+                  "that does not wait, which allocates: execute it once through XLAExecuteSharded");
     const rx::Plan& P = ex->plan;
     if (num_args != (int)P.param_types.size())
       throw Error("INVALID_ARGUMENT: executable expects " + std::to_string(P.param_types.size()) + " arguments, got " + std::to_string(num_args));
@@ -972,7 +1030,6 @@ RX_EXPORT int RxExecuteNoAlloc(RxExecutable* ex, int num_args, RxBuffer** args, 
     if (used > RX_NOALLOC_SCRATCH_BYTES)
       throw Error("RESOURCE_EXHAUSTED: the temporaries of this executable take " + std::to_string(used) + " bytes; RxExecuteNoAlloc holds at most " +
                   std::to_string(RX_NOALLOC_SCRATCH_BYTES) + " (use XLAExecuteSharded)");
-    std::lock_guard<std::mutex> lock(ex->mu);
     std::lock_guard<std::mutex> slock(dev->scratch_mu);
     HIP_CHECK(hipSetDevice(dev->ordinal));
     std::vector<void*> ptrs, argv;
@@ -1011,6 +1068,7 @@ RX_EXPORT void FreeFuture(RxFuture* f) {
 }
 // The event of a future, recorded on its device's stream the first time the future is asked about.
 static void future_event(RxFuture* f) {
+  std::lock_guard<std::mutex> l(f->device->future_mu);   // two threads may ask the same future at once
   if (f->ev || f->done) return;
   if (!f->device->client || !f->device->client->alive.load()) { f->done = true; return; }   // FreeClient drained the stream
   HIP_CHECK(hipSetDevice(f->device->ordinal));

@@ -459,8 +459,9 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
           // double rounds to the same float as the division (see rx_div_uniform)
           // a result that is rounded to a narrow float, divided by a value that is the same along the minor dimension
           // (the sum of a softmax row, a quantization scale): its reciprocal, a division of its own that the compiler
-          // computes once per row, times the dividend -- within an ulp of float32 of the quotient
-          if (CT == "float" && is_narrow_float(dt) && excess_precision && n.ty.rank() > 0 && minor_uniform(n.in[1])) return def("(" + a + " * (1.0f / " + b + "))");
+          // computes once per row, times the dividend -- within an ulp of float32 of the quotient (rx_div_minor_uniform, which
+          // also covers subnormal divisors whose reciprocal would overflow)
+          if (CT == "float" && is_narrow_float(dt) && excess_precision && n.ty.rank() > 0 && minor_uniform(n.in[1])) return def("rx_div_minor_uniform(" + a + ", " + b + ")");
           if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
           return def("(" + a + " / " + b + ")");
         }

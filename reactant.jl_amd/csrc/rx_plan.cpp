@@ -3168,9 +3168,9 @@ struct Planner {
       // group needs at once, a chunk waited 5.4 us on average, with this window 3.7 (2^26 f32, time stamps inside
       // the kernel).  Every workgroup waits only for lower-numbered ones, which the dispatcher
       // started no later (workgroups start in index order on each die: an assumption about the dispatcher).  Waits are
-      // bounded: one that expires sets the device's fault word, and the next call that waits for the device raises an
-      // error instead of handing out the result; RX_SINGLE_PASS_SCAN=0 selects the two-launch form, which never
-      // waits.  Nothing is cleared between runs: a flag is the row's epoch, a word that
+      // bounded: one that expires sets the device's fault word, the next call that waits for the device raises an
+      // error instead of handing out the result, and from then on the host rebuilds every executable with such a kernel
+      // in the two-launch form (also what RX_SINGLE_PASS_SCAN=0 selects), which never waits.  Nothing is cleared between runs: a flag is the row's epoch, a word that
       // the row's last chunk advances once its carry is complete -- by then every chunk of the row has published, so
       // has read the epoch (one counter of finished workgroups would cost 60 ns each: atomics on one address from
       // eight dies).  The data is read once and written once.
@@ -3193,7 +3193,8 @@ struct Planner {
           const int spin_limit = getenv("RX_SCAN_SPIN_LIMIT") ? std::max(0, atoi(getenv("RX_SCAN_SPIN_LIMIT"))) : (1 << 16);
           o << "// scan along the minor dimension of " << ty.str() << " (" << sNC << " chunks per row, one launch): " << describe(rn.in[0]) << "\n";
           o << sg << " {\n";
-          o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n  __shared__ " << ACC << " wsum[" << T * (kBlock / 64) << "];\n";
+          o << "  __shared__ " << ACC << " lds[" << kBlock / 64 << "];\n  __shared__ " << ACC << " wsum[" << T * (kBlock / 64) << "];\n  __shared__ int anyw;\n";
+          o << "  bool bad = false;   // a wait of this thread expired\n";
           o << "  const " << it << " c = (" << it << ")(blockIdx.x % " << sNC << "u), row = (" << it << ")(blockIdx.x / " << sNC << "u);\n";
           decompose(o, "row", 0, a);
           for (int d = a + 1; d < ty.rank(); ++d) o << "  const " << it << " q" << d << " = 0;\n";
@@ -3258,9 +3259,11 @@ struct Planner {
           o << "    run = " << red_apply(rn.red, dt, "run", "total") << ";\n  }\n";
           // the last chunk of a group also publishes the group's total
           o << "  if (c % " << GS << " == " << GS - 1 << ") {\n";
-          o << "    " << ACC << " part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + (" + it + ")threadIdx.x)") << ", epoch, " << spin_limit << ", fault);\n";
+          o << "    " << ACC << " part = rx_peek_partial<" << ACC << ">(" << slot_of("(c - " + std::to_string(GS - 1) + " + (" + it + ")threadIdx.x)") << ", epoch, " << spin_limit << ", fault, &bad);\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
-          o << "    if (threadIdx.x == 0) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS)) << ", part, epoch);\n";
+          // a group total built from a slot that never arrived is not published: the chunks that need it expire in turn
+          o << "    const bool gbad = rx_block_any(bad, &anyw);\n";
+          o << "    if (threadIdx.x == 0 && !gbad) rx_publish_partial<" << ACC << ">(" << slot_of(std::to_string(sNC) + " + c / " + std::to_string(GS)) << ", part, epoch);\n";
           o << "  }\n";
           // carry
           o << "  " << ACC << " carry = (" << ACC << ")" << initv << ";\n";
@@ -3268,11 +3271,14 @@ struct Planner {
           o << "    " << ACC << " part = " << IDENT << ";\n";
           o << "    for (" << it << " k = threadIdx.x; k < ngr + (c - c0); k += " << kBlock << ") {\n";
           o << "      const " << it << " idx = k < ngr ? " << sNC << " + k : c0 + (k - ngr);\n";
-          o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch, " + std::to_string(spin_limit) + ", fault)") << ";\n    }\n";
+          o << "      part = " << red_apply(rn.red, dt, "part", "rx_peek_partial<" + ACC + ">(" + slot_of("idx") + ", epoch, " + std::to_string(spin_limit) + ", fault, &bad)") << ";\n    }\n";
           o << "    part = rx_block_reduce<" << ACC << ", decltype(" << OP << "), " << kBlock / 64 << ">(part, " << OP << ", lds);\n";
           o << "    if (c != 0) carry = " << red_apply(rn.red, dt, "carry", "part") << ";\n  }\n";
-          // the row's last chunk has, through its carry, heard from every chunk of the row: the next run's epoch
-          o << "  if (c == " << sNC - 1 << " && threadIdx.x == 0) slots[" << outer * SL * NW << " + row] = (unsigned long long)(epoch == 0xffffffffu ? 0u : epoch);\n";
+          // the row's last chunk has, through its carry, heard from every chunk of the row: the next run's epoch.  Not
+          // when one of its waits expired: a chunk that has not started yet would read the new epoch and publish under it
+          // (the host rebuilds the executable without waits before it runs again, so the stale flags are never read)
+          o << "  if (c == " << sNC - 1 << ") {\n    const bool rbad = rx_block_any(bad, &anyw);\n";
+          o << "    if (threadIdx.x == 0 && !rbad) slots[" << outer * SL * NW << " + row] = (unsigned long long)(epoch == 0xffffffffu ? 0u : epoch);\n  }\n";
           // results
           o << "#pragma unroll\n  for (int t = 0; t < " << T << "; ++t) {\n";
           o << "    const " << it << " pb = c * " << sCH << " + t * " << TILE << " + (" << it << ")threadIdx.x * " << V << ";\n";

@@ -135,6 +135,34 @@ def test_fp8_linear_8192_rows_sampled(rx, client):
     assert float(np.max(np.max(np.abs(g64 - r64), axis=1) / np.max(np.abs(r64), axis=1))) <= 1e-2
 
 
+def test_fp8_dot_8192_componentwise(rx, client):
+    """The 8192-long e4m3 contraction of the FP8 layer on its own at full size (both operands [rows][k], f32 result, no
+    scale, no norm), on sampled rows: |got - ref|_ij <= 1e-2 (|A8| . |W8|)_ij with the reference accumulated in float64.
+    Products of two e4m3 values are exact in float32, so what this bounds is the f32 accumulation over 8192 terms in the
+    order the kernel takes them, and a dropped K tile or a wrong fragment shows as an entry of its own."""
+    n, rows = 8192, 48
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, size=(n, n), dtype=np.uint8)
+    w = rng.integers(0, 256, size=(n, n), dtype=np.uint8)
+    for c in (a, w):
+        c[(c & 0x7F) == 0x7F] = 0x38                                       # no NaN codes
+    ta, to = "tensor<%dx%dxf8E4M3FN>" % (n, n), "tensor<%dx%dxf32>" % (n, n)
+    text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
+            "    %%0 = stablehlo.dot_general %%arg0, %%arg1, contracting_dims = [1] x [1], precision = [DEFAULT, DEFAULT] : (%s, %s) -> %s\n"
+            "    return %%0 : %s\n  }\n}\n" % (ta, ta, to, ta, ta, to, to))
+    exe = rx.xla_compile(client, text)
+    assert [l["kind"] for l in exe.launches()] == ["gemm_f8"], exe.report()
+    out = exe.execute_sharded([_upload(rx, client, a, "f8E4M3FN"), _upload(rx, client, w, "f8E4M3FN")])
+    got = _download(out[0]).reshape(n, n)
+    pick = np.concatenate([np.arange(4), np.linspace(4, n - 5, rows - 8).astype(int), np.arange(n - 4, n)])
+    af = lf.e4m3fn_bits_to_f32(a[pick]).astype(np.float64)
+    wf = lf.e4m3fn_bits_to_f32(w).astype(np.float64)
+    ref, bound = af @ wf.T, np.abs(af) @ np.abs(wf).T
+    assert contraction_err(got[pick], ref, bound) <= 1e-2
+    # and far inside it: float32 accumulation of exact products
+    assert contraction_err(got[pick], ref, bound) <= 1e-4
+
+
 def test_tensors_of_more_than_2_31_elements(rx, client):
     """Index arithmetic switches to 64 bits when a tensor has 2^31 elements or more: an elementwise
     map with a shifted slice and a pad, a full reduction, a row and a column reduction, bit for bit

@@ -405,15 +405,15 @@ def test_division_by_a_row_value_special_cases(rx, client):
     subnormal against dividends of every kind.  Finite quotients within an ulp of the exact one (or both zero / both
     beyond the largest bf16), infinities and NaNs where IEEE division has them."""
     big, tiny = 3.0e38, 1.2e-38
-    divisors = np.array([1.0, -3.0, 0.0, -0.0, np.inf, -np.inf, np.nan, big, -big, tiny, 4.0e-39, 1.0e-30, 7.0e20, 0.333], dtype=np.float64)
-    dividends = np.array([0.0, -0.0, 1.0, -1.0, 2.5, np.inf, -np.inf, np.nan, big, -big, tiny, 1.0e-20, 6.0e15, 0.1, 100.0, -7.0], dtype=np.float64)
+    divisors = np.array([1.0, -3.0, 0.0, -0.0, np.inf, -np.inf, np.nan, big, -big, tiny, 4.0e-39, 2.0e-39, 1.0e-39, 1.0e-40, 9.2e-41, -9.2e-41, 1.0e-30, 5.0e-20, 7.0e20, 0.333], dtype=np.float64)
+    dividends = np.array([0.0, -0.0, 1.0, -1.0, 2.5, np.inf, -np.inf, np.nan, big, -big, tiny, 1.0e-20, 6.0e15, 0.1, 100.0, -7.0, 1.0e-35, 9.2e-41, 3.0e-39], dtype=np.float64)
     rows, cols = len(divisors), 64
     x = np.tile(np.resize(dividends, cols), (rows, 1))
     ty, tr = P._tt([rows, cols], "bf16"), P._tt([rows], "bf16")
     text = ("module {\n  func.func @main(%%arg0: %s, %%arg1: %s) -> %s {\n"
             "    %%0 = stablehlo.broadcast_in_dim %%arg1, dims = [0] : (%s) -> %s\n"
             "    %%1 = stablehlo.divide %%arg0, %%0 : %s\n    return %%1 : %s\n  }\n}\n" % (ty, tr, ty, tr, ty, ty, ty))
-    assert "(1.0f / " in rx.compile_offline(text, with_source=True)
+    assert "rx_div_minor_uniform(" in rx.compile_offline(text, with_source=True)
     a, b = I.tensor(x, "bf16"), I.tensor(divisors, "bf16")
     got, _ = gpu_run(rx, client, text, [a, b])
     g = got[0].a.astype(np.float64)
@@ -474,7 +474,7 @@ def test_softmax_rows_with_extreme_sums(rx, client, dt):
             "    %%3 = stablehlo.divide %%0, %%2 : %s\n    return %%3 : %s\n  }\n}\n" % (ty, ty, dt, ty, ty, dt, tr, tr, ty, ty, ty))
     a = I.tensor(x, dt)
     got, exe = gpu_run(rx, client, text, [a])
-    assert "(1.0f / " in rx.compile_offline(text, with_source=True)
+    assert "rx_div_minor_uniform(" in rx.compile_offline(text, with_source=True)
     xv = a.a.astype(np.float64)
     e = np.exp(xv)
     exact = e / e.sum(axis=1, keepdims=True)

@@ -148,17 +148,28 @@ def test_prefix_scans_of_long_rows_in_one_launch(rx, client, monkeypatch, shape,
 def test_a_wait_that_expires_is_reported(rx, client, monkeypatch):
     """A workgroup of the one-launch scan waits, for a bounded number of polls, for totals that lower-numbered workgroups
     publish.  With the bound forced to zero polls from the host some wait expires (every kernel still runs to its end): the
-    kernel sets the device's fault word and the next call that waits for the device raises instead of returning the result."""
+    kernel sets the device's fault word and the next call that waits for the device raises instead of returning the result.
+    The same executable is then rebuilt in the two-launch form on its next execution and gives the right answer, as does
+    every executable compiled through that client afterwards (a client of its own: the switch is per client)."""
+    client = rx.Client()
     text = NN.cumulative([1 << 24], "f32", 0, "add", False)
     args = _args([[1 << 24]], "f32", seed=3)
+    ref = np.cumsum(args[0].a.astype(np.float64))
     monkeypatch.setenv("RX_SCAN_SPIN_LIMIT", "0")
     exe = rx.xla_compile(client, text)
+    assert [l["kind"] for l in exe.launches()] == ["scan"]
     with pytest.raises(rx.ReactantInternalError, match="bounded wait for another workgroup"):
         for _ in range(3):       # a run in which every slot happens to be there in time is possible, three in a row are not
             gpu_run(rx, client, text, args, exe=exe)
+    # the same executable again, the zero bound still set: it no longer waits
+    for _ in range(2):
+        got, _ = gpu_run(rx, client, text, args, exe=exe)
+        _close(got[0].a, ref, 1e-5 * np.sqrt(1 << 24))
+    assert [l["kind"] for l in exe.launches()] == ["scan_totals", "scan"]
     monkeypatch.delenv("RX_SCAN_SPIN_LIMIT")
-    got, _ = gpu_run(rx, client, text, args)          # the device is usable afterwards and the word was cleared
-    _close(got[0].a, np.cumsum(args[0].a.astype(np.float64)), 1e-5 * np.sqrt(1 << 24))
+    got, exe2 = gpu_run(rx, client, text, args)          # the device is usable afterwards and the word was cleared
+    assert [l["kind"] for l in exe2.launches()] == ["scan_totals", "scan"]
+    _close(got[0].a, ref, 1e-5 * np.sqrt(1 << 24))
 
 
 def test_scan_of_a_fused_producer_and_into_a_consumer(rx, client):

@@ -393,6 +393,73 @@ def test_c_restatement_of_sinsum_add_is_pinned():
     assert abs(build_c.sinsum_add(lib, x, y) - ref) <= 1e-6 * mag
 
 
+def _c_oracle():
+    from oracle import build_c
+    srcs = [os.path.join(os.path.dirname(build_c.SO), "..", f) for f in ("stencil_cpu.c", "reduce_cpu.c", "dense_cpu.c")]
+    if not os.path.exists(build_c.SO) or any(os.path.getmtime(build_c.SO) < os.path.getmtime(f) for f in srcs):
+        build_c.build(force=True)
+    return build_c, build_c.load()
+
+
+def test_c_restatement_of_the_dense_layers_is_pinned():
+    """oracle/dense_cpu.c (bias + gelu, softmax, dequantizing scale + RMSNorm: the elementwise parts of the CPU baselines
+    of the two dense programs).  Closed forms that a wrong constant, a dropped term or a swapped operand would miss --
+    gelu(0) = 0, gelu(x) - gelu(-x) = x, gelu(large) = x, a softmax row sums to one and keeps the order of its inputs, a
+    constant row gives 1/n, RMSNorm output has unit mean square and the input's signs, and both are invariant under what
+    they should be (softmax under a shift, RMSNorm under a positive factor) -- and the numpy interpreter's evaluation of
+    the same modules on seeded bf16 / e4m3 data (float64 accumulation, rounding where the module stores)."""
+    build_c, lib = _c_oracle()
+    bf = lambda a: lf.bf16_bits_to_f32(lf.f32_to_bf16_bits(np.asarray(a, dtype=np.float32)))
+    ones = np.eye(8, dtype=np.float32)
+    # one layer with identity weights: bias + gelu alone
+    x = bf(np.array([[0.0, 1.0, -1.0, 3.0, -3.0, 20.0, -20.0, 0.5]], dtype=np.float32))
+    g = build_c.mlp_f32(lib, x, [ones], [np.zeros(8, np.float32)], softmax=False)[0]
+    assert g[0] == 0.0 and g[5] == 20.0 and abs(g[6]) == 0.0
+    assert abs((g[1] - g[2]) - 1.0) <= 2.0 ** -7 and abs((g[3] - g[4]) - 3.0) <= 2.0 ** -6      # gelu(x) - gelu(-x) = x
+    assert abs(g[1] - 0.8411919906082768) <= 2.0 ** -8 and abs(g[7] - 0.34571400982514394) <= 2.0 ** -9   # tanh form, float64 values
+    gb = build_c.mlp_f32(lib, np.zeros((1, 8), np.float32), [ones], [x[0].copy()], softmax=False)[0]
+    assert np.array_equal(gb, g)                                                               # the bias enters like the product
+    # softmax
+    fp = __import__("ctypes").POINTER(__import__("ctypes").c_float)
+    r = np.array([[1.0, 2.0, 3.0, 4.0], [7.0, 7.0, 7.0, 7.0], [101.0, 102.0, 103.0, 104.0]], dtype=np.float32)
+    lib.rx_oracle_softmax_rows_bf16(r.ctypes.data_as(fp), 3, 4)
+    assert np.all(np.abs(r.sum(axis=1) - 1.0) <= 2.0 ** -7) and np.all(np.diff(r[0]) > 0)
+    assert np.array_equal(r[1], np.full(4, 0.25, np.float32)) and np.array_equal(r[0], r[2])    # shift invariance
+    assert abs(r[0][3] - 0.6439142598879724) <= 2.0 ** -9
+    # RMSNorm
+    v = np.array([[3.0, -4.0, 0.0, 0.0], [30.0, -40.0, 0.0, 0.0]], dtype=np.float32)
+    lib.rx_oracle_scale_rmsnorm_bf16(v.ctypes.data_as(fp), 1.0, 0.0, 2, 4)
+    assert np.array_equal(v[0], v[1]) and abs(v[0][0] - 1.2) <= 2.0 ** -8 and abs(v[0][1] + 1.6) <= 2.0 ** -8
+    v2 = np.array([[3.0, -4.0, 0.0, 0.0]], dtype=np.float32)
+    lib.rx_oracle_scale_rmsnorm_bf16(v2.ctypes.data_as(fp), 2.0, 0.0, 1, 4)
+    assert np.array_equal(v2[0], v[0])                                                          # the scale cancels in the norm
+    # against the interpreter: the whole dense network and the FP8 layer on seeded data
+    batch, widths = 24, (32, 64, 48, 40)
+    rng = np.random.default_rng(0)
+    raw = [lf.f32_to_bf16_bits(rng.normal(size=(batch, widths[0])).astype(np.float32))]
+    for l in range(3):
+        lim = np.sqrt(6.0 / (widths[l] + widths[l + 1]))
+        raw.append(lf.f32_to_bf16_bits(rng.uniform(-lim, lim, size=(widths[l], widths[l + 1])).astype(np.float32)))
+        raw.append(lf.f32_to_bf16_bits((rng.normal(size=(widths[l + 1],)) * 0.1).astype(np.float32)))
+    args = [I.Tensor.from_bytes(a.tobytes(), "bf16", a.shape) for a in raw]
+    ref = run(P.mlp(batch, widths), args, hifi=True, excess=True)[0].a.astype(np.float64)
+    f32 = [lf.bf16_bits_to_f32(a) for a in raw]
+    got = build_c.mlp_f32(lib, f32[0], f32[1::2], f32[2::2])
+    assert np.max(np.abs(got - ref)) <= 2e-2 * np.max(np.abs(ref))
+    n, k = 40, 64
+    act = lf.f32_to_bf16_bits(rng.normal(size=(batch, k)).astype(np.float32))
+    codes = rng.integers(0, 256, size=(n, k), dtype=np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x38
+    sw = np.float32(0.0123)
+    ref = run(P.fp8_linear(batch, k, n), [I.Tensor.from_bytes(act.tobytes(), "bf16", (batch, k)), I.Tensor.from_bytes(codes.tobytes(), "f8E4M3FN", (n, k)),
+                                          I.Tensor(sw, "f32")], hifi=True, excess=True)[0].a.astype(np.float64)
+    a32 = lf.bf16_bits_to_f32(act)
+    sa = np.float32(np.abs(a32).max()) / np.float32(448.0)
+    q = lf.e4m3fn_bits_to_f32(lf.f32_to_e4m3fn_bits(np.clip(a32 / sa, -448.0, 448.0).astype(np.float32)))
+    got = build_c.fp8_linear_f32(lib, q, lf.e4m3fn_bits_to_f32(codes), sa * sw)
+    assert np.max(np.abs(got - ref)) <= 1e-2 * np.max(np.abs(ref))
+
+
 def test_conditionals_against_plain_python():
     x = np.arange(8, dtype=np.float32) / 4
     for s in (2.0, -3.0):
