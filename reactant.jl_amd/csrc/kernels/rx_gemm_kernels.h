@@ -731,8 +731,8 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
 // Operand tiles go global -> LDS as buffer loads: the per-thread part of an address is one 32-bit offset that never
 // changes (two where the swizzle alternates between loads), the K tile and the row block of load i go into the scalar
 // offset, and rows past the end of the operand are outside the buffer's range and read as zero: no address
-// arithmetic and no clamping in the main loop.  Two LDS stages per operand, A stages first so that one address
-// register per operand reaches both of its stages.
+// arithmetic and no clamping in the main loop.  Two LDS stages per operand (three for the 256 x 128 tiles, where they
+// fit), A stages first so that one address register per operand reaches all of its stages.
 // Measured against the skeleton above on the same devices: 8192^3 e4m3 484-491 us against 538-560; bf16
 // 8192 x 4096 x 4096 with bias + GELU 235-238 us against 245-257 ([m][k] x [k][n]; no difference for [m][k] x [n][k]),
 // K = 1024: 74 against 77; 256 x 128 tiles of 8192 x 1024 x 4096: 65 against 66.5.  128 x 128 tiles on four wavefronts
@@ -868,23 +868,25 @@ struct rx_dma_s {
   }
 };
 
-template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2>
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2>
 RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NBUF = 4;
   constexpr int NT = WM * WN * 64;
   constexpr int NA = BM / WM / 16, NB = BN / WN / 16;
   static_assert(NA % NBUF == 0 && D >= 1 && D < NBUF && D <= NA, "streaming depth");
+  static_assert(NSTG == 2 || NSTG == 3, "LDS stages per operand");
   constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BKB : BM * ESZ;   // LDS tiles: rows x bytes
   constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BKB : BN * ESZ;
   constexpr int A_SZ = BM * BKB, B_SZ = BN * BKB;
   typedef rx_dma_s<EL, A_ROWS, A_COLS, NT, A_KC> DMA_A;
   typedef rx_dma_s<EL, B_ROWS, B_COLS, NT, B_KC> DMA_B;
+  constexpr int NLT = DMA_A::NL + DMA_B::NL;   // direct loads per thread and K tile
   static_assert((long long)M * K * ESZ < (1ll << 32) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
   static_assert(K % BK == 0, "whole K tiles");
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
   RX_LDS rx_u8* const ldsa = (RX_LDS rx_u8*)rx_smem;
-  RX_LDS rx_u8* const ldsb = ldsa + 2 * A_SZ;
+  RX_LDS rx_u8* const ldsb = ldsa + NSTG * A_SZ;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
@@ -907,9 +909,9 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
   DMA_B dma_b;
   dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * K * ESZ), tid);
   dma_b.init(B + batch * (long long)N * K, B_GLDB, B_KC ? n0 : n0 * ESZ, (unsigned)((long long)N * K * ESZ), tid);
-  // tile kt lies in stage kt % 2 of both operands
-  auto issue = [&](int kt, auto ST) {
-    constexpr int st = decltype(ST)::value;
+  // tile kt lies in stage kt % NSTG of both operands
+  // (st is a constant at every call, so the stage's offset folds into the instruction)
+  auto issue = [&](int kt, int st) __attribute__((always_inline)) {
     dma_a.issue((unsigned)kt * KA, ldsa + st * A_SZ, wave);
     dma_b.issue((unsigned)kt * KB, ldsb + st * B_SZ, wave);
   };
@@ -920,11 +922,12 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
     if constexpr (A_KC) fa[decltype(BUF)::value] = rx_frag_s<EL>::template kc<A_COLS>(st, o, lane);
     else fa[decltype(BUF)::value] = rx_frag_s<EL>::template tr<A_COLS>(st, o, lane);
   };
-  auto read_b = [&](auto J, auto ST) {
-    constexpr int j = decltype(J)::value, st = decltype(ST)::value;
+  // the B fragments of tile kt live in register set kt % 2
+  auto read_b = [&](auto J, auto PAR, auto ST) {
+    constexpr int j = decltype(J)::value, par = decltype(PAR)::value, st = decltype(ST)::value;
     const int o = wn * (BN / WN) + 16 * j;
-    if constexpr (B_KC) fb[st][j] = rx_frag_s<EL>::template kc<B_COLS>(ldsb + st * B_SZ, o, lane);
-    else fb[st][j] = rx_frag_s<EL>::template tr<B_COLS>(ldsb + st * B_SZ, o, lane);
+    if constexpr (B_KC) fb[par][j] = rx_frag_s<EL>::template kc<B_COLS>(ldsb + st * B_SZ, o, lane);
+    else fb[par][j] = rx_frag_s<EL>::template tr<B_COLS>(ldsb + st * B_SZ, o, lane);
   };
   auto publish = [&]() {
     asm volatile("" ::: "memory");   // compiler-only fences: LDS reads must not move across the barrier
@@ -932,40 +935,42 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
     asm volatile("" ::: "memory");
   };
 
-  issue(0, rx_int<0>{});
-  if (KT > 1) issue(1, rx_int<1>{});
-  if (KT > 1) rx_wait_vmcnt<DMA_A::NL + DMA_B::NL>(); else rx_wait_vmcnt<0>();
+  rx_static_for<0, NSTG>([&](auto S) { if constexpr (decltype(S)::value < KT) issue(decltype(S)::value, decltype(S)::value); });
+  if constexpr (KT >= NSTG) rx_wait_vmcnt<(NSTG - 1) * NLT>(); else rx_wait_vmcnt<0>();
   publish();
-  rx_static_for<0, NB>([&](auto J) { read_b(J, rx_int<0>{}); });
+  rx_static_for<0, NB>([&](auto J) { read_b(J, rx_int<0>{}, rx_int<0>{}); });
   rx_static_for<0, D>([&](auto I) { read_a(I, rx_int<0>{}, decltype(I)::value); });
 
   // The barrier that publishes tile kt+1 sits before the first read of it, D blocks before the end of tile kt: by
-  // then every wavefront has issued its last reads of tile kt, so the stages of tile kt take tile kt+2.  The B
-  // fragments of tile kt+1 are read with its first D blocks of A, BPB of them per block.
+  // then every wavefront has issued its last reads of tile kt, so the stages of tile kt take tile kt+NSTG.  The B
+  // fragments of tile kt+1 are read with its first D blocks of A, BPB of them per block.  With three stages a request
+  // has two K tiles to land instead of one (tiles of 256 x 128, whose K tile is half as long as that of 256 x 256:
+  // the wait for the requests of the 8192 x 1024 x 4096 bf16 layer 9.4 -> 0.5 us per workgroup, 62.3 -> 59.9 us).
   constexpr int BPB = (NB + D - 1) / D;
   constexpr int RDS_A = A_KC ? 2 : 4, RDS_B = B_KC ? 2 : 4;   // LDS read instructions per fragment
   constexpr int NMB = NB * EL::NMF;                           // MFMAs per block of A
-  // MODE 0: tile kt+2 exists, 1: it may not, 2: last tile
-  auto tile = [&](auto P, auto MODE, int kt) {
+  // MODE 0: tile kt+NSTG exists, 1: it does not but tile kt+1 does, 2: last tile
+  auto tile = [&](auto P, auto ST, auto MODE, int kt) {
     constexpr int p = decltype(P)::value, mode = decltype(MODE)::value;
     constexpr bool last = mode == 2;
-    const rx_int<p> cur{};
-    const rx_int<p ^ 1> nxt{};
+    typedef decltype(ST) CUR;                                   // stage of this tile
+    typedef rx_int<(decltype(ST)::value + 1) % NSTG> NXT;       // stage of the next one
     rx_static_for<0, NA>([&](auto I) {
       constexpr int i = decltype(I)::value;
       constexpr int t = i + D;                   // block whose read goes out now
       constexpr int nb0 = t >= NA ? (t - NA) * BPB : 0;
       constexpr int nb1 = t >= NA ? (nb0 + BPB < NB ? nb0 + BPB : NB) : 0;
       if constexpr (t < NA) {
-        read_a(rx_int<t % NBUF>{}, cur, t);
+        read_a(rx_int<t % NBUF>{}, CUR{}, t);
       } else if constexpr (!last) {
         if constexpr (t == NA) {
-          rx_wait_vmcnt<0>();
+          // tile kt+1 has landed once only the NSTG-2 tiles after it are still in flight
+          if constexpr (mode == 0) rx_wait_vmcnt<(NSTG - 2) * NLT>(); else rx_wait_vmcnt<0>();
           publish();
-          if (mode == 0 || kt + 2 < KT) issue(kt + 2, cur);
+          if constexpr (mode == 0) issue(kt + NSTG, CUR::value);
         }
-        read_a(rx_int<t % NBUF>{}, nxt, t - NA);
-        rx_static_for<nb0, nb1>([&](auto J) { read_b(J, nxt); });
+        read_a(rx_int<t % NBUF>{}, NXT{}, t - NA);
+        rx_static_for<nb0, nb1>([&](auto J) { read_b(J, rx_int<p ^ 1>{}, NXT{}); });
       }
       // the B fragment is the row operand: a lane ends with four consecutive n of one m
       rx_static_for<0, NB>([&](auto J) {
@@ -994,21 +999,19 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
       }
     });
   };
-  int kt = 0;
-  for (; kt + 3 < KT; kt += 2) {      // steady state: no branches inside a tile
-    tile(rx_int<0>{}, rx_int<0>{}, kt);
-    tile(rx_int<1>{}, rx_int<0>{}, kt + 1);
-  }
-  for (; kt + 2 < KT; kt += 2) {
-    tile(rx_int<0>{}, rx_int<1>{}, kt);
-    tile(rx_int<1>{}, rx_int<1>{}, kt + 1);
-  }
-  if (kt + 1 < KT) {
-    tile(rx_int<0>{}, rx_int<1>{}, kt);
-    tile(rx_int<1>{}, rx_int<2>{}, kt + 1);
-  } else {
-    tile(rx_int<0>{}, rx_int<2>{}, kt);
-  }
+  // The steady state has no branches inside a tile: it is unrolled over one period of (stage, B register set), and the
+  // tiles that cannot request a successor any more are written out one by one (KT is a compile-time constant).
+  constexpr int U = NSTG % 2 == 0 ? NSTG : 2 * NSTG;
+  constexpr int NSTEADY = KT > NSTG ? ((KT - NSTG) / U) * U : 0;
+  for (int kt = 0; kt < NSTEADY; kt += U)
+    rx_static_for<0, U>([&](auto UU) {
+      constexpr int u = decltype(UU)::value;
+      tile(rx_int<u % 2>{}, rx_int<u % NSTG>{}, rx_int<0>{}, kt + u);
+    });
+  rx_static_for<NSTEADY, KT>([&](auto KK) {
+    constexpr int k = decltype(KK)::value;
+    tile(rx_int<k % 2>{}, rx_int<k % NSTG>{}, rx_int<(k + NSTG < KT ? 0 : (k + 1 < KT ? 1 : 2))>{}, k);
+  });
   RX_SCHED_FENCE();
 
 #pragma unroll

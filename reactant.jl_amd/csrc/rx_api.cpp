@@ -267,6 +267,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_TRANSPOSE_BLOCK")) o.transpose_block = std::max(1, std::min(64, atoi(e)));
   if (const char* e = getenv("RX_MARCH2_PREFETCH")) o.march2_prefetch = atoi(e) == 2 ? 2 : 1;
   if (const char* e = getenv("RX_MARCH2_EDGE")) o.march2_edge = atoi(e) != 0;
+  if (const char* e = getenv("RX_MARCH2_LDS_BALLAST")) o.march2_lds_ballast = std::max(0, atoi(e));
   if (const char* e = getenv("RX_MARCH2_PLANES")) o.march2_planes = atoi(e) > 0 ? atoi(e) : o.march2_planes;
   if (const char* e = getenv("RX_MARCH2_TILE")) { int v[2]; if (sscanf(e, "%d,%d", &v[0], &v[1]) == 2) { o.march2_tile[0] = v[0]; o.march2_tile[1] = v[1]; } }
   if (const char* e = getenv("RX_LDS_TILE")) { int v[3]; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) == 3) { o.lds_tile[0] = v[0]; o.lds_tile[1] = v[1]; o.lds_tile[2] = v[2]; } }

@@ -129,7 +129,13 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
     // 256x128 tiles: wavefronts of 64x64 (4 + 4 fragments per K tile for 16 MFMA blocks) instead of 128x32 (8 + 2):
     // the 8192 x 1024 x 4096 bf16 layer 68.3 -> 66.6 us
     if (BN == 128 && !tuned) { WM = 4; WN = 2; }
-    c.lds_bytes = (unsigned)(2 * (BM + BN) * 128);
+    // three LDS stages where they fit (256x128 tiles: 144 KB): a request then has two K tiles to land instead of one
+    int sstages = (BM + BN) * 128 * 3 <= 160 * 1024 ? 3 : 2;
+    if (const char* e = getenv("RX_GEMM_STREAM_STAGES")) {
+      if ((atoi(e) != 2 && atoi(e) != 3) || (BM + BN) * 128 * atoi(e) > 160 * 1024) refuse("RX_GEMM_STREAM_STAGES is 2, or 3 where three stages fit 160 KB");
+      sstages = atoi(e);
+    }
+    c.lds_bytes = (unsigned)(sstages * (BM + BN) * 128);
     c.block = nt;
     c.grid[0] = (unsigned)gemm_grid((M + BM - 1) / BM, (N + BN - 1) / BN, rb, cb);
     c.grid[1] = (unsigned)batch;
@@ -139,10 +145,12 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       << ", " << N << ", " << K << ", " << rb << ", " << cb;
     c.targs = t.str();
     c.skeleton = "rx_gemm_body_s";
+    c.depth = 2;
     if (const char* e = getenv("RX_GEMM_STREAM_DEPTH")) {
       if (atoi(e) < 1 || atoi(e) > 3) refuse("RX_GEMM_STREAM_DEPTH is 1, 2 or 3");
       c.depth = atoi(e);
     }
+    c.stream_stages = sstages;
     c.stype_a = el + "::elem";
     c.ok = true;
     return c;
@@ -218,6 +226,7 @@ std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const s
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn" : fa.type) << ", " << (fb.type.empty() ? "rx_no_fn" : fb.type);
   if (c.split > 1) o << ", " << c.split;
   if (c.depth > 0) o << ", " << c.depth;
+  if (c.stream_stages > 0) o << ", " << c.stream_stages;
   o << ">(A, B, epi";
   if (fn) o << ", " << (fa.type.empty() ? "rx_no_fn()" : "la") << ", " << (fb.type.empty() ? "rx_no_fn()" : "lb");
   o << ");\n}\n\n";

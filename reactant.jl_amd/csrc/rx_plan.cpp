@@ -1738,6 +1738,7 @@ struct Planner {
     L.kind = "map_stencil_lds2";
     L.grid[0] = (unsigned)launch_blocks;
     L.block[0] = R0.nb;
+    L.lds_bytes = (unsigned)opt.march2_lds_ballast;   // occupancy experiments: dynamic LDS that the kernel never touches
     for (size_t k = 0; k < R0.inputs.size(); ++k) {
       if ((int)k == R0.prev_slot) continue;
       L.args.push_back(buffer_for(R0.inputs[k]));

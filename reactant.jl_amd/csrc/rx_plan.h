@@ -69,6 +69,7 @@ struct PlanOptions {
   int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
   bool transpose_vectors = true;   // transposing maps move 16-byte vectors where the dimensions allow it
   int transpose_block = 8;         // their tiles are taken in blocks of this many by this many (1: plain order)
+  int march2_lds_ballast = 0;   // bytes of LDS the marching stencil kernel declares and never uses: lowers its occupancy (measurements only)
   int march2_prefetch = 2;   // planes that the marching stencil kernel requests ahead of their use (1 or 2)
   // Runs of in-place update steps over small arrays (time loops of stencils): up to `chain_steps`
   // consecutive steps per launch, the arrays held in LDS tiles in between (0: 64 for vectors, 16
