@@ -321,6 +321,13 @@ def _mfma_ceiling(rx, client, entry, kind):
         return
     entry["sustained_mfma"] = {"random_operands": {"TFLOP/s": tf_r, "clock_MHz": mhz_r}, "zero_operands": {"TFLOP/s": tf_z, "clock_MHz": mhz_z},
                                "kernel_frac_of_random": entry["roofline"]["achieved"] / tf_r if tf_r else None}
+    # the config's large GEMM kernel with a clock probe inside (plain scaling epilogue, pseudo-random operands): the clock
+    # it runs at, read over a sleep of known length in the middle of the K loop, beside the ratio of the same two counters
+    # over the workgroups' lifetimes (lower: the cycle counter stands still while a compute unit has nothing to issue)
+    try:
+        entry["gemm_clock_probe"] = rx.gemm_clock_probe(dev, kind)
+    except Exception as e:
+        entry["gemm_clock_probe"] = {"error": str(e)[:200]}
 
 
 def _cw_err(got, ref, bound):

@@ -173,6 +173,12 @@ float RxCalibrationCopy(RxDevice *device, size_t bytes, int iters);
  * e4m3; operands pseudo-random, or all zero (`zero_operands` != 0: no toggling in the multipliers).  Writes the
  * TFLOP/s and the average shader clock in MHz; returns 0, or 1 with a message (RxLastError). */
 int RxMfmaCeiling(RxDevice *device, int kind, int zero_operands, double *tflops, double *clock_mhz);
+/* No counterpart in the reference (measurement aid).  The benchmark's two large GEMM kernels (kind 0: bf16
+ * 8192 x 4096 x 4096, kind 1: f8E4M3FN 8192^3) launched back to back with a clock probe inside: out5 = { us per
+ * launch, TFLOP/s, cycle counter / real-time counter over the workgroups' lifetimes in MHz, the same over a sleep of
+ * known length in the middle of the K loop in MHz (the clock the kernel runs at), cycles counted over that sleep
+ * (65024 by the sleep instruction's definition) }. */
+int RxGemmClockProbe(RxDevice *device, int kind, double *out5);
 
 #ifdef __cplusplus
 }

@@ -122,6 +122,7 @@ SIGNATURES = {
     "RxDeviceSynchronize": (None, [_vp]),
     "RxCalibrationCopy": (ctypes.c_float, [_vp, _sz, _i]),
     "RxMfmaCeiling": (_i, [_vp, _i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
+    "RxGemmClockProbe": (_i, [_vp, _i, ctypes.POINTER(ctypes.c_double)]),
 }
 for _name, (_res, _args) in SIGNATURES.items():
     _fn = getattr(lib, _name)
@@ -479,6 +480,17 @@ def mfma_ceiling(device, kind, zero_operands=False):
     tf, mhz = ctypes.c_double(), ctypes.c_double()
     _call("RxMfmaCeiling", device.handle, {"bf16": 0, "f8": 1}[kind], 1 if zero_operands else 0, ctypes.byref(tf), ctypes.byref(mhz))
     return tf.value, mhz.value
+
+
+def gemm_clock_probe(device, kind):
+    """The benchmark's large GEMM kernel of `kind` ("bf16": 8192 x 4096 x 4096, "f8": 8192^3) launched back to back with a
+    clock probe inside: dict with us per launch, TFLOP/s, the ratio of the shader-cycle counter to the real-time counter
+    over the workgroups' lifetimes (MHz), the same ratio over a sleep of known length in the middle of the K loop (MHz:
+    the clock the kernel runs at) and the cycles counted over that sleep (65024 nominal)."""
+    out = (ctypes.c_double * 5)()
+    _call("RxGemmClockProbe", device.handle, {"bf16": 0, "f8": 1}[kind], out)
+    return {"us_per_launch": out[0], "TFLOP/s": out[1], "lifetime_cycles_over_real_time_MHz": out[2], "clock_MHz": out[3],
+            "cycles_over_a_sleep_of_65024": out[4]}
 
 
 def compile_offline(mlir_text, with_source=False):

@@ -708,7 +708,8 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
         TRAITS::coords(lane, rg, &dm, &dn);
         const int m = m0 + wm * (BM / WM) + 32 * i + dm;
         const int n = n0 + wn * (BN / WN) + 32 * j + dn;
-        if (m < M && n < N) {
+        constexpr bool WHOLE = M % BM == 0 && N % BN == 0;   // no bounds test: the epilogue becomes straight-line code
+        if (WHOLE || (m < M && n < N)) {
           const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
           if constexpr (BATCHED) epi(v, (int)batch, m, n);
           else if constexpr (SPLIT > 1) epi(v, (int)blockIdx.y, m, n);
@@ -868,8 +869,28 @@ struct rx_dma_s {
   }
 };
 
-template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2>
-RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi) {
+// Clock probe for measurements (the library's RxGemmClockProbe; the kernels of compiled programs never carry it): in
+// the middle of the K loop of its tile, wavefront 0 of every 16th workgroup sleeps 8 x s_sleep 127 -- 65024 shader
+// cycles by the instruction's definition -- and records what the shader-cycle counter and the 100 MHz real-time
+// counter advanced meanwhile.  cycles / real time is the clock the compute unit ran at while the rest of the chip
+// kept multiplying; the same two counters over a workgroup's whole lifetime read lower, because the cycle counter
+// does not advance while the compute unit has nothing to issue.
+struct rx_clock_probe {
+  static constexpr bool none = false;
+  unsigned long long* out;   // per workgroup: [0] cycles, [1] real-time ticks over the sleep
+  RX_MEM void mid(int kt, int at, int wave, int lane) const {
+    if (kt == at && (blockIdx.x & 15) == 0 && wave == 0) {
+      const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+#pragma unroll
+      for (int q = 0; q < 8; ++q) __builtin_amdgcn_s_sleep(127);
+      const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+      if (lane == 0) { out[blockIdx.x * 2] = c1 - c0; out[blockIdx.x * 2 + 1] = r1 - r0; }
+    }
+  }
+};
+
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2, class Probe = rx_no_fn>
+RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, const Probe& probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NBUF = 4;
   constexpr int NT = WM * WN * 64;
@@ -964,6 +985,7 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
         read_a(rx_int<t % NBUF>{}, CUR{}, t);
       } else if constexpr (!last) {
         if constexpr (t == NA) {
+          if constexpr (!Probe::none) probe.mid(kt, KT / 2, wave, lane);
           // tile kt+1 has landed once only the NSTG-2 tiles after it are still in flight
           if constexpr (mode == 0) rx_wait_vmcnt<(NSTG - 2) * NLT>(); else rx_wait_vmcnt<0>();
           publish();
@@ -1020,7 +1042,11 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
     for (int j = 0; j < NB; ++j) {
       const int m = m0 + wm * (BM / WM) + 16 * i + (lane & 15);
       const int n = n0 + wn * (BN / WN) + 16 * j + 4 * (lane >> 4);
-      if (m < M && n < N) {
+      // Whole tiles need no bounds test, and without it the epilogue is straight-line code: the compiler then requests
+      // what the functor reads (a bias, the C operand) for all blocks ahead of the arithmetic instead of one
+      // request, one wait and one store per block.
+      constexpr bool WHOLE = M % BM == 0 && N % BN == 0;
+      if (WHOLE || (m < M && n < N)) {
         const float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
         if constexpr (BATCHED) epi(v, (int)batch, m, n);
         else epi(v, m, n);

@@ -19,6 +19,7 @@
 #include "rx_embedded.inc"
 #include "rx_ir.h"
 #include "rx_plan.h"
+#include "rx_gemm.h"
 
 #define RX_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -337,6 +338,10 @@ RxBuffer* new_buffer(RxClient* c, RxDevice* d, const rx::TType& ty, Mem mem) {
 }
 
 // AOT kernels ------------------------------------------------------------------
+}  // namespace
+#include "kernels/rx_preamble.h"
+#include "kernels/rx_gemm_kernels.h"
+namespace {
 __global__ __launch_bounds__(256) void rx_copy16(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * 256;
@@ -405,6 +410,46 @@ __global__ __launch_bounds__(256) void rx_mfma_probe(unsigned long long* ticks, 
   if ((tid & 63) == 0) {
     ticks[(blockIdx.x * 4 + (tid >> 6)) * 2] = t1 - t0;
     ticks[(blockIdx.x * 4 + (tid >> 6)) * 2 + 1] = w1 - w0;
+  }
+}
+
+// The two large GEMM kernels of the benchmark (the 8192 x 4096 x 4096 bf16 layer, operands [m][k] x [k][n], and the
+// 8192^3 e4m3 product, [m][k] x [n][k]) as the planner instantiates them, with a plain scaling epilogue and the clock
+// probe of rx_gemm_kernels.h: RxGemmClockProbe.
+struct rx_probe_epi {
+  rx_u16* __restrict__ out;
+  int ld;
+  template <int NV> __device__ __forceinline__ void operator()(const float (&acc)[NV], int m, int n) const {
+    rx_vec<rx_u16, NV> res;
+#pragma unroll
+    for (int l = 0; l < NV; ++l) res.v[l] = rx_f32_to_bf16(acc[l] * 0.001f);
+    *reinterpret_cast<rx_vec<rx_u16, NV>*>(out + (long long)m * ld + n) = res;
+  }
+};
+template <int KIND>
+__global__ __launch_bounds__(512) void rx_gemm_clock_probe(const void* __restrict__ A, const void* __restrict__ B, rx_u16* __restrict__ out,
+                                                           unsigned long long* __restrict__ sleep_ticks, unsigned long long* __restrict__ life_ticks) {
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  rx_clock_probe probe{sleep_ticks};
+  if constexpr (KIND == 0) {
+    rx_probe_epi epi{out, 4096};
+    rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096, 4, 8, false, rx_probe_epi, 2, 2, rx_clock_probe>((const rx_u16*)A, (const rx_u16*)B, epi, probe);
+  } else {
+    rx_probe_epi epi{out, 8192};
+    rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192, 4, 8, false, rx_probe_epi, 2, 2, rx_clock_probe>((const rx_u8*)A, (const rx_u8*)B, epi, probe);
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0) { life_ticks[blockIdx.x * 2] = c1 - c0; life_ticks[blockIdx.x * 2 + 1] = r1 - r0; }
+}
+// pseudo-random operands: bf16 values in (-2, 2) with random mantissas, or e4m3 codes of moderate exponent (no NaN codes)
+__global__ __launch_bounds__(256) void rx_probe_fill(unsigned* __restrict__ words, size_t nwords, int kind, unsigned seed) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < nwords; i += stride) {
+    unsigned s = ((unsigned)i + seed) * 2654435761u + 12345u;
+    s ^= s >> 15; s *= 2246822519u; s ^= s >> 13;
+    words[i] = kind == 0 ? ((s & 0x807f807fu) | 0x3f003f00u) : ((s & 0xa7a7a7a7u) | 0x30303030u);
   }
 }
 
@@ -1134,6 +1179,54 @@ RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tf
     for (int i = 0; i < 1024; ++i) { c += (double)h[2 * i]; w += (double)h[2 * i + 1]; }
     if (tflops) *tflops = flop_per_iter * iters * 1024 / (ms * 1e-3) / 1e12;
     if (clock_mhz) *clock_mhz = w > 0 ? c / w * 100.0 : 0.0;   // the real-time counter ticks at 100 MHz
+    return 0;
+  }, 1);
+}
+
+RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out5) {
+  return guarded([&]() -> int {
+    check_device(d);
+    if (kind != 0 && kind != 1) throw Error("INVALID_ARGUMENT: kind is 0 (bf16 8192 x 4096 x 4096) or 1 (f8E4M3FN 8192^3)");
+    if (!out5) throw Error("INVALID_ARGUMENT: null result array");
+    HIP_CHECK(hipSetDevice(d->ordinal));
+    const size_t M = 8192, N = kind == 0 ? 4096 : 8192, K = kind == 0 ? 4096 : 8192, esz = kind == 0 ? 2 : 1;
+    const unsigned grid = (unsigned)rx::gemm_grid((int64_t)(M / 256), (int64_t)(N / 256), 4, 8);
+    Allocation a(d, M * K * esz), b(d, N * K * esz), o(d, M * N * 2), sl(d, grid * 16), lf(d, grid * 16);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, (unsigned*)a.ptr, M * K * esz / 4, kind, 1u);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, (unsigned*)b.ptr, N * K * esz / 4, kind, 77u);
+    HIP_CHECK(hipMemsetAsync(sl.ptr, 0, grid * 16, d->stream));
+    HIP_CHECK(hipMemsetAsync(lf.ptr, 0, grid * 16, d->stream));
+    const int lds = 2 * 512 * 128;
+    auto fn = kind == 0 ? rx_gemm_clock_probe<0> : rx_gemm_clock_probe<1>;
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    hipEvent_t e0, e1;
+    HIP_CHECK(hipEventCreate(&e0));
+    HIP_CHECK(hipEventCreate(&e1));
+    const int warm = 5, reps = 20;   // back to back, so that the clock has settled under the power limit
+    for (int i = 0; i < warm; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
+    HIP_CHECK(hipEventRecord(e0, d->stream));
+    for (int i = 0; i < reps; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
+    HIP_CHECK(hipEventRecord(e1, d->stream));
+    HIP_CHECK(hipEventSynchronize(e1));
+    float ms = 0;
+    HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    std::vector<unsigned long long> hs(grid * 2), hl(grid * 2);
+    HIP_CHECK(hipMemcpy(hs.data(), sl.ptr, grid * 16, hipMemcpyDeviceToHost));
+    HIP_CHECK(hipMemcpy(hl.data(), lf.ptr, grid * 16, hipMemcpyDeviceToHost));
+    double sc = 0, sr = 0, lc = 0, lr = 0;
+    int ns = 0;
+    for (unsigned w = 0; w < grid; ++w) {
+      if (hs[2 * w + 1]) { sc += (double)hs[2 * w]; sr += (double)hs[2 * w + 1]; ++ns; }
+      lc += (double)hl[2 * w]; lr += (double)hl[2 * w + 1];
+    }
+    const double us = ms * 1e3 / reps;
+    out5[0] = us;                                                   // per launch; the sleeping wavefronts lengthen it by a few per cent
+    out5[1] = 2.0 * M * N * K / (us * 1e-6) / 1e12;                 // TFLOP/s
+    out5[2] = lr > 0 ? lc / lr * 100.0 : 0.0;                       // cycle counter / real time over the workgroups' lifetimes, MHz
+    out5[3] = sr > 0 ? sc / sr * 100.0 : 0.0;                       // the same over the sleeps: the clock, MHz
+    out5[4] = ns > 0 ? sc / ns : 0.0;                               // cycles counted over a sleep of 65024 nominal cycles
     return 0;
   }, 1);
 }

@@ -1466,7 +1466,7 @@ struct Planner {
     const int64_t APLANE = AY * AX, BPLANE = BY * BX, AV = AY * AXV;
     const int64_t RA = hP.lo[0] + hP.hi[0] + 2, RB = hR.lo[0] + hR.hi[0] + 2;   // a stencil's reach plus the plane being written
     const int es = info(rn.ty.dt).size;
-    if ((RA * APLANE + RB * BPLANE) * es > 64 * 1024) return false;
+    if ((RA * APLANE + RB * BPLANE) * es > 80 * 1024) return false;   // two workgroups per compute unit at least
     const int64_t NLA = (AV + NB - 1) / NB;   // 16-byte loads per thread for one source plane
     if (NLA > 8) return false;
     const std::string st = info(rn.ty.dt).stype;
@@ -1727,8 +1727,16 @@ struct Planner {
     }
     int64_t lds_a = 0, lds_b = 0, launch_blocks = 0;
     for (auto& R : regions) { lds_a = std::max(lds_a, R.lds_a); lds_b = std::max(lds_b, R.lds_b); launch_blocks += R.blocks; }
-    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsA[" << lds_a << "];\n";
-    o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << lds_b << "];\n";
+    // the two rings: static LDS up to the 64 KB that a static array may take, dynamic beyond
+    const int es_k = info(rn.ty.dt).size;
+    const bool dyn_lds = (lds_a + lds_b) * es_k > 64 * 1024;
+    if (dyn_lds) {
+      o << "  extern __shared__ __attribute__((aligned(16))) " << st << " rx_rings[];\n";
+      o << "  " << st << "* const ldsA = rx_rings;\n  " << st << "* const ldsB = rx_rings + " << lds_a << ";\n";
+    } else {
+      o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsA[" << lds_a << "];\n";
+      o << "  __shared__ __attribute__((aligned(16))) " << st << " ldsB[" << lds_b << "];\n";
+    }
     if (split) o << "  if (blockIdx.x < " << R0.blocks << "u) {\n" << R0.text << "  } else {\n" << regions[1].text << "  }\n";
     else o << R0.text;
     o << "}\n\n";
@@ -1738,7 +1746,7 @@ struct Planner {
     L.kind = "map_stencil_lds2";
     L.grid[0] = (unsigned)launch_blocks;
     L.block[0] = R0.nb;
-    L.lds_bytes = (unsigned)opt.march2_lds_ballast;   // occupancy experiments: dynamic LDS that the kernel never touches
+    L.lds_bytes = (unsigned)((dyn_lds ? (lds_a + lds_b) * es_k : 0) + opt.march2_lds_ballast);   // the ballast (occupancy experiments) is never touched
     for (size_t k = 0; k < R0.inputs.size(); ++k) {
       if ((int)k == R0.prev_slot) continue;
       L.args.push_back(buffer_for(R0.inputs[k]));
