@@ -699,7 +699,7 @@ def main():
         "roofline": main_res["roofline"],
         "copy_kernel_GBs": 2.0 * (1 << 30) / (copy_ms * 1e-3) / 1e9 if copy_ms > 0 else None,
     }
-    for key in ("check", "cpu_baseline", "whole_step_frac", "sustained_mfma"):
+    for key in ("check", "cpu_baseline", "whole_step_frac", "sustained_mfma", "gemm_clock_probe", "with_launch_events"):
         if key in main_res:
             out[key] = main_res[key]
     if "kernels" in main_res:

@@ -442,14 +442,24 @@ __global__ __launch_bounds__(512) void rx_gemm_clock_probe(const void* __restric
   const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
   if (threadIdx.x == 0) { life_ticks[blockIdx.x * 2] = c1 - c0; life_ticks[blockIdx.x * 2 + 1] = r1 - r0; }
 }
-// pseudo-random operands: bf16 values in (-2, 2) with random mantissas, or e4m3 codes of moderate exponent (no NaN codes)
-__global__ __launch_bounds__(256) void rx_probe_fill(unsigned* __restrict__ words, size_t nwords, int kind, unsigned seed) {
+// Pseudo-random operands shaped like the benchmark's: mode 0 bf16 ~ N(0, 1) (activations), mode 1 bf16 uniform in
+// +-0.027 (Glorot weights of a 4096-wide layer), mode 2 e4m3 of N(0, 1) scaled to an absmax of 448 at 5.5 sigma (a tensor
+// quantized with a per-tensor scale).  The normal is a sum of four uniforms.
+__global__ __launch_bounds__(256) void rx_probe_fill(void* __restrict__ dst, size_t n, int mode, unsigned seed) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * 256;
-  for (; i < nwords; i += stride) {
+  for (; i < n; i += stride) {
     unsigned s = ((unsigned)i + seed) * 2654435761u + 12345u;
-    s ^= s >> 15; s *= 2246822519u; s ^= s >> 13;
-    words[i] = kind == 0 ? ((s & 0x807f807fu) | 0x3f003f00u) : ((s & 0xa7a7a7a7u) | 0x30303030u);
+    float u[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      s ^= s >> 15; s *= 2246822519u; s ^= s >> 13; s *= 3266489917u; s ^= s >> 16;
+      u[k] = (float)(s >> 8) * (1.0f / 16777216.0f);
+    }
+    const float g = (u[0] + u[1] + u[2] + u[3] - 2.0f) * 1.7320508f;   // variance 4 / 12 -> 1
+    if (mode == 0) ((rx_u16*)dst)[i] = rx_f32_to_bf16(g);
+    else if (mode == 1) ((rx_u16*)dst)[i] = rx_f32_to_bf16((u[0] * 2.0f - 1.0f) * 0.027f);
+    else ((rx_u8*)dst)[i] = rx_f32_to_e4m3(g * (448.0f / 5.5f));
   }
 }
 
@@ -1192,8 +1202,8 @@ RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out5) {
     const size_t M = 8192, N = kind == 0 ? 4096 : 8192, K = kind == 0 ? 4096 : 8192, esz = kind == 0 ? 2 : 1;
     const unsigned grid = (unsigned)rx::gemm_grid((int64_t)(M / 256), (int64_t)(N / 256), 4, 8);
     Allocation a(d, M * K * esz), b(d, N * K * esz), o(d, M * N * 2), sl(d, grid * 16), lf(d, grid * 16);
-    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, (unsigned*)a.ptr, M * K * esz / 4, kind, 1u);
-    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, (unsigned*)b.ptr, N * K * esz / 4, kind, 77u);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, a.ptr, M * K, kind == 0 ? 0 : 2, 1u);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, b.ptr, N * K, kind == 0 ? 1 : 2, 77u);
     HIP_CHECK(hipMemsetAsync(sl.ptr, 0, grid * 16, d->stream));
     HIP_CHECK(hipMemsetAsync(lf.ptr, 0, grid * 16, d->stream));
     const int lds = 2 * 512 * 128;
