@@ -100,6 +100,12 @@ void ExecutableFree(RxExecutable *exec);                             /* API.cpp:
 RxClient *PjRtLoadedExecutableGetClient(RxExecutable *exec);         /* API.cpp:807  */
 /* API.cpp:2064-2071: there are no HLO modules here; *nmodules is set to 0. */
 void PjRtLoadedExecutableGetHloModules(RxExecutable *exec, void **hlo_modules, int32_t *nmodules);
+/* pjrt_hlo_module_cost_analysis_properties (API.cpp:3238-3260; Julia: XLA.cost_analysis, src/xla/Stats.jl:86-115) takes a
+ * HeldHloModule, which this library does not keep.  This entry point fills the same struct of eleven floats
+ * (JLHloCostAnalysisProperties: flops, transcendentals, bytes accessed, optimal seconds, utilization, operand 0 / 1
+ * utilization, operand 0 / 1 bytes accessed, output root bytes accessed, reserved) for an executable, counted over the
+ * StableHLO module it was compiled from. */
+void RxExecutableCostAnalysis(RxExecutable *exec, float *properties11);
 /* API.cpp:1585-1630.  Results are owning handles; *futures is set to 1 and one
  * future per result is returned.  A donated argument (is_arg_donatable[i] != 0)
  * gives up its storage: the handle stays valid only for PjRtBufferFree. */

@@ -77,6 +77,7 @@ function __init__()
     install_routes!()
     install_compile!()
     install_execute!()
+    install_cost_analysis!()
     register!()
     return nothing
 end

@@ -72,3 +72,29 @@ function execute_no_alloc!(exec::PJRT.LoadedExecutable, args::Vector{PJRT.Buffer
     rc == 0 || error("RxExecuteNoAlloc failed: " * unsafe_string(ccall(sym(:RxLastError), Cstring, ())))
     return results
 end
+
+"""
+    XLA.cost_analysis(exec::PJRT.LoadedExecutable)
+
+Reference: `cost_analysis(exec)` asks every HLO module of the executable
+(src/xla/LoadedExecutable.jl:14-18 -> `pjrt_hlo_module_cost_analysis_properties`, src/xla/PJRT/Client.jl:83-90).
+An executable of this library keeps no HLO module (`get_hlo_modules` returns none), so the same
+`JLHloCostAnalysisProperties` comes from `RxExecutableCostAnalysis`, counted over the StableHLO module
+the executable was compiled from.
+"""
+function install_cost_analysis!()
+    Core.eval(
+        PJRT,
+        quote
+            function XLA.cost_analysis(exec::LoadedExecutable)
+                $(owns)(exec.exec) || return invoke(XLA.cost_analysis, Tuple{XLA.AbstractLoadedExecutable}, exec)
+                props = Ref{MLIR.API.JLHloCostAnalysisProperties}()
+                GC.@preserve exec props begin
+                    ccall($(sym)(:RxExecutableCostAnalysis), Cvoid, (Ptr{Cvoid}, Ptr{Cvoid}), exec.exec, props)
+                end
+                return props[]
+            end
+        end,
+    )
+    return nothing
+end

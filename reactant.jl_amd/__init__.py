@@ -123,6 +123,7 @@ SIGNATURES = {
     "RxCalibrationCopy": (ctypes.c_float, [_vp, _sz, _i]),
     "RxMfmaCeiling": (_i, [_vp, _i, _i, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "RxGemmClockProbe": (_i, [_vp, _i, ctypes.POINTER(ctypes.c_double)]),
+    "RxExecutableCostAnalysis": (None, [_vp, ctypes.POINTER(ctypes.c_float)]),
 }
 for _name, (_res, _args) in SIGNATURES.items():
     _fn = getattr(lib, _name)
@@ -397,6 +398,14 @@ class LoadedExecutable:
             out.append({"kernel": kn.value.decode(), "kind": kd.value.decode(), "algorithmic_bytes": b.value,
                         "flops": f.value})
         return out
+
+    def cost_analysis(self):
+        """XLA.cost_analysis(exec) (src/xla/Stats.jl:86-115): the fields of HloCostAnalysisProperties as a dict."""
+        props = (ctypes.c_float * 11)()
+        _call("RxExecutableCostAnalysis", self.handle, props)
+        names = ("flops", "transcendentals", "bytes_accessed", "optimal_seconds", "utilization", "operand0_utilization",
+                 "operand1_utilization", "operand0_bytes_accessed", "operand1_bytes_accessed", "output_root_bytes_accessed", "reserved0")
+        return dict(zip(names, [float(v) for v in props]))
 
     def get_hlo_modules(self):
         n = ctypes.c_int32(-1)

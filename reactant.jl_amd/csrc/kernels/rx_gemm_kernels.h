@@ -183,8 +183,18 @@ struct rx_tile_copy {
         const int rr = row0 + v / VPR;
         const int cc = col0 + (v % VPR) * VE;
         union { E e[VE]; rx_u32x4 q; } u;
+        if constexpr (FN::vec_width == VE) {
+          // a whole vector inside the matrix: the functor's vector form shares the index arithmetic between the lanes
+          if (rr < nrows && cc + VE <= ncols) {
+            fn.vec(batch, rr, cc, u.e);
+          } else {
 #pragma unroll
-        for (int k = 0; k < VE; ++k) u.e[k] = (rr < nrows && cc + k < ncols) ? fn(batch, rr, cc + k) : E(0);
+            for (int k = 0; k < VE; ++k) u.e[k] = (rr < nrows && cc + k < ncols) ? fn(batch, rr, cc + k) : E(0);
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < VE; ++k) u.e[k] = (rr < nrows && cc + k < ncols) ? fn(batch, rr, cc + k) : E(0);
+        }
         r[i] = u.q;
       }
     }
@@ -229,7 +239,7 @@ RX_DEV bool rx_gemm_tile(unsigned bid, int* bm, int* bn) {
 // An operand can also be a functor (LA / LB other than rx_no_fn): the fusion code generator
 // writes one when the operand is a cheap expansion of smaller data (the window matrix of a
 // convolution, a broadcast), so that the expanded matrix never exists in memory.
-struct rx_no_fn { static constexpr bool none = true; };
+struct rx_no_fn { static constexpr bool none = true; static constexpr int vec_width = 0; };
 
 template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
           class LA = rx_no_fn, class LB = rx_no_fn>

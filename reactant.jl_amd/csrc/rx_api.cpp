@@ -976,6 +976,34 @@ RX_EXPORT void PjRtLoadedExecutableGetHloModules(RxExecutable* ex, void** mods, 
   (void)mods;
   guarded_void([&] { check_exec(ex); if (n) *n = 0; });
 }
+// The counterpart of pjrt_hlo_module_cost_analysis_properties (API.cpp:3238-3260) for an executable of this library,
+// which keeps no HLO module: the same eleven floats, counted over the StableHLO module as it was compiled.  The optimal
+// time is that of the plan's launches at the device's peaks (each launch the larger of its arithmetic and its memory time).
+RX_EXPORT void RxExecutableCostAnalysis(RxExecutable* ex, float* props11) {
+  guarded_void([&] {
+    check_exec(ex);
+    if (!props11) throw Error("INVALID_ARGUMENT: null properties");
+    std::lock_guard<std::mutex> lock(ex->mu);
+    const rx::Plan& P = ex->plan;
+    double optimal = 0;
+    for (auto& L : P.launches) {
+      const double peak = L.kind == "gemm_f8" ? 5.0e15 : (L.kind == "gemm_bf16" || L.kind == "gemm_f16") ? 2.5e15 : L.kind == "gemm_f64" ? 78.6e12 : 157.3e12;
+      optimal += std::max(L.flops / peak, L.algo_bytes / 8.0e12);
+    }
+    const double mem_time = P.hlo_bytes_accessed / 8.0e12;
+    props11[0] = (float)P.hlo_flops;
+    props11[1] = (float)P.hlo_transcendentals;
+    props11[2] = (float)P.hlo_bytes_accessed;
+    props11[3] = (float)optimal;
+    props11[4] = (float)(mem_time > 0 ? std::min(1.0, optimal / mem_time) : 0.0);   // utilization: optimal time over the time of every op's own traffic
+    props11[5] = P.hlo_bytes_accessed > 0 ? (float)(P.hlo_operand_bytes[0] / P.hlo_bytes_accessed) : 0.f;
+    props11[6] = P.hlo_bytes_accessed > 0 ? (float)(P.hlo_operand_bytes[1] / P.hlo_bytes_accessed) : 0.f;
+    props11[7] = (float)P.hlo_operand_bytes[0];
+    props11[8] = (float)P.hlo_operand_bytes[1];
+    props11[9] = (float)P.hlo_output_bytes;
+    props11[10] = 0.f;
+  });
+}
 RX_EXPORT const char* RxExecutableReport(RxExecutable* ex) { return guarded([&]() -> const char* { check_exec(ex); return ex->report.c_str(); }, ""); }
 RX_EXPORT int RxExecutableNumLaunches(RxExecutable* ex) { return guarded([&] { check_exec(ex); return (int)ex->plan.launches.size(); }, 0); }
 RX_EXPORT int RxExecutableNumResults(RxExecutable* ex) { return guarded([&] { check_exec(ex); return (int)ex->plan.result_types.size(); }, 0); }

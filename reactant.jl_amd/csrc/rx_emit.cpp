@@ -592,6 +592,32 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
         if (ok && groups.size() > 1) {
           for (auto& gq : groups) {
             if (gq.a1 - gq.a0 == 1 && gq.b1 - gq.b0 == 1) { oi[gq.b0] = ix[gq.a0]; continue; }
+            // One source dimension whose index is lane `off` of an aligned vector (var a multiple of `align`), split into
+            // dimensions the innermost of which is a whole number of vectors: var splits by itself and the lane is added
+            // to the innermost component -- the lanes of a vector then share every division.
+            {
+              int k0 = -1, nz = 0, last = -1;
+              for (size_t k = gq.a0; k < gq.a1; ++k) if (nd[k] != 1) { k0 = (int)k; ++nz; }
+              for (size_t k = gq.b0; k < gq.b1; ++k) if (od[k] != 1) last = (int)k;
+              if (nz == 1 && last >= 0) {
+                const Ix& sx = ix[k0];
+                if (!sx.is_const() && sx.align > 1 && sx.off >= 0 && sx.off < sx.align && od[last] % sx.align == 0) {
+                  int64_t stride = nd[k0];
+                  for (size_t k = gq.b0; k < gq.b1; ++k) {
+                    stride /= std::max<int64_t>(od[k], 1);
+                    if (od[k] == 1) continue;
+                    std::string c2 = sx.var;
+                    if (stride > 1) c2 = "(" + c2 + " / " + std::to_string(stride) + ")";
+                    bool first = true;
+                    for (size_t q = gq.b0; q < k; ++q) first = first && od[q] == 1;
+                    if (!first) c2 = c2 + " % " + std::to_string(od[k]);
+                    oi[k] = temp_index(c2, 0, od[k] - 1);
+                    if ((int)k == last) { oi[k].off = sx.off; oi[k].align = sx.align; oi[k].hi = od[k] - sx.align; oi[k].lo = 0; oi[k].lo += sx.off; oi[k].hi += sx.off; }
+                  }
+                  continue;
+                }
+              }
+            }
             // linear index inside the group
             std::string e;
             int64_t total = 1, lo = 0, hi = 0;

@@ -18,9 +18,12 @@ struct Ix {
   std::string var;
   int64_t off = 0;
   int64_t lo = 0, hi = 0;
+  // `var` is known to be a multiple of `align` (the first lane of a vector of `align` consecutive elements, off = lane):
+  // a reshape then splits var alone and adds the lane to the innermost component, so the divisions are shared by the lanes
+  int64_t align = 1;
   bool is_const() const { return var.empty(); }
   std::string str() const;
-  std::string key() const { return var + "+" + std::to_string(off); }
+  std::string key() const { return var + "+" + std::to_string(off) + (align > 1 ? "@" + std::to_string(align) : ""); }
 };
 using Index = std::vector<Ix>;
 

@@ -3833,7 +3833,41 @@ struct Planner {
       o << "  __device__ __forceinline__ " << E << " operator()(long long ob_, int r_, int c_) const {\n";
       o << "    const " << eit << " ob = (" << eit << ")ob_, r = (" << eit << ")r_, c = (" << eit << ")c_;\n    (void)ob;\n";
       o << code;
-      o << "    return " << e.store_value(xt.dt, v) << ";\n  }\n};\n\n";
+      o << "    return " << e.store_value(xt.dt, v) << ";\n  }\n";
+      // The same for a whole 16-byte vector of consecutive columns starting at a multiple of the vector width: the
+      // index arithmetic that does not depend on the lane (the splitting of row and column numbers into the operand's
+      // own coordinates) is written once per lane in the text but on the same expressions, so it is computed once.
+      const int VE = 16 / (int)info(xt.dt).size;
+      const int64_t minor = xt.dims[xt.rank() - 1];
+      if (VE > 1 && minor % VE == 0 && xt.rank() == nbd + 2) {
+        Emitter ev(g, [&](int y) { return mat[y] != 0; });
+        ev.excess_precision = opt.excess_precision;
+        ev.idx64 = e.idx64;
+        ev.set_root({}, {}, false);
+        ev.indent = 4;
+        ev.inputs = e.inputs;
+        std::vector<std::string> vals;
+        for (int l = 0; l < VE; ++l) {
+          Index il = ix;
+          il[xt.rank() - 1].off = l;
+          il[xt.rank() - 1].align = VE;
+          il[xt.rank() - 1].hi = xt.dims[xt.rank() - 1] - 1;
+          vals.push_back(ev.store_value(xt.dt, ev.emit(x, il)));
+        }
+        if (ev.inputs == e.inputs) {
+          o << "  static constexpr int vec_width = " << VE << ";\n";
+          o << "  __device__ __forceinline__ void vec(long long ob_, int r_, int c_, " << E << "* out) const {\n";
+          o << "    const " << eit << " ob = (" << eit << ")ob_, r = (" << eit << ")r_, c = (" << eit << ")c_;\n    (void)ob;\n";
+          o << ev.take_code();
+          for (int l = 0; l < VE; ++l) o << "    out[" << l << "] = " << vals[l] << ";\n";
+          o << "  }\n";
+        } else {
+          o << "  static constexpr int vec_width = 0;\n";
+        }
+      } else {
+        o << "  static constexpr int vec_width = 0;\n";
+      }
+      o << "};\n\n";
       fn.type = kbase + "_" + tag;
       fn.ctor = fn.type + " " + (side == 0 ? "la" : "lb") + "{";
       for (size_t k = 0; k < inputs.size(); ++k) {
@@ -4209,12 +4243,65 @@ std::string Plan::report() const {
     o << "  [" << i << "] " << L.kernel << " kind=" << L.kind << " grid=" << L.grid[0] << "x" << L.grid[1] << "x" << L.grid[2] << " block=" << L.block[0]
       << " lds=" << L.lds_bytes << " algo_bytes=" << (long long)L.algo_bytes << " flops=" << (long long)L.flops << " :: " << L.desc << "\n";
   }
+  o << "module costs: flops=" << (long long)hlo_flops << " transcendentals=" << (long long)hlo_transcendentals << " bytes_accessed=" << (long long)hlo_bytes_accessed
+    << " output_bytes=" << (long long)hlo_output_bytes << "\n";
   return o.str();
+}
+
+// Operation counts of the module as written, in the conventions of XLA's HloCostAnalysis: a product counts 2 M N K,
+// every other arithmetic op one operation per result element (a reduction one per reduced element), transcendental ops
+// are counted apart, and every op reads its operands and writes its result once.
+static void count_hlo_costs(const Graph& g, Plan* plan) {
+  const size_t N = g.nodes.size();
+  std::vector<char> live(N, 0);
+  std::vector<int> stack(g.results.begin(), g.results.end());
+  while (!stack.empty()) {
+    const int x = stack.back();
+    stack.pop_back();
+    if (live[x]) continue;
+    live[x] = 1;
+    for (int i : g.nodes[x].in) stack.push_back(i);
+  }
+  static const char* const kTrans[] = {"exponential", "exponential_minus_one", "log", "log_plus_one", "logistic", "tanh", "sine", "cosine", "tan",
+                                       "rsqrt", "sqrt", "cbrt", "erf", "power", "atan2"};
+  double flops = 0, trans = 0, bytes = 0;
+  for (size_t x = 0; x < N; ++x) {
+    if (!live[x]) continue;
+    const Node& n = g.nodes[x];
+    const double numel = (double)n.ty.numel();
+    bool is_trans = n.k == OpK::Gelu;
+    for (const char* t : kTrans) is_trans = is_trans || n.op == t;
+    switch (n.k) {
+      case OpK::Param: case OpK::Constant: case OpK::Iota: break;
+      case OpK::DotGeneral: {
+        double kk = 1;
+        for (int64_t d : n.a2) kk *= (double)g.nodes[n.in[0]].ty.dims[d];
+        flops += 2.0 * numel * kk;
+        break;
+      }
+      case OpK::Reduce: case OpK::Scan: flops += (double)g.nodes[n.in[0]].ty.numel(); break;
+      case OpK::Unary: case OpK::Binary: case OpK::Gelu:
+        if (is_trans) trans += numel; else flops += numel;
+        break;
+      case OpK::Compare: case OpK::Select: case OpK::Clamp: case OpK::Scatter: flops += numel; break;
+      default: break;   // data movement
+    }
+    if (n.k != OpK::Param && n.k != OpK::Constant) {
+      bytes += (double)n.ty.bytes();
+      for (int i : n.in) bytes += (double)g.nodes[i].ty.bytes();
+    }
+  }
+  plan->hlo_flops = flops;
+  plan->hlo_transcendentals = trans;
+  plan->hlo_bytes_accessed = bytes;
+  for (size_t k = 0; k < 2 && k < g.params.size(); ++k) plan->hlo_operand_bytes[k] = (double)g.nodes[g.params[k]].ty.bytes();
+  for (int r : g.results) plan->hlo_output_bytes += (double)g.nodes[r].ty.bytes();
 }
 
 Plan make_plan(const Graph& g, const PlanOptions& opt) {
   Planner p(g, opt);
   p.run();
+  count_hlo_costs(g, &p.plan);
   return std::move(p.plan);
 }
 

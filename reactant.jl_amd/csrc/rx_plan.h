@@ -38,6 +38,11 @@ struct Plan {
   std::vector<int> result_buffers;     // per @main result: buffer id
   std::vector<TType> param_types, result_types;
   std::vector<int> aliasing_output;    // per argument: result index it may alias, or -1
+  // Counts over the live nodes of the module as written (what XLA's HloCostAnalysis reports for a module, reference
+  // deps/ReactantExtra/API.cpp:3224-3260): arithmetic operations (2 M N K per product, one per element of every other
+  // arithmetic op and of every reduced element), elements of transcendental ops, and per-op bytes read and written
+  double hlo_flops = 0, hlo_transcendentals = 0, hlo_bytes_accessed = 0, hlo_output_bytes = 0;
+  double hlo_operand_bytes[2] = {0, 0};
   std::string report() const;          // text summary for debugging
 };
 

@@ -369,3 +369,20 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     # the 32x32 MFMA shapes are a request for the ring skeleton
     monkeypatch.setenv("RX_GEMM_MFMA32", "1")
     assert "rx_gemm_body_dl<rx_mma_bf16, 256, 256, 64" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
+
+
+def test_cost_analysis_counts_of_the_module(rx):
+    """The counts behind RxExecutableCostAnalysis (the reference's cost_analysis, src/xla/Stats.jl:86-115), in the plan
+    report: sum(sin.(x) .+ y) over n elements is n additions + n reduced elements, n transcendentals, and every op reads
+    its operands and writes its result once; a product counts 2 M N K."""
+    import re
+    n = 1 << 16
+    rep = rx.compile_offline(P.sinsum_add(n))
+    m = re.search(r"module costs: flops=(\d+) transcendentals=(\d+) bytes_accessed=(\d+) output_bytes=(\d+)", rep)
+    assert m, rep
+    flops, trans, nbytes, out = map(int, m.groups())
+    assert flops == 2 * n and trans == n and out == 4
+    assert nbytes == (4 * n + 4 * n) + (8 * n + 4 * n) + (4 * n + 4 + 4)      # sine, add, reduce (operand + init + result)
+    rep = rx.compile_offline(P.gemm(64, 128, 256))
+    flops = int(re.search(r"module costs: flops=(\d+)", rep).group(1))
+    assert flops == 2 * 64 * 128 * 256 + 3 * 64 * 128                            # the product, alpha, beta, the sum

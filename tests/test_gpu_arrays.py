@@ -201,3 +201,20 @@ def test_futures_are_asked_late_or_never(rx):
         own.close()
     assert unasked.is_ready()                                              # FreeClient waited for the stream
     unasked.wait()
+
+
+def test_cost_analysis_of_an_executable(rx, client):
+    from _loader import load_programs
+    P = load_programs()
+    """XLA.cost_analysis(exec) (reference src/xla/Stats.jl:86-115): the eleven HloCostAnalysisProperties fields through the
+    C ABI, for the fused sin + add + sum and for a matrix product."""
+    n = 1 << 20
+    exe = rx.xla_compile(client, P.sinsum_add(n))
+    c = exe.cost_analysis()
+    assert c["flops"] == 2.0 * n and c["transcendentals"] == float(n)
+    assert c["operand0_bytes_accessed"] == 4.0 * n and c["operand1_bytes_accessed"] == 4.0 * n and c["output_root_bytes_accessed"] == 4.0
+    assert c["bytes_accessed"] >= 8.0 * n and 0.0 < c["utilization"] <= 1.0
+    assert c["optimal_seconds"] == pytest.approx(8.0 * n / 8.0e12, rel=0.05)      # one pass over both vectors at the HBM peak
+    exe = rx.xla_compile(client, P.gemm(512, 512, 512))
+    c = exe.cost_analysis()
+    assert c["flops"] == 2.0 * 512 ** 3 + 3.0 * 512 ** 2 and c["transcendentals"] == 0.0
