@@ -59,3 +59,16 @@ RX_CHECK_S(rx_check_s_bf16_nt, rx_el_bf16, 256, 128, 4, 2, true, true, 64)
 RX_CHECK_S(rx_check_s_bf16_nt24, rx_el_bf16, 256, 128, 2, 4, true, true, 64)
 RX_CHECK_S(rx_check_s_f16_tn, rx_el_f16, 256, 256, 2, 4, false, false, 192)
 RX_CHECK_S(rx_check_s_f16_tt, rx_el_f16, 256, 128, 4, 2, false, true, 128)
+
+// the ping-pong form of the 256x256 streaming tiles
+#define RX_CHECK_PP(NAME, EL, AKC, BKC, K)                                                                               \
+  extern "C" __global__ __launch_bounds__(512) void NAME(const EL::elem* A, const EL::elem* B, float* out) {              \
+    rx_check_epi<float, 512> epi{out};                                                                                     \
+    rx_gemm_body_pp<EL, 256, 256, 2, 4, AKC, BKC, 512, 512, K, 0, 0, false, rx_check_epi<float, 512>>(A, B, epi);           \
+  }
+RX_CHECK_PP(rx_check_pp_bf16_nn, rx_el_bf16, true, false, 512)
+RX_CHECK_PP(rx_check_pp_bf16_nt, rx_el_bf16, true, true, 128)
+RX_CHECK_PP(rx_check_pp_f16_tn, rx_el_f16, false, false, 256)
+RX_CHECK_PP(rx_check_pp_f16_tt, rx_el_f16, false, true, 256)
+RX_CHECK_PP(rx_check_pp_f8_nt, rx_el_f8, true, true, 512)
+RX_CHECK_PP(rx_check_pp_f8_tn, rx_el_f8, false, false, 256)

@@ -144,6 +144,17 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
     t << el << ", " << BM << ", " << BN << ", " << WM << ", " << WN << ", " << (a_kc ? "true" : "false") << ", " << (b_kc ? "true" : "false") << ", " << M
       << ", " << N << ", " << K << ", " << rb << ", " << cb;
     c.targs = t.str();
+    c.stype_a = el + "::elem";
+    // 16-bit operands on 256 x 256 tiles with an even number of K tiles: the ping-pong form of the same tiles
+    // (rx_gemm_body_pp: one wavefront of a SIMD multiplies a whole K tile while the other reads its fragments);
+    // RX_GEMM_PINGPONG=0 keeps the interleaved form, =1 also sends 8-bit operands there
+    const int pp = getenv("RX_GEMM_PINGPONG") ? atoi(getenv("RX_GEMM_PINGPONG")) : (esize == 2 ? 1 : 0);
+    if (pp != 0 && BM == 256 && BN == 256 && WM == 2 && WN == 4 && (K / bk) % 2 == 0 && !getenv("RX_GEMM_STREAM_STAGES") && !getenv("RX_GEMM_STREAM_DEPTH")) {
+      c.lds_bytes = (unsigned)(2 * (BM + BN) * 128);
+      c.skeleton = "rx_gemm_body_pp";
+      c.ok = true;
+      return c;
+    }
     c.skeleton = "rx_gemm_body_s";
     c.depth = 2;
     if (const char* e = getenv("RX_GEMM_STREAM_DEPTH")) {

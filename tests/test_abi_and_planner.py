@@ -350,8 +350,18 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     big = P.fp8_linear(8192, 8192, 8192)
     assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
     mlp = rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
-    assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in mlp      # the 4096^2 layer
+    # 16-bit operands on 256x256 tiles with an even number of K tiles: the ping-pong form of the same tiles
+    assert "rx_gemm_body_pp<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in mlp     # the 4096^2 layer
+    assert "rx_gemm_body_pp<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 1024" in mlp     # the first layer
     assert "rx_gemm_body_s<rx_el_bf16, 256, 128, 4, 2, true, false, 8192, 1024, 4096" in mlp      # the last layer: 256x128 tiles, wavefronts of 64x64
+    monkeypatch.setenv("RX_GEMM_PINGPONG", "0")
+    assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
+    monkeypatch.setenv("RX_GEMM_PINGPONG", "1")
+    assert "rx_gemm_body_pp<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    monkeypatch.delenv("RX_GEMM_PINGPONG")
+    # an odd number of K tiles (K = 64 * 65) stays with the interleaved form
+    odd_kt = rx.compile_offline(_dot("tensor<8192x4160xbf16>", "tensor<4160x4096xbf16>", "tensor<8192x4096xf32>", "contracting_dims = [1] x [0]"), with_source=True)
+    assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4160" in odd_kt
     monkeypatch.setenv("RX_GEMM_STREAM", "0")
     src = rx.compile_offline(big, with_source=True)
     assert "rx_gemm_body_s<" not in src and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in src

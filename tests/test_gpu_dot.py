@@ -106,6 +106,11 @@ STREAM_CASES = [
     ("bf16", "bf16", 4000, 4104, 192, False, False, 0),
     ("f16", "f16", 4008, 4100, 320, False, True, 0),
     ("f16", "f32", 2040, 2056, 256, True, False, 5),
+    # an even number of K tiles on 256x256 tiles: 16-bit operands take the ping-pong form, in every operand order
+    ("bf16", "bf16", 4000, 4104, 256, True, False, 0),
+    ("bf16", "f32", 4000, 4104, 384, False, False, 0),
+    ("f16", "f16", 4008, 4100, 768, False, True, 0),
+    ("bf16", "bf16", 2040, 2056, 128, False, True, 5),
     # 256x128 tiles (the tall products whose 256x256 tiles would not fill the chip)
     ("bf16", "bf16", 8000, 1032, 192, True, False, 0),
     ("bf16", "f32", 8000, 1028, 128, True, True, 0),
@@ -117,10 +122,12 @@ STREAM_CASES = [
 @pytest.mark.parametrize("dt,out_dt,M,N,K,a_kc,b_kc,batch", STREAM_CASES)
 def test_streaming_skeleton(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
     """8- and 16-bit operands on the eight-wavefront tiles take the skeleton that streams one operand through the 16x16
-    MFMA shapes: every operand order, batched, rows past the end of an operand (read as zero by the buffer loads), odd and
-    even tile counts along K."""
+    MFMA shapes, or its ping-pong form: every operand order, batched, rows past the end of an operand (read as zero by the
+    buffer loads), odd and even tile counts along K."""
     text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch)
-    assert "rx_gemm_body_s<" in rx.compile_offline(text, with_source=True)
+    # 16-bit operands on 256x256 tiles with an even number of K tiles: the ping-pong form of the same tiles
+    pingpong = dt != "f8E4M3FN" and N > 2000 and (K // 64) % 2 == 0
+    assert ("rx_gemm_body_pp<" if pingpong else "rx_gemm_body_s<") in rx.compile_offline(text, with_source=True)
     a = I.tensor(np.random.default_rng(5).normal(size=a_shape), dt)
     b = I.tensor(np.random.default_rng(6).normal(size=b_shape), dt)
     got, exe = gpu_run(rx, client, text, [a, b])
