@@ -321,11 +321,15 @@ def _mfma_ceiling(rx, client, entry, kind):
         return
     entry["sustained_mfma"] = {"random_operands": {"TFLOP/s": tf_r, "clock_MHz": mhz_r}, "zero_operands": {"TFLOP/s": tf_z, "clock_MHz": mhz_z},
                                "kernel_frac_of_random": entry["roofline"]["achieved"] / tf_r if tf_r else None}
-    # the config's large GEMM kernel with a clock probe inside (plain scaling epilogue, pseudo-random operands): the clock
-    # it runs at, read over a sleep of known length in the middle of the K loop, beside the ratio of the same two counters
-    # over the workgroups' lifetimes (lower: the cycle counter stands still while a compute unit has nothing to issue)
+    # the config's large GEMM kernel with a probe inside (plain scaling epilogue, pseudo-random operands, 150 ms under load
+    # before the timed launches): the ratio of the shader-cycle counter to the real-time counter over a sleep of known
+    # length in the middle of the K loop (the compute unit of the sleeping wavefront soon idles at a barrier: the chip's
+    # clock) and over the workgroups' lifetimes; for bf16 also the ping-pong body that the compiled program runs on, with
+    # the same ratio over its compute phases (MFMAs issued back to back: the clock of a compute unit whose pipes are full)
     try:
         entry["gemm_clock_probe"] = rx.gemm_clock_probe(dev, kind)
+        if kind == "bf16":
+            entry["gemm_clock_probe"]["pingpong_body"] = rx.gemm_clock_probe(dev, "bf16_pingpong")
     except Exception as e:
         entry["gemm_clock_probe"] = {"error": str(e)[:200]}
 

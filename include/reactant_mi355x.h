@@ -180,11 +180,16 @@ float RxCalibrationCopy(RxDevice *device, size_t bytes, int iters);
  * TFLOP/s and the average shader clock in MHz; returns 0, or 1 with a message (RxLastError). */
 int RxMfmaCeiling(RxDevice *device, int kind, int zero_operands, double *tflops, double *clock_mhz);
 /* No counterpart in the reference (measurement aid).  The benchmark's two large GEMM kernels (kind 0: bf16
- * 8192 x 4096 x 4096, kind 1: f8E4M3FN 8192^3) launched back to back with a clock probe inside: out5 = { us per
- * launch, TFLOP/s, cycle counter / real-time counter over the workgroups' lifetimes in MHz, the same over a sleep of
- * known length in the middle of the K loop in MHz (the clock the kernel runs at), cycles counted over that sleep
- * (65024 by the sleep instruction's definition) }. */
-int RxGemmClockProbe(RxDevice *device, int kind, double *out5);
+ * 8192 x 4096 x 4096 on the interleaved streaming body, kind 1: f8E4M3FN 8192^3, kind 2: the bf16 product on the
+ * ping-pong body that compiled programs take) launched back to back, timed once the device has been under that load
+ * for 150 ms, with a probe inside: out8 = { us per launch, TFLOP/s, cycle counter / real-time counter over the
+ * workgroups' lifetimes in MHz, [kinds 0, 1] the same over a sleep of known length that one wavefront of every 16th
+ * workgroup takes in the middle of its K loop in MHz (the rest of its workgroup soon waits at a barrier: the clock
+ * of an idle compute unit on the loaded chip), cycles counted over that sleep (65024 by the sleep instruction's
+ * definition), [kind 2] cycles counted per compute phase (64 MFMAs issued back to back by one wavefront: 1024 at
+ * the full rate), cycle counter / real-time counter over those phases in MHz (the clock of a compute unit while
+ * its MFMA pipes are full), nanoseconds per compute phase }. */
+int RxGemmClockProbe(RxDevice *device, int kind, double *out8);
 
 #ifdef __cplusplus
 }

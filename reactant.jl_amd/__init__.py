@@ -492,14 +492,22 @@ def mfma_ceiling(device, kind, zero_operands=False):
 
 
 def gemm_clock_probe(device, kind):
-    """The benchmark's large GEMM kernel of `kind` ("bf16": 8192 x 4096 x 4096, "f8": 8192^3) launched back to back with a
-    clock probe inside: dict with us per launch, TFLOP/s, the ratio of the shader-cycle counter to the real-time counter
-    over the workgroups' lifetimes (MHz), the same ratio over a sleep of known length in the middle of the K loop (MHz:
-    the clock the kernel runs at) and the cycles counted over that sleep (65024 nominal)."""
-    out = (ctypes.c_double * 5)()
-    _call("RxGemmClockProbe", device.handle, {"bf16": 0, "f8": 1}[kind], out)
-    return {"us_per_launch": out[0], "TFLOP/s": out[1], "lifetime_cycles_over_real_time_MHz": out[2], "clock_MHz": out[3],
-            "cycles_over_a_sleep_of_65024": out[4]}
+    """The benchmark's large GEMM kernel of `kind` ("bf16": 8192 x 4096 x 4096 on the interleaved streaming body, "f8":
+    8192^3, "bf16_pingpong": the bf16 product on the ping-pong body that compiled programs take) launched back to back, timed
+    once the device has been under that load for 150 ms, with a probe inside: dict with us per launch, TFLOP/s, the ratio of
+    the shader-cycle counter to the real-time counter over the workgroups' lifetimes (MHz); for "bf16" and "f8" the same
+    ratio over a sleep of known length that one wavefront takes in the middle of the K loop (MHz: its workgroup soon waits at
+    a barrier, so this is the clock of an idle compute unit on the loaded chip) and the cycles counted over that sleep (65024
+    nominal); for "bf16_pingpong" the cycles counted per compute phase (64 MFMAs issued back to back: 1024 at the full rate),
+    the same ratio over those phases (MHz: the clock of a compute unit while its MFMA pipes are full) and ns per phase."""
+    out = (ctypes.c_double * 8)()
+    _call("RxGemmClockProbe", device.handle, {"bf16": 0, "f8": 1, "bf16_pingpong": 2}[kind], out)
+    res = {"us_per_launch": out[0], "TFLOP/s": out[1], "lifetime_cycles_over_real_time_MHz": out[2]}
+    if kind == "bf16_pingpong":
+        res.update({"cycles_per_compute_phase_of_64_MFMAs": out[5], "compute_phase_cycles_over_real_time_MHz": out[6], "ns_per_compute_phase": out[7]})
+    else:
+        res.update({"clock_MHz": out[3], "cycles_over_a_sleep_of_65024": out[4]})
+    return res
 
 
 def compile_offline(mlir_text, with_source=False):

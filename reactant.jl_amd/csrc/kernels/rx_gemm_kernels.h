@@ -903,6 +903,21 @@ struct rx_clock_probe {
   }
 };
 
+// Probe of the ping-pong body (RxGemmClockProbe, kind 2): what the shader-cycle counter and the real-time counter
+// advance over the compute phases of wavefronts 0 and 4 of every workgroup -- stretches in which a wavefront issues
+// nothing but MFMAs, back to back.  cycles / phases says whether the MFMAs issue at their full rate (16 cycles each for
+// the 16 x 16 x 32 shapes), cycles / real time is the clock the compute unit runs at while its MFMA pipes are full.
+struct rx_phase_probe {
+  static constexpr bool none = false;
+  unsigned long long* out;   // per workgroup and group: [0] cycles, [1] real-time ticks, [2] phases
+  unsigned long long c = 0, t = 0, c0 = 0, t0 = 0, n = 0;
+  RX_MEM void begin() { c0 = __builtin_readcyclecounter(); t0 = __builtin_amdgcn_s_memrealtime(); }
+  RX_MEM void end() { c += __builtin_readcyclecounter() - c0; t += __builtin_amdgcn_s_memrealtime() - t0; ++n; }
+  RX_MEM void flush(int wave, int lane) const {
+    if ((wave & 3) == 0 && lane == 0) { unsigned long long* o = out + (blockIdx.x * 2 + (wave >> 2)) * 3; o[0] = c; o[1] = t; o[2] = n; }
+  }
+};
+
 template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2, class Probe = rx_no_fn>
 RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, const Probe& probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
@@ -1087,8 +1102,8 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 // bf16 8192 x 4096 x 4096 with bias + GELU 199.7 -> 190.0 us, K = 1024: 65.6 -> 64.6 us; for e4m3 8192^3 it gains
 // nothing (both operands [row][k]: its memory phase is as long as its compute phase), so only 16-bit operands take it.
 // ---------------------------------------------------------------------------
-template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi>
-RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi) {
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, class Probe = rx_no_fn>
+RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, Probe probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NSTG = 2;
   constexpr int NTL = 256;                                   // threads that request
@@ -1157,6 +1172,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
   };
   auto fragments_in = [&]() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); };
   auto multiply = [&]() {
+    if constexpr (!Probe::none) probe.begin();
     __builtin_amdgcn_s_setprio(1);
     rx_static_for<0, NA>([&](auto I) {
       constexpr int i = decltype(I)::value;
@@ -1164,6 +1180,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
       rx_static_for<0, NB>([&](auto J) { EL::mma(acc[i][decltype(J)::value], fb[decltype(J)::value], fa[i]); });
     });
     __builtin_amdgcn_s_setprio(0);
+    if constexpr (!Probe::none) { __builtin_amdgcn_sched_barrier(0); probe.end(); }
   };
 
   if (grp == 0) {
@@ -1219,6 +1236,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
     step(rx_int<1>{}, rx_int<1>{});
   }
   RX_SCHED_FENCE();
+  if constexpr (!Probe::none) probe.flush(wave, lane);
 
 #pragma unroll
   for (int i = 0; i < NA; ++i) {

@@ -431,7 +431,11 @@ __global__ __launch_bounds__(512) void rx_gemm_clock_probe(const void* __restric
                                                            unsigned long long* __restrict__ sleep_ticks, unsigned long long* __restrict__ life_ticks) {
   const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
   rx_clock_probe probe{sleep_ticks};
-  if constexpr (KIND == 0) {
+  if constexpr (KIND == 2) {
+    // the bf16 layer on the ping-pong body, as the planner instantiates it: sleep_ticks takes the phase probe's figures
+    rx_probe_epi epi{out, 4096};
+    rx_gemm_body_pp<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096, 4, 8, false, rx_probe_epi, rx_phase_probe>((const rx_u16*)A, (const rx_u16*)B, epi, rx_phase_probe{sleep_ticks});
+  } else if constexpr (KIND == 0) {
     rx_probe_epi epi{out, 4096};
     rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096, 4, 8, false, rx_probe_epi, 2, 2, rx_clock_probe>((const rx_u16*)A, (const rx_u16*)B, epi, probe);
   } else {
@@ -1221,27 +1225,38 @@ RX_EXPORT int RxMfmaCeiling(RxDevice* d, int kind, int zero_operands, double* tf
   }, 1);
 }
 
-RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out5) {
+RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out8) {
   return guarded([&]() -> int {
     check_device(d);
-    if (kind != 0 && kind != 1) throw Error("INVALID_ARGUMENT: kind is 0 (bf16 8192 x 4096 x 4096) or 1 (f8E4M3FN 8192^3)");
-    if (!out5) throw Error("INVALID_ARGUMENT: null result array");
+    if (kind < 0 || kind > 2) throw Error("INVALID_ARGUMENT: kind is 0 (bf16 8192 x 4096 x 4096), 1 (f8E4M3FN 8192^3) or 2 (the bf16 product on the ping-pong body)");
+    if (!out8) throw Error("INVALID_ARGUMENT: null result array");
     HIP_CHECK(hipSetDevice(d->ordinal));
-    const size_t M = 8192, N = kind == 0 ? 4096 : 8192, K = kind == 0 ? 4096 : 8192, esz = kind == 0 ? 2 : 1;
+    const size_t M = 8192, N = kind == 1 ? 8192 : 4096, K = kind == 1 ? 8192 : 4096, esz = kind == 1 ? 1 : 2;
     const unsigned grid = (unsigned)rx::gemm_grid((int64_t)(M / 256), (int64_t)(N / 256), 4, 8);
-    Allocation a(d, M * K * esz), b(d, N * K * esz), o(d, M * N * 2), sl(d, grid * 16), lf(d, grid * 16);
-    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, a.ptr, M * K, kind == 0 ? 0 : 2, 1u);
-    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, b.ptr, N * K, kind == 0 ? 1 : 2, 77u);
-    HIP_CHECK(hipMemsetAsync(sl.ptr, 0, grid * 16, d->stream));
+    Allocation a(d, M * K * esz), b(d, N * K * esz), o(d, M * N * 2), sl(d, grid * 48), lf(d, grid * 16);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, a.ptr, M * K, kind == 1 ? 2 : 0, 1u);
+    hipLaunchKernelGGL(rx_probe_fill, dim3(4096), dim3(256), 0, d->stream, b.ptr, N * K, kind == 1 ? 2 : 1, 77u);
+    HIP_CHECK(hipMemsetAsync(sl.ptr, 0, grid * 48, d->stream));
     HIP_CHECK(hipMemsetAsync(lf.ptr, 0, grid * 16, d->stream));
     const int lds = 2 * 512 * 128;
-    auto fn = kind == 0 ? rx_gemm_clock_probe<0> : rx_gemm_clock_probe<1>;
+    auto fn = kind == 0 ? rx_gemm_clock_probe<0> : (kind == 1 ? rx_gemm_clock_probe<1> : rx_gemm_clock_probe<2>);
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     hipEvent_t e0, e1;
     HIP_CHECK(hipEventCreate(&e0));
     HIP_CHECK(hipEventCreate(&e1));
-    const int warm = 5, reps = 20;   // back to back, so that the clock has settled under the power limit
-    for (int i = 0; i < warm; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
+    // Back to back, and not timed before the device has been under this load for 150 ms: after an idle period the first
+    // 20 ms or so of a load run up to 20 % slower (8192 x 4096 x 4096 bf16: 246 us per launch 5 ms after the start,
+    // 201 us from 22 ms on), whatever the kernel.
+    const int reps = 20;
+    HIP_CHECK(hipEventRecord(e0, d->stream));
+    for (;;) {
+      for (int i = 0; i < 20; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
+      HIP_CHECK(hipEventRecord(e1, d->stream));
+      HIP_CHECK(hipEventSynchronize(e1));
+      float warm_ms = 0;
+      HIP_CHECK(hipEventElapsedTime(&warm_ms, e0, e1));
+      if (warm_ms >= 150.f) break;
+    }
     HIP_CHECK(hipEventRecord(e0, d->stream));
     for (int i = 0; i < reps; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
     HIP_CHECK(hipEventRecord(e1, d->stream));
@@ -1250,21 +1265,26 @@ RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out5) {
     HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    std::vector<unsigned long long> hs(grid * 2), hl(grid * 2);
-    HIP_CHECK(hipMemcpy(hs.data(), sl.ptr, grid * 16, hipMemcpyDeviceToHost));
+    std::vector<unsigned long long> hs(grid * 6), hl(grid * 2);
+    HIP_CHECK(hipMemcpy(hs.data(), sl.ptr, grid * 48, hipMemcpyDeviceToHost));
     HIP_CHECK(hipMemcpy(hl.data(), lf.ptr, grid * 16, hipMemcpyDeviceToHost));
     double sc = 0, sr = 0, lc = 0, lr = 0;
     int ns = 0;
+    double pc = 0, pr = 0, pn = 0;
     for (unsigned w = 0; w < grid; ++w) {
-      if (hs[2 * w + 1]) { sc += (double)hs[2 * w]; sr += (double)hs[2 * w + 1]; ++ns; }
+      if (kind == 2) { for (int g = 0; g < 2; ++g) { pc += (double)hs[(2 * w + g) * 3]; pr += (double)hs[(2 * w + g) * 3 + 1]; pn += (double)hs[(2 * w + g) * 3 + 2]; } }
+      else if (hs[2 * w + 1]) { sc += (double)hs[2 * w]; sr += (double)hs[2 * w + 1]; ++ns; }
       lc += (double)hl[2 * w]; lr += (double)hl[2 * w + 1];
     }
     const double us = ms * 1e3 / reps;
-    out5[0] = us;                                                   // per launch; the sleeping wavefronts lengthen it by a few per cent
-    out5[1] = 2.0 * M * N * K / (us * 1e-6) / 1e12;                 // TFLOP/s
-    out5[2] = lr > 0 ? lc / lr * 100.0 : 0.0;                       // cycle counter / real time over the workgroups' lifetimes, MHz
-    out5[3] = sr > 0 ? sc / sr * 100.0 : 0.0;                       // the same over the sleeps: the clock, MHz
-    out5[4] = ns > 0 ? sc / ns : 0.0;                               // cycles counted over a sleep of 65024 nominal cycles
+    out8[0] = us;                                                   // per launch; the sleeping wavefronts lengthen it by a few per cent
+    out8[1] = 2.0 * M * N * K / (us * 1e-6) / 1e12;                 // TFLOP/s
+    out8[2] = lr > 0 ? lc / lr * 100.0 : 0.0;                       // cycle counter / real time over the workgroups' lifetimes, MHz
+    out8[3] = sr > 0 ? sc / sr * 100.0 : 0.0;                       // the same over the sleeps, MHz (kinds 0 and 1)
+    out8[4] = ns > 0 ? sc / ns : 0.0;                               // cycles counted over a sleep of 65024 nominal cycles
+    out8[5] = pn > 0 ? pc / pn : 0.0;                               // kind 2: cycles per compute phase of 64 MFMAs issued back to back
+    out8[6] = pr > 0 ? pc / pr * 100.0 : 0.0;                       // kind 2: cycle counter / real time over those phases, MHz
+    out8[7] = pn > 0 ? pr / pn * 10.0 : 0.0;                        // kind 2: nanoseconds per compute phase
     return 0;
   }, 1);
 }
