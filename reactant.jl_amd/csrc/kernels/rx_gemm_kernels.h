@@ -1091,31 +1091,39 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 // apart: in its memory phase a wavefront reads all its fragments of one K tile from LDS (8 of A, 4 of B: 96
 // registers), in its compute phase it issues that tile's 64 (16-bit) or 32 (8-bit) MFMAs back to back at raised
 // priority, with nothing in between that could wait for memory, while the other wavefront of the SIMD is in its
-// memory phase.  Two barriers per K tile keep the phases apart.  Wavefronts 0-3 request every operand tile (256
-// threads cover it), their requests spread between the LDS reads of their memory phase, where a request that has to
-// wait for the load path delays no MFMA; wavefronts 4-7 never request.
-//   interval 2t:   group 0 reads tile t (stage t % 2) and requests tile t + 1 into the other stage, group 1 multiplies tile t - 1
-//   interval 2t+1: group 0 multiplies tile t and then waits for tile t + 1 to land,              group 1 reads tile t
+// memory phase.  Two barriers per K tile keep the phases apart.  Requests go out in memory phases only, between the
+// LDS reads, where a request that has to wait for the load path delays no MFMA.
+//   interval 2t:   group 0 (wavefronts 0-3) reads tile t (stage t % 2) and requests tile t + 1 into the other stage,
+//                  group 1 multiplies tile t - 1
+//   interval 2t+1: group 0 multiplies tile t and then waits for tile t + 1 to land, group 1 reads tile t
 // The stage of tile t - 1 is free when interval 2t begins (group 1 read it in interval 2t - 1), and tile t + 1 is first
-// read in interval 2t + 2.
+// read in interval 2t + 2.  With B stored [k][n] group 0 requests both operands (256 threads cover a tile).  With B
+// stored [n][k] a wavefront's request fills eight whole rows of the LDS tile, and rows 64 wn .. 64 wn + 63 of B are
+// read by wavefronts wn and wn + 4 alone: group 0 requests A only, and every wavefront of group 1 requests its 64 rows
+// of B of tile t + 2 in its own memory phase of tile t, into the stage it is reading, once its B fragments have
+// arrived (wavefront wn read them an interval earlier); that halves the requests of group 0, whose memory phase is
+// otherwise as long as a compute phase for 8-bit operands.
 // Measured after 150 ms under load (the first 20 ms after an idle period run up to 20 % slower, whatever the kernel):
-// bf16 8192 x 4096 x 4096 with bias + GELU 199.7 -> 190.0 us, K = 1024: 65.6 -> 64.6 us; for e4m3 8192^3 it gains
-// nothing (both operands [row][k]: its memory phase is as long as its compute phase), so only 16-bit operands take it.
+// bf16 8192 x 4096 x 4096 [m][k] x [k][n] with bias + GELU 199.7 -> 190.0 us, K = 1024: 65.6 -> 64.6 us; e4m3 8192^3
+// [m][k] x [n][k] 386 -> 360 us (with group 0 requesting both operands: 411).
 // ---------------------------------------------------------------------------
 template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, class Probe = rx_no_fn>
 RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, Probe probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NSTG = 2;
-  constexpr int NTL = 256;                                   // threads that request
+  constexpr int NTL = 256;                                   // threads of group 0
   constexpr int NA = BM / WM / 16, NB = BN / WN / 16;
   constexpr int A_ROWS = A_KC ? BM : BK, A_COLS = A_KC ? BKB : BM * ESZ;
   constexpr int B_ROWS = B_KC ? BN : BK, B_COLS = B_KC ? BKB : BN * ESZ;
   constexpr int A_SZ = BM * BKB, B_SZ = BN * BKB;
+  constexpr int BSL = BN / WN;                               // rows of B that one wavefront column reads
   typedef rx_dma_s<EL, A_ROWS, A_COLS, NTL, A_KC> DMA_A;
-  typedef rx_dma_s<EL, B_ROWS, B_COLS, NTL, B_KC> DMA_B;
-  constexpr int NLT = DMA_A::NL + DMA_B::NL;                 // requests per requesting thread and K tile
+  typedef rx_dma_s<EL, B_ROWS, B_COLS, NTL, B_KC> DMA_B;     // B requested by group 0 ([k][n])
+  constexpr int NLA = DMA_A::NL;
+  constexpr int NLB = B_KC ? BSL * 8 / 64 : DMA_B::NL;       // [n][k]: a wavefront's request covers 8 rows of 128 bytes
+  constexpr int NL0 = B_KC ? NLA : NLA + NLB;                // requests per thread of group 0 and K tile
   constexpr int NFR = NA + NB;                               // fragments per wavefront and K tile
-  static_assert(WM * WN == 8, "two wavefronts per SIMD");
+  static_assert(WM == 2 && WN == 4, "wavefronts w and w + 4 share a SIMD and a column of B");
   static_assert((long long)M * K * ESZ < (1ll << 32) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
   constexpr int KT = K / BK;
   static_assert(K % BK == 0 && KT >= 2 && KT % 2 == 0, "an even number of whole K tiles");
@@ -1142,24 +1150,52 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
   DMA_A dma_a;
   DMA_B dma_b;
   dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * K * ESZ), tid & (NTL - 1));
-  dma_b.init(B + batch * (long long)N * K, B_GLDB, B_KC ? n0 : n0 * ESZ, (unsigned)((long long)N * K * ESZ), tid & (NTL - 1));
+  // [n][k]: slot `lane` of a wavefront's request q is row 8 q + lane / 8 of its rows, position lane % 8, and the swizzle
+  // puts chunk c of row r at position c ^ ((r / 2) & 7): for odd q (row bit 3 set) bit 2 of the chunk flips
+  unsigned slab0 = 0, slab1 = 0;
+  if constexpr (B_KC) {
+    dma_b.rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(B + batch * (long long)N * K), 0, (unsigned)((long long)N * K * ESZ), 0x00020000);
+    slab0 = (unsigned)(n0 + wn * BSL + (lane >> 3)) * B_GLDB + (unsigned)(((lane & 7) ^ (lane >> 4)) * 16);
+    slab1 = slab0 ^ 64u;
+  } else {
+    dma_b.init(B + batch * (long long)N * K, B_GLDB, n0 * ESZ, (unsigned)((long long)N * K * ESZ), tid & (NTL - 1));
+  }
   rx_i32x8 fa[NA], fb[NB];
-  // request q of a tile: those of A first (st and q are constants at every call)
+  // request q of a tile by group 0: those of A first (st and q are constants at every call)
   auto request = [&](int kt, int st, int q) __attribute__((always_inline)) {
-    if (q < DMA_A::NL) dma_a.one(q, (unsigned)kt * KA, ldsa + st * A_SZ, wave);
-    else dma_b.one(q - DMA_A::NL, (unsigned)kt * KB, ldsb + st * B_SZ, wave);
+    if (q < NLA) dma_a.one(q, (unsigned)kt * KA, ldsa + st * A_SZ, wave);
+    else if constexpr (!B_KC) dma_b.one(q - NLA, (unsigned)kt * KB, ldsb + st * B_SZ, wave);
   };
+  // request q of this wavefront's rows of B ([n][k])
+  auto request_rows = [&](int kt, int st, int q) __attribute__((always_inline)) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(dma_b.rsrc, (RX_LDS void*)(ldsb + st * B_SZ + wn * BSL * BKB + q * 1024), 16, (q & 1) ? slab1 : slab0,
+                                             (unsigned)kt * KB + (unsigned)q * 8u * B_GLDB, 0, 0);
+  };
+  // [row][k] fragments (what rx_frag_s::kc reads) from two addresses per lane and operand: its row within a block of 16
+  // and its two chunks, which the swizzle keeps 64 bytes apart; stage and block fold into the instruction's offset
+  const unsigned lane_off = (unsigned)(lane & 15) * 128u + (unsigned)(((lane >> 4) ^ ((lane & 15) >> 1)) * 16);
+  RX_LDS rx_u8* const pa0 = ldsa + (unsigned)(wm * (BM / WM)) * 128u + lane_off;
+  RX_LDS rx_u8* const pa1 = ldsa + (unsigned)(wm * (BM / WM)) * 128u + (lane_off ^ 64u);
+  RX_LDS rx_u8* const pb0 = ldsb + (unsigned)(wn * BSL) * 128u + lane_off;
+  RX_LDS rx_u8* const pb1 = ldsb + (unsigned)(wn * BSL) * 128u + (lane_off ^ 64u);
   // fragment f of a tile: those of B first
   auto read = [&](auto ST, auto F) {
     constexpr int st = decltype(ST)::value, f = decltype(F)::value;
     if constexpr (f < NB) {
-      const int o = wn * (BN / WN) + 16 * f;
-      if constexpr (B_KC) fb[f] = rx_frag_s<EL>::template kc<B_COLS>(ldsb + st * B_SZ, o, lane);
-      else fb[f] = rx_frag_s<EL>::template tr<B_COLS>(ldsb + st * B_SZ, o, lane);
+      if constexpr (B_KC) {
+        struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(pb0 + (st * B_SZ + f * 2048)), *(const RX_LDS rx_i32x4*)(pb1 + (st * B_SZ + f * 2048))};
+        fb[f] = __builtin_bit_cast(rx_i32x8, both);
+      } else {
+        fb[f] = rx_frag_s<EL>::template tr<B_COLS>(ldsb + st * B_SZ, wn * BSL + 16 * f, lane);
+      }
     } else {
-      const int o = wm * (BM / WM) + 16 * (f - NB);
-      if constexpr (A_KC) fa[f - NB] = rx_frag_s<EL>::template kc<A_COLS>(ldsa + st * A_SZ, o, lane);
-      else fa[f - NB] = rx_frag_s<EL>::template tr<A_COLS>(ldsa + st * A_SZ, o, lane);
+      constexpr int i = f - NB;
+      if constexpr (A_KC) {
+        struct { rx_i32x4 a, b; } both = {*(const RX_LDS rx_i32x4*)(pa0 + (st * A_SZ + i * 2048)), *(const RX_LDS rx_i32x4*)(pa1 + (st * A_SZ + i * 2048))};
+        fa[i] = __builtin_bit_cast(rx_i32x8, both);
+      } else {
+        fa[i] = rx_frag_s<EL>::template tr<A_COLS>(ldsa + st * A_SZ, wm * (BM / WM) + 16 * i, lane);
+      }
     }
   };
   // end of a phase: nothing moves across it, neither in the compiler's schedule nor at run time
@@ -1185,8 +1221,15 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
 
   if (grp == 0) {
 #pragma unroll
-    for (int q = 0; q < NLT; ++q) request(0, 0, q);
+    for (int q = 0; q < NL0; ++q) request(0, 0, q);
     rx_wait_vmcnt<0>();
+  } else if constexpr (B_KC) {
+    // its rows of B of tiles 0 and 1: group 1 requests two tiles ahead
+#pragma unroll
+    for (int q = 0; q < NLB; ++q) request_rows(0, 0, q);
+#pragma unroll
+    for (int q = 0; q < NLB; ++q) request_rows(1, 1, q);
+    rx_wait_vmcnt<NLB>();
   }
   phase_end();                 // tile 0 is in LDS
   if (grp == 1) phase_end();   // group 1 runs one interval behind
@@ -1196,10 +1239,10 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
     auto step = [&](auto UU, auto REQ, int k) {
       constexpr int u = decltype(UU)::value;
       if constexpr (decltype(REQ)::value != 0) {
-        rx_static_for<0, NLT>([&](auto Q) {
+        rx_static_for<0, NL0>([&](auto Q) {
           constexpr int q = decltype(Q)::value;
           request(k + 1, (u + 1) % 2, q);
-          rx_static_for<q * NFR / NLT, (q + 1) * NFR / NLT>([&](auto F) { read(rx_int<u>{}, F); });
+          rx_static_for<q * NFR / NL0, (q + 1) * NFR / NL0>([&](auto F) { read(rx_int<u>{}, F); });
           __builtin_amdgcn_sched_barrier(0);
         });
       } else {
@@ -1209,7 +1252,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
       phase_end();
       multiply();
       __builtin_amdgcn_sched_barrier(0);
-      rx_wait_vmcnt<0>();      // tile k + 1 has landed
+      rx_wait_vmcnt<0>();      // what this group requested of tile k + 1 has landed
       phase_end();
     };
     for (int kt = 0; kt < KT - 2; kt += 2) {
@@ -1219,21 +1262,37 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
     step(rx_int<0>{}, rx_int<1>{}, KT - 2);
     step(rx_int<1>{}, rx_int<0>{}, KT - 1);
   } else {
-    auto step = [&](auto UU, auto LAST) {
+    // REQ: tile k + 2 exists ([n][k] only); LAST: group 0 has left the loop, its last barrier was the one in this step
+    auto step = [&](auto UU, auto REQ, auto LAST, int k) {
       constexpr int u = decltype(UU)::value;
-      rx_static_for<0, NFR>([&](auto F) { read(rx_int<u>{}, F); });
+      constexpr bool req = B_KC && decltype(REQ)::value != 0;
+      rx_static_for<0, NB>([&](auto F) { read(rx_int<u>{}, F); });
+      if constexpr (req) {
+        fragments_in();        // this wavefront's B fragments of tile k are in registers: its rows of the stage are free
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      rx_static_for<0, NA>([&](auto I) {
+        constexpr int i = decltype(I)::value;
+        if constexpr (req) {
+#pragma unroll
+          for (int q = i * NLB / NA; q < (i + 1) * NLB / NA; ++q) request_rows(k + 2, u, q);
+        }
+        read(rx_int<u>{}, rx_int<NB + i>{});
+        if constexpr (req) __builtin_amdgcn_sched_barrier(0);
+      });
       fragments_in();
+      // its rows of B of tile k + 1, requested a K tile ago, have landed; the requests just made may still be under way
+      if constexpr (B_KC) { if constexpr (req) rx_wait_vmcnt<NLB>(); else rx_wait_vmcnt<0>(); }
       phase_end();
       multiply();
-      // group 0 has left the loop by then: its last barrier was the one above
       if constexpr (decltype(LAST)::value == 0) phase_end();
     };
     for (int kt = 0; kt < KT - 2; kt += 2) {
-      step(rx_int<0>{}, rx_int<0>{});
-      step(rx_int<1>{}, rx_int<0>{});
+      step(rx_int<0>{}, rx_int<1>{}, rx_int<0>{}, kt);
+      step(rx_int<1>{}, rx_int<1>{}, rx_int<0>{}, kt + 1);
     }
-    step(rx_int<0>{}, rx_int<0>{});
-    step(rx_int<1>{}, rx_int<1>{});
+    step(rx_int<0>{}, rx_int<0>{}, rx_int<0>{}, KT - 2);
+    step(rx_int<1>{}, rx_int<0>{}, rx_int<1>{}, KT - 1);
   }
   RX_SCHED_FENCE();
   if constexpr (!Probe::none) probe.flush(wave, lane);

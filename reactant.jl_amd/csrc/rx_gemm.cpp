@@ -145,10 +145,12 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
       << ", " << N << ", " << K << ", " << rb << ", " << cb;
     c.targs = t.str();
     c.stype_a = el + "::elem";
-    // 16-bit operands on 256 x 256 tiles with an even number of K tiles: the ping-pong form of the same tiles
-    // (rx_gemm_body_pp: one wavefront of a SIMD multiplies a whole K tile while the other reads its fragments);
-    // RX_GEMM_PINGPONG=0 keeps the interleaved form, =1 also sends 8-bit operands there
-    const int pp = getenv("RX_GEMM_PINGPONG") ? atoi(getenv("RX_GEMM_PINGPONG")) : (esize == 2 ? 1 : 0);
+    // 256 x 256 tiles with an even number of K tiles: the ping-pong form of the same tiles (rx_gemm_body_pp: one
+    // wavefront of a SIMD multiplies a whole K tile while the other reads its fragments) for 16-bit operands, and for
+    // 8-bit operands when B is stored [n][k] (then the requests are shared between the two groups of wavefronts; with
+    // one group requesting everything the 8-bit form is slower than the interleaved one).  RX_GEMM_PINGPONG=0 keeps
+    // the interleaved form, =1 takes the ping-pong form wherever it exists.
+    const int pp = getenv("RX_GEMM_PINGPONG") ? atoi(getenv("RX_GEMM_PINGPONG")) : ((esize == 2 || b_kc) ? 1 : 0);
     if (pp != 0 && BM == 256 && BN == 256 && WM == 2 && WN == 4 && (K / bk) % 2 == 0 && !getenv("RX_GEMM_STREAM_STAGES") && !getenv("RX_GEMM_STREAM_DEPTH")) {
       c.lds_bytes = (unsigned)(2 * (BM + BN) * 128);
       c.skeleton = "rx_gemm_body_pp";

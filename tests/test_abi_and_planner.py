@@ -348,7 +348,9 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     # 8- and 16-bit operands on eight-wavefront tiles with whole K tiles of 128 bytes: the 16x16 MFMA skeleton that streams
     # one operand (with_source shows the call)
     big = P.fp8_linear(8192, 8192, 8192)
-    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    # 256x256 tiles, an even number of K tiles, B stored [n][k]: the ping-pong form of those tiles; B stored [k][n]: the interleaved form
+    assert "rx_gemm_body_pp<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, false, 8192, 8192, 8192" in rx.compile_offline(P.fp8_linear(8192, 8192, 8192, weight_layout="kn"), with_source=True)
     mlp = rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
     # 16-bit operands on 256x256 tiles with an even number of K tiles: the ping-pong form of the same tiles
     assert "rx_gemm_body_pp<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in mlp     # the 4096^2 layer
@@ -356,8 +358,9 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     assert "rx_gemm_body_s<rx_el_bf16, 256, 128, 4, 2, true, false, 8192, 1024, 4096" in mlp      # the last layer: 256x128 tiles, wavefronts of 64x64
     monkeypatch.setenv("RX_GEMM_PINGPONG", "0")
     assert "rx_gemm_body_s<rx_el_bf16, 256, 256, 2, 4, true, false, 8192, 4096, 4096" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)
+    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
     monkeypatch.setenv("RX_GEMM_PINGPONG", "1")
-    assert "rx_gemm_body_pp<rx_el_f8, 256, 256, 2, 4, true, true, 8192, 8192, 8192" in rx.compile_offline(big, with_source=True)
+    assert "rx_gemm_body_pp<rx_el_f8, 256, 256, 2, 4, true, false, 8192, 8192, 8192" in rx.compile_offline(P.fp8_linear(8192, 8192, 8192, weight_layout="kn"), with_source=True)
     monkeypatch.delenv("RX_GEMM_PINGPONG")
     # an odd number of K tiles (K = 64 * 65) stays with the interleaved form
     odd_kt = rx.compile_offline(_dot("tensor<8192x4160xbf16>", "tensor<4160x4096xbf16>", "tensor<8192x4096xf32>", "contracting_dims = [1] x [0]"), with_source=True)
@@ -375,7 +378,7 @@ def test_gemm_takes_the_streaming_skeleton_where_it_fits(monkeypatch):
     assert "rx_gemm_body_s<" not in huge and "rx_gemm_body_dl<rx_mma_f8, 256, 256, 128" in huge
     below = rx.compile_offline(_dot("tensor<32768x65536xf8E4M3FN>", "tensor<8192x65536xf8E4M3FN>", "tensor<32768x8192xf32>", "contracting_dims = [1] x [1]"),
                                with_source=True)
-    assert "rx_gemm_body_s<rx_el_f8, 256, 256, 2, 4, true, true, 32768, 8192, 65536" in below
+    assert "rx_gemm_body_pp<rx_el_f8, 256, 256, 2, 4, true, true, 32768, 8192, 65536" in below
     # the 32x32 MFMA shapes are a request for the ring skeleton
     monkeypatch.setenv("RX_GEMM_MFMA32", "1")
     assert "rx_gemm_body_dl<rx_mma_bf16, 256, 256, 64" in rx.compile_offline(P.mlp(8192, [1024, 4096, 4096, 1024]), with_source=True)

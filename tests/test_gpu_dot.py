@@ -101,6 +101,8 @@ STREAM_CASES = [
     ("f8E4M3FN", "bf16", 4016, 4100, 640, False, True, 0),
     ("f8E4M3FN", "f32", 2048, 2064, 512, True, True, 4),
     ("f8E4M3FN", "bf16", 2040, 2064, 256, True, False, 5),
+    ("f8E4M3FN", "bf16", 4000, 4112, 512, True, True, 0),
+    ("f8E4M3FN", "f32", 4016, 4100, 256, False, True, 0),
     ("bf16", "bf16", 4000, 4104, 64, True, False, 0),
     ("bf16", "f32", 4000, 4104, 128, True, True, 0),
     ("bf16", "bf16", 4000, 4104, 192, False, False, 0),
@@ -125,8 +127,8 @@ def test_streaming_skeleton(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
     MFMA shapes, or its ping-pong form: every operand order, batched, rows past the end of an operand (read as zero by the
     buffer loads), odd and even tile counts along K."""
     text, a_shape, b_shape = dot_module(M, N, K, dt, out_dt, a_kc, b_kc, batch)
-    # 16-bit operands on 256x256 tiles with an even number of K tiles: the ping-pong form of the same tiles
-    pingpong = dt != "f8E4M3FN" and N > 2000 and (K // 64) % 2 == 0
+    # 256x256 tiles with an even number of K tiles: the ping-pong form of the same tiles (8-bit operands: when B is [n][k])
+    pingpong = N > 2000 and (K * (1 if dt == "f8E4M3FN" else 2) // 128) % 2 == 0 and (dt != "f8E4M3FN" or b_kc)
     assert ("rx_gemm_body_pp<" if pingpong else "rx_gemm_body_s<") in rx.compile_offline(text, with_source=True)
     a = I.tensor(np.random.default_rng(5).normal(size=a_shape), dt)
     b = I.tensor(np.random.default_rng(6).normal(size=b_shape), dt)
