@@ -1,6 +1,6 @@
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload stencil] [--no-others] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms 150] [--workload stencil] [--no-others] [--no-cpu]
 
 Prints ONE JSON line.  The headline workload is the 3-D diffusion/advection stencil,
 Float64 512x512x256 with 3-cell halos, 10 timesteps traced into one module.  A "step" is one execution of that module (10 timesteps)
@@ -17,6 +17,9 @@ on every launch is reported beside it.  Every workload's result is verified afte
 the stencil bit for bit against the C restatement, the others on sampled rows against float64 / the numpy oracle.
 `roofline.traffic` is read from profiles/bench_all_configs_hbm_traffic.txt (rocprofv3 counters) and is null when the
 kernel name or launch size there does not match this run's launch list.
+Before the W warm-up steps of a workload come untimed executions of it until the device has been under that load for
+`--settle-ms` milliseconds (`load_before_warmup_ms` in the line): after an idle period -- compilation, a host-side check, a
+CPU baseline -- the first 20 ms or so of a load run up to 20 % slower on this part, whatever the kernel.
 `--workload conv|cumsum|maxpool|colsum|transpose` run one of the windowed / layout ops instead, `--workload polybench` /
 `polybench_linalg` the reference's polybench stencil and linear-algebra suites (never part of `others`).
 """
@@ -40,7 +43,7 @@ if ROOT not in sys.path:
 # of this run's launch list; otherwise `traffic` is null.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "bench_all_configs_hbm_traffic.txt")
 _FULL_SIZE = [True]   # cleared by --small
-OPTS = {"check": True, "cpu": True}
+OPTS = {"check": True, "cpu": True, "settle_ms": 150.0}
 
 
 def _traffic_table():
@@ -112,6 +115,13 @@ def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
     Returns (seconds for the timed steps, per-launch mean ms over the timed steps, last results)."""
     dev = client.default_device()
     res = None
+    # untimed executions until the device has been under this workload for OPTS["settle_ms"] (see _settle), then the W warm-up steps
+    t_load = time.perf_counter()
+    while OPTS["settle_ms"] > 0 and (time.perf_counter() - t_load) * 1e3 < OPTS["settle_ms"]:
+        for _ in range(10):
+            bufs, don = make_args(res)
+            res = exe.execute_profiled(bufs, don)
+        dev.synchronize()
     for _ in range(warmup):
         bufs, don = make_args(res)
         res = exe.execute_profiled(bufs, don)
@@ -128,12 +138,25 @@ def _time_steps(rx, client, exe, make_args, steps, warmup, carry=None):
     return t1 - t0, np.asarray(mean_ms), res
 
 
+def _settle(dev, run_one):
+    """Untimed executions until the device has been under the workload for OPTS["settle_ms"] milliseconds.  After an idle
+    period (compilation, a host-side check, the CPU baseline of the previous workload) the first 20 ms or so of a load run
+    up to 20 % slower on this part, whatever the kernel (a bf16 8192 x 4096 x 4096 product: 246 us per launch 5 ms after the
+    start, 201 us from 22 ms on); five warm-up steps of 0.3 ms end inside that window."""
+    t0 = time.perf_counter()
+    while OPTS["settle_ms"] > 0 and (time.perf_counter() - t0) * 1e3 < OPTS["settle_ms"]:
+        for _ in range(10):
+            run_one()
+        dev.synchronize()
+
+
 def _time_plain(client, exe, bufs, steps, warmup):
     """K steps as a caller runs them: queued without waiting, no event pair on the launches (a pair
     costs a few microseconds of stream time, which shows on steps of less than 0.1 ms).  The K steps are run five
     times, each run queued whole and timed by the host clock around a synchronization (whose wake-up, some tens of
     microseconds, is spread over the K steps of a run); returns the median of the runs' seconds per step."""
     dev = client.default_device()
+    _settle(dev, lambda: exe.execute_sharded(bufs))
     for _ in range(warmup):
         exe.execute_sharded(bufs)
     dev.synchronize()
@@ -673,6 +696,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
+    ap.add_argument("--settle-ms", type=float, default=150.0, help="untimed executions of a workload before its warm-up steps until the device has been under that load this long (0: none)")
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--no-check", action="store_true", help="skip the verification of the results after the timed regions (profiling runs)")
@@ -691,13 +715,14 @@ def main():
              "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
              "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "colsum": dict(n=1024), "transpose": dict(n=1024), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
-    OPTS["check"], OPTS["cpu"] = not args.no_check, not args.no_cpu
+    OPTS["check"], OPTS["cpu"], OPTS["settle_ms"] = not args.no_check, not args.no_cpu, args.settle_ms
     kw = small[args.workload] if args.small else {}
     main_res = table[args.workload](rx, client, P, args.steps, args.warmup, **kw)
     copy_ms = rx._call("RxCalibrationCopy", client.default_device().handle, 1 << 30, 10)
     out = {
         "metric": "achieved HBM GB/s (map/reduce/stencil) + dot_general TFLOP/s, % of peak, 1 GPU",
         "value": main_res["value"], "unit": main_res["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "load_before_warmup_ms": args.settle_ms,
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": main_res.get("higher_is_better", True), "scaling": "weak", "vs_baseline": None,
         "dtype": main_res["dtype"], "data": "synthetic", "config": {"workload": main_res["workload"]},
         "roofline": main_res["roofline"],
