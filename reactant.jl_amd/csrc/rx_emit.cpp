@@ -955,6 +955,7 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
     case OpK::Reduce:
     case OpK::Scan:
     case OpK::Scatter:
+    case OpK::Conv:
     case OpK::DotGeneral:
       throw Error("internal: reduce/dot_general reached the emitter without a buffer or binding");
   }

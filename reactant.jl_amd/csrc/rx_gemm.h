@@ -44,4 +44,16 @@ struct GemmOperandFn {
 std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const std::string& epi_params, const std::string& epi_ctor, bool batched,
                           const GemmOperandFn& fa = {}, const GemmOperandFn& fb = {});
 
+// Tiling of the direct-convolution kernel (rx_conv_body in kernels/rx_gemm_kernels.h): f32 images [B, C, H, W], filters
+// [O, C, KH, KW], result [B, O, HO, WO], unit strides and dilations, `pl` zero columns before the image.  ok = false
+// when the kernel does not cover the case (the convolution is then lowered to a matrix product on the window matrix).
+struct ConvChoice {
+  bool ok = false;
+  int rows = 0;             // rows of the result per workgroup
+  int slab = 0;             // channels per LDS stage
+  unsigned grid[2] = {1, 1};
+  unsigned lds_bytes = 0;
+};
+ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW, int64_t HO, int64_t WO, int64_t pl);
+
 }  // namespace rx

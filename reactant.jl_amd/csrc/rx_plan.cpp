@@ -307,7 +307,7 @@ struct Planner {
     for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
     for (int r : g.results) nuse[r]++;
     auto is_leaf = [](const Node& n) {
-      return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral;
+      return n.k == OpK::Param || (n.k == OpK::Constant && !n.splat) || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv || n.k == OpK::DotGeneral;
     };
     for (const Node& d : g.nodes) {
       if (d.k != OpK::DotGeneral || d.ty.rank() < 2 || !d.a4.empty()) continue;
@@ -662,7 +662,7 @@ struct Planner {
       st.pop_back();
       if (!seen.insert(x).second) continue;
       const Node& n = g.nodes[x];
-      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) continue;
+      if (n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv || n.k == OpK::DotGeneral) continue;
       if (n.k == OpK::Constant) continue;
       if (x != id && prev_mat[x]) continue;
       if (is_arith(n.k)) cost += (n.k == OpK::Unary || n.k == OpK::Gelu) ? 2 : 1;
@@ -680,7 +680,7 @@ struct Planner {
       if (!seen.insert(x).second || seen.size() > 64) continue;
       const Node& n = g.nodes[x];
       if (n.k == OpK::DotGeneral) return true;
-      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter) continue;
+      if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv) continue;
       if (x != id && prev_mat[x]) continue;
       for (int i : n.in) st.push_back(i);
     }
@@ -712,10 +712,11 @@ struct Planner {
       const Node& n = g.nodes[x];
       // contexts in which x is evaluated
       std::set<Ctx> U;
-      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral ||
+      bool forced = is_result[x] || n.k == OpK::Param || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv || n.k == OpK::DotGeneral ||
                     (n.k == OpK::Constant && !n.splat);
       for (int u : users[x]) {
         const Node& un = g.nodes[u];
+        if (un.k == OpK::Conv) { forced = true; continue; }   // the direct-convolution kernel reads its operands from memory
         if (un.k == OpK::DotGeneral) {
           const int side = un.in[0] == x ? 0 : 1;
           if (fused_operands.count({u, side})) U.insert({u, "/operand" + std::to_string(side)});
@@ -758,7 +759,7 @@ struct Planner {
             if (!(cn.k == OpK::Convert || cn.k == OpK::Unary)) break;
             int p = cn.in[0];
             const Node& pn = g.nodes[p];
-            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce || pn.k == OpK::Scan || pn.k == OpK::Scatter) break;
+            if (pn.k == OpK::DotGeneral || pn.k == OpK::Param || pn.k == OpK::Constant || pn.k == OpK::Reduce || pn.k == OpK::Scan || pn.k == OpK::Scatter || pn.k == OpK::Conv) break;
             if (users[p].size() != 1 || is_result[p]) break;
             cur = p;
             if (info(pn.ty.dt).size < info(g.nodes[best].ty.dt).size) best = cur;
@@ -879,6 +880,7 @@ struct Planner {
         case OpK::Gather: nm = "gather"; break;
         case OpK::Scan: nm = "scan"; break;
         case OpK::Scatter: nm = "scatter"; break;
+        case OpK::Conv: nm = "convolution"; break;
         case OpK::Reduce: nm = "reduce"; break;
         case OpK::DotGeneral: nm = "dot_general"; break;
         case OpK::Iota: nm = "iota"; break;
@@ -1014,7 +1016,7 @@ struct Planner {
   bool probe_stencil(int root, StencilProbe* sp) {
     const Node& rn = g.nodes[root];
     const auto& dims = rn.ty.dims;
-    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::Scan || rn.k == OpK::Scatter || rn.k == OpK::DotGeneral) return false;
+    if (!opt.lds_stencil || rn.ty.rank() != 3 || rn.k == OpK::Reduce || rn.k == OpK::Scan || rn.k == OpK::Scatter || rn.k == OpK::Conv || rn.k == OpK::DotGeneral) return false;
     sp->vec = pick_vec(rn.ty);
     if (rn.ty.numel() < opt.slab_min_numel || sp->vec < 2) return false;
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
@@ -1971,7 +1973,7 @@ struct Planner {
     // rank 3: only small arrays, whose steps are bound by the launch gap (32^3 and 64^3 heat steps: 1.6x and 1.4x
     // faster in chains of four); at 128^3 the redundant halo cells cost more than the launches saved
     if (r < 1 || r > 3 || (r > opt.chain_max_rank && !(r == 3 && n.ty.numel() <= opt.chain_rank3_numel))) return false;
-    if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) return false;
+    if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv || n.k == OpK::DotGeneral) return false;
     const int es = info(n.ty.dt).size;
     if (es != 4 && es != 8) return false;
     if (n.ty.numel() < 2 || n.ty.numel() >= opt.slab_min_numel) return false;
@@ -2706,6 +2708,87 @@ struct Planner {
     L.args.push_back(buffer_for(root));
     L.algo_bytes = algo_bytes(em.inputs, {});
     L.desc = describe(rn.in[2]) + " scatter";
+    plan.launches.push_back(L);
+  }
+
+  // ------------------------------------------------------------------ direct convolution
+  // `root` is the convolution itself or the elementwise root that consumes it at the identity index (a bias, an
+  // activation): that cone becomes the kernel's epilogue functor, as for a dot_general.
+  void emit_conv(int root, int conv) {
+    const Node& cn = g.nodes[conv];
+    const Node& rn = g.nodes[root];
+    const TType& xt = g.nodes[cn.in[0]].ty;
+    const TType& wt = g.nodes[cn.in[1]].ty;
+    const ConvChoice cc = choose_conv(xt.dims[0], xt.dims[1], xt.dims[2], xt.dims[3], wt.dims[0], wt.dims[2], wt.dims[3], cn.ty.dims[2], cn.ty.dims[3], cn.a0[2]);
+    if (!cc.ok) throw Error("internal: convolution node without a tiling");
+    const int n = rn.ty.rank();
+    Emitter em(g, [&](int x) { return mat[x] && x != root; });
+    em.excess_precision = opt.excess_precision;
+    em.idx64 = needs64(cone_nodes(root));
+    const std::string it = em.idx_t();
+    std::vector<std::string> vars;
+    for (int k = 0; k < n; ++k) vars.push_back("i" + std::to_string(k));
+    em.set_root(rn.ty.dims, vars, true);
+    em.vec = 4;
+    em.direct_expr = vec_name;
+    em.indent = 6;
+    em.bound[conv] = "accv";
+    const std::string val = root == conv ? std::string("accv") : em.emit(root, root_index(rn.ty.dims));
+    const std::string ebody = em.take_code();
+    const std::string ost = info(rn.ty.dt).stype;
+    std::ostringstream o;
+    o << "// convolution epilogue: " << describe(root) << "\n";
+    o << "struct @K@_epi {\n";
+    for (size_t k = 0; k < em.inputs.size(); ++k)
+      o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
+    o << "  " << ost << "* __restrict__ out0;\n";
+    o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const float (&acc)[NV]";
+    for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
+    o << ") const {\n";
+    {
+      Index rix = root_index(rn.ty.dims);
+      rix[n - 1].var = "i" + std::to_string(n - 1) + "b";
+      o << "    const " << it << " lin0 = " << em.linear(rix, rn.ty.dims) << ";\n";
+    }
+    for (auto& sd : em.direct_vecs) {
+      const int slot = sd.first;
+      const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
+      o << "    const rx_vec<" << st << ", NV> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", NV>*>(in" << slot << " + lin0);\n";
+    }
+    o << "    rx_vec<" << ost << ", NV> res;\n";
+    o << "#pragma unroll\n    for (int l = 0; l < NV; ++l) {\n";
+    o << "      const " << it << " i" << n - 1 << " = i" << n - 1 << "b + l;\n";
+    o << "      const float accv = acc[l];\n";
+    o << ebody;
+    o << "      res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n    }\n";
+    o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+    o << "  }\n};\n\n";
+    o << "// direct convolution: " << xt.str() << " * " << wt.str() << " -> " << cn.ty.str() << ", " << cc.rows << " rows of the result per workgroup, channels in slabs of " << cc.slab << "\n";
+    o << "extern \"C\" __global__ __launch_bounds__(256) void @K@_conv(const float* __restrict__ X, const float* __restrict__ Wt";
+    for (size_t k = 0; k < em.inputs.size(); ++k) o << ", const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ e" << k;
+    o << ", " << ost << "* __restrict__ out0) {\n";
+    o << "  @K@_epi epi{";
+    for (size_t k = 0; k < em.inputs.size(); ++k) o << "e" << k << ", ";
+    o << "out0};\n";
+    o << "  rx_conv_body<" << xt.dims[0] << ", " << xt.dims[1] << ", " << xt.dims[2] << ", " << xt.dims[3] << ", " << wt.dims[0] << ", " << wt.dims[2] << ", " << wt.dims[3] << ", "
+      << cn.a0[0] << ", " << cn.a0[2] << ", " << cn.ty.dims[2] << ", " << cn.ty.dims[3] << ", " << cc.rows << ", " << cc.slab << ", @K@_epi>(X, Wt, epi);\n}\n\n";
+    const std::string kb_final = finalize(o.str());
+    Launch L;
+    L.kernel = named("@K@_conv", kb_final);
+    L.kind = "conv";
+    L.grid[0] = cc.grid[0];
+    L.grid[1] = cc.grid[1];
+    L.block[0] = 256;
+    L.lds_bytes = cc.lds_bytes;
+    L.args.push_back(buffer_for(cn.in[0]));
+    L.args.push_back(buffer_for(cn.in[1]));
+    for (int i : em.inputs) L.args.push_back(buffer_for(i));
+    L.args.push_back(buffer_for(root));
+    std::vector<int> all_in{cn.in[0], cn.in[1]};
+    for (int i : em.inputs) if (std::find(all_in.begin(), all_in.end(), i) == all_in.end()) all_in.push_back(i);
+    L.algo_bytes = algo_bytes(all_in, {root});
+    L.flops = 2.0 * (double)cn.ty.numel() * (double)(wt.dims[1] * wt.dims[2] * wt.dims[3]);
+    L.desc = describe(root);
     plan.launches.push_back(L);
   }
 
@@ -4030,13 +4113,13 @@ struct Planner {
     // dot epilogues: an elementwise root that consumes a dot result at the identity index
     epilogue_of.clear();
     for (int x = 0; x < N; ++x) {
-      if (!live[x] || g.nodes[x].k != OpK::DotGeneral) continue;
+      if (!live[x] || (g.nodes[x].k != OpK::DotGeneral && g.nodes[x].k != OpK::Conv)) continue;
       if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
       if (ctx[x].size() != 1) continue;
       const Ctx& c = *ctx[x].begin();
       if (!c.second.empty()) continue;
       const Node& r = g.nodes[c.first];
-      if (r.k == OpK::Reduce || r.k == OpK::Scan || r.k == OpK::Scatter || r.k == OpK::DotGeneral) continue;
+      if (r.k == OpK::Reduce || r.k == OpK::Scan || r.k == OpK::Scatter || r.k == OpK::Conv || r.k == OpK::DotGeneral) continue;
       if (r.ty.dims != g.nodes[x].ty.dims) continue;
       // the root must not be the anchor of a row group (its reductions need the full row)
       if (!row_phases(c.first).empty()) continue;
@@ -4090,7 +4173,8 @@ struct Planner {
       if (absorbed_roots.count(x)) {
         int dot = -1;
         for (auto& kv : epilogue_of) if (kv.second == x) dot = kv.first;
-        jobs.push_back({x, [this, x, dot] { emit_dot(x, dot); }});
+        if (g.nodes[dot].k == OpK::Conv) jobs.push_back({x, [this, x, dot] { emit_conv(x, dot); }});
+        else jobs.push_back({x, [this, x, dot] { emit_dot(x, dot); }});
         continue;
       }
       if (n.k == OpK::Scan) {
@@ -4099,6 +4183,11 @@ struct Planner {
       }
       if (n.k == OpK::Scatter) {
         jobs.push_back({x, [this, x] { emit_scatter(x); }});
+        continue;
+      }
+      if (n.k == OpK::Conv) {
+        if (epilogue_of.count(x)) continue;  // emitted with its root
+        jobs.push_back({x, [this, x] { emit_conv(x, x); }});
         continue;
       }
       if (reshape_alias.count(x)) continue;
@@ -4129,7 +4218,7 @@ struct Planner {
       auto plain_map_root = [&](int x) {
         const Node& n = g.nodes[x];
         if (!live[x] || !mat[x]) return false;
-        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::DotGeneral) return false;
+        if (n.k == OpK::Param || n.k == OpK::Constant || n.k == OpK::Reduce || n.k == OpK::Scan || n.k == OpK::Scatter || n.k == OpK::Conv || n.k == OpK::DotGeneral) return false;
         if (reshape_alias.count(x)) return false;
         if (absorbed_roots.count(x) || !row_phases(x).empty()) return false;
         return true;
@@ -4207,7 +4296,7 @@ struct Planner {
     // row groups claim their reductions before those would be emitted on their own
     for (auto& j : jobs) {
       const Node& n = g.nodes[j.first];
-      if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::Scatter && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
+      if (n.k != OpK::Reduce && n.k != OpK::Scan && n.k != OpK::Scatter && n.k != OpK::Conv && n.k != OpK::DotGeneral && !absorbed_roots.count(j.first))
         for (int p : row_phases(j.first)) { fused_reduces.insert(p); row_anchor[p] = j.first; }
     }
     lap("job list, chains");
@@ -4277,6 +4366,11 @@ static void count_hlo_costs(const Graph& g, Plan* plan) {
         double kk = 1;
         for (int64_t d : n.a2) kk *= (double)g.nodes[n.in[0]].ty.dims[d];
         flops += 2.0 * numel * kk;
+        break;
+      }
+      case OpK::Conv: {
+        const TType& wt = g.nodes[n.in[1]].ty;
+        flops += 2.0 * numel * (double)(wt.dims[1] * wt.dims[2] * wt.dims[3]);
         break;
       }
       case OpK::Reduce: case OpK::Scan: flops += (double)g.nodes[n.in[0]].ty.numel(); break;

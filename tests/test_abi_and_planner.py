@@ -250,10 +250,16 @@ def test_windowed_ops_plan(monkeypatch):
     # pooling: the window view is index arithmetic inside a reduction kernel
     rep = rx.compile_offline(NN.reduce_window([8, 16, 32, 32], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])[0])
     assert "launches: 1" in rep and "window reduce" in rep
-    # convolution with few output features: one MFMA product (64-row tiles) that evaluates the window matrix while
-    # it loads its tiles, then bias + relu + layout in one map; the reshaped weights share the argument's buffer
+    # f32 convolution, unit strides, 64 output features: the direct-convolution kernel with bias + relu as its epilogue,
+    # seven rows of the result per workgroup (256 workgroups)
     conv = NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0]
     kinds = lambda rep: [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
+    rep = rx.compile_offline(conv, with_source=True)
+    assert kinds(rep) == ["conv"] and "grid=256x1x1" in rep, rep
+    assert "rx_conv_body<32, 64, 56, 56, 64, 3, 3, 1, 1, 56, 56, 7, 8, " in rep
+    # without it: one MFMA product (64-row tiles) that evaluates the window matrix while it loads its tiles, then
+    # bias + relu + layout in one map; the reshaped weights share the argument's buffer
+    monkeypatch.setenv("RX_CONV_DIRECT", "0")
     rep = rx.compile_offline(conv, with_source=True)
     assert kinds(rep) == ["gemm_f32", "map"], rep
     assert "rx_gemm_body<rx_mma_f32, 64, 128" in rep and "dot operand B computed on the fly" in rep
@@ -264,6 +270,10 @@ def test_windowed_ops_plan(monkeypatch):
     rep = rx.compile_offline(conv, with_source=True)
     assert kinds(rep) == ["map", "gemm_f32", "map"] and "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rep
     monkeypatch.delenv("RX_FUSE_DOT_OPERANDS")
+    monkeypatch.delenv("RX_CONV_DIRECT")
+    # strides, few output features, other element types: the matrix product
+    assert "kind=conv" not in rx.compile_offline(NN.convolution([1, 3, 33, 35], [16, 3, 5, 5], "f32", strides=[2, 2], padding=[[2, 2], [2, 2]])[0])
+    assert "kind=conv" not in rx.compile_offline(NN.convolution([2, 32, 28, 28], [64, 32, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0])
     with pytest.raises(Exception, match="batch_group_count and feature_group_count"):
         rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 4, 4, 4], "f32", groups=2)[0].replace("batch_group_count = 1", "batch_group_count = 2"))
 

@@ -249,7 +249,18 @@ def test_convolution_reference_grid(rx, client, groups):
 
 CONVS = [
     # x, w, dtype, dims, kwargs, expected kind of the product
-    ([4, 64, 56, 56], [64, 64, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "gemm_f32"),
+    # f32, unit strides and dilations, at least 33 output features: the direct-convolution kernel (bias + relu in its epilogue)
+    ([4, 64, 56, 56], [64, 64, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "conv"),
+    # the same as a matrix product on the window matrix
+    ([4, 64, 56, 56], [64, 64, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu", env={"RX_CONV_DIRECT": "0"}), "gemm_f32"),
+    # a 5x3 filter, uneven padding, channels that are not whole slabs of 8, 48 features (three of the four wavefronts), a ragged last tile
+    ([3, 20, 30, 36], [48, 20, 5, 3], "f32", None, dict(padding=[[2, 1], [0, 2]]), "conv"),
+    # rows of the image and of the result that are not whole 16-byte vectors, no padding, 40 features
+    ([2, 9, 21, 23], [40, 9, 3, 3], "f32", None, dict(), "conv"),
+    # channels-last images and [rows, columns, in, out] filters: transposes around the kernel
+    ([2, 12, 16, 8], [3, 3, 8, 64], "f32", "[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]", dict(padding=[[1, 1], [1, 1]]), "conv"),
+    # a 1x1 filter (a product over the channels), 7x7 images, bias + relu
+    ([8, 128, 7, 7], [96, 128, 1, 1], "f32", None, dict(epilogue="bias_relu"), "conv"),
     ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
     ([1, 3, 33, 35], [16, 3, 5, 5], "f32", None, dict(strides=[2, 2], padding=[[2, 2], [2, 2]]), "gemm_f32"),
     ([16, 16, 8, 2], [4, 4, 8, 4], "f32", "[1, 0, f, b]x[1, 0, i, o]->[1, 0, f, b]", dict(), None),
@@ -258,14 +269,18 @@ CONVS = [
     ([2, 3, 8, 8, 8], [3, 3, 3, 3, 3], "f32", "[b, f, 2, 1, 0]x[o, i, 2, 1, 0]->[b, f, 2, 1, 0]", dict(padding=[[1, 1], [1, 1], [1, 1]]), None),
     ([2, 6, 20, 20], [12, 3, 3, 3], "f64", None, dict(groups=2, generic=True), None),
     ([8, 32, 14, 14], [32, 1, 3, 3], "f32", None, dict(groups=32, padding=[[1, 1], [1, 1]]), None),
-    # more than 128 output features: the window matrix is written to memory instead of being evaluated by the product
-    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "gemm_f32"),
+    # 160 output features: three groups of 64 features in the direct kernel's grid
+    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "conv"),
+    # bf16 with more than 128 output features: the window matrix is written to memory instead of being evaluated by the product
+    ([2, 160, 14, 14], [160, 160, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
 ]
 
 
 @pytest.mark.parametrize("xs,ws,dt,dims,kw,kind", CONVS)
-def test_convolution_layouts_and_types(rx, client, xs, ws, dt, dims, kw, kind):
+def test_convolution_layouts_and_types(rx, client, xs, ws, dt, dims, kw, kind, monkeypatch):
     kw = dict(kw)
+    for k, v in kw.pop("env", {}).items():
+        monkeypatch.setenv(k, v)
     if dims:
         kw["dims"] = dims
     text, out_shape = NN.convolution(xs, ws, dt, **kw)
@@ -318,7 +333,7 @@ def test_vgg_style_forward_pass(rx, client, sizes):
     assert np.allclose(got[0].a.sum(axis=1), 1.0, atol=1e-5)
     _close(got[0].a, ref[0].a, 1e-4)
     if sizes["cmid"] >= 64:
-        assert any(l["kind"] == "gemm_f32" for l in exe.launches())
+        assert any(l["kind"] == "conv" for l in exe.launches())
 
 
 @pytest.mark.parametrize("bh,seq,dim,dt,tol", [(6, 40, 16, "f32", 1e-5), (8, 256, 64, "f32", 1e-4), (8, 256, 64, "bf16", 2e-2)])
