@@ -1485,11 +1485,21 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
       else pstage1[i] = in ? src[q] : 0.f;
     }
     const int o = og + (tid & 63), part = tid >> 6;
+    // whole slabs, whole groups of 64 features and whole quarters: plain consecutive loads, which the compiler widens;
+    // else loads at clamped positions inside the filter array and a select (a load under a branch of its own is not
+    // combined with its neighbours and costs the kernel 12 %)
+    constexpr bool WFULL = C % CB == 0 && O % 64 == 0 && CB * TAPS % 4 == 0;
+    const float* wsrc = w + ((long long)(o < O ? o : O - 1) * C + c0) * TAPS;
+    const int left = (C - c0) * TAPS;                               // words of this feature from channel c0 on
 #pragma unroll
     for (int i = 0; i < WPT; ++i) {
       const int e = part * WPT + i;                                 // (channel of the slab, tap)
-      const int c = c0 + e / TAPS;
-      wstage[i] = (e < CB * TAPS && c < C && o < O) ? w[((long long)o * C + c0) * TAPS + e] : 0.f;
+      if constexpr (WFULL) {
+        wstage[i] = wsrc[e];
+      } else {
+        const float v = wsrc[e < left ? e : left - 1];
+        wstage[i] = (e < CB * TAPS && e < left && o < O) ? v : 0.f;
+      }
     }
   };
   auto store_slab = [&](int st) {
