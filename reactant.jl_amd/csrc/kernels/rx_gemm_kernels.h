@@ -1425,13 +1425,13 @@ RX_DEV void rx_gemm_body_f64(const double* __restrict__ A, const double* __restr
 
 // ===========================================================================
 // Direct convolution of f32 images on v_mfma_f32_16x16x4_f32: x [B][C][H][W], w [O][C][KH][KW], out [B][O][HO][WO],
-// unit strides and dilations, zero padding PT / PL rows and columns before the image (what lies after it follows from
-// HO and WO).  A workgroup of four wavefronts computes TR whole rows of the result of one image for 64 output
+// strides SH / SW, filter dilations DH / DW, zero padding PT / PL rows and columns before the image (what lies after it
+// follows from HO and WO).  A workgroup of four wavefronts computes TR whole rows of the result of one image for 64 output
 // features, wavefront v the features 16 v .. 16 v + 15 of the group; blockIdx.y is the group of features.  The
-// channels pass through LDS in slabs of CB, two stages: the patch of the image that the tile reads, [CB][TR + KH - 1]
-// [PW] with the image's column 0 at column OFF and zeros around it, and the slab's weights as [tap][quad of channels]
+// channels pass through LDS in slabs of CB, two stages (one if there is one slab): the patch of the image that the tile
+// reads, [CB][(TR - 1) SH + (KH - 1) DH + 1][PW] with the image's column 0 at column OFF and zeros around it, and the slab's weights as [tap][quad of channels]
 // [channel of the quad][80] features.  One k step of the MFMA is four channels of one tap: the pixel operand of lane
-// (pixel % 16, channel = lane / 16) is patch[channel][row + dy][column + dx], i.e. one address per lane and pixel block
+// (pixel % 16, channel = lane / 16) is patch[channel][row SH + dy DH][column SW + dx DW], i.e. one address per lane and pixel block
 // plus a constant per step; the feature operand is one LDS word per step.  Every element of the image is read from
 // memory once per tile (and per group of features) instead of once per tap.  The channel pitch of the patch is
 // 16 mod 64 words, so that the four channels of a step read different banks.
@@ -1440,12 +1440,13 @@ RX_DEV void rx_gemm_body_f64(const double* __restrict__ A, const double* __restr
 // 119 us for the same product as an implicit GEMM (the window matrix evaluated while its tiles are loaded) plus 9 us for
 // the map that brings its [feature][image, pixel] result into this layout.
 // ===========================================================================
-template <int B, int C, int H, int W, int O, int KH, int KW, int PT, int PL, int HO, int WO, int TR, int CB, class Epi>
+template <int B, int C, int H, int W, int O, int KH, int KW, int SH, int SW, int DH, int DW, int PT, int PL, int HO, int WO, int TR, int CB, class Epi>
 RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ w, const Epi& epi) {
   constexpr int TAPS = KH * KW;
-  constexpr int PR = TR + KH - 1;                                   // rows of the patch
+  constexpr int PR = (TR - 1) * SH + (KH - 1) * DH + 1;             // rows of the patch
   constexpr int OFF = (PL + 3) / 4 * 4;                             // column of the image's column 0
-  constexpr int PW = (OFF + WO + KW - 1 - PL + 3) / 4 * 4;          // row pitch: columns -PL .. WO + KW - 2 - PL of the image
+  constexpr int LASTC = (WO - 1) * SW + (KW - 1) * DW - PL;         // last column of the image that a tile reads (may lie in the padding)
+  constexpr int PW = (OFF + (LASTC + 1 > W ? LASTC + 1 : W) + 3) / 4 * 4;   // row pitch
   constexpr int PCH = (PR * PW + 47) / 64 * 64 + 16;                // channel pitch, 16 mod 64
   constexpr int NPX = TR * WO, NPB = (NPX + 15) / 16;               // pixels and blocks of 16 pixels of a tile
   constexpr int NQ = CB / 4, NSTEP = TAPS * NQ;                     // k steps per slab
@@ -1455,13 +1456,14 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
   constexpr int TILES = (HO + TR - 1) / TR;
   static_assert(CB % 4 == 0 && OFF >= PL && PW >= OFF + W, "patch layout");
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
-  float* const patch = (float*)rx_smem;                             // [2][PATCH]
-  float* const wl = patch + 2 * PATCH;                              // [2][WSLAB]
+  constexpr int NSTG = NSLAB > 1 ? 2 : 1;                           // one slab needs no second stage
+  float* const patch = (float*)rx_smem;                             // [NSTG][PATCH]
+  float* const wl = patch + NSTG * PATCH;                           // [NSTG][WSLAB]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = blockIdx.x / TILES, y0 = (blockIdx.x % TILES) * TR;
   const int og = blockIdx.y * 64;
-  // both patch stages start as zeros: the columns around the image are never written afterwards
-  for (int i = tid; i < 2 * PATCH; i += 256) patch[i] = 0.f;
+  // the patch stages start as zeros: the columns around the image are never written afterwards
+  for (int i = tid; i < NSTG * PATCH; i += 256) patch[i] = 0.f;
   __syncthreads();
 
   // Loaders.  Patch: the CB * PR rows of a slab, W words each, as 16-byte vectors where the rows are aligned; weights:
@@ -1478,7 +1480,7 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
     for (int i = 0; i < NLP; ++i) {
       const int v = i * 256 + tid;
       const int row = v / EPR, q = v % EPR;                         // row = channel of the slab * PR + row of the patch
-      const int c = c0 + row / PR, y = y0 - PT + row % PR;
+      const int c = c0 + row / PR, y = y0 * SH - PT + row % PR;
       const bool in = v < NLD && c < C && y >= 0 && y < H;
       const float* src = x + (((long long)b * C + c) * H + y) * W;
       if constexpr (VEC) pstage[i] = in ? *(const rx_f32x4*)(src + 4 * q) : rx_f32x4{0.f, 0.f, 0.f, 0.f};
@@ -1530,7 +1532,7 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
   for (int pb = 0; pb < NPB; ++pb) {
     int p = pb * 16 + li;
     if (p >= NPX) p = NPX - 1;                                      // ragged last block: those rows of the result are not stored
-    poff[pb] = kk * PCH + (p / WO) * PW + (p % WO) + OFF - PL;
+    poff[pb] = kk * PCH + (p / WO) * SH * PW + (p % WO) * SW + OFF - PL;
   }
   const int woff = kk * WST + wave * 16 + li;
   rx_f32x4 acc[NPB];
@@ -1550,7 +1552,7 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
         const float fw = ww[(tap * NQ + q) * 4 * WST + woff];
-        const int koff = q * 4 * PCH + (tap / KW) * PW + (tap % KW);
+        const int koff = q * 4 * PCH + (tap / KW) * DH * PW + (tap % KW) * DW;
 #pragma unroll
         for (int pb = 0; pb < NPB; ++pb)
           acc[pb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pp[poff[pb] + koff], fw, acc[pb], 0, 0, 0);

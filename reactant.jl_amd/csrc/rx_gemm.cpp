@@ -1,6 +1,7 @@
 #include "rx_gemm.h"
 
 #include <cstdlib>
+#include <algorithm>
 #include <sstream>
 #include <stdexcept>
 
@@ -246,21 +247,24 @@ std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const s
   return o.str();
 }
 
-ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW, int64_t HO, int64_t WO, int64_t pl) {
+ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW, int64_t HO, int64_t WO, int64_t pl,
+                       int64_t sh, int64_t sw, int64_t dh, int64_t dw) {
   ConvChoice c;
   if (getenv("RX_CONV_DIRECT") && atoi(getenv("RX_CONV_DIRECT")) == 0) return c;
   if (getenv("RX_MFMA") && atoi(getenv("RX_MFMA")) == 0) return c;
   if (B < 1 || C < 1 || O < 1 || HO < 1 || WO < 1 || KH < 1 || KW < 1) return c;
   // four wavefronts of 16 features each: with fewer than 33 features half of them would idle; a tile is whole rows of
   // the result, at most 25 blocks of 16 pixels (100 accumulator registers); taps unroll, so the filter is small
-  if (O < 33 || WO > 400 || KH * KW > 49 || KH > H + 64 || KW > W + 64) return c;
+  if (O < 33 || WO > 400 || KH * KW > 49 || KH > H + 64 || KW > W + 64 || sh < 1 || sw < 1 || dh < 1 || dw < 1 || sh > 4 || sw > 4) return c;
   if (B * C * H * W >= ((int64_t)1 << 31) || B * O * HO * WO >= ((int64_t)1 << 31)) return c;
   const int64_t groups = (O + 63) / 64;
   const int slab = C >= 8 ? 8 : 4;
+  const int64_t stages = (C + slab - 1) / slab > 1 ? 2 : 1;
   auto lds_of = [&](int64_t tr) {
-    const int64_t pr = tr + KH - 1, off = (pl + 3) / 4 * 4, pw = (off + WO + KW - 1 - pl + 3) / 4 * 4;
+    const int64_t pr = (tr - 1) * sh + (KH - 1) * dh + 1, off = (pl + 3) / 4 * 4, lastc = (WO - 1) * sw + (KW - 1) * dw - pl;
+    const int64_t pw = (off + std::max<int64_t>(lastc + 1, W) + 3) / 4 * 4;
     const int64_t pch = (pr * pw + 47) / 64 * 64 + 16;
-    return (2 * slab * pch + 2 * KH * KW * (slab / 4) * 4 * 80) * 4;
+    return (stages * slab * pch + stages * KH * KW * (slab / 4) * 4 * 80) * 4;
   };
   // rows per workgroup: least padded work (ragged last tile, ragged last pixel block, workgroups in whole rounds of
   // the 256 compute units) among the tiles that fit
@@ -270,10 +274,15 @@ ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, in
     const int64_t tiles = (HO + tr - 1) / tr, npb = (tr * WO + 15) / 16;
     const int64_t wgs = B * tiles * groups;
     const double rounds = (double)((wgs + 255) / 256);
-    const double cost = rounds * (double)npb * (1.0 + 0.02 * (double)(tr + KH - 1) / (double)tr);   // time of the slowest compute unit, patch loads included
+    // time of the slowest compute unit: the MFMAs of its pixel blocks, the filter it reads once per tile (about one pixel block's worth) and the patch loads
+    const double cost = rounds * ((double)npb + 1.0) * (1.0 + 0.02 * (double)((tr - 1) * sh + (KH - 1) * dh + 1) / (double)tr);
     if (c.rows == 0 || cost < best) { best = cost; c.rows = (int)tr; }
   }
   if (c.rows == 0) return c;
+  // A workgroup reads its 64 features' whole filter for one tile of one image: with small images (14 x 14: 13 pixel
+  // blocks per image, 0.107 against 0.103 ms for 256 -> 256 features; 7 x 7: 0.152 against 0.099 ms for 512 -> 512) the
+  // matrix product on the window matrix, whose tiles span images, is as fast or faster
+  if (HO * WO < 224) { c.rows = 0; return c; }
   if (const char* e = getenv("RX_CONV_ROWS")) {
     const int v = atoi(e);
     if (v >= 1 && v <= HO && (int64_t)v * WO <= 400 && lds_of(v) <= 160 * 1024) c.rows = v;

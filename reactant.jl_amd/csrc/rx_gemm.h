@@ -45,7 +45,7 @@ std::string gemm_instance(const GemmChoice& c, const std::string& kbase, const s
                           const GemmOperandFn& fa = {}, const GemmOperandFn& fb = {});
 
 // Tiling of the direct-convolution kernel (rx_conv_body in kernels/rx_gemm_kernels.h): f32 images [B, C, H, W], filters
-// [O, C, KH, KW], result [B, O, HO, WO], unit strides and dilations, `pl` zero columns before the image.  ok = false
+// [O, C, KH, KW], result [B, O, HO, WO], strides sh / sw, filter dilations dh / dw, `pl` zero columns before the image.  ok = false
 // when the kernel does not cover the case (the convolution is then lowered to a matrix product on the window matrix).
 struct ConvChoice {
   bool ok = false;
@@ -54,6 +54,7 @@ struct ConvChoice {
   unsigned grid[2] = {1, 1};
   unsigned lds_bytes = 0;
 };
-ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW, int64_t HO, int64_t WO, int64_t pl);
+ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, int64_t KH, int64_t KW, int64_t HO, int64_t WO, int64_t pl,
+                       int64_t sh = 1, int64_t sw = 1, int64_t dh = 1, int64_t dw = 1);
 
 }  // namespace rx

@@ -79,8 +79,8 @@ struct Node {
   //       a2 = scatter_dims_to_operand_dims, a4[0] = index_vector_dim, a5 = input_batching_dims,
   //       a6 = scatter_indices_batching_dims; op = "assign", "subtract", "divide" or "combine" (then `red` is the monoid)
   //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
-  //   Conv (image [B, C, H, W], filter [O, C, KH, KW]) -> [B, O, HO, WO]: unit strides and dilations, zero padding
-  //       a0 = {rows before, rows after, columns before, columns after} (the direct-convolution kernel's operation)
+  //   Conv (image [B, C, H, W], filter [O, C, KH, KW]) -> [B, O, HO, WO]: zero padding a0 = {rows before, rows after,
+  //       columns before, columns after}, a1 = strides, a2 = filter dilations (the direct-convolution kernel's operation)
   std::vector<int64_t> a0, a1, a2, a3, a4, a5, a6;
   Red red = Red::Add;
   // Constant payload: either one splat element or dense bytes in storage format

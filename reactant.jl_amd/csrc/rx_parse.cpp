@@ -1936,13 +1936,14 @@ struct Builder {
     if (C != I * G || O % G != 0) fail("convolution: feature counts do not match feature_group_count");
     if (B % BG != 0 || O % BG != 0) fail("convolution: batch and output feature counts must be multiples of batch_group_count");
     const int64_t Bo = B / BG;    // batch entries of the result
-    // f32 images with two spatial dims, unit strides and dilations, no groups and non-negative padding: the direct-convolution
+    // f32 images with two spatial dims, no input dilation, no groups and non-negative padding: the direct-convolution
     // kernel (OpK::Conv; rx_conv_body in kernels/rx_gemm_kernels.h) where its tiling covers the shapes
-    if (nsp == 2 && xct.dt == DT::F32 && G == 1 && BG == 1 && st[0] == 1 && st[1] == 1 && ld[0] == 1 && ld[1] == 1 && rd[0] == 1 && rd[1] == 1 &&
-        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0) {
+    if (nsp == 2 && xct.dt == DT::F32 && G == 1 && BG == 1 && st[0] >= 1 && st[1] >= 1 && ld[0] == 1 && ld[1] == 1 && rd[0] >= 1 && rd[1] >= 1 &&
+        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1) {
       const int64_t KH = wct.dims[2], KW = wct.dims[3];
-      const int64_t HO = xct.dims[2] + pad[0] + pad[1] - KH + 1, WO = xct.dims[3] + pad[2] + pad[3] - KW + 1;
-      if (HO >= 1 && WO >= 1 && KH >= 1 && KW >= 1 && choose_conv(B, C, xct.dims[2], xct.dims[3], O, KH, KW, HO, WO, pad[2]).ok) {
+      const int64_t eh = xct.dims[2] + pad[0] + pad[1] - ((KH - 1) * rd[0] + 1), ew = xct.dims[3] + pad[2] + pad[3] - ((KW - 1) * rd[1] + 1);
+      const int64_t HO = eh >= 0 ? eh / st[0] + 1 : 0, WO = ew >= 0 ? ew / st[1] + 1 : 0;
+      if (HO >= 1 && WO >= 1 && choose_conv(B, C, xct.dims[2], xct.dims[3], O, KH, KW, HO, WO, pad[2], st[0], st[1], rd[0], rd[1]).ok) {
         std::vector<int64_t> want(r);
         want[cd[2].d0] = B; want[cd[2].d1] = O; want[cd[2].sp[0]] = HO; want[cd[2].sp[1]] = WO;
         if (want != out.dims) fail("convolution: result shape mismatch");
@@ -1950,6 +1951,8 @@ struct Builder {
         cv.k = OpK::Conv;
         cv.in = {xc, wc};
         cv.a0 = {pad[0], pad[1], pad[2], pad[3]};
+        cv.a1 = {st[0], st[1]};
+        cv.a2 = {rd[0], rd[1]};
         cv.ty = TType{out.dt, {B, O, HO, WO}};
         int cur = g.add(cv);
         // [B, O, rows, columns] -> the result's own dimension order

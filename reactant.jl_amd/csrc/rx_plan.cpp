@@ -2719,7 +2719,8 @@ struct Planner {
     const Node& rn = g.nodes[root];
     const TType& xt = g.nodes[cn.in[0]].ty;
     const TType& wt = g.nodes[cn.in[1]].ty;
-    const ConvChoice cc = choose_conv(xt.dims[0], xt.dims[1], xt.dims[2], xt.dims[3], wt.dims[0], wt.dims[2], wt.dims[3], cn.ty.dims[2], cn.ty.dims[3], cn.a0[2]);
+    const ConvChoice cc = choose_conv(xt.dims[0], xt.dims[1], xt.dims[2], xt.dims[3], wt.dims[0], wt.dims[2], wt.dims[3], cn.ty.dims[2], cn.ty.dims[3], cn.a0[2],
+                                      cn.a1[0], cn.a1[1], cn.a2[0], cn.a2[1]);
     if (!cc.ok) throw Error("internal: convolution node without a tiling");
     const int n = rn.ty.rank();
     Emitter em(g, [&](int x) { return mat[x] && x != root; });
@@ -2771,7 +2772,7 @@ struct Planner {
     for (size_t k = 0; k < em.inputs.size(); ++k) o << "e" << k << ", ";
     o << "out0};\n";
     o << "  rx_conv_body<" << xt.dims[0] << ", " << xt.dims[1] << ", " << xt.dims[2] << ", " << xt.dims[3] << ", " << wt.dims[0] << ", " << wt.dims[2] << ", " << wt.dims[3] << ", "
-      << cn.a0[0] << ", " << cn.a0[2] << ", " << cn.ty.dims[2] << ", " << cn.ty.dims[3] << ", " << cc.rows << ", " << cc.slab << ", @K@_epi>(X, Wt, epi);\n}\n\n";
+      << cn.a1[0] << ", " << cn.a1[1] << ", " << cn.a2[0] << ", " << cn.a2[1] << ", " << cn.a0[0] << ", " << cn.a0[2] << ", " << cn.ty.dims[2] << ", " << cn.ty.dims[3] << ", " << cc.rows << ", " << cc.slab << ", @K@_epi>(X, Wt, epi);\n}\n\n";
     const std::string kb_final = finalize(o.str());
     Launch L;
     L.kernel = named("@K@_conv", kb_final);

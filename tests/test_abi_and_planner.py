@@ -256,7 +256,7 @@ def test_windowed_ops_plan(monkeypatch):
     kinds = lambda rep: [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
     rep = rx.compile_offline(conv, with_source=True)
     assert kinds(rep) == ["conv"] and "grid=256x1x1" in rep, rep
-    assert "rx_conv_body<32, 64, 56, 56, 64, 3, 3, 1, 1, 56, 56, 7, 8, " in rep
+    assert "rx_conv_body<32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 56, 56, 7, 8, " in rep
     # without it: one MFMA product (64-row tiles) that evaluates the window matrix while it loads its tiles, then
     # bias + relu + layout in one map; the reshaped weights share the argument's buffer
     monkeypatch.setenv("RX_CONV_DIRECT", "0")
@@ -271,8 +271,12 @@ def test_windowed_ops_plan(monkeypatch):
     assert kinds(rep) == ["map", "gemm_f32", "map"] and "rx_gemm_body_dl<rx_mma_f32, 64, 128" in rep
     monkeypatch.delenv("RX_FUSE_DOT_OPERANDS")
     monkeypatch.delenv("RX_CONV_DIRECT")
-    # strides, few output features, other element types: the matrix product
+    # a strided stem (three channels: one slab, one LDS stage): two rows of the result per workgroup
+    rep = rx.compile_offline(NN.convolution([32, 3, 224, 224], [64, 3, 7, 7], "f32", strides=[2, 2], padding=[[3, 3], [3, 3]])[0], with_source=True)
+    assert kinds(rep) == ["conv"] and "rx_conv_body<32, 3, 224, 224, 64, 7, 7, 2, 2, 1, 1, 3, 3, 112, 112, 2, 4, " in rep, rep
+    # few output features, input dilation, other element types: the matrix product
     assert "kind=conv" not in rx.compile_offline(NN.convolution([1, 3, 33, 35], [16, 3, 5, 5], "f32", strides=[2, 2], padding=[[2, 2], [2, 2]])[0])
+    assert "kind=conv" not in rx.compile_offline(NN.convolution([2, 8, 20, 20], [64, 8, 3, 3], "f32", lhs_dil=[2, 2], padding=[[2, 2], [2, 2]])[0])
     assert "kind=conv" not in rx.compile_offline(NN.convolution([2, 32, 28, 28], [64, 32, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0])
     with pytest.raises(Exception, match="batch_group_count and feature_group_count"):
         rx.compile_offline(NN.convolution([2, 8, 16, 16], [4, 4, 4, 4], "f32", groups=2)[0].replace("batch_group_count = 1", "batch_group_count = 2"))

@@ -258,9 +258,14 @@ CONVS = [
     # rows of the image and of the result that are not whole 16-byte vectors, no padding, 40 features
     ([2, 9, 21, 23], [40, 9, 3, 3], "f32", None, dict(), "conv"),
     # channels-last images and [rows, columns, in, out] filters: transposes around the kernel
-    ([2, 12, 16, 8], [3, 3, 8, 64], "f32", "[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]", dict(padding=[[1, 1], [1, 1]]), "conv"),
+    ([2, 16, 20, 8], [3, 3, 8, 64], "f32", "[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]", dict(padding=[[1, 1], [1, 1]]), "conv"),
+    # strides: a 7x7/2 stem with three channels (one slab, one LDS stage) and a 3x3/2 layer with two groups of 64 features
+    ([2, 3, 64, 64], [64, 3, 7, 7], "f32", None, dict(strides=[2, 2], padding=[[3, 3], [3, 3]]), "conv"),
+    ([3, 24, 30, 28], [128, 24, 3, 3], "f32", None, dict(strides=[2, 1], padding=[[1, 1], [1, 0]], epilogue="bias_relu"), "conv"),
+    # a dilated filter with unequal strides, flipped (NNlib's true convolution)
+    ([2, 16, 24, 28], [48, 16, 3, 3], "f32", None, dict(strides=[1, 2], rhs_dil=[2, 3], padding=[[2, 2], [3, 3]], flip=True), "conv"),
     # a 1x1 filter (a product over the channels), 7x7 images, bias + relu
-    ([8, 128, 7, 7], [96, 128, 1, 1], "f32", None, dict(epilogue="bias_relu"), "conv"),
+    ([8, 128, 16, 16], [96, 128, 1, 1], "f32", None, dict(epilogue="bias_relu"), "conv"),
     ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
     ([1, 3, 33, 35], [16, 3, 5, 5], "f32", None, dict(strides=[2, 2], padding=[[2, 2], [2, 2]]), "gemm_f32"),
     ([16, 16, 8, 2], [4, 4, 8, 4], "f32", "[1, 0, f, b]x[1, 0, i, o]->[1, 0, f, b]", dict(), None),
@@ -270,7 +275,9 @@ CONVS = [
     ([2, 6, 20, 20], [12, 3, 3, 3], "f64", None, dict(groups=2, generic=True), None),
     ([8, 32, 14, 14], [32, 1, 3, 3], "f32", None, dict(groups=32, padding=[[1, 1], [1, 1]]), None),
     # 160 output features: three groups of 64 features in the direct kernel's grid
-    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "conv"),
+    ([2, 160, 20, 20], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "conv"),
+    # small images: the matrix product, whose tiles span images (more than 128 output features: the window matrix is written to memory)
+    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "gemm_f32"),
     # bf16 with more than 128 output features: the window matrix is written to memory instead of being evaluated by the product
     ([2, 160, 14, 14], [160, 160, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
 ]
