@@ -1248,6 +1248,8 @@ RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out8) {
     // 20 ms or so of a load run up to 20 % slower (8192 x 4096 x 4096 bf16: 246 us per launch 5 ms after the start,
     // 201 us from 22 ms on), whatever the kernel.
     const int reps = 20;
+    // RX_PROBE_SETTLE_MS: that time (counter runs, which record every dispatch, set it to 0)
+    const float settle_ms = getenv("RX_PROBE_SETTLE_MS") ? (float)atof(getenv("RX_PROBE_SETTLE_MS")) : 150.f;
     HIP_CHECK(hipEventRecord(e0, d->stream));
     for (;;) {
       for (int i = 0; i < 20; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
@@ -1255,7 +1257,7 @@ RX_EXPORT int RxGemmClockProbe(RxDevice* d, int kind, double* out8) {
       HIP_CHECK(hipEventSynchronize(e1));
       float warm_ms = 0;
       HIP_CHECK(hipEventElapsedTime(&warm_ms, e0, e1));
-      if (warm_ms >= 150.f) break;
+      if (warm_ms >= settle_ms) break;
     }
     HIP_CHECK(hipEventRecord(e0, d->stream));
     for (int i = 0; i < reps; ++i) hipLaunchKernelGGL(fn, dim3(grid), dim3(512), lds, d->stream, a.ptr, b.ptr, (rx_u16*)o.ptr, (unsigned long long*)sl.ptr, (unsigned long long*)lf.ptr);
