@@ -1091,8 +1091,9 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 // apart: in its memory phase a wavefront reads all its fragments of one K tile from LDS (8 of A, 4 of B: 96
 // registers), in its compute phase it issues that tile's 64 (16-bit) or 32 (8-bit) MFMAs back to back at raised
 // priority, with nothing in between that could wait for memory, while the other wavefront of the SIMD is in its
-// memory phase.  Two barriers per K tile keep the phases apart.  Requests go out in memory phases only, between the
-// LDS reads, where a request that has to wait for the load path delays no MFMA.
+// memory phase.  Two barriers per K tile keep the phases apart (the results do not depend on which wavefronts share a
+// SIMD, only the overlap does).  Requests go out in memory phases only, between the LDS reads, where a request that has
+// to wait for the load path delays no MFMA.
 //   interval 2t:   group 0 (wavefronts 0-3) reads tile t (stage t % 2) and requests tile t + 1 into the other stage,
 //                  group 1 multiplies tile t - 1
 //   interval 2t+1: group 0 multiplies tile t and then waits for tile t + 1 to land, group 1 reads tile t
