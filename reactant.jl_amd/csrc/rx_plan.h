@@ -58,9 +58,11 @@ struct PlanOptions {
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
   int slab_ytiles = 0;          // stencil kernels: y-tiles per XCD slab (0: one slab per XCD)
   int lds_tile[3] = {3, 4, 128};  // outputs per workgroup tile (slowest .. fastest dimension)
-  // full reductions in one launch: the last workgroup to finish combines the partials.  Off: the
-  // device-scope release fence every workgroup needs before taking its ticket (an L2 write-back on
-  // this multi-die part) made the sinsum kernel 2x slower than the two-launch form.
+  // full reductions in one launch: every workgroup publishes its partial as flagged words and the
+  // workgroup with the last index waits for all of them and combines.  Off: it saves the 1-workgroup
+  // combine launch (1.4 us of an 85 us step over 2^26 elements, 1.2 us of a 485 us FP8 step), and it
+  // adds a wait between workgroups whose expiry would go unreported.  (An earlier form with a
+  // device-scope release fence before a ticket -- an L2 write-back on this multi-die part -- was 2x slower.)
   bool single_pass_reduce = false;
   bool single_pass_scan = true;      // long scanned rows in one launch (chunk totals travel as flagged words)
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
