@@ -1463,9 +1463,6 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = blockIdx.x / TILES, y0 = (blockIdx.x % TILES) * TR;
   const int og = blockIdx.y * 64;
-  // the patch stages start as zeros: the columns around the image are never written afterwards
-  for (int i = tid; i < NSTG * PATCH; i += 256) patch[i] = 0.f;
-  __syncthreads();
 
   // Loaders.  Patch: the CB * PR rows of a slab, W words each, as 16-byte vectors where the rows are aligned; weights:
   // thread (feature tid % 64, quarter tid / 64) takes a quarter of the feature's CB * TAPS consecutive words.
@@ -1541,26 +1538,68 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
   for (int pb = 0; pb < NPB; ++pb) acc[pb] = rx_f32x4{0.f, 0.f, 0.f, 0.f};
 
   load_slab(0);
+  // the patch stages start as zeros (the columns around the image are never written afterwards), under the first loads
+  for (int i = tid; i < NSTG * PATCH; i += 256) patch[i] = 0.f;
+  __syncthreads();
   store_slab(0);
   __syncthreads();
+  // One wavefront per SIMD: nothing else hides the LDS latency, so the operands of k step ks + 1 are read into a second
+  // register set while the MFMAs of step ks run, one read between two MFMAs (a scheduling barrier after every pair keeps
+  // that order: left alone the compiler reads a whole step's operands and then waits for them with the MFMA pipe idle).  The next slab goes
+  // into the other stage in the middle of a slab, between two barriers (every wavefront has left the previous slab; the
+  // stage is complete), so that the last step of a slab can already read the first operands of the next one.
+  float pa[2][NPB], fw[2];
+  // operand `pb` of step KS into register set BUF (pb = -1: the filter word)
+  auto fetch = [&](auto BUF, auto KS, int pb, const float* pp, const float* ww) __attribute__((always_inline)) {
+    constexpr int buf = decltype(BUF)::value, ks = decltype(KS)::value, tap = ks / NQ, q = ks % NQ;
+    constexpr int koff = q * 4 * PCH + (tap / KW) * DH * PW + (tap % KW) * DW;
+    if (pb < 0) fw[buf] = ww[ks * 4 * WST + woff];
+    else pa[buf][pb] = pp[poff[pb] + koff];
+  };
+  auto fetch_all = [&](auto BUF, auto KS, const float* pp, const float* ww) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pb = -1; pb < NPB; ++pb) fetch(BUF, KS, pb, pp, ww);
+  };
+  constexpr bool AHEAD = NSTEP % 2 == 0 && NSTEP >= 4;              // the register sets alternate in step with the slabs
+  if constexpr (AHEAD) fetch_all(rx_int<0>{}, rx_int<0>{}, patch, wl);
   for (int s = 0; s < NSLAB; ++s) {
     const int st = s & 1;
-    if (s + 1 < NSLAB) load_slab((s + 1) * CB);
+    const bool more = s + 1 < NSLAB;
+    if (more) load_slab((s + 1) * CB);
     const float* pp = patch + st * PATCH;
     const float* ww = wl + st * WSLAB;
-#pragma unroll
-    for (int tap = 0; tap < TAPS; ++tap) {
-#pragma unroll
-      for (int q = 0; q < NQ; ++q) {
-        const float fw = ww[(tap * NQ + q) * 4 * WST + woff];
-        const int koff = q * 4 * PCH + (tap / KW) * DH * PW + (tap % KW) * DW;
-#pragma unroll
-        for (int pb = 0; pb < NPB; ++pb)
-          acc[pb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pp[poff[pb] + koff], fw, acc[pb], 0, 0, 0);
+    if constexpr (!AHEAD) fetch_all(rx_int<0>{}, rx_int<0>{}, pp, ww);
+    rx_static_for<0, NSTEP>([&](auto KS) {
+      constexpr int ks = decltype(KS)::value;
+      if constexpr (AHEAD && ks == NSTEP / 2) {
+        if (more) {
+          __syncthreads();
+          store_slab(st ^ 1);
+          __syncthreads();
+        }
       }
+      // where the next step's operands come from: this slab, or (last step) the first step of the next one
+      constexpr bool last = ks + 1 == NSTEP;
+      const float* np = last ? patch + (st ^ 1) * PATCH : pp;
+      const float* nw = last ? wl + (st ^ 1) * WSLAB : ww;
+      const bool rd = last ? (AHEAD && more) : true;
+      typedef rx_int<last ? 0 : (ks + 1) % 2> NB_;
+      typedef rx_int<last ? 0 : ks + 1> NK_;
+      if (rd) fetch(NB_{}, NK_{}, -1, np, nw);
+      constexpr int GRP = 5;
+#pragma unroll
+      for (int g = 0; g < NPB; g += GRP) {
+#pragma unroll
+        for (int pb = g; pb < g + GRP && pb < NPB; ++pb) if (rd) fetch(NB_{}, NK_{}, pb, np, nw);
+#pragma unroll
+        for (int pb = g; pb < g + GRP && pb < NPB; ++pb) acc[pb] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[ks % 2][pb], fw[ks % 2], acc[pb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);                     // a few reads, a few MFMAs: the order of the groups stays as written
+      }
+    });
+    if constexpr (!AHEAD) {
+      if (more) store_slab(st ^ 1);
+      __syncthreads();
     }
-    if (s + 1 < NSLAB) store_slab(st ^ 1);
-    __syncthreads();
   }
   // a lane holds pixels 4 (lane / 16) .. + 3 of each block for feature lane % 16 of its wavefront; the epilogue functor
   // (bias, activation, store) takes them at (image, feature, row, first column)

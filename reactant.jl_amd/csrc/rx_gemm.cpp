@@ -279,10 +279,10 @@ ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, in
     if (c.rows == 0 || cost < best) { best = cost; c.rows = (int)tr; }
   }
   if (c.rows == 0) return c;
-  // A workgroup reads its 64 features' whole filter for one tile of one image: with small images (14 x 14: 13 pixel
-  // blocks per image, 0.107 against 0.103 ms for 256 -> 256 features; 7 x 7: 0.152 against 0.099 ms for 512 -> 512) the
-  // matrix product on the window matrix, whose tiles span images, is as fast or faster
-  if (HO * WO < 224) { c.rows = 0; return c; }
+  // A workgroup reads its 64 features' whole filter for one tile of one image: with small images the matrix product
+  // on the window matrix, whose tiles span images, is faster (32 images, 7 x 7, 512 -> 512 features: 0.127 against
+  // 0.099 ms; 14 x 14, 256 -> 256: 0.084 against 0.103 ms).  RX_CONV_MIN_PIXELS moves the limit.
+  if (HO * WO < (getenv("RX_CONV_MIN_PIXELS") ? atoi(getenv("RX_CONV_MIN_PIXELS")) : 128)) { c.rows = 0; return c; }
   if (const char* e = getenv("RX_CONV_ROWS")) {
     const int v = atoi(e);
     if (v >= 1 && v <= HO && (int64_t)v * WO <= 400 && lds_of(v) <= 160 * 1024) c.rows = v;

@@ -277,7 +277,9 @@ CONVS = [
     # 160 output features: three groups of 64 features in the direct kernel's grid
     ([2, 160, 20, 20], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "conv"),
     # small images: the matrix product, whose tiles span images (more than 128 output features: the window matrix is written to memory)
-    ([2, 160, 14, 14], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "gemm_f32"),
+    ([2, 160, 10, 10], [160, 160, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "gemm_f32"),
+    # 14 x 14 images: 13 blocks of 16 pixels per image in the direct kernel
+    ([3, 96, 14, 14], [96, 96, 3, 3], "f32", None, dict(padding=[[1, 1], [1, 1]]), "conv"),
     # bf16 with more than 128 output features: the window matrix is written to memory instead of being evaluated by the product
     ([2, 160, 14, 14], [160, 160, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
 ]
