@@ -279,13 +279,27 @@ ConvChoice choose_conv(int64_t B, int64_t C, int64_t H, int64_t W, int64_t O, in
     if (c.rows == 0 || cost < best) { best = cost; c.rows = (int)tr; }
   }
   if (c.rows == 0) return c;
-  // A workgroup reads its 64 features' whole filter for one tile of one image: with small images the matrix product
-  // on the window matrix, whose tiles span images, is faster (32 images, 7 x 7, 512 -> 512 features: 0.127 against
-  // 0.099 ms; 14 x 14, 256 -> 256: 0.084 against 0.103 ms).  RX_CONV_MIN_PIXELS moves the limit.
-  if (HO * WO < (getenv("RX_CONV_MIN_PIXELS") ? atoi(getenv("RX_CONV_MIN_PIXELS")) : 128)) { c.rows = 0; return c; }
   if (const char* e = getenv("RX_CONV_ROWS")) {
     const int v = atoi(e);
     if (v >= 1 && v <= HO && (int64_t)v * WO <= 400 && lds_of(v) <= 160 * 1024) c.rows = v;
+  }
+  // Against the matrix product on the window matrix, whose tiles span images and which can slice the channels: a
+  // workgroup of this kernel passes all channels of its 64 features through LDS for one tile of one image, about 1.5 us
+  // per slab however few pixels the tile has.  Estimates in microseconds, fitted to 3 x 3 layers of 64 to 512 features
+  // on 7 x 7 to 56 x 56 images in batches of 4 and 32 (512 -> 512 on 14 x 14, 4 images: 0.097 ms direct against 0.055;
+  // 32 images of 256 -> 256: 0.086 against 0.103): slabs of max(1.5 us, 1.35 x their MFMA time) here; 70 TFLOP/s, a
+  // window matrix written and read when there are more than 128 features, a layout map of the result and two more
+  // launches there.
+  {
+    const int64_t tiles = (HO + c.rows - 1) / c.rows, npb = (c.rows * WO + 15) / 16;
+    const double rounds = (double)((B * tiles * groups + 255) / 256);
+    const double nslab = (double)((C + slab - 1) / slab), nstep = (double)(KH * KW * (slab / 4));
+    const double direct_us = rounds * nslab * std::max(1.5, 1.35 * (double)npb * nstep * 32.0 / 2200.0) + 5.0;
+    const double flops = 2.0 * (double)B * (double)O * (double)HO * (double)WO * (double)C * (double)(KH * KW);
+    const double window_bytes = O > 128 ? 2.0 * 4.0 * (double)B * (double)C * (double)(KH * KW) * (double)HO * (double)WO : 0.0;
+    const double product_us = flops / 70e6 + (window_bytes + 2.0 * 4.0 * (double)B * (double)O * (double)HO * (double)WO) / 5e6 + 5.0 + 8.0;   // three launches
+    const char* force = getenv("RX_CONV_DIRECT");   // 2: this kernel wherever it covers the case
+    if (direct_us > product_us && !(force && atoi(force) == 2)) { c.rows = 0; return c; }
   }
   c.slab = slab;
   c.grid[0] = (unsigned)(B * ((HO + c.rows - 1) / c.rows));
