@@ -239,7 +239,14 @@ RX_DEV bool rx_gemm_tile(unsigned bid, int* bm, int* bn) {
 // An operand can also be a functor (LA / LB other than rx_no_fn): the fusion code generator
 // writes one when the operand is a cheap expansion of smaller data (the window matrix of a
 // convolution, a broadcast), so that the expanded matrix never exists in memory.
-struct rx_no_fn { static constexpr bool none = true; static constexpr int vec_width = 0; };
+struct rx_no_fn {
+  static constexpr bool none = true;
+  static constexpr int vec_width = 0;
+  static constexpr int C = 0;                 // as a K-offset functor: none
+  RX_DEV unsigned at(int) { return 0u; }
+  RX_DEV int row(int) { return 0; }
+  RX_DEV int col(int) { return 0; }
+};
 
 template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
           class LA = rx_no_fn, class LB = rx_no_fn>
@@ -571,7 +578,7 @@ RX_DEV void rx_tile_load_direct(const E* __restrict__ g, long long gld, int row0
 // SPLIT > 1: workgroup (x, y) contracts the y-th of SPLIT equal slices of K and hands the epilogue
 // (y, m, n): partial products that a reduction over the leading index adds up (few output tiles, long K).
 template <class MMA, int BM, int BN, int BK, int WM, int WN, int S, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
-          int SPLIT = 1>
+          int SPLIT = 1, class KOff = rx_no_fn>
 RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi) {
   typedef typename MMA::elem E;
   typedef rx_mma_traits<MMA> TRAITS;
@@ -609,7 +616,12 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
   auto issue = [&](int kt) {
     RX_LDS E* st = lds + (kt % S) * STAGE;
     const int k0 = kbase + kt * BK;
-    if (A_KC) rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, A_GLD, m0, k0, M, K, st, tid);
+    if constexpr (!KOff::none) {
+      // row shifts (rx_tap_shift): the first operand has KOff::C columns; a shifted row beyond its last one belongs to a
+      // result that the epilogue does not keep, so the clamped read is as good as a zero
+      static_assert(A_KC && !BATCHED && SPLIT == 1 && BK * (int)sizeof(E) == 128, "row shifts: [row][k] operand, K tiles of 128 bytes");
+      rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, (long long)KOff::C, m0 + KOff::row(kt), KOff::col(kt), M, KOff::C, st, tid);
+    } else if (A_KC) rx_tile_load_direct<E, A_ROWS, A_COLS, NT, true>(Ab, A_GLD, m0, k0, M, K, st, tid);
     else rx_tile_load_direct<E, A_ROWS, A_COLS, NT, false, TRAITS::TR_SWZ>(Ab, A_GLD, k0, m0, K, M, st, tid);
     if (B_KC) rx_tile_load_direct<E, B_ROWS, B_COLS, NT, true>(Bb, B_GLD, n0, k0, N, K, st + A_SZ, tid);
     else rx_tile_load_direct<E, B_ROWS, B_COLS, NT, false, TRAITS::TR_SWZ>(Bb, B_GLD, k0, n0, K, N, st + A_SZ, tid);
@@ -918,7 +930,29 @@ struct rx_phase_probe {
   }
 };
 
-template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2, class Probe = rx_no_fn>
+// A product whose first operand is read through row shifts (KOff of the streaming bodies): K is cut into taps of C
+// elements, and tap t = (ty, tx) of a KW-wide window contracts rows m + ty * SY + tx * SX of a matrix of C columns with
+// columns t * C .. t * C + C - 1 of the second operand; rows beyond the matrix read as zeros.  With the matrix a zero-
+// padded image in [image, row, column, channel] order and SY the padded row length this is a convolution with unit
+// strides, evaluated on the padded grid: no window matrix exists, the operand tiles still arrive as plain buffer loads
+// with a scalar offset per K tile.
+template <int C_, int KW_, int SY_, int SX_, int ESZ_>
+struct rx_tap_shift {
+  static constexpr bool none = false;
+  static constexpr int C = C_;                                // elements per row of the first operand
+  static constexpr int CT = C_ * ESZ_ / 128;                  // K tiles per tap
+  static_assert(C_ * ESZ_ % 128 == 0, "a tap is whole K tiles");
+  // byte offset of K tile kt, to be added to (row of the tile) * C * ESZ
+  RX_DEV unsigned at(int kt) {
+    const int tap = kt / CT, part = kt % CT;
+    return (unsigned)((tap / KW_) * SY_ + (tap % KW_) * SX_) * (unsigned)(C_ * ESZ_) + (unsigned)part * 128u;
+  }
+  // the same as a row shift and a first column (elements)
+  RX_DEV int row(int kt) { const int tap = kt / CT; return (tap / KW_) * SY_ + (tap % KW_) * SX_; }
+  RX_DEV int col(int kt) { return (kt % CT) * (128 / ESZ_); }
+};
+
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, int D = 2, int NSTG = 2, class Probe = rx_no_fn, class KOff = rx_no_fn>
 RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, const Probe& probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NBUF = 4;
@@ -932,7 +966,9 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
   typedef rx_dma_s<EL, A_ROWS, A_COLS, NT, A_KC> DMA_A;
   typedef rx_dma_s<EL, B_ROWS, B_COLS, NT, B_KC> DMA_B;
   constexpr int NLT = DMA_A::NL + DMA_B::NL;   // direct loads per thread and K tile
-  static_assert((long long)M * K * ESZ < (1ll << 32) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
+  constexpr long long AROW = KOff::none ? (long long)K : (long long)KOff::C;   // elements per row of the first operand as stored
+  static_assert(KOff::none || (A_KC && !BATCHED), "row shifts: the first operand is [row][k]");
+  static_assert((long long)M * AROW * ESZ < (1ll << 31) * (KOff::none ? 2 : 1) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
   static_assert(K % BK == 0, "whole K tiles");
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
   RX_LDS rx_u8* const ldsa = (RX_LDS rx_u8*)rx_smem;
@@ -945,7 +981,7 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
   if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
   const int m0 = bm * BM, n0 = bn * BN;
   const long long batch = BATCHED ? blockIdx.y : 0;
-  constexpr unsigned A_GLDB = (A_KC ? K : M) * ESZ, B_GLDB = (B_KC ? K : N) * ESZ;
+  constexpr unsigned A_GLDB = (A_KC ? (unsigned)AROW : M) * ESZ, B_GLDB = (B_KC ? K : N) * ESZ;
   constexpr int KT = K / BK;
   constexpr unsigned KA = A_KC ? BKB : BK * A_GLDB, KB = B_KC ? BKB : BK * B_GLDB;   // byte step of one K tile
 
@@ -957,12 +993,13 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 
   DMA_A dma_a;
   DMA_B dma_b;
-  dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * K * ESZ), tid);
+  dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * AROW * ESZ), tid);
   dma_b.init(B + batch * (long long)N * K, B_GLDB, B_KC ? n0 : n0 * ESZ, (unsigned)((long long)N * K * ESZ), tid);
   // tile kt lies in stage kt % NSTG of both operands
   // (st is a constant at every call, so the stage's offset folds into the instruction)
   auto issue = [&](int kt, int st) __attribute__((always_inline)) {
-    dma_a.issue((unsigned)kt * KA, ldsa + st * A_SZ, wave);
+    if constexpr (KOff::none) dma_a.issue((unsigned)kt * KA, ldsa + st * A_SZ, wave);
+    else dma_a.issue(KOff::at(kt), ldsa + st * A_SZ, wave);
     dma_b.issue((unsigned)kt * KB, ldsb + st * B_SZ, wave);
   };
   rx_i32x8 fa[NBUF], fb[2][NB];
@@ -1108,7 +1145,7 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 // bf16 8192 x 4096 x 4096 [m][k] x [k][n] with bias + GELU 199.7 -> 190.0 us, K = 1024: 65.6 -> 64.6 us; e4m3 8192^3
 // [m][k] x [n][k] 386 -> 360 us (with group 0 requesting both operands: 411).
 // ---------------------------------------------------------------------------
-template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, class Probe = rx_no_fn>
+template <class EL, int BM, int BN, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi, class Probe = rx_no_fn, class KOff = rx_no_fn>
 RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typename EL::elem* __restrict__ B, const Epi& epi, Probe probe = Probe()) {
   constexpr int ESZ = sizeof(typename EL::elem);
   constexpr int BKB = 128, BK = BKB / ESZ, NSTG = 2;
@@ -1125,7 +1162,9 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
   constexpr int NL0 = B_KC ? NLA : NLA + NLB;                // requests per thread of group 0 and K tile
   constexpr int NFR = NA + NB;                               // fragments per wavefront and K tile
   static_assert(WM == 2 && WN == 4, "wavefronts w and w + 4 share a SIMD and a column of B");
-  static_assert((long long)M * K * ESZ < (1ll << 32) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
+  constexpr long long AROW = KOff::none ? (long long)K : (long long)KOff::C;   // elements per row of the first operand as stored
+  static_assert(KOff::none || (A_KC && !BATCHED), "row shifts: the first operand is [row][k]");
+  static_assert((long long)M * AROW * ESZ < (1ll << 31) * (KOff::none ? 2 : 1) && (long long)N * K * ESZ < (1ll << 32), "32-bit operand offsets");
   constexpr int KT = K / BK;
   static_assert(K % BK == 0 && KT >= 2 && KT % 2 == 0, "an even number of whole K tiles");
   extern __shared__ __attribute__((aligned(16))) unsigned char rx_smem[];
@@ -1140,7 +1179,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
   if (!rx_gemm_tile<GM, GN, RB, CB>(blockIdx.x, &bm, &bn)) return;
   const int m0 = bm * BM, n0 = bn * BN;
   const long long batch = BATCHED ? blockIdx.y : 0;
-  constexpr unsigned A_GLDB = (A_KC ? K : M) * ESZ, B_GLDB = (B_KC ? K : N) * ESZ;
+  constexpr unsigned A_GLDB = (A_KC ? (unsigned)AROW : M) * ESZ, B_GLDB = (B_KC ? K : N) * ESZ;
   constexpr unsigned KA = A_KC ? BKB : BK * A_GLDB, KB = B_KC ? BKB : BK * B_GLDB;
 
   rx_f32x4v acc[NA][NB];
@@ -1150,7 +1189,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
     for (int j = 0; j < NB; ++j) acc[i][j] = rx_f32x4v{0.f, 0.f, 0.f, 0.f};
   DMA_A dma_a;
   DMA_B dma_b;
-  dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * K * ESZ), tid & (NTL - 1));
+  dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * AROW * ESZ), tid & (NTL - 1));
   // [n][k]: slot `lane` of a wavefront's request q is row 8 q + lane / 8 of its rows, position lane % 8, and the swizzle
   // puts chunk c of row r at position c ^ ((r / 2) & 7): for odd q (row bit 3 set) bit 2 of the chunk flips
   unsigned slab0 = 0, slab1 = 0;
@@ -1164,7 +1203,10 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
   rx_i32x8 fa[NA], fb[NB];
   // request q of a tile by group 0: those of A first (st and q are constants at every call)
   auto request = [&](int kt, int st, int q) __attribute__((always_inline)) {
-    if (q < NLA) dma_a.one(q, (unsigned)kt * KA, ldsa + st * A_SZ, wave);
+    if (q < NLA) {
+      if constexpr (KOff::none) dma_a.one(q, (unsigned)kt * KA, ldsa + st * A_SZ, wave);
+      else dma_a.one(q, KOff::at(kt), ldsa + st * A_SZ, wave);
+    }
     else if constexpr (!B_KC) dma_b.one(q - NLA, (unsigned)kt * KB, ldsb + st * B_SZ, wave);
   };
   // request q of this wavefront's rows of B ([n][k])

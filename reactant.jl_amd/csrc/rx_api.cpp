@@ -991,7 +991,7 @@ RX_EXPORT void RxExecutableCostAnalysis(RxExecutable* ex, float* props11) {
     const rx::Plan& P = ex->plan;
     double optimal = 0;
     for (auto& L : P.launches) {
-      const double peak = L.kind == "gemm_f8" ? 5.0e15 : (L.kind == "gemm_bf16" || L.kind == "gemm_f16") ? 2.5e15 : L.kind == "gemm_f64" ? 78.6e12 : 157.3e12;
+      const double peak = L.kind == "gemm_f8" ? 5.0e15 : (L.kind == "gemm_bf16" || L.kind == "gemm_f16" || L.kind == "conv_bf16" || L.kind == "conv_f16") ? 2.5e15 : L.kind == "gemm_f64" ? 78.6e12 : 157.3e12;
       optimal += std::max(L.flops / peak, L.algo_bytes / 8.0e12);
     }
     const double mem_time = P.hlo_bytes_accessed / 8.0e12;

@@ -191,6 +191,7 @@ GemmChoice choose_gemm(DT a, DT b, DT out, int64_t batch, int64_t M, int64_t N, 
         << (b_kc ? "true" : "false") << ", " << M << ", " << N << ", " << K << ", " << rb << ", " << cb;
       c.targs = t.str();
       c.skeleton = "rx_gemm_body_dl";
+      c.bk = dbk;
       c.stype_a = dmma + "::elem";
       c.ok = true;
       return c;

@@ -18,6 +18,7 @@ struct GemmChoice {
   int split = 1;            // slices of K, one per blockIdx.y (partial products; rx_gemm_body_dl only)
   int depth = 0;            // rx_gemm_body_s: blocks of the streamed operand read ahead (0: the skeleton's default)
   int stream_stages = 0;    // rx_gemm_body_s: LDS stages per operand (0: not that skeleton)
+  int bk = 0;               // rx_gemm_body_dl: elements of K per tile
 };
 
 // Workgroups to launch for a gm x gn grid of tiles: the kernels walk the tiles in blocks of 4 x 8,

@@ -1809,8 +1809,9 @@ struct Planner {
     const int es_out = info(rn.ty.dt).size;
     int V = (es_out == 2 || es_out == 4 || es_out == 8) ? 16 / es_out : 1;
     for (auto& kv : staged) if ((int)info(g.nodes[kv.first].ty.dt).size != es_out) V = 1;
-    if (V > 1 && (q < 0 || dims[q] % V != 0 || dims[n - 1] % V != 0 || dims[q] < 64 || dims[n - 1] < 64 || !opt.transpose_vectors)) V = 1;
-    const int TQ = TS, TM = V > 1 ? (es_out == 8 ? 64 : 128) : TS, LD = V > 1 ? TQ + V : TS + 1;
+    if (V > 1 && (q < 0 || dims[q] % V != 0 || dims[n - 1] % V != 0 || dims[q] < 64 || dims[n - 1] < 32 || !opt.transpose_vectors)) V = 1;
+    // a minor dimension of at most 64 (the rows of a 56 x 56 image) takes tiles of 64 rows: 128 would be half empty
+    const int TQ = TS, TM = V > 1 ? ((es_out == 8 || dims[n - 1] <= 64) ? 64 : 128) : TS, LD = V > 1 ? TQ + V : TS + 1;
     int64_t lds_total = 0;
     for (auto& kv : staged) lds_total += (int64_t)TM * LD * info(g.nodes[kv.first].ty.dt).size;
     if (lds_total > 64 * 1024) return false;
@@ -2719,9 +2720,13 @@ struct Planner {
     const Node& rn = g.nodes[root];
     const TType& xt = g.nodes[cn.in[0]].ty;
     const TType& wt = g.nodes[cn.in[1]].ty;
-    const ConvChoice cc = choose_conv(xt.dims[0], xt.dims[1], xt.dims[2], xt.dims[3], wt.dims[0], wt.dims[2], wt.dims[3], cn.ty.dims[2], cn.ty.dims[3], cn.a0[2],
-                                      cn.a1[0], cn.a1[1], cn.a2[0], cn.a2[1]);
-    if (!cc.ok) throw Error("internal: convolution node without a tiling");
+    const bool shifted = !cn.a3.empty();   // the product with row shifts (16-bit images)
+    ConvChoice cc;
+    if (!shifted) {
+      cc = choose_conv(xt.dims[0], xt.dims[1], xt.dims[2], xt.dims[3], wt.dims[0], wt.dims[2], wt.dims[3], cn.ty.dims[2], cn.ty.dims[3], cn.a0[2],
+                       cn.a1[0], cn.a1[1], cn.a2[0], cn.a2[1]);
+      if (!cc.ok) throw Error("internal: convolution node without a tiling");
+    }
     const int n = rn.ty.rank();
     Emitter em(g, [&](int x) { return mat[x] && x != root; });
     em.excess_precision = opt.excess_precision;
@@ -2744,8 +2749,17 @@ struct Planner {
       o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
     o << "  " << ost << "* __restrict__ out0;\n";
     o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const float (&acc)[NV]";
-    for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
-    o << ") const {\n";
+    if (shifted) {
+      // called with (row of the product, first column): the row is a position of the padded grid, of which the
+      // result keeps the first HO rows and WO columns of every image
+      if (n != 4) throw Error("internal: shifted product with a result of another rank");
+      o << ", " << it << " row_, " << it << " i3b) const {\n";
+      o << "    const " << it << " i2 = row_ % " << cn.a3[4] << ", i1 = (row_ / " << cn.a3[4] << ") % " << cn.a3[3] << ", i0 = row_ / " << cn.a3[3] * cn.a3[4] << ";\n";
+      o << "    if (i1 >= " << rn.ty.dims[1] << " || i2 >= " << rn.ty.dims[2] << ") return;\n";
+    } else {
+      for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
+      o << ") const {\n";
+    }
     {
       Index rix = root_index(rn.ty.dims);
       rix[n - 1].var = "i" + std::to_string(n - 1) + "b";
@@ -2764,6 +2778,45 @@ struct Planner {
     o << "      res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n    }\n";
     o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
     o << "  }\n};\n\n";
+    if (shifted) {
+      // [rows of the padded images, C] x [O, taps * C] -> [rows, O] on a streaming GEMM skeleton whose K tiles of the
+      // first operand carry the tap's row shift (rx_tap_shift)
+      if (rn.ty.dims != cn.ty.dims || cn.ty.dims[0] * cn.a3[3] * cn.a3[4] != xt.dims[0]) throw Error("internal: shifted product with a result of another shape");
+      const GemmChoice gc = choose_gemm(xt.dt, wt.dt, cn.ty.dt, 1, xt.dims[0], wt.dims[0], wt.dims[1], true, true);
+      const bool dl = gc.skeleton == "rx_gemm_body_dl";
+      if (!gc.ok || (gc.skeleton != "rx_gemm_body_pp" && gc.skeleton != "rx_gemm_body_s" && !(dl && gc.bk * (int)info(xt.dt).size == 128 && gc.split == 1)))
+        throw Error("internal: shifted product without a skeleton that loads tiles straight into LDS");
+      o << "// convolution as a product with row shifts: " << xt.str() << " x " << wt.str() << " -> " << cn.ty.str() << ", window " << wt.dims[1] / xt.dims[1] / cn.a3[0] << " x " << cn.a3[0]
+        << ", row shifts " << cn.a3[1] << " / " << cn.a3[2] << "\n";
+      o << "extern \"C\" __global__ __launch_bounds__(" << gc.block << ") void @K@_conv(const " << gc.stype_a << "* __restrict__ A, const " << gc.stype_a << "* __restrict__ B";
+      for (size_t k = 0; k < em.inputs.size(); ++k) o << ", const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ e" << k;
+      o << ", " << ost << "* __restrict__ out0) {\n";
+      o << "  @K@_epi epi{";
+      for (size_t k = 0; k < em.inputs.size(); ++k) o << "e" << k << ", ";
+      o << "out0};\n";
+      o << "  " << gc.skeleton << "<" << gc.targs << ", false, @K@_epi";
+      if (gc.depth > 0) o << ", " << gc.depth;
+      if (gc.stream_stages > 0) o << ", " << gc.stream_stages;
+      o << (dl ? ", 1" : ", rx_no_fn") << ", rx_tap_shift<" << xt.dims[1] << ", " << cn.a3[0] << ", " << cn.a3[1] << ", " << cn.a3[2] << ", " << info(xt.dt).size << ">>(A, B, epi);\n}\n\n";
+      const std::string kb = finalize(o.str());
+      Launch L;
+      L.kernel = named("@K@_conv", kb);
+      L.kind = "conv_" + gc.kind.substr(5);   // conv_bf16, conv_f16
+      L.grid[0] = gc.grid[0]; L.grid[1] = gc.grid[1]; L.grid[2] = gc.grid[2];
+      L.block[0] = gc.block;
+      L.lds_bytes = gc.lds_bytes;
+      L.args.push_back(buffer_for(cn.in[0]));
+      L.args.push_back(buffer_for(cn.in[1]));
+      for (int i : em.inputs) L.args.push_back(buffer_for(i));
+      L.args.push_back(buffer_for(root));
+      std::vector<int> all_in{cn.in[0], cn.in[1]};
+      for (int i : em.inputs) if (std::find(all_in.begin(), all_in.end(), i) == all_in.end()) all_in.push_back(i);
+      L.algo_bytes = algo_bytes(all_in, {root});
+      L.flops = 2.0 * (double)cn.ty.numel() * (double)wt.dims[1];   // of the results that are kept
+      L.desc = describe(root);
+      plan.launches.push_back(L);
+      return;
+    }
     o << "// direct convolution: " << xt.str() << " * " << wt.str() << " -> " << cn.ty.str() << ", " << cc.rows << " rows of the result per workgroup, channels in slabs of " << cc.slab << "\n";
     o << "extern \"C\" __global__ __launch_bounds__(256) void @K@_conv(const float* __restrict__ X, const float* __restrict__ Wt";
     for (size_t k = 0; k < em.inputs.size(); ++k) o << ", const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ e" << k;
@@ -4371,7 +4424,7 @@ static void count_hlo_costs(const Graph& g, Plan* plan) {
       }
       case OpK::Conv: {
         const TType& wt = g.nodes[n.in[1]].ty;
-        flops += 2.0 * numel * (double)(wt.dims[1] * wt.dims[2] * wt.dims[3]);
+        flops += 2.0 * numel * (double)(wt.rank() == 2 ? wt.dims[1] : wt.dims[1] * wt.dims[2] * wt.dims[3]);
         break;
       }
       case OpK::Reduce: case OpK::Scan: flops += (double)g.nodes[n.in[0]].ty.numel(); break;

@@ -267,6 +267,19 @@ CONVS = [
     # a 1x1 filter (a product over the channels), 7x7 images, bias + relu
     ([8, 128, 16, 16], [96, 128, 1, 1], "f32", None, dict(epilogue="bias_relu"), "conv"),
     ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
+    # 16-bit images with whole 128-byte runs of channels, unit strides: a product over the zero-padded [image, row, column,
+    # channel] data with one row shift per tap (no window matrix) -- 64 x 64 and 128 x 64 tiles of the direct-to-LDS skeleton,
+    ([2, 64, 40, 40], [128, 64, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "conv_bf16"),
+    ([4, 64, 64, 64], [64, 64, 5, 5], "bf16", None, dict(padding=[[2, 2], [2, 2]], flip=True), "conv_bf16"),
+    # f16, a dilated 2 x 3 filter, uneven padding; a 1 x 1 filter; channels-last images and [rows, columns, in, out] filters
+    ([2, 128, 30, 26], [64, 128, 2, 3], "f16", None, dict(padding=[[0, 1], [2, 0]], rhs_dil=[2, 1]), "conv_f16"),
+    ([2, 64, 24, 24], [128, 64, 1, 1], "bf16", None, dict(), "conv_bf16"),
+    ([2, 20, 16, 64], [3, 3, 64, 128], "bf16", "[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]", dict(padding=[[1, 1], [1, 1]]), "conv_bf16"),
+    # the streaming skeletons: 256 x 128 tiles, and 256 x 256 tiles in the ping-pong form
+    ([8, 64, 94, 94], [128, 64, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "conv_bf16"),
+    ([4, 64, 90, 90], [512, 64, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "conv_bf16"),
+    # the same data through the window matrix
+    ([2, 64, 40, 40], [128, 64, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu", env={"RX_CONV_SHIFT": "0"}), "gemm_bf16"),
     ([1, 3, 33, 35], [16, 3, 5, 5], "f32", None, dict(strides=[2, 2], padding=[[2, 2], [2, 2]]), "gemm_f32"),
     ([16, 16, 8, 2], [4, 4, 8, 4], "f32", "[1, 0, f, b]x[1, 0, i, o]->[1, 0, f, b]", dict(), None),
     ([2, 16, 16, 8], [4, 4, 8, 4], "f32", "[b, 1, 0, f]x[1, 0, i, o]->[b, 1, 0, f]", dict(padding=[[1, 2], [0, 1]]), None),

@@ -40,6 +40,9 @@ def corpus():
         "maxpool": NN.reduce_window([4, 8, 32, 32], "f32", "maximum", [1, 1, 2, 2], strides=[1, 1, 2, 2])[0],
         "conv": NN.convolution([2, 8, 16, 16], [4, 8, 3, 3], "f32", padding=[[1, 1], [1, 1]])[0],
         "conv_groups": NN.convolution([2, 8, 16, 16], [4, 4, 3, 3], "f32", groups=2)[0],
+        "conv_direct": NN.convolution([32, 64, 56, 56], [64, 64, 3, 3], "f32", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0],
+        "conv_shifted": NN.convolution([32, 256, 56, 56], [256, 256, 3, 3], "bf16", padding=[[1, 1], [1, 1]], epilogue="bias_relu")[0],
+        "conv_shifted_small": NN.convolution([2, 20, 16, 64], [3, 3, 64, 128], "f16", padding=[[1, 0], [2, 1]], rhs_dil=[1, 2], dims="[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]")[0],
         "vgg": NN.vgg_block(), "attention": NN.attention_block(),
         "argmax": NN.argreduce([64, 100], "f32", 1),
         "pool_grad": NN.select_and_scatter([2, 4, 16, 16], "f32", [1, 1, 2, 2], strides=[1, 1, 2, 2]),
