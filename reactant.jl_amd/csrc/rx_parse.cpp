@@ -1972,25 +1972,28 @@ struct Builder {
         return cur;
       }
     }
-    // 16-bit images with two spatial dims, unit strides, no input dilation, no groups, non-negative padding and whole
-    // 128-byte K tiles of channels: the images are zero-padded and laid out [image, row, column, channel], the filter
+    // 16-bit images with two spatial dims, unit strides, no input dilation, no groups and non-negative padding, whose
+    // channels are whole 128-byte K tiles or can be padded to that: the images are zero-padded and laid out [image, row, column, channel], the filter
     // [feature, tap, channel], and the convolution is a matrix product whose first operand is read through one row
     // shift per tap (OpK::Conv with a3; rx_tap_shift in kernels/rx_gemm_kernels.h) -- evaluated on the padded grid,
     // [image, padded row, padded column, feature], from which the result is sliced and transposed.  No window matrix
     // exists.  Taken where the product gets a GEMM skeleton that loads its tiles straight into LDS; RX_CONV_SHIFT=0
     // keeps the window matrix.
     if (nsp == 2 && (xct.dt == DT::BF16 || xct.dt == DT::F16) && G == 1 && BG == 1 && st[0] == 1 && st[1] == 1 && ld[0] == 1 && ld[1] == 1 && rd[0] >= 1 && rd[1] >= 1 &&
-        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1 && (C * 2) % 128 == 0 && O % 8 == 0 &&
+        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1 && 2 * ((C + 63) / 64 * 64) <= 3 * C && O % 8 == 0 &&
         !(getenv("RX_CONV_SHIFT") && atoi(getenv("RX_CONV_SHIFT")) == 0) && !(getenv("RX_MFMA") && atoi(getenv("RX_MFMA")) == 0)) {
       const int64_t KH = wct.dims[2], KW = wct.dims[3];
       const int64_t HP = xct.dims[2] + pad[0] + pad[1], WP = xct.dims[3] + pad[2] + pad[3];
       const int64_t HO = HP - (KH - 1) * rd[0], WO = WP - (KW - 1) * rd[1];
-      const int64_t MP = B * HP * WP, KK = KH * KW * C;
+      // channels that are not whole K tiles (96, 160) are padded with zero channels to the next multiple of 64, in the
+      // images and in the filter, when that adds at most half
+      const int64_t CP = (C + 63) / 64 * 64;
+      const int64_t MP = B * HP * WP, KK = KH * KW * CP;
       GemmChoice gc;
       // few results and a long contraction: the product on the window matrix is cut along K (split_dots in the planner,
       // the same test), which this form is not (512 -> 512 features on four 14 x 14 images: 0.026 against 0.061 ms)
       const bool sliced = ((B * HO * WO + 63) / 64) * ((O + 63) / 64) < 256 && KK >= 1024 && !(getenv("RX_SPLIT_K") && atoi(getenv("RX_SPLIT_K")) == 0);
-      if (HO >= 1 && WO >= 1 && !sliced && MP * C * 2 < ((int64_t)1 << 31) && O * KK * 2 < ((int64_t)1 << 31) && KH * KW <= 1024)
+      if (HO >= 1 && WO >= 1 && !sliced && MP * CP * 2 < ((int64_t)1 << 31) && O * KK * 2 < ((int64_t)1 << 31) && KH * KW <= 1024)
         gc = choose_gemm(xct.dt, xct.dt, xct.dt, 1, MP, O, KK, true, true);
       if (gc.ok && (gc.skeleton == "rx_gemm_body_pp" || gc.skeleton == "rx_gemm_body_s" || (gc.skeleton == "rx_gemm_body_dl" && gc.bk * 2 == 128 && gc.split == 1))) {
         std::vector<int64_t> want(r);
@@ -1998,15 +2001,20 @@ struct Builder {
         if (want != out.dims) fail("convolution: result shape mismatch");
         auto add_node = [&](OpK k, std::vector<int> in, TType t) { Node n; n.k = k; n.in = std::move(in); n.ty = std::move(t); return n; };
         int xi = xc;
-        if (pad[0] || pad[1] || pad[2] || pad[3]) {
-          Node pn = add_node(OpK::Pad, {xi, zero_of(xct.dt)}, TType{xct.dt, {B, C, HP, WP}});
-          pn.a0 = {0, 0, pad[0], pad[2]}; pn.a1 = {0, 0, pad[1], pad[3]}; pn.a2 = {0, 0, 0, 0};
+        if (pad[0] || pad[1] || pad[2] || pad[3] || CP != C) {
+          Node pn = add_node(OpK::Pad, {xi, zero_of(xct.dt)}, TType{xct.dt, {B, CP, HP, WP}});
+          pn.a0 = {0, 0, pad[0], pad[2]}; pn.a1 = {0, CP - C, pad[1], pad[3]}; pn.a2 = {0, 0, 0, 0};
           xi = g.add(pn);
         }
-        { Node t = add_node(OpK::Transpose, {xi}, TType{xct.dt, {B, HP, WP, C}}); t.a0 = {0, 2, 3, 1}; xi = g.add(t); }
-        xi = g.add(add_node(OpK::Reshape, {xi}, TType{xct.dt, {MP, C}}));
+        { Node t = add_node(OpK::Transpose, {xi}, TType{xct.dt, {B, HP, WP, CP}}); t.a0 = {0, 2, 3, 1}; xi = g.add(t); }
+        xi = g.add(add_node(OpK::Reshape, {xi}, TType{xct.dt, {MP, CP}}));
         int wi = wc;
-        { Node t = add_node(OpK::Transpose, {wi}, TType{xct.dt, {O, KH, KW, C}}); t.a0 = {0, 2, 3, 1}; wi = g.add(t); }
+        if (CP != C) {
+          Node pn = add_node(OpK::Pad, {wi, zero_of(xct.dt)}, TType{xct.dt, {O, CP, KH, KW}});
+          pn.a0 = {0, 0, 0, 0}; pn.a1 = {0, CP - C, 0, 0}; pn.a2 = {0, 0, 0, 0};
+          wi = g.add(pn);
+        }
+        { Node t = add_node(OpK::Transpose, {wi}, TType{xct.dt, {O, KH, KW, CP}}); t.a0 = {0, 2, 3, 1}; wi = g.add(t); }
         wi = g.add(add_node(OpK::Reshape, {wi}, TType{xct.dt, {O, KK}}));
         // the kernel's epilogue keeps the rows of the padded grid that are results and writes them side by side:
         // [B, HO, WO, O]

@@ -291,7 +291,10 @@ def test_windowed_ops_plan(monkeypatch):
     assert "conv_bf16" in kinds(rep) and "rx_gemm_body_dl<rx_mma_bf16_16, 128, 128, 64, " in rep and ", 1, rx_tap_shift<256, 3, 58, 1, 2>>" in rep, rep
     # not that form: strides, channels that are not whole 128-byte runs, a product that is cut along K, the switch
     assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([32, 64, 56, 56], [128, 64, 3, 3], "bf16", strides=[2, 2], padding=[[1, 1], [1, 1]])[0]))
-    assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([32, 96, 56, 56], [128, 96, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0]))
+    assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([32, 32, 56, 56], [128, 32, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0]))
+    # 96 channels: padded with zero channels to 128, in the images' layout map and in the filter's
+    rep = rx.compile_offline(NN.convolution([32, 96, 56, 56], [128, 96, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0], with_source=True)
+    assert "conv_bf16" in kinds(rep) and "rx_tap_shift<128, 3, 58, 1, 2>>" in rep, rep
     assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([4, 512, 14, 14], [512, 512, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0]))
     monkeypatch.setenv("RX_CONV_SHIFT", "0")
     assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([32, 256, 56, 56], [256, 256, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0]))
