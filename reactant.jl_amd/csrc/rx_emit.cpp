@@ -181,6 +181,7 @@ std::string Emitter::emit_load(int node, const Index& ix) {
   int slot = slot_of(node);
   LoadRecord rec;
   rec.node = node;
+  rec.minor_follows = !dims.empty() && !root_vars_.empty() && ix[dims.size() - 1].var == root_vars_.back();
   if (dims.size() == root_vars_.size() && !dims.empty()) {
     rec.affine = true;
     for (size_t d = 0; d < dims.size(); ++d) {
@@ -799,6 +800,26 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
       std::string cond;
       for (auto& c : conds) cond += (cond.empty() ? "" : " && ") + c;
       if (cond.empty()) cond = "true";
+      if (clamp_guards && pre.empty()) {
+        // Reads at positions clamped into the operand and a select instead of a branch: the loads of a lane's
+        // consecutive elements are then unconditional and at consecutive addresses, and the compiler combines them
+        // into one vector load (under a branch of their own, eight 16-bit elements are eight loads).
+        Index ci = oi;
+        for (size_t d = 0; d < ix.size(); ++d) {
+          const int64_t sd = o.ty.dims[d];
+          const Ix q0 = shifted(ix[d], -n.a0[d]);
+          if (q0.lo >= 0 && q0.hi <= sd - 1) continue;
+          Ix t;
+          t.var = fresh("t");
+          t.lo = std::max<int64_t>(q0.lo, 0);
+          t.hi = std::min<int64_t>(q0.hi, sd - 1);
+          line("const " + idx_t() + " " + t.var + " = rx_min<" + idx_t() + ">(rx_max<" + idx_t() + ">(" + q0.str() + ", 0), " + std::to_string(sd - 1) + ");");
+          ci[d] = t;
+        }
+        std::string inner = emit(n.in[0], ci);
+        line("const " + CT + " " + v + " = (" + cond + ") ? " + inner + " : " + pv + ";");
+        return v;
+      }
       if (branchless_guards) {
         const int unsafe0 = unsafe_loads_;
         const std::string before = take_code();

@@ -34,6 +34,7 @@ struct LoadRecord {
   // per input dimension: which root variable indexes it with offset 0 (-1: anything else).  A
   // permutation of the root variables that is not the identity marks a transposed read.
   std::vector<int> root_var;
+  bool minor_follows = false;   // the input's minor dimension is indexed by the root's minor variable (any offset)
 };
 
 class Emitter {
@@ -75,6 +76,7 @@ class Emitter {
   // preloaded vector (so evaluating it at a point the guard excludes cannot fault), evaluate both
   // sides and select, instead of branching per element
   bool branchless_guards = false;
+  bool clamp_guards = false;   // pad: read at positions clamped into the operand and select, instead of a branch around the read
 
   std::string emit(int node, const Index& ix);
   std::string take_code() { std::string s = out_.str(); out_.str(""); return s; }

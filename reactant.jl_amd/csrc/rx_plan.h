@@ -67,6 +67,7 @@ struct PlanOptions {
   bool single_pass_scan = true;      // long scanned rows in one launch (chunk totals travel as flagged words)
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
+  bool clamp_pad_reads = true;     // maps over 8- and 16-bit elements: padded reads at clamped positions and a select, so that a lane's loads combine
   bool stencil_fuse_steps = true;  // two consecutive stencil steps in one kernel: the first step's result lives only in LDS
   int lds_tile2[3] = {4, 8, 64};   // outputs per workgroup tile of the two-step kernel
   int lds2_threads = 512;          // its workgroup size
