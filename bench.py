@@ -516,7 +516,7 @@ def _window_entry(name, exe, secs, steps, mean_ms, algo_bytes, flops, dtype, bou
         entry.update(value=ach, unit="TFLOP/s")
         dot = [i for i, l in enumerate(launches) if l["flops"] > 0]
         kms = float(mean_ms[dot[0]]) if dot else float(mean_ms[big])
-        kach = flops / (kms * 1e-3) / 1e12
+        kach = (launches[dot[0]]["flops"] if dot else flops) / (kms * 1e-3) / 1e12   # that launch's own flops (a chain has several)
         entry["roofline"] = {"bound": "mfma", "kernel": launches[dot[0] if dot else big]["kernel"], "kernel_ms": kms, "achieved": kach,
                              "peak": PEAK_TFLOPS[bound_kind], "unit": "TFLOP/s", "frac": kach / PEAK_TFLOPS[bound_kind], "traffic": None}
     else:
@@ -539,6 +539,20 @@ def bench_conv(rx, client, P, steps, warmup, batch=32, cin=64, cout=64, hw=56):
     flops = 2.0 * batch * cout * hw * hw * cin * 9
     return _window_entry("conv 3x3 pad 1 f32 %dx%dx%dx%d -> %d features, bias + relu" % (batch, cin, hw, hw, cout), exe, secs, steps, mean_ms,
                          0.0, flops, "f32", "f32")
+
+
+def bench_conv16(rx, client, P, steps, warmup, batch=32, channels=256, hw=56, layers=3):
+    """Three 3x3 convolutions of 256 -> 256 features with bias + relu in bf16 (the body of a VGG block): the products with
+    row shifts, the maps between them and the layout maps at both ends."""
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    text, shapes = NN.conv_chain(batch, channels, hw, layers, "bf16")
+    exe = rx.xla_compile(client, text)
+    rng = np.random.default_rng(0)
+    bufs = [_upload(rx, client, rx.encode((rng.normal(size=s) * (0.02 if len(s) == 4 and k > 0 else 1.0)).astype(np.float32), "bf16"), "bf16") for k, s in enumerate(shapes)]
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
+    flops = layers * 2.0 * batch * channels * hw * hw * channels * 9
+    return _window_entry("%d x (conv 3x3 pad 1 bf16 %dx%dx%dx%d -> %d features, bias + relu)" % (layers, batch, channels, hw, hw, channels), exe, secs, steps, mean_ms,
+                         0.0, flops, "bf16", "bf16")
 
 
 def bench_cumsum(rx, client, P, steps, warmup, n=1 << 26):
@@ -695,7 +709,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "conv16", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
     ap.add_argument("--settle-ms", type=float, default=150.0, help="untimed executions of a workload before its warm-up steps until the device has been under that load this long (0: none)")
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
@@ -710,9 +724,9 @@ def main():
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
-             "conv": bench_conv, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "colsum": bench_colsum, "transpose": bench_transpose, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
+             "conv": bench_conv, "conv16": bench_conv16, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "colsum": bench_colsum, "transpose": bench_transpose, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
-             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28),
+             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28), "conv16": dict(batch=2, channels=64, hw=28),
              "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "colsum": dict(n=1024), "transpose": dict(n=1024), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
     OPTS["check"], OPTS["cpu"], OPTS["settle_ms"] = not args.no_check, not args.no_cpu, args.settle_ms

@@ -141,6 +141,32 @@ def convolution(x_shape, w_shape, dt, dims="[b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1,
     return ("module {\n  func.func @main(%s) -> %s {\n%s    return %s : %s\n  }\n}\n" % (args, to, body, res, to)), out
 
 
+def conv_chain(batch, channels, hw, layers, dt, k=3):
+    """`layers` k x k convolutions (padding k // 2, unit strides) of `channels` -> `channels` features on `batch` images of
+    hw x hw, each followed by a per-feature bias and a relu (the body of a VGG block as LuxLib fuses it); arguments: the
+    images [batch, channels, hw, hw], then a filter [channels, channels, k, k] and a bias [channels] per layer."""
+    t = tt([batch, channels, hw, hw], dt)
+    tw = tt([channels, channels, k, k], dt)
+    tb = tt([channels], dt)
+    args = ["%%arg0: %s" % t]
+    body = ""
+    cur = "%arg0"
+    for l in range(layers):
+        w, b = "%%arg%d" % (1 + 2 * l), "%%arg%d" % (2 + 2 * l)
+        args += ["%s: %s" % (w, tw), "%s: %s" % (b, tb)]
+        body += ("    %%c%d = stablehlo.convolution(%s, %s) dim_numbers = [b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0], window = {stride = [1, 1], "
+                 "pad = [[%d, %d], [%d, %d]], lhs_dilate = [1, 1], rhs_dilate = [1, 1]} {batch_group_count = 1 : i64, feature_group_count = 1 : i64, "
+                 "precision_config = [#stablehlo<precision DEFAULT>, #stablehlo<precision DEFAULT>]} : (%s, %s) -> %s\n"
+                 % (l, cur, w, k // 2, k // 2, k // 2, k // 2, t, tw, t))
+        body += "    %%b%d = stablehlo.broadcast_in_dim %s, dims = [1] : (%s) -> %s\n" % (l, b, tb, t)
+        body += "    %%a%d = stablehlo.add %%c%d, %%b%d : %s\n" % (l, l, l, t)
+        body += "    %%z%d = stablehlo.constant dense<0.000000e+00> : %s\n" % (l, t)
+        body += "    %%r%d = stablehlo.maximum %%a%d, %%z%d : %s\n" % (l, l, l, t)
+        cur = "%%r%d" % l
+    shapes = [[batch, channels, hw, hw]] + [[channels, channels, k, k], [channels]] * layers
+    return ("module {\n  func.func @main(%s) -> %s {\n%s    return %s : %s\n  }\n}\n" % (", ".join(args), t, body, cur, t)), shapes
+
+
 def batch_norm(shape, dt, feature_index, epsilon=1e-5, training=False):
     """`stablehlo.batch_norm_inference` / `batch_norm_training` in the generic form they print in
     (built by the reference's src/Ops.jl:4012-4092)."""

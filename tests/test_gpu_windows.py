@@ -342,6 +342,23 @@ def test_batch_norm(rx, client, shape, dt, feature, training):
         _close(g.a, r.a, tol)
 
 
+@pytest.mark.parametrize("dt,kind", [("bf16", "conv_bf16"), ("f16", "conv_f16"), ("f32", "conv")])
+def test_chain_of_convolutions_with_bias_and_relu(rx, client, dt, kind):
+    """Two 3x3 layers of 64 -> 64 features with bias + relu: in 16 bits the products with row shifts, with one map between
+    them (bias, relu and zero padding, channels-last to channels-last) and the layout maps at both ends; in f32 the direct
+    kernel with its epilogue.  Against the oracle, layer by layer rounding included."""
+    text, shapes = NN.conv_chain(3, 64, 40, 2, dt)
+    rng = np.random.default_rng(5)
+    args = [I.tensor((rng.normal(size=s) * (0.05 if len(s) == 4 and k > 0 else 1.0)).astype(np.float32), dt) for k, s in enumerate(shapes)]
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    assert kinds.count(kind) == 2, kinds
+    if dt != "f32":
+        assert kinds == ["map", "map", kind, "map", "map", kind, "map_transposed"], kinds
+    ref = oracle_run(text, args, hifi=True)
+    _close(got[0].a, ref[0].a, 2e-2 if dt == "bf16" else (4e-3 if dt == "f16" else 1e-4))
+
+
 @pytest.mark.parametrize("sizes", [dict(batch=2, cin=3, cmid=8, hw=16, classes=10), dict(batch=4, cin=3, cmid=64, hw=32, classes=100)])
 def test_vgg_style_forward_pass(rx, client, sizes):
     text, shapes = NN.vgg_block(**sizes)
