@@ -43,6 +43,12 @@ static __device__ __forceinline__ V rx_load_nt(const T* p) {
     return *reinterpret_cast<const V*>(p);
   }
 }
+// a vector at an address that is a multiple of the element size only (padded rows start anywhere)
+template <typename V, typename T>
+static __device__ __forceinline__ V rx_load_unaligned(const T* p) {
+  struct __attribute__((packed, aligned(alignof(T)))) U { V v; };
+  return reinterpret_cast<const U*>(p)->v;
+}
 template <typename T, typename V>
 static __device__ __forceinline__ void rx_store(T* p, const V& v) {
   *reinterpret_cast<V*>(p) = v;

@@ -282,6 +282,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_FUSE_DOT_OPERANDS")) o.fuse_dot_operands = atoi(e) != 0;
   if (const char* e = getenv("RX_BRANCHLESS")) o.branchless_guards = atoi(e) != 0;
   if (const char* e = getenv("RX_CLAMP_PADS")) o.clamp_pad_reads = atoi(e) != 0;
+  if (const char* e = getenv("RX_TRANSPOSE_OFFSETS")) o.transpose_offsets = atoi(e) != 0;
   if (const char* e = getenv("RX_STENCIL_FUSE")) o.stencil_fuse_steps = atoi(e) != 0;
   if (const char* e = getenv("RX_SPLIT_K")) o.split_k = atoi(e) != 0;
   if (const char* e = getenv("RX_IN_PLACE")) o.in_place_updates = atoi(e) != 0;

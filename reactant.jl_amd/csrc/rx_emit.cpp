@@ -196,11 +196,11 @@ std::string Emitter::emit_load(int node, const Index& ix) {
     for (size_t d = 0; d < dims.size() && permuted; ++d) {
       int which = -1;
       for (size_t v = 0; v < root_vars_.size(); ++v)
-        if (ix[d].var == root_vars_[v] && ix[d].off == 0) which = (int)v;
-      if (which < 0 || used[which] || root_dims_[which] != dims[d]) permuted = false;
-      else { used[which] = 1; rec.root_var.push_back(which); }
+        if (ix[d].var == root_vars_[v] && (ix[d].off == 0 || offset_perms)) which = (int)v;
+      if (which < 0 || used[which] || (root_dims_[which] != dims[d] && !offset_perms)) permuted = false;
+      else { used[which] = 1; rec.root_var.push_back(which); rec.root_off.push_back(ix[d].off); }
     }
-    if (!permuted) rec.root_var.clear();
+    if (!permuted) { rec.root_var.clear(); rec.root_off.clear(); }
   }
   loads.push_back(rec);
   if (permuted && perm_hook) {

@@ -35,6 +35,7 @@ struct LoadRecord {
   // permutation of the root variables that is not the identity marks a transposed read.
   std::vector<int> root_var;
   bool minor_follows = false;   // the input's minor dimension is indexed by the root's minor variable (any offset)
+  std::vector<int64_t> root_off;   // with root_var: constant offset of every input dimension's index (offset_perms)
 };
 
 class Emitter {
@@ -76,6 +77,7 @@ class Emitter {
   // preloaded vector (so evaluating it at a point the guard excludes cannot fault), evaluate both
   // sides and select, instead of branching per element
   bool branchless_guards = false;
+  bool offset_perms = false;   // a transposed read may carry constant offsets and read an input of other extents (a padded or sliced transpose)
   bool clamp_guards = false;   // pad: read at positions clamped into the operand and select, instead of a branch around the read
 
   std::string emit(int node, const Index& ix);

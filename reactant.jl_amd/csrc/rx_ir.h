@@ -81,7 +81,7 @@ struct Node {
   //   Scan (inclusive prefix combine with `red`): a0[0] = dimension, a1[0] = 1 if it runs from the end
   //   Conv (image [B, C, H, W], filter [O, C, KH, KW]) -> [B, O, HO, WO]: zero padding a0 = {rows before, rows after,
   //       columns before, columns after}, a1 = strides, a2 = filter dilations (the direct-convolution kernel's operation)
-  //   Conv with a3 = {KW, SY, SX, HP, WP} (product with row shifts): operands [M, C] with M = B * HP * WP and
+  //   Conv with a3 = {KW, SY, SX, HP, WP} (product with row shifts): operands [M, C] with M = B * HP * WP (or [B, HP, WP, C]) and
   //       [O, taps * C]; p[m][o] = sum over taps t = (ty, tx), tx < KW, and c of in0[m + ty * SY + tx * SX][c] * in1[o][t * C + c]
   //       (rows beyond M read as zeros): a unit-stride convolution of zero-padded [image, row, column, channel] data on
   //       the padded grid; the result [B, HO, WO, O] keeps p at m = (b * HP + y) * WP + x for y < HO, x < WO

@@ -2006,8 +2006,8 @@ struct Builder {
           pn.a0 = {0, 0, pad[0], pad[2]}; pn.a1 = {0, CP - C, pad[1], pad[3]}; pn.a2 = {0, 0, 0, 0};
           xi = g.add(pn);
         }
+        // (the product takes [B, HP, WP, CP] as the matrix [B * HP * WP, CP]: the layout map keeps its four dimensions)
         { Node t = add_node(OpK::Transpose, {xi}, TType{xct.dt, {B, HP, WP, CP}}); t.a0 = {0, 2, 3, 1}; xi = g.add(t); }
-        xi = g.add(add_node(OpK::Reshape, {xi}, TType{xct.dt, {MP, CP}}));
         int wi = wc;
         if (CP != C) {
           Node pn = add_node(OpK::Pad, {wi, zero_of(xct.dt)}, TType{xct.dt, {O, CP, KH, KW}});

@@ -1781,6 +1781,7 @@ struct Planner {
       em.set_root(dims, vars, false);
       em.vec = 1;
       em.indent = 6;
+      em.offset_perms = opt.transpose_offsets;
     };
     // pass 1: which reads are transposed, and against which root dimension
     Emitter probe(g, [&](int x) { return x != root && mat[x]; });
@@ -1788,8 +1789,17 @@ struct Planner {
     probe.emit(root, root_index(dims));
     int q = -1;                      // root dimension that indexes the staged inputs' minor dimension
     std::map<int, std::vector<int>> staged;   // node -> root_var
+    // constant offsets of the staged reads (a transpose of a padded or sliced operand): the tile is then read at
+    // positions clamped into the operand, and whatever guards the read in the map (the pad's test) guards the tile read
+    std::map<int, std::vector<int64_t>> staged_off;
+    std::set<int> conflicting;
     for (auto& l : probe.loads) {
       if (l.root_var.empty()) continue;
+      {
+        auto so = staged_off.find(l.node);
+        if (so != staged_off.end() && so->second != l.root_off) conflicting.insert(l.node);
+        staged_off[l.node] = l.root_off;
+      }
       const int in_minor_var = l.root_var.back();
       if (in_minor_var == n - 1) continue;                     // its minor dim already follows the output's
       if (dims[in_minor_var] < 16 || dims[n - 1] < 16) continue;
@@ -1801,15 +1811,27 @@ struct Planner {
       if (it2 != staged.end() && it2->second != l.root_var) continue;
       staged[l.node] = l.root_var;
     }
+    for (int c : conflicting) staged.erase(c);   // read at several offsets: not one tile
     if (staged.empty()) return false;
+    auto plain = [&](int node) {   // the read is a pure permutation of an operand of the root's extents
+      const Node& in = g.nodes[node];
+      const auto& rv = staged[node];
+      for (int d = 0; d < in.ty.rank(); ++d)
+        if (staged_off[node][d] != 0 || in.ty.dims[d] != dims[rv[d]]) return false;
+      return true;
+    };
     // Whole 16-byte vectors on both sides where the two dimensions allow it: a tile of 64 input columns x 128 input
     // rows (64 x 64 for 8-byte elements) is read with 16-byte loads, parked with a row pitch of 64 + V, and written as
     // output rows of 512 bytes, each lane storing the V elements it gathered from V tile rows (8192^2 f32 transpose:
     // 134 -> 105 us; the 4-byte form moves a 256-byte row segment per wavefront instruction).
     const int es_out = info(rn.ty.dt).size;
     int V = (es_out == 2 || es_out == 4 || es_out == 8) ? 16 / es_out : 1;
-    for (auto& kv : staged) if ((int)info(g.nodes[kv.first].ty.dt).size != es_out) V = 1;
-    if (V > 1 && (q < 0 || dims[q] % V != 0 || dims[n - 1] % V != 0 || dims[q] < 64 || dims[n - 1] < 32 || !opt.transpose_vectors)) V = 1;
+    for (auto& kv : staged) if ((int)info(g.nodes[kv.first].ty.dt).size != es_out || (!plain(kv.first) && g.nodes[kv.first].ty.dims.back() < 16 / es_out)) V = 1;
+    bool all_offset = true;   // every staged read carries offsets: its vectors are tested against the operand's row one by one
+    for (auto& kv : staged) all_offset = all_offset && !plain(kv.first);
+    if (V > 1 && (q < 0 || dims[n - 1] % V != 0 || dims[n - 1] < 32 || !opt.transpose_vectors)) V = 1;
+    if (V > 1 && !all_offset && (dims[q] % V != 0 || dims[q] < 64)) V = 1;
+    if (V > 1 && all_offset && dims[q] < 16) V = 1;
     // a minor dimension of at most 64 (the rows of a 56 x 56 image) takes tiles of 64 rows: 128 would be half empty
     const int TQ = TS, TM = V > 1 ? ((es_out == 8 || dims[n - 1] <= 64) ? 64 : 128) : TS, LD = V > 1 ? TQ + V : TS + 1;
     int64_t lds_total = 0;
@@ -1881,12 +1903,44 @@ struct Planner {
       for (int d = in.ty.rank() - 2; d >= 0; --d) stride[d] = stride[d + 1] * in.ty.dims[d + 1];
       std::string base = "0";
       int64_t stride_m = 0;
+      const bool pl = plain(kv.first);
+      const auto& off = staged_off[kv.first];
+      int64_t off_m = 0, off_q = 0, dim_m = 0, dim_q = 0;
       for (int d = 0; d < in.ty.rank(); ++d) {
-        if (rv[d] == n - 1) { stride_m = stride[d]; continue; }
-        if (rv[d] == q) continue;   // the input's minor dimension
-        base += " + i" + std::to_string(rv[d]) + " * " + std::to_string(stride[d]) + (em.idx64 ? "LL" : "");
+        if (rv[d] == n - 1) { stride_m = stride[d]; off_m = off[d]; dim_m = in.ty.dims[d]; continue; }
+        if (rv[d] == q) { off_q = off[d]; dim_q = in.ty.dims[d]; continue; }   // the input's minor dimension
+        std::string coord = "i" + std::to_string(rv[d]);
+        if (!pl && (off[d] != 0 || in.ty.dims[d] < dims[rv[d]]))
+          coord = "rx_min<" + it + ">(rx_max<" + it + ">(" + coord + " + (" + std::to_string(off[d]) + "), 0), " + std::to_string(in.ty.dims[d] - 1) + ")";
+        base += " + " + coord + " * " + std::to_string(stride[d]) + (em.idx64 ? "LL" : "");
       }
       o << "  {\n    const " << it << " base = " << base << ";\n";
+      if (!pl) {
+        // offsets: rows and columns of the operand at clamped positions; a vector that lies inside the operand's row
+        // is one load (at any element address), one that crosses its ends is read element by element
+        const std::string st = info(in.ty.dt).stype;
+        if (V > 1) {
+          const int LPR = TQ / V, RPP = kBlock / LPR;
+          const std::string vts = "rx_vec<" + st + ", " + std::to_string(V) + ">";
+          o << "#pragma unroll\n    for (int r = 0; r < " << TM / RPP << "; ++r) {\n";
+          o << "      const int tb = r * " << RPP << " + (int)threadIdx.x / " << LPR << ", ta = ((int)threadIdx.x % " << LPR << ") * " << V << ";\n";
+          o << "      const " << it << " rr = rx_min<" << it << ">(rx_max<" << it << ">(m0 + tb + (" << off_m << "), 0), " << dim_m - 1 << ");\n";
+          o << "      const " << it << " cc = q0 + ta + (" << off_q << ");\n";
+          o << "      const " << st << "* src = in" << slot << " + base + rr * " << stride_m << (em.idx64 ? "LL" : "") << ";\n";
+          o << "      if (cc >= 0 && cc + " << V << " <= " << dim_q << ") {\n";
+          o << "        rx_store(tile" << slot << " + tb * " << LD << " + ta, rx_load_unaligned<" << vts << ">(src + cc));\n";
+          o << "      } else {\n#pragma unroll\n        for (int e = 0; e < " << V << "; ++e) tile" << slot << "[tb * " << LD << " + ta + e] = src[rx_min<" << it << ">(rx_max<" << it << ">(cc + e, 0), " << dim_q - 1 << ")];\n      }\n";
+          o << "    }\n  }\n";
+        } else {
+          o << "#pragma unroll\n    for (int r = 0; r < " << TS / ROWS << "; ++r) {\n";
+          o << "      const int tb = r * " << ROWS << " + grp, ta = lane;\n";
+          o << "      const " << it << " rr = rx_min<" << it << ">(rx_max<" << it << ">(m0 + tb + (" << off_m << "), 0), " << dim_m - 1 << ");\n";
+          o << "      const " << it << " cc = rx_min<" << it << ">(rx_max<" << it << ">(q0 + ta + (" << off_q << "), 0), " << dim_q - 1 << ");\n";
+          o << "      tile" << slot << "[tb * " << TS + 1 << " + ta] = in" << slot << "[base + rr * " << stride_m << (em.idx64 ? "LL" : "") << " + cc];\n";
+          o << "    }\n  }\n";
+        }
+        continue;
+      }
       if (V > 1) {
         const int LPR = TQ / V, RPP = kBlock / LPR;    // lanes per input row, rows per pass
         const std::string vts = "rx_vec<" + std::string(info(in.ty.dt).stype) + ", " + std::to_string(V) + ">";
@@ -2798,12 +2852,13 @@ struct Planner {
     if (shifted) {
       // [rows of the padded images, C] x [O, taps * C] -> [rows, O] on a streaming GEMM skeleton whose K tiles of the
       // first operand carry the tap's row shift (rx_tap_shift)
-      if (rn.ty.dims != cn.ty.dims || cn.ty.dims[0] * cn.a3[3] * cn.a3[4] != xt.dims[0]) throw Error("internal: shifted product with a result of another shape");
-      const GemmChoice gc = choose_gemm(xt.dt, wt.dt, cn.ty.dt, 1, xt.dims[0], wt.dims[0], wt.dims[1], true, true);
+      const int64_t xrows = xt.numel() / xt.dims.back(), xcols = xt.dims.back();   // the first operand as a matrix (its leading dimensions are the rows)
+      if (rn.ty.dims != cn.ty.dims || cn.ty.dims[0] * cn.a3[3] * cn.a3[4] != xrows) throw Error("internal: shifted product with a result of another shape");
+      const GemmChoice gc = choose_gemm(xt.dt, wt.dt, cn.ty.dt, 1, xrows, wt.dims[0], wt.dims[1], true, true);
       const bool dl = gc.skeleton == "rx_gemm_body_dl";
       if (!gc.ok || (gc.skeleton != "rx_gemm_body_pp" && gc.skeleton != "rx_gemm_body_s" && !(dl && gc.bk * (int)info(xt.dt).size == 128 && gc.split == 1)))
         throw Error("internal: shifted product without a skeleton that loads tiles straight into LDS");
-      o << "// convolution as a product with row shifts: " << xt.str() << " x " << wt.str() << " -> " << cn.ty.str() << ", window " << wt.dims[1] / xt.dims[1] / cn.a3[0] << " x " << cn.a3[0]
+      o << "// convolution as a product with row shifts: " << xt.str() << " x " << wt.str() << " -> " << cn.ty.str() << ", window " << wt.dims[1] / xcols / cn.a3[0] << " x " << cn.a3[0]
         << ", row shifts " << cn.a3[1] << " / " << cn.a3[2] << "\n";
       o << "extern \"C\" __global__ __launch_bounds__(" << gc.block << ") void @K@_conv(const " << gc.stype_a << "* __restrict__ A, const " << gc.stype_a << "* __restrict__ B";
       for (size_t k = 0; k < em.inputs.size(); ++k) o << ", const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ e" << k;
@@ -2814,7 +2869,7 @@ struct Planner {
       o << "  " << gc.skeleton << "<" << gc.targs << ", false, @K@_epi";
       if (gc.depth > 0) o << ", " << gc.depth;
       if (gc.stream_stages > 0) o << ", " << gc.stream_stages;
-      o << (dl ? ", 1" : ", rx_no_fn") << ", rx_tap_shift<" << xt.dims[1] << ", " << cn.a3[0] << ", " << cn.a3[1] << ", " << cn.a3[2] << ", " << info(xt.dt).size << ">>(A, B, epi);\n}\n\n";
+      o << (dl ? ", 1" : ", rx_no_fn") << ", rx_tap_shift<" << xcols << ", " << cn.a3[0] << ", " << cn.a3[1] << ", " << cn.a3[2] << ", " << info(xt.dt).size << ">>(A, B, epi);\n}\n\n";
       const std::string kb = finalize(o.str());
       Launch L;
       L.kernel = named("@K@_conv", kb);

@@ -76,6 +76,7 @@ struct PlanOptions {
   bool march2_edge = true;         // a nearly empty last tile column is covered by tiles a quarter as wide, four times as tall
   int march2_planes = 22;          // planes per workgroup, about (the extent is cut into equal chunks)
   bool transpose_vectors = true;   // transposing maps move 16-byte vectors where the dimensions allow it
+  bool transpose_offsets = true;   // a transposed read of a padded or sliced operand is staged through the LDS tiles too
   int transpose_block = 8;         // their tiles are taken in blocks of this many by this many (1: plain order)
   int march2_lds_ballast = 0;   // bytes of LDS the marching stencil kernel declares and never uses: lowers its occupancy (measurements only)
   int march2_prefetch = 2;   // planes that the marching stencil kernel requests ahead of their use (1 or 2)

@@ -283,10 +283,10 @@ def test_windowed_ops_plan(monkeypatch):
     # 16-bit images, whole 128-byte runs of channels, unit strides: pad + layout map, filter layout map, the product with
     # one row shift per tap on the skeleton the product's shape gets, and the transposing map of the result
     rep = rx.compile_offline(NN.convolution([32, 256, 56, 56], [256, 256, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0], with_source=True)
-    assert kinds(rep) == ["map", "map", "conv_bf16", "map_transposed"], rep
+    assert kinds(rep) == ["map_transposed", "map", "conv_bf16", "map_transposed"], rep
     assert "rx_gemm_body_pp<rx_el_bf16, 256, 256, 2, 4, true, true, 107648, 256, 2304, " in rep and "rx_tap_shift<256, 3, 58, 1, 2>>(A, B, epi)" in rep
     rep = rx.compile_offline(NN.convolution([32, 64, 112, 112], [128, 64, 3, 3], "f16", padding=[[1, 1], [1, 1]], rhs_dil=[1, 2])[0], with_source=True)
-    assert kinds(rep) == ["map", "map", "conv_f16", "map_transposed"] and "rx_gemm_body_s<rx_el_f16, 256, 128, 4, 2, true, true, " in rep and "rx_tap_shift<64, 3, 228, 1, 2>>" in rep, rep
+    assert kinds(rep) == ["map_transposed", "map", "conv_f16", "map_transposed"] and "rx_gemm_body_s<rx_el_f16, 256, 128, 4, 2, true, true, " in rep and "rx_tap_shift<64, 3, 228, 1, 2>>" in rep, rep
     rep = rx.compile_offline(NN.convolution([4, 256, 56, 56], [256, 256, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0], with_source=True)
     assert "conv_bf16" in kinds(rep) and "rx_gemm_body_dl<rx_mma_bf16_16, 128, 128, 64, " in rep and ", 1, rx_tap_shift<256, 3, 58, 1, 2>>" in rep, rep
     # not that form: strides, channels that are not whole 128-byte runs, a product that is cut along K, the switch

@@ -393,6 +393,49 @@ def test_transpose_through_lds_tiles(rx, client, shape, perm, dt):
     assert np.array_equal(got[0].a, oracle_run(text, [x])[0].a)
 
 
+@pytest.mark.parametrize("shape,low,high,perm,dt", [
+    ((6, 200, 121), (0, 2, 1), (0, 1, 3), (0, 2, 1), "f32"),          # scalar tiles, padding on both tiled dimensions
+    ((4, 128, 30, 26), (0, 0, 1, 1), (0, 0, 1, 1), (0, 2, 3, 1), "bf16"),   # [B, C, H, W] -> padded [B, H, W, C]: vector tiles, rows that start at odd elements
+    ((2, 64, 40, 56), (0, 0, 0, 3), (0, 64, 2, 0), (0, 2, 3, 1), "f16"),    # zero channels after the last one, columns before the first
+    ((5, 72, 200), (1, 0, 0), (0, 8, 5), (0, 2, 1), "f64"),
+    ((250, 300), (0, 7), (32, 0), (1, 0), "i32")])
+def test_transpose_of_a_padded_operand_through_lds_tiles(rx, client, shape, low, high, perm, dt):
+    """transpose(pad(x)): the tiles are read at positions clamped into x (a vector inside a row of x at any element
+    address, one that crosses the row's ends element by element) and the pad's test guards the read of the tile; bit-exact."""
+    padded = tuple(s + l + h for s, l, h in zip(shape, low, high))
+    out_shape = tuple(padded[p] for p in perm)
+    zero = "0" if dt == "i32" else "0.000000e+00"
+    lst = lambda v: ", ".join(str(x) for x in v)
+    text = ("module { func.func @main(%%a: %s) -> %s {\n  %%z = stablehlo.constant dense<%s> : tensor<%s>\n"
+            "  %%p = stablehlo.pad %%a, %%z, low = [%s], high = [%s], interior = [%s] : (%s, tensor<%s>) -> %s\n"
+            "  %%0 = stablehlo.transpose %%p, dims = [%s] : (%s) -> %s\n  return %%0 : %s } }"
+            % (_tt_(shape, dt), _tt_(out_shape, dt), zero, dt, lst(low), lst(high), lst([0] * len(shape)), _tt_(shape, dt), dt, _tt_(padded, dt),
+               lst(perm), _tt_(padded, dt), _tt_(out_shape, dt), _tt_(out_shape, dt)))
+    rng = np.random.default_rng(3)
+    x = I.tensor(rng.integers(-1000, 1000, size=shape), dt) if dt == "i32" else I.tensor(rng.normal(size=shape), dt)
+    got, exe = gpu_run(rx, client, text, [x])
+    assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
+    want = np.transpose(np.pad(x.a, list(zip(low, high))), perm)
+    assert got[0].a.shape == want.shape and np.array_equal(got[0].a, want)
+    assert np.array_equal(got[0].a, oracle_run(text, [x])[0].a)
+
+
+def test_transpose_of_a_slice_through_lds_tiles(rx, client):
+    """transpose(x[1:, 3:131, 8:200]): offsets without any guard."""
+    shape, start, limit, perm = (4, 140, 210), (1, 3, 8), (4, 131, 200), (0, 2, 1)
+    sl = tuple(l - s for s, l in zip(start, limit))
+    out_shape = tuple(sl[p] for p in perm)
+    lst = lambda v: ", ".join(str(x) for x in v)
+    text = ("module { func.func @main(%%a: %s) -> %s {\n  %%s = stablehlo.slice %%a [%s] : (%s) -> %s\n"
+            "  %%0 = stablehlo.transpose %%s, dims = [%s] : (%s) -> %s\n  return %%0 : %s } }"
+            % (_tt_(shape, "f32"), _tt_(out_shape, "f32"), ", ".join("%d:%d" % (a, b) for a, b in zip(start, limit)), _tt_(shape, "f32"), _tt_(sl, "f32"),
+               lst(perm), _tt_(sl, "f32"), _tt_(out_shape, "f32"), _tt_(out_shape, "f32")))
+    x = I.tensor(np.random.default_rng(4).normal(size=shape), "f32")
+    got, exe = gpu_run(rx, client, text, [x])
+    assert [l["kind"] for l in exe.launches()] == ["map_transposed"]
+    assert np.array_equal(got[0].a, np.transpose(x.a[1:, 3:131, 8:200], perm))
+
+
 @pytest.mark.parametrize("block", ["1", "3", "16"])
 @pytest.mark.parametrize("shape,perm,dt", [((1100, 1300), (1, 0), "f32"), ((3, 700, 129), (0, 2, 1), "f32"), ((2, 1000, 72), (0, 2, 1), "f64")])
 def test_transposing_tiles_in_blocks_of_other_sizes(rx, client, monkeypatch, block, shape, perm, dt):
