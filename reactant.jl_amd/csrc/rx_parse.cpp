@@ -1979,11 +1979,15 @@ struct Builder {
     // [image, padded row, padded column, feature], from which the result is sliced and transposed.  No window matrix
     // exists.  Taken where the product gets a GEMM skeleton that loads its tiles straight into LDS; RX_CONV_SHIFT=0
     // keeps the window matrix.
-    if (nsp == 2 && (xct.dt == DT::BF16 || xct.dt == DT::F16) && G == 1 && BG == 1 && st[0] == 1 && st[1] == 1 && ld[0] == 1 && ld[1] == 1 && rd[0] >= 1 && rd[1] >= 1 &&
+    // A strided 1 x 1 filter without padding reads every st-th pixel only: the images are sliced first, and the
+    // convolution has unit strides.
+    const bool pointwise = nsp == 2 && wct.dims[2] == 1 && wct.dims[3] == 1 && pad[0] == 0 && pad[1] == 0 && pad[2] == 0 && pad[3] == 0 && st[0] >= 1 && st[1] >= 1;
+    if (nsp == 2 && (xct.dt == DT::BF16 || xct.dt == DT::F16) && G == 1 && BG == 1 && ((st[0] == 1 && st[1] == 1) || pointwise) && ld[0] == 1 && ld[1] == 1 && rd[0] >= 1 && rd[1] >= 1 &&
         pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1 && 2 * ((C + 63) / 64 * 64) <= 3 * C && O % 8 == 0 &&
         !(getenv("RX_CONV_SHIFT") && atoi(getenv("RX_CONV_SHIFT")) == 0) && !(getenv("RX_MFMA") && atoi(getenv("RX_MFMA")) == 0)) {
       const int64_t KH = wct.dims[2], KW = wct.dims[3];
-      const int64_t HP = xct.dims[2] + pad[0] + pad[1], WP = xct.dims[3] + pad[2] + pad[3];
+      const int64_t HS = (xct.dims[2] - 1) / st[0] + 1, WS = (xct.dims[3] - 1) / st[1] + 1;   // the images after the slice (unit strides: as they are)
+      const int64_t HP = HS + pad[0] + pad[1], WP = WS + pad[2] + pad[3];
       const int64_t HO = HP - (KH - 1) * rd[0], WO = WP - (KW - 1) * rd[1];
       // channels that are not whole K tiles (96, 160) are padded with zero channels to the next multiple of 64, in the
       // images and in the filter, when that adds at most half
@@ -2001,6 +2005,11 @@ struct Builder {
         if (want != out.dims) fail("convolution: result shape mismatch");
         auto add_node = [&](OpK k, std::vector<int> in, TType t) { Node n; n.k = k; n.in = std::move(in); n.ty = std::move(t); return n; };
         int xi = xc;
+        if (st[0] > 1 || st[1] > 1) {
+          Node sl = add_node(OpK::Slice, {xi}, TType{xct.dt, {B, C, HS, WS}});
+          sl.a0 = {0, 0, 0, 0}; sl.a1 = {B, C, xct.dims[2], xct.dims[3]}; sl.a2 = {1, 1, st[0], st[1]};
+          xi = g.add(sl);
+        }
         if (pad[0] || pad[1] || pad[2] || pad[3] || CP != C) {
           Node pn = add_node(OpK::Pad, {xi, zero_of(xct.dt)}, TType{xct.dt, {B, CP, HP, WP}});
           pn.a0 = {0, 0, pad[0], pad[2]}; pn.a1 = {0, CP - C, pad[1], pad[3]}; pn.a2 = {0, 0, 0, 0};

@@ -275,6 +275,8 @@ CONVS = [
     ([2, 128, 30, 26], [64, 128, 2, 3], "f16", None, dict(padding=[[0, 1], [2, 0]], rhs_dil=[2, 1]), "conv_f16"),
     ([2, 64, 24, 24], [128, 64, 1, 1], "bf16", None, dict(), "conv_bf16"),
     ([2, 20, 16, 64], [3, 3, 64, 128], "bf16", "[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]", dict(padding=[[1, 1], [1, 1]]), "conv_bf16"),
+    # a strided 1 x 1 filter: the images are sliced, then the product (one tap)
+    ([8, 64, 57, 56], [128, 64, 1, 1], "bf16", None, dict(strides=[2, 3]), "conv_bf16"),
     # 96 channels: zero channels up to 128
     ([8, 96, 48, 48], [64, 96, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "conv_bf16"),
     # the streaming skeletons: 256 x 128 tiles, and 256 x 256 tiles in the ping-pong form
