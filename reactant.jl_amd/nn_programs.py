@@ -205,7 +205,7 @@ def vgg_block(batch=2, cin=3, cmid=8, hw=16, classes=10, dt="f32"):
         "(" + ", ".join([A1, F1, F1, F1, F1]) + ") -> " + A1,
         "%z1 = stablehlo.constant dense<0.000000e+00> : " + A1,
         "%r1 = stablehlo.maximum %bn, %z1 : " + A1,
-        "%ninf = stablehlo.constant dense<0xFF800000> : " + S if dt == "f32" else "%ninf = stablehlo.constant dense<0xFFF0000000000000> : " + S,
+        "%ninf = stablehlo.constant dense<" + _init_literal("maximum", dt) + "> : " + S,
         "%p1 = " + pool % ("%r1", "%ninf", S, S, S, S, A1, S, P1),
         "%c2 = " + conv % ("%p1", "%arg6", P1, W2, A2),
         "%b2 = stablehlo.broadcast_in_dim %arg7, dims = [1] : (" + F2 + ") -> " + A2,

@@ -382,6 +382,29 @@ def test_vgg_style_forward_pass(rx, client, sizes):
         assert any(l["kind"] == "conv" for l in exe.launches())
 
 
+def test_vgg_style_forward_pass_in_bf16(rx, client):
+    """The same op sequence on bf16 images of 64 channels: both convolutions are products with row shifts, whose
+    channels-last results the batch norm, the pooling window and the mean pool read through the transposes' index maps."""
+    sizes = dict(batch=4, cin=64, cmid=64, hw=32, classes=100)
+    text, shapes = NN.vgg_block(dt="bf16", **sizes)
+    rng = np.random.default_rng(19)
+    args = []
+    for k, sh in enumerate(shapes):
+        if k == 5:      # running variance
+            args.append(I.tensor(rng.uniform(0.5, 2.0, size=sh), "bf16"))
+        elif len(sh) == 4 and k > 0:
+            args.append(I.tensor(rng.normal(size=sh) / np.sqrt(np.prod(sh[1:])), "bf16"))
+        else:
+            args.append(I.tensor(rng.normal(size=sh), "bf16"))
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    assert kinds.count("conv_bf16") == 2, kinds
+    ref = oracle_run(text, args, hifi=True)
+    assert got[0].a.shape == (sizes["batch"], sizes["classes"])
+    assert np.allclose(got[0].a.astype(np.float64).sum(axis=1), 1.0, atol=2e-2)
+    _close(got[0].a, ref[0].a, 3e-2)
+
+
 @pytest.mark.parametrize("bh,seq,dim,dt,tol", [(6, 40, 16, "f32", 1e-5), (8, 256, 64, "f32", 1e-4), (8, 256, 64, "bf16", 2e-2)])
 def test_attention_block(rx, client, bh, seq, dim, dt, tol):
     text, shapes = NN.attention_block(bh, seq, dim, dt)
