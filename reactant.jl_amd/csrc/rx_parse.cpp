@@ -1983,14 +1983,15 @@ struct Builder {
     // convolution has unit strides.
     const bool pointwise = nsp == 2 && wct.dims[2] == 1 && wct.dims[3] == 1 && pad[0] == 0 && pad[1] == 0 && pad[2] == 0 && pad[3] == 0 && st[0] >= 1 && st[1] >= 1;
     if (nsp == 2 && (xct.dt == DT::BF16 || xct.dt == DT::F16) && G == 1 && BG == 1 && ((st[0] == 1 && st[1] == 1) || pointwise) && ld[0] == 1 && ld[1] == 1 && rd[0] >= 1 && rd[1] >= 1 &&
-        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1 && 2 * ((C + 63) / 64 * 64) <= 3 * C && O % 8 == 0 &&
+        pad[0] >= 0 && pad[1] >= 0 && pad[2] >= 0 && pad[3] >= 0 && wct.dims[2] >= 1 && wct.dims[3] >= 1 && (double)((C + 63) / 64 * 64) <= (getenv("RX_CONV_SHIFT_WASTE") ? atof(getenv("RX_CONV_SHIFT_WASTE")) : 4.0) * (double)C && O % 8 == 0 &&
         !(getenv("RX_CONV_SHIFT") && atoi(getenv("RX_CONV_SHIFT")) == 0) && !(getenv("RX_MFMA") && atoi(getenv("RX_MFMA")) == 0)) {
       const int64_t KH = wct.dims[2], KW = wct.dims[3];
       const int64_t HS = (xct.dims[2] - 1) / st[0] + 1, WS = (xct.dims[3] - 1) / st[1] + 1;   // the images after the slice (unit strides: as they are)
       const int64_t HP = HS + pad[0] + pad[1], WP = WS + pad[2] + pad[3];
       const int64_t HO = HP - (KH - 1) * rd[0], WO = WP - (KW - 1) * rd[1];
-      // channels that are not whole K tiles (96, 160) are padded with zero channels to the next multiple of 64, in the
-      // images and in the filter, when that adds at most half
+      // channels that are not whole K tiles (96, 160; 16, 32) are padded with zero channels to the next multiple of 64, in
+      // the images and in the filter, up to four times their number (32 -> 64 features on 32 x 112^2: 0.186 -> 0.099 ms,
+      // 16 -> 32 on 16 x 224^2: 0.179 -> 0.121; three channels would be 21 times: 0.19 -> 0.33); RX_CONV_SHIFT_WASTE
       const int64_t CP = (C + 63) / 64 * 64;
       const int64_t MP = B * HP * WP, KK = KH * KW * CP;
       GemmChoice gc;

@@ -266,7 +266,9 @@ CONVS = [
     ([2, 16, 24, 28], [48, 16, 3, 3], "f32", None, dict(strides=[1, 2], rhs_dil=[2, 3], padding=[[2, 2], [3, 3]], flip=True), "conv"),
     # a 1x1 filter (a product over the channels), 7x7 images, bias + relu
     ([8, 128, 16, 16], [96, 128, 1, 1], "f32", None, dict(epilogue="bias_relu"), "conv"),
-    ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
+    ([2, 8, 28, 28], [64, 8, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "gemm_bf16"),
+    # 32 channels: zero channels up to 64
+    ([2, 32, 28, 28], [64, 32, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]]), "conv_bf16"),
     # 16-bit images with whole 128-byte runs of channels, unit strides: a product over the zero-padded [image, row, column,
     # channel] data with one row shift per tap (no window matrix) -- 64 x 64 and 128 x 64 tiles of the direct-to-LDS skeleton,
     ([2, 64, 40, 40], [128, 64, 3, 3], "bf16", None, dict(padding=[[1, 1], [1, 1]], epilogue="bias_relu"), "conv_bf16"),
