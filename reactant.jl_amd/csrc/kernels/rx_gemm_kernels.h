@@ -930,6 +930,12 @@ struct rx_phase_probe {
   }
 };
 
+// An epilogue functor may supply the accumulators' first values (`has_init`, `init(v, n)`: what it would otherwise add
+// to every row of columns n .. n + NV - 1, a bias): the products are then summed onto them, and the epilogue saves the
+// addition and the operand's loads and conversions for every block of rows (an eighth of its instructions for bias + GELU).
+template <class E, class = void> struct rx_epi_has_init { static constexpr bool value = false; };
+template <class E> struct rx_epi_has_init<E, decltype((void)E::has_init)> { static constexpr bool value = E::has_init; };
+
 // A product whose first operand is read through row shifts (KOff of the streaming bodies): K is cut into taps of C
 // elements, and tap t = (ty, tx) of a KW-wide window contracts rows m + ty * SY + tx * SX of a matrix of C columns with
 // columns t * C .. t * C + C - 1 of the second operand; rows beyond the matrix read as zeros.  With the matrix a zero-
@@ -987,9 +993,12 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
 
   rx_f32x4v acc[NA][NB];
 #pragma unroll
-  for (int i = 0; i < NA; ++i)
+  for (int j = 0; j < NB; ++j) {
+    float v0[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (rx_epi_has_init<Epi>::value && !BATCHED) epi.init(v0, n0 + wn * (BN / WN) + 16 * j + 4 * (lane >> 4));
 #pragma unroll
-    for (int j = 0; j < NB; ++j) acc[i][j] = rx_f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < NA; ++i) acc[i][j] = rx_f32x4v{v0[0], v0[1], v0[2], v0[3]};
+  }
 
   DMA_A dma_a;
   DMA_B dma_b;
@@ -1184,9 +1193,12 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
 
   rx_f32x4v acc[NA][NB];
 #pragma unroll
-  for (int i = 0; i < NA; ++i)
+  for (int j = 0; j < NB; ++j) {
+    float v0[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (rx_epi_has_init<Epi>::value && !BATCHED) epi.init(v0, n0 + wn * (BN / WN) + 16 * j + 4 * (lane >> 4));
 #pragma unroll
-    for (int j = 0; j < NB; ++j) acc[i][j] = rx_f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < NA; ++i) acc[i][j] = rx_f32x4v{v0[0], v0[1], v0[2], v0[3]};
+  }
   DMA_A dma_a;
   DMA_B dma_b;
   dma_a.init(A + batch * (long long)M * K, A_GLDB, A_KC ? m0 : m0 * ESZ, (unsigned)((long long)M * AROW * ESZ), tid & (NTL - 1));

@@ -3990,6 +3990,13 @@ struct Planner {
     // Epilogue: the cone from the root down to the dot accumulator, evaluated on NV
     // consecutive elements of the minor output dimension (vector loads of same-shaped
     // operands such as C in alpha*A*B + beta*C, one vector store).
+    const bool fuse_a = fused_operands.count({dot, 0}) != 0, fuse_b = fused_operands.count({dot, 1}) != 0;
+    GemmChoice gc;
+    const int ksplit = d.a4.empty() ? 1 : (int)d.a4[0];
+    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, fuse_a || fuse_b, ksplit);
+    if ((fuse_a || fuse_b) && !gc.ok) throw Error("internal: a fused dot_general operand without a GEMM skeleton");
+    if (ksplit > 1 && (!gc.ok || gc.split != ksplit || root != dot)) throw Error("internal: a dot_general cut along K without the skeleton that slices K");
+
     Emitter em(g, [&](int x) { return mat[x] && x != root; });
     em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(root)) || lt.numel() >= ((int64_t)1 << 31) || rt.numel() >= ((int64_t)1 << 31);
@@ -4001,17 +4008,34 @@ struct Planner {
     em.direct_expr = vec_name;
     em.indent = 6;
     const std::string DCT = info(d.ty.dt).ctype;
+    // The product's only consumer adds a vector along the result's columns (a bias): the streaming skeletons take it as
+    // the accumulators' first values (rx_epi_has_init), and the epilogue starts behind the addition.  Only where narrow
+    // results keep their float32 values inside a kernel anyway (the sum is then rounded once either way).
+    int init_add = -1, init_vec = -1;
+    if (opt.epilogue_init && opt.excess_precision && root != dot && gc.ok && (gc.skeleton == "rx_gemm_body_pp" || gc.skeleton == "rx_gemm_body_s") && d.a0.empty() &&
+        n == 2 && is_float(d.ty.dt) && d.ty.dt != DT::F64) {
+      int users = 0, add = -1;
+      for (int x : cone_nodes(root))
+        for (int i : g.nodes[x].in)
+          if (i == dot) { ++users; add = x; }
+      if (users == 1 && g.nodes[add].k == OpK::Binary && g.nodes[add].op == "add" && g.nodes[add].ty.dims == d.ty.dims && g.nodes[add].ty.dt == d.ty.dt) {
+        const Node& an = g.nodes[add];
+        const int other = an.in[0] == dot ? an.in[1] : an.in[0];
+        const Node& bn = g.nodes[other];
+        if (other != dot && bn.k == OpK::BroadcastInDim && !mat[other] && bn.a0.size() == 1 && bn.a0[0] == n - 1 && mat[bn.in[0]] && g.nodes[bn.in[0]].ty.rank() == 1 &&
+            g.nodes[bn.in[0]].ty.dims[0] == d.ty.dims[n - 1] && g.nodes[bn.in[0]].ty.dt == d.ty.dt) {
+          init_add = add;
+          init_vec = bn.in[0];
+        }
+      }
+    }
+    if (init_add >= 0) em.bound[init_add] = "accv";
     em.bound[dot] = "accv";
     std::string val = root == dot ? std::string("accv") : em.emit(root, root_index(rn.ty.dims));
     std::string ebody = em.take_code();
+    const int init_slot = init_vec >= 0 ? em.slot_of(init_vec) : -1;
     const std::string ACC = is_float(d.ty.dt) ? (d.ty.dt == DT::F64 ? "double" : "float") : info(d.ty.dt).ctype;
 
-    const bool fuse_a = fused_operands.count({dot, 0}) != 0, fuse_b = fused_operands.count({dot, 1}) != 0;
-    GemmChoice gc;
-    const int ksplit = d.a4.empty() ? 1 : (int)d.a4[0];
-    if (opt.mfma && f.ok && n >= 2) gc = choose_gemm(lt.dt, rt.dt, d.ty.dt, f.batch, f.M, f.N, f.K, f.a_k_contig, f.b_k_contig, fuse_a || fuse_b, ksplit);
-    if ((fuse_a || fuse_b) && !gc.ok) throw Error("internal: a fused dot_general operand without a GEMM skeleton");
-    if (ksplit > 1 && (!gc.ok || gc.split != ksplit || root != dot)) throw Error("internal: a dot_general cut along K without the skeleton that slices K");
     std::ostringstream o;
     // operand functors: element (row, column) of the operand as it would be stored, evaluated from the fused cone
     GemmOperandFn fn_a, fn_b;
@@ -4094,6 +4118,12 @@ struct Planner {
       o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
     const std::string ost = info(rn.ty.dt).stype;
     o << "  " << ost << "* __restrict__ out0;\n";
+    if (init_slot >= 0) {
+      o << "  static constexpr bool has_init = true;\n";
+      o << "  template <int NV>\n  __device__ __forceinline__ void init(float (&v)[NV], int n) const {\n";
+      o << "#pragma unroll\n    for (int l = 0; l < NV; ++l) v[l] = (float)" << em.load_conv(d.ty.dt, "in" + std::to_string(init_slot) + "[rx_min<int>(n + l, " + std::to_string(d.ty.dims[n - 1] - 1) + ")]") << ";\n";
+      o << "  }\n";
+    }
     o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const " << ACC << " (&acc)[NV]";
     for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
     o << ") const {\n";

@@ -54,6 +54,7 @@ struct PlanOptions {
   bool dot_as_reduce = true;    // dot_generals with a vector-like operand run as multiply + reduce
   bool fuse_dot_operands = true;  // a dot operand that expands much smaller data is evaluated inside the GEMM's tile loads
   bool split_k = true;          // matrix products with few output tiles and a long contraction: K in slices, partial products, a reduction
+  bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
   int slab_ytiles = 0;          // stencil kernels: y-tiles per XCD slab (0: one slab per XCD)

@@ -140,6 +140,34 @@ def test_streaming_skeleton(rx, client, dt, out_dt, M, N, K, a_kc, b_kc, batch):
     assert max_rel_to_scale(got[0].a, ref[0].a) <= (1e-2 if out_dt in ("bf16", "f16") else 1e-5 * np.sqrt(K))
 
 
+@pytest.mark.parametrize("dt,M,N,K", [("bf16", 4000, 4104, 256), ("f16", 8000, 1032, 192)])
+def test_bias_as_the_accumulators_first_values(rx, client, monkeypatch, dt, M, N, K):
+    """relu(x W + b) on the streaming skeletons, ragged last tiles in both directions: the bias is the accumulators' first
+    values (the epilogue functor's `init`), which must give what adding it in the epilogue gives, up to the order of the
+    float32 additions, and what the oracle gives."""
+    t = lambda s: "tensor<" + "x".join(str(v) for v in s) + "x" + dt + ">"
+    text = ("module {\n  func.func @main(%%x: %s, %%w: %s, %%b: %s) -> %s {\n"
+            "    %%0 = stablehlo.dot_general %%x, %%w, contracting_dims = [1] x [0] : (%s, %s) -> %s\n"
+            "    %%1 = stablehlo.broadcast_in_dim %%b, dims = [1] : (%s) -> %s\n    %%2 = stablehlo.add %%0, %%1 : %s\n"
+            "    %%z = stablehlo.constant dense<0.000000e+00> : %s\n    %%3 = stablehlo.maximum %%2, %%z : %s\n    return %%3 : %s\n  }\n}\n"
+            % (t([M, K]), t([K, N]), t([N]), t([M, N]), t([M, K]), t([K, N]), t([M, N]), t([N]), t([M, N]), t([M, N]), t([M, N]), t([M, N]), t([M, N])))
+    rng = np.random.default_rng(9)
+    args = [I.tensor(rng.normal(size=(M, K)), dt), I.tensor(rng.normal(size=(K, N)) / np.sqrt(K), dt), I.tensor(rng.normal(size=(N,)) * 3.0, dt)]
+    src = rx.compile_offline(text, with_source=True)
+    assert "has_init = true" in src and "void init(float (&v)[NV], int n)" in src
+    got, exe = gpu_run(rx, client, text, args)
+    assert [l["kind"] for l in exe.launches()] == ["gemm_" + dt]
+    monkeypatch.setenv("RX_EPILOGUE_INIT", "0")
+    assert "has_init" not in rx.compile_offline(text, with_source=True)
+    plain, _ = gpu_run(rx, client, text, args)
+    ref = oracle_run(text, args, hifi=True)
+    tol = 1e-2 if dt == "bf16" else 2e-3
+    assert max_rel_to_scale(got[0].a, ref[0].a) <= tol and max_rel_to_scale(plain[0].a, ref[0].a) <= tol
+    # the two forms differ by float32 rounding of the sums only: at most an ulp of the narrow result here and there
+    g, p = got[0].a.astype(np.float64), plain[0].a.astype(np.float64)
+    assert np.mean(g != p) < 0.02 and np.max(np.abs(g - p)) <= (2.0 ** -7 if dt == "bf16" else 2.0 ** -10) * np.abs(p).max()
+
+
 def test_int_dot_general_reference_vectors(rx, client):
     """Known answers of the reference's own test (test/core/ops.jl:249-278)."""
     t = ("module {\n  func.func @main(%arg0: tensor<4xi32>, %arg1: tensor<4xi32>) -> tensor<i32> {\n"
