@@ -285,7 +285,9 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_TRANSPOSE_OFFSETS")) o.transpose_offsets = atoi(e) != 0;
   if (const char* e = getenv("RX_STENCIL_FUSE")) o.stencil_fuse_steps = atoi(e) != 0;
   if (const char* e = getenv("RX_SPLIT_K")) o.split_k = atoi(e) != 0;
+  if (const char* e = getenv("RX_EPILOGUES")) o.product_epilogues = atoi(e) != 0;
   if (const char* e = getenv("RX_EPILOGUE_INIT")) o.epilogue_init = atoi(e) != 0;
+  if (const char* e = getenv("RX_CHAIN_CONVS")) o.chain_convs = atoi(e) != 0;
   if (const char* e = getenv("RX_IN_PLACE")) o.in_place_updates = atoi(e) != 0;
   if (const char* e = getenv("RX_CHAIN_STEPS")) o.chain_steps = atoi(e);
   if (const char* e = getenv("RX_CHAIN_TILE")) { int v[3] = {0, 0, 0}; if (sscanf(e, "%d,%d,%d", &v[0], &v[1], &v[2]) >= 1) { o.chain_tile[0] = v[0]; o.chain_tile[1] = v[1]; o.chain_tile[2] = v[2]; } }

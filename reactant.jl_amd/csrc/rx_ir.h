@@ -85,6 +85,8 @@ struct Node {
   //       [O, taps * C]; p[m][o] = sum over taps t = (ty, tx), tx < KW, and c of in0[m + ty * SY + tx * SX][c] * in1[o][t * C + c]
   //       (rows beyond M read as zeros): a unit-stride convolution of zero-padded [image, row, column, channel] data on
   //       the padded grid; the result [B, HO, WO, O] keeps p at m = (b * HP + y) * WP + x for y < HO, x < WO
+  //       with a3 = {KW, SY, SX, HP, WP, HO, WO, shift} the result is [B, HP, WP, O]: row m of p, zero where it is not a
+  //       result, at row m + shift, and zeros in the rows before `shift` (the next such product's zero-padded operand)
   std::vector<int64_t> a0, a1, a2, a3, a4, a5, a6;
   Red red = Red::Add;
   // Constant payload: either one splat element or dense bytes in storage format

@@ -108,6 +108,10 @@ std::string red_apply(Red r, DT dt, const std::string& a, const std::string& b) 
   return a;
 }
 
+// Thrown while planning when a convolution in the grid form did not take the whole elementwise chain that follows
+// it into its kernel: the module is then planned again without that rewrite.
+struct ChainNotAbsorbed {};
+
 struct Planner {
   Graph g;  // canonicalized copy
   PlanOptions opt;
@@ -176,6 +180,163 @@ struct Planner {
     normalize_dots();
     align_dots();
     split_dots();
+    chain_convs();
+  }
+
+  // Two convolutions in the product-with-row-shifts form (OpK::Conv with a3) with nothing between them but elementwise
+  // ops whose other operands vary along the channels only (bias, batch norm, activation) and the zero padding of the
+  // second one, on the same padded grid (same batch, HP x WP): the first product keeps its rows on that grid instead of
+  // packing the results -- the epilogue writes row m to row m + (top padding * WP + left padding), zero where row m is
+  // not a result, and zeros to the rows before that offset -- which is the second product's zero-padded operand: a
+  // result's grid position (y, x) moves to (y + top, x + left), and the positions that are not results (the last rows
+  // and columns of every image's grid) move onto the borders, each border position exactly once.  The elementwise ops
+  // become the first product's epilogue; the map between the two products disappears.
+  void chain_convs() {
+    if (!opt.chain_convs || !opt.mfma) return;
+    const int N = (int)g.nodes.size();
+    std::vector<int> nuse(N, 0);
+    for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
+    for (int r : g.results) nuse[r]++;
+    auto elementwise = [](OpK k) { return k == OpK::Unary || k == OpK::Binary || k == OpK::Clamp || k == OpK::Gelu || k == OpK::Convert || k == OpK::Select || k == OpK::Compare; };
+    // value varies along dimension 1 (the channels of [B, C, H, W]) only
+    std::vector<signed char> vec_memo(N, -1);
+    std::function<bool(int, int)> channel_only = [&](int x, int depth) -> bool {
+      if (vec_memo[x] >= 0) return vec_memo[x] != 0;
+      const Node& n = g.nodes[x];
+      bool ok = false;
+      if (n.k == OpK::Constant) ok = n.splat;
+      else if (n.k == OpK::BroadcastInDim) {
+        const TType& st = g.nodes[n.in[0]].ty;
+        ok = n.ty.rank() == 4 && (st.rank() == 0 || (st.rank() == 1 && n.a0.size() == 1 && n.a0[0] == 1 && st.dims[0] == n.ty.dims[1]));
+      } else if (elementwise(n.k) && depth < 12) {
+        ok = !n.in.empty();
+        for (int i : n.in) ok = ok && channel_only(i, depth + 1);
+      }
+      vec_memo[x] = ok ? 1 : 0;
+      return ok;
+    };
+    struct Match { int c1, t1, pad, t2, c2; std::vector<int> chain; int64_t shift; };
+    std::vector<Match> matches;
+    std::vector<char> taken(N, 0);
+    for (const Node& c2 : g.nodes) {
+      if (c2.k != OpK::Conv || c2.a3.size() != 5) continue;
+      Match m;
+      m.c2 = c2.id;
+      m.t2 = c2.in[0];
+      const Node& t2 = g.nodes[m.t2];
+      if (t2.k != OpK::Transpose || t2.a0 != std::vector<int64_t>{0, 2, 3, 1} || nuse[m.t2] != 1) continue;
+      int cur = t2.in[0];
+      m.pad = -1;
+      int64_t pt = 0, pl = 0;
+      if (g.nodes[cur].k == OpK::Pad) {
+        const Node& p = g.nodes[cur];
+        const Node& pv = g.nodes[p.in[1]];
+        bool zero = pv.k == OpK::Constant && pv.splat;
+        for (uint8_t b : pv.data) zero = zero && b == 0;
+        if (!zero || nuse[cur] != 1 || p.a0.size() != 4 || p.a0[0] || p.a0[1] || p.a1[0] || p.a1[1] || p.a2 != std::vector<int64_t>{0, 0, 0, 0} ||
+            p.a0[2] < 0 || p.a0[3] < 0 || p.a1[2] < 0 || p.a1[3] < 0) continue;
+        m.pad = cur;
+        pt = p.a0[2];
+        pl = p.a0[3];
+        cur = p.in[0];
+      }
+      bool ok = true;
+      m.t1 = -1;
+      for (int depth = 0; depth < 16 && ok; ++depth) {
+        const Node& n = g.nodes[cur];
+        if (nuse[cur] != 1 || taken[cur]) { ok = false; break; }
+        if (n.k == OpK::Transpose) {
+          ok = n.a0 == std::vector<int64_t>{0, 3, 1, 2};
+          m.t1 = cur;
+          break;
+        }
+        if (!elementwise(n.k) || n.k == OpK::Compare || n.k == OpK::Select || n.ty.rank() != 4) { ok = false; break; }
+        int tensor = -1;
+        for (int i : n.in) {
+          if (channel_only(i, 0)) continue;
+          if (tensor >= 0) ok = false;
+          tensor = i;
+        }
+        if (tensor < 0) ok = false;
+        m.chain.push_back(cur);
+        cur = tensor;
+      }
+      if (!ok || m.t1 < 0) continue;
+      m.c1 = g.nodes[m.t1].in[0];
+      const Node& c1 = g.nodes[m.c1];
+      if (c1.k != OpK::Conv || c1.a3.size() != 5 || nuse[m.c1] != 1 || taken[m.c1] || m.c1 == m.c2) continue;
+      // the same grid, the second operand's channels as the first product delivers them, results where the padding puts them
+      const TType& x2 = t2.ty;   // [B, HP, WP, C]
+      if (x2.rank() != 4 || c1.ty.rank() != 4 || x2.dims[0] != c1.ty.dims[0] || x2.dims[1] != c1.a3[3] || x2.dims[2] != c1.a3[4] || x2.dims[3] != c1.ty.dims[3] ||
+          c2.a3[3] != c1.a3[3] || c2.a3[4] != c1.a3[4] || x2.dims[1] - c1.ty.dims[1] < pt || x2.dims[2] - c1.ty.dims[2] < pl)
+        continue;
+      if (m.pad >= 0) {
+        const Node& p = g.nodes[m.pad];
+        if (c1.ty.dims[1] + pt + p.a1[2] != x2.dims[1] || c1.ty.dims[2] + pl + p.a1[3] != x2.dims[2]) continue;
+      } else if (c1.ty.dims[1] != x2.dims[1] || c1.ty.dims[2] != x2.dims[2]) continue;
+      m.shift = pt * c1.a3[4] + pl;
+      for (int x : m.chain) taken[x] = 1;
+      taken[m.c1] = taken[m.t1] = taken[m.t2] = 1;
+      if (m.pad >= 0) taken[m.pad] = 1;
+      matches.push_back(m);
+    }
+    if (matches.empty()) return;
+    std::map<int, const Match*> by_c1, by_t1, by_chain, by_pad, by_t2;
+    for (auto& m : matches) {
+      by_c1[m.c1] = &m; by_t1[m.t1] = &m; by_t2[m.t2] = &m;
+      if (m.pad >= 0) by_pad[m.pad] = &m;
+      for (int x : m.chain) by_chain[x] = &m;
+    }
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(N, -1);
+    // a channel-only value rebuilt on [B, HP, WP, C]
+    std::function<int(int, const std::vector<int64_t>&, std::map<int, int>&)> rebuild_vec = [&](int x, const std::vector<int64_t>& dims, std::map<int, int>& memo) -> int {
+      auto it = memo.find(x);
+      if (it != memo.end()) return it->second;
+      Node c = g.nodes[x];
+      c.ty.dims = dims;
+      if (c.k == OpK::BroadcastInDim) {
+        c.in = {remap[c.in[0]]};
+        if (!c.a0.empty()) c.a0 = {3};
+      } else if (c.k != OpK::Constant) {
+        for (int& i : c.in) i = rebuild_vec(i, dims, memo);
+      }
+      return memo[x] = out.add(c);
+    };
+    std::map<const Match*, std::map<int, int>> memos;
+    for (const Node& n : g.nodes) {
+      if (by_c1.count(n.id)) {
+        const Match& m = *by_c1[n.id];
+        Node c = n;
+        for (int& i : c.in) i = remap[i];
+        c.a3 = {n.a3[0], n.a3[1], n.a3[2], n.a3[3], n.a3[4], n.ty.dims[1], n.ty.dims[2], m.shift};
+        c.ty.dims = {n.ty.dims[0], n.a3[3], n.a3[4], n.ty.dims[3]};
+        remap[n.id] = out.add(c);
+        continue;
+      }
+      if (by_t1.count(n.id)) { remap[n.id] = remap[n.in[0]]; continue; }
+      if (by_chain.count(n.id)) {
+        const Match& m = *by_chain[n.id];
+        const Node& c1 = g.nodes[m.c1];
+        const std::vector<int64_t> dims{c1.ty.dims[0], c1.a3[3], c1.a3[4], c1.ty.dims[3]};
+        Node c = n;
+        c.ty.dims = dims;
+        for (int& i : c.in) i = channel_only(i, 0) ? rebuild_vec(i, dims, memos[&m]) : remap[i];
+        remap[n.id] = out.add(c);
+        continue;
+      }
+      if (by_pad.count(n.id)) { remap[n.id] = remap[n.in[0]]; continue; }
+      if (by_t2.count(n.id)) { remap[n.id] = remap[n.in[0]]; continue; }
+      Node c = n;
+      for (int& i : c.in) i = remap[i];
+      remap[n.id] = out.add(c);
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // A dot_general with several batch, free or contracting dims, or with them in another order than
@@ -2799,6 +2960,17 @@ struct Planner {
       if (!cc.ok) throw Error("internal: convolution node without a tiling");
     }
     const int n = rn.ty.rank();
+    if (shifted && cn.a3.size() == 8) {
+      // The grid form zeroes the rows that are not results and moves the rows inside this kernel, after the
+      // elementwise ops it has taken in.  That is only right when nothing elementwise is left to run
+      // afterwards (it would turn the zeros into f(0)) and when every reader expects the moved rows.
+      bool whole = !std::count(g.results.begin(), g.results.end(), root) && !users[root].empty();
+      for (int u : users[root]) {
+        const Node& un = g.nodes[u];
+        whole = whole && un.k == OpK::Conv && !un.a3.empty() && un.in[0] == root && un.in[1] != root;
+      }
+      if (!whole) throw ChainNotAbsorbed();
+    }
     Emitter em(g, [&](int x) { return mat[x] && x != root; });
     em.excess_precision = opt.excess_precision;
     em.idx64 = needs64(cone_nodes(root));
@@ -2826,7 +2998,12 @@ struct Planner {
       if (n != 4) throw Error("internal: shifted product with a result of another rank");
       o << ", " << it << " row_, " << it << " i3b) const {\n";
       o << "    const " << it << " i2 = row_ % " << cn.a3[4] << ", i1 = (row_ / " << cn.a3[4] << ") % " << cn.a3[3] << ", i0 = row_ / " << cn.a3[3] * cn.a3[4] << ";\n";
-      o << "    if (i1 >= " << rn.ty.dims[1] << " || i2 >= " << rn.ty.dims[2] << ") return;\n";
+      if (cn.a3.size() == 8) {
+        // the grid form (chain_convs): every row is written, the ones that are not results as zeros
+        o << "    const bool result_ = i1 < " << cn.a3[5] << " && i2 < " << cn.a3[6] << ";\n";
+      } else {
+        o << "    if (i1 >= " << rn.ty.dims[1] << " || i2 >= " << rn.ty.dims[2] << ") return;\n";
+      }
     } else {
       for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
       o << ") const {\n";
@@ -2847,7 +3024,18 @@ struct Planner {
     o << "      const float accv = acc[l];\n";
     o << ebody;
     o << "      res.v[l] = " << em.store_value(rn.ty.dt, val) << ";\n    }\n";
-    o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+    if (shifted && cn.a3.size() == 8) {
+      // row m goes to row m + shift (the position of the same pixel in the next product's zero-padded operand); rows that
+      // are not results carry zeros onto the borders; the rows before the shift are zeros too, written by the call for the
+      // product row of the same number
+      const int64_t rows = cn.ty.dims[0] * cn.a3[3] * cn.a3[4], ncol = cn.ty.dims[3];
+      o << "    rx_vec<" << ost << ", NV> zero_;\n#pragma unroll\n    for (int l = 0; l < NV; ++l) zero_.v[l] = 0;\n";
+      o << "    if (!result_) res = zero_;\n";
+      o << "    if (row_ + " << cn.a3[7] << " < " << rows << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0 + " << cn.a3[7] * ncol << ") = res;\n";
+      if (cn.a3[7] > 0) o << "    if (row_ < " << cn.a3[7] << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = zero_;\n";
+    } else {
+      o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+    }
     o << "  }\n};\n\n";
     if (shifted) {
       // [rows of the padded images, C] x [O, taps * C] -> [rows, O] on a streaming GEMM skeleton whose K tiles of the
@@ -2884,7 +3072,8 @@ struct Planner {
       std::vector<int> all_in{cn.in[0], cn.in[1]};
       for (int i : em.inputs) if (std::find(all_in.begin(), all_in.end(), i) == all_in.end()) all_in.push_back(i);
       L.algo_bytes = algo_bytes(all_in, {root});
-      L.flops = 2.0 * (double)cn.ty.numel() * (double)wt.dims[1];   // of the results that are kept
+      // of the results that are kept
+      L.flops = 2.0 * (double)(cn.a3.size() == 8 ? cn.ty.dims[0] * cn.a3[5] * cn.a3[6] * cn.ty.dims[3] : cn.ty.numel()) * (double)wt.dims[1];
       L.desc = describe(root);
       plan.launches.push_back(L);
       return;
@@ -4268,7 +4457,7 @@ struct Planner {
 
     // dot epilogues: an elementwise root that consumes a dot result at the identity index
     epilogue_of.clear();
-    for (int x = 0; x < N; ++x) {
+    for (int x = 0; x < N && opt.product_epilogues; ++x) {
       if (!live[x] || (g.nodes[x].k != OpK::DotGeneral && g.nodes[x].k != OpK::Conv)) continue;
       if (std::find(g.results.begin(), g.results.end(), x) != g.results.end()) continue;
       if (ctx[x].size() != 1) continue;
@@ -4549,10 +4738,16 @@ static void count_hlo_costs(const Graph& g, Plan* plan) {
 }
 
 Plan make_plan(const Graph& g, const PlanOptions& opt) {
-  Planner p(g, opt);
-  p.run();
-  count_hlo_costs(g, &p.plan);
-  return std::move(p.plan);
+  try {
+    Planner p(g, opt);
+    p.run();
+    count_hlo_costs(g, &p.plan);
+    return std::move(p.plan);
+  } catch (const ChainNotAbsorbed&) {
+    PlanOptions plain = opt;
+    plain.chain_convs = false;
+    return make_plan(g, plain);
+  }
 }
 
 }  // namespace rx

@@ -54,6 +54,8 @@ struct PlanOptions {
   bool dot_as_reduce = true;    // dot_generals with a vector-like operand run as multiply + reduce
   bool fuse_dot_operands = true;  // a dot operand that expands much smaller data is evaluated inside the GEMM's tile loads
   bool split_k = true;          // matrix products with few output tiles and a long contraction: K in slices, partial products, a reduction
+  bool chain_convs = true;      // two 16-bit convolutions with only channel-wise elementwise ops and padding between them share the padded grid: no map in between
+  bool product_epilogues = true;  // the elementwise ops that consume a product or convolution run in its kernel (off: a map after it; for comparisons)
   bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles

@@ -299,6 +299,22 @@ def test_windowed_ops_plan(monkeypatch):
     monkeypatch.setenv("RX_CONV_SHIFT", "0")
     assert "conv_bf16" not in kinds(rx.compile_offline(NN.convolution([32, 256, 56, 56], [256, 256, 3, 3], "bf16", padding=[[1, 1], [1, 1]])[0]))
     monkeypatch.delenv("RX_CONV_SHIFT")
+    # two such convolutions with bias + relu between them share the padded grid: the first one's kernel writes the
+    # second one's zero-padded operand and no map runs between them; the switch, and a first convolution whose kernel
+    # does not hold the ops between them (then the module is planned again without it), leave the maps in
+    text = NN.conv_chain(32, 256, 56, 2, "bf16")[0]
+    chained = ["map_transposed", "map", "conv_bf16", "map", "conv_bf16", "map_transposed"]
+    unchained = ["map_transposed", "map", "conv_bf16", "map", "map", "conv_bf16", "map_transposed"]
+    rep = rx.compile_offline(text, with_source=True)
+    assert kinds(rep) == chained and "zero_" in rep, rep
+    monkeypatch.setenv("RX_CHAIN_CONVS", "0")
+    rep = rx.compile_offline(text, with_source=True)
+    assert kinds(rep) == unchained and "zero_" not in rep, rep
+    monkeypatch.delenv("RX_CHAIN_CONVS")
+    monkeypatch.setenv("RX_EPILOGUES", "0")
+    rep = rx.compile_offline(text, with_source=True)
+    assert kinds(rep) == unchained and "zero_" not in rep, rep
+    monkeypatch.delenv("RX_EPILOGUES")
 
 
 def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):

@@ -348,21 +348,39 @@ def test_batch_norm(rx, client, shape, dt, feature, training):
         _close(g.a, r.a, tol)
 
 
-@pytest.mark.parametrize("dt,kind", [("bf16", "conv_bf16"), ("f16", "conv_f16"), ("f32", "conv")])
-def test_chain_of_convolutions_with_bias_and_relu(rx, client, dt, kind):
-    """Two 3x3 layers of 64 -> 64 features with bias + relu: in 16 bits the products with row shifts, with one map between
-    them (bias, relu and zero padding, channels-last to channels-last) and the layout maps at both ends; in f32 the direct
-    kernel with its epilogue.  Against the oracle, layer by layer rounding included."""
-    text, shapes = NN.conv_chain(3, 64, 40, 2, dt)
+@pytest.mark.parametrize("dt,kind,chained", [("bf16", "conv_bf16", True), ("bf16", "conv_bf16", False), ("f16", "conv_f16", True), ("f16", "conv_f16", False), ("f32", "conv", True)])
+def test_chain_of_convolutions_with_bias_and_relu(rx, client, monkeypatch, dt, kind, chained):
+    """Three 3x3 layers of 64 -> 64 features with bias + relu.  In 16 bits the products with row shifts: chained, a product
+    writes bias + relu of its results straight into the next one's zero-padded operand (same grid, rows moved by the
+    padding, zeros where a row is not a result), so only the filters' layout maps lie between the products; unchained
+    (RX_CHAIN_CONVS=0), one map between them does that.  In f32 the direct kernel with its epilogue.  Against the oracle."""
+    if not chained:
+        monkeypatch.setenv("RX_CHAIN_CONVS", "0")
+    text, shapes = NN.conv_chain(3, 64, 40, 3, dt)
     rng = np.random.default_rng(5)
     args = [I.tensor((rng.normal(size=s) * (0.05 if len(s) == 4 and k > 0 else 1.0)).astype(np.float32), dt) for k, s in enumerate(shapes)]
     got, exe = gpu_run(rx, client, text, args)
     kinds = [l["kind"] for l in exe.launches()]
-    assert kinds.count(kind) == 2, kinds
-    if dt != "f32":
-        assert kinds == ["map_transposed", "map", kind, "map", "map", kind, "map_transposed"], kinds
+    assert kinds.count(kind) == 3, kinds
+    if dt != "f32" and chained:
+        assert kinds == ["map_transposed", "map", kind, "map", kind, "map", kind, "map_transposed"], kinds
+    elif dt != "f32":
+        assert kinds == ["map_transposed", "map", kind, "map", "map", kind, "map", "map", kind, "map_transposed"], kinds
     ref = oracle_run(text, args, hifi=True)
     _close(got[0].a, ref[0].a, 2e-2 if dt == "bf16" else (4e-3 if dt == "f16" else 1e-4))
+
+
+def test_chain_of_convolutions_when_the_kernels_take_no_epilogues(rx, client, monkeypatch):
+    """RX_EPILOGUES=0: bias + relu run as a map after each product, so a product cannot write the next one's operand;
+    the module is planned without the chaining and the results are the same."""
+    monkeypatch.setenv("RX_EPILOGUES", "0")
+    text, shapes = NN.conv_chain(2, 64, 24, 2, "bf16")
+    rng = np.random.default_rng(6)
+    args = [I.tensor((rng.normal(size=s) * (0.05 if len(s) == 4 and k > 0 else 1.0)).astype(np.float32), "bf16") for k, s in enumerate(shapes)]
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    assert kinds == ["map_transposed", "map", "conv_bf16", "map", "map", "conv_bf16", "map_transposed"], kinds
+    _close(got[0].a, oracle_run(text, args, hifi=True)[0].a, 2e-2)
 
 
 @pytest.mark.parametrize("sizes", [dict(batch=2, cin=3, cmid=8, hw=16, classes=10), dict(batch=4, cin=3, cmid=64, hw=32, classes=100)])
