@@ -248,6 +248,12 @@ struct rx_no_fn {
   RX_DEV int col(int) { return 0; }
 };
 
+// An epilogue functor that declares `static constexpr bool masks_rows = true` tests the row it is called with itself
+// (it guards its stores only): the skeleton then calls it for the rows past the product's last one too, and with whole
+// column tiles the epilogue is straight-line code, in which what depends on the column alone is computed once.
+template <class E, class = void> struct rx_epi_masks_rows { static constexpr bool value = false; };
+template <class E> struct rx_epi_masks_rows<E, decltype((void)E::masks_rows)> { static constexpr bool value = E::masks_rows; };
+
 template <class MMA, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, int M, int N, int K, int RB, int CB, bool BATCHED, class Epi,
           class LA = rx_no_fn, class LB = rx_no_fn>
 RX_DEV void rx_gemm_body(const typename MMA::elem* __restrict__ A, const typename MMA::elem* __restrict__ B, const Epi& epi, const LA& la = LA(),
@@ -730,7 +736,7 @@ RX_DEV void rx_gemm_body_dl(const typename MMA::elem* __restrict__ A, const type
         TRAITS::coords(lane, rg, &dm, &dn);
         const int m = m0 + wm * (BM / WM) + 32 * i + dm;
         const int n = n0 + wn * (BN / WN) + 32 * j + dn;
-        constexpr bool WHOLE = M % BM == 0 && N % BN == 0;   // no bounds test: the epilogue becomes straight-line code
+        constexpr bool WHOLE = (M % BM == 0 || rx_epi_masks_rows<Epi>::value) && N % BN == 0;   // no bounds test: the epilogue becomes straight-line code
         if (WHOLE || (m < M && n < N)) {
           const float v[4] = {acc[i][j][4 * rg], acc[i][j][4 * rg + 1], acc[i][j][4 * rg + 2], acc[i][j][4 * rg + 3]};
           if constexpr (BATCHED) epi(v, (int)batch, m, n);
@@ -1120,7 +1126,7 @@ RX_DEV void rx_gemm_body_s(const typename EL::elem* __restrict__ A, const typena
       // Whole tiles need no bounds test, and without it the epilogue is straight-line code: the compiler then requests
       // what the functor reads (a bias, the C operand) for all blocks ahead of the arithmetic instead of one
       // request, one wait and one store per block.
-      constexpr bool WHOLE = M % BM == 0 && N % BN == 0;
+      constexpr bool WHOLE = (M % BM == 0 || rx_epi_masks_rows<Epi>::value) && N % BN == 0;
       if (WHOLE || (m < M && n < N)) {
         const float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
         if constexpr (BATCHED) epi(v, (int)batch, m, n);
@@ -1358,7 +1364,7 @@ RX_DEV void rx_gemm_body_pp(const typename EL::elem* __restrict__ A, const typen
     for (int j = 0; j < NB; ++j) {
       const int m = m0 + wm * (BM / WM) + 16 * i + (lane & 15);
       const int n = n0 + wn * (BN / WN) + 16 * j + 4 * (lane >> 4);
-      constexpr bool WHOLE = M % BM == 0 && N % BN == 0;
+      constexpr bool WHOLE = (M % BM == 0 || rx_epi_masks_rows<Epi>::value) && N % BN == 0;
       if (WHOLE || (m < M && n < N)) {
         const float v[4] = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
         if constexpr (BATCHED) epi(v, (int)batch, m, n);

@@ -205,6 +205,25 @@ RX_DEV float rx_gelu_chain_fast(float x, float k1, float k3) {
 // behave as in the division (1/0 = inf, 0 * inf = NaN, ...); double has the range for
 // subnormal divisors.
 RX_DEV float rx_div_uniform(float x, float y) { return (float)((double)x * (1.0 / (double)y)); }
+// Marks a value as used here: the compiler then computes it at this point instead of moving the whole computation
+// into a conditional store that follows (where equal subexpressions of neighbouring calls could no longer be merged).
+template <class V>
+RX_DEV void rx_keep_value(V& v) {
+  if constexpr (sizeof(V) % 4 == 0) {
+    unsigned w[sizeof(V) / 4];
+    __builtin_memcpy(w, &v, sizeof(V));
+#pragma unroll
+    for (unsigned k = 0; k < sizeof(V) / 4; ++k) asm volatile("" : "+v"(w[k]));
+    __builtin_memcpy(&v, w, sizeof(V));
+  }
+}
+// A read of memory that nothing writes while the kernel runs (a bias, batch-norm statistics), through the constant
+// address space: the compiler may then merge equal reads across the kernel's stores, which for a struct member that is
+// only declared __restrict__ it does not.
+template <class T>
+RX_DEV T rx_load_const(const T* p, long long i) {
+  return ((const __attribute__((address_space(4))) T*)p)[i];
+}
 // x / y for a result that is rounded to a narrow float, where y does not vary along the minor dimension (the sum of a
 // softmax row): x times the reciprocal of y, a division that is computed once per row.  The reciprocal of a divisor
 // below 2^-128 would overflow although the quotient is finite (1e-20 / 1e-39), so divisors below 2^-64 are scaled by

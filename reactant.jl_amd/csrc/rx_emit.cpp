@@ -244,7 +244,9 @@ std::string Emitter::emit_load(int node, const Index& ix) {
             std::to_string(vec) + "])";
     }
   } else {
-    raw = "in" + std::to_string(slot) + "[" + (dims.empty() ? std::string("0") : linear(ix, dims)) + "]";
+    const std::string at = dims.empty() ? std::string("0") : linear(ix, dims);
+    if (const_vectors && dims.size() <= 1) raw = "rx_load_const(in" + std::to_string(slot) + ", " + at + ")";
+    else raw = "in" + std::to_string(slot) + "[" + at + "]";
     if (!dims.empty()) ++unsafe_loads_;
   }
   std::string v = fresh();
@@ -291,6 +293,28 @@ bool Emitter::minor_uniform(int node, int depth) const {
       return minor_uniform(n.in[0], depth + 1);
     case OpK::Binary:
       return minor_uniform(n.in[0], depth + 1) && minor_uniform(n.in[1], depth + 1);
+    default:
+      return false;
+  }
+}
+
+bool Emitter::minor_only(int node, int depth) const {
+  const Node& n = g_.nodes[node];
+  if (n.ty.rank() == 0) return true;
+  if (depth > 8) return false;
+  switch (n.k) {
+    case OpK::Constant: return n.splat;
+    case OpK::BroadcastInDim: {
+      const Node& o = g_.nodes[n.in[0]];
+      for (size_t d = 0; d < n.a0.size(); ++d)
+        if (n.a0[d] != n.ty.rank() - 1 && o.ty.dims[d] != 1) return false;
+      return true;
+    }
+    case OpK::Convert:
+    case OpK::Unary:
+      return minor_only(n.in[0], depth + 1);
+    case OpK::Binary:
+      return minor_only(n.in[0], depth + 1) && minor_only(n.in[1], depth + 1);
     default:
       return false;
   }
@@ -462,7 +486,10 @@ std::string Emitter::emit_op(const Node& n, const Index& ix) {
           // (the sum of a softmax row, a quantization scale): its reciprocal, a division of its own that the compiler
           // computes once per row, times the dividend -- within an ulp of float32 of the quotient (rx_div_minor_uniform, which
           // also covers subnormal divisors whose reciprocal would overflow)
-          if (CT == "float" && is_narrow_float(dt) && excess_precision && n.ty.rank() > 0 && minor_uniform(n.in[1])) return def("rx_div_minor_uniform(" + a + ", " + b + ")");
+          // (in a product's epilogue a thread handles many rows of the same columns: there the same holds for a divisor
+          // that varies along the minor dimension only, a per-feature standard deviation)
+          if (CT == "float" && is_narrow_float(dt) && excess_precision && n.ty.rank() > 0 && (minor_uniform(n.in[1]) || (columns_reused && n.ty.rank() >= 2 && minor_only(n.in[1]))))
+            return def("rx_div_minor_uniform(" + a + ", " + b + ")");
           if (CT == "float" && n.ty.rank() > 0 && is_uniform(n.in[1])) return def("rx_div_uniform(" + a + ", " + b + ")");
           return def("(" + a + " / " + b + ")");
         }

@@ -78,6 +78,8 @@ class Emitter {
   // sides and select, instead of branching per element
   bool branchless_guards = false;
   bool offset_perms = false;   // a transposed read may carry constant offsets and read an input of other extents (a padded or sliced transpose)
+  bool const_vectors = false;  // vectors and scalars are read through the constant address space (nothing in the kernel writes them): equal reads merge across stores
+  bool columns_reused = false; // the code runs for many rows of the same columns in one thread (a product's epilogue): values that vary along the minor dimension only are computed once
   bool clamp_guards = false;   // pad: read at positions clamped into the operand and select, instead of a branch around the read
 
   std::string emit(int node, const Index& ix);
@@ -112,6 +114,7 @@ class Emitter {
 
   bool is_uniform(int node, int depth = 0) const;
   bool minor_uniform(int node, int depth = 0) const;
+  bool minor_only(int node, int depth = 0) const;   // the value varies along the minor dimension at most
   std::string emit_load(int node, const Index& ix);
   std::string emit_op(const Node& n, const Index& ix);
   bool match_gelu_chain(const Node& n, int* xnode, double* ka, double* kb) const;

@@ -180,7 +180,146 @@ struct Planner {
     normalize_dots();
     align_dots();
     split_dots();
+    pools_between_convs();
     chain_convs();
+  }
+
+  // Between two convolutions in the product-with-row-shifts form the values live as [image, row, column, channel]: the
+  // first one's result is transposed to [image, channel, row, column] for the ops of the module and the second one's
+  // operand is transposed back.  When everything in between can run in either layout -- elementwise ops whose other
+  // operands vary along the channels only, padding with a scalar, pooling windows (a window view and its reduction)
+  // -- and a pooling window is among them, those ops are rebuilt on the channel-minor layout and both transposes
+  // disappear: the elementwise ops before the first window become the first product's epilogue, the window's reads
+  // run along the channels (16-byte loads) instead of across a transposed operand, and the layout map of the second
+  // product's operand is a plain padding map of the pooled values.  (Chains without a window are chain_convs's.)
+  void pools_between_convs() {
+    if (!opt.nhwc_pools || !opt.mfma) return;
+    const int N = (int)g.nodes.size();
+    std::vector<int> nuse(N, 0);
+    std::vector<std::vector<int>> use(N);
+    for (auto& n : g.nodes) for (int i : n.in) { nuse[i]++; use[i].push_back(n.id); }
+    for (int r : g.results) nuse[r]++;
+    auto elementwise = [](OpK k) { return k == OpK::Unary || k == OpK::Binary || k == OpK::Clamp || k == OpK::Gelu || k == OpK::Convert || k == OpK::Select || k == OpK::Compare; };
+    std::vector<signed char> vec_memo(N, -1);
+    std::function<bool(int, int)> channel_only = [&](int x, int depth) -> bool {
+      if (vec_memo[x] >= 0) return vec_memo[x] != 0;
+      const Node& n = g.nodes[x];
+      bool ok = false;
+      if (n.k == OpK::Constant) ok = n.splat;
+      else if (n.k == OpK::BroadcastInDim) {
+        const TType& st = g.nodes[n.in[0]].ty;
+        ok = n.ty.rank() == 4 && (st.rank() == 0 || (st.rank() == 1 && n.a0.size() == 1 && n.a0[0] == 1 && st.dims[0] == n.ty.dims[1]));
+      } else if (elementwise(n.k) && depth < 12) {
+        ok = !n.in.empty();
+        for (int i : n.in) ok = ok && channel_only(i, depth + 1);
+      }
+      vec_memo[x] = ok ? 1 : 0;
+      return ok;
+    };
+    enum Role : char { None = 0, T1, Elem, PadOp, Win, Red, T2 };
+    std::vector<char> role(N, None);
+    bool any = false;
+    for (const Node& t1 : g.nodes) {
+      if (t1.k != OpK::Transpose || t1.a0 != std::vector<int64_t>{0, 3, 1, 2} || nuse[t1.id] != 1) continue;
+      const Node& c1 = g.nodes[t1.in[0]];
+      if (c1.k != OpK::Conv || c1.a3.size() != 5 || nuse[c1.id] != 1) continue;
+      std::vector<std::pair<int, char>> found{{t1.id, T1}};
+      int cur = t1.id;
+      bool ok = false, pooled = false;
+      for (int depth = 0; depth < 24; ++depth) {
+        if (nuse[cur] != 1 || use[cur].size() != 1) break;
+        const Node& u = g.nodes[use[cur][0]];
+        if (u.k == OpK::Transpose) {
+          ok = u.a0 == std::vector<int64_t>{0, 2, 3, 1} && nuse[u.id] == 1 && use[u.id].size() == 1 && g.nodes[use[u.id][0]].k == OpK::Conv &&
+               g.nodes[use[u.id][0]].a3.size() == 5 && g.nodes[use[u.id][0]].in[0] == u.id;
+          found.push_back({u.id, T2});
+          break;
+        }
+        if (u.ty.rank() != 4 && u.k != OpK::Window) break;
+        if (elementwise(u.k) && u.k != OpK::Compare && u.k != OpK::Select) {
+          int tensors = 0;
+          for (int i : u.in) if (i == cur) ++tensors; else if (!channel_only(i, 0)) tensors = 99;
+          if (tensors != 1) break;
+          found.push_back({u.id, Elem});
+          cur = u.id;
+        } else if (u.k == OpK::Pad) {
+          if (u.in[0] != cur || u.in[1] == cur || g.nodes[u.in[1]].ty.rank() != 0) break;
+          found.push_back({u.id, PadOp});
+          cur = u.id;
+        } else if (u.k == OpK::Window) {
+          if (g.nodes[cur].ty.rank() != 4 || nuse[u.id] != 1 || use[u.id].size() != 1) break;
+          const Node& r = g.nodes[use[u.id][0]];
+          if (r.k != OpK::Reduce || r.in[0] != u.id || r.a0 != std::vector<int64_t>{0, 1, 2, 3} || g.nodes[r.in[1]].ty.rank() != 0) break;
+          found.push_back({u.id, Win});
+          found.push_back({r.id, Red});
+          pooled = true;
+          cur = r.id;
+        } else break;
+      }
+      if (!ok || !pooled) continue;
+      for (auto& f : found) role[f.first] = f.second;
+      any = true;
+    }
+    if (!any) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(N, -1);
+    // old dimension i is new dimension P[i]
+    static const int P[4] = {0, 3, 1, 2};
+    auto permuted = [&](const std::vector<int64_t>& v) { std::vector<int64_t> r(4); for (int i = 0; i < 4; ++i) r[P[i]] = v[i]; return r; };
+    std::map<std::pair<int, std::vector<int64_t>>, int> memo;
+    std::function<int(int, const std::vector<int64_t>&)> rebuild_vec = [&](int x, const std::vector<int64_t>& dims) -> int {
+      auto it = memo.find({x, dims});
+      if (it != memo.end()) return it->second;
+      Node c = g.nodes[x];
+      c.ty.dims = dims;
+      if (c.k == OpK::BroadcastInDim) {
+        c.in = {remap[c.in[0]]};
+        if (!c.a0.empty()) c.a0 = {3};
+      } else if (c.k != OpK::Constant) {
+        for (int& i : c.in) i = rebuild_vec(i, dims);
+      }
+      return memo[{x, dims}] = out.add(c);
+    };
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      switch (role[n.id]) {
+        case T1: case T2:
+          remap[n.id] = remap[n.in[0]];
+          continue;
+        case Elem: {
+          c.ty.dims = permuted(n.ty.dims);
+          for (int& i : c.in) i = role[i] != None ? remap[i] : rebuild_vec(i, c.ty.dims);
+          break;
+        }
+        case PadOp:
+          c.ty.dims = permuted(n.ty.dims);
+          c.a0 = permuted(n.a0); c.a1 = permuted(n.a1); c.a2 = permuted(n.a2);
+          for (int& i : c.in) i = remap[i];
+          break;
+        case Win: {
+          c.a0 = permuted(n.a0); c.a1 = permuted(n.a1); c.a2 = permuted(n.a2);
+          const std::vector<int64_t> k = permuted(std::vector<int64_t>(n.ty.dims.begin(), n.ty.dims.begin() + 4));
+          const std::vector<int64_t> o = permuted(std::vector<int64_t>(n.ty.dims.begin() + 4, n.ty.dims.end()));
+          c.ty.dims = k;
+          c.ty.dims.insert(c.ty.dims.end(), o.begin(), o.end());
+          for (int& i : c.in) i = remap[i];
+          break;
+        }
+        case Red:
+          c.ty.dims = permuted(n.ty.dims);
+          for (int& i : c.in) i = remap[i];
+          break;
+        default:
+          for (int& i : c.in) i = remap[i];
+      }
+      remap[n.id] = out.add(c);
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // Two convolutions in the product-with-row-shifts form (OpK::Conv with a3) with nothing between them but elementwise
@@ -867,6 +1006,27 @@ struct Planner {
       if (live[x]) for (int i : g.nodes[x].in) users[i].push_back(x);
     std::vector<char> is_result(N, 0);
     for (int r : g.results) is_result[r] = 1;
+
+    // The elementwise ops that follow a convolution one after the other (conversion to the images' type, batch norm,
+    // bias, activation) end where something reads their value at other positions (a pooling window, a layout change):
+    // the value is written there, so that the chain runs once per element in the convolution's kernel, in the
+    // type it ends in, instead of once per read in the reader's.
+    if (opt.product_epilogues && opt.conv_tails) {
+      auto pointwise = [](OpK k) { return k == OpK::Unary || k == OpK::Binary || k == OpK::Clamp || k == OpK::Convert || k == OpK::Select || k == OpK::Gelu; };
+      for (int c = 0; c < N; ++c) {
+        if (!live[c] || g.nodes[c].k != OpK::Conv) continue;
+        int cur = c;
+        while (!is_result[cur] && users[cur].size() == 1) {
+          const Node& un = g.nodes[users[cur][0]];
+          if (!pointwise(un.k) || un.ty.dims != g.nodes[c].ty.dims) break;
+          cur = un.id;
+        }
+        if (cur == c || is_result[cur]) continue;
+        bool index_reader = !users[cur].empty();
+        for (int u : users[cur]) index_reader = index_reader && (is_index_op(g.nodes[u].k) || g.nodes[u].k == OpK::Reduce);
+        if (index_reader) force_mat[cur] = 1;
+      }
+    }
 
     for (int x = N - 1; x >= 0; --x) {
       if (!live[x]) continue;
@@ -2982,15 +3142,28 @@ struct Planner {
     em.direct_expr = vec_name;
     em.indent = 6;
     em.bound[conv] = "accv";
+    em.columns_reused = shifted;
+    em.const_vectors = shifted;
     const std::string val = root == conv ? std::string("accv") : em.emit(root, root_index(rn.ty.dims));
     const std::string ebody = em.take_code();
     const std::string ost = info(rn.ty.dt).stype;
+    // The compact form of the shifted product drops the rows that are not results.  When the epilogue reads per-feature
+    // vectors only (bias, batch norm) the test guards the store alone: the arithmetic is then straight-line code over all
+    // the rows a thread handles, and what depends on the column only (the vectors' loads and conversions, a square root,
+    // a reciprocal) is computed once per column instead of once per row.
+    bool vectors_only = shifted && !em.inputs.empty();
+    for (int i : em.inputs) vectors_only = vectors_only && g.nodes[i].ty.rank() <= 1;
+    for (auto& l : em.loads) vectors_only = vectors_only && (g.nodes[l.node].ty.rank() == 0 || l.minor_follows);   // read at the column only: in range on every row
+    const bool late_mask = vectors_only && cn.a3.size() == 5;
+    // (the grid form computes every row anyway and guards its stores by the row number: it takes the rows past the last one too)
+    const bool grid_all_rows = vectors_only && cn.a3.size() == 8;
     std::ostringstream o;
     o << "// convolution epilogue: " << describe(root) << "\n";
     o << "struct @K@_epi {\n";
     for (size_t k = 0; k < em.inputs.size(); ++k)
       o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
     o << "  " << ost << "* __restrict__ out0;\n";
+    if (late_mask || grid_all_rows) o << "  static constexpr bool masks_rows = true;\n";
     o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const float (&acc)[NV]";
     if (shifted) {
       // called with (row of the product, first column): the row is a position of the padded grid, of which the
@@ -3001,6 +3174,8 @@ struct Planner {
       if (cn.a3.size() == 8) {
         // the grid form (chain_convs): every row is written, the ones that are not results as zeros
         o << "    const bool result_ = i1 < " << cn.a3[5] << " && i2 < " << cn.a3[6] << ";\n";
+      } else if (late_mask) {
+        o << "    const bool keep_ = i0 < " << rn.ty.dims[0] << " && i1 < " << rn.ty.dims[1] << " && i2 < " << rn.ty.dims[2] << ";\n";
       } else {
         o << "    if (i1 >= " << rn.ty.dims[1] << " || i2 >= " << rn.ty.dims[2] << ") return;\n";
       }
@@ -3031,10 +3206,12 @@ struct Planner {
       const int64_t rows = cn.ty.dims[0] * cn.a3[3] * cn.a3[4], ncol = cn.ty.dims[3];
       o << "    rx_vec<" << ost << ", NV> zero_;\n#pragma unroll\n    for (int l = 0; l < NV; ++l) zero_.v[l] = 0;\n";
       o << "    if (!result_) res = zero_;\n";
+      if (grid_all_rows) o << "    rx_keep_value(res);\n";
       o << "    if (row_ + " << cn.a3[7] << " < " << rows << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0 + " << cn.a3[7] * ncol << ") = res;\n";
       if (cn.a3[7] > 0) o << "    if (row_ < " << cn.a3[7] << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = zero_;\n";
     } else {
-      o << "    *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+      if (late_mask) o << "    rx_keep_value(res);\n";
+      o << "    " << (late_mask ? "if (keep_) " : "") << "*reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
     }
     o << "  }\n};\n\n";
     if (shifted) {
@@ -3333,10 +3510,21 @@ struct Planner {
     // are one 16-byte access (the per-output order of the sum does not change); the chunk loop is unrolled to keep
     // eight such loads in flight (column sum of an 8192 x 8192 f32 matrix: 4.1 -> 6.3 TB/s).
     int VEC = 1;
-    if (!kept.empty() && !red.empty() && kept.back() == inn.ty.rank() - 1 && (info(inn.ty.dt).size == 4 || info(inn.ty.dt).size == 8) &&
-        info(dt).size == info(inn.ty.dt).size) {
-      const int v = 16 / info(inn.ty.dt).size;
-      if (inn.ty.dims[kept.back()] % v == 0 && nout / v >= 64 && red_len >= 16) VEC = v;
+    // 16-bit elements take it for short reductions too (pooling windows: eight outputs per thread, 16-byte loads where the
+    // window view's minor dimension is the operand's).
+    const int esz = info(inn.ty.dt).size;
+    if (!kept.empty() && !red.empty() && kept.back() == inn.ty.rank() - 1 && (esz == 2 || esz == 4 || esz == 8) && info(dt).size == esz) {
+      const int v = 16 / esz;
+      // (not when the reads are transposed or gathered: eight outputs along the minor dimension would be eight strides apart)
+      bool short_ok = esz == 2 && opt.window_reduce_vectors && red_len >= 2;
+      if (short_ok)
+        for (int x : cone_nodes(rn.in[0])) {
+          const OpK k = g.nodes[x].k;
+          if (x != rn.in[0] && mat[x]) continue;
+          if (is_index_op(k) && k != OpK::Window && k != OpK::BroadcastInDim && k != OpK::Pad) short_ok = false;
+        }
+      const bool long_enough = esz == 2 ? short_ok : red_len >= 16;
+      if (inn.ty.dims[kept.back()] % v == 0 && nout / v >= 64 && long_enough) VEC = v;
     }
     const int64_t nthr = nout / VEC;
     int64_t split = 1;

@@ -56,6 +56,8 @@ struct PlanOptions {
   bool split_k = true;          // matrix products with few output tiles and a long contraction: K in slices, partial products, a reduction
   bool chain_convs = true;      // two 16-bit convolutions with only channel-wise elementwise ops and padding between them share the padded grid: no map in between
   bool product_epilogues = true;  // the elementwise ops that consume a product or convolution run in its kernel (off: a map after it; for comparisons)
+  bool conv_tails = true;       // the elementwise chain after a convolution is written where a window, reduction or layout change reads it (it runs in the convolution's kernel)
+  bool nhwc_pools = true;       // pooling windows (and the elementwise ops and padding around them) between two 16-bit convolutions run on the channel-minor layout: no transposes
   bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles
@@ -68,6 +70,7 @@ struct PlanOptions {
   // device-scope release fence before a ticket -- an L2 write-back on this multi-die part -- was 2x slower.)
   bool single_pass_reduce = false;
   bool single_pass_scan = true;      // long scanned rows in one launch (chunk totals travel as flagged words)
+  bool window_reduce_vectors = true;  // reductions over 16-bit elements that keep the minor dimension (pooling windows): eight outputs per thread
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool clamp_pad_reads = true;     // maps over 8- and 16-bit elements: padded reads at clamped positions and a select, so that a lane's loads combine

@@ -234,6 +234,67 @@ def vgg_block(batch=2, cin=3, cmid=8, hw=16, classes=10, dt="f32"):
     return ("module {\n  func.func @main(%s) -> %s {\n    %s\n    return %%out : %s\n  }\n}\n" % (sig, OUT, "\n    ".join(lines), OUT)), shapes
 
 
+VGG11_LAYERS = (64, "M", 128, "M", 256, 256, "M", 512, 512, "M", 512, 512, "M")
+
+
+def vgg11(batch=4, hw=224, classes=1000, dt="f32", layers=VGG11_LAYERS, dense=4096, cin=3):
+    """Forward pass of VGG-11 with batch norm in test mode, the model of benchmark/nn/vision.jl:24-34
+    (`Vision.VGG(11; batchnorm=true)` on [224, 224, 3, 4]): per entry of `layers` a 3x3 convolution (padding 1, no bias) +
+    batch_norm_inference + relu, or ("M") a 2x2 max pool; then flatten, two dense layers of `dense` features with relu and
+    one of `classes` (logits).  Arguments: the images [batch, cin, hw, hw]; per convolution its filter and the batch
+    norm's scale, offset, mean, variance; per dense layer its matrix [in, out] and its bias."""
+    S = tt([], dt)
+    conv = ("stablehlo.convolution(%s, %s) dim_numbers = [b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0], window = {stride = [1, 1], "
+            "pad = [[1, 1], [1, 1]], rhs_dilate = [1, 1]} {batch_group_count = 1 : i64, feature_group_count = 1 : i64} : (%s, %s) -> %s")
+    pool = ("\"stablehlo.reduce_window\"(%s, %%ninf) <{base_dilations = array<i64: 1, 1, 1, 1>, padding = dense<0> : tensor<4x2xi64>, "
+            "window_dilations = array<i64: 1, 1, 1, 1>, window_dimensions = array<i64: 1, 1, 2, 2>, window_strides = array<i64: 1, 1, 2, 2>}> ({\n"
+            "    ^bb0(%%p: %s, %%q: %s):\n      %%m = stablehlo.maximum %%p, %%q : %s\n      stablehlo.return %%m : %s\n    }) : (%s, %s) -> %s")
+    lines = ["%ninf = stablehlo.constant dense<" + _init_literal("maximum", dt) + "> : " + S]
+    args, shapes = [tt([batch, cin, hw, hw], dt)], [[batch, cin, hw, hw]]
+    cur, c, h, flops = "%arg0", cin, hw, 0.0
+    for k, l in enumerate(layers):
+        T = tt([batch, c, h, h], dt)
+        if l == "M":
+            P = tt([batch, c, h // 2, h // 2], dt)
+            lines.append("%%l%d = " % k + pool % (cur, S, S, S, S, T, S, P))
+            h //= 2
+        else:
+            A, F = tt([batch, l, h, h], dt), tt([l], dt)
+            a = len(args)
+            args += [tt([l, c, 3, 3], dt), F, F, F, F]
+            shapes += [[l, c, 3, 3], [l], [l], [l], [l]]
+            lines.append("%%c%d = " % k + conv % (cur, "%%arg%d" % a, T, tt([l, c, 3, 3], dt), A))
+            lines.append("%%n%d = \"stablehlo.batch_norm_inference\"(%%c%d, %%arg%d, %%arg%d, %%arg%d, %%arg%d) <{epsilon = 1.000000e-05 : f32, feature_index = 1 : i64}> : (%s) -> %s"
+                         % (k, k, a + 1, a + 2, a + 3, a + 4, ", ".join([A, F, F, F, F]), A))
+            lines.append("%%z%d = stablehlo.constant dense<0.000000e+00> : %s" % (k, A))
+            lines.append("%%l%d = stablehlo.maximum %%n%d, %%z%d : %s" % (k, k, k, A))
+            flops += 2.0 * batch * l * h * h * c * 9
+            c = l
+        cur = "%%l%d" % k
+    feat = c * h * h
+    lines.append("%%f = stablehlo.reshape %s : (%s) -> %s" % (cur, tt([batch, c, h, h], dt), tt([batch, feat], dt)))
+    cur = "%f"
+    for k, n in enumerate((dense, dense, classes)):
+        X, W, Bv, O = tt([batch, feat], dt), tt([feat, n], dt), tt([n], dt), tt([batch, n], dt)
+        a = len(args)
+        args += [W, Bv]
+        shapes += [[feat, n], [n]]
+        lines.append("%%d%d = stablehlo.dot_general %s, %%arg%d, contracting_dims = [1] x [0] : (%s, %s) -> %s" % (k, cur, a, X, W, O))
+        lines.append("%%bb%d = stablehlo.broadcast_in_dim %%arg%d, dims = [1] : (%s) -> %s" % (k, a + 1, Bv, O))
+        lines.append("%%s%d = stablehlo.add %%d%d, %%bb%d : %s" % (k, k, k, O))
+        cur = "%%s%d" % k
+        if k < 2:
+            lines.append("%%dz%d = stablehlo.constant dense<0.000000e+00> : %s" % (k, O))
+            lines.append("%%e%d = stablehlo.maximum %%s%d, %%dz%d : %s" % (k, k, k, O))
+            cur = "%%e%d" % k
+        flops += 2.0 * batch * feat * n
+        feat = n
+    OUT = tt([batch, classes], dt)
+    sig = ", ".join("%%arg%d: %s" % (k, t) for k, t in enumerate(args))
+    text = "module {\n  func.func @main(%s) -> %s {\n    %s\n    return %s : %s\n  }\n}\n" % (sig, OUT, "\n    ".join(lines), cur, OUT)
+    return text, shapes, flops
+
+
 def attention_block(batch_heads=6, seq=40, dim=16, dt="f32"):
     """softmax(q k^T / sqrt(d)) v on [batch*heads, seq, dim] operands: the two batched products and the
     row softmax of NNlib.dot_product_attention, which the ViT of benchmark/nn/vision.jl:5-22 runs."""

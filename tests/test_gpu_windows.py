@@ -427,6 +427,47 @@ def test_vgg_style_forward_pass_in_bf16(rx, client):
     _close(got[0].a, ref[0].a, 3e-2)
 
 
+def _vgg11_args(shapes, dt, seed=23):
+    rng = np.random.default_rng(seed)
+    args = []
+    for k, sh in enumerate(shapes):
+        if len(sh) == 1 and 0 < k <= 40 and (k - 1) % 5 == 4:       # running variances
+            args.append(I.tensor(rng.uniform(0.5, 2.0, size=sh), dt))
+        elif len(sh) == 1 and 0 < k <= 40 and (k - 1) % 5 == 1:     # batch norm scales
+            args.append(I.tensor(rng.uniform(0.8, 1.6, size=sh), dt))
+        elif len(sh) == 4 and k > 0:
+            args.append(I.tensor(rng.normal(size=sh) * np.sqrt(2.0 / np.prod(sh[1:])), dt))
+        elif len(sh) == 2:
+            args.append(I.tensor(rng.normal(size=sh) * np.sqrt(2.0 / sh[0]), dt))
+        else:
+            args.append(I.tensor(rng.normal(size=sh) * (1.0 if k == 0 else 0.3), dt))
+    return args
+
+
+@pytest.mark.parametrize("dt,nhwc", [("f32", True), ("bf16", True), ("bf16", False), ("f16", True)])
+def test_vgg11_forward_pass(rx, client, monkeypatch, dt, nhwc):
+    """The whole VGG-11 forward pass with batch norm in test mode (eight 3x3 convolutions + batch norm + relu, five
+    2x2 max pools, three dense layers) at small sizes.  In 16 bits the pooling windows between two products with row
+    shifts run on the channel-minor layout (no transposes between them; RX_NHWC_POOLS=0: through the transposes),
+    the batch norm + relu as the products' epilogues.  Against the oracle."""
+    if not nhwc:
+        monkeypatch.setenv("RX_NHWC_POOLS", "0")
+    layers = (64, "M", 64, "M", 64, 64, "M", 64, 64, "M", 64, 64, "M")
+    text, shapes, _ = NN.vgg11(batch=4, hw=64, classes=10, dt=dt, layers=layers, dense=96, cin=3)
+    args = _vgg11_args(shapes, dt)
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    if dt != "f32":
+        assert kinds.count("conv_" + dt) == 7, kinds
+        pools = [ln.split("::")[1] for ln in rx.compile_offline(text).splitlines() if "kind=reduce_generic" in ln and "window" in ln]
+        assert len(pools) == 5
+        # the pools between two products: pure window reductions on the channel-minor layout when the rewrite is on
+        assert sum(d.strip() == "window reduce" for d in pools) == (4 if nhwc else 1), pools
+    ref = oracle_run(text, args, hifi=True)
+    assert got[0].a.shape == (4, 10)
+    _close(got[0].a, ref[0].a, {"f32": 2e-4, "bf16": 5e-2, "f16": 8e-3}[dt])
+
+
 @pytest.mark.parametrize("bh,seq,dim,dt,tol", [(6, 40, 16, "f32", 1e-5), (8, 256, 64, "f32", 1e-4), (8, 256, 64, "bf16", 2e-2)])
 def test_attention_block(rx, client, bh, seq, dim, dt, tol):
     text, shapes = NN.attention_block(bh, seq, dim, dt)
