@@ -515,6 +515,7 @@ def _window_entry(name, exe, secs, steps, mean_ms, algo_bytes, flops, dtype, bou
         ach = flops / (secs / steps) / 1e12
         entry.update(value=ach, unit="TFLOP/s")
         dot = [i for i, l in enumerate(launches) if l["flops"] > 0]
+        dot.sort(key=lambda i: -float(mean_ms[i]))      # the longest of the launches that multiply
         kms = float(mean_ms[dot[0]]) if dot else float(mean_ms[big])
         kach = (launches[dot[0]]["flops"] if dot else flops) / (kms * 1e-3) / 1e12   # that launch's own flops (a chain has several)
         entry["roofline"] = {"bound": "mfma", "kernel": launches[dot[0] if dot else big]["kernel"], "kernel_ms": kms, "achieved": kach,
@@ -553,6 +554,38 @@ def bench_conv16(rx, client, P, steps, warmup, batch=32, channels=256, hw=56, la
     flops = layers * 2.0 * batch * channels * hw * hw * channels * 9
     return _window_entry("%d x (conv 3x3 pad 1 bf16 %dx%dx%dx%d -> %d features, bias + relu)" % (layers, batch, channels, hw, hw, channels), exe, secs, steps, mean_ms,
                          0.0, flops, "bf16", "bf16")
+
+
+def bench_vgg11(rx, client, P, steps, warmup, batch=4, dt="f32", hw=224, layers=None, dense=4096):
+    """Forward pass of VGG-11 with batch norm in test mode on `batch` images of 224 x 224 (the model and input of
+    benchmark/nn/vision.jl:24-34, there in f32 on 4 images): eight 3x3 convolutions + batch norm + relu, five max pools,
+    three dense layers; `value` counts the convolutions' and dense layers' flops."""
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    text, shapes, flops = NN.vgg11(batch=batch, hw=hw, dt=dt, layers=layers or NN.VGG11_LAYERS, dense=dense)
+    exe = rx.xla_compile(client, text)
+    rng = np.random.default_rng(0)
+    nconv = sum(1 for l in (layers or NN.VGG11_LAYERS) if l != "M")
+
+    def values(k, s):
+        if len(s) == 1 and 0 < k <= 5 * nconv and (k - 1) % 5 == 4:
+            return rng.uniform(0.5, 2.0, size=s)                       # running variances
+        if len(s) == 4 and k > 0:
+            return rng.normal(size=s) * np.sqrt(2.0 / np.prod(s[1:]))
+        if len(s) == 2:
+            return rng.normal(size=s) * np.sqrt(2.0 / s[0])
+        return rng.normal(size=s)
+    bufs = [_upload(rx, client, rx.encode(values(k, s).astype(np.float32), dt) if dt != "f32" else values(k, s).astype(np.float32), dt) for k, s in enumerate(shapes)]
+    # a step of 24 to 35 launches: timed as a caller runs it; the per-launch times come from a second pass with an event pair on every launch
+    plain = _time_plain(client, exe, bufs, steps, warmup)
+    secs, mean_ms, _ = _time_steps(rx, client, exe, lambda prev: (bufs, [0] * len(bufs)), steps, warmup)
+    entry = _window_entry("VGG-11 (batch norm, test mode) forward, %s, %d x 3 x %d x %d" % (dt, batch, hw, hw), exe, plain * steps, steps, mean_ms, 0.0, flops, dt, dt)
+    entry["with_launch_events"] = {"ms_per_step": 1e3 * secs / steps, "kernel_ms_sum": float(np.sum(mean_ms))}
+    entry["roofline"]["timed_in"] = "with_launch_events"
+    return entry
+
+
+def bench_vgg11_bf16(rx, client, P, steps, warmup, batch=32, **kw):
+    return bench_vgg11(rx, client, P, steps, warmup, batch=batch, dt="bf16", **kw)
 
 
 def bench_cumsum(rx, client, P, steps, warmup, n=1 << 26):
@@ -709,7 +742,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "conv16", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
+    ap.add_argument("--workload", default="stencil", choices=["stencil", "sinsum", "gemm", "mlp", "fp8", "conv", "conv16", "vgg11", "vgg11_bf16", "cumsum", "maxpool", "colsum", "transpose", "polybench", "polybench_linalg"])
     ap.add_argument("--settle-ms", type=float, default=150.0, help="untimed executions of a workload before its warm-up steps until the device has been under that load this long (0: none)")
     ap.add_argument("--no-others", action="store_true", help="skip the other four configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
@@ -724,9 +757,9 @@ def main():
     P = importlib.import_module("reactant_jl_amd.programs")
     client = rx.set_default_backend("gpu")
     table = {"stencil": bench_stencil, "sinsum": bench_sinsum, "gemm": bench_gemm, "mlp": bench_mlp, "fp8": bench_fp8,
-             "conv": bench_conv, "conv16": bench_conv16, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "colsum": bench_colsum, "transpose": bench_transpose, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
+             "conv": bench_conv, "conv16": bench_conv16, "vgg11": bench_vgg11, "vgg11_bf16": bench_vgg11_bf16, "cumsum": bench_cumsum, "maxpool": bench_maxpool, "colsum": bench_colsum, "transpose": bench_transpose, "polybench": bench_polybench, "polybench_linalg": bench_polybench_linalg}
     small = {"stencil": dict(nx=128, ny=128, nz=64), "sinsum": dict(n=1 << 22), "gemm": dict(n=1024),
-             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28), "conv16": dict(batch=2, channels=64, hw=28),
+             "mlp": dict(batch=1024, widths=(256, 512, 512, 256)), "fp8": dict(n=1024), "conv": dict(batch=2, hw=28), "conv16": dict(batch=2, channels=64, hw=28), "vgg11": dict(batch=2, hw=32, dense=64), "vgg11_bf16": dict(batch=2, hw=32, dense=64),
              "cumsum": dict(n=1 << 20), "maxpool": dict(batch=4), "colsum": dict(n=1024), "transpose": dict(n=1024), "polybench": dict(scale=16), "polybench_linalg": dict(scale=8)}
     _FULL_SIZE[0] = not args.small
     OPTS["check"], OPTS["cpu"], OPTS["settle_ms"] = not args.no_check, not args.no_cpu, args.settle_ms

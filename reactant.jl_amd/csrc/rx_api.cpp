@@ -286,7 +286,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_STENCIL_FUSE")) o.stencil_fuse_steps = atoi(e) != 0;
   if (const char* e = getenv("RX_SPLIT_K")) o.split_k = atoi(e) != 0;
   if (const char* e = getenv("RX_WINDOW_VECTORS")) o.window_reduce_vectors = atoi(e) != 0;
-  if (const char* e = getenv("RX_CONV_TAILS")) o.conv_tails = atoi(e) != 0;
+  if (const char* e = getenv("RX_CONV_TAILS")) o.conv_tails = atoi(e);
   if (const char* e = getenv("RX_NHWC_POOLS")) o.nhwc_pools = atoi(e) != 0;
   if (const char* e = getenv("RX_EPILOGUES")) o.product_epilogues = atoi(e) != 0;
   if (const char* e = getenv("RX_EPILOGUE_INIT")) o.epilogue_init = atoi(e) != 0;

@@ -1022,6 +1022,10 @@ struct Planner {
           cur = un.id;
         }
         if (cur == c || is_result[cur]) continue;
+        // (measured on VGG-11: with 16-bit results the readers, bound by memory, get twice as fast and the convolutions
+        // pay less than that; with f32 results the division and square root of a batch norm cost the convolution
+        // kernels more than the pooling kernels gain)
+        if (opt.conv_tails < 2 && info(g.nodes[cur].ty.dt).size >= 4) continue;
         bool index_reader = !users[cur].empty();
         for (int u : users[cur]) index_reader = index_reader && (is_index_op(g.nodes[u].k) || g.nodes[u].k == OpK::Reduce);
         if (index_reader) force_mat[cur] = 1;

@@ -56,7 +56,7 @@ struct PlanOptions {
   bool split_k = true;          // matrix products with few output tiles and a long contraction: K in slices, partial products, a reduction
   bool chain_convs = true;      // two 16-bit convolutions with only channel-wise elementwise ops and padding between them share the padded grid: no map in between
   bool product_epilogues = true;  // the elementwise ops that consume a product or convolution run in its kernel (off: a map after it; for comparisons)
-  bool conv_tails = true;       // the elementwise chain after a convolution is written where a window, reduction or layout change reads it (it runs in the convolution's kernel)
+  int conv_tails = 1;           // the elementwise chain after a convolution is written where a window, reduction or layout change reads it, so that it runs in the convolution's kernel: 1 when it ends in a type narrower than the f32 accumulators, 2 always, 0 never
   bool nhwc_pools = true;       // pooling windows (and the elementwise ops and padding around them) between two 16-bit convolutions run on the channel-minor layout: no transposes
   bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers

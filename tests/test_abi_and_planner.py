@@ -317,6 +317,43 @@ def test_windowed_ops_plan(monkeypatch):
     monkeypatch.delenv("RX_EPILOGUES")
 
 
+def test_vgg11_forward_pass_plans(monkeypatch):
+    """VGG-11 with batch norm in test mode (benchmark/nn/vision.jl:24-34).  In f32 on 4 images: the direct kernel where it
+    covers the layer; batch norm + relu run in the pooling kernel that reads the convolution (RX_CONV_TAILS=2: in the
+    convolution's epilogue, the pools as pure window reductions).  In bf16 on 32 images: seven products with row shifts
+    with batch norm + relu as their epilogues (results narrower than the accumulators are written where a window reads
+    them); the pools between two of them run channel-minor -- no transposing map on either side, a padding map after
+    them -- and take eight outputs per thread; convolutions that follow one another directly are chained."""
+    import _nn_modules as NN
+    parse = lambda rep: [(ln.split("kind=")[1].split()[0], ln.split("::")[1].strip()) for ln in rep.splitlines() if "kind=" in ln]
+    f32 = parse(rx.compile_offline(NN.vgg11(batch=4, dt="f32")[0]))
+    assert [k for k, _ in f32].count("conv") == 6
+    assert [d for k, d in f32 if k == "conv"].count("convolution") == 4 and sum("window" in d and "divide" in d for _, d in f32) >= 4, f32
+    monkeypatch.setenv("RX_CONV_TAILS", "2")
+    f32 = parse(rx.compile_offline(NN.vgg11(batch=4, dt="f32")[0]))
+    assert all("divide" in d and "maximum" in d for k, d in f32 if k == "conv")
+    assert [d for k, d in f32 if k == "reduce_generic" and "window" in d][:4] == ["window reduce"] * 4
+    monkeypatch.delenv("RX_CONV_TAILS")
+    text = NN.vgg11(batch=32, dt="bf16")[0]
+    rep = rx.compile_offline(text, with_source=True)
+    bf16 = parse(rep)
+    kinds = [k for k, _ in bf16]
+    assert kinds.count("conv_bf16") == 7 and kinds.count("conv") == 1 and kinds.count("map_transposed") == 1, kinds
+    assert [d for k, d in bf16 if "window" in d][:4] == ["window reduce"] * 4
+    assert [d for k, d in bf16 if k == "map" and d.startswith("pad")] == ["pad"] * 3
+    assert "static constexpr bool masks_rows = true;" in rep and "rx_keep_value(res);" in rep and "rx_load_const(in0, " in rep
+    i = rep.index("// reduce (generic): window over dims -> tensor<32x56x56x128xbf16>")
+    assert "threadIdx.x) * 8;" in rep[i:i + 400]
+    monkeypatch.setenv("RX_NHWC_POOLS", "0")
+    off = parse(rx.compile_offline(text))
+    assert [k for k, _ in off].count("map_transposed") == 4 and sum("transpose window" in d for _, d in off) == 4, off
+    monkeypatch.delenv("RX_NHWC_POOLS")
+    monkeypatch.setenv("RX_CONV_TAILS", "0")
+    off = parse(rx.compile_offline(text))
+    assert sum("window" in d and "divide" in d for _, d in off) == 5, off
+    monkeypatch.delenv("RX_CONV_TAILS")
+
+
 def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
     """The reference's polybench stencils (benchmark/polybench/stencil.jl) at its sizes: 1024 or 256
     trips of a `stablehlo.while` unroll into runs of update steps, which share chain kernels."""
