@@ -1101,6 +1101,111 @@ struct Planner {
     }
   }
 
+  // Plain maps that read nothing but arguments and constants of the module (the layout maps of a network's filters, a
+  // conversion of its first images) depend on no other launch: they go to the front of the launch list, and when
+  // there are several they run as one launch -- each map's kernel becomes a device function that takes the workgroup
+  // number as its first parameter, and one kernel sends ranges of workgroup numbers to them.  Small maps cost a launch
+  // each (4 us between dependent launches) for a microsecond of work.
+  void merge_parameter_maps() {
+    if (!opt.merge_parameter_maps) return;
+    std::map<std::string, std::string> text_of;   // kernel symbol prefix -> its text
+    for (auto& kv : dedupe) text_of[kv.second] = named(kv.first, kv.second);
+    std::vector<size_t> picked;
+    std::vector<char> written(plan.buffers.size(), 0);
+    for (auto& L : plan.launches)
+      for (int k = 0; k < L.n_outputs; ++k) written[L.args[L.args.size() - 1 - k]] = 1;
+    for (size_t li = 0; li < plan.launches.size(); ++li) {
+      const Launch& L = plan.launches[li];
+      if (L.kind != "map" || L.grid[1] != 1 || L.grid[2] != 1 || L.block[0] != (unsigned)kBlock || L.lds_bytes != 0 || L.n_outputs != 1 || L.args.empty()) continue;
+      bool ok = L.grid[0] <= 16384;
+      for (size_t a = 0; a + 1 < L.args.size(); ++a) {
+        const BufferDesc& B = plan.buffers[L.args[a]];
+        ok = ok && (B.kind == BufferDesc::Param || B.kind == BufferDesc::Const) && !written[L.args[a]];
+      }
+      const BufferDesc& O = plan.buffers[L.args.back()];
+      ok = ok && O.kind == BufferDesc::Temp && !O.is_result;   // operands prepared for later launches, not results of the module
+      // the only launch that writes its result
+      int writers = 0;
+      for (auto& M : plan.launches)
+        for (int k = 0; k < M.n_outputs; ++k) writers += M.args[M.args.size() - 1 - k] == L.args.back();
+      ok = ok && writers == 1;
+      const size_t us = L.kernel.rfind("_map");
+      if (!ok || us == std::string::npos || us + 4 != L.kernel.size()) continue;
+      auto it = text_of.find(L.kernel.substr(0, us));
+      if (it == text_of.end()) continue;
+      const std::string& t = it->second;
+      const std::string sig = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + L.kernel + "(";
+      const size_t at = t.find(sig);
+      if (at == std::string::npos || t.find("__global__", at + sig.size()) != std::string::npos || t.find("__global__") != at + 11 ||
+          t.find("gridDim") != std::string::npos || t.find("blockIdx.y") != std::string::npos || t.find("blockIdx.z") != std::string::npos || t.find("__shared__") != std::string::npos)
+        continue;
+      picked.push_back(li);
+    }
+    if (picked.size() < 2) return;
+    std::vector<Launch> front, rest;
+    for (size_t li = 0, q = 0; li < plan.launches.size(); ++li) {
+      if (q < picked.size() && picked[q] == li) { front.push_back(plan.launches[li]); ++q; }
+      else rest.push_back(plan.launches[li]);
+    }
+    {
+      std::ostringstream o;
+      o << "// " << front.size() << " maps of the module's arguments in one launch\n";
+      std::set<std::string> defined;
+      std::vector<std::vector<std::pair<std::string, std::string>>> params(front.size());   // per map: (type, name)
+      for (size_t f = 0; f < front.size(); ++f) {
+        const Launch& L = front[f];
+        const std::string& t = text_of[L.kernel.substr(0, L.kernel.size() - 4)];
+        const std::string sig = "extern \"C\" __global__ __launch_bounds__(" + std::to_string(kBlock) + ") void " + L.kernel + "(";
+        const size_t at = t.find(sig), close = t.find(") {", at);
+        const std::string plist = t.substr(at + sig.size(), close - at - sig.size());
+        for (size_t q = 0; q < plist.size();) {
+          size_t e = plist.find(", ", q);
+          if (e == std::string::npos) e = plist.size();
+          const std::string d = plist.substr(q, e - q);
+          const size_t sp = d.rfind(' ');
+          params[f].push_back({d.substr(0, sp), d.substr(sp + 1)});
+          q = e + 2;
+        }
+        if (params[f].size() != L.args.size()) return;   // not the text this pass understands: leave the plan as it is
+        if (!defined.insert(L.kernel).second) continue;
+        std::string body = t.substr(close + 3);
+        for (size_t q; (q = body.find("blockIdx.x")) != std::string::npos;) body.replace(q, 10, "bid_");
+        o << "static __device__ __forceinline__ void " << L.kernel << "_part(const unsigned bid_, " << plist << ") {" << body;
+      }
+      o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void @K@_maps(";
+      for (size_t f = 0; f < front.size(); ++f)
+        for (size_t a = 0; a < params[f].size(); ++a) o << (f + a ? ", " : "") << params[f][a].first << " m" << f << "_" << params[f][a].second;
+      o << ") {\n";
+      Launch F;
+      unsigned first = 0;
+      for (size_t f = 0; f < front.size(); ++f) {
+        const Launch& L = front[f];
+        o << "  if (blockIdx.x < " << first + L.grid[0] << "u) { " << L.kernel << "_part(blockIdx.x - " << first << "u";
+        for (size_t a = 0; a < params[f].size(); ++a) o << ", m" << f << "_" << params[f][a].second;
+        o << "); return; }\n";
+        first += L.grid[0];
+        // results last, as every launch has them
+        for (size_t a = 0; a + 1 < L.args.size(); ++a) F.args.push_back(L.args[a]);
+        F.algo_bytes += L.algo_bytes;
+        F.desc += (f ? " | " : "") + L.desc;
+      }
+      o << "}\n\n";
+      // the kernel's parameters are in the maps' order (inputs and result of each map together); the launch's argument
+      // list must follow that order too, so it is rebuilt here and all results count as outputs only for the liveness
+      F.args.clear();
+      for (auto& L : front) for (int a : L.args) F.args.push_back(a);
+      const std::string base = finalize(o.str());
+      F.kernel = named("@K@_maps", base);
+      F.kind = "map";
+      F.grid[0] = first;
+      F.block[0] = kBlock;
+      F.n_outputs = 1;
+      front.assign(1, F);
+    }
+    plan.launches = front;
+    plan.launches.insert(plan.launches.end(), rest.begin(), rest.end());
+  }
+
   // ------------------------------------------------------------------ buffers
   int buffer_for(int node) {
     if (buf_of[node] >= 0) return buf_of[node];
@@ -4846,6 +4951,7 @@ struct Planner {
       plan.buffers[b].is_result = true;
       plan.result_buffers.push_back(b);
     }
+    merge_parameter_maps();
     // liveness over the launch list
     for (size_t li = 0; li < plan.launches.size(); ++li) {
       auto& L = plan.launches[li];

@@ -303,8 +303,9 @@ def test_windowed_ops_plan(monkeypatch):
     # second one's zero-padded operand and no map runs between them; the switch, and a first convolution whose kernel
     # does not hold the ops between them (then the module is planned again without it), leave the maps in
     text = NN.conv_chain(32, 256, 56, 2, "bf16")[0]
-    chained = ["map_transposed", "map", "conv_bf16", "map", "conv_bf16", "map_transposed"]
-    unchained = ["map_transposed", "map", "conv_bf16", "map", "map", "conv_bf16", "map_transposed"]
+    # (the two filters' layout maps read arguments only: they run first, as one launch)
+    chained = ["map", "map_transposed", "conv_bf16", "conv_bf16", "map_transposed"]
+    unchained = ["map", "map_transposed", "conv_bf16", "map", "conv_bf16", "map_transposed"]
     rep = rx.compile_offline(text, with_source=True)
     assert kinds(rep) == chained and "zero_" in rep, rep
     monkeypatch.setenv("RX_CHAIN_CONVS", "0")
@@ -344,6 +345,12 @@ def test_vgg11_forward_pass_plans(monkeypatch):
     assert "static constexpr bool masks_rows = true;" in rep and "rx_keep_value(res);" in rep and "rx_load_const(in0, " in rep
     i = rep.index("// reduce (generic): window over dims -> tensor<32x56x56x128xbf16>")
     assert "threadIdx.x) * 8;" in rep[i:i + 400]
+    # the conversions of the first images and filter and the seven filter layout maps read arguments only: one launch, first
+    assert kinds[0] == "map" and "rx_mod_k31_maps kind=map grid=9211x1x1" in rep and rep.count("_map_part(blockIdx.x - ") == 9, kinds
+    assert len(kinds) == 27
+    monkeypatch.setenv("RX_MERGE_MAPS", "0")
+    assert len(parse(rx.compile_offline(text))) == 35
+    monkeypatch.delenv("RX_MERGE_MAPS")
     monkeypatch.setenv("RX_NHWC_POOLS", "0")
     off = parse(rx.compile_offline(text))
     assert [k for k, _ in off].count("map_transposed") == 4 and sum("transpose window" in d for _, d in off) == 4, off
