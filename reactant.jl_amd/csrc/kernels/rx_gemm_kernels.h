@@ -1668,19 +1668,30 @@ RX_DEV void rx_conv_body(const float* __restrict__ x, const float* __restrict__ 
 #pragma unroll
     for (int pb = 0; pb < NPB; ++pb) {
       const int p = pb * 16 + 4 * kk;
+      // (a functor that declares masks_rows takes the test as its last argument and guards its store with it: its
+      // arithmetic is then straight-line code over all the blocks of the lane, whose feature is the same in all of them)
       if constexpr (WO % 4 == 0) {
         // whole vectors: a row of the result and the rows left in the image are multiples of 4 words
-        if (p < NPX && y0 * WO + p < HO * WO) {
+        const bool inside = p < NPX && y0 * WO + p < HO * WO;
+        if constexpr (rx_epi_masks_rows<Epi>::value) {
+          const float v[4] = {acc[pb][0], acc[pb][1], acc[pb][2], acc[pb][3]};
+          epi(v, b, o, y0 + p / WO, p % WO, inside);
+        } else if (inside) {
           const float v[4] = {acc[pb][0], acc[pb][1], acc[pb][2], acc[pb][3]};
           epi(v, b, o, y0 + p / WO, p % WO);
         }
       } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (p + r < NPX && y0 * WO + p + r < HO * WO) {
+        for (int r = 0; r < 4; ++r) {
+          const bool inside = p + r < NPX && y0 * WO + p + r < HO * WO;
+          if constexpr (rx_epi_masks_rows<Epi>::value) {
+            const float v[1] = {acc[pb][r]};
+            epi(v, b, o, y0 + (p + r) / WO, (p + r) % WO, inside);
+          } else if (inside) {
             const float v[1] = {acc[pb][r]};
             epi(v, b, o, y0 + (p + r) / WO, (p + r) % WO);
           }
+        }
       }
     }
   }

@@ -3252,7 +3252,7 @@ struct Planner {
     em.indent = 6;
     em.bound[conv] = "accv";
     em.columns_reused = shifted;
-    em.const_vectors = shifted;
+    em.const_vectors = true;
     const std::string val = root == conv ? std::string("accv") : em.emit(root, root_index(rn.ty.dims));
     const std::string ebody = em.take_code();
     const std::string ost = info(rn.ty.dt).stype;
@@ -3264,6 +3264,19 @@ struct Planner {
     for (int i : em.inputs) vectors_only = vectors_only && g.nodes[i].ty.rank() <= 1;
     for (auto& l : em.loads) vectors_only = vectors_only && (g.nodes[l.node].ty.rank() == 0 || l.minor_follows);   // read at the column only: in range on every row
     const bool late_mask = vectors_only && cn.a3.size() == 5;
+    // The direct kernel: a lane holds one feature for all its pixels.  An epilogue that reads nothing but per-feature
+    // vectors (broadcast along the result's feature dimension) takes the kernel's bounds test as an argument and guards
+    // its store with it, for the same reason.
+    bool direct_mask = !shifted && !em.inputs.empty() && n == 4;
+    for (int i : em.inputs) {
+      const Node& in = g.nodes[i];
+      direct_mask = direct_mask && in.ty.rank() <= 1;
+      if (in.ty.rank() == 1)
+        for (int u : users[i]) {
+          const Node& un = g.nodes[u];
+          direct_mask = direct_mask && un.k == OpK::BroadcastInDim && un.ty.rank() == 4 && un.a0 == std::vector<int64_t>{1} && in.ty.dims[0] == rn.ty.dims[1];
+        }
+    }
     // (the grid form computes every row anyway and guards its stores by the row number: it takes the rows past the last one too)
     const bool grid_all_rows = vectors_only && cn.a3.size() == 8;
     std::ostringstream o;
@@ -3272,7 +3285,7 @@ struct Planner {
     for (size_t k = 0; k < em.inputs.size(); ++k)
       o << "  const " << info(g.nodes[em.inputs[k]].ty.dt).stype << "* __restrict__ in" << k << ";\n";
     o << "  " << ost << "* __restrict__ out0;\n";
-    if (late_mask || grid_all_rows) o << "  static constexpr bool masks_rows = true;\n";
+    if (late_mask || grid_all_rows || direct_mask) o << "  static constexpr bool masks_rows = true;\n";
     o << "  template <int NV>\n  __device__ __forceinline__ void operator()(const float (&acc)[NV]";
     if (shifted) {
       // called with (row of the product, first column): the row is a position of the padded grid, of which the
@@ -3290,6 +3303,7 @@ struct Planner {
       }
     } else {
       for (int k = 0; k < n; ++k) o << ", " << it << " i" << k << (k == n - 1 ? "b" : "");
+      if (direct_mask) o << ", const bool keep_";
       o << ") const {\n";
     }
     {
@@ -3319,8 +3333,8 @@ struct Planner {
       o << "    if (row_ + " << cn.a3[7] << " < " << rows << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0 + " << cn.a3[7] * ncol << ") = res;\n";
       if (cn.a3[7] > 0) o << "    if (row_ < " << cn.a3[7] << ") *reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = zero_;\n";
     } else {
-      if (late_mask) o << "    rx_keep_value(res);\n";
-      o << "    " << (late_mask ? "if (keep_) " : "") << "*reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
+      if (late_mask || direct_mask) o << "    rx_keep_value(res);\n";
+      o << "    " << (late_mask || direct_mask ? "if (keep_) " : "") << "*reinterpret_cast<rx_vec<" << ost << ", NV>*>(out0 + lin0) = res;\n";
     }
     o << "  }\n};\n\n";
     if (shifted) {
