@@ -98,6 +98,7 @@ class Emitter {
   void push_scope() { scopes_.emplace_back(); }
   void pop_scope() { scopes_.pop_back(); }
   std::string linear(const Index& ix, const std::vector<int64_t>& dims) const;
+  bool minor_uniform(int node, int depth = 0) const;   // the value does not vary along the node's last dimension
 
  private:
   const Graph& g_;
@@ -113,7 +114,6 @@ class Emitter {
   bool allow_direct_ = false;
 
   bool is_uniform(int node, int depth = 0) const;
-  bool minor_uniform(int node, int depth = 0) const;
   bool minor_only(int node, int depth = 0) const;   // the value varies along the minor dimension at most
   std::string emit_load(int node, const Index& ix);
   std::string emit_op(const Node& n, const Index& ix);

@@ -3649,11 +3649,45 @@ struct Planner {
       const bool long_enough = esz == 2 ? short_ok : red_len >= 16;
       if (inn.ty.dims[kept.back()] % v == 0 && nout / v >= 64 && long_enough) VEC = v;
     }
-    const int64_t nthr = nout / VEC;
+    // A kept minor dimension that one vector covers (the few rows of a skinny matrix product, written as a reduction
+    // over k of x[b][k] * w[k][n] with the result as [n][b]): a thread then takes RB consecutive values of the
+    // next kept dimension as well, an RB x VEC block of the result.  What varies along that dimension only (w) is then
+    // read RB elements at a time, one 16-byte load instead of four 4-byte ones, and what does not (x) once for the block.
+    int RB = 1, wnode = -1;
+    Emitter emr(g, [&](int x) { return mat[x]; });
+    std::string wbody, wval;
+    if (opt.reduce_row_blocks && VEC > 1 && esz == 4 && kept.size() >= 2 && red.size() == 1 && inn.ty.dims[kept.back()] == VEC &&
+        inn.ty.dims[kept[kept.size() - 2]] % 4 == 0 && red_len >= 256 && nout / VEC / 4 >= 256 && !mat[rn.in[0]] && inn.k == OpK::Binary && inn.op == "multiply") {
+      for (int side = 0; side < 2; ++side)
+        if (em.minor_uniform(inn.in[side]) && !em.minor_uniform(inn.in[1 - side]) && g.nodes[inn.in[side]].ty.dims == inn.ty.dims) wnode = inn.in[side];
+      if (wnode >= 0) {
+        // the kernel's text again, in two parts: the operand that the block shares (for eight reduction steps ahead of
+        // the arithmetic, so that eight 16-byte loads are in flight), then the rest with that operand's value in scope
+        RB = 4;
+        emr.excess_precision = opt.excess_precision;
+        emr.idx64 = em.idx64;
+        emr.set_root({}, {}, false);
+        emr.indent = 8;
+        emr.push_scope();
+        wval = emr.emit(wnode, ix);
+        wbody = emr.take_code();
+        emr.pop_scope();
+        emr.bound[wnode] = "wq_";
+        emr.indent = 10;
+        val = emr.emit(rn.in[0], ix);
+        body = emr.take_code();
+        emr.indent = 2;
+        initv = emr.emit(rn.in[1], Index{});
+        ibody = emr.take_code();
+      }
+    }
+    Emitter& eu = RB > 1 ? emr : em;     // the emitter whose inputs the kernel takes
+    const int64_t nthr = nout / VEC / RB;
     int64_t split = 1;
     if (!red.empty() && nout > 0 && nthr <= 32 * 1024 && red_len >= 64) {
       const int64_t ds = inn.ty.dims[red[ks]];
-      split = std::min<int64_t>({ds, (512 * 1024 + nthr - 1) / nthr, 1024, std::max<int64_t>(1, red_len / 16)});
+      // (threads of a block carry many times the bytes in flight: a quarter of the threads suffices, and the partials stay small; twice the threads, or sixteen steps per block, measured slower)
+      split = std::min<int64_t>({ds, ((RB > 1 ? 128 : 512) * 1024 + nthr - 1) / nthr, 1024, std::max<int64_t>(1, red_len / 16)});
     }
     const bool two_pass = split >= 2;
     const int64_t chunk = two_pass ? (inn.ty.dims[red[ks]] + split - 1) / split : 0;
@@ -3661,21 +3695,49 @@ struct Planner {
     std::ostringstream o;
     o << "// reduce (generic" << (two_pass ? ", reduced dimension cut into " + std::to_string(split) + " chunks" : std::string()) << "): " << describe(rn.in[0])
       << " over dims -> " << rn.ty.str() << "\n";
-    o << signature(kname, em.inputs, {{two_pass ? ACC : std::string(info(dt).stype), two_pass ? "partial" : "out0"}}) << " {\n";
-    if (VEC > 1) o << "  const " << it << " oid = ((" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x) * " << VEC << ";\n";
+    o << signature(kname, eu.inputs, {{two_pass ? ACC : std::string(info(dt).stype), two_pass ? "partial" : "out0"}}) << " {\n";
+    if (VEC > 1) o << "  const " << it << " oid = ((" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x) * " << VEC * RB << ";\n";
     else o << "  const " << it << " oid = (" << it << ")blockIdx.x * " << kBlock << " + threadIdx.x;\n";
     o << "  if (oid >= " << nout << ") return;\n";
     o << "  " << it << " rr = oid;\n";
     for (int k = (int)kept.size() - 1; k >= 0; --k) {
-      o << "  const " << it << " o" << k << (VEC > 1 && k == (int)kept.size() - 1 ? "b" : "") << " = rr % " << inn.ty.dims[kept[k]] << ";\n";
+      o << "  const " << it << " o" << k << ((VEC > 1 && k == (int)kept.size() - 1) || (RB > 1 && k == (int)kept.size() - 2) ? "b" : "") << " = rr % " << inn.ty.dims[kept[k]] << ";\n";
       o << "  rr /= " << inn.ty.dims[kept[k]] << ";\n";
     }
     if (VEC > 1) {
-      o << "  " << ACC << " accv[" << VEC << "];\n#pragma unroll\n  for (int l = 0; l < " << VEC << "; ++l) accv[l] = " << red_identity(rn.red, dt) << ";\n";
+      o << "  " << ACC << " accv[" << VEC * RB << "];\n#pragma unroll\n  for (int l = 0; l < " << VEC * RB << "; ++l) accv[l] = " << red_identity(rn.red, dt) << ";\n";
     } else {
       o << "  " << ACC << " acc = " << red_identity(rn.red, dt) << ";\n";
     }
-    for (size_t k = 0; k < red.size(); ++k) {
+    if (RB > 1) {
+      // one reduced dimension: blocks of eight steps, the shared operand's values of a block first
+      const std::string wct = info(g.nodes[wnode].ty.dt).ctype;
+      const std::string ok2 = "o" + std::to_string(kept.size() - 2), ok1 = "o" + std::to_string(kept.size() - 1);
+      if (two_pass) {
+        o << "  const " << it << " r0_end = rx_min<" << it << ">(((" << it << ")blockIdx.y + 1) * " << chunk << ", " << inn.ty.dims[red[0]] << ");\n";
+        o << "  " << it << " r0s = (" << it << ")blockIdx.y * " << chunk << ";\n";
+      } else {
+        o << "  const " << it << " r0_end = " << inn.ty.dims[red[0]] << ";\n  " << it << " r0s = 0;\n";
+      }
+      auto steps = [&](int U) {
+        o << "    " << wct << " wq[" << U * RB << "];\n";
+        o << "#pragma unroll\n    for (int u = 0; u < " << U << "; ++u) {\n      const " << it << " r0 = r0s + u;\n";
+        o << "#pragma unroll\n      for (int j = 0; j < " << RB << "; ++j) {\n        const " << it << " " << ok2 << " = " << ok2 << "b + j, " << ok1 << " = " << ok1 << "b;\n";
+        o << wbody << "        wq[u * " << RB << " + j] = " << wval << ";\n      }\n    }\n";
+        o << "#pragma unroll\n    for (int u = 0; u < " << U << "; ++u) {\n      const " << it << " r0 = r0s + u;\n";
+        o << "#pragma unroll\n      for (int j = 0; j < " << RB << "; ++j) {\n        const " << it << " " << ok2 << " = " << ok2 << "b + j;\n        const " << wct << " wq_ = wq[u * " << RB << " + j];\n";
+        o << "#pragma unroll\n        for (int l = 0; l < " << VEC << "; ++l) {\n          const " << it << " " << ok1 << " = " << ok1 << "b + l;\n";
+        o << body;
+        const std::string slot = "accv[j * " + std::to_string(VEC) + " + l]";
+        o << "          " << slot << " = " << red_apply(rn.red, dt, slot, "(" + ACC + ")" + val) << ";\n        }\n      }\n    }\n";
+      };
+      o << "  for (; r0s + 8 <= r0_end; r0s += 8) {\n";
+      steps(8);
+      o << "  }\n  for (; r0s < r0_end; ++r0s) {\n";
+      steps(1);
+      o << "  }\n";
+    }
+    for (size_t k = 0; k < red.size() && RB == 1; ++k) {
       const std::string pad(2 + 2 * k, ' ');
       const std::string unroll = VEC > 1 && k + 1 == red.size() ? "#pragma unroll 8\n" : "";
       if (two_pass && k == ks) {
@@ -3685,7 +3747,8 @@ struct Planner {
         o << unroll << pad << "for (" << it << " r" << k << " = 0; r" << k << " < " << inn.ty.dims[red[k]] << "; ++r" << k << ") {\n";
       }
     }
-    if (VEC > 1) {
+    if (RB > 1) {
+    } else if (VEC > 1) {
       const std::string pad(2 + 2 * red.size(), ' ');
       o << "#pragma unroll\n" << pad << "for (int l = 0; l < " << VEC << "; ++l) {\n";
       o << pad << "  const " << it << " o" << kept.size() - 1 << " = o" << kept.size() - 1 << "b + l;\n";
@@ -3696,14 +3759,14 @@ struct Planner {
       o << body;
       o << std::string(4 + 2 * red.size(), ' ') << "acc = " << red_apply(rn.red, dt, "acc", "(" + ACC + ")" + val) << ";\n";
     }
-    for (int k = (int)red.size() - 1; k >= 0; --k) o << std::string(2 + 2 * k, ' ') << "}\n";
+    for (int k = (int)red.size() - 1; k >= 0 && RB == 1; --k) o << std::string(2 + 2 * k, ' ') << "}\n";
     std::string rv = is_narrow_float(dt) ? Emitter::round_narrow(dt, "r") : std::string("(") + info(dt).ctype + ")r";
     std::vector<int> fin_inputs;
     int comb_lanes = 1;      // wavefronts of the combine kernel that share an output
     if (!two_pass) {
       o << ibody;
       if (VEC > 1) {
-        o << "#pragma unroll\n  for (int l = 0; l < " << VEC << "; ++l) {\n";
+        o << "#pragma unroll\n  for (int l = 0; l < " << VEC * RB << "; ++l) {\n";
         o << "    const " << ACC << " r = " << red_apply(rn.red, dt, "accv[l]", "(" + ACC + ")" + initv) << ";\n";
         o << "    out0[oid + l] = " << Emitter::store_conv(dt, rv) << ";\n  }\n}\n\n";
       } else {
@@ -3711,7 +3774,7 @@ struct Planner {
         o << "  out0[oid] = " << Emitter::store_conv(dt, rv) << ";\n}\n\n";
       }
     } else {
-      if (VEC > 1) o << "#pragma unroll\n  for (int l = 0; l < " << VEC << "; ++l) partial[(" << it << ")blockIdx.y * " << nout << " + oid + l] = accv[l];\n}\n\n";
+      if (VEC > 1) o << "#pragma unroll\n  for (int l = 0; l < " << VEC * RB << "; ++l) partial[(" << it << ")blockIdx.y * " << nout << " + oid + l] = accv[l];\n}\n\n";
       else o << "  partial[(" << it << ")blockIdx.y * " << nout << " + oid] = acc;\n}\n\n";
       // the init value may read buffers of its own: evaluate it with a fresh numbering
       Emitter e3(g, [&](int x) { return mat[x]; });
@@ -3756,8 +3819,8 @@ struct Planner {
     L.grid[0] = (unsigned)((nthr + kBlock - 1) / kBlock);
     L.grid[1] = (unsigned)(two_pass ? split : 1);
     L.block[0] = kBlock;
-    for (int i : em.inputs) L.args.push_back(buffer_for(i));
-    L.algo_bytes = algo_bytes(em.inputs, {root});
+    for (int i : eu.inputs) L.args.push_back(buffer_for(i));
+    L.algo_bytes = algo_bytes(eu.inputs, {root});
     L.desc = describe(rn.in[0]) + " reduce";
     if (!two_pass) {
       L.args.push_back(buffer_for(root));

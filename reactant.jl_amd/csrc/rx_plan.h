@@ -72,6 +72,7 @@ struct PlanOptions {
   bool single_pass_reduce = false;
   bool single_pass_scan = true;      // long scanned rows in one launch (chunk totals travel as flagged words)
   bool window_reduce_vectors = true;  // reductions over 16-bit elements that keep the minor dimension (pooling windows): eight outputs per thread
+  bool reduce_row_blocks = true;   // reductions whose kept minor dimension is one vector long (skinny matrix products): a thread takes four values of the next kept dimension too
   bool lds_transpose = true;       // maps with transposed reads: stage 64x64 tiles through LDS
   bool branchless_guards = true;   // stencil kernels: evaluate pad/update guards as selects when every guarded read is a tile read
   bool clamp_pad_reads = true;     // maps over 8- and 16-bit elements: padded reads at clamped positions and a select, so that a lane's loads combine

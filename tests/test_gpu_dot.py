@@ -219,6 +219,9 @@ VECTOR_CASES = [
     ((200, 6, 300), (300, 6), (6, 200), "batching_dims = [1] x [1], contracting_dims = [2] x [0]", "f32", None),
     ((300, 700), (700,), (300,), "contracting_dims = [1] x [0]", "i32", ["row"]),
     ((300, 700), (700,), (300,), "contracting_dims = [1] x [0]", "f8E4M3FN", None),
+    # four rows times a wide matrix (a dense layer on a batch of four): 4 x 4 blocks of the result per thread
+    ((4, 1003), (1003, 2048), (4, 2048), "contracting_dims = [1] x [0]", "f32", ["reduce_generic"]),
+    ((4, 4100), (4100, 1024), (4, 1024), "contracting_dims = [1] x [0]", "i32", ["reduce_generic"]),
 ]
 
 
@@ -251,6 +254,14 @@ def test_dot_general_with_a_vector_like_operand(rx, client, ls, rs, os_, attrs, 
         assert err <= 1e-12
     else:
         assert err <= 1e-5 * np.sqrt(100003 if not os_ else 1000)
+
+
+def test_four_rows_times_a_wide_matrix_plan():
+    """x[4][k] w[k][n] as a reduction over k with the result as [n][4]: a thread owns four n and the four rows, and reads
+    w sixteen bytes at a time for eight k ahead of the arithmetic (RX_REDUCE_ROW_BLOCKS=0: one n per thread)."""
+    from _loader import load_pkg
+    rep = load_pkg().compile_offline(_dot_text([4, 1003], [1003, 2048], [4, 2048], "contracting_dims = [1] x [0]", "f32"), with_source=True)
+    assert "threadIdx.x) * 16;" in rep and "float wq[32];" in rep and "for (; r0s + 8 <= r0_end; r0s += 8)" in rep, rep
 
 
 def test_short_contractions_keep_the_scalar_loop(rx, client):
