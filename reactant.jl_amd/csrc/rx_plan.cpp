@@ -1142,6 +1142,7 @@ struct Planner {
       picked.push_back(li);
     }
     if (picked.size() < 2) return;
+    if (picked.size() > 64) picked.resize(64);   // the merged kernel takes every map's pointers as parameters
     std::vector<Launch> front, rest;
     for (size_t li = 0, q = 0; li < plan.launches.size(); ++li) {
       if (q < picked.size() && picked[q] == li) { front.push_back(plan.launches[li]); ++q; }
