@@ -121,6 +121,7 @@ struct Planner {
   std::vector<std::set<Ctx>> ctx;
   std::vector<char> prev_mat;       // materialization decided by the previous analysis sweep (used for producers)
   std::vector<char> force_mat;      // chosen cut points below a dot_general with several consumers
+  std::set<int> layout_entries;     // transposes that bring a tensor into a channel-minor region: written by a transposing map, not read across the layout by their readers
   std::vector<int> buf_of;          // node -> buffer id (materialized nodes)
   std::map<int, int> fuse_prev;     // stencil root -> the stencil step it evaluates in LDS instead of reading from memory
   std::set<int> lds_only;           // the steps absorbed that way: no launch, no buffer
@@ -182,6 +183,190 @@ struct Planner {
     split_dots();
     pools_between_convs();
     chain_convs();
+    channel_minor_regions();
+  }
+
+  // What pools_between_convs does for a chain, for a region: a connected set of values between products with row
+  // shifts in which every op can run on either layout -- elementwise ops on tensors of one shape (residual additions
+  // among them) whose other operands vary along the channels only, padding with a scalar, pooling windows -- with any
+  // number of readers.  The region is rebuilt on [image, row, column, channel]; the transposes after the products
+  // that feed it and before the products that read it disappear, a tensor that enters it from elsewhere is transposed
+  // once on the way in, and a value that something outside reads (a reduction over the pixels, the module's result) is
+  // transposed once on the way out.  Done when the transposes that disappear move at least twice the bytes of those
+  // that are added.
+  void channel_minor_regions() {
+    if (!opt.nhwc_regions || !opt.nhwc_pools || !opt.mfma) return;
+    const int N = (int)g.nodes.size();
+    std::vector<std::vector<int>> use(N);
+    std::vector<char> is_res(N, 0);
+    for (auto& n : g.nodes) for (int i : n.in) use[i].push_back(n.id);
+    for (int r : g.results) is_res[r] = 1;
+    auto elementwise = [](OpK k) { return k == OpK::Unary || k == OpK::Binary || k == OpK::Clamp || k == OpK::Gelu || k == OpK::Convert || k == OpK::Select || k == OpK::Compare; };
+    std::vector<signed char> vec_memo(N, -1);
+    std::function<bool(int, int)> channel_only = [&](int x, int depth) -> bool {
+      if (vec_memo[x] >= 0) return vec_memo[x] != 0;
+      const Node& n = g.nodes[x];
+      bool ok = false;
+      if (n.k == OpK::Constant) ok = n.splat;
+      else if (n.k == OpK::BroadcastInDim) {
+        const TType& st = g.nodes[n.in[0]].ty;
+        ok = n.ty.rank() == 4 && (st.rank() == 0 || (st.rank() == 1 && n.a0.size() == 1 && n.a0[0] == 1 && st.dims[0] == n.ty.dims[1]));
+      } else if (elementwise(n.k) && depth < 12) {
+        ok = !n.in.empty();
+        for (int i : n.in) ok = ok && channel_only(i, depth + 1);
+      }
+      vec_memo[x] = ok ? 1 : 0;
+      return ok;
+    };
+    auto shifted_conv = [&](int x) { return g.nodes[x].k == OpK::Conv && !g.nodes[x].a3.empty(); };
+    enum Role : char { None = 0, T1, Elem, PadOp, Win, Red, T2 };
+    std::vector<char> role(N, None);
+    for (const Node& n : g.nodes) {
+      if (n.k == OpK::Transpose && n.ty.rank() == 4) {
+        if (n.a0 == std::vector<int64_t>{0, 3, 1, 2} && g.nodes[n.in[0]].k == OpK::Conv && g.nodes[n.in[0]].a3.size() == 5 && use[n.in[0]].size() == 1 && !is_res[n.in[0]])
+          role[n.id] = T1;
+        else if (n.a0 == std::vector<int64_t>{0, 2, 3, 1} && !is_res[n.id] && !use[n.id].empty()) {
+          bool all = true;
+          for (int u : use[n.id]) all = all && shifted_conv(u) && g.nodes[u].in[0] == n.id && g.nodes[u].in[1] != n.id;
+          if (all) role[n.id] = T2;
+        }
+      } else if (n.ty.rank() == 4 && elementwise(n.k) && n.k != OpK::Compare && n.k != OpK::Select && !channel_only(n.id, 0)) {
+        bool ok = !n.in.empty();
+        for (int i : n.in) ok = ok && (channel_only(i, 0) || (g.nodes[i].ty.rank() == 4 && g.nodes[i].ty.dims == n.ty.dims));
+        if (ok) role[n.id] = Elem;
+      } else if (n.k == OpK::Pad && n.ty.rank() == 4 && g.nodes[n.in[1]].ty.rank() == 0 && n.in[0] != n.in[1] && !channel_only(n.in[0], 0)) {
+        role[n.id] = PadOp;
+      } else if (n.k == OpK::Window && g.nodes[n.in[0]].ty.rank() == 4 && use[n.id].size() == 1 && !is_res[n.id]) {
+        const Node& r = g.nodes[use[n.id][0]];
+        if (r.k == OpK::Reduce && r.in[0] == n.id && r.a0 == std::vector<int64_t>{0, 1, 2, 3} && g.nodes[r.in[1]].ty.rank() == 0) { role[n.id] = Win; role[r.id] = Red; }
+      }
+    }
+    // the tensor operands of a member
+    auto tensor_ins = [&](const Node& n) {
+      std::vector<int> t;
+      if (role[n.id] == Elem) { for (int i : n.in) if (!channel_only(i, 0)) t.push_back(i); }
+      else if (role[n.id] == PadOp || role[n.id] == Win || role[n.id] == Red || role[n.id] == T2) t.push_back(n.in[0]);
+      return t;
+    };
+    // components over tensor edges between members
+    std::vector<int> comp(N);
+    for (int i = 0; i < N; ++i) comp[i] = i;
+    std::function<int(int)> find = [&](int x) { while (comp[x] != x) x = comp[x] = comp[comp[x]]; return x; };
+    for (const Node& n : g.nodes) {
+      if (role[n.id] == None) continue;
+      for (int i : tensor_ins(n)) if (role[i] != None && role[i] != T2) comp[find(n.id)] = find(i);
+    }
+    struct Tally { double saved = 0, added = 0; int t1 = 0, t2 = 0; std::set<int> entries, exits; };
+    std::map<int, Tally> tally;
+    for (const Node& n : g.nodes) {
+      if (role[n.id] == None) continue;
+      Tally& t = tally[find(n.id)];
+      if (role[n.id] == T1) { t.saved += (double)n.ty.bytes(); ++t.t1; }
+      if (role[n.id] == T2) { t.saved += (double)n.ty.bytes(); ++t.t2; }
+      for (int i : tensor_ins(n))
+        if (role[i] == None || role[i] == T2) { if (t.entries.insert(i).second) t.added += (double)g.nodes[i].ty.bytes(); }
+      if (role[n.id] == T2 || role[n.id] == Win) continue;      // read by the products / by its reduction only
+      bool outside = is_res[n.id];
+      for (int u : use[n.id]) {
+        bool inside = role[u] != None && role[u] != T1;
+        if (inside) { bool reads = false; for (int i : tensor_ins(g.nodes[u])) reads = reads || i == n.id; inside = reads; }
+        outside = outside || !inside;
+      }
+      if (outside && t.exits.insert(n.id).second) t.added += (double)n.ty.bytes();
+    }
+    std::set<int> chosen;
+    for (auto& kv : tally)
+      if (kv.second.t1 >= 1 && kv.second.t2 >= 1 && kv.second.saved >= 2.0 * kv.second.added) chosen.insert(kv.first);
+    if (chosen.empty()) return;
+    auto member = [&](int x) { return role[x] != None && chosen.count(find(x)) > 0; };
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(N, -1), nhwc(N, -1);
+    static const int P[4] = {0, 3, 1, 2};      // old dimension i is new dimension P[i]
+    auto permuted = [&](const std::vector<int64_t>& v) { std::vector<int64_t> r(4); for (int i = 0; i < 4; ++i) r[P[i]] = v[i]; return r; };
+    std::map<std::pair<int, std::vector<int64_t>>, int> memo;
+    std::function<int(int, const std::vector<int64_t>&)> rebuild_vec = [&](int x, const std::vector<int64_t>& dims) -> int {
+      auto it = memo.find({x, dims});
+      if (it != memo.end()) return it->second;
+      Node c = g.nodes[x];
+      c.ty.dims = dims;
+      if (c.k == OpK::BroadcastInDim) {
+        c.in = {remap[c.in[0]]};
+        if (!c.a0.empty()) c.a0 = {3};
+      } else if (c.k != OpK::Constant) {
+        for (int& i : c.in) i = rebuild_vec(i, dims);
+      }
+      return memo[{x, dims}] = out.add(c);
+    };
+    // the value of old node x in the old layout (members of a chosen region exist in the new layout only)
+    std::function<int(int)> old_layout = [&](int x) -> int {
+      if (remap[x] >= 0) return remap[x];
+      Node t;
+      t.k = OpK::Transpose;
+      t.in = {nhwc[x]};
+      t.a0 = {0, 3, 1, 2};
+      t.ty = g.nodes[x].ty;
+      return remap[x] = out.add(t);
+    };
+    std::function<int(int)> new_layout = [&](int x) -> int {
+      if (nhwc[x] >= 0) return nhwc[x];
+      Node t;
+      t.k = OpK::Transpose;
+      t.in = {old_layout(x)};
+      t.a0 = {0, 2, 3, 1};
+      t.ty.dt = g.nodes[x].ty.dt;
+      t.ty.dims = permuted(g.nodes[x].ty.dims);
+      nhwc[x] = out.add(t);
+      layout_entries.insert(nhwc[x]);
+      return nhwc[x];
+    };
+    layout_entries.clear();
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      if (!member(n.id)) {
+        for (int& i : c.in) i = old_layout(i);
+        remap[n.id] = out.add(c);
+        continue;
+      }
+      switch (role[n.id]) {
+        case T1:
+          nhwc[n.id] = old_layout(n.in[0]);      // the product's own result
+          continue;
+        case T2:
+          remap[n.id] = new_layout(n.in[0]);     // what the products read
+          continue;
+        case Elem:
+          c.ty.dims = permuted(n.ty.dims);
+          for (int& i : c.in) i = channel_only(i, 0) ? rebuild_vec(i, c.ty.dims) : new_layout(i);
+          break;
+        case PadOp:
+          c.ty.dims = permuted(n.ty.dims);
+          c.a0 = permuted(n.a0); c.a1 = permuted(n.a1); c.a2 = permuted(n.a2);
+          c.in = {new_layout(n.in[0]), old_layout(n.in[1])};
+          break;
+        case Win: {
+          c.a0 = permuted(n.a0); c.a1 = permuted(n.a1); c.a2 = permuted(n.a2);
+          const std::vector<int64_t> k = permuted(std::vector<int64_t>(n.ty.dims.begin(), n.ty.dims.begin() + 4));
+          const std::vector<int64_t> o = permuted(std::vector<int64_t>(n.ty.dims.begin() + 4, n.ty.dims.end()));
+          c.ty.dims = k;
+          c.ty.dims.insert(c.ty.dims.end(), o.begin(), o.end());
+          c.in = {new_layout(n.in[0])};
+          break;
+        }
+        case Red:
+          c.ty.dims = permuted(n.ty.dims);
+          c.in = {nhwc[n.in[0]], old_layout(n.in[1])};
+          break;
+        default:
+          break;
+      }
+      nhwc[n.id] = out.add(c);
+    }
+    for (int p : g.params) out.params.push_back(old_layout(p));
+    for (int r : g.results) out.results.push_back(old_layout(r));
+    g = std::move(out);
   }
 
   // Between two convolutions in the product-with-row-shifts form the values live as [image, row, column, channel]: the
@@ -1011,6 +1196,8 @@ struct Planner {
     // bias, activation) end where something reads their value at other positions (a pooling window, a layout change):
     // the value is written there, so that the chain runs once per element in the convolution's kernel, in the
     // type it ends in, instead of once per read in the reader's.
+    for (int x : layout_entries)
+      if (x < N && live[x] && !users[x].empty()) force_mat[x] = 1;
     if (opt.product_epilogues && opt.conv_tails) {
       auto pointwise = [](OpK k) { return k == OpK::Unary || k == OpK::Binary || k == OpK::Clamp || k == OpK::Convert || k == OpK::Select || k == OpK::Gelu; };
       for (int c = 0; c < N; ++c) {

@@ -59,6 +59,7 @@ struct PlanOptions {
   int conv_tails = 1;           // the elementwise chain after a convolution is written where a window, reduction or layout change reads it, so that it runs in the convolution's kernel: 1 when it ends in a type narrower than the f32 accumulators, 2 always, 0 never
   bool nhwc_pools = true;       // pooling windows (and the elementwise ops and padding around them) between two 16-bit convolutions run on the channel-minor layout: no transposes
   bool merge_parameter_maps = true;  // plain maps that read only the module's arguments run first, several of them as one launch
+  bool nhwc_regions = true;     // the same for regions with several readers per value (residual additions): transposed once on the way in and out where needed
   bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles

@@ -295,6 +295,38 @@ def vgg11(batch=4, hw=224, classes=1000, dt="f32", layers=VGG11_LAYERS, dense=40
     return text, shapes, flops
 
 
+def resnet_stage(batch=2, channels=64, hw=16, blocks=2, dt="f32"):
+    """`blocks` basic residual blocks on `batch` images of `channels` x hw x hw: 3x3 convolution (padding 1) + batch
+    norm (test mode) + relu + 3x3 convolution + batch norm, the block's input added, relu (the identity blocks of a
+    ResNet stage as Lux / Boltz build them).  Arguments: the images, then per block the two filters, each followed
+    by its batch norm's scale, offset, mean, variance.  Returns (text, shapes, flops)."""
+    T, W, F = tt([batch, channels, hw, hw], dt), tt([channels, channels, 3, 3], dt), tt([channels], dt)
+    conv = ("stablehlo.convolution(%s, %s) dim_numbers = [b, f, 1, 0]x[o, i, 1, 0]->[b, f, 1, 0], window = {stride = [1, 1], "
+            "pad = [[1, 1], [1, 1]], rhs_dilate = [1, 1]} {batch_group_count = 1 : i64, feature_group_count = 1 : i64} : (" + T + ", " + W + ") -> " + T)
+    args, shapes, lines = [T], [[batch, channels, hw, hw]], ["%zero = stablehlo.constant dense<0.000000e+00> : " + T]
+    cur = "%arg0"
+    for b in range(blocks):
+        inp = cur
+        for half in range(2):
+            a = len(args)
+            args += [W, F, F, F, F]
+            shapes += [[channels, channels, 3, 3]] + [[channels]] * 4
+            k = "%d_%d" % (b, half)
+            lines.append("%%c%s = " % k + conv % (cur, "%%arg%d" % a))
+            lines.append("%%n%s = \"stablehlo.batch_norm_inference\"(%%c%s, %%arg%d, %%arg%d, %%arg%d, %%arg%d) <{epsilon = 1.000000e-05 : f32, feature_index = 1 : i64}> : (%s) -> %s"
+                         % (k, k, a + 1, a + 2, a + 3, a + 4, ", ".join([T, F, F, F, F]), T))
+            cur = "%%n%s" % k
+            if half == 0:
+                lines.append("%%r%s = stablehlo.maximum %s, %%zero : %s" % (k, cur, T))
+                cur = "%%r%s" % k
+        lines.append("%%s%d = stablehlo.add %s, %s : %s" % (b, cur, inp, T))
+        lines.append("%%o%d = stablehlo.maximum %%s%d, %%zero : %s" % (b, b, T))
+        cur = "%%o%d" % b
+    sig = ", ".join("%%arg%d: %s" % (k, t) for k, t in enumerate(args))
+    text = "module {\n  func.func @main(%s) -> %s {\n    %s\n    return %s : %s\n  }\n}\n" % (sig, T, "\n    ".join(lines), cur, T)
+    return text, shapes, blocks * 2 * 2.0 * batch * channels * hw * hw * channels * 9
+
+
 def attention_block(batch_heads=6, seq=40, dim=16, dt="f32"):
     """softmax(q k^T / sqrt(d)) v on [batch*heads, seq, dim] operands: the two batched products and the
     row softmax of NNlib.dot_product_attention, which the ViT of benchmark/nn/vision.jl:5-22 runs."""

@@ -468,6 +468,40 @@ def test_vgg11_forward_pass(rx, client, monkeypatch, dt, nhwc):
     _close(got[0].a, ref[0].a, {"f32": 2e-4, "bf16": 5e-2, "f16": 8e-3}[dt])
 
 
+@pytest.mark.parametrize("dt,regions", [("bf16", True), ("bf16", False), ("f16", True), ("f32", True)])
+def test_residual_stage(rx, client, monkeypatch, dt, regions):
+    """Three basic residual blocks (convolution + batch norm + relu + convolution + batch norm, the block's input added,
+    relu).  In 16 bits the products with row shifts keep the values channel-minor through the whole stage: a block is
+    two products -- batch norm + relu, and batch norm + the addition + relu, as their epilogues -- and a padding map; the
+    stage's input is transposed once on the way in, its result once on the way out (RX_NHWC_REGIONS=0: a transposing
+    map on either side of every second product).  Against the oracle."""
+    if not regions:
+        monkeypatch.setenv("RX_NHWC_REGIONS", "0")
+    text, shapes, _ = NN.resnet_stage(batch=3, channels=64, hw=24, blocks=3, dt=dt)
+    rng = np.random.default_rng(31)
+    args = []
+    for k, sh in enumerate(shapes):
+        if len(sh) == 1 and (k - 1) % 5 == 4:
+            args.append(I.tensor(rng.uniform(0.5, 2.0, size=sh), dt))
+        elif len(sh) == 1 and (k - 1) % 5 == 1:
+            args.append(I.tensor(rng.uniform(0.5, 1.0, size=sh), dt))
+        elif len(sh) == 4 and k > 0:
+            args.append(I.tensor(rng.normal(size=sh) * np.sqrt(1.0 / np.prod(sh[1:])), dt))
+        else:
+            args.append(I.tensor(rng.normal(size=sh) * (1.0 if k == 0 else 0.2), dt))
+    got, exe = gpu_run(rx, client, text, args)
+    kinds = [l["kind"] for l in exe.launches()]
+    if dt != "f32":
+        kind = "conv_" + dt
+        assert kinds.count(kind) == 6, kinds
+        if regions:
+            assert kinds == ["map", "map_transposed", kind, "map_transposed", kind, "map", kind, kind, "map", kind, kind, "map_transposed"], kinds
+        else:
+            assert kinds.count("map_transposed") == 6, kinds
+    ref = oracle_run(text, args, hifi=True)
+    _close(got[0].a, ref[0].a, {"f32": 1e-4, "bf16": 3e-2, "f16": 5e-3}[dt])
+
+
 @pytest.mark.parametrize("bh,seq,dim,dt,tol", [(6, 40, 16, "f32", 1e-5), (8, 256, 64, "f32", 1e-4), (8, 256, 64, "bf16", 2e-2)])
 def test_attention_block(rx, client, bh, seq, dim, dt, tol):
     text, shapes = NN.attention_block(bh, seq, dim, dt)

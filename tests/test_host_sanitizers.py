@@ -45,6 +45,7 @@ def corpus():
         "conv_shifted_small": NN.convolution([2, 20, 16, 64], [3, 3, 64, 128], "f16", padding=[[1, 0], [2, 1]], rhs_dil=[1, 2], dims="[b, 0, 1, f]x[0, 1, i, o]->[b, 0, 1, f]")[0],
         "vgg": NN.vgg_block(), "attention": NN.attention_block(),
         "conv_chain": NN.conv_chain(32, 256, 56, 3, "bf16")[0], "vgg11_f32": NN.vgg11(batch=4, dt="f32")[0], "vgg11_bf16": NN.vgg11(batch=32, dt="bf16")[0],
+        "resnet_stage": NN.resnet_stage(batch=32, channels=128, hw=28, blocks=3, dt="bf16")[0], "resnet_stage_f32": NN.resnet_stage(batch=2, channels=64, hw=16, blocks=2, dt="f32")[0],
         "vgg11_small": NN.vgg11(batch=4, hw=64, classes=10, dt="f16", layers=(64, "M", 64, "M", 64, 64, "M", 64, 64, "M", 64, 64, "M"), dense=96)[0],
         "argmax": NN.argreduce([64, 100], "f32", 1),
         "pool_grad": NN.select_and_scatter([2, 4, 16, 16], "f32", [1, 1, 2, 2], strides=[1, 1, 2, 2]),
