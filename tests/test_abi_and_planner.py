@@ -361,6 +361,24 @@ def test_vgg11_forward_pass_plans(monkeypatch):
     monkeypatch.delenv("RX_CONV_TAILS")
 
 
+def test_residual_blocks_plan_channel_minor(monkeypatch):
+    """Three basic residual blocks in bf16: the filters' layout maps as one launch, the first product's padded operand
+    and the block input's layout (two transposing maps), then per block two products (the second one's epilogue adds
+    the block's input) and one padding map; the result is transposed once.  Without the regions: a transposing map
+    after and before every second product."""
+    import _nn_modules as NN
+    kinds = lambda rep: [ln.split("kind=")[1].split()[0] for ln in rep.splitlines() if "kind=" in ln]
+    text = NN.resnet_stage(batch=32, channels=128, hw=28, blocks=3, dt="bf16")[0]
+    c = "conv_bf16"
+    assert kinds(rx.compile_offline(text)) == ["map", "map_transposed", c, "map_transposed", c, "map", c, c, "map", c, c, "map_transposed"]
+    monkeypatch.setenv("RX_NHWC_REGIONS", "0")
+    off = kinds(rx.compile_offline(text))
+    assert off.count(c) == 6 and off.count("map_transposed") == 6, off
+    monkeypatch.delenv("RX_NHWC_REGIONS")
+    # f32 runs on the direct kernel in the module's own layout: nothing to do
+    assert "map_transposed" not in kinds(rx.compile_offline(NN.resnet_stage(batch=4, channels=64, hw=28, blocks=2, dt="f32")[0]))
+
+
 def test_time_loops_over_small_arrays_plan_as_chain_kernels(monkeypatch):
     """The reference's polybench stencils (benchmark/polybench/stencil.jl) at its sizes: 1024 or 256
     trips of a `stablehlo.while` unroll into runs of update steps, which share chain kernels."""
