@@ -3448,9 +3448,18 @@ struct Planner {
     // vectors only (bias, batch norm) the test guards the store alone: the arithmetic is then straight-line code over all
     // the rows a thread handles, and what depends on the column only (the vectors' loads and conversions, a square root,
     // a reciprocal) is computed once per column instead of once per row.
-    bool vectors_only = shifted && !em.inputs.empty();
-    for (int i : em.inputs) vectors_only = vectors_only && g.nodes[i].ty.rank() <= 1;
-    for (auto& l : em.loads) vectors_only = vectors_only && (g.nodes[l.node].ty.rank() == 0 || l.minor_follows);   // read at the column only: in range on every row
+    // (Tensors of the result's own shape that are read at the result's position -- the other operand of a residual
+    // addition -- may take part in the compact form: their vectors are read at a position clamped into the tensor.)
+    bool vectors_only = shifted && !em.inputs.empty(), clamped_reads = false;
+    for (auto& l : em.loads) {
+      const Node& ln = g.nodes[l.node];
+      bool ok = ln.ty.rank() == 0 || (ln.ty.rank() <= 1 && l.minor_follows);      // read at the column only: in range on every row
+      if (!ok && cn.a3.size() == 5 && l.affine && ln.ty.dims == rn.ty.dims && std::all_of(l.off.begin(), l.off.end(), [](int64_t v) { return v == 0; })) ok = clamped_reads = true;
+      vectors_only = vectors_only && ok;
+    }
+    for (auto& sd : em.direct_vecs) vectors_only = vectors_only && sd.second == 0;
+    if (clamped_reads) for (int i : em.inputs) vectors_only = vectors_only && (g.nodes[i].ty.rank() <= 1 || g.nodes[i].ty.dims == rn.ty.dims);
+    else for (int i : em.inputs) vectors_only = vectors_only && g.nodes[i].ty.rank() <= 1;
     const bool late_mask = vectors_only && cn.a3.size() == 5;
     // The direct kernel: a lane holds one feature for all its pixels.  An epilogue that reads nothing but per-feature
     // vectors (broadcast along the result's feature dimension) takes the kernel's bounds test as an argument and guards
@@ -3499,10 +3508,11 @@ struct Planner {
       rix[n - 1].var = "i" + std::to_string(n - 1) + "b";
       o << "    const " << it << " lin0 = " << em.linear(rix, rn.ty.dims) << ";\n";
     }
+    if (late_mask && !em.direct_vecs.empty()) o << "    const " << it << " lin0c = rx_min<" << it << ">(lin0, " << rn.ty.numel() << " - NV);\n";
     for (auto& sd : em.direct_vecs) {
       const int slot = sd.first;
       const std::string st = info(g.nodes[em.inputs[slot]].ty.dt).stype;
-      o << "    const rx_vec<" << st << ", NV> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", NV>*>(in" << slot << " + lin0);\n";
+      o << "    const rx_vec<" << st << ", NV> d" << slot << " = *reinterpret_cast<const rx_vec<" << st << ", NV>*>(in" << slot << " + " << (late_mask ? "lin0c" : "lin0") << ");\n";
     }
     o << "    rx_vec<" << ost << ", NV> res;\n";
     o << "#pragma unroll\n    for (int l = 0; l < NV; ++l) {\n";
