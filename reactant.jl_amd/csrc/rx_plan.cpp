@@ -192,8 +192,8 @@ struct Planner {
   // number of readers.  The region is rebuilt on [image, row, column, channel]; the transposes after the products
   // that feed it and before the products that read it disappear, a tensor that enters it from elsewhere is transposed
   // once on the way in, and a value that something outside reads (a reduction over the pixels, the module's result) is
-  // transposed once on the way out.  Done when the transposes that disappear move at least twice the bytes of those
-  // that are added.
+  // transposed once on the way out.  Done when the transposes that disappear move at least one and a half times the
+  // bytes of those that are added.
   void channel_minor_regions() {
     if (!opt.nhwc_regions || !opt.nhwc_pools || !opt.mfma) return;
     const int N = (int)g.nodes.size();
@@ -276,7 +276,7 @@ struct Planner {
     }
     std::set<int> chosen;
     for (auto& kv : tally)
-      if (kv.second.t1 >= 1 && kv.second.t2 >= 1 && kv.second.saved >= 2.0 * kv.second.added) chosen.insert(kv.first);
+      if (kv.second.t1 >= 1 && kv.second.t2 >= 1 && kv.second.saved >= opt.nhwc_region_ratio * kv.second.added) chosen.insert(kv.first);
     if (chosen.empty()) return;
     auto member = [&](int x) { return role[x] != None && chosen.count(find(x)) > 0; };
     Graph out;
