@@ -292,6 +292,7 @@ rx::PlanOptions plan_options() {
   if (const char* e = getenv("RX_REDUCE_ROW_BLOCKS")) o.reduce_row_blocks = atoi(e) != 0;
   if (const char* e = getenv("RX_NHWC_REGIONS")) o.nhwc_regions = atoi(e) != 0;
   if (const char* e = getenv("RX_NHWC_REGION_RATIO")) o.nhwc_region_ratio = atof(e);
+  if (const char* e = getenv("RX_PAD_INTO_POOLS")) o.pad_into_pools = atoi(e) != 0;
   if (const char* e = getenv("RX_EPILOGUES")) o.product_epilogues = atoi(e) != 0;
   if (const char* e = getenv("RX_EPILOGUE_INIT")) o.epilogue_init = atoi(e) != 0;
   if (const char* e = getenv("RX_CHAIN_CONVS")) o.chain_convs = atoi(e) != 0;

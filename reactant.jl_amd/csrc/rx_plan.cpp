@@ -184,6 +184,87 @@ struct Planner {
     pools_between_convs();
     chain_convs();
     channel_minor_regions();
+    pad_into_pools();
+  }
+
+  // Zero padding of a pooled value, where the windows do not overlap (size = stride, no dilation, the extent a whole
+  // number of windows), is the pooling of the operand padded by that many windows: a window made of padding alone
+  // reduces to zero -- the maximum of -inf and zeros, or a sum of zeros -- and the other windows are the same ones.
+  // The padding then sits in the pooling kernel's reads and the padding map of the pooled value (the operand of the
+  // next convolution) disappears.
+  void pad_into_pools() {
+    if (!opt.pad_into_pools) return;
+    const int N = (int)g.nodes.size();
+    std::vector<int> nuse(N, 0);
+    for (auto& n : g.nodes) for (int i : n.in) nuse[i]++;
+    for (int r : g.results) nuse[r]++;
+    auto zero = [&](int x) {
+      const Node& c = g.nodes[x];
+      if (c.k != OpK::Constant || !c.splat || c.ty.rank() != 0) return false;
+      for (uint8_t b : c.data) if (b) return false;
+      return true;
+    };
+    std::map<int, int> pad_of_win, pad_of_red;   // window / reduction -> the padding that moves
+    std::set<int> moved;
+    for (const Node& p : g.nodes) {
+      if (p.k != OpK::Pad || !zero(p.in[1]) || !is_float(p.ty.dt)) continue;
+      const Node& r = g.nodes[p.in[0]];
+      if (r.k != OpK::Reduce || nuse[r.id] != 1 || (r.red != Red::Max && r.red != Red::Add)) continue;
+      const Node& w = g.nodes[r.in[0]];
+      const int rank = p.ty.rank();
+      if (w.k != OpK::Window || nuse[w.id] != 1 || g.nodes[w.in[0]].ty.rank() != rank || (int)r.a0.size() != rank) continue;
+      // (not along the minor dimension: the pooling kernel's vectors of outputs would no longer be whole)
+      bool ok = p.a0[rank - 1] == 0 && p.a1[rank - 1] == 0;
+      for (int d = 0; d < rank; ++d) {
+        ok = ok && r.a0[d] == d && w.a0[d] == w.a1[d] && w.a2[d] == 1 && g.nodes[w.in[0]].ty.dims[d] % w.a0[d] == 0 && p.a0[d] >= 0 && p.a1[d] >= 0 && p.a2[d] == 0;
+      }
+      // the reduction starts from the identity: -inf for a maximum, zero for a sum
+      const Node& init = g.nodes[r.in[1]];
+      if (init.k != OpK::Constant || !init.splat || init.ty.rank() != 0) continue;
+      const double iv = splat_as_double(init);
+      ok = ok && (r.red == Red::Max ? (std::isinf(iv) && iv < 0) : iv == 0.0);
+      if (!ok) continue;
+      pad_of_win[w.id] = p.id;
+      pad_of_red[r.id] = p.id;
+      moved.insert(p.id);
+    }
+    if (moved.empty()) return;
+    Graph out;
+    out.name = g.name;
+    out.module_name = g.module_name;
+    out.aliasing_output = g.aliasing_output;
+    std::vector<int> remap(N, -1);
+    for (const Node& n : g.nodes) {
+      Node c = n;
+      for (int& i : c.in) i = remap[i];
+      if (pad_of_win.count(n.id)) {
+        const Node& p = g.nodes[pad_of_win[n.id]];
+        const int rank = p.ty.rank();
+        Node np = p;            // the padding, on the operand, in units of windows
+        np.in = {remap[n.in[0]], remap[p.in[1]] >= 0 ? remap[p.in[1]] : -1};
+        if (np.in[1] < 0) {     // the zero comes later in the list than the window: give the new padding one of its own
+          Node z = g.nodes[p.in[1]];
+          np.in[1] = out.add(z);
+        }
+        np.ty = g.nodes[n.in[0]].ty;
+        for (int d = 0; d < rank; ++d) {
+          np.a0[d] = p.a0[d] * n.a0[d];
+          np.a1[d] = p.a1[d] * n.a0[d];
+          np.ty.dims[d] += np.a0[d] + np.a1[d];
+        }
+        c.in = {out.add(np)};
+        for (int d = 0; d < rank; ++d) c.ty.dims[rank + d] = p.ty.dims[d];
+      } else if (pad_of_red.count(n.id)) {
+        c.ty.dims = g.nodes[pad_of_red[n.id]].ty.dims;
+      } else if (moved.count(n.id)) {
+        remap[n.id] = remap[n.in[0]];
+        continue;
+      }
+      remap[n.id] = out.add(c);
+    }
+    for (int p : g.params) out.params.push_back(remap[p]);
+    for (int r : g.results) out.results.push_back(remap[r]);
+    g = std::move(out);
   }
 
   // What pools_between_convs does for a chain, for a region: a connected set of values between products with row
@@ -3809,9 +3890,9 @@ struct Planner {
     for (size_t k = 0; k < kept.size(); ++k) { ix[kept[k]].var = "o" + std::to_string(k); ix[kept[k]].hi = inn.ty.dims[kept[k]] - 1; }
     for (size_t k = 0; k < red.size(); ++k) { ix[red[k]].var = "r" + std::to_string(k); ix[red[k]].hi = inn.ty.dims[red[k]] - 1; }
     em.indent = 4 + 2 * (int)red.size();
-    Emitter e2(g, [&](int x) { return mat[x]; });
-    e2.excess_precision = opt.excess_precision;
-    e2.inputs = {};
+    // 16-bit elements whose minor dimension is kept (eight outputs per thread, below): padded reads at clamped
+    // positions and a select, so that the eight loads of a window element stay one 16-byte load
+    em.clamp_guards = opt.clamp_pad_reads && opt.window_reduce_vectors && info(inn.ty.dt).size == 2 && !kept.empty() && kept.back() == inn.ty.rank() - 1;
     std::string val = em.emit(rn.in[0], ix);
     std::string body = em.take_code();
     em.indent = 2;

@@ -61,6 +61,7 @@ struct PlanOptions {
   bool merge_parameter_maps = true;  // plain maps that read only the module's arguments run first, several of them as one launch
   bool nhwc_regions = true;     // the same for regions with several readers per value (residual additions): transposed once on the way in and out where needed
   double nhwc_region_ratio = 1.5;   // a region is rebuilt when the transposes that disappear move this many times the bytes of those that are added (two residual blocks: 3 against 2 tensors, 0.129 -> 0.115 ms)
+  bool pad_into_pools = true;   // zero padding of a pooled value (windows that do not overlap) moves onto the pooling's operand: no padding map
   bool epilogue_init = true;    // a bias added to a product on the streaming skeletons becomes the accumulators' first values
   bool row_fusion = true;       // fuse row reductions with their elementwise consumers
   bool lds_stencil = true;      // 3-D maps that read an input at several offsets stage it through LDS halo tiles

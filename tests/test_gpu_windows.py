@@ -462,7 +462,7 @@ def test_vgg11_forward_pass(rx, client, monkeypatch, dt, nhwc):
         pools = [ln.split("::")[1] for ln in rx.compile_offline(text).splitlines() if "kind=reduce_generic" in ln and "window" in ln]
         assert len(pools) == 5
         # the pools between two products: pure window reductions on the channel-minor layout when the rewrite is on
-        assert sum(d.strip() == "window reduce" for d in pools) == (4 if nhwc else 1), pools
+        assert sum("divide" not in d for d in pools) == (4 if nhwc else 1), pools
     ref = oracle_run(text, args, hifi=True)
     assert got[0].a.shape == (4, 10)
     _close(got[0].a, ref[0].a, {"f32": 2e-4, "bf16": 5e-2, "f16": 8e-3}[dt])
