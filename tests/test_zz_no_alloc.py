@@ -62,6 +62,15 @@ def test_no_alloc_matches_execute_sharded_on_two_calls_in_a_row(rx, client):
 }
 """
     _compare(rx, client, t, [np.arange(300, dtype=np.float32)], ["f32"])
+    # two chained 16-bit convolutions: the filters' layout maps as one launch with two results, the padded images, the
+    # first product's result on the second one's padded grid -- all of them temporaries in the array
+    import importlib
+    NN = importlib.import_module("reactant_jl_amd.nn_programs")
+    text, shapes = NN.conv_chain(2, 64, 24, 2, "bf16")
+    rng = np.random.default_rng(4)
+    arrays = [rx.encode((rng.normal(size=sh) * (0.05 if len(sh) == 4 and k > 0 else 1.0)).astype(np.float32), "bf16") for k, sh in enumerate(shapes)]
+    exe, _, _ = _compare(rx, client, text, arrays, ["bf16"] * len(shapes))
+    assert [l["kind"] for l in exe.launches()] == ["map", "map_transposed", "conv_bf16", "conv_bf16", "map_transposed"]
 
 
 def test_no_alloc_rejects_what_does_not_fit(rx, client):
